@@ -1,0 +1,77 @@
+"""Builds libmni_rocm.so (HIP kernels + C ABI) for gfx950 with hipcc.
+
+Usage: python -m framework_amd.build [--force]
+
+The library is built in-tree (framework_amd/lib/libmni_rocm.so).  hipcc
+cross-compiles gfx950 code objects without a GPU, so this runs anywhere the
+ROCm toolchain is installed.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "lib", "obj")
+LIB = os.path.join(HERE, "lib", "libmni_rocm.so")
+SOURCES = ["device.hip", "gemm_mfma.hip", "gemm_skinny.hip", "gemm.hip", "elementwise.hip", "engine.hip"]
+HEADERS = ["common.h", "gemm_internal.h", os.path.join("..", "..", "include", "mni_rocm.h")]
+
+# -packed-fp32-ops is switched off for device code: hipcc must not form
+# v_pk_*_f32 from ordinary float arithmetic on this target.
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _hipcc():
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    return "hipcc"
+
+
+def _stale(target, deps):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def _run(cmd):
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in p.stdout.splitlines() if "not a recognized feature for this target" not in l)
+    if p.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build(force=False, verbose=True):
+    os.makedirs(OBJ, exist_ok=True)
+    hipcc = _hipcc()
+    headers = [os.path.normpath(os.path.join(CSRC, h)) for h in HEADERS]
+    jobs = []
+    objs = []
+    for src in SOURCES:
+        s = os.path.join(CSRC, src)
+        o = os.path.join(OBJ, src.replace(".hip", ".o"))
+        objs.append(o)
+        if force or _stale(o, [s] + headers):
+            jobs.append([hipcc] + FLAGS + ["-c", s, "-o", o])
+    with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as ex:
+        for out in ex.map(_run, jobs):
+            if verbose and out.strip():
+                print(out)
+    if force or jobs or _stale(LIB, objs):
+        out = _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+        if verbose and out.strip():
+            print(out)
+    if verbose:
+        print("built %s (%d translation units recompiled)" % (LIB, len(jobs)))
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv)

@@ -1,0 +1,90 @@
+// Shared declarations of libmni_rocm.so: device context, allocator, error
+// reporting and the internal launchers the C ABI and the engine are built on.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/mni_rocm.h"
+
+namespace mni {
+
+// ---- error reporting -------------------------------------------------------
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define MNI_HIP_CHECK(expr)                                                              \
+    do {                                                                                 \
+        hipError_t e_ = (expr);                                                          \
+        if (e_ != hipSuccess)                                                            \
+            return ::mni::set_error(MNI_ERR_HIP, "%s failed: %s (%s:%d)", #expr,         \
+                                    hipGetErrorString(e_), __FILE__, __LINE__);          \
+    } while (0)
+
+#define MNI_TRY(expr)              \
+    do {                           \
+        int rc_ = (expr);          \
+        if (rc_ != MNI_OK) return rc_; \
+    } while (0)
+
+// ---- device context --------------------------------------------------------
+struct DeviceCtx {
+    bool ready = false;
+    int device = 0;
+    int compute_units = 0;
+    int clock_khz = 0;
+    char name[256] = {0};
+    hipStream_t stream = nullptr;
+};
+DeviceCtx &ctx();
+int ensure_init();  // initialises device 0 on first use
+
+// ---- caching allocator -----------------------------------------------------
+int dev_alloc(void **p, size_t bytes);  // contents undefined
+int dev_free(void *p);
+int dev_clear_cache();
+size_t dev_cached_bytes();  // bytes held in free lists
+
+// ---- launch helpers --------------------------------------------------------
+int check_launch(const char *what);  // hipGetLastError after a kernel launch
+
+// gemm.hip
+int sgemm(const mni_gemm_desc &d);
+
+// elementwise.hip: internal launchers (device pointers, element strides)
+struct StridedDesc {
+    int ndim;
+    int64_t shape[MNI_MAX_DIMS];
+    int64_t a_strides[MNI_MAX_DIMS];
+    int64_t b_strides[MNI_MAX_DIMS];
+};
+enum BinOp { BIN_ADD = 0, BIN_SUB = 1, BIN_MUL = 2 };
+enum UnOp { UN_RELU = 0, UN_GELU = 1, UN_NEG = 2, UN_SCALE = 3, UN_COPY = 4 };
+
+int k_fill(float *dst, float v, int64_t n);
+int k_axpy(float *dst, const float *src, float alpha, int64_t n);
+int k_scale_inplace(float *dst, float s, int64_t n);
+int k_strided_copy(float *dst, const float *src, const int64_t *shape, const int64_t *strides, int ndim);
+int k_binary_broadcast(float *out, const float *a, const float *b, const StridedDesc &d, int op);
+int k_binary_same(float *out, const float *a, const float *b, int64_t n, int op);
+int k_add_bias(float *out, const float *a, const float *bias, int64_t rows, int64_t cols);
+int k_unary(float *out, const float *x, int64_t n, int op, float s);
+// out = g * f'(x) for relu/gelu
+int k_unary_backward(float *out, const float *g, const float *x, int64_t n, int op);
+int k_mul_backward_same(float *ga, float *gb, const float *g, const float *a, const float *b, int64_t n);
+int k_colsum(float *out, const float *a, int64_t rows, int64_t cols);
+// out[o, i] = (sum_d a[o, d, i]) / div
+int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t inner, float div);
+// out[o, d, i] = g[o, i] / div
+int k_expand_dim(float *out, const float *g, int64_t outer, int64_t dim, int64_t inner, float div);
+// generic unbroadcast: out (orig shape, contiguous) = sum of g over broadcast dims
+int k_unbroadcast(float *out, const float *g, const int64_t *gshape, int gnd, const int64_t *oshape, int ond);
+int k_cross_entropy(float *loss, float *softmax, const float *logits, const int32_t *targets,
+                    int64_t n, int64_t v);
+int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t *targets,
+                             const float *grad_scalar, int64_t n, int64_t v);
+int k_sumsq_f64(double *out, const float *g, int64_t n);  // out += sum g^2 (device double)
+int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, float b1, float b2,
+            float eps, float wd, float bc1, float bc2);
+
+}  // namespace mni

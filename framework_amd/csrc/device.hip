@@ -1,0 +1,221 @@
+// Device singleton, caching allocator, copies and timing marks.
+// Counterpart of the cuda arm's GpuDevice (src/native/src/device.rs:29-48) and
+// CachingAllocator (src/native/src/allocator.rs:46-84) in the reference: one
+// device, one stream, kernels prebuilt into this library.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+namespace mni {
+
+static char g_err_shared[1024];
+
+int set_error(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err_shared, sizeof g_err_shared, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+DeviceCtx &ctx() {
+    static DeviceCtx c;
+    return c;
+}
+
+static int init_device(int device) {
+    DeviceCtx &c = ctx();
+    if (c.ready) {
+        if (device != c.device)
+            return set_error(MNI_ERR_INVALID, "library already initialised on device %d", c.device);
+        return MNI_OK;
+    }
+    int count = 0;
+    MNI_HIP_CHECK(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count)
+        return set_error(MNI_ERR_INVALID, "device %d out of range (%d visible)", device, count);
+    MNI_HIP_CHECK(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    MNI_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return set_error(MNI_ERR_INVALID, "libmni_rocm is built for gfx950 only, found %s", prop.gcnArchName);
+    c.device = device;
+    c.compute_units = prop.multiProcessorCount;
+    c.clock_khz = prop.clockRate;
+    snprintf(c.name, sizeof c.name, "%s (%s)", prop.name, prop.gcnArchName);
+    // Default priority on purpose: streams of mixed priority are avoided.
+    MNI_HIP_CHECK(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
+    c.ready = true;
+    return MNI_OK;
+}
+
+int ensure_init() {
+    if (ctx().ready) return MNI_OK;
+    return init_device(0);
+}
+
+int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return set_error(MNI_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+    return MNI_OK;
+}
+
+// ---- allocator --------------------------------------------------------------
+// Exact-size free lists keyed by the rounded request, like the reference's
+// allocator; sizes are rounded up to 256 B so that every buffer is aligned for
+// 16-byte vector access and small tensors share lists.
+struct Allocator {
+    std::unordered_map<size_t, std::vector<void *>> free_lists;
+    std::unordered_map<void *, size_t> live;  // ptr -> rounded size
+    size_t total = 0;
+    size_t cached = 0;
+};
+static Allocator &allocator() {
+    static Allocator a;
+    return a;
+}
+static size_t round_size(size_t bytes) {
+    if (bytes == 0) bytes = 4;
+    return (bytes + 255) & ~(size_t)255;
+}
+
+int dev_alloc(void **p, size_t bytes) {
+    MNI_TRY(ensure_init());
+    Allocator &a = allocator();
+    size_t sz = round_size(bytes);
+    auto it = a.free_lists.find(sz);
+    if (it != a.free_lists.end() && !it->second.empty()) {
+        *p = it->second.back();
+        it->second.pop_back();
+        a.cached -= sz;
+        a.live[*p] = sz;
+        return MNI_OK;
+    }
+    hipError_t e = hipMalloc(p, sz);
+    if (e != hipSuccess) {
+        // Give cached blocks back to the driver and retry once.
+        (void)hipGetLastError();
+        dev_clear_cache();
+        e = hipMalloc(p, sz);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return set_error(MNI_ERR_NOMEM, "hipMalloc(%zu) failed: %s", sz, hipGetErrorString(e));
+        }
+    }
+    a.total += sz;
+    a.live[*p] = sz;
+    return MNI_OK;
+}
+
+int dev_free(void *p) {
+    if (!p) return MNI_OK;
+    Allocator &a = allocator();
+    auto it = a.live.find(p);
+    if (it == a.live.end()) return set_error(MNI_ERR_INVALID, "free of a pointer this library did not allocate");
+    a.free_lists[it->second].push_back(p);
+    a.cached += it->second;
+    a.live.erase(it);
+    return MNI_OK;
+}
+
+int dev_clear_cache() {
+    Allocator &a = allocator();
+    bool any = false;
+    for (auto &kv : a.free_lists) any = any || !kv.second.empty();
+    if (!any) return MNI_OK;
+    // Cached blocks may still be read by queued kernels.
+    if (ctx().ready) MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+    for (auto &kv : a.free_lists) {
+        for (void *p : kv.second) {
+            (void)hipFree(p);
+            a.total -= kv.first;
+        }
+        kv.second.clear();
+    }
+    a.free_lists.clear();
+    a.cached = 0;
+    return MNI_OK;
+}
+
+size_t dev_cached_bytes() { return allocator().cached; }
+
+}  // namespace mni
+
+using namespace mni;
+
+extern "C" {
+
+int mni_rocm_init(int device) { return init_device(device); }
+
+int mni_rocm_device_info(char *name, size_t name_cap, int *compute_units, int *clock_khz) {
+    MNI_TRY(ensure_init());
+    if (name && name_cap) snprintf(name, name_cap, "%s", ctx().name);
+    if (compute_units) *compute_units = ctx().compute_units;
+    if (clock_khz) *clock_khz = ctx().clock_khz;
+    return MNI_OK;
+}
+
+const char *mni_rocm_last_error(void) { return g_err_shared; }
+
+int mni_rocm_malloc(void **ptr, size_t bytes) {
+    if (!ptr) return set_error(MNI_ERR_INVALID, "null out pointer");
+    return dev_alloc(ptr, bytes);
+}
+int mni_rocm_free(void *ptr) { return dev_free(ptr); }
+int mni_rocm_clear_cache(void) { return dev_clear_cache(); }
+
+int mni_rocm_h2d(void *dst, const void *src, size_t bytes) {
+    MNI_TRY(ensure_init());
+    if (bytes == 0) return MNI_OK;
+    MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
+    MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+    return MNI_OK;
+}
+int mni_rocm_d2h(void *dst, const void *src, size_t bytes) {
+    MNI_TRY(ensure_init());
+    if (bytes == 0) return MNI_OK;
+    MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
+    MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+    return MNI_OK;
+}
+int mni_rocm_d2d(void *dst, const void *src, size_t bytes) {
+    MNI_TRY(ensure_init());
+    if (bytes == 0) return MNI_OK;
+    MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx().stream));
+    return MNI_OK;
+}
+int mni_rocm_sync(void) {
+    MNI_TRY(ensure_init());
+    MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+    return MNI_OK;
+}
+
+int mni_rocm_event_create(void **event) {
+    MNI_TRY(ensure_init());
+    if (!event) return set_error(MNI_ERR_INVALID, "null out pointer");
+    hipEvent_t e;
+    MNI_HIP_CHECK(hipEventCreate(&e));
+    *event = (void *)e;
+    return MNI_OK;
+}
+int mni_rocm_event_record(void *event) {
+    MNI_TRY(ensure_init());
+    MNI_HIP_CHECK(hipEventRecord((hipEvent_t)event, ctx().stream));
+    return MNI_OK;
+}
+int mni_rocm_event_elapsed_ms(void *start, void *stop, float *ms) {
+    MNI_HIP_CHECK(hipEventSynchronize((hipEvent_t)stop));
+    MNI_HIP_CHECK(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return MNI_OK;
+}
+int mni_rocm_event_destroy(void *event) {
+    MNI_HIP_CHECK(hipEventDestroy((hipEvent_t)event));
+    return MNI_OK;
+}
+
+}  // extern "C"

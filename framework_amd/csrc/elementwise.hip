@@ -1,0 +1,685 @@
+// Bandwidth-bound support kernels around the GEMM path: fills, copies,
+// strided gathers (views made contiguous on the device), broadcast binary ops,
+// the Linear bias add and its column-sum gradient, activations, reductions
+// along one dim, cross-entropy and the AdamW update.  They replace the
+// per-element host loops of the reference's cpu arm (file:line at each kernel)
+// and the 256-thread one-element-per-thread kernels of its cuda arm
+// (src/native/kernels/elementwise.cu) with 16-byte accesses where the layout
+// allows.
+#include "common.h"
+
+namespace mni {
+
+static constexpr int TPB = 256;
+
+static inline unsigned grid_for(int64_t n, int per_block) {
+    int64_t b = (n + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    if (b > 0x7fffffffLL) b = 0x7fffffffLL;
+    return (unsigned)b;
+}
+static inline bool al16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+__device__ __forceinline__ float d_gelu(float x) {
+    // src/native/src/ops/activation.rs:15-18
+    const float s = 0.7978845608028654f;
+    return 0.5f * x * (1.0f + tanhf(s * (x + 0.044715f * x * x * x)));
+}
+__device__ __forceinline__ float d_gelu_grad(float x) {
+    // src/native/src/ops/activation.rs:20-28
+    const float s = 0.7978845608028654f;
+    const float inner = s * (x + 0.044715f * x * x * x);
+    const float th = tanhf(inner);
+    const float sech2 = 1.0f - th * th;
+    const float d_inner = s * (1.0f + 3.0f * 0.044715f * x * x);
+    return 0.5f * (1.0f + th) + 0.5f * x * sech2 * d_inner;
+}
+
+// ---- fill / axpy / scale ------------------------------------------------------
+__global__ void fill_kernel(float *__restrict__ dst, float v, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = v;
+}
+__global__ void fill4_kernel(float4 *__restrict__ dst, float v, int64_t n4) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const float4 f = make_float4(v, v, v, v);
+    for (; i < n4; i += stride) dst[i] = f;
+}
+int k_fill(float *dst, float v, int64_t n) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (al16(dst) && (n % 4) == 0) {
+        hipLaunchKernelGGL(fill4_kernel, dim3(grid_for(n / 4, TPB * 4)), dim3(TPB), 0, ctx().stream,
+                           reinterpret_cast<float4 *>(dst), v, n / 4);
+    } else {
+        hipLaunchKernelGGL(fill_kernel, dim3(grid_for(n, TPB * 4)), dim3(TPB), 0, ctx().stream, dst, v, n);
+    }
+    return check_launch("fill");
+}
+
+// dst += alpha * src  (src/native/src/tensor.rs:272-290 accumulate_grad / add_inplace)
+__global__ void axpy_kernel(float *__restrict__ dst, const float *__restrict__ src, float alpha, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] += alpha * src[i];
+}
+__global__ void axpy4_kernel(float4 *__restrict__ dst, const float4 *__restrict__ src, float alpha, int64_t n4) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += stride) {
+        float4 d = dst[i];
+        const float4 s = src[i];
+        d.x += alpha * s.x; d.y += alpha * s.y; d.z += alpha * s.z; d.w += alpha * s.w;
+        dst[i] = d;
+    }
+}
+int k_axpy(float *dst, const float *src, float alpha, int64_t n) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (al16(dst) && al16(src) && (n % 4) == 0) {
+        hipLaunchKernelGGL(axpy4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+                           reinterpret_cast<float4 *>(dst), reinterpret_cast<const float4 *>(src), alpha, n / 4);
+    } else {
+        hipLaunchKernelGGL(axpy_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, dst, src, alpha, n);
+    }
+    return check_launch("axpy");
+}
+
+__global__ void scale_kernel(float *__restrict__ dst, float s, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] *= s;
+}
+int k_scale_inplace(float *dst, float s, int64_t n) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(scale_kernel, dim3(grid_for(n, TPB * 4)), dim3(TPB), 0, ctx().stream, dst, s, n);
+    return check_launch("scale");
+}
+
+// ---- strided gather -------------------------------------------------------------
+// dst[i] = src[sum_d coord_d(i) * stride_d]: make_contiguous_data
+// (src/native/src/tensor.rs:292-309) and permute_f32
+// (src/native/kernels/elementwise.cu:67-81) without the 4-dim / i32 limits.
+struct GatherDesc {
+    int ndim;
+    int64_t shape[MNI_MAX_DIMS];
+    int64_t strides[MNI_MAX_DIMS];
+};
+__global__ void gather_kernel(float *__restrict__ dst, const float *__restrict__ src, const GatherDesc d, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) {
+        int64_t rem = i, off = 0;
+        for (int k = d.ndim - 1; k >= 0; --k) {
+            const int64_t c = rem % d.shape[k];
+            rem /= d.shape[k];
+            off += c * d.strides[k];
+        }
+        dst[i] = src[off];
+    }
+}
+// Batched 2-D transpose through LDS for the common "swap the last two dims"
+// view: src element (b, r, c) at b*bs + r*1 + c*cs_ (row axis contiguous in
+// memory), dst contiguous [b][r][c].
+__global__ void transpose_tile_kernel(float *__restrict__ dst, const float *__restrict__ src, int64_t rows,
+                                      int64_t cols, int64_t src_col_stride, int64_t src_bs) {
+    __shared__ float tile[32][33];
+    const int64_t b = blockIdx.z;
+    const int64_t r0 = (int64_t)blockIdx.y * 32, c0 = (int64_t)blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    const float *s = src + b * src_bs;
+    float *d = dst + b * rows * cols;
+    for (int j = ty; j < 32; j += 8) {
+        const int64_t r = r0 + tx, c = c0 + j;  // read along r (contiguous)
+        if (r < rows && c < cols) tile[j][tx] = s[r + c * src_col_stride];
+    }
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8) {
+        const int64_t r = r0 + j, c = c0 + tx;  // write along c (contiguous)
+        if (r < rows && c < cols) d[r * cols + c] = tile[tx][j];
+    }
+}
+int k_strided_copy(float *dst, const float *src, const int64_t *shape, const int64_t *strides, int ndim) {
+    MNI_TRY(ensure_init());
+    if (ndim < 0 || ndim > MNI_MAX_DIMS) return set_error(MNI_ERR_INVALID, "strided_copy: ndim %d out of range", ndim);
+    int64_t n = 1;
+    for (int i = 0; i < ndim; ++i) {
+        if (shape[i] < 0) return set_error(MNI_ERR_INVALID, "strided_copy: negative extent");
+        n *= shape[i];
+    }
+    if (n == 0) return MNI_OK;
+    // Fast path: last two dims swapped relative to memory, leading dims with
+    // one uniform stride.
+    if (ndim >= 2 && strides[ndim - 2] == 1 && shape[ndim - 2] > 1 && shape[ndim - 1] > 1) {
+        const int64_t rows = shape[ndim - 2], cols = shape[ndim - 1];
+        int64_t batch = 1, bs = 0;
+        bool uniform = true;
+        if (ndim > 2) {
+            bs = strides[ndim - 3];
+            int64_t expect = bs;
+            for (int k = ndim - 3; k >= 0; --k) {
+                if (shape[k] != 1 && strides[k] != expect) uniform = false;
+                expect *= shape[k];
+                batch *= shape[k];
+            }
+        }
+        if (uniform && batch <= 65535) {
+            dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32), (unsigned)batch);
+            if (grid.y <= 65535) {
+                hipLaunchKernelGGL(transpose_tile_kernel, grid, dim3(256), 0, ctx().stream, dst, src, rows, cols,
+                                   strides[ndim - 1], bs);
+                return check_launch("transpose_tile");
+            }
+        }
+    }
+    GatherDesc d;
+    d.ndim = ndim;
+    for (int i = 0; i < ndim; ++i) { d.shape[i] = shape[i]; d.strides[i] = strides[i]; }
+    hipLaunchKernelGGL(gather_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, dst, src, d, n);
+    return check_launch("gather");
+}
+
+// ---- broadcast binary -----------------------------------------------------------
+// broadcast_binary (src/native/src/ops/elementwise.rs:20-56): operands are
+// addressed by their own strides with 0 on broadcast dims, so views need no copy.
+__device__ __forceinline__ float bin_apply(float x, float y, int op) {
+    return op == BIN_ADD ? x + y : op == BIN_SUB ? x - y : x * y;
+}
+__global__ void binary_bcast_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b,
+                                    const StridedDesc d, int64_t n, int op) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) {
+        int64_t rem = i, ao = 0, bo = 0;
+        for (int k = d.ndim - 1; k >= 0; --k) {
+            const int64_t c = rem % d.shape[k];
+            rem /= d.shape[k];
+            ao += c * d.a_strides[k];
+            bo += c * d.b_strides[k];
+        }
+        out[i] = bin_apply(a[ao], b[bo], op);
+    }
+}
+int k_binary_broadcast(float *out, const float *a, const float *b, const StridedDesc &d, int op) {
+    MNI_TRY(ensure_init());
+    int64_t n = 1;
+    for (int i = 0; i < d.ndim; ++i) n *= d.shape[i];
+    if (n <= 0) return MNI_OK;
+    hipLaunchKernelGGL(binary_bcast_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, d, n, op);
+    return check_launch("binary_broadcast");
+}
+
+__global__ void binary_same_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b,
+                                   int64_t n, int op) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) out[i] = bin_apply(a[i], b[i], op);
+}
+__global__ void binary_same4_kernel(float4 *__restrict__ out, const float4 *__restrict__ a,
+                                    const float4 *__restrict__ b, int64_t n4, int op) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += step) {
+        const float4 x = a[i], y = b[i];
+        out[i] = make_float4(bin_apply(x.x, y.x, op), bin_apply(x.y, y.y, op), bin_apply(x.z, y.z, op),
+                             bin_apply(x.w, y.w, op));
+    }
+}
+int k_binary_same(float *out, const float *a, const float *b, int64_t n, int op) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (al16(out) && al16(a) && al16(b) && (n % 4) == 0) {
+        hipLaunchKernelGGL(binary_same4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+                           reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(a),
+                           reinterpret_cast<const float4 *>(b), n / 4, op);
+    } else {
+        hipLaunchKernelGGL(binary_same_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, n, op);
+    }
+    return check_launch("binary_same");
+}
+
+// out[r, c] = a[r, c] + bias[c]   (src/native/kernels/elementwise.cu:43-47)
+__global__ void add_bias_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ bias,
+                                int64_t n, int64_t cols) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) out[i] = a[i] + bias[i % cols];
+}
+__global__ void add_bias4_kernel(float4 *__restrict__ out, const float4 *__restrict__ a,
+                                 const float4 *__restrict__ bias, int64_t n4, int64_t cols4) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += step) {
+        const float4 x = a[i], y = bias[i % cols4];
+        out[i] = make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w);
+    }
+}
+int k_add_bias(float *out, const float *a, const float *bias, int64_t rows, int64_t cols) {
+    const int64_t n = rows * cols;
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (al16(out) && al16(a) && al16(bias) && (cols % 4) == 0) {
+        hipLaunchKernelGGL(add_bias4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+                           reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(a),
+                           reinterpret_cast<const float4 *>(bias), n / 4, cols / 4);
+    } else {
+        hipLaunchKernelGGL(add_bias_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, bias, n, cols);
+    }
+    return check_launch("add_bias");
+}
+
+// ---- unary ----------------------------------------------------------------------
+__device__ __forceinline__ float un_apply(float x, int op, float s) {
+    switch (op) {
+    case UN_RELU: return fmaxf(x, 0.0f);  // f32::max(x, 0.0), activation.rs:116
+    case UN_GELU: return d_gelu(x);
+    case UN_NEG: return -x;
+    case UN_SCALE: return x * s;
+    default: return x;
+    }
+}
+__global__ void unary_kernel(float *__restrict__ out, const float *__restrict__ x, int64_t n, int op, float s) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) out[i] = un_apply(x[i], op, s);
+}
+__global__ void unary4_kernel(float4 *__restrict__ out, const float4 *__restrict__ x, int64_t n4, int op, float s) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += step) {
+        const float4 v = x[i];
+        out[i] = make_float4(un_apply(v.x, op, s), un_apply(v.y, op, s), un_apply(v.z, op, s), un_apply(v.w, op, s));
+    }
+}
+int k_unary(float *out, const float *x, int64_t n, int op, float s) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (al16(out) && al16(x) && (n % 4) == 0) {
+        hipLaunchKernelGGL(unary4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+                           reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(x), n / 4, op, s);
+    } else {
+        hipLaunchKernelGGL(unary_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, n, op, s);
+    }
+    return check_launch("unary");
+}
+
+// relu_backward / gelu_backward (src/native/src/ops/activation.rs:74-84,154-164)
+__global__ void unary_bwd_kernel(float *__restrict__ out, const float *__restrict__ g, const float *__restrict__ x,
+                                 int64_t n, int op) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) {
+        const float xv = x[i], gv = g[i];
+        out[i] = op == UN_RELU ? (xv > 0.0f ? gv : 0.0f) : gv * d_gelu_grad(xv);
+    }
+}
+int k_unary_backward(float *out, const float *g, const float *x, int64_t n, int op) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(unary_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, x, n, op);
+    return check_launch("unary_backward");
+}
+
+// mul_backward for equal shapes (src/native/src/ops/elementwise.rs:348-390)
+__global__ void mul_bwd_kernel(float *__restrict__ ga, float *__restrict__ gb, const float *__restrict__ g,
+                               const float *__restrict__ a, const float *__restrict__ b, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) {
+        const float gv = g[i], av = a[i], bv = b[i];
+        ga[i] = gv * bv;
+        gb[i] = gv * av;
+    }
+}
+int k_mul_backward_same(float *ga, float *gb, const float *g, const float *a, const float *b, int64_t n) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(mul_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, ga, gb, g, a, b, n);
+    return check_launch("mul_backward");
+}
+
+// ---- column sum -------------------------------------------------------------------
+// out[c] = sum_r a[r, c]: the bias gradient (unbroadcast of [rows, C] to [C],
+// src/native/src/utils.rs:39-66) and the batch reduction of a broadcast matmul
+// operand.  Two deterministic passes: row blocks into partials, then partials
+// in block order.
+static constexpr int CS_ROWS = 128;  // rows per block in pass 1
+__global__ void colsum_partial_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t rows,
+                                      int64_t cols) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * CS_ROWS;
+    const int64_t r1 = min(rows, r0 + CS_ROWS);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int64_t r = r0;
+    for (; r + 3 < r1; r += 4) {
+        s0 += a[r * cols + c];
+        s1 += a[(r + 1) * cols + c];
+        s2 += a[(r + 2) * cols + c];
+        s3 += a[(r + 3) * cols + c];
+    }
+    for (; r < r1; ++r) s0 += a[r * cols + c];
+    part[(int64_t)blockIdx.y * cols + c] = (s0 + s1) + (s2 + s3);
+}
+__global__ void colsum_final_kernel(float *__restrict__ out, const float *__restrict__ part, int64_t nparts,
+                                    int64_t cols) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    float s = 0.f;
+    for (int64_t p = 0; p < nparts; ++p) s += part[p * cols + c];
+    out[c] = s;
+}
+int k_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
+    if (cols <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (rows <= 0) return k_fill(out, 0.0f, cols);
+    const int64_t nparts = (rows + CS_ROWS - 1) / CS_ROWS;
+    if (nparts > 65535) return set_error(MNI_ERR_INVALID, "colsum: too many rows (%lld)", (long long)rows);
+    const dim3 block(TPB);
+    const unsigned gx = (unsigned)((cols + TPB - 1) / TPB);
+    if (nparts == 1) {
+        hipLaunchKernelGGL(colsum_partial_kernel, dim3(gx, 1), block, 0, ctx().stream, out, a, rows, cols);
+        return check_launch("colsum");
+    }
+    void *part = nullptr;
+    MNI_TRY(dev_alloc(&part, (size_t)nparts * cols * sizeof(float)));
+    hipLaunchKernelGGL(colsum_partial_kernel, dim3(gx, (unsigned)nparts), block, 0, ctx().stream, (float *)part, a, rows, cols);
+    int rc = check_launch("colsum_partial");
+    if (rc == MNI_OK) {
+        hipLaunchKernelGGL(colsum_final_kernel, dim3(gx), block, 0, ctx().stream, out, (const float *)part, nparts, cols);
+        rc = check_launch("colsum_final");
+    }
+    dev_free(part);
+    return rc;
+}
+
+// ---- reduce / expand along one dim ----------------------------------------------------
+// sum / mean along `dim` (src/native/src/ops/reduce.rs:13-46,169-184): input
+// viewed as [outer, dim, inner].
+__global__ void reduce_inner_kernel(float *__restrict__ out, const float *__restrict__ a, int64_t outer, int64_t dim,
+                                    int64_t inner, float div) {
+    // one thread per output, consecutive threads along `inner` (coalesced);
+    // terms are added in increasing d like the reference's flat-order loop.
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= outer * inner) return;
+    const int64_t o = idx / inner, i = idx - o * inner;
+    const float *p = a + o * dim * inner + i;
+    float s = 0.f;
+    for (int64_t d = 0; d < dim; ++d) s += p[d * inner];
+    out[idx] = s / div;
+}
+__global__ void reduce_rows_kernel(float *__restrict__ out, const float *__restrict__ a, int64_t outer, int64_t dim,
+                                   float div) {
+    // inner == 1: one wavefront per row, lanes stride the row.
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= outer) return;
+    const float *p = a + row * dim;
+    float s = 0.f;
+    for (int64_t d = lane; d < dim; d += 64) s += p[d];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (lane == 0) out[row] = s / div;
+}
+int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t inner, float div) {
+    const int64_t n = outer * inner;
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (inner == 1 && dim >= 256) {
+        hipLaunchKernelGGL(reduce_rows_kernel, dim3(grid_for(outer, 4)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, div);
+        return check_launch("reduce_rows");
+    }
+    hipLaunchKernelGGL(reduce_inner_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, inner, div);
+    return check_launch("reduce_inner");
+}
+
+// sum_backward / mean_backward (src/native/src/ops/reduce.rs:94-118,232-263)
+__global__ void expand_dim_kernel(float *__restrict__ out, const float *__restrict__ g, int64_t outer, int64_t dim,
+                                  int64_t inner, float div, int64_t n) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; idx < n; idx += step) {
+        const int64_t o = idx / (dim * inner);
+        const int64_t i = idx % inner;
+        out[idx] = g[o * inner + i] / div;
+    }
+}
+int k_expand_dim(float *out, const float *g, int64_t outer, int64_t dim, int64_t inner, float div) {
+    const int64_t n = outer * dim * inner;
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(expand_dim_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, outer, dim, inner, div, n);
+    return check_launch("expand_dim");
+}
+
+// ---- generic unbroadcast ----------------------------------------------------------------
+// One thread per output element; it walks the broadcast coordinates in the
+// reference's flat order (src/native/src/utils.rs:55-64), so the sum order per
+// element is the reference's.
+struct UnbDesc {
+    int gnd;                          // grad dims
+    int64_t gshape[MNI_MAX_DIMS];
+    int64_t gstr[MNI_MAX_DIMS];
+    int64_t oshape_al[MNI_MAX_DIMS];  // orig shape right-aligned to gnd (1 where missing)
+    int nred;                         // reduced dims, outermost first
+    int red_dim[MNI_MAX_DIMS];
+};
+__global__ void unbroadcast_kernel(float *__restrict__ out, const float *__restrict__ g, const UnbDesc d, int64_t on,
+                                   int64_t red_total) {
+    const int64_t oi = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (oi >= on) return;
+    // base offset in g from the output coordinate
+    int64_t rem = oi, base = 0;
+    for (int k = d.gnd - 1; k >= 0; --k) {
+        const int64_t ext = d.oshape_al[k];
+        const int64_t c = rem % ext;
+        rem /= ext;
+        base += c * d.gstr[k];
+    }
+    float s = 0.f;
+    for (int64_t t = 0; t < red_total; ++t) {
+        int64_t r = t, off = 0;
+        for (int k = d.nred - 1; k >= 0; --k) {
+            const int dim = d.red_dim[k];
+            const int64_t c = r % d.gshape[dim];
+            r /= d.gshape[dim];
+            off += c * d.gstr[dim];
+        }
+        s += g[base + off];
+    }
+    out[oi] = s;
+}
+int k_unbroadcast(float *out, const float *g, const int64_t *gshape, int gnd, const int64_t *oshape, int ond) {
+    MNI_TRY(ensure_init());
+    if (gnd > MNI_MAX_DIMS || ond > gnd) return set_error(MNI_ERR_INVALID, "unbroadcast: bad ranks %d -> %d", gnd, ond);
+    UnbDesc d;
+    d.gnd = gnd;
+    int64_t gs = 1;
+    for (int k = gnd - 1; k >= 0; --k) { d.gshape[k] = gshape[k]; d.gstr[k] = gs; gs *= gshape[k]; }
+    const int off = gnd - ond;
+    int64_t on = 1, red_total = 1;
+    d.nred = 0;
+    for (int k = 0; k < gnd; ++k) {
+        const int64_t ext = k < off ? 1 : oshape[k - off];
+        d.oshape_al[k] = ext;
+        on *= ext;
+        if (ext == 1 && gshape[k] != 1) { d.red_dim[d.nred++] = k; red_total *= gshape[k]; }
+        else if (ext != gshape[k]) return set_error(MNI_ERR_INVALID, "unbroadcast: shapes do not broadcast");
+    }
+    if (on <= 0) return MNI_OK;
+    hipLaunchKernelGGL(unbroadcast_kernel, dim3(grid_for(on, TPB)), dim3(TPB), 0, ctx().stream, out, g, d, on, red_total);
+    return check_launch("unbroadcast");
+}
+
+// ---- cross-entropy --------------------------------------------------------------------
+// src/native/src/ops/loss.rs:24-67: per row max, exp, normalise, -ln p[target];
+// loss = mean over rows.  One wavefront per row; the row losses are summed by
+// a single wavefront in a fixed order.
+__global__ void ce_rows_kernel(float *__restrict__ row_loss, float *__restrict__ sm, const float *__restrict__ logits,
+                               const int32_t *__restrict__ targets, int64_t n, int64_t v) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n) return;
+    const float *x = logits + row * v;
+    float *p = sm + row * v;
+    float mx = -INFINITY;
+    for (int64_t j = lane; j < v; j += 64) mx = fmaxf(mx, x[j]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+    for (int64_t j = lane; j < v; j += 64) {
+        const float e = expf(x[j] - mx);
+        p[j] = e;
+        sum += e;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    for (int64_t j = lane; j < v; j += 64) p[j] = p[j] / sum;
+    if (lane == 0) {
+        const int32_t t = targets[row];
+        const float e = expf(x[t] - mx);
+        row_loss[row] = -logf(e / sum);
+    }
+}
+__global__ void ce_mean_kernel(float *__restrict__ loss, const float *__restrict__ row_loss, int64_t n) {
+    const int lane = threadIdx.x;
+    float s = 0.f;
+    for (int64_t i = lane; i < n; i += 64) s += row_loss[i];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (lane == 0) loss[0] = s / (float)n;
+}
+int k_cross_entropy(float *loss, float *softmax, const float *logits, const int32_t *targets, int64_t n, int64_t v) {
+    MNI_TRY(ensure_init());
+    if (n <= 0 || v <= 0) return set_error(MNI_ERR_INVALID, "cross_entropy: empty logits");
+    void *rl = nullptr;
+    MNI_TRY(dev_alloc(&rl, (size_t)n * sizeof(float)));
+    hipLaunchKernelGGL(ce_rows_kernel, dim3(grid_for(n, 4)), dim3(TPB), 0, ctx().stream, (float *)rl, softmax, logits, targets, n, v);
+    int rc = check_launch("ce_rows");
+    if (rc == MNI_OK) {
+        hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(64), 0, ctx().stream, loss, (const float *)rl, n);
+        rc = check_launch("ce_mean");
+    }
+    dev_free(rl);
+    return rc;
+}
+// src/native/src/ops/loss.rs:131-149: (softmax - onehot) * (grad / n)
+__global__ void ce_bwd_kernel(float *__restrict__ dl, const float *__restrict__ sm, const int32_t *__restrict__ targets,
+                              const float *__restrict__ grad, int64_t n, int64_t v) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    const float scale = grad[0] / (float)n;
+    for (; idx < n * v; idx += step) {
+        const int64_t row = idx / v, j = idx - row * v;
+        float p = sm[idx];
+        if (j == targets[row]) p -= 1.0f;
+        dl[idx] = p * scale;
+    }
+}
+int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t *targets, const float *grad_scalar,
+                             int64_t n, int64_t v) {
+    MNI_TRY(ensure_init());
+    if (n * v <= 0) return MNI_OK;
+    hipLaunchKernelGGL(ce_bwd_kernel, dim3(grid_for(n * v, TPB * 2)), dim3(TPB), 0, ctx().stream, dlogits, softmax, targets, grad_scalar, n, v);
+    return check_launch("ce_backward");
+}
+
+// ---- optimiser -----------------------------------------------------------------------
+// grad_norm (src/native/src/ops/optimizer.rs:126-138): f64 accumulation.
+__global__ void sumsq_kernel(double *__restrict__ part, const float *__restrict__ g, int64_t n) {
+    __shared__ double sh[4];
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    double s = 0.0;
+    for (; i < n; i += step) { const double v = (double)g[i]; s += v * v; }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) part[blockIdx.x] = (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+__global__ void sumsq_final_kernel(double *__restrict__ out, const double *__restrict__ part, int nparts) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        double s = 0.0;
+        for (int p = 0; p < nparts; ++p) s += part[p];
+        out[0] += s;
+    }
+}
+int k_sumsq_f64(double *out, const float *g, int64_t n) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    int blocks = (int)grid_for(n, TPB * 8);
+    if (blocks > 1024) blocks = 1024;
+    void *part = nullptr;
+    MNI_TRY(dev_alloc(&part, (size_t)blocks * sizeof(double)));
+    hipLaunchKernelGGL(sumsq_kernel, dim3(blocks), dim3(TPB), 0, ctx().stream, (double *)part, g, n);
+    int rc = check_launch("sumsq");
+    if (rc == MNI_OK) {
+        hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), dim3(64), 0, ctx().stream, out, (const double *)part, blocks);
+        rc = check_launch("sumsq_final");
+    }
+    dev_free(part);
+    return rc;
+}
+
+// adamw_step, cpu arm (src/native/src/ops/optimizer.rs:21-65): decoupled decay
+// only when weight_decay > 0.
+__global__ void adamw_kernel(float *__restrict__ p, float *__restrict__ m, float *__restrict__ v,
+                             const float *__restrict__ g, int64_t n, float lr, float b1, float b2, float eps, float wd,
+                             float bc1, float bc2) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) {
+        const float gv = g[i];
+        float pv = p[i];
+        if (wd > 0.0f) pv *= 1.0f - lr * wd;
+        const float mv = b1 * m[i] + (1.0f - b1) * gv;
+        const float vv = b2 * v[i] + (1.0f - b2) * gv * gv;
+        m[i] = mv;
+        v[i] = vv;
+        const float m_hat = mv / bc1;
+        const float v_hat = vv / bc2;
+        p[i] = pv - lr * m_hat / (sqrtf(v_hat) + eps);
+    }
+}
+int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, float b1, float b2, float eps, float wd,
+            float bc1, float bc2) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(adamw_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, p, m, v, g, n, lr, b1, b2, eps, wd, bc1, bc2);
+    return check_launch("adamw");
+}
+
+}  // namespace mni
+
+using namespace mni;
+
+extern "C" {
+int mni_rocm_strided_copy(float *dst, const float *src, const int64_t *shape, const int64_t *src_strides, int ndim) {
+    if (!dst || !src || (ndim > 0 && (!shape || !src_strides))) return set_error(MNI_ERR_INVALID, "strided_copy: null argument");
+    return k_strided_copy(dst, src, shape, src_strides, ndim);
+}
+int mni_rocm_add_bias(float *out, const float *a, const float *bias, int64_t rows, int64_t cols) {
+    if (rows < 0 || cols < 0) return set_error(MNI_ERR_INVALID, "add_bias: negative extent");
+    if (rows * cols > 0 && (!out || !a || !bias)) return set_error(MNI_ERR_INVALID, "add_bias: null argument");
+    return k_add_bias(out, a, bias, rows, cols);
+}
+int mni_rocm_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
+    if (rows < 0 || cols < 0) return set_error(MNI_ERR_INVALID, "colsum: negative extent");
+    if (cols > 0 && (!out || (rows > 0 && !a))) return set_error(MNI_ERR_INVALID, "colsum: null argument");
+    return k_colsum(out, a, rows, cols);
+}
+int mni_rocm_axpy(float *dst, const float *src, float alpha, int64_t n) {
+    if (n < 0) return set_error(MNI_ERR_INVALID, "axpy: negative length");
+    if (n > 0 && (!dst || !src)) return set_error(MNI_ERR_INVALID, "axpy: null argument");
+    return k_axpy(dst, src, alpha, n);
+}
+int mni_rocm_fill(float *dst, float value, int64_t n) {
+    if (n < 0) return set_error(MNI_ERR_INVALID, "fill: negative length");
+    if (n > 0 && !dst) return set_error(MNI_ERR_INVALID, "fill: null argument");
+    return k_fill(dst, value, n);
+}
+}

@@ -1,0 +1,1215 @@
+// Engine level of libmni_rocm.so: a device-resident counterpart of the
+// reference's Engine { store, tape } (src/native/src/lib.rs:19-39) for the
+// matmul path and its callers.  Tensors are ids into a slot vector with LIFO
+// id recycling (src/native/src/tensor.rs:96-113); buffers live in HBM and are
+// reference-counted, so permute() is a zero-copy view and a transposed matmul
+// operand is only a pair of swapped strides handed to the GEMM.  In-place
+// writers (gradient accumulation, zero_grad, clipping, AdamW) copy a shared
+// buffer first, which keeps the reference's value semantics (its permute
+// clones the buffer, src/native/src/ops/layout.rs:125).
+#include <math.h>
+#include <string.h>
+
+#include <memory>
+#include <vector>
+
+#include "common.h"
+
+namespace mni {
+namespace {
+
+struct Buf {
+    float *p = nullptr;
+    size_t n = 0;  // floats
+    ~Buf() { if (p) dev_free(p); }
+};
+using BufP = std::shared_ptr<Buf>;
+
+static BufP new_buf(size_t n) {
+    void *p = nullptr;
+    if (dev_alloc(&p, (n ? n : 1) * sizeof(float)) != MNI_OK) return nullptr;
+    BufP b = std::make_shared<Buf>();
+    b->p = (float *)p;
+    b->n = n;
+    return b;
+}
+
+using Shape = std::vector<int64_t>;
+
+// src/native/src/tensor.rs:27-37 GpuTensor
+struct Tensor {
+    bool live = false;
+    BufP buf;
+    Shape shape, strides;
+    int64_t size = 0;
+    bool requires_grad = false;
+    int64_t grad = -1;
+    BufP adam_m, adam_v;
+};
+
+enum Op {  // subset of src/native/src/autograd.rs:28-62 plus the fused Linear
+    OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
+    OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY, OP_LINEAR
+};
+
+// src/native/src/autograd.rs:65-70 TapeEntry
+struct Entry {
+    int op;
+    uint32_t output_id;
+    uint32_t inputs[3];
+    int n_inputs;
+    Shape saved_shape;   // Shape / TensorAndShape / Permutation original shape
+    Shape saved_perm;
+    float scalar = 0.f;
+    int act = 0;         // OP_LINEAR: epilogue
+    uint32_t aux = MNI_BAD_ID;  // cross-entropy softmax / linear pre-activation
+    std::shared_ptr<void> targets;  // device int32 targets
+    int64_t ce_n = 0, ce_v = 0;
+};
+
+struct Tape {
+    std::vector<Entry> entries;
+    bool enabled = true;
+    void record(Entry &&e) { if (enabled) entries.push_back(std::move(e)); }
+};
+
+struct Engine {
+    std::vector<Tensor> tensors;
+    std::vector<uint32_t> free_ids;
+    Tape tape;
+};
+static Engine &eng() {
+    static Engine e;
+    return e;
+}
+
+// ---- shape helpers -----------------------------------------------------------
+static Shape compute_strides(const Shape &shape) {  // tensor.rs:7-17
+    Shape s(shape.size(), 0);
+    if (shape.empty()) return s;
+    s.back() = 1;
+    for (int i = (int)shape.size() - 2; i >= 0; --i) s[i] = s[i + 1] * shape[i + 1];
+    return s;
+}
+static int64_t shape_size(const Shape &shape) {  // tensor.rs:19-21
+    int64_t p = 1;
+    for (int64_t d : shape) p *= d;
+    return p < 1 ? 1 : p;
+}
+static int64_t shape_size(const int64_t *s, int n) {
+    int64_t p = 1;
+    for (int i = 0; i < n; ++i) p *= s[i];
+    return p < 1 ? 1 : p;
+}
+static bool is_contiguous(const Tensor &t) {  // tensor.rs:41-53
+    int64_t expected = 1;
+    for (int i = (int)t.shape.size() - 1; i >= 0; --i) {
+        if (t.strides[i] != expected) return false;
+        expected *= t.shape[i];
+    }
+    return true;
+}
+static bool broadcast_shape(const Shape &a, const Shape &b, Shape *out) {  // utils.rs:3-20
+    const size_t n = a.size() > b.size() ? a.size() : b.size();
+    out->assign(n, 0);
+    for (size_t i = 0; i < n; ++i) {
+        const int64_t da = i < n - a.size() ? 1 : a[i - (n - a.size())];
+        const int64_t db = i < n - b.size() ? 1 : b[i - (n - b.size())];
+        if (da == db) (*out)[i] = da;
+        else if (da == 1) (*out)[i] = db;
+        else if (db == 1) (*out)[i] = da;
+        else return false;
+    }
+    return true;
+}
+
+// ---- store ----------------------------------------------------------------------
+static Tensor *get(uint32_t id) {  // tensor.rs:115-117
+    Engine &e = eng();
+    if (id >= e.tensors.size() || !e.tensors[id].live) {
+        set_error(MNI_ERR_FREED, "tensor already freed (id %u)", id);
+        return nullptr;
+    }
+    return &e.tensors[id];
+}
+// Shapes are taken by value: a caller may pass a reference into the slot
+// vector, which emplace_back can reallocate.
+static uint32_t insert(BufP buf, Shape shape, Shape strides, int64_t size) {  // tensor.rs:104-113
+    Engine &e = eng();
+    uint32_t id;
+    if (!e.free_ids.empty()) {
+        id = e.free_ids.back();
+        e.free_ids.pop_back();
+    } else {
+        id = (uint32_t)e.tensors.size();
+        e.tensors.emplace_back();
+    }
+    Tensor &t = e.tensors[id];
+    t = Tensor();
+    t.live = true;
+    t.buf = std::move(buf);
+    t.shape = std::move(shape);
+    t.strides = std::move(strides);
+    t.size = size;
+    return id;
+}
+static uint32_t insert_contig(BufP buf, Shape shape) {
+    Shape strides = compute_strides(shape);
+    const int64_t size = shape_size(shape);
+    return insert(std::move(buf), std::move(shape), std::move(strides), size);
+}
+static void free_tensor(uint32_t id) {  // tensor.rs:169-174 (cuda arm :351-356)
+    Engine &e = eng();
+    if (id >= e.tensors.size() || !e.tensors[id].live) return;
+    e.tensors[id] = Tensor();
+    e.free_ids.push_back(id);
+}
+
+// A contiguous device buffer with the tensor's logical contents: its own
+// buffer when already contiguous, else a gathered temporary
+// (make_contiguous_data, tensor.rs:292-309, on the device).
+static BufP contiguous_buf(const Tensor &t) {
+    if (is_contiguous(t)) return t.buf;
+    BufP out = new_buf((size_t)t.size);
+    if (!out) return nullptr;
+    if (k_strided_copy(out->p, t.buf->p, t.shape.data(), t.strides.data(), (int)t.shape.size()) != MNI_OK) return nullptr;
+    return out;
+}
+static BufP clone_buf(const BufP &src, size_t n) {
+    BufP out = new_buf(n);
+    if (!out) return nullptr;
+    if (n && mni_rocm_d2d(out->p, src->p, n * sizeof(float)) != MNI_OK) return nullptr;
+    return out;
+}
+// Copy-on-write before an in-place update.
+static int make_unique(Tensor &t) {
+    if (t.buf.use_count() <= 1) return MNI_OK;
+    BufP c = clone_buf(t.buf, t.buf->n);
+    if (!c) return MNI_ERR_NOMEM;
+    t.buf = std::move(c);
+    return MNI_OK;
+}
+static uint32_t zeros(const Shape &shape) {  // tensor.rs:412-420
+    const int64_t n = shape_size(shape);
+    BufP b = new_buf((size_t)n);
+    if (!b || k_fill(b->p, 0.0f, n) != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(b), shape);
+}
+static uint32_t filled(const Shape &shape, float v) {
+    const int64_t n = shape_size(shape);
+    BufP b = new_buf((size_t)n);
+    if (!b || k_fill(b->p, v, n) != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(b), shape);
+}
+static int64_t ensure_grad(uint32_t id) {  // tensor.rs:144-152
+    Tensor *t = get(id);
+    if (!t) return -1;
+    if (t->grad >= 0) return t->grad;
+    const Shape shape = t->shape;
+    const uint32_t g = zeros(shape);
+    if (g == MNI_BAD_ID) return -1;
+    get(id)->grad = g;
+    return g;
+}
+// tensor.rs:475-491 accumulate_grad / :493-508 add_inplace: raw buffer order,
+// src.size elements.
+static int add_into(uint32_t dst, uint32_t src) {
+    Tensor *s = get(src), *d = get(dst);
+    if (!s || !d) return MNI_ERR_FREED;
+    if ((int64_t)d->buf->n < s->size) return set_error(MNI_ERR_INVALID, "add_inplace: destination smaller than source");
+    MNI_TRY(make_unique(*d));
+    return k_axpy(d->buf->p, s->buf->p, 1.0f, s->size);
+}
+
+static bool to_shape(const int64_t *shape, int nd, Shape *out) {
+    if (nd < 0 || nd > MNI_MAX_DIMS || (nd > 0 && !shape)) {
+        set_error(MNI_ERR_INVALID, "rank %d out of range (max %d)", nd, MNI_MAX_DIMS);
+        return false;
+    }
+    out->assign(shape, shape + nd);
+    for (int64_t d : *out)
+        if (d < 0) { set_error(MNI_ERR_INVALID, "negative extent"); return false; }
+    return true;
+}
+
+// ---- matmul ------------------------------------------------------------------------
+// Describe the last two dims of `t` as a GEMM operand; leading dims collapse
+// to one batch stride when they can, otherwise the tensor is gathered once on
+// the device.  `keep` holds whatever buffer the descriptor points into.
+static int make_operand(const Tensor &t, bool transpose, mni_operand *op, BufP *keep) {
+    const int nd = (int)t.shape.size();
+    Shape strides = t.strides;
+    *keep = t.buf;
+    int64_t bcount = 1;
+    for (int i = 0; i < nd - 2; ++i) bcount *= t.shape[i];
+    if (bcount < 1) bcount = 1;
+    int64_t bstride = 0;
+    bool ok = true;
+    if (bcount > 1) {
+        // innermost non-unit batch dim gives the stride; outer ones must nest
+        int64_t expect = -1;
+        for (int i = nd - 3; i >= 0; --i) {
+            if (t.shape[i] == 1) continue;
+            if (expect < 0) { bstride = strides[i]; expect = bstride * t.shape[i]; }
+            else { if (strides[i] != expect) ok = false; expect *= t.shape[i]; }
+        }
+    }
+    if (!ok) {
+        BufP c = contiguous_buf(t);
+        if (!c) return MNI_ERR_NOMEM;
+        *keep = c;
+        strides = compute_strides(t.shape);
+        bstride = t.shape[nd - 2] * t.shape[nd - 1];
+    }
+    op->ptr = (*keep)->p;
+    op->row_stride = strides[nd - 2];
+    op->col_stride = strides[nd - 1];
+    if (transpose) std::swap(op->row_stride, op->col_stride);
+    op->batch_stride = bstride;
+    op->batch_count = bcount;
+    return MNI_OK;
+}
+
+// C = op(A) * op(B) on tensors, batch rule of ops/matmul.rs:54-60.
+// ta / tb: use the operand with its last two dims swapped (transpose_last2,
+// ops/matmul.rs:258-284, without the copy).
+static uint32_t matmul_tensors(uint32_t a, bool ta, uint32_t b, bool tb, const float *bias, int epilogue) {
+    Tensor *A = get(a), *B = get(b);
+    if (!A || !B) return MNI_BAD_ID;
+    const int and_ = (int)A->shape.size(), bnd = (int)B->shape.size();
+    if (and_ < 2 || bnd < 2) {
+        set_error(MNI_ERR_INVALID, "matmul requires at least 2D tensors");
+        return MNI_BAD_ID;
+    }
+    int64_t m = A->shape[and_ - 2], k = A->shape[and_ - 1];
+    if (ta) std::swap(m, k);
+    int64_t k2 = B->shape[bnd - 2], n = B->shape[bnd - 1];
+    if (tb) std::swap(k2, n);
+    if (k != k2) {
+        set_error(MNI_ERR_INVALID, "matmul inner dimensions must match: %lld vs %lld", (long long)k, (long long)k2);
+        return MNI_BAD_ID;
+    }
+    const Shape a_batch(A->shape.begin(), A->shape.end() - 2), b_batch(B->shape.begin(), B->shape.end() - 2);
+    Shape out_shape;
+    if (!broadcast_shape(a_batch, b_batch, &out_shape)) {
+        set_error(MNI_ERR_INVALID, "matmul batch shapes are not broadcastable");
+        return MNI_BAD_ID;
+    }
+    if (out_shape.size() + 2 > MNI_MAX_DIMS) {
+        set_error(MNI_ERR_INVALID, "matmul result rank exceeds %d", MNI_MAX_DIMS);
+        return MNI_BAD_ID;
+    }
+    const int64_t batch = shape_size(out_shape);
+    out_shape.push_back(m);
+    out_shape.push_back(n);
+
+    mni_gemm_desc d;
+    memset(&d, 0, sizeof d);
+    BufP keep_a, keep_b;
+    if (make_operand(*A, ta, &d.A, &keep_a) != MNI_OK || make_operand(*B, tb, &d.B, &keep_b) != MNI_OK) return MNI_BAD_ID;
+    BufP out = new_buf((size_t)shape_size(out_shape));
+    if (!out) return MNI_BAD_ID;
+    d.M = m; d.N = n; d.K = k; d.batch = batch;
+    d.C = out->p; d.ldc = n; d.c_batch_stride = m * n;
+    d.bias = bias; d.epilogue = epilogue;
+    if (sgemm(d) != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(out), out_shape);
+}
+
+// Sum `full` (contiguous, full_shape) down to `orig_shape`
+// (utils::unbroadcast, src/native/src/utils.rs:39-66).  Returns a tensor id;
+// when nothing is reduced the result shares full's buffer.
+static uint32_t unbroadcast_tensor(uint32_t full, const Shape &orig_shape) {
+    Tensor *F = get(full);
+    if (!F) return MNI_BAD_ID;
+    if (F->shape == orig_shape) return insert_contig(F->buf, orig_shape);
+    const Shape fshape = F->shape;
+    BufP src = contiguous_buf(*F);
+    if (!src) return MNI_BAD_ID;
+    const int64_t on = shape_size(orig_shape);
+    BufP out = new_buf((size_t)on);
+    if (!out) return MNI_BAD_ID;
+    // Leading-dims reduction ([R.., C..] -> [C..], or [1.., C..]) is a column sum.
+    size_t lead = 0;
+    while (lead < orig_shape.size() && orig_shape[lead] == 1) ++lead;
+    const size_t core = orig_shape.size() - lead;
+    bool suffix = fshape.size() >= orig_shape.size();
+    for (size_t i = 0; suffix && i < core; ++i) suffix = fshape[fshape.size() - core + i] == orig_shape[lead + i];
+    int rc;
+    if (suffix) {
+        rc = k_colsum(out->p, src->p, shape_size(fshape) / on, on);
+    } else {
+        rc = k_unbroadcast(out->p, src->p, fshape.data(), (int)fshape.size(), orig_shape.data(), (int)orig_shape.size());
+    }
+    if (rc != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(out), orig_shape);
+}
+
+// ops/matmul.rs:199-222 matmul_backward: dA = unbroadcast(dC * B^T),
+// dB = unbroadcast(A^T * dC); both always.
+static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    const uint32_t a = e.inputs[0], b = e.inputs[1];
+    Tensor *A = get(a), *B = get(b), *G = get(grad);
+    if (!A || !B || !G) return MNI_ERR_FREED;
+    const Shape a_shape = A->shape, b_shape = B->shape;
+
+    // dA
+    {
+        const uint32_t full = matmul_tensors(grad, false, b, true, nullptr, MNI_EPI_NONE);
+        if (full == MNI_BAD_ID) return MNI_ERR_INVALID;
+        const uint32_t ga = unbroadcast_tensor(full, a_shape);
+        free_tensor(full);
+        if (ga == MNI_BAD_ID) return MNI_ERR_INVALID;
+        out[0] = ga;
+    }
+    // dB.  When B has no batch of its own and A / dC stack their batch
+    // matrices at a uniform row pitch, sum over the batch inside one product
+    // by extending K to batch * M (the split-K path then fills the machine).
+    {
+        A = get(a); B = get(b); G = get(grad);
+        const int and_ = (int)A->shape.size(), gnd = (int)G->shape.size();
+        int64_t b_bcount = 1;
+        for (size_t i = 0; i + 2 < b_shape.size(); ++i) b_bcount *= b_shape[i];
+        int64_t g_batch = 1;
+        for (int i = 0; i < gnd - 2; ++i) g_batch *= G->shape[i];
+        bool folded = false;
+        if (b_bcount == 1 && g_batch > 1 && is_contiguous(*A) && is_contiguous(*G)) {
+            int64_t a_batch = 1;
+            for (int i = 0; i < and_ - 2; ++i) a_batch *= A->shape[i];
+            if (a_batch == g_batch) {
+                const int64_t m = A->shape[and_ - 2], k = A->shape[and_ - 1], n = G->shape[gnd - 1];
+                mni_gemm_desc d;
+                memset(&d, 0, sizeof d);
+                BufP outb = new_buf((size_t)(k * n));
+                if (!outb) return MNI_ERR_NOMEM;
+                d.M = k; d.N = n; d.K = g_batch * m; d.batch = 1;
+                d.A.ptr = A->buf->p; d.A.row_stride = 1; d.A.col_stride = k; d.A.batch_count = 1;
+                d.B.ptr = G->buf->p; d.B.row_stride = n; d.B.col_stride = 1; d.B.batch_count = 1;
+                d.C = outb->p; d.ldc = n; d.c_batch_stride = k * n;
+                MNI_TRY(sgemm(d));
+                Shape kn = {k, n};
+                const uint32_t full = insert_contig(std::move(outb), kn);
+                // b_shape may carry leading ones ([1, K, N]); same element count.
+                Tensor *F = get(full);
+                F->shape = b_shape;
+                F->strides = compute_strides(b_shape);
+                out[1] = full;
+                folded = true;
+            }
+        }
+        if (!folded) {
+            const uint32_t full = matmul_tensors(a, true, grad, false, nullptr, MNI_EPI_NONE);
+            if (full == MNI_BAD_ID) return MNI_ERR_INVALID;
+            const uint32_t gb = unbroadcast_tensor(full, b_shape);
+            free_tensor(full);
+            if (gb == MNI_BAD_ID) return MNI_ERR_INVALID;
+            out[1] = gb;
+        }
+    }
+    return MNI_OK;
+}
+
+// ---- elementwise ---------------------------------------------------------------------
+// ops/elementwise.rs:20-73,237-248,474-485
+static uint32_t binary_op(uint32_t a, uint32_t b, int op) {
+    Tensor *A = get(a), *B = get(b);
+    if (!A || !B) return MNI_BAD_ID;
+    Shape out_shape;
+    if (!broadcast_shape(A->shape, B->shape, &out_shape)) {
+        set_error(MNI_ERR_INVALID, "shapes are not broadcastable");
+        return MNI_BAD_ID;
+    }
+    const int64_t n = shape_size(out_shape);
+    BufP out = new_buf((size_t)n);
+    if (!out) return MNI_BAD_ID;
+    int rc;
+    const bool a_c = is_contiguous(*A), b_c = is_contiguous(*B);
+    if (A->shape == B->shape && a_c && b_c) {
+        rc = k_binary_same(out->p, A->buf->p, B->buf->p, n, op);
+    } else if (op == BIN_ADD && a_c && b_c && A->shape == out_shape && B->shape.size() == 1 &&
+               B->shape[0] == out_shape.back()) {
+        rc = k_add_bias(out->p, A->buf->p, B->buf->p, n / out_shape.back(), out_shape.back());
+    } else {
+        StridedDesc d;
+        d.ndim = (int)out_shape.size();
+        const int ao = d.ndim - (int)A->shape.size(), bo = d.ndim - (int)B->shape.size();
+        for (int i = 0; i < d.ndim; ++i) {
+            d.shape[i] = out_shape[i];
+            d.a_strides[i] = (i < ao || A->shape[i - ao] == 1) ? 0 : A->strides[i - ao];
+            d.b_strides[i] = (i < bo || B->shape[i - bo] == 1) ? 0 : B->strides[i - bo];
+        }
+        rc = k_binary_broadcast(out->p, A->buf->p, B->buf->p, d, op);
+    }
+    if (rc != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(out), out_shape);
+    Entry e;
+    e.op = op == BIN_ADD ? OP_ADD : op == BIN_SUB ? OP_SUB : OP_MUL;
+    e.output_id = id; e.n_inputs = 2; e.inputs[0] = a; e.inputs[1] = b;
+    e.saved_shape = out_shape;
+    eng().tape.record(std::move(e));
+    return id;
+}
+
+static uint32_t negated(uint32_t g) {
+    Tensor *G = get(g);
+    BufP src = contiguous_buf(*G);
+    BufP out = src ? new_buf((size_t)G->size) : nullptr;
+    if (!out || k_unary(out->p, src->p, G->size, UN_NEG, 0.f) != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(out), G->shape);
+}
+
+// ops/elementwise.rs:199-211 add_backward, :558-571 sub_backward
+static int addsub_backward(uint32_t grad, const Entry &e, int64_t *out, bool is_sub) {
+    Tensor *A = get(e.inputs[0]), *B = get(e.inputs[1]);
+    if (!A || !B || !get(grad)) return MNI_ERR_FREED;
+    const Shape a_shape = A->shape, b_shape = B->shape;
+    const uint32_t ga = unbroadcast_tensor(grad, a_shape);
+    if (ga == MNI_BAD_ID) return MNI_ERR_INVALID;
+    out[0] = ga;
+    uint32_t gb;
+    if (is_sub) {
+        const uint32_t ng = negated(grad);
+        if (ng == MNI_BAD_ID) return MNI_ERR_INVALID;
+        gb = unbroadcast_tensor(ng, b_shape);
+        free_tensor(ng);
+    } else {
+        gb = unbroadcast_tensor(grad, b_shape);
+    }
+    if (gb == MNI_BAD_ID) return MNI_ERR_INVALID;
+    out[1] = gb;
+    return MNI_OK;
+}
+
+// ops/elementwise.rs:348-390 mul_backward
+static int mul_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    const uint32_t a = e.inputs[0], b = e.inputs[1];
+    Tensor *A = get(a), *B = get(b), *G = get(grad);
+    if (!A || !B || !G) return MNI_ERR_FREED;
+    const Shape a_shape = A->shape, b_shape = B->shape, g_shape = G->shape;
+    const int64_t n = shape_size(g_shape);
+    BufP gsrc = contiguous_buf(*G);
+    BufP ga_full = new_buf((size_t)n), gb_full = new_buf((size_t)n);
+    if (!gsrc || !ga_full || !gb_full) return MNI_ERR_NOMEM;
+    if (a_shape == g_shape && b_shape == g_shape && is_contiguous(*A) && is_contiguous(*B)) {
+        MNI_TRY(k_mul_backward_same(ga_full->p, gb_full->p, gsrc->p, A->buf->p, B->buf->p, n));
+    } else {
+        // ga_full = g * b (b broadcast), gb_full = g * a (a broadcast)
+        StridedDesc d;
+        d.ndim = (int)g_shape.size();
+        const Shape gstr = compute_strides(g_shape);
+        const int ao = d.ndim - (int)a_shape.size(), bo = d.ndim - (int)b_shape.size();
+        for (int i = 0; i < d.ndim; ++i) {
+            d.shape[i] = g_shape[i];
+            d.a_strides[i] = gstr[i];
+            d.b_strides[i] = (i < bo || b_shape[i - bo] == 1) ? 0 : B->strides[i - bo];
+        }
+        MNI_TRY(k_binary_broadcast(ga_full->p, gsrc->p, B->buf->p, d, BIN_MUL));
+        for (int i = 0; i < d.ndim; ++i)
+            d.b_strides[i] = (i < ao || a_shape[i - ao] == 1) ? 0 : A->strides[i - ao];
+        MNI_TRY(k_binary_broadcast(gb_full->p, gsrc->p, A->buf->p, d, BIN_MUL));
+    }
+    const uint32_t fa = insert_contig(std::move(ga_full), g_shape);
+    const uint32_t fb = insert_contig(std::move(gb_full), g_shape);
+    const uint32_t ga = unbroadcast_tensor(fa, a_shape);
+    const uint32_t gb = unbroadcast_tensor(fb, b_shape);
+    free_tensor(fa);
+    free_tensor(fb);
+    if (ga == MNI_BAD_ID || gb == MNI_BAD_ID) return MNI_ERR_INVALID;
+    out[0] = ga; out[1] = gb;
+    return MNI_OK;
+}
+
+// ops/activation.rs:34-44,114-124; elementwise neg / mul_scalar
+static uint32_t unary_op(uint32_t a, int un, int tape_op, float s) {
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    BufP src = contiguous_buf(*A);
+    BufP out = src ? new_buf((size_t)A->size) : nullptr;
+    if (!out || k_unary(out->p, src->p, A->size, un, s) != MNI_OK) return MNI_BAD_ID;
+    const Shape shape = A->shape;
+    const uint32_t id = insert_contig(std::move(out), shape);
+    Entry e;
+    e.op = tape_op; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a; e.scalar = s;
+    eng().tape.record(std::move(e));
+    return id;
+}
+
+// ops/activation.rs:74-84,154-164 and the neg / mul_scalar backward
+static int unary_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *G = get(grad);
+    if (!G) return MNI_ERR_FREED;
+    const Shape shape = G->shape;
+    const int64_t n = G->size;
+    BufP g = contiguous_buf(*G);
+    BufP o = g ? new_buf((size_t)n) : nullptr;
+    if (!o) return MNI_ERR_NOMEM;
+    if (e.op == OP_RELU || e.op == OP_GELU) {
+        Tensor *X = get(e.inputs[0]);
+        if (!X) return MNI_ERR_FREED;
+        BufP x = contiguous_buf(*X);
+        if (!x) return MNI_ERR_NOMEM;
+        MNI_TRY(k_unary_backward(o->p, g->p, x->p, n, e.op == OP_RELU ? UN_RELU : UN_GELU));
+    } else if (e.op == OP_NEG) {
+        MNI_TRY(k_unary(o->p, g->p, n, UN_NEG, 0.f));
+    } else {
+        MNI_TRY(k_unary(o->p, g->p, n, UN_SCALE, e.scalar));
+    }
+    out[0] = insert_contig(std::move(o), shape);
+    return MNI_OK;
+}
+
+// ---- reductions ----------------------------------------------------------------------
+static int resolve_dim(int64_t dim, int nd) { return (int)(dim < 0 ? nd + dim : dim); }  // reduce.rs:5-7
+
+// ops/reduce.rs:13-46 sum, :169-184 mean.  The reference's mean also leaves an
+// unreachable Sum entry and tensor behind; only the Mean entry is recorded.
+static uint32_t reduce_op(uint32_t a, int64_t dim, bool mean) {
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    const int nd = (int)A->shape.size();
+    const int d = resolve_dim(dim, nd);
+    if (d < 0 || d >= nd) {
+        set_error(MNI_ERR_INVALID, "reduce dim %lld out of range for rank %d", (long long)dim, nd);
+        return MNI_BAD_ID;
+    }
+    const Shape a_shape = A->shape;
+    Shape out_shape = a_shape;
+    out_shape[d] = 1;
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < d; ++i) outer *= a_shape[i];
+    for (int i = d + 1; i < nd; ++i) inner *= a_shape[i];
+    BufP src = contiguous_buf(*A);
+    BufP out = src ? new_buf((size_t)shape_size(out_shape)) : nullptr;
+    if (!out) return MNI_BAD_ID;
+    if (k_reduce_dim(out->p, src->p, outer, a_shape[d], inner, mean ? (float)a_shape[d] : 1.0f) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(out), out_shape);
+    Entry e;
+    e.op = mean ? OP_MEAN : OP_SUM; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a;
+    e.saved_shape = a_shape;
+    eng().tape.record(std::move(e));
+    return id;
+}
+
+// ops/reduce.rs:94-118 sum_backward, :232-263 mean_backward
+static int reduce_backward(uint32_t grad, const Entry &e, int64_t *out, bool mean) {
+    Tensor *G = get(grad);
+    if (!G) return MNI_ERR_FREED;
+    const Shape &orig = e.saved_shape;
+    const Shape gshape = G->shape;
+    if (gshape.size() != orig.size()) return set_error(MNI_ERR_INVALID, "reduce backward: rank mismatch");
+    float div = 1.0f;
+    if (mean)
+        for (size_t d = 0; d < orig.size(); ++d)
+            if (gshape[d] == 1 && orig[d] > 1) div = (float)orig[d];
+    BufP g = contiguous_buf(*G);
+    const int64_t on = shape_size(orig);
+    BufP o = g ? new_buf((size_t)on) : nullptr;
+    if (!o) return MNI_ERR_NOMEM;
+    // One expanded dim is the common case; otherwise broadcast generically.
+    int nexp = 0, ed = -1;
+    for (size_t d = 0; d < orig.size(); ++d)
+        if (gshape[d] == 1 && orig[d] != 1) { ++nexp; ed = (int)d; }
+    if (nexp <= 1) {
+        int64_t outer = 1, inner = 1, dimn = 1;
+        if (nexp == 1) {
+            for (int i = 0; i < ed; ++i) outer *= orig[i];
+            for (size_t i = ed + 1; i < orig.size(); ++i) inner *= orig[i];
+            dimn = orig[ed];
+        } else {
+            inner = on;
+        }
+        MNI_TRY(k_expand_dim(o->p, g->p, outer, dimn, inner, div));
+    } else {
+        // g broadcast to orig (as a broadcast multiply by one), then divided.
+        BufP one = new_buf(1);
+        if (!one) return MNI_ERR_NOMEM;
+        MNI_TRY(k_fill(one->p, 1.0f, 1));
+        StridedDesc d;
+        d.ndim = (int)orig.size();
+        const Shape gstr = compute_strides(gshape);
+        for (int i = 0; i < d.ndim; ++i) {
+            d.shape[i] = orig[i];
+            d.a_strides[i] = gshape[i] == 1 ? 0 : gstr[i];
+            d.b_strides[i] = 0;
+        }
+        MNI_TRY(k_binary_broadcast(o->p, g->p, one->p, d, BIN_MUL));
+        if (div != 1.0f) MNI_TRY(k_expand_dim(o->p, o->p, 1, 1, on, div));
+    }
+    out[0] = insert_contig(std::move(o), orig);
+    return MNI_OK;
+}
+
+// ---- layout ------------------------------------------------------------------------------
+// ops/layout.rs:66-89 view: always a copy with the new shape.
+static uint32_t view_op(uint32_t a, const Shape &new_shape) {
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    const Shape orig = A->shape;
+    const int64_t n = A->size;
+    if (shape_size(new_shape) != n) {
+        set_error(MNI_ERR_INVALID, "view: %lld elements cannot be viewed as %lld", (long long)n, (long long)shape_size(new_shape));
+        return MNI_BAD_ID;
+    }
+    BufP out = new_buf((size_t)n);
+    if (!out) return MNI_BAD_ID;
+    int rc = is_contiguous(*A) ? mni_rocm_d2d(out->p, A->buf->p, (size_t)n * sizeof(float))
+                               : k_strided_copy(out->p, A->buf->p, A->shape.data(), A->strides.data(), (int)A->shape.size());
+    if (rc != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(out), new_shape);
+    Entry e;
+    e.op = OP_VIEW; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a; e.saved_shape = orig;
+    eng().tape.record(std::move(e));
+    return id;
+}
+// ops/layout.rs:92-105 view_backward
+static int view_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *G = get(grad);
+    if (!G) return MNI_ERR_FREED;
+    BufP g = contiguous_buf(*G);
+    if (!g) return MNI_ERR_NOMEM;
+    out[0] = insert_contig(g, e.saved_shape);  // shares the buffer; writers copy first
+    return MNI_OK;
+}
+// ops/layout.rs:112-134 permute: a view (shared buffer, permuted strides)
+static uint32_t permute_op(uint32_t a, const Shape &dims) {
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    const int nd = (int)A->shape.size();
+    if ((int)dims.size() != nd) {
+        set_error(MNI_ERR_INVALID, "permute: %zu dims given for a rank-%d tensor", dims.size(), nd);
+        return MNI_BAD_ID;
+    }
+    Shape ns(nd), nst(nd);
+    std::vector<bool> seen(nd, false);
+    for (int i = 0; i < nd; ++i) {
+        if (dims[i] < 0 || dims[i] >= nd || seen[dims[i]]) {
+            set_error(MNI_ERR_INVALID, "permute: dims are not a permutation");
+            return MNI_BAD_ID;
+        }
+        seen[dims[i]] = true;
+        ns[i] = A->shape[dims[i]];
+        nst[i] = A->strides[dims[i]];
+    }
+    const Shape a_shape = A->shape;
+    const uint32_t id = insert(A->buf, ns, nst, A->size);
+    Entry e;
+    e.op = OP_PERMUTE; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a;
+    e.saved_shape = a_shape; e.saved_perm = dims;
+    eng().tape.record(std::move(e));
+    return id;
+}
+// ops/layout.rs:162-195 permute_backward: grad (contiguous, permuted shape)
+// scattered back = a gather of grad through the inverse permutation.
+static int permute_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *G = get(grad);
+    if (!G) return MNI_ERR_FREED;
+    const int nd = (int)e.saved_perm.size();
+    BufP g = contiguous_buf(*G);
+    if (!g) return MNI_ERR_NOMEM;
+    const Shape gstr = compute_strides(G->shape);
+    // out[coord_orig] = g[coord_perm], coord_perm[i] = coord_orig[perm[i]]
+    Shape src_strides(nd);
+    for (int i = 0; i < nd; ++i) src_strides[e.saved_perm[i]] = gstr[i];
+    BufP o = new_buf((size_t)shape_size(e.saved_shape));
+    if (!o) return MNI_ERR_NOMEM;
+    MNI_TRY(k_strided_copy(o->p, g->p, e.saved_shape.data(), src_strides.data(), nd));
+    out[0] = insert_contig(std::move(o), e.saved_shape);
+    return MNI_OK;
+}
+
+// ---- loss ------------------------------------------------------------------------------------
+// ops/loss.rs:24-67 cross_entropy
+static uint32_t cross_entropy_op(uint32_t logits, const int64_t *targets, size_t nt) {
+    Tensor *L = get(logits);
+    if (!L) return MNI_BAD_ID;
+    const Shape shape = L->shape;
+    if (shape.empty()) { set_error(MNI_ERR_INVALID, "cross_entropy: scalar logits"); return MNI_BAD_ID; }
+    const int64_t v = shape.back();
+    const int64_t n = v ? shape_size(shape) / v : 0;
+    if (n <= 0 || v <= 0) { set_error(MNI_ERR_INVALID, "cross_entropy: empty logits"); return MNI_BAD_ID; }
+    if ((int64_t)nt < n) { set_error(MNI_ERR_INVALID, "cross_entropy: %zu targets for %lld rows", nt, (long long)n); return MNI_BAD_ID; }
+    std::vector<int32_t> t32((size_t)n);
+    for (int64_t i = 0; i < n; ++i) {
+        if (targets[i] < 0 || targets[i] >= v) {
+            set_error(MNI_ERR_INVALID, "cross_entropy: target %lld out of range [0, %lld)", (long long)targets[i], (long long)v);
+            return MNI_BAD_ID;
+        }
+        t32[(size_t)i] = (int32_t)targets[i];
+    }
+    void *tp = nullptr;
+    if (dev_alloc(&tp, (size_t)n * sizeof(int32_t)) != MNI_OK) return MNI_BAD_ID;
+    std::shared_ptr<void> tdev(tp, [](void *p) { dev_free(p); });
+    if (mni_rocm_h2d(tp, t32.data(), (size_t)n * sizeof(int32_t)) != MNI_OK) return MNI_BAD_ID;
+    BufP x = contiguous_buf(*L);
+    BufP sm = x ? new_buf((size_t)(n * v)) : nullptr;
+    BufP loss = sm ? new_buf(1) : nullptr;
+    if (!loss) return MNI_BAD_ID;
+    if (k_cross_entropy(loss->p, sm->p, x->p, (const int32_t *)tp, n, v) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t loss_id = insert_contig(std::move(loss), Shape{1});
+    const uint32_t sm_id = insert_contig(std::move(sm), shape);
+    Entry e;
+    e.op = OP_CROSSENTROPY; e.output_id = loss_id; e.n_inputs = 1; e.inputs[0] = logits;
+    e.aux = sm_id; e.targets = tdev; e.ce_n = n; e.ce_v = v;
+    eng().tape.record(std::move(e));
+    return loss_id;
+}
+// ops/loss.rs:131-149
+static int cross_entropy_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *G = get(grad), *S = get(e.aux);
+    if (!G || !S) return MNI_ERR_FREED;
+    const Shape shape = S->shape;
+    BufP o = new_buf((size_t)(e.ce_n * e.ce_v));
+    if (!o) return MNI_ERR_NOMEM;
+    MNI_TRY(k_cross_entropy_backward(o->p, S->buf->p, (const int32_t *)e.targets.get(), G->buf->p, e.ce_n, e.ce_v));
+    out[0] = insert_contig(std::move(o), shape);
+    return MNI_OK;
+}
+
+// ---- fused Linear ------------------------------------------------------------------------------
+static uint32_t linear_op(uint32_t x, uint32_t w, uint32_t bias, int act) {
+    Tensor *X = get(x), *W = get(w), *Bv = get(bias);
+    if (!X || !W || !Bv) return MNI_BAD_ID;
+    if (act < MNI_EPI_BIAS || act > MNI_EPI_BIAS_GELU) { set_error(MNI_ERR_INVALID, "linear: unknown activation %d", act); return MNI_BAD_ID; }
+    if (W->shape.size() != 2) { set_error(MNI_ERR_INVALID, "linear: weight must be [in, out]"); return MNI_BAD_ID; }
+    if (Bv->shape.size() != 1 || Bv->shape[0] != W->shape[1] || !is_contiguous(*Bv)) {
+        set_error(MNI_ERR_INVALID, "linear: bias must be a contiguous [out] vector");
+        return MNI_BAD_ID;
+    }
+    // GELU needs its pre-activation in backward: keep z and apply the
+    // activation as a second pass; bias and ReLU ride in the GEMM epilogue.
+    const BufP bias_buf = Bv->buf;
+    uint32_t out, aux = MNI_BAD_ID;
+    if (act == MNI_EPI_BIAS_GELU) {
+        aux = matmul_tensors(x, false, w, false, bias_buf->p, MNI_EPI_BIAS);
+        if (aux == MNI_BAD_ID) return MNI_BAD_ID;
+        Tensor *Z = get(aux);
+        BufP o = new_buf((size_t)Z->size);
+        if (!o || k_unary(o->p, Z->buf->p, Z->size, UN_GELU, 0.f) != MNI_OK) return MNI_BAD_ID;
+        out = insert_contig(std::move(o), Z->shape);
+    } else {
+        out = matmul_tensors(x, false, w, false, bias_buf->p, act);
+        if (out == MNI_BAD_ID) return MNI_BAD_ID;
+    }
+    Entry e;
+    e.op = OP_LINEAR; e.output_id = out; e.n_inputs = 3;
+    e.inputs[0] = x; e.inputs[1] = w; e.inputs[2] = bias;
+    e.act = act; e.aux = aux;
+    eng().tape.record(std::move(e));
+    return out;
+}
+static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    uint32_t g = grad;
+    bool own_g = false;
+    if (e.act != MNI_EPI_BIAS) {
+        // dZ = dOut * act'(z); for ReLU the output has the sign of z.
+        Tensor *G = get(grad), *Z = get(e.act == MNI_EPI_BIAS_GELU ? e.aux : e.output_id);
+        if (!G || !Z) return MNI_ERR_FREED;
+        BufP gb = contiguous_buf(*G);
+        BufP o = gb ? new_buf((size_t)G->size) : nullptr;
+        if (!o) return MNI_ERR_NOMEM;
+        MNI_TRY(k_unary_backward(o->p, gb->p, Z->buf->p, G->size, e.act == MNI_EPI_BIAS_GELU ? UN_GELU : UN_RELU));
+        g = insert_contig(std::move(o), G->shape);
+        own_g = true;
+    }
+    Entry mm;
+    mm.op = OP_MATMUL; mm.n_inputs = 2; mm.inputs[0] = e.inputs[0]; mm.inputs[1] = e.inputs[1];
+    int rc = matmul_backward(g, mm, out);
+    if (rc == MNI_OK) {
+        Tensor *Bv = get(e.inputs[2]);
+        if (!Bv) rc = MNI_ERR_FREED;
+        else {
+            const Shape bshape = Bv->shape;
+            const uint32_t gb = unbroadcast_tensor(g, bshape);
+            if (gb == MNI_BAD_ID) rc = MNI_ERR_INVALID;
+            else out[2] = gb;
+        }
+    }
+    if (own_g) free_tensor(g);
+    return rc;
+}
+
+// ---- backward --------------------------------------------------------------------------------
+static int dispatch_backward(const Entry &e, uint32_t grad, int64_t *out) {  // autograd.rs:180-222
+    out[0] = out[1] = out[2] = -1;
+    switch (e.op) {
+    case OP_ADD: return addsub_backward(grad, e, out, false);
+    case OP_SUB: return addsub_backward(grad, e, out, true);
+    case OP_MUL: return mul_backward(grad, e, out);
+    case OP_NEG: case OP_MULSCALAR: case OP_RELU: case OP_GELU: return unary_backward(grad, e, out);
+    case OP_MATMUL: return matmul_backward(grad, e, out);
+    case OP_SUM: return reduce_backward(grad, e, out, false);
+    case OP_MEAN: return reduce_backward(grad, e, out, true);
+    case OP_VIEW: return view_backward(grad, e, out);
+    case OP_PERMUTE: return permute_backward(grad, e, out);
+    case OP_CONTIGUOUS: out[0] = grad; return MNI_OK;  // layout.rs:229-231
+    case OP_CROSSENTROPY: return cross_entropy_backward(grad, e, out);
+    case OP_LINEAR: return linear_backward(grad, e, out);
+    }
+    return set_error(MNI_ERR_INVALID, "unknown tape op %d", e.op);
+}
+
+// autograd.rs:96-171 Tape::backward
+static int tape_backward(Tape &tp, uint32_t loss) {
+    if (!get(loss)) return MNI_ERR_FREED;
+    const size_t nslots = eng().tensors.size() + 1;
+    std::vector<int64_t> out2entry(nslots, -1);
+    for (size_t i = 0; i < tp.entries.size(); ++i)
+        if (tp.entries[i].output_id < nslots) out2entry[tp.entries[i].output_id] = (int64_t)i;  // later entry wins
+
+    std::vector<char> relevant(nslots, 0), visited(nslots, 0);
+    {
+        std::vector<uint32_t> stack{loss};
+        while (!stack.empty()) {
+            const uint32_t tid = stack.back();
+            stack.pop_back();
+            if (tid >= nslots || relevant[tid]) continue;
+            relevant[tid] = 1;
+            const int64_t idx = out2entry[tid];
+            if (idx >= 0)
+                for (int i = 0; i < tp.entries[idx].n_inputs; ++i) stack.push_back(tp.entries[idx].inputs[i]);
+        }
+    }
+    // Post-order DFS, inputs in order (autograd.rs:120-137), without recursion.
+    std::vector<uint32_t> order;
+    {
+        struct Frame { uint32_t tid; int next; };
+        std::vector<Frame> st;
+        visited[loss] = 1;
+        st.push_back({loss, 0});
+        while (!st.empty()) {
+            Frame &f = st.back();
+            const int64_t idx = out2entry[f.tid];
+            bool pushed = false;
+            if (idx >= 0) {
+                const Entry &en = tp.entries[idx];
+                while (f.next < en.n_inputs) {
+                    const uint32_t inp = en.inputs[f.next++];
+                    if (inp < nslots && relevant[inp] && !visited[inp]) {
+                        visited[inp] = 1;
+                        st.push_back({inp, 0});
+                        pushed = true;
+                        break;
+                    }
+                }
+            }
+            if (!pushed) {
+                order.push_back(st.back().tid);
+                st.pop_back();
+            }
+        }
+    }
+    std::vector<int64_t> grads(nslots, -1);
+    {
+        const Shape shape = get(loss)->shape;
+        const uint32_t g = filled(shape, 1.0f);  // ones_like for any loss shape, autograd.rs:143
+        if (g == MNI_BAD_ID) return MNI_ERR_NOMEM;
+        grads[loss] = g;
+    }
+    for (size_t oi = order.size(); oi-- > 0;) {
+        const uint32_t tid = order[oi];
+        if (grads[tid] < 0) continue;
+        const int64_t idx = out2entry[tid];
+        if (idx < 0) continue;
+        const Entry &en = tp.entries[idx];
+        int64_t ig[3];
+        MNI_TRY(dispatch_backward(en, (uint32_t)grads[tid], ig));
+        for (int i = 0; i < en.n_inputs; ++i) {
+            if (ig[i] < 0) continue;
+            const uint32_t inp = en.inputs[i];
+            Tensor *T = get(inp);
+            if (!T) return MNI_ERR_FREED;
+            if (T->requires_grad) {
+                const int64_t gid = ensure_grad(inp);
+                if (gid < 0) return MNI_ERR_NOMEM;
+                MNI_TRY(add_into((uint32_t)gid, (uint32_t)ig[i]));
+            }
+            if (grads[inp] >= 0) MNI_TRY(add_into((uint32_t)grads[inp], (uint32_t)ig[i]));
+            else grads[inp] = ig[i];
+        }
+    }
+    return MNI_OK;
+}
+
+// ---- optimiser ------------------------------------------------------------------------------------
+static float powi_f32(float a, int b) {  // f32::powi (compiler-rt __powisf2)
+    const bool recip = b < 0;
+    float r = 1.0f;
+    while (true) {
+        if (b & 1) r *= a;
+        b /= 2;
+        if (b == 0) break;
+        a *= a;
+    }
+    return recip ? 1.0f / r : r;
+}
+
+// ops/optimizer.rs:126-138 grad_norm
+static int grad_norm(const uint32_t *ids, size_t n, float *out) {
+    void *acc = nullptr;
+    MNI_TRY(dev_alloc(&acc, sizeof(double)));
+    std::shared_ptr<void> guard(acc, [](void *p) { dev_free(p); });
+    MNI_HIP_CHECK(hipMemsetAsync(acc, 0, sizeof(double), ctx().stream));
+    for (size_t p = 0; p < n; ++p) {
+        Tensor *T = get(ids[p]);
+        if (!T) return MNI_ERR_FREED;
+        if (T->grad < 0) continue;
+        Tensor *G = get((uint32_t)T->grad);
+        if (!G) return MNI_ERR_FREED;
+        MNI_TRY(k_sumsq_f64((double *)acc, G->buf->p, G->size));
+    }
+    double sq = 0.0;
+    MNI_TRY(mni_rocm_d2h(&sq, acc, sizeof(double)));
+    *out = sqrtf((float)sq);
+    return MNI_OK;
+}
+
+// ops/optimizer.rs:21-65 adamw_step
+static int adamw_step(const uint32_t *ids, size_t n, float lr, float b1, float b2, float eps, float wd, uint32_t step) {
+    const float bc1 = 1.0f - powi_f32(b1, (int)step);
+    const float bc2 = 1.0f - powi_f32(b2, (int)step);
+    for (size_t p = 0; p < n; ++p) {
+        Tensor *T = get(ids[p]);
+        if (!T) return MNI_ERR_FREED;
+        if (T->grad < 0) continue;
+        Tensor *G = get((uint32_t)T->grad);
+        if (!G) return MNI_ERR_FREED;
+        BufP g = contiguous_buf(*G);
+        if (!g) return MNI_ERR_NOMEM;
+        const int64_t size = T->size;
+        if (!T->adam_m) {
+            T->adam_m = new_buf((size_t)size);
+            T->adam_v = new_buf((size_t)size);
+            if (!T->adam_m || !T->adam_v) return MNI_ERR_NOMEM;
+            MNI_TRY(k_fill(T->adam_m->p, 0.f, size));
+            MNI_TRY(k_fill(T->adam_v->p, 0.f, size));
+        }
+        MNI_TRY(make_unique(*T));
+        MNI_TRY(k_adamw(T->buf->p, T->adam_m->p, T->adam_v->p, g->p, size, lr, b1, b2, eps, wd, bc1, bc2));
+    }
+    return MNI_OK;
+}
+
+static int scale_grads(const uint32_t *ids, size_t n, float scale) {
+    for (size_t p = 0; p < n; ++p) {
+        Tensor *T = get(ids[p]);
+        if (!T) return MNI_ERR_FREED;
+        if (T->grad < 0) continue;
+        Tensor *G = get((uint32_t)T->grad);
+        if (!G) return MNI_ERR_FREED;
+        MNI_TRY(make_unique(*G));
+        MNI_TRY(k_scale_inplace(G->buf->p, scale, (int64_t)G->buf->n));
+    }
+    return MNI_OK;
+}
+
+}  // namespace
+}  // namespace mni
+
+using namespace mni;
+
+// ============================================================================
+// Exported engine surface (one function per #[napi] export of lib.rs)
+// ============================================================================
+extern "C" {
+
+uint32_t mni_zeros(const int64_t *shape, int ndim) {
+    Shape s;
+    if (ensure_init() != MNI_OK || !to_shape(shape, ndim, &s)) return MNI_BAD_ID;
+    return zeros(s);
+}
+uint32_t mni_ones(const int64_t *shape, int ndim) {
+    Shape s;
+    if (ensure_init() != MNI_OK || !to_shape(shape, ndim, &s)) return MNI_BAD_ID;
+    return filled(s, 1.0f);
+}
+uint32_t mni_from_float32(const float *data, size_t len, const int64_t *shape, int ndim) {
+    Shape s;
+    if (ensure_init() != MNI_OK || !to_shape(shape, ndim, &s)) return MNI_BAD_ID;
+    const int64_t n = shape_size(s);
+    if ((int64_t)len < n || (n > 0 && !data)) {
+        set_error(MNI_ERR_INVALID, "from_float32: %zu values for shape of %lld elements", len, (long long)n);
+        return MNI_BAD_ID;
+    }
+    BufP b = new_buf((size_t)n);
+    if (!b || mni_rocm_h2d(b->p, data, (size_t)n * sizeof(float)) != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(b), s);
+}
+int mni_tensor_shape(uint32_t id, int64_t *out, int cap) {
+    Tensor *t = get(id);
+    if (!t) return -1;
+    for (int i = 0; i < (int)t->shape.size() && i < cap; ++i) out[i] = t->shape[i];
+    return (int)t->shape.size();
+}
+int64_t mni_tensor_size(uint32_t id) {
+    Tensor *t = get(id);
+    return t ? t->size : -1;
+}
+int mni_to_float32(uint32_t id, float *out, size_t cap) {
+    Tensor *t = get(id);
+    if (!t) return MNI_ERR_FREED;
+    if ((int64_t)cap < t->size) return set_error(MNI_ERR_INVALID, "to_float32: buffer of %zu for %lld elements", cap, (long long)t->size);
+    BufP b = contiguous_buf(*t);
+    if (!b) return MNI_ERR_NOMEM;
+    return mni_rocm_d2h(out, b->p, (size_t)t->size * sizeof(float));
+}
+int mni_get_scalar(uint32_t id, double *out) {
+    Tensor *t = get(id);
+    if (!t) return MNI_ERR_FREED;
+    float v = 0.f;
+    MNI_TRY(mni_rocm_d2h(&v, t->buf->p, sizeof(float)));
+    *out = (double)v;
+    return MNI_OK;
+}
+void mni_free_tensor(uint32_t id) { free_tensor(id); }
+int mni_set_requires_grad(uint32_t id, int requires_) {
+    Tensor *t = get(id);
+    if (!t) return MNI_ERR_FREED;
+    t->requires_grad = requires_ != 0;
+    return MNI_OK;
+}
+int mni_get_grad(uint32_t id, uint32_t *out) {
+    Tensor *t = get(id);
+    if (!t) return -1;
+    if (t->grad < 0) return 0;
+    if (out) *out = (uint32_t)t->grad;
+    return 1;
+}
+int mni_backward(uint32_t loss) {
+    // The tape is consumed and replaced by a fresh, enabled one (lib.rs:135).
+    Tape old = std::move(eng().tape);
+    eng().tape = Tape();
+    return tape_backward(old, loss);
+}
+int mni_zero_grad(const uint32_t *ids, size_t n) {
+    for (size_t p = 0; p < n; ++p) {
+        Tensor *t = get(ids[p]);
+        if (!t) return MNI_ERR_FREED;
+        if (t->grad < 0) continue;
+        Tensor *g = get((uint32_t)t->grad);
+        if (!g) return MNI_ERR_FREED;
+        if (g->buf.use_count() > 1) {  // shared: replace instead of copy + clear
+            g->buf = new_buf(g->buf->n);
+            if (!g->buf) return MNI_ERR_NOMEM;
+        }
+        MNI_TRY(k_fill(g->buf->p, 0.0f, (int64_t)g->buf->n));
+    }
+    return MNI_OK;
+}
+void mni_no_grad_start(void) { eng().tape.enabled = false; }
+void mni_no_grad_end(void) { eng().tape.enabled = true; }
+
+uint32_t mni_add(uint32_t a, uint32_t b) { return binary_op(a, b, BIN_ADD); }
+uint32_t mni_mul(uint32_t a, uint32_t b) { return binary_op(a, b, BIN_MUL); }
+uint32_t mni_sub(uint32_t a, uint32_t b) { return binary_op(a, b, BIN_SUB); }
+uint32_t mni_neg(uint32_t a) { return unary_op(a, UN_NEG, OP_NEG, 0.f); }
+uint32_t mni_mul_scalar(uint32_t a, double s) { return unary_op(a, UN_SCALE, OP_MULSCALAR, (float)s); }
+uint32_t mni_gelu(uint32_t a) { return unary_op(a, UN_GELU, OP_GELU, 0.f); }
+uint32_t mni_relu(uint32_t a) { return unary_op(a, UN_RELU, OP_RELU, 0.f); }
+
+uint32_t mni_matmul(uint32_t a, uint32_t b) {
+    const uint32_t out = matmul_tensors(a, false, b, false, nullptr, MNI_EPI_NONE);
+    if (out == MNI_BAD_ID) return out;
+    Entry e;
+    e.op = OP_MATMUL; e.output_id = out; e.n_inputs = 2; e.inputs[0] = a; e.inputs[1] = b;
+    eng().tape.record(std::move(e));
+    return out;
+}
+uint32_t mni_linear(uint32_t x, uint32_t w, uint32_t bias, int act) { return linear_op(x, w, bias, act); }
+
+uint32_t mni_sum_op(uint32_t a, int64_t dim) { return reduce_op(a, dim, false); }
+uint32_t mni_mean_op(uint32_t a, int64_t dim) { return reduce_op(a, dim, true); }
+uint32_t mni_sum_all(uint32_t a) {
+    Tensor *t = get(a);
+    if (!t) return MNI_BAD_ID;
+    uint32_t cur = a;
+    for (int d = (int)t->shape.size() - 1; d >= 0 && cur != MNI_BAD_ID; --d) cur = reduce_op(cur, d, false);
+    return cur;
+}
+uint32_t mni_mean_all(uint32_t a) {
+    Tensor *t = get(a);
+    if (!t) return MNI_BAD_ID;
+    uint32_t cur = a;
+    for (int d = (int)t->shape.size() - 1; d >= 0 && cur != MNI_BAD_ID; --d) cur = reduce_op(cur, d, true);
+    return cur;
+}
+uint32_t mni_view(uint32_t a, const int64_t *shape, int ndim) {
+    Shape s;
+    if (!to_shape(shape, ndim, &s)) return MNI_BAD_ID;
+    return view_op(a, s);
+}
+uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim) {
+    Shape s;
+    if (!to_shape(dims, ndim, &s)) return MNI_BAD_ID;
+    return permute_op(a, s);
+}
+uint32_t mni_contiguous(uint32_t a) {  // layout.rs:218-227
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    if (is_contiguous(*A)) return a;
+    BufP b = contiguous_buf(*A);
+    if (!b) return MNI_BAD_ID;
+    const Shape shape = A->shape;
+    const uint32_t id = insert_contig(std::move(b), shape);
+    Entry e;
+    e.op = OP_CONTIGUOUS; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a;
+    eng().tape.record(std::move(e));
+    return id;
+}
+uint32_t mni_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n) {
+    if (!targets) { set_error(MNI_ERR_INVALID, "cross_entropy: null targets"); return MNI_BAD_ID; }
+    return cross_entropy_op(logits, targets, n);
+}
+int mni_adamw_step(const uint32_t *ids, size_t n, double lr, double beta1, double beta2, double eps,
+                   double weight_decay, int64_t step) {
+    return adamw_step(ids, n, (float)lr, (float)beta1, (float)beta2, (float)eps, (float)weight_decay, (uint32_t)step);
+}
+double mni_grad_norm(const uint32_t *ids, size_t n) {
+    float norm = 0.f;
+    if (grad_norm(ids, n, &norm) != MNI_OK) return -1.0;
+    return (double)norm;
+}
+int mni_clip_grad_norm(const uint32_t *ids, size_t n, double max_norm) {  // optimizer.rs:160-173
+    float norm = 0.f;
+    MNI_TRY(grad_norm(ids, n, &norm));
+    const float mx = (float)max_norm;
+    if (norm > mx) MNI_TRY(scale_grads(ids, n, mx / norm));
+    return MNI_OK;
+}
+double mni_clip_and_step(const uint32_t *ids, size_t n, double lr, double beta1, double beta2, double eps,
+                         double weight_decay, int64_t step, double max_grad_norm) {  // optimizer.rs:224-245
+    float norm = 0.f;
+    if (grad_norm(ids, n, &norm) != MNI_OK) return -1.0;
+    const float mg = (float)max_grad_norm;
+    if (mg > 0.0f && norm > mg)
+        if (scale_grads(ids, n, mg / norm) != MNI_OK) return -1.0;
+    if (adamw_step(ids, n, (float)lr, (float)beta1, (float)beta2, (float)eps, (float)weight_decay, (uint32_t)step) != MNI_OK)
+        return -1.0;
+    return (double)norm;
+}
+void mni_reset_engine(void) {
+    Engine &e = eng();
+    e.tensors.clear();
+    e.free_ids.clear();
+    e.tape = Tape();
+}
+int mni_gc_tensors(const uint32_t *keep, size_t n) {
+    Engine &e = eng();
+    const size_t len = e.tensors.size();
+    std::vector<char> k(len + 1, 0);
+    for (size_t i = 0; i < n; ++i)
+        if (keep[i] < len) k[keep[i]] = 1;
+    for (size_t id = 0; id < len; ++id)
+        if (!k[id] && e.tensors[id].live) free_tensor((uint32_t)id);
+    e.tape = Tape();
+    // The reference drops its allocator cache here (lib.rs:704).  Blocks stay
+    // cached for the next step unless the cache has grown large: returning
+    // them to the driver every step would cost a device-wide sync per block.
+    if (dev_cached_bytes() > ((size_t)64 << 30)) return dev_clear_cache();
+    return MNI_OK;
+}
+void *mni_dev_ptr(uint32_t id) {
+    Tensor *t = get(id);
+    return t ? (void *)t->buf->p : nullptr;
+}
+
+}  // extern "C"

@@ -1,0 +1,207 @@
+// mni_rocm_sgemm: validation, kernel choice (MFMA tile kernel vs the skinny
+// bandwidth kernels), operand-layout classification and the split-K plan.
+#include "common.h"
+#include "gemm_internal.h"
+
+namespace mni {
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// 0: K axis contiguous, 1: the other axis contiguous, 2: arbitrary.  `ks` is
+// the stride along K, `os` the stride along M (for A) or N (for B).  A batch
+// stride only matters when more than one batch matrix is addressed.
+static int classify(const float *p, int64_t ks, int64_t os, int64_t bs, int64_t bcount) {
+    const bool batch_ok = bcount <= 1 || (bs % 4) == 0;
+    if (!aligned16(p) || !batch_ok) return 2;
+    if (ks == 1 && (os % 4) == 0) return 0;
+    if (os == 1 && (ks % 4) == 0) return 1;
+    return 2;
+}
+
+static int validate(const mni_gemm_desc &d) {
+    if (d.M < 0 || d.N < 0 || d.K < 0 || d.batch < 0)
+        return set_error(MNI_ERR_INVALID, "sgemm: negative extent (M=%lld N=%lld K=%lld batch=%lld)",
+                         (long long)d.M, (long long)d.N, (long long)d.K, (long long)d.batch);
+    if (d.M > 0x7fffffffLL || d.N > 0x7fffffffLL || d.K > 0x7fffffffLL || d.batch > 0x7fffffffLL)
+        return set_error(MNI_ERR_INVALID, "sgemm: extent exceeds 2^31-1");
+    if (d.M == 0 || d.N == 0 || d.batch == 0) return MNI_OK;
+    if (!d.C) return set_error(MNI_ERR_INVALID, "sgemm: C is null");
+    if (d.K > 0 && (!d.A.ptr || !d.B.ptr)) return set_error(MNI_ERR_INVALID, "sgemm: operand pointer is null");
+    if (d.A.batch_count < 1 || d.B.batch_count < 1)
+        return set_error(MNI_ERR_INVALID, "sgemm: operand batch_count must be >= 1");
+    if (d.ldc < d.N) return set_error(MNI_ERR_INVALID, "sgemm: ldc (%lld) < N (%lld)", (long long)d.ldc, (long long)d.N);
+    if (d.epilogue < MNI_EPI_NONE || d.epilogue > MNI_EPI_BIAS_GELU)
+        return set_error(MNI_ERR_INVALID, "sgemm: unknown epilogue %d", d.epilogue);
+    if (d.epilogue != MNI_EPI_NONE && !d.bias)
+        return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
+    if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_SKINNY)
+        return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
+    return MNI_OK;
+}
+
+static int finish_split(const float *ws, float *out, const float *bias, int slices, int batch, int rows, int cols,
+                        int64_t o_rs, int64_t o_cs, int64_t o_bs, int epilogue, int accumulate, int bias_on_rows) {
+    ReduceLaunch r;
+    r.ws = ws; r.out = out; r.bias = bias;
+    r.slices = slices; r.batch = batch; r.rows = rows; r.cols = cols;
+    r.o_rs = o_rs; r.o_cs = o_cs; r.o_bs = o_bs;
+    r.epilogue = epilogue; r.accumulate = accumulate; r.bias_on_rows = bias_on_rows;
+    return launch_splitk_reduce(r);
+}
+
+// ---- skinny path --------------------------------------------------------------
+// Returns 1 when it handled the product, 0 when the shape/layout is not
+// eligible, < 0 ... never; errors are returned through *rc.
+static bool try_skinny(const mni_gemm_desc &d, int *rc) {
+    *rc = MNI_OK;
+    if (d.K == 0) return false;
+    SkinnyLaunch s;
+    bool swapped;
+    if (d.M <= 16) swapped = false;
+    else if (d.N <= 16) swapped = true;
+    else return false;
+
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        if (!swapped) {
+            s.rows = (int)d.M; s.cols = (int)d.N;
+            s.X = d.A.ptr; s.x_rs = d.A.row_stride; s.x_cs = d.A.col_stride;
+            s.x_bs = d.A.batch_stride; s.x_bcount = (int)d.A.batch_count;
+            s.W = d.B.ptr; s.w_rs = d.B.row_stride; s.w_cs = d.B.col_stride;
+            s.w_bs = d.B.batch_stride; s.w_bcount = (int)d.B.batch_count;
+            s.o_rs = d.ldc; s.o_cs = 1; s.bias_on_rows = 0;
+        } else {
+            // C^T = B^T * A^T: the few columns of C become the rows of X.
+            s.rows = (int)d.N; s.cols = (int)d.M;
+            s.X = d.B.ptr; s.x_rs = d.B.col_stride; s.x_cs = d.B.row_stride;
+            s.x_bs = d.B.batch_stride; s.x_bcount = (int)d.B.batch_count;
+            s.W = d.A.ptr; s.w_rs = d.A.col_stride; s.w_cs = d.A.row_stride;
+            s.w_bs = d.A.batch_stride; s.w_bcount = (int)d.A.batch_count;
+            s.o_rs = 1; s.o_cs = d.ldc; s.bias_on_rows = 1;
+        }
+        s.K = (int)d.K; s.batch = (int)d.batch;
+        s.out = d.C; s.o_bs = d.c_batch_stride; s.bias = d.bias;
+        s.epilogue = d.epilogue; s.accumulate = d.accumulate;
+        s.ws = nullptr; s.split_k = 1; s.k_per_slice = s.K;
+
+        const bool w_batch_ok = s.w_bcount <= 1 || (s.w_bs % 4) == 0;
+        const bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
+        const bool x_batch_ok = s.x_bcount <= 1 || (s.x_bs % 4) == 0;
+        const bool w_dots = s.w_rs == 1 && (s.w_cs % 4) == 0 && (s.K % 4) == 0 && aligned16(s.W) && w_batch_ok &&
+                            s.x_cs == 1 && (s.x_rs % 4) == 0 && aligned16(s.X) && x_batch_ok;
+
+        if (w_cols) {
+            // Enough workgroups to keep every CU streaming: aim at ~4 per CU.
+            const int groups = (s.cols + skinny_cols_block_cols() - 1) / skinny_cols_block_cols();
+            int split = d.split_k;
+            if (split == 0) {
+                const int64_t target = 4LL * (ctx().compute_units > 0 ? ctx().compute_units : 256);
+                const int64_t have = (int64_t)groups * s.batch;
+                split = (int)((target + have - 1) / have);
+                const int max_split = (s.K + 63) / 64;  // at least 64 K rows per slice
+                if (split > max_split) split = max_split;
+                if (split < 1) split = 1;
+            }
+            int kps = (s.K + split - 1) / split;
+            kps = (kps + 31) & ~31;
+            split = (s.K + kps - 1) / kps;
+            s.split_k = split; s.k_per_slice = kps;
+            void *ws = nullptr;
+            if (split > 1) {
+                const size_t bytes = (size_t)split * s.batch * s.rows * s.cols * sizeof(float);
+                *rc = dev_alloc(&ws, bytes);
+                if (*rc != MNI_OK) return true;
+                s.ws = (float *)ws;
+            }
+            *rc = launch_skinny_cols(s);
+            if (*rc == MNI_OK && split > 1)
+                *rc = finish_split(s.ws, s.out, s.bias, split, s.batch, s.rows, s.cols, s.o_rs, s.o_cs, s.o_bs,
+                                   s.epilogue, s.accumulate, s.bias_on_rows);
+            if (ws) dev_free(ws);
+            return true;
+        }
+        if (w_dots && d.split_k <= 1) {
+            *rc = launch_skinny_dots(s);
+            return true;
+        }
+        // Both extents small: the other orientation may be eligible.
+        if (attempt == 0 && !swapped && d.N <= 16) swapped = true;
+        else break;
+    }
+    return false;
+}
+
+// ---- MFMA path ----------------------------------------------------------------
+static int run_mfma(const mni_gemm_desc &d) {
+    GemmLaunch g;
+    g.A = d.A.ptr; g.B = d.B.ptr; g.C = d.C; g.bias = d.bias; g.ws = nullptr;
+    g.M = (int)d.M; g.N = (int)d.N; g.K = (int)d.K; g.batch = (int)d.batch;
+    g.a_rs = d.A.row_stride; g.a_cs = d.A.col_stride; g.a_bs = d.A.batch_stride;
+    g.b_rs = d.B.row_stride; g.b_cs = d.B.col_stride; g.b_bs = d.B.batch_stride;
+    g.a_bcount = (int)d.A.batch_count; g.b_bcount = (int)d.B.batch_count;
+    g.ldc = d.ldc; g.c_bs = d.c_batch_stride;
+    g.epilogue = d.epilogue; g.accumulate = d.accumulate;
+    const int bm = gemm_mfma_tile_m(), bn = gemm_mfma_tile_n(), bk = gemm_mfma_tile_k();
+    g.tiles_m = (g.M + bm - 1) / bm;
+    g.tiles_n = (g.N + bn - 1) / bn;
+
+    // op(A)(m, k): K stride = col_stride, M stride = row_stride.
+    const int amode = g.K == 0 ? 2 : classify(g.A, g.a_cs, g.a_rs, g.a_bs, g.a_bcount);
+    // op(B)(k, n): K stride = row_stride, N stride = col_stride.
+    const int bmode = g.K == 0 ? 2 : classify(g.B, g.b_rs, g.b_cs, g.b_bs, g.b_bcount);
+
+    // Split K when the output tiles alone cannot fill the machine (two
+    // workgroups fit on each CU).  Slices are whole K steps.
+    int split = d.split_k;
+    const int ktiles = (g.K + bk - 1) / bk;
+    if (split == 0) {
+        const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * g.batch;
+        const int64_t slots = 2LL * (ctx().compute_units > 0 ? ctx().compute_units : 256);
+        split = 1;
+        if (tiles * 4 < slots * 3) {
+            split = (int)((slots + tiles - 1) / tiles);
+            const int max_split = ktiles / 8 > 0 ? ktiles / 8 : 1;  // >= 8 K steps per slice
+            if (split > max_split) split = max_split;
+            if (split > 64) split = 64;
+        }
+    }
+    if (split > ktiles) split = ktiles > 0 ? ktiles : 1;
+    int tiles_per_slice = ktiles > 0 ? (ktiles + split - 1) / split : 1;
+    split = ktiles > 0 ? (ktiles + tiles_per_slice - 1) / tiles_per_slice : 1;
+    g.split_k = split;
+    g.k_per_slice = split > 1 ? tiles_per_slice * bk : (g.K > 0 ? g.K : 1);
+
+    void *ws = nullptr;
+    if (split > 1) {
+        const size_t bytes = (size_t)split * g.batch * g.M * g.N * sizeof(float);
+        MNI_TRY(dev_alloc(&ws, bytes));
+        g.ws = (float *)ws;
+    }
+    int rc = launch_gemm_mfma(g, amode, bmode);
+    if (rc == MNI_OK && split > 1)
+        rc = finish_split(g.ws, g.C, g.bias, split, g.batch, g.M, g.N, g.ldc, 1, g.c_bs, g.epilogue, g.accumulate, 0);
+    if (ws) dev_free(ws);
+    return rc;
+}
+
+int sgemm(const mni_gemm_desc &d) {
+    MNI_TRY(ensure_init());
+    MNI_TRY(validate(d));
+    if (d.M == 0 || d.N == 0 || d.batch == 0) return MNI_OK;
+    if (d.algo != MNI_ALGO_MFMA) {
+        int rc;
+        if (try_skinny(d, &rc)) return rc;
+        if (d.algo == MNI_ALGO_SKINNY)
+            return set_error(MNI_ERR_INVALID,
+                             "sgemm: shape/layout not eligible for the skinny kernels "
+                             "(needs min(M,N) <= 16 and 16-byte aligned unit-stride W)");
+    }
+    return run_mfma(d);
+}
+
+}  // namespace mni
+
+extern "C" int mni_rocm_sgemm(const mni_gemm_desc *desc) {
+    if (!desc) return mni::set_error(MNI_ERR_INVALID, "sgemm: null descriptor");
+    return mni::sgemm(*desc);
+}

@@ -1,0 +1,66 @@
+// Launch descriptors shared by the GEMM kernels and their dispatcher.
+#pragma once
+#include <stdint.h>
+
+namespace mni {
+
+// Everything a GEMM kernel needs, passed by value as the kernel argument.
+// op(A)[b](m, k) = A[(b % a_bcount) * a_bs + m * a_rs + k * a_cs]
+// op(B)[b](k, n) = B[(b % b_bcount) * b_bs + k * b_rs + n * b_cs]
+struct GemmLaunch {
+    const float *A;
+    const float *B;
+    float *C;
+    const float *bias;
+    float *ws;  // split-K partials [slice][batch][M][N]
+    int M, N, K, batch;
+    int64_t a_rs, a_cs, a_bs;
+    int64_t b_rs, b_cs, b_bs;
+    int a_bcount, b_bcount;
+    int64_t ldc, c_bs;
+    int split_k, k_per_slice;
+    int tiles_m, tiles_n;
+    int epilogue, accumulate;
+};
+
+int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode);
+int gemm_mfma_tile_m();
+int gemm_mfma_tile_n();
+int gemm_mfma_tile_k();
+
+// Skinny (GEMV-shaped) products: X (MR x K, MR <= 16) against a large W.
+//   out[b](i, j) = sum_k X[b](i, k) * W[b](k, j),  i < rows, j < cols
+// written at out[b * o_bs + i * o_rs + j * o_cs] (or to split-K partials).
+struct SkinnyLaunch {
+    const float *X;
+    const float *W;
+    float *out;
+    const float *bias;  // indexed by bias_on_rows ? i : j
+    float *ws;          // partials [slice][batch][rows][cols]
+    int rows, cols, K, batch;
+    int64_t x_rs, x_cs, x_bs;  // X(i, k)
+    int64_t w_rs, w_cs, w_bs;  // W(k, j)
+    int x_bcount, w_bcount;
+    int64_t o_rs, o_cs, o_bs;
+    int split_k, k_per_slice;
+    int epilogue, accumulate, bias_on_rows;
+};
+// W with unit stride along j (cols): lanes own columns, K split over waves.
+int launch_skinny_cols(const SkinnyLaunch &s);
+// W with unit stride along k: one wavefront per output column, shuffle reduce.
+int launch_skinny_dots(const SkinnyLaunch &s);
+int skinny_cols_block_cols();
+
+// Sums split-K partials ws[slice][batch][rows][cols] in slice order and
+// applies the epilogue; out addressed with (o_bs, o_rs, o_cs).
+struct ReduceLaunch {
+    const float *ws;
+    float *out;
+    const float *bias;
+    int slices, batch, rows, cols;
+    int64_t o_rs, o_cs, o_bs;
+    int epilogue, accumulate, bias_on_rows;
+};
+int launch_splitk_reduce(const ReduceLaunch &r);
+
+}  // namespace mni

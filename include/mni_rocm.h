@@ -1,0 +1,190 @@
+/*
+ * mni_rocm.h -- C ABI of libmni_rocm.so, the MI355X (gfx950) backend for the
+ * fp32 matrix-multiply path of mni-ml/framework.
+ *
+ * Two layers are exported:
+ *
+ *   1. Kernel level (mni_rocm_*): raw device pointers and sizes.  This is what
+ *      a `rocm` cargo feature of the reference's Rust native layer binds with
+ *      `extern "C"` from its own TensorStore/ops arms; each entry names the
+ *      reference call site it replaces.
+ *
+ *   2. Engine level (mni_*): a self-contained counterpart of the reference's
+ *      `Engine { store, tape }` behind its N-API bridge, one function per
+ *      `#[napi]` export of src/native/src/lib.rs that the matmul path and its
+ *      callers use.  Tensors are opaque u32 ids exactly as on the JS side.
+ *
+ * Conventions: no function throws or aborts.  Status-returning functions
+ * return 0 on success and a non-zero MNI_ERR_* code on failure; id-returning
+ * functions return MNI_BAD_ID on failure.  The message of the most recent
+ * failure on the calling thread's library instance is available from
+ * mni_rocm_last_error().  All work is issued on one library-owned HIP stream;
+ * calls are stream-ordered, and only the documented functions synchronise.
+ * The library is not re-entrant across threads (same contract as the
+ * reference's single global mutex, src/native/src/lib.rs:27-39).
+ */
+#ifndef MNI_ROCM_H
+#define MNI_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MNI_OK 0
+#define MNI_ERR_INVALID 1   /* bad argument / shape mismatch (reference: panic)   */
+#define MNI_ERR_FREED 2     /* "tensor already freed" (src/native/src/tensor.rs:116) */
+#define MNI_ERR_HIP 3       /* a HIP runtime call failed                           */
+#define MNI_ERR_NOMEM 4     /* device allocation failed                            */
+#define MNI_BAD_ID UINT32_MAX
+
+/* ------------------------------------------------------------------------- *
+ * 1. Kernel level
+ * ------------------------------------------------------------------------- */
+
+/* Device singleton: replaces GpuDevice::instance() of the cuda arm
+ * (src/native/src/device.rs:29-48): one device, one stream, code objects
+ * prebuilt into the library (no runtime compilation). Idempotent. */
+int mni_rocm_init(int device);
+/* Name reported by the HIP runtime and its compute-unit count / clock (kHz),
+ * for roofline bookkeeping.  Any out pointer may be NULL. */
+int mni_rocm_device_info(char *name, size_t name_cap, int *compute_units, int *clock_khz);
+const char *mni_rocm_last_error(void);
+
+/* Caching device allocator: replaces CachingAllocator of the cuda arm
+ * (src/native/src/allocator.rs:46-84).  Exact-size free lists; unlike the
+ * reference's cuda arm, memory handed to zero-initialised tensors is cleared
+ * on reuse. */
+int mni_rocm_malloc(void **ptr, size_t bytes);
+int mni_rocm_free(void *ptr);
+int mni_rocm_clear_cache(void);
+/* Copies.  h2d/d2h synchronise the stream before returning (the reference's
+ * memcpy_stod / memcpy_dtov, src/native/src/tensor.rs:364-387,460-469). */
+int mni_rocm_h2d(void *dst, const void *src, size_t bytes);
+int mni_rocm_d2h(void *dst, const void *src, size_t bytes);
+int mni_rocm_d2d(void *dst, const void *src, size_t bytes);
+int mni_rocm_sync(void);
+
+/* Stream-ordered timing marks on the library's stream (HIP events). */
+int mni_rocm_event_create(void **event);
+int mni_rocm_event_record(void *event);
+int mni_rocm_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
+int mni_rocm_event_destroy(void *event);
+
+/* One operand of a product.  op(X) is addressed as
+ *   X[batch b, row r, col c] = ptr[(b % batch_count) * batch_stride + r * row_stride + c * col_stride]
+ * with strides in elements, so a transposed or permuted view is just a
+ * different pair of strides: nothing is materialised.  `b % batch_count` is
+ * the reference's batch rule (src/native/src/ops/matmul.rs:55-56). */
+typedef struct {
+    const float *ptr;
+    int64_t row_stride;
+    int64_t col_stride;
+    int64_t batch_stride;
+    int64_t batch_count; /* >= 1 */
+} mni_operand;
+
+enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_GELU = 3 };
+enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2 };
+
+/* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
+ * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),
+ * the permute_f32 transposes feeding them (:287-326), the host gather of
+ * non-contiguous operands (src/native/src/tensor.rs:510-517) and, with a bias
+ * epilogue, add_bias_f32 (src/native/src/ops/elementwise.rs:105-130). */
+typedef struct {
+    int64_t M, N, K, batch;
+    mni_operand A; /* op(A): rows = M, cols = K */
+    mni_operand B; /* op(B): rows = K, cols = N */
+    float *C;
+    int64_t ldc;
+    int64_t c_batch_stride;
+    const float *bias;   /* N floats, or NULL when epilogue == MNI_EPI_NONE */
+    int32_t epilogue;    /* MNI_EPI_*                                       */
+    int32_t accumulate;  /* non-zero: C += result                            */
+    int32_t split_k;     /* 0 = choose, 1 = never, n > 1 = exactly n slices */
+    int32_t algo;        /* MNI_ALGO_*                                      */
+} mni_gemm_desc;
+int mni_rocm_sgemm(const mni_gemm_desc *desc);
+
+/* dst (contiguous, `shape`) = gather of src by `src_strides` (elements).
+ * Replaces permute_f32 (src/native/kernels/elementwise.cu:67-81) and the host
+ * gather in ensure_contiguous (src/native/src/tensor.rs:510-517); up to 8 dims. */
+int mni_rocm_strided_copy(float *dst, const float *src, const int64_t *shape,
+                          const int64_t *src_strides, int ndim);
+/* out[r, c] = a[r, c] + bias[c]   (add_bias_f32, src/native/kernels/elementwise.cu:43-47) */
+int mni_rocm_add_bias(float *out, const float *a, const float *bias, int64_t rows, int64_t cols);
+/* out[c] = sum_r a[r, c]          (bias gradient; replaces the host unbroadcast of
+ * add_backward, src/native/src/ops/elementwise.rs:213-231) */
+int mni_rocm_colsum(float *out, const float *a, int64_t rows, int64_t cols);
+/* dst[i] += alpha * src[i]        (add_f32 in accumulate_grad / add_inplace,
+ * src/native/src/tensor.rs:475-508) */
+int mni_rocm_axpy(float *dst, const float *src, float alpha, int64_t n);
+/* dst[i] = value                  (fill_f32, src/native/src/tensor.rs:395-442) */
+int mni_rocm_fill(float *dst, float value, int64_t n);
+
+/* ------------------------------------------------------------------------- *
+ * 2. Engine level: mirrors src/native/src/lib.rs export by export.
+ * ------------------------------------------------------------------------- */
+
+#define MNI_MAX_DIMS 8
+
+uint32_t mni_zeros(const int64_t *shape, int ndim);                       /* lib.rs:45-50   */
+uint32_t mni_ones(const int64_t *shape, int ndim);                        /* lib.rs:52-57   */
+uint32_t mni_from_float32(const float *data, size_t len,
+                          const int64_t *shape, int ndim);                /* lib.rs:73-78   */
+int mni_tensor_shape(uint32_t id, int64_t *out, int cap);                 /* lib.rs:80-84; returns ndim or -1 */
+int64_t mni_tensor_size(uint32_t id);                                     /* lib.rs:86-90   */
+int mni_to_float32(uint32_t id, float *out, size_t cap);                  /* lib.rs:92-97   */
+int mni_get_scalar(uint32_t id, double *out);                             /* lib.rs:99-103  */
+void mni_free_tensor(uint32_t id);                                        /* lib.rs:105-109 */
+int mni_set_requires_grad(uint32_t id, int requires);                     /* lib.rs:115-119 */
+int mni_get_grad(uint32_t id, uint32_t *out);                             /* lib.rs:121-125; 1 = has grad, 0 = none, -1 = error */
+int mni_backward(uint32_t loss);                                          /* lib.rs:131-137 */
+int mni_zero_grad(const uint32_t *ids, size_t n);                         /* lib.rs:139-146 */
+void mni_no_grad_start(void);                                             /* lib.rs:148-152 */
+void mni_no_grad_end(void);                                               /* lib.rs:154-158 */
+uint32_t mni_add(uint32_t a, uint32_t b);                                 /* lib.rs:164-169 */
+uint32_t mni_mul(uint32_t a, uint32_t b);                                 /* lib.rs:171-176 */
+uint32_t mni_sub(uint32_t a, uint32_t b);                                 /* lib.rs:178-183 */
+uint32_t mni_neg(uint32_t a);                                             /* lib.rs:185-190 */
+uint32_t mni_mul_scalar(uint32_t a, double s);                            /* lib.rs:192-197 */
+uint32_t mni_matmul(uint32_t a, uint32_t b);                              /* lib.rs:199-204 */
+uint32_t mni_gelu(uint32_t a);                                            /* lib.rs:206-211 */
+uint32_t mni_relu(uint32_t a);                                            /* lib.rs:213-218 */
+uint32_t mni_sum_op(uint32_t a, int64_t dim);                             /* lib.rs:234-239 */
+uint32_t mni_mean_op(uint32_t a, int64_t dim);                            /* lib.rs:241-246 */
+uint32_t mni_sum_all(uint32_t a);                                         /* lib.rs:255-265 */
+uint32_t mni_mean_all(uint32_t a);                                        /* lib.rs:267-277 */
+uint32_t mni_view(uint32_t a, const int64_t *shape, int ndim);            /* lib.rs:279-285 */
+uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim);          /* lib.rs:287-293 */
+uint32_t mni_contiguous(uint32_t a);                                      /* lib.rs:295-300 */
+uint32_t mni_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n); /* lib.rs:328-336 */
+int mni_adamw_step(const uint32_t *ids, size_t n, double lr, double beta1, double beta2,
+                   double eps, double weight_decay, int64_t step);        /* lib.rs:400-412 */
+double mni_grad_norm(const uint32_t *ids, size_t n);                      /* lib.rs:414-419; < 0 on error */
+int mni_clip_grad_norm(const uint32_t *ids, size_t n, double max_norm);   /* lib.rs:421-426 */
+double mni_clip_and_step(const uint32_t *ids, size_t n, double lr, double beta1, double beta2,
+                         double eps, double weight_decay, int64_t step,
+                         double max_grad_norm);                           /* lib.rs:428-442; < 0 on error */
+void mni_reset_engine(void);                                              /* lib.rs:460-468 */
+int mni_gc_tensors(const uint32_t *keep, size_t n);                       /* lib.rs:693-706 */
+
+/* Opt-in fused Linear: out = x * w + bias in one product with a bias
+ * epilogue, recorded as one tape entry whose backward yields dX, dW and db.
+ * The reference composes this from `matmul` then `add` (src/nn.ts:23-25); a
+ * caller feature-detects this export the way the reference detects its
+ * cuda-only fused ops (src/nn.ts:116, test/native.test.ts:13).
+ * act: MNI_EPI_BIAS (none), MNI_EPI_BIAS_RELU or MNI_EPI_BIAS_GELU. */
+uint32_t mni_linear(uint32_t x, uint32_t w, uint32_t bias, int act);
+
+/* Device address of a tensor's buffer (cuda arm: TensorStore::dev_ptr,
+ * src/native/src/tensor.rs:358-361). NULL on error. */
+void *mni_dev_ptr(uint32_t id);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MNI_ROCM_H */

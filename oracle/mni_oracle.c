@@ -1,0 +1,1185 @@
+/*
+ * mni_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * A plain-C, single-threaded restatement of the pure-Rust CPU backend of
+ * mni-ml/framework for the fp32 matmul path: tensor store, autograd tape and
+ * the handful of ops the path and its callers touch.  It exists only so that
+ * the tests, the smoke check and the cpu_baseline leg of the benchmark have
+ * something to compare the HIP backend against.  Nothing in the shipped
+ * library links, loads or calls this file.
+ *
+ * Build: gcc -O3 -ffp-contract=off -fno-fast-math (no -march=native) so every
+ * sum is the same sequence of separately rounded f32 multiplies and adds the
+ * reference's release build performs (Rust never contracts a*b+c to an FMA;
+ * src/native/Cargo.toml:30-32 sets opt-level 3 on the x86-64 baseline target).
+ *
+ * Every function cites the reference lines it restates (paths relative to the
+ * reference checkout).  What pins each function is listed next to it as
+ * "pinned by": reference-held test vectors (the test suites under test/), closed forms and
+ * brute force in tests/test_oracle_*.py.  Transcendentals (expf, logf, tanhf,
+ * sqrtf, powf) come from glibc, not Rust's libm: they may differ by an ulp or
+ * two from the reference, which is far inside the parity tolerance.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_MAX_DIMS 8
+#define ORC_BAD UINT32_MAX
+
+typedef struct {
+    int live;
+    float *data;            /* raw buffer, `size` floats                     */
+    size_t shape[ORC_MAX_DIMS];
+    size_t strides[ORC_MAX_DIMS]; /* in elements                             */
+    int ndim;
+    size_t size;
+    int requires_grad;
+    long grad;              /* tensor id of .grad, or -1                     */
+    float *adam_m, *adam_v; /* lazily created by adamw_step                  */
+} orc_tensor;
+
+/* tensor.rs:96-100 TensorStore{tensors, free_ids, alloc} */
+typedef struct {
+    orc_tensor *t;
+    size_t len, cap;
+    size_t *free_ids;
+    size_t nfree, capfree;
+} orc_store;
+
+enum orc_op { /* subset of autograd.rs:28-62 BackwardOp */
+    OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
+    OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY
+};
+
+/* autograd.rs:65-70 TapeEntry + the SavedContext variants the subset needs */
+typedef struct {
+    int op;
+    size_t output_id;
+    size_t input_ids[2];
+    int n_inputs;
+    size_t saved_ids[2];          /* Tensor / Tensors / TensorsAndShape ids  */
+    size_t saved_shape[ORC_MAX_DIMS]; /* Shape / TensorAndShape / Permutation orig */
+    int saved_ndim;
+    size_t saved_perm[ORC_MAX_DIMS];
+    float saved_scalar;
+    size_t *targets;              /* Indices(targets, n, v, sm_id)           */
+    size_t ce_n, ce_v, ce_sm;
+} orc_entry;
+
+typedef struct {
+    orc_entry *e;
+    size_t len, cap;
+    int enabled;
+} orc_tape;
+
+static orc_store g_store;
+static orc_tape g_tape = {0, 0, 0, 1};
+static char g_err[512];
+
+static uint32_t fail(const char *msg) {
+    snprintf(g_err, sizeof g_err, "%s", msg);
+    return ORC_BAD;
+}
+const char *orc_last_error(void) { return g_err; }
+
+/* ---- shape helpers ------------------------------------------------------ */
+
+/* tensor.rs:7-17 compute_strides */
+static void compute_strides(const size_t *shape, int ndim, size_t *strides) {
+    if (ndim == 0) return;
+    strides[ndim - 1] = 1;
+    for (int i = ndim - 2; i >= 0; --i) strides[i] = strides[i + 1] * shape[i + 1];
+}
+
+/* tensor.rs:19-21 shape_size: product, at least 1 */
+static size_t shape_size(const size_t *shape, int ndim) {
+    size_t p = 1;
+    for (int i = 0; i < ndim; ++i) p *= shape[i];
+    return p < 1 ? 1 : p;
+}
+
+/* tensor.rs:41-53 is_contiguous: every dim checked, size-1 dims included */
+static int is_contiguous(const orc_tensor *t) {
+    if (t->ndim == 0) return 1;
+    size_t expected = 1;
+    for (int i = t->ndim - 1; i >= 0; --i) {
+        if (t->strides[i] != expected) return 0;
+        expected *= t->shape[i];
+    }
+    return 1;
+}
+
+/* utils.rs:3-20 broadcast_shape; returns -1 where the reference panics */
+static int broadcast_shape(const size_t *a, int na, const size_t *b, int nb, size_t *out) {
+    int n = na > nb ? na : nb;
+    for (int i = 0; i < n; ++i) {
+        size_t da = i < n - na ? 1 : a[i - (n - na)];
+        size_t db = i < n - nb ? 1 : b[i - (n - nb)];
+        if (da == db) out[i] = da;
+        else if (da == 1) out[i] = db;
+        else if (db == 1) out[i] = da;
+        else return -1;
+    }
+    return n;
+}
+
+static int same_shape(const size_t *a, int na, const size_t *b, int nb) {
+    if (na != nb) return 0;
+    for (int i = 0; i < na; ++i) if (a[i] != b[i]) return 0;
+    return 1;
+}
+
+/* utils.rs:39-66 unbroadcast: sum a grad of grad_shape down to orig_shape,
+ * visiting grad elements in flat order (so each output receives its terms in
+ * increasing flat index). */
+static float *unbroadcast(const float *g, const size_t *gshape, int gnd,
+                          const size_t *oshape, int ond) {
+    size_t osz = shape_size(oshape, ond);
+    if (same_shape(gshape, gnd, oshape, ond)) {
+        float *out = (float *)malloc(osz * sizeof(float));
+        memcpy(out, g, osz * sizeof(float));
+        return out;
+    }
+    float *out = (float *)calloc(osz, sizeof(float));
+    size_t gstr[ORC_MAX_DIMS], ostr[ORC_MAX_DIMS];
+    compute_strides(gshape, gnd, gstr);
+    compute_strides(oshape, ond, ostr);
+    int offset = gnd - ond;
+    size_t gsz = shape_size(gshape, gnd);
+    for (size_t i = 0; i < gsz; ++i) {
+        size_t rem = i, out_idx = 0;
+        for (int d = 0; d < gnd; ++d) {
+            size_t c = rem / gstr[d];
+            rem %= gstr[d];
+            if (d >= offset) {
+                int od = d - offset;
+                out_idx += (oshape[od] == 1 ? 0 : c) * ostr[od];
+            }
+        }
+        out[out_idx] += g[i];
+    }
+    return out;
+}
+
+/* ---- store -------------------------------------------------------------- */
+
+/* tensor.rs:104-113 insert: pop the most recently freed id, else append */
+static size_t store_insert(float *data, const size_t *shape, const size_t *strides, int ndim, size_t size) {
+    size_t id;
+    if (g_store.nfree) {
+        id = g_store.free_ids[--g_store.nfree];
+    } else {
+        if (g_store.len == g_store.cap) {
+            g_store.cap = g_store.cap ? g_store.cap * 2 : 64;
+            g_store.t = (orc_tensor *)realloc(g_store.t, g_store.cap * sizeof(orc_tensor));
+        }
+        id = g_store.len++;
+    }
+    orc_tensor *t = &g_store.t[id];
+    memset(t, 0, sizeof *t);
+    t->live = 1;
+    t->data = data;
+    t->ndim = ndim;
+    for (int i = 0; i < ndim; ++i) { t->shape[i] = shape[i]; t->strides[i] = strides[i]; }
+    t->size = size;
+    t->grad = -1;
+    return id;
+}
+
+/* tensor.rs:263-270 from_vec (takes ownership of data) */
+static size_t from_vec(float *data, const size_t *shape, int ndim) {
+    size_t strides[ORC_MAX_DIMS];
+    compute_strides(shape, ndim, strides);
+    return store_insert(data, shape, strides, ndim, shape_size(shape, ndim));
+}
+
+/* tensor.rs:115-117 get: "tensor already freed" panic -> NULL */
+static orc_tensor *get(size_t id) {
+    if (id >= g_store.len || !g_store.t[id].live) return NULL;
+    return &g_store.t[id];
+}
+
+/* tensor.rs:169-174 free */
+static void store_free(size_t id) {
+    if (id >= g_store.len || !g_store.t[id].live) return;
+    orc_tensor *t = &g_store.t[id];
+    free(t->data); free(t->adam_m); free(t->adam_v);
+    t->live = 0; t->data = NULL; t->adam_m = t->adam_v = NULL;
+    if (g_store.nfree == g_store.capfree) {
+        g_store.capfree = g_store.capfree ? g_store.capfree * 2 : 64;
+        g_store.free_ids = (size_t *)realloc(g_store.free_ids, g_store.capfree * sizeof(size_t));
+    }
+    g_store.free_ids[g_store.nfree++] = id;
+}
+
+/* tensor.rs:292-309 make_contiguous_data: gather by strides in flat order */
+static float *make_contiguous_data(const orc_tensor *t) {
+    float *out = (float *)calloc(t->size ? t->size : 1, sizeof(float));
+    size_t ostr[ORC_MAX_DIMS];
+    compute_strides(t->shape, t->ndim, ostr);
+    for (size_t i = 0; i < t->size; ++i) {
+        size_t src = 0, rem = i;
+        for (int d = 0; d < t->ndim; ++d) {
+            size_t c = rem / ostr[d];
+            rem %= ostr[d];
+            src += c * t->strides[d];
+        }
+        out[i] = t->data[src];
+    }
+    return out;
+}
+
+/* tensor.rs:184-191 to_host: always a fresh copy */
+static float *to_host(const orc_tensor *t) {
+    if (is_contiguous(t)) {
+        float *out = (float *)malloc((t->size ? t->size : 1) * sizeof(float));
+        memcpy(out, t->data, t->size * sizeof(float));
+        return out;
+    }
+    return make_contiguous_data(t);
+}
+
+/* tensor.rs:311-318 ensure_contiguous: same id when already contiguous */
+static size_t ensure_contiguous(size_t id) {
+    orc_tensor *t = get(id);
+    if (is_contiguous(t)) return id;
+    float *d = make_contiguous_data(t);
+    size_t shape[ORC_MAX_DIMS]; int nd = t->ndim;
+    memcpy(shape, t->shape, sizeof shape);
+    return from_vec(d, shape, nd);
+}
+
+/* tensor.rs:207-215 zeros / :217-226 ones */
+static size_t zeros(const size_t *shape, int ndim) {
+    size_t n = shape_size(shape, ndim);
+    return from_vec((float *)calloc(n, sizeof(float)), shape, ndim);
+}
+static size_t ones(const size_t *shape, int ndim) {
+    size_t n = shape_size(shape, ndim);
+    float *d = (float *)malloc(n * sizeof(float));
+    for (size_t i = 0; i < n; ++i) d[i] = 1.0f;
+    return from_vec(d, shape, ndim);
+}
+
+/* tensor.rs:144-152 ensure_grad */
+static size_t ensure_grad(size_t id) {
+    orc_tensor *t = get(id);
+    if (t->grad >= 0) return (size_t)t->grad;
+    size_t shape[ORC_MAX_DIMS]; int nd = t->ndim;
+    memcpy(shape, t->shape, sizeof shape);
+    size_t g = zeros(shape, nd);
+    get(id)->grad = (long)g;
+    return g;
+}
+
+/* tensor.rs:272-280 accumulate_grad: raw-buffer order, src.size elements */
+static void accumulate_grad(size_t dst, size_t src) {
+    size_t gid = ensure_grad(dst);
+    orc_tensor *s = get(src), *g = get(gid);
+    for (size_t i = 0; i < s->size; ++i) g->data[i] += s->data[i];
+}
+
+/* tensor.rs:283-290 add_inplace */
+static void add_inplace(size_t dst, size_t src) {
+    orc_tensor *s = get(src), *d = get(dst);
+    for (size_t i = 0; i < s->size; ++i) d->data[i] += s->data[i];
+}
+
+/* ---- tape --------------------------------------------------------------- */
+
+/* autograd.rs:90-94 record */
+static orc_entry *tape_record(orc_tape *tp, int op, size_t out, int n_in, size_t in0, size_t in1) {
+    static orc_entry dummy;
+    if (!tp->enabled) { memset(&dummy, 0, sizeof dummy); return &dummy; }
+    if (tp->len == tp->cap) {
+        tp->cap = tp->cap ? tp->cap * 2 : 64;
+        tp->e = (orc_entry *)realloc(tp->e, tp->cap * sizeof(orc_entry));
+    }
+    orc_entry *e = &tp->e[tp->len++];
+    memset(e, 0, sizeof *e);
+    e->op = op; e->output_id = out; e->n_inputs = n_in;
+    e->input_ids[0] = in0; e->input_ids[1] = in1;
+    e->saved_ids[0] = in0; e->saved_ids[1] = in1;
+    return e;
+}
+
+static void tape_clear(orc_tape *tp) {
+    for (size_t i = 0; i < tp->len; ++i) free(tp->e[i].targets);
+    free(tp->e);
+    tp->e = NULL; tp->len = tp->cap = 0; tp->enabled = 1;
+}
+
+/* ---- matmul (the path) -------------------------------------------------- */
+
+/* ops/matmul.rs:18-78 matmul, cpu arm.  Both operands are materialised
+ * contiguous (:20-21) and cloned (:45-46); the batch index of an operand is
+ * `batch % operand_batch_size` (:55-56); the hot loop is i-k-j with an f32
+ * accumulator that starts at +0.0 (:62-69).
+ * pinned by: test/tensor.test.ts:222-240 vectors, f64 brute force, A*I=A,
+ * ones*ones=K, integer-exact cases (tests/test_oracle_matmul.py). */
+static uint32_t matmul_impl(size_t a, size_t b, orc_tape *tp) {
+    if (!get(a) || !get(b)) return fail("tensor already freed");
+    size_t a_id = ensure_contiguous(a);
+    size_t b_id = ensure_contiguous(b);
+    orc_tensor *A = get(a_id), *B = get(b_id);
+    if (A->ndim < 2 || B->ndim < 2) return fail("matmul requires at least 2D tensors");
+    size_t m = A->shape[A->ndim - 2], k = A->shape[A->ndim - 1];
+    size_t k2 = B->shape[B->ndim - 2], n = B->shape[B->ndim - 1];
+    if (k != k2) return fail("matmul inner dimensions must match");
+
+    size_t out_shape[ORC_MAX_DIMS];
+    int nb = broadcast_shape(A->shape, A->ndim - 2, B->shape, B->ndim - 2, out_shape);
+    if (nb < 0) return fail("shapes are not broadcastable");
+    if (nb + 2 > ORC_MAX_DIMS) return fail("too many dims");
+    size_t batch_size = shape_size(out_shape, nb);
+    out_shape[nb] = m; out_shape[nb + 1] = n;
+    size_t a_bs = shape_size(A->shape, A->ndim - 2);
+    size_t b_bs = shape_size(B->shape, B->ndim - 2);
+
+    float *a_data = to_host(A);
+    float *b_data = to_host(B);
+    size_t out_size = shape_size(out_shape, nb + 2);
+    float *out = (float *)calloc(out_size, sizeof(float));
+    size_t a_mat = m * k, b_mat = k * n, c_mat = m * n;
+
+    for (size_t batch = 0; batch < batch_size; ++batch) {
+        size_t a_bi = a_bs == 1 ? 0 : batch % a_bs;
+        size_t b_bi = b_bs == 1 ? 0 : batch % b_bs;
+        const float *ap = a_data + a_bi * a_mat;
+        const float *bp = b_data + b_bi * b_mat;
+        float *cp = out + batch * c_mat;
+        for (size_t i = 0; i < m; ++i) {
+            for (size_t kk = 0; kk < k; ++kk) {
+                float a_val = ap[i * k + kk];
+                const float *brow = bp + kk * n;
+                float *crow = cp + i * n;
+                for (size_t j = 0; j < n; ++j) crow[j] += a_val * brow[j];
+            }
+        }
+    }
+    free(a_data); free(b_data);
+    size_t out_id = from_vec(out, out_shape, nb + 2);
+    tape_record(tp, OP_MATMUL, out_id, 2, a, b); /* original ids, :73-76 */
+    return (uint32_t)out_id;
+}
+
+/* ops/matmul.rs:329-333 matmul_no_grad: a throwaway disabled tape */
+static uint32_t matmul_no_grad(size_t a, size_t b) {
+    orc_tape dummy = {0, 0, 0, 0};
+    return matmul_impl(a, b, &dummy);
+}
+
+/* ops/matmul.rs:258-284 transpose_last2, cpu arm
+ * pinned by: (A*B)^T = B^T*A^T and numpy transpose in tests. */
+static size_t transpose_last2(size_t a) {
+    orc_tensor *t = get(a);
+    size_t shape[ORC_MAX_DIMS]; int nd = t->ndim;
+    memcpy(shape, t->shape, sizeof shape);
+    size_t a_id = ensure_contiguous(a);
+    float *data = to_host(get(a_id));
+    size_t m = shape[nd - 2], n = shape[nd - 1];
+    size_t bs = 1;
+    for (int i = 0; i < nd - 2; ++i) bs *= shape[i];
+    if (bs < 1) bs = 1;
+    size_t total = get(a_id)->size;
+    float *out = (float *)calloc(total ? total : 1, sizeof(float));
+    size_t mat = m * n;
+    for (size_t b = 0; b < bs; ++b) {
+        size_t off = b * mat;
+        for (size_t i = 0; i < m; ++i)
+            for (size_t j = 0; j < n; ++j) out[off + j * m + i] = data[off + i * n + j];
+    }
+    free(data);
+    shape[nd - 2] = n; shape[nd - 1] = m;
+    return from_vec(out, shape, nd);
+}
+
+/* ops/matmul.rs:199-222 matmul_backward, cpu arm: both grads always.
+ * pinned by: dX/dY of test/autograd.test.ts:42-46 in closed form, f64 central
+ * differences on small cases, broadcast-batch sums vs numpy. */
+static int matmul_backward(size_t grad, const orc_entry *e, long *out) {
+    size_t a = e->saved_ids[0], b = e->saved_ids[1];
+    if (!get(a) || !get(b) || !get(grad)) { fail("tensor already freed"); return -1; }
+    size_t a_shape[ORC_MAX_DIMS], b_shape[ORC_MAX_DIMS];
+    int a_nd = get(a)->ndim, b_nd = get(b)->ndim;
+    memcpy(a_shape, get(a)->shape, sizeof a_shape);
+    memcpy(b_shape, get(b)->shape, sizeof b_shape);
+
+    size_t b_t = transpose_last2(b);
+    uint32_t grad_a = matmul_no_grad(grad, b_t);
+    if (grad_a == ORC_BAD) return -1;
+    float *gad = to_host(get(grad_a));
+    float *ga = unbroadcast(gad, get(grad_a)->shape, get(grad_a)->ndim, a_shape, a_nd);
+    free(gad);
+    out[0] = (long)from_vec(ga, a_shape, a_nd);
+
+    size_t a_t = transpose_last2(a);
+    uint32_t grad_b = matmul_no_grad(a_t, grad);
+    if (grad_b == ORC_BAD) return -1;
+    float *gbd = to_host(get(grad_b));
+    float *gb = unbroadcast(gbd, get(grad_b)->shape, get(grad_b)->ndim, b_shape, b_nd);
+    free(gbd);
+    out[1] = (long)from_vec(gb, b_shape, b_nd);
+    return 0;
+}
+
+/* ---- elementwise -------------------------------------------------------- */
+
+/* ops/elementwise.rs:20-56 broadcast_binary; op: 0 add, 1 sub, 2 mul
+ * pinned by: test/tensor.test.ts:248-256 broadcast values, numpy broadcasting. */
+static uint32_t broadcast_binary(size_t a, size_t b, int op, size_t *out_shape, int *out_nd) {
+    orc_tensor *A = get(a), *B = get(b);
+    if (!A || !B) return fail("tensor already freed");
+    int nd = broadcast_shape(A->shape, A->ndim, B->shape, B->ndim, out_shape);
+    if (nd < 0) return fail("shapes are not broadcastable");
+    size_t out_size = shape_size(out_shape, nd);
+    size_t ostr[ORC_MAX_DIMS], astr[ORC_MAX_DIMS], bstr[ORC_MAX_DIMS];
+    compute_strides(out_shape, nd, ostr);
+    compute_strides(A->shape, A->ndim, astr);
+    compute_strides(B->shape, B->ndim, bstr);
+    float *ad = to_host(A), *bd = to_host(B);
+    float *out = (float *)calloc(out_size, sizeof(float));
+    int a_off = nd - A->ndim, b_off = nd - B->ndim;
+    for (size_t i = 0; i < out_size; ++i) {
+        size_t coord[ORC_MAX_DIMS], rem = i;
+        for (int d = 0; d < nd; ++d) { coord[d] = rem / ostr[d]; rem %= ostr[d]; }
+        size_t ai = 0, bi = 0;
+        for (int d = 0; d < A->ndim; ++d) ai += (A->shape[d] == 1 ? 0 : coord[d + a_off]) * astr[d];
+        for (int d = 0; d < B->ndim; ++d) bi += (B->shape[d] == 1 ? 0 : coord[d + b_off]) * bstr[d];
+        float x = ad[ai], y = bd[bi];
+        out[i] = op == 0 ? x + y : op == 1 ? x - y : x * y;
+    }
+    free(ad); free(bd);
+    *out_nd = nd;
+    return (uint32_t)from_vec(out, out_shape, nd);
+}
+
+/* ops/elementwise.rs:62-73 add, :237-248 mul, :474-485 sub */
+static uint32_t binary_op(size_t a, size_t b, int op) {
+    size_t shape[ORC_MAX_DIMS]; int nd;
+    uint32_t out = broadcast_binary(a, b, op, shape, &nd);
+    if (out == ORC_BAD) return out;
+    orc_entry *e = tape_record(&g_tape, op == 0 ? OP_ADD : op == 1 ? OP_SUB : OP_MUL, out, 2, a, b);
+    memcpy(e->saved_shape, shape, sizeof shape);
+    e->saved_ndim = nd;
+    return out;
+}
+
+/* ops/elementwise.rs:199-211 add_backward, :558-571 sub_backward */
+static int addsub_backward(size_t grad, const orc_entry *e, long *out, int is_sub) {
+    orc_tensor *A = get(e->saved_ids[0]), *B = get(e->saved_ids[1]), *G = get(grad);
+    if (!A || !B || !G) { fail("tensor already freed"); return -1; }
+    size_t a_shape[ORC_MAX_DIMS], b_shape[ORC_MAX_DIMS], g_shape[ORC_MAX_DIMS];
+    int a_nd = A->ndim, b_nd = B->ndim, g_nd = G->ndim;
+    memcpy(a_shape, A->shape, sizeof a_shape);
+    memcpy(b_shape, B->shape, sizeof b_shape);
+    memcpy(g_shape, G->shape, sizeof g_shape);
+    size_t gsz = G->size;
+    float *gd = to_host(G);
+    float *ga = unbroadcast(gd, g_shape, g_nd, a_shape, a_nd);
+    if (is_sub) for (size_t i = 0; i < gsz; ++i) gd[i] = -gd[i];
+    float *gb = unbroadcast(gd, g_shape, g_nd, b_shape, b_nd);
+    free(gd);
+    out[0] = (long)from_vec(ga, a_shape, a_nd);
+    out[1] = (long)from_vec(gb, b_shape, b_nd);
+    return 0;
+}
+
+/* ops/elementwise.rs:348-390 mul_backward */
+static int mul_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *A = get(e->saved_ids[0]), *B = get(e->saved_ids[1]), *G = get(grad);
+    if (!A || !B || !G) { fail("tensor already freed"); return -1; }
+    size_t a_shape[ORC_MAX_DIMS], b_shape[ORC_MAX_DIMS], g_shape[ORC_MAX_DIMS];
+    int a_nd = A->ndim, b_nd = B->ndim, nd = G->ndim;
+    memcpy(a_shape, A->shape, sizeof a_shape);
+    memcpy(b_shape, B->shape, sizeof b_shape);
+    memcpy(g_shape, G->shape, sizeof g_shape);
+    float *ad = to_host(A), *bd = to_host(B), *gd = to_host(G);
+    size_t gsz = shape_size(g_shape, nd);
+    size_t ostr[ORC_MAX_DIMS], astr[ORC_MAX_DIMS], bstr[ORC_MAX_DIMS];
+    compute_strides(g_shape, nd, ostr);
+    compute_strides(a_shape, a_nd, astr);
+    compute_strides(b_shape, b_nd, bstr);
+    float *ga_full = (float *)calloc(gsz, sizeof(float));
+    float *gb_full = (float *)calloc(gsz, sizeof(float));
+    int a_off = nd - a_nd, b_off = nd - b_nd;
+    for (size_t i = 0; i < gsz; ++i) {
+        size_t coord[ORC_MAX_DIMS], rem = i;
+        for (int d = 0; d < nd; ++d) { coord[d] = rem / ostr[d]; rem %= ostr[d]; }
+        size_t ai = 0, bi = 0;
+        for (int d = 0; d < a_nd; ++d) ai += (a_shape[d] == 1 ? 0 : coord[d + a_off]) * astr[d];
+        for (int d = 0; d < b_nd; ++d) bi += (b_shape[d] == 1 ? 0 : coord[d + b_off]) * bstr[d];
+        ga_full[i] = gd[i] * bd[bi];
+        gb_full[i] = gd[i] * ad[ai];
+    }
+    float *ga = unbroadcast(ga_full, g_shape, nd, a_shape, a_nd);
+    float *gb = unbroadcast(gb_full, g_shape, nd, b_shape, b_nd);
+    free(ad); free(bd); free(gd); free(ga_full); free(gb_full);
+    out[0] = (long)from_vec(ga, a_shape, a_nd);
+    out[1] = (long)from_vec(gb, b_shape, b_nd);
+    return 0;
+}
+
+/* ---- unary ops ---------------------------------------------------------- */
+
+/* ops/activation.rs:15-18 gelu_scalar (tanh approximation) */
+static float gelu_scalar(float x) {
+    float s = sqrtf(2.0f / 3.14159265358979323846f);
+    return 0.5f * x * (1.0f + tanhf(s * (x + 0.044715f * x * x * x)));
+}
+/* ops/activation.rs:20-28 gelu_grad_scalar */
+static float gelu_grad_scalar(float x) {
+    float s = sqrtf(2.0f / 3.14159265358979323846f);
+    float inner = s * (x + 0.044715f * x * x * x);
+    float th = tanhf(inner);
+    float sech2 = 1.0f - th * th;
+    float d_inner = s * (1.0f + 3.0f * 0.044715f * x * x);
+    return 0.5f * (1.0f + th) + 0.5f * x * sech2 * d_inner;
+}
+
+/* ops/activation.rs:34-44 gelu_forward, :114-124 relu_forward;
+ * ops/elementwise.rs neg / mul_scalar (same map-over-to_host shape).
+ * kind: 0 relu, 1 gelu, 2 neg, 3 mul_scalar
+ * pinned by: test/nn.test.ts:17-27 relu/gelu anchors, f64 closed forms. */
+static uint32_t unary_op(size_t a, int kind, float s) {
+    orc_tensor *A = get(a);
+    if (!A) return fail("tensor already freed");
+    float *d = to_host(A);
+    for (size_t i = 0; i < A->size; ++i) {
+        float x = d[i];
+        d[i] = kind == 0 ? (x > 0.0f ? x : 0.0f) /* f32::max(x, 0.0) */
+             : kind == 1 ? gelu_scalar(x)
+             : kind == 2 ? -x : x * s;
+    }
+    size_t shape[ORC_MAX_DIMS]; int nd = A->ndim;
+    memcpy(shape, A->shape, sizeof shape);
+    size_t out = from_vec(d, shape, nd);
+    static const int ops[4] = {OP_RELU, OP_GELU, OP_NEG, OP_MULSCALAR};
+    orc_entry *e = tape_record(&g_tape, ops[kind], out, 1, a, 0);
+    e->saved_scalar = s;
+    return (uint32_t)out;
+}
+
+/* ops/activation.rs:74-84 gelu_backward, :154-164 relu_backward; neg and
+ * mul_scalar backward scale the grad. */
+static int unary_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *G = get(grad);
+    if (!G) { fail("tensor already freed"); return -1; }
+    float *gd = to_host(G);
+    size_t shape[ORC_MAX_DIMS]; int nd = G->ndim; size_t n = G->size;
+    memcpy(shape, G->shape, sizeof shape);
+    if (e->op == OP_RELU || e->op == OP_GELU) {
+        orc_tensor *X = get(e->saved_ids[0]);
+        if (!X) { free(gd); fail("tensor already freed"); return -1; }
+        float *xd = to_host(X);
+        for (size_t i = 0; i < n; ++i)
+            gd[i] = e->op == OP_RELU ? (xd[i] > 0.0f ? gd[i] : 0.0f) : gd[i] * gelu_grad_scalar(xd[i]);
+        free(xd);
+    } else if (e->op == OP_NEG) {
+        for (size_t i = 0; i < n; ++i) gd[i] = -gd[i];
+    } else {
+        for (size_t i = 0; i < n; ++i) gd[i] = gd[i] * e->saved_scalar;
+    }
+    out[0] = (long)from_vec(gd, shape, nd);
+    return 0;
+}
+
+/* ---- reductions --------------------------------------------------------- */
+
+/* ops/reduce.rs:5-7 resolve_dim */
+static int resolve_dim(int dim, int ndim) { return dim < 0 ? ndim + dim : dim; }
+
+/* ops/reduce.rs:13-46 sum along dim (kept as size 1), flat-order accumulation */
+static uint32_t sum_impl(size_t a, int dim, orc_tape *tp) {
+    orc_tensor *A = get(a);
+    if (!A) return fail("tensor already freed");
+    int nd = A->ndim;
+    int d = resolve_dim(dim, nd);
+    if (d < 0 || d >= nd) return fail("reduce dim out of range");
+    size_t a_shape[ORC_MAX_DIMS], out_shape[ORC_MAX_DIMS];
+    memcpy(a_shape, A->shape, sizeof a_shape);
+    memcpy(out_shape, A->shape, sizeof out_shape);
+    out_shape[d] = 1;
+    float *ad = to_host(A);
+    size_t out_size = shape_size(out_shape, nd);
+    float *out = (float *)calloc(out_size, sizeof(float));
+    size_t astr[ORC_MAX_DIMS], ostr[ORC_MAX_DIMS];
+    compute_strides(a_shape, nd, astr);
+    compute_strides(out_shape, nd, ostr);
+    size_t total = shape_size(a_shape, nd);
+    for (size_t i = 0; i < total; ++i) {
+        size_t oi = 0, rem = i;
+        for (int dd = 0; dd < nd; ++dd) {
+            size_t c = rem / astr[dd];
+            rem %= astr[dd];
+            oi += (dd == d ? 0 : c) * ostr[dd];
+        }
+        out[oi] += ad[i];
+    }
+    free(ad);
+    size_t out_id = from_vec(out, out_shape, nd);
+    orc_entry *e = tape_record(tp, OP_SUM, out_id, 1, a, 0);
+    memcpy(e->saved_shape, a_shape, sizeof a_shape);
+    e->saved_ndim = nd;
+    return (uint32_t)out_id;
+}
+
+/* ops/reduce.rs:169-184 mean = sum (recorded) then divide (recorded as Mean
+ * with the same input) */
+static uint32_t mean_impl(size_t a, int dim) {
+    orc_tensor *A = get(a);
+    if (!A) return fail("tensor already freed");
+    int nd = A->ndim;
+    int d = resolve_dim(dim, nd);
+    if (d < 0 || d >= nd) return fail("reduce dim out of range");
+    size_t a_shape[ORC_MAX_DIMS];
+    memcpy(a_shape, A->shape, sizeof a_shape);
+    float count = (float)a_shape[d];
+    uint32_t s = sum_impl(a, dim, &g_tape);
+    if (s == ORC_BAD) return s;
+    orc_tensor *S = get(s);
+    float *sd = to_host(S);
+    for (size_t i = 0; i < S->size; ++i) sd[i] = sd[i] / count;
+    size_t shape[ORC_MAX_DIMS]; int snd = S->ndim;
+    memcpy(shape, S->shape, sizeof shape);
+    size_t out = from_vec(sd, shape, snd);
+    orc_entry *e = tape_record(&g_tape, OP_MEAN, out, 1, a, 0);
+    memcpy(e->saved_shape, a_shape, sizeof a_shape);
+    e->saved_ndim = nd;
+    return (uint32_t)out;
+}
+
+/* ops/reduce.rs:94-118 sum_backward; :232-263 mean_backward (divisor = the
+ * LAST dim with grad 1 and orig > 1, else 1) */
+static int reduce_backward(size_t grad, const orc_entry *e, long *out, int is_mean) {
+    orc_tensor *G = get(grad);
+    if (!G) { fail("tensor already freed"); return -1; }
+    int nd = e->saved_ndim;
+    const size_t *orig = e->saved_shape;
+    size_t gshape[ORC_MAX_DIMS];
+    memcpy(gshape, G->shape, sizeof gshape);
+    float *gd = to_host(G);
+    size_t osz = shape_size(orig, nd);
+    size_t gstr[ORC_MAX_DIMS], ostr[ORC_MAX_DIMS];
+    compute_strides(gshape, G->ndim, gstr);
+    compute_strides(orig, nd, ostr);
+    float div = 1.0f;
+    if (is_mean)
+        for (int d = 0; d < nd; ++d)
+            if (gshape[d] == 1 && orig[d] > 1) div = (float)orig[d];
+    float *o = (float *)calloc(osz, sizeof(float));
+    for (size_t i = 0; i < osz; ++i) {
+        size_t gi = 0, rem = i;
+        for (int d = 0; d < nd; ++d) {
+            size_t c = rem / ostr[d];
+            rem %= ostr[d];
+            gi += (gshape[d] == 1 ? 0 : c) * gstr[d];
+        }
+        o[i] = is_mean ? gd[gi] / div : gd[gi];
+    }
+    free(gd);
+    out[0] = (long)from_vec(o, orig, nd);
+    return 0;
+}
+
+/* ---- layout ------------------------------------------------------------- */
+
+/* ops/layout.rs:66-77 view (always a copy) */
+static uint32_t view_impl(size_t a, const size_t *new_shape, int nd) {
+    orc_tensor *A = get(a);
+    if (!A) return fail("tensor already freed");
+    size_t orig[ORC_MAX_DIMS]; int ond = A->ndim;
+    memcpy(orig, A->shape, sizeof orig);
+    size_t a_id = ensure_contiguous(a);
+    float *d = to_host(get(a_id));
+    size_t out = from_vec(d, new_shape, nd);
+    orc_entry *e = tape_record(&g_tape, OP_VIEW, out, 1, a, 0);
+    memcpy(e->saved_shape, orig, sizeof orig);
+    e->saved_ndim = ond;
+    return (uint32_t)out;
+}
+
+/* ops/layout.rs:112-134 permute: cloned raw buffer + permuted shape/strides */
+static uint32_t permute_impl(size_t a, const size_t *dims, int nd) {
+    orc_tensor *A = get(a);
+    if (!A) return fail("tensor already freed");
+    if (nd != A->ndim) return fail("permute dims length mismatch");
+    size_t ns[ORC_MAX_DIMS], nst[ORC_MAX_DIMS], a_shape[ORC_MAX_DIMS];
+    memcpy(a_shape, A->shape, sizeof a_shape);
+    for (int i = 0; i < nd; ++i) {
+        if (dims[i] >= (size_t)nd) return fail("permute dim out of range");
+        ns[i] = A->shape[dims[i]];
+        nst[i] = A->strides[dims[i]];
+    }
+    size_t size = A->size;
+    float *d = (float *)malloc((size ? size : 1) * sizeof(float));
+    memcpy(d, A->data, size * sizeof(float));
+    size_t out = store_insert(d, ns, nst, nd, size);
+    orc_entry *e = tape_record(&g_tape, OP_PERMUTE, out, 1, a, 0);
+    memcpy(e->saved_shape, a_shape, sizeof a_shape);
+    e->saved_ndim = nd;
+    for (int i = 0; i < nd; ++i) e->saved_perm[i] = dims[i];
+    return (uint32_t)out;
+}
+
+/* ops/layout.rs:162-195 permute_backward: inverse-permutation scatter */
+static int permute_backward(size_t grad, const orc_entry *e, long *out) {
+    if (!get(grad)) { fail("tensor already freed"); return -1; }
+    int nd = e->saved_ndim;
+    size_t inv[ORC_MAX_DIMS];
+    for (int i = 0; i < nd; ++i) inv[e->saved_perm[i]] = (size_t)i;
+    size_t gc = ensure_contiguous(grad);
+    orc_tensor *G = get(gc);
+    float *d = to_host(G);
+    size_t sstr[ORC_MAX_DIMS], ostr[ORC_MAX_DIMS];
+    compute_strides(G->shape, nd, sstr);
+    compute_strides(e->saved_shape, nd, ostr);
+    size_t size = shape_size(G->shape, nd);
+    float *o = (float *)calloc(size, sizeof(float));
+    for (size_t i = 0; i < size; ++i) {
+        size_t coord[ORC_MAX_DIMS], rem = i;
+        for (int dd = 0; dd < nd; ++dd) { coord[dd] = rem / sstr[dd]; rem %= sstr[dd]; }
+        size_t oi = 0;
+        for (int dd = 0; dd < nd; ++dd) oi += coord[inv[dd]] * ostr[dd];
+        o[oi] = d[i];
+    }
+    free(d);
+    out[0] = (long)from_vec(o, e->saved_shape, nd);
+    return 0;
+}
+
+/* ops/layout.rs:92-97 view_backward */
+static int view_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *G = get(grad);
+    if (!G) { fail("tensor already freed"); return -1; }
+    float *d = to_host(G);
+    out[0] = (long)from_vec(d, e->saved_shape, e->saved_ndim);
+    return 0;
+}
+
+/* ---- loss --------------------------------------------------------------- */
+
+/* ops/loss.rs:24-67 cross_entropy, cpu arm (-ln p, no epsilon)
+ * pinned by: f64 log-softmax closed form; test/nn.test.ts:70-76 ordering. */
+static uint32_t cross_entropy_impl(size_t logits, const int64_t *targets, size_t nt) {
+    orc_tensor *L = get(logits);
+    if (!L) return fail("tensor already freed");
+    int nd = L->ndim;
+    if (nd < 1) return fail("cross_entropy needs at least 1 dim");
+    size_t shape[ORC_MAX_DIMS];
+    memcpy(shape, L->shape, sizeof shape);
+    size_t v = shape[nd - 1];
+    size_t n = shape_size(shape, nd) / v;
+    if (nt < n) return fail("index out of bounds: targets shorter than rows");
+    float *data = to_host(L);
+    float *sm = (float *)calloc((n * v) > 0 ? n * v : 1, sizeof(float));
+    float loss_sum = 0.0f;
+    for (size_t i = 0; i < n; ++i) {
+        size_t off = i * v;
+        float mx = -INFINITY;
+        for (size_t j = 0; j < v; ++j) mx = data[off + j] > mx ? data[off + j] : mx;
+        float sum = 0.0f;
+        for (size_t j = 0; j < v; ++j) {
+            float ex = expf(data[off + j] - mx);
+            sm[off + j] = ex;
+            sum += ex;
+        }
+        for (size_t j = 0; j < v; ++j) sm[off + j] /= sum;
+        if (targets[i] < 0 || (size_t)targets[i] >= v) {
+            free(data); free(sm);
+            return fail("index out of bounds: target class");
+        }
+        loss_sum += -logf(sm[off + (size_t)targets[i]]);
+    }
+    free(data);
+    float *lv = (float *)malloc(sizeof(float));
+    lv[0] = loss_sum / (float)n;
+    size_t one = 1;
+    size_t loss_id = from_vec(lv, &one, 1);
+    size_t sm_id = from_vec(sm, shape, nd);
+    orc_entry *e = tape_record(&g_tape, OP_CROSSENTROPY, loss_id, 1, logits, 0);
+    if (g_tape.enabled) {
+        e->targets = (size_t *)malloc((n ? n : 1) * sizeof(size_t));
+        for (size_t i = 0; i < n; ++i) e->targets[i] = (size_t)targets[i];
+    }
+    e->ce_n = n; e->ce_v = v; e->ce_sm = sm_id;
+    return (uint32_t)loss_id;
+}
+
+/* ops/loss.rs:131-149 cross_entropy_backward */
+static int cross_entropy_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *G = get(grad), *S = get(e->ce_sm);
+    if (!G || !S) { fail("tensor already freed"); return -1; }
+    float grad_val = G->data[0];
+    float *dl = to_host(S);
+    size_t shape[ORC_MAX_DIMS]; int nd = S->ndim;
+    memcpy(shape, S->shape, sizeof shape);
+    for (size_t i = 0; i < e->ce_n; ++i) {
+        size_t off = i * e->ce_v;
+        dl[off + e->targets[i]] -= 1.0f;
+        float scale = grad_val / (float)e->ce_n;
+        for (size_t j = 0; j < e->ce_v; ++j) dl[off + j] *= scale;
+    }
+    out[0] = (long)from_vec(dl, shape, nd);
+    return 0;
+}
+
+/* ---- backward ----------------------------------------------------------- */
+
+/* autograd.rs:180-222 dispatch_backward */
+static int dispatch_backward(const orc_entry *e, size_t grad, long *out) {
+    out[0] = out[1] = -1;
+    switch (e->op) {
+    case OP_ADD: return addsub_backward(grad, e, out, 0);
+    case OP_SUB: return addsub_backward(grad, e, out, 1);
+    case OP_MUL: return mul_backward(grad, e, out);
+    case OP_NEG: case OP_MULSCALAR: case OP_RELU: case OP_GELU: return unary_backward(grad, e, out);
+    case OP_MATMUL: return matmul_backward(grad, e, out);
+    case OP_SUM: return reduce_backward(grad, e, out, 0);
+    case OP_MEAN: return reduce_backward(grad, e, out, 1);
+    case OP_VIEW: return view_backward(grad, e, out);
+    case OP_PERMUTE: return permute_backward(grad, e, out);
+    case OP_CONTIGUOUS: out[0] = (long)grad; return 0; /* layout.rs:229-231 */
+    case OP_CROSSENTROPY: return cross_entropy_backward(grad, e, out);
+    }
+    return -1;
+}
+
+typedef struct {
+    const orc_entry *entries;
+    const long *out2entry;
+    const unsigned char *relevant;
+    unsigned char *visited;
+    size_t *order;
+    size_t norder;
+    size_t nslots;
+} dfs_ctx;
+
+/* autograd.rs:120-137 recursive post-order DFS */
+static void dfs(dfs_ctx *c, size_t tid) {
+    if (tid >= c->nslots || c->visited[tid]) return;
+    c->visited[tid] = 1;
+    long idx = c->out2entry[tid];
+    if (idx >= 0) {
+        const orc_entry *e = &c->entries[idx];
+        for (int i = 0; i < e->n_inputs; ++i)
+            if (e->input_ids[i] < c->nslots && c->relevant[e->input_ids[i]]) dfs(c, e->input_ids[i]);
+    }
+    c->order[c->norder++] = tid;
+}
+
+/* autograd.rs:96-171 Tape::backward.
+ * pinned by: gradient values of test/autograd.test.ts:19-46 in closed form,
+ * the shared-input case diff.mul(diff) -> 2*diff*g, end-to-end regression of
+ * test/module.test.ts:113-130 converging. */
+static int tape_backward(orc_tape *tp, size_t loss_id) {
+    if (!get(loss_id)) { fail("tensor already freed"); return -1; }
+    size_t nslots = g_store.len + 1;
+    long *out2entry = (long *)malloc(nslots * sizeof(long));
+    for (size_t i = 0; i < nslots; ++i) out2entry[i] = -1;
+    for (size_t i = 0; i < tp->len; ++i)
+        if (tp->e[i].output_id < nslots) out2entry[tp->e[i].output_id] = (long)i; /* later entry wins */
+
+    unsigned char *relevant = (unsigned char *)calloc(nslots, 1);
+    unsigned char *visited = (unsigned char *)calloc(nslots, 1);
+    size_t *stack = (size_t *)malloc((2 * tp->len + 2) * sizeof(size_t));
+    size_t sp = 0;
+    stack[sp++] = loss_id;
+    while (sp) {
+        size_t tid = stack[--sp];
+        if (tid >= nslots || relevant[tid]) continue;
+        relevant[tid] = 1;
+        long idx = out2entry[tid];
+        if (idx >= 0)
+            for (int i = 0; i < tp->e[idx].n_inputs; ++i) stack[sp++] = tp->e[idx].input_ids[i];
+    }
+    free(stack);
+
+    dfs_ctx c = {tp->e, out2entry, relevant, visited, (size_t *)malloc(nslots * sizeof(size_t)), 0, nslots};
+    dfs(&c, loss_id);
+
+    /* grads: tensor id -> grad id.  Backward creates tensors, so ids beyond
+     * nslots can appear as grad ids but never as keys. */
+    long *grads = (long *)malloc(nslots * sizeof(long));
+    for (size_t i = 0; i < nslots; ++i) grads[i] = -1;
+    {
+        orc_tensor *L = get(loss_id);
+        size_t shape[ORC_MAX_DIMS]; int nd = L->ndim;
+        memcpy(shape, L->shape, sizeof shape);
+        grads[loss_id] = (long)ones(shape, nd); /* ones_like for any shape, :143 */
+    }
+    int rc = 0;
+    for (size_t oi = c.norder; oi-- > 0 && rc == 0;) { /* reversed post-order */
+        size_t tid = c.order[oi];
+        if (grads[tid] < 0) continue;
+        long idx = out2entry[tid];
+        if (idx < 0) continue;
+        orc_entry e = tp->e[idx];
+        long ig[2];
+        if (dispatch_backward(&e, (size_t)grads[tid], ig) != 0) { rc = -1; break; }
+        for (int i = 0; i < e.n_inputs; ++i) {
+            if (ig[i] < 0) continue;
+            size_t inp = e.input_ids[i];
+            orc_tensor *T = get(inp);
+            if (!T) { fail("tensor already freed"); rc = -1; break; }
+            if (T->requires_grad) accumulate_grad(inp, (size_t)ig[i]);
+            if (inp < nslots && grads[inp] >= 0) add_inplace((size_t)grads[inp], (size_t)ig[i]);
+            else if (inp < nslots) grads[inp] = ig[i];
+        }
+    }
+    free(out2entry); free(relevant); free(visited); free(c.order); free(grads);
+    return rc;
+}
+
+/* ---- optimiser ---------------------------------------------------------- */
+
+/* ops/optimizer.rs:126-138 grad_norm: f64 accumulation, f32 sqrt */
+static float grad_norm_impl(const uint32_t *ids, size_t n) {
+    double sq = 0.0;
+    for (size_t p = 0; p < n; ++p) {
+        orc_tensor *T = get(ids[p]);
+        if (!T || T->grad < 0) continue;
+        orc_tensor *G = get((size_t)T->grad);
+        for (size_t i = 0; i < G->size; ++i) sq += (double)G->data[i] * (double)G->data[i];
+    }
+    return sqrtf((float)sq);
+}
+
+/* f32::powi: repeated multiplication (llvm.powi); exponentiation by squaring
+ * as compiler-rt's __powisf2 does. */
+static float powi_f32(float a, int b) {
+    int recip = b < 0;
+    float r = 1.0f;
+    while (1) {
+        if (b & 1) r *= a;
+        b /= 2;
+        if (b == 0) break;
+        a *= a;
+    }
+    return recip ? 1.0f / r : r;
+}
+
+/* ops/optimizer.rs:21-65 adamw_step, cpu arm
+ * pinned by: one-step closed form (first Adam step moves by lr*sign(g) up to
+ * eps), regression convergence. */
+static void adamw_step_impl(const uint32_t *ids, size_t n, float lr, float b1, float b2,
+                            float eps, float wd, uint32_t step) {
+    float bc1 = 1.0f - powi_f32(b1, (int)step);
+    float bc2 = 1.0f - powi_f32(b2, (int)step);
+    for (size_t p = 0; p < n; ++p) {
+        orc_tensor *T = get(ids[p]);
+        if (!T || T->grad < 0) continue;
+        size_t size = T->size;
+        float *gd = to_host(get((size_t)T->grad));
+        if (!T->adam_m) {
+            T->adam_m = (float *)calloc(size, sizeof(float));
+            T->adam_v = (float *)calloc(size, sizeof(float));
+        }
+        float *m = T->adam_m, *v = T->adam_v, *data = T->data;
+        for (size_t i = 0; i < size; ++i) {
+            float g = gd[i];
+            if (wd > 0.0f) data[i] *= 1.0f - lr * wd;
+            m[i] = b1 * m[i] + (1.0f - b1) * g;
+            v[i] = b2 * v[i] + (1.0f - b2) * g * g;
+            float m_hat = m[i] / bc1;
+            float v_hat = v[i] / bc2;
+            data[i] -= lr * m_hat / (sqrtf(v_hat) + eps);
+        }
+        free(gd);
+    }
+}
+
+/* ========================================================================= *
+ * Exported surface: one function per N-API export of src/native/src/lib.rs
+ * that the path's callers use (names follow lib.rs, prefixed orc_).
+ * ========================================================================= */
+
+static int conv_shape(const int64_t *shape, int nd, size_t *out) {
+    if (nd < 0 || nd > ORC_MAX_DIMS) { fail("too many dims"); return -1; }
+    for (int i = 0; i < nd; ++i) out[i] = (size_t)shape[i];
+    return 0;
+}
+
+uint32_t orc_zeros(const int64_t *shape, int nd) { /* lib.rs:45-50 */
+    size_t s[ORC_MAX_DIMS];
+    if (conv_shape(shape, nd, s)) return ORC_BAD;
+    return (uint32_t)zeros(s, nd);
+}
+uint32_t orc_ones(const int64_t *shape, int nd) { /* lib.rs:52-57 */
+    size_t s[ORC_MAX_DIMS];
+    if (conv_shape(shape, nd, s)) return ORC_BAD;
+    return (uint32_t)ones(s, nd);
+}
+/* lib.rs:73-78 from_float32 -> tensor.rs:252-261 from_slice */
+uint32_t orc_from_float32(const float *data, size_t len, const int64_t *shape, int nd) {
+    size_t s[ORC_MAX_DIMS];
+    if (conv_shape(shape, nd, s)) return ORC_BAD;
+    size_t n = shape_size(s, nd);
+    if (len < n) return fail("range end index out of range for slice");
+    float *d = (float *)malloc(n * sizeof(float));
+    memcpy(d, data, n * sizeof(float));
+    return (uint32_t)from_vec(d, s, nd);
+}
+int orc_tensor_shape(uint32_t id, int64_t *out, int cap) { /* lib.rs:80-84 */
+    orc_tensor *t = get(id);
+    if (!t) { fail("tensor already freed"); return -1; }
+    for (int i = 0; i < t->ndim && i < cap; ++i) out[i] = (int64_t)t->shape[i];
+    return t->ndim;
+}
+int64_t orc_tensor_size(uint32_t id) { /* lib.rs:86-90 */
+    orc_tensor *t = get(id);
+    if (!t) { fail("tensor already freed"); return -1; }
+    return (int64_t)t->size;
+}
+int orc_to_float32(uint32_t id, float *out, size_t cap) { /* lib.rs:92-97 */
+    orc_tensor *t = get(id);
+    if (!t) { fail("tensor already freed"); return -1; }
+    if (cap < t->size) { fail("output buffer too small"); return -1; }
+    float *d = to_host(t);
+    memcpy(out, d, t->size * sizeof(float));
+    free(d);
+    return 0;
+}
+int orc_get_scalar(uint32_t id, double *out) { /* lib.rs:99-103 */
+    orc_tensor *t = get(id);
+    if (!t) { fail("tensor already freed"); return -1; }
+    *out = (double)t->data[0];
+    return 0;
+}
+void orc_free_tensor(uint32_t id) { store_free(id); } /* lib.rs:105-109 */
+int orc_set_requires_grad(uint32_t id, int r) { /* lib.rs:115-119 */
+    orc_tensor *t = get(id);
+    if (!t) { fail("tensor already freed"); return -1; }
+    t->requires_grad = r;
+    return 0;
+}
+/* lib.rs:121-125 get_grad: 1 and *out when a grad exists, 0 when None */
+int orc_get_grad(uint32_t id, uint32_t *out) {
+    orc_tensor *t = get(id);
+    if (!t) { fail("tensor already freed"); return -1; }
+    if (t->grad < 0) return 0;
+    *out = (uint32_t)t->grad;
+    return 1;
+}
+/* lib.rs:131-137 backward: the tape is swapped for a fresh enabled one */
+int orc_backward(uint32_t loss) {
+    orc_tape old = g_tape;
+    g_tape.e = NULL; g_tape.len = g_tape.cap = 0; g_tape.enabled = 1;
+    int rc = tape_backward(&old, loss);
+    tape_clear(&old);
+    return rc;
+}
+int orc_zero_grad(const uint32_t *ids, size_t n) { /* lib.rs:139-146, tensor.rs:197-205 */
+    for (size_t p = 0; p < n; ++p) {
+        orc_tensor *t = get(ids[p]);
+        if (!t) { fail("tensor already freed"); return -1; }
+        if (t->grad >= 0) {
+            orc_tensor *g = get((size_t)t->grad);
+            if (!g) { fail("tensor already freed"); return -1; }
+            for (size_t i = 0; i < g->size; ++i) g->data[i] = 0.0f;
+        }
+    }
+    return 0;
+}
+void orc_no_grad_start(void) { g_tape.enabled = 0; } /* lib.rs:148-152 */
+void orc_no_grad_end(void) { g_tape.enabled = 1; }   /* lib.rs:154-158 */
+
+uint32_t orc_add(uint32_t a, uint32_t b) { return binary_op(a, b, 0); } /* lib.rs:164-169 */
+uint32_t orc_sub(uint32_t a, uint32_t b) { return binary_op(a, b, 1); } /* lib.rs:178-183 */
+uint32_t orc_mul(uint32_t a, uint32_t b) { return binary_op(a, b, 2); } /* lib.rs:171-176 */
+uint32_t orc_neg(uint32_t a) { return unary_op(a, 2, 0.0f); }            /* lib.rs:185-190 */
+uint32_t orc_mul_scalar(uint32_t a, double s) { return unary_op(a, 3, (float)s); } /* lib.rs:192-197 */
+uint32_t orc_matmul(uint32_t a, uint32_t b) { return matmul_impl(a, b, &g_tape); } /* lib.rs:199-204 */
+uint32_t orc_gelu(uint32_t a) { return unary_op(a, 1, 0.0f); }           /* lib.rs:206-211 */
+uint32_t orc_relu(uint32_t a) { return unary_op(a, 0, 0.0f); }           /* lib.rs:213-218 */
+uint32_t orc_sum_op(uint32_t a, int64_t dim) { return sum_impl(a, (int)dim, &g_tape); } /* lib.rs:234-239 */
+uint32_t orc_mean_op(uint32_t a, int64_t dim) { return mean_impl(a, (int)dim); }         /* lib.rs:241-246 */
+uint32_t orc_sum_all(uint32_t a) { /* lib.rs:255-265 */
+    orc_tensor *t = get(a);
+    if (!t) return fail("tensor already freed");
+    uint32_t cur = a;
+    for (int d = t->ndim - 1; d >= 0 && cur != ORC_BAD; --d) cur = sum_impl(cur, d, &g_tape);
+    return cur;
+}
+uint32_t orc_mean_all(uint32_t a) { /* lib.rs:267-277 */
+    orc_tensor *t = get(a);
+    if (!t) return fail("tensor already freed");
+    uint32_t cur = a;
+    for (int d = t->ndim - 1; d >= 0 && cur != ORC_BAD; --d) cur = mean_impl(cur, d);
+    return cur;
+}
+uint32_t orc_view(uint32_t a, const int64_t *shape, int nd) { /* lib.rs:279-285 */
+    size_t s[ORC_MAX_DIMS];
+    if (conv_shape(shape, nd, s)) return ORC_BAD;
+    return view_impl(a, s, nd);
+}
+uint32_t orc_permute(uint32_t a, const int64_t *dims, int nd) { /* lib.rs:287-293 */
+    size_t s[ORC_MAX_DIMS];
+    if (conv_shape(dims, nd, s)) return ORC_BAD;
+    return permute_impl(a, s, nd);
+}
+uint32_t orc_contiguous(uint32_t a) { /* lib.rs:295-300 -> layout.rs:218-227 */
+    if (!get(a)) return fail("tensor already freed");
+    size_t out = ensure_contiguous(a);
+    if (out != a) tape_record(&g_tape, OP_CONTIGUOUS, out, 1, a, 0);
+    return (uint32_t)out;
+}
+uint32_t orc_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n) { /* lib.rs:328-336 */
+    return cross_entropy_impl(logits, targets, n);
+}
+void orc_adamw_step(const uint32_t *ids, size_t n, double lr, double b1, double b2, double eps,
+                    double wd, int64_t step) { /* lib.rs:400-412 */
+    adamw_step_impl(ids, n, (float)lr, (float)b1, (float)b2, (float)eps, (float)wd, (uint32_t)step);
+}
+double orc_grad_norm(const uint32_t *ids, size_t n) { return (double)grad_norm_impl(ids, n); } /* lib.rs:414-419 */
+/* lib.rs:428-442 -> ops/optimizer.rs:224-245 clip_and_step */
+double orc_clip_and_step(const uint32_t *ids, size_t n, double lr, double b1, double b2, double eps,
+                         double wd, int64_t step, double max_grad_norm) {
+    float norm = grad_norm_impl(ids, n);
+    float mg = (float)max_grad_norm;
+    if (mg > 0.0f && norm > mg) {
+        float scale = mg / norm;
+        for (size_t p = 0; p < n; ++p) {
+            orc_tensor *T = get(ids[p]);
+            if (!T || T->grad < 0) continue;
+            orc_tensor *G = get((size_t)T->grad);
+            for (size_t i = 0; i < G->size; ++i) G->data[i] *= scale;
+        }
+    }
+    adamw_step_impl(ids, n, (float)lr, (float)b1, (float)b2, (float)eps, (float)wd, (uint32_t)step);
+    return (double)norm;
+}
+void orc_reset_engine(void) { /* lib.rs:460-468 */
+    for (size_t i = 0; i < g_store.len; ++i)
+        if (g_store.t[i].live) { free(g_store.t[i].data); free(g_store.t[i].adam_m); free(g_store.t[i].adam_v); }
+    free(g_store.t); free(g_store.free_ids);
+    memset(&g_store, 0, sizeof g_store);
+    tape_clear(&g_tape);
+}
+void orc_gc_tensors(const uint32_t *keep, size_t n) { /* lib.rs:693-706 */
+    size_t len = g_store.len;
+    unsigned char *k = (unsigned char *)calloc(len + 1, 1);
+    for (size_t i = 0; i < n; ++i) if (keep[i] < len) k[keep[i]] = 1;
+    for (size_t id = 0; id < len; ++id)
+        if (!k[id] && g_store.t[id].live) store_free(id);
+    free(k);
+    tape_clear(&g_tape);
+}
+
+/* Raw kernel-level check: C[M,N] = A[M,K] * B[K,N] with the reference's loop
+ * order and rounding, no store/tape/clones.  Used to pin the HIP GEMM on
+ * shapes where building tensors through the engine would only add copies.
+ * Same loop as ops/matmul.rs:62-69. */
+void orc_sgemm_ikj(const float *a, const float *b, float *c, size_t m, size_t n, size_t k) {
+    memset(c, 0, m * n * sizeof(float));
+    for (size_t i = 0; i < m; ++i)
+        for (size_t kk = 0; kk < k; ++kk) {
+            float a_val = a[i * k + kk];
+            const float *brow = b + kk * n;
+            float *crow = c + i * n;
+            for (size_t j = 0; j < n; ++j) crow[j] += a_val * brow[j];
+        }
+}
