@@ -1,0 +1,197 @@
+"""Host-side mirror of the reference's TypeScript API for the matmul path.
+
+`bind(native)` returns a namespace with Tensor, Linear, ReLU, Adam, mseLoss,
+crossEntropyLoss ... whose methods forward tensor ids to `native`, an object
+with the reference's N-API export names (src/tensor.ts, src/nn.ts,
+src/optimizer.ts, src/module.ts).  The default namespace of the package is
+bound to the HIP backend; tests bind a second one to the CPU oracle and run
+the same script against both.
+"""
+import math
+from types import SimpleNamespace
+
+import numpy as np
+
+
+def bind(native):
+    class Tensor:  # src/tensor.ts:9-252
+        def __init__(self, id, shape=None):
+            self._id = id
+            self._shape = list(shape) if shape is not None else [int(s) for s in native.tensorShape(id)]
+
+        @property
+        def shape(self):
+            return self._shape
+
+        @property
+        def size(self):
+            n = 1
+            for s in self._shape:
+                n *= s
+            return n
+
+        @property
+        def dims(self):
+            return len(self._shape)
+
+        # gradient
+        @property
+        def grad(self):
+            gid = native.getGrad(self._id)
+            return None if gid is None else Tensor(gid)
+
+        def backward(self):
+            native.backward(self._id)
+
+        def requiresGrad(self):
+            return native.getGrad(self._id) is not None
+
+        # data transfer
+        def toFloat32(self):
+            return native.toFloat32(self._id)
+
+        def item(self):
+            return native.getScalar(self._id)
+
+        def numpy(self):
+            return np.asarray(self.toFloat32(), dtype=np.float32).reshape(self._shape)
+
+        def free(self):
+            native.freeTensor(self._id)
+
+        # creation
+        @staticmethod
+        def fromFloat32(data, shape):
+            return Tensor(native.fromFloat32(np.asarray(data, dtype=np.float32), list(shape)), shape)
+
+        @staticmethod
+        def zeros(shape):
+            return Tensor(native.zeros(list(shape)), shape)
+
+        @staticmethod
+        def ones(shape):
+            return Tensor(native.ones(list(shape)), shape)
+
+        # elementwise (src/tensor.ts:101-133): a number becomes a [1] tensor for
+        # add/sub and a scalar multiply for mul
+        def add(self, other):
+            if isinstance(other, (int, float)):
+                other = Tensor.fromFloat32([other], [1])
+            return Tensor(native.add(self._id, other._id))
+
+        def sub(self, other):
+            if isinstance(other, (int, float)):
+                other = Tensor.fromFloat32([other], [1])
+            return Tensor(native.sub(self._id, other._id))
+
+        def mul(self, other):
+            if isinstance(other, (int, float)):
+                return Tensor(native.mulScalar(self._id, other))
+            return Tensor(native.mul(self._id, other._id))
+
+        def neg(self):
+            return Tensor(native.neg(self._id))
+
+        def relu(self):
+            return Tensor(native.relu(self._id))
+
+        def gelu(self):  # src/nn.ts gelu() -> native.gelu
+            return Tensor(native.gelu(self._id))
+
+        def sum(self, dim=None):
+            return Tensor(native.sumAll(self._id) if dim is None else native.sumOp(self._id, dim))
+
+        def mean(self, dim=None):
+            return Tensor(native.meanAll(self._id) if dim is None else native.meanOp(self._id, dim))
+
+        def view(self, *shape):
+            return Tensor(native.view(self._id, list(shape)))
+
+        def permute(self, *dims):
+            return Tensor(native.permute(self._id, list(dims)))
+
+        def contiguous(self):
+            return Tensor(native.contiguous(self._id))
+
+        def matmul(self, other):  # src/tensor.ts:207-209
+            return Tensor(native.matmul(self._id, other._id))
+
+        def setRequiresGrad(self, requires):
+            native.setRequiresGrad(self._id, requires)
+            return self
+
+    class Parameter:  # src/module.ts
+        def __init__(self, value):
+            self.value = value
+
+    class Module:
+        def parameters(self):
+            out = []
+            for v in self.__dict__.values():
+                if isinstance(v, Parameter):
+                    out.append(v)
+                elif isinstance(v, Module):
+                    out.extend(v.parameters())
+                elif isinstance(v, (list, tuple)):
+                    for m in v:
+                        if isinstance(m, Module):
+                            out.extend(m.parameters())
+            return out
+
+        def __call__(self, x):
+            return self.forward(x)
+
+    class Linear(Module):  # src/nn.ts:8-26: weight is [in, out], bound 1/sqrt(in) for both
+        def __init__(self, inFeatures, outFeatures, weight=None, bias=None, fused=False):
+            self.inFeatures, self.outFeatures = inFeatures, outFeatures
+            bound = 1.0 / math.sqrt(inFeatures)
+            if weight is None:
+                weight = np.random.uniform(-bound, bound, (inFeatures, outFeatures)).astype(np.float32)
+            if bias is None:
+                bias = np.random.uniform(-bound, bound, (outFeatures,)).astype(np.float32)
+            self.weight = Parameter(Tensor.fromFloat32(weight, [inFeatures, outFeatures]).setRequiresGrad(True))
+            self.bias = Parameter(Tensor.fromFloat32(bias, [outFeatures]).setRequiresGrad(True))
+            # opt-in fused path, feature-detected like the reference's cuda-only ops
+            self.fused = fused and hasattr(native, "linear")
+
+        def forward(self, x):
+            if self.fused:
+                return Tensor(native.linear(x._id, self.weight.value._id, self.bias.value._id))
+            return x.matmul(self.weight.value).add(self.bias.value)
+
+    class ReLU(Module):
+        def forward(self, x):
+            return x.relu()
+
+    class GELU(Module):
+        def forward(self, x):
+            return x.gelu()
+
+    def mseLoss(pred, target):  # src/nn.ts:161-165: mean(-1) twice
+        diff = pred.sub(target)
+        sq = diff.mul(diff)
+        return Tensor(native.meanOp(Tensor(native.meanOp(sq._id, -1))._id, -1))
+
+    def crossEntropyLoss(logits, targets):  # src/nn.ts:90-100
+        V = logits.shape[-1]
+        BT = logits.size // V
+        flat = logits.view(BT, V)
+        flat_targets = [int(t) for row in targets for t in (row if isinstance(row, (list, tuple, np.ndarray)) else [row])]
+        return Tensor(native.crossEntropyLoss(flat._id, flat_targets))
+
+    class Adam:  # src/optimizer.ts:33-70: options object, defaults lr 6e-4, beta2 0.95
+        def __init__(self, parameters, lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weightDecay=0.0):
+            self.parameters = list(parameters)
+            self.lr, self.beta1, self.beta2, self.eps, self.weightDecay = lr, beta1, beta2, eps, weightDecay
+            self.t = 0
+
+        def zeroGrad(self):
+            native.zeroGrad([p.value._id for p in self.parameters])
+
+        def step(self, maxGradNorm=0.0):
+            self.t += 1
+            ids = [p.value._id for p in self.parameters]
+            return native.clipAndStep(ids, self.lr, self.beta1, self.beta2, self.eps, self.weightDecay, self.t, maxGradNorm)
+
+    return SimpleNamespace(native=native, Tensor=Tensor, Parameter=Parameter, Module=Module, Linear=Linear, ReLU=ReLU,
+                           GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, Adam=Adam)

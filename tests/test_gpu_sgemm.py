@@ -1,0 +1,361 @@
+"""Kernel-level parity of mni_rocm_sgemm (through the C ABI) with the CPU
+oracle's i-k-j loop.  Integer-valued inputs must match bit for bit (any
+summation order is exact), normal inputs within
+1e-4 * sqrt(K) * max|a| * max|b|."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from framework_amd import native as N
+from framework_amd import synth
+from helpers import gemm_tol, max_err
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+class Dev:
+    """Device buffers freed at the end of a test."""
+
+    def __init__(self, r):
+        self.r, self.ptrs = r, []
+
+    def put(self, a):
+        p = self.r.to_device(a)
+        self.ptrs.append(p)
+        return p
+
+    def empty(self, n, fill=None):
+        p = self.r.malloc(max(n, 1) * 4)
+        self.ptrs.append(p)
+        if fill is not None:
+            self.r.fill(p, fill, n)
+        return p
+
+    def close(self):
+        for p in self.ptrs:
+            self.r.free(p)
+
+
+@pytest.fixture()
+def dev(rocm):
+    d = Dev(rocm)
+    yield d
+    d.close()
+
+
+def run_gemm(dev, a, b, ta=False, tb=False, **kw):
+    """a, b are the arrays as stored; op(A) = a.T when ta."""
+    r = dev.r
+    batch = a.shape[0] if a.ndim == 3 else 1
+    a3 = a.reshape((batch,) + a.shape[-2:])
+    b3 = b.reshape((-1,) + b.shape[-2:])
+    M, K = (a3.shape[2], a3.shape[1]) if ta else (a3.shape[1], a3.shape[2])
+    Nn = b3.shape[1] if tb else b3.shape[2]
+    batch = max(a3.shape[0], b3.shape[0])
+    dA, dB = dev.put(a3), dev.put(b3)
+    dC = dev.empty(batch * M * Nn, fill=-7.0)
+    r.sgemm(M, Nn, K, dA, dB, dC, batch=batch,
+            a_strides=(1, a3.shape[2]) if ta else (a3.shape[2], 1),
+            b_strides=(1, b3.shape[2]) if tb else (b3.shape[2], 1),
+            a_batch=(a3.shape[1] * a3.shape[2], a3.shape[0]), b_batch=(b3.shape[1] * b3.shape[2], b3.shape[0]), **kw)
+    return r.to_host(dC, (batch, M, Nn))
+
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (17, 63, 65), (64, 64, 16), (128, 128, 32), (129, 127, 33), (256, 384, 160), (1000, 300, 200)]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_mfma_integer_exact_all_layouts(dev, m, n, k, ta, tb):
+    a = synth.small_ints(m + k, (k, m) if ta else (m, k), 4)
+    b = synth.small_ints(n + k, (n, k) if tb else (k, n), 4, stream=1)
+    got = run_gemm(dev, a, b, ta, tb, algo=N.ALGO_MFMA)[0]
+    want = ((a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(np.float32)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 48, 96), (300, 200, 1000), (512, 512, 512)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_mfma_normal_inputs_vs_oracle(dev, oracle_native, m, n, k, ta, tb):
+    a = synth.normal(m, (k, m) if ta else (m, k))
+    b = synth.normal(n, (n, k) if tb else (k, n), stream=1)
+    got = run_gemm(dev, a, b, ta, tb, algo=N.ALGO_MFMA)[0]
+    want = oracle_native.sgemm_ikj(a.T if ta else a, b.T if tb else b)
+    assert max_err(got, want) <= gemm_tol(k, a, b)
+
+
+def test_golden_cases(dev):
+    with open(os.path.join(GOLDEN, "matmul_cases.json")) as f:
+        cases = json.load(f)["cases"]
+    for c in cases:
+        gen = (lambda s, sh, st: synth.small_ints(s, sh, 4, st)) if c["kind"] == "int" else (lambda s, sh, st: synth.normal(s, sh, 1.0, st))
+        a, b = gen(c["seed"], (c["m"], c["k"]), 0), gen(c["seed"], (c["k"], c["n"]), 1)
+        want = np.array(c["out"], dtype=np.float32).reshape(c["m"], c["n"])
+        for algo in (N.ALGO_AUTO, N.ALGO_MFMA):
+            got = run_gemm(dev, a, b, algo=algo)[0]
+            if c["kind"] == "int":
+                assert np.array_equal(got, want), (c["seed"], algo)
+            else:
+                assert max_err(got, want) <= gemm_tol(c["k"], a, b), (c["seed"], algo)
+
+
+@pytest.mark.parametrize("split", [2, 3, 7, 16])
+def test_split_k_equals_unsplit(dev, split):
+    a = synth.small_ints(1, (1000, 200), 4)  # stored K x M: TN like a weight gradient
+    b = synth.small_ints(2, (1000, 130), 4, stream=1)
+    base = run_gemm(dev, a, b, ta=True, algo=N.ALGO_MFMA, split_k=1)[0]
+    got = run_gemm(dev, a, b, ta=True, algo=N.ALGO_MFMA, split_k=split)[0]
+    assert np.array_equal(got, base)
+    an, bn = synth.normal(3, (4096, 96)), synth.normal(4, (4096, 80), stream=1)
+    base = run_gemm(dev, an, bn, ta=True, algo=N.ALGO_MFMA, split_k=1)[0]
+    got = run_gemm(dev, an, bn, ta=True, algo=N.ALGO_MFMA, split_k=split)[0]
+    assert max_err(got, base) <= gemm_tol(4096, an, bn)
+
+
+def test_auto_split_k_on_tall_k(dev, oracle_native):
+    a = synth.normal(5, (8192, 128))
+    b = synth.normal(5, (8192, 256), stream=1)
+    got = run_gemm(dev, a, b, ta=True)[0]  # 2 tiles only: the planner must split
+    want = oracle_native.sgemm_ikj(a.T, b)
+    assert max_err(got, want) <= gemm_tol(8192, a, b)
+
+
+def test_batched_and_batch_broadcast(dev):
+    a = synth.small_ints(1, (5, 70, 40), 4)
+    b = synth.small_ints(2, (5, 40, 90), 4, stream=1)
+    got = run_gemm(dev, a, b, algo=N.ALGO_MFMA)
+    assert np.array_equal(got, np.matmul(a.astype(np.int64), b.astype(np.int64)).astype(np.float32))
+    w = synth.small_ints(3, (1, 40, 90), 4, stream=2)  # batch_count 1: reused by every batch
+    got = run_gemm(dev, a, w, algo=N.ALGO_MFMA)
+    assert np.array_equal(got, np.matmul(a.astype(np.int64), w.astype(np.int64)).astype(np.float32))
+
+
+def test_batch_modulo_rule(dev, rocm):
+    # operand batch index = b % batch_count (src/native/src/ops/matmul.rs:55-56)
+    a = synth.small_ints(1, (2, 8, 6), 4)
+    b = synth.small_ints(2, (3, 6, 5), 4, stream=1)
+    dA, dB, dC = dev.put(a), dev.put(b), dev.empty(6 * 8 * 5)
+    rocm.sgemm(8, 5, 6, dA, dB, dC, batch=6, a_batch=(48, 2), b_batch=(30, 3), algo=N.ALGO_MFMA)
+    got = rocm.to_host(dC, (6, 8, 5))
+    for i in range(6):
+        assert np.array_equal(got[i], a[i % 2] @ b[i % 3])
+
+
+def test_arbitrary_strides_and_unaligned_pointers(dev, rocm):
+    big_a = synth.small_ints(1, (2 * 37, 2 * 29 + 1), 4)
+    big_b = synth.small_ints(2, (3 * 29, 3 * 41 + 2), 4, stream=1)
+    a = big_a[::2, 1::2][:37, :29]   # row stride 2*ld, col stride 2, offset 1 element
+    b = big_b[::3, 2::3][:29, :41]
+    dA, dB, dC = dev.put(big_a), dev.put(big_b), dev.empty(37 * 41)
+    rocm.sgemm(37, 41, 29, dA + 4, dB + 8, dC, a_strides=(2 * big_a.shape[1], 2), b_strides=(3 * big_b.shape[1], 3))
+    assert np.array_equal(rocm.to_host(dC, (37, 41)), (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+    # contiguous but based 4 bytes off a 16-byte boundary, odd leading dimension
+    a2 = synth.small_ints(3, (130 * 131 + 1,), 4)
+    b2 = synth.small_ints(4, (131 * 129 + 1,), 4, stream=1)
+    dA, dB, dC = dev.put(a2), dev.put(b2), dev.empty(130 * 129)
+    rocm.sgemm(130, 129, 131, dA + 4, dB + 4, dC)
+    want = a2[1:].reshape(130, 131).astype(np.int64) @ b2[1:].reshape(131, 129).astype(np.int64)
+    assert np.array_equal(rocm.to_host(dC, (130, 129)), want.astype(np.float32))
+
+
+@pytest.mark.parametrize("algo", [N.ALGO_MFMA, N.ALGO_SKINNY])
+@pytest.mark.parametrize("epi", [N.EPI_BIAS, N.EPI_BIAS_RELU, N.EPI_BIAS_GELU])
+def test_bias_epilogues(dev, rocm, algo, epi):
+    m = 130 if algo == N.ALGO_MFMA else 7
+    a = synth.small_ints(1, (m, 64), 3)
+    b = synth.small_ints(2, (64, 256), 3, stream=1)
+    bias = synth.small_ints(3, (256,), 3, stream=2)
+    dbias = dev.put(bias)
+    got = run_gemm(dev, a, b, algo=algo, bias=dbias, epilogue=epi)[0]
+    z = (a.astype(np.int64) @ b.astype(np.int64) + bias.astype(np.int64)).astype(np.float64)
+    if epi == N.EPI_BIAS:
+        assert np.array_equal(got, z.astype(np.float32))
+    elif epi == N.EPI_BIAS_RELU:
+        assert np.array_equal(got, np.maximum(z, 0).astype(np.float32))
+    else:
+        want = 0.5 * z * (1 + np.tanh(np.sqrt(2 / np.pi) * (z + 0.044715 * z ** 3)))
+        assert max_err(got, want) <= 1e-5 * max(1.0, np.abs(z).max())
+    # split-K applies the epilogue once, in the reduction
+    if algo == N.ALGO_MFMA:
+        got2 = run_gemm(dev, a, b, algo=algo, bias=dbias, epilogue=epi, split_k=2)[0]
+        assert max_err(got2, got) <= 1e-6 * max(1.0, np.abs(z).max())
+
+
+def test_accumulate(dev, rocm):
+    a = synth.small_ints(1, (100, 50), 3)
+    b = synth.small_ints(2, (50, 60), 3, stream=1)
+    c0 = synth.small_ints(3, (100, 60), 3, stream=2)
+    dA, dB, dC = dev.put(a), dev.put(b), dev.put(c0)
+    rocm.sgemm(100, 60, 50, dA, dB, dC, accumulate=True, algo=N.ALGO_MFMA)
+    assert np.array_equal(rocm.to_host(dC, (100, 60)), c0 + (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+
+
+def test_ldc_padding_is_untouched(dev, rocm):
+    a = synth.small_ints(1, (33, 20), 3)
+    b = synth.small_ints(2, (20, 45), 3, stream=1)
+    dA, dB = dev.put(a), dev.put(b)
+    dC = dev.empty(33 * 64, fill=-7.0)
+    rocm.sgemm(33, 45, 20, dA, dB, dC, ldc=64, algo=N.ALGO_MFMA)
+    got = rocm.to_host(dC, (33, 64))
+    assert np.array_equal(got[:, :45], (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+    assert np.all(got[:, 45:] == -7.0)
+
+
+def test_empty_and_zero_k(dev, rocm):
+    dC = dev.empty(12, fill=5.0)
+    rocm.sgemm(3, 4, 0, None, None, dC)  # K = 0: an empty sum
+    assert np.all(rocm.to_host(dC, (3, 4)) == 0.0)
+    rocm.sgemm(0, 4, 3, None, None, None)  # nothing to do
+    rocm.sgemm(3, 0, 3, None, None, None)
+
+
+# ---- skinny kernels ----------------------------------------------------------------
+
+@pytest.mark.parametrize("m", [1, 2, 4, 5, 8, 13, 16])
+def test_skinny_cols_integer_exact(dev, m):
+    a = synth.small_ints(m, (m, 700), 4)
+    b = synth.small_ints(m + 1, (700, 520), 4, stream=1)
+    got = run_gemm(dev, a, b, algo=N.ALGO_SKINNY)[0]
+    assert np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+    for split in (1, 3):
+        got = run_gemm(dev, a, b, algo=N.ALGO_SKINNY, split_k=split)[0]
+        assert np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+
+
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_skinny_dots_integer_exact(dev, m):
+    a = synth.small_ints(m, (m, 1024), 4)
+    bt = synth.small_ints(m + 1, (300, 1024), 4, stream=1)  # B stored as its transpose: K contiguous
+    got = run_gemm(dev, a, bt, tb=True, algo=N.ALGO_SKINNY)[0]
+    assert np.array_equal(got, (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float32))
+
+
+def test_skinny_few_output_columns(dev):
+    # [rows, K] x [K, 4]: the few columns become the skinny side (C^T = B^T A^T)
+    at = synth.small_ints(1, (64, 1000), 4)  # A stored K x M
+    b = synth.small_ints(2, (64, 4), 4, stream=1)
+    got = run_gemm(dev, at, b, ta=True, algo=N.ALGO_SKINNY)[0]
+    assert np.array_equal(got, (at.T.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+    a = synth.small_ints(3, (1000, 64), 4)
+    bt = synth.small_ints(4, (4, 64), 4, stream=1)
+    got = run_gemm(dev, a, bt, tb=True, algo=N.ALGO_SKINNY)[0]
+    assert np.array_equal(got, (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float32))
+
+
+def test_skinny_batched_and_vs_oracle(dev, oracle_native):
+    a = synth.normal(1, (3, 2, 4096), 0.02)
+    w = synth.normal(2, (1, 4096, 512), 0.02, stream=1)
+    got = run_gemm(dev, a, w, algo=N.ALGO_SKINNY)
+    for i in range(3):
+        assert max_err(got[i], oracle_native.sgemm_ikj(a[i], w[0])) <= gemm_tol(4096, a, w)
+
+
+def test_skinny_ineligible_is_an_error_only_when_forced(dev, rocm):
+    a = synth.small_ints(1, (40, 30), 3)
+    b = synth.small_ints(2, (30, 50), 3, stream=1)
+    with pytest.raises(N.MniError, match="not eligible"):
+        run_gemm(dev, a, b, algo=N.ALGO_SKINNY)
+    a = synth.small_ints(1, (3, 30), 3)
+    b = synth.small_ints(2, (30, 50), 3, stream=1)  # N % 4 != 0: auto falls back to MFMA
+    got = run_gemm(dev, a, b)[0]
+    assert np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+
+
+# ---- argument checking: status codes, never an abort --------------------------------------
+
+def test_invalid_arguments_are_reported(dev, rocm):
+    dC = dev.empty(16)
+    dA = dev.put(np.zeros((4, 4), np.float32))
+    with pytest.raises(N.MniError, match="negative"):
+        rocm.sgemm(-1, 4, 4, dA, dA, dC)
+    with pytest.raises(N.MniError, match="ldc"):
+        rocm.sgemm(4, 4, 4, dA, dA, dC, ldc=2)
+    with pytest.raises(N.MniError, match="null"):
+        rocm.sgemm(4, 4, 4, None, dA, dC)
+    with pytest.raises(N.MniError, match="bias"):
+        rocm.sgemm(4, 4, 4, dA, dA, dC, epilogue=N.EPI_BIAS)
+    with pytest.raises(N.MniError, match="batch_count"):
+        rocm.sgemm(4, 4, 4, dA, dA, dC, a_batch=(0, 0))
+
+
+# ---- support kernels of the C ABI ----------------------------------------------------------
+
+def test_strided_copy_add_bias_colsum_axpy_fill(dev, rocm):
+    x = synth.normal(1, (3, 40, 50))
+    src = dev.put(x)
+    dst = dev.empty(x.size)
+    rocm.strided_copy(dst, src, [3, 50, 40], [2000, 1, 50])  # swap last two dims
+    assert np.array_equal(rocm.to_host(dst, (3, 50, 40)), x.transpose(0, 2, 1))
+    rocm.strided_copy(dst, src, [50, 3, 40], [1, 2000, 50])  # general permutation
+    assert np.array_equal(rocm.to_host(dst, (50, 3, 40)), x.transpose(2, 0, 1))
+    a = synth.small_ints(2, (300, 96), 5)
+    bias = synth.small_ints(3, (96,), 5, stream=1)
+    da, db, out = dev.put(a), dev.put(bias), dev.empty(a.size)
+    rocm.add_bias(out, da, db, 300, 96)
+    assert np.array_equal(rocm.to_host(out, (300, 96)), a + bias)
+    cs = dev.empty(96)
+    rocm.colsum(cs, da, 300, 96)
+    assert np.array_equal(rocm.to_host(cs, (96,)), a.sum(0))
+    big = synth.normal(4, (5000, 33))
+    dbig, cs2 = dev.put(big), dev.empty(33)
+    rocm.colsum(cs2, dbig, 5000, 33)
+    assert max_err(rocm.to_host(cs2, (33,)), big.astype(np.float64).sum(0)) <= gemm_tol(5000, big, np.ones(1))
+    rocm.axpy(out, da, 2.0, a.size)
+    assert np.array_equal(rocm.to_host(out, (300, 96)), a + bias + 2 * a)
+    rocm.fill(out, 3.5, 7)
+    assert np.all(rocm.to_host(out, (7,)) == 3.5)
+
+
+# ---- benchmark configurations at full size ---------------------------------------------------
+
+def _check_rows(got_rows, stats, K, amax, bmax):
+    tol = 1e-4 * np.sqrt(K) * amax * bmax
+    for row, st in zip(got_rows, stats):
+        assert max_err(row[:8], st["head"]) <= tol
+        # |sum of N errors| <= N * tol
+        assert abs(float(row.astype(np.float64).sum()) - st["sum"]) <= tol * row.size
+        assert abs(float((row.astype(np.float64) ** 2).sum()) - st["sumsq"]) <= 2 * tol * np.abs(row).max() * row.size
+
+
+def test_config2_4096_cubed(dev, rocm, oracle_native):
+    with open(os.path.join(GOLDEN, "config_samples.json")) as f:
+        gold = json.load(f)["config2"]
+    a = synth.normal(1, (4096, 4096))
+    b = synth.normal(1, (4096, 4096), stream=1)
+    got = run_gemm(dev, a, b)[0]
+    _check_rows(got[gold["rows"]], gold["stats"], 4096, np.abs(a).max(), np.abs(b).max())
+    # live oracle on another 16 rows, every element
+    rows = list(range(1000, 1016))
+    assert max_err(got[rows], oracle_native.sgemm_ikj(a[rows], b)) <= gemm_tol(4096, a, b)
+    # C 1 = A (B 1) in float64: touches every element of C
+    ones = np.ones(4096)
+    lhs = got.astype(np.float64) @ ones
+    rhs = a.astype(np.float64) @ (b.astype(np.float64) @ ones)
+    assert np.max(np.abs(lhs - rhs)) <= 4096 * gemm_tol(4096, a, b)
+
+
+def test_config5a_decode_gemv(dev, rocm):
+    with open(os.path.join(GOLDEN, "config_samples.json")) as f:
+        gold = json.load(f)["config5a"]
+    x = synth.normal(4, (4, 4096), 0.02)
+    w = synth.normal(4, (4096, 4096), 0.02, stream=1)
+    got = run_gemm(dev, x, w)[0]
+    _check_rows(got, gold["stats"], 4096, np.abs(x).max(), np.abs(w).max())
+    want = x.astype(np.float64) @ w.astype(np.float64)
+    assert max_err(got, want) <= gemm_tol(4096, x, w)
+
+
+def test_config5b_tall_k_weight_gradient(dev, rocm):
+    with open(os.path.join(GOLDEN, "config_samples.json")) as f:
+        gold = json.load(f)["config5b"]
+    X = synth.normal(5, (65536, 1024))
+    dY = synth.normal(5, (65536, 1024), stream=1)
+    got = run_gemm(dev, X, dY, ta=True)[0]  # X^T as a view: strides (1, 1024)
+    _check_rows(got[gold["rows"]], gold["stats"], 65536, np.abs(X).max(), np.abs(dY).max())
+    # a sampled block in float64
+    rows, cols = slice(100, 116), slice(900, 932)
+    want = X[:, rows].astype(np.float64).T @ dY[:, cols].astype(np.float64)
+    assert max_err(got[rows, cols], want) <= gemm_tol(65536, X, dY)
