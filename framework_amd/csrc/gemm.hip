@@ -91,19 +91,22 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
                             s.x_cs == 1 && (s.x_rs % 4) == 0 && aligned16(s.X) && x_batch_ok;
 
         if (w_cols) {
-            // Enough workgroups to keep every CU streaming: aim at ~4 per CU.
+            // Slice K until about 4 workgroups per CU exist (every CU streams,
+            // nearly all of W is requested at once); a slice is a whole number
+            // of workgroup passes.
             const int groups = (s.cols + skinny_cols_block_cols() - 1) / skinny_cols_block_cols();
+            const int pass = skinny_cols_rows_per_pass();
             int split = d.split_k;
             if (split == 0) {
                 const int64_t target = 4LL * (ctx().compute_units > 0 ? ctx().compute_units : 256);
                 const int64_t have = (int64_t)groups * s.batch;
                 split = (int)((target + have - 1) / have);
-                const int max_split = (s.K + 63) / 64;  // at least 64 K rows per slice
+                const int max_split = (s.K + pass - 1) / pass;
                 if (split > max_split) split = max_split;
                 if (split < 1) split = 1;
             }
             int kps = (s.K + split - 1) / split;
-            kps = (kps + 31) & ~31;
+            kps = (kps + pass - 1) / pass * pass;
             split = (s.K + kps - 1) / kps;
             s.split_k = split; s.k_per_slice = kps;
             void *ws = nullptr;
@@ -114,9 +117,14 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
                 s.ws = (float *)ws;
             }
             *rc = launch_skinny_cols(s);
-            if (*rc == MNI_OK && split > 1)
-                *rc = finish_split(s.ws, s.out, s.bias, split, s.batch, s.rows, s.cols, s.o_rs, s.o_cs, s.o_bs,
-                                   s.epilogue, s.accumulate, s.bias_on_rows);
+            if (*rc == MNI_OK && split > 1) {
+                ReduceLaunch r;
+                r.ws = s.ws; r.out = s.out; r.bias = s.bias;
+                r.slices = split; r.batch = s.batch; r.rows = s.rows; r.cols = s.cols;
+                r.o_rs = s.o_rs; r.o_cs = s.o_cs; r.o_bs = s.o_bs;
+                r.epilogue = s.epilogue; r.accumulate = s.accumulate; r.bias_on_rows = s.bias_on_rows;
+                *rc = launch_skinny_reduce(r);
+            }
             if (ws) dev_free(ws);
             return true;
         }

@@ -45,11 +45,12 @@ struct SkinnyLaunch {
     int split_k, k_per_slice;
     int epilogue, accumulate, bias_on_rows;
 };
-// W with unit stride along j (cols): lanes own columns, K split over waves.
+// W with unit stride along j (cols): lanes own columns, K split over wavefronts and slices.
 int launch_skinny_cols(const SkinnyLaunch &s);
 // W with unit stride along k: one wavefront per output column, shuffle reduce.
 int launch_skinny_dots(const SkinnyLaunch &s);
 int skinny_cols_block_cols();
+int skinny_cols_rows_per_pass();  // K rows one workgroup covers per trip
 
 // Sums split-K partials ws[slice][batch][rows][cols] in slice order and
 // applies the epilogue; out addressed with (o_bs, o_rs, o_cs).
@@ -62,5 +63,6 @@ struct ReduceLaunch {
     int epilogue, accumulate, bias_on_rows;
 };
 int launch_splitk_reduce(const ReduceLaunch &r);
+int launch_skinny_reduce(const ReduceLaunch &r);  // few outputs, many slices
 
 }  // namespace mni
