@@ -42,6 +42,13 @@ static constexpr int PAD = 2;               // float4 of padding per K-quad slic
 static constexpr int SLICE = BM + PAD;      // float4 per K-quad slice
 static constexpr int NTHREADS = 256;
 
+// Row r of a tile sits at float4 slot r ^ ((r >> 4) & 3) of its K-quad slice.
+// Within an aligned group of 16 rows this is a permutation, so the MFMA operand
+// reads (16 consecutive rows per LDS pass) stay conflict-free; it spreads the
+// 16 rows 4*j + i that the micro-tile stores write in one pass over all 16
+// bank groups (they would otherwise collide four ways).
+__device__ __forceinline__ int lds_row(int r) { return r ^ ((r >> 4) & 3); }
+
 // ---- global -> register loads ---------------------------------------------
 // Register layout LAYOUT 0 (K contiguous): thread owns float4 #(tid + 256 i),
 //   i = 0..3, where float4 #f is row f/8, K quad f%8.
@@ -108,14 +115,14 @@ __device__ __forceinline__ void store_lds(float4 *__restrict__ tile, int tid, co
         for (int i = 0; i < 4; ++i) {
             int f = tid + NTHREADS * i;
             int row = f >> 3, q = f & 7;
-            tile[q * SLICE + row] = v[i];
+            tile[q * SLICE + lds_row(row)] = v[i];
         }
     } else {
         int r4 = tid & 31, q = tid >> 5;
-        tile[q * SLICE + 4 * r4 + 0] = make_float4(v[0].x, v[1].x, v[2].x, v[3].x);
-        tile[q * SLICE + 4 * r4 + 1] = make_float4(v[0].y, v[1].y, v[2].y, v[3].y);
-        tile[q * SLICE + 4 * r4 + 2] = make_float4(v[0].z, v[1].z, v[2].z, v[3].z);
-        tile[q * SLICE + 4 * r4 + 3] = make_float4(v[0].w, v[1].w, v[2].w, v[3].w);
+        tile[q * SLICE + lds_row(4 * r4 + 0)] = make_float4(v[0].x, v[1].x, v[2].x, v[3].x);
+        tile[q * SLICE + lds_row(4 * r4 + 1)] = make_float4(v[0].y, v[1].y, v[2].y, v[3].y);
+        tile[q * SLICE + lds_row(4 * r4 + 2)] = make_float4(v[0].z, v[1].z, v[2].z, v[3].z);
+        tile[q * SLICE + lds_row(4 * r4 + 3)] = make_float4(v[0].w, v[1].w, v[2].w, v[3].w);
     }
 }
 
@@ -220,32 +227,60 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_mfma_kernel(const GemmLaunch
     __syncthreads();
 
     const int r = lane & 31, h = lane >> 5;
+    // float4 slots of this lane's two A row blocks and two B column blocks
+    const int a_row0 = lds_row(wm * 64 + r), a_row1 = lds_row(wm * 64 + 32 + r);
+    const int b_row0 = lds_row(wn * 64 + r), b_row1 = lds_row(wn * 64 + 32 + r);
+    constexpr int NCHUNK = KQ / 2;  // chunks of 8 K values: 16 MFMAs each
+
+    // One chunk = 8 K values = 16 MFMAs in 4 groups of 4 (group j uses element
+    // j of each operand float4).  The four ds_read_b128 of the NEXT chunk are
+    // issued after the first three groups, and in the last chunk of a step the LDS
+    // writes of the next stage take their place, so LDS traffic is spread under
+    // the MFMAs instead of bunching up in front of a wait.  sched_barrier keeps
+    // the compiler from regrouping them.
+    float4 fa0, fa1, fb0, fb1;     // fragments in use
+    float4 na0, na1, nb0, nb1;     // fragments of the next chunk
+    auto mfma4 = [&](int j) {
+        const float a0 = j == 0 ? fa0.x : j == 1 ? fa0.y : j == 2 ? fa0.z : fa0.w;
+        const float a1 = j == 0 ? fa1.x : j == 1 ? fa1.y : j == 2 ? fa1.z : fa1.w;
+        const float b0 = j == 0 ? fb0.x : j == 1 ? fb0.y : j == 2 ? fb0.z : fb0.w;
+        const float b1 = j == 0 ? fb1.x : j == 1 ? fb1.y : j == 2 ? fb1.z : fb1.w;
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    };
+
     for (int kt = 0; kt < nkt; ++kt) {
         const int cur = kt & 1;
         const bool more = kt + 1 < nkt;
-        if (more) load_tiles(kt + 1);
+        if (more) load_tiles(kt + 1);  // global loads of the next K step fly during this step's MFMAs
 
-        const float4 *__restrict__ As = lds[cur][0] + wm * 64 + r;
-        const float4 *__restrict__ Bs = lds[cur][1] + wn * 64 + r;
+        const float4 *As = lds[cur][0], *Bs = lds[cur][1];
+        fa0 = As[h * SLICE + a_row0]; fa1 = As[h * SLICE + a_row1];
+        fb0 = Bs[h * SLICE + b_row0]; fb1 = Bs[h * SLICE + b_row1];
 #pragma unroll
-        for (int c = 0; c < KQ / 2; ++c) {
-            const int q = 2 * c + h;
-            const float4 a0 = As[q * SLICE], a1 = As[q * SLICE + 32];
-            const float4 b0 = Bs[q * SLICE], b1 = Bs[q * SLICE + 32];
-            const float av0[4] = {a0.x, a0.y, a0.z, a0.w}, av1[4] = {a1.x, a1.y, a1.z, a1.w};
-            const float bv0[4] = {b0.x, b0.y, b0.z, b0.w}, bv1[4] = {b1.x, b1.y, b1.z, b1.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv0[j], acc[0][0], 0, 0, 0);
-                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[j], bv1[j], acc[0][1], 0, 0, 0);
-                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv0[j], acc[1][0], 0, 0, 0);
-                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[j], bv1[j], acc[1][1], 0, 0, 0);
-            }
-        }
-
-        if (more) {
-            store_lds<AL>(lds[cur ^ 1][0], tid, ra);
-            store_lds<BL>(lds[cur ^ 1][1], tid, rb);
+        for (int c = 0; c < NCHUNK; ++c) {
+            const bool last = c == NCHUNK - 1;
+            const int qn = (2 * (c + 1) + h) * SLICE;
+            __builtin_amdgcn_sched_barrier(0);
+            mfma4(0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) { na0 = As[qn + a_row0]; na1 = As[qn + a_row1]; }
+            else if (more) store_lds<AL>(lds[cur ^ 1][0], tid, ra);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma4(1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) nb0 = Bs[qn + b_row0];
+            else if (more) store_lds<BL>(lds[cur ^ 1][1], tid, rb);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma4(2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) nb1 = Bs[qn + b_row1];
+            __builtin_amdgcn_sched_barrier(0);
+            mfma4(3);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) { fa0 = na0; fa1 = na1; fb0 = nb0; fb1 = nb1; }
         }
         __syncthreads();
     }
