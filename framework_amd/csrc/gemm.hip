@@ -35,7 +35,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_SKINNY)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_MFMA_SMALL)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -149,7 +149,19 @@ static int run_mfma(const mni_gemm_desc &d) {
     g.a_bcount = (int)d.A.batch_count; g.b_bcount = (int)d.B.batch_count;
     g.ldc = d.ldc; g.c_bs = d.c_batch_stride;
     g.epilogue = d.epilogue; g.accumulate = d.accumulate;
-    const int bm = gemm_mfma_tile_m(), bn = gemm_mfma_tile_n(), bk = gemm_mfma_tile_k();
+    // Tile shape: 128 x 128 for dense products; a 64-wide side when that
+    // extent is at most 64 (no half-empty tiles), and 64 x 64 when K is short
+    // and 128 x 128 tiles would leave the machine with few, short-lived
+    // workgroups (small tiles: 4 resident per CU, cheaper prologue/epilogue).
+    const int bk = gemm_mfma_tile_k();
+    const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
+    int bm = g.M <= 64 ? 64 : 128, bn = g.N <= 64 ? 64 : 128;
+    if (d.algo == MNI_ALGO_MFMA_SMALL) {
+        bm = bn = 64;
+    } else if (d.algo == MNI_ALGO_AUTO) {
+        const int64_t big_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
+        if (g.K <= 256 && big_tiles < 4LL * cus) bm = bn = 64;
+    }
     g.tiles_m = (g.M + bm - 1) / bm;
     g.tiles_n = (g.N + bn - 1) / bn;
 
@@ -164,7 +176,7 @@ static int run_mfma(const mni_gemm_desc &d) {
     const int ktiles = (g.K + bk - 1) / bk;
     if (split == 0) {
         const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * g.batch;
-        const int64_t slots = 2LL * (ctx().compute_units > 0 ? ctx().compute_units : 256);
+        const int64_t slots = (bm * bn >= 128 * 128 ? 2LL : 4LL) * cus;
         split = 1;
         if (tiles * 4 < slots * 3) {
             split = (int)((slots + tiles - 1) / tiles);
@@ -185,7 +197,7 @@ static int run_mfma(const mni_gemm_desc &d) {
         MNI_TRY(dev_alloc(&ws, bytes));
         g.ws = (float *)ws;
     }
-    int rc = launch_gemm_mfma(g, amode, bmode);
+    int rc = launch_gemm_mfma(g, amode, bmode, bm, bn);
     if (rc == MNI_OK && split > 1)
         rc = finish_split(g.ws, g.C, g.bias, split, g.batch, g.M, g.N, g.ldc, 1, g.c_bs, g.epilogue, g.accumulate, 0);
     if (ws) dev_free(ws);
@@ -196,7 +208,7 @@ int sgemm(const mni_gemm_desc &d) {
     MNI_TRY(ensure_init());
     MNI_TRY(validate(d));
     if (d.M == 0 || d.N == 0 || d.batch == 0) return MNI_OK;
-    if (d.algo != MNI_ALGO_MFMA) {
+    if (d.algo == MNI_ALGO_AUTO || d.algo == MNI_ALGO_SKINNY) {
         int rc;
         if (try_skinny(d, &rc)) return rc;
         if (d.algo == MNI_ALGO_SKINNY)

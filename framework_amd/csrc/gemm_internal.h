@@ -23,9 +23,8 @@ struct GemmLaunch {
     int epilogue, accumulate;
 };
 
-int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode);
-int gemm_mfma_tile_m();
-int gemm_mfma_tile_n();
+// tile_m, tile_n in {128, 64}; g.tiles_m / g.tiles_n count tiles of that size
+int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int tile_n);
 int gemm_mfma_tile_k();
 
 // Skinny (GEMV-shaped) products: X (MR x K, MR <= 16) against a large W.

@@ -8,10 +8,13 @@
 //
 // Tiling.  A workgroup of 256 threads (4 wavefronts, 2 x 2) owns a 128 x 128
 // tile of C and walks K in steps of 32.  Each wavefront owns 64 x 64 as 2 x 2
-// blocks of v_mfma_f32_32x32x2_f32 (16 accumulator VGPRs per block).  Tiles are
-// staged through LDS, double-buffered, one barrier per K step: while the MFMAs
-// of step t run out of LDS stage t&1, the global loads of step t+1 are in
-// flight into registers and are written to the other stage afterwards.
+// blocks of v_mfma_f32_32x32x2_f32 (16 accumulator VGPRs per block).  Narrow
+// or short-K products use 64-wide tile sides (one MFMA block per wavefront along
+// that side) from the same template.  Tiles are
+// staged through LDS, double-buffered, one barrier per K step.  Global loads
+// run a full K step ahead: the registers that carried tile t+1 into LDS during
+// the last MFMAs of step t are refilled with tile t+2 right away, so a load has
+// a whole step of MFMAs to land before it is needed.
 //
 // LDS layout.  Both operand tiles are stored "K-quad major":
 //     tile[k/4][row][k%4]        (row = m for A, n for B; one float4 per row)
@@ -36,10 +39,9 @@ namespace mni {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-static constexpr int BM = 128, BN = 128, BK = 32;
+static constexpr int BK = 32;
 static constexpr int KQ = BK / 4;           // K quads per tile
 static constexpr int PAD = 2;               // float4 of padding per K-quad slice
-static constexpr int SLICE = BM + PAD;      // float4 per K-quad slice
 static constexpr int NTHREADS = 256;
 
 // Row r of a tile sits at float4 slot r ^ ((r >> 4) & 3) of its K-quad slice.
@@ -50,37 +52,42 @@ static constexpr int NTHREADS = 256;
 __device__ __forceinline__ int lds_row(int r) { return r ^ ((r >> 4) & 3); }
 
 // ---- global -> register loads ---------------------------------------------
+// A tile side has ROWS = 128 or 64 rows (m for A, n for B) and BK = 32 K values.
 // Register layout LAYOUT 0 (K contiguous): thread owns float4 #(tid + 256 i),
-//   i = 0..3, where float4 #f is row f/8, K quad f%8.
+//   i < ROWS/32, where float4 #f is row f/8, K quad f%8.
 // Register layout LAYOUT 1 (M/N contiguous): thread owns the 4 x 4 micro-tile
-//   rows 4*(tid%32)..+3, K quad tid/32; v[j] holds k = 4*quad + j across the
-//   four rows.
+//   rows 4*(tid % (ROWS/4))..+3, K quad tid / (ROWS/4) (threads whose quad is
+//   >= 8 own nothing: half of them when ROWS = 64); v[j] holds k = 4*quad + j
+//   across the four rows.
 
-template <int LAYOUT>
+template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t ld, int tid, float4 (&v)[4]) {
     if (LAYOUT == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < ROWS / 32; ++i) {
             int f = tid + NTHREADS * i;
             int row = f >> 3, q = f & 7;
             v[i] = *reinterpret_cast<const float4 *>(p + (int64_t)row * ld + 4 * q);
         }
     } else {
-        int r4 = tid & 31, q = tid >> 5;
+        constexpr int R4 = ROWS / 4;
+        int r4 = tid % R4, q = tid / R4;
+        if (q < KQ) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            v[j] = *reinterpret_cast<const float4 *>(p + 4 * r4 + (int64_t)(4 * q + j) * ld);
+            for (int j = 0; j < 4; ++j)
+                v[j] = *reinterpret_cast<const float4 *>(p + 4 * r4 + (int64_t)(4 * q + j) * ld);
+        }
     }
 }
 
 // Guarded element-wise load: element (row, k) lives at p[row * rs + k * cs];
 // rows >= rmax or k >= kmax read as zero.
-template <int LAYOUT>
+template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void load_guarded(const float *__restrict__ p, int64_t rs, int64_t cs, int rmax,
                                              int kmax, int tid, float4 (&v)[4]) {
     if (LAYOUT == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < ROWS / 32; ++i) {
             int f = tid + NTHREADS * i;
             int row = f >> 3, q = f & 7;
             float t[4];
@@ -92,37 +99,44 @@ __device__ __forceinline__ void load_guarded(const float *__restrict__ p, int64_
             v[i] = make_float4(t[0], t[1], t[2], t[3]);
         }
     } else {
-        int r4 = tid & 31, q = tid >> 5;
+        constexpr int R4 = ROWS / 4;
+        int r4 = tid % R4, q = tid / R4;
+        if (q < KQ) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            int k = 4 * q + j;
-            float t[4];
+            for (int j = 0; j < 4; ++j) {
+                int k = 4 * q + j;
+                float t[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                int row = 4 * r4 + e;
-                t[e] = (row < rmax && k < kmax) ? p[(int64_t)row * rs + (int64_t)k * cs] : 0.0f;
+                for (int e = 0; e < 4; ++e) {
+                    int row = 4 * r4 + e;
+                    t[e] = (row < rmax && k < kmax) ? p[(int64_t)row * rs + (int64_t)k * cs] : 0.0f;
+                }
+                v[j] = make_float4(t[0], t[1], t[2], t[3]);
             }
-            v[j] = make_float4(t[0], t[1], t[2], t[3]);
         }
     }
 }
 
 // ---- register -> LDS --------------------------------------------------------
-template <int LAYOUT>
+template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void store_lds(float4 *__restrict__ tile, int tid, const float4 (&v)[4]) {
+    constexpr int SLICE = ROWS + PAD;
     if (LAYOUT == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < ROWS / 32; ++i) {
             int f = tid + NTHREADS * i;
             int row = f >> 3, q = f & 7;
             tile[q * SLICE + lds_row(row)] = v[i];
         }
     } else {
-        int r4 = tid & 31, q = tid >> 5;
-        tile[q * SLICE + lds_row(4 * r4 + 0)] = make_float4(v[0].x, v[1].x, v[2].x, v[3].x);
-        tile[q * SLICE + lds_row(4 * r4 + 1)] = make_float4(v[0].y, v[1].y, v[2].y, v[3].y);
-        tile[q * SLICE + lds_row(4 * r4 + 2)] = make_float4(v[0].z, v[1].z, v[2].z, v[3].z);
-        tile[q * SLICE + lds_row(4 * r4 + 3)] = make_float4(v[0].w, v[1].w, v[2].w, v[3].w);
+        constexpr int R4 = ROWS / 4;
+        int r4 = tid % R4, q = tid / R4;
+        if (q < KQ) {
+            tile[q * SLICE + lds_row(4 * r4 + 0)] = make_float4(v[0].x, v[1].x, v[2].x, v[3].x);
+            tile[q * SLICE + lds_row(4 * r4 + 1)] = make_float4(v[0].y, v[1].y, v[2].y, v[3].y);
+            tile[q * SLICE + lds_row(4 * r4 + 2)] = make_float4(v[0].z, v[1].z, v[2].z, v[3].z);
+            tile[q * SLICE + lds_row(4 * r4 + 3)] = make_float4(v[0].w, v[1].w, v[2].w, v[3].w);
+        }
     }
 }
 
@@ -132,13 +146,26 @@ __device__ __forceinline__ float gelu_tanh(float x) {
     return 0.5f * x * (1.0f + tanhf(s * (x + 0.044715f * x * x * x)));
 }
 
+__device__ __forceinline__ float pick(const float4 &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
+
 // MODE: 0 = K axis contiguous + 16-byte aligned, 1 = M/N axis contiguous +
 // aligned, 2 = arbitrary strides (always guarded scalar loads, layout 0).
-template <int AMODE, int BMODE>
-__global__ __launch_bounds__(NTHREADS, 2) void gemm_mfma_kernel(const GemmLaunch g) {
+// TM x TN: 32 x 32 MFMA blocks per wavefront; the workgroup tile is
+// (64 TM) x (64 TN): 128 x 128 for the dense case, 64-wide sides for narrow or
+// short-K products where smaller tiles waste less and fill the machine better.
+template <int AMODE, int BMODE, int TM, int TN>
+__global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_kernel(const GemmLaunch g) {
     constexpr int AL = AMODE == 1 ? 1 : 0;
     constexpr int BL = BMODE == 1 ? 1 : 0;
-    __shared__ float4 lds[2][2][KQ * SLICE];
+    constexpr int BM = 64 * TM, BN = 64 * TN;
+    constexpr int SLICE_A = BM + PAD, SLICE_B = BN + PAD;
+    // One LDS block: two stages of the A tile, two of the B tile; the epilogue
+    // reuses it to turn the MFMA accumulator layout into row-contiguous 16-byte
+    // stores.
+    constexpr int STAGE_A = KQ * SLICE_A, STAGE_B = KQ * SLICE_B;
+    __shared__ float4 lds[2 * STAGE_A + 2 * STAGE_B];
+    auto stage_a = [&](int st) -> float4 * { return lds + st * STAGE_A; };
+    auto stage_b = [&](int st) -> float4 * { return lds + 2 * STAGE_A + st * STAGE_B; };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -190,105 +217,130 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_mfma_kernel(const GemmLaunch
     const int64_t a_ld = AMODE == 0 ? g.a_rs : g.a_cs;
     const int64_t b_ld = BMODE == 0 ? g.b_cs : g.b_rs;
 
-    floatx16 acc[2][2];
+    floatx16 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
     float4 ra[4], rb[4];
 
-    auto load_tiles = [&](int kt) {
+    auto load_a = [&](int kt) {  // A tile: rows = m, element (m, k) at Ap[m * a_rs + k * a_cs]
         const int k0 = kt * BK;
         const int krem = klen - k0;
-        // A tile: rows = m, element (m, k) at Ap[m * a_rs + k * a_cs]
         if (a_full && krem >= BK) {
-            if (AMODE == 0) load_fast<0>(Ap + (int64_t)k0, a_ld, tid, ra);
-            else load_fast<1>(Ap + (int64_t)k0 * a_ld, a_ld, tid, ra);
+            if (AMODE == 0) load_fast<0, BM>(Ap + (int64_t)k0, a_ld, tid, ra);
+            else load_fast<1, BM>(Ap + (int64_t)k0 * a_ld, a_ld, tid, ra);
         } else {
-            load_guarded<AL>(Ap + (int64_t)k0 * g.a_cs, g.a_rs, g.a_cs, mrem, krem, tid, ra);
+            load_guarded<AL, BM>(Ap + (int64_t)k0 * g.a_cs, g.a_rs, g.a_cs, mrem, krem, tid, ra);
         }
-        // B tile: rows = n, element (n, k) at Bp[n * b_cs + k * b_rs]
+    };
+    auto load_b = [&](int kt) {  // B tile: rows = n, element (n, k) at Bp[n * b_cs + k * b_rs]
+        const int k0 = kt * BK;
+        const int krem = klen - k0;
         if (b_full && krem >= BK) {
-            if (BMODE == 0) load_fast<0>(Bp + (int64_t)k0, b_ld, tid, rb);
-            else load_fast<1>(Bp + (int64_t)k0 * b_ld, b_ld, tid, rb);
+            if (BMODE == 0) load_fast<0, BN>(Bp + (int64_t)k0, b_ld, tid, rb);
+            else load_fast<1, BN>(Bp + (int64_t)k0 * b_ld, b_ld, tid, rb);
         } else {
-            load_guarded<BL>(Bp + (int64_t)k0 * g.b_rs, g.b_cs, g.b_rs, nrem, krem, tid, rb);
+            load_guarded<BL, BN>(Bp + (int64_t)k0 * g.b_rs, g.b_cs, g.b_rs, nrem, krem, tid, rb);
         }
     };
 
+    // Prologue: tile 0 goes to LDS stage 0, tile 1 into the staging registers.
     if (nkt > 0) {
-        load_tiles(0);
-        store_lds<AL>(lds[0][0], tid, ra);
-        store_lds<BL>(lds[0][1], tid, rb);
+        load_a(0);
+        load_b(0);
+        store_lds<AL, BM>(stage_a(0), tid, ra);
+        store_lds<BL, BN>(stage_b(0), tid, rb);
+        if (nkt > 1) { load_a(1); load_b(1); }
     }
     __syncthreads();
 
     const int r = lane & 31, h = lane >> 5;
-    // float4 slots of this lane's two A row blocks and two B column blocks
-    const int a_row0 = lds_row(wm * 64 + r), a_row1 = lds_row(wm * 64 + 32 + r);
-    const int b_row0 = lds_row(wn * 64 + r), b_row1 = lds_row(wn * 64 + 32 + r);
-    constexpr int NCHUNK = KQ / 2;  // chunks of 8 K values: 16 MFMAs each
+    // float4 slots of this lane's A row blocks and B column blocks
+    int a_row[TM], b_row[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a_row[i] = lds_row(wm * (32 * TM) + 32 * i + r);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b_row[j] = lds_row(wn * (32 * TN) + 32 * j + r);
+    constexpr int NCHUNK = KQ / 2;  // chunks of 8 K values
 
-    // One chunk = 8 K values = 16 MFMAs in 4 groups of 4 (group j uses element
-    // j of each operand float4).  The four ds_read_b128 of the NEXT chunk are
-    // issued after the first three groups, and in the last chunk of a step the LDS
+    // One chunk = 8 K values = 4 groups of TM x TN MFMAs (group j uses element
+    // j of each operand float4).  The ds_read_b128 of the NEXT chunk are issued
+    // after the first three groups, and in the last chunk of a step the LDS
     // writes of the next stage take their place, so LDS traffic is spread under
     // the MFMAs instead of bunching up in front of a wait.  sched_barrier keeps
     // the compiler from regrouping them.
-    float4 fa0, fa1, fb0, fb1;     // fragments in use
-    float4 na0, na1, nb0, nb1;     // fragments of the next chunk
-    auto mfma4 = [&](int j) {
-        const float a0 = j == 0 ? fa0.x : j == 1 ? fa0.y : j == 2 ? fa0.z : fa0.w;
-        const float a1 = j == 0 ? fa1.x : j == 1 ? fa1.y : j == 2 ? fa1.z : fa1.w;
-        const float b0 = j == 0 ? fb0.x : j == 1 ? fb0.y : j == 2 ? fb0.z : fb0.w;
-        const float b1 = j == 0 ? fb1.x : j == 1 ? fb1.y : j == 2 ? fb1.z : fb1.w;
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    float4 fa[TM], fb[TN];  // fragments in use
+    float4 na[TM], nb[TN];  // fragments of the next chunk
+    auto mfma_group = [&](int j) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int jj = 0; jj < TN; ++jj)
+                acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(pick(fa[i], j), pick(fb[jj], j), acc[i][jj], 0, 0, 0);
     };
 
     for (int kt = 0; kt < nkt; ++kt) {
         const int cur = kt & 1;
         const bool more = kt + 1 < nkt;
-        if (more) load_tiles(kt + 1);  // global loads of the next K step fly during this step's MFMAs
+        const bool more2 = kt + 2 < nkt;
 
-        const float4 *As = lds[cur][0], *Bs = lds[cur][1];
-        fa0 = As[h * SLICE + a_row0]; fa1 = As[h * SLICE + a_row1];
-        fb0 = Bs[h * SLICE + b_row0]; fb1 = Bs[h * SLICE + b_row1];
+        const float4 *As = stage_a(cur), *Bs = stage_b(cur);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = As[h * SLICE_A + a_row[i]];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = Bs[h * SLICE_B + b_row[j]];
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const bool last = c == NCHUNK - 1;
-            const int qn = (2 * (c + 1) + h) * SLICE;
+            const int qa = (2 * (c + 1) + h) * SLICE_A, qb = (2 * (c + 1) + h) * SLICE_B;
             __builtin_amdgcn_sched_barrier(0);
-            mfma4(0);
+            mfma_group(0);
             __builtin_amdgcn_sched_barrier(0);
-            if (!last) { na0 = As[qn + a_row0]; na1 = As[qn + a_row1]; }
-            else if (more) store_lds<AL>(lds[cur ^ 1][0], tid, ra);
+            if (!last) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) na[i] = As[qa + a_row[i]];
+            } else if (more) {
+                // The staging registers hold tile kt+1 (requested a whole K step
+                // ago); once they are in LDS they are refilled with tile kt+2.
+                store_lds<AL, BM>(stage_a(cur ^ 1), tid, ra);
+                if (more2) load_a(kt + 2);
+            }
             __builtin_amdgcn_sched_barrier(0);
-            mfma4(1);
+            mfma_group(1);
             __builtin_amdgcn_sched_barrier(0);
-            if (!last) nb0 = Bs[qn + b_row0];
-            else if (more) store_lds<BL>(lds[cur ^ 1][1], tid, rb);
+            if (!last) nb[0] = Bs[qb + b_row[0]];
+            else if (more) {
+                store_lds<BL, BN>(stage_b(cur ^ 1), tid, rb);
+                if (more2) load_b(kt + 2);
+            }
             __builtin_amdgcn_sched_barrier(0);
-            mfma4(2);
+            mfma_group(2);
             __builtin_amdgcn_sched_barrier(0);
-            if (!last) nb1 = Bs[qn + b_row1];
+            if (!last && TN > 1) nb[TN - 1] = Bs[qb + b_row[TN - 1]];
             __builtin_amdgcn_sched_barrier(0);
-            mfma4(3);
+            mfma_group(3);
             __builtin_amdgcn_sched_barrier(0);
-            if (!last) { fa0 = na0; fa1 = na1; fb0 = nb0; fb1 = nb1; }
+            if (!last) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[i] = na[i];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) fb[j] = nb[j];
+            }
         }
         __syncthreads();
     }
 
     // ---- epilogue -----------------------------------------------------------
     // A 32 x 32 MFMA block leaves lane l with column l%32 and rows
-    // 8*(e/4) + 4*(l/32) + e%4, e = 0..15: each store instruction writes two
-    // runs of 32 consecutive floats.
+    // 8*(e/4) + 4*(l/32) + e%4, e = 0..15.  Storing that directly costs one
+    // 4-byte store per value; instead every wavefront passes its 32-row strips
+    // through a private LDS patch and writes them back out as 16-byte stores
+    // along the rows (4x fewer store instructions, which is what bounds
+    // short-K, output-heavy products).
     float *__restrict__ Cb;
     int64_t ldc;
     const bool partial = g.split_k > 1;
@@ -299,52 +351,90 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_mfma_kernel(const GemmLaunch
         Cb = g.C + (int64_t)batch * g.c_bs;
         ldc = g.ldc;
     }
+    constexpr int WN = 32 * TN;          // columns of a wavefront's strip
+    constexpr int PW = WN + 4;           // patch row pitch in floats (16-byte multiple)
+    constexpr int LANES_PER_ROW = WN / 4;
+    constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+    float *patch = reinterpret_cast<float *>(lds) + wave * (32 * PW);
+    const int prow = lane / LANES_PER_ROW, pc4 = lane % LANES_PER_ROW;
+    const int col = n0 + wn * WN + 4 * pc4;
+    const bool vec_ok = partial ? ((g.N & 3) == 0)
+                                : ((ldc & 3) == 0 && (g.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(g.C) & 15) == 0);
+    float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (!partial && g.epilogue != MNI_EPI_NONE) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int col = n0 + wn * 64 + j * 32 + r;
-        const bool col_ok = col < g.N;
-        float bias = 0.0f;
-        if (!partial && g.epilogue != MNI_EPI_NONE && col_ok) bias = g.bias[col];
+        for (int e = 0; e < 4; ++e)
+            if (col + e < g.N) bias4[e] = g.bias[col + e];
+    }
+    // all wavefronts are past their last LDS read (barrier at the end of the K loop)
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int row_base = m0 + wm * 64 + i * 32 + 4 * h;
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int row = row_base + 8 * (e >> 2) + (e & 3);
-                if (col_ok && row < g.M) {
-                    float v = acc[i][j][e];
-                    float *dst = Cb + (int64_t)row * ldc + col;
-                    if (!partial) {
-                        v += bias;
-                        if (g.epilogue == MNI_EPI_BIAS_RELU) v = fmaxf(v, 0.0f);
-                        else if (g.epilogue == MNI_EPI_BIAS_GELU) v = gelu_tanh(v);
-                        if (g.accumulate) v += *dst;
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) patch[(8 * (e >> 2) + 4 * h + (e & 3)) * PW + 32 * j + r] = acc[i][j][e];
+        __syncthreads();
+#pragma unroll
+        for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
+            const int lr = prow + ROWS_PER_PASS * pass;
+            const int row = m0 + wm * (32 * TM) + 32 * i + lr;
+            const float4 t = *reinterpret_cast<const float4 *>(patch + lr * PW + 4 * pc4);
+            float v[4] = {t.x, t.y, t.z, t.w};
+            if (row < g.M && col < g.N) {
+                float *dst = Cb + (int64_t)row * ldc + col;
+                if (!partial) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] += bias4[e];
+                        if (g.epilogue == MNI_EPI_BIAS_RELU) v[e] = fmaxf(v[e], 0.0f);
+                        else if (g.epilogue == MNI_EPI_BIAS_GELU) v[e] = gelu_tanh(v[e]);
                     }
-                    *dst = v;
+                }
+                if (vec_ok && col + 3 < g.N) {
+                    if (!partial && g.accumulate) {
+                        const float4 c = *reinterpret_cast<const float4 *>(dst);
+                        v[0] += c.x; v[1] += c.y; v[2] += c.z; v[3] += c.w;
+                    }
+                    *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (col + e < g.N) dst[e] = (!partial && g.accumulate) ? v[e] + dst[e] : v[e];
+                    }
                 }
             }
         }
+        __syncthreads();
     }
 }
 
-int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode) {
-    const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * g.batch * g.split_k;
-    if (blocks <= 0) return MNI_OK;
-    if (blocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "sgemm: too many tiles (%lld)", (long long)blocks);
-    dim3 grid((unsigned)blocks), block(NTHREADS);
+template <int TM, int TN>
+static void launch_modes(const GemmLaunch &g, int amode, int bmode, dim3 grid) {
+    dim3 block(NTHREADS);
     hipStream_t s = ctx().stream;
-#define MNI_LAUNCH(AM, BMO) hipLaunchKernelGGL((gemm_mfma_kernel<AM, BMO>), grid, block, 0, s, g)
+#define MNI_LAUNCH(AM, BMO) hipLaunchKernelGGL((gemm_mfma_kernel<AM, BMO, TM, TN>), grid, block, 0, s, g)
     if (amode == 2 || bmode == 2) MNI_LAUNCH(2, 2);
     else if (amode == 0 && bmode == 0) MNI_LAUNCH(0, 0);
     else if (amode == 0 && bmode == 1) MNI_LAUNCH(0, 1);
     else if (amode == 1 && bmode == 0) MNI_LAUNCH(1, 0);
     else MNI_LAUNCH(1, 1);
 #undef MNI_LAUNCH
+}
+
+// tile_m / tile_n: 128 or 64 (g.tiles_m / g.tiles_n must be counted in those units)
+int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int tile_n) {
+    const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * g.batch * g.split_k;
+    if (blocks <= 0) return MNI_OK;
+    if (blocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "sgemm: too many tiles (%lld)", (long long)blocks);
+    dim3 grid((unsigned)blocks);
+    if (tile_m == 128 && tile_n == 128) launch_modes<2, 2>(g, amode, bmode, grid);
+    else if (tile_m == 128 && tile_n == 64) launch_modes<2, 1>(g, amode, bmode, grid);
+    else if (tile_m == 64 && tile_n == 128) launch_modes<1, 2>(g, amode, bmode, grid);
+    else if (tile_m == 64 && tile_n == 64) launch_modes<1, 1>(g, amode, bmode, grid);
+    else return set_error(MNI_ERR_INVALID, "sgemm: unsupported tile %d x %d", tile_m, tile_n);
     return check_launch("gemm_mfma_kernel");
 }
 
-int gemm_mfma_tile_m() { return BM; }
-int gemm_mfma_tile_n() { return BN; }
 int gemm_mfma_tile_k() { return BK; }
 
 }  // namespace mni

@@ -87,7 +87,10 @@ typedef struct {
 } mni_operand;
 
 enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_GELU = 3 };
-enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2 };
+/* MFMA = the MFMA tile kernel with its own choice of tile; MFMA_SMALL = the same
+ * kernel forced to 64 x 64 tiles; SKINNY = the bandwidth kernels (error if the
+ * shape or layout is not eligible). */
+enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),

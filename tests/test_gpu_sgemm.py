@@ -77,6 +77,20 @@ def test_mfma_integer_exact_all_layouts(dev, m, n, k, ta, tb):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 50, 200), (50, 300, 200), (256, 384, 160), (512, 512, 64)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("algo", [N.ALGO_MFMA, N.ALGO_MFMA_SMALL])
+def test_mfma_tile_shapes_integer_exact(dev, m, n, k, ta, tb, algo):
+    # 128x64 / 64x128 tiles (an extent <= 64), forced 64x64 tiles, short K
+    a = synth.small_ints(m + k, (k, m) if ta else (m, k), 4)
+    b = synth.small_ints(n + k, (n, k) if tb else (k, n), 4, stream=1)
+    got = run_gemm(dev, a, b, ta, tb, algo=algo)[0]
+    want = ((a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(np.float32)
+    assert np.array_equal(got, want)
+    got = run_gemm(dev, a, b, ta, tb, algo=algo, split_k=2)[0]
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("m,n,k", [(64, 48, 96), (300, 200, 1000), (512, 512, 512)])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 def test_mfma_normal_inputs_vs_oracle(dev, oracle_native, m, n, k, ta, tb):
