@@ -160,7 +160,10 @@ static int run_mfma(const mni_gemm_desc &d) {
         bm = bn = 64;
     } else if (d.algo == MNI_ALGO_AUTO) {
         const int64_t big_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
-        if (g.K <= 256 && big_tiles < 4LL * cus) bm = bn = 64;
+        const int ksteps = (g.K + bk - 1) / bk;
+        const int64_t big_split = d.split_k > 0 ? d.split_k : (ksteps / 8 > 0 ? ksteps / 8 : 1);
+        if (bm == 128 && bn == 128 && ((g.K <= 256 && big_tiles < 4LL * cus) || big_tiles * big_split < 2LL * cus))
+            bm = bn = 64;
     }
     g.tiles_m = (g.M + bm - 1) / bm;
     g.tiles_n = (g.N + bn - 1) / bn;
