@@ -70,7 +70,28 @@ def build(force=False, verbose=True):
             print(out)
     if verbose:
         print("built %s (%d translation units recompiled)" % (LIB, len(jobs)))
+    build_node_addon(force or bool(jobs), verbose)
     return LIB
+
+
+NODE_ADDON = os.path.join(HERE, "lib", "mni_rocm.node")
+NODE_INCLUDE = "/usr/include/node"
+
+
+def build_node_addon(force=False, verbose=True):
+    """The Node-API shim (csrc/napi_shim.cpp) over the engine-level ABI.  Needs
+    only g++ and node_api.h; skipped where the Node headers are not installed."""
+    src = os.path.join(CSRC, "napi_shim.cpp")
+    if not os.path.exists(os.path.join(NODE_INCLUDE, "node_api.h")):
+        if verbose:
+            print("node_api.h not found: Node addon not built")
+        return None
+    if force or _stale(NODE_ADDON, [src, LIB, os.path.normpath(os.path.join(CSRC, HEADERS[2]))]):
+        _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I" + NODE_INCLUDE, src, "-o", NODE_ADDON,
+              "-L" + os.path.dirname(LIB), "-lmni_rocm", "-Wl,-rpath,$ORIGIN"])
+        if verbose:
+            print("built %s" % NODE_ADDON)
+    return NODE_ADDON
 
 
 if __name__ == "__main__":

@@ -1,0 +1,118 @@
+// Drives the Node-API addon (framework_amd/lib/mni_rocm.node) the way the
+// reference's TypeScript layer drives its native addon: a Tensor class that
+// only forwards ids (cf. src/tensor.ts), Linear / mseLoss / Adam on top of it
+// (cf. src/nn.ts, src/optimizer.ts), and the assertions the reference's own
+// suite makes about the matmul path (test/tensor.test.ts MatMul section,
+// test/autograd.test.ts, test/nn.test.ts, test/module.test.ts).  Needs a GPU.
+'use strict';
+const path = require('path');
+const native = require(path.join(__dirname, '..', '..', 'framework_amd', 'lib', 'mni_rocm.node'));
+
+let passed = 0, failed = 0;
+function assert(cond, msg) { if (cond) { passed++; } else { failed++; console.log('FAIL: ' + msg); } }
+function assertClose(a, b, tol, msg) { assert(Math.abs(a - b) <= tol, msg + ' (got ' + a + ', want ' + b + ')'); }
+
+class Tensor {
+  constructor(id, shape) { this._id = id; this._shape = shape || native.tensorShape(id).map(Number); }
+  get shape() { return this._shape; }
+  get grad() { const g = native.getGrad(this._id); return g == null ? null : new Tensor(g); }
+  static fromFloat32(data, shape) { return new Tensor(native.fromFloat32(data, shape), shape); }
+  toFloat32() { return native.toFloat32(this._id); }
+  setRequiresGrad(r) { native.setRequiresGrad(this._id, r); return this; }
+  matmul(o) { return new Tensor(native.matmul(this._id, o._id)); }
+  add(o) { return new Tensor(native.add(this._id, o._id)); }
+  sub(o) { return new Tensor(native.sub(this._id, o._id)); }
+  mul(o) { return typeof o === 'number' ? new Tensor(native.mulScalar(this._id, o)) : new Tensor(native.mul(this._id, o._id)); }
+  relu() { return new Tensor(native.relu(this._id)); }
+  sum(dim) { return new Tensor(dim === undefined ? native.sumAll(this._id) : native.sumOp(this._id, dim)); }
+  permute(...dims) { return new Tensor(native.permute(this._id, dims)); }
+  backward() { native.backward(this._id); }
+}
+function lcg(seed) { let s = seed >>> 0; return () => { s = (Math.imul(s, 1664525) + 1013904223) >>> 0; return s / 4294967296; }; }
+function randArray(n, rnd, lo, hi) { const a = new Float32Array(n); for (let i = 0; i < n; i++) a[i] = lo + (hi - lo) * rnd(); return a; }
+class Linear {
+  constructor(inF, outF, rnd, fused) {
+    const b = 1 / Math.sqrt(inF);
+    this.weight = Tensor.fromFloat32(randArray(inF * outF, rnd, -b, b), [inF, outF]).setRequiresGrad(true);
+    this.bias = Tensor.fromFloat32(randArray(outF, rnd, -b, b), [outF]).setRequiresGrad(true);
+    this.fused = fused && typeof native.linear === 'function';   // the reference's feature-detection idiom
+  }
+  forward(x) {
+    if (this.fused) return new Tensor(native.linear(x._id, this.weight._id, this.bias._id, 1));
+    return x.matmul(this.weight).add(this.bias);
+  }
+  parameters() { return [this.weight, this.bias]; }
+}
+function mseLoss(pred, target) {  // mean(-1) twice, as the reference does
+  const d = pred.sub(target); const sq = d.mul(d);
+  return new Tensor(native.meanOp(native.meanOp(sq._id, -1), -1));
+}
+
+// ---- MatMul (test/tensor.test.ts) ------------------------------------------------------
+const mm = Tensor.fromFloat32(new Float32Array([1, 2, 3, 4]), [2, 2]).matmul(Tensor.fromFloat32(new Float32Array([5, 6, 7, 8]), [2, 2])).toFloat32();
+assertClose(mm[0], 19, 1e-3, 'matmul [0,0]'); assertClose(mm[1], 22, 1e-3, 'matmul [0,1]');
+assertClose(mm[2], 43, 1e-3, 'matmul [1,0]'); assertClose(mm[3], 50, 1e-3, 'matmul [1,1]');
+const ns = Tensor.fromFloat32(new Float32Array([1, 2, 3, 4, 5, 6]), [2, 3]).matmul(Tensor.fromFloat32(new Float32Array([1, 2, 3, 4, 5, 6]), [3, 2]));
+assert(ns.shape[0] === 2 && ns.shape[1] === 2, 'matmul [2,3]x[3,2] -> [2,2]');
+assertClose(ns.toFloat32()[0], 22, 1e-3, 'matmul non-square [0,0]');
+const rnd = lcg(7);
+const bm = Tensor.fromFloat32(randArray(60, rnd, 0, 1), [4, 3, 5]).matmul(Tensor.fromFloat32(randArray(40, rnd, 0, 1), [4, 5, 2]));
+assert(bm.shape.join() === '4,3,2', 'batched matmul shape');
+
+// ---- a larger product against a JS triple loop, through a permuted view ---------------
+{
+  const M = 70, K = 45, N = 90;
+  const a = randArray(M * K, rnd, -1, 1), bt = randArray(N * K, rnd, -1, 1);  // bt is B^T, viewed through permute
+  const got = Tensor.fromFloat32(a, [M, K]).matmul(Tensor.fromFloat32(bt, [N, K]).permute(1, 0)).toFloat32();
+  let worst = 0;
+  for (let i = 0; i < M; i++) for (let j = 0; j < N; j++) {
+    let s = 0; for (let k = 0; k < K; k++) s += a[i * K + k] * bt[j * K + k];
+    worst = Math.max(worst, Math.abs(s - got[i * N + j]));
+  }
+  assert(worst <= 1e-4 * Math.sqrt(K), 'permuted-view matmul vs JS loop, max err ' + worst);
+}
+
+// ---- autograd through matmul (test/autograd.test.ts) -------------------------------------
+const mmX = Tensor.fromFloat32(new Float32Array([1, 0, 0, 1]), [2, 2]).setRequiresGrad(true);
+const mmY = Tensor.fromFloat32(new Float32Array([3, 4, 5, 6]), [2, 2]).setRequiresGrad(true);
+mmX.matmul(mmY).sum().backward();
+assert(mmX.grad !== null, 'matmul grad exists');
+assert(Array.from(mmX.grad.toFloat32()).join() === '7,11,7,11', 'dX = G Y^T');
+assert(Array.from(mmY.grad.toFloat32()).join() === '1,1,1,1', 'dY = X^T G');
+
+// ---- Linear and losses (test/nn.test.ts) ------------------------------------------------------
+for (const fused of [false, true]) {
+  const lin = new Linear(3, 2, lcg(3), fused);
+  const out = lin.forward(Tensor.fromFloat32(randArray(12, rnd, 0, 1), [4, 3]));
+  assert(out.shape[0] === 4 && out.shape[1] === 2, 'linear [4,3] -> [4,2] fused=' + fused);
+  assert(lin.parameters().length === 2, 'linear has weight + bias');
+}
+const p = Tensor.fromFloat32(new Float32Array([1, 2, 3, 4]), [2, 2]);
+assertClose(mseLoss(p, Tensor.fromFloat32(new Float32Array([1, 2, 3, 4]), [2, 2])).toFloat32()[0], 0, 1e-4, 'mseLoss identical = 0');
+assertClose(mseLoss(p, Tensor.fromFloat32(new Float32Array([2, 3, 4, 5]), [2, 2])).toFloat32()[0], 1.0, 1e-4, 'mseLoss off-by-1 = 1.0');
+
+// ---- end-to-end regression (test/module.test.ts) --------------------------------------------------
+{
+  const X = Tensor.fromFloat32(new Float32Array([0, 1, 2, 3, 4, 5]), [6, 1]);
+  const Y = Tensor.fromFloat32(new Float32Array([1, 3, 5, 7, 9, 11]), [6, 1]);
+  const net = new Linear(1, 1, lcg(11), false);
+  const ids = net.parameters().map(t => t._id);
+  let early = null, t = 0;
+  for (let i = 0; i < 200; i++) {
+    native.zeroGrad(ids);
+    const loss = mseLoss(net.forward(X), Y);
+    if (i === 10) early = loss.toFloat32()[0];
+    loss.backward();
+    native.clipAndStep(ids, 0.05, 0.9, 0.95, 1e-8, 0, ++t, 0);   // Adam {lr: 0.05}
+    native.gcTensors([X._id, Y._id].concat(ids, ids.map(id => native.getGrad(id))));
+  }
+  const final = mseLoss(net.forward(X), Y).toFloat32()[0];
+  assert(final < early, 'training reduces loss'); assert(final < 1.0, 'training converges to low loss (' + final + ')');
+}
+
+// ---- misuse raises a JS Error where the reference panics ---------------------------------------------
+try { Tensor.fromFloat32(new Float32Array(6), [2, 3]).matmul(Tensor.fromFloat32(new Float32Array(8), [4, 2])); assert(false, 'K mismatch must throw'); }
+catch (e) { assert(/inner dimensions/.test(e.message), 'K mismatch message: ' + e.message); }
+
+console.log(passed + ' passed, ' + failed + ' failed');
+process.exit(failed ? 1 : 0);
