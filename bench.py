@@ -97,18 +97,14 @@ def bench_extras(r):
     x = synth.normal(4, (4, 4096), 0.02)
     w = synth.normal(4, (4096, 4096), 0.02, stream=1)
     dx, dw, dy = r.to_device(x), r.to_device(w), r.malloc(4 * 4096 * 4)
-    ms = time_launches(r, lambda: r.sgemm(4, 4096, 4096, dx, dw, dy), 5, 50)
+    # launches of a few microseconds are issued from C (mni_rocm_sgemm_timed) so that the host stays ahead
+    ms = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 10, 200)
     by = 4.0 * (4096 * 4096 + 2 * 4 * 4096)
     out["config5a_gemv"] = {"us": ms * 1e3, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / PEAK_HBM_GBPS,
                             "note": "W (64 MiB) is re-read every launch and fits the 256 MiB Infinity Cache"}
     # the same product over 8 different W in turn (512 MiB working set): HBM-resident
     ws = [r.to_device(w) for _ in range(8)]
-    state = {"i": 0}
-
-    def rot():
-        r.sgemm(4, 4096, 4096, dx, ws[state["i"] % 8], dy)
-        state["i"] += 1
-    ms = time_launches(r, rot, 8, 64)
+    ms = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, p, dy) for p in ws], 16, 200)
     out["config5a_gemv_cold"] = {"us": ms * 1e3, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / PEAK_HBM_GBPS}
     for p in ws + [dx, dw, dy]:
         r.free(p)
@@ -127,12 +123,12 @@ def bench_extras(r):
     dq, dk, dds = r.to_device(q), r.to_device(q), r.to_device(ds)
     s_out, g_out = r.malloc(32 * 512 * 512 * 4), r.malloc(32 * 512 * 64 * 4)
     fl = 2.0 * 32 * 512 * 512 * 64
-    ms_f = time_launches(r, lambda: r.sgemm(512, 512, 64, dq, dk, s_out, batch=32, a_batch=(512 * 64, 32),
-                                            b_strides=(1, 64), b_batch=(512 * 64, 32)), 3, 20)
-    ms_q = time_launches(r, lambda: r.sgemm(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32),
-                                            b_batch=(512 * 64, 32)), 3, 20)
-    ms_k = time_launches(r, lambda: r.sgemm(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64),
-                                            a_batch=(512 * 64, 32), b_batch=(512 * 512, 32)), 3, 20)
+    ms_f = r.sgemm_timed([r.gemm_desc(512, 512, 64, dq, dk, s_out, batch=32, a_batch=(512 * 64, 32),
+                                      b_strides=(1, 64), b_batch=(512 * 64, 32))], 5, 100)
+    ms_q = r.sgemm_timed([r.gemm_desc(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32),
+                                      b_batch=(512 * 64, 32))], 5, 100)
+    ms_k = r.sgemm_timed([r.gemm_desc(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64),
+                                      a_batch=(512 * 64, 32), b_batch=(512 * 512, 32))], 5, 100)
     by = 4.0 * 32 * (512 * 64 * 2 + 512 * 512)
     out["config3_attention_scores"] = {
         "fwd_us": ms_f * 1e3, "dq_us": ms_q * 1e3, "dkT_us": ms_k * 1e3,

@@ -35,6 +35,15 @@ struct DeviceCtx {
     int clock_khz = 0;
     char name[256] = {0};
     hipStream_t stream = nullptr;
+    // Workgroup b of a 1-D grid runs on XCD b % xcd_count when the start-up
+    // probe confirmed it (0 = not confirmed; kernels that rely on sharing one
+    // XCD's L2 are then not used).
+    int xcd_count = 0;
+    // Arrival flags of the single-launch skinny kernel: [unit][slice], each
+    // launch marks them with a fresh epoch so they never need clearing.
+    unsigned *skinny_flags = nullptr;
+    size_t skinny_flag_cap = 0;  // entries
+    unsigned skinny_epoch = 0;
 };
 DeviceCtx &ctx();
 int ensure_init();  // initialises device 0 on first use

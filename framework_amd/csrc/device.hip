@@ -28,6 +28,38 @@ DeviceCtx &ctx() {
     return c;
 }
 
+// Which XCD a workgroup runs on: the hardware id, read by one lane.
+__global__ void xcc_probe_kernel(unsigned *out) {
+    if (threadIdx.x == 0) {
+        unsigned v;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(v));
+        out[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)] = v & 0xf;
+    }
+}
+
+// Confirms that workgroups are dealt to the XCDs round-robin by linear id
+// (x fastest; workgroup b on XCD b % count), also in a 2-D/3-D grid, which the
+// single-launch skinny kernel relies on to keep a column group's partial sums
+// inside one XCD's L2.
+static int probe_xcd_mapping(DeviceCtx &c) {
+    const dim3 grid(24, 29, 3);  // 24 = a multiple of 8 XCDs, as the skinny kernel's grids are
+    constexpr int BLOCKS = 24 * 29 * 3;
+    unsigned *dev = nullptr;
+    MNI_HIP_CHECK(hipMalloc((void **)&dev, BLOCKS * sizeof(unsigned)));
+    hipLaunchKernelGGL(xcc_probe_kernel, grid, dim3(64), 0, c.stream, dev);
+    std::vector<unsigned> host(BLOCKS);
+    hipError_t e = hipMemcpyAsync(host.data(), dev, BLOCKS * sizeof(unsigned), hipMemcpyDeviceToHost, c.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
+    (void)hipFree(dev);
+    if (e != hipSuccess) return set_error(MNI_ERR_HIP, "XCD probe failed: %s", hipGetErrorString(e));
+    unsigned count = 0;
+    for (unsigned v : host) count = v + 1 > count ? v + 1 : count;
+    bool round_robin = count > 0;
+    for (int b = 0; b < BLOCKS && round_robin; ++b) round_robin = host[b] == (unsigned)b % count;
+    c.xcd_count = round_robin ? (int)count : 0;
+    return MNI_OK;
+}
+
 static int init_device(int device) {
     DeviceCtx &c = ctx();
     if (c.ready) {
@@ -50,6 +82,11 @@ static int init_device(int device) {
     snprintf(c.name, sizeof c.name, "%s (%s)", prop.name, prop.gcnArchName);
     // Default priority on purpose: streams of mixed priority are avoided.
     MNI_HIP_CHECK(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
+    MNI_TRY(probe_xcd_mapping(c));
+    c.skinny_flag_cap = 1 << 16;
+    MNI_HIP_CHECK(hipMalloc((void **)&c.skinny_flags, c.skinny_flag_cap * sizeof(unsigned)));
+    MNI_HIP_CHECK(hipMemset(c.skinny_flags, 0, c.skinny_flag_cap * sizeof(unsigned)));
+    c.skinny_epoch = 0;
     c.ready = true;
     return MNI_OK;
 }
@@ -158,6 +195,11 @@ int mni_rocm_device_info(char *name, size_t name_cap, int *compute_units, int *c
     if (compute_units) *compute_units = ctx().compute_units;
     if (clock_khz) *clock_khz = ctx().clock_khz;
     return MNI_OK;
+}
+
+int mni_rocm_device_xcds(void) {
+    if (ensure_init() != MNI_OK) return -1;
+    return ctx().xcd_count;
 }
 
 const char *mni_rocm_last_error(void) { return g_err_shared; }

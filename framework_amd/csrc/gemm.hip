@@ -35,7 +35,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_MFMA_SMALL)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_SKINNY_TWO_PASS)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -83,6 +83,7 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         s.out = d.C; s.o_bs = d.c_batch_stride; s.bias = d.bias;
         s.epilogue = d.epilogue; s.accumulate = d.accumulate;
         s.ws = nullptr; s.split_k = 1; s.k_per_slice = s.K;
+        s.groups = 0; s.fused = 0; s.xcds = 0; s.flags = nullptr; s.epoch = 0;
 
         const bool w_batch_ok = s.w_bcount <= 1 || (s.w_bs % 4) == 0;
         const bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
@@ -95,6 +96,7 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
             // nearly all of W is requested at once); a slice is a whole number
             // of workgroup passes.
             const int groups = (s.cols + skinny_cols_block_cols() - 1) / skinny_cols_block_cols();
+            s.groups = groups;
             const int pass = skinny_cols_rows_per_pass();
             int split = d.split_k;
             if (split == 0) {
@@ -116,8 +118,20 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
                 if (*rc != MNI_OK) return true;
                 s.ws = (float *)ws;
             }
-            *rc = launch_skinny_cols(s);
-            if (*rc == MNI_OK && split > 1) {
+            // One launch when the partials of a unit can stay inside one XCD's
+            // L2 and its arrival flags fit the library's flag array.
+            DeviceCtx &c = ctx();
+            const int64_t flag_count = (int64_t)groups * s.batch * split;
+            if (split > 1 && d.algo != MNI_ALGO_SKINNY_TWO_PASS && c.xcd_count > 0 && c.skinny_flags &&
+                flag_count <= (int64_t)c.skinny_flag_cap) {
+                if (++c.skinny_epoch == 0) {  // wrapped: old marks could match again
+                    *rc = k_fill((float *)c.skinny_flags, 0.0f, (int64_t)c.skinny_flag_cap);
+                    c.skinny_epoch = 1;
+                }
+                s.fused = 1; s.xcds = c.xcd_count; s.flags = c.skinny_flags; s.epoch = c.skinny_epoch;
+            }
+            if (*rc == MNI_OK) *rc = launch_skinny_cols(s);
+            if (*rc == MNI_OK && split > 1 && !s.fused) {
                 ReduceLaunch r;
                 r.ws = s.ws; r.out = s.out; r.bias = s.bias;
                 r.slices = split; r.batch = s.batch; r.rows = s.rows; r.cols = s.cols;
@@ -211,10 +225,10 @@ int sgemm(const mni_gemm_desc &d) {
     MNI_TRY(ensure_init());
     MNI_TRY(validate(d));
     if (d.M == 0 || d.N == 0 || d.batch == 0) return MNI_OK;
-    if (d.algo == MNI_ALGO_AUTO || d.algo == MNI_ALGO_SKINNY) {
+    if (d.algo == MNI_ALGO_AUTO || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS) {
         int rc;
         if (try_skinny(d, &rc)) return rc;
-        if (d.algo == MNI_ALGO_SKINNY)
+        if (d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS)
             return set_error(MNI_ERR_INVALID,
                              "sgemm: shape/layout not eligible for the skinny kernels "
                              "(needs min(M,N) <= 16 and 16-byte aligned unit-stride W)");
@@ -227,4 +241,29 @@ int sgemm(const mni_gemm_desc &d) {
 extern "C" int mni_rocm_sgemm(const mni_gemm_desc *desc) {
     if (!desc) return mni::set_error(MNI_ERR_INVALID, "sgemm: null descriptor");
     return mni::sgemm(*desc);
+}
+
+extern "C" int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms) {
+    using namespace mni;
+    if (!descs || count <= 0 || iters <= 0 || warmup < 0 || !avg_ms)
+        return set_error(MNI_ERR_INVALID, "sgemm_timed: bad arguments");
+    MNI_TRY(ensure_init());
+    int next = 0;
+    for (int i = 0; i < warmup; ++i, next = (next + 1) % count) MNI_TRY(sgemm(descs[next]));
+    hipEvent_t e0, e1;
+    MNI_HIP_CHECK(hipEventCreate(&e0));
+    MNI_HIP_CHECK(hipEventCreate(&e1));
+    int rc = MNI_OK;
+    hipError_t he = hipEventRecord(e0, ctx().stream);
+    for (int i = 0; i < iters && rc == MNI_OK && he == hipSuccess; ++i, next = (next + 1) % count) rc = sgemm(descs[next]);
+    if (he == hipSuccess) he = hipEventRecord(e1, ctx().stream);
+    if (he == hipSuccess) he = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != MNI_OK) return rc;
+    if (he != hipSuccess) return set_error(MNI_ERR_HIP, "sgemm_timed: %s", hipGetErrorString(he));
+    *avg_ms = ms / (float)iters;
+    return MNI_OK;
 }

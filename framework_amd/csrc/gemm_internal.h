@@ -37,12 +37,19 @@ struct SkinnyLaunch {
     const float *bias;  // indexed by bias_on_rows ? i : j
     float *ws;          // partials [slice][batch][rows][cols]
     int rows, cols, K, batch;
+    int groups;  // column groups of skinny_cols_block_cols() (skinny_cols only)
     int64_t x_rs, x_cs, x_bs;  // X(i, k)
     int64_t w_rs, w_cs, w_bs;  // W(k, j)
     int x_bcount, w_bcount;
     int64_t o_rs, o_cs, o_bs;
     int split_k, k_per_slice;
     int epilogue, accumulate, bias_on_rows;
+    // Single-launch form (fused != 0, split_k > 1): arrival flags
+    // [unit][split_k] with unit = b * groups + column group, the value that
+    // marks this launch, and the number of XCDs the units are dealt over.
+    int fused, xcds;
+    unsigned *flags;
+    unsigned epoch;
 };
 // W with unit stride along j (cols): lanes own columns, K split over wavefronts and slices.
 int launch_skinny_cols(const SkinnyLaunch &s);

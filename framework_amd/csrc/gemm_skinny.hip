@@ -27,33 +27,81 @@ __device__ __forceinline__ float sk_epilogue(float v, float bias, int epilogue) 
 }
 
 // ---- W contiguous along columns ---------------------------------------------
-// grid = (column groups of 256, K slices, batch), 256 threads = 4 wavefronts.
+// Work item = (column group of 256, K slice, batch), 256 threads = 4 wavefronts.
 // A wavefront reads whole 1 KiB pieces of W rows (every lane one 16-byte load
 // per row, SK_UNROLL rows in flight), which is the access pattern that streams
 // HBM best; the X values of a row are the same for all lanes, so they are
 // fetched with wave-uniform (scalar) loads.  The 4 wavefronts interleave groups
 // of SK_UNROLL rows and are summed through LDS in wave order.  K is sliced
 // across workgroups until about 4 workgroups per CU exist; each slice leaves a
-// partial that skinny_reduce_kernel sums in slice order, so the result does not
-// depend on scheduling.  (Single-launch variants -- arrival counters with
-// device-scope fences, float atomics, write-through partial stores, or one
-// workgroup owning all of K for 16 columns -- were measured slower on MI355X:
-// cross-XCD communication inside a kernel costs more than a second launch.)
-template <int MR, bool XC>
+// partial [slice][batch][rows][cols] and the slices are summed in a fixed
+// order, so the result does not depend on scheduling.
+//
+// Who sums the slices:
+//  * FUSED = false: a second launch (skinny_reduce_kernel).
+//  * FUSED = true: the same launch.  All slices of a (batch, column group) unit
+//    are given to workgroups of ONE XCD (1-D grid, workgroup b runs on XCD
+//    b % xcds -- confirmed by a probe when the library starts), so the partials
+//    never have to leave that XCD's L2.  A workgroup stores its partial, waits
+//    for the stores to be acknowledged, then sets its own arrival flag to this
+//    launch's epoch (a plain store to a private address).  The workgroups
+//    holding the last R = min(rows, slices) slices of a unit then act as
+//    reducers, one output row each: they poll the unit's flags with loads that
+//    skip the CU's L1, read the row's partials from L2 and apply the epilogue.
+//    Reducers have the highest workgroup ids of the grid, so everything they
+//    wait for has been dispatched before them and never waits itself; the poll
+//    is bounded all the same and a reducer that gives up writes NaN.
+//    Measured on MI355X for x[4,4096] W[4096,4096]: 12.2 us against 15.8 us for
+//    two launches.  What does not work here: one arrival counter per unit
+//    (returning atomics on one address serialise at ~145 ns each in L2: +9 us
+//    for 64 slices), device-scope fences (L2 write-back per workgroup) and
+//    float atomics.
+static constexpr int SK_SPIN_LIMIT = 1 << 18;
+
+__device__ __forceinline__ unsigned sk_load_flag(const unsigned *p) {
+    // sc1: served by the XCD's L2, never by the CU's L1 (a plain load would
+    // keep hitting the stale L1 line)
+    unsigned v;
+    asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+
+// TAIL = false promises that every slice is a whole number of SK_UNROLL-row
+// groups (K % SK_UNROLL == 0), which removes the guarded path and its address
+// arithmetic from the kernel; this kernel lives for a few microseconds, so the
+// length of its prologue shows.
+template <int MR, bool XC, bool FUSED, bool TAIL>
 __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLaunch s) {
     constexpr int U = SK_UNROLL;
     __shared__ float4 red[SK_WAVES - 1][MR][64];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int col0 = blockIdx.x * SK_COLS + 4 * lane;
-    const int slice = blockIdx.y, b = blockIdx.z;
+    int group, slice, b, unit = 0;
+    // A workgroup past the last unit is not turned away here but given an empty
+    // K range and dismissed after the loop: an early return would make the
+    // kernel wait for one kernel-argument fetch before it may start the next.
+    bool alive = true;
+    if (FUSED) {
+        // grid = (units rounded up to a multiple of the XCD count, slices):
+        // workgroups are dealt to XCDs by linear id, so unit u stays on XCD
+        // u % xcds in every slice row of the grid.
+        unit = blockIdx.x;
+        slice = blockIdx.y;
+        alive = unit < s.groups * s.batch;
+        if (s.batch == 1) { b = 0; group = unit; }
+        else { b = unit / s.groups; group = unit - b * s.groups; }
+    } else {
+        group = blockIdx.x; slice = blockIdx.y; b = blockIdx.z;
+    }
+    const int col0 = group * SK_COLS + 4 * lane;
     const int k_begin = slice * s.k_per_slice;
-    const int k_end = min(s.K, k_begin + s.k_per_slice);
+    const int k_end = alive ? min(s.K, k_begin + s.k_per_slice) : k_begin;
     const bool col_ok = col0 < s.cols;  // cols % 4 == 0 is a launch precondition
 
-    const float *__restrict__ X = s.X + (int64_t)(b % s.x_bcount) * s.x_bs;
-    const float *__restrict__ W = s.W + (int64_t)(b % s.w_bcount) * s.w_bs + (col_ok ? col0 : 0);
+    const int xb = s.x_bcount > 1 ? b % s.x_bcount : 0, wb = s.w_bcount > 1 ? b % s.w_bcount : 0;
+    const float *__restrict__ X = s.X + (int64_t)xb * s.x_bs;
+    const float *__restrict__ W = s.W + (int64_t)wb * s.w_bs + (col_ok ? col0 : 0);
 
     float4 acc[MR];
 #pragma unroll
@@ -61,35 +109,44 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
 
     for (int k0 = k_begin + wave * U; k0 < k_end; k0 += SK_WAVES * U) {
         f32x4 w[U];
-        if (k0 + U <= k_end) {
+        if (!TAIL || k0 + U <= k_end) {
             // whole group inside the slice: no clamps, no guards
             const float *__restrict__ wp = W + (int64_t)k0 * s.w_rs;
 #pragma unroll
             for (int u = 0; u < U; ++u)
                 w[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(wp + (int64_t)u * s.w_rs));
+            // X is requested four rows at a time without looking at s.rows
+            // (rows past it re-read the last row and are never stored):
+            // guarding each row would put one scalar-load round trip after
+            // the other.
 #pragma unroll
-            for (int i = 0; i < MR; ++i) {
-                if (i < s.rows) {
-                    float xv[U];
+            for (int i0 = 0; i0 < MR; i0 += 4) {
+                float xv[4][U];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int ii = min(i0 + i, s.rows - 1);
                     if (XC) {  // X rows contiguous along k: one scalar load of U floats
-                        const float *__restrict__ xr = X + (int64_t)i * s.x_rs + k0;
+                        const float *__restrict__ xr = X + (int64_t)ii * s.x_rs + k0;
 #pragma unroll
-                        for (int u = 0; u < U; ++u) xv[u] = xr[u];
+                        for (int u = 0; u < U; ++u) xv[i][u] = xr[u];
                     } else {
-                        const float *__restrict__ xr = X + (int64_t)i * s.x_rs + (int64_t)k0 * s.x_cs;
+                        const float *__restrict__ xr = X + (int64_t)ii * s.x_rs + (int64_t)k0 * s.x_cs;
 #pragma unroll
-                        for (int u = 0; u < U; ++u) xv[u] = xr[(int64_t)u * s.x_cs];
+                        for (int u = 0; u < U; ++u) xv[i][u] = xr[(int64_t)u * s.x_cs];
                     }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
-                        acc[i].x += xv[u] * w[u].x;
-                        acc[i].y += xv[u] * w[u].y;
-                        acc[i].z += xv[u] * w[u].z;
-                        acc[i].w += xv[u] * w[u].w;
+                        acc[i0 + i].x += xv[i][u] * w[u].x;
+                        acc[i0 + i].y += xv[i][u] * w[u].y;
+                        acc[i0 + i].z += xv[i][u] * w[u].z;
+                        acc[i0 + i].w += xv[i][u] * w[u].w;
                     }
                 }
             }
-        } else {
+        } else if (TAIL) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 // rows past the slice re-read its last row and meet x == 0
@@ -113,28 +170,99 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
         }
     }
 
+    if (FUSED && !alive) return;
+
     // ---- sum the wavefronts in wave order -------------------------------------
     if (wave > 0) {
 #pragma unroll
         for (int i = 0; i < MR; ++i) red[wave - 1][i][lane] = acc[i];
     }
     __syncthreads();
-    if (wave != 0 || !col_ok) return;
+    if (wave == 0) {
 #pragma unroll
-    for (int i = 0; i < MR; ++i) {
+        for (int i = 0; i < MR; ++i) {
 #pragma unroll
-        for (int w = 0; w < SK_WAVES - 1; ++w) {
-            const float4 p = red[w][i][lane];
-            acc[i].x += p.x; acc[i].y += p.y; acc[i].z += p.z; acc[i].w += p.w;
+            for (int w = 0; w < SK_WAVES - 1; ++w) {
+                const float4 p = red[w][i][lane];
+                acc[i].x += p.x; acc[i].y += p.y; acc[i].z += p.z; acc[i].w += p.w;
+            }
+        }
+        if (s.split_k > 1 && col_ok) {
+            float *ws = s.ws + (((int64_t)slice * s.batch + b) * s.rows) * (int64_t)s.cols + col0;
+#pragma unroll
+            for (int i = 0; i < MR; ++i)
+                if (i < s.rows) *reinterpret_cast<float4 *>(ws + (int64_t)i * s.cols) = acc[i];
         }
     }
-    if (s.split_k > 1) {
-        float *ws = s.ws + (((int64_t)slice * s.batch + b) * s.rows) * (int64_t)s.cols + col0;
+
+    if (FUSED) {
+        unsigned *flags = s.flags + (int64_t)unit * s.split_k;
+        if (wave == 0) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the partial has reached L2
+            if (lane == 0) flags[slice] = s.epoch;
+        }
+        const int reducers = min(s.rows, s.split_k);
+        const int q = s.split_k - 1 - slice;
+        if (q >= reducers) return;
+
+        // Every wavefront of a reducer polls on its own (lane l watches slices l, l + 64, ...).
+        bool arrived = false;
+        for (int spin = 0; spin < SK_SPIN_LIMIT && !arrived; ++spin) {
+            bool all = true;
+            for (int s0 = 0; s0 < s.split_k; s0 += 64) {
+                const int sl = s0 + lane;
+                const unsigned v = sl < s.split_k ? sk_load_flag(flags + sl) : s.epoch;
+                all = all && v == s.epoch;
+            }
+            arrived = __all(all);
+            if (!arrived) __builtin_amdgcn_s_sleep(2);
+        }
+
+        constexpr int TB = 16;  // partials in flight per lane
+        const int64_t slice_stride = (int64_t)s.batch * s.rows * s.cols;
+        for (int row = q; row < s.rows; row += reducers) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+            if (!arrived) {
+                const float nan = __builtin_nanf("");
+                t = f32x4{nan, nan, nan, nan};
+            } else if (col_ok) {
+                const float *p = s.ws + ((int64_t)b * s.rows + row) * (int64_t)s.cols + col0;
+                for (int s0 = wave; s0 < s.split_k; s0 += SK_WAVES * TB) {
+                    f32x4 v[TB];
 #pragma unroll
-        for (int i = 0; i < MR; ++i)
-            if (i < s.rows) *reinterpret_cast<float4 *>(ws + (int64_t)i * s.cols) = acc[i];
+                    for (int j = 0; j < TB; ++j) {
+                        const int sl = s0 + j * SK_WAVES;
+                        v[j] = sl < s.split_k ? *reinterpret_cast<const f32x4 *>(p + (int64_t)sl * slice_stride)
+                                              : f32x4{0.f, 0.f, 0.f, 0.f};
+                    }
+#pragma unroll
+                    for (int j = 0; j < TB; ++j) t += v[j];
+                }
+            }
+            __syncthreads();  // red is free again
+            if (wave > 0) red[wave - 1][0][lane] = make_float4(t.x, t.y, t.z, t.w);
+            __syncthreads();
+            if (wave == 0 && col_ok) {
+                float r[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                for (int w = 0; w < SK_WAVES - 1; ++w) {
+                    const float4 pw = red[w][0][lane];
+                    r[0] += pw.x; r[1] += pw.y; r[2] += pw.z; r[3] += pw.w;
+                }
+                float *out = s.out + (int64_t)b * s.o_bs;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (s.epilogue != MNI_EPI_NONE)
+                        r[e] = sk_epilogue(r[e], s.bias[s.bias_on_rows ? row : col0 + e], s.epilogue);
+                    float *dst = out + (int64_t)row * s.o_rs + (int64_t)(col0 + e) * s.o_cs;
+                    *dst = s.accumulate ? r[e] + *dst : r[e];
+                }
+            }
+        }
         return;
     }
+
+    if (wave != 0 || !col_ok || s.split_k > 1) return;
     float *out = s.out + (int64_t)b * s.o_bs;
 #pragma unroll
     for (int i = 0; i < MR; ++i) {
@@ -238,11 +366,11 @@ __global__ __launch_bounds__(256) void skinny_dots_kernel(const SkinnyLaunch s) 
     float *out = s.out + (int64_t)b * s.o_bs;
 #pragma unroll
     for (int i = 0; i < MR; ++i) {
-        if (i >= s.rows) break;
+        if (i >= s.rows) continue;
 #pragma unroll
         for (int c = 0; c < JW; ++c) {
             const int j = j0 + c;
-            if (j >= s.cols) break;
+            if (j >= s.cols) continue;
             float *dst = out + (int64_t)i * s.o_rs + (int64_t)j * s.o_cs;
             float r = acc[i][c];
             if (s.epilogue != MNI_EPI_NONE) r = sk_epilogue(r, s.bias[s.bias_on_rows ? i : j], s.epilogue);
@@ -272,21 +400,39 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const ReduceLaunch r
 int skinny_cols_block_cols() { return SK_COLS; }
 int skinny_cols_rows_per_pass() { return SK_WAVES * SK_UNROLL; }
 
+template <int MR>
+static void launch_skinny_cols_mr(const SkinnyLaunch &s, dim3 grid, bool fused) {
+    const dim3 block(SK_THREADS);
+    hipStream_t st = ctx().stream;
+    const int variant = (s.x_cs == 1 ? 4 : 0) | (fused ? 2 : 0) | (s.K % SK_UNROLL != 0 ? 1 : 0);
+    switch (variant) {
+#define MNI_SK(V, XC, FUSED, TAIL) \
+    case V: hipLaunchKernelGGL((skinny_cols_kernel<MR, XC, FUSED, TAIL>), grid, block, 0, st, s); break;
+        MNI_SK(0, false, false, false) MNI_SK(1, false, false, true)
+        MNI_SK(2, false, true, false)  MNI_SK(3, false, true, true)
+        MNI_SK(4, true, false, false)  MNI_SK(5, true, false, true)
+        MNI_SK(6, true, true, false)   MNI_SK(7, true, true, true)
+#undef MNI_SK
+    }
+}
+
 int launch_skinny_cols(const SkinnyLaunch &s) {
     if (s.rows <= 0 || s.cols <= 0 || s.batch <= 0) return MNI_OK;
-    dim3 grid((s.cols + SK_COLS - 1) / SK_COLS, s.split_k, s.batch), block(SK_THREADS);
-    hipStream_t st = ctx().stream;
-    const bool xc = s.x_cs == 1;
-#define MNI_SK(MR)                                                                          \
-    do {                                                                                    \
-        if (xc) hipLaunchKernelGGL((skinny_cols_kernel<MR, true>), grid, block, 0, st, s);  \
-        else hipLaunchKernelGGL((skinny_cols_kernel<MR, false>), grid, block, 0, st, s);    \
-    } while (0)
-    if (s.rows <= 4) MNI_SK(4);
-    else if (s.rows <= 8) MNI_SK(8);
-    else if (s.rows <= 16) MNI_SK(16);
+    const int groups = (s.cols + SK_COLS - 1) / SK_COLS;
+    if (s.groups != groups) return set_error(MNI_ERR_INVALID, "skinny launch: column group count not set");
+    if (s.k_per_slice % SK_UNROLL != 0 && s.split_k > 1)
+        return set_error(MNI_ERR_INVALID, "skinny launch: a K slice must be whole groups of %d rows", SK_UNROLL);
+    const bool fused = s.fused && s.split_k > 1;
+    dim3 grid(groups, s.split_k, s.batch);
+    if (fused) {
+        if (s.xcds <= 0 || !s.flags || !s.ws) return set_error(MNI_ERR_INVALID, "single-launch skinny product without flags/partials");
+        const int64_t units = (int64_t)groups * s.batch;
+        grid = dim3((unsigned)((units + s.xcds - 1) / s.xcds * s.xcds), s.split_k);
+    }
+    if (s.rows <= 4) launch_skinny_cols_mr<4>(s, grid, fused);
+    else if (s.rows <= 8) launch_skinny_cols_mr<8>(s, grid, fused);
+    else if (s.rows <= 16) launch_skinny_cols_mr<16>(s, grid, fused);
     else return set_error(MNI_ERR_INVALID, "skinny kernel takes at most 16 rows, got %d", s.rows);
-#undef MNI_SK
     return check_launch("skinny_cols_kernel");
 }
 

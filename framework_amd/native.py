@@ -23,7 +23,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmni_rocm.so")
 BAD_ID = 0xFFFFFFFF
 MAX_DIMS = 8
 EPI_NONE, EPI_BIAS, EPI_BIAS_RELU, EPI_BIAS_GELU = 0, 1, 2, 3
-ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL = 0, 1, 2, 3
+ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL, ALGO_SKINNY_TWO_PASS = 0, 1, 2, 3, 4
 
 _f32p = C.POINTER(C.c_float)
 _i64p = C.POINTER(C.c_int64)
@@ -51,6 +51,7 @@ class GemmDesc(C.Structure):
 SIGNATURES = {
     "mni_rocm_init": (C.c_int, [C.c_int]),
     "mni_rocm_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "mni_rocm_device_xcds": (C.c_int, []),
     "mni_rocm_last_error": (C.c_char_p, []),
     "mni_rocm_malloc": (C.c_int, [C.POINTER(C.c_void_p), C.c_size_t]),
     "mni_rocm_free": (C.c_int, [C.c_void_p]),
@@ -64,6 +65,7 @@ SIGNATURES = {
     "mni_rocm_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "mni_rocm_event_destroy": (C.c_int, [C.c_void_p]),
     "mni_rocm_sgemm": (C.c_int, [C.POINTER(GemmDesc)]),
+    "mni_rocm_sgemm_timed": (C.c_int, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
     "mni_rocm_strided_copy": (C.c_int, [C.c_void_p, C.c_void_p, _i64p, _i64p, C.c_int]),
     "mni_rocm_add_bias": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
     "mni_rocm_colsum": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
@@ -156,6 +158,12 @@ class Rocm:
         self._check(self.lib.mni_rocm_device_info(name, 256, C.byref(cus), C.byref(khz)))
         return {"name": name.value.decode(), "compute_units": cus.value, "clock_khz": khz.value}
 
+    def device_xcds(self):
+        n = self.lib.mni_rocm_device_xcds()
+        if n < 0:
+            raise MniError(self.lib.mni_rocm_last_error().decode())
+        return n
+
     def malloc(self, nbytes):
         p = C.c_void_p()
         self._check(self.lib.mni_rocm_malloc(C.byref(p), nbytes))
@@ -197,10 +205,23 @@ class Rocm:
     def event_destroy(self, event):
         self._check(self.lib.mni_rocm_event_destroy(event))
 
-    def sgemm(self, M, N, K, A, B, Cptr, *, batch=1, a_strides=None, b_strides=None, a_batch=(0, 1), b_batch=(0, 1),
-              ldc=None, c_batch_stride=None, bias=None, epilogue=EPI_NONE, accumulate=False, split_k=0, algo=ALGO_AUTO):
+    def sgemm(self, M, N, K, A, B, Cptr, **kw):
         """C = epilogue(op(A) * op(B)).  a_strides / b_strides are (row, col)
         element strides of op(A) (M x K) and op(B) (K x N); default row-major."""
+        d = self.gemm_desc(M, N, K, A, B, Cptr, **kw)
+        self._check(self.lib.mni_rocm_sgemm(C.byref(d)))
+
+    def sgemm_timed(self, descs, warmup, iters):
+        """Average ms per launch of the products in `descs` (made by gemm_desc),
+        cycled back to back and issued from C."""
+        arr = (GemmDesc * len(descs))(*descs)
+        ms = C.c_float(0)
+        self._check(self.lib.mni_rocm_sgemm_timed(arr, len(descs), warmup, iters, C.byref(ms)))
+        return ms.value
+
+    @staticmethod
+    def gemm_desc(M, N, K, A, B, Cptr, *, batch=1, a_strides=None, b_strides=None, a_batch=(0, 1), b_batch=(0, 1),
+                  ldc=None, c_batch_stride=None, bias=None, epilogue=EPI_NONE, accumulate=False, split_k=0, algo=ALGO_AUTO):
         d = GemmDesc()
         d.M, d.N, d.K, d.batch = M, N, K, batch
         ars, acs = a_strides if a_strides is not None else (K, 1)
@@ -215,7 +236,7 @@ class Rocm:
         d.accumulate = 1 if accumulate else 0
         d.split_k = split_k
         d.algo = algo
-        self._check(self.lib.mni_rocm_sgemm(C.byref(d)))
+        return d
 
     def strided_copy(self, dst, src, shape, strides):
         self._check(self.lib.mni_rocm_strided_copy(dst, src, _i64_array(shape), _i64_array(strides), len(shape)))

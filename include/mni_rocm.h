@@ -51,6 +51,11 @@ int mni_rocm_init(int device);
 /* Name reported by the HIP runtime and its compute-unit count / clock (kHz),
  * for roofline bookkeeping.  Any out pointer may be NULL. */
 int mni_rocm_device_info(char *name, size_t name_cap, int *compute_units, int *clock_khz);
+/* Number of XCDs (dies with an L2 of their own) that workgroups were seen to be
+ * dealt over round-robin when the library started; 0 if that could not be
+ * confirmed, in which case kernels that keep partial sums inside one XCD's L2
+ * are not used.  < 0 on error.  No counterpart in the reference. */
+int mni_rocm_device_xcds(void);
 const char *mni_rocm_last_error(void);
 
 /* Caching device allocator: replaces CachingAllocator of the cuda arm
@@ -89,8 +94,9 @@ typedef struct {
 enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_GELU = 3 };
 /* MFMA = the MFMA tile kernel with its own choice of tile; MFMA_SMALL = the same
  * kernel forced to 64 x 64 tiles; SKINNY = the bandwidth kernels (error if the
- * shape or layout is not eligible). */
-enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3 };
+ * shape or layout is not eligible); SKINNY_TWO_PASS = the same with the K-slice
+ * partials summed by a second launch instead of inside the first. */
+enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),
@@ -111,6 +117,12 @@ typedef struct {
     int32_t algo;        /* MNI_ALGO_*                                      */
 } mni_gemm_desc;
 int mni_rocm_sgemm(const mni_gemm_desc *desc);
+/* Measurement aid (no counterpart in the reference): runs descs[0], descs[1],
+ * ... descs[count-1], descs[0], ... back to back on the library's stream,
+ * `warmup` untimed launches and then `iters` launches between two HIP events,
+ * and returns the average milliseconds per launch.  Issuing from C keeps the
+ * host ahead of kernels that take only a few microseconds. */
+int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms);
 
 /* dst (contiguous, `shape`) = gather of src by `src_strides` (elements).
  * Replaces permute_f32 (src/native/kernels/elementwise.cu:67-81) and the host

@@ -228,15 +228,64 @@ def test_empty_and_zero_k(dev, rocm):
 
 # ---- skinny kernels ----------------------------------------------------------------
 
+def test_single_launch_skinny_path_is_available(rocm):
+    # MI355X deals workgroups over its 8 XCDs round-robin; were the probe to fail,
+    # ALGO_SKINNY would quietly run as ALGO_SKINNY_TWO_PASS and the tests below
+    # would cover one path twice.
+    assert rocm.device_xcds() == 8
+
+
+SKINNY_ALGOS = [N.ALGO_SKINNY, N.ALGO_SKINNY_TWO_PASS]  # slices summed inside the launch / by a second launch
+
+
+@pytest.mark.parametrize("algo", SKINNY_ALGOS)
 @pytest.mark.parametrize("m", [1, 2, 4, 5, 8, 13, 16])
-def test_skinny_cols_integer_exact(dev, m):
+def test_skinny_cols_integer_exact(dev, m, algo):
     a = synth.small_ints(m, (m, 700), 4)
     b = synth.small_ints(m + 1, (700, 520), 4, stream=1)
-    got = run_gemm(dev, a, b, algo=N.ALGO_SKINNY)[0]
-    assert np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
-    for split in (1, 3):
-        got = run_gemm(dev, a, b, algo=N.ALGO_SKINNY, split_k=split)[0]
-        assert np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b, algo=algo)[0], want)
+    for split in (1, 3, 11):  # 3 slices < 13 rows: reducers take several rows each
+        assert np.array_equal(run_gemm(dev, a, b, algo=algo, split_k=split)[0], want)
+
+
+@pytest.mark.parametrize("algo", SKINNY_ALGOS)
+def test_skinny_cols_many_slices_few_columns(dev, algo):
+    # one column group, hundreds of K slices: more arrival flags than lanes
+    a = synth.small_ints(1, (4, 32768), 2)
+    b = synth.small_ints(2, (32768, 96), 2, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b, algo=algo)[0], want)
+    assert np.array_equal(run_gemm(dev, a, b, algo=algo, split_k=200)[0], want)
+
+
+@pytest.mark.parametrize("algo", SKINNY_ALGOS)
+def test_skinny_cols_batched_units_epilogue_accumulate(dev, rocm, algo):
+    # 5 batches x 3 column groups = 15 units over the XCDs; bias + ReLU and accumulate in the slice reduction
+    a = synth.small_ints(1, (5, 6, 1024), 3)
+    w = synth.small_ints(2, (5, 1024, 640), 3, stream=1)
+    bias = synth.small_ints(3, (640,), 3, stream=2)
+    c0 = synth.small_ints(4, (5, 6, 640), 3, stream=3)
+    dA, dW, dbias, dC = dev.put(a), dev.put(w), dev.put(bias), dev.put(c0)
+    rocm.sgemm(6, 640, 1024, dA, dW, dC, batch=5, a_batch=(6 * 1024, 5), b_batch=(1024 * 640, 5),
+               bias=dbias, epilogue=N.EPI_BIAS_RELU, accumulate=True, split_k=7, algo=algo)
+    z = np.einsum("bmk,bkn->bmn", a.astype(np.int64), w.astype(np.int64)) + bias.astype(np.int64)
+    assert np.array_equal(rocm.to_host(dC, (5, 6, 640)), (np.maximum(z, 0) + c0).astype(np.float32))
+
+
+def test_skinny_single_launch_repeats_and_matches_two_pass(dev, rocm):
+    # the arrival flags are reused launch after launch (fresh epoch each time)
+    a = synth.normal(1, (4, 4096), 1.0)
+    w = synth.normal(2, (4096, 1024), 0.05, stream=1)
+    two = run_gemm(dev, a, w, algo=N.ALGO_SKINNY_TWO_PASS)[0]
+    dA, dW, dC = dev.put(a), dev.put(w), dev.empty(4 * 1024)
+    first = None
+    for _ in range(50):
+        rocm.sgemm(4, 1024, 4096, dA, dW, dC, algo=N.ALGO_SKINNY)
+        got = rocm.to_host(dC, (4, 1024))
+        first = got if first is None else first
+        assert np.array_equal(got, first)  # fixed summation order: the same bits every launch
+    assert max_err(first, two) <= gemm_tol(4096, a, w)
 
 
 @pytest.mark.parametrize("m", [1, 4, 16])
@@ -247,11 +296,12 @@ def test_skinny_dots_integer_exact(dev, m):
     assert np.array_equal(got, (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float32))
 
 
-def test_skinny_few_output_columns(dev):
+@pytest.mark.parametrize("algo", SKINNY_ALGOS)
+def test_skinny_few_output_columns(dev, algo):
     # [rows, K] x [K, 4]: the few columns become the skinny side (C^T = B^T A^T)
     at = synth.small_ints(1, (64, 1000), 4)  # A stored K x M
     b = synth.small_ints(2, (64, 4), 4, stream=1)
-    got = run_gemm(dev, at, b, ta=True, algo=N.ALGO_SKINNY)[0]
+    got = run_gemm(dev, at, b, ta=True, algo=algo)[0]
     assert np.array_equal(got, (at.T.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
     a = synth.small_ints(3, (1000, 64), 4)
     bt = synth.small_ints(4, (4, 64), 4, stream=1)
@@ -373,3 +423,17 @@ def test_config5b_tall_k_weight_gradient(dev, rocm):
     rows, cols = slice(100, 116), slice(900, 932)
     want = X[:, rows].astype(np.float64).T @ dY[:, cols].astype(np.float64)
     assert max_err(got[rows, cols], want) <= gemm_tol(65536, X, dY)
+
+
+def test_sgemm_timed_runs_the_products_and_reports_a_duration(dev, rocm):
+    a = synth.small_ints(1, (64, 48), 3)
+    bs = [synth.small_ints(2 + i, (48, 80), 3, stream=1) for i in range(3)]
+    dA, dBs = dev.put(a), [dev.put(b) for b in bs]
+    dCs = [dev.empty(64 * 80) for _ in bs]
+    descs = [rocm.gemm_desc(64, 80, 48, dA, dB, dC) for dB, dC in zip(dBs, dCs)]
+    ms = rocm.sgemm_timed(descs, 2, 7)  # 9 launches cycle over the 3 products
+    assert 0.0 < ms < 10.0
+    for b, dC in zip(bs, dCs):
+        assert np.array_equal(rocm.to_host(dC, (64, 80)), (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+    with pytest.raises(N.MniError):
+        rocm.sgemm_timed(descs, 0, 0)
