@@ -45,7 +45,7 @@ PEAK_HBM_GBPS = 8000.0
 # HBM bytes per gemm_mfma_kernel launch at 4096^3, from the rocprofv3 --pmc
 # runs summarised in profiles/gemm_mfma_4096_pmc.txt (FETCH_SIZE + WRITE_SIZE,
 # scaled by a copy kernel of known size).  None until measured.
-MEASURED_HBM_BYTES_4096 = 814.9e6
+MEASURED_HBM_BYTES_4096 = 786.7e6
 
 
 def time_launches(r, fn, warmup, iters):
@@ -285,7 +285,7 @@ def main():
         "config": {"workload": "single fp32 matmul A[4096,4096] x B[4096,4096], A,B ~ N(0,1) seed 1, row-major, forward only",
                    "M": 4096, "N": 4096, "K": 4096, "device": info["name"].strip(), "compute_units": info["compute_units"],
                    "max_err_vs_f64_sample": err},
-        "roofline": {"bound": "mfma", "kernel": "gemm_mfma_kernel<0,1>", "achieved": achieved,
+        "roofline": {"bound": "mfma", "kernel": "gemm_mfma_kernel<0, 1, 2, 2>", "achieved": achieved,
                      "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MATRIX_TFLOPS,
                      "kernel_ms": kernel_ms, "algorithmic_flops": flops, "traffic": MEASURED_HBM_BYTES_4096},
     }
