@@ -70,9 +70,18 @@ __device__ __forceinline__ unsigned sk_load_flag(const unsigned *p) {
 // groups (K % SK_UNROLL == 0), which removes the guarded path and its address
 // arithmetic from the kernel; this kernel lives for a few microseconds, so the
 // length of its prologue shows.
-template <int MR, bool XC, bool FUSED, bool TAIL>
+template <int MR, bool XC, bool FUSED, bool TAIL, bool LEAN>
 __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLaunch s) {
     constexpr int U = SK_UNROLL;
+    // LEAN (the decode shape): one batch, exactly MR rows, whole 256-column
+    // groups, row-major output, no epilogue -- known at compile time, so the
+    // general case's address arithmetic and guards drop out of a kernel whose
+    // whole life is a few microseconds.
+    static_assert(!LEAN || (XC && FUSED && !TAIL), "LEAN implies XC, FUSED, !TAIL");
+    const int rows = LEAN ? MR : s.rows, batch = LEAN ? 1 : s.batch;
+    const int epilogue = LEAN ? (int)MNI_EPI_NONE : s.epilogue, accumulate = LEAN ? 0 : s.accumulate;
+    const int64_t o_cs = LEAN ? 1 : s.o_cs;
+    const int x_bcount = LEAN ? 1 : s.x_bcount, w_bcount = LEAN ? 1 : s.w_bcount;
     __shared__ float4 red[SK_WAVES - 1][MR][64];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -88,8 +97,8 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
         // u % xcds in every slice row of the grid.
         unit = blockIdx.x;
         slice = blockIdx.y;
-        alive = unit < s.groups * s.batch;
-        if (s.batch == 1) { b = 0; group = unit; }
+        alive = unit < s.groups * batch;
+        if (batch == 1) { b = 0; group = unit; }
         else { b = unit / s.groups; group = unit - b * s.groups; }
     } else {
         group = blockIdx.x; slice = blockIdx.y; b = blockIdx.z;
@@ -97,9 +106,9 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
     const int col0 = group * SK_COLS + 4 * lane;
     const int k_begin = slice * s.k_per_slice;
     const int k_end = alive ? min(s.K, k_begin + s.k_per_slice) : k_begin;
-    const bool col_ok = col0 < s.cols;  // cols % 4 == 0 is a launch precondition
+    const bool col_ok = LEAN || col0 < s.cols;  // cols % 4 == 0 is a launch precondition
 
-    const int xb = s.x_bcount > 1 ? b % s.x_bcount : 0, wb = s.w_bcount > 1 ? b % s.w_bcount : 0;
+    const int xb = x_bcount > 1 ? b % x_bcount : 0, wb = w_bcount > 1 ? b % w_bcount : 0;
     const float *__restrict__ X = s.X + (int64_t)xb * s.x_bs;
     const float *__restrict__ W = s.W + (int64_t)wb * s.w_bs + (col_ok ? col0 : 0);
 
@@ -115,7 +124,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
 #pragma unroll
             for (int u = 0; u < U; ++u)
                 w[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(wp + (int64_t)u * s.w_rs));
-            // X is requested four rows at a time without looking at s.rows
+            // X is requested four rows at a time without looking at rows
             // (rows past it re-read the last row and are never stored):
             // guarding each row would put one scalar-load round trip after
             // the other.
@@ -124,7 +133,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
                 float xv[4][U];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const int ii = min(i0 + i, s.rows - 1);
+                    const int ii = min(i0 + i, rows - 1);
                     if (XC) {  // X rows contiguous along k: one scalar load of U floats
                         const float *__restrict__ xr = X + (int64_t)ii * s.x_rs + k0;
 #pragma unroll
@@ -155,7 +164,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
             }
 #pragma unroll
             for (int i = 0; i < MR; ++i) {
-                if (i < s.rows) {
+                if (i < rows) {
                     const float *__restrict__ xr = X + (int64_t)i * s.x_rs + (int64_t)k0 * s.x_cs;
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
@@ -188,10 +197,10 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
             }
         }
         if (s.split_k > 1 && col_ok) {
-            float *ws = s.ws + (((int64_t)slice * s.batch + b) * s.rows) * (int64_t)s.cols + col0;
+            float *ws = s.ws + (((int64_t)slice * batch + b) * rows) * (int64_t)s.cols + col0;
 #pragma unroll
             for (int i = 0; i < MR; ++i)
-                if (i < s.rows) *reinterpret_cast<float4 *>(ws + (int64_t)i * s.cols) = acc[i];
+                if (i < rows) *reinterpret_cast<float4 *>(ws + (int64_t)i * s.cols) = acc[i];
         }
     }
 
@@ -201,7 +210,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the partial has reached L2
             if (lane == 0) flags[slice] = s.epoch;
         }
-        const int reducers = min(s.rows, s.split_k);
+        const int reducers = min(rows, s.split_k);
         const int q = s.split_k - 1 - slice;
         if (q >= reducers) return;
 
@@ -219,14 +228,14 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
         }
 
         constexpr int TB = 16;  // partials in flight per lane
-        const int64_t slice_stride = (int64_t)s.batch * s.rows * s.cols;
-        for (int row = q; row < s.rows; row += reducers) {
+        const int64_t slice_stride = (int64_t)batch * rows * s.cols;
+        for (int row = q; row < rows; row += reducers) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
             if (!arrived) {
                 const float nan = __builtin_nanf("");
                 t = f32x4{nan, nan, nan, nan};
             } else if (col_ok) {
-                const float *p = s.ws + ((int64_t)b * s.rows + row) * (int64_t)s.cols + col0;
+                const float *p = s.ws + ((int64_t)b * rows + row) * (int64_t)s.cols + col0;
                 for (int s0 = wave; s0 < s.split_k; s0 += SK_WAVES * TB) {
                     f32x4 v[TB];
 #pragma unroll
@@ -250,12 +259,16 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
                     r[0] += pw.x; r[1] += pw.y; r[2] += pw.z; r[3] += pw.w;
                 }
                 float *out = s.out + (int64_t)b * s.o_bs;
+                if (LEAN) {
+                    *reinterpret_cast<float4 *>(out + (int64_t)row * s.o_rs + col0) = make_float4(r[0], r[1], r[2], r[3]);
+                    continue;
+                }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    if (s.epilogue != MNI_EPI_NONE)
-                        r[e] = sk_epilogue(r[e], s.bias[s.bias_on_rows ? row : col0 + e], s.epilogue);
-                    float *dst = out + (int64_t)row * s.o_rs + (int64_t)(col0 + e) * s.o_cs;
-                    *dst = s.accumulate ? r[e] + *dst : r[e];
+                    if (epilogue != MNI_EPI_NONE)
+                        r[e] = sk_epilogue(r[e], s.bias[s.bias_on_rows ? row : col0 + e], epilogue);
+                    float *dst = out + (int64_t)row * s.o_rs + (int64_t)(col0 + e) * o_cs;
+                    *dst = accumulate ? r[e] + *dst : r[e];
                 }
             }
         }
@@ -266,13 +279,13 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
     float *out = s.out + (int64_t)b * s.o_bs;
 #pragma unroll
     for (int i = 0; i < MR; ++i) {
-        if (i < s.rows) {
+        if (i < rows) {
             float r[4] = {acc[i].x, acc[i].y, acc[i].z, acc[i].w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                if (s.epilogue != MNI_EPI_NONE) r[e] = sk_epilogue(r[e], s.bias[s.bias_on_rows ? i : col0 + e], s.epilogue);
-                float *dst = out + (int64_t)i * s.o_rs + (int64_t)(col0 + e) * s.o_cs;
-                *dst = s.accumulate ? r[e] + *dst : r[e];
+                if (epilogue != MNI_EPI_NONE) r[e] = sk_epilogue(r[e], s.bias[s.bias_on_rows ? i : col0 + e], epilogue);
+                float *dst = out + (int64_t)i * s.o_rs + (int64_t)(col0 + e) * o_cs;
+                *dst = accumulate ? r[e] + *dst : r[e];
             }
         }
     }
@@ -405,9 +418,16 @@ static void launch_skinny_cols_mr(const SkinnyLaunch &s, dim3 grid, bool fused) 
     const dim3 block(SK_THREADS);
     hipStream_t st = ctx().stream;
     const int variant = (s.x_cs == 1 ? 4 : 0) | (fused ? 2 : 0) | (s.K % SK_UNROLL != 0 ? 1 : 0);
+    const bool lean = variant == 6 && s.batch == 1 && s.rows == MR && s.cols % SK_COLS == 0 && s.o_cs == 1 &&
+                      s.o_rs % 4 == 0 && (reinterpret_cast<uintptr_t>(s.out) & 15) == 0 &&
+                      s.epilogue == MNI_EPI_NONE && !s.accumulate;
+    if (lean) {
+        hipLaunchKernelGGL((skinny_cols_kernel<MR, true, true, false, true>), grid, block, 0, st, s);
+        return;
+    }
     switch (variant) {
 #define MNI_SK(V, XC, FUSED, TAIL) \
-    case V: hipLaunchKernelGGL((skinny_cols_kernel<MR, XC, FUSED, TAIL>), grid, block, 0, st, s); break;
+    case V: hipLaunchKernelGGL((skinny_cols_kernel<MR, XC, FUSED, TAIL, false>), grid, block, 0, st, s); break;
         MNI_SK(0, false, false, false) MNI_SK(1, false, false, true)
         MNI_SK(2, false, true, false)  MNI_SK(3, false, true, true)
         MNI_SK(4, true, false, false)  MNI_SK(5, true, false, true)

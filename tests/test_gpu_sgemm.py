@@ -249,6 +249,16 @@ def test_skinny_cols_integer_exact(dev, m, algo):
         assert np.array_equal(run_gemm(dev, a, b, algo=algo, split_k=split)[0], want)
 
 
+@pytest.mark.parametrize("m", [4, 8, 16])
+def test_skinny_cols_decode_shape_integer_exact(dev, m):
+    # whole column groups, full row blocks, plain output: the specialised single-launch kernel
+    a = synth.small_ints(m, (m, 2048), 4)
+    b = synth.small_ints(m + 1, (2048, 768), 4, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b, algo=N.ALGO_SKINNY)[0], want)
+    assert np.array_equal(run_gemm(dev, a, b, algo=N.ALGO_SKINNY, split_k=5)[0], want)
+
+
 @pytest.mark.parametrize("algo", SKINNY_ALGOS)
 def test_skinny_cols_many_slices_few_columns(dev, algo):
     # one column group, hundreds of K slices: more arrival flags than lanes
