@@ -1,6 +1,7 @@
 // Shared declarations of libmni_rocm.so: device context, allocator, error
 // reporting and the internal launchers the C ABI and the engine are built on.
 #pragma once
+#include <mutex>
 
 #include <hip/hip_runtime.h>
 #include <stddef.h>
@@ -46,6 +47,13 @@ struct DeviceCtx {
     unsigned skinny_epoch = 0;
 };
 DeviceCtx &ctx();
+
+// Every extern "C" entry point holds this for its whole duration: the engine
+// and the allocator are single-threaded by design, as the reference's Engine
+// behind its one mutex is (src/native/src/lib.rs:27-39).  Recursive because
+// engine-level entry points call kernel-level ones.
+std::recursive_mutex &api_mutex();
+#define MNI_API_GUARD std::lock_guard<std::recursive_mutex> mni_api_guard_(mni::api_mutex())
 int ensure_init();  // initialises device 0 on first use
 
 // ---- caching allocator -----------------------------------------------------

@@ -13,7 +13,8 @@
 
 namespace mni {
 
-static char g_err_shared[1024];
+// Per thread, so that a message read after a failed call is that call's own.
+static thread_local char g_err_shared[1024];
 
 int set_error(int code, const char *fmt, ...) {
     va_list ap;
@@ -21,6 +22,11 @@ int set_error(int code, const char *fmt, ...) {
     vsnprintf(g_err_shared, sizeof g_err_shared, fmt, ap);
     va_end(ap);
     return code;
+}
+
+std::recursive_mutex &api_mutex() {
+    static std::recursive_mutex m;
+    return m;
 }
 
 DeviceCtx &ctx() {
@@ -187,9 +193,10 @@ using namespace mni;
 
 extern "C" {
 
-int mni_rocm_init(int device) { return init_device(device); }
+int mni_rocm_init(int device) { MNI_API_GUARD; return init_device(device); }
 
 int mni_rocm_device_info(char *name, size_t name_cap, int *compute_units, int *clock_khz) {
+    MNI_API_GUARD;
     MNI_TRY(ensure_init());
     if (name && name_cap) snprintf(name, name_cap, "%s", ctx().name);
     if (compute_units) *compute_units = ctx().compute_units;
@@ -198,6 +205,7 @@ int mni_rocm_device_info(char *name, size_t name_cap, int *compute_units, int *c
 }
 
 int mni_rocm_device_xcds(void) {
+    MNI_API_GUARD;
     if (ensure_init() != MNI_OK) return -1;
     return ctx().xcd_count;
 }
@@ -205,13 +213,15 @@ int mni_rocm_device_xcds(void) {
 const char *mni_rocm_last_error(void) { return g_err_shared; }
 
 int mni_rocm_malloc(void **ptr, size_t bytes) {
+    MNI_API_GUARD;
     if (!ptr) return set_error(MNI_ERR_INVALID, "null out pointer");
     return dev_alloc(ptr, bytes);
 }
-int mni_rocm_free(void *ptr) { return dev_free(ptr); }
-int mni_rocm_clear_cache(void) { return dev_clear_cache(); }
+int mni_rocm_free(void *ptr) { MNI_API_GUARD; return dev_free(ptr); }
+int mni_rocm_clear_cache(void) { MNI_API_GUARD; return dev_clear_cache(); }
 
 int mni_rocm_h2d(void *dst, const void *src, size_t bytes) {
+    MNI_API_GUARD;
     MNI_TRY(ensure_init());
     if (bytes == 0) return MNI_OK;
     MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
@@ -219,6 +229,7 @@ int mni_rocm_h2d(void *dst, const void *src, size_t bytes) {
     return MNI_OK;
 }
 int mni_rocm_d2h(void *dst, const void *src, size_t bytes) {
+    MNI_API_GUARD;
     MNI_TRY(ensure_init());
     if (bytes == 0) return MNI_OK;
     MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
@@ -226,18 +237,21 @@ int mni_rocm_d2h(void *dst, const void *src, size_t bytes) {
     return MNI_OK;
 }
 int mni_rocm_d2d(void *dst, const void *src, size_t bytes) {
+    MNI_API_GUARD;
     MNI_TRY(ensure_init());
     if (bytes == 0) return MNI_OK;
     MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx().stream));
     return MNI_OK;
 }
 int mni_rocm_sync(void) {
+    MNI_API_GUARD;
     MNI_TRY(ensure_init());
     MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
     return MNI_OK;
 }
 
 int mni_rocm_event_create(void **event) {
+    MNI_API_GUARD;
     MNI_TRY(ensure_init());
     if (!event) return set_error(MNI_ERR_INVALID, "null out pointer");
     hipEvent_t e;
@@ -246,16 +260,19 @@ int mni_rocm_event_create(void **event) {
     return MNI_OK;
 }
 int mni_rocm_event_record(void *event) {
+    MNI_API_GUARD;
     MNI_TRY(ensure_init());
     MNI_HIP_CHECK(hipEventRecord((hipEvent_t)event, ctx().stream));
     return MNI_OK;
 }
 int mni_rocm_event_elapsed_ms(void *start, void *stop, float *ms) {
+    MNI_API_GUARD;
     MNI_HIP_CHECK(hipEventSynchronize((hipEvent_t)stop));
     MNI_HIP_CHECK(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
     return MNI_OK;
 }
 int mni_rocm_event_destroy(void *event) {
+    MNI_API_GUARD;
     MNI_HIP_CHECK(hipEventDestroy((hipEvent_t)event));
     return MNI_OK;
 }

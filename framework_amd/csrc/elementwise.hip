@@ -659,25 +659,30 @@ using namespace mni;
 
 extern "C" {
 int mni_rocm_strided_copy(float *dst, const float *src, const int64_t *shape, const int64_t *src_strides, int ndim) {
+    MNI_API_GUARD;
     if (!dst || !src || (ndim > 0 && (!shape || !src_strides))) return set_error(MNI_ERR_INVALID, "strided_copy: null argument");
     return k_strided_copy(dst, src, shape, src_strides, ndim);
 }
 int mni_rocm_add_bias(float *out, const float *a, const float *bias, int64_t rows, int64_t cols) {
+    MNI_API_GUARD;
     if (rows < 0 || cols < 0) return set_error(MNI_ERR_INVALID, "add_bias: negative extent");
     if (rows * cols > 0 && (!out || !a || !bias)) return set_error(MNI_ERR_INVALID, "add_bias: null argument");
     return k_add_bias(out, a, bias, rows, cols);
 }
 int mni_rocm_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
+    MNI_API_GUARD;
     if (rows < 0 || cols < 0) return set_error(MNI_ERR_INVALID, "colsum: negative extent");
     if (cols > 0 && (!out || (rows > 0 && !a))) return set_error(MNI_ERR_INVALID, "colsum: null argument");
     return k_colsum(out, a, rows, cols);
 }
 int mni_rocm_axpy(float *dst, const float *src, float alpha, int64_t n) {
+    MNI_API_GUARD;
     if (n < 0) return set_error(MNI_ERR_INVALID, "axpy: negative length");
     if (n > 0 && (!dst || !src)) return set_error(MNI_ERR_INVALID, "axpy: null argument");
     return k_axpy(dst, src, alpha, n);
 }
 int mni_rocm_fill(float *dst, float value, int64_t n) {
+    MNI_API_GUARD;
     if (n < 0) return set_error(MNI_ERR_INVALID, "fill: negative length");
     if (n > 0 && !dst) return set_error(MNI_ERR_INVALID, "fill: null argument");
     return k_fill(dst, value, n);

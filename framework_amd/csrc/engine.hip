@@ -1013,16 +1013,19 @@ using namespace mni;
 extern "C" {
 
 uint32_t mni_zeros(const int64_t *shape, int ndim) {
+    MNI_API_GUARD;
     Shape s;
     if (ensure_init() != MNI_OK || !to_shape(shape, ndim, &s)) return MNI_BAD_ID;
     return zeros(s);
 }
 uint32_t mni_ones(const int64_t *shape, int ndim) {
+    MNI_API_GUARD;
     Shape s;
     if (ensure_init() != MNI_OK || !to_shape(shape, ndim, &s)) return MNI_BAD_ID;
     return filled(s, 1.0f);
 }
 uint32_t mni_from_float32(const float *data, size_t len, const int64_t *shape, int ndim) {
+    MNI_API_GUARD;
     Shape s;
     if (ensure_init() != MNI_OK || !to_shape(shape, ndim, &s)) return MNI_BAD_ID;
     const int64_t n = shape_size(s);
@@ -1035,16 +1038,19 @@ uint32_t mni_from_float32(const float *data, size_t len, const int64_t *shape, i
     return insert_contig(std::move(b), s);
 }
 int mni_tensor_shape(uint32_t id, int64_t *out, int cap) {
+    MNI_API_GUARD;
     Tensor *t = get(id);
     if (!t) return -1;
     for (int i = 0; i < (int)t->shape.size() && i < cap; ++i) out[i] = t->shape[i];
     return (int)t->shape.size();
 }
 int64_t mni_tensor_size(uint32_t id) {
+    MNI_API_GUARD;
     Tensor *t = get(id);
     return t ? t->size : -1;
 }
 int mni_to_float32(uint32_t id, float *out, size_t cap) {
+    MNI_API_GUARD;
     Tensor *t = get(id);
     if (!t) return MNI_ERR_FREED;
     if ((int64_t)cap < t->size) return set_error(MNI_ERR_INVALID, "to_float32: buffer of %zu for %lld elements", cap, (long long)t->size);
@@ -1053,6 +1059,7 @@ int mni_to_float32(uint32_t id, float *out, size_t cap) {
     return mni_rocm_d2h(out, b->p, (size_t)t->size * sizeof(float));
 }
 int mni_get_scalar(uint32_t id, double *out) {
+    MNI_API_GUARD;
     Tensor *t = get(id);
     if (!t) return MNI_ERR_FREED;
     float v = 0.f;
@@ -1060,14 +1067,16 @@ int mni_get_scalar(uint32_t id, double *out) {
     *out = (double)v;
     return MNI_OK;
 }
-void mni_free_tensor(uint32_t id) { free_tensor(id); }
+void mni_free_tensor(uint32_t id) { MNI_API_GUARD; free_tensor(id); }
 int mni_set_requires_grad(uint32_t id, int requires_) {
+    MNI_API_GUARD;
     Tensor *t = get(id);
     if (!t) return MNI_ERR_FREED;
     t->requires_grad = requires_ != 0;
     return MNI_OK;
 }
 int mni_get_grad(uint32_t id, uint32_t *out) {
+    MNI_API_GUARD;
     Tensor *t = get(id);
     if (!t) return -1;
     if (t->grad < 0) return 0;
@@ -1075,12 +1084,14 @@ int mni_get_grad(uint32_t id, uint32_t *out) {
     return 1;
 }
 int mni_backward(uint32_t loss) {
+    MNI_API_GUARD;
     // The tape is consumed and replaced by a fresh, enabled one (lib.rs:135).
     Tape old = std::move(eng().tape);
     eng().tape = Tape();
     return tape_backward(old, loss);
 }
 int mni_zero_grad(const uint32_t *ids, size_t n) {
+    MNI_API_GUARD;
     for (size_t p = 0; p < n; ++p) {
         Tensor *t = get(ids[p]);
         if (!t) return MNI_ERR_FREED;
@@ -1095,18 +1106,19 @@ int mni_zero_grad(const uint32_t *ids, size_t n) {
     }
     return MNI_OK;
 }
-void mni_no_grad_start(void) { eng().tape.enabled = false; }
-void mni_no_grad_end(void) { eng().tape.enabled = true; }
+void mni_no_grad_start(void) { MNI_API_GUARD; eng().tape.enabled = false; }
+void mni_no_grad_end(void) { MNI_API_GUARD; eng().tape.enabled = true; }
 
-uint32_t mni_add(uint32_t a, uint32_t b) { return binary_op(a, b, BIN_ADD); }
-uint32_t mni_mul(uint32_t a, uint32_t b) { return binary_op(a, b, BIN_MUL); }
-uint32_t mni_sub(uint32_t a, uint32_t b) { return binary_op(a, b, BIN_SUB); }
-uint32_t mni_neg(uint32_t a) { return unary_op(a, UN_NEG, OP_NEG, 0.f); }
-uint32_t mni_mul_scalar(uint32_t a, double s) { return unary_op(a, UN_SCALE, OP_MULSCALAR, (float)s); }
-uint32_t mni_gelu(uint32_t a) { return unary_op(a, UN_GELU, OP_GELU, 0.f); }
-uint32_t mni_relu(uint32_t a) { return unary_op(a, UN_RELU, OP_RELU, 0.f); }
+uint32_t mni_add(uint32_t a, uint32_t b) { MNI_API_GUARD; return binary_op(a, b, BIN_ADD); }
+uint32_t mni_mul(uint32_t a, uint32_t b) { MNI_API_GUARD; return binary_op(a, b, BIN_MUL); }
+uint32_t mni_sub(uint32_t a, uint32_t b) { MNI_API_GUARD; return binary_op(a, b, BIN_SUB); }
+uint32_t mni_neg(uint32_t a) { MNI_API_GUARD; return unary_op(a, UN_NEG, OP_NEG, 0.f); }
+uint32_t mni_mul_scalar(uint32_t a, double s) { MNI_API_GUARD; return unary_op(a, UN_SCALE, OP_MULSCALAR, (float)s); }
+uint32_t mni_gelu(uint32_t a) { MNI_API_GUARD; return unary_op(a, UN_GELU, OP_GELU, 0.f); }
+uint32_t mni_relu(uint32_t a) { MNI_API_GUARD; return unary_op(a, UN_RELU, OP_RELU, 0.f); }
 
 uint32_t mni_matmul(uint32_t a, uint32_t b) {
+    MNI_API_GUARD;
     const uint32_t out = matmul_tensors(a, false, b, false, nullptr, MNI_EPI_NONE);
     if (out == MNI_BAD_ID) return out;
     Entry e;
@@ -1114,11 +1126,12 @@ uint32_t mni_matmul(uint32_t a, uint32_t b) {
     eng().tape.record(std::move(e));
     return out;
 }
-uint32_t mni_linear(uint32_t x, uint32_t w, uint32_t bias, int act) { return linear_op(x, w, bias, act); }
+uint32_t mni_linear(uint32_t x, uint32_t w, uint32_t bias, int act) { MNI_API_GUARD; return linear_op(x, w, bias, act); }
 
-uint32_t mni_sum_op(uint32_t a, int64_t dim) { return reduce_op(a, dim, false); }
-uint32_t mni_mean_op(uint32_t a, int64_t dim) { return reduce_op(a, dim, true); }
+uint32_t mni_sum_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return reduce_op(a, dim, false); }
+uint32_t mni_mean_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return reduce_op(a, dim, true); }
 uint32_t mni_sum_all(uint32_t a) {
+    MNI_API_GUARD;
     Tensor *t = get(a);
     if (!t) return MNI_BAD_ID;
     uint32_t cur = a;
@@ -1126,6 +1139,7 @@ uint32_t mni_sum_all(uint32_t a) {
     return cur;
 }
 uint32_t mni_mean_all(uint32_t a) {
+    MNI_API_GUARD;
     Tensor *t = get(a);
     if (!t) return MNI_BAD_ID;
     uint32_t cur = a;
@@ -1133,11 +1147,13 @@ uint32_t mni_mean_all(uint32_t a) {
     return cur;
 }
 uint32_t mni_view(uint32_t a, const int64_t *shape, int ndim) {
+    MNI_API_GUARD;
     Shape s;
     if (!to_shape(shape, ndim, &s)) return MNI_BAD_ID;
     return view_op(a, s);
 }
 uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim) {
+    MNI_API_GUARD;
     Shape s;
     if (!to_shape(dims, ndim, &s)) return MNI_BAD_ID;
     return permute_op(a, s);
@@ -1156,14 +1172,17 @@ uint32_t mni_contiguous(uint32_t a) {  // layout.rs:218-227
     return id;
 }
 uint32_t mni_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n) {
+    MNI_API_GUARD;
     if (!targets) { set_error(MNI_ERR_INVALID, "cross_entropy: null targets"); return MNI_BAD_ID; }
     return cross_entropy_op(logits, targets, n);
 }
 int mni_adamw_step(const uint32_t *ids, size_t n, double lr, double beta1, double beta2, double eps,
                    double weight_decay, int64_t step) {
+    MNI_API_GUARD;
     return adamw_step(ids, n, (float)lr, (float)beta1, (float)beta2, (float)eps, (float)weight_decay, (uint32_t)step);
 }
 double mni_grad_norm(const uint32_t *ids, size_t n) {
+    MNI_API_GUARD;
     float norm = 0.f;
     if (grad_norm(ids, n, &norm) != MNI_OK) return -1.0;
     return (double)norm;
@@ -1187,12 +1206,14 @@ double mni_clip_and_step(const uint32_t *ids, size_t n, double lr, double beta1,
     return (double)norm;
 }
 void mni_reset_engine(void) {
+    MNI_API_GUARD;
     Engine &e = eng();
     e.tensors.clear();
     e.free_ids.clear();
     e.tape = Tape();
 }
 int mni_gc_tensors(const uint32_t *keep, size_t n) {
+    MNI_API_GUARD;
     Engine &e = eng();
     const size_t len = e.tensors.size();
     std::vector<char> k(len + 1, 0);
@@ -1208,6 +1229,7 @@ int mni_gc_tensors(const uint32_t *keep, size_t n) {
     return MNI_OK;
 }
 void *mni_dev_ptr(uint32_t id) {
+    MNI_API_GUARD;
     Tensor *t = get(id);
     return t ? (void *)t->buf->p : nullptr;
 }

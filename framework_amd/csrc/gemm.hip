@@ -239,11 +239,13 @@ int sgemm(const mni_gemm_desc &d) {
 }  // namespace mni
 
 extern "C" int mni_rocm_sgemm(const mni_gemm_desc *desc) {
+    MNI_API_GUARD;
     if (!desc) return mni::set_error(MNI_ERR_INVALID, "sgemm: null descriptor");
     return mni::sgemm(*desc);
 }
 
 extern "C" int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms) {
+    MNI_API_GUARD;
     using namespace mni;
     if (!descs || count <= 0 || iters <= 0 || warmup < 0 || !avg_ms)
         return set_error(MNI_ERR_INVALID, "sgemm_timed: bad arguments");

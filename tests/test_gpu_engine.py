@@ -463,3 +463,33 @@ def test_errors_where_the_reference_panics(gpu):
         t.matmul(other)
     with pytest.raises(N.MniError, match="out of range"):
         gpu.crossEntropyLoss(Tn.ones([2, 3]), [[0], [3]])
+
+
+def test_entry_points_serialise_concurrent_callers(rocm_native):
+    # The reference funnels every export through one mutex (src/native/src/lib.rs:27-39);
+    # ctypes drops the GIL during a call, so these threads really do race into the library.
+    import threading
+    T = rocm_native
+    errors = []
+
+    def worker(seed):
+        try:
+            for it in range(40):
+                a = synth.small_ints(seed + it, (17, 9), 3)
+                b = synth.small_ints(seed + it, (9, 23), 3, stream=1)
+                ia, ib = T.fromFloat32(a.ravel(), [17, 9]), T.fromFloat32(b.ravel(), [9, 23])
+                ic = T.matmul(ia, ib)
+                got = np.asarray(T.toFloat32(ic)).reshape(17, 23)
+                if not np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)):
+                    errors.append((seed, it))
+                for i in (ia, ib, ic):
+                    T.freeTensor(i)
+        except Exception as e:  # noqa: BLE001 - reported through the assertion below
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(100 * k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert errors == []
