@@ -200,6 +200,26 @@ def bench_extras(r):
         ids += [g for g in (api.native.getGrad(p.value._id) for p in params1) if g is not None]
         return ids
     out["config1_readme_mlp_step"] = {"ms": time_step(step1, keep1, 20, 5)}
+    # attention on the batched GEMM at the config-3 shapes: flashAttention(q, k, v) [32, 512, 64], causal
+    api.native.resetEngine()
+    bh, s, d = 32, 512, 64
+    qa, ka, va = (T(synth.normal(2, (bh, s, d), stream=i) / np.float32(8 if i < 2 else 1), True) for i in range(3))
+    wa = T(synth.normal(2, (bh, s, d), stream=3))
+
+    def keep_att():
+        ids = [t._id for t in (qa, ka, va, wa)]
+        return ids + [g for g in (api.native.getGrad(t._id) for t in (qa, ka, va)) if g is not None]
+    ms_fwd = time_step(lambda: api.flashAttention(qa, ka, va, 0.125, True), keep_att, 20, 5)
+
+    def att_step():
+        api.native.zeroGrad([qa._id, ka._id, va._id])
+        api.flashAttention(qa, ka, va, 0.125, True).mul(wa).sum().backward()
+    ms_all = time_step(att_step, keep_att, 20, 5)
+    dense = 2.0 * bh * s * s * d  # one s x s x d product, mask not exploited
+    out["attention_32x512x64_causal"] = {"fwd_ms": ms_fwd, "fwd_bwd_ms": ms_all,
+                                         "fwd_TFLOP/s_dense_count": 2 * dense / ms_fwd / 1e9,
+                                         "fwd_bwd_TFLOP/s_dense_count": 7 * dense / ms_all / 1e9,
+                                         "note": "wall clock per call incl. host issue and a trailing sync; 2 products forward, 5 backward"}
     api.native.resetEngine()
     return out
 

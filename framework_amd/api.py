@@ -179,6 +179,12 @@ def bind(native):
         flat_targets = [int(t) for row in targets for t in (row if isinstance(row, (list, tuple, np.ndarray)) else [row])]
         return Tensor(native.crossEntropyLoss(flat._id, flat_targets))
 
+    def softmax(x, dim=-1):  # src/nn.ts:77-79
+        return Tensor(native.softmaxOp(x._id, dim))
+
+    def flashAttention(q, k, v, scale, causal=True):  # src/nn.ts:107-110
+        return Tensor(native.flashAttention(q._id, k._id, v._id, scale, causal))
+
     class Adam:  # src/optimizer.ts:33-70: options object, defaults lr 6e-4, beta2 0.95
         def __init__(self, parameters, lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weightDecay=0.0):
             self.parameters = list(parameters)
@@ -194,4 +200,5 @@ def bind(native):
             return native.clipAndStep(ids, self.lr, self.beta1, self.beta2, self.eps, self.weightDecay, self.t, maxGradNorm)
 
     return SimpleNamespace(native=native, Tensor=Tensor, Parameter=Parameter, Module=Module, Linear=Linear, ReLU=ReLU,
-                           GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, Adam=Adam)
+                           GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, softmax=softmax,
+                           flashAttention=flashAttention, Adam=Adam)

@@ -100,6 +100,14 @@ int k_cross_entropy(float *loss, float *softmax, const float *logits, const int3
                     int64_t n, int64_t v);
 int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t *targets,
                              const float *grad_scalar, int64_t n, int64_t v);
+// attention.hip
+int k_softmax(float *out, const float *x, int64_t outer, int64_t n, int64_t inner);
+int k_softmax_backward(float *out, const float *sm, const float *g, int64_t outer, int64_t n, int64_t inner);
+int k_attn_softmax(float *scores, float *lse, int64_t rows, int64_t s, float scale, int causal);
+int k_rowdot(float *out, const float *a, const float *b, int64_t rows, int64_t d);
+int k_attn_backward(float *scores, float *dp, const float *lse, const float *di, int64_t rows, int64_t s, float scale,
+                    int causal);
+
 int k_sumsq_f64(double *out, const float *g, int64_t n);  // out += sum g^2 (device double)
 int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, float b1, float b2,
             float eps, float wd, float bc1, float bc2);

@@ -49,7 +49,8 @@ struct Tensor {
 
 enum Op {  // subset of src/native/src/autograd.rs:28-62 plus the fused Linear
     OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
-    OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY, OP_LINEAR
+    OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY, OP_LINEAR,
+    OP_SOFTMAX, OP_FLASHATTENTION
 };
 
 // src/native/src/autograd.rs:65-70 TapeEntry
@@ -62,7 +63,8 @@ struct Entry {
     Shape saved_perm;
     float scalar = 0.f;
     int act = 0;         // OP_LINEAR: epilogue
-    uint32_t aux = MNI_BAD_ID;  // cross-entropy softmax / linear pre-activation
+    uint32_t aux = MNI_BAD_ID;  // cross-entropy softmax / linear pre-activation / softmax output / attention output
+    uint32_t aux2 = MNI_BAD_ID; // attention log-sum-exp
     std::shared_ptr<void> targets;  // device int32 targets
     int64_t ce_n = 0, ce_v = 0;
 };
@@ -765,6 +767,126 @@ static int cross_entropy_backward(uint32_t grad, const Entry &e, int64_t *out) {
     return MNI_OK;
 }
 
+// ---- softmax -----------------------------------------------------------------------------------
+// ops/norm.rs:10-50.  The tape keeps the dim as it was passed (:47).
+static uint32_t softmax_op(uint32_t a, int64_t dim) {
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    const Shape shape = A->shape;
+    const int nd = (int)shape.size();
+    const int d = (int)(dim < 0 ? nd + dim : dim);
+    if (d < 0 || d >= nd) { set_error(MNI_ERR_INVALID, "softmax: dim %lld out of range for %d dims", (long long)dim, nd); return MNI_BAD_ID; }
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < d; ++i) outer *= shape[i];
+    for (int i = d + 1; i < nd; ++i) inner *= shape[i];
+    BufP src = contiguous_buf(*A);
+    BufP out = src ? new_buf((size_t)A->size) : nullptr;
+    if (!out || k_softmax(out->p, src->p, outer, shape[d], inner) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(out), shape);
+    Entry e;
+    e.op = OP_SOFTMAX; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a; e.scalar = (float)dim; e.aux = id;
+    eng().tape.record(std::move(e));
+    return id;
+}
+// ops/norm.rs:96-123.  The saved dim is read back with Rust's saturating
+// `as usize`, so a negative dim (the TypeScript default -1, src/nn.ts:77)
+// reduces along dim 0 in the reference; kept so that gradients match it.
+static int softmax_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *G = get(grad), *S = get(e.aux);
+    if (!G || !S) return MNI_ERR_FREED;
+    const Shape shape = S->shape;
+    const int nd = (int)shape.size();
+    const int d = e.scalar > 0.f ? (int)e.scalar : 0;
+    if (d >= nd) return set_error(MNI_ERR_INVALID, "softmax backward: dim %d out of range", d);
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < d; ++i) outer *= shape[i];
+    for (int i = d + 1; i < nd; ++i) inner *= shape[i];
+    BufP g = contiguous_buf(*G), sm = contiguous_buf(*S);
+    BufP o = (g && sm) ? new_buf((size_t)S->size) : nullptr;
+    if (!o) return MNI_ERR_NOMEM;
+    MNI_TRY(k_softmax_backward(o->p, sm->p, g->p, outer, shape[d], inner));
+    out[0] = insert_contig(std::move(o), shape);
+    return MNI_OK;
+}
+
+// ---- attention on the batched GEMM ----------------------------------------------------------------
+// One batched product through the kernel-level entry: C[b] = op(A)[b] op(B)[b],
+// operands given as contiguous [bh, rows, cols] buffers, optionally transposed.
+static int attn_gemm(float *c, const float *a, bool ta, const float *b, bool tb, int64_t bh, int64_t m, int64_t n,
+                     int64_t k) {
+    mni_gemm_desc d;
+    memset(&d, 0, sizeof d);
+    d.M = m; d.N = n; d.K = k; d.batch = bh;
+    // a is stored [bh][m][k] (or [bh][k][m] when ta); b is [bh][k][n] (or [bh][n][k] when tb)
+    d.A = ta ? mni_operand{a, 1, m, k * m, bh} : mni_operand{a, k, 1, m * k, bh};
+    d.B = tb ? mni_operand{b, 1, k, n * k, bh} : mni_operand{b, n, 1, k * n, bh};
+    d.C = c; d.ldc = n; d.c_batch_stride = m * n;
+    return sgemm(d);
+}
+
+// ops/attention.rs:14-78: q, k, v are taken as [bh, s, d] from their first
+// three dims.  scores = q k^T and out = P v run on the GEMM kernels; the row
+// kernel in between applies scale, the causal mask and the normalisation and
+// leaves lse = max + ln(sum) for the backward pass.
+static uint32_t flash_attention_op(uint32_t q, uint32_t k, uint32_t v, float scale, bool causal) {
+    Tensor *Q = get(q), *K = get(k), *V = get(v);
+    if (!Q || !K || !V) return MNI_BAD_ID;
+    if (Q->shape.size() < 3) { set_error(MNI_ERR_INVALID, "flash_attention: q must be [bh, s, d]"); return MNI_BAD_ID; }
+    const int64_t bh = Q->shape[0], s = Q->shape[1], d = Q->shape[2];
+    const int64_t total = bh * s * d;
+    if (K->size < total || V->size < total) {
+        set_error(MNI_ERR_INVALID, "flash_attention: k / v hold fewer than bh*s*d = %lld values", (long long)total);
+        return MNI_BAD_ID;
+    }
+    BufP qc = contiguous_buf(*Q), kc = contiguous_buf(*K), vc = contiguous_buf(*V);
+    BufP scores = (qc && kc && vc) ? new_buf((size_t)(bh * s * s)) : nullptr;
+    BufP lse = scores ? new_buf((size_t)(bh * s)) : nullptr;
+    BufP out = lse ? new_buf((size_t)total) : nullptr;
+    if (!out) return MNI_BAD_ID;
+    if (total > 0) {
+        if (attn_gemm(scores->p, qc->p, false, kc->p, true, bh, s, s, d) != MNI_OK) return MNI_BAD_ID;
+        if (k_attn_softmax(scores->p, lse->p, bh * s, s, scale, causal ? 1 : 0) != MNI_OK) return MNI_BAD_ID;
+        if (attn_gemm(out->p, scores->p, false, vc->p, false, bh, s, d, s) != MNI_OK) return MNI_BAD_ID;
+    }
+    const uint32_t out_id = insert_contig(std::move(out), Shape{bh, s, d});
+    const uint32_t lse_id = insert_contig(std::move(lse), Shape{bh, s});
+    Entry e;
+    e.op = OP_FLASHATTENTION; e.output_id = out_id; e.n_inputs = 3;
+    e.inputs[0] = q; e.inputs[1] = k; e.inputs[2] = v;
+    e.aux = out_id; e.aux2 = lse_id; e.scalar = scale; e.act = causal ? 1 : 0;
+    eng().tape.record(std::move(e));
+    return out_id;
+}
+// ops/attention.rs:143-202: di = rowsum(dO * O); P recomputed from lse;
+// dV = P^T dO, dP = dO V^T, dS = P (dP - di) scale, dQ = dS K, dK = dS^T Q.
+static int flash_attention_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *Q = get(e.inputs[0]), *K = get(e.inputs[1]), *V = get(e.inputs[2]);
+    Tensor *O = get(e.aux), *L = get(e.aux2), *G = get(grad);
+    if (!Q || !K || !V || !O || !L || !G) return MNI_ERR_FREED;
+    const int64_t bh = Q->shape[0], s = Q->shape[1], d = Q->shape[2];
+    const int64_t total = bh * s * d;
+    BufP qc = contiguous_buf(*Q), kc = contiguous_buf(*K), vc = contiguous_buf(*V);
+    BufP oc = contiguous_buf(*O), lc = contiguous_buf(*L), gc = contiguous_buf(*G);
+    if (!qc || !kc || !vc || !oc || !lc || !gc) return MNI_ERR_NOMEM;
+    BufP p = new_buf((size_t)(bh * s * s)), ds = new_buf((size_t)(bh * s * s)), di = new_buf((size_t)(bh * s));
+    BufP dq = new_buf((size_t)total), dk = new_buf((size_t)total), dv = new_buf((size_t)total);
+    if (!p || !ds || !di || !dq || !dk || !dv) return MNI_ERR_NOMEM;
+    if (total > 0) {
+        MNI_TRY(k_rowdot(di->p, gc->p, oc->p, bh * s, d));
+        MNI_TRY(attn_gemm(p->p, qc->p, false, kc->p, true, bh, s, s, d));   // q k^T
+        MNI_TRY(attn_gemm(ds->p, gc->p, false, vc->p, true, bh, s, s, d));  // dO v^T
+        MNI_TRY(k_attn_backward(p->p, ds->p, lc->p, di->p, bh * s, s, e.scalar, e.act));
+        MNI_TRY(attn_gemm(dv->p, p->p, true, gc->p, false, bh, s, d, s));   // P^T dO
+        MNI_TRY(attn_gemm(dq->p, ds->p, false, kc->p, false, bh, s, d, s)); // dS k
+        MNI_TRY(attn_gemm(dk->p, ds->p, true, qc->p, false, bh, s, d, s));  // dS^T q
+    }
+    const Shape shape{bh, s, d};
+    out[0] = insert_contig(std::move(dq), shape);
+    out[1] = insert_contig(std::move(dk), shape);
+    out[2] = insert_contig(std::move(dv), shape);
+    return MNI_OK;
+}
+
 // ---- fused Linear ------------------------------------------------------------------------------
 static uint32_t linear_op(uint32_t x, uint32_t w, uint32_t bias, int act) {
     Tensor *X = get(x), *W = get(w), *Bv = get(bias);
@@ -844,6 +966,8 @@ static int dispatch_backward(const Entry &e, uint32_t grad, int64_t *out) {  // 
     case OP_CONTIGUOUS: out[0] = grad; return MNI_OK;  // layout.rs:229-231
     case OP_CROSSENTROPY: return cross_entropy_backward(grad, e, out);
     case OP_LINEAR: return linear_backward(grad, e, out);
+    case OP_SOFTMAX: return softmax_backward(grad, e, out);                  // autograd.rs:204
+    case OP_FLASHATTENTION: return flash_attention_backward(grad, e, out);   // autograd.rs:210
     }
     return set_error(MNI_ERR_INVALID, "unknown tape op %d", e.op);
 }
@@ -1170,6 +1294,11 @@ uint32_t mni_contiguous(uint32_t a) {  // layout.rs:218-227
     e.op = OP_CONTIGUOUS; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a;
     eng().tape.record(std::move(e));
     return id;
+}
+uint32_t mni_softmax_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return softmax_op(a, dim); }
+uint32_t mni_flash_attention(uint32_t q, uint32_t k, uint32_t v, double scale, int causal) {
+    MNI_API_GUARD;
+    return flash_attention_op(q, k, v, (float)scale, causal != 0);
 }
 uint32_t mni_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n) {
     MNI_API_GUARD;

@@ -122,6 +122,7 @@ UNARY(Gelu, mni_gelu)                    // lib.rs:206-211
 UNARY(Relu, mni_relu)                    // lib.rs:213-218
 WITH_DIM(SumOp, mni_sum_op)              // lib.rs:234-239
 WITH_DIM(MeanOp, mni_mean_op)            // lib.rs:241-246
+WITH_DIM(SoftmaxOp, mni_softmax_op)      // lib.rs:302-307
 UNARY(SumAll, mni_sum_all)               // lib.rs:255-265
 UNARY(MeanAll, mni_mean_all)             // lib.rs:267-277
 WITH_SHAPE(View, mni_view)               // lib.rs:279-285
@@ -255,6 +256,11 @@ napi_value GcTensors(napi_env env, napi_callback_info info) {  // lib.rs:693-706
     return ret_rc(env, mni_gc_tensors(ids.data(), ids.size()));
 }
 // Opt-in fused Linear (no counterpart in lib.rs; feature-detected by callers).
+napi_value FlashAttention(napi_env env, napi_callback_info info) {  // lib.rs:575-584
+    Args a(env, info);
+    return ret_id(env, mni_flash_attention(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_u32(env, a.v[2]),
+                                           get_f64(env, a.v[3]), get_bool(env, a.v[4]) ? 1 : 0));
+}
 napi_value Linear(napi_env env, napi_callback_info info) {
     Args a(env, info);
     const int act = a.n > 3 ? (int)get_i64(env, a.v[3]) : MNI_EPI_BIAS;
@@ -277,6 +283,7 @@ NAPI_MODULE_INIT() {
         EXPORT("contiguous", Contiguous), EXPORT("crossEntropyLoss", CrossEntropyLoss), EXPORT("adamwStep", AdamwStep),
         EXPORT("gradNorm", GradNorm), EXPORT("clipGradNorm", ClipGradNorm), EXPORT("clipAndStep", ClipAndStep),
         EXPORT("resetEngine", ResetEngine), EXPORT("gcTensors", GcTensors), EXPORT("linear", Linear),
+        EXPORT("softmaxOp", SoftmaxOp), EXPORT("flashAttention", FlashAttention),
 #undef EXPORT
     };
     napi_define_properties(env, exports, sizeof(props) / sizeof(props[0]), props);

@@ -100,6 +100,8 @@ SIGNATURES = {
     "mni_view": (C.c_uint32, [C.c_uint32, _i64p, C.c_int]),
     "mni_permute": (C.c_uint32, [C.c_uint32, _i64p, C.c_int]),
     "mni_contiguous": (C.c_uint32, [C.c_uint32]),
+    "mni_softmax_op": (C.c_uint32, [C.c_uint32, C.c_int64]),
+    "mni_flash_attention": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double, C.c_int]),
     "mni_cross_entropy_loss": (C.c_uint32, [C.c_uint32, _i64p, C.c_size_t]),
     "mni_adamw_step": (C.c_int, [_u32p, C.c_size_t, C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, C.c_int64]),
     "mni_grad_norm": (C.c_double, [_u32p, C.c_size_t]),
@@ -382,6 +384,12 @@ class Native:
 
     def contiguous(self, a):
         return self._id(self.lib.mni_contiguous(a))
+
+    def softmaxOp(self, a, dim):
+        return self._id(self.lib.mni_softmax_op(a, dim))
+
+    def flashAttention(self, q, k, v, scale, causal):
+        return self._id(self.lib.mni_flash_attention(q, k, v, scale, 1 if causal else 0))
 
     def crossEntropyLoss(self, logits, targets):
         return self._id(self.lib.mni_cross_entropy_loss(logits, _i64_array(targets), len(targets)))

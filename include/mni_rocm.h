@@ -175,7 +175,16 @@ uint32_t mni_sum_all(uint32_t a);                                         /* lib
 uint32_t mni_mean_all(uint32_t a);                                        /* lib.rs:267-277 */
 uint32_t mni_view(uint32_t a, const int64_t *shape, int ndim);            /* lib.rs:279-285 */
 uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim);          /* lib.rs:287-293 */
-uint32_t mni_contiguous(uint32_t a);                                      /* lib.rs:295-300 */
+uint32_t mni_contiguous(uint32_t a);                                      /* softmax_op (src/native/src/lib.rs:302-307 -> ops/norm.rs:10-50); backward as
+ * ops/norm.rs:96-123, including its reading of a negative saved dim as dim 0. */
+uint32_t mni_softmax_op(uint32_t a, int64_t dim);
+/* flash_attention (src/native/src/lib.rs:575-584 -> ops/attention.rs:14-78,
+ * backward :143-202): q, k, v taken as [bh, s, d] from their first three dims;
+ * returns out [bh, s, d].  Built on the batched GEMM (q k^T, P v and the five
+ * backward products) with row kernels for scale / causal mask / normalisation,
+ * in place of the per-key loop of kernels/flash_attention.cu. */
+uint32_t mni_flash_attention(uint32_t q, uint32_t k, uint32_t v, double scale, int causal);
+/* lib.rs:295-300 */
 uint32_t mni_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n); /* lib.rs:328-336 */
 int mni_adamw_step(const uint32_t *ids, size_t n, double lr, double beta1, double beta2,
                    double eps, double weight_decay, int64_t step);        /* lib.rs:400-412 */

@@ -51,22 +51,25 @@ typedef struct {
 
 enum orc_op { /* subset of autograd.rs:28-62 BackwardOp */
     OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
-    OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY
+    OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY,
+    OP_SOFTMAX, OP_FLASHATTENTION
 };
 
 /* autograd.rs:65-70 TapeEntry + the SavedContext variants the subset needs */
 typedef struct {
     int op;
     size_t output_id;
-    size_t input_ids[2];
+    size_t input_ids[3];
     int n_inputs;
-    size_t saved_ids[2];          /* Tensor / Tensors / TensorsAndShape ids  */
+    size_t saved_ids[3];          /* Tensor / Tensors / TensorsAndShape ids  */
     size_t saved_shape[ORC_MAX_DIMS]; /* Shape / TensorAndShape / Permutation orig */
     int saved_ndim;
     size_t saved_perm[ORC_MAX_DIMS];
     float saved_scalar;
     size_t *targets;              /* Indices(targets, n, v, sm_id)           */
     size_t ce_n, ce_v, ce_sm;
+    size_t fa_out, fa_lse;        /* FlashAttention{q,k,v,out,lse,scale,s,d,causal} */
+    int fa_causal;
 } orc_entry;
 
 typedef struct {
@@ -827,11 +830,196 @@ static int cross_entropy_backward(size_t grad, const orc_entry *e, long *out) {
     return 0;
 }
 
+/* ---- softmax ------------------------------------------------------------ */
+
+/* ops/norm.rs:10-50 softmax, cpu arm: per (outer, inner) line -- running max,
+ * exp(x - max) stored and summed in index order, then divided by the sum.
+ * The tape keeps `dim as f32` exactly as passed (possibly negative), :47.
+ * pinned by: test/nn.test.ts:46-54 (rows of [1,2,3] sum to 1, positive,
+ * ordered), float64 closed form on random lines, shift invariance. */
+static uint32_t softmax_impl(size_t a, int dim) {
+    orc_tensor *A = get(a);
+    if (!A) return fail("tensor already freed");
+    int nd = A->ndim;
+    size_t shape[ORC_MAX_DIMS];
+    memcpy(shape, A->shape, sizeof shape);
+    int d = dim < 0 ? nd + dim : dim; /* :13 */
+    if (d < 0 || d >= nd) return fail("index out of bounds: softmax dim");
+    float *x = to_host(A);
+    size_t total = shape_size(shape, nd), dim_size = shape[d];
+    size_t outer = 1, inner = 1;
+    for (int i = 0; i < d; ++i) outer *= shape[i];
+    for (int i = d + 1; i < nd; ++i) inner *= shape[i];
+    if (outer < 1) outer = 1;
+    if (inner < 1) inner = 1;
+    float *out = (float *)calloc(total ? total : 1, sizeof(float));
+    for (size_t o = 0; o < outer; ++o)
+        for (size_t i = 0; i < inner; ++i) {
+            float mx = -INFINITY;
+            for (size_t t = 0; t < dim_size; ++t) {
+                float v = x[o * dim_size * inner + t * inner + i];
+                mx = v > mx ? v : mx;
+            }
+            float sum = 0.0f;
+            for (size_t t = 0; t < dim_size; ++t) {
+                size_t idx = o * dim_size * inner + t * inner + i;
+                float e = expf(x[idx] - mx);
+                out[idx] = e;
+                sum += e;
+            }
+            for (size_t t = 0; t < dim_size; ++t) out[o * dim_size * inner + t * inner + i] /= sum;
+        }
+    free(x);
+    size_t out_id = from_vec(out, shape, nd);
+    orc_entry *e = tape_record(&g_tape, OP_SOFTMAX, out_id, 1, a, 0);
+    e->saved_scalar = (float)dim; /* ScalarAndTensor(dim as f32, out_id) */
+    e->saved_ids[0] = out_id;
+    return (uint32_t)out_id;
+}
+
+/* ops/norm.rs:96-123 softmax_backward: dx = sm * (g - sum(g * sm)) along the
+ * saved dim.  The dim comes back as `*dim_f as usize`: Rust's float-to-integer
+ * cast saturates, so a NEGATIVE saved dim (softmax(x, -1), the TypeScript
+ * default, src/nn.ts:77) becomes 0 and the reduction runs along dim 0 --
+ * reproduced here as the reference behaves, not as it presumably intends.
+ * pinned by: float64 Jacobian-vector product for dim >= 0; for dim = -1 on a
+ * 2-D input the result must equal the dim-0 formula (tests/test_oracle_attention.py). */
+static int softmax_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *S = get(e->saved_ids[0]), *G = get(grad);
+    if (!S || !G) { fail("tensor already freed"); return -1; }
+    int nd = S->ndim;
+    size_t shape[ORC_MAX_DIMS];
+    memcpy(shape, S->shape, sizeof shape);
+    size_t d = e->saved_scalar > 0.0f ? (size_t)e->saved_scalar : 0; /* saturating cast */
+    if ((int)d >= nd) { fail("index out of bounds: softmax dim"); return -1; }
+    float *sm = to_host(S), *g = to_host(G);
+    size_t total = shape_size(shape, nd), dim_size = shape[d];
+    size_t outer = 1, inner = 1;
+    for (size_t i = 0; i < d; ++i) outer *= shape[i];
+    for (int i = (int)d + 1; i < nd; ++i) inner *= shape[i];
+    if (outer < 1) outer = 1;
+    if (inner < 1) inner = 1;
+    float *o_ = (float *)calloc(total ? total : 1, sizeof(float));
+    for (size_t o = 0; o < outer; ++o)
+        for (size_t i = 0; i < inner; ++i) {
+            float dot = 0.0f;
+            for (size_t t = 0; t < dim_size; ++t) {
+                size_t idx = o * dim_size * inner + t * inner + i;
+                dot += g[idx] * sm[idx];
+            }
+            for (size_t t = 0; t < dim_size; ++t) {
+                size_t idx = o * dim_size * inner + t * inner + i;
+                o_[idx] = sm[idx] * (g[idx] - dot);
+            }
+        }
+    free(sm); free(g);
+    out[0] = (long)from_vec(o_, shape, nd);
+    return 0;
+}
+
+/* ---- attention ---------------------------------------------------------- */
+
+/* ops/attention.rs:14-78 flash_attention, cpu arm.  q, k, v are read as
+ * [bh, s, d] from their first three dims (:21-24); per (b, row) an online
+ * softmax over col < col_end (row + 1 when causal): running max, running sum
+ * and accumulator rescaled by exp(old_max - new_max) (:41-53), then
+ * out = acc / sum and lse = max + ln(sum) (:56-60).
+ * pinned by: float64 softmax(q k^T scale) v with and without the causal mask,
+ * v = ones -> out = ones, causal row 0 = v[0], equal scores -> mean of v,
+ * lse against float64 log-sum-exp (tests/test_oracle_attention.py). */
+static uint32_t flash_attention_impl(size_t q, size_t k, size_t v, float scale, int causal) {
+    orc_tensor *Q = get(q), *K = get(k), *V = get(v);
+    if (!Q || !K || !V) return fail("tensor already freed");
+    if (Q->ndim < 3) return fail("index out of bounds: flash_attention needs [bh, s, d]");
+    size_t bh = Q->shape[0], s = Q->shape[1], d = Q->shape[2];
+    if (K->size < bh * s * d || V->size < bh * s * d) return fail("index out of bounds: flash_attention k/v shorter than q");
+    float *qd = to_host(Q), *kd = to_host(K), *vd = to_host(V);
+    float *out = (float *)calloc((bh * s * d) > 0 ? bh * s * d : 1, sizeof(float));
+    float *lse = (float *)calloc((bh * s) > 0 ? bh * s : 1, sizeof(float));
+    float *acc = (float *)malloc((d ? d : 1) * sizeof(float));
+    for (size_t b = 0; b < bh; ++b)
+        for (size_t row = 0; row < s; ++row) {
+            size_t col_end = causal ? row + 1 : s;
+            float running_max = -INFINITY, running_sum = 0.0f;
+            for (size_t dd = 0; dd < d; ++dd) acc[dd] = 0.0f;
+            for (size_t col = 0; col < col_end; ++col) {
+                float dot = 0.0f;
+                for (size_t dd = 0; dd < d; ++dd) dot += qd[b * s * d + row * d + dd] * kd[b * s * d + col * d + dd];
+                dot *= scale;
+                float old_max = running_max;
+                running_max = running_max > dot ? running_max : dot; /* f32::max */
+                float exp_diff = expf(old_max - running_max);
+                running_sum = running_sum * exp_diff + expf(dot - running_max);
+                for (size_t dd = 0; dd < d; ++dd)
+                    acc[dd] = acc[dd] * exp_diff + expf(dot - running_max) * vd[b * s * d + col * d + dd];
+            }
+            float inv_sum = 1.0f / running_sum;
+            for (size_t dd = 0; dd < d; ++dd) out[b * s * d + row * d + dd] = acc[dd] * inv_sum;
+            lse[b * s + row] = running_max + logf(running_sum);
+        }
+    free(acc); free(qd); free(kd); free(vd);
+    size_t oshape[3] = {bh, s, d}, lshape[2] = {bh, s};
+    size_t out_id = from_vec(out, oshape, 3);
+    size_t lse_id = from_vec(lse, lshape, 2);
+    orc_entry *e = tape_record(&g_tape, OP_FLASHATTENTION, out_id, 3, q, k);
+    e->input_ids[2] = v; e->saved_ids[2] = v;
+    e->fa_out = out_id; e->fa_lse = lse_id; e->saved_scalar = scale; e->fa_causal = causal;
+    return (uint32_t)out_id;
+}
+
+/* ops/attention.rs:143-202 flash_attention_backward, cpu arm: di = sum(dO * O)
+ * per row, p = exp(dot * scale - lse), dv += p dO, dp = dO . v,
+ * ds = p (dp - di) scale, dq += ds k, dk += ds q, all accumulated in f32 in
+ * (b, row, col) order.
+ * pinned by: float64 central finite differences of sum(w * out) in q, k, v
+ * (causal and not), sum over rows of dS = 0 identity through dq for k = const. */
+static int flash_attention_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *Q = get(e->input_ids[0]), *K = get(e->input_ids[1]), *V = get(e->input_ids[2]);
+    orc_tensor *O = get(e->fa_out), *L = get(e->fa_lse), *G = get(grad);
+    if (!Q || !K || !V || !O || !L || !G) { fail("tensor already freed"); return -1; }
+    size_t bh = Q->shape[0], s = Q->shape[1], d = Q->shape[2];
+    float scale = e->saved_scalar;
+    float *qd = to_host(Q), *kd = to_host(K), *vd = to_host(V), *od = to_host(O), *ld = to_host(L), *gd = to_host(G);
+    size_t total = bh * s * d;
+    float *dq = (float *)calloc(total ? total : 1, sizeof(float));
+    float *dk = (float *)calloc(total ? total : 1, sizeof(float));
+    float *dv = (float *)calloc(total ? total : 1, sizeof(float));
+    for (size_t b = 0; b < bh; ++b)
+        for (size_t row = 0; row < s; ++row) {
+            size_t col_end = e->fa_causal ? row + 1 : s;
+            float lse_val = ld[b * s + row];
+            float di = 0.0f;
+            for (size_t dd = 0; dd < d; ++dd) di += gd[b * s * d + row * d + dd] * od[b * s * d + row * d + dd];
+            for (size_t col = 0; col < col_end; ++col) {
+                float dot = 0.0f;
+                for (size_t dd = 0; dd < d; ++dd) dot += qd[b * s * d + row * d + dd] * kd[b * s * d + col * d + dd];
+                dot *= scale;
+                float p = expf(dot - lse_val);
+                float dp = 0.0f;
+                for (size_t dd = 0; dd < d; ++dd) {
+                    dp += gd[b * s * d + row * d + dd] * vd[b * s * d + col * d + dd];
+                    dv[b * s * d + col * d + dd] += p * gd[b * s * d + row * d + dd];
+                }
+                float ds = p * (dp - di) * scale;
+                for (size_t dd = 0; dd < d; ++dd) {
+                    dq[b * s * d + row * d + dd] += ds * kd[b * s * d + col * d + dd];
+                    dk[b * s * d + col * d + dd] += ds * qd[b * s * d + row * d + dd];
+                }
+            }
+        }
+    free(qd); free(kd); free(vd); free(od); free(ld); free(gd);
+    size_t shape[3] = {bh, s, d};
+    out[0] = (long)from_vec(dq, shape, 3);
+    out[1] = (long)from_vec(dk, shape, 3);
+    out[2] = (long)from_vec(dv, shape, 3);
+    return 0;
+}
+
 /* ---- backward ----------------------------------------------------------- */
 
 /* autograd.rs:180-222 dispatch_backward */
 static int dispatch_backward(const orc_entry *e, size_t grad, long *out) {
-    out[0] = out[1] = -1;
+    out[0] = out[1] = out[2] = -1;
     switch (e->op) {
     case OP_ADD: return addsub_backward(grad, e, out, 0);
     case OP_SUB: return addsub_backward(grad, e, out, 1);
@@ -844,6 +1032,8 @@ static int dispatch_backward(const orc_entry *e, size_t grad, long *out) {
     case OP_PERMUTE: return permute_backward(grad, e, out);
     case OP_CONTIGUOUS: out[0] = (long)grad; return 0; /* layout.rs:229-231 */
     case OP_CROSSENTROPY: return cross_entropy_backward(grad, e, out);
+    case OP_SOFTMAX: return softmax_backward(grad, e, out);           /* autograd.rs:204 */
+    case OP_FLASHATTENTION: return flash_attention_backward(grad, e, out); /* autograd.rs:210 */
     }
     return -1;
 }
@@ -918,7 +1108,7 @@ static int tape_backward(orc_tape *tp, size_t loss_id) {
         long idx = out2entry[tid];
         if (idx < 0) continue;
         orc_entry e = tp->e[idx];
-        long ig[2];
+        long ig[3];
         if (dispatch_backward(&e, (size_t)grads[tid], ig) != 0) { rc = -1; break; }
         for (int i = 0; i < e.n_inputs; ++i) {
             if (ig[i] < 0) continue;
@@ -1126,6 +1316,10 @@ uint32_t orc_contiguous(uint32_t a) { /* lib.rs:295-300 -> layout.rs:218-227 */
     size_t out = ensure_contiguous(a);
     if (out != a) tape_record(&g_tape, OP_CONTIGUOUS, out, 1, a, 0);
     return (uint32_t)out;
+}
+uint32_t orc_softmax_op(uint32_t a, int64_t dim) { return softmax_impl(a, (int)dim); } /* lib.rs:302-307 */
+uint32_t orc_flash_attention(uint32_t q, uint32_t k, uint32_t v, double scale, int causal) { /* lib.rs:575-584 */
+    return flash_attention_impl(q, k, v, (float)scale, causal);
 }
 uint32_t orc_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n) { /* lib.rs:328-336 */
     return cross_entropy_impl(logits, targets, n);

@@ -59,6 +59,8 @@ class OracleNative:
             "orc_view": (u32, [u32, _i64p, C.c_int]), "orc_permute": (u32, [u32, _i64p, C.c_int]),
             "orc_contiguous": (u32, [u32]),
             "orc_cross_entropy_loss": (u32, [u32, _i64p, C.c_size_t]),
+            "orc_softmax_op": (u32, [u32, C.c_int64]),
+            "orc_flash_attention": (u32, [u32, u32, u32, C.c_double, C.c_int]),
             "orc_adamw_step": (None, [_u32p, C.c_size_t] + [C.c_double] * 5 + [C.c_int64]),
             "orc_grad_norm": (C.c_double, [_u32p, C.c_size_t]),
             "orc_clip_and_step": (C.c_double, [_u32p, C.c_size_t] + [C.c_double] * 5 + [C.c_int64, C.c_double]),
@@ -187,6 +189,12 @@ class OracleNative:
 
     def crossEntropyLoss(self, logits, targets):
         return self._id(self.lib.orc_cross_entropy_loss(logits, _i64(targets), len(targets)))
+
+    def softmaxOp(self, a, dim):
+        return self._id(self.lib.orc_softmax_op(a, dim))
+
+    def flashAttention(self, q, k, v, scale, causal):
+        return self._id(self.lib.orc_flash_attention(q, k, v, scale, 1 if causal else 0))
 
     def adamwStep(self, ids, lr, beta1, beta2, eps, weight_decay, step):
         self.lib.orc_adamw_step(_u32(ids), len(ids), lr, beta1, beta2, eps, weight_decay, step)

@@ -110,6 +110,24 @@ assertClose(mseLoss(p, Tensor.fromFloat32(new Float32Array([2, 3, 4, 5]), [2, 2]
   assert(final < early, 'training reduces loss'); assert(final < 1.0, 'training converges to low loss (' + final + ')');
 }
 
+// ---- softmax / flashAttention (test/nn.test.ts:46-54, test/native.test.ts:13-23) -----------------------
+{
+  const sm = native.toFloat32(native.softmaxOp(Tensor.fromFloat32(new Float32Array([1, 2, 3, 1, 2, 3]), [2, 3])._id, 1));
+  assertClose(sm[0] + sm[1] + sm[2], 1.0, 1e-4, 'softmax row0 sums to 1');
+  assertClose(sm[3] + sm[4] + sm[5], 1.0, 1e-4, 'softmax row1 sums to 1');
+  assert(sm.every(v => v > 0) && sm[2] > sm[1] && sm[1] > sm[0], 'softmax positive and ordered');
+  assert(typeof native.flashAttention === 'function', 'flashAttention is exported');
+  const nHeads = 2, seqLen = 4, headDim = 8;
+  const mk = () => Tensor.fromFloat32(randArray(nHeads * seqLen * headDim, rnd, 0, 1), [nHeads, seqLen, headDim]);
+  const q = mk(), k = mk(), v = mk();
+  const att = new Tensor(native.flashAttention(q._id, k._id, v._id, 1.0 / Math.sqrt(headDim), true));
+  assert(att.shape.join() === [nHeads, seqLen, headDim].join(), 'attention output shape');
+  const a = att.toFloat32(), vv = v.toFloat32();
+  let worst = 0;  // causal row 0 attends to key 0 only
+  for (let h = 0; h < nHeads; h++) for (let d = 0; d < headDim; d++) worst = Math.max(worst, Math.abs(a[h * seqLen * headDim + d] - vv[h * seqLen * headDim + d]));
+  assert(worst < 1e-6, 'causal attention row 0 equals v[0]');
+}
+
 // ---- misuse raises a JS Error where the reference panics ---------------------------------------------
 try { Tensor.fromFloat32(new Float32Array(6), [2, 3]).matmul(Tensor.fromFloat32(new Float32Array(8), [4, 2])); assert(false, 'K mismatch must throw'); }
 catch (e) { assert(/inner dimensions/.test(e.message), 'K mismatch message: ' + e.message); }

@@ -1,0 +1,133 @@
+"""softmax and flash_attention on the GPU against the CPU oracle, through the
+engine-level C ABI.  Tolerances: softmax outputs and attention weights live in
+[0, 1] and are compared to 2e-6 absolute; attention outputs are convex
+combinations of rows of v, compared to 1e-5 * max|v|; gradients are sums of s
+products, compared to 1e-4 * sqrt(s) * (product of the operand maxima)."""
+import math
+
+import numpy as np
+import pytest
+
+from framework_amd import synth
+from framework_amd.api import bind
+from helpers import max_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(api, a, grad=False):
+    a = np.asarray(a, dtype=np.float32)
+    t = api.Tensor.fromFloat32(a, list(a.shape))
+    return t.setRequiresGrad(True) if grad else t
+
+
+@pytest.fixture()
+def both(rocm_native, oracle_native):
+    gpu, cpu = bind(rocm_native), bind(oracle_native)
+    yield gpu, cpu
+    rocm_native.resetEngine()
+    oracle_native.resetEngine()
+
+
+@pytest.mark.parametrize("shape,dim", [((2, 3), 1), ((64, 1000), 1), ((64, 1000), 0), ((3, 50, 7), 1), ((3, 50, 7), -1),
+                                       ((5,), 0), ((2, 3, 4, 5), 2), ((1, 4097), 1)])
+def test_softmax_forward_and_backward_match_the_oracle(both, shape, dim):
+    gpu, cpu = both
+    x = synth.normal(1, shape, 2.0)
+    w = synth.normal(2, shape, stream=1)
+    res = []
+    for api in (gpu, cpu):
+        X = _t(api, x, True)
+        y = api.softmax(X, dim)
+        y.mul(_t(api, w)).sum().backward()
+        res.append((y.numpy(), X.grad.numpy()))
+    assert max_err(res[0][0], res[1][0]) <= 2e-6
+    assert max_err(res[0][1], res[1][1]) <= 1e-5 * float(np.abs(w).max())
+
+
+def test_softmax_negative_dim_gradient_is_the_reference_one(both):
+    # dim = -1 is saved as -1.0 and read back as 0 by the reference's backward
+    gpu, cpu = both
+    x, w = synth.normal(3, (6, 9)), synth.normal(4, (6, 9), stream=1)
+    grads = []
+    for api in (gpu, cpu):
+        X = _t(api, x, True)
+        api.softmax(X, -1).mul(_t(api, w)).sum().backward()
+        grads.append(X.grad.numpy())
+    assert max_err(grads[0], grads[1]) <= 1e-5
+    x64 = x.astype(np.float64)
+    s = np.exp(x64 - x64.max(1, keepdims=True))
+    s /= s.sum(1, keepdims=True)
+    assert max_err(grads[0], s * (w - (w * s).sum(0, keepdims=True))) <= 1e-5
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bh,s,d", [(2, 4, 8), (3, 37, 20), (1, 1, 4), (4, 130, 64), (2, 1100, 16)])
+def test_attention_forward_and_backward_match_the_oracle(both, bh, s, d, causal):
+    gpu, cpu = both
+    q, k, v = (synth.normal(5, (bh, s, d), stream=i) for i in range(3))
+    w = synth.normal(5, (bh, s, d), stream=4)
+    scale = 1.0 / math.sqrt(d)
+    res = []
+    for api in (gpu, cpu):
+        Q, K, V = _t(api, q, True), _t(api, k, True), _t(api, v, True)
+        out = api.flashAttention(Q, K, V, scale, causal)
+        assert out.shape == [bh, s, d]
+        out.mul(_t(api, w)).sum().backward()
+        res.append([out.numpy(), Q.grad.numpy(), K.grad.numpy(), V.grad.numpy()])
+    mq, mk, mv, mw = (float(np.abs(a).max()) for a in (q, k, v, w))
+    assert max_err(res[0][0], res[1][0]) <= 1e-5 * mv
+    gtol = 1e-4 * math.sqrt(s)
+    assert max_err(res[0][3], res[1][3]) <= gtol * mw                      # dv = P^T dO
+    assert max_err(res[0][1], res[1][1]) <= gtol * mw * mv * mk * scale * 2  # dq = dS k
+    assert max_err(res[0][2], res[1][2]) <= gtol * mw * mv * mq * scale * 2  # dk = dS^T q
+
+
+def test_attention_known_answers_on_the_gpu(both):
+    gpu, _ = both
+    bh, s, d = 2, 70, 8
+    q, k = synth.normal(6, (bh, s, d)), synth.normal(6, (bh, s, d), stream=1)
+    v = synth.normal(6, (bh, s, d), stream=2)
+    ones = np.ones((bh, s, d), np.float32)
+    assert max_err(gpu.flashAttention(_t(gpu, q), _t(gpu, k), _t(gpu, ones), 0.3, False).numpy(), ones) <= 2e-6
+    out = gpu.flashAttention(_t(gpu, q), _t(gpu, k), _t(gpu, v), 0.3, True).numpy()
+    assert max_err(out[:, 0, :], v[:, 0, :]) <= 1e-6
+    zero = np.zeros_like(q)
+    prefix = np.cumsum(v.astype(np.float64), axis=1) / np.arange(1, s + 1)[None, :, None]
+    assert max_err(gpu.flashAttention(_t(gpu, zero), _t(gpu, k), _t(gpu, v), 0.3, True).numpy(), prefix) <= 1e-5
+
+
+def test_attention_config3_shape_against_the_oracle(both):
+    # batch 32, 512 x 64: the attention-score shapes of the measured configuration
+    gpu, cpu = both
+    bh, s, d = 32, 512, 64
+    q, k = synth.normal(2, (bh, s, d)) / np.float32(8), synth.normal(2, (bh, s, d), stream=1) / np.float32(8)
+    v = synth.normal(2, (bh, s, d), stream=2)
+    w = synth.normal(2, (bh, s, d), stream=3)
+    res = []
+    for api in (gpu, cpu):
+        Q, K, V = _t(api, q, True), _t(api, k, True), _t(api, v, True)
+        out = api.flashAttention(Q, K, V, 0.125, True)
+        out.mul(_t(api, w)).sum().backward()
+        res.append([out.numpy(), Q.grad.numpy(), K.grad.numpy(), V.grad.numpy()])
+    mq, mk, mv, mw = (float(np.abs(a).max()) for a in (q, k, v, w))
+    assert max_err(res[0][0], res[1][0]) <= 1e-5 * mv
+    gtol = 1e-4 * math.sqrt(s)
+    assert max_err(res[0][3], res[1][3]) <= gtol * mw
+    assert max_err(res[0][1], res[1][1]) <= gtol * mw * mv * mk * 0.125 * 2
+    assert max_err(res[0][2], res[1][2]) <= gtol * mw * mv * mq * 0.125 * 2
+
+
+def test_attention_misuse_is_an_error(rocm_native):
+    from framework_amd import native as N
+    T = rocm_native
+    q = T.fromFloat32(np.zeros(8, np.float32), [2, 4])
+    with pytest.raises(N.MniError, match="bh, s, d"):
+        T.flashAttention(q, q, q, 1.0, True)
+    q3 = T.fromFloat32(np.zeros(24, np.float32), [2, 3, 4])
+    short = T.fromFloat32(np.zeros(12, np.float32), [1, 3, 4])
+    with pytest.raises(N.MniError, match="fewer than"):
+        T.flashAttention(q3, short, q3, 1.0, True)
+    with pytest.raises(N.MniError, match="out of range"):
+        T.softmaxOp(q3, 3)
+    T.resetEngine()
