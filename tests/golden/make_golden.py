@@ -12,6 +12,11 @@
   full-size product computed by the CPU oracle's i-k-j loop: per row the f64
   sum, the f64 sum of squares and the first 8 values.
 
+* attention_cases.json -- the reference's softmax assertion input
+  (test/nn.test.ts:46-54) and small seeded flash_attention cases: outputs and
+  the gradients of sum(w * out), computed by the CPU oracle
+  (`python tests/golden/make_golden.py attention` writes only this file).
+
 Nothing here executes reference code; the oracle is this repository's own C
 restatement (oracle/mni_oracle.c).
 """
@@ -39,8 +44,36 @@ def row_stats(rows):
              "head": [float(x) for x in r[:8]]} for r in rows]
 
 
+def attention_cases(orc):
+    from framework_amd.api import bind
+    api = bind(orc)
+    T = api.Tensor
+    sm = api.softmax(T.fromFloat32(np.array([1, 2, 3, 1, 2, 3], np.float32), [2, 3]), 1).toFloat32()
+    cases = []
+    for i, (bh, s, d, causal) in enumerate([(2, 4, 8, True), (1, 7, 3, False), (2, 19, 8, True)]):
+        seed = 200 + i
+        q, k, v, w = (synth.normal(seed, (bh, s, d), 1.0, st) for st in range(4))
+        scale = 1.0 / float(np.sqrt(d))
+        Q, K, V = (T.fromFloat32(a, [bh, s, d]).setRequiresGrad(True) for a in (q, k, v))
+        out = api.flashAttention(Q, K, V, scale, causal)
+        out.mul(T.fromFloat32(w, [bh, s, d])).sum().backward()
+        cases.append({"bh": bh, "s": s, "d": d, "causal": causal, "scale": scale, "seed": seed,
+                      "out": [float(x) for x in out.toFloat32()], "dq": [float(x) for x in Q.grad.toFloat32()],
+                      "dk": [float(x) for x in K.grad.toFloat32()], "dv": [float(x) for x in V.grad.toFloat32()]})
+        orc.resetEngine()
+    dump("attention_cases.json", {
+        "softmax_rows_123": {"input": [1, 2, 3, 1, 2, 3], "shape": [2, 3], "dim": 1, "out": [float(x) for x in sm],
+                             "source": "input of test/nn.test.ts:46-54; values from the oracle"},
+        "generator": "framework_amd.synth.normal(seed, (bh, s, d), 1, stream): q, k, v, w = streams 0..3; loss = sum(w * out)",
+        "cases": cases})
+
+
 def main():
     orc = OracleNative()
+    if sys.argv[1:] == ["attention"]:
+        attention_cases(orc)
+        return
+    attention_cases(orc)
 
     dump("reference_vectors.json", {
         "matmul_2x2": {"a": [1, 2, 3, 4], "a_shape": [2, 2], "b": [5, 6, 7, 8], "b_shape": [2, 2],

@@ -45,3 +45,25 @@ def test_matmul_cases_on_oracle(oracle_native):
         assert np.array_equal(got.ravel(), np.array(c["out"], dtype=np.float32)), c["seed"]
         if c["kind"] == "int":  # exact in integers too
             assert np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
+
+
+def _attention_case(api, c):
+    bh, s, d = c["bh"], c["s"], c["d"]
+    q, k, v, w = (synth.normal(c["seed"], (bh, s, d), 1.0, st) for st in range(4))
+    T = api.Tensor
+    Q, K, V = (T.fromFloat32(a, [bh, s, d]).setRequiresGrad(True) for a in (q, k, v))
+    out = api.flashAttention(Q, K, V, c["scale"], c["causal"])
+    out.mul(T.fromFloat32(w, [bh, s, d])).sum().backward()
+    return {"out": out.toFloat32(), "dq": Q.grad.toFloat32(), "dk": K.grad.toFloat32(), "dv": V.grad.toFloat32()}
+
+
+def test_attention_fixtures_on_oracle(orc):
+    g = load("attention_cases.json")
+    v = g["softmax_rows_123"]
+    sm = orc.softmax(orc.Tensor.fromFloat32(v["input"], v["shape"]), v["dim"]).toFloat32()
+    assert np.allclose(sm, v["out"], rtol=0, atol=1e-7)
+    assert abs(sum(v["out"][:3]) - 1.0) < 1e-6 and v["out"][2] > v["out"][1] > v["out"][0]  # test/nn.test.ts:51-54
+    for c in g["cases"]:
+        got = _attention_case(orc, c)
+        for key in ("out", "dq", "dk", "dv"):  # libm's expf may differ in the last place between machines
+            assert np.allclose(got[key], c[key], rtol=0, atol=2e-6), (c["seed"], key)

@@ -131,3 +131,25 @@ def test_attention_misuse_is_an_error(rocm_native):
     with pytest.raises(N.MniError, match="out of range"):
         T.softmaxOp(q3, 3)
     T.resetEngine()
+
+
+def test_attention_golden_fixtures_on_the_gpu(rocm_native):
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "attention_cases.json")) as f:
+        g = json.load(f)
+    api = bind(rocm_native)
+    v = g["softmax_rows_123"]
+    sm = api.softmax(api.Tensor.fromFloat32(v["input"], v["shape"]), v["dim"]).toFloat32()
+    assert np.allclose(sm, v["out"], rtol=0, atol=2e-6)
+    for c in g["cases"]:
+        bh, s, d = c["bh"], c["s"], c["d"]
+        q, k, vv, w = (synth.normal(c["seed"], (bh, s, d), 1.0, st) for st in range(4))
+        Q, K, V = (_t(api, a, True) for a in (q, k, vv))
+        out = api.flashAttention(Q, K, V, c["scale"], c["causal"])
+        out.mul(_t(api, w)).sum().backward()
+        mv, mw = float(np.abs(vv).max()), float(np.abs(w).max())
+        assert max_err(out.numpy().ravel(), np.array(c["out"])) <= 1e-5 * mv
+        for key, T in (("dq", Q), ("dk", K), ("dv", V)):
+            assert max_err(T.grad.numpy().ravel(), np.array(c[key])) <= 1e-4 * math.sqrt(s) * mw * mv * 4, (c["seed"], key)
+    rocm_native.resetEngine()
