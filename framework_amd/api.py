@@ -142,7 +142,7 @@ def bind(native):
             return self.forward(x)
 
     class Linear(Module):  # src/nn.ts:8-26: weight is [in, out], bound 1/sqrt(in) for both
-        def __init__(self, inFeatures, outFeatures, weight=None, bias=None, fused=False):
+        def __init__(self, inFeatures, outFeatures, weight=None, bias=None, fused=False, activation=None):
             self.inFeatures, self.outFeatures = inFeatures, outFeatures
             bound = 1.0 / math.sqrt(inFeatures)
             if weight is None:
@@ -153,11 +153,15 @@ def bind(native):
             self.bias = Parameter(Tensor.fromFloat32(bias, [outFeatures]).setRequiresGrad(True))
             # opt-in fused path, feature-detected like the reference's cuda-only ops
             self.fused = fused and hasattr(native, "linear")
+            # None, "relu" or "gelu": applied by forward(); with the fused path it rides in native.linear
+            self.activation = activation
 
         def forward(self, x):
             if self.fused:
-                return Tensor(native.linear(x._id, self.weight.value._id, self.bias.value._id))
-            return x.matmul(self.weight.value).add(self.bias.value)
+                act = {None: 1, "relu": 2, "gelu": 3}[self.activation]  # MNI_EPI_BIAS / _RELU / _GELU
+                return Tensor(native.linear(x._id, self.weight.value._id, self.bias.value._id, act))
+            y = x.matmul(self.weight.value).add(self.bias.value)
+            return y if self.activation is None else (y.relu() if self.activation == "relu" else y.gelu())
 
     class ReLU(Module):
         def forward(self, x):
@@ -182,6 +186,9 @@ def bind(native):
     def softmax(x, dim=-1):  # src/nn.ts:77-79
         return Tensor(native.softmaxOp(x._id, dim))
 
+    def biasGelu(x, bias):  # src/nn.ts:153-155
+        return Tensor(native.biasGelu(x._id, bias._id))
+
     def flashAttention(q, k, v, scale, causal=True):  # src/nn.ts:107-110
         return Tensor(native.flashAttention(q._id, k._id, v._id, scale, causal))
 
@@ -200,5 +207,5 @@ def bind(native):
             return native.clipAndStep(ids, self.lr, self.beta1, self.beta2, self.eps, self.weightDecay, self.t, maxGradNorm)
 
     return SimpleNamespace(native=native, Tensor=Tensor, Parameter=Parameter, Module=Module, Linear=Linear, ReLU=ReLU,
-                           GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, softmax=softmax,
+                           GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, softmax=softmax, biasGelu=biasGelu,
                            flashAttention=flashAttention, Adam=Adam)

@@ -100,6 +100,9 @@ int k_cross_entropy(float *loss, float *softmax, const float *logits, const int3
                     int64_t n, int64_t v);
 int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t *targets,
                              const float *grad_scalar, int64_t n, int64_t v);
+int k_bias_gelu(float *out, const float *x, const float *bias, int64_t rows, int64_t cols);
+int k_bias_gelu_backward(float *dx, float *dbias, const float *g, const float *x, const float *bias, int64_t rows,
+                         int64_t cols);
 // attention.hip
 int k_softmax(float *out, const float *x, int64_t outer, int64_t n, int64_t inner);
 int k_softmax_backward(float *out, const float *sm, const float *g, int64_t outer, int64_t n, int64_t inner);

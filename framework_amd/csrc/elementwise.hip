@@ -369,7 +369,15 @@ __global__ void colsum_final_kernel(float *__restrict__ out, const float *__rest
     const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= cols) return;
     float s = 0.f;
-    for (int64_t p = 0; p < nparts; ++p) s += part[p * cols + c];
+    int64_t p = 0;
+    for (; p + 7 < nparts; p += 8) {  // 8 loads in flight, added in order
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = part[(p + e) * cols + c];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += v[e];
+    }
+    for (; p < nparts; ++p) s += part[p * cols + c];
     out[c] = s;
 }
 int k_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
@@ -393,6 +401,100 @@ int k_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
         rc = check_launch("colsum_final");
     }
     dev_free(part);
+    return rc;
+}
+
+// ---- fused bias + GELU (src/native/src/ops/fused.rs:247-273, 316-351) ------------------
+// forward: out = gelu(x + bias[col]); backward: dx = g * gelu'(x + bias[col])
+// and dbias = column sums of dx, taken in the same pass over row blocks
+// (partials per block, summed in block order: deterministic).
+__global__ void bias_gelu_kernel(float *__restrict__ out, const float *__restrict__ x, const float *__restrict__ bias,
+                                 int64_t n, int64_t cols) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) out[i] = d_gelu(x[i] + bias[i % cols]);
+}
+__global__ void bias_gelu4_kernel(float4 *__restrict__ out, const float4 *__restrict__ x, const float4 *__restrict__ bias,
+                                  int64_t n4, int64_t cols4) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += step) {
+        const float4 v = x[i], b = bias[i % cols4];
+        out[i] = make_float4(d_gelu(v.x + b.x), d_gelu(v.y + b.y), d_gelu(v.z + b.z), d_gelu(v.w + b.w));
+    }
+}
+int k_bias_gelu(float *out, const float *x, const float *bias, int64_t rows, int64_t cols) {
+    const int64_t n = rows * cols;
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (cols % 4 == 0 && al16(out) && al16(x) && al16(bias))
+        hipLaunchKernelGGL(bias_gelu4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream, (float4 *)out,
+                           (const float4 *)x, (const float4 *)bias, n / 4, cols / 4);
+    else
+        hipLaunchKernelGGL(bias_gelu_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, bias, n, cols);
+    return check_launch("bias_gelu");
+}
+static constexpr int BG_ROWS = 16;  // rows per block in the backward pass
+template <typename V, int W>
+__global__ void bias_gelu_bwd_kernel(V *__restrict__ dx, V *__restrict__ part, const V *__restrict__ g,
+                                     const V *__restrict__ x, const V *__restrict__ bias, int64_t rows, int64_t colsv) {
+    // colsv = columns in units of V (float or float4); thread = one V column, BG_ROWS rows
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= colsv) return;
+    const int64_t r0 = (int64_t)blockIdx.y * BG_ROWS;
+    const int64_t r1 = min(rows, r0 + BG_ROWS);
+    float b[W], s[W];
+    {
+        const V bv = bias[c];
+        const float *bp = reinterpret_cast<const float *>(&bv);
+#pragma unroll
+        for (int e = 0; e < W; ++e) { b[e] = bp[e]; s[e] = 0.f; }
+    }
+    for (int64_t r = r0; r < r1; ++r) {
+        const V gv = g[r * colsv + c], xv = x[r * colsv + c];
+        const float *gp = reinterpret_cast<const float *>(&gv), *xp = reinterpret_cast<const float *>(&xv);
+        V ov;
+        float *op = reinterpret_cast<float *>(&ov);
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            op[e] = gp[e] * d_gelu_grad(xp[e] + b[e]);
+            s[e] += op[e];
+        }
+        dx[r * colsv + c] = ov;
+    }
+    V sv;
+    float *sp = reinterpret_cast<float *>(&sv);
+#pragma unroll
+    for (int e = 0; e < W; ++e) sp[e] = s[e];
+    part[(int64_t)blockIdx.y * colsv + c] = sv;
+}
+int k_bias_gelu_backward(float *dx, float *dbias, const float *g, const float *x, const float *bias, int64_t rows,
+                         int64_t cols) {
+    if (cols <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (rows <= 0) return k_fill(dbias, 0.0f, cols);
+    const int64_t nparts = (rows + BG_ROWS - 1) / BG_ROWS;
+    if (nparts > 65535) return set_error(MNI_ERR_INVALID, "bias_gelu backward: too many rows (%lld)", (long long)rows);
+    const bool vec = cols % 4 == 0 && al16(dx) && al16(g) && al16(x) && al16(bias) && al16(dbias);
+    const int64_t colsv = vec ? cols / 4 : cols;
+    const dim3 block(TPB);
+    const unsigned gx = (unsigned)((colsv + TPB - 1) / TPB);
+    void *part = nullptr;
+    if (nparts > 1) MNI_TRY(dev_alloc(&part, (size_t)nparts * cols * sizeof(float)));
+    float *dst = nparts > 1 ? (float *)part : dbias;
+    if (vec)
+        hipLaunchKernelGGL((bias_gelu_bwd_kernel<float4, 4>), dim3(gx, (unsigned)nparts), block, 0, ctx().stream, (float4 *)dx,
+                           (float4 *)dst, (const float4 *)g, (const float4 *)x, (const float4 *)bias, rows, colsv);
+    else
+        hipLaunchKernelGGL((bias_gelu_bwd_kernel<float, 1>), dim3(gx, (unsigned)nparts), block, 0, ctx().stream, dx, dst, g, x,
+                           bias, rows, colsv);
+    int rc = check_launch("bias_gelu_backward");
+    if (rc == MNI_OK && nparts > 1) {
+        hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned)((cols + TPB - 1) / TPB)), block, 0, ctx().stream, dbias,
+                           (const float *)part, nparts, cols);
+        rc = check_launch("colsum_final");
+    }
+    if (part) dev_free(part);
     return rc;
 }
 

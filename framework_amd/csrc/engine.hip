@@ -50,7 +50,7 @@ struct Tensor {
 enum Op {  // subset of src/native/src/autograd.rs:28-62 plus the fused Linear
     OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
     OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY, OP_LINEAR,
-    OP_SOFTMAX, OP_FLASHATTENTION
+    OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU
 };
 
 // src/native/src/autograd.rs:65-70 TapeEntry
@@ -767,6 +767,41 @@ static int cross_entropy_backward(uint32_t grad, const Entry &e, int64_t *out) {
     return MNI_OK;
 }
 
+// ---- fused bias + GELU ------------------------------------------------------------------------------
+// ops/fused.rs:247-273: out = gelu(x + bias[i % c]), c = last extent of x.
+static uint32_t bias_gelu_op(uint32_t x, uint32_t bias) {
+    Tensor *X = get(x), *Bv = get(bias);
+    if (!X || !Bv) return MNI_BAD_ID;
+    if (X->shape.empty()) { set_error(MNI_ERR_INVALID, "bias_gelu: x must have at least one dim"); return MNI_BAD_ID; }
+    const Shape shape = X->shape;
+    const int64_t c = shape.back();
+    if (Bv->size < c) { set_error(MNI_ERR_INVALID, "bias_gelu: bias holds %lld values, last extent is %lld", (long long)Bv->size, (long long)c); return MNI_BAD_ID; }
+    BufP xs = contiguous_buf(*X), bs = contiguous_buf(*Bv);
+    BufP out = (xs && bs) ? new_buf((size_t)X->size) : nullptr;
+    if (!out || k_bias_gelu(out->p, xs->p, bs->p, c ? X->size / c : 0, c) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(out), shape);
+    Entry e;
+    e.op = OP_BIASGELU; e.output_id = id; e.n_inputs = 2; e.inputs[0] = x; e.inputs[1] = bias;
+    eng().tape.record(std::move(e));
+    return id;
+}
+// ops/fused.rs:316-351: dx = grad * gelu'(x + bias), dbias = column sums of dx.
+static int bias_gelu_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *X = get(e.inputs[0]), *Bv = get(e.inputs[1]), *G = get(grad);
+    if (!X || !Bv || !G) return MNI_ERR_FREED;
+    const Shape shape = X->shape, bshape = Bv->shape;
+    const int64_t c = shape.back(), rows = c ? X->size / c : 0;
+    BufP xs = contiguous_buf(*X), bs = contiguous_buf(*Bv), gs = contiguous_buf(*G);
+    BufP dx = (xs && bs && gs) ? new_buf((size_t)X->size) : nullptr;
+    BufP db = dx ? new_buf((size_t)Bv->size) : nullptr;
+    if (!db) return MNI_ERR_NOMEM;
+    if (Bv->size > c) MNI_TRY(k_fill(db->p, 0.0f, Bv->size));  // entries past the last extent receive nothing
+    MNI_TRY(k_bias_gelu_backward(dx->p, db->p, gs->p, xs->p, bs->p, rows, c));
+    out[0] = insert_contig(std::move(dx), shape);
+    out[1] = insert_contig(std::move(db), bshape);
+    return MNI_OK;
+}
+
 // ---- softmax -----------------------------------------------------------------------------------
 // ops/norm.rs:10-50.  The tape keeps the dim as it was passed (:47).
 static uint32_t softmax_op(uint32_t a, int64_t dim) {
@@ -897,16 +932,18 @@ static uint32_t linear_op(uint32_t x, uint32_t w, uint32_t bias, int act) {
         set_error(MNI_ERR_INVALID, "linear: bias must be a contiguous [out] vector");
         return MNI_BAD_ID;
     }
-    // GELU needs its pre-activation in backward: keep z and apply the
-    // activation as a second pass; bias and ReLU ride in the GEMM epilogue.
+    // GELU needs its pre-activation in backward: the product is kept without
+    // the bias and one pass applies bias + GELU (ops/fused.rs:247-273); plain
+    // bias and ReLU ride in the GEMM epilogue.
     const BufP bias_buf = Bv->buf;
     uint32_t out, aux = MNI_BAD_ID;
     if (act == MNI_EPI_BIAS_GELU) {
-        aux = matmul_tensors(x, false, w, false, bias_buf->p, MNI_EPI_BIAS);
+        aux = matmul_tensors(x, false, w, false, nullptr, MNI_EPI_NONE);
         if (aux == MNI_BAD_ID) return MNI_BAD_ID;
         Tensor *Z = get(aux);
+        const int64_t c = Z->shape.back();
         BufP o = new_buf((size_t)Z->size);
-        if (!o || k_unary(o->p, Z->buf->p, Z->size, UN_GELU, 0.f) != MNI_OK) return MNI_BAD_ID;
+        if (!o || k_bias_gelu(o->p, Z->buf->p, bias_buf->p, c ? Z->size / c : 0, c) != MNI_OK) return MNI_BAD_ID;
         out = insert_contig(std::move(o), Z->shape);
     } else {
         out = matmul_tensors(x, false, w, false, bias_buf->p, act);
@@ -922,14 +959,28 @@ static uint32_t linear_op(uint32_t x, uint32_t w, uint32_t bias, int act) {
 static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
     uint32_t g = grad;
     bool own_g = false;
-    if (e.act != MNI_EPI_BIAS) {
-        // dZ = dOut * act'(z); for ReLU the output has the sign of z.
-        Tensor *G = get(grad), *Z = get(e.act == MNI_EPI_BIAS_GELU ? e.aux : e.output_id);
+    int64_t db_id = -1;
+    if (e.act == MNI_EPI_BIAS_GELU) {
+        // dZ = dOut * gelu'(z + bias) and db = column sums of dZ in one pass (ops/fused.rs:316-351)
+        Tensor *G = get(grad), *Z = get(e.aux), *Bv = get(e.inputs[2]);
+        if (!G || !Z || !Bv) return MNI_ERR_FREED;
+        const int64_t c = Z->shape.back();
+        BufP gb = contiguous_buf(*G);
+        BufP o = gb ? new_buf((size_t)G->size) : nullptr;
+        BufP db = o ? new_buf((size_t)c) : nullptr;
+        if (!db) return MNI_ERR_NOMEM;
+        MNI_TRY(k_bias_gelu_backward(o->p, db->p, gb->p, Z->buf->p, Bv->buf->p, c ? Z->size / c : 0, c));
+        g = insert_contig(std::move(o), G->shape);
+        db_id = insert_contig(std::move(db), Bv->shape);
+        own_g = true;
+    } else if (e.act == MNI_EPI_BIAS_RELU) {
+        // dZ = dOut where the output is positive (the output has the sign of z)
+        Tensor *G = get(grad), *Z = get(e.output_id);
         if (!G || !Z) return MNI_ERR_FREED;
         BufP gb = contiguous_buf(*G);
         BufP o = gb ? new_buf((size_t)G->size) : nullptr;
         if (!o) return MNI_ERR_NOMEM;
-        MNI_TRY(k_unary_backward(o->p, gb->p, Z->buf->p, G->size, e.act == MNI_EPI_BIAS_GELU ? UN_GELU : UN_RELU));
+        MNI_TRY(k_unary_backward(o->p, gb->p, Z->buf->p, G->size, UN_RELU));
         g = insert_contig(std::move(o), G->shape);
         own_g = true;
     }
@@ -937,15 +988,18 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
     mm.op = OP_MATMUL; mm.n_inputs = 2; mm.inputs[0] = e.inputs[0]; mm.inputs[1] = e.inputs[1];
     int rc = matmul_backward(g, mm, out);
     if (rc == MNI_OK) {
-        Tensor *Bv = get(e.inputs[2]);
-        if (!Bv) rc = MNI_ERR_FREED;
+        if (db_id >= 0) out[2] = db_id;
         else {
-            const Shape bshape = Bv->shape;
-            const uint32_t gb = unbroadcast_tensor(g, bshape);
-            if (gb == MNI_BAD_ID) rc = MNI_ERR_INVALID;
-            else out[2] = gb;
+            Tensor *Bv = get(e.inputs[2]);
+            if (!Bv) rc = MNI_ERR_FREED;
+            else {
+                const Shape bshape = Bv->shape;
+                const uint32_t gb = unbroadcast_tensor(g, bshape);
+                if (gb == MNI_BAD_ID) rc = MNI_ERR_INVALID;
+                else out[2] = gb;
+            }
         }
-    }
+    } else if (db_id >= 0) free_tensor((uint32_t)db_id);
     if (own_g) free_tensor(g);
     return rc;
 }
@@ -966,6 +1020,7 @@ static int dispatch_backward(const Entry &e, uint32_t grad, int64_t *out) {  // 
     case OP_CONTIGUOUS: out[0] = grad; return MNI_OK;  // layout.rs:229-231
     case OP_CROSSENTROPY: return cross_entropy_backward(grad, e, out);
     case OP_LINEAR: return linear_backward(grad, e, out);
+    case OP_BIASGELU: return bias_gelu_backward(grad, e, out);               // autograd.rs BiasGelu
     case OP_SOFTMAX: return softmax_backward(grad, e, out);                  // autograd.rs:204
     case OP_FLASHATTENTION: return flash_attention_backward(grad, e, out);   // autograd.rs:210
     }
@@ -1295,6 +1350,7 @@ uint32_t mni_contiguous(uint32_t a) {  // layout.rs:218-227
     eng().tape.record(std::move(e));
     return id;
 }
+uint32_t mni_bias_gelu(uint32_t x, uint32_t bias) { MNI_API_GUARD; return bias_gelu_op(x, bias); }
 uint32_t mni_softmax_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return softmax_op(a, dim); }
 uint32_t mni_flash_attention(uint32_t q, uint32_t k, uint32_t v, double scale, int causal) {
     MNI_API_GUARD;

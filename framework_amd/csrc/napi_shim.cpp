@@ -118,6 +118,7 @@ BINARY(Mul, mni_mul)                     // lib.rs:171-176
 BINARY(Sub, mni_sub)                     // lib.rs:178-183
 UNARY(Neg, mni_neg)                      // lib.rs:185-190
 BINARY(Matmul, mni_matmul)               // lib.rs:199-204
+BINARY(BiasGelu, mni_bias_gelu)          // lib.rs:526-531
 UNARY(Gelu, mni_gelu)                    // lib.rs:206-211
 UNARY(Relu, mni_relu)                    // lib.rs:213-218
 WITH_DIM(SumOp, mni_sum_op)              // lib.rs:234-239
@@ -283,7 +284,7 @@ NAPI_MODULE_INIT() {
         EXPORT("contiguous", Contiguous), EXPORT("crossEntropyLoss", CrossEntropyLoss), EXPORT("adamwStep", AdamwStep),
         EXPORT("gradNorm", GradNorm), EXPORT("clipGradNorm", ClipGradNorm), EXPORT("clipAndStep", ClipAndStep),
         EXPORT("resetEngine", ResetEngine), EXPORT("gcTensors", GcTensors), EXPORT("linear", Linear),
-        EXPORT("softmaxOp", SoftmaxOp), EXPORT("flashAttention", FlashAttention),
+        EXPORT("softmaxOp", SoftmaxOp), EXPORT("biasGelu", BiasGelu), EXPORT("flashAttention", FlashAttention),
 #undef EXPORT
     };
     napi_define_properties(env, exports, sizeof(props) / sizeof(props[0]), props);

@@ -101,6 +101,7 @@ SIGNATURES = {
     "mni_permute": (C.c_uint32, [C.c_uint32, _i64p, C.c_int]),
     "mni_contiguous": (C.c_uint32, [C.c_uint32]),
     "mni_softmax_op": (C.c_uint32, [C.c_uint32, C.c_int64]),
+    "mni_bias_gelu": (C.c_uint32, [C.c_uint32, C.c_uint32]),
     "mni_flash_attention": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double, C.c_int]),
     "mni_cross_entropy_loss": (C.c_uint32, [C.c_uint32, _i64p, C.c_size_t]),
     "mni_adamw_step": (C.c_int, [_u32p, C.c_size_t, C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, C.c_int64]),
@@ -387,6 +388,9 @@ class Native:
 
     def softmaxOp(self, a, dim):
         return self._id(self.lib.mni_softmax_op(a, dim))
+
+    def biasGelu(self, x, bias):
+        return self._id(self.lib.mni_bias_gelu(x, bias))
 
     def flashAttention(self, q, k, v, scale, causal):
         return self._id(self.lib.mni_flash_attention(q, k, v, scale, 1 if causal else 0))

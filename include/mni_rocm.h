@@ -175,7 +175,10 @@ uint32_t mni_sum_all(uint32_t a);                                         /* lib
 uint32_t mni_mean_all(uint32_t a);                                        /* lib.rs:267-277 */
 uint32_t mni_view(uint32_t a, const int64_t *shape, int ndim);            /* lib.rs:279-285 */
 uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim);          /* lib.rs:287-293 */
-uint32_t mni_contiguous(uint32_t a);                                      /* softmax_op (src/native/src/lib.rs:302-307 -> ops/norm.rs:10-50); backward as
+uint32_t mni_contiguous(uint32_t a);                                      /* bias_gelu (src/native/src/lib.rs:526-531 -> ops/fused.rs:247-273, backward :316-351):
+ * out = gelu(x + bias) along the last extent; backward yields dx and the column sums dbias in one pass. */
+uint32_t mni_bias_gelu(uint32_t x, uint32_t bias);
+/* softmax_op (src/native/src/lib.rs:302-307 -> ops/norm.rs:10-50); backward as
  * ops/norm.rs:96-123, including its reading of a negative saved dim as dim 0. */
 uint32_t mni_softmax_op(uint32_t a, int64_t dim);
 /* flash_attention (src/native/src/lib.rs:575-584 -> ops/attention.rs:14-78,

@@ -52,7 +52,7 @@ typedef struct {
 enum orc_op { /* subset of autograd.rs:28-62 BackwardOp */
     OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
     OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY,
-    OP_SOFTMAX, OP_FLASHATTENTION
+    OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU
 };
 
 /* autograd.rs:65-70 TapeEntry + the SavedContext variants the subset needs */
@@ -830,6 +830,64 @@ static int cross_entropy_backward(size_t grad, const orc_entry *e, long *out) {
     return 0;
 }
 
+/* ---- fused bias + GELU ---------------------------------------------------- */
+
+/* ops/fused.rs:247-273 bias_gelu, cpu arm: val = x[i] + bias[i % c] with c the
+ * last extent of x, GELU with the literal constant 0.7978845608 (:263).
+ * pinned by: equality with gelu(add(x, bias)) of this oracle to rounding,
+ * float64 closed form, shape assertion of test/native.test.ts:39-43. */
+static uint32_t bias_gelu_impl(size_t x, size_t bias) {
+    orc_tensor *X = get(x), *B = get(bias);
+    if (!X || !B) return fail("tensor already freed");
+    if (X->ndim < 1) return fail("called `Option::unwrap()` on a `None` value: bias_gelu of a scalar");
+    size_t shape[ORC_MAX_DIMS]; int nd = X->ndim;
+    memcpy(shape, X->shape, sizeof shape);
+    size_t c = shape[nd - 1], total = shape_size(shape, nd);
+    if (B->size < c) return fail("index out of bounds: bias shorter than the last extent");
+    float *xd = to_host(X), *bd = to_host(B);
+    float *out = (float *)calloc(total ? total : 1, sizeof(float));
+    for (size_t i = 0; i < total; ++i) {
+        float val = xd[i] + bd[i % c];
+        float inner = 0.7978845608f * (val + 0.044715f * val * val * val);
+        out[i] = 0.5f * val * (1.0f + tanhf(inner));
+    }
+    free(xd); free(bd);
+    size_t out_id = from_vec(out, shape, nd);
+    tape_record(&g_tape, OP_BIASGELU, out_id, 2, x, bias);
+    return (uint32_t)out_id;
+}
+
+/* ops/fused.rs:316-351 bias_gelu_backward: g = grad * gelu'(x + bias);
+ * dx = g, dbias[j] += g in flat index order (i.e. down each column).
+ * pinned by: float64 derivative, dbias = column sums of dx, finite differences. */
+static int bias_gelu_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *X = get(e->saved_ids[0]), *B = get(e->saved_ids[1]), *G = get(grad);
+    if (!X || !B || !G) { fail("tensor already freed"); return -1; }
+    size_t shape[ORC_MAX_DIMS], bshape[ORC_MAX_DIMS]; int nd = X->ndim, bnd = B->ndim;
+    memcpy(shape, X->shape, sizeof shape);
+    memcpy(bshape, B->shape, sizeof bshape);
+    size_t c = shape[nd - 1], total = shape_size(shape, nd);
+    float *xd = to_host(X), *bd = to_host(B), *gd = to_host(G);
+    float *dx = (float *)calloc(total ? total : 1, sizeof(float));
+    float *db = (float *)calloc(B->size ? B->size : 1, sizeof(float));
+    for (size_t i = 0; i < total; ++i) {
+        size_t j = i % c;
+        float val = xd[i] + bd[j];
+        float inner = 0.7978845608f * (val + 0.044715f * val * val * val);
+        float th = tanhf(inner);
+        float sech2 = 1.0f - th * th;
+        float d_inner = 0.7978845608f * (1.0f + 3.0f * 0.044715f * val * val);
+        float dgelu = 0.5f * (1.0f + th) + 0.5f * val * sech2 * d_inner;
+        float g = gd[i] * dgelu;
+        dx[i] = g;
+        db[j] += g;
+    }
+    free(xd); free(bd); free(gd);
+    out[0] = (long)from_vec(dx, shape, nd);
+    out[1] = (long)from_vec(db, bshape, bnd);
+    return 0;
+}
+
 /* ---- softmax ------------------------------------------------------------ */
 
 /* ops/norm.rs:10-50 softmax, cpu arm: per (outer, inner) line -- running max,
@@ -1032,6 +1090,7 @@ static int dispatch_backward(const orc_entry *e, size_t grad, long *out) {
     case OP_PERMUTE: return permute_backward(grad, e, out);
     case OP_CONTIGUOUS: out[0] = (long)grad; return 0; /* layout.rs:229-231 */
     case OP_CROSSENTROPY: return cross_entropy_backward(grad, e, out);
+    case OP_BIASGELU: return bias_gelu_backward(grad, e, out);        /* autograd.rs BiasGelu */
     case OP_SOFTMAX: return softmax_backward(grad, e, out);           /* autograd.rs:204 */
     case OP_FLASHATTENTION: return flash_attention_backward(grad, e, out); /* autograd.rs:210 */
     }
@@ -1317,6 +1376,7 @@ uint32_t orc_contiguous(uint32_t a) { /* lib.rs:295-300 -> layout.rs:218-227 */
     if (out != a) tape_record(&g_tape, OP_CONTIGUOUS, out, 1, a, 0);
     return (uint32_t)out;
 }
+uint32_t orc_bias_gelu(uint32_t x, uint32_t bias) { return bias_gelu_impl(x, bias); } /* lib.rs:526-531 */
 uint32_t orc_softmax_op(uint32_t a, int64_t dim) { return softmax_impl(a, (int)dim); } /* lib.rs:302-307 */
 uint32_t orc_flash_attention(uint32_t q, uint32_t k, uint32_t v, double scale, int causal) { /* lib.rs:575-584 */
     return flash_attention_impl(q, k, v, (float)scale, causal);

@@ -60,6 +60,7 @@ class OracleNative:
             "orc_contiguous": (u32, [u32]),
             "orc_cross_entropy_loss": (u32, [u32, _i64p, C.c_size_t]),
             "orc_softmax_op": (u32, [u32, C.c_int64]),
+            "orc_bias_gelu": (u32, [u32, u32]),
             "orc_flash_attention": (u32, [u32, u32, u32, C.c_double, C.c_int]),
             "orc_adamw_step": (None, [_u32p, C.c_size_t] + [C.c_double] * 5 + [C.c_int64]),
             "orc_grad_norm": (C.c_double, [_u32p, C.c_size_t]),
@@ -192,6 +193,9 @@ class OracleNative:
 
     def softmaxOp(self, a, dim):
         return self._id(self.lib.orc_softmax_op(a, dim))
+
+    def biasGelu(self, x, bias):
+        return self._id(self.lib.orc_bias_gelu(x, bias))
 
     def flashAttention(self, q, k, v, scale, causal):
         return self._id(self.lib.orc_flash_attention(q, k, v, scale, 1 if causal else 0))

@@ -116,6 +116,8 @@ assertClose(mseLoss(p, Tensor.fromFloat32(new Float32Array([2, 3, 4, 5]), [2, 2]
   assertClose(sm[0] + sm[1] + sm[2], 1.0, 1e-4, 'softmax row0 sums to 1');
   assertClose(sm[3] + sm[4] + sm[5], 1.0, 1e-4, 'softmax row1 sums to 1');
   assert(sm.every(v => v > 0) && sm[2] > sm[1] && sm[1] > sm[0], 'softmax positive and ordered');
+  const bg = new Tensor(native.biasGelu(Tensor.fromFloat32(randArray(8, rnd, 0, 1), [2, 4])._id, Tensor.fromFloat32(randArray(4, rnd, 0, 1), [4])._id));
+  assert(bg.shape[0] === 2 && bg.shape[1] === 4, 'biasGelu shape');   // test/native.test.ts:39-43
   assert(typeof native.flashAttention === 'function', 'flashAttention is exported');
   const nHeads = 2, seqLen = 4, headDim = 8;
   const mk = () => Tensor.fromFloat32(randArray(nHeads * seqLen * headDim, rnd, 0, 1), [nHeads, seqLen, headDim]);

@@ -153,3 +153,46 @@ def test_attention_golden_fixtures_on_the_gpu(rocm_native):
         for key, T in (("dq", Q), ("dk", K), ("dv", V)):
             assert max_err(T.grad.numpy().ravel(), np.array(c[key])) <= 1e-4 * math.sqrt(s) * mw * mv * 4, (c["seed"], key)
     rocm_native.resetEngine()
+
+
+@pytest.mark.parametrize("shape", [(2, 4), (300, 257), (4096, 1024), (3, 50, 8), (7,)])
+def test_bias_gelu_forward_and_backward_match_the_oracle(both, shape):
+    gpu, cpu = both
+    x = synth.normal(7, shape, 1.5)
+    b = synth.normal(8, (shape[-1],), 1.0, stream=1)
+    w = synth.normal(9, shape, 1.0, stream=2)
+    res = []
+    for api in (gpu, cpu):
+        X, B = _t(api, x, True), _t(api, b, True)
+        out = api.biasGelu(X, B)
+        out.mul(_t(api, w)).sum().backward()
+        res.append((out.numpy(), X.grad.numpy(), B.grad.numpy()))
+    rows = int(np.prod(shape[:-1])) if len(shape) > 1 else 1
+    mw = float(np.abs(w).max())
+    assert max_err(res[0][0], res[1][0]) <= 1e-5 * float(np.abs(x).max() + np.abs(b).max())
+    assert max_err(res[0][1], res[1][1]) <= 1e-5 * mw * 1.2
+    assert max_err(res[0][2], res[1][2]) <= 1e-4 * math.sqrt(rows) * mw * 1.2  # column sums over `rows` terms
+
+
+def test_fused_linear_gelu_equals_the_unfused_chain(both):
+    # Linear(fused) with GELU = matmul, then bias + GELU in one pass; its backward
+    # takes dGELU and the bias gradient in one pass.  Same values as matmul -> add -> gelu.
+    gpu, cpu = both
+    x = synth.normal(1, (130, 70))
+    wt = synth.uniform(2, (70, 90), -0.2, 0.2, stream=1)
+    b = synth.normal(3, (90,), 0.3, stream=2)
+    r = synth.normal(4, (130, 90), 1.0, stream=3)
+    grads = []
+    for api, fused in ((gpu, True), (gpu, False), (cpu, False)):
+        X, W, B = _t(api, x, True), _t(api, wt, True), _t(api, b, True)
+        if fused:
+            y = api.Tensor(api.native.linear(X._id, W._id, B._id, 3))
+        else:
+            y = X.matmul(W).add(B).gelu()
+        y.mul(_t(api, r)).sum().backward()
+        grads.append([y.numpy(), X.grad.numpy(), W.grad.numpy(), B.grad.numpy()])
+    for other in (1, 2):
+        assert max_err(grads[0][0], grads[other][0]) <= 1e-4 * math.sqrt(70) * 0.2 * 4
+        assert max_err(grads[0][1], grads[other][1]) <= 1e-4 * math.sqrt(90) * 0.2 * 5
+        assert max_err(grads[0][2], grads[other][2]) <= 1e-4 * math.sqrt(130) * 4 * 5
+        assert max_err(grads[0][3], grads[other][3]) <= 1e-4 * math.sqrt(130) * 5

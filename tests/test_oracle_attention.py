@@ -160,3 +160,49 @@ def test_attention_key_gradient_vanishes_for_constant_keys(orc):
     orc.flashAttention(Q, K, V, 1.0, False).sum().backward()
     assert max_err(Q.grad.numpy(), np.zeros((bh, s, d))) < 1e-6
     assert max_err(V.grad.numpy(), np.ones((bh, s, d))) < 1e-6  # each column gets s * (1/s)
+
+
+# ---- fused bias + GELU (ops/fused.rs:247-273, 316-351) -------------------------
+
+def _gelu64(z):
+    return 0.5 * z * (1 + np.tanh(np.sqrt(2 / np.pi) * (z + 0.044715 * z ** 3)))
+
+
+def _dgelu64(z):
+    s = np.sqrt(2 / np.pi)
+    th = np.tanh(s * (z + 0.044715 * z ** 3))
+    return 0.5 * (1 + th) + 0.5 * z * (1 - th * th) * s * (1 + 3 * 0.044715 * z * z)
+
+
+@pytest.mark.parametrize("shape", [(2, 4), (5, 7), (3, 4, 6), (9,)])
+def test_bias_gelu_forward_vs_float64_and_composition(orc, shape):
+    x = synth.normal(11, shape, 2.0)
+    b = synth.normal(12, (shape[-1],), 1.0, stream=1)
+    out = orc.biasGelu(_t(orc, x), _t(orc, b))
+    assert out.shape == list(shape)  # test/native.test.ts:39-43 checks the shape only
+    z = x.astype(np.float64) + b.astype(np.float64)
+    assert max_err(out.numpy(), _gelu64(z)) < 1e-6
+    composed = _t(orc, x).add(_t(orc, b)).gelu().numpy()  # the unfused path of the same oracle
+    assert max_err(out.numpy(), composed) < 5e-7
+
+
+def test_bias_gelu_backward_vs_float64_and_column_sums(orc):
+    x = synth.normal(13, (6, 5), 1.5)
+    b = synth.normal(14, (5,), 1.0, stream=1)
+    w = synth.normal(15, (6, 5), 1.0, stream=2)
+    X, B = _t(orc, x, True), _t(orc, b, True)
+    orc.biasGelu(X, B).mul(_t(orc, w)).sum().backward()
+    z = x.astype(np.float64) + b.astype(np.float64)
+    dx = w.astype(np.float64) * _dgelu64(z)
+    assert max_err(X.grad.numpy(), dx) < 1e-6
+    assert max_err(B.grad.numpy(), dx.sum(axis=0)) < 1e-5
+    # dbias is exactly the f32 column sum of dx taken down the rows
+    got_dx = X.grad.numpy()
+    col = np.zeros(5, np.float32)
+    for r in range(6):
+        col = col + got_dx[r]
+    assert np.array_equal(B.grad.numpy(), col)
+    # finite differences of the float64 closed form, as a check on the closed form itself
+    eps = 1e-6
+    fd = ((_gelu64(z + eps) - _gelu64(z - eps)) / (2 * eps)) * w
+    assert max_err(dx, fd) < 1e-6
