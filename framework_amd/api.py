@@ -113,6 +113,36 @@ def bind(native):
         def contiguous(self):
             return Tensor(native.contiguous(self._id))
 
+        def exp(self):
+            return Tensor(native.expOp(self._id))
+
+        def log(self):
+            return Tensor(native.logOp(self._id))
+
+        def sigmoid(self):
+            return Tensor(native.sigmoid(self._id))
+
+        def pow(self, exponent):
+            return Tensor(native.powOp(self._id, exponent))
+
+        def div(self, other):
+            return Tensor(native.div(self._id, other._id))
+
+        def lt(self, other):
+            return Tensor(native.lt(self._id, other._id))
+
+        def eq(self, other):
+            return Tensor(native.eqOp(self._id, other._id))
+
+        def gt(self, other):
+            return Tensor(native.gt(self._id, other._id))
+
+        def isClose(self, other, tol=1e-5):
+            return Tensor(native.isClose(self._id, other._id, tol))
+
+        def max(self, dim):
+            return Tensor(native.maxOp(self._id, dim))
+
         def matmul(self, other):  # src/tensor.ts:207-209
             return Tensor(native.matmul(self._id, other._id))
 
@@ -186,6 +216,9 @@ def bind(native):
     def softmax(x, dim=-1):  # src/nn.ts:77-79
         return Tensor(native.softmaxOp(x._id, dim))
 
+    def layerNorm(x, gamma, beta, eps=1e-5):  # src/nn.ts LayerNorm -> native.layernormOp
+        return Tensor(native.layernormOp(x._id, gamma._id, beta._id, eps))
+
     def biasGelu(x, bias):  # src/nn.ts:153-155
         return Tensor(native.biasGelu(x._id, bias._id))
 
@@ -207,5 +240,5 @@ def bind(native):
             return native.clipAndStep(ids, self.lr, self.beta1, self.beta2, self.eps, self.weightDecay, self.t, maxGradNorm)
 
     return SimpleNamespace(native=native, Tensor=Tensor, Parameter=Parameter, Module=Module, Linear=Linear, ReLU=ReLU,
-                           GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, softmax=softmax, biasGelu=biasGelu,
+                           GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, softmax=softmax, biasGelu=biasGelu, layerNorm=layerNorm,
                            flashAttention=flashAttention, Adam=Adam)

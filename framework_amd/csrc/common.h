@@ -75,19 +75,24 @@ struct StridedDesc {
     int64_t a_strides[MNI_MAX_DIMS];
     int64_t b_strides[MNI_MAX_DIMS];
 };
-enum BinOp { BIN_ADD = 0, BIN_SUB = 1, BIN_MUL = 2 };
-enum UnOp { UN_RELU = 0, UN_GELU = 1, UN_NEG = 2, UN_SCALE = 3, UN_COPY = 4 };
+enum BinOp { BIN_ADD = 0, BIN_SUB = 1, BIN_MUL = 2, BIN_DIV = 3, BIN_LT = 4, BIN_EQ = 5, BIN_GT = 6, BIN_CLOSE = 7 };
+enum UnOp { UN_RELU = 0, UN_GELU = 1, UN_NEG = 2, UN_SCALE = 3, UN_COPY = 4, UN_EXP = 5, UN_LOG = 6, UN_SIGMOID = 7, UN_POW = 8 };
 
 int k_fill(float *dst, float v, int64_t n);
 int k_axpy(float *dst, const float *src, float alpha, int64_t n);
 int k_scale_inplace(float *dst, float s, int64_t n);
 int k_strided_copy(float *dst, const float *src, const int64_t *shape, const int64_t *strides, int ndim);
-int k_binary_broadcast(float *out, const float *a, const float *b, const StridedDesc &d, int op);
-int k_binary_same(float *out, const float *a, const float *b, int64_t n, int op);
+// `p` is the tolerance of BIN_CLOSE (|a - b| < p)
+int k_binary_broadcast(float *out, const float *a, const float *b, const StridedDesc &d, int op, float p = 0.f);
+int k_binary_same(float *out, const float *a, const float *b, int64_t n, int op, float p = 0.f);
+// ga = g / b, gb = -g * a / (b * b); g contiguous over d.shape, a / b addressed by d.a_strides / d.b_strides
+int k_div_backward(float *ga, float *gb, const float *g, const float *a, const float *b, const StridedDesc &d);
 int k_add_bias(float *out, const float *a, const float *bias, int64_t rows, int64_t cols);
 int k_unary(float *out, const float *x, int64_t n, int op, float s);
 // out = g * f'(x) for relu/gelu
 int k_unary_backward(float *out, const float *g, const float *x, int64_t n, int op);
+// exp: g * out, log: g / x, sigmoid: g * o * (1 - o), pow: g * s * x^(s - 1); `saved` is out or x accordingly
+int k_unary2_backward(float *out, const float *g, const float *saved, int64_t n, int op, float s);
 int k_mul_backward_same(float *ga, float *gb, const float *g, const float *a, const float *b, int64_t n);
 int k_colsum(float *out, const float *a, int64_t rows, int64_t cols);
 // out[o, i] = (sum_d a[o, d, i]) / div
@@ -103,6 +108,13 @@ int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t
 int k_bias_gelu(float *out, const float *x, const float *bias, int64_t rows, int64_t cols);
 int k_bias_gelu_backward(float *dx, float *dbias, const float *g, const float *x, const float *bias, int64_t rows,
                          int64_t cols);
+// out[o, i] = max_d a[o, d, i]; backward: g[o, i] where |x - max| < 1e-6, else 0
+int k_max_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t inner);
+int k_max_backward(float *out, const float *x, const float *mx, const float *g, int64_t outer, int64_t dim, int64_t inner);
+int k_layernorm(float *out, float *mean, float *rstd, const float *x, const float *gamma, const float *beta, int64_t rows,
+                int64_t c, float eps);
+int k_layernorm_backward(float *dx, float *dgamma, float *dbeta, const float *g, const float *x, const float *gamma,
+                         const float *mean, const float *rstd, int64_t rows, int64_t c);
 // attention.hip
 int k_softmax(float *out, const float *x, int64_t outer, int64_t n, int64_t inner);
 int k_softmax_backward(float *out, const float *sm, const float *g, int64_t outer, int64_t n, int64_t inner);

@@ -185,11 +185,20 @@ int k_strided_copy(float *dst, const float *src, const int64_t *shape, const int
 // ---- broadcast binary -----------------------------------------------------------
 // broadcast_binary (src/native/src/ops/elementwise.rs:20-56): operands are
 // addressed by their own strides with 0 on broadcast dims, so views need no copy.
-__device__ __forceinline__ float bin_apply(float x, float y, int op) {
-    return op == BIN_ADD ? x + y : op == BIN_SUB ? x - y : x * y;
+__device__ __forceinline__ float bin_apply(float x, float y, int op, float p) {
+    switch (op) {
+    case BIN_ADD: return x + y;
+    case BIN_SUB: return x - y;
+    case BIN_MUL: return x * y;
+    case BIN_DIV: return x / y;                               // elementwise.rs:918-928
+    case BIN_LT: return x < y ? 1.0f : 0.0f;                  // :1099-1103
+    case BIN_EQ: return x == y ? 1.0f : 0.0f;                 // :1152-1156
+    case BIN_GT: return x > y ? 1.0f : 0.0f;                  // :1205-1209
+    default: return fabsf(x - y) < p ? 1.0f : 0.0f;           // is_close, :1258-1288
+    }
 }
 __global__ void binary_bcast_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b,
-                                    const StridedDesc d, int64_t n, int op) {
+                                    const StridedDesc d, int64_t n, int op, float p) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t step = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += step) {
@@ -200,45 +209,72 @@ __global__ void binary_bcast_kernel(float *__restrict__ out, const float *__rest
             ao += c * d.a_strides[k];
             bo += c * d.b_strides[k];
         }
-        out[i] = bin_apply(a[ao], b[bo], op);
+        out[i] = bin_apply(a[ao], b[bo], op, p);
     }
 }
-int k_binary_broadcast(float *out, const float *a, const float *b, const StridedDesc &d, int op) {
+int k_binary_broadcast(float *out, const float *a, const float *b, const StridedDesc &d, int op, float p) {
     MNI_TRY(ensure_init());
     int64_t n = 1;
     for (int i = 0; i < d.ndim; ++i) n *= d.shape[i];
     if (n <= 0) return MNI_OK;
-    hipLaunchKernelGGL(binary_bcast_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, d, n, op);
+    hipLaunchKernelGGL(binary_bcast_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, d, n, op, p);
     return check_launch("binary_broadcast");
 }
 
 __global__ void binary_same_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b,
-                                   int64_t n, int op) {
+                                   int64_t n, int op, float p) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t step = (int64_t)gridDim.x * blockDim.x;
-    for (; i < n; i += step) out[i] = bin_apply(a[i], b[i], op);
+    for (; i < n; i += step) out[i] = bin_apply(a[i], b[i], op, p);
 }
 __global__ void binary_same4_kernel(float4 *__restrict__ out, const float4 *__restrict__ a,
-                                    const float4 *__restrict__ b, int64_t n4, int op) {
+                                    const float4 *__restrict__ b, int64_t n4, int op, float p) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t step = (int64_t)gridDim.x * blockDim.x;
     for (; i < n4; i += step) {
         const float4 x = a[i], y = b[i];
-        out[i] = make_float4(bin_apply(x.x, y.x, op), bin_apply(x.y, y.y, op), bin_apply(x.z, y.z, op),
-                             bin_apply(x.w, y.w, op));
+        out[i] = make_float4(bin_apply(x.x, y.x, op, p), bin_apply(x.y, y.y, op, p), bin_apply(x.z, y.z, op, p),
+                             bin_apply(x.w, y.w, op, p));
     }
 }
-int k_binary_same(float *out, const float *a, const float *b, int64_t n, int op) {
+int k_binary_same(float *out, const float *a, const float *b, int64_t n, int op, float p) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (al16(out) && al16(a) && al16(b) && (n % 4) == 0) {
         hipLaunchKernelGGL(binary_same4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
                            reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(a),
-                           reinterpret_cast<const float4 *>(b), n / 4, op);
+                           reinterpret_cast<const float4 *>(b), n / 4, op, p);
     } else {
-        hipLaunchKernelGGL(binary_same_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, n, op);
+        hipLaunchKernelGGL(binary_same_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, n, op, p);
     }
     return check_launch("binary_same");
+}
+
+// div_backward (src/native/src/ops/elementwise.rs:991-1029) before the unbroadcast
+__global__ void div_bwd_kernel(float *__restrict__ ga, float *__restrict__ gb, const float *__restrict__ g,
+                               const float *__restrict__ a, const float *__restrict__ b, const StridedDesc d, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) {
+        int64_t rem = i, ao = 0, bo = 0;
+        for (int k = d.ndim - 1; k >= 0; --k) {
+            const int64_t c = rem % d.shape[k];
+            rem /= d.shape[k];
+            ao += c * d.a_strides[k];
+            bo += c * d.b_strides[k];
+        }
+        const float gv = g[i], bv = b[bo];
+        ga[i] = gv / bv;
+        gb[i] = -gv * a[ao] / (bv * bv);
+    }
+}
+int k_div_backward(float *ga, float *gb, const float *g, const float *a, const float *b, const StridedDesc &d) {
+    MNI_TRY(ensure_init());
+    int64_t n = 1;
+    for (int i = 0; i < d.ndim; ++i) n *= d.shape[i];
+    if (n <= 0) return MNI_OK;
+    hipLaunchKernelGGL(div_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, ga, gb, g, a, b, d, n);
+    return check_launch("div_backward");
 }
 
 // out[r, c] = a[r, c] + bias[c]   (src/native/kernels/elementwise.cu:43-47)
@@ -278,6 +314,10 @@ __device__ __forceinline__ float un_apply(float x, int op, float s) {
     case UN_GELU: return d_gelu(x);
     case UN_NEG: return -x;
     case UN_SCALE: return x * s;
+    case UN_EXP: return expf(x);                        // elementwise.rs:760-770
+    case UN_LOG: return logf(x);                        // :839-849
+    case UN_SIGMOID: return 1.0f / (1.0f + expf(-x));   // activation.rs:194-204
+    case UN_POW: return powf(x, s);                     // elementwise.rs:1341-1351
     default: return x;
     }
 }
@@ -321,6 +361,24 @@ int k_unary_backward(float *out, const float *g, const float *x, int64_t n, int 
     MNI_TRY(ensure_init());
     hipLaunchKernelGGL(unary_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, x, n, op);
     return check_launch("unary_backward");
+}
+
+// exp / log / sigmoid / pow backward (elementwise.rs:800-809, 879-888, 1375-1386; activation.rs:231-241)
+__global__ void unary2_bwd_kernel(float *__restrict__ out, const float *__restrict__ g, const float *__restrict__ saved,
+                                  int64_t n, int op, float s) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) {
+        const float gv = g[i], v = saved[i];
+        out[i] = op == UN_EXP ? gv * v : op == UN_LOG ? gv / v : op == UN_SIGMOID ? gv * v * (1.0f - v)
+                                                               : gv * s * powf(v, s - 1.0f);
+    }
+}
+int k_unary2_backward(float *out, const float *g, const float *saved, int64_t n, int op, float s) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(unary2_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, saved, n, op, s);
+    return check_launch("unary2_backward");
 }
 
 // mul_backward for equal shapes (src/native/src/ops/elementwise.rs:348-390)
@@ -495,6 +553,162 @@ int k_bias_gelu_backward(float *dx, float *dbias, const float *g, const float *x
         rc = check_launch("colsum_final");
     }
     if (part) dev_free(part);
+    return rc;
+}
+
+// ---- max along one dim (src/native/src/ops/reduce.rs:333-368, 416-447) --------------------
+__global__ void max_dim_kernel(float *__restrict__ out, const float *__restrict__ a, int64_t outer, int64_t dim,
+                               int64_t inner) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= outer * inner) return;
+    const int64_t o = idx / inner, i = idx - o * inner;
+    const float *p = a + o * dim * inner + i;
+    float m = -INFINITY;
+    for (int64_t d = 0; d < dim; ++d) {
+        const float v = p[d * inner];
+        if (v > m) m = v;  // strict >, like the reference (a NaN never replaces the maximum)
+    }
+    out[idx] = m;
+}
+__global__ void max_rows_kernel(float *__restrict__ out, const float *__restrict__ a, int64_t outer, int64_t dim) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= outer) return;
+    const float *p = a + row * dim;
+    float m = -INFINITY;
+    for (int64_t d = lane; d < dim; d += 64) {
+        const float v = p[d];
+        if (v > m) m = v;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float o = __shfl_xor(m, off, 64);
+        if (o > m) m = o;
+    }
+    if (lane == 0) out[row] = m;
+}
+int k_max_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t inner) {
+    const int64_t n = outer * inner;
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (inner == 1 && dim >= 256)
+        hipLaunchKernelGGL(max_rows_kernel, dim3(grid_for(outer, 4)), dim3(TPB), 0, ctx().stream, out, a, outer, dim);
+    else
+        hipLaunchKernelGGL(max_dim_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, inner);
+    return check_launch("max_dim");
+}
+__global__ void max_bwd_kernel(float *__restrict__ out, const float *__restrict__ x, const float *__restrict__ mx,
+                               const float *__restrict__ g, int64_t dim, int64_t inner, int64_t n) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; idx < n; idx += step) {
+        const int64_t o = idx / (dim * inner), i = idx % inner;
+        const int64_t mi = o * inner + i;
+        out[idx] = fabsf(x[idx] - mx[mi]) < 1e-6f ? g[mi] : 0.0f;
+    }
+}
+int k_max_backward(float *out, const float *x, const float *mx, const float *g, int64_t outer, int64_t dim, int64_t inner) {
+    const int64_t n = outer * dim * inner;
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(max_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, mx, g, dim, inner, n);
+    return check_launch("max_backward");
+}
+
+// ---- layernorm over the last extent (src/native/src/ops/norm.rs:167-215, 273-322) -------------
+// One wavefront per row: mean, biased variance (second pass over the centred
+// values, as the reference), rstd = 1 / sqrt(var / c + eps).
+__device__ __forceinline__ float ew_wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__global__ void layernorm_kernel(float *__restrict__ out, float *__restrict__ mean, float *__restrict__ rstd,
+                                 const float *__restrict__ x, const float *__restrict__ gamma,
+                                 const float *__restrict__ beta, int64_t rows, int64_t c, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *p = x + row * c;
+    float s = 0.f;
+    for (int64_t j = lane; j < c; j += 64) s += p[j];
+    const float m = ew_wave_sum(s) / (float)c;
+    float v = 0.f;
+    for (int64_t j = lane; j < c; j += 64) { const float d = p[j] - m; v += d * d; }
+    const float r = 1.0f / sqrtf(ew_wave_sum(v) / (float)c + eps);
+    for (int64_t j = lane; j < c; j += 64) out[row * c + j] = (p[j] - m) * r * gamma[j] + beta[j];
+    if (lane == 0) { mean[row] = m; rstd[row] = r; }
+}
+int k_layernorm(float *out, float *mean, float *rstd, const float *x, const float *gamma, const float *beta, int64_t rows,
+                int64_t c, float eps) {
+    if (rows <= 0 || c <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(layernorm_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, mean, rstd, x, gamma, beta,
+                       rows, c, eps);
+    return check_launch("layernorm");
+}
+// dx per row (one wavefront per row)
+__global__ void layernorm_bwd_rows_kernel(float *__restrict__ dx, const float *__restrict__ g, const float *__restrict__ x,
+                                          const float *__restrict__ gamma, const float *__restrict__ mean,
+                                          const float *__restrict__ rstd, int64_t rows, int64_t c) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float m = mean[row], r = rstd[row];
+    const float *px = x + row * c, *pg = g + row * c;
+    float sum_dg = 0.f, sum_dgx = 0.f;
+    for (int64_t j = lane; j < c; j += 64) {
+        const float xhat = (px[j] - m) * r, dg = pg[j] * gamma[j];
+        sum_dg += dg;
+        sum_dgx += dg * xhat;
+    }
+    sum_dg = ew_wave_sum(sum_dg);
+    sum_dgx = ew_wave_sum(sum_dgx);
+    for (int64_t j = lane; j < c; j += 64) {
+        const float xhat = (px[j] - m) * r, dg = pg[j] * gamma[j];
+        dx[row * c + j] = r * (dg - sum_dg / (float)c - xhat * sum_dgx / (float)c);
+    }
+}
+// dgamma / dbeta: column sums of g * xhat and g over row blocks, partials summed in block order
+__global__ void layernorm_bwd_cols_kernel(float *__restrict__ pgamma, float *__restrict__ pbeta, const float *__restrict__ g,
+                                          const float *__restrict__ x, const float *__restrict__ mean,
+                                          const float *__restrict__ rstd, int64_t rows, int64_t c) {
+    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= c) return;
+    const int64_t r0 = (int64_t)blockIdx.y * BG_ROWS;
+    const int64_t r1 = min(rows, r0 + BG_ROWS);
+    float sg = 0.f, sb = 0.f;
+    for (int64_t r = r0; r < r1; ++r) {
+        const float gv = g[r * c + j];
+        sg += gv * ((x[r * c + j] - mean[r]) * rstd[r]);
+        sb += gv;
+    }
+    pgamma[(int64_t)blockIdx.y * c + j] = sg;
+    pbeta[(int64_t)blockIdx.y * c + j] = sb;
+}
+int k_layernorm_backward(float *dx, float *dgamma, float *dbeta, const float *g, const float *x, const float *gamma,
+                         const float *mean, const float *rstd, int64_t rows, int64_t c) {
+    if (c <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (rows <= 0) { MNI_TRY(k_fill(dgamma, 0.0f, c)); return k_fill(dbeta, 0.0f, c); }
+    hipLaunchKernelGGL(layernorm_bwd_rows_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, dx, g, x, gamma, mean,
+                       rstd, rows, c);
+    MNI_TRY(check_launch("layernorm_backward_rows"));
+    const int64_t nparts = (rows + BG_ROWS - 1) / BG_ROWS;
+    if (nparts > 65535) return set_error(MNI_ERR_INVALID, "layernorm backward: too many rows (%lld)", (long long)rows);
+    void *part = nullptr;
+    MNI_TRY(dev_alloc(&part, (size_t)2 * nparts * c * sizeof(float)));
+    float *pg = (float *)part, *pb = pg + nparts * c;
+    const unsigned gx = (unsigned)((c + TPB - 1) / TPB);
+    hipLaunchKernelGGL(layernorm_bwd_cols_kernel, dim3(gx, (unsigned)nparts), dim3(TPB), 0, ctx().stream, pg, pb, g, x, mean,
+                       rstd, rows, c);
+    int rc = check_launch("layernorm_backward_cols");
+    if (rc == MNI_OK) {
+        hipLaunchKernelGGL(colsum_final_kernel, dim3(gx), dim3(TPB), 0, ctx().stream, dgamma, (const float *)pg, nparts, c);
+        hipLaunchKernelGGL(colsum_final_kernel, dim3(gx), dim3(TPB), 0, ctx().stream, dbeta, (const float *)pb, nparts, c);
+        rc = check_launch("colsum_final");
+    }
+    dev_free(part);
     return rc;
 }
 

@@ -50,7 +50,8 @@ struct Tensor {
 enum Op {  // subset of src/native/src/autograd.rs:28-62 plus the fused Linear
     OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
     OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY, OP_LINEAR,
-    OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU
+    OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU,
+    OP_EXP, OP_LOG, OP_DIV, OP_SIGMOID, OP_POW, OP_MAX, OP_LAYERNORM
 };
 
 // src/native/src/autograd.rs:65-70 TapeEntry
@@ -413,7 +414,9 @@ static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out) {
 
 // ---- elementwise ---------------------------------------------------------------------
 // ops/elementwise.rs:20-73,237-248,474-485
-static uint32_t binary_op(uint32_t a, uint32_t b, int op) {
+// div (:918-928) is recorded like add / sub / mul; the comparisons lt / eq / gt / is_close (:1099-1288)
+// produce 1.0 / 0.0 and record nothing.
+static uint32_t binary_op(uint32_t a, uint32_t b, int op, float tol = 0.f) {
     Tensor *A = get(a), *B = get(b);
     if (!A || !B) return MNI_BAD_ID;
     Shape out_shape;
@@ -427,7 +430,7 @@ static uint32_t binary_op(uint32_t a, uint32_t b, int op) {
     int rc;
     const bool a_c = is_contiguous(*A), b_c = is_contiguous(*B);
     if (A->shape == B->shape && a_c && b_c) {
-        rc = k_binary_same(out->p, A->buf->p, B->buf->p, n, op);
+        rc = k_binary_same(out->p, A->buf->p, B->buf->p, n, op, tol);
     } else if (op == BIN_ADD && a_c && b_c && A->shape == out_shape && B->shape.size() == 1 &&
                B->shape[0] == out_shape.back()) {
         rc = k_add_bias(out->p, A->buf->p, B->buf->p, n / out_shape.back(), out_shape.back());
@@ -440,12 +443,13 @@ static uint32_t binary_op(uint32_t a, uint32_t b, int op) {
             d.a_strides[i] = (i < ao || A->shape[i - ao] == 1) ? 0 : A->strides[i - ao];
             d.b_strides[i] = (i < bo || B->shape[i - bo] == 1) ? 0 : B->strides[i - bo];
         }
-        rc = k_binary_broadcast(out->p, A->buf->p, B->buf->p, d, op);
+        rc = k_binary_broadcast(out->p, A->buf->p, B->buf->p, d, op, tol);
     }
     if (rc != MNI_OK) return MNI_BAD_ID;
     const uint32_t id = insert_contig(std::move(out), out_shape);
+    if (op >= BIN_LT) return id;
     Entry e;
-    e.op = op == BIN_ADD ? OP_ADD : op == BIN_SUB ? OP_SUB : OP_MUL;
+    e.op = op == BIN_ADD ? OP_ADD : op == BIN_SUB ? OP_SUB : op == BIN_MUL ? OP_MUL : OP_DIV;
     e.output_id = id; e.n_inputs = 2; e.inputs[0] = a; e.inputs[1] = b;
     e.saved_shape = out_shape;
     eng().tape.record(std::move(e));
@@ -767,6 +771,142 @@ static int cross_entropy_backward(uint32_t grad, const Entry &e, int64_t *out) {
     return MNI_OK;
 }
 
+// ops/elementwise.rs:991-1029 div_backward: da = g / b, db = -g a / b^2, then unbroadcast
+static int div_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *A = get(e.inputs[0]), *B = get(e.inputs[1]), *G = get(grad);
+    if (!A || !B || !G) return MNI_ERR_FREED;
+    const Shape a_shape = A->shape, b_shape = B->shape, g_shape = G->shape;
+    const int64_t n = shape_size(g_shape);
+    BufP gsrc = contiguous_buf(*G);
+    BufP ga_full = new_buf((size_t)n), gb_full = new_buf((size_t)n);
+    if (!gsrc || !ga_full || !gb_full) return MNI_ERR_NOMEM;
+    StridedDesc d;
+    d.ndim = (int)g_shape.size();
+    const int ao = d.ndim - (int)a_shape.size(), bo = d.ndim - (int)b_shape.size();
+    for (int i = 0; i < d.ndim; ++i) {
+        d.shape[i] = g_shape[i];
+        d.a_strides[i] = (i < ao || a_shape[i - ao] == 1) ? 0 : A->strides[i - ao];
+        d.b_strides[i] = (i < bo || b_shape[i - bo] == 1) ? 0 : B->strides[i - bo];
+    }
+    MNI_TRY(k_div_backward(ga_full->p, gb_full->p, gsrc->p, A->buf->p, B->buf->p, d));
+    const uint32_t fa = insert_contig(std::move(ga_full), g_shape);
+    const uint32_t fb = insert_contig(std::move(gb_full), g_shape);
+    const uint32_t ga = unbroadcast_tensor(fa, a_shape);
+    const uint32_t gb = unbroadcast_tensor(fb, b_shape);
+    free_tensor(fa);
+    free_tensor(fb);
+    if (ga == MNI_BAD_ID || gb == MNI_BAD_ID) return MNI_ERR_INVALID;
+    out[0] = ga; out[1] = gb;
+    return MNI_OK;
+}
+
+// exp / log / pow (ops/elementwise.rs:760-770, 839-849, 1341-1351) and sigmoid
+// (ops/activation.rs:194-204).  exp and sigmoid save their output, log and pow
+// their input, as the reference's tape does.
+static uint32_t unary2_op(uint32_t a, int un, int tape_op, float s) {
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    BufP src = contiguous_buf(*A);
+    BufP out = src ? new_buf((size_t)A->size) : nullptr;
+    if (!out || k_unary(out->p, src->p, A->size, un, s) != MNI_OK) return MNI_BAD_ID;
+    const Shape shape = A->shape;
+    const uint32_t id = insert_contig(std::move(out), shape);
+    Entry e;
+    e.op = tape_op; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a; e.scalar = s;
+    e.aux = (un == UN_EXP || un == UN_SIGMOID) ? id : a;
+    eng().tape.record(std::move(e));
+    return id;
+}
+static int unary2_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *G = get(grad), *S = get(e.aux);
+    if (!G || !S) return MNI_ERR_FREED;
+    const Shape shape = G->shape;
+    BufP g = contiguous_buf(*G), sv = contiguous_buf(*S);
+    BufP o = (g && sv) ? new_buf((size_t)G->size) : nullptr;
+    if (!o) return MNI_ERR_NOMEM;
+    const int un = e.op == OP_EXP ? UN_EXP : e.op == OP_LOG ? UN_LOG : e.op == OP_SIGMOID ? UN_SIGMOID : UN_POW;
+    MNI_TRY(k_unary2_backward(o->p, g->p, sv->p, G->size, un, e.scalar));
+    out[0] = insert_contig(std::move(o), shape);
+    return MNI_OK;
+}
+
+// ops/reduce.rs:333-368 max along dim (kept as size 1), :416-447 its backward
+static uint32_t max_op(uint32_t a, int64_t dim) {
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    const int nd = (int)A->shape.size();
+    const int d = (int)(dim < 0 ? nd + dim : dim);
+    if (d < 0 || d >= nd) { set_error(MNI_ERR_INVALID, "max dim %lld out of range for rank %d", (long long)dim, nd); return MNI_BAD_ID; }
+    const Shape a_shape = A->shape;
+    Shape out_shape = a_shape;
+    out_shape[d] = 1;
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < d; ++i) outer *= a_shape[i];
+    for (int i = d + 1; i < nd; ++i) inner *= a_shape[i];
+    BufP src = contiguous_buf(*A);
+    BufP out = src ? new_buf((size_t)shape_size(out_shape)) : nullptr;
+    if (!out || k_max_dim(out->p, src->p, outer, a_shape[d], inner) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(out), out_shape);
+    Entry e;
+    e.op = OP_MAX; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a; e.aux = id; e.scalar = (float)d;
+    eng().tape.record(std::move(e));
+    return id;
+}
+static int max_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *X = get(e.inputs[0]), *M = get(e.aux), *G = get(grad);
+    if (!X || !M || !G) return MNI_ERR_FREED;
+    const Shape shape = X->shape;
+    const int nd = (int)shape.size(), d = (int)e.scalar;
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < d; ++i) outer *= shape[i];
+    for (int i = d + 1; i < nd; ++i) inner *= shape[i];
+    BufP x = contiguous_buf(*X), m = contiguous_buf(*M), g = contiguous_buf(*G);
+    BufP o = (x && m && g) ? new_buf((size_t)X->size) : nullptr;
+    if (!o) return MNI_ERR_NOMEM;
+    MNI_TRY(k_max_backward(o->p, x->p, m->p, g->p, outer, shape[d], inner));
+    out[0] = insert_contig(std::move(o), shape);
+    return MNI_OK;
+}
+
+// ops/norm.rs:167-215 layernorm over the last extent; saves mean and rstd per row
+static uint32_t layernorm_op(uint32_t x, uint32_t gamma, uint32_t beta, float eps) {
+    Tensor *X = get(x), *Gm = get(gamma), *Bt = get(beta);
+    if (!X || !Gm || !Bt) return MNI_BAD_ID;
+    if (X->shape.empty()) { set_error(MNI_ERR_INVALID, "layernorm: x must have at least one dim"); return MNI_BAD_ID; }
+    const Shape shape = X->shape;
+    const int64_t c = shape.back(), rows = c ? X->size / c : 0;
+    if (Gm->size < c || Bt->size < c) { set_error(MNI_ERR_INVALID, "layernorm: gamma / beta hold fewer than %lld values", (long long)c); return MNI_BAD_ID; }
+    BufP xs = contiguous_buf(*X), gs = contiguous_buf(*Gm), bs = contiguous_buf(*Bt);
+    BufP out = (xs && gs && bs) ? new_buf((size_t)X->size) : nullptr;
+    BufP mean = out ? new_buf((size_t)rows) : nullptr, rstd = mean ? new_buf((size_t)rows) : nullptr;
+    if (!rstd || k_layernorm(out->p, mean->p, rstd->p, xs->p, gs->p, bs->p, rows, c, eps) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t out_id = insert_contig(std::move(out), shape);
+    const uint32_t mean_id = insert_contig(std::move(mean), Shape{rows});
+    const uint32_t rstd_id = insert_contig(std::move(rstd), Shape{rows});
+    Entry e;
+    e.op = OP_LAYERNORM; e.output_id = out_id; e.n_inputs = 3;
+    e.inputs[0] = x; e.inputs[1] = gamma; e.inputs[2] = beta; e.aux = mean_id; e.aux2 = rstd_id;
+    eng().tape.record(std::move(e));
+    return out_id;
+}
+// ops/norm.rs:273-322
+static int layernorm_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *X = get(e.inputs[0]), *Gm = get(e.inputs[1]), *Mn = get(e.aux), *Rs = get(e.aux2), *G = get(grad);
+    if (!X || !Gm || !Mn || !Rs || !G) return MNI_ERR_FREED;
+    const Shape shape = X->shape, gshape = Gm->shape;
+    const int64_t c = shape.back(), rows = c ? X->size / c : 0;
+    BufP xs = contiguous_buf(*X), gs = contiguous_buf(*Gm), g = contiguous_buf(*G);
+    BufP dx = (xs && gs && g) ? new_buf((size_t)X->size) : nullptr;
+    BufP dgamma = dx ? new_buf((size_t)Gm->size) : nullptr, dbeta = dgamma ? new_buf((size_t)Gm->size) : nullptr;
+    if (!dbeta) return MNI_ERR_NOMEM;
+    if (Gm->size > c) { MNI_TRY(k_fill(dgamma->p, 0.0f, Gm->size)); MNI_TRY(k_fill(dbeta->p, 0.0f, Gm->size)); }
+    MNI_TRY(k_layernorm_backward(dx->p, dgamma->p, dbeta->p, g->p, xs->p, gs->p, Mn->buf->p, Rs->buf->p, rows, c));
+    out[0] = insert_contig(std::move(dx), shape);
+    out[1] = insert_contig(std::move(dgamma), gshape);
+    out[2] = insert_contig(std::move(dbeta), gshape);
+    return MNI_OK;
+}
+
 // ---- fused bias + GELU ------------------------------------------------------------------------------
 // ops/fused.rs:247-273: out = gelu(x + bias[i % c]), c = last extent of x.
 static uint32_t bias_gelu_op(uint32_t x, uint32_t bias) {
@@ -1020,6 +1160,10 @@ static int dispatch_backward(const Entry &e, uint32_t grad, int64_t *out) {  // 
     case OP_CONTIGUOUS: out[0] = grad; return MNI_OK;  // layout.rs:229-231
     case OP_CROSSENTROPY: return cross_entropy_backward(grad, e, out);
     case OP_LINEAR: return linear_backward(grad, e, out);
+    case OP_EXP: case OP_LOG: case OP_SIGMOID: case OP_POW: return unary2_backward(grad, e, out);
+    case OP_DIV: return div_backward(grad, e, out);
+    case OP_MAX: return max_backward(grad, e, out);
+    case OP_LAYERNORM: return layernorm_backward(grad, e, out);
     case OP_BIASGELU: return bias_gelu_backward(grad, e, out);               // autograd.rs BiasGelu
     case OP_SOFTMAX: return softmax_backward(grad, e, out);                  // autograd.rs:204
     case OP_FLASHATTENTION: return flash_attention_backward(grad, e, out);   // autograd.rs:210
@@ -1349,6 +1493,20 @@ uint32_t mni_contiguous(uint32_t a) {  // layout.rs:218-227
     e.op = OP_CONTIGUOUS; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a;
     eng().tape.record(std::move(e));
     return id;
+}
+uint32_t mni_exp_op(uint32_t a) { MNI_API_GUARD; return unary2_op(a, UN_EXP, OP_EXP, 0.f); }
+uint32_t mni_log_op(uint32_t a) { MNI_API_GUARD; return unary2_op(a, UN_LOG, OP_LOG, 0.f); }
+uint32_t mni_sigmoid(uint32_t a) { MNI_API_GUARD; return unary2_op(a, UN_SIGMOID, OP_SIGMOID, 0.f); }
+uint32_t mni_pow_op(uint32_t a, double exponent) { MNI_API_GUARD; return unary2_op(a, UN_POW, OP_POW, (float)exponent); }
+uint32_t mni_div(uint32_t a, uint32_t b) { MNI_API_GUARD; return binary_op(a, b, BIN_DIV); }
+uint32_t mni_lt(uint32_t a, uint32_t b) { MNI_API_GUARD; return binary_op(a, b, BIN_LT); }
+uint32_t mni_eq_op(uint32_t a, uint32_t b) { MNI_API_GUARD; return binary_op(a, b, BIN_EQ); }
+uint32_t mni_gt(uint32_t a, uint32_t b) { MNI_API_GUARD; return binary_op(a, b, BIN_GT); }
+uint32_t mni_is_close(uint32_t a, uint32_t b, double tol) { MNI_API_GUARD; return binary_op(a, b, BIN_CLOSE, (float)tol); }
+uint32_t mni_max_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return max_op(a, dim); }
+uint32_t mni_layernorm_op(uint32_t x, uint32_t gamma, uint32_t beta, double eps) {
+    MNI_API_GUARD;
+    return layernorm_op(x, gamma, beta, (float)eps);
 }
 uint32_t mni_bias_gelu(uint32_t x, uint32_t bias) { MNI_API_GUARD; return bias_gelu_op(x, bias); }
 uint32_t mni_softmax_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return softmax_op(a, dim); }

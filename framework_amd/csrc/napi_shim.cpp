@@ -119,6 +119,14 @@ BINARY(Sub, mni_sub)                     // lib.rs:178-183
 UNARY(Neg, mni_neg)                      // lib.rs:185-190
 BINARY(Matmul, mni_matmul)               // lib.rs:199-204
 BINARY(BiasGelu, mni_bias_gelu)          // lib.rs:526-531
+UNARY(ExpOp, mni_exp_op)                 // lib.rs:220-225
+UNARY(LogOp, mni_log_op)                 // lib.rs:227-232
+UNARY(Sigmoid, mni_sigmoid)              // lib.rs:374-379
+BINARY(Div, mni_div)                     // lib.rs:339-344
+BINARY(Lt, mni_lt)                       // lib.rs:346-351
+BINARY(EqOp, mni_eq_op)                  // lib.rs:353-358
+BINARY(Gt, mni_gt)                       // lib.rs:360-365
+WITH_DIM(MaxOp, mni_max_op)              // lib.rs:248-253
 UNARY(Gelu, mni_gelu)                    // lib.rs:206-211
 UNARY(Relu, mni_relu)                    // lib.rs:213-218
 WITH_DIM(SumOp, mni_sum_op)              // lib.rs:234-239
@@ -257,6 +265,18 @@ napi_value GcTensors(napi_env env, napi_callback_info info) {  // lib.rs:693-706
     return ret_rc(env, mni_gc_tensors(ids.data(), ids.size()));
 }
 // Opt-in fused Linear (no counterpart in lib.rs; feature-detected by callers).
+napi_value PowOp(napi_env env, napi_callback_info info) {  // lib.rs:381-386
+    Args a(env, info);
+    return ret_id(env, mni_pow_op(get_u32(env, a.v[0]), get_f64(env, a.v[1])));
+}
+napi_value IsClose(napi_env env, napi_callback_info info) {  // lib.rs:367-372
+    Args a(env, info);
+    return ret_id(env, mni_is_close(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_f64(env, a.v[2])));
+}
+napi_value LayernormOp(napi_env env, napi_callback_info info) {  // lib.rs:309-315
+    Args a(env, info);
+    return ret_id(env, mni_layernorm_op(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_u32(env, a.v[2]), get_f64(env, a.v[3])));
+}
 napi_value FlashAttention(napi_env env, napi_callback_info info) {  // lib.rs:575-584
     Args a(env, info);
     return ret_id(env, mni_flash_attention(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_u32(env, a.v[2]),
@@ -284,7 +304,10 @@ NAPI_MODULE_INIT() {
         EXPORT("contiguous", Contiguous), EXPORT("crossEntropyLoss", CrossEntropyLoss), EXPORT("adamwStep", AdamwStep),
         EXPORT("gradNorm", GradNorm), EXPORT("clipGradNorm", ClipGradNorm), EXPORT("clipAndStep", ClipAndStep),
         EXPORT("resetEngine", ResetEngine), EXPORT("gcTensors", GcTensors), EXPORT("linear", Linear),
-        EXPORT("softmaxOp", SoftmaxOp), EXPORT("biasGelu", BiasGelu), EXPORT("flashAttention", FlashAttention),
+        EXPORT("softmaxOp", SoftmaxOp), EXPORT("biasGelu", BiasGelu),
+        EXPORT("expOp", ExpOp), EXPORT("logOp", LogOp), EXPORT("sigmoid", Sigmoid), EXPORT("powOp", PowOp),
+        EXPORT("div", Div), EXPORT("lt", Lt), EXPORT("eqOp", EqOp), EXPORT("gt", Gt), EXPORT("isClose", IsClose),
+        EXPORT("maxOp", MaxOp), EXPORT("layernormOp", LayernormOp), EXPORT("flashAttention", FlashAttention),
 #undef EXPORT
     };
     napi_define_properties(env, exports, sizeof(props) / sizeof(props[0]), props);

@@ -102,6 +102,13 @@ SIGNATURES = {
     "mni_contiguous": (C.c_uint32, [C.c_uint32]),
     "mni_softmax_op": (C.c_uint32, [C.c_uint32, C.c_int64]),
     "mni_bias_gelu": (C.c_uint32, [C.c_uint32, C.c_uint32]),
+    "mni_exp_op": (C.c_uint32, [C.c_uint32]), "mni_log_op": (C.c_uint32, [C.c_uint32]),
+    "mni_sigmoid": (C.c_uint32, [C.c_uint32]), "mni_pow_op": (C.c_uint32, [C.c_uint32, C.c_double]),
+    "mni_div": (C.c_uint32, [C.c_uint32, C.c_uint32]), "mni_lt": (C.c_uint32, [C.c_uint32, C.c_uint32]),
+    "mni_eq_op": (C.c_uint32, [C.c_uint32, C.c_uint32]), "mni_gt": (C.c_uint32, [C.c_uint32, C.c_uint32]),
+    "mni_is_close": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_double]),
+    "mni_max_op": (C.c_uint32, [C.c_uint32, C.c_int64]),
+    "mni_layernorm_op": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double]),
     "mni_flash_attention": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double, C.c_int]),
     "mni_cross_entropy_loss": (C.c_uint32, [C.c_uint32, _i64p, C.c_size_t]),
     "mni_adamw_step": (C.c_int, [_u32p, C.c_size_t, C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, C.c_int64]),
@@ -391,6 +398,39 @@ class Native:
 
     def biasGelu(self, x, bias):
         return self._id(self.lib.mni_bias_gelu(x, bias))
+
+    def expOp(self, a):
+        return self._id(self.lib.mni_exp_op(a))
+
+    def logOp(self, a):
+        return self._id(self.lib.mni_log_op(a))
+
+    def sigmoid(self, a):
+        return self._id(self.lib.mni_sigmoid(a))
+
+    def powOp(self, a, exponent):
+        return self._id(self.lib.mni_pow_op(a, exponent))
+
+    def div(self, a, b):
+        return self._id(self.lib.mni_div(a, b))
+
+    def lt(self, a, b):
+        return self._id(self.lib.mni_lt(a, b))
+
+    def eqOp(self, a, b):
+        return self._id(self.lib.mni_eq_op(a, b))
+
+    def gt(self, a, b):
+        return self._id(self.lib.mni_gt(a, b))
+
+    def isClose(self, a, b, tol):
+        return self._id(self.lib.mni_is_close(a, b, tol))
+
+    def maxOp(self, a, dim):
+        return self._id(self.lib.mni_max_op(a, dim))
+
+    def layernormOp(self, x, gamma, beta, eps):
+        return self._id(self.lib.mni_layernorm_op(x, gamma, beta, eps))
 
     def flashAttention(self, q, k, v, scale, causal):
         return self._id(self.lib.mni_flash_attention(q, k, v, scale, 1 if causal else 0))

@@ -175,7 +175,24 @@ uint32_t mni_sum_all(uint32_t a);                                         /* lib
 uint32_t mni_mean_all(uint32_t a);                                        /* lib.rs:267-277 */
 uint32_t mni_view(uint32_t a, const int64_t *shape, int ndim);            /* lib.rs:279-285 */
 uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim);          /* lib.rs:287-293 */
-uint32_t mni_contiguous(uint32_t a);                                      /* bias_gelu (src/native/src/lib.rs:526-531 -> ops/fused.rs:247-273, backward :316-351):
+uint32_t mni_contiguous(uint32_t a);                                      /* Remaining elementwise / reduction exports of src/native/src/lib.rs, all on the device:
+ * exp_op (:220-225), log_op (:227-232), sigmoid (:374-379), pow_op (:381-386; powf),
+ * div (:339-344; broadcasting, backward da = g / b, db = -g a / b^2),
+ * lt / eq_op / gt / is_close (:346-372; 1.0 or 0.0, nothing recorded),
+ * max_op (:248-253; dim kept as size 1, the gradient goes to every element within 1e-6 of the maximum),
+ * layernorm_op (:309-315; over the last extent, backward yields dx, dgamma, dbeta). */
+uint32_t mni_exp_op(uint32_t a);
+uint32_t mni_log_op(uint32_t a);
+uint32_t mni_sigmoid(uint32_t a);
+uint32_t mni_pow_op(uint32_t a, double exponent);
+uint32_t mni_div(uint32_t a, uint32_t b);
+uint32_t mni_lt(uint32_t a, uint32_t b);
+uint32_t mni_eq_op(uint32_t a, uint32_t b);
+uint32_t mni_gt(uint32_t a, uint32_t b);
+uint32_t mni_is_close(uint32_t a, uint32_t b, double tol);
+uint32_t mni_max_op(uint32_t a, int64_t dim);
+uint32_t mni_layernorm_op(uint32_t x, uint32_t gamma, uint32_t beta, double eps);
+/* bias_gelu (src/native/src/lib.rs:526-531 -> ops/fused.rs:247-273, backward :316-351):
  * out = gelu(x + bias) along the last extent; backward yields dx and the column sums dbias in one pass. */
 uint32_t mni_bias_gelu(uint32_t x, uint32_t bias);
 /* softmax_op (src/native/src/lib.rs:302-307 -> ops/norm.rs:10-50); backward as

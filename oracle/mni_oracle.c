@@ -52,7 +52,8 @@ typedef struct {
 enum orc_op { /* subset of autograd.rs:28-62 BackwardOp */
     OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
     OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY,
-    OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU
+    OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU,
+    OP_EXP, OP_LOG, OP_DIV, OP_SIGMOID, OP_POW, OP_MAX, OP_LAYERNORM
 };
 
 /* autograd.rs:65-70 TapeEntry + the SavedContext variants the subset needs */
@@ -431,8 +432,10 @@ static int matmul_backward(size_t grad, const orc_entry *e, long *out) {
 
 /* ---- elementwise -------------------------------------------------------- */
 
-/* ops/elementwise.rs:20-56 broadcast_binary; op: 0 add, 1 sub, 2 mul
+/* ops/elementwise.rs:20-56 broadcast_binary; op: 0 add, 1 sub, 2 mul, 3 div,
+ * 4 lt, 5 eq, 6 gt (1.0 / 0.0, :1099-1216), 7 is_close with tolerance `tol` (:1258-1288)
  * pinned by: test/tensor.test.ts:248-256 broadcast values, numpy broadcasting. */
+static float g_binary_tol;
 static uint32_t broadcast_binary(size_t a, size_t b, int op, size_t *out_shape, int *out_nd) {
     orc_tensor *A = get(a), *B = get(b);
     if (!A || !B) return fail("tensor already freed");
@@ -453,7 +456,9 @@ static uint32_t broadcast_binary(size_t a, size_t b, int op, size_t *out_shape, 
         for (int d = 0; d < A->ndim; ++d) ai += (A->shape[d] == 1 ? 0 : coord[d + a_off]) * astr[d];
         for (int d = 0; d < B->ndim; ++d) bi += (B->shape[d] == 1 ? 0 : coord[d + b_off]) * bstr[d];
         float x = ad[ai], y = bd[bi];
-        out[i] = op == 0 ? x + y : op == 1 ? x - y : x * y;
+        out[i] = op == 0 ? x + y : op == 1 ? x - y : op == 2 ? x * y : op == 3 ? x / y
+               : op == 4 ? (x < y ? 1.0f : 0.0f) : op == 5 ? (x == y ? 1.0f : 0.0f) : op == 6 ? (x > y ? 1.0f : 0.0f)
+               : (fabsf(x - y) < g_binary_tol ? 1.0f : 0.0f);
     }
     free(ad); free(bd);
     *out_nd = nd;
@@ -523,6 +528,94 @@ static int mul_backward(size_t grad, const orc_entry *e, long *out) {
     free(ad); free(bd); free(gd); free(ga_full); free(gb_full);
     out[0] = (long)from_vec(ga, a_shape, a_nd);
     out[1] = (long)from_vec(gb, b_shape, b_nd);
+    return 0;
+}
+
+/* ops/elementwise.rs:918-928 div; comparisons record nothing on the tape */
+static uint32_t div_op(size_t a, size_t b) {
+    size_t shape[ORC_MAX_DIMS]; int nd;
+    uint32_t out = broadcast_binary(a, b, 3, shape, &nd);
+    if (out == ORC_BAD) return out;
+    tape_record(&g_tape, OP_DIV, out, 2, a, b);
+    return out;
+}
+static uint32_t compare_op(size_t a, size_t b, int op, float tol) {
+    size_t shape[ORC_MAX_DIMS]; int nd;
+    g_binary_tol = tol;
+    return broadcast_binary(a, b, op, shape, &nd);
+}
+/* ops/elementwise.rs:991-1029 div_backward: da = g / b, db = -g * a / (b * b), unbroadcast.
+ * pinned by: float64 closed form with and without broadcasting. */
+static int div_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *A = get(e->saved_ids[0]), *B = get(e->saved_ids[1]), *G = get(grad);
+    if (!A || !B || !G) { fail("tensor already freed"); return -1; }
+    size_t a_shape[ORC_MAX_DIMS], b_shape[ORC_MAX_DIMS], g_shape[ORC_MAX_DIMS];
+    int a_nd = A->ndim, b_nd = B->ndim, nd = G->ndim;
+    memcpy(a_shape, A->shape, sizeof a_shape);
+    memcpy(b_shape, B->shape, sizeof b_shape);
+    memcpy(g_shape, G->shape, sizeof g_shape);
+    float *ad = to_host(A), *bd = to_host(B), *gd = to_host(G);
+    size_t gsz = shape_size(g_shape, nd);
+    size_t ostr[ORC_MAX_DIMS], astr[ORC_MAX_DIMS], bstr[ORC_MAX_DIMS];
+    compute_strides(g_shape, nd, ostr);
+    compute_strides(a_shape, a_nd, astr);
+    compute_strides(b_shape, b_nd, bstr);
+    float *ga_full = (float *)calloc(gsz ? gsz : 1, sizeof(float));
+    float *gb_full = (float *)calloc(gsz ? gsz : 1, sizeof(float));
+    int a_off = nd - a_nd, b_off = nd - b_nd;
+    for (size_t i = 0; i < gsz; ++i) {
+        size_t coord[ORC_MAX_DIMS], rem = i;
+        for (int d = 0; d < nd; ++d) { coord[d] = rem / ostr[d]; rem %= ostr[d]; }
+        size_t ai = 0, bi = 0;
+        for (int d = 0; d < a_nd; ++d) ai += (a_shape[d] == 1 ? 0 : coord[d + a_off]) * astr[d];
+        for (int d = 0; d < b_nd; ++d) bi += (b_shape[d] == 1 ? 0 : coord[d + b_off]) * bstr[d];
+        ga_full[i] = gd[i] / bd[bi];
+        gb_full[i] = -gd[i] * ad[ai] / (bd[bi] * bd[bi]);
+    }
+    float *ga = unbroadcast(ga_full, g_shape, nd, a_shape, a_nd);
+    float *gb = unbroadcast(gb_full, g_shape, nd, b_shape, b_nd);
+    free(ad); free(bd); free(gd); free(ga_full); free(gb_full);
+    out[0] = (long)from_vec(ga, a_shape, a_nd);
+    out[1] = (long)from_vec(gb, b_shape, b_nd);
+    return 0;
+}
+
+/* ops/elementwise.rs:760-770 exp, :839-849 log, :1341-1351 pow (powf);
+ * ops/activation.rs:194-204 sigmoid.  kind: 0 exp, 1 log, 2 sigmoid, 3 pow.
+ * Saved: exp and sigmoid keep their OUTPUT, log and pow their input.
+ * pinned by: float64 closed forms; derivative identities. */
+static uint32_t unary2_op(size_t a, int kind, float s) {
+    orc_tensor *A = get(a);
+    if (!A) return fail("tensor already freed");
+    float *d = to_host(A);
+    for (size_t i = 0; i < A->size; ++i) {
+        float x = d[i];
+        d[i] = kind == 0 ? expf(x) : kind == 1 ? logf(x) : kind == 2 ? 1.0f / (1.0f + expf(-x)) : powf(x, s);
+    }
+    size_t shape[ORC_MAX_DIMS]; int nd = A->ndim;
+    memcpy(shape, A->shape, sizeof shape);
+    size_t out = from_vec(d, shape, nd);
+    static const int ops[4] = {OP_EXP, OP_LOG, OP_SIGMOID, OP_POW};
+    orc_entry *e = tape_record(&g_tape, ops[kind], out, 1, a, 0);
+    e->saved_scalar = s;
+    e->saved_ids[0] = (kind == 0 || kind == 2) ? out : a;
+    return (uint32_t)out;
+}
+/* ops/elementwise.rs:800-809 exp_backward (g * out), :879-888 log_backward (g / x),
+ * :1375-1386 pow_backward (g * e * x^(e-1)); ops/activation.rs:231-241 sigmoid_backward (g * o * (1 - o)) */
+static int unary2_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *G = get(grad), *S = get(e->saved_ids[0]);
+    if (!G || !S) { fail("tensor already freed"); return -1; }
+    float *gd = to_host(G), *sd = to_host(S);
+    size_t shape[ORC_MAX_DIMS]; int nd = G->ndim; size_t n = G->size;
+    memcpy(shape, G->shape, sizeof shape);
+    for (size_t i = 0; i < n; ++i) {
+        float g = gd[i], v = sd[i];
+        gd[i] = e->op == OP_EXP ? g * v : e->op == OP_LOG ? g / v : e->op == OP_SIGMOID ? g * v * (1.0f - v)
+              : g * e->saved_scalar * powf(v, e->saved_scalar - 1.0f);
+    }
+    free(sd);
+    out[0] = (long)from_vec(gd, shape, nd);
     return 0;
 }
 
@@ -830,6 +923,143 @@ static int cross_entropy_backward(size_t grad, const orc_entry *e, long *out) {
     return 0;
 }
 
+/* ops/reduce.rs:333-368 max along dim (kept as size 1): strict `>` against a
+ * running maximum that starts at -inf, in flat order.
+ * pinned by: numpy max; ties; backward mask. */
+static uint32_t max_impl(size_t a, int dim) {
+    orc_tensor *A = get(a);
+    if (!A) return fail("tensor already freed");
+    int nd = A->ndim;
+    int d = resolve_dim(dim, nd);
+    if (d < 0 || d >= nd) return fail("index out of bounds: max dim");
+    size_t shape[ORC_MAX_DIMS], oshape[ORC_MAX_DIMS], astr[ORC_MAX_DIMS], ostr[ORC_MAX_DIMS];
+    memcpy(shape, A->shape, sizeof shape);
+    memcpy(oshape, shape, sizeof oshape);
+    oshape[d] = 1;
+    compute_strides(shape, nd, astr);
+    compute_strides(oshape, nd, ostr);
+    size_t total = shape_size(shape, nd), osz = shape_size(oshape, nd);
+    float *ad = to_host(A);
+    float *out = (float *)malloc((osz ? osz : 1) * sizeof(float));
+    for (size_t i = 0; i < osz; ++i) out[i] = -INFINITY;
+    for (size_t i = 0; i < total; ++i) {
+        size_t oi = 0, rem = i;
+        for (int dd = 0; dd < nd; ++dd) {
+            size_t coord = rem / astr[dd];
+            rem %= astr[dd];
+            oi += (dd == d ? 0 : coord) * ostr[dd];
+        }
+        if (ad[i] > out[oi]) out[oi] = ad[i];
+    }
+    free(ad);
+    size_t out_id = from_vec(out, oshape, nd);
+    orc_entry *e = tape_record(&g_tape, OP_MAX, out_id, 1, a, 0);
+    e->saved_ids[1] = out_id;
+    return (uint32_t)out_id;
+}
+/* ops/reduce.rs:416-447 max_backward: the grad goes to every element within
+ * 1e-6 of the maximum (ties all receive it). */
+static int max_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *X = get(e->saved_ids[0]), *M = get(e->saved_ids[1]), *G = get(grad);
+    if (!X || !M || !G) { fail("tensor already freed"); return -1; }
+    int nd = X->ndim;
+    size_t shape[ORC_MAX_DIMS], mshape[ORC_MAX_DIMS], xstr[ORC_MAX_DIMS], mstr[ORC_MAX_DIMS];
+    memcpy(shape, X->shape, sizeof shape);
+    memcpy(mshape, M->shape, sizeof mshape);
+    compute_strides(shape, nd, xstr);
+    compute_strides(mshape, nd, mstr);
+    float *xd = to_host(X), *md = to_host(M), *gd = to_host(G);
+    size_t total = shape_size(shape, nd);
+    float *o = (float *)calloc(total ? total : 1, sizeof(float));
+    for (size_t i = 0; i < total; ++i) {
+        size_t mi = 0, rem = i;
+        for (int dd = 0; dd < nd; ++dd) {
+            size_t coord = rem / xstr[dd];
+            rem %= xstr[dd];
+            mi += (mshape[dd] == 1 ? 0 : coord) * mstr[dd];
+        }
+        if (fabsf(xd[i] - md[mi]) < 1e-6f) o[i] = gd[mi];
+    }
+    free(xd); free(md); free(gd);
+    out[0] = (long)from_vec(o, shape, nd);
+    return 0;
+}
+
+/* ops/norm.rs:167-215 layernorm over the last extent: mean, biased variance
+ * (two passes, f32, index order), rstd = 1 / sqrt(var / c + eps).
+ * pinned by: float64 closed form; normalised rows have mean 0, variance 1 when
+ * gamma = 1, beta = 0; finite differences of the backward. */
+static uint32_t layernorm_impl(size_t x, size_t gamma, size_t beta, float eps) {
+    orc_tensor *X = get(x), *Gm = get(gamma), *Bt = get(beta);
+    if (!X || !Gm || !Bt) return fail("tensor already freed");
+    int nd = X->ndim;
+    if (nd < 1) return fail("index out of bounds: layernorm of a scalar");
+    size_t shape[ORC_MAX_DIMS];
+    memcpy(shape, X->shape, sizeof shape);
+    size_t c = shape[nd - 1];
+    size_t n = c ? shape_size(shape, nd) / c : 0;
+    if (Gm->size < c || Bt->size < c) return fail("index out of bounds: gamma/beta shorter than the last extent");
+    float *xd = to_host(X), *gd = to_host(Gm), *bd = to_host(Bt);
+    float *mean = (float *)calloc(n ? n : 1, sizeof(float)), *rstd = (float *)calloc(n ? n : 1, sizeof(float));
+    float *out = (float *)calloc((n * c) > 0 ? n * c : 1, sizeof(float));
+    for (size_t row = 0; row < n; ++row) {
+        size_t off = row * c;
+        float sum = 0.0f;
+        for (size_t j = 0; j < c; ++j) sum += xd[off + j];
+        float m = sum / (float)c;
+        mean[row] = m;
+        float var = 0.0f;
+        for (size_t j = 0; j < c; ++j) { float d = xd[off + j] - m; var += d * d; }
+        float r = 1.0f / sqrtf(var / (float)c + eps);
+        rstd[row] = r;
+        for (size_t j = 0; j < c; ++j) out[off + j] = (xd[off + j] - m) * r * gd[j] + bd[j];
+    }
+    free(xd); free(gd); free(bd);
+    size_t mean_id = from_vec(mean, &n, 1), rstd_id = from_vec(rstd, &n, 1);
+    size_t out_id = from_vec(out, shape, nd);
+    orc_entry *e = tape_record(&g_tape, OP_LAYERNORM, out_id, 3, x, gamma);
+    e->input_ids[2] = beta; e->saved_ids[2] = beta;
+    e->fa_out = mean_id; e->fa_lse = rstd_id; /* Tensors[x, gamma, mean, rstd] */
+    return (uint32_t)out_id;
+}
+/* ops/norm.rs:273-322 layernorm_backward */
+static int layernorm_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *X = get(e->input_ids[0]), *Gm = get(e->input_ids[1]), *Mn = get(e->fa_out), *Rs = get(e->fa_lse), *G = get(grad);
+    if (!X || !Gm || !Mn || !Rs || !G) { fail("tensor already freed"); return -1; }
+    int nd = X->ndim, gnd = Gm->ndim;
+    size_t shape[ORC_MAX_DIMS], gshape[ORC_MAX_DIMS];
+    memcpy(shape, X->shape, sizeof shape);
+    memcpy(gshape, Gm->shape, sizeof gshape);
+    size_t c = shape[nd - 1], n = c ? shape_size(shape, nd) / c : 0;
+    float *xd = to_host(X), *gm = to_host(Gm), *mn = to_host(Mn), *rs = to_host(Rs), *gd = to_host(G);
+    float *dx = (float *)calloc((n * c) > 0 ? n * c : 1, sizeof(float));
+    float *dgamma = (float *)calloc(Gm->size ? Gm->size : 1, sizeof(float));
+    float *dbeta = (float *)calloc(Gm->size ? Gm->size : 1, sizeof(float));
+    for (size_t row = 0; row < n; ++row) {
+        size_t off = row * c;
+        float m = mn[row], r = rs[row];
+        float sum_dg = 0.0f, sum_dgx = 0.0f;
+        for (size_t j = 0; j < c; ++j) {
+            float xhat = (xd[off + j] - m) * r;
+            float dg = gd[off + j] * gm[j];
+            sum_dg += dg;
+            sum_dgx += dg * xhat;
+            dgamma[j] += gd[off + j] * xhat;
+            dbeta[j] += gd[off + j];
+        }
+        for (size_t j = 0; j < c; ++j) {
+            float xhat = (xd[off + j] - m) * r;
+            float dg = gd[off + j] * gm[j];
+            dx[off + j] = r * (dg - sum_dg / (float)c - xhat * sum_dgx / (float)c);
+        }
+    }
+    free(xd); free(gm); free(mn); free(rs); free(gd);
+    out[0] = (long)from_vec(dx, shape, nd);
+    out[1] = (long)from_vec(dgamma, gshape, gnd);
+    out[2] = (long)from_vec(dbeta, gshape, gnd);
+    return 0;
+}
+
 /* ---- fused bias + GELU ---------------------------------------------------- */
 
 /* ops/fused.rs:247-273 bias_gelu, cpu arm: val = x[i] + bias[i % c] with c the
@@ -1090,6 +1320,10 @@ static int dispatch_backward(const orc_entry *e, size_t grad, long *out) {
     case OP_PERMUTE: return permute_backward(grad, e, out);
     case OP_CONTIGUOUS: out[0] = (long)grad; return 0; /* layout.rs:229-231 */
     case OP_CROSSENTROPY: return cross_entropy_backward(grad, e, out);
+    case OP_EXP: case OP_LOG: case OP_SIGMOID: case OP_POW: return unary2_backward(grad, e, out);
+    case OP_DIV: return div_backward(grad, e, out);
+    case OP_MAX: return max_backward(grad, e, out);
+    case OP_LAYERNORM: return layernorm_backward(grad, e, out);
     case OP_BIASGELU: return bias_gelu_backward(grad, e, out);        /* autograd.rs BiasGelu */
     case OP_SOFTMAX: return softmax_backward(grad, e, out);           /* autograd.rs:204 */
     case OP_FLASHATTENTION: return flash_attention_backward(grad, e, out); /* autograd.rs:210 */
@@ -1375,6 +1609,19 @@ uint32_t orc_contiguous(uint32_t a) { /* lib.rs:295-300 -> layout.rs:218-227 */
     size_t out = ensure_contiguous(a);
     if (out != a) tape_record(&g_tape, OP_CONTIGUOUS, out, 1, a, 0);
     return (uint32_t)out;
+}
+uint32_t orc_exp_op(uint32_t a) { return unary2_op(a, 0, 0.0f); }   /* lib.rs:220-225 */
+uint32_t orc_log_op(uint32_t a) { return unary2_op(a, 1, 0.0f); }   /* lib.rs:227-232 */
+uint32_t orc_sigmoid(uint32_t a) { return unary2_op(a, 2, 0.0f); }  /* lib.rs:374-379 */
+uint32_t orc_pow_op(uint32_t a, double e) { return unary2_op(a, 3, (float)e); } /* lib.rs:381-386 */
+uint32_t orc_div(uint32_t a, uint32_t b) { return div_op(a, b); }   /* lib.rs:339-344 */
+uint32_t orc_lt(uint32_t a, uint32_t b) { return compare_op(a, b, 4, 0.0f); }    /* lib.rs:346-351 */
+uint32_t orc_eq_op(uint32_t a, uint32_t b) { return compare_op(a, b, 5, 0.0f); } /* lib.rs:353-358 */
+uint32_t orc_gt(uint32_t a, uint32_t b) { return compare_op(a, b, 6, 0.0f); }    /* lib.rs:360-365 */
+uint32_t orc_is_close(uint32_t a, uint32_t b, double tol) { return compare_op(a, b, 7, (float)tol); } /* lib.rs:367-372 */
+uint32_t orc_max_op(uint32_t a, int64_t dim) { return max_impl(a, (int)dim); }   /* lib.rs:248-253 */
+uint32_t orc_layernorm_op(uint32_t x, uint32_t gamma, uint32_t beta, double eps) { /* lib.rs:309-315 */
+    return layernorm_impl(x, gamma, beta, (float)eps);
 }
 uint32_t orc_bias_gelu(uint32_t x, uint32_t bias) { return bias_gelu_impl(x, bias); } /* lib.rs:526-531 */
 uint32_t orc_softmax_op(uint32_t a, int64_t dim) { return softmax_impl(a, (int)dim); } /* lib.rs:302-307 */

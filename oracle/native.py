@@ -61,6 +61,11 @@ class OracleNative:
             "orc_cross_entropy_loss": (u32, [u32, _i64p, C.c_size_t]),
             "orc_softmax_op": (u32, [u32, C.c_int64]),
             "orc_bias_gelu": (u32, [u32, u32]),
+            "orc_exp_op": (u32, [u32]), "orc_log_op": (u32, [u32]), "orc_sigmoid": (u32, [u32]),
+            "orc_pow_op": (u32, [u32, C.c_double]), "orc_div": (u32, [u32, u32]),
+            "orc_lt": (u32, [u32, u32]), "orc_eq_op": (u32, [u32, u32]), "orc_gt": (u32, [u32, u32]),
+            "orc_is_close": (u32, [u32, u32, C.c_double]), "orc_max_op": (u32, [u32, C.c_int64]),
+            "orc_layernorm_op": (u32, [u32, u32, u32, C.c_double]),
             "orc_flash_attention": (u32, [u32, u32, u32, C.c_double, C.c_int]),
             "orc_adamw_step": (None, [_u32p, C.c_size_t] + [C.c_double] * 5 + [C.c_int64]),
             "orc_grad_norm": (C.c_double, [_u32p, C.c_size_t]),
@@ -196,6 +201,39 @@ class OracleNative:
 
     def biasGelu(self, x, bias):
         return self._id(self.lib.orc_bias_gelu(x, bias))
+
+    def expOp(self, a):
+        return self._id(self.lib.orc_exp_op(a))
+
+    def logOp(self, a):
+        return self._id(self.lib.orc_log_op(a))
+
+    def sigmoid(self, a):
+        return self._id(self.lib.orc_sigmoid(a))
+
+    def powOp(self, a, exponent):
+        return self._id(self.lib.orc_pow_op(a, exponent))
+
+    def div(self, a, b):
+        return self._id(self.lib.orc_div(a, b))
+
+    def lt(self, a, b):
+        return self._id(self.lib.orc_lt(a, b))
+
+    def eqOp(self, a, b):
+        return self._id(self.lib.orc_eq_op(a, b))
+
+    def gt(self, a, b):
+        return self._id(self.lib.orc_gt(a, b))
+
+    def isClose(self, a, b, tol):
+        return self._id(self.lib.orc_is_close(a, b, tol))
+
+    def maxOp(self, a, dim):
+        return self._id(self.lib.orc_max_op(a, dim))
+
+    def layernormOp(self, x, gamma, beta, eps):
+        return self._id(self.lib.orc_layernorm_op(x, gamma, beta, eps))
 
     def flashAttention(self, q, k, v, scale, causal):
         return self._id(self.lib.orc_flash_attention(q, k, v, scale, 1 if causal else 0))
