@@ -220,6 +220,27 @@ def bench_extras(r):
                                          "fwd_TFLOP/s_dense_count": 2 * dense / ms_fwd / 1e9,
                                          "fwd_bwd_TFLOP/s_dense_count": 7 * dense / ms_all / 1e9,
                                          "note": "wall clock per call incl. host issue and a trailing sync; 2 products forward, 5 backward"}
+    # KV-cache decode: 8 x 32 heads of 128, 4096 cached positions, one new token per call
+    api.native.resetEngine()
+    bsz, nh, hd, hist = 8, 32, 128, 4096
+    for quantized in (False, True):
+        cache = api.KvCache(bsz, nh, hd, hist + 64, quantized)
+        kk = T(synth.normal(6, (bsz, nh, 1, hd)))
+        for _ in range(hist):
+            cache.append(kk, kk)
+        qq = T(synth.normal(6, (bsz, nh, 1, hd), stream=1))
+        for _ in range(3):
+            cache.decodeStep(qq, kk, kk, 0.088)
+        r.sync()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            cache.decodeStep(qq, kk, kk, 0.088)
+        r.sync()
+        us = (time.perf_counter() - t0) / 20 * 1e6
+        by = 2.0 * bsz * nh * (hist + 12) * hd * (1 if quantized else 4)
+        out["kv_decode_8x32x128_hist4096_" + ("int8" if quantized else "fp32")] = {"us": us, "GB/s": by / us / 1e3}
+        cache.free()
+        api.native.gcTensors([])
     api.native.resetEngine()
     return out
 

@@ -225,6 +225,31 @@ def bind(native):
     def flashAttention(q, k, v, scale, causal=True):  # src/nn.ts:107-110
         return Tensor(native.flashAttention(q._id, k._id, v._id, scale, causal))
 
+    class KvCache:  # src/nn.ts:111-151
+        def __init__(self, batchSize, numHeads, headDim, maxSeqLen, quantized=True):
+            if not hasattr(native, "kvCacheCreate"):
+                raise RuntimeError("kv cache is not available in this native build")
+            requested = quantized and hasattr(native, "flashAttention")
+            self.cacheId = native.kvCacheCreate(batchSize, numHeads, headDim, maxSeqLen, requested)
+
+        def decodeStep(self, q, k, v, scale):
+            return Tensor(native.kvCacheDecodeStep(self.cacheId, q._id, k._id, v._id, scale))
+
+        def append(self, k, v):
+            native.kvCacheAppend(self.cacheId, k._id, v._id)
+
+        def length(self):
+            return int(native.kvCacheLen(self.cacheId))
+
+        def isQuantized(self):
+            return bool(native.kvCacheQuantized(self.cacheId))
+
+        def reset(self):
+            native.kvCacheReset(self.cacheId)
+
+        def free(self):
+            native.kvCacheFree(self.cacheId)
+
     class Adam:  # src/optimizer.ts:33-70: options object, defaults lr 6e-4, beta2 0.95
         def __init__(self, parameters, lr=6e-4, beta1=0.9, beta2=0.95, eps=1e-8, weightDecay=0.0):
             self.parameters = list(parameters)
@@ -241,4 +266,4 @@ def bind(native):
 
     return SimpleNamespace(native=native, Tensor=Tensor, Parameter=Parameter, Module=Module, Linear=Linear, ReLU=ReLU,
                            GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, softmax=softmax, biasGelu=biasGelu, layerNorm=layerNorm,
-                           flashAttention=flashAttention, Adam=Adam)
+                           flashAttention=flashAttention, KvCache=KvCache, Adam=Adam)

@@ -206,4 +206,333 @@ int k_attn_backward(float *scores, float *dp, const float *lse, const float *di,
     return check_launch("attn_backward");
 }
 
+
+// ---- device-resident KV cache -----------------------------------------------------------
+// Counterpart of ops/kv_cache.rs, whose cache lives in host memory and whose
+// decode loops over the history on the CPU (its cuda arm only quantises on the
+// device).  Storage here is [bh, max_seq, d] in HBM, fp32 or int8 with one f32
+// scale per row.
+
+// append, fp32: row r of k / v goes to position pos of its head (:159-167)
+__global__ void kv_append_f32_kernel(float *__restrict__ kc, float *__restrict__ vc, const float *__restrict__ k,
+                                     const float *__restrict__ v, int64_t n, int64_t d, int64_t max_seq, int64_t pos) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    const int64_t row = idx / d, dd = idx - row * d;
+    const int64_t dst = (row * max_seq + pos) * d + dd;
+    kc[dst] = k[idx];
+    vc[dst] = v[idx];
+}
+// append, int8: quantize_row_i8 (:357-370) -- scale = max(max|x| / 127, 1e-8),
+// q = clamp(round(x * (1 / scale)), -127, 127), round half away from zero.
+// One wavefront per (row, k or v).
+__global__ void kv_append_i8_kernel(signed char *__restrict__ kc, signed char *__restrict__ vc, float *__restrict__ ks,
+                                    float *__restrict__ vs, const float *__restrict__ k, const float *__restrict__ v,
+                                    int64_t bh, int64_t d, int64_t max_seq, int64_t pos) {
+    const int lane = threadIdx.x & 63;
+    const int64_t job = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (job >= 2 * bh) return;
+    const int64_t row = job >> 1;
+    const bool is_v = job & 1;
+    const float *src = (is_v ? v : k) + row * d;
+    signed char *dst = (is_v ? vc : kc) + (row * max_seq + pos) * d;
+    float mx = 0.f;
+    for (int64_t j = lane; j < d; j += 64) mx = fmaxf(mx, fabsf(src[j]));
+    mx = wave_max(mx);
+    float scale = mx / 127.0f;
+    if (!(scale > 1e-8f)) scale = 1e-8f;
+    const float inv = 1.0f / scale;
+    for (int64_t j = lane; j < d; j += 64) {
+        float q = roundf(src[j] * inv);
+        q = q < -127.0f ? -127.0f : q > 127.0f ? 127.0f : q;
+        dst[j] = (signed char)q;
+    }
+    if (lane == 0) (is_v ? vs : ks)[row * max_seq + pos] = scale;
+}
+int k_kv_append(void *kc, void *vc, float *ks, float *vs, const float *k, const float *v, int64_t bh, int64_t d,
+                int64_t max_seq, int64_t pos, int quantized) {
+    if (bh * d <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (quantized)
+        hipLaunchKernelGGL(kv_append_i8_kernel, dim3(rows_grid(2 * bh)), dim3(ATT_TPB), 0, ctx().stream, (signed char *)kc,
+                           (signed char *)vc, ks, vs, k, v, bh, d, max_seq, pos);
+    else
+        hipLaunchKernelGGL(kv_append_f32_kernel, dim3((unsigned)((bh * d + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB), 0,
+                           ctx().stream, (float *)kc, (float *)vc, k, v, bh * d, d, max_seq, pos);
+    return check_launch("kv_append");
+}
+
+// decode (:259-287): attention of one query row per head over positions
+// [0, len).  grid = (bh, splits): a workgroup takes a chunk of the history --
+// one thread per key for the scores (the query sits in LDS), block-wide max and
+// sum, then threads own output columns for the weighted sum of the values.  With
+// more than one split the chunks leave (acc, max, sum) behind and
+// kv_combine_kernel merges them (the usual log-sum-exp merge); the merge order is
+// fixed, so results do not depend on scheduling.
+struct KvDecode {
+    const void *kc, *vc;
+    const float *ks, *vs, *q;
+    float *out, *part;  // part: [bh][splits][d + 2]
+    int64_t d, max_seq;
+    int len, splits, chunk;
+    float scale;
+};
+static constexpr int KV_CHUNK_MAX = 2048;
+
+__device__ __forceinline__ float block_reduce(float v, float *red, bool is_max) {
+    v = is_max ? wave_max(v) : wave_sum(v);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int i = 1; i < ATT_TPB / 64; ++i) r = is_max ? fmaxf(r, red[i]) : r + red[i];
+    return r;
+}
+
+template <bool Q8>
+__global__ __launch_bounds__(ATT_TPB) void kv_decode_kernel(const KvDecode a) {
+    extern __shared__ float sm[];
+    float *qs = sm;                 // [d]
+    float *sc = sm + a.d;           // [chunk]
+    float *red = sc + a.chunk;      // [ATT_TPB]
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const int sp = blockIdx.y;
+    const int t0 = sp * a.chunk;
+    const int n = min(a.len, t0 + a.chunk) - t0;
+    const int64_t d = a.d;
+    for (int64_t dd = tid; dd < d; dd += ATT_TPB) qs[dd] = a.q[row * d + dd];
+    __syncthreads();
+    // scores
+    for (int i = tid; i < n; i += ATT_TPB) {
+        const int64_t pos = row * a.max_seq + t0 + i;
+        float dot = 0.f;
+        if (Q8) {
+            const signed char *kp = (const signed char *)a.kc + pos * d;
+            const float s = a.ks[pos];
+            for (int64_t dd = 0; dd < d; ++dd) dot += qs[dd] * ((float)kp[dd] * s);
+        } else {
+            const float *kp = (const float *)a.kc + pos * d;
+            for (int64_t dd = 0; dd < d; ++dd) dot += qs[dd] * kp[dd];
+        }
+        sc[i] = dot * a.scale;
+    }
+    __syncthreads();
+    float m = -INFINITY;
+    for (int i = tid; i < n; i += ATT_TPB) m = fmaxf(m, sc[i]);
+    m = block_reduce(m, red, true);
+    float l = 0.f;
+    for (int i = tid; i < n; i += ATT_TPB) {
+        const float w = expf(sc[i] - m);
+        sc[i] = w;
+        l += w;
+    }
+    l = block_reduce(l, red, false);
+    __syncthreads();
+    // weighted sum of the values: threads own columns, groups split the keys
+    const int lanes = d <= ATT_TPB ? (int)d : ATT_TPB;
+    const int groups = d <= ATT_TPB ? ATT_TPB / (int)d : 1;
+    float *pout = a.part + ((int64_t)row * a.splits + sp) * (d + 2);
+    for (int64_t base = 0; base < d; base += lanes) {
+        const int col = tid % lanes, grp = tid / lanes;
+        const int64_t dd = base + col;
+        float acc = 0.f;
+        if (grp < groups && dd < d) {
+            for (int i = grp; i < n; i += groups) {
+                const int64_t pos = row * a.max_seq + t0 + i;
+                const float vv = Q8 ? (float)((const signed char *)a.vc)[pos * d + dd] * a.vs[pos]
+                                    : ((const float *)a.vc)[pos * d + dd];
+                acc += sc[i] * vv;
+            }
+        }
+        __syncthreads();
+        red[tid] = acc;
+        __syncthreads();
+        if (tid < lanes && base + tid < d) {
+            float s = 0.f;
+            for (int g = 0; g < groups; ++g) s += red[g * lanes + tid];
+            if (a.splits == 1) a.out[row * d + base + tid] = l > 0.f ? s * (1.0f / l) : 0.f;
+            else pout[base + tid] = s;
+        }
+    }
+    if (a.splits > 1 && tid == 0) { pout[d] = m; pout[d + 1] = l; }
+}
+// The same decode for head dims up to 256 (fp32, multiples of 4) or up to 1024
+// (int8, multiples of 16): every row of the cache is read as 16-byte pieces by
+// LPR neighbouring lanes -- 4 fp32 or 16 int8 values per lane -- so loads are
+// coalesced; a dot product is finished with log2(LPR) butterfly steps, and the
+// value pass keeps those 4 / 16 columns per lane.
+template <bool Q8, int LPR>
+__global__ __launch_bounds__(ATT_TPB) void kv_decode_vec_kernel(const KvDecode a) {
+    constexpr int E = Q8 ? 16 : 4;         // elements per lane
+    constexpr int RPP = 64 / LPR;          // rows per wavefront pass
+    constexpr int GROUPS = ATT_TPB / LPR;  // key groups in the value pass
+    extern __shared__ float sm[];
+    float *sc = sm;                         // [chunk]
+    float *red = sm + a.chunk;              // [ATT_TPB]
+    float *redv = red + ATT_TPB;            // [ATT_TPB][E]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l = lane % LPR, sub = lane / LPR;
+    const int64_t row = blockIdx.x;
+    const int sp = blockIdx.y;
+    const int t0 = sp * a.chunk;
+    const int n = min(a.len, t0 + a.chunk) - t0;
+    const int pieces = (int)(a.d / E);
+    const int64_t base = row * a.max_seq + t0;
+    auto load = [&](const void *cache, const float *scales, int64_t pos, int piece, float (&v)[E]) {
+        if (Q8) {
+            const int4 w = reinterpret_cast<const int4 *>(reinterpret_cast<const signed char *>(cache) + pos * a.d)[piece];
+            const float s = scales[pos];
+            const int ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int b8 = 0; b8 < 4; ++b8) v[4 * j + b8] = (float)(signed char)((ws[j] >> (8 * b8)) & 0xff) * s;
+        } else {
+            const float4 f = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(cache) + pos * a.d)[piece];
+            v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+        }
+    };
+    float qv[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) qv[e] = l < pieces ? a.q[row * a.d + l * E + e] : 0.f;
+    // scores
+    for (int i0 = wave * RPP; i0 < n; i0 += (ATT_TPB / 64) * RPP) {
+        const int i = i0 + sub;
+        float part = 0.f;
+        if (i < n && l < pieces) {
+            float kv[E];
+            load(a.kc, a.ks, base + i, l, kv);
+#pragma unroll
+            for (int e = 0; e < E; ++e) part += qv[e] * kv[e];
+        }
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        if (i < n && l == 0) sc[i] = part * a.scale;
+    }
+    __syncthreads();
+    float m = -INFINITY;
+    for (int i = tid; i < n; i += ATT_TPB) m = fmaxf(m, sc[i]);
+    m = block_reduce(m, red, true);
+    float lsum = 0.f;
+    for (int i = tid; i < n; i += ATT_TPB) {
+        const float w = expf(sc[i] - m);
+        sc[i] = w;
+        lsum += w;
+    }
+    lsum = block_reduce(lsum, red, false);
+    __syncthreads();
+    // values: lane lv of key group grp accumulates columns E * lv .. E * lv + E - 1
+    const int lv = tid % LPR, grp = tid / LPR;
+    float acc[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[e] = 0.f;
+    if (lv < pieces) {
+        for (int i = grp; i < n; i += GROUPS) {
+            float vv[E];
+            load(a.vc, a.vs, base + i, lv, vv);
+            const float w = sc[i];
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc[e] += w * vv[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) redv[e * ATT_TPB + tid] = acc[e];
+    __syncthreads();
+    float *pout = a.part + ((int64_t)row * a.splits + sp) * (a.d + 2);
+    const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+    // one thread per output column: column c = E * piece + e lives at redv[e][g * LPR + piece]
+    for (int c = tid; c < (int)a.d; c += ATT_TPB) {
+        const int piece = c / E, e = c % E;
+        float s1 = 0.f;
+        for (int g = 0; g < GROUPS; ++g) s1 += redv[e * ATT_TPB + g * LPR + piece];
+        if (a.splits == 1) a.out[row * a.d + c] = s1 * inv;
+        else pout[c] = s1;
+    }
+    if (a.splits > 1 && tid == 0) { pout[a.d] = m; pout[a.d + 1] = lsum; }
+}
+template <bool Q8>
+static bool launch_kv_decode_vec(const KvDecode &a, dim3 grid, size_t lds) {
+    const int pieces = (int)(a.d / (Q8 ? 16 : 4));
+    hipStream_t st = ctx().stream;
+#define MNI_KVV(L) hipLaunchKernelGGL((kv_decode_vec_kernel<Q8, L>), grid, dim3(ATT_TPB), lds, st, a)
+    if (pieces <= 1) MNI_KVV(1);
+    else if (pieces <= 2) MNI_KVV(2);
+    else if (pieces <= 4) MNI_KVV(4);
+    else if (pieces <= 8) MNI_KVV(8);
+    else if (pieces <= 16) MNI_KVV(16);
+    else if (pieces <= 32) MNI_KVV(32);
+    else if (pieces <= 64) MNI_KVV(64);
+    else return false;
+#undef MNI_KVV
+    return true;
+}
+
+__global__ void kv_combine_kernel(float *__restrict__ out, const float *__restrict__ part, int64_t d, int splits) {
+    const int64_t row = blockIdx.x;
+    const float *p = part + row * splits * (d + 2);
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, p[s * (d + 2) + d]);
+    float l = 0.f;
+    for (int s = 0; s < splits; ++s) l += p[s * (d + 2) + d + 1] * expf(p[s * (d + 2) + d] - m);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    for (int64_t dd = threadIdx.x; dd < d; dd += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < splits; ++s) acc += p[s * (d + 2) + dd] * expf(p[s * (d + 2) + d] - m);
+        out[row * d + dd] = acc * inv;
+    }
+}
+int k_kv_decode(float *out, const void *kc, const void *vc, const float *ks, const float *vs, const float *q, int64_t bh,
+                int64_t d, int64_t max_seq, int64_t len, float scale, int quantized) {
+    if (bh <= 0 || d <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    if (len <= 0) return k_fill(out, 0.0f, bh * d);
+    if (d > 4096) return set_error(MNI_ERR_INVALID, "kv cache decode: head_dim %lld above 4096", (long long)d);
+    if (bh > 0x7fffffff || len > 0x7ffffff0) return set_error(MNI_ERR_INVALID, "kv cache decode: extent out of range");
+    // enough workgroups to occupy the device, chunks of at most KV_CHUNK_MAX keys
+    const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
+    int64_t splits = (2LL * cus + bh - 1) / bh;
+    const int64_t max_by_len = (len + 127) / 128;
+    if (splits > max_by_len) splits = max_by_len;
+    const int64_t min_by_chunk = (len + KV_CHUNK_MAX - 1) / KV_CHUNK_MAX;
+    if (splits < min_by_chunk) splits = min_by_chunk;
+    if (splits < 1) splits = 1;
+    int64_t chunk = (len + splits - 1) / splits;
+    chunk = (chunk + 63) / 64 * 64;
+    splits = (len + chunk - 1) / chunk;
+    if (splits > 65535) return set_error(MNI_ERR_INVALID, "kv cache decode: history of %lld positions is too long", (long long)len);
+    KvDecode a;
+    a.kc = kc; a.vc = vc; a.ks = ks; a.vs = vs; a.q = q; a.out = out; a.part = nullptr;
+    a.d = d; a.max_seq = max_seq; a.len = (int)len; a.splits = (int)splits; a.chunk = (int)chunk; a.scale = scale;
+    void *part = nullptr;
+    if (splits > 1) {
+        MNI_TRY(dev_alloc(&part, (size_t)(bh * splits * (d + 2)) * sizeof(float)));
+        a.part = (float *)part;
+    } else {
+        a.part = out;  // not written when splits == 1; keeps the pointer arithmetic in bounds
+    }
+    const dim3 grid((unsigned)bh, (unsigned)splits);
+    // 16-byte pieces of a row: 4 fp32 or 16 int8 values (rows are then 16-byte aligned in the cache)
+    const int per_lane = quantized ? 16 : 4;
+    bool launched = false;
+    if (d % per_lane == 0 && d / per_lane <= 64) {
+        const size_t ldsv = (size_t)(chunk + ATT_TPB + per_lane * ATT_TPB) * sizeof(float);
+        launched = quantized ? launch_kv_decode_vec<true>(a, grid, ldsv) : launch_kv_decode_vec<false>(a, grid, ldsv);
+    }
+    if (!launched) {
+        const size_t lds = (size_t)(d + chunk + ATT_TPB) * sizeof(float);
+        if (quantized) hipLaunchKernelGGL((kv_decode_kernel<true>), grid, dim3(ATT_TPB), lds, ctx().stream, a);
+        else hipLaunchKernelGGL((kv_decode_kernel<false>), grid, dim3(ATT_TPB), lds, ctx().stream, a);
+    }
+    int rc = check_launch("kv_decode");
+    if (rc == MNI_OK && splits > 1) {
+        hipLaunchKernelGGL(kv_combine_kernel, dim3((unsigned)bh), dim3(ATT_TPB), 0, ctx().stream, out, (const float *)part, d,
+                           (int)splits);
+        rc = check_launch("kv_combine");
+    }
+    if (part) dev_free(part);
+    return rc;
+}
+
 }  // namespace mni

@@ -122,6 +122,10 @@ int k_attn_softmax(float *scores, float *lse, int64_t rows, int64_t s, float sca
 int k_rowdot(float *out, const float *a, const float *b, int64_t rows, int64_t d);
 int k_attn_backward(float *scores, float *dp, const float *lse, const float *di, int64_t rows, int64_t s, float scale,
                     int causal);
+int k_kv_append(void *kc, void *vc, float *ks, float *vs, const float *k, const float *v, int64_t bh, int64_t d,
+                int64_t max_seq, int64_t pos, int quantized);
+int k_kv_decode(float *out, const void *kc, const void *vc, const float *ks, const float *vs, const float *q, int64_t bh,
+                int64_t d, int64_t max_seq, int64_t len, float scale, int quantized);
 
 int k_sumsq_f64(double *out, const float *g, int64_t n);  // out += sum g^2 (device double)
 int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, float b1, float b2,

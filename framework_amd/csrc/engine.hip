@@ -10,7 +10,9 @@
 #include <math.h>
 #include <string.h>
 
+#include <map>
 #include <memory>
+#include <string>
 #include <vector>
 
 #include "common.h"
@@ -76,10 +78,20 @@ struct Tape {
     void record(Entry &&e) { if (enabled) entries.push_back(std::move(e)); }
 };
 
+// ops/kv_cache.rs:20-47 KvCacheConfig + KvCache, storage on the device
+struct KvCache {
+    int64_t batch = 0, heads = 0, d = 0, max_seq = 0, len = 0;
+    bool quantized = false;
+    std::shared_ptr<void> keys, vals;      // [bh, max_seq, d] float or int8
+    std::shared_ptr<void> kscale, vscale;  // [bh, max_seq] float (quantized only)
+};
+
 struct Engine {
     std::vector<Tensor> tensors;
     std::vector<uint32_t> free_ids;
     Tape tape;
+    std::map<uint32_t, KvCache> kv_caches;  // lib.rs:23-24
+    uint32_t next_kv_cache_id = 1;          // lib.rs:36
 };
 static Engine &eng() {
     static Engine e;
@@ -1062,6 +1074,100 @@ static int flash_attention_backward(uint32_t grad, const Entry &e, int64_t *out)
     return MNI_OK;
 }
 
+// ---- KV cache ------------------------------------------------------------------------------------
+static std::shared_ptr<void> dev_block(size_t bytes) {
+    void *p = nullptr;
+    if (dev_alloc(&p, bytes ? bytes : 4) != MNI_OK) return nullptr;
+    return std::shared_ptr<void>(p, [](void *q) { dev_free(q); });
+}
+static std::string shape_text(const Shape &s) {  // Rust's {:?} of a slice
+    std::string t = "[";
+    for (size_t i = 0; i < s.size(); ++i) t += (i ? ", " : "") + std::to_string(s[i]);
+    return t + "]";
+}
+// ops/kv_cache.rs:83-111, 336-349: [B,H,S,D] or [BH,S,D] with S = 1 and the cache's extents
+static bool kv_validate(const KvCache &c, const Shape &shape, const char *op, std::string *why) {
+    int64_t b, h, sl, d;
+    if (shape.size() == 4) { b = shape[0]; h = shape[1]; sl = shape[2]; d = shape[3]; }
+    else if (shape.size() == 3) { b = 1; h = shape[0]; sl = shape[1]; d = shape[2]; }
+    else { *why = "expected [B,H,S,D] or [BH,S,D], got shape " + shape_text(shape); return false; }
+    if (sl != 1) { *why = std::string("kv cache ") + op + " expects seq_len=1, got " + std::to_string(sl); return false; }
+    if (b != c.batch || h != c.heads || d != c.d) {
+        *why = std::string("kv cache ") + op + " shape mismatch: expected [B=" + std::to_string(c.batch) + ", H=" +
+               std::to_string(c.heads) + ", S=1, D=" + std::to_string(c.d) + "], got [B=" + std::to_string(b) + ", H=" +
+               std::to_string(h) + ", S=1, D=" + std::to_string(d) + "]";
+        return false;
+    }
+    return true;
+}
+// ops/kv_cache.rs:113-171 append_inner
+static bool kv_append_inner(KvCache &c, const Tensor &K, const Tensor &V, std::string *why) {
+    if (c.len >= c.max_seq) {
+        *why = "kv cache is full (len=" + std::to_string(c.len) + ", max_seq_len=" + std::to_string(c.max_seq) + ")";
+        return false;
+    }
+    const int64_t bh = c.batch * c.heads;
+    BufP kb = contiguous_buf(K), vb = contiguous_buf(V);
+    if (!kb || !vb) { *why = mni_rocm_last_error(); return false; }
+    if (k_kv_append(c.keys.get(), c.vals.get(), (float *)c.kscale.get(), (float *)c.vscale.get(), kb->p, vb->p, bh, c.d,
+                    c.max_seq, c.len, c.quantized ? 1 : 0) != MNI_OK) {
+        *why = mni_rocm_last_error();
+        return false;
+    }
+    c.len += 1;
+    return true;
+}
+static uint32_t kv_cache_create(int64_t batch, int64_t heads, int64_t d, int64_t max_seq, bool quantized) {
+    if (batch < 0 || heads < 0 || d < 0 || max_seq < 0) { set_error(MNI_ERR_INVALID, "kv cache: negative extent"); return MNI_BAD_ID; }
+    KvCache c;
+    c.batch = batch; c.heads = heads; c.d = d; c.max_seq = max_seq; c.quantized = quantized;
+    const size_t cap = (size_t)(batch * heads * max_seq * d), rows = (size_t)(batch * heads * max_seq);
+    c.keys = dev_block(cap * (quantized ? 1 : sizeof(float)));
+    c.vals = dev_block(cap * (quantized ? 1 : sizeof(float)));
+    if (quantized) { c.kscale = dev_block(rows * sizeof(float)); c.vscale = dev_block(rows * sizeof(float)); }
+    if (!c.keys || !c.vals || (quantized && (!c.kscale || !c.vscale))) return MNI_BAD_ID;
+    Engine &e = eng();
+    const uint32_t id = e.next_kv_cache_id++;
+    e.kv_caches[id] = std::move(c);
+    return id;
+}
+static int kv_cache_append(uint32_t id, uint32_t k, uint32_t v) {  // lib.rs:661-676, kv_cache.rs:173-181
+    auto it = eng().kv_caches.find(id);
+    if (it == eng().kv_caches.end()) return set_error(MNI_ERR_INVALID, "invalid kv cache id: %u", id);
+    Tensor *K = get(k), *V = get(v);
+    if (!K || !V) return MNI_ERR_FREED;
+    std::string why;
+    bool ok = true;
+    if (K->shape != V->shape) { why = "k/v shapes must match for kv cache append"; ok = false; }
+    ok = ok && kv_validate(it->second, K->shape, "append", &why) && kv_append_inner(it->second, *K, *V, &why);
+    return ok ? MNI_OK : set_error(MNI_ERR_INVALID, "kv cache append failed: %s", why.c_str());
+}
+static uint32_t kv_cache_decode_step(uint32_t id, uint32_t q, uint32_t k, uint32_t v, float scale) {  // lib.rs:641-659
+    auto it = eng().kv_caches.find(id);
+    if (it == eng().kv_caches.end()) { set_error(MNI_ERR_INVALID, "invalid kv cache id: %u", id); return MNI_BAD_ID; }
+    KvCache &c = it->second;
+    Tensor *Q = get(q), *K = get(k), *V = get(v);
+    if (!Q || !K || !V) return MNI_BAD_ID;
+    std::string why;
+    bool ok = true;
+    if (Q->shape != K->shape || Q->shape != V->shape) { why = "q/k/v shapes must match for kv cache decode"; ok = false; }
+    ok = ok && kv_validate(c, Q->shape, "decode", &why) && kv_append_inner(c, *K, *V, &why);
+    BufP qb, out;
+    const int64_t bh = c.batch * c.heads;
+    if (ok) {
+        qb = contiguous_buf(*Q);
+        out = qb ? new_buf((size_t)(bh * c.d)) : nullptr;
+        if (!out || k_kv_decode(out->p, c.keys.get(), c.vals.get(), (const float *)c.kscale.get(), (const float *)c.vscale.get(),
+                                qb->p, bh, c.d, c.max_seq, c.len, scale, c.quantized ? 1 : 0) != MNI_OK) {
+            why = mni_rocm_last_error();
+            ok = false;
+        }
+    }
+    if (!ok) { set_error(MNI_ERR_INVALID, "kv cache decode failed: %s", why.c_str()); return MNI_BAD_ID; }
+    const Shape out_shape = Q->shape.size() == 4 ? Shape{c.batch, c.heads, 1, c.d} : Shape{bh, 1, c.d};
+    return insert_contig(std::move(out), out_shape);
+}
+
 // ---- fused Linear ------------------------------------------------------------------------------
 static uint32_t linear_op(uint32_t x, uint32_t w, uint32_t bias, int act) {
     Tensor *X = get(x), *W = get(w), *Bv = get(bias);
@@ -1508,6 +1614,32 @@ uint32_t mni_layernorm_op(uint32_t x, uint32_t gamma, uint32_t beta, double eps)
     MNI_API_GUARD;
     return layernorm_op(x, gamma, beta, (float)eps);
 }
+uint32_t mni_kv_cache_create(int64_t batch_size, int64_t num_heads, int64_t head_dim, int64_t max_seq_len, int quantized) {
+    MNI_API_GUARD;
+    if (ensure_init() != MNI_OK) return MNI_BAD_ID;
+    return kv_cache_create(batch_size, num_heads, head_dim, max_seq_len, quantized != 0);
+}
+int64_t mni_kv_cache_len(uint32_t cache_id) {
+    MNI_API_GUARD;
+    auto it = eng().kv_caches.find(cache_id);
+    return it == eng().kv_caches.end() ? 0 : it->second.len;
+}
+int mni_kv_cache_quantized(uint32_t cache_id) {
+    MNI_API_GUARD;
+    auto it = eng().kv_caches.find(cache_id);
+    return it != eng().kv_caches.end() && it->second.quantized ? 1 : 0;
+}
+void mni_kv_cache_reset(uint32_t cache_id) {
+    MNI_API_GUARD;
+    auto it = eng().kv_caches.find(cache_id);
+    if (it != eng().kv_caches.end()) it->second.len = 0;  // positions past len are never read
+}
+void mni_kv_cache_free(uint32_t cache_id) { MNI_API_GUARD; eng().kv_caches.erase(cache_id); }
+int mni_kv_cache_append(uint32_t cache_id, uint32_t k, uint32_t v) { MNI_API_GUARD; return kv_cache_append(cache_id, k, v); }
+uint32_t mni_kv_cache_decode_step(uint32_t cache_id, uint32_t q, uint32_t k, uint32_t v, double scale) {
+    MNI_API_GUARD;
+    return kv_cache_decode_step(cache_id, q, k, v, (float)scale);
+}
 uint32_t mni_bias_gelu(uint32_t x, uint32_t bias) { MNI_API_GUARD; return bias_gelu_op(x, bias); }
 uint32_t mni_softmax_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return softmax_op(a, dim); }
 uint32_t mni_flash_attention(uint32_t q, uint32_t k, uint32_t v, double scale, int causal) {
@@ -1554,6 +1686,8 @@ void mni_reset_engine(void) {
     e.tensors.clear();
     e.free_ids.clear();
     e.tape = Tape();
+    e.kv_caches.clear();       // lib.rs:466-467
+    e.next_kv_cache_id = 1;
 }
 int mni_gc_tensors(const uint32_t *keep, size_t n) {
     MNI_API_GUARD;

@@ -265,6 +265,40 @@ napi_value GcTensors(napi_env env, napi_callback_info info) {  // lib.rs:693-706
     return ret_rc(env, mni_gc_tensors(ids.data(), ids.size()));
 }
 // Opt-in fused Linear (no counterpart in lib.rs; feature-detected by callers).
+napi_value KvCacheCreate(napi_env env, napi_callback_info info) {  // lib.rs:586-607
+    Args a(env, info);
+    return ret_id(env, mni_kv_cache_create(get_i64(env, a.v[0]), get_i64(env, a.v[1]), get_i64(env, a.v[2]), get_i64(env, a.v[3]),
+                                           get_bool(env, a.v[4]) ? 1 : 0));
+}
+napi_value KvCacheLen(napi_env env, napi_callback_info info) {  // lib.rs:609-616
+    Args a(env, info);
+    return make_f64(env, (double)mni_kv_cache_len(get_u32(env, a.v[0])));
+}
+napi_value KvCacheQuantized(napi_env env, napi_callback_info info) {  // lib.rs:618-625
+    Args a(env, info);
+    napi_value v;
+    napi_get_boolean(env, mni_kv_cache_quantized(get_u32(env, a.v[0])) != 0, &v);
+    return v;
+}
+napi_value KvCacheReset(napi_env env, napi_callback_info info) {  // lib.rs:627-633
+    Args a(env, info);
+    mni_kv_cache_reset(get_u32(env, a.v[0]));
+    return undefined(env);
+}
+napi_value KvCacheFree(napi_env env, napi_callback_info info) {  // lib.rs:635-639
+    Args a(env, info);
+    mni_kv_cache_free(get_u32(env, a.v[0]));
+    return undefined(env);
+}
+napi_value KvCacheAppend(napi_env env, napi_callback_info info) {  // lib.rs:661-676
+    Args a(env, info);
+    return ret_rc(env, mni_kv_cache_append(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_u32(env, a.v[2])));
+}
+napi_value KvCacheDecodeStep(napi_env env, napi_callback_info info) {  // lib.rs:641-659
+    Args a(env, info);
+    return ret_id(env, mni_kv_cache_decode_step(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_u32(env, a.v[2]),
+                                                get_u32(env, a.v[3]), get_f64(env, a.v[4])));
+}
 napi_value PowOp(napi_env env, napi_callback_info info) {  // lib.rs:381-386
     Args a(env, info);
     return ret_id(env, mni_pow_op(get_u32(env, a.v[0]), get_f64(env, a.v[1])));
@@ -307,7 +341,10 @@ NAPI_MODULE_INIT() {
         EXPORT("softmaxOp", SoftmaxOp), EXPORT("biasGelu", BiasGelu),
         EXPORT("expOp", ExpOp), EXPORT("logOp", LogOp), EXPORT("sigmoid", Sigmoid), EXPORT("powOp", PowOp),
         EXPORT("div", Div), EXPORT("lt", Lt), EXPORT("eqOp", EqOp), EXPORT("gt", Gt), EXPORT("isClose", IsClose),
-        EXPORT("maxOp", MaxOp), EXPORT("layernormOp", LayernormOp), EXPORT("flashAttention", FlashAttention),
+        EXPORT("maxOp", MaxOp), EXPORT("layernormOp", LayernormOp),
+        EXPORT("kvCacheCreate", KvCacheCreate), EXPORT("kvCacheLen", KvCacheLen), EXPORT("kvCacheQuantized", KvCacheQuantized),
+        EXPORT("kvCacheReset", KvCacheReset), EXPORT("kvCacheFree", KvCacheFree), EXPORT("kvCacheAppend", KvCacheAppend),
+        EXPORT("kvCacheDecodeStep", KvCacheDecodeStep), EXPORT("flashAttention", FlashAttention),
 #undef EXPORT
     };
     napi_define_properties(env, exports, sizeof(props) / sizeof(props[0]), props);

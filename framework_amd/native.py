@@ -102,6 +102,10 @@ SIGNATURES = {
     "mni_contiguous": (C.c_uint32, [C.c_uint32]),
     "mni_softmax_op": (C.c_uint32, [C.c_uint32, C.c_int64]),
     "mni_bias_gelu": (C.c_uint32, [C.c_uint32, C.c_uint32]),
+    "mni_kv_cache_create": (C.c_uint32, [C.c_int64] * 4 + [C.c_int]), "mni_kv_cache_len": (C.c_int64, [C.c_uint32]),
+    "mni_kv_cache_quantized": (C.c_int, [C.c_uint32]), "mni_kv_cache_reset": (None, [C.c_uint32]),
+    "mni_kv_cache_free": (None, [C.c_uint32]), "mni_kv_cache_append": (C.c_int, [C.c_uint32] * 3),
+    "mni_kv_cache_decode_step": (C.c_uint32, [C.c_uint32] * 4 + [C.c_double]),
     "mni_exp_op": (C.c_uint32, [C.c_uint32]), "mni_log_op": (C.c_uint32, [C.c_uint32]),
     "mni_sigmoid": (C.c_uint32, [C.c_uint32]), "mni_pow_op": (C.c_uint32, [C.c_uint32, C.c_double]),
     "mni_div": (C.c_uint32, [C.c_uint32, C.c_uint32]), "mni_lt": (C.c_uint32, [C.c_uint32, C.c_uint32]),
@@ -398,6 +402,27 @@ class Native:
 
     def biasGelu(self, x, bias):
         return self._id(self.lib.mni_bias_gelu(x, bias))
+
+    def kvCacheCreate(self, batchSize, numHeads, headDim, maxSeqLen, quantized):
+        return self._id(self.lib.mni_kv_cache_create(batchSize, numHeads, headDim, maxSeqLen, 1 if quantized else 0))
+
+    def kvCacheLen(self, cacheId):
+        return self.lib.mni_kv_cache_len(cacheId)
+
+    def kvCacheQuantized(self, cacheId):
+        return bool(self.lib.mni_kv_cache_quantized(cacheId))
+
+    def kvCacheReset(self, cacheId):
+        self.lib.mni_kv_cache_reset(cacheId)
+
+    def kvCacheFree(self, cacheId):
+        self.lib.mni_kv_cache_free(cacheId)
+
+    def kvCacheAppend(self, cacheId, k, v):
+        self._rc(self.lib.mni_kv_cache_append(cacheId, k, v))
+
+    def kvCacheDecodeStep(self, cacheId, q, k, v, scale):
+        return self._id(self.lib.mni_kv_cache_decode_step(cacheId, q, k, v, scale))
 
     def expOp(self, a):
         return self._id(self.lib.mni_exp_op(a))

@@ -175,7 +175,22 @@ uint32_t mni_sum_all(uint32_t a);                                         /* lib
 uint32_t mni_mean_all(uint32_t a);                                        /* lib.rs:267-277 */
 uint32_t mni_view(uint32_t a, const int64_t *shape, int ndim);            /* lib.rs:279-285 */
 uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim);          /* lib.rs:287-293 */
-uint32_t mni_contiguous(uint32_t a);                                      /* Remaining elementwise / reduction exports of src/native/src/lib.rs, all on the device:
+uint32_t mni_contiguous(uint32_t a);                                      /* KV cache for incremental decoding (src/native/src/lib.rs:586-676 -> ops/kv_cache.rs): per cache
+ * [batch * heads, max_seq_len, head_dim] keys and values in device memory, fp32 or int8 with one f32 scale per
+ * row (quantize_row_i8, kv_cache.rs:357-370).  The reference keeps the cache in host memory and decodes on the
+ * CPU; here append and decode are kernels.  Ids start at 1 and restart after mni_reset_engine.
+ * create: new cache id, MNI_BAD_ID on error.  len / quantized: 0 for an unknown id.  reset / free: no-ops for
+ * an unknown id.  append(k, v): k, v of shape [B,H,1,D] or [BH,1,D].  decode_step(q, k, v, scale): appends
+ * k, v, then attends q over every cached position; returns the output tensor ([B,H,1,D] or [BH,1,D]).
+ * Errors carry the reference's texts ("kv cache decode failed: kv cache decode expects seq_len=1, got 2", ...). */
+uint32_t mni_kv_cache_create(int64_t batch_size, int64_t num_heads, int64_t head_dim, int64_t max_seq_len, int quantized);
+int64_t mni_kv_cache_len(uint32_t cache_id);
+int mni_kv_cache_quantized(uint32_t cache_id);
+void mni_kv_cache_reset(uint32_t cache_id);
+void mni_kv_cache_free(uint32_t cache_id);
+int mni_kv_cache_append(uint32_t cache_id, uint32_t k, uint32_t v);
+uint32_t mni_kv_cache_decode_step(uint32_t cache_id, uint32_t q, uint32_t k, uint32_t v, double scale);
+/* Remaining elementwise / reduction exports of src/native/src/lib.rs, all on the device:
  * exp_op (:220-225), log_op (:227-232), sigmoid (:374-379), pow_op (:381-386; powf),
  * div (:339-344; broadcasting, backward da = g / b, db = -g a / b^2),
  * lt / eq_op / gt / is_close (:346-372; 1.0 or 0.0, nothing recorded),

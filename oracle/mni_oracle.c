@@ -1486,6 +1486,181 @@ static int conv_shape(const int64_t *shape, int nd, size_t *out) {
     return 0;
 }
 
+/* ---- KV cache --------------------------------------------------------------
+ * ops/kv_cache.rs, cpu arm (:20-334, quantisation helpers :336-383): per cache
+ * fp32 or int8 (+ per-row f32 scale) storage [bh, max_seq, d]; append writes
+ * position `len`; decode_step appends k, v and runs the online-softmax attention
+ * of q over positions 0..len (:259-287).
+ * pinned by: float64 softmax attention over the appended history, the
+ * quantisation bound |x - q * scale| <= scale / 2 and its exact arithmetic on
+ * hand-picked rows, the error cases of test/native.test.ts:112-151. */
+typedef struct {
+    int live, quantized;
+    size_t batch, heads, d, max_seq, len;
+    float *k32, *v32, *kscale, *vscale;
+    signed char *k8, *v8;
+} orc_kv;
+static orc_kv *g_kv;
+static size_t g_kv_cap;
+static uint32_t g_kv_next = 1; /* lib.rs:36 */
+
+static orc_kv *kv_get(uint32_t id) {
+    if (id == 0 || id >= g_kv_cap || !g_kv[id].live) return NULL;
+    return &g_kv[id];
+}
+static void kv_release(orc_kv *c) {
+    free(c->k32); free(c->v32); free(c->kscale); free(c->vscale); free(c->k8); free(c->v8);
+    memset(c, 0, sizeof *c);
+}
+static void kv_clear_storage(orc_kv *c) { /* :73-81 reset */
+    size_t cap = c->batch * c->heads * c->max_seq * c->d, sc = c->batch * c->heads * c->max_seq;
+    c->len = 0;
+    memset(c->k32, 0, cap * sizeof(float)); memset(c->v32, 0, cap * sizeof(float));
+    memset(c->k8, 0, cap); memset(c->v8, 0, cap);
+    for (size_t i = 0; i < sc; ++i) { c->kscale[i] = 1.0f; c->vscale[i] = 1.0f; }
+}
+uint32_t orc_kv_cache_create(int64_t batch, int64_t heads, int64_t head_dim, int64_t max_seq, int quantized) { /* lib.rs:586-607 */
+    uint32_t id = g_kv_next++;
+    if (id >= g_kv_cap) {
+        size_t ncap = g_kv_cap ? g_kv_cap * 2 : 16;
+        while (ncap <= id) ncap *= 2;
+        g_kv = (orc_kv *)realloc(g_kv, ncap * sizeof(orc_kv));
+        memset(g_kv + g_kv_cap, 0, (ncap - g_kv_cap) * sizeof(orc_kv));
+        g_kv_cap = ncap;
+    }
+    orc_kv *c = &g_kv[id];
+    c->live = 1; c->quantized = quantized != 0;
+    c->batch = (size_t)batch; c->heads = (size_t)heads; c->d = (size_t)head_dim; c->max_seq = (size_t)max_seq;
+    size_t cap = c->batch * c->heads * c->max_seq * c->d, sc = c->batch * c->heads * c->max_seq;
+    c->k32 = (float *)malloc((cap ? cap : 1) * sizeof(float)); c->v32 = (float *)malloc((cap ? cap : 1) * sizeof(float));
+    c->k8 = (signed char *)malloc(cap ? cap : 1); c->v8 = (signed char *)malloc(cap ? cap : 1);
+    c->kscale = (float *)malloc((sc ? sc : 1) * sizeof(float)); c->vscale = (float *)malloc((sc ? sc : 1) * sizeof(float));
+    kv_clear_storage(c);
+    return id;
+}
+int64_t orc_kv_cache_len(uint32_t id) { orc_kv *c = kv_get(id); return c ? (int64_t)c->len : 0; }       /* lib.rs:609-616 */
+int orc_kv_cache_quantized(uint32_t id) { orc_kv *c = kv_get(id); return c ? c->quantized : 0; }        /* lib.rs:618-625 */
+void orc_kv_cache_reset(uint32_t id) { orc_kv *c = kv_get(id); if (c) kv_clear_storage(c); }             /* lib.rs:627-633 */
+void orc_kv_cache_free(uint32_t id) { orc_kv *c = kv_get(id); if (c) kv_release(c); }                    /* lib.rs:635-639 */
+
+/* :336-349 parse_bhsd */
+static int kv_parse_bhsd(const orc_tensor *t, size_t *b, size_t *h, size_t *s_, size_t *d, char *err, size_t cap) {
+    if (t->ndim == 4) { *b = t->shape[0]; *h = t->shape[1]; *s_ = t->shape[2]; *d = t->shape[3]; return 0; }
+    if (t->ndim == 3) { *b = 1; *h = t->shape[0]; *s_ = t->shape[1]; *d = t->shape[2]; return 0; }
+    size_t n = (size_t)snprintf(err, cap, "expected [B,H,S,D] or [BH,S,D], got shape [");
+    for (int i = 0; i < t->ndim && n < cap; ++i) n += (size_t)snprintf(err + n, cap - n, i ? ", %zu" : "%zu", t->shape[i]);
+    if (n < cap) snprintf(err + n, cap - n, "]");
+    return -1;
+}
+/* :83-111 validate_single_step_shape */
+static int kv_validate(const orc_kv *c, const orc_tensor *t, const char *op, char *err, size_t cap) {
+    size_t b, h, s_, d;
+    if (kv_parse_bhsd(t, &b, &h, &s_, &d, err, cap) != 0) return -1;
+    if (s_ != 1) { snprintf(err, cap, "kv cache %s expects seq_len=1, got %zu", op, s_); return -1; }
+    if (b != c->batch || h != c->heads || d != c->d) {
+        snprintf(err, cap, "kv cache %s shape mismatch: expected [B=%zu, H=%zu, S=1, D=%zu], got [B=%zu, H=%zu, S=1, D=%zu]",
+                 op, c->batch, c->heads, c->d, b, h, d);
+        return -1;
+    }
+    return 0;
+}
+/* :357-370 quantize_row_i8: scale = max(max|x| / 127, 1e-8); q = clamp(round(x * (1 / scale)), -127, 127) */
+static float kv_quantize_row(const float *in, size_t d, signed char *out) {
+    float max_abs = 0.0f;
+    for (size_t i = 0; i < d; ++i) { float a = fabsf(in[i]); max_abs = a > max_abs ? a : max_abs; }
+    float scale = max_abs / 127.0f;
+    if (!(scale > 1e-8f)) scale = 1e-8f;
+    float inv = 1.0f / scale;
+    for (size_t i = 0; i < d; ++i) {
+        float q = roundf(in[i] * inv); /* f32::round: half away from zero */
+        q = q < -127.0f ? -127.0f : q > 127.0f ? 127.0f : q;
+        out[i] = (signed char)q;
+    }
+    return scale;
+}
+/* :113-171 append_inner */
+static int kv_append_inner(orc_kv *c, const orc_tensor *K, const orc_tensor *V, char *err, size_t cap) {
+    if (c->len >= c->max_seq) { snprintf(err, cap, "kv cache is full (len=%zu, max_seq_len=%zu)", c->len, c->max_seq); return -1; }
+    size_t bh = c->batch * c->heads, d = c->d, pos = c->len;
+    if (K->size != bh * d || V->size != bh * d) { snprintf(err, cap, "expected %zu elements for single-step tensor, got %zu", bh * d, K->size != bh * d ? K->size : V->size); return -1; }
+    float *kd = to_host(K), *vd = to_host(V);
+    for (size_t row = 0; row < bh; ++row) {
+        size_t src = row * d, dst = (row * c->max_seq + pos) * d;
+        if (c->quantized) {
+            c->kscale[row * c->max_seq + pos] = kv_quantize_row(kd + src, d, c->k8 + dst);
+            c->vscale[row * c->max_seq + pos] = kv_quantize_row(vd + src, d, c->v8 + dst);
+        } else {
+            memcpy(c->k32 + dst, kd + src, d * sizeof(float));
+            memcpy(c->v32 + dst, vd + src, d * sizeof(float));
+        }
+    }
+    free(kd); free(vd);
+    c->len += 1;
+    return 0;
+}
+static int same_dims(const orc_tensor *a, const orc_tensor *b) { return same_shape(a->shape, a->ndim, b->shape, b->ndim); }
+
+int orc_kv_cache_append(uint32_t id, uint32_t k, uint32_t v) { /* lib.rs:661-676, kv_cache.rs:173-181 */
+    orc_kv *c = kv_get(id);
+    if (!c) { snprintf(g_err, sizeof g_err, "invalid kv cache id: %u", id); return -1; }
+    orc_tensor *K = get(k), *V = get(v);
+    if (!K || !V) { fail("tensor already freed"); return -1; }
+    char why[400];
+    int rc = 0;
+    if (!same_dims(K, V)) { snprintf(why, sizeof why, "k/v shapes must match for kv cache append"); rc = -1; }
+    if (rc == 0) rc = kv_validate(c, K, "append", why, sizeof why);
+    if (rc == 0) rc = kv_append_inner(c, K, V, why, sizeof why);
+    if (rc != 0) snprintf(g_err, sizeof g_err, "kv cache append failed: %s", why);
+    return rc;
+}
+uint32_t orc_kv_cache_decode_step(uint32_t id, uint32_t q, uint32_t k, uint32_t v, double scale_) { /* lib.rs:641-659, kv_cache.rs:183-306 */
+    orc_kv *c = kv_get(id);
+    if (!c) { snprintf(g_err, sizeof g_err, "invalid kv cache id: %u", id); return ORC_BAD; }
+    orc_tensor *Q = get(q), *K = get(k), *V = get(v);
+    if (!Q || !K || !V) return fail("tensor already freed");
+    char why[400];
+    int rc = 0;
+    if (!same_dims(Q, K) || !same_dims(Q, V)) { snprintf(why, sizeof why, "q/k/v shapes must match for kv cache decode"); rc = -1; }
+    if (rc == 0) rc = kv_validate(c, Q, "decode", why, sizeof why);
+    if (rc == 0) rc = kv_append_inner(c, K, V, why, sizeof why);
+    if (rc != 0) { snprintf(g_err, sizeof g_err, "kv cache decode failed: %s", why); return ORC_BAD; }
+    float scale = (float)scale_;
+    size_t bh = c->batch * c->heads, d = c->d, cur = c->len;
+    int q_nd = Q->ndim;
+    float *qd = to_host(Q);
+    float *out = (float *)calloc((bh * d) > 0 ? bh * d : 1, sizeof(float));
+    float *acc = (float *)malloc((d ? d : 1) * sizeof(float));
+    for (size_t row = 0; row < bh; ++row) {
+        float running_max = -INFINITY, running_sum = 0.0f;
+        for (size_t dd = 0; dd < d; ++dd) acc[dd] = 0.0f;
+        for (size_t col = 0; col < cur; ++col) {
+            size_t off = (row * c->max_seq + col) * d;
+            float ks = c->kscale[row * c->max_seq + col], vs = c->vscale[row * c->max_seq + col];
+            float dot = 0.0f;
+            for (size_t dd = 0; dd < d; ++dd) {
+                float kv = c->quantized ? (float)c->k8[off + dd] * ks : c->k32[off + dd]; /* :372-383 dequantize */
+                dot += qd[row * d + dd] * kv;
+            }
+            dot *= scale;
+            float old_max = running_max;
+            running_max = running_max > dot ? running_max : dot;
+            float exp_diff = expf(old_max - running_max);
+            float w = expf(dot - running_max);
+            running_sum = running_sum * exp_diff + w;
+            for (size_t dd = 0; dd < d; ++dd) {
+                float vv = c->quantized ? (float)c->v8[off + dd] * vs : c->v32[off + dd];
+                acc[dd] = acc[dd] * exp_diff + w * vv;
+            }
+        }
+        float inv_sum = running_sum > 0.0f ? 1.0f / running_sum : 0.0f;
+        for (size_t dd = 0; dd < d; ++dd) out[row * d + dd] = acc[dd] * inv_sum;
+    }
+    free(acc); free(qd);
+    size_t s4[4] = {c->batch, c->heads, 1, d}, s3[3] = {bh, 1, d};
+    return (uint32_t)(q_nd == 4 ? from_vec(out, s4, 4) : from_vec(out, s3, 3));
+}
+
+/* ---- public surface ------------------------------------------------------ */
 uint32_t orc_zeros(const int64_t *shape, int nd) { /* lib.rs:45-50 */
     size_t s[ORC_MAX_DIMS];
     if (conv_shape(shape, nd, s)) return ORC_BAD;
@@ -1654,6 +1829,8 @@ double orc_clip_and_step(const uint32_t *ids, size_t n, double lr, double b1, do
     return (double)norm;
 }
 void orc_reset_engine(void) { /* lib.rs:460-468 */
+    for (size_t i = 0; i < g_kv_cap; ++i) if (g_kv[i].live) kv_release(&g_kv[i]);
+    g_kv_next = 1;
     for (size_t i = 0; i < g_store.len; ++i)
         if (g_store.t[i].live) { free(g_store.t[i].data); free(g_store.t[i].adam_m); free(g_store.t[i].adam_v); }
     free(g_store.t); free(g_store.free_ids);

@@ -61,6 +61,10 @@ class OracleNative:
             "orc_cross_entropy_loss": (u32, [u32, _i64p, C.c_size_t]),
             "orc_softmax_op": (u32, [u32, C.c_int64]),
             "orc_bias_gelu": (u32, [u32, u32]),
+            "orc_kv_cache_create": (u32, [C.c_int64] * 4 + [C.c_int]), "orc_kv_cache_len": (C.c_int64, [u32]),
+            "orc_kv_cache_quantized": (C.c_int, [u32]), "orc_kv_cache_reset": (None, [u32]), "orc_kv_cache_free": (None, [u32]),
+            "orc_kv_cache_append": (C.c_int, [u32, u32, u32]),
+            "orc_kv_cache_decode_step": (u32, [u32, u32, u32, u32, C.c_double]),
             "orc_exp_op": (u32, [u32]), "orc_log_op": (u32, [u32]), "orc_sigmoid": (u32, [u32]),
             "orc_pow_op": (u32, [u32, C.c_double]), "orc_div": (u32, [u32, u32]),
             "orc_lt": (u32, [u32, u32]), "orc_eq_op": (u32, [u32, u32]), "orc_gt": (u32, [u32, u32]),
@@ -201,6 +205,28 @@ class OracleNative:
 
     def biasGelu(self, x, bias):
         return self._id(self.lib.orc_bias_gelu(x, bias))
+
+    def kvCacheCreate(self, batchSize, numHeads, headDim, maxSeqLen, quantized):
+        return self.lib.orc_kv_cache_create(batchSize, numHeads, headDim, maxSeqLen, 1 if quantized else 0)
+
+    def kvCacheLen(self, cacheId):
+        return self.lib.orc_kv_cache_len(cacheId)
+
+    def kvCacheQuantized(self, cacheId):
+        return bool(self.lib.orc_kv_cache_quantized(cacheId))
+
+    def kvCacheReset(self, cacheId):
+        self.lib.orc_kv_cache_reset(cacheId)
+
+    def kvCacheFree(self, cacheId):
+        self.lib.orc_kv_cache_free(cacheId)
+
+    def kvCacheAppend(self, cacheId, k, v):
+        if self.lib.orc_kv_cache_append(cacheId, k, v) != 0:
+            raise self._err()
+
+    def kvCacheDecodeStep(self, cacheId, q, k, v, scale):
+        return self._id(self.lib.orc_kv_cache_decode_step(cacheId, q, k, v, scale))
 
     def expOp(self, a):
         return self._id(self.lib.orc_exp_op(a))

@@ -130,6 +130,38 @@ assertClose(mseLoss(p, Tensor.fromFloat32(new Float32Array([2, 3, 4, 5]), [2, 2]
   assert(worst < 1e-6, 'causal attention row 0 equals v[0]');
 }
 
+// ---- KV cache (test/native.test.ts:48-151) -----------------------------------------------------------
+{
+  const batch = 1, heads = 2, headDim = 8, maxSeq = 16, steps = 6, scale = 1 / Math.sqrt(headDim);
+  const mk = (s) => Tensor.fromFloat32(randArray(batch * heads * s * headDim, rnd, 0, 1), [batch, heads, s, headDim]);
+  const fp = native.kvCacheCreate(batch, heads, headDim, maxSeq, false), qc = native.kvCacheCreate(batch, heads, headDim, maxSeq, true);
+  assert(native.kvCacheQuantized(qc) === true && native.kvCacheQuantized(fp) === false, 'quantized flag');
+  let maxAbsDiff = 0;
+  for (let t = 0; t < steps; t++) {
+    const q = mk(1), k = mk(1), v = mk(1);
+    const a = native.toFloat32(native.kvCacheDecodeStep(fp, q._id, k._id, v._id, scale));
+    const b = native.toFloat32(native.kvCacheDecodeStep(qc, q._id, k._id, v._id, scale));
+    for (let i = 0; i < a.length; i++) maxAbsDiff = Math.max(maxAbsDiff, Math.abs(a[i] - b[i]));
+    assert(a.length === batch * heads * headDim, 'decode output size');
+  }
+  assert(Number(native.kvCacheLen(fp)) === steps && Number(native.kvCacheLen(qc)) === steps, 'kv cache length tracks decode steps');
+  assert(maxAbsDiff < 0.15, 'quantized kv decode drift bounded (' + maxAbsDiff.toFixed(4) + ')');
+  let threw = false;
+  try { const t2 = mk(2); native.kvCacheDecodeStep(fp, t2._id, t2._id, t2._id, scale); } catch (e) { threw = /seq_len=1/.test(e.message); }
+  assert(threw, 'decode step rejects seq_len != 1');
+  const small = native.kvCacheCreate(batch, heads, headDim, 2, false);
+  native.kvCacheAppend(small, mk(1)._id, mk(1)._id); native.kvCacheAppend(small, mk(1)._id, mk(1)._id);
+  threw = false;
+  try { native.kvCacheAppend(small, mk(1)._id, mk(1)._id); } catch (e) { threw = /kv cache is full/.test(e.message); }
+  assert(threw, 'append rejects capacity overflow');
+  native.kvCacheReset(fp);
+  assert(Number(native.kvCacheLen(fp)) === 0, 'kv cache reset clears logical length');
+  native.kvCacheFree(fp);
+  threw = false;
+  try { native.kvCacheDecodeStep(fp, mk(1)._id, mk(1)._id, mk(1)._id, scale); } catch (e) { threw = /invalid kv cache id/.test(e.message); }
+  assert(threw, 'free invalidates kv cache handle');
+}
+
 // ---- misuse raises a JS Error where the reference panics ---------------------------------------------
 try { Tensor.fromFloat32(new Float32Array(6), [2, 3]).matmul(Tensor.fromFloat32(new Float32Array(8), [4, 2])); assert(false, 'K mismatch must throw'); }
 catch (e) { assert(/inner dimensions/.test(e.message), 'K mismatch message: ' + e.message); }
