@@ -119,8 +119,11 @@ struct Allocator {
     size_t cached = 0;
 };
 static Allocator &allocator() {
-    static Allocator a;
-    return a;
+    // Never destroyed: tensors of the engine (another translation unit's
+    // static) return their buffers here while the process exits, in an order
+    // the language does not fix; the driver reclaims device memory itself.
+    static Allocator *a = new Allocator;
+    return *a;
 }
 static size_t round_size(size_t bytes) {
     if (bytes == 0) bytes = 4;

@@ -94,8 +94,10 @@ struct Engine {
     uint32_t next_kv_cache_id = 1;          // lib.rs:36
 };
 static Engine &eng() {
-    static Engine e;
-    return e;
+    // Never destroyed: releasing device buffers from a static destructor would
+    // run after the HIP runtime may already have shut down.
+    static Engine *e = new Engine;
+    return *e;
 }
 
 // ---- shape helpers -----------------------------------------------------------
@@ -1216,8 +1218,10 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
         BufP db = o ? new_buf((size_t)c) : nullptr;
         if (!db) return MNI_ERR_NOMEM;
         MNI_TRY(k_bias_gelu_backward(o->p, db->p, gb->p, Z->buf->p, Bv->buf->p, c ? Z->size / c : 0, c));
-        g = insert_contig(std::move(o), G->shape);
-        db_id = insert_contig(std::move(db), Bv->shape);
+        // shapes are copied first: an insert may move the tensor table and leave G / Bv dangling
+        const Shape gshape = G->shape, bshape = Bv->shape;
+        g = insert_contig(std::move(o), gshape);
+        db_id = insert_contig(std::move(db), bshape);
         own_g = true;
     } else if (e.act == MNI_EPI_BIAS_RELU) {
         // dZ = dOut where the output is positive (the output has the sign of z)
