@@ -72,6 +72,14 @@ def bind(native):
         def ones(shape):
             return Tensor(native.ones(list(shape)), shape)
 
+        @staticmethod
+        def rand(shape):  # src/tensor.ts rand -> native.randTensor, uniform [0, 1)
+            return Tensor(native.randTensor(list(shape)), shape)
+
+        @staticmethod
+        def randn(shape):
+            return Tensor(native.randnTensor(list(shape)), shape)
+
         # elementwise (src/tensor.ts:101-133): a number becomes a [1] tensor for
         # add/sub and a scalar multiply for mul
         def add(self, other):
@@ -193,6 +201,22 @@ def bind(native):
             y = x.matmul(self.weight.value).add(self.bias.value)
             return y if self.activation is None else (y.relu() if self.activation == "relu" else y.gelu())
 
+    class Embedding(Module):  # src/nn.ts:46-71: weight [vocab, dim], bound 1/sqrt(dim)
+        def __init__(self, vocabSize, embedDim, weight=None):
+            self.vocabSize, self.embedDim = vocabSize, embedDim
+            bound = 1.0 / math.sqrt(embedDim)
+            if weight is None:
+                weight = np.random.uniform(-bound, bound, (vocabSize, embedDim)).astype(np.float32)
+            self.weight = Parameter(Tensor.fromFloat32(weight, [vocabSize, embedDim]).setRequiresGrad(True))
+
+        def forward(self, indices):
+            batch, seqLen = len(indices), len(indices[0])
+            flat = [int(i) for row in indices for i in row]
+            return Tensor(native.embeddingForward(self.weight.value._id, flat, batch, seqLen))
+
+        def forwardGpu(self, intBufId, batch, seqLen):
+            return Tensor(native.embeddingForwardGpu(self.weight.value._id, intBufId, batch, seqLen))
+
     class ReLU(Module):
         def forward(self, x):
             return x.relu()
@@ -212,6 +236,20 @@ def bind(native):
         flat = logits.view(BT, V)
         flat_targets = [int(t) for row in targets for t in (row if isinstance(row, (list, tuple, np.ndarray)) else [row])]
         return Tensor(native.crossEntropyLoss(flat._id, flat_targets))
+
+    def crossEntropyLossGpu(logits, intBufId):  # src/nn.ts:102-105
+        return Tensor(native.crossEntropyLossGpu(logits._id, intBufId))
+
+    def dropout(x, rate=0.0, inference=False):  # src/nn.ts:85-88
+        if inference or rate == 0:
+            return x
+        return Tensor(native.dropoutOp(x._id, rate, True))
+
+    def residualLayerNorm(x, residual, gamma, beta, eps=1e-5):  # src/nn.ts:149-151
+        return Tensor(native.residualLayernorm(x._id, residual._id, gamma._id, beta._id, eps))
+
+    def tile(x, reps):  # src/nn.ts:251-253
+        return Tensor(native.tile(x._id, list(reps)))
 
     def softmax(x, dim=-1):  # src/nn.ts:77-79
         return Tensor(native.softmaxOp(x._id, dim))
@@ -264,6 +302,32 @@ def bind(native):
             ids = [p.value._id for p in self.parameters]
             return native.clipAndStep(ids, self.lr, self.beta1, self.beta2, self.eps, self.weightDecay, self.t, maxGradNorm)
 
-    return SimpleNamespace(native=native, Tensor=Tensor, Parameter=Parameter, Module=Module, Linear=Linear, ReLU=ReLU,
+    class GradScaler:  # src/optimizer.ts:72-121
+        def __init__(self, initScale=65536.0, growthFactor=2.0, backoffFactor=0.5, growthInterval=2000):
+            self.scale, self.growthFactor, self.backoffFactor = initScale, growthFactor, backoffFactor
+            self.growthInterval, self.stepsSinceGrowth = growthInterval, 0
+
+        def getScale(self):
+            return self.scale
+
+        def scaleLoss(self, loss):
+            return loss.mul(self.scale)
+
+        def unscaleAndStep(self, optimizer, maxGradNorm=0.0):
+            ids = [p.value._id for p in optimizer.parameters]
+            if native.scaleGrads(ids, 1.0 / self.scale):
+                self.scale *= self.backoffFactor
+                self.stepsSinceGrowth = 0
+                optimizer.zeroGrad()
+                return {"gradNorm": 0, "skipped": True}
+            gradNorm = optimizer.step(maxGradNorm)
+            self.stepsSinceGrowth += 1
+            if self.stepsSinceGrowth >= self.growthInterval:
+                self.scale *= self.growthFactor
+                self.stepsSinceGrowth = 0
+            return {"gradNorm": gradNorm, "skipped": False}
+
+    return SimpleNamespace(native=native, Embedding=Embedding, crossEntropyLossGpu=crossEntropyLossGpu, dropout=dropout,
+                           residualLayerNorm=residualLayerNorm, tile=tile, GradScaler=GradScaler, Tensor=Tensor, Parameter=Parameter, Module=Module, Linear=Linear, ReLU=ReLU,
                            GELU=GELU, mseLoss=mseLoss, crossEntropyLoss=crossEntropyLoss, softmax=softmax, biasGelu=biasGelu, layerNorm=layerNorm,
                            flashAttention=flashAttention, KvCache=KvCache, Adam=Adam)

@@ -127,6 +127,22 @@ int k_kv_append(void *kc, void *vc, float *ks, float *vs, const float *k, const 
 int k_kv_decode(float *out, const void *kc, const void *vc, const float *ks, const float *vs, const float *q, int64_t bh,
                 int64_t d, int64_t max_seq, int64_t len, float scale, int quantized);
 
+// sequence.hip
+// mode 0: uniform [0, 1), 1: standard normal, 2: the raw Philox words; element i is word i % 4 of block offset + i / 4
+int k_random_fill(float *out, int64_t n, uint64_t seed, uint64_t offset, int mode);
+// out = x * (u >= rate) * scale with the uniforms of (seed, offset); also the backward, with the gradient as x
+int k_dropout(float *out, const float *x, int64_t n, float rate, float scale, uint64_t seed, uint64_t offset);
+int k_sample_windows(int32_t *inputs, int32_t *targets, const int32_t *data, const int32_t *starts, int64_t block, int64_t batch);
+int k_embedding_forward(float *out, const float *w, const int32_t *idx, int64_t tokens, int64_t dim);
+// dw[v] = sum of g[t] over idx[t] == v in increasing t; `work` holds 3 * vocab + 2 + 2 * tokens int32 values
+int k_embedding_backward(float *dw, const float *g, const int32_t *idx, int64_t tokens, int64_t vocab, int64_t dim,
+                         int32_t *work);
+int k_tile(float *out, const float *in, const int64_t *in_shape, const int64_t *reps, int ndim);
+int k_residual_layernorm(float *out, float *res, float *mean, float *rstd, const float *x, const float *residual,
+                         const float *gamma, const float *beta, int64_t rows, int64_t c, float eps);
+// g *= s; *flag = 1 if any scaled value is infinite or NaN (flag is not cleared here)
+int k_scale_check(float *g, float s, int64_t n, float *flag);
+
 int k_sumsq_f64(double *out, const float *g, int64_t n);  // out += sum g^2 (device double)
 int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, float b1, float b2,
             float eps, float wd, float bc1, float bc2);

@@ -8,6 +8,11 @@
 // allows.
 #include "common.h"
 
+// The reference's cpu arm rounds every multiply and every add separately (Rust
+// never contracts a * b + c); these kernels are bandwidth-bound, so they do
+// the same and stay as close to it as the summation order allows.
+#pragma clang fp contract(off)
+
 namespace mni {
 
 static constexpr int TPB = 256;

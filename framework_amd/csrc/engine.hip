@@ -12,6 +12,7 @@
 
 #include <map>
 #include <memory>
+#include <random>
 #include <string>
 #include <vector>
 
@@ -53,14 +54,15 @@ enum Op {  // subset of src/native/src/autograd.rs:28-62 plus the fused Linear
     OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
     OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY, OP_LINEAR,
     OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU,
-    OP_EXP, OP_LOG, OP_DIV, OP_SIGMOID, OP_POW, OP_MAX, OP_LAYERNORM
+    OP_EXP, OP_LOG, OP_DIV, OP_SIGMOID, OP_POW, OP_MAX, OP_LAYERNORM,
+    OP_EMBEDDING, OP_DROPOUT, OP_RESIDUALLAYERNORM
 };
 
 // src/native/src/autograd.rs:65-70 TapeEntry
 struct Entry {
     int op;
     uint32_t output_id;
-    uint32_t inputs[3];
+    uint32_t inputs[4];
     int n_inputs;
     Shape saved_shape;   // Shape / TensorAndShape / Permutation original shape
     Shape saved_perm;
@@ -68,8 +70,10 @@ struct Entry {
     int act = 0;         // OP_LINEAR: epilogue
     uint32_t aux = MNI_BAD_ID;  // cross-entropy softmax / linear pre-activation / softmax output / attention output
     uint32_t aux2 = MNI_BAD_ID; // attention log-sum-exp
-    std::shared_ptr<void> targets;  // device int32 targets
+    uint32_t aux3 = MNI_BAD_ID; // residual + layernorm: the saved sum x + residual
+    std::shared_ptr<void> targets;  // device int32 targets / embedding indices
     int64_t ce_n = 0, ce_v = 0;
+    uint64_t rng_seed = 0, rng_offset = 0;  // dropout: where its mask starts in the random stream
 };
 
 struct Tape {
@@ -86,12 +90,30 @@ struct KvCache {
     std::shared_ptr<void> kscale, vscale;  // [bh, max_seq] float (quantized only)
 };
 
+// ops/data.rs:13-27 IntBuffer, on the device.  lo / hi bound the values it can
+// hold (a batch sampled from a dataset inherits the dataset's bounds), so an
+// index can be checked against a table without reading the device.
+struct IntBuf {
+    bool live = false;
+    std::shared_ptr<void> data;  // int32
+    int64_t len = 0;
+    int32_t lo = 0, hi = 0;
+};
+
 struct Engine {
     std::vector<Tensor> tensors;
     std::vector<uint32_t> free_ids;
     Tape tape;
     std::map<uint32_t, KvCache> kv_caches;  // lib.rs:23-24
     uint32_t next_kv_cache_id = 1;          // lib.rs:36
+    std::vector<IntBuf> int_bufs;           // ops/data.rs:24-27 IntStore
+    std::vector<uint32_t> int_free;
+    // Random numbers: Philox blocks (seed, offset) on the device, a Mersenne
+    // twister for the host-side window starts.  Seeded from the system's
+    // entropy like the reference's thread_rng unless mni_seed() fixes it.
+    bool rng_ready = false;
+    uint64_t rng_seed = 0, rng_offset = 0;
+    std::mt19937_64 host_rng;
 };
 static Engine &eng() {
     // Never destroyed: releasing device buffers from a static destructor would
@@ -1254,9 +1276,336 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
     return rc;
 }
 
+// ---- random numbers ------------------------------------------------------------------------------
+static void rng_init(Engine &e) {
+    if (e.rng_ready) return;
+    std::random_device rd;
+    e.rng_seed = ((uint64_t)rd() << 32) ^ (uint64_t)rd();
+    e.rng_offset = 0;
+    e.host_rng.seed(e.rng_seed);
+    e.rng_ready = true;
+}
+// Reserve the Philox blocks for n elements and return where they start.
+static uint64_t rng_take(int64_t n) {
+    Engine &e = eng();
+    rng_init(e);
+    const uint64_t at = e.rng_offset;
+    e.rng_offset += (uint64_t)((n + 3) / 4);
+    return at;
+}
+// tensor.rs:228-250 rand (uniform [0, 1)) / randn (standard normal)
+static uint32_t random_tensor(const Shape &shape, int mode) {
+    const int64_t n = shape_size(shape);
+    BufP b = new_buf((size_t)n);
+    if (!b) return MNI_BAD_ID;
+    const uint64_t at = rng_take(n);
+    if (k_random_fill(b->p, n, eng().rng_seed, at, mode) != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(b), shape);
+}
+
+// ---- dropout (ops/dropout.rs) --------------------------------------------------------------------
+// The mask is not stored: the tape keeps where it starts in the random stream
+// and the backward regenerates it.
+static uint32_t dropout_op(uint32_t x, float rate, bool training) {
+    Tensor *X = get(x);
+    if (!X) return MNI_BAD_ID;
+    if (!training || rate == 0.0f) return x;  // the same id, dropout.rs:30-32
+    const Shape shape = X->shape;
+    const int64_t n = X->size;
+    BufP src = contiguous_buf(*X);
+    BufP out = src ? new_buf((size_t)n) : nullptr;
+    if (!out) return MNI_BAD_ID;
+    const float scale = 1.0f / (1.0f - rate);
+    const uint64_t at = rng_take(n);
+    if (k_dropout(out->p, src->p, n, rate, scale, eng().rng_seed, at) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(out), shape);
+    Entry e;
+    e.op = OP_DROPOUT; e.output_id = id; e.n_inputs = 1; e.inputs[0] = x; e.scalar = rate;
+    e.rng_seed = eng().rng_seed; e.rng_offset = at;
+    eng().tape.record(std::move(e));
+    return id;
+}
+static int dropout_backward(uint32_t grad, const Entry &e, int64_t *out) {  // dropout.rs:114-126
+    Tensor *G = get(grad);
+    if (!G) return MNI_ERR_FREED;
+    const Shape shape = G->shape;
+    BufP g = contiguous_buf(*G);
+    BufP o = g ? new_buf((size_t)G->size) : nullptr;
+    if (!o) return MNI_ERR_NOMEM;
+    const float scale = 1.0f / (1.0f - e.scalar);
+    MNI_TRY(k_dropout(o->p, g->p, G->size, e.scalar, scale, e.rng_seed, e.rng_offset));
+    out[0] = insert_contig(std::move(o), shape);
+    return MNI_OK;
+}
+
+// ---- integer buffers and datasets (ops/data.rs) ------------------------------------------------------
+static IntBuf *get_int(uint32_t id) {  // data.rs:49-51
+    Engine &e = eng();
+    if (id >= e.int_bufs.size() || !e.int_bufs[id].live) {
+        set_error(MNI_ERR_FREED, "int buffer already freed (id %u)", id);
+        return nullptr;
+    }
+    return &e.int_bufs[id];
+}
+static uint32_t insert_int(IntBuf &&b) {  // data.rs:37-47: LIFO id recycling
+    Engine &e = eng();
+    b.live = true;
+    if (!e.int_free.empty()) {
+        const uint32_t id = e.int_free.back();
+        e.int_free.pop_back();
+        e.int_bufs[id] = std::move(b);
+        return id;
+    }
+    e.int_bufs.push_back(std::move(b));
+    return (uint32_t)e.int_bufs.size() - 1;
+}
+static std::shared_ptr<void> dev_ints(size_t n) {
+    void *p = nullptr;
+    if (dev_alloc(&p, (n ? n : 1) * sizeof(int32_t)) != MNI_OK) return nullptr;
+    return std::shared_ptr<void>(p, [](void *q) { dev_free(q); });
+}
+static uint32_t create_dataset(const int32_t *data, size_t len) {  // data.rs:69-77
+    IntBuf b;
+    b.data = dev_ints(len);
+    if (!b.data) return MNI_BAD_ID;
+    b.len = (int64_t)len;
+    if (len) {
+        b.lo = b.hi = data[0];
+        for (size_t i = 1; i < len; ++i) {
+            if (data[i] < b.lo) b.lo = data[i];
+            if (data[i] > b.hi) b.hi = data[i];
+        }
+        if (mni_rocm_h2d(b.data.get(), data, len * sizeof(int32_t)) != MNI_OK) return MNI_BAD_ID;
+    }
+    return insert_int(std::move(b));
+}
+// data.rs:112-155: batch_size windows of block_size tokens, each starting at a
+// uniform offset in [0, len - block_size - 1); targets are the inputs shifted
+// by one token.  Only the offsets cross the bus.
+static int sample_batch(uint32_t dataset, int64_t block, int64_t batch, uint32_t *out_ids) {
+    IntBuf *ds = get_int(dataset);
+    if (!ds) return MNI_ERR_FREED;
+    if (block <= 0 || batch <= 0) return set_error(MNI_ERR_INVALID, "sample_batch: block_size and batch_size must be positive");
+    const int64_t range = ds->len - block - 1;
+    if (range <= 0)
+        return set_error(MNI_ERR_INVALID, "sample_batch: cannot sample empty range (dataset of %lld tokens, block_size %lld)",
+                         (long long)ds->len, (long long)block);
+    if (ds->len > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "sample_batch: dataset too large for 32-bit offsets");
+    Engine &e = eng();
+    rng_init(e);
+    std::vector<int32_t> starts((size_t)batch);
+    std::uniform_int_distribution<int64_t> pick(0, range - 1);
+    for (auto &s : starts) s = (int32_t)pick(e.host_rng);
+    std::shared_ptr<void> dstarts = dev_ints((size_t)batch);
+    IntBuf inp, tgt;
+    inp.data = dev_ints((size_t)(batch * block));
+    tgt.data = dev_ints((size_t)(batch * block));
+    if (!dstarts || !inp.data || !tgt.data) return MNI_ERR_NOMEM;
+    MNI_TRY(mni_rocm_h2d(dstarts.get(), starts.data(), (size_t)batch * sizeof(int32_t)));
+    const std::shared_ptr<void> src = ds->data;
+    inp.len = tgt.len = batch * block;
+    inp.lo = tgt.lo = ds->lo;
+    inp.hi = tgt.hi = ds->hi;
+    MNI_TRY(k_sample_windows((int32_t *)inp.data.get(), (int32_t *)tgt.data.get(), (const int32_t *)src.get(),
+                             (const int32_t *)dstarts.get(), block, batch));
+    // the offsets buffer returns to the allocator here; the stream orders its reuse after the kernel
+    out_ids[0] = insert_int(std::move(inp));
+    out_ids[1] = insert_int(std::move(tgt));
+    return MNI_OK;
+}
+
+// ---- embedding (ops/embedding.rs) ------------------------------------------------------------------
+static uint32_t embedding_common(uint32_t weight, std::shared_ptr<void> idx, int64_t batch, int64_t seq_len) {
+    Tensor *W = get(weight);
+    if (!W) return MNI_BAD_ID;
+    const int64_t dim = W->shape[1], tokens = batch * seq_len;
+    BufP w = contiguous_buf(*W);
+    BufP out = w ? new_buf((size_t)(tokens * dim)) : nullptr;
+    if (!out) return MNI_BAD_ID;
+    if (k_embedding_forward(out->p, w->p, (const int32_t *)idx.get(), tokens, dim) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(out), Shape{batch, seq_len, dim});
+    Entry e;
+    e.op = OP_EMBEDDING; e.output_id = id; e.n_inputs = 1; e.inputs[0] = weight;
+    e.targets = std::move(idx); e.ce_n = tokens;
+    eng().tape.record(std::move(e));
+    return id;
+}
+static bool embedding_check(uint32_t weight, int64_t batch, int64_t seq_len, int64_t have, int64_t lo, int64_t hi) {
+    Tensor *W = get(weight);
+    if (!W) return false;
+    if (W->shape.size() != 2) { set_error(MNI_ERR_INVALID, "embedding: weight must be [vocab, dim]"); return false; }
+    if (batch < 0 || seq_len < 0 || batch * seq_len > have) {
+        set_error(MNI_ERR_INVALID, "embedding: %lld indices for batch %lld x seq_len %lld", (long long)have, (long long)batch,
+                  (long long)seq_len);
+        return false;
+    }
+    if (batch * seq_len > 0 && (lo < 0 || hi >= W->shape[0])) {
+        set_error(MNI_ERR_INVALID, "embedding: index %lld out of range for %lld rows", (long long)(lo < 0 ? lo : hi),
+                  (long long)W->shape[0]);
+        return false;
+    }
+    return true;
+}
+static uint32_t embedding_forward(uint32_t weight, const int64_t *indices, size_t n, int64_t batch, int64_t seq_len) {
+    const int64_t tokens = batch * seq_len;
+    int64_t lo = 0, hi = 0;
+    if (batch >= 0 && seq_len >= 0 && tokens <= (int64_t)n && tokens > 0) {
+        lo = hi = indices[0];
+        for (int64_t i = 1; i < tokens; ++i) {
+            if (indices[i] < lo) lo = indices[i];
+            if (indices[i] > hi) hi = indices[i];
+        }
+    }
+    if (!embedding_check(weight, batch, seq_len, (int64_t)n, lo, hi)) return MNI_BAD_ID;
+    std::vector<int32_t> i32((size_t)tokens);
+    for (int64_t i = 0; i < tokens; ++i) i32[(size_t)i] = (int32_t)indices[i];
+    std::shared_ptr<void> dev = dev_ints((size_t)tokens);
+    if (!dev) return MNI_BAD_ID;
+    if (tokens && mni_rocm_h2d(dev.get(), i32.data(), (size_t)tokens * sizeof(int32_t)) != MNI_OK) return MNI_BAD_ID;
+    return embedding_common(weight, std::move(dev), batch, seq_len);
+}
+static uint32_t embedding_forward_gpu(uint32_t weight, uint32_t int_buf, int64_t batch, int64_t seq_len) {
+    IntBuf *b = get_int(int_buf);
+    if (!b) return MNI_BAD_ID;
+    if (!embedding_check(weight, batch, seq_len, b->len, b->lo, b->hi)) return MNI_BAD_ID;
+    return embedding_common(weight, b->data, batch, seq_len);
+}
+static int embedding_backward(uint32_t grad, const Entry &e, int64_t *out) {  // embedding.rs:104-128
+    Tensor *W = get(e.inputs[0]), *G = get(grad);
+    if (!W || !G) return MNI_ERR_FREED;
+    const Shape wshape = W->shape;
+    const int64_t vocab = wshape[0], dim = wshape[1], tokens = e.ce_n;
+    if (G->size < tokens * dim) return set_error(MNI_ERR_INVALID, "embedding backward: gradient smaller than the output");
+    BufP g = contiguous_buf(*G);
+    BufP dw = g ? new_buf((size_t)(vocab * dim)) : nullptr;
+    std::shared_ptr<void> work = dw ? dev_ints((size_t)(3 * vocab + 2 + 2 * tokens)) : nullptr;
+    if (!work) return MNI_ERR_NOMEM;
+    MNI_TRY(k_embedding_backward(dw->p, g->p, (const int32_t *)e.targets.get(), tokens, vocab, dim, (int32_t *)work.get()));
+    out[0] = insert_contig(std::move(dw), wshape);
+    return MNI_OK;
+}
+
+// lib.rs:679-691 + ops/loss.rs:190-229: cross-entropy with the targets in an
+// integer buffer; the logits are viewed as [rows, classes] first (a View entry
+// on the tape, like the reference).
+static uint32_t cross_entropy_gpu_op(uint32_t logits, uint32_t int_buf) {
+    Tensor *L = get(logits);
+    IntBuf *T = get_int(int_buf);
+    if (!L || !T) return MNI_BAD_ID;
+    if (L->shape.empty()) { set_error(MNI_ERR_INVALID, "cross_entropy: scalar logits"); return MNI_BAD_ID; }
+    const int64_t v = L->shape.back();
+    const int64_t n = v ? L->size / v : 0;
+    if (n <= 0 || v <= 0) { set_error(MNI_ERR_INVALID, "cross_entropy: empty logits"); return MNI_BAD_ID; }
+    if (T->len < n) { set_error(MNI_ERR_INVALID, "cross_entropy: %lld targets for %lld rows", (long long)T->len, (long long)n); return MNI_BAD_ID; }
+    if (T->lo < 0 || T->hi >= v) {
+        set_error(MNI_ERR_INVALID, "cross_entropy: target %lld out of range [0, %lld)", (long long)(T->lo < 0 ? T->lo : T->hi), (long long)v);
+        return MNI_BAD_ID;
+    }
+    const std::shared_ptr<void> tdev = T->data;
+    const uint32_t flat = view_op(logits, Shape{n, v});
+    if (flat == MNI_BAD_ID) return MNI_BAD_ID;
+    Tensor *F = get(flat);
+    BufP x = contiguous_buf(*F);
+    BufP sm = x ? new_buf((size_t)(n * v)) : nullptr;
+    BufP loss = sm ? new_buf(1) : nullptr;
+    if (!loss) return MNI_BAD_ID;
+    if (k_cross_entropy(loss->p, sm->p, x->p, (const int32_t *)tdev.get(), n, v) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t loss_id = insert_contig(std::move(loss), Shape{1});
+    const uint32_t sm_id = insert_contig(std::move(sm), Shape{n, v});
+    Entry e;
+    e.op = OP_CROSSENTROPY; e.output_id = loss_id; e.n_inputs = 1; e.inputs[0] = flat;
+    e.aux = sm_id; e.targets = tdev; e.ce_n = n; e.ce_v = v;
+    eng().tape.record(std::move(e));
+    return loss_id;
+}
+
+// ---- tile (ops/pooling.rs:276-309; not recorded on the tape there either) ----------------------------
+static uint32_t tile_op(uint32_t a, const int64_t *reps, int n) {
+    Tensor *A = get(a);
+    if (!A) return MNI_BAD_ID;
+    const int nd = (int)A->shape.size();
+    if (n != nd) { set_error(MNI_ERR_INVALID, "tile: reps must match tensor dimensions"); return MNI_BAD_ID; }
+    if (nd < 1) { set_error(MNI_ERR_INVALID, "tile: the tensor must have at least one dim"); return MNI_BAD_ID; }
+    const Shape shape = A->shape;
+    Shape out_shape(nd);
+    for (int i = 0; i < nd; ++i) {
+        if (reps[i] < 0) { set_error(MNI_ERR_INVALID, "tile: negative repeat count"); return MNI_BAD_ID; }
+        out_shape[i] = shape[i] * reps[i];
+    }
+    BufP src = contiguous_buf(*A);
+    BufP out = src ? new_buf((size_t)shape_size(out_shape)) : nullptr;
+    if (!out || k_tile(out->p, src->p, shape.data(), reps, nd) != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(out), out_shape);
+}
+
+// ---- residual + layernorm (ops/fused.rs:23-78, 134-186) ----------------------------------------------
+static uint32_t residual_layernorm_op(uint32_t x, uint32_t residual, uint32_t gamma, uint32_t beta, float eps) {
+    Tensor *X = get(x), *R = get(residual), *Gm = get(gamma), *Bt = get(beta);
+    if (!X || !R || !Gm || !Bt) return MNI_BAD_ID;
+    if (X->shape.empty()) { set_error(MNI_ERR_INVALID, "residual_layernorm: x must have at least one dim"); return MNI_BAD_ID; }
+    const Shape shape = X->shape;
+    const int64_t c = shape.back(), rows = c ? X->size / c : 0;
+    if (R->size < X->size) { set_error(MNI_ERR_INVALID, "residual_layernorm: residual holds fewer values than x"); return MNI_BAD_ID; }
+    if (Gm->size < c || Bt->size < c) { set_error(MNI_ERR_INVALID, "residual_layernorm: gamma / beta hold fewer than %lld values", (long long)c); return MNI_BAD_ID; }
+    BufP xs = contiguous_buf(*X), rs = contiguous_buf(*R), gs = contiguous_buf(*Gm), bs = contiguous_buf(*Bt);
+    BufP out = (xs && rs && gs && bs) ? new_buf((size_t)X->size) : nullptr;
+    BufP res = out ? new_buf((size_t)X->size) : nullptr;
+    BufP mean = res ? new_buf((size_t)rows) : nullptr, rstd = mean ? new_buf((size_t)rows) : nullptr;
+    if (!rstd || k_residual_layernorm(out->p, res->p, mean->p, rstd->p, xs->p, rs->p, gs->p, bs->p, rows, c, eps) != MNI_OK)
+        return MNI_BAD_ID;
+    // ids are handed out in the reference's order: res, mean, rstd, out
+    const uint32_t res_id = insert_contig(std::move(res), shape);
+    const uint32_t mean_id = insert_contig(std::move(mean), Shape{rows});
+    const uint32_t rstd_id = insert_contig(std::move(rstd), Shape{rows});
+    const uint32_t out_id = insert_contig(std::move(out), shape);
+    Entry e;
+    e.op = OP_RESIDUALLAYERNORM; e.output_id = out_id; e.n_inputs = 4;
+    e.inputs[0] = x; e.inputs[1] = residual; e.inputs[2] = gamma; e.inputs[3] = beta;
+    e.aux = mean_id; e.aux2 = rstd_id; e.aux3 = res_id;
+    eng().tape.record(std::move(e));
+    return out_id;
+}
+// The same tensor is returned for x and for the residual, as the reference does.
+static int residual_layernorm_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *S = get(e.aux3), *Gm = get(e.inputs[2]), *Mn = get(e.aux), *Rs = get(e.aux2), *G = get(grad);
+    if (!S || !Gm || !Mn || !Rs || !G) return MNI_ERR_FREED;
+    const Shape shape = S->shape, gshape = Gm->shape;
+    const int64_t c = shape.back(), rows = c ? S->size / c : 0;
+    BufP gs = contiguous_buf(*Gm), g = contiguous_buf(*G);
+    BufP dx = (gs && g) ? new_buf((size_t)S->size) : nullptr;
+    BufP dgamma = dx ? new_buf((size_t)Gm->size) : nullptr, dbeta = dgamma ? new_buf((size_t)Gm->size) : nullptr;
+    if (!dbeta) return MNI_ERR_NOMEM;
+    if (Gm->size > c) { MNI_TRY(k_fill(dgamma->p, 0.0f, Gm->size)); MNI_TRY(k_fill(dbeta->p, 0.0f, Gm->size)); }
+    MNI_TRY(k_layernorm_backward(dx->p, dgamma->p, dbeta->p, g->p, S->buf->p, gs->p, Mn->buf->p, Rs->buf->p, rows, c));
+    out[0] = out[1] = insert_contig(std::move(dx), shape);
+    out[2] = insert_contig(std::move(dgamma), gshape);
+    out[3] = insert_contig(std::move(dbeta), gshape);
+    return MNI_OK;
+}
+
+// ops/mixed_precision.rs:17-32: grads *= inv_scale, true when any scaled value is inf or NaN
+static int scale_grads_checked(const uint32_t *ids, size_t n, float inv_scale, int *found) {
+    BufP flag = new_buf(1);
+    if (!flag) return MNI_ERR_NOMEM;
+    MNI_TRY(k_fill(flag->p, 0.0f, 1));
+    for (size_t p = 0; p < n; ++p) {
+        Tensor *T = get(ids[p]);
+        if (!T) return MNI_ERR_FREED;
+        if (T->grad < 0) continue;
+        Tensor *G = get((uint32_t)T->grad);
+        if (!G) return MNI_ERR_FREED;
+        MNI_TRY(make_unique(*G));
+        MNI_TRY(k_scale_check(G->buf->p, inv_scale, (int64_t)G->buf->n, flag->p));
+    }
+    float f = 0.f;
+    MNI_TRY(mni_rocm_d2h(&f, flag->p, sizeof(float)));
+    *found = f != 0.0f;
+    return MNI_OK;
+}
+
 // ---- backward --------------------------------------------------------------------------------
 static int dispatch_backward(const Entry &e, uint32_t grad, int64_t *out) {  // autograd.rs:180-222
-    out[0] = out[1] = out[2] = -1;
+    out[0] = out[1] = out[2] = out[3] = -1;
     switch (e.op) {
     case OP_ADD: return addsub_backward(grad, e, out, false);
     case OP_SUB: return addsub_backward(grad, e, out, true);
@@ -1277,6 +1626,9 @@ static int dispatch_backward(const Entry &e, uint32_t grad, int64_t *out) {  // 
     case OP_BIASGELU: return bias_gelu_backward(grad, e, out);               // autograd.rs BiasGelu
     case OP_SOFTMAX: return softmax_backward(grad, e, out);                  // autograd.rs:204
     case OP_FLASHATTENTION: return flash_attention_backward(grad, e, out);   // autograd.rs:210
+    case OP_EMBEDDING: return embedding_backward(grad, e, out);
+    case OP_DROPOUT: return dropout_backward(grad, e, out);
+    case OP_RESIDUALLAYERNORM: return residual_layernorm_backward(grad, e, out);
     }
     return set_error(MNI_ERR_INVALID, "unknown tape op %d", e.op);
 }
@@ -1344,7 +1696,7 @@ static int tape_backward(Tape &tp, uint32_t loss) {
         const int64_t idx = out2entry[tid];
         if (idx < 0) continue;
         const Entry &en = tp.entries[idx];
-        int64_t ig[3];
+        int64_t ig[4];
         MNI_TRY(dispatch_backward(en, (uint32_t)grads[tid], ig));
         for (int i = 0; i < en.n_inputs; ++i) {
             if (ig[i] < 0) continue;
@@ -1667,6 +2019,7 @@ double mni_grad_norm(const uint32_t *ids, size_t n) {
     return (double)norm;
 }
 int mni_clip_grad_norm(const uint32_t *ids, size_t n, double max_norm) {  // optimizer.rs:160-173
+    MNI_API_GUARD;
     float norm = 0.f;
     MNI_TRY(grad_norm(ids, n, &norm));
     const float mx = (float)max_norm;
@@ -1675,6 +2028,7 @@ int mni_clip_grad_norm(const uint32_t *ids, size_t n, double max_norm) {  // opt
 }
 double mni_clip_and_step(const uint32_t *ids, size_t n, double lr, double beta1, double beta2, double eps,
                          double weight_decay, int64_t step, double max_grad_norm) {  // optimizer.rs:224-245
+    MNI_API_GUARD;
     float norm = 0.f;
     if (grad_norm(ids, n, &norm) != MNI_OK) return -1.0;
     const float mg = (float)max_grad_norm;
@@ -1692,6 +2046,8 @@ void mni_reset_engine(void) {
     e.tape = Tape();
     e.kv_caches.clear();       // lib.rs:466-467
     e.next_kv_cache_id = 1;
+    e.int_bufs.clear();        // lib.rs:465
+    e.int_free.clear();
 }
 int mni_gc_tensors(const uint32_t *keep, size_t n) {
     MNI_API_GUARD;
@@ -1709,6 +2065,100 @@ int mni_gc_tensors(const uint32_t *keep, size_t n) {
     if (dev_cached_bytes() > ((size_t)64 << 30)) return dev_clear_cache();
     return MNI_OK;
 }
+// ---- token-side ops ------------------------------------------------------------------------
+uint32_t mni_rand_tensor(const int64_t *shape, int ndim) {  // lib.rs:60-64
+    MNI_API_GUARD;
+    Shape s;
+    if (ensure_init() != MNI_OK || !to_shape(shape, ndim, &s)) return MNI_BAD_ID;
+    return random_tensor(s, 0);
+}
+uint32_t mni_randn_tensor(const int64_t *shape, int ndim) {  // lib.rs:67-71
+    MNI_API_GUARD;
+    Shape s;
+    if (ensure_init() != MNI_OK || !to_shape(shape, ndim, &s)) return MNI_BAD_ID;
+    return random_tensor(s, 1);
+}
+int mni_seed(uint64_t seed) {
+    MNI_API_GUARD;
+    Engine &e = eng();
+    e.rng_seed = seed;
+    e.rng_offset = 0;
+    e.host_rng.seed(seed);
+    e.rng_ready = true;
+    return MNI_OK;
+}
+int mni_philox_words(uint64_t seed, uint64_t offset, uint32_t *out, size_t n) {
+    MNI_API_GUARD;
+    MNI_TRY(ensure_init());
+    BufP b = new_buf(n);
+    if (!b) return MNI_ERR_NOMEM;
+    MNI_TRY(k_random_fill(b->p, (int64_t)n, seed, offset, 2));
+    return mni_rocm_d2h(out, b->p, n * sizeof(uint32_t));
+}
+uint32_t mni_dropout_op(uint32_t x, double rate, int training) {  // lib.rs:388-394
+    MNI_API_GUARD;
+    return dropout_op(x, (float)rate, training != 0);
+}
+uint32_t mni_create_dataset(const int32_t *data, size_t len) {  // lib.rs:476-479
+    MNI_API_GUARD;
+    if (ensure_init() != MNI_OK) return MNI_BAD_ID;
+    if (len && !data) { set_error(MNI_ERR_INVALID, "create_dataset: null data"); return MNI_BAD_ID; }
+    return create_dataset(data, len);
+}
+int mni_sample_batch(uint32_t dataset, int64_t block_size, int64_t batch_size, uint32_t *out_ids) {  // lib.rs:483-490
+    MNI_API_GUARD;
+    return sample_batch(dataset, block_size, batch_size, out_ids);
+}
+int mni_free_int_buffer(uint32_t id) {  // lib.rs:494-497, data.rs:53-56
+    MNI_API_GUARD;
+    Engine &e = eng();
+    if (id >= e.int_bufs.size()) return set_error(MNI_ERR_INVALID, "int buffer id %u out of range", id);
+    e.int_bufs[id] = IntBuf();
+    e.int_free.push_back(id);
+    return MNI_OK;
+}
+int64_t mni_int_buffer_len(uint32_t id) {
+    MNI_API_GUARD;
+    IntBuf *b = get_int(id);
+    return b ? b->len : -1;
+}
+int mni_int_buffer_to_host(uint32_t id, int32_t *out, size_t cap) {
+    MNI_API_GUARD;
+    IntBuf *b = get_int(id);
+    if (!b) return MNI_ERR_FREED;
+    if ((int64_t)cap < b->len) return set_error(MNI_ERR_INVALID, "int_buffer_to_host: room for %zu of %lld values", cap, (long long)b->len);
+    return b->len ? mni_rocm_d2h(out, b->data.get(), (size_t)b->len * sizeof(int32_t)) : MNI_OK;
+}
+uint32_t mni_embedding_forward(uint32_t weight, const int64_t *indices, size_t n, int64_t batch, int64_t seq_len) {  // lib.rs:319-326
+    MNI_API_GUARD;
+    if (n && !indices) { set_error(MNI_ERR_INVALID, "embedding: null indices"); return MNI_BAD_ID; }
+    return embedding_forward(weight, indices, n, batch, seq_len);
+}
+uint32_t mni_embedding_forward_gpu(uint32_t weight, uint32_t int_buf, int64_t batch, int64_t seq_len) {  // lib.rs:501-511
+    MNI_API_GUARD;
+    return embedding_forward_gpu(weight, int_buf, batch, seq_len);
+}
+uint32_t mni_cross_entropy_loss_gpu(uint32_t logits, uint32_t int_buf) {  // lib.rs:679-691
+    MNI_API_GUARD;
+    return cross_entropy_gpu_op(logits, int_buf);
+}
+uint32_t mni_residual_layernorm(uint32_t x, uint32_t residual, uint32_t gamma, uint32_t beta, double eps) {  // lib.rs:515-523
+    MNI_API_GUARD;
+    return residual_layernorm_op(x, residual, gamma, beta, (float)eps);
+}
+int mni_scale_grads(const uint32_t *ids, size_t n, double inv_scale, int *found_inf) {  // lib.rs:450-454
+    MNI_API_GUARD;
+    int found = 0;
+    MNI_TRY(scale_grads_checked(ids, n, (float)inv_scale, &found));
+    if (found_inf) *found_inf = found;
+    return MNI_OK;
+}
+uint32_t mni_tile(uint32_t input, const int64_t *reps, int n) {  // lib.rs:568-573
+    MNI_API_GUARD;
+    if (n > 0 && !reps) { set_error(MNI_ERR_INVALID, "tile: null reps"); return MNI_BAD_ID; }
+    return tile_op(input, reps, n);
+}
+
 void *mni_dev_ptr(uint32_t id) {
     MNI_API_GUARD;
     Tensor *t = get(id);

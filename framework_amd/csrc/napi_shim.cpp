@@ -322,6 +322,91 @@ napi_value Linear(napi_env env, napi_callback_info info) {
     return ret_id(env, mni_linear(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_u32(env, a.v[2]), act));
 }
 
+FROM_SHAPE(RandTensor, mni_rand_tensor)    // lib.rs:60-64
+FROM_SHAPE(RandnTensor, mni_randn_tensor)  // lib.rs:67-71
+WITH_SHAPE(Tile, mni_tile)                 // lib.rs:568-573
+BINARY(CrossEntropyLossGpu, mni_cross_entropy_loss_gpu)  // lib.rs:679-691
+napi_value Seed(napi_env env, napi_callback_info info) {  // no counterpart in the reference: fixes the random stream
+    Args a(env, info);
+    return ret_rc(env, mni_seed((uint64_t)get_f64(env, a.v[0])));
+}
+napi_value PhiloxWords(napi_env env, napi_callback_info info) {  // no counterpart: the raw generator, for known-answer checks
+    Args a(env, info);
+    const size_t n = (size_t)get_i64(env, a.v[2]);
+    napi_value ab, out;
+    void *data = nullptr;
+    napi_create_arraybuffer(env, n * sizeof(uint32_t), &data, &ab);
+    if (mni_philox_words((uint64_t)get_f64(env, a.v[0]), (uint64_t)get_f64(env, a.v[1]), (uint32_t *)data, n) != MNI_OK)
+        return throw_last(env);
+    napi_create_typedarray(env, napi_uint32_array, n, ab, 0, &out);
+    return out;
+}
+napi_value DropoutOp(napi_env env, napi_callback_info info) {  // lib.rs:388-394
+    Args a(env, info);
+    return ret_id(env, mni_dropout_op(get_u32(env, a.v[0]), get_f64(env, a.v[1]), get_bool(env, a.v[2]) ? 1 : 0));
+}
+napi_value CreateDataset(napi_env env, napi_callback_info info) {  // lib.rs:476-479
+    Args a(env, info);
+    napi_typedarray_type type;
+    size_t len = 0, off = 0;
+    void *data = nullptr;
+    napi_value ab;
+    if (napi_get_typedarray_info(env, a.v[0], &type, &len, &data, &ab, &off) != napi_ok || type != napi_int32_array) {
+        napi_throw_type_error(env, nullptr, "createDataset expects an Int32Array");
+        return nullptr;
+    }
+    return ret_id(env, mni_create_dataset((const int32_t *)data, len));
+}
+napi_value SampleBatch(napi_env env, napi_callback_info info) {  // lib.rs:483-490
+    Args a(env, info);
+    uint32_t ids[2] = {0, 0};
+    if (mni_sample_batch(get_u32(env, a.v[0]), get_i64(env, a.v[1]), get_i64(env, a.v[2]), ids) != MNI_OK) return throw_last(env);
+    napi_value arr;
+    napi_create_array_with_length(env, 2, &arr);
+    napi_set_element(env, arr, 0, make_u32(env, ids[0]));
+    napi_set_element(env, arr, 1, make_u32(env, ids[1]));
+    return arr;
+}
+napi_value FreeIntBuffer(napi_env env, napi_callback_info info) {  // lib.rs:494-497
+    Args a(env, info);
+    return ret_rc(env, mni_free_int_buffer(get_u32(env, a.v[0])));
+}
+napi_value IntBufferToInt32(napi_env env, napi_callback_info info) {  // no counterpart in the reference: reads a buffer back
+    Args a(env, info);
+    const uint32_t id = get_u32(env, a.v[0]);
+    const int64_t n = mni_int_buffer_len(id);
+    if (n < 0) return throw_last(env);
+    napi_value ab, out;
+    void *data = nullptr;
+    napi_create_arraybuffer(env, (size_t)n * sizeof(int32_t), &data, &ab);
+    if (mni_int_buffer_to_host(id, (int32_t *)data, (size_t)n) != MNI_OK) return throw_last(env);
+    napi_create_typedarray(env, napi_int32_array, (size_t)n, ab, 0, &out);
+    return out;
+}
+napi_value EmbeddingForward(napi_env env, napi_callback_info info) {  // lib.rs:319-326
+    Args a(env, info);
+    std::vector<int64_t> idx = get_i64_array(env, a.v[1]);
+    return ret_id(env, mni_embedding_forward(get_u32(env, a.v[0]), idx.data(), idx.size(), get_i64(env, a.v[2]), get_i64(env, a.v[3])));
+}
+napi_value EmbeddingForwardGpu(napi_env env, napi_callback_info info) {  // lib.rs:501-511
+    Args a(env, info);
+    return ret_id(env, mni_embedding_forward_gpu(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_i64(env, a.v[2]), get_i64(env, a.v[3])));
+}
+napi_value ResidualLayernorm(napi_env env, napi_callback_info info) {  // lib.rs:515-523
+    Args a(env, info);
+    return ret_id(env, mni_residual_layernorm(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_u32(env, a.v[2]), get_u32(env, a.v[3]),
+                                              get_f64(env, a.v[4])));
+}
+napi_value ScaleGrads(napi_env env, napi_callback_info info) {  // lib.rs:450-454
+    Args a(env, info);
+    std::vector<uint32_t> ids = get_u32_array(env, a.v[0]);
+    int found = 0;
+    if (mni_scale_grads(ids.data(), ids.size(), get_f64(env, a.v[1]), &found) != MNI_OK) return throw_last(env);
+    napi_value v;
+    napi_get_boolean(env, found != 0, &v);
+    return v;
+}
+
 }  // namespace
 
 NAPI_MODULE_INIT() {
@@ -345,6 +430,12 @@ NAPI_MODULE_INIT() {
         EXPORT("kvCacheCreate", KvCacheCreate), EXPORT("kvCacheLen", KvCacheLen), EXPORT("kvCacheQuantized", KvCacheQuantized),
         EXPORT("kvCacheReset", KvCacheReset), EXPORT("kvCacheFree", KvCacheFree), EXPORT("kvCacheAppend", KvCacheAppend),
         EXPORT("kvCacheDecodeStep", KvCacheDecodeStep), EXPORT("flashAttention", FlashAttention),
+        EXPORT("randTensor", RandTensor), EXPORT("randnTensor", RandnTensor), EXPORT("seed", Seed), EXPORT("philoxWords", PhiloxWords), EXPORT("tile", Tile),
+        EXPORT("dropoutOp", DropoutOp), EXPORT("createDataset", CreateDataset), EXPORT("sampleBatch", SampleBatch),
+        EXPORT("freeIntBuffer", FreeIntBuffer), EXPORT("intBufferToInt32", IntBufferToInt32),
+        EXPORT("embeddingForward", EmbeddingForward), EXPORT("embeddingForwardGpu", EmbeddingForwardGpu),
+        EXPORT("crossEntropyLossGpu", CrossEntropyLossGpu), EXPORT("residualLayernorm", ResidualLayernorm),
+        EXPORT("scaleGrads", ScaleGrads),
 #undef EXPORT
     };
     napi_define_properties(env, exports, sizeof(props) / sizeof(props[0]), props);

@@ -114,6 +114,21 @@ SIGNATURES = {
     "mni_max_op": (C.c_uint32, [C.c_uint32, C.c_int64]),
     "mni_layernorm_op": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double]),
     "mni_flash_attention": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_double, C.c_int]),
+    "mni_rand_tensor": (C.c_uint32, [_i64p, C.c_int]), "mni_randn_tensor": (C.c_uint32, [_i64p, C.c_int]),
+    "mni_seed": (C.c_int, [C.c_uint64]),
+    "mni_philox_words": (C.c_int, [C.c_uint64, C.c_uint64, C.c_void_p, C.c_size_t]),
+    "mni_dropout_op": (C.c_uint32, [C.c_uint32, C.c_double, C.c_int]),
+    "mni_create_dataset": (C.c_uint32, [C.c_void_p, C.c_size_t]),
+    "mni_sample_batch": (C.c_int, [C.c_uint32, C.c_int64, C.c_int64, _u32p]),
+    "mni_free_int_buffer": (C.c_int, [C.c_uint32]),
+    "mni_int_buffer_len": (C.c_int64, [C.c_uint32]),
+    "mni_int_buffer_to_host": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t]),
+    "mni_embedding_forward": (C.c_uint32, [C.c_uint32, _i64p, C.c_size_t, C.c_int64, C.c_int64]),
+    "mni_embedding_forward_gpu": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_int64, C.c_int64]),
+    "mni_cross_entropy_loss_gpu": (C.c_uint32, [C.c_uint32, C.c_uint32]),
+    "mni_residual_layernorm": (C.c_uint32, [C.c_uint32] * 4 + [C.c_double]),
+    "mni_scale_grads": (C.c_int, [_u32p, C.c_size_t, C.c_double, C.POINTER(C.c_int)]),
+    "mni_tile": (C.c_uint32, [C.c_uint32, _i64p, C.c_int]),
     "mni_cross_entropy_loss": (C.c_uint32, [C.c_uint32, _i64p, C.c_size_t]),
     "mni_adamw_step": (C.c_int, [_u32p, C.c_size_t, C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, C.c_int64]),
     "mni_grad_norm": (C.c_double, [_u32p, C.c_size_t]),
@@ -462,6 +477,64 @@ class Native:
 
     def crossEntropyLoss(self, logits, targets):
         return self._id(self.lib.mni_cross_entropy_loss(logits, _i64_array(targets), len(targets)))
+
+    # token-side ops
+    def randTensor(self, shape):
+        return self._id(self.lib.mni_rand_tensor(_i64_array(shape), len(shape)))
+
+    def randnTensor(self, shape):
+        return self._id(self.lib.mni_randn_tensor(_i64_array(shape), len(shape)))
+
+    def seed(self, seed):
+        self._rc(self.lib.mni_seed(seed))
+
+    def philoxWords(self, seed, offset, n):
+        out = np.empty(n, dtype=np.uint32)
+        self._rc(self.lib.mni_philox_words(seed, offset, out.ctypes.data, n))
+        return out
+
+    def dropoutOp(self, x, rate, training):
+        return self._id(self.lib.mni_dropout_op(x, rate, 1 if training else 0))
+
+    def createDataset(self, data):
+        a = np.ascontiguousarray(data, dtype=np.int32)
+        return self._id(self.lib.mni_create_dataset(a.ctypes.data, a.size))
+
+    def sampleBatch(self, datasetId, blockSize, batchSize):
+        out = (C.c_uint32 * 2)()
+        self._rc(self.lib.mni_sample_batch(datasetId, blockSize, batchSize, out))
+        return [int(out[0]), int(out[1])]
+
+    def freeIntBuffer(self, id):
+        self._rc(self.lib.mni_free_int_buffer(id))
+
+    def intBufferToHost(self, id):
+        n = self.lib.mni_int_buffer_len(id)
+        if n < 0:
+            raise self._err()
+        out = np.empty(n, dtype=np.int32)
+        self._rc(self.lib.mni_int_buffer_to_host(id, out.ctypes.data, n))
+        return out
+
+    def embeddingForward(self, weight, indices, batch, seqLen):
+        return self._id(self.lib.mni_embedding_forward(weight, _i64_array(indices), len(indices), batch, seqLen))
+
+    def embeddingForwardGpu(self, weight, intBufId, batch, seqLen):
+        return self._id(self.lib.mni_embedding_forward_gpu(weight, intBufId, batch, seqLen))
+
+    def crossEntropyLossGpu(self, logits, intBufId):
+        return self._id(self.lib.mni_cross_entropy_loss_gpu(logits, intBufId))
+
+    def residualLayernorm(self, x, residual, gamma, beta, eps):
+        return self._id(self.lib.mni_residual_layernorm(x, residual, gamma, beta, eps))
+
+    def scaleGrads(self, ids, invScale):
+        found = C.c_int(0)
+        self._rc(self.lib.mni_scale_grads(_u32_array(ids), len(ids), invScale, C.byref(found)))
+        return bool(found.value)
+
+    def tile(self, a, reps):
+        return self._id(self.lib.mni_tile(a, _i64_array(reps), len(reps)))
 
     # optimiser
     def adamwStep(self, ids, lr, beta1, beta2, eps, weight_decay, step):

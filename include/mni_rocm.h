@@ -207,6 +207,46 @@ uint32_t mni_gt(uint32_t a, uint32_t b);
 uint32_t mni_is_close(uint32_t a, uint32_t b, double tol);
 uint32_t mni_max_op(uint32_t a, int64_t dim);
 uint32_t mni_layernorm_op(uint32_t x, uint32_t gamma, uint32_t beta, double eps);
+/* Token side of a language-model step, device-resident.
+ * rand_tensor / randn_tensor (src/native/src/lib.rs:60-71 -> tensor.rs:228-250): uniform [0, 1) in steps
+ *   of 2^-24 and standard normal, drawn from a Philox4x32-10 stream on the device.  Like the reference's
+ *   thread RNG the stream is seeded from system entropy; mni_seed (no counterpart in the reference) fixes
+ *   it, and mni_philox_words exposes the raw generator (word i of the result is word i % 4 of block
+ *   offset + i / 4 under key `seed`) so that it can be checked against the published test vectors.
+ * dropout_op (lib.rs:388-394 -> ops/dropout.rs:25-58, backward :114-126): returns x itself when not
+ *   training or rate == 0; else x * mask * 1/(1-rate) with mask = (u >= rate).  The mask is regenerated
+ *   from the stream position in the backward instead of being stored.
+ * create_dataset / sample_batch / free_int_buffer (lib.rs:476-497 -> ops/data.rs): int32 buffers in their
+ *   own id space (LIFO recycling); sample_batch writes the ids of the inputs and targets buffers
+ *   ([batch_size, block_size] windows at uniform starts in [0, len - block_size - 1), targets shifted by
+ *   one) to out_ids[0..1].  mni_int_buffer_len / _to_host have no counterpart (the reference never reads
+ *   these buffers back); they exist for tests and debugging.
+ * embedding_forward (lib.rs:319-326 -> ops/embedding.rs:25-53) and embedding_forward_gpu (:501-511):
+ *   out[b, t, :] = weight[index[b, t], :]; backward (:104-128) adds the gradient rows of equal indices
+ *   in token order, on the device, deterministically.  Indices outside the table are an error.
+ * cross_entropy_loss_gpu (lib.rs:679-691 -> ops/loss.rs:190-229): logits viewed as [rows, classes],
+ *   targets taken from an int buffer.
+ * residual_layernorm (lib.rs:515-523 -> ops/fused.rs:23-78, backward :134-186): layernorm(x + residual)
+ *   in one pass; x and residual receive the same gradient tensor.
+ * scale_grads (lib.rs:450-454 -> ops/mixed_precision.rs:17-32): grads *= inv_scale; *found_inf = 1 when
+ *   any scaled value is infinite or NaN.
+ * tile (lib.rs:568-573 -> ops/pooling.rs:276-309): repeat along every dim; not differentiable. */
+uint32_t mni_rand_tensor(const int64_t *shape, int ndim);
+uint32_t mni_randn_tensor(const int64_t *shape, int ndim);
+int mni_seed(uint64_t seed);
+int mni_philox_words(uint64_t seed, uint64_t offset, uint32_t *out, size_t n);
+uint32_t mni_dropout_op(uint32_t x, double rate, int training);
+uint32_t mni_create_dataset(const int32_t *data, size_t len);
+int mni_sample_batch(uint32_t dataset, int64_t block_size, int64_t batch_size, uint32_t *out_ids);
+int mni_free_int_buffer(uint32_t id);
+int64_t mni_int_buffer_len(uint32_t id); /* < 0 on error */
+int mni_int_buffer_to_host(uint32_t id, int32_t *out, size_t cap);
+uint32_t mni_embedding_forward(uint32_t weight, const int64_t *indices, size_t n, int64_t batch, int64_t seq_len);
+uint32_t mni_embedding_forward_gpu(uint32_t weight, uint32_t int_buf, int64_t batch, int64_t seq_len);
+uint32_t mni_cross_entropy_loss_gpu(uint32_t logits, uint32_t int_buf);
+uint32_t mni_residual_layernorm(uint32_t x, uint32_t residual, uint32_t gamma, uint32_t beta, double eps);
+int mni_scale_grads(const uint32_t *ids, size_t n, double inv_scale, int *found_inf);
+uint32_t mni_tile(uint32_t input, const int64_t *reps, int n);
 /* bias_gelu (src/native/src/lib.rs:526-531 -> ops/fused.rs:247-273, backward :316-351):
  * out = gelu(x + bias) along the last extent; backward yields dx and the column sums dbias in one pass. */
 uint32_t mni_bias_gelu(uint32_t x, uint32_t bias);

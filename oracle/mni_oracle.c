@@ -53,16 +53,17 @@ enum orc_op { /* subset of autograd.rs:28-62 BackwardOp */
     OP_ADD, OP_MUL, OP_SUB, OP_NEG, OP_MULSCALAR, OP_MATMUL, OP_GELU, OP_RELU,
     OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY,
     OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU,
-    OP_EXP, OP_LOG, OP_DIV, OP_SIGMOID, OP_POW, OP_MAX, OP_LAYERNORM
+    OP_EXP, OP_LOG, OP_DIV, OP_SIGMOID, OP_POW, OP_MAX, OP_LAYERNORM,
+    OP_EMBEDDING, OP_DROPOUT, OP_RESIDUALLAYERNORM
 };
 
 /* autograd.rs:65-70 TapeEntry + the SavedContext variants the subset needs */
 typedef struct {
     int op;
     size_t output_id;
-    size_t input_ids[3];
+    size_t input_ids[4];
     int n_inputs;
-    size_t saved_ids[3];          /* Tensor / Tensors / TensorsAndShape ids  */
+    size_t saved_ids[4];          /* Tensor / Tensors / TensorsAndShape ids  */
     size_t saved_shape[ORC_MAX_DIMS]; /* Shape / TensorAndShape / Permutation orig */
     int saved_ndim;
     size_t saved_perm[ORC_MAX_DIMS];
@@ -71,6 +72,8 @@ typedef struct {
     size_t ce_n, ce_v, ce_sm;
     size_t fa_out, fa_lse;        /* FlashAttention{q,k,v,out,lse,scale,s,d,causal} */
     int fa_causal;
+    size_t emb_batch, emb_seq;    /* Indices(indices, batch, seq_len, weight) */
+    size_t drop_mask;             /* DropoutMask(mask_id, rate): rate in saved_scalar */
 } orc_entry;
 
 typedef struct {
@@ -1303,11 +1306,381 @@ static int flash_attention_backward(size_t grad, const orc_entry *e, long *out) 
     return 0;
 }
 
+/* ---- token-side ops: random numbers, dropout, datasets, embedding, tile, residual layernorm ---- */
+
+/* Philox4x32-10 (Salmon, Moraes, Dror, Shaw, SC'11), the generator the HIP
+ * backend draws rand / randn / dropout masks from.  The reference draws from
+ * rand 0.8's unseedable thread RNG (tensor.rs:228-250, dropout.rs:37-44), so
+ * no stream can match it; what its consumers rely on is the distribution
+ * (uniform on multiples of 2^-24 in [0, 1); standard normal).
+ * pinned by: the known-answer vectors published with the generator
+ * (Random123 kat_vectors), moments of the outputs. */
+static void philox4x32_10(uint64_t counter, uint64_t seed, uint32_t out[4]) {
+    uint32_t c0 = (uint32_t)counter, c1 = (uint32_t)(counter >> 32), c2 = 0, c3 = 0;
+    uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+/* the general form (4-word counter, 2-word key) for the published vectors */
+void orc_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; ++r) {
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+        uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+void orc_philox_words(uint64_t seed, uint64_t offset, uint32_t *out, size_t n) {
+    for (size_t i = 0; i < n; i += 4) {
+        uint32_t w[4];
+        philox4x32_10(offset + i / 4, seed, w);
+        for (size_t j = 0; j < 4 && i + j < n; ++j) out[i + j] = w[j];
+    }
+}
+static float u01(uint32_t w) { return (float)(w >> 8) * 5.9604644775390625e-8f; }
+static uint64_t g_rng_seed = 0, g_rng_offset = 0;
+void orc_seed(uint64_t seed) { g_rng_seed = seed; g_rng_offset = 0; }
+static uint64_t rng_take(size_t n) {
+    uint64_t at = g_rng_offset;
+    g_rng_offset += (n + 3) / 4;
+    return at;
+}
+/* mode 0: uniform [0, 1) (tensor.rs:228-238); 1: standard normal by Box-Muller (tensor.rs:240-250) */
+static uint32_t random_tensor(const size_t *shape, int nd, int mode) {
+    size_t n = shape_size(shape, nd);
+    float *d = (float *)malloc((n + 4) * sizeof(float));
+    uint64_t at = rng_take(n);
+    for (size_t i = 0; i < n; i += 4) {
+        uint32_t w[4];
+        float v[4];
+        philox4x32_10(at + i / 4, g_rng_seed, w);
+        if (mode == 0) {
+            for (int j = 0; j < 4; ++j) v[j] = u01(w[j]);
+        } else {
+            for (int j = 0; j < 4; j += 2) {
+                float u1 = (float)((w[j] >> 8) + 1u) * 5.9604644775390625e-8f, u2 = u01(w[j + 1]);
+                float r = sqrtf(-2.0f * logf(u1)), a = 6.283185307179586f * u2;
+                v[j] = r * cosf(a);
+                v[j + 1] = r * sinf(a);
+            }
+        }
+        for (size_t j = 0; j < 4 && i + j < n; ++j) d[i + j] = v[j];
+    }
+    return (uint32_t)from_vec(d, shape, nd);
+}
+
+/* ops/dropout.rs:25-58 dropout_forward, cpu arm: the input id itself when not
+ * training or rate == 0; else mask = (u >= rate), out = x * mask * scale with
+ * scale = 1 / (1 - rate), mask kept as a tensor.
+ * pinned by: out is 0 or x / (1 - rate) elementwise, kept fraction ~ 1 - rate,
+ * backward equals forward applied to the gradient with the same mask. */
+static uint32_t dropout_impl(size_t x, float rate, int training) {
+    orc_tensor *X = get(x);
+    if (!X) return fail("tensor already freed");
+    if (!training || rate == 0.0f) return (uint32_t)x;
+    float *xd = to_host(X);
+    size_t shape[ORC_MAX_DIMS]; int nd = X->ndim;
+    memcpy(shape, X->shape, sizeof shape);
+    size_t size = X->size;
+    float scale = 1.0f / (1.0f - rate);
+    float *mask = (float *)malloc((size + 4) * sizeof(float)), *out = (float *)malloc((size + 4) * sizeof(float));
+    uint64_t at = rng_take(size);
+    for (size_t i = 0; i < size; i += 4) {
+        uint32_t w[4];
+        philox4x32_10(at + i / 4, g_rng_seed, w);
+        for (size_t j = 0; j < 4 && i + j < size; ++j) {
+            mask[i + j] = u01(w[j]) >= rate ? 1.0f : 0.0f;
+            out[i + j] = xd[i + j] * mask[i + j] * scale;
+        }
+    }
+    free(xd);
+    size_t mask_id = from_vec(mask, shape, nd);
+    size_t out_id = from_vec(out, shape, nd);
+    orc_entry *e = tape_record(&g_tape, OP_DROPOUT, out_id, 1, x, 0);
+    e->drop_mask = mask_id; e->saved_scalar = rate;
+    return (uint32_t)out_id;
+}
+/* ops/dropout.rs:114-126 */
+static int dropout_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *G = get(grad), *M = get(e->drop_mask);
+    if (!G || !M) { fail("tensor already freed"); return -1; }
+    float *gd = to_host(G), *md = to_host(M);
+    size_t shape[ORC_MAX_DIMS]; int nd = G->ndim;
+    memcpy(shape, G->shape, sizeof shape);
+    float scale = 1.0f / (1.0f - e->saved_scalar);
+    size_t n = G->size;
+    float *o = (float *)malloc((n ? n : 1) * sizeof(float));
+    for (size_t i = 0; i < n; ++i) o[i] = gd[i] * md[i] * scale;
+    free(gd); free(md);
+    out[0] = (long)from_vec(o, shape, nd);
+    return 0;
+}
+
+/* ops/data.rs:13-56 IntBuffer / IntStore (cpu arm: host vectors, LIFO id recycling) */
+typedef struct { int live; int32_t *data; size_t len; } orc_intbuf;
+static orc_intbuf *g_int;
+static size_t g_int_len, g_int_cap, *g_int_free, g_int_nfree, g_int_capfree;
+static size_t int_insert(int32_t *data, size_t len) {
+    if (g_int_nfree) {
+        size_t id = g_int_free[--g_int_nfree];
+        g_int[id].live = 1; g_int[id].data = data; g_int[id].len = len;
+        return id;
+    }
+    if (g_int_len == g_int_cap) {
+        g_int_cap = g_int_cap ? g_int_cap * 2 : 16;
+        g_int = (orc_intbuf *)realloc(g_int, g_int_cap * sizeof(orc_intbuf));
+    }
+    g_int[g_int_len].live = 1; g_int[g_int_len].data = data; g_int[g_int_len].len = len;
+    return g_int_len++;
+}
+static orc_intbuf *int_get(size_t id) {
+    if (id >= g_int_len || !g_int[id].live) { fail("int buffer already freed"); return NULL; }
+    return &g_int[id];
+}
+static void int_clear(void) {
+    for (size_t i = 0; i < g_int_len; ++i) if (g_int[i].live) free(g_int[i].data);
+    free(g_int); free(g_int_free);
+    g_int = NULL; g_int_free = NULL; g_int_len = g_int_cap = g_int_nfree = g_int_capfree = 0;
+}
+uint32_t orc_create_dataset(const int32_t *data, size_t len) { /* lib.rs:476-479, data.rs:59-66 */
+    int32_t *d = (int32_t *)malloc((len ? len : 1) * sizeof(int32_t));
+    memcpy(d, data, len * sizeof(int32_t));
+    return (uint32_t)int_insert(d, len);
+}
+void orc_free_int_buffer(uint32_t id) { /* lib.rs:494-497, data.rs:53-56 */
+    if (id >= g_int_len) return;
+    if (g_int[id].live) free(g_int[id].data);
+    g_int[id].live = 0; g_int[id].data = NULL;
+    if (g_int_nfree == g_int_capfree) {
+        g_int_capfree = g_int_capfree ? g_int_capfree * 2 : 16;
+        g_int_free = (size_t *)realloc(g_int_free, g_int_capfree * sizeof(size_t));
+    }
+    g_int_free[g_int_nfree++] = id;
+}
+int64_t orc_int_buffer_len(uint32_t id) { orc_intbuf *b = int_get(id); return b ? (int64_t)b->len : -1; }
+int orc_int_buffer_to_host(uint32_t id, int32_t *out, size_t cap) {
+    orc_intbuf *b = int_get(id);
+    if (!b || cap < b->len) return -1;
+    memcpy(out, b->data, b->len * sizeof(int32_t));
+    return 0;
+}
+/* ops/data.rs:79-109 sample_batch, cpu arm, with the window starts supplied by
+ * the caller in place of rng.gen_range(0..len - block_size - 1): inputs are
+ * data[start + t], targets data[start + t + 1].
+ * pinned by: windows of an arange dataset; range of valid starts. */
+int orc_sample_batch_at(uint32_t dataset, int64_t block, int64_t batch, const int64_t *starts, uint32_t *out_ids) {
+    orc_intbuf *ds = int_get(dataset);
+    if (!ds) return -1;
+    if (block <= 0 || batch <= 0 || (int64_t)ds->len - block - 1 <= 0) { fail("cannot sample empty range"); return -1; }
+    size_t total = (size_t)(batch * block);
+    int32_t *inp = (int32_t *)malloc(total * sizeof(int32_t)), *tgt = (int32_t *)malloc(total * sizeof(int32_t));
+    for (int64_t b = 0; b < batch; ++b) {
+        if (starts[b] < 0 || starts[b] >= (int64_t)ds->len - block - 1) { free(inp); free(tgt); fail("start outside the sampled range"); return -1; }
+        for (int64_t t = 0; t < block; ++t) {
+            inp[b * block + t] = ds->data[starts[b] + t];
+            tgt[b * block + t] = ds->data[starts[b] + t + 1];
+        }
+    }
+    out_ids[0] = (uint32_t)int_insert(inp, total);
+    out_ids[1] = (uint32_t)int_insert(tgt, total);
+    return 0;
+}
+
+/* ops/embedding.rs:25-53 embedding_forward, cpu arm
+ * pinned by: numpy fancy indexing; backward against np.add.at and, bitwise,
+ * a sequential float32 loop in token order. */
+static uint32_t embedding_impl(size_t weight, const size_t *indices, size_t batch, size_t seq_len) {
+    orc_tensor *W = get(weight);
+    if (!W) return fail("tensor already freed");
+    if (W->ndim < 2) return fail("index out of bounds: embedding weight needs 2 dims");
+    size_t dim = W->shape[1], rows = W->shape[0];
+    float *wd = to_host(W);
+    float *out = (float *)calloc((batch * seq_len * dim) > 0 ? batch * seq_len * dim : 1, sizeof(float));
+    for (size_t b = 0; b < batch; ++b)
+        for (size_t t = 0; t < seq_len; ++t) {
+            size_t idx = indices[b * seq_len + t];
+            if (idx >= rows) { free(wd); free(out); return fail("index out of bounds: embedding index"); }
+            memcpy(out + (b * seq_len + t) * dim, wd + idx * dim, dim * sizeof(float));
+        }
+    free(wd);
+    size_t shape[3] = {batch, seq_len, dim};
+    size_t out_id = from_vec(out, shape, 3);
+    orc_entry *e = tape_record(&g_tape, OP_EMBEDDING, out_id, 1, weight, 0);
+    if (g_tape.enabled) {
+        size_t n = batch * seq_len;
+        e->targets = (size_t *)malloc((n ? n : 1) * sizeof(size_t));
+        memcpy(e->targets, indices, n * sizeof(size_t));
+    }
+    e->emb_batch = batch; e->emb_seq = seq_len;
+    return (uint32_t)out_id;
+}
+/* ops/embedding.rs:104-128 embedding_backward: dw rows accumulate in token order */
+static int embedding_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *W = get(e->input_ids[0]), *G = get(grad);
+    if (!W || !G) { fail("tensor already freed"); return -1; }
+    size_t wshape[ORC_MAX_DIMS]; int wnd = W->ndim;
+    memcpy(wshape, W->shape, sizeof wshape);
+    size_t vocab = wshape[0], dim = wshape[1];
+    float *gd = to_host(G);
+    float *dw = (float *)calloc((vocab * dim) > 0 ? vocab * dim : 1, sizeof(float));
+    for (size_t b = 0; b < e->emb_batch; ++b)
+        for (size_t t = 0; t < e->emb_seq; ++t) {
+            size_t idx = e->targets[b * e->emb_seq + t];
+            const float *src = gd + (b * e->emb_seq + t) * dim;
+            float *dst = dw + idx * dim;
+            for (size_t j = 0; j < dim; ++j) dst[j] += src[j];
+        }
+    free(gd);
+    out[0] = (long)from_vec(dw, wshape, wnd);
+    return 0;
+}
+
+/* ops/pooling.rs:276-309 tile (nothing recorded on the tape)
+ * pinned by: numpy.tile. */
+static uint32_t tile_impl(size_t input, const size_t *reps, int nreps) {
+    orc_tensor *A = get(input);
+    if (!A) return fail("tensor already freed");
+    int nd = A->ndim;
+    if (nreps != nd) return fail("tile: reps must match tensor dimensions");
+    if (nd < 1) return fail("attempt to subtract with overflow: tile of a scalar");
+    size_t shape[ORC_MAX_DIMS], out_shape[ORC_MAX_DIMS], in_strides[ORC_MAX_DIMS], out_strides[ORC_MAX_DIMS];
+    memcpy(shape, A->shape, sizeof shape);
+    float *data = to_host(A);
+    for (int i = 0; i < nd; ++i) out_shape[i] = shape[i] * reps[i];
+    size_t out_size = shape_size(out_shape, nd);
+    int empty = 0;
+    for (int i = 0; i < nd; ++i) if (out_shape[i] == 0) empty = 1;
+    compute_strides(shape, nd, in_strides);
+    compute_strides(out_shape, nd, out_strides);
+    float *o = (float *)calloc(out_size ? out_size : 1, sizeof(float));
+    for (size_t i = 0; i < out_size && !empty; ++i) {
+        size_t src = 0, rem = i;
+        for (int d = 0; d < nd; ++d) {
+            size_t coord = rem / out_strides[d];
+            rem %= out_strides[d];
+            src += (coord % shape[d]) * in_strides[d];
+        }
+        o[i] = data[src];
+    }
+    free(data);
+    return (uint32_t)from_vec(o, out_shape, nd);
+}
+
+/* ops/fused.rs:23-78 residual_layernorm, cpu arm: res = x + residual, then the
+ * layernorm of norm.rs over the last extent; saves [res, gamma, mean, rstd].
+ * pinned by: equality with layernorm(add(x, residual)) of this oracle, bit for
+ * bit; float64 closed form. */
+static uint32_t residual_layernorm_impl(size_t x, size_t residual, size_t gamma, size_t beta, float eps) {
+    orc_tensor *X = get(x), *R = get(residual), *Gm = get(gamma), *Bt = get(beta);
+    if (!X || !R || !Gm || !Bt) return fail("tensor already freed");
+    int nd = X->ndim;
+    if (nd < 1) return fail("called `Option::unwrap()` on a `None` value: residual_layernorm of a scalar");
+    size_t shape[ORC_MAX_DIMS];
+    memcpy(shape, X->shape, sizeof shape);
+    size_t c = shape[nd - 1];
+    size_t n = c ? shape_size(shape, nd) / c : 0;
+    if (R->size < n * c) return fail("index out of bounds: residual shorter than x");
+    if (Gm->size < c || Bt->size < c) return fail("index out of bounds: gamma/beta shorter than the last extent");
+    float *xd = to_host(X), *rd = to_host(R), *gd = to_host(Gm), *bd = to_host(Bt);
+    float *res = (float *)calloc((n * c) > 0 ? n * c : 1, sizeof(float));
+    float *out = (float *)calloc((n * c) > 0 ? n * c : 1, sizeof(float));
+    float *mean = (float *)calloc(n ? n : 1, sizeof(float)), *rstd = (float *)calloc(n ? n : 1, sizeof(float));
+    for (size_t row = 0; row < n; ++row) {
+        size_t off = row * c;
+        float sum = 0.0f;
+        for (size_t j = 0; j < c; ++j) {
+            float val = xd[off + j] + rd[off + j];
+            res[off + j] = val;
+            sum += val;
+        }
+        float m = sum / (float)c;
+        mean[row] = m;
+        float var = 0.0f;
+        for (size_t j = 0; j < c; ++j) { float d = res[off + j] - m; var += d * d; }
+        float r = 1.0f / sqrtf(var / (float)c + eps);
+        rstd[row] = r;
+        for (size_t j = 0; j < c; ++j) out[off + j] = (res[off + j] - m) * r * gd[j] + bd[j];
+    }
+    free(xd); free(rd); free(gd); free(bd);
+    size_t res_id = from_vec(res, shape, nd);
+    size_t mean_id = from_vec(mean, &n, 1), rstd_id = from_vec(rstd, &n, 1);
+    size_t out_id = from_vec(out, shape, nd);
+    orc_entry *e = tape_record(&g_tape, OP_RESIDUALLAYERNORM, out_id, 4, x, residual);
+    e->input_ids[2] = gamma; e->input_ids[3] = beta;
+    e->saved_ids[0] = res_id; e->saved_ids[1] = gamma; e->saved_ids[2] = mean_id; e->saved_ids[3] = rstd_id;
+    return (uint32_t)out_id;
+}
+/* ops/fused.rs:134-186: the layernorm backward on the saved sum; the one dx
+ * tensor is returned for x and for the residual. */
+static int residual_layernorm_backward(size_t grad, const orc_entry *e, long *out) {
+    orc_tensor *S = get(e->saved_ids[0]), *Gm = get(e->saved_ids[1]), *Mn = get(e->saved_ids[2]), *Rs = get(e->saved_ids[3]), *G = get(grad);
+    if (!S || !Gm || !Mn || !Rs || !G) { fail("tensor already freed"); return -1; }
+    int nd = S->ndim, gnd = Gm->ndim;
+    size_t shape[ORC_MAX_DIMS], gshape[ORC_MAX_DIMS];
+    memcpy(shape, S->shape, sizeof shape);
+    memcpy(gshape, Gm->shape, sizeof gshape);
+    size_t c = shape[nd - 1], n = c ? shape_size(shape, nd) / c : 0;
+    float *xd = to_host(S), *gm = to_host(Gm), *mn = to_host(Mn), *rs = to_host(Rs), *gd = to_host(G);
+    float *dx = (float *)calloc((n * c) > 0 ? n * c : 1, sizeof(float));
+    size_t gsz = Gm->size > c ? Gm->size : c;
+    float *dgamma = (float *)calloc(gsz ? gsz : 1, sizeof(float));
+    float *dbeta = (float *)calloc(gsz ? gsz : 1, sizeof(float));
+    for (size_t row = 0; row < n; ++row) {
+        size_t off = row * c;
+        float m = mn[row], r = rs[row];
+        float sum_dg = 0.0f, sum_dgx = 0.0f;
+        for (size_t j = 0; j < c; ++j) {
+            float xhat = (xd[off + j] - m) * r;
+            float dg = gd[off + j] * gm[j];
+            sum_dg += dg;
+            sum_dgx += dg * xhat;
+            dgamma[j] += gd[off + j] * xhat;
+            dbeta[j] += gd[off + j];
+        }
+        for (size_t j = 0; j < c; ++j) {
+            float xhat = (xd[off + j] - m) * r;
+            float dg = gd[off + j] * gm[j];
+            dx[off + j] = r * (dg - sum_dg / (float)c - xhat * sum_dgx / (float)c);
+        }
+    }
+    free(xd); free(gm); free(mn); free(rs); free(gd);
+    out[0] = out[1] = (long)from_vec(dx, shape, nd);
+    out[2] = (long)from_vec(dgamma, gshape, gnd); /* c sums under gamma's shape, fused.rs:176-185 */
+    out[3] = (long)from_vec(dbeta, gshape, gnd);
+    return 0;
+}
+
+/* ops/mixed_precision.rs:17-32 scale_grads, cpu arm */
+int orc_scale_grads(const uint32_t *ids, size_t n, double inv_scale_) {
+    float inv_scale = (float)inv_scale_;
+    int found = 0;
+    for (size_t p = 0; p < n; ++p) {
+        orc_tensor *T = get(ids[p]);
+        if (!T || T->grad < 0) continue;
+        orc_tensor *G = get((size_t)T->grad);
+        if (!G) continue;
+        for (size_t i = 0; i < G->size; ++i) {
+            G->data[i] *= inv_scale;
+            if (isinf(G->data[i]) || isnan(G->data[i])) found = 1;
+        }
+    }
+    return found;
+}
+
 /* ---- backward ----------------------------------------------------------- */
 
 /* autograd.rs:180-222 dispatch_backward */
 static int dispatch_backward(const orc_entry *e, size_t grad, long *out) {
-    out[0] = out[1] = out[2] = -1;
+    out[0] = out[1] = out[2] = out[3] = -1;
     switch (e->op) {
     case OP_ADD: return addsub_backward(grad, e, out, 0);
     case OP_SUB: return addsub_backward(grad, e, out, 1);
@@ -1327,6 +1700,9 @@ static int dispatch_backward(const orc_entry *e, size_t grad, long *out) {
     case OP_BIASGELU: return bias_gelu_backward(grad, e, out);        /* autograd.rs BiasGelu */
     case OP_SOFTMAX: return softmax_backward(grad, e, out);           /* autograd.rs:204 */
     case OP_FLASHATTENTION: return flash_attention_backward(grad, e, out); /* autograd.rs:210 */
+    case OP_EMBEDDING: return embedding_backward(grad, e, out);
+    case OP_DROPOUT: return dropout_backward(grad, e, out);
+    case OP_RESIDUALLAYERNORM: return residual_layernorm_backward(grad, e, out);
     }
     return -1;
 }
@@ -1401,7 +1777,7 @@ static int tape_backward(orc_tape *tp, size_t loss_id) {
         long idx = out2entry[tid];
         if (idx < 0) continue;
         orc_entry e = tp->e[idx];
-        long ig[3];
+        long ig[4];
         if (dispatch_backward(&e, (size_t)grads[tid], ig) != 0) { rc = -1; break; }
         for (int i = 0; i < e.n_inputs; ++i) {
             if (ig[i] < 0) continue;
@@ -1828,7 +2204,62 @@ double orc_clip_and_step(const uint32_t *ids, size_t n, double lr, double b1, do
     adamw_step_impl(ids, n, (float)lr, (float)b1, (float)b2, (float)eps, (float)wd, (uint32_t)step);
     return (double)norm;
 }
+uint32_t orc_rand_tensor(const int64_t *shape, int nd) { /* lib.rs:60-64 */
+    size_t s[ORC_MAX_DIMS];
+    if (conv_shape(shape, nd, s) != 0) return ORC_BAD;
+    return random_tensor(s, nd, 0);
+}
+uint32_t orc_randn_tensor(const int64_t *shape, int nd) { /* lib.rs:67-71 */
+    size_t s[ORC_MAX_DIMS];
+    if (conv_shape(shape, nd, s) != 0) return ORC_BAD;
+    return random_tensor(s, nd, 1);
+}
+uint32_t orc_dropout_op(uint32_t x, double rate, int training) { return dropout_impl(x, (float)rate, training); } /* lib.rs:388-394 */
+uint32_t orc_embedding_forward(uint32_t weight, const int64_t *indices, size_t n, int64_t batch, int64_t seq_len) { /* lib.rs:319-326 */
+    if (batch < 0 || seq_len < 0 || (size_t)(batch * seq_len) > n) return fail("index out of bounds: fewer indices than batch * seq_len");
+    size_t *idx = (size_t *)malloc((n ? n : 1) * sizeof(size_t));
+    for (size_t i = 0; i < n; ++i) idx[i] = (size_t)indices[i];
+    uint32_t r = embedding_impl(weight, idx, (size_t)batch, (size_t)seq_len);
+    free(idx);
+    return r;
+}
+uint32_t orc_embedding_forward_gpu(uint32_t weight, uint32_t int_buf, int64_t batch, int64_t seq_len) { /* lib.rs:501-511, embedding.rs (GpuIndices arm) */
+    orc_intbuf *b = int_get(int_buf);
+    if (!b) return ORC_BAD;
+    if (batch < 0 || seq_len < 0 || (size_t)(batch * seq_len) > b->len) return fail("index out of bounds: fewer indices than batch * seq_len");
+    size_t *idx = (size_t *)malloc((b->len ? b->len : 1) * sizeof(size_t));
+    for (size_t i = 0; i < b->len; ++i) idx[i] = (size_t)b->data[i];
+    uint32_t r = embedding_impl(weight, idx, (size_t)batch, (size_t)seq_len);
+    free(idx);
+    return r;
+}
+uint32_t orc_cross_entropy_loss_gpu(uint32_t logits, uint32_t int_buf) { /* lib.rs:679-691 -> loss.rs:190-229 */
+    orc_tensor *L = get(logits);
+    orc_intbuf *b = int_get(int_buf);
+    if (!L || !b) return ORC_BAD;
+    if (L->ndim < 1) return fail("index out of bounds: cross_entropy of a scalar");
+    size_t v = L->shape[L->ndim - 1];
+    if (v == 0) return fail("attempt to divide by zero");
+    size_t flat[2] = {L->size / v, v};
+    uint32_t f = view_impl(logits, flat, 2);
+    if (f == ORC_BAD) return ORC_BAD;
+    int64_t *t = (int64_t *)malloc((b->len ? b->len : 1) * sizeof(int64_t));
+    for (size_t i = 0; i < b->len; ++i) t[i] = b->data[i];
+    uint32_t r = cross_entropy_impl(f, t, b->len);
+    free(t);
+    return r;
+}
+uint32_t orc_residual_layernorm(uint32_t x, uint32_t residual, uint32_t gamma, uint32_t beta, double eps) { /* lib.rs:515-523 */
+    return residual_layernorm_impl(x, residual, gamma, beta, (float)eps);
+}
+uint32_t orc_tile(uint32_t input, const int64_t *reps, int n) { /* lib.rs:568-573 */
+    size_t r[ORC_MAX_DIMS];
+    if (n < 0 || n > ORC_MAX_DIMS) return fail("tile: reps must match tensor dimensions");
+    for (int i = 0; i < n; ++i) { if (reps[i] < 0) return fail("negative repeat count"); r[i] = (size_t)reps[i]; }
+    return tile_impl(input, r, n);
+}
 void orc_reset_engine(void) { /* lib.rs:460-468 */
+    int_clear();
     for (size_t i = 0; i < g_kv_cap; ++i) if (g_kv[i].live) kv_release(&g_kv[i]);
     g_kv_next = 1;
     for (size_t i = 0; i < g_store.len; ++i)

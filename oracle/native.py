@@ -76,6 +76,20 @@ class OracleNative:
             "orc_clip_and_step": (C.c_double, [_u32p, C.c_size_t] + [C.c_double] * 5 + [C.c_int64, C.c_double]),
             "orc_reset_engine": (None, []), "orc_gc_tensors": (None, [_u32p, C.c_size_t]),
             "orc_sgemm_ikj": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]),
+            "orc_philox4x32_10": (None, [_u32p, _u32p, _u32p]),
+            "orc_philox_words": (None, [C.c_uint64, C.c_uint64, C.c_void_p, C.c_size_t]),
+            "orc_seed": (None, [C.c_uint64]),
+            "orc_rand_tensor": (u32, [_i64p, C.c_int]), "orc_randn_tensor": (u32, [_i64p, C.c_int]),
+            "orc_dropout_op": (u32, [u32, C.c_double, C.c_int]),
+            "orc_create_dataset": (u32, [C.c_void_p, C.c_size_t]), "orc_free_int_buffer": (None, [u32]),
+            "orc_int_buffer_len": (C.c_int64, [u32]), "orc_int_buffer_to_host": (C.c_int, [u32, C.c_void_p, C.c_size_t]),
+            "orc_sample_batch_at": (C.c_int, [u32, C.c_int64, C.c_int64, _i64p, _u32p]),
+            "orc_embedding_forward": (u32, [u32, _i64p, C.c_size_t, C.c_int64, C.c_int64]),
+            "orc_embedding_forward_gpu": (u32, [u32, u32, C.c_int64, C.c_int64]),
+            "orc_cross_entropy_loss_gpu": (u32, [u32, u32]),
+            "orc_residual_layernorm": (u32, [u32, u32, u32, u32, C.c_double]),
+            "orc_scale_grads": (C.c_int, [_u32p, C.c_size_t, C.c_double]),
+            "orc_tile": (u32, [u32, _i64p, C.c_int]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(lib, name)
@@ -278,6 +292,68 @@ class OracleNative:
 
     def gcTensors(self, keep):
         self.lib.orc_gc_tensors(_u32(keep), len(keep))
+
+    # token-side ops
+    def philox(self, ctr, key):
+        out = (C.c_uint32 * 4)()
+        self.lib.orc_philox4x32_10(_u32(ctr), _u32(key), out)
+        return [int(v) for v in out]
+
+    def philoxWords(self, seed, offset, n):
+        out = np.empty(n, dtype=np.uint32)
+        self.lib.orc_philox_words(seed, offset, out.ctypes.data, n)
+        return out
+
+    def seed(self, seed):
+        self.lib.orc_seed(seed)
+
+    def randTensor(self, shape):
+        return self._id(self.lib.orc_rand_tensor(_i64(shape), len(shape)))
+
+    def randnTensor(self, shape):
+        return self._id(self.lib.orc_randn_tensor(_i64(shape), len(shape)))
+
+    def dropoutOp(self, x, rate, training):
+        return self._id(self.lib.orc_dropout_op(x, rate, 1 if training else 0))
+
+    def createDataset(self, data):
+        a = np.ascontiguousarray(data, dtype=np.int32)
+        return self._id(self.lib.orc_create_dataset(a.ctypes.data, a.size))
+
+    def freeIntBuffer(self, id):
+        self.lib.orc_free_int_buffer(id)
+
+    def intBufferToHost(self, id):
+        n = self.lib.orc_int_buffer_len(id)
+        if n < 0:
+            raise self._err()
+        out = np.empty(n, dtype=np.int32)
+        self._rc(self.lib.orc_int_buffer_to_host(id, out.ctypes.data, n))
+        return out
+
+    # the reference draws the window starts from its thread RNG; the oracle takes them as an argument
+    def sampleBatchAt(self, datasetId, blockSize, batchSize, starts):
+        out = (C.c_uint32 * 2)()
+        self._rc(self.lib.orc_sample_batch_at(datasetId, blockSize, batchSize, _i64(starts), out))
+        return [int(out[0]), int(out[1])]
+
+    def embeddingForward(self, weight, indices, batch, seqLen):
+        return self._id(self.lib.orc_embedding_forward(weight, _i64(indices), len(indices), batch, seqLen))
+
+    def embeddingForwardGpu(self, weight, intBufId, batch, seqLen):
+        return self._id(self.lib.orc_embedding_forward_gpu(weight, intBufId, batch, seqLen))
+
+    def crossEntropyLossGpu(self, logits, intBufId):
+        return self._id(self.lib.orc_cross_entropy_loss_gpu(logits, intBufId))
+
+    def residualLayernorm(self, x, residual, gamma, beta, eps):
+        return self._id(self.lib.orc_residual_layernorm(x, residual, gamma, beta, eps))
+
+    def scaleGrads(self, ids, invScale):
+        return bool(self.lib.orc_scale_grads(_u32(ids), len(ids), invScale))
+
+    def tile(self, a, reps):
+        return self._id(self.lib.orc_tile(a, _i64(reps), len(reps)))
 
     # raw loop of ops/matmul.rs:62-69 on host arrays
     def sgemm_ikj(self, a, b):

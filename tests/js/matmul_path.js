@@ -162,6 +162,54 @@ assertClose(mseLoss(p, Tensor.fromFloat32(new Float32Array([2, 3, 4, 5]), [2, 2]
   assert(threw, 'free invalidates kv cache handle');
 }
 
+// ---- token-side ops (test/nn.test.ts:176-251, test/native.test.ts:28-36) --------------------------------
+{
+  native.seed(7);
+  const w = native.philoxWords(0, 0, 4);
+  assert(w[0] === 0x6627e8d5 && w[3] === 0x9b00dbd8, 'philox known answer');
+  const r = native.toFloat32(native.randTensor([1000]));
+  assert(r.every(v => v >= 0 && v < 1), 'rand in [0, 1)');
+  const z = native.toFloat32(native.randnTensor([4000]));
+  let m = 0; for (const v of z) m += v / z.length;
+  assert(Math.abs(m) < 0.1, 'randn mean near 0');
+  const tiled = new Tensor(native.tile(Tensor.fromFloat32(new Float32Array([1, 2, 3]), [1, 3])._id, [2, 1]));
+  const td = tiled.toFloat32();
+  assert(tiled.shape[0] === 2 && tiled.shape[1] === 3 && td[0] === 1 && td[3] === 1 && td[5] === 3, 'tile [1,3] x [2,1]');
+  const weight = Tensor.fromFloat32(randArray(40, rnd, -0.5, 0.5), [10, 4]).setRequiresGrad(true);
+  const emb = new Tensor(native.embeddingForward(weight._id, [0, 1, 2, 3, 4, 5], 2, 3));
+  assert(emb.shape.join() === '2,3,4', 'embedding shape');
+  const same = native.toFloat32(native.embeddingForward(weight._id, [0, 0, 0, 0], 2, 2));
+  assert(same[0] === same[4], 'same index = same embedding');
+  let threw = false;
+  try { native.embeddingForward(weight._id, [10], 1, 1); } catch (e) { threw = /out of range/.test(e.message); }
+  assert(threw, 'embedding index out of range throws');
+  const x4 = Tensor.fromFloat32(new Float32Array([1, 2, 3, 4]), [4]);
+  assert(native.dropoutOp(x4._id, 0.5, false) === x4._id && native.dropoutOp(x4._id, 0.0, true) === x4._id, 'dropout passthrough');
+  const dropped = native.toFloat32(native.dropoutOp(native.ones([1000]), 0.5, true));
+  const zeros = dropped.filter(v => v === 0).length;
+  assert(zeros > 100 && zeros < 900 && dropped.every(v => v === 0 || v === 2), 'dropout rate 0.5');
+  const rln = new Tensor(native.residualLayernorm(native.randTensor([2, 4]), native.randTensor([2, 4]), native.ones([4]), native.zeros([4]), 1e-5));
+  const rd = rln.toFloat32();
+  assert(rln.shape.join() === '2,4' && Math.abs(rd[0] + rd[1] + rd[2] + rd[3]) < 1e-4, 'residualLayernorm rows have zero mean');
+  const data = new Int32Array(500); for (let i = 0; i < 500; i++) data[i] = i % 10;
+  const ds = native.createDataset(data);
+  const [inp, tgt] = native.sampleBatch(ds, 8, 4);
+  const a = native.intBufferToInt32(inp), b = native.intBufferToInt32(tgt);
+  let ok = a.length === 32 && b.length === 32;
+  for (let i = 0; i < 32; i++) ok = ok && b[i] === (a[i] + 1) % 10;
+  assert(ok, 'sampleBatch targets are the inputs shifted by one');
+  const e2 = new Tensor(native.embeddingForwardGpu(weight._id, inp, 4, 8));
+  const logits = e2.matmul(Tensor.fromFloat32(randArray(40, rnd, -0.5, 0.5), [4, 10]));
+  const loss = new Tensor(native.crossEntropyLossGpu(logits._id, tgt));
+  loss.mul(1024).backward();
+  assert(native.scaleGrads([weight._id], 1 / 1024) === false, 'scaleGrads reports finite gradients');
+  assert(Math.abs(loss.toFloat32()[0] - Math.log(10)) < 0.5, 'cross-entropy on buffered targets near ln(10)');
+  native.freeIntBuffer(inp); native.freeIntBuffer(tgt);
+  threw = false;
+  try { native.intBufferToInt32(inp); } catch (e) { threw = /int buffer already freed/.test(e.message); }
+  assert(threw, 'freed int buffer is rejected');
+}
+
 // ---- misuse raises a JS Error where the reference panics ---------------------------------------------
 try { Tensor.fromFloat32(new Float32Array(6), [2, 3]).matmul(Tensor.fromFloat32(new Float32Array(8), [4, 2])); assert(false, 'K mismatch must throw'); }
 catch (e) { assert(/inner dimensions/.test(e.message), 'K mismatch message: ' + e.message); }
