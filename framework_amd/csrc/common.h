@@ -144,6 +144,11 @@ int k_residual_layernorm(float *out, float *res, float *mean, float *rstd, const
 int k_scale_check(float *g, float s, int64_t n, float *flag);
 
 int k_sumsq_f64(double *out, const float *g, int64_t n);  // out += sum g^2 (device double)
+// The same in two steps, so that many tensors share one final sum: partials of
+// one tensor (sumsq_blocks(n) doubles), then out += sum of all partials.
+int sumsq_blocks(int64_t n);
+int k_sumsq_partials(double *part, const float *g, int64_t n);
+int k_sumsq_finish(double *out, const double *part, int nparts);
 int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, float b1, float b2,
             float eps, float wd, float bc1, float bc2);
 

@@ -865,6 +865,49 @@ __global__ void ce_rows_kernel(float *__restrict__ row_loss, float *__restrict__
         row_loss[row] = -logf(e / sum);
     }
 }
+// The same with the row held in registers (NV 16-byte pieces per lane): the
+// logits are read once and the probabilities written once.
+template <int NV>
+__global__ void ce_rows_cached_kernel(float *__restrict__ row_loss, float *__restrict__ sm, const float *__restrict__ logits,
+                                      const int32_t *__restrict__ targets, int64_t n, int64_t v) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n) return;
+    const int64_t v4 = v >> 2;
+    const float4 *x = reinterpret_cast<const float4 *>(logits + row * v);
+    float4 *p = reinterpret_cast<float4 *>(sm + row * v);
+    float4 r[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t j = lane + 64 * i;
+        r[i] = j < v4 ? x[j] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) mx = fmaxf(fmaxf(mx, fmaxf(r[i].x, r[i].y)), fmaxf(r[i].z, r[i].w));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        if (lane + 64 * i < v4) {
+            r[i].x = expf(r[i].x - mx); r[i].y = expf(r[i].y - mx); r[i].z = expf(r[i].z - mx); r[i].w = expf(r[i].w - mx);
+            sum += r[i].x; sum += r[i].y; sum += r[i].z; sum += r[i].w;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t j = lane + 64 * i;
+        if (j < v4) p[j] = make_float4(r[i].x / sum, r[i].y / sum, r[i].z / sum, r[i].w / sum);
+    }
+    if (lane == 0) {
+        const int32_t t = targets[row];
+        const float e = expf(logits[row * v + t] - mx);
+        row_loss[row] = -logf(e / sum);
+    }
+}
 __global__ void ce_mean_kernel(float *__restrict__ loss, const float *__restrict__ row_loss, int64_t n) {
     const int lane = threadIdx.x;
     float s = 0.f;
@@ -878,7 +921,17 @@ int k_cross_entropy(float *loss, float *softmax, const float *logits, const int3
     if (n <= 0 || v <= 0) return set_error(MNI_ERR_INVALID, "cross_entropy: empty logits");
     void *rl = nullptr;
     MNI_TRY(dev_alloc(&rl, (size_t)n * sizeof(float)));
-    hipLaunchKernelGGL(ce_rows_kernel, dim3(grid_for(n, 4)), dim3(TPB), 0, ctx().stream, (float *)rl, softmax, logits, targets, n, v);
+    const bool vec = (v % 4) == 0 && al16(logits) && al16(softmax);
+    const dim3 grid(grid_for(n, 4)), block(TPB);
+    hipStream_t st = ctx().stream;
+    if (vec && v <= 64 * 4 * 2)
+        hipLaunchKernelGGL(ce_rows_cached_kernel<2>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
+    else if (vec && v <= 64 * 4 * 8)
+        hipLaunchKernelGGL(ce_rows_cached_kernel<8>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
+    else if (vec && v <= 64 * 4 * 32)
+        hipLaunchKernelGGL(ce_rows_cached_kernel<32>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
+    else
+        hipLaunchKernelGGL(ce_rows_kernel, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
     int rc = check_launch("ce_rows");
     if (rc == MNI_OK) {
         hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(64), 0, ctx().stream, loss, (const float *)rl, n);
@@ -922,26 +975,41 @@ __global__ void sumsq_kernel(double *__restrict__ part, const float *__restrict_
     __syncthreads();
     if (threadIdx.x == 0) part[blockIdx.x] = (sh[0] + sh[1]) + (sh[2] + sh[3]);
 }
+// out[0] += sum of part[0..nparts): one workgroup, fixed order
 __global__ void sumsq_final_kernel(double *__restrict__ out, const double *__restrict__ part, int nparts) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        double s = 0.0;
-        for (int p = 0; p < nparts; ++p) s += part[p];
-        out[0] += s;
-    }
+    __shared__ double sh[4];
+    double s = 0.0;
+    for (int p = threadIdx.x; p < nparts; p += blockDim.x) s += part[p];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) out[0] += (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+int sumsq_blocks(int64_t n) {
+    if (n <= 0) return 0;
+    int blocks = (int)grid_for(n, TPB * 8);
+    return blocks > 1024 ? 1024 : blocks;
+}
+int k_sumsq_partials(double *part, const float *g, int64_t n) {
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(sumsq_kernel, dim3(sumsq_blocks(n)), dim3(TPB), 0, ctx().stream, part, g, n);
+    return check_launch("sumsq");
+}
+int k_sumsq_finish(double *out, const double *part, int nparts) {
+    if (nparts <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), dim3(TPB), 0, ctx().stream, out, part, nparts);
+    return check_launch("sumsq_final");
 }
 int k_sumsq_f64(double *out, const float *g, int64_t n) {
     if (n <= 0) return MNI_OK;
-    MNI_TRY(ensure_init());
-    int blocks = (int)grid_for(n, TPB * 8);
-    if (blocks > 1024) blocks = 1024;
+    const int blocks = sumsq_blocks(n);
     void *part = nullptr;
     MNI_TRY(dev_alloc(&part, (size_t)blocks * sizeof(double)));
-    hipLaunchKernelGGL(sumsq_kernel, dim3(blocks), dim3(TPB), 0, ctx().stream, (double *)part, g, n);
-    int rc = check_launch("sumsq");
-    if (rc == MNI_OK) {
-        hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), dim3(64), 0, ctx().stream, out, (const double *)part, blocks);
-        rc = check_launch("sumsq_final");
-    }
+    int rc = k_sumsq_partials((double *)part, g, n);
+    if (rc == MNI_OK) rc = k_sumsq_finish(out, (const double *)part, blocks);
     dev_free(part);
     return rc;
 }

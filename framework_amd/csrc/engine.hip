@@ -48,6 +48,10 @@ struct Tensor {
     bool requires_grad = false;
     int64_t grad = -1;
     BufP adam_m, adam_v;
+    // A gradient that is known to hold only zeros (fresh, or just cleared):
+    // the first accumulation into it shares the incoming buffer instead of
+    // adding to zeros.  Every in-place writer goes through make_unique().
+    bool known_zero = false;
 };
 
 enum Op {  // subset of src/native/src/autograd.rs:28-62 plus the fused Linear
@@ -222,6 +226,7 @@ static BufP clone_buf(const BufP &src, size_t n) {
 }
 // Copy-on-write before an in-place update.
 static int make_unique(Tensor &t) {
+    t.known_zero = false;
     if (t.buf.use_count() <= 1) return MNI_OK;
     BufP c = clone_buf(t.buf, t.buf->n);
     if (!c) return MNI_ERR_NOMEM;
@@ -247,6 +252,7 @@ static int64_t ensure_grad(uint32_t id) {  // tensor.rs:144-152
     const Shape shape = t->shape;
     const uint32_t g = zeros(shape);
     if (g == MNI_BAD_ID) return -1;
+    get(g)->known_zero = true;
     get(id)->grad = g;
     return g;
 }
@@ -256,6 +262,11 @@ static int add_into(uint32_t dst, uint32_t src) {
     Tensor *s = get(src), *d = get(dst);
     if (!s || !d) return MNI_ERR_FREED;
     if ((int64_t)d->buf->n < s->size) return set_error(MNI_ERR_INVALID, "add_inplace: destination smaller than source");
+    if (d->known_zero && d->buf->n == s->buf->n && s->size == (int64_t)s->buf->n) {
+        d->buf = s->buf;  // 0 + x = x: share x (a later in-place writer of either tensor copies first)
+        d->known_zero = false;
+        return MNI_OK;
+    }
     MNI_TRY(make_unique(*d));
     return k_axpy(d->buf->p, s->buf->p, 1.0f, s->size);
 }
@@ -682,7 +693,7 @@ static int reduce_backward(uint32_t grad, const Entry &e, int64_t *out, bool mea
 }
 
 // ---- layout ------------------------------------------------------------------------------
-// ops/layout.rs:66-89 view: always a copy with the new shape.
+// ops/layout.rs:66-89 view: a tensor of the same contents under the new shape.
 static uint32_t view_op(uint32_t a, const Shape &new_shape) {
     Tensor *A = get(a);
     if (!A) return MNI_BAD_ID;
@@ -692,11 +703,18 @@ static uint32_t view_op(uint32_t a, const Shape &new_shape) {
         set_error(MNI_ERR_INVALID, "view: %lld elements cannot be viewed as %lld", (long long)n, (long long)shape_size(new_shape));
         return MNI_BAD_ID;
     }
-    BufP out = new_buf((size_t)n);
-    if (!out) return MNI_BAD_ID;
-    int rc = is_contiguous(*A) ? mni_rocm_d2d(out->p, A->buf->p, (size_t)n * sizeof(float))
-                               : k_strided_copy(out->p, A->buf->p, A->shape.data(), A->strides.data(), (int)A->shape.size());
-    if (rc != MNI_OK) return MNI_BAD_ID;
+    // The reference copies (layout.rs:70-77); with reference-counted buffers a
+    // contiguous source is shared instead, and any in-place writer copies first.
+    BufP out;
+    if (is_contiguous(*A) && (int64_t)A->buf->n == n) {
+        out = A->buf;
+    } else {
+        out = new_buf((size_t)n);
+        if (!out) return MNI_BAD_ID;
+        const int rc = is_contiguous(*A) ? mni_rocm_d2d(out->p, A->buf->p, (size_t)n * sizeof(float))
+                                         : k_strided_copy(out->p, A->buf->p, A->shape.data(), A->strides.data(), (int)A->shape.size());
+        if (rc != MNI_OK) return MNI_BAD_ID;
+    }
     const uint32_t id = insert_contig(std::move(out), new_shape);
     Entry e;
     e.op = OP_VIEW; e.output_id = id; e.n_inputs = 1; e.inputs[0] = a; e.saved_shape = orig;
@@ -1730,20 +1748,31 @@ static float powi_f32(float a, int b) {  // f32::powi (compiler-rt __powisf2)
 
 // ops/optimizer.rs:126-138 grad_norm
 static int grad_norm(const uint32_t *ids, size_t n, float *out) {
-    void *acc = nullptr;
-    MNI_TRY(dev_alloc(&acc, sizeof(double)));
-    std::shared_ptr<void> guard(acc, [](void *p) { dev_free(p); });
-    MNI_HIP_CHECK(hipMemsetAsync(acc, 0, sizeof(double), ctx().stream));
+    // Per-tensor partial sums land in one buffer; a single kernel adds them up.
+    std::vector<Tensor *> gs;
+    int64_t nparts = 0;
     for (size_t p = 0; p < n; ++p) {
         Tensor *T = get(ids[p]);
         if (!T) return MNI_ERR_FREED;
         if (T->grad < 0) continue;
         Tensor *G = get((uint32_t)T->grad);
         if (!G) return MNI_ERR_FREED;
-        MNI_TRY(k_sumsq_f64((double *)acc, G->buf->p, G->size));
+        gs.push_back(G);
+        nparts += sumsq_blocks(G->size);
     }
+    void *acc = nullptr;
+    MNI_TRY(dev_alloc(&acc, (size_t)(nparts + 1) * sizeof(double)));
+    std::shared_ptr<void> guard(acc, [](void *p) { dev_free(p); });
+    double *total = (double *)acc, *part = total + 1;
+    MNI_TRY(k_fill((float *)total, 0.0f, 2));  // one double
+    int64_t at = 0;
+    for (Tensor *G : gs) {
+        MNI_TRY(k_sumsq_partials(part + at, G->buf->p, G->size));
+        at += sumsq_blocks(G->size);
+    }
+    MNI_TRY(k_sumsq_finish(total, part, (int)nparts));
     double sq = 0.0;
-    MNI_TRY(mni_rocm_d2h(&sq, acc, sizeof(double)));
+    MNI_TRY(mni_rocm_d2h(&sq, total, sizeof(double)));
     *out = sqrtf((float)sq);
     return MNI_OK;
 }
@@ -1883,11 +1912,14 @@ int mni_zero_grad(const uint32_t *ids, size_t n) {
         if (t->grad < 0) continue;
         Tensor *g = get((uint32_t)t->grad);
         if (!g) return MNI_ERR_FREED;
+        bool fill = !g->known_zero;
         if (g->buf.use_count() > 1) {  // shared: replace instead of copy + clear
             g->buf = new_buf(g->buf->n);
             if (!g->buf) return MNI_ERR_NOMEM;
+            fill = true;
         }
-        MNI_TRY(k_fill(g->buf->p, 0.0f, (int64_t)g->buf->n));
+        if (fill) MNI_TRY(k_fill(g->buf->p, 0.0f, (int64_t)g->buf->n));
+        g->known_zero = true;
     }
     return MNI_OK;
 }
@@ -1944,6 +1976,7 @@ uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim) {
     return permute_op(a, s);
 }
 uint32_t mni_contiguous(uint32_t a) {  // layout.rs:218-227
+    MNI_API_GUARD;
     Tensor *A = get(a);
     if (!A) return MNI_BAD_ID;
     if (is_contiguous(*A)) return a;
@@ -2162,6 +2195,7 @@ uint32_t mni_tile(uint32_t input, const int64_t *reps, int n) {  // lib.rs:568-5
 void *mni_dev_ptr(uint32_t id) {
     MNI_API_GUARD;
     Tensor *t = get(id);
+    if (t) t->known_zero = false;  // the caller may write through the pointer
     return t ? (void *)t->buf->p : nullptr;
 }
 

@@ -195,6 +195,24 @@ def test_int_buffer_forms_equal_the_host_forms(both):
         gpu.crossEntropyLossGpu(_t(gpu, np.zeros((4, 50))), bad)
 
 
+@pytest.mark.parametrize("n,v", [(5, 3), (33, 512), (17, 516), (64, 2048), (9, 2050), (40, 8192), (6, 8196), (3, 20000)])
+def test_cross_entropy_row_kernels_match_the_oracle(both, n, v):
+    # every row-kernel variant: scalar rows, rows cached in registers at three depths, long rows
+    logits = synth.normal(n + v, (n, v)) * 3.0
+    targets = [[int(t)] for t in np.random.default_rng(v).integers(0, v, size=n)]
+    res = []
+    for api in both:
+        lg = _t(api, logits, True)
+        loss = api.crossEntropyLoss(lg, targets)
+        loss.mul(3.0).backward()
+        res.append((loss.item(), lg.grad.numpy()))
+    assert abs(res[0][0] - res[1][0]) < 4e-6 * abs(res[1][0])
+    assert max_err(res[0][1], res[1][1]) < 4e-6 * float(np.abs(res[1][1]).max())   # the row sum runs in another order
+    lp = logits.astype(np.float64)
+    want = np.mean(np.log(np.exp(lp - lp.max(1, keepdims=True)).sum(1)) + lp.max(1) - lp[np.arange(n), [t[0] for t in targets]])
+    assert abs(res[0][0] - want) < 1e-5 * abs(want)
+
+
 def test_tile_matches_numpy_and_the_oracle(both):
     gpu, cpu = both
     t = gpu.tile(_t(gpu, [[1, 2, 3]]), [2, 1])                   # test/nn.test.ts:181-190
