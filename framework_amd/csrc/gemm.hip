@@ -35,7 +35,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_SKINNY_TWO_PASS)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_MFMA_STREAMK)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -48,6 +48,19 @@ static int finish_split(const float *ws, float *out, const float *bias, int slic
     r.o_rs = o_rs; r.o_cs = o_cs; r.o_bs = o_bs;
     r.epilogue = epilogue; r.accumulate = accumulate; r.bias_on_rows = bias_on_rows;
     return launch_splitk_reduce(r);
+}
+
+// A fresh value for the arrival marks of a single-launch reduction (skinny
+// fused kernel, stream-K): marks from earlier launches never match it, so the
+// array needs no clearing except when the counter wraps.
+static int next_epoch(unsigned *epoch) {
+    DeviceCtx &c = ctx();
+    if (++c.skinny_epoch == 0) {
+        MNI_TRY(k_fill((float *)c.skinny_flags, 0.0f, (int64_t)c.skinny_flag_cap));
+        c.skinny_epoch = 1;
+    }
+    *epoch = c.skinny_epoch;
+    return MNI_OK;
 }
 
 // ---- skinny path --------------------------------------------------------------
@@ -124,11 +137,8 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
             const int64_t flag_count = (int64_t)groups * s.batch * split;
             if (split > 1 && d.algo != MNI_ALGO_SKINNY_TWO_PASS && c.xcd_count > 0 && c.skinny_flags &&
                 flag_count <= (int64_t)c.skinny_flag_cap) {
-                if (++c.skinny_epoch == 0) {  // wrapped: old marks could match again
-                    *rc = k_fill((float *)c.skinny_flags, 0.0f, (int64_t)c.skinny_flag_cap);
-                    c.skinny_epoch = 1;
-                }
-                s.fused = 1; s.xcds = c.xcd_count; s.flags = c.skinny_flags; s.epoch = c.skinny_epoch;
+                *rc = next_epoch(&s.epoch);
+                s.fused = 1; s.xcds = c.xcd_count; s.flags = c.skinny_flags;
             }
             if (*rc == MNI_OK) *rc = launch_skinny_cols(s);
             if (*rc == MNI_OK && split > 1 && !s.fused) {
@@ -163,21 +173,72 @@ static int run_mfma(const mni_gemm_desc &d) {
     g.a_bcount = (int)d.A.batch_count; g.b_bcount = (int)d.B.batch_count;
     g.ldc = d.ldc; g.c_bs = d.c_batch_stride;
     g.epilogue = d.epilogue; g.accumulate = d.accumulate;
-    // Tile shape: 128 x 128 for dense products; a 64-wide side when that
-    // extent is at most 64 (no half-empty tiles), and 64 x 64 when K is short
-    // and 128 x 128 tiles would leave the machine with few, short-lived
-    // workgroups (small tiles: 4 resident per CU, cheaper prologue/epilogue).
     const int bk = gemm_mfma_tile_k();
-    const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
+    DeviceCtx &c = ctx();
+    const int cus = c.compute_units > 0 ? c.compute_units : 256;
+    const int ktiles = (g.K + bk - 1) / bk;
+    const bool sk_device = c.xcd_count > 0 && c.skinny_flags && cus % c.xcd_count == 0;
+
+    // Can the K steps of tiles of this shape be dealt over the stream-K grid?
+    // In every XCD's stream-K region each workgroup must own at least
+    // `min_steps` K steps (with none, a finisher would wait for a partial that
+    // nobody writes; with few, the fix-up costs more than it saves).
+    auto streamk_fits = [&](int tm, int tn, int min_steps) {
+        if (!sk_device || ktiles <= 0 || d.split_k > 1) return false;
+        const int64_t wpx = (int64_t)cus / c.xcd_count * gemm_mfma_resident_per_cu(tm, tn);
+        const int64_t total = (int64_t)((g.M + tm - 1) / tm) * ((g.N + tn - 1) / tn) * g.batch;
+        if (total * ktiles > 0x7fffffffLL || wpx > 256 || (size_t)(wpx * c.xcd_count) > c.skinny_flag_cap) return false;
+        for (int64_t xt = total / c.xcd_count; xt <= (total + c.xcd_count - 1) / c.xcd_count; ++xt) {
+            const int64_t left = xt % wpx;
+            const int64_t region = left == 0 ? 0 : (xt >= wpx ? left + wpx : left);
+            if (region > 0 && region * ktiles < wpx * min_steps) return false;
+        }
+        return true;
+    };
+
+    // Tile shape and work distribution.  A side is 64 wide when that extent is
+    // at most 64 (no half-empty tiles).  Otherwise: 128 x 128 tiles when every
+    // resident workgroup gets a good stretch of K steps out of them, 64 x 64
+    // when not.  With the tile chosen: one workgroup per tile when the tiles
+    // fill their rounds on the machine well; else stream-K, which has no
+    // rounds to fill; else (device mapping unknown, tiny product) K slices and
+    // a reduction pass.
     int bm = g.M <= 64 ? 64 : 128, bn = g.N <= 64 ? 64 : 128;
+    bool streamk = false;
+    bool whole_tiles = false;  // one workgroup per tile, no K slices
     if (d.algo == MNI_ALGO_MFMA_SMALL) {
         bm = bn = 64;
-    } else if (d.algo == MNI_ALGO_AUTO) {
-        const int64_t big_tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
-        const int ksteps = (g.K + bk - 1) / bk;
-        const int64_t big_split = d.split_k > 0 ? d.split_k : (ksteps / 8 > 0 ? ksteps / 8 : 1);
-        if (bm == 128 && bn == 128 && ((g.K <= 256 && big_tiles < 4LL * cus) || big_tiles * big_split < 2LL * cus))
-            bm = bn = 64;
+    } else if (d.algo == MNI_ALGO_AUTO || d.algo == MNI_ALGO_MFMA_STREAMK) {
+        const int64_t big_tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
+        const int64_t big_slots = (int64_t)cus * gemm_mfma_resident_per_cu(bm, bn);
+        if (ktiles >= 8 && d.split_k == 0 && sk_device) {
+            if (big_tiles * ktiles >= 20 * big_slots) {
+                // plenty of K steps per workgroup slot: big tiles
+                const int64_t rounds = (big_tiles + big_slots - 1) / big_slots;
+                whole_tiles = big_tiles * 100 >= rounds * big_slots * 93;
+                // (under 3/16 of the slots: long K over few tiles, left to the K slices below)
+                if (!whole_tiles && big_tiles * 16 >= 3 * big_slots) streamk = streamk_fits(bm, bn, 8);
+            } else {
+                const int64_t tiles = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) * g.batch;
+                const int64_t slots = (int64_t)cus * gemm_mfma_resident_per_cu(64, 64);
+                const int64_t rounds = (tiles + slots - 1) / slots;
+                whole_tiles = tiles * 100 >= rounds * slots * 70;
+                if (!whole_tiles) streamk = streamk_fits(64, 64, 8);
+                if (whole_tiles || streamk) bm = bn = 64;
+            }
+        } else {
+            // short K, a requested split, or no stream-K on this device: 64 x 64 when
+            // 128 x 128 tiles would leave the machine with few, short-lived workgroups
+            const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
+            const int64_t big_split = d.split_k > 0 ? d.split_k : (ktiles / 8 > 0 ? ktiles / 8 : 1);
+            if (bm == 128 && bn == 128 && ((g.K <= 256 && t128 < 4LL * cus) || t128 * big_split < 2LL * cus)) bm = bn = 64;
+        }
+        if (d.algo == MNI_ALGO_MFMA_STREAMK && !streamk) {
+            if (!sk_device) return set_error(MNI_ERR_INVALID, "sgemm: stream-K needs a confirmed workgroup-to-XCD mapping");
+            if (d.split_k > 1) return set_error(MNI_ERR_INVALID, "sgemm: stream-K does not take a split_k");
+            if (!streamk_fits(bm, bn, 1)) return set_error(MNI_ERR_INVALID, "sgemm: product too small for the stream-K grid");
+            streamk = true;
+        }
     }
     g.tiles_m = (g.M + bm - 1) / bm;
     g.tiles_n = (g.N + bn - 1) / bn;
@@ -187,10 +248,26 @@ static int run_mfma(const mni_gemm_desc &d) {
     // op(B)(k, n): K stride = row_stride, N stride = col_stride.
     const int bmode = g.K == 0 ? 2 : classify(g.B, g.b_rs, g.b_cs, g.b_bs, g.b_bcount);
 
+    g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0;
+    void *ws = nullptr;
+    if (streamk) {
+        g.split_k = 1;
+        g.k_per_slice = g.K;
+        g.streamk = 1;
+        g.sk_xcds = c.xcd_count;
+        g.sk_wpx = cus / c.xcd_count * gemm_mfma_resident_per_cu(bm, bn);
+        g.sk_flags = c.skinny_flags;
+        MNI_TRY(next_epoch(&g.sk_epoch));
+        MNI_TRY(dev_alloc(&ws, (size_t)g.sk_xcds * g.sk_wpx * bm * bn * sizeof(float)));
+        g.ws = (float *)ws;
+        const int rc = launch_gemm_mfma(g, amode, bmode, bm, bn);
+        dev_free(ws);
+        return rc;
+    }
+
     // Split K when the output tiles alone cannot fill the machine (two
     // workgroups fit on each CU).  Slices are whole K steps.
-    int split = d.split_k;
-    const int ktiles = (g.K + bk - 1) / bk;
+    int split = whole_tiles ? 1 : d.split_k;
     if (split == 0) {
         const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * g.batch;
         const int64_t slots = (bm * bn >= 128 * 128 ? 2LL : 4LL) * cus;
@@ -208,7 +285,6 @@ static int run_mfma(const mni_gemm_desc &d) {
     g.split_k = split;
     g.k_per_slice = split > 1 ? tiles_per_slice * bk : (g.K > 0 ? g.K : 1);
 
-    void *ws = nullptr;
     if (split > 1) {
         const size_t bytes = (size_t)split * g.batch * g.M * g.N * sizeof(float);
         MNI_TRY(dev_alloc(&ws, bytes));

@@ -21,10 +21,18 @@ struct GemmLaunch {
     int split_k, k_per_slice;
     int tiles_m, tiles_n;
     int epilogue, accumulate;
+    // Stream-K form (streamk != 0, split_k == 1): the grid is xcds * sk_wpx
+    // persistent workgroups; `ws` then holds one tile-sized partial per
+    // workgroup and sk_flags one arrival mark per workgroup, set to sk_epoch.
+    int streamk, sk_wpx, sk_xcds;
+    unsigned *sk_flags;
+    unsigned sk_epoch;
 };
 
 // tile_m, tile_n in {128, 64}; g.tiles_m / g.tiles_n count tiles of that size
 int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int tile_n);
+// workgroups that stay resident per CU for a tile shape (what the stream-K grid is sized by)
+int gemm_mfma_resident_per_cu(int tile_m, int tile_n);
 int gemm_mfma_tile_k();
 
 // Skinny (GEMV-shaped) products: X (MR x K, MR <= 16) against a large W.

@@ -32,6 +32,23 @@
 // a 4(k) x 4(mn) micro-tile with 16-byte loads along M/N and transposed in
 // registers on the way to LDS.  Anything else (arbitrary strides, unaligned
 // bases, edge tiles) takes guarded scalar loads into the same register layout.
+//
+// Work distribution.  Classic form: one workgroup per (tile, batch, K slice);
+// with more than one slice the partials go to a workspace and a second kernel
+// adds them.  Stream-K form (Osama et al., "Stream-K", PPoPP'23, restricted to
+// one XCD at a time): a fixed grid of resident workgroups; every XCD owns a
+// contiguous run of whole tiles.  Whole rounds of one tile per workgroup are
+// done tile by tile; the tiles that do not fill a round (with one full round,
+// when there is one) have their K steps dealt evenly over the XCD's
+// workgroups, so a workgroup's share may start and end in the middle of a tile.
+// A workgroup walks its share backwards: the piece at the end (the head of a
+// tile somebody else finishes) is computed first and parked in the workspace
+// with an arrival mark; whole tiles follow; the piece at the start (the tail
+// of a tile begun by lower-numbered workgroups) comes last, by which time
+// their partials arrived long ago.  Whoever holds a tile's last K step adds
+// the parked partials in workgroup order and runs the epilogue, so the sum
+// order is fixed by the shape alone.  Partials never leave the XCD's L2, and
+// a workgroup only ever waits for lower-numbered (earlier dispatched) ones.
 #include "common.h"
 #include "gemm_internal.h"
 
@@ -43,6 +60,14 @@ static constexpr int BK = 32;
 static constexpr int KQ = BK / 4;           // K quads per tile
 static constexpr int PAD = 2;               // float4 of padding per K-quad slice
 static constexpr int NTHREADS = 256;
+static constexpr int SK_WAIT_LIMIT = 1 << 20;  // polls before a finisher gives up and writes NaN
+
+__device__ __forceinline__ unsigned load_mark(const unsigned *p) {
+    // sc1: answered by the XCD's L2, never by this CU's L1
+    unsigned v;
+    asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
 
 // Row r of a tile sits at float4 slot r ^ ((r >> 4) & 3) of its K-quad slice.
 // Within an aligned group of 16 rows this is a permutation, so the MFMA operand
@@ -85,6 +110,10 @@ __device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t l
 template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void load_guarded(const float *__restrict__ p, int64_t rs, int64_t cs, int rmax,
                                              int kmax, int tid, float4 (&v)[4]) {
+    // Edge tiles and K tails only.  The empty asm makes the element addresses
+    // get computed here, on use: computed once ahead of the K loop they would
+    // occupy sixteen register pairs for the whole loop.
+    asm volatile("" : "+v"(tid));
     if (LAYOUT == 0) {
 #pragma unroll
         for (int i = 0; i < ROWS / 32; ++i) {
@@ -153,8 +182,17 @@ __device__ __forceinline__ float pick(const float4 &v, int j) { return j == 0 ? 
 // TM x TN: 32 x 32 MFMA blocks per wavefront; the workgroup tile is
 // (64 TM) x (64 TN): 128 x 128 for the dense case, 64-wide sides for narrow or
 // short-K products where smaller tiles waste less and fill the machine better.
-template <int AMODE, int BMODE, int TM, int TN>
-__global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_kernel(const GemmLaunch g) {
+// SK: the stream-K form (a loop over this workgroup's segments); otherwise the
+// body runs once for the (tile, batch, slice) named by the workgroup id.
+template <int AMODE, int BMODE, int TM, int TN, bool SK>
+__global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_kernel(const GemmLaunch launch_args) {
+    // The launch descriptor is read through the kernel-argument segment, so
+    // that the stream-K form can read it afresh for every segment (scalar
+    // loads) instead of holding all of it in scalar registers across the loop.
+    (void)launch_args;
+    typedef const GemmLaunch __attribute__((address_space(4))) *LaunchPtr;
+    LaunchPtr gp = (LaunchPtr)__builtin_amdgcn_kernarg_segment_ptr();
+#define g (*gp)
     constexpr int AL = AMODE == 1 ? 1 : 0;
     constexpr int BL = BMODE == 1 ? 1 : 0;
     constexpr int BM = 64 * TM, BN = 64 * TN;
@@ -167,28 +205,118 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     auto stage_a = [&](int st) -> float4 * { return lds + st * STAGE_A; };
     auto stage_b = [&](int st) -> float4 * { return lds + 2 * STAGE_A + st * STAGE_B; };
 
-    const int tid = threadIdx.x;
+    // ---- segments of work ----------------------------------------------------
+    enum { ROLE_FULL = 0, ROLE_SLICE = 1, ROLE_PART = 2, ROLE_FINISH = 3 };
+    const int tiles = g.tiles_m * g.tiles_n;
+    const int ksteps = (g.K + BK - 1) / BK;
+    // Stream-K.  The XCD's run of tiles splits into a stream-K region (its
+    // first sk_tiles tiles, whose K steps are dealt evenly: this workgroup's
+    // share is [seg_lo, seg_hi)) and whole rounds of one tile per workgroup
+    // after it.  The region is what does not fill a round, plus one full
+    // round when there is one, so that a share is at least a tile's worth.
+    // Only seg_hi (end of what is left of the share) and dp_tile (next whole
+    // tile) are carried from segment to segment; everything else is derived
+    // again from the workgroup id at the top of a segment, which keeps the
+    // scalar registers free across the K loop.
+    int seg_hi = 0, dp_tile = 0;
+    struct Share { int x, i, tile0, tiles, units, lo, hi, dp0; };
+    auto share_of = [&](unsigned bid) {
+        Share sh;
+        sh.x = (int)(bid % g.sk_xcds);
+        sh.i = (int)(bid / g.sk_xcds);
+        const int total = tiles * g.batch;
+        const int q = total / g.sk_xcds, rem = total % g.sk_xcds;
+        sh.tile0 = sh.x < rem ? sh.x * (q + 1) : rem * (q + 1) + (sh.x - rem) * q;
+        sh.tiles = q + (sh.x < rem ? 1 : 0);
+        const int rounds = sh.tiles / g.sk_wpx, left = sh.tiles - rounds * g.sk_wpx;
+        const int sk_tiles = left == 0 ? 0 : (rounds > 0 ? left + g.sk_wpx : left);
+        sh.units = sk_tiles * ksteps;
+        sh.lo = (int)((int64_t)sh.i * sh.units / g.sk_wpx);
+        sh.hi = (int)((int64_t)(sh.i + 1) * sh.units / g.sk_wpx);
+        sh.dp0 = sk_tiles + sh.i;
+        return sh;
+    };
+    if (SK) {
+        const Share sh = share_of(blockIdx.x);
+        seg_hi = sh.hi;
+        dp_tile = sh.dp0;
+        if (seg_hi <= sh.lo && dp_tile >= sh.tiles) return;
+    }
+
+    do {
+    // Everything a thread derives from its id is derived again for every
+    // segment (the empty asm hides that it never changes): hoisted out of the
+    // segment loop, those addresses would stay live across it and spill.
+    int tid = threadIdx.x;
+    unsigned bid = blockIdx.x;
+    if (SK) {
+        asm volatile("" : "+v"(tid));
+        asm volatile("" : "+s"(gp));
+        asm volatile("" : "+s"(bid));
+    }
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
+    const int r = lane & 31, h = lane >> 5;
+    // float4 slots of this lane's A row blocks and B column blocks
+    int a_row[TM], b_row[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a_row[i] = lds_row(wm * (32 * TM) + 32 * i + r);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b_row[j] = lds_row(wn * (32 * TN) + 32 * j + r);
 
-    // ---- workgroup -> (tile, batch, slice) ---------------------------------
-    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
-    // Renumber so that every XCD works on one contiguous run of tiles, then
-    // walk tiles in column-grouped order so concurrently resident tiles share
-    // A row panels and B column panels in that L2.
-    int64_t pid = blockIdx.x;
-    {
+    int64_t pid;
+    int role, k_begin, k_end, slice = 0;
+    // ROLE_FINISH: fin = c_first | c_count << 15, the workgroups (index within
+    // the XCD) whose partials belong to this tile; bit 30 of fin: more segments follow
+    int fin = 0;
+    if (!SK) {
+        // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
+        // Renumber so that every XCD works on one contiguous run of tiles.
+        pid = blockIdx.x;
         const int64_t total = gridDim.x;
-        const int64_t q = total >> 3, r = total & 7;
+        const int64_t q = total >> 3, rr = total & 7;
         const int64_t x = pid & 7, i = pid >> 3;
-        pid = (x < r ? x * (q + 1) : r * (q + 1) + (x - r) * q) + i;
+        pid = (x < rr ? x * (q + 1) : rr * (q + 1) + (x - rr) * q) + i;
+        role = g.split_k > 1 ? ROLE_SLICE : ROLE_FULL;
+        k_begin = 0;  // set below from the slice
+        k_end = 0;
+    } else {
+        const Share sh = share_of(bid);
+        if (seg_hi > sh.lo) {
+            const int lt = (seg_hi - 1) / ksteps;
+            const int tstart = lt * ksteps;
+            const int sb = sh.lo > tstart ? sh.lo : tstart;
+            const int kb = sb - tstart, ke = seg_hi - tstart;
+            pid = sh.tile0 + lt;
+            role = ke < ksteps ? ROLE_PART : (kb == 0 ? ROLE_FULL : ROLE_FINISH);
+            if (role == ROLE_FINISH) {
+                const int c_first = (int)((((int64_t)tstart + 1) * g.sk_wpx - 1) / sh.units);  // owner of the tile's first K step
+                fin = c_first | (sh.i - c_first) << 15;
+            }
+            k_begin = kb * BK;
+            k_end = min(g.K, ke * BK);
+            seg_hi = sb;
+        } else {
+            pid = sh.tile0 + dp_tile;
+            dp_tile += g.sk_wpx;
+            role = ROLE_FULL;
+            k_begin = 0;
+            k_end = g.K;
+        }
+        if (seg_hi > sh.lo || dp_tile < sh.tiles) fin |= 1 << 30;
     }
-    const int tiles = g.tiles_m * g.tiles_n;
+    // Tiles are walked in column-grouped order so that concurrently resident
+    // tiles share A row panels and B column panels in the XCD's L2.
     const int z = (int)(pid / tiles);
     int t = (int)(pid - (int64_t)z * tiles);
-    const int batch = z / g.split_k;
-    const int slice = z - batch * g.split_k;
+    int batch = z;
+    if (!SK) {
+        batch = z / g.split_k;
+        slice = z - batch * g.split_k;
+        k_begin = slice * g.k_per_slice;
+        k_end = min(g.K, k_begin + g.k_per_slice);
+    }
     int tm, tn;
     {
         const int GROUP = 8;
@@ -201,8 +329,6 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         tn = in_group / gsz;
     }
     const int m0 = tm * BM, n0 = tn * BN;
-    const int k_begin = slice * g.k_per_slice;
-    const int k_end = min(g.K, k_begin + g.k_per_slice);
     const int klen = max(k_end - k_begin, 0);
     const int nkt = (klen + BK - 1) / BK;
 
@@ -258,13 +384,6 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     }
     __syncthreads();
 
-    const int r = lane & 31, h = lane >> 5;
-    // float4 slots of this lane's A row blocks and B column blocks
-    int a_row[TM], b_row[TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i) a_row[i] = lds_row(wm * (32 * TM) + 32 * i + r);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) b_row[j] = lds_row(wn * (32 * TN) + 32 * j + r);
     constexpr int NCHUNK = KQ / 2;  // chunks of 8 K values
 
     // One chunk = 8 K values = 4 groups of TM x TN MFMAs (group j uses element
@@ -348,7 +467,7 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     // short-K, output-heavy products).
     float *__restrict__ Cb;
     int64_t ldc;
-    const bool partial = g.split_k > 1;
+    const bool partial = role == ROLE_SLICE;
     if (partial) {
         Cb = g.ws + ((int64_t)slice * g.batch + batch) * (int64_t)g.M * g.N;
         ldc = g.N;
@@ -362,15 +481,34 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
     float *patch = reinterpret_cast<float *>(lds) + wave * (32 * PW);
     const int prow = lane / LANES_PER_ROW, pc4 = lane % LANES_PER_ROW;
-    const int col = n0 + wn * WN + 4 * pc4;
+    const int coll = wn * WN + 4 * pc4;  // column within the tile
+    const int col = n0 + coll;
     const bool vec_ok = partial ? ((g.N & 3) == 0)
                                 : ((ldc & 3) == 0 && (g.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(g.C) & 15) == 0);
     float bias4[4] = {0.f, 0.f, 0.f, 0.f};
-    if (!partial && g.epilogue != MNI_EPI_NONE) {
+    if (!partial && !(SK && role == ROLE_PART) && g.epilogue != MNI_EPI_NONE) {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             if (col + e < g.N) bias4[e] = g.bias[col + e];
     }
+    // Stream-K: a finisher makes sure the partials of its tile have arrived
+    // (they were parked at the very start of their owners' lives).
+    bool lost = false;
+    const int c_first = fin & 0x7fff, c_count = (fin >> 15) & 0x7fff;
+    const int sk_x = SK ? (int)(bid % g.sk_xcds) : 0;
+    if (SK && role == ROLE_FINISH) {
+        bool ok = true;
+        if (tid < c_count) {
+            const unsigned *mark = g.sk_flags + (sk_x + g.sk_xcds * (c_first + tid));
+            ok = false;
+            for (int spin = 0; spin < SK_WAIT_LIMIT; ++spin) {
+                if (load_mark(mark) == g.sk_epoch) { ok = true; break; }
+                __builtin_amdgcn_s_sleep(4);
+            }
+        }
+        lost = __syncthreads_or(!ok) != 0;
+    }
+    float *const slot = g.ws + (int64_t)bid * (BM * BN);  // ROLE_PART: where this workgroup parks its tile
     // all wavefronts are past their last LDS read (barrier at the end of the K loop)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -382,9 +520,29 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
 #pragma unroll
         for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
             const int lr = prow + ROWS_PER_PASS * pass;
-            const int row = m0 + wm * (32 * TM) + 32 * i + lr;
-            const float4 t = *reinterpret_cast<const float4 *>(patch + lr * PW + 4 * pc4);
-            float v[4] = {t.x, t.y, t.z, t.w};
+            const int rowl = wm * (32 * TM) + 32 * i + lr;  // row within the tile
+            const int row = m0 + rowl;
+            const float4 t4 = *reinterpret_cast<const float4 *>(patch + lr * PW + 4 * pc4);
+            float v[4] = {t4.x, t4.y, t4.z, t4.w};
+            if (SK && role == ROLE_PART) {
+                *reinterpret_cast<float4 *>(slot + rowl * BN + coll) = t4;
+                continue;
+            }
+            if (SK && role == ROLE_FINISH) {
+                // four partials requested at a time, added in workgroup order
+                for (int c0 = 0; c0 < c_count; c0 += 4) {
+                    float4 pv[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float *ps = g.ws + (int64_t)(sk_x + g.sk_xcds * (c_first + c0 + j)) * (BM * BN);
+                        pv[j] = c0 + j < c_count ? *reinterpret_cast<const float4 *>(ps + rowl * BN + coll)
+                                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { v[0] += pv[j].x; v[1] += pv[j].y; v[2] += pv[j].z; v[3] += pv[j].w; }
+                }
+                if (lost) v[0] = v[1] = v[2] = v[3] = __builtin_nanf("");
+            }
             if (row < g.M && col < g.N) {
                 float *dst = Cb + (int64_t)row * ldc + col;
                 if (!partial) {
@@ -411,13 +569,25 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         }
         __syncthreads();
     }
+    if (SK && role == ROLE_PART) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of the tile has reached L2
+        __syncthreads();
+        if (tid == 0) g.sk_flags[bid] = g.sk_epoch;
+    }
+    if (!(fin >> 30)) break;
+    } while (SK);  // segments
+#undef g
 }
 
 template <int TM, int TN>
 static void launch_modes(const GemmLaunch &g, int amode, int bmode, dim3 grid) {
     dim3 block(NTHREADS);
     hipStream_t s = ctx().stream;
-#define MNI_LAUNCH(AM, BMO) hipLaunchKernelGGL((gemm_mfma_kernel<AM, BMO, TM, TN>), grid, block, 0, s, g)
+#define MNI_LAUNCH(AM, BMO)                                                                        \
+    do {                                                                                           \
+        if (g.streamk) hipLaunchKernelGGL((gemm_mfma_kernel<AM, BMO, TM, TN, true>), grid, block, 0, s, g);   \
+        else hipLaunchKernelGGL((gemm_mfma_kernel<AM, BMO, TM, TN, false>), grid, block, 0, s, g);            \
+    } while (0)
     if (amode == 2 || bmode == 2) MNI_LAUNCH(2, 2);
     else if (amode == 0 && bmode == 0) MNI_LAUNCH(0, 0);
     else if (amode == 0 && bmode == 1) MNI_LAUNCH(0, 1);
@@ -428,8 +598,13 @@ static void launch_modes(const GemmLaunch &g, int amode, int bmode, dim3 grid) {
 
 // tile_m / tile_n: 128 or 64 (g.tiles_m / g.tiles_n must be counted in those units)
 int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int tile_n) {
-    const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * g.batch * g.split_k;
-    if (blocks <= 0) return MNI_OK;
+    if ((int64_t)g.tiles_m * g.tiles_n * g.batch <= 0) return MNI_OK;
+    if (g.streamk) {
+        // what the kernel's arithmetic assumes about its grid and buffers
+        if (g.split_k != 1 || g.sk_xcds < 1 || g.sk_wpx < 1 || g.sk_wpx > NTHREADS || !g.ws || !g.sk_flags)
+            return set_error(MNI_ERR_INVALID, "sgemm: inconsistent stream-K launch");
+    }
+    const int64_t blocks = g.streamk ? (int64_t)g.sk_xcds * g.sk_wpx : (int64_t)g.tiles_m * g.tiles_n * g.batch * g.split_k;
     if (blocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "sgemm: too many tiles (%lld)", (long long)blocks);
     dim3 grid((unsigned)blocks);
     if (tile_m == 128 && tile_n == 128) launch_modes<2, 2>(g, amode, bmode, grid);
@@ -441,5 +616,7 @@ int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int 
 }
 
 int gemm_mfma_tile_k() { return BK; }
+// 128-wide tiles: two waves per SIMD by registers (and two tiles' LDS); 64 x 64: four.
+int gemm_mfma_resident_per_cu(int tile_m, int tile_n) { return tile_m * tile_n > 64 * 64 ? 2 : 4; }
 
 }  // namespace mni

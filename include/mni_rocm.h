@@ -92,11 +92,15 @@ typedef struct {
 } mni_operand;
 
 enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_GELU = 3 };
-/* MFMA = the MFMA tile kernel with its own choice of tile; MFMA_SMALL = the same
- * kernel forced to 64 x 64 tiles; SKINNY = the bandwidth kernels (error if the
- * shape or layout is not eligible); SKINNY_TWO_PASS = the same with the K-slice
- * partials summed by a second launch instead of inside the first. */
-enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4 };
+/* MFMA = the MFMA tile kernel, one workgroup per tile and K slice, 128-wide tiles;
+ * MFMA_SMALL = the same forced to 64 x 64 tiles; MFMA_STREAMK = the tile kernel
+ * with the K steps of all tiles dealt evenly over a resident grid (error if the
+ * device's workgroup-to-XCD mapping was not confirmed); SKINNY = the bandwidth
+ * kernels (error if the shape or layout is not eligible); SKINNY_TWO_PASS = the
+ * same with the K-slice partials summed by a second launch instead of inside
+ * the first.  AUTO picks among them. */
+enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
+       MNI_ALGO_MFMA_STREAMK = 5 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),

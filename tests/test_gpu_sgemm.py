@@ -226,6 +226,75 @@ def test_empty_and_zero_k(dev, rocm):
     rocm.sgemm(3, 0, 3, None, None, None)
 
 
+# ---- stream-K distribution of the tile kernel -------------------------------------------
+# Shapes that land in each form of the stream-K grid on a 256-CU / 8-XCD device:
+# a pure stream-K region (fewer tiles than resident workgroups), whole rounds plus a
+# region, ragged tile counts per XCD, edge tiles and K tails, 64 x 64 tiles.
+STREAMK_SHAPES = [(768, 776, 1000), (1000, 1000, 1000), (1500, 1300, 520), (4096, 768, 768), (2100, 2050, 300), (640, 3000, 777),
+                  (520, 260, 4100)]
+
+
+@pytest.mark.parametrize("m,n,k", STREAMK_SHAPES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_streamk_integer_exact_all_layouts(dev, m, n, k, ta, tb):
+    a = synth.small_ints(m + k, (k, m) if ta else (m, k), 3)
+    b = synth.small_ints(n + k, (n, k) if tb else (k, n), 3, stream=1)
+    want = ((a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(np.float32)
+    for algo in (N.ALGO_MFMA_STREAMK, N.ALGO_AUTO):
+        assert np.array_equal(run_gemm(dev, a, b, ta, tb, algo=algo)[0], want), algo
+
+
+def test_streamk_normal_inputs_batched_epilogue_accumulate(dev, rocm, oracle_native):
+    a = synth.normal(1, (3, 700, 900))
+    b = synth.normal(2, (1, 900, 650), stream=1)                      # one B for every batch (batch % 1)
+    bias = synth.normal(3, (650,), stream=2)
+    got = run_gemm(dev, a, b, algo=N.ALGO_MFMA_STREAMK, bias=dev.put(bias), epilogue=N.EPI_BIAS_RELU)
+    for i in range(3):
+        want = np.maximum(oracle_native.sgemm_ikj(a[i], b[0]) + bias, 0)
+        assert max_err(got[i], want) <= gemm_tol(900, a, b)
+    # accumulate: C += A B, with a padded ldc that must stay untouched
+    a2, b2 = synth.small_ints(4, (1100, 600), 3), synth.small_ints(5, (600, 1030), 3, stream=1)
+    c0 = synth.small_ints(6, (1100, 1040), 3, stream=2)
+    dA, dB, dC = dev.put(a2), dev.put(b2), dev.put(c0)
+    rocm.sgemm(1100, 1030, 600, dA, dB, dC, ldc=1040, accumulate=True, algo=N.ALGO_MFMA_STREAMK)
+    out = rocm.to_host(dC, (1100, 1040))
+    assert np.array_equal(out[:, :1030], c0[:, :1030] + (a2.astype(np.int64) @ b2.astype(np.int64)).astype(np.float32))
+    assert np.array_equal(out[:, 1030:], c0[:, 1030:])
+
+
+def test_streamk_repeats_and_agrees_with_the_tile_per_workgroup_form(dev, rocm):
+    # every launch marks arrivals with a fresh value, so back-to-back launches (also of
+    # other shapes and of the skinny kernel, which shares the marks) cannot see old ones
+    a, b = synth.normal(7, (1300, 1100)), synth.normal(8, (1100, 900), stream=1)
+    base = run_gemm(dev, a, b, algo=N.ALGO_MFMA)[0]
+    dA, dB = dev.put(a), dev.put(b)
+    dC = dev.empty(1300 * 900)
+    x, w = dev.put(synth.normal(9, (4, 4096))), dev.put(synth.normal(10, (4096, 512), stream=1))
+    dY = dev.empty(4 * 512)
+    for it in range(6):
+        rocm.fill(dC, -3.0, 1300 * 900)
+        rocm.sgemm(1300, 900, 1100, dA, dB, dC, algo=N.ALGO_MFMA_STREAMK)
+        if it % 2:
+            rocm.sgemm(4, 512, 4096, x, w, dY)                                 # skinny single-launch kernel in between
+        got = rocm.to_host(dC, (1300, 900))
+        assert max_err(got, base) <= gemm_tol(1100, a, b) * 1e-2              # same products, another order of the K sum
+        assert np.all(np.isfinite(got))
+    first = rocm.to_host(dC, (1300, 900)).copy()
+    rocm.sgemm(1300, 900, 1100, dA, dB, dC, algo=N.ALGO_MFMA_STREAMK)
+    assert np.array_equal(rocm.to_host(dC, (1300, 900)), first)              # the sum order is fixed by the shape
+
+
+def test_streamk_is_refused_where_it_cannot_work(dev, rocm):
+    a, b = dev.put(np.ones((64, 64), np.float32)), dev.put(np.ones((64, 64), np.float32))
+    c = dev.empty(64 * 64)
+    with pytest.raises(N.MniError, match="too small"):
+        rocm.sgemm(64, 64, 64, a, b, c, algo=N.ALGO_MFMA_STREAMK)
+    with pytest.raises(N.MniError, match="split_k"):
+        rocm.sgemm(64, 64, 64, a, b, c, algo=N.ALGO_MFMA_STREAMK, split_k=2)
+    rocm.sgemm(64, 64, 64, a, b, c)                                           # the planner falls back by itself
+    assert np.all(rocm.to_host(c, (64, 64)) == 64.0)
+
+
 # ---- skinny kernels ----------------------------------------------------------------
 
 def test_single_launch_skinny_path_is_available(rocm):
