@@ -241,6 +241,90 @@ def bench_extras(r):
         out["kv_decode_8x32x128_hist4096_" + ("int8" if quantized else "fp32")] = {"us": us, "GB/s": by / us / 1e3}
         cache.free()
         api.native.gcTensors([])
+    # language-model training step: 2 blocks of width 768 (12 heads), 8 x 512 tokens, vocabulary 8192;
+    # dataset windows, embeddings, dropout, attention, residual + layernorm, GELU MLP, cross-entropy on
+    # buffered targets, clipped AdamW -- everything device-resident
+    api.native.resetEngine()
+    nat = api.native
+    V, D, H, Tn, Bn, L = 8192, 768, 12, 512, 8, 2
+    hd_ = D // H
+    nat.seed(1)
+    u = lambda seed, shape, b: synth.uniform(seed, shape, -b, b)
+    lin = lambda sd, i, o, act=None: api.Linear(i, o, weight=u(sd, (i, o), 1 / math.sqrt(i)), bias=np.zeros(o, np.float32), fused=True, activation=act)
+    tok, pos = api.Embedding(V, D, weight=u(1, (V, D), 0.05)), api.Embedding(Tn, D, weight=u(2, (Tn, D), 0.05))
+    layers = [dict(q=lin(10 + l, D, D), k=lin(20 + l, D, D), v=lin(30 + l, D, D), proj=lin(40 + l, D, D), fc=lin(50 + l, D, 4 * D, "gelu"),
+                   out=lin(60 + l, 4 * D, D), g1=api.Parameter(T(np.ones(D, np.float32), True)), b1=api.Parameter(T(np.zeros(D, np.float32), True)),
+                   g2=api.Parameter(T(np.ones(D, np.float32), True)), b2=api.Parameter(T(np.zeros(D, np.float32), True))) for l in range(L)]
+    head = lin(3, D, V)
+    lm_params = [tok.weight, pos.weight] + head.parameters()
+    for ly in layers:
+        for kname in ("q", "k", "v", "proj", "fc", "out"):
+            lm_params += ly[kname].parameters()
+        lm_params += [ly["g1"], ly["b1"], ly["g2"], ly["b2"]]
+    lm_opt = api.Adam(lm_params, lr=1e-3)
+    ds = nat.createDataset((np.arange(1 << 20, dtype=np.int64) * 2654435761 % V).astype(np.int32))
+    posidx = [list(range(Tn))] * Bn
+    heads = lambda t: t.view(Bn, Tn, H, hd_).permute(0, 2, 1, 3).contiguous().view(Bn * H, Tn, hd_)
+
+    def lm_step():
+        inp, tgt = nat.sampleBatch(ds, Tn, Bn)
+        h = api.dropout(tok.forwardGpu(inp, Bn, Tn).add(pos.forward(posidx)), 0.1)
+        for ly in layers:
+            att = api.flashAttention(heads(ly["q"].forward(h)), heads(ly["k"].forward(h)), heads(ly["v"].forward(h)), 1 / math.sqrt(hd_), True)
+            att = att.view(Bn, H, Tn, hd_).permute(0, 2, 1, 3).contiguous().view(Bn, Tn, D)
+            h1 = api.residualLayerNorm(api.dropout(ly["proj"].forward(att), 0.1), h, ly["g1"].value, ly["b1"].value)
+            h = api.residualLayerNorm(api.dropout(ly["out"].forward(ly["fc"].forward(h1)), 0.1), h1, ly["g2"].value, ly["b2"].value)
+        loss = api.crossEntropyLossGpu(head.forward(h), tgt)
+        lm_opt.zeroGrad()
+        loss.backward()
+        lm_opt.step(1.0)
+        nat.freeIntBuffer(inp)
+        nat.freeIntBuffer(tgt)
+
+    def keep_lm():
+        ids = [p.value._id for p in lm_params]
+        return ids + [g for g in (nat.getGrad(p.value._id) for p in lm_params) if g is not None]
+    ms = time_step(lm_step, keep_lm, 10, 3)
+    per_tok = 6.0 * (L * 12 * D * D + D * V) + L * 3.5 * 4 * Tn * D  # matmul FLOPs per token, fwd + bwd (attention counted dense)
+    out["lm_step_2x768_8x512_vocab8192"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3, "matmul_TFLOP/s": per_tok * Bn * Tn / ms / 1e9}
+    # token-side kernels on their own (wall clock per call incl. host issue; bytes = algorithmic)
+    api.native.resetEngine()
+    xt, rt = T(synth.normal(7, (8192, 768))), T(synth.normal(7, (8192, 768), stream=1))
+    gm, bt = T(np.ones(768, np.float32)), T(np.zeros(768, np.float32))
+    wemb = T(u(8, (32768, 768), 0.05), True)
+    idx = np.asarray(synth.integers(9, (8192,), 0, 32768), dtype=np.int64)
+
+    def keep_tok():
+        g = nat.getGrad(wemb._id)
+        return [t._id for t in (xt, rt, gm, bt, wemb)] + ([g] if g is not None else [])
+
+    def timed(fn, n=20):
+        # every call is followed by a collection (untimed), as in a training loop, so buffers come from the allocator's cache
+        total = 0.0
+        for it in range(n + 3):
+            r.sync()
+            t0 = time.perf_counter()
+            fn()
+            r.sync()
+            if it >= 3:
+                total += time.perf_counter() - t0
+            nat.gcTensors(keep_tok())
+        return total / n * 1e6
+    nb = 8192 * 768 * 4.0
+    us_d = timed(lambda: nat.dropoutOp(xt._id, 0.1, True))
+    us_l = timed(lambda: nat.residualLayernorm(xt._id, rt._id, gm._id, bt._id, 1e-5))
+    us_e = timed(lambda: nat.embeddingForward(wemb._id, idx, 8, 1024))
+
+    def emb_fb():
+        nat.zeroGrad([wemb._id])
+        api.Tensor(nat.embeddingForward(wemb._id, idx, 8, 1024)).mul(xt.view(8, 1024, 768)).sum().backward()
+    us_eb = timed(emb_fb, 10)
+    out["token_ops_8192x768"] = {
+        "dropout_us": us_d, "dropout_GB/s": 2 * nb / us_d / 1e3,
+        "residual_layernorm_us": us_l, "residual_layernorm_GB/s": 4 * nb / us_l / 1e3,
+        "embedding_forward_us": us_e, "embedding_forward_GB/s": 2 * nb / us_e / 1e3,
+        "embedding_forward_backward_vocab32768_us": us_eb,
+        "note": "one call, then a sync; embedding_forward includes the host-to-device copy of 8192 indices"}
     api.native.resetEngine()
     return out
 

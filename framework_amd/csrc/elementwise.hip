@@ -126,6 +126,26 @@ __global__ void gather_kernel(float *__restrict__ dst, const float *__restrict__
         dst[i] = src[off];
     }
 }
+// The same when the innermost dim has unit stride in the source and a length
+// that is a multiple of 4, with 16-byte aligned pieces (heads split off and
+// merged back, [b, t, h, d] <-> [b, h, t, d]): one 16-byte access per four
+// elements and a quarter of the index arithmetic.  d.shape / d.strides describe
+// the dims above the innermost one; inner4 = innermost length / 4.
+__global__ void gather4_kernel(float4 *__restrict__ dst, const float *__restrict__ src, const GatherDesc d, int64_t inner4,
+                               int64_t n4) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += step) {
+        int64_t rem = i / inner4;
+        int64_t off = (i - rem * inner4) * 4;
+        for (int k = d.ndim - 1; k >= 0; --k) {
+            const int64_t c = rem % d.shape[k];
+            rem /= d.shape[k];
+            off += c * d.strides[k];
+        }
+        dst[i] = *reinterpret_cast<const float4 *>(src + off);
+    }
+}
 // Batched 2-D transpose through LDS for the common "swap the last two dims"
 // view: src element (b, r, c) at b*bs + r*1 + c*cs_ (row axis contiguous in
 // memory), dst contiguous [b][r][c].
@@ -181,6 +201,17 @@ int k_strided_copy(float *dst, const float *src, const int64_t *shape, const int
         }
     }
     GatherDesc d;
+    if (ndim >= 1 && strides[ndim - 1] == 1 && (shape[ndim - 1] % 4) == 0 && al16(dst) && al16(src)) {
+        bool aligned = true;
+        for (int i = 0; i < ndim - 1; ++i) aligned = aligned && (strides[i] % 4) == 0;
+        if (aligned) {
+            d.ndim = ndim - 1;
+            for (int i = 0; i < ndim - 1; ++i) { d.shape[i] = shape[i]; d.strides[i] = strides[i]; }
+            hipLaunchKernelGGL(gather4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+                               reinterpret_cast<float4 *>(dst), src, d, shape[ndim - 1] / 4, n / 4);
+            return check_launch("gather4");
+        }
+    }
     d.ndim = ndim;
     for (int i = 0; i < ndim; ++i) { d.shape[i] = shape[i]; d.strides[i] = strides[i]; }
     hipLaunchKernelGGL(gather_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, dst, src, d, n);

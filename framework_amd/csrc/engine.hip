@@ -50,8 +50,10 @@ struct Tensor {
     BufP adam_m, adam_v;
     // A gradient that is known to hold only zeros (fresh, or just cleared):
     // the first accumulation into it shares the incoming buffer instead of
-    // adding to zeros.  Every in-place writer goes through make_unique().
-    bool known_zero = false;
+    // adding to zeros, and the zeros themselves are only written
+    // (zero_filled) when somebody reads the tensor before that: get() does it.
+    // Every in-place writer goes through make_unique().
+    bool known_zero = false, zero_filled = false;
 };
 
 enum Op {  // subset of src/native/src/autograd.rs:28-62 plus the fused Linear
@@ -167,13 +169,22 @@ static bool broadcast_shape(const Shape &a, const Shape &b, Shape *out) {  // ut
 }
 
 // ---- store ----------------------------------------------------------------------
-static Tensor *get(uint32_t id) {  // tensor.rs:115-117
+// The slot as it is: a cleared gradient may not have had its zeros written yet.
+static Tensor *peek(uint32_t id) {
     Engine &e = eng();
     if (id >= e.tensors.size() || !e.tensors[id].live) {
         set_error(MNI_ERR_FREED, "tensor already freed (id %u)", id);
         return nullptr;
     }
     return &e.tensors[id];
+}
+static Tensor *get(uint32_t id) {  // tensor.rs:115-117
+    Tensor *t = peek(id);
+    if (t && t->known_zero && !t->zero_filled) {
+        if (k_fill(t->buf->p, 0.0f, (int64_t)t->buf->n) != MNI_OK) return nullptr;
+        t->zero_filled = true;
+    }
+    return t;
 }
 // Shapes are taken by value: a caller may pass a reference into the slot
 // vector, which emplace_back can reallocate.
@@ -250,16 +261,19 @@ static int64_t ensure_grad(uint32_t id) {  // tensor.rs:144-152
     if (!t) return -1;
     if (t->grad >= 0) return t->grad;
     const Shape shape = t->shape;
-    const uint32_t g = zeros(shape);
-    if (g == MNI_BAD_ID) return -1;
-    get(g)->known_zero = true;
+    BufP b = new_buf((size_t)shape_size(shape));
+    if (!b) return -1;
+    const uint32_t g = insert_contig(std::move(b), shape);
+    Tensor *G = peek(g);
+    G->known_zero = true;  // zeros on demand
+    G->zero_filled = false;
     get(id)->grad = g;
     return g;
 }
 // tensor.rs:475-491 accumulate_grad / :493-508 add_inplace: raw buffer order,
 // src.size elements.
 static int add_into(uint32_t dst, uint32_t src) {
-    Tensor *s = get(src), *d = get(dst);
+    Tensor *s = get(src), *d = peek(dst);
     if (!s || !d) return MNI_ERR_FREED;
     if ((int64_t)d->buf->n < s->size) return set_error(MNI_ERR_INVALID, "add_inplace: destination smaller than source");
     if (d->known_zero && d->buf->n == s->buf->n && s->size == (int64_t)s->buf->n) {
@@ -267,6 +281,7 @@ static int add_into(uint32_t dst, uint32_t src) {
         d->known_zero = false;
         return MNI_OK;
     }
+    if (!get(dst)) return MNI_ERR_HIP;  // writes the pending zeros
     MNI_TRY(make_unique(*d));
     return k_axpy(d->buf->p, s->buf->p, 1.0f, s->size);
 }
@@ -1910,16 +1925,15 @@ int mni_zero_grad(const uint32_t *ids, size_t n) {
         Tensor *t = get(ids[p]);
         if (!t) return MNI_ERR_FREED;
         if (t->grad < 0) continue;
-        Tensor *g = get((uint32_t)t->grad);
+        Tensor *g = peek((uint32_t)t->grad);
         if (!g) return MNI_ERR_FREED;
-        bool fill = !g->known_zero;
+        if (g->known_zero) continue;
         if (g->buf.use_count() > 1) {  // shared: replace instead of copy + clear
             g->buf = new_buf(g->buf->n);
             if (!g->buf) return MNI_ERR_NOMEM;
-            fill = true;
         }
-        if (fill) MNI_TRY(k_fill(g->buf->p, 0.0f, (int64_t)g->buf->n));
-        g->known_zero = true;
+        g->known_zero = true;  // the zeros are written when somebody asks for them
+        g->zero_filled = false;
     }
     return MNI_OK;
 }

@@ -517,7 +517,8 @@ class Native:
         return out
 
     def embeddingForward(self, weight, indices, batch, seqLen):
-        return self._id(self.lib.mni_embedding_forward(weight, _i64_array(indices), len(indices), batch, seqLen))
+        idx = np.ascontiguousarray(indices, dtype=np.int64)  # a numpy array passes through without a per-element copy
+        return self._id(self.lib.mni_embedding_forward(weight, idx.ctypes.data_as(_i64p), idx.size, batch, seqLen))
 
     def embeddingForwardGpu(self, weight, intBufId, batch, seqLen):
         return self._id(self.lib.mni_embedding_forward_gpu(weight, intBufId, batch, seqLen))
