@@ -330,9 +330,9 @@ def bench_extras(r):
 
 
 def run_for_counters(r, which):
-    """Launch sequence for hardware-counter runs: gather_kernel x3 on a
-    contiguous 16M-float buffer (64 MiB read, 64 MiB written: the yardstick the
-    counters are scaled by), then the product x5."""
+    """Launch sequence for hardware-counter runs: the strided-copy kernel x3 on
+    a contiguous 16M-float buffer (64 MiB read, 64 MiB written: the yardstick
+    the counters are scaled by), then the product x5."""
     n = 4096 * 4096
     src = r.to_device(synth.normal(9, (n,)))
     dst = r.malloc(n * 4)
@@ -342,6 +342,11 @@ def run_for_counters(r, which):
         a, b = r.to_device(synth.normal(1, (4096, 4096))), r.to_device(synth.normal(1, (4096, 4096), stream=1))
         for _ in range(5):
             r.sgemm(4096, 4096, 4096, a, b, dst)
+    elif which == "streamk":
+        # a mid-size product whose 192 tiles do not fill a round: the planner deals its K steps (stream-K)
+        a, b = r.to_device(synth.normal(1, (4096, 3072))), r.to_device(synth.normal(1, (3072, 768), stream=1))
+        for _ in range(5):
+            r.sgemm(4096, 768, 3072, a, b, dst)
     else:
         x, w = r.to_device(synth.normal(4, (4, 4096), 0.02)), r.to_device(synth.normal(4, (4096, 4096), 0.02, stream=1))
         for _ in range(5):
@@ -386,7 +391,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
-    ap.add_argument("--counters", choices=["gemm", "gemv"], default=None,
+    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk"], default=None,
                     help="for rocprofv3 --pmc runs: launch a copy kernel of known size (64 MiB read + 64 MiB "
                          "written) 3 times, then the chosen product 5 times, and exit")
     args = ap.parse_args()
@@ -410,7 +415,7 @@ def main():
         "config": {"workload": "single fp32 matmul A[4096,4096] x B[4096,4096], A,B ~ N(0,1) seed 1, row-major, forward only",
                    "M": 4096, "N": 4096, "K": 4096, "device": info["name"].strip(), "compute_units": info["compute_units"],
                    "max_err_vs_f64_sample": err},
-        "roofline": {"bound": "mfma", "kernel": "gemm_mfma_kernel<0, 1, 2, 2>", "achieved": achieved,
+        "roofline": {"bound": "mfma", "kernel": "gemm_mfma_kernel<0, 1, 2, 2, false>", "achieved": achieved,
                      "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MATRIX_TFLOPS,
                      "kernel_ms": kernel_ms, "algorithmic_flops": flops, "traffic": MEASURED_HBM_BYTES_4096},
     }
