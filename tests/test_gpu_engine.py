@@ -493,3 +493,38 @@ def test_entry_points_serialise_concurrent_callers(rocm_native):
     for t in threads:
         t.join()
     assert errors == []
+
+
+def test_cleared_gradients_read_as_zeros_and_accumulate_from_zero(gpu):
+    # zeroGrad only marks a gradient; the zeros appear when it is read, and the first accumulation replaces them
+    Tn = gpu.Tensor
+    w = Tn.fromFloat32(np.arange(6, dtype=np.float32).reshape(2, 3), [2, 3]).setRequiresGrad(True)
+    u = Tn.fromFloat32(np.ones((2, 3), np.float32), [2, 3]).setRequiresGrad(True)
+    x = Tn.fromFloat32(np.array([[1, 2, 3], [4, 5, 6]], np.float32), [2, 3])
+    w.mul(x).sum().backward()
+    assert np.array_equal(w.grad.numpy(), x.numpy()) and u.grad is None
+    gpu.native.zeroGrad([w._id, u._id])
+    assert not np.any(w.grad.numpy())                                    # read before any accumulation: zeros
+    gview = w.grad.permute(1, 0)                                         # a view of the cleared gradient
+    w.mul(x).sum().backward()
+    w.mul(x).sum().backward()                                            # second accumulation adds
+    assert np.array_equal(w.grad.numpy(), 2 * x.numpy())
+    assert not np.any(gview.numpy())                                     # the view kept the zeros it was taken from
+    gpu.native.zeroGrad([w._id])
+    gpu.native.zeroGrad([w._id])                                         # twice in a row
+    assert gpu.native.gradNorm([w._id, u._id]) == 0.0                    # a reader other than toFloat32
+    w.mul(x).sum().backward()
+    assert np.array_equal(w.grad.numpy(), x.numpy())
+    # a gradient shared with the tape's tensor is not corrupted by scaling it in place afterwards
+    gpu.native.zeroGrad([w._id])
+    loss = w.mul(x).sum()
+    loss.backward()
+    assert gpu.native.scaleGrads([w._id], 0.5) is False
+    assert np.array_equal(w.grad.numpy(), 0.5 * x.numpy()) and np.array_equal(x.numpy(), np.array([[1, 2, 3], [4, 5, 6]], np.float32))
+    # an optimiser step on a parameter whose gradient stayed cleared leaves it alone (zero gradient, zero moments)
+    opt = gpu.Adam([gpu.Parameter(w), gpu.Parameter(u)], lr=0.1)
+    before = u.numpy().copy()
+    opt.zeroGrad()
+    w.mul(x).sum().backward()
+    opt.step()
+    assert np.array_equal(u.numpy(), before) and not np.array_equal(w.numpy(), np.arange(6, dtype=np.float32).reshape(2, 3))

@@ -480,6 +480,24 @@ def test_config2_4096_cubed(dev, rocm, oracle_native):
     assert np.max(np.abs(lhs - rhs)) <= 4096 * gemm_tol(4096, a, b)
 
 
+@pytest.mark.parametrize("m,n,k,ta,tb", [(4096, 768, 3072, False, False), (768, 3072, 4096, True, False), (4096, 768, 768, False, True),
+                                          (3000, 3000, 1000, False, False)])
+def test_streamk_at_training_sizes(dev, oracle_native, m, n, k, ta, tb):
+    # the mid-size products of a transformer step, which the planner hands to stream-K (128 x 128 and 64 x 64 tiles)
+    a = synth.normal(m, (k, m) if ta else (m, k))
+    b = synth.normal(n, (n, k) if tb else (k, n), stream=1)
+    A, B = (a.T if ta else a), (b.T if tb else b)
+    got = run_gemm(dev, a, b, ta, tb)[0]
+    rows = [0, 1, 127, 128, m // 2, m - 1]
+    assert max_err(got[rows], oracle_native.sgemm_ikj(np.ascontiguousarray(A[rows]), np.ascontiguousarray(B))) <= gemm_tol(k, a, b)
+    ones = np.ones(n)
+    lhs = got.astype(np.float64) @ ones                                        # C 1 = A (B 1): touches every element of C
+    rhs = A.astype(np.float64) @ (B.astype(np.float64) @ ones)
+    assert np.max(np.abs(lhs - rhs)) <= n * gemm_tol(k, a, b)
+    forced = run_gemm(dev, a, b, ta, tb, algo=N.ALGO_MFMA_STREAMK)[0]
+    assert max_err(forced, got) <= gemm_tol(k, a, b)
+
+
 def test_config5a_decode_gemv(dev, rocm):
     with open(os.path.join(GOLDEN, "config_samples.json")) as f:
         gold = json.load(f)["config5a"]
