@@ -151,5 +151,19 @@ int k_sumsq_partials(double *part, const float *g, int64_t n);
 int k_sumsq_finish(double *out, const double *part, int nparts);
 int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, float b1, float b2,
             float eps, float wd, float bc1, float bc2);
+// Many tensors in one launch.  Tensor i owns workgroups [block_start[i], block_start[i + 1]), one per
+// MULTI_CHUNK elements (multi_tensor_blocks(n[i]) of them).  k_sumsq_multi writes one partial per workgroup.
+constexpr int MULTI_MAX = 48;
+constexpr int MULTI_CHUNK = 4096;
+struct MultiTensor {
+    int count;
+    int block_start[MULTI_MAX + 1];
+    float *p[MULTI_MAX], *m[MULTI_MAX], *v[MULTI_MAX];
+    const float *g[MULTI_MAX];
+    int64_t n[MULTI_MAX];
+};
+int multi_tensor_blocks(int64_t n);
+int k_adamw_multi(const MultiTensor &t, float lr, float b1, float b2, float eps, float wd, float bc1, float bc2);
+int k_sumsq_multi(const MultiTensor &t, double *part);
 
 }  // namespace mni

@@ -1073,6 +1073,79 @@ int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, f
     return check_launch("adamw");
 }
 
+// The same for up to MULTI_MAX tensors in one launch (a training step updates
+// dozens of parameters, most of them a few hundred values long): the table
+// rides in the kernel arguments, a workgroup takes MULTI_CHUNK elements of the
+// tensor its index falls into.
+template <bool ADAM>
+__global__ void multi_tensor_kernel(const MultiTensor t, double *__restrict__ part, float lr, float b1, float b2, float eps,
+                                    float wd, float bc1, float bc2) {
+    int ti = 0;
+    while (ti + 1 < t.count && (int)blockIdx.x >= t.block_start[ti + 1]) ++ti;
+    const int64_t n = t.n[ti];
+    const int64_t lo = (int64_t)((int)blockIdx.x - t.block_start[ti]) * MULTI_CHUNK;
+    const int64_t hi = lo + MULTI_CHUNK < n ? lo + MULTI_CHUNK : n;
+    const float *__restrict__ g = t.g[ti];
+    if (ADAM) {
+        float *__restrict__ p = t.p[ti], *__restrict__ m = t.m[ti], *__restrict__ v = t.v[ti];
+        const bool vec = (n % 4) == 0;  // allocator blocks are 256-byte aligned; lo is a multiple of 4
+        auto upd = [&](float gv, float &pv, float &mv, float &vv) {
+            if (wd > 0.0f) pv *= 1.0f - lr * wd;
+            mv = b1 * mv + (1.0f - b1) * gv;
+            vv = b2 * vv + (1.0f - b2) * gv * gv;
+            const float m_hat = mv / bc1;
+            const float v_hat = vv / bc2;
+            pv = pv - lr * m_hat / (sqrtf(v_hat) + eps);
+        };
+        if (vec) {
+            for (int64_t i = lo + 4 * threadIdx.x; i < hi; i += 4 * blockDim.x) {
+                const float4 g4 = *reinterpret_cast<const float4 *>(g + i);
+                float4 p4 = *reinterpret_cast<float4 *>(p + i), m4 = *reinterpret_cast<float4 *>(m + i), v4 = *reinterpret_cast<float4 *>(v + i);
+                upd(g4.x, p4.x, m4.x, v4.x); upd(g4.y, p4.y, m4.y, v4.y); upd(g4.z, p4.z, m4.z, v4.z); upd(g4.w, p4.w, m4.w, v4.w);
+                *reinterpret_cast<float4 *>(p + i) = p4;
+                *reinterpret_cast<float4 *>(m + i) = m4;
+                *reinterpret_cast<float4 *>(v + i) = v4;
+            }
+        } else {
+            for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) upd(g[i], p[i], m[i], v[i]);
+        }
+    } else {
+        __shared__ double sh[4];
+        double sq = 0.0;
+        for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) { const double x = (double)g[i]; sq += x * x; }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+        if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = sq;
+        __syncthreads();
+        if (threadIdx.x == 0) part[blockIdx.x] = (sh[0] + sh[1]) + (sh[2] + sh[3]);
+    }
+}
+int multi_tensor_blocks(int64_t n) { return (int)((n + MULTI_CHUNK - 1) / MULTI_CHUNK); }
+static int multi_check(const MultiTensor &t) {
+    if (t.count < 1 || t.count > MULTI_MAX) return set_error(MNI_ERR_INVALID, "multi-tensor launch: %d tensors", t.count);
+    int at = 0;
+    for (int i = 0; i < t.count; ++i) {
+        if (t.block_start[i] != at || t.n[i] <= 0) return set_error(MNI_ERR_INVALID, "multi-tensor launch: inconsistent table");
+        at += multi_tensor_blocks(t.n[i]);
+    }
+    if (t.block_start[t.count] != at) return set_error(MNI_ERR_INVALID, "multi-tensor launch: inconsistent table");
+    return MNI_OK;
+}
+int k_adamw_multi(const MultiTensor &t, float lr, float b1, float b2, float eps, float wd, float bc1, float bc2) {
+    MNI_TRY(ensure_init());
+    MNI_TRY(multi_check(t));
+    hipLaunchKernelGGL(multi_tensor_kernel<true>, dim3(t.block_start[t.count]), dim3(TPB), 0, ctx().stream, t, (double *)nullptr, lr, b1,
+                       b2, eps, wd, bc1, bc2);
+    return check_launch("adamw_multi");
+}
+int k_sumsq_multi(const MultiTensor &t, double *part) {
+    MNI_TRY(ensure_init());
+    MNI_TRY(multi_check(t));
+    hipLaunchKernelGGL(multi_tensor_kernel<false>, dim3(t.block_start[t.count]), dim3(TPB), 0, ctx().stream, t, part, 0.f, 0.f, 0.f,
+                       0.f, 0.f, 0.f, 0.f);
+    return check_launch("sumsq_multi");
+}
+
 }  // namespace mni
 
 using namespace mni;

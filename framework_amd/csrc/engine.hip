@@ -10,6 +10,7 @@
 #include <math.h>
 #include <string.h>
 
+#include <algorithm>
 #include <map>
 #include <memory>
 #include <random>
@@ -1763,7 +1764,8 @@ static float powi_f32(float a, int b) {  // f32::powi (compiler-rt __powisf2)
 
 // ops/optimizer.rs:126-138 grad_norm
 static int grad_norm(const uint32_t *ids, size_t n, float *out) {
-    // Per-tensor partial sums land in one buffer; a single kernel adds them up.
+    // Workgroups of multi-tensor launches leave one partial sum each in one
+    // buffer; a single kernel adds them up.
     std::vector<Tensor *> gs;
     int64_t nparts = 0;
     for (size_t p = 0; p < n; ++p) {
@@ -1772,8 +1774,9 @@ static int grad_norm(const uint32_t *ids, size_t n, float *out) {
         if (T->grad < 0) continue;
         Tensor *G = get((uint32_t)T->grad);
         if (!G) return MNI_ERR_FREED;
+        if (G->size <= 0) continue;
         gs.push_back(G);
-        nparts += sumsq_blocks(G->size);
+        nparts += multi_tensor_blocks(G->size);
     }
     void *acc = nullptr;
     MNI_TRY(dev_alloc(&acc, (size_t)(nparts + 1) * sizeof(double)));
@@ -1781,9 +1784,21 @@ static int grad_norm(const uint32_t *ids, size_t n, float *out) {
     double *total = (double *)acc, *part = total + 1;
     MNI_TRY(k_fill((float *)total, 0.0f, 2));  // one double
     int64_t at = 0;
-    for (Tensor *G : gs) {
-        MNI_TRY(k_sumsq_partials(part + at, G->buf->p, G->size));
-        at += sumsq_blocks(G->size);
+    for (size_t first = 0; first < gs.size(); first += MULTI_MAX) {
+        MultiTensor t;
+        memset(&t, 0, sizeof t);
+        t.count = (int)std::min<size_t>(MULTI_MAX, gs.size() - first);
+        int blocks = 0;
+        for (int i = 0; i < t.count; ++i) {
+            Tensor *G = gs[first + i];
+            t.block_start[i] = blocks;
+            t.g[i] = G->buf->p;
+            t.n[i] = G->size;
+            blocks += multi_tensor_blocks(G->size);
+        }
+        t.block_start[t.count] = blocks;
+        MNI_TRY(k_sumsq_multi(t, part + at));
+        at += blocks;
     }
     MNI_TRY(k_sumsq_finish(total, part, (int)nparts));
     double sq = 0.0;
@@ -1796,6 +1811,19 @@ static int grad_norm(const uint32_t *ids, size_t n, float *out) {
 static int adamw_step(const uint32_t *ids, size_t n, float lr, float b1, float b2, float eps, float wd, uint32_t step) {
     const float bc1 = 1.0f - powi_f32(b1, (int)step);
     const float bc2 = 1.0f - powi_f32(b2, (int)step);
+    MultiTensor t;
+    memset(&t, 0, sizeof t);
+    std::vector<BufP> keep;  // gathered copies of non-contiguous gradients, alive until their launch is queued
+    int blocks = 0;
+    auto flush = [&]() -> int {
+        if (t.count == 0) return MNI_OK;
+        t.block_start[t.count] = blocks;
+        const int rc = k_adamw_multi(t, lr, b1, b2, eps, wd, bc1, bc2);
+        memset(&t, 0, sizeof t);
+        blocks = 0;
+        keep.clear();
+        return rc;
+    };
     for (size_t p = 0; p < n; ++p) {
         Tensor *T = get(ids[p]);
         if (!T) return MNI_ERR_FREED;
@@ -1805,6 +1833,8 @@ static int adamw_step(const uint32_t *ids, size_t n, float lr, float b1, float b
         BufP g = contiguous_buf(*G);
         if (!g) return MNI_ERR_NOMEM;
         const int64_t size = T->size;
+        if (size <= 0) continue;
+        if ((int64_t)g->n < size) return set_error(MNI_ERR_INVALID, "adamw: gradient smaller than its parameter");
         if (!T->adam_m) {
             T->adam_m = new_buf((size_t)size);
             T->adam_v = new_buf((size_t)size);
@@ -1813,9 +1843,17 @@ static int adamw_step(const uint32_t *ids, size_t n, float lr, float b1, float b
             MNI_TRY(k_fill(T->adam_v->p, 0.f, size));
         }
         MNI_TRY(make_unique(*T));
-        MNI_TRY(k_adamw(T->buf->p, T->adam_m->p, T->adam_v->p, g->p, size, lr, b1, b2, eps, wd, bc1, bc2));
+        // the same parameter twice in one list must see its first update: start a new launch
+        bool repeated = false;
+        for (int i = 0; i < t.count; ++i) repeated = repeated || t.p[i] == T->buf->p;
+        if (repeated || t.count == MULTI_MAX) MNI_TRY(flush());
+        const int i = t.count++;
+        t.block_start[i] = blocks;
+        t.p[i] = T->buf->p; t.m[i] = T->adam_m->p; t.v[i] = T->adam_v->p; t.g[i] = g->p; t.n[i] = size;
+        blocks += multi_tensor_blocks(size);
+        keep.push_back(std::move(g));
     }
-    return MNI_OK;
+    return flush();
 }
 
 static int scale_grads(const uint32_t *ids, size_t n, float scale) {
