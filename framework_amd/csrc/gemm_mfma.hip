@@ -558,7 +558,11 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
                         const float4 c = *reinterpret_cast<const float4 *>(dst);
                         v[0] += c.x; v[1] += c.y; v[2] += c.z; v[3] += c.w;
                     }
-                    *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                    // streaming store: C is written once and not read again by this kernel, so
+                    // it need not displace the operand panels in L2
+                    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+                    const f32x4_t o4 = {v[0], v[1], v[2], v[3]};
+                    __builtin_nontemporal_store(o4, reinterpret_cast<f32x4_t *>(dst));
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
