@@ -363,6 +363,7 @@ __global__ __launch_bounds__(ATT_TPB) void kv_decode_kernel(const KvDecode a) {
 // LPR neighbouring lanes -- 4 fp32 or 16 int8 values per lane -- so loads are
 // coalesced; a dot product is finished with log2(LPR) butterfly steps, and the
 // value pass keeps those 4 / 16 columns per lane.
+static constexpr int KV_UNROLL = 4;  // cache rows in flight per lane
 template <bool Q8, int LPR>
 __global__ __launch_bounds__(ATT_TPB) void kv_decode_vec_kernel(const KvDecode a) {
     constexpr int E = Q8 ? 16 : 4;         // elements per lane
@@ -397,19 +398,28 @@ __global__ __launch_bounds__(ATT_TPB) void kv_decode_vec_kernel(const KvDecode a
     float qv[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) qv[e] = l < pieces ? a.q[row * a.d + l * E + e] : 0.f;
-    // scores
-    for (int i0 = wave * RPP; i0 < n; i0 += (ATT_TPB / 64) * RPP) {
-        const int i = i0 + sub;
-        float part = 0.f;
-        if (i < n && l < pieces) {
-            float kv[E];
-            load(a.kc, a.ks, base + i, l, kv);
+    // scores: KV_UNROLL rows of the cache are requested before the first is used
+    // (one 16-byte load per lane in flight does not cover the memory latency)
+    constexpr int ROWS_PER_TRIP = (ATT_TPB / 64) * RPP;
+    for (int i0 = wave * RPP; i0 < n; i0 += ROWS_PER_TRIP * KV_UNROLL) {
+        float kv[KV_UNROLL][E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) part += qv[e] * kv[e];
+        for (int u = 0; u < KV_UNROLL; ++u) {
+            const int i = i0 + u * ROWS_PER_TRIP + sub;
+            if (i < n && l < pieces) load(a.kc, a.ks, base + i, l, kv[u]);
         }
 #pragma unroll
-        for (int off = LPR / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
-        if (i < n && l == 0) sc[i] = part * a.scale;
+        for (int u = 0; u < KV_UNROLL; ++u) {
+            const int i = i0 + u * ROWS_PER_TRIP + sub;
+            float part = 0.f;
+            if (i < n && l < pieces) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) part += qv[e] * kv[u][e];
+            }
+#pragma unroll
+            for (int off = LPR / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+            if (i < n && l == 0) sc[i] = part * a.scale;
+        }
     }
     __syncthreads();
     float m = -INFINITY;
@@ -429,12 +439,20 @@ __global__ __launch_bounds__(ATT_TPB) void kv_decode_vec_kernel(const KvDecode a
 #pragma unroll
     for (int e = 0; e < E; ++e) acc[e] = 0.f;
     if (lv < pieces) {
-        for (int i = grp; i < n; i += GROUPS) {
-            float vv[E];
-            load(a.vc, a.vs, base + i, lv, vv);
-            const float w = sc[i];
+        for (int i0 = grp; i0 < n; i0 += GROUPS * KV_UNROLL) {
+            float vv[KV_UNROLL][E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) acc[e] += w * vv[e];
+            for (int u = 0; u < KV_UNROLL; ++u)
+                if (i0 + u * GROUPS < n) load(a.vc, a.vs, base + i0 + u * GROUPS, lv, vv[u]);
+#pragma unroll
+            for (int u = 0; u < KV_UNROLL; ++u) {
+                const int i = i0 + u * GROUPS;
+                if (i < n) {
+                    const float w = sc[i];
+#pragma unroll
+                    for (int e = 0; e < E; ++e) acc[e] += w * vv[u][e];
+                }
+            }
         }
     }
 #pragma unroll
@@ -492,7 +510,7 @@ int k_kv_decode(float *out, const void *kc, const void *vc, const float *ks, con
     if (bh > 0x7fffffff || len > 0x7ffffff0) return set_error(MNI_ERR_INVALID, "kv cache decode: extent out of range");
     // enough workgroups to occupy the device, chunks of at most KV_CHUNK_MAX keys
     const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
-    int64_t splits = (2LL * cus + bh - 1) / bh;
+    int64_t splits = (4LL * cus + bh - 1) / bh;
     const int64_t max_by_len = (len + 127) / 128;
     if (splits > max_by_len) splits = max_by_len;
     const int64_t min_by_chunk = (len + KV_CHUNK_MAX - 1) / KV_CHUNK_MAX;
