@@ -33,6 +33,16 @@
 // registers on the way to LDS.  Anything else (arbitrary strides, unaligned
 // bases, edge tiles) takes guarded scalar loads into the same register layout.
 //
+// K loop.  Tile kt+1 sits in staging registers while tile kt is multiplied out
+// of LDS; in the last quarter of a step the staged tile goes to the other LDS
+// stage and tile kt+2 is requested, so a request has a whole step to arrive.
+// The loop exists twice.  The general form chooses between fast and guarded
+// loads per step.  The steady form (interior tile, K a whole number of steps)
+// has no such choice and loads unconditionally: when the staging registers
+// have two possible producers the compiler merges them with register copies
+// that wait for the data right behind the request, which stalls every step
+// for a memory round trip.
+//
 // Work distribution.  Classic form: one workgroup per (tile, batch, K slice);
 // with more than one slice the partials go to a workspace and a second kernel
 // adds them.  Stream-K form (Osama et al., "Stream-K", PPoPP'23, restricted to
@@ -51,6 +61,7 @@
 // a workgroup only ever waits for lower-numbered (earlier dispatched) ones.
 #include "common.h"
 #include "gemm_internal.h"
+#include <type_traits>
 
 namespace mni {
 
@@ -97,11 +108,14 @@ __device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t l
     } else {
         constexpr int R4 = ROWS / 4;
         int r4 = tid % R4, q = tid / R4;
-        if (q < KQ) {
+        // Threads beyond the tile (half of them when ROWS = 64) own nothing;
+        // they load what their partner 8 quads below loads and never store
+        // it.  Loading under a predicate instead would make every load a merge
+        // with the old register contents, which waits for the data on the spot.
+        q %= KQ;
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                v[j] = *reinterpret_cast<const float4 *>(p + 4 * r4 + (int64_t)(4 * q + j) * ld);
-        }
+        for (int j = 0; j < 4; ++j)
+            v[j] = *reinterpret_cast<const float4 *>(p + 4 * r4 + (int64_t)(4 * q + j) * ld);
     }
 }
 
@@ -160,11 +174,24 @@ __device__ __forceinline__ void store_lds(float4 *__restrict__ tile, int tid, co
     } else {
         constexpr int R4 = ROWS / 4;
         int r4 = tid % R4, q = tid / R4;
-        if (q < KQ) {
-            tile[q * SLICE + lds_row(4 * r4 + 0)] = make_float4(v[0].x, v[1].x, v[2].x, v[3].x);
-            tile[q * SLICE + lds_row(4 * r4 + 1)] = make_float4(v[0].y, v[1].y, v[2].y, v[3].y);
-            tile[q * SLICE + lds_row(4 * r4 + 2)] = make_float4(v[0].z, v[1].z, v[2].z, v[3].z);
-            tile[q * SLICE + lds_row(4 * r4 + 3)] = make_float4(v[0].w, v[1].w, v[2].w, v[3].w);
+        // The 4 x 4 transpose is sixteen register moves, written out so that
+        // they stay here, a whole K step after the loads were issued.  Left to
+        // the compiler they end up merged into the loop-carried copy of the
+        // staging registers, right behind the loads, and wait for data that
+        // was only just requested.
+        float4 o[4];
+#define MNI_TRANSPOSE_ROW(dst, c)                                                                     \
+    asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7"        \
+                 : "=&v"(dst.x), "=&v"(dst.y), "=&v"(dst.z), "=&v"(dst.w)                              \
+                 : "v"(v[0].c), "v"(v[1].c), "v"(v[2].c), "v"(v[3].c))
+        MNI_TRANSPOSE_ROW(o[0], x);
+        MNI_TRANSPOSE_ROW(o[1], y);
+        MNI_TRANSPOSE_ROW(o[2], z);
+        MNI_TRANSPOSE_ROW(o[3], w);
+#undef MNI_TRANSPOSE_ROW
+        if (NTHREADS / R4 <= KQ || q < KQ) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) tile[q * SLICE + lds_row(4 * r4 + e)] = o[e];
         }
     }
 }
@@ -353,34 +380,39 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
 
     float4 ra[4], rb[4];
 
-    auto load_a = [&](int kt) {  // A tile: rows = m, element (m, k) at Ap[m * a_rs + k * a_cs]
+    // STEADY: the tile is interior and K is a whole number of steps, so every
+    // load of the K loop is a fast one; the loop then has no branch that
+    // produces staging registers on two paths.
+    auto load_a = [&](int kt, auto steady) {  // A tile: rows = m, element (m, k) at Ap[m * a_rs + k * a_cs]
         const int k0 = kt * BK;
         const int krem = klen - k0;
-        if (a_full && krem >= BK) {
+        if (decltype(steady)::value || (a_full && krem >= BK)) {
             if (AMODE == 0) load_fast<0, BM>(Ap + (int64_t)k0, a_ld, tid, ra);
             else load_fast<1, BM>(Ap + (int64_t)k0 * a_ld, a_ld, tid, ra);
         } else {
             load_guarded<AL, BM>(Ap + (int64_t)k0 * g.a_cs, g.a_rs, g.a_cs, mrem, krem, tid, ra);
         }
     };
-    auto load_b = [&](int kt) {  // B tile: rows = n, element (n, k) at Bp[n * b_cs + k * b_rs]
+    auto load_b = [&](int kt, auto steady) {  // B tile: rows = n, element (n, k) at Bp[n * b_cs + k * b_rs]
         const int k0 = kt * BK;
         const int krem = klen - k0;
-        if (b_full && krem >= BK) {
+        if (decltype(steady)::value || (b_full && krem >= BK)) {
             if (BMODE == 0) load_fast<0, BN>(Bp + (int64_t)k0, b_ld, tid, rb);
             else load_fast<1, BN>(Bp + (int64_t)k0 * b_ld, b_ld, tid, rb);
         } else {
             load_guarded<BL, BN>(Bp + (int64_t)k0 * g.b_rs, g.b_cs, g.b_rs, nrem, krem, tid, rb);
         }
     };
+    typedef std::integral_constant<bool, false> General;
+    typedef std::integral_constant<bool, true> Steady;
 
     // Prologue: tile 0 goes to LDS stage 0, tile 1 into the staging registers.
     if (nkt > 0) {
-        load_a(0);
-        load_b(0);
+        load_a(0, General());
+        load_b(0, General());
         store_lds<AL, BM>(stage_a(0), tid, ra);
         store_lds<BL, BN>(stage_b(0), tid, rb);
-        if (nkt > 1) { load_a(1); load_b(1); }
+        if (nkt > 1) { load_a(1, General()); load_b(1, General()); }
     }
     __syncthreads();
 
@@ -407,10 +439,16 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         __builtin_amdgcn_s_setprio(0);
     };
 
+    auto k_loop = [&](auto steady) {
+    constexpr bool ST = decltype(steady)::value;
     for (int kt = 0; kt < nkt; ++kt) {
         const int cur = kt & 1;
-        const bool more = kt + 1 < nkt;
-        const bool more2 = kt + 2 < nkt;
+        // Steady form: the stores and loads run unconditionally (the last two
+        // steps park and fetch the final tile again, which nobody reads), so
+        // the staging registers have one producer.
+        const bool more = ST || kt + 1 < nkt;
+        const bool more2 = ST || kt + 2 < nkt;
+        const int kt2 = ST ? min(kt + 2, nkt - 1) : kt + 2;
 
         const float4 *As = stage_a(cur), *Bs = stage_b(cur);
 #pragma unroll
@@ -431,7 +469,7 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
                 // The staging registers hold tile kt+1 (requested a whole K step
                 // ago); once they are in LDS they are refilled with tile kt+2.
                 store_lds<AL, BM>(stage_a(cur ^ 1), tid, ra);
-                if (more2) load_a(kt + 2);
+                if (more2) load_a(kt2, steady);
             }
             __builtin_amdgcn_sched_barrier(0);
             mfma_group(1);
@@ -439,7 +477,7 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
             if (!last) nb[0] = Bs[qb + b_row[0]];
             else if (more) {
                 store_lds<BL, BN>(stage_b(cur ^ 1), tid, rb);
-                if (more2) load_b(kt + 2);
+                if (more2) load_b(kt2, steady);
             }
             __builtin_amdgcn_sched_barrier(0);
             mfma_group(2);
@@ -457,6 +495,9 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         }
         __syncthreads();
     }
+    };
+    if (AMODE != 2 && BMODE != 2 && a_full && b_full && klen % BK == 0) k_loop(Steady());
+    else k_loop(General());
 
     // ---- epilogue -----------------------------------------------------------
     // A 32 x 32 MFMA block leaves lane l with column l%32 and rows
