@@ -426,17 +426,15 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     // the compiler from regrouping them.
     float4 fa[TM], fb[TN];  // fragments in use
     float4 na[TM], nb[TN];  // fragments of the next chunk
-    // The wavefront raises its issue priority while it feeds the matrix pipe, so
-    // that the other resident wavefront's loads and LDS traffic fill the gaps
-    // instead of delaying the MFMAs (+2.5 % at 4096^3 on MI355X).
+    // Both resident wavefronts of a SIMD issue at the default priority: raising
+    // it around the MFMAs paid off only while the K loop still stalled on its
+    // loads, and costs 2 % at 4096^3 now that it does not.
     auto mfma_group = [&](int j) {
-        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int jj = 0; jj < TN; ++jj)
                 acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(pick(fa[i], j), pick(fb[jj], j), acc[i][jj], 0, 0, 0);
-        __builtin_amdgcn_s_setprio(0);
     };
 
     auto k_loop = [&](auto steady) {
