@@ -179,6 +179,11 @@ static int run_mfma(const mni_gemm_desc &d) {
     const int ktiles = (g.K + bk - 1) / bk;
     const bool sk_device = c.xcd_count > 0 && c.skinny_flags && cus % c.xcd_count == 0;
 
+    // op(A)(m, k): K stride = col_stride, M stride = row_stride.
+    const int amode = g.K == 0 ? 2 : classify(g.A, g.a_cs, g.a_rs, g.a_bs, g.a_bcount);
+    // op(B)(k, n): K stride = row_stride, N stride = col_stride.
+    const int bmode = g.K == 0 ? 2 : classify(g.B, g.b_rs, g.b_cs, g.b_bs, g.b_bcount);
+
     // Can the K steps of tiles of this shape be dealt over the stream-K grid?
     // In every XCD's stream-K region each workgroup must own at least
     // `min_steps` K steps (with none, a finisher would wait for a partial that
@@ -216,6 +221,24 @@ static int run_mfma(const mni_gemm_desc &d) {
                 // plenty of K steps per workgroup slot: big tiles
                 const int64_t rounds = (big_tiles + big_slots - 1) / big_slots;
                 whole_tiles = big_tiles * 100 >= rounds * big_slots * 93;
+                if (!whole_tiles && bm == 128 && bn == 128 && (amode == 0 || bmode == 0)) {
+                    // Tiles halved along one side may fill their rounds where
+                    // 128 x 128 does not.  Over a few rounds they beat stream-K
+                    // (they run within 5 % of the big tile; over many rounds
+                    // stream-K's fix-up of one last round costs less than that).
+                    // The short side goes to an operand that is K-contiguous: one
+                    // that is transposed on the way to LDS keeps all threads busy
+                    // with its loads only at 128.
+                    const int hm = amode == 0 ? 64 : 128, hn = amode == 0 ? 128 : 64;
+                    const int64_t half_tiles = (int64_t)((g.M + hm - 1) / hm) * ((g.N + hn - 1) / hn) * g.batch;
+                    const int64_t half_slots = (int64_t)cus * gemm_mfma_resident_per_cu(hm, hn);
+                    const int64_t half_rounds = (half_tiles + half_slots - 1) / half_slots;
+                    if (half_rounds <= 3 && half_tiles * 100 >= half_rounds * half_slots * 93) {
+                        whole_tiles = true;
+                        bm = hm;
+                        bn = hn;
+                    }
+                }
                 // (under 3/16 of the slots: long K over few tiles, left to the K slices below)
                 if (!whole_tiles && big_tiles * 16 >= 3 * big_slots) streamk = streamk_fits(bm, bn, 8);
             } else {
@@ -242,11 +265,6 @@ static int run_mfma(const mni_gemm_desc &d) {
     }
     g.tiles_m = (g.M + bm - 1) / bm;
     g.tiles_n = (g.N + bn - 1) / bn;
-
-    // op(A)(m, k): K stride = col_stride, M stride = row_stride.
-    const int amode = g.K == 0 ? 2 : classify(g.A, g.a_cs, g.a_rs, g.a_bs, g.a_bcount);
-    // op(B)(k, n): K stride = row_stride, N stride = col_stride.
-    const int bmode = g.K == 0 ? 2 : classify(g.B, g.b_rs, g.b_cs, g.b_bs, g.b_bcount);
 
     g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0;
     void *ws = nullptr;
