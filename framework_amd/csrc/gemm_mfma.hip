@@ -37,8 +37,9 @@
 // of LDS; in the last quarter of a step the staged tile goes to the other LDS
 // stage and tile kt+2 is requested, so a request has a whole step to arrive.
 // The loop exists twice.  The general form chooses between fast and guarded
-// loads per step.  The steady form (interior tile, K a whole number of steps)
-// has no such choice and loads unconditionally: when the staging registers
+// loads per step.  The steady form (interior tile, whole K steps; a partial
+// last step and the two before it are left to the general form) has no such
+// choice and loads unconditionally: when the staging registers
 // have two possible producers the compiler merges them with register copies
 // that wait for the data right behind the request, which stalls every step
 // for a memory round trip.
@@ -96,18 +97,21 @@ __device__ __forceinline__ int lds_row(int r) { return r ^ ((r >> 4) & 3); }
 //   >= 8 own nothing: half of them when ROWS = 64); v[j] holds k = 4*quad + j
 //   across the four rows.
 
+// Rows at or beyond `rows` (an edge tile; a multiple of 4 for layout 1) are
+// read from the last valid row or row quad instead: what they contribute lands
+// in accumulator rows / columns that the epilogue never stores.
 template <int LAYOUT, int ROWS>
-__device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t ld, int tid, float4 (&v)[4]) {
+__device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t ld, int rows, int tid, float4 (&v)[4]) {
     if (LAYOUT == 0) {
 #pragma unroll
         for (int i = 0; i < ROWS / 32; ++i) {
             int f = tid + NTHREADS * i;
-            int row = f >> 3, q = f & 7;
+            int row = min(f >> 3, rows - 1), q = f & 7;
             v[i] = *reinterpret_cast<const float4 *>(p + (int64_t)row * ld + 4 * q);
         }
     } else {
         constexpr int R4 = ROWS / 4;
-        int r4 = tid % R4, q = tid / R4;
+        int r4 = min(tid % R4, rows / 4 - 1), q = tid / R4;
         // Threads beyond the tile (half of them when ROWS = 64) own nothing;
         // they load what their partner 8 quads below loads and never store
         // it.  Loading under a predicate instead would make every load a merge
@@ -364,8 +368,12 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     const float *__restrict__ Bp =
         g.B + (int64_t)(batch % g.b_bcount) * g.b_bs + (int64_t)n0 * g.b_cs + (int64_t)k_begin * g.b_rs;
     const int mrem = g.M - m0, nrem = g.N - n0;
-    const bool a_full = AMODE != 2 && mrem >= BM;
-    const bool b_full = BMODE != 2 && nrem >= BN;
+    // Fast loads also serve an edge tile (rows beyond the edge re-read the last
+    // valid ones), except that 16-byte loads along M/N need the edge on a
+    // multiple of 4.
+    const int a_rows = min(mrem, BM), b_rows = min(nrem, BN);
+    const bool a_fast = AMODE == 0 || (AMODE == 1 && a_rows % 4 == 0);
+    const bool b_fast = BMODE == 0 || (BMODE == 1 && b_rows % 4 == 0);
     // leading dimension seen by the fast loaders
     const int64_t a_ld = AMODE == 0 ? g.a_rs : g.a_cs;
     const int64_t b_ld = BMODE == 0 ? g.b_cs : g.b_rs;
@@ -386,9 +394,9 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     auto load_a = [&](int kt, auto steady) {  // A tile: rows = m, element (m, k) at Ap[m * a_rs + k * a_cs]
         const int k0 = kt * BK;
         const int krem = klen - k0;
-        if (decltype(steady)::value || (a_full && krem >= BK)) {
-            if (AMODE == 0) load_fast<0, BM>(Ap + (int64_t)k0, a_ld, tid, ra);
-            else load_fast<1, BM>(Ap + (int64_t)k0 * a_ld, a_ld, tid, ra);
+        if (decltype(steady)::value || (a_fast && krem >= BK)) {
+            if (AMODE == 0) load_fast<0, BM>(Ap + (int64_t)k0, a_ld, a_rows, tid, ra);
+            else load_fast<1, BM>(Ap + (int64_t)k0 * a_ld, a_ld, a_rows, tid, ra);
         } else {
             load_guarded<AL, BM>(Ap + (int64_t)k0 * g.a_cs, g.a_rs, g.a_cs, mrem, krem, tid, ra);
         }
@@ -396,9 +404,9 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     auto load_b = [&](int kt, auto steady) {  // B tile: rows = n, element (n, k) at Bp[n * b_cs + k * b_rs]
         const int k0 = kt * BK;
         const int krem = klen - k0;
-        if (decltype(steady)::value || (b_full && krem >= BK)) {
-            if (BMODE == 0) load_fast<0, BN>(Bp + (int64_t)k0, b_ld, tid, rb);
-            else load_fast<1, BN>(Bp + (int64_t)k0 * b_ld, b_ld, tid, rb);
+        if (decltype(steady)::value || (b_fast && krem >= BK)) {
+            if (BMODE == 0) load_fast<0, BN>(Bp + (int64_t)k0, b_ld, b_rows, tid, rb);
+            else load_fast<1, BN>(Bp + (int64_t)k0 * b_ld, b_ld, b_rows, tid, rb);
         } else {
             load_guarded<BL, BN>(Bp + (int64_t)k0 * g.b_rs, g.b_cs, g.b_rs, nrem, krem, tid, rb);
         }
@@ -437,9 +445,9 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
                 acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(pick(fa[i], j), pick(fb[jj], j), acc[i][jj], 0, 0, 0);
     };
 
-    auto k_loop = [&](auto steady) {
+    auto k_loop = [&](auto steady, int kt_begin, int kt_end) {
     constexpr bool ST = decltype(steady)::value;
-    for (int kt = 0; kt < nkt; ++kt) {
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
         const int cur = kt & 1;
         // Steady form: the stores and loads run unconditionally (the last two
         // steps park and fetch the final tile again, which nobody reads), so
@@ -494,8 +502,13 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         __syncthreads();
     }
     };
-    if (AMODE != 2 && BMODE != 2 && a_full && b_full && klen % BK == 0) k_loop(Steady());
-    else k_loop(General());
+    // An interior tile runs the steady form; when K ends in a partial step, up
+    // to the step that requests that last tile (two steps ahead), and the
+    // general form takes the remaining three.
+    int nsteady = 0;
+    if (AMODE != 2 && BMODE != 2 && a_fast && b_fast) nsteady = klen % BK == 0 ? nkt : max(nkt - 3, 0);
+    k_loop(Steady(), 0, nsteady);
+    k_loop(General(), nsteady, nkt);
 
     // ---- epilogue -----------------------------------------------------------
     // A 32 x 32 MFMA block leaves lane l with column l%32 and rows

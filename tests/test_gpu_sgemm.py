@@ -101,6 +101,35 @@ def test_mfma_normal_inputs_vs_oracle(dev, oracle_native, m, n, k, ta, tb):
     assert max_err(got, want) <= gemm_tol(k, a, b)
 
 
+@pytest.mark.parametrize("m,n,k,lda,ldb", [
+    (1004, 300, 200, 200, 300),    # both edges on a multiple of 4: fast loads, rows beyond the edge re-read
+    (1001, 302, 200, 200, 320),    # B is a view into wider rows, its edge (46 columns) is not a multiple of 4
+    (1002, 300, 203, 208, 300),    # K tail inside padded rows of A
+    (1000, 1004, 517, 520, 1004),  # long enough for the steady K loop before the tail
+])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_edge_tiles_in_padded_buffers(dev, m, n, k, lda, ldb, ta, tb):
+    """Edge tiles and K tails of operands that sit in wider (16-byte aligned) rows: the extent is smaller than the
+    leading dimension, so the 16-byte load paths are eligible and have to stop at the edge by themselves.  The
+    padding holds a large value that must not leak into the result."""
+    r = dev.r
+    # op(A) is m x k; stored k x m (leading dimension padded) when ta
+    ea, eb = (k, m) if ta else (m, k), (n, k) if tb else (k, n)
+    pa = lda if not ta else ((m + 3) // 4 * 4 + 4)
+    pb = ldb if not tb else ((k + 3) // 4 * 4 + 4)
+    a = np.full((ea[0], pa), 1e30, dtype=np.float32)
+    b = np.full((eb[0], pb), 1e30, dtype=np.float32)
+    a[:, :ea[1]] = synth.small_ints(m + k, ea, 4)
+    b[:, :eb[1]] = synth.small_ints(n + k, eb, 4, stream=1)
+    dA, dB = dev.put(a), dev.put(b)
+    dC = dev.empty(m * n, fill=-7.0)
+    want = ((a[:, :ea[1]].T if ta else a[:, :ea[1]]).astype(np.int64) @ (b[:, :eb[1]].T if tb else b[:, :eb[1]]).astype(np.int64)).astype(np.float32)
+    for algo in (N.ALGO_AUTO, N.ALGO_MFMA, N.ALGO_MFMA_SMALL):
+        r.fill(dC, -7.0, m * n)
+        r.sgemm(m, n, k, dA, dB, dC, a_strides=(1, pa) if ta else (pa, 1), b_strides=(1, pb) if tb else (pb, 1), algo=algo)
+        assert np.array_equal(r.to_host(dC, (m, n)), want), algo
+
+
 def test_golden_cases(dev):
     with open(os.path.join(GOLDEN, "matmul_cases.json")) as f:
         cases = json.load(f)["cases"]
