@@ -8,13 +8,12 @@ namespace mni {
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // 0: K axis contiguous, 1: the other axis contiguous, 2: arbitrary.  `ks` is
-// the stride along K, `os` the stride along M (for A) or N (for B).  A batch
-// stride only matters when more than one batch matrix is addressed.
-static int classify(const float *p, int64_t ks, int64_t os, int64_t bs, int64_t bcount) {
-    const bool batch_ok = bcount <= 1 || (bs % 4) == 0;
-    if (!aligned16(p) || !batch_ok) return 2;
-    if (ks == 1 && (os % 4) == 0) return 0;
-    if (os == 1 && (ks % 4) == 0) return 1;
+// the stride along K, `os` the stride along M (for A) or N (for B).  Base
+// address, leading dimension and batch stride do not matter: the tile kernel's
+// 16-byte loads work from any 4-byte aligned address.
+static int classify(int64_t ks, int64_t os) {
+    if (ks == 1) return 0;
+    if (os == 1) return 1;
     return 2;
 }
 
@@ -180,9 +179,9 @@ static int run_mfma(const mni_gemm_desc &d) {
     const bool sk_device = c.xcd_count > 0 && c.skinny_flags && cus % c.xcd_count == 0;
 
     // op(A)(m, k): K stride = col_stride, M stride = row_stride.
-    const int amode = g.K == 0 ? 2 : classify(g.A, g.a_cs, g.a_rs, g.a_bs, g.a_bcount);
+    const int amode = g.K == 0 ? 2 : classify(g.a_cs, g.a_rs);
     // op(B)(k, n): K stride = row_stride, N stride = col_stride.
-    const int bmode = g.K == 0 ? 2 : classify(g.B, g.b_rs, g.b_cs, g.b_bs, g.b_bcount);
+    const int bmode = g.K == 0 ? 2 : classify(g.b_rs, g.b_cs);
 
     // Can the K steps of tiles of this shape be dealt over the stream-K grid?
     // In every XCD's stream-K region each workgroup must own at least

@@ -30,8 +30,12 @@
 // with 16-byte loads along K and stored to LDS as is.  An operand whose M/N
 // axis has unit stride (B row-major, or A given as its transpose) is loaded as
 // a 4(k) x 4(mn) micro-tile with 16-byte loads along M/N and transposed in
-// registers on the way to LDS.  Anything else (arbitrary strides, unaligned
-// bases, edge tiles) takes guarded scalar loads into the same register layout.
+// registers on the way to LDS.  The 16-byte loads need no more than the 4-byte
+// alignment every float has (the memory system splits a load that straddles a
+// cache line), so odd leading dimensions and offset bases take these paths
+// too.  Anything else (neither axis contiguous, K tails, edges of an M/N-
+// contiguous operand off a multiple of 4) takes guarded scalar loads into the
+// same register layout.
 //
 // K loop.  Tile kt+1 sits in staging registers while tile kt is multiplied out
 // of LDS; in the last quarter of a step the staged tile goes to the other LDS
@@ -208,8 +212,8 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 
 __device__ __forceinline__ float pick(const float4 &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
 
-// MODE: 0 = K axis contiguous + 16-byte aligned, 1 = M/N axis contiguous +
-// aligned, 2 = arbitrary strides (always guarded scalar loads, layout 0).
+// MODE: 0 = K axis contiguous, 1 = M/N axis contiguous, 2 = arbitrary strides
+// (always guarded scalar loads, layout 0).
 // TM x TN: 32 x 32 MFMA blocks per wavefront; the workgroup tile is
 // (64 TM) x (64 TN): 128 x 128 for the dense case, 64-wide sides for narrow or
 // short-K products where smaller tiles waste less and fill the machine better.

@@ -130,6 +130,27 @@ def test_edge_tiles_in_padded_buffers(dev, m, n, k, lda, ldb, ta, tb):
         assert np.array_equal(r.to_host(dC, (m, n)), want), algo
 
 
+@pytest.mark.parametrize("m,n,k", [(257, 259, 261), (1000, 1001, 515)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_odd_leading_dimensions_and_offset_bases(dev, m, n, k, ta, tb):
+    """Rows that start on no 16-byte boundary (odd leading dimensions; operands that begin one, two or three floats
+    into their allocation) still take the 16-byte load paths; the result must not change."""
+    r = dev.r
+    a = synth.small_ints(m + k, (k, m) if ta else (m, k), 4)
+    b = synth.small_ints(n + k, (n, k) if tb else (k, n), 4, stream=1)
+    want = ((a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(np.float32)
+    for off_a, off_b in ((0, 0), (1, 2), (3, 1)):
+        fa = np.concatenate([np.full(off_a, 1e30, np.float32), a.ravel()])
+        fb = np.concatenate([np.full(off_b, 1e30, np.float32), b.ravel()])
+        dA, dB = dev.put(fa), dev.put(fb)
+        dC = dev.empty(m * n, fill=-7.0)
+        for algo in (N.ALGO_AUTO, N.ALGO_MFMA_SMALL):
+            r.fill(dC, -7.0, m * n)
+            r.sgemm(m, n, k, dA + 4 * off_a, dB + 4 * off_b, dC, a_strides=(1, a.shape[1]) if ta else (a.shape[1], 1),
+                    b_strides=(1, b.shape[1]) if tb else (b.shape[1], 1), algo=algo)
+            assert np.array_equal(r.to_host(dC, (m, n)), want), (off_a, off_b, algo)
+
+
 def test_golden_cases(dev):
     with open(os.path.join(GOLDEN, "matmul_cases.json")) as f:
         cases = json.load(f)["cases"]
