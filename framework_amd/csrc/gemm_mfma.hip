@@ -539,8 +539,9 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     const int prow = lane / LANES_PER_ROW, pc4 = lane % LANES_PER_ROW;
     const int coll = wn * WN + 4 * pc4;  // column within the tile
     const int col = n0 + coll;
-    const bool vec_ok = partial ? ((g.N & 3) == 0)
-                                : ((ldc & 3) == 0 && (g.c_bs & 3) == 0 && (reinterpret_cast<uintptr_t>(g.C) & 15) == 0);
+    // 16-byte stores (and the loads of an accumulating epilogue) go to any
+    // 4-byte aligned address, as the operand loads do
+    constexpr bool vec_ok = true;
     float bias4[4] = {0.f, 0.f, 0.f, 0.f};
     if (!partial && !(SK && role == ROLE_PART) && g.epilogue != MNI_EPI_NONE) {
 #pragma unroll
