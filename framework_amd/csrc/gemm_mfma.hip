@@ -39,7 +39,10 @@
 //
 // K loop.  Tile kt+1 sits in staging registers while tile kt is multiplied out
 // of LDS; in the last quarter of a step the staged tile goes to the other LDS
-// stage and tile kt+2 is requested, so a request has a whole step to arrive.
+// stage and tile kt+2 is requested, so a request has a whole step to arrive
+// (the steady form deals these transfers out in pieces, one or two behind each
+// MFMA of that quarter; LDS is read in the first three quarters and written
+// in the last).
 // The loop exists twice.  The general form chooses between fast and guarded
 // loads per step.  The steady form (interior tile, whole K steps; a partial
 // last step and the two before it are left to the general form) has no such
@@ -200,6 +203,42 @@ __device__ __forceinline__ void store_lds(float4 *__restrict__ tile, int tid, co
         if (NTHREADS / R4 <= KQ || q < KQ) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) tile[q * SLICE + lds_row(4 * r4 + e)] = o[e];
+        }
+    }
+}
+
+// One piece of a tile transfer, so that the last chunk of a K step can deal
+// them out one per MFMA.  A tile side is `pieces<LAYOUT, ROWS>()` pieces: for
+// layout 0 float4 #i is stored (first half) and then loaded anew (second
+// half); for layout 1 pieces 0..3 transpose and store row e of the micro-tile
+// and pieces 4..7 load v[j].
+template <int LAYOUT, int ROWS>
+__device__ constexpr int tile_pieces() { return LAYOUT == 0 ? 2 * (ROWS / 32) : 8; }
+
+template <int LAYOUT, int ROWS>
+__device__ __forceinline__ void tile_piece(int x, float4 *__restrict__ tile, const float *__restrict__ p, int64_t ld,
+                                           int rows, int tid, float4 (&v)[4]) {
+    constexpr int SLICE = ROWS + PAD;
+    if (LAYOUT == 0) {
+        constexpr int NV = ROWS / 32;
+        const int i = x < NV ? x : x - NV;
+        const int f = tid + NTHREADS * i;
+        const int row = f >> 3, q = f & 7;
+        if (x < NV) tile[q * SLICE + lds_row(row)] = v[i];
+        else v[i] = *reinterpret_cast<const float4 *>(p + (int64_t)min(row, rows - 1) * ld + 4 * q);
+    } else {
+        constexpr int R4 = ROWS / 4;
+        const int r4 = tid % R4, q = tid / R4;
+        if (x < 4) {
+            float4 o;
+            if (x == 0) asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7" : "=&v"(o.x), "=&v"(o.y), "=&v"(o.z), "=&v"(o.w) : "v"(v[0].x), "v"(v[1].x), "v"(v[2].x), "v"(v[3].x));
+            if (x == 1) asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7" : "=&v"(o.x), "=&v"(o.y), "=&v"(o.z), "=&v"(o.w) : "v"(v[0].y), "v"(v[1].y), "v"(v[2].y), "v"(v[3].y));
+            if (x == 2) asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7" : "=&v"(o.x), "=&v"(o.y), "=&v"(o.z), "=&v"(o.w) : "v"(v[0].z), "v"(v[1].z), "v"(v[2].z), "v"(v[3].z));
+            if (x == 3) asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7" : "=&v"(o.x), "=&v"(o.y), "=&v"(o.z), "=&v"(o.w) : "v"(v[0].w), "v"(v[1].w), "v"(v[2].w), "v"(v[3].w));
+            if (NTHREADS / R4 <= KQ || q < KQ) tile[q * SLICE + lds_row(4 * r4 + x)] = o;
+        } else {
+            const int j = x - 4;
+            v[j] = *reinterpret_cast<const float4 *>(p + 4 * min(r4, rows / 4 - 1) + (int64_t)(4 * (q % KQ) + j) * ld);
         }
     }
 }
@@ -469,6 +508,34 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         for (int c = 0; c < NCHUNK; ++c) {
             const bool last = c == NCHUNK - 1;
             const int qa = (2 * (c + 1) + h) * SLICE_A, qb = (2 * (c + 1) + h) * SLICE_B;
+            if (ST && last) {
+                // Steady form: the staged tile goes to LDS and tile kt+2 is
+                // requested piece by piece, one or two pieces behind each MFMA, so
+                // that none of it has to be issued with the matrix pipe idle.
+                constexpr int PA = tile_pieces<AL, BM>(), PB = tile_pieces<BL, BN>();
+                constexpr int SLOTS = 4 * TM * TN, PER = (PA + PB + SLOTS - 1) / SLOTS;
+                const float *pa = AMODE == 0 ? Ap + (int64_t)kt2 * BK : Ap + (int64_t)kt2 * BK * a_ld;
+                const float *pb = BMODE == 0 ? Bp + (int64_t)kt2 * BK : Bp + (int64_t)kt2 * BK * b_ld;
+                int slot = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int jj = 0; jj < TN; ++jj) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(pick(fa[i], j), pick(fb[jj], j), acc[i][jj], 0, 0, 0);
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int x = slot * PER; x < (slot + 1) * PER; ++x) {
+                                if (x < PA) tile_piece<AL, BM>(x, stage_a(cur ^ 1), pa, a_ld, a_rows, tid, ra);
+                                else if (x < PA + PB) tile_piece<BL, BN>(x - PA, stage_b(cur ^ 1), pb, b_ld, b_rows, tid, rb);
+                            }
+                            ++slot;
+                        }
+                __builtin_amdgcn_sched_barrier(0);
+                continue;
+            }
             __builtin_amdgcn_sched_barrier(0);
             mfma_group(0);
             __builtin_amdgcn_sched_barrier(0);
