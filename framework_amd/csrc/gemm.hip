@@ -220,11 +220,12 @@ static int run_mfma(const mni_gemm_desc &d) {
                 // plenty of K steps per workgroup slot: big tiles
                 const int64_t rounds = (big_tiles + big_slots - 1) / big_slots;
                 whole_tiles = big_tiles * 100 >= rounds * big_slots * 93;
-                if (!whole_tiles && bm == 128 && bn == 128 && (amode == 0 || bmode == 0)) {
+                if (!whole_tiles && bm == 128 && bn == 128 && (amode == 0 || bmode == 0) && ktiles <= 64) {
                     // Tiles halved along one side may fill their rounds where
-                    // 128 x 128 does not.  Over a few rounds they beat stream-K
-                    // (they run within 5 % of the big tile; over many rounds
-                    // stream-K's fix-up of one last round costs less than that).
+                    // 128 x 128 does not.  Over a few rounds of moderate K they
+                    // beat stream-K (they run within 5 % of the big tile; over
+                    // many rounds or a long K stream-K's fix-up of one last
+                    // round costs less than that).
                     // The short side goes to an operand that is K-contiguous: one
                     // that is transposed on the way to LDS keeps all threads busy
                     // with its loads only at 128.
