@@ -178,7 +178,7 @@ def bench_extras(r):
                 if g is not None:
                     ids.append(g)
             return ids
-        ms = time_step(step4, keep4, 10, 3)
+        ms = time_step(step4, keep4, 20, 15)  # 30 ms of warm-up: the clocks take tens of milliseconds to settle after an idle spell
         out["config4_ffn_step" + ("_fused_linear" if fused else "")] = {
             "ms": ms, "gemm_TFLOP/s_if_all_gemm": 6 * 2.0 * rows * d * h / ms / 1e9}
     # config 1: README MLP step (32x10 -> 64 -> 3, cross-entropy, Adam): launch-latency bound
@@ -284,7 +284,7 @@ def bench_extras(r):
     def keep_lm():
         ids = [p.value._id for p in lm_params]
         return ids + [g for g in (nat.getGrad(p.value._id) for p in lm_params) if g is not None]
-    ms = time_step(lm_step, keep_lm, 10, 3)
+    ms = time_step(lm_step, keep_lm, 15, 6)
     per_tok = 6.0 * (L * 12 * D * D + D * V) + L * 3.5 * 4 * Tn * D  # matmul FLOPs per token, fwd + bwd (attention counted dense)
     out["lm_step_2x768_8x512_vocab8192"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3, "matmul_TFLOP/s": per_tok * Bn * Tn / ms / 1e9}
     # token-side kernels on their own (wall clock per call incl. host issue; bytes = algorithmic)
