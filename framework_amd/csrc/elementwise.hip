@@ -458,22 +458,35 @@ __global__ void colsum_partial_kernel(float *__restrict__ part, const float *__r
     for (; r < r1; ++r) s0 += a[r * cols + c];
     part[(int64_t)blockIdx.y * cols + c] = (s0 + s1) + (s2 + s3);
 }
+// Pass 2: 64 columns per block, the partials dealt to four thread groups as
+// contiguous quarters (a quarter of the loads per thread, all in flight at
+// once for the usual few dozen partials); the four group sums are added in
+// group order, so the result depends on the shape only.
+static constexpr int CF_COLS = 64, CF_GROUPS = 4;
 __global__ void colsum_final_kernel(float *__restrict__ out, const float *__restrict__ part, int64_t nparts,
                                     int64_t cols) {
-    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= cols) return;
+    __shared__ float sums[CF_GROUPS][CF_COLS];
+    const int cx = threadIdx.x % CF_COLS, grp = threadIdx.x / CF_COLS;
+    const int64_t c = (int64_t)blockIdx.x * CF_COLS + cx;
+    const int64_t per = (nparts + CF_GROUPS - 1) / CF_GROUPS;
+    const int64_t p0 = min(nparts, grp * per), p1 = min(nparts, p0 + per);
     float s = 0.f;
-    int64_t p = 0;
-    for (; p + 7 < nparts; p += 8) {  // 8 loads in flight, added in order
-        float v[8];
+    if (c < cols) {
+        int64_t p = p0;
+        for (; p + 7 < p1; p += 8) {  // 8 loads in flight, added in order
+            float v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = part[(p + e) * cols + c];
+            for (int e = 0; e < 8; ++e) v[e] = part[(p + e) * cols + c];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) s += v[e];
+            for (int e = 0; e < 8; ++e) s += v[e];
+        }
+        for (; p < p1; ++p) s += part[p * cols + c];
     }
-    for (; p < nparts; ++p) s += part[p * cols + c];
-    out[c] = s;
+    sums[grp][cx] = s;
+    __syncthreads();
+    if (grp == 0 && c < cols) out[c] = ((sums[0][cx] + sums[1][cx]) + sums[2][cx]) + sums[3][cx];
 }
+static inline dim3 colsum_final_grid(int64_t cols) { return dim3((unsigned)((cols + CF_COLS - 1) / CF_COLS)); }
 int k_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
     if (cols <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
@@ -491,7 +504,7 @@ int k_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
     hipLaunchKernelGGL(colsum_partial_kernel, dim3(gx, (unsigned)nparts), block, 0, ctx().stream, (float *)part, a, rows, cols);
     int rc = check_launch("colsum_partial");
     if (rc == MNI_OK) {
-        hipLaunchKernelGGL(colsum_final_kernel, dim3(gx), block, 0, ctx().stream, out, (const float *)part, nparts, cols);
+        hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, out, (const float *)part, nparts, cols);
         rc = check_launch("colsum_final");
     }
     dev_free(part);
@@ -584,7 +597,7 @@ int k_bias_gelu_backward(float *dx, float *dbias, const float *g, const float *x
                            bias, rows, colsv);
     int rc = check_launch("bias_gelu_backward");
     if (rc == MNI_OK && nparts > 1) {
-        hipLaunchKernelGGL(colsum_final_kernel, dim3((unsigned)((cols + TPB - 1) / TPB)), block, 0, ctx().stream, dbias,
+        hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dbias,
                            (const float *)part, nparts, cols);
         rc = check_launch("colsum_final");
     }
@@ -740,8 +753,8 @@ int k_layernorm_backward(float *dx, float *dgamma, float *dbeta, const float *g,
                        rstd, rows, c);
     int rc = check_launch("layernorm_backward_cols");
     if (rc == MNI_OK) {
-        hipLaunchKernelGGL(colsum_final_kernel, dim3(gx), dim3(TPB), 0, ctx().stream, dgamma, (const float *)pg, nparts, c);
-        hipLaunchKernelGGL(colsum_final_kernel, dim3(gx), dim3(TPB), 0, ctx().stream, dbeta, (const float *)pb, nparts, c);
+        hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(c), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dgamma, (const float *)pg, nparts, c);
+        hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(c), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dbeta, (const float *)pb, nparts, c);
         rc = check_launch("colsum_final");
     }
     dev_free(part);
