@@ -45,7 +45,7 @@ PEAK_HBM_GBPS = 8000.0
 # HBM bytes per gemm_mfma_kernel launch at 4096^3, from the rocprofv3 --pmc
 # runs summarised in profiles/gemm_mfma_4096_pmc.txt (FETCH_SIZE + WRITE_SIZE,
 # scaled by a copy kernel of known size).  None until measured.
-MEASURED_HBM_BYTES_4096 = 827.4e6
+MEASURED_HBM_BYTES_4096 = 797.2e6
 
 
 def time_launches(r, fn, warmup, iters):
