@@ -106,6 +106,10 @@ def bench_extras(r):
     by = 4.0 * (4096 * 4096 + 2 * 4 * 4096)
     out["config5a_gemv"] = {"us": ms * 1e3, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / PEAK_HBM_GBPS,
                             "note": "W (64 MiB) is re-read every launch and fits the 256 MiB Infinity Cache"}
+    # the same after 3000 launches (~40 ms) of it: memory-bound work runs ~5 % slower once the part has been
+    # streaming for a while than in a short burst
+    ms = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 3000, 1000)
+    out["config5a_gemv_sustained"] = {"us": ms * 1e3, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / PEAK_HBM_GBPS}
     # the same product over 8 different W in turn (512 MiB working set): HBM-resident
     ws = [r.to_device(w) for _ in range(8)]
     ms = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, p, dy) for p in ws], 16, 200)
