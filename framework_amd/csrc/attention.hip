@@ -363,10 +363,10 @@ __global__ __launch_bounds__(ATT_TPB) void kv_decode_kernel(const KvDecode a) {
 // LPR neighbouring lanes -- 4 fp32 or 16 int8 values per lane -- so loads are
 // coalesced; a dot product is finished with log2(LPR) butterfly steps, and the
 // value pass keeps those 4 / 16 columns per lane.
-static constexpr int KV_UNROLL = 4;  // cache rows in flight per lane
 template <bool Q8, int LPR>
 __global__ __launch_bounds__(ATT_TPB) void kv_decode_vec_kernel(const KvDecode a) {
     constexpr int E = Q8 ? 16 : 4;         // elements per lane
+    constexpr int KV_UNROLL = 4;           // cache rows in flight per lane (8 measured the same for int8, slower for fp32)
     constexpr int RPP = 64 / LPR;          // rows per wavefront pass
     constexpr int GROUPS = ATT_TPB / LPR;  // key groups in the value pass
     extern __shared__ float sm[];
@@ -381,18 +381,28 @@ __global__ __launch_bounds__(ATT_TPB) void kv_decode_vec_kernel(const KvDecode a
     const int n = min(a.len, t0 + a.chunk) - t0;
     const int pieces = (int)(a.d / E);
     const int64_t base = row * a.max_seq + t0;
-    auto load = [&](const void *cache, const float *scales, int64_t pos, int piece, float (&v)[E]) {
+    // A 16-byte piece of a cache row is requested as it is stored (and, for
+    // int8, the row's scale); it is widened to floats only where it is used, so
+    // that the requests of a trip are all issued before the first wait.
+    auto request = [&](const void *cache, const float *scales, int64_t pos, int piece, int4 &w, float &s) {
         if (Q8) {
-            const int4 w = reinterpret_cast<const int4 *>(reinterpret_cast<const signed char *>(cache) + pos * a.d)[piece];
-            const float s = scales[pos];
-            const int ws[4] = {w.x, w.y, w.z, w.w};
+            w = reinterpret_cast<const int4 *>(reinterpret_cast<const signed char *>(cache) + pos * a.d)[piece];
+            s = scales[pos];
+        } else {
+            w = reinterpret_cast<const int4 *>(reinterpret_cast<const float *>(cache) + pos * a.d)[piece];
+            s = 1.0f;
+        }
+    };
+    auto widen = [&](const int4 &w, float s, float (&v)[E]) {
+        const int ws[4] = {w.x, w.y, w.z, w.w};
+        if (Q8) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int b8 = 0; b8 < 4; ++b8) v[4 * j + b8] = (float)(signed char)((ws[j] >> (8 * b8)) & 0xff) * s;
         } else {
-            const float4 f = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(cache) + pos * a.d)[piece];
-            v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = __int_as_float(ws[j]);
         }
     };
     float qv[E];
@@ -402,19 +412,24 @@ __global__ __launch_bounds__(ATT_TPB) void kv_decode_vec_kernel(const KvDecode a
     // (one 16-byte load per lane in flight does not cover the memory latency)
     constexpr int ROWS_PER_TRIP = (ATT_TPB / 64) * RPP;
     for (int i0 = wave * RPP; i0 < n; i0 += ROWS_PER_TRIP * KV_UNROLL) {
-        float kv[KV_UNROLL][E];
+        int4 kw[KV_UNROLL];
+        float ksc[KV_UNROLL];
 #pragma unroll
         for (int u = 0; u < KV_UNROLL; ++u) {
             const int i = i0 + u * ROWS_PER_TRIP + sub;
-            if (i < n && l < pieces) load(a.kc, a.ks, base + i, l, kv[u]);
+            kw[u] = make_int4(0, 0, 0, 0);
+            ksc[u] = 0.f;
+            if (i < n && l < pieces) request(a.kc, a.ks, base + i, l, kw[u], ksc[u]);
         }
 #pragma unroll
         for (int u = 0; u < KV_UNROLL; ++u) {
             const int i = i0 + u * ROWS_PER_TRIP + sub;
             float part = 0.f;
             if (i < n && l < pieces) {
+                float kv[E];
+                widen(kw[u], ksc[u], kv);
 #pragma unroll
-                for (int e = 0; e < E; ++e) part += qv[e] * kv[u][e];
+                for (int e = 0; e < E; ++e) part += qv[e] * kv[e];
             }
 #pragma unroll
             for (int off = LPR / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
@@ -440,17 +455,23 @@ __global__ __launch_bounds__(ATT_TPB) void kv_decode_vec_kernel(const KvDecode a
     for (int e = 0; e < E; ++e) acc[e] = 0.f;
     if (lv < pieces) {
         for (int i0 = grp; i0 < n; i0 += GROUPS * KV_UNROLL) {
-            float vv[KV_UNROLL][E];
+            int4 vw[KV_UNROLL];
+            float vsc[KV_UNROLL];
 #pragma unroll
-            for (int u = 0; u < KV_UNROLL; ++u)
-                if (i0 + u * GROUPS < n) load(a.vc, a.vs, base + i0 + u * GROUPS, lv, vv[u]);
+            for (int u = 0; u < KV_UNROLL; ++u) {
+                vw[u] = make_int4(0, 0, 0, 0);
+                vsc[u] = 0.f;
+                if (i0 + u * GROUPS < n) request(a.vc, a.vs, base + i0 + u * GROUPS, lv, vw[u], vsc[u]);
+            }
 #pragma unroll
             for (int u = 0; u < KV_UNROLL; ++u) {
                 const int i = i0 + u * GROUPS;
                 if (i < n) {
                     const float w = sc[i];
+                    float vv[E];
+                    widen(vw[u], vsc[u], vv);
 #pragma unroll
-                    for (int e = 0; e < E; ++e) acc[e] += w * vv[u][e];
+                    for (int e = 0; e < E; ++e) acc[e] += w * vv[e];
                 }
             }
         }
