@@ -548,6 +548,20 @@ def test_streamk_at_training_sizes(dev, oracle_native, m, n, k, ta, tb):
     assert max_err(forced, got) <= gemm_tol(k, a, b)
 
 
+@pytest.mark.parametrize("m,n,k,ta,tb", [(2048, 2048, 1536, False, False), (2048, 2048, 1536, False, True), (2048, 2048, 1536, True, False),
+                                          (4096, 3072, 768, False, False), (4096, 3072, 776, False, True)])
+def test_planner_half_width_tiles(dev, m, n, k, ta, tb):
+    """Products whose 128 x 128 tiles fill their rounds badly while 64 x 128 / 128 x 64 tiles fill theirs: with a
+    K-contiguous operand the planner takes the half-width tiles (whole tiles, steady K loop, the last case with a
+    K tail), otherwise stream-K; every choice must give the integer-exact result, and so must the forced ones."""
+    a = synth.small_ints(m + k, (k, m) if ta else (m, k), 3)
+    b = synth.small_ints(n + k, (n, k) if tb else (k, n), 3, stream=1)
+    # float64 holds these sums of small integers exactly (and runs on the host BLAS, unlike an int64 product)
+    want = ((a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)).astype(np.float32)
+    for algo in (N.ALGO_AUTO, N.ALGO_MFMA, N.ALGO_MFMA_SMALL, N.ALGO_MFMA_STREAMK):
+        assert np.array_equal(run_gemm(dev, a, b, ta, tb, algo=algo)[0], want), algo
+
+
 def test_config5a_decode_gemv(dev, rocm):
     with open(os.path.join(GOLDEN, "config_samples.json")) as f:
         gold = json.load(f)["config5a"]
