@@ -159,6 +159,197 @@ int k_attn_softmax(float *scores, float *lse, int64_t rows, int64_t s, float sca
     return check_launch("attn_softmax");
 }
 
+// ---- attention forward in one kernel --------------------------------------------------
+// out = softmax(scale * q k^T [+ causal mask]) v and lse = max + ln(sum) per query
+// (ops/attention.rs:14-78), for head dims 32, 64, 96, 128, without the s x s
+// score matrix ever leaving the chip.  A workgroup owns 128 queries (32 per
+// wavefront) and walks the keys 32 at a time with the running-maximum
+// recurrence of the reference.  Both products run on v_mfma_f32_32x32x2_f32 and
+// are taken transposed, which puts one query in every lane:
+//   S^T = K Q^T   A = the key tile (LDS, [d/4][key] float4), B = the lane's own
+//                 query row (registers); lane (query r, half h) receives the
+//                 scores of keys 8(e/4) + 4h + e%4, e = 0..15, so the row
+//                 maximum and sum are 15 in-lane steps and one exchange
+//                 between the halves;
+//   O^T += V^T P^T  the probabilities stay where they are: MFMA j of chunk c
+//                 contracts keys 8c + 4h + j, which is exactly accumulator
+//                 element 4c + j of S^T, so P^T is fed to the matrix pipe as
+//                 operand B straight from the registers; A = V^T read from the
+//                 value tile in LDS.  Rescaling the running output is one
+//                 factor per lane.
+typedef float att_f16 __attribute__((ext_vector_type(16)));
+static constexpr int AF_QUERIES = 128, AF_KEYS = 32;
+template <int DB>  // head dim = 32 * DB
+__global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__restrict__ out, float *__restrict__ lse,
+                                                                 const float *__restrict__ q, const float *__restrict__ k,
+                                                                 const float *__restrict__ v, int s, int qblocks, float scale,
+                                                                 int causal) {
+    constexpr int D = 32 * DB, DQ = D / 4;
+    constexpr int KPITCH = AF_KEYS + 1;  // float4 per d-quad slice (+1: the tile stores of 16 consecutive quads spread over the banks)
+    constexpr int VPITCH = D + 8;        // floats per key row (+8: the two lane halves, 4 keys apart, use different banks)
+    constexpr int KSTAGE = DQ * KPITCH, VSTAGE = AF_KEYS * VPITCH;
+    constexpr int NLD = AF_KEYS * DQ / ATT_TPB;  // float4 of each tile per thread (1 .. 4)
+    __shared__ float4 kt[2 * KSTAGE];
+    __shared__ __align__(16) float vt[2 * VSTAGE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int64_t bh = blockIdx.x / qblocks;
+    // blocks of late queries have the most keys to visit under the causal mask: they go first
+    const int qb = qblocks - 1 - (int)(blockIdx.x % qblocks);
+    const int qi = qb * AF_QUERIES + wave * 32 + r;  // this lane's query
+    const int ql = min(qi, s - 1);                   // (queries beyond the end compute on the last one and store nothing)
+    const float *qrow = q + (bh * s + ql) * (int64_t)D;
+    const float *kbase = k + bh * s * (int64_t)D, *vbase = v + bh * s * (int64_t)D;
+    float4 qf[D / 8];  // the d quads 2c + h of the lane's query
+#pragma unroll
+    for (int c = 0; c < D / 8; ++c) qf[c] = *reinterpret_cast<const float4 *>(qrow + 4 * (2 * c + h));
+    att_f16 oacc[DB];
+#pragma unroll
+    for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[b][e] = 0.f;
+    float m = -INFINITY, l = 0.f;
+    // keys this workgroup needs: all of them, or those up to its last query
+    const int nkeys = causal ? min(s, (qb + 1) * AF_QUERIES) : s;
+    const int nsteps = (nkeys + AF_KEYS - 1) / AF_KEYS;
+    const int wave_first = qb * AF_QUERIES + wave * 32;                  // first query of this wavefront
+    const int wave_last = min(wave_first + 31, s - 1);                   // and its last
+    const float scale2 = scale * 1.4426950408889634f;                    // scores in units of log2
+
+    // Tiles travel global -> registers -> LDS; the registers are filled for step
+    // i + 1 before step i is computed and parked in the other LDS stage after it,
+    // so a request has a whole step to arrive and one barrier per step orders
+    // everything.  Requests and stores are unconditional (the last step fetches
+    // its own tile again into a stage nobody reads): a predicated refill would
+    // be merged with the old register contents right behind the loads.
+    float4 kreg[NLD], vreg[NLD];
+    // where this thread's pieces of a tile come from and go to (the same for every step)
+    int src_off[NLD], k_slot[NLD], v_slot[NLD], key_of[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int f = tid + ATT_TPB * i;
+        key_of[i] = f / DQ;
+        src_off[i] = 4 * (f % DQ);
+        k_slot[i] = (f % DQ) * KPITCH + f / DQ;
+        v_slot[i] = (f / DQ) * VPITCH + 4 * (f % DQ);
+    }
+#define MNI_AF_REQUEST(STEP)                                                                          \
+    _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
+        const int64_t src = (int64_t)min((STEP) * AF_KEYS + key_of[i], s - 1) * D + src_off[i];        \
+        kreg[i] = *reinterpret_cast<const float4 *>(kbase + src);                                     \
+        vreg[i] = *reinterpret_cast<const float4 *>(vbase + src);                                     \
+    }
+#define MNI_AF_PARK(STAGE)                                                                            \
+    _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
+        kt[(STAGE) * KSTAGE + k_slot[i]] = kreg[i];                                                   \
+        *reinterpret_cast<float4 *>(vt + (STAGE) * VSTAGE + v_slot[i]) = vreg[i];                     \
+    }
+    MNI_AF_REQUEST(0)
+    MNI_AF_PARK(0)
+    __syncthreads();
+    for (int step = 0; step < nsteps; ++step) {
+        const int k0 = step * AF_KEYS;
+        const int cur = step & 1;
+        MNI_AF_REQUEST(min(step + 1, nsteps - 1))
+        // a wavefront whose queries all come before this key tile has nothing to add (causal)
+        if (!causal || k0 <= wave_last) {
+            const float4 *ks = kt + cur * KSTAGE;
+            const float *vs = vt + cur * VSTAGE;
+            // key fragments are fetched from LDS one d chunk ahead of the MFMAs that use them
+            att_f16 sacc;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
+            float4 ka = ks[h * KPITCH + r];
+#pragma unroll
+            for (int c = 0; c < D / 8; ++c) {
+                float4 na = ka;
+                if (c + 1 < D / 8) na = ks[(2 * (c + 1) + h) * KPITCH + r];
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qf[c].x, sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qf[c].y, sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qf[c].z, sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.w, qf[c].w, sacc, 0, 0, 0);
+                ka = na;
+            }
+            // From here on in units of log2: p = 2^(x - max) is one v_exp_f32.  Only a tile that
+            // reaches past the last key or across the diagonal of this wavefront needs the mask.
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sacc[e] *= scale2;
+            if (k0 + AF_KEYS > s || (causal && k0 + AF_KEYS - 1 > wave_first)) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = k0 + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (!(key < s && (!causal || key <= ql))) sacc[e] = -INFINITY;
+                }
+            }
+            float mx = m;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[e]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            // (key 0 is allowed for every query, so mx is finite from the first step on)
+            const float alpha = __builtin_amdgcn_exp2f(m - mx);
+            float psum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                sacc[e] = __builtin_amdgcn_exp2f(sacc[e] - mx);
+                psum += sacc[e];
+            }
+            psum += __shfl_xor(psum, 32, 64);
+            l = l * alpha + psum;
+            m = mx;
+            // once the running maxima have settled nothing needs rescaling
+            const bool rescale = __any(alpha != 1.0f) != 0;
+#pragma unroll
+            for (int b = 0; b < DB; ++b) {
+                if (rescale) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) oacc[b][e] *= alpha;
+                }
+#pragma unroll
+                for (int c = 0; c < AF_KEYS / 8; ++c)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[(8 * c + 4 * h + j) * VPITCH + 32 * b + r], sacc[4 * c + j],
+                                                                       oacc[b], 0, 0, 0);
+            }
+        }
+        MNI_AF_PARK(cur ^ 1)
+        __syncthreads();
+    }
+#undef MNI_AF_REQUEST
+#undef MNI_AF_PARK
+    if (qi < s) {
+        const float inv = 1.0f / l;
+        float *orow = out + (bh * s + qi) * (int64_t)D;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4)  // accumulator elements 4 g4 .. 4 g4 + 3 are d = 32 b + 8 g4 + 4 h + 0..3
+                *reinterpret_cast<float4 *>(orow + 32 * b + 8 * g4 + 4 * h) =
+                    make_float4(oacc[b][4 * g4] * inv, oacc[b][4 * g4 + 1] * inv, oacc[b][4 * g4 + 2] * inv, oacc[b][4 * g4 + 3] * inv);
+        if (h == 0) lse[bh * s + qi] = m * 0.6931471805599453f + logf(l);  // back from log2 units
+    }
+}
+bool attn_fused_supported(int64_t d) { return d == 32 || d == 64 || d == 96 || d == 128; }
+int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k, const float *v, int64_t bh, int64_t s, int64_t d,
+                         float scale, int causal) {
+    if (bh <= 0 || s <= 0) return MNI_OK;
+    if (!attn_fused_supported(d)) return set_error(MNI_ERR_INVALID, "fused attention: head dim %lld is not 32, 64, 96 or 128", (long long)d);
+    MNI_TRY(ensure_init());
+    const int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
+    if (s > 0x7fffff00LL || bh * qblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
+    hipStream_t st = ctx().stream;
+#define MNI_AF(DBV) hipLaunchKernelGGL(attn_fused_fwd_kernel<DBV>, grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, scale, causal)
+    switch (d / 32) {
+        case 1: MNI_AF(1); break;
+        case 2: MNI_AF(2); break;
+        case 3: MNI_AF(3); break;
+        default: MNI_AF(4); break;
+    }
+#undef MNI_AF
+    return check_launch("attn_fused_forward");
+}
+
 // di[row] = sum_d a[row][d] * b[row][d] (ops/attention.rs:167-170)
 __global__ void rowdot_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, int64_t rows,
                               int64_t d) {

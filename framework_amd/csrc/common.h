@@ -120,6 +120,10 @@ int k_softmax(float *out, const float *x, int64_t outer, int64_t n, int64_t inne
 int k_softmax_backward(float *out, const float *sm, const float *g, int64_t outer, int64_t n, int64_t inner);
 int k_attn_softmax(float *scores, float *lse, int64_t rows, int64_t s, float scale, int causal);
 int k_rowdot(float *out, const float *a, const float *b, int64_t rows, int64_t d);
+// Attention forward in one kernel (out [bh,s,d], lse [bh,s]); head dims 32, 64, 96, 128 only.
+bool attn_fused_supported(int64_t d);
+int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k, const float *v, int64_t bh, int64_t s, int64_t d,
+                         float scale, int causal);
 int k_attn_backward(float *scores, float *dp, const float *lse, const float *di, int64_t rows, int64_t s, float scale,
                     int causal);
 int k_kv_append(void *kc, void *vc, float *ks, float *vs, const float *k, const float *v, int64_t bh, int64_t d,

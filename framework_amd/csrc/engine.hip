@@ -1070,9 +1070,11 @@ static int attn_gemm(float *c, const float *a, bool ta, const float *b, bool tb,
 }
 
 // ops/attention.rs:14-78: q, k, v are taken as [bh, s, d] from their first
-// three dims.  scores = q k^T and out = P v run on the GEMM kernels; the row
-// kernel in between applies scale, the causal mask and the normalisation and
-// leaves lse = max + ln(sum) for the backward pass.
+// three dims.  Head dims 32, 64, 96 and 128 run the forward in one kernel that
+// keeps the scores on the chip; otherwise scores = q k^T and out = P v run on
+// the GEMM kernels and the row kernel in between applies scale, the causal
+// mask and the normalisation.  Either way lse = max + ln(sum) is left for the
+// backward pass, which recomputes P from it.
 static uint32_t flash_attention_op(uint32_t q, uint32_t k, uint32_t v, float scale, bool causal) {
     Tensor *Q = get(q), *K = get(k), *V = get(v);
     if (!Q || !K || !V) return MNI_BAD_ID;
@@ -1084,11 +1086,16 @@ static uint32_t flash_attention_op(uint32_t q, uint32_t k, uint32_t v, float sca
         return MNI_BAD_ID;
     }
     BufP qc = contiguous_buf(*Q), kc = contiguous_buf(*K), vc = contiguous_buf(*V);
-    BufP scores = (qc && kc && vc) ? new_buf((size_t)(bh * s * s)) : nullptr;
-    BufP lse = scores ? new_buf((size_t)(bh * s)) : nullptr;
+    if (!qc || !kc || !vc) return MNI_BAD_ID;
+    BufP lse = new_buf((size_t)(bh * s));
     BufP out = lse ? new_buf((size_t)total) : nullptr;
     if (!out) return MNI_BAD_ID;
-    if (total > 0) {
+    if (total > 0 && attn_fused_supported(d)) {
+        // head dims 32 .. 128: one kernel, the scores never reach memory
+        if (k_attn_fused_forward(out->p, lse->p, qc->p, kc->p, vc->p, bh, s, d, scale, causal ? 1 : 0) != MNI_OK) return MNI_BAD_ID;
+    } else if (total > 0) {
+        BufP scores = new_buf((size_t)(bh * s * s));
+        if (!scores) return MNI_BAD_ID;
         if (attn_gemm(scores->p, qc->p, false, kc->p, true, bh, s, s, d) != MNI_OK) return MNI_BAD_ID;
         if (k_attn_softmax(scores->p, lse->p, bh * s, s, scale, causal ? 1 : 0) != MNI_OK) return MNI_BAD_ID;
         if (attn_gemm(out->p, scores->p, false, vc->p, false, bh, s, d, s) != MNI_OK) return MNI_BAD_ID;

@@ -62,7 +62,9 @@ def test_softmax_negative_dim_gradient_is_the_reference_one(both):
 
 
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("bh,s,d", [(2, 4, 8), (3, 37, 20), (1, 1, 4), (4, 130, 64), (2, 1100, 16)])
+@pytest.mark.parametrize("bh,s,d", [(2, 4, 8), (3, 37, 20), (1, 1, 4), (4, 130, 64), (2, 1100, 16),
+                                    # head dims of the one-kernel forward: key / query tails, one block, several blocks
+                                    (2, 300, 32), (1, 257, 96), (2, 129, 128), (1, 31, 64), (3, 1, 32), (1, 640, 64)])
 def test_attention_forward_and_backward_match_the_oracle(both, bh, s, d, causal):
     gpu, cpu = both
     q, k, v = (synth.normal(5, (bh, s, d), stream=i) for i in range(3))
