@@ -163,7 +163,7 @@ int k_attn_softmax(float *scores, float *lse, int64_t rows, int64_t s, float sca
 // out = softmax(scale * q k^T [+ causal mask]) v and lse = max + ln(sum) per query
 // (ops/attention.rs:14-78), for head dims 32, 64, 96, 128, without the s x s
 // score matrix ever leaving the chip.  A workgroup owns 128 queries (32 per
-// wavefront) and walks the keys 32 at a time with the running-maximum
+// wavefront) and walks the keys 32 or 64 at a time with the running-maximum
 // recurrence of the reference.  Both products run on v_mfma_f32_32x32x2_f32 and
 // are taken transposed, which puts one query in every lane:
 //   S^T = K Q^T   A = the key tile (LDS, [d/4][key] float4), B = the lane's own
@@ -178,17 +178,17 @@ int k_attn_softmax(float *scores, float *lse, int64_t rows, int64_t s, float sca
 //                 value tile in LDS.  Rescaling the running output is one
 //                 factor per lane.
 typedef float att_f16 __attribute__((ext_vector_type(16)));
-static constexpr int AF_QUERIES = 128, AF_KEYS = 32;
-template <int DB>  // head dim = 32 * DB
+static constexpr int AF_QUERIES = 128;
+template <int DB, int NB>  // head dim = 32 * DB, keys per step = 32 * NB
 __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__restrict__ out, float *__restrict__ lse,
-                                                                 const float *__restrict__ q, const float *__restrict__ k,
-                                                                 const float *__restrict__ v, int s, int qblocks, float scale,
-                                                                 int causal) {
-    constexpr int D = 32 * DB, DQ = D / 4;
-    constexpr int KPITCH = AF_KEYS + 1;  // float4 per d-quad slice (+1: the tile stores of 16 consecutive quads spread over the banks)
-    constexpr int VPITCH = D + 8;        // floats per key row (+8: the two lane halves, 4 keys apart, use different banks)
-    constexpr int KSTAGE = DQ * KPITCH, VSTAGE = AF_KEYS * VPITCH;
-    constexpr int NLD = AF_KEYS * DQ / ATT_TPB;  // float4 of each tile per thread (1 .. 4)
+                                                                    const float *__restrict__ q, const float *__restrict__ k,
+                                                                    const float *__restrict__ v, int s, int qblocks, float scale,
+                                                                    int causal) {
+    constexpr int D = 32 * DB, DQ = D / 4, KEYS = 32 * NB;
+    constexpr int KPITCH = KEYS + 1;  // float4 per d-quad slice (+1: the tile stores of consecutive quads spread over the banks)
+    constexpr int VPITCH = D + 8;     // floats per key row (+8: the two lane halves, 4 keys apart, use different banks)
+    constexpr int KSTAGE = DQ * KPITCH, VSTAGE = KEYS * VPITCH;
+    constexpr int NLD = KEYS * DQ / ATT_TPB;  // float4 of each tile per thread (1 .. 4)
     __shared__ float4 kt[2 * KSTAGE];
     __shared__ __align__(16) float vt[2 * VSTAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -211,10 +211,10 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
     float m = -INFINITY, l = 0.f;
     // keys this workgroup needs: all of them, or those up to its last query
     const int nkeys = causal ? min(s, (qb + 1) * AF_QUERIES) : s;
-    const int nsteps = (nkeys + AF_KEYS - 1) / AF_KEYS;
-    const int wave_first = qb * AF_QUERIES + wave * 32;                  // first query of this wavefront
-    const int wave_last = min(wave_first + 31, s - 1);                   // and its last
-    const float scale2 = scale * 1.4426950408889634f;                    // scores in units of log2
+    const int nsteps = (nkeys + KEYS - 1) / KEYS;
+    const int wave_first = qb * AF_QUERIES + wave * 32;  // first query of this wavefront
+    const int wave_last = min(wave_first + 31, s - 1);   // and its last
+    const float scale2 = scale * 1.4426950408889634f;    // scores in units of log2
 
     // Tiles travel global -> registers -> LDS; the registers are filled for step
     // i + 1 before step i is computed and parked in the other LDS stage after it,
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
     }
 #define MNI_AF_REQUEST(STEP)                                                                          \
     _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
-        const int64_t src = (int64_t)min((STEP) * AF_KEYS + key_of[i], s - 1) * D + src_off[i];        \
+        const int64_t src = (int64_t)min((STEP) * KEYS + key_of[i], s - 1) * D + src_off[i];           \
         kreg[i] = *reinterpret_cast<const float4 *>(kbase + src);                                     \
         vreg[i] = *reinterpret_cast<const float4 *>(vbase + src);                                     \
     }
@@ -248,51 +248,66 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
     MNI_AF_PARK(0)
     __syncthreads();
     for (int step = 0; step < nsteps; ++step) {
-        const int k0 = step * AF_KEYS;
+        const int k0 = step * KEYS;
         const int cur = step & 1;
         MNI_AF_REQUEST(min(step + 1, nsteps - 1))
         // a wavefront whose queries all come before this key tile has nothing to add (causal)
         if (!causal || k0 <= wave_last) {
             const float4 *ks = kt + cur * KSTAGE;
             const float *vs = vt + cur * VSTAGE;
-            // key fragments are fetched from LDS one d chunk ahead of the MFMAs that use them
-            att_f16 sacc;
+            att_f16 sacc[NB];
+            bool live[NB];  // under the causal mask the later 32 keys of a step may all lie past this wavefront
 #pragma unroll
-            for (int e = 0; e < 16; ++e) sacc[e] = 0.f;
-            float4 ka = ks[h * KPITCH + r];
+            for (int nb = 0; nb < NB; ++nb) {
+                live[nb] = !causal || k0 + 32 * nb <= wave_last;
 #pragma unroll
-            for (int c = 0; c < D / 8; ++c) {
-                float4 na = ka;
-                if (c + 1 < D / 8) na = ks[(2 * (c + 1) + h) * KPITCH + r];
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qf[c].x, sacc, 0, 0, 0);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qf[c].y, sacc, 0, 0, 0);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qf[c].z, sacc, 0, 0, 0);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.w, qf[c].w, sacc, 0, 0, 0);
-                ka = na;
+                for (int e = 0; e < 16; ++e) sacc[nb][e] = 0.f;
+                if (live[nb]) {
+                    // key fragments are fetched from LDS one d chunk ahead of the MFMAs that use them
+                    float4 ka = ks[h * KPITCH + 32 * nb + r];
+#pragma unroll
+                    for (int c = 0; c < D / 8; ++c) {
+                        float4 na = ka;
+                        if (c + 1 < D / 8) na = ks[(2 * (c + 1) + h) * KPITCH + 32 * nb + r];
+                        sacc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qf[c].x, sacc[nb], 0, 0, 0);
+                        sacc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qf[c].y, sacc[nb], 0, 0, 0);
+                        sacc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qf[c].z, sacc[nb], 0, 0, 0);
+                        sacc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.w, qf[c].w, sacc[nb], 0, 0, 0);
+                        ka = na;
+                    }
+                }
             }
             // From here on in units of log2: p = 2^(x - max) is one v_exp_f32.  Only a tile that
             // reaches past the last key or across the diagonal of this wavefront needs the mask.
 #pragma unroll
-            for (int e = 0; e < 16; ++e) sacc[e] *= scale2;
-            if (k0 + AF_KEYS > s || (causal && k0 + AF_KEYS - 1 > wave_first)) {
+            for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int key = k0 + 8 * (e >> 2) + 4 * h + (e & 3);
-                    if (!(key < s && (!causal || key <= ql))) sacc[e] = -INFINITY;
-                }
+                for (int e = 0; e < 16; ++e) sacc[nb][e] *= scale2;
+            if (k0 + KEYS > s || (causal && k0 + KEYS - 1 > wave_first)) {
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int key = k0 + 32 * nb + 8 * (e >> 2) + 4 * h + (e & 3);
+                        if (!(key < s && (!causal || key <= ql))) sacc[nb][e] = -INFINITY;
+                    }
             }
             float mx = m;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[e]);
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[nb][e]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             // (key 0 is allowed for every query, so mx is finite from the first step on)
             const float alpha = __builtin_amdgcn_exp2f(m - mx);
             float psum = 0.f;
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                sacc[e] = __builtin_amdgcn_exp2f(sacc[e] - mx);
-                psum += sacc[e];
-            }
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    sacc[nb][e] = __builtin_amdgcn_exp2f(sacc[nb][e] - mx);
+                    psum += sacc[nb][e];
+                }
             psum += __shfl_xor(psum, 32, 64);
             l = l * alpha + psum;
             m = mx;
@@ -305,11 +320,15 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
                     for (int e = 0; e < 16; ++e) oacc[b][e] *= alpha;
                 }
 #pragma unroll
-                for (int c = 0; c < AF_KEYS / 8; ++c)
+                for (int nb = 0; nb < NB; ++nb) {
+                    if (!live[nb]) continue;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[(8 * c + 4 * h + j) * VPITCH + 32 * b + r], sacc[4 * c + j],
-                                                                       oacc[b], 0, 0, 0);
+                    for (int c = 0; c < 4; ++c)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[(32 * nb + 8 * c + 4 * h + j) * VPITCH + 32 * b + r],
+                                                                           sacc[nb][4 * c + j], oacc[b], 0, 0, 0);
+                }
             }
         }
         MNI_AF_PARK(cur ^ 1)
@@ -339,12 +358,13 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
     if (s > 0x7fffff00LL || bh * qblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
-#define MNI_AF(DBV) hipLaunchKernelGGL(attn_fused_fwd_kernel<DBV>, grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, scale, causal)
+#define MNI_AF(DBV, NBV) hipLaunchKernelGGL((attn_fused_fwd_kernel<DBV, NBV>), grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, scale, causal)
     switch (d / 32) {
-        case 1: MNI_AF(1); break;
-        case 2: MNI_AF(2); break;
-        case 3: MNI_AF(3); break;
-        default: MNI_AF(4); break;
+        // 64 keys per step while two workgroups still fit a CU's LDS, 32 beyond
+        case 1: MNI_AF(1, 2); break;
+        case 2: MNI_AF(2, 2); break;
+        case 3: MNI_AF(3, 1); break;
+        default: MNI_AF(4, 1); break;
     }
 #undef MNI_AF
     return check_launch("attn_fused_forward");
