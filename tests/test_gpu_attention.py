@@ -85,6 +85,25 @@ def test_attention_forward_and_backward_match_the_oracle(both, bh, s, d, causal)
     assert max_err(res[0][2], res[1][2]) <= gtol * mw * mv * mq * scale * 2  # dk = dS^T q
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bh,s,d", [(2, 4096, 64), (1, 3001, 128), (3, 1000, 32)])
+def test_long_attention_forward_against_float64(rocm_native, bh, s, d, causal):
+    """Sequences of thousands of positions through the one-kernel forward (dozens of key steps, query and key
+    tails, every wavefront's diagonal) against a float64 softmax(q k^T) v."""
+    rocm_native.resetEngine()
+    gpu = bind(rocm_native)
+    q, k, v = (synth.normal(9, (bh, s, d), stream=i) for i in range(3))
+    scale = 1.0 / math.sqrt(d)
+    got = gpu.flashAttention(_t(gpu, q), _t(gpu, k), _t(gpu, v), scale, causal).numpy()
+    for b in range(bh):
+        sc = (q[b].astype(np.float64) @ k[b].astype(np.float64).T) * scale
+        if causal:
+            sc = np.where(np.tri(s, dtype=bool), sc, -np.inf)
+        p = np.exp(sc - sc.max(1, keepdims=True))
+        want = (p / p.sum(1, keepdims=True)) @ v[b].astype(np.float64)
+        assert max_err(got[b], want) <= 1e-5 * float(np.abs(v).max())
+
+
 def test_attention_known_answers_on_the_gpu(both):
     gpu, _ = both
     bh, s, d = 2, 70, 8
