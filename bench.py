@@ -224,6 +224,13 @@ def bench_extras(r):
         api.native.zeroGrad([qa._id, ka._id, va._id])
         api.flashAttention(qa, ka, va, 0.125, True).mul(wa).sum().backward()
     ms_all = time_step(att_step, keep_att, 20, 5)
+    # the one-kernel forward on long sequences ([8, 8192, 64] and [16, 4096, 128], causal): useful flops = half of dense
+    for lb, ls, ld in ((8, 8192, 64), (16, 4096, 128)):
+        ql, kl, vl = (T(synth.normal(2, (lb, ls, ld), stream=i)) for i in range(3))
+        keep_long = lambda: [ql._id, kl._id, vl._id] + keep_att()
+        ms_long = time_step(lambda: api.flashAttention(ql, kl, vl, 1.0 / math.sqrt(ld), True), keep_long, 10, 3)
+        out["attention_fwd_%dx%dx%d_causal" % (lb, ls, ld)] = {"ms": ms_long, "useful_TFLOP/s": 2.0 * lb * ls * ls * ld / ms_long / 1e9}
+        api.native.gcTensors(keep_att())
     dense = 2.0 * bh * s * s * d  # one s x s x d product, mask not exploited
     out["attention_32x512x64_causal"] = {"fwd_ms": ms_fwd, "fwd_bwd_ms": ms_all,
                                          "fwd_TFLOP/s_dense_count": 2 * dense / ms_fwd / 1e9,
@@ -356,6 +363,14 @@ def run_for_counters(r, which):
         a, b = r.to_device(synth.normal(1, (4096, 3072))), r.to_device(synth.normal(1, (3072, 768), stream=1))
         for _ in range(5):
             r.sgemm(4096, 768, 3072, a, b, dst)
+    elif which == "attention":
+        # the one-kernel attention forward on [8, 8192, 64], causal, through the engine entry point
+        from framework_amd.api import bind
+        api = bind(N.Native())
+        q, k, v = (api.Tensor.fromFloat32(synth.normal(2, (8, 8192, 64), stream=i), [8, 8192, 64]) for i in range(3))
+        for _ in range(5):
+            api.flashAttention(q, k, v, 0.125, True)
+            api.native.gcTensors([q._id, k._id, v._id])
     else:
         x, w = r.to_device(synth.normal(4, (4, 4096), 0.02)), r.to_device(synth.normal(4, (4096, 4096), 0.02, stream=1))
         for _ in range(5):
@@ -400,7 +415,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
-    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk"], default=None,
+    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "attention"], default=None,
                     help="for rocprofv3 --pmc runs: launch a copy kernel of known size (64 MiB read + 64 MiB "
                          "written) 3 times, then the chosen product 5 times, and exit")
     args = ap.parse_args()
