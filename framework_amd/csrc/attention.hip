@@ -370,6 +370,327 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
     return check_launch("attn_fused_forward");
 }
 
+// ---- attention backward, query side -----------------------------------------------------
+// dq = dS k with dS = P (dP - di) scale, P = exp(scale q k^T - lse), dP = dO v^T
+// (ops/attention.rs:143-202), for the head dims of the one-kernel forward and
+// with the same layout: a workgroup owns 128 queries, one per lane, and walks
+// the keys 32 at a time.  S^T = K Q^T and dP^T = V dO^T take the key / value
+// tiles from LDS ([d/4][key] float4) and the lane's own q / dO rows from
+// registers; lse and di are one scalar per lane; dS^T stays in the accumulator
+// registers and is operand B of dQ^T += K^T dS^T, whose operand A is the key
+// tile once more, kept in LDS a second time as plain [key][d] rows.
+template <int DB>
+__global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_kernel(float *__restrict__ dq, const float *__restrict__ q,
+                                                                       const float *__restrict__ k, const float *__restrict__ v,
+                                                                       const float *__restrict__ dout, const float *__restrict__ lse,
+                                                                       const float *__restrict__ di, int s, int qblocks, float scale,
+                                                                       int causal) {
+    constexpr int D = 32 * DB, DQ = D / 4, KEYS = 32;
+    constexpr int TPITCH = KEYS + 1;  // float4 per d-quad slice of a [d/4][key] tile
+    constexpr int RPITCH = D + 8;     // floats per row of the [key][d] copy of the key tile
+    constexpr int TSTAGE = DQ * TPITCH, RSTAGE = KEYS * RPITCH;
+    constexpr int NLD = KEYS * DQ / ATT_TPB;  // float4 of each tile per thread (1 .. 4)
+    __shared__ float4 kt[2 * TSTAGE];
+    __shared__ float4 vt[2 * TSTAGE];
+    __shared__ __align__(16) float kr[2 * RSTAGE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int64_t bh = blockIdx.x / qblocks;
+    const int qb = qblocks - 1 - (int)(blockIdx.x % qblocks);  // late query blocks (most keys under the mask) first
+    const int qi = qb * AF_QUERIES + wave * 32 + r;
+    const int ql = min(qi, s - 1);
+    const int64_t row = bh * s + ql;
+    const float *kbase = k + bh * s * (int64_t)D, *vbase = v + bh * s * (int64_t)D;
+    float4 qf[D / 8], gf[D / 8];  // the d quads 2c + h of the lane's q and dO rows
+#pragma unroll
+    for (int c = 0; c < D / 8; ++c) {
+        qf[c] = *reinterpret_cast<const float4 *>(q + row * D + 4 * (2 * c + h));
+        gf[c] = *reinterpret_cast<const float4 *>(dout + row * D + 4 * (2 * c + h));
+    }
+    const float lse2 = lse[row] * 1.4426950408889634f, dil = di[row];
+    const float scale2 = scale * 1.4426950408889634f;
+    att_f16 qacc[DB];
+#pragma unroll
+    for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) qacc[b][e] = 0.f;
+    const int nkeys = causal ? min(s, (qb + 1) * AF_QUERIES) : s;
+    const int nsteps = (nkeys + KEYS - 1) / KEYS;
+    const int wave_first = qb * AF_QUERIES + wave * 32;
+    const int wave_last = min(wave_first + 31, s - 1);
+
+    float4 kreg[NLD], vreg[NLD];
+    int src_off[NLD], t_slot[NLD], r_slot[NLD], key_of[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int f = tid + ATT_TPB * i;
+        key_of[i] = f / DQ;
+        src_off[i] = 4 * (f % DQ);
+        t_slot[i] = (f % DQ) * TPITCH + f / DQ;
+        r_slot[i] = (f / DQ) * RPITCH + 4 * (f % DQ);
+    }
+#define MNI_AB_REQUEST(STEP)                                                                          \
+    _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
+        const int64_t src = (int64_t)min((STEP) * KEYS + key_of[i], s - 1) * D + src_off[i];           \
+        kreg[i] = *reinterpret_cast<const float4 *>(kbase + src);                                     \
+        vreg[i] = *reinterpret_cast<const float4 *>(vbase + src);                                     \
+    }
+#define MNI_AB_PARK(STAGE)                                                                            \
+    _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
+        kt[(STAGE) * TSTAGE + t_slot[i]] = kreg[i];                                                   \
+        vt[(STAGE) * TSTAGE + t_slot[i]] = vreg[i];                                                   \
+        *reinterpret_cast<float4 *>(kr + (STAGE) * RSTAGE + r_slot[i]) = kreg[i];                     \
+    }
+    MNI_AB_REQUEST(0)
+    MNI_AB_PARK(0)
+    __syncthreads();
+    for (int step = 0; step < nsteps; ++step) {
+        const int k0 = step * KEYS;
+        const int cur = step & 1;
+        MNI_AB_REQUEST(min(step + 1, nsteps - 1))
+        if (!causal || k0 <= wave_last) {
+            const float4 *ks = kt + cur * TSTAGE, *vs = vt + cur * TSTAGE;
+            const float *krow = kr + cur * RSTAGE;
+            att_f16 sacc, pacc;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; pacc[e] = 0.f; }
+#pragma unroll
+            for (int c = 0; c < D / 8; ++c) {
+                const float4 ka = ks[(2 * c + h) * TPITCH + r], va = vs[(2 * c + h) * TPITCH + r];
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qf[c].x, sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(va.x, gf[c].x, pacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qf[c].y, sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(va.y, gf[c].y, pacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qf[c].z, sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(va.z, gf[c].z, pacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.w, qf[c].w, sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(va.w, gf[c].w, pacc, 0, 0, 0);
+            }
+            // dS^T = P^T (dP^T - di) scale, 0 where the mask (or the end of the keys) forbids
+            const bool edge = k0 + KEYS > s || (causal && k0 + KEYS - 1 > wave_first);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float p = __builtin_amdgcn_exp2f(sacc[e] * scale2 - lse2);
+                float ds = p * (pacc[e] - dil) * scale;
+                if (edge) {
+                    const int key = k0 + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (!(key < s && (!causal || key <= ql))) ds = 0.f;
+                }
+                sacc[e] = ds;
+            }
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        qacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[(8 * c + 4 * h + j) * RPITCH + 32 * b + r], sacc[4 * c + j],
+                                                                       qacc[b], 0, 0, 0);
+        }
+        MNI_AB_PARK(cur ^ 1)
+        __syncthreads();
+    }
+#undef MNI_AB_REQUEST
+#undef MNI_AB_PARK
+    if (qi < s) {
+        float *orow = dq + (bh * s + qi) * (int64_t)D;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4)
+                *reinterpret_cast<float4 *>(orow + 32 * b + 8 * g4 + 4 * h) =
+                    make_float4(qacc[b][4 * g4], qacc[b][4 * g4 + 1], qacc[b][4 * g4 + 2], qacc[b][4 * g4 + 3]);
+    }
+}
+int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const float *v, const float *dout, const float *lse,
+                             const float *di, int64_t bh, int64_t s, int64_t d, float scale, int causal) {
+    if (bh <= 0 || s <= 0) return MNI_OK;
+    if (!attn_fused_supported(d)) return set_error(MNI_ERR_INVALID, "fused attention: head dim %lld is not 32, 64, 96 or 128", (long long)d);
+    MNI_TRY(ensure_init());
+    const int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
+    if (s > 0x7fffff00LL || bh * qblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
+    hipStream_t st = ctx().stream;
+#define MNI_AB(DBV) hipLaunchKernelGGL(attn_fused_bwd_dq_kernel<DBV>, grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, scale, causal)
+    switch (d / 32) {
+        case 1: MNI_AB(1); break;
+        case 2: MNI_AB(2); break;
+        case 3: MNI_AB(3); break;
+        default: MNI_AB(4); break;
+    }
+#undef MNI_AB
+    return check_launch("attn_fused_backward_dq");
+}
+
+// ---- attention backward, key side ---------------------------------------------------------
+// dv = P^T dO and dk = dS^T q with the roles swapped: a workgroup owns 128 keys,
+// one per lane (its k and v rows in registers), and walks the queries 32 at a
+// time.  S = Q K^T and dP = dO V^T take the query / dO tiles from LDS
+// ([d/4][query] float4); lane (key r, half h) receives queries 8(e/4) + 4h + e%4,
+// whose lse and di come from LDS four at a time.  P and dS stay in the
+// accumulator registers as operand B of dV^T += dO^T P and dK^T += Q^T dS, whose
+// operands A are the dO / query tiles once more, kept as plain [query][d] rows.
+// Under the causal mask a key block starts at its own first query.
+template <int DB>
+__global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv_kernel(
+    float *__restrict__ dk, float *__restrict__ dv, const float *__restrict__ q, const float *__restrict__ k,
+    const float *__restrict__ v, const float *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ di, int s,
+    int kblocks, float scale, int causal) {
+    constexpr int D = 32 * DB, DQ = D / 4, QT = 32;
+    constexpr int TPITCH = QT + 1, RPITCH = D + 8;
+    constexpr int TSTAGE = DQ * TPITCH, RSTAGE = QT * RPITCH;
+    constexpr int NLD = QT * DQ / ATT_TPB;
+    __shared__ float4 qt[2 * TSTAGE];
+    __shared__ float4 gt[2 * TSTAGE];
+    __shared__ __align__(16) float qr[2 * RSTAGE];
+    __shared__ __align__(16) float gr[2 * RSTAGE];
+    __shared__ __align__(16) float lt[2 * QT];
+    __shared__ __align__(16) float dt[2 * QT];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int64_t bh = blockIdx.x / kblocks;
+    const int kb = (int)(blockIdx.x % kblocks);  // early key blocks see the most queries under the mask: they come first anyway
+    const int kj = kb * AF_QUERIES + wave * 32 + r;  // this lane's key
+    const int kl = min(kj, s - 1);
+    const int64_t base = bh * s;
+    const float *qbase = q + base * (int64_t)D, *gbase = dout + base * (int64_t)D;
+    float4 kf[D / 8], vf[D / 8];  // the d quads 2c + h of the lane's k and v rows
+#pragma unroll
+    for (int c = 0; c < D / 8; ++c) {
+        kf[c] = *reinterpret_cast<const float4 *>(k + (base + kl) * D + 4 * (2 * c + h));
+        vf[c] = *reinterpret_cast<const float4 *>(v + (base + kl) * D + 4 * (2 * c + h));
+    }
+    const float scale2 = scale * 1.4426950408889634f;
+    att_f16 kacc[DB], vacc[DB];
+#pragma unroll
+    for (int b = 0; b < DB; ++b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { kacc[b][e] = 0.f; vacc[b][e] = 0.f; }
+    const int q_begin = causal ? kb * AF_QUERIES : 0;  // queries before the block's first key see none of its keys
+    const int nsteps = (s - q_begin + QT - 1) / QT;    // >= 1: the block holds at least one key < s
+    const int wave_first = kb * AF_QUERIES + wave * 32;  // first key of this wavefront
+
+    float4 qreg[NLD], greg[NLD];
+    float lreg, dreg;
+    int src_off[NLD], t_slot[NLD], r_slot[NLD], row_of[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int f = tid + ATT_TPB * i;
+        row_of[i] = f / DQ;
+        src_off[i] = 4 * (f % DQ);
+        t_slot[i] = (f % DQ) * TPITCH + f / DQ;
+        r_slot[i] = (f / DQ) * RPITCH + 4 * (f % DQ);
+    }
+#define MNI_AK_REQUEST(STEP)                                                                          \
+    _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
+        const int64_t src = (int64_t)min(q_begin + (STEP) * QT + row_of[i], s - 1) * D + src_off[i];   \
+        qreg[i] = *reinterpret_cast<const float4 *>(qbase + src);                                     \
+        greg[i] = *reinterpret_cast<const float4 *>(gbase + src);                                     \
+    }                                                                                                 \
+    lreg = lse[base + min(q_begin + (STEP) * QT + (tid & 31), s - 1)] * 1.4426950408889634f;           \
+    dreg = di[base + min(q_begin + (STEP) * QT + (tid & 31), s - 1)];
+#define MNI_AK_PARK(STAGE)                                                                            \
+    _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
+        qt[(STAGE) * TSTAGE + t_slot[i]] = qreg[i];                                                   \
+        gt[(STAGE) * TSTAGE + t_slot[i]] = greg[i];                                                   \
+        *reinterpret_cast<float4 *>(qr + (STAGE) * RSTAGE + r_slot[i]) = qreg[i];                     \
+        *reinterpret_cast<float4 *>(gr + (STAGE) * RSTAGE + r_slot[i]) = greg[i];                     \
+    }                                                                                                 \
+    if (tid < QT) { lt[(STAGE) * QT + tid] = lreg; dt[(STAGE) * QT + tid] = dreg; }
+    MNI_AK_REQUEST(0)
+    MNI_AK_PARK(0)
+    __syncthreads();
+    for (int step = 0; step < nsteps; ++step) {
+        const int q0 = q_begin + step * QT;
+        const int cur = step & 1;
+        MNI_AK_REQUEST(min(step + 1, nsteps - 1))
+        // a wavefront whose keys all come after this query tile receives nothing from it (causal)
+        if (!causal || q0 + QT - 1 >= wave_first) {
+            const float4 *qs = qt + cur * TSTAGE, *gs = gt + cur * TSTAGE;
+            const float *qrow = qr + cur * RSTAGE, *grow = gr + cur * RSTAGE;
+            att_f16 sacc, pacc;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; pacc[e] = 0.f; }
+#pragma unroll
+            for (int c = 0; c < D / 8; ++c) {
+                const float4 qa = qs[(2 * c + h) * TPITCH + r], ga = gs[(2 * c + h) * TPITCH + r];
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.x, kf[c].x, sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ga.x, vf[c].x, pacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.y, kf[c].y, sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ga.y, vf[c].y, pacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.z, kf[c].z, sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ga.z, vf[c].z, pacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.w, kf[c].w, sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ga.w, vf[c].w, pacc, 0, 0, 0);
+            }
+            // P and dS for the queries 8 g + 4 h + 0..3 of accumulator elements 4 g .. 4 g + 3
+            const bool edge = q0 + QT > s || kj >= s || (causal && q0 < wave_first + 32);
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const float4 l4 = *reinterpret_cast<const float4 *>(lt + cur * QT + 8 * g4 + 4 * h);
+                const float4 d4 = *reinterpret_cast<const float4 *>(dt + cur * QT + 8 * g4 + 4 * h);
+                const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int e = 4 * g4 + j;
+                    float p = __builtin_amdgcn_exp2f(sacc[e] * scale2 - ls[j]);
+                    if (edge) {
+                        const int query = q0 + 8 * g4 + 4 * h + j;
+                        if (!(query < s && kj < s && (!causal || kj <= query))) p = 0.f;
+                    }
+                    sacc[e] = p;
+                    pacc[e] = p * (pacc[e] - dd[j]) * scale;
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int at = (8 * c + 4 * h + j) * RPITCH + 32 * b + r;
+                        vacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(grow[at], sacc[4 * c + j], vacc[b], 0, 0, 0);
+                        kacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(qrow[at], pacc[4 * c + j], kacc[b], 0, 0, 0);
+                    }
+        }
+        MNI_AK_PARK(cur ^ 1)
+        __syncthreads();
+    }
+#undef MNI_AK_REQUEST
+#undef MNI_AK_PARK
+    if (kj < s) {
+        float *krow = dk + (base + kj) * (int64_t)D, *vrow = dv + (base + kj) * (int64_t)D;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                *reinterpret_cast<float4 *>(krow + 32 * b + 8 * g4 + 4 * h) =
+                    make_float4(kacc[b][4 * g4], kacc[b][4 * g4 + 1], kacc[b][4 * g4 + 2], kacc[b][4 * g4 + 3]);
+                *reinterpret_cast<float4 *>(vrow + 32 * b + 8 * g4 + 4 * h) =
+                    make_float4(vacc[b][4 * g4], vacc[b][4 * g4 + 1], vacc[b][4 * g4 + 2], vacc[b][4 * g4 + 3]);
+            }
+    }
+}
+int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float *k, const float *v, const float *dout,
+                              const float *lse, const float *di, int64_t bh, int64_t s, int64_t d, float scale, int causal) {
+    if (bh <= 0 || s <= 0) return MNI_OK;
+    if (!attn_fused_supported(d)) return set_error(MNI_ERR_INVALID, "fused attention: head dim %lld is not 32, 64, 96 or 128", (long long)d);
+    MNI_TRY(ensure_init());
+    const int64_t kblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
+    if (s > 0x7fffff00LL || bh * kblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    const dim3 grid((unsigned)(bh * kblocks)), block(ATT_TPB);
+    hipStream_t st = ctx().stream;
+#define MNI_AK(DBV) hipLaunchKernelGGL(attn_fused_bwd_dkv_kernel<DBV>, grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, scale, causal)
+    switch (d / 32) {
+        case 1: MNI_AK(1); break;
+        case 2: MNI_AK(2); break;
+        case 3: MNI_AK(3); break;
+        default: MNI_AK(4); break;
+    }
+#undef MNI_AK
+    return check_launch("attn_fused_backward_dkv");
+}
+
 // di[row] = sum_d a[row][d] * b[row][d] (ops/attention.rs:167-170)
 __global__ void rowdot_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, int64_t rows,
                               int64_t d) {

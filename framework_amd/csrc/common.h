@@ -124,6 +124,11 @@ int k_rowdot(float *out, const float *a, const float *b, int64_t rows, int64_t d
 bool attn_fused_supported(int64_t d);
 int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k, const float *v, int64_t bh, int64_t s, int64_t d,
                          float scale, int causal);
+// dq of the attention backward in one kernel (same head dims); di[row] = sum_d dO * O.
+int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const float *v, const float *dout, const float *lse,
+                             const float *di, int64_t bh, int64_t s, int64_t d, float scale, int causal);
+int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float *k, const float *v, const float *dout,
+                              const float *lse, const float *di, int64_t bh, int64_t s, int64_t d, float scale, int causal);
 int k_attn_backward(float *scores, float *dp, const float *lse, const float *di, int64_t rows, int64_t s, float scale,
                     int causal);
 int k_kv_append(void *kc, void *vc, float *ks, float *vs, const float *k, const float *v, int64_t bh, int64_t d,

@@ -1120,10 +1120,17 @@ static int flash_attention_backward(uint32_t grad, const Entry &e, int64_t *out)
     BufP qc = contiguous_buf(*Q), kc = contiguous_buf(*K), vc = contiguous_buf(*V);
     BufP oc = contiguous_buf(*O), lc = contiguous_buf(*L), gc = contiguous_buf(*G);
     if (!qc || !kc || !vc || !oc || !lc || !gc) return MNI_ERR_NOMEM;
-    BufP p = new_buf((size_t)(bh * s * s)), ds = new_buf((size_t)(bh * s * s)), di = new_buf((size_t)(bh * s));
+    BufP di = new_buf((size_t)(bh * s));
     BufP dq = new_buf((size_t)total), dk = new_buf((size_t)total), dv = new_buf((size_t)total);
-    if (!p || !ds || !di || !dq || !dk || !dv) return MNI_ERR_NOMEM;
-    if (total > 0) {
+    if (!di || !dq || !dk || !dv) return MNI_ERR_NOMEM;
+    if (total > 0 && attn_fused_supported(d)) {
+        // head dims 32 .. 128: two kernels that recompute P from lse, nothing of size s x s is stored
+        MNI_TRY(k_rowdot(di->p, gc->p, oc->p, bh * s, d));
+        MNI_TRY(k_attn_fused_backward_dq(dq->p, qc->p, kc->p, vc->p, gc->p, lc->p, di->p, bh, s, d, e.scalar, e.act));
+        MNI_TRY(k_attn_fused_backward_dkv(dk->p, dv->p, qc->p, kc->p, vc->p, gc->p, lc->p, di->p, bh, s, d, e.scalar, e.act));
+    } else if (total > 0) {
+        BufP p = new_buf((size_t)(bh * s * s)), ds = new_buf((size_t)(bh * s * s));
+        if (!p || !ds) return MNI_ERR_NOMEM;
         MNI_TRY(k_rowdot(di->p, gc->p, oc->p, bh * s, d));
         MNI_TRY(attn_gemm(p->p, qc->p, false, kc->p, true, bh, s, s, d));   // q k^T
         MNI_TRY(attn_gemm(ds->p, gc->p, false, vc->p, true, bh, s, s, d));  // dO v^T
