@@ -104,6 +104,34 @@ def test_long_attention_forward_against_float64(rocm_native, bh, s, d, causal):
         assert max_err(got[b], want) <= 1e-5 * float(np.abs(v).max())
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bh,s,d", [(2, 1500, 64), (1, 1031, 128), (2, 700, 32)])
+def test_long_attention_backward_against_float64(rocm_native, bh, s, d, causal):
+    """The two backward kernels over dozens of key / query steps against the closed form in float64:
+    dV = P^T dO, dP = dO V^T, dS = P (dP - rowsum(dO O)) scale, dQ = dS K, dK = dS^T Q."""
+    rocm_native.resetEngine()
+    gpu = bind(rocm_native)
+    q, k, v, w = (synth.normal(10, (bh, s, d), stream=i) for i in range(4))
+    scale = 1.0 / math.sqrt(d)
+    Q, K, V = (_t(gpu, a, True) for a in (q, k, v))
+    gpu.flashAttention(Q, K, V, scale, causal).mul(_t(gpu, w)).sum().backward()
+    got = [T.grad.numpy() for T in (Q, K, V)]
+    for b in range(bh):
+        q64, k64, v64, w64 = (a[b].astype(np.float64) for a in (q, k, v, w))
+        sc = (q64 @ k64.T) * scale
+        if causal:
+            sc = np.where(np.tri(s, dtype=bool), sc, -np.inf)
+        p = np.exp(sc - sc.max(1, keepdims=True))
+        p /= p.sum(1, keepdims=True)
+        o = p @ v64
+        dp = w64 @ v64.T
+        ds = p * (dp - (w64 * o).sum(1, keepdims=True)) * scale
+        tol = 1e-4 * math.sqrt(s) * float(np.abs(w).max()) * float(np.abs(v).max())
+        assert max_err(got[2][b], p.T @ w64) <= tol
+        assert max_err(got[0][b], ds @ k64) <= tol * float(np.abs(k).max()) * scale * 2
+        assert max_err(got[1][b], ds.T @ q64) <= tol * float(np.abs(q).max()) * scale * 2
+
+
 def test_attention_known_answers_on_the_gpu(both):
     gpu, _ = both
     bh, s, d = 2, 70, 8
