@@ -259,9 +259,11 @@ uint32_t mni_bias_gelu(uint32_t x, uint32_t bias);
 uint32_t mni_softmax_op(uint32_t a, int64_t dim);
 /* flash_attention (src/native/src/lib.rs:575-584 -> ops/attention.rs:14-78,
  * backward :143-202): q, k, v taken as [bh, s, d] from their first three dims;
- * returns out [bh, s, d].  Built on the batched GEMM (q k^T, P v and the five
- * backward products) with row kernels for scale / causal mask / normalisation,
- * in place of the per-key loop of kernels/flash_attention.cu. */
+ * returns out [bh, s, d].  Head dims 32, 64, 96 and 128 run the forward in one
+ * MFMA kernel and the backward in two (scores and probabilities never reach
+ * memory); other head dims are built on the batched GEMM (q k^T, P v and the
+ * five backward products) with row kernels for scale / causal mask /
+ * normalisation.  Either replaces the per-key loop of kernels/flash_attention.cu. */
 uint32_t mni_flash_attention(uint32_t q, uint32_t k, uint32_t v, double scale, int causal);
 /* lib.rs:295-300 */
 uint32_t mni_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n); /* lib.rs:328-336 */
