@@ -178,12 +178,27 @@ int k_attn_softmax(float *scores, float *lse, int64_t rows, int64_t s, float sca
 //                 value tile in LDS.  Rescaling the running output is one
 //                 factor per lane.
 typedef float att_f16 __attribute__((ext_vector_type(16)));
+
+// Which block of which head a workgroup takes.  Under the causal mask the blocks of a head differ in
+// work by a factor of up to their number, and the kernels below keep two workgroups on a CU, so what
+// counts is the sum of the two that share one.  The hardware hands workgroup x and workgroup x + CUs to
+// the same CU while the first two per CU are being placed.  So the first `pair` workgroups take the
+// heaviest blocks in falling order and the next `pair` the blocks that follow in rising order -- heavy
+// meets light on every CU -- and whatever is left goes on in falling order to the slots that free up.
+// rank 0 is the heaviest block; pair = CUs when two workgroups fit a CU, a huge value otherwise.
+__device__ __forceinline__ void attn_item(int nblocks, int pair, int &rank, int64_t &bh) {
+    const int total = (int)gridDim.x, heads = total / nblocks;
+    int t = (int)blockIdx.x;
+    if (t >= pair && t - pair < pair) t = pair + min(total - pair, pair) - 1 - (t - pair);
+    rank = t / heads;
+    bh = t % heads;
+}
 static constexpr int AF_QUERIES = 128;
 template <int DB, int NB>  // head dim = 32 * DB, keys per step = 32 * NB
 __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__restrict__ out, float *__restrict__ lse,
                                                                     const float *__restrict__ q, const float *__restrict__ k,
-                                                                    const float *__restrict__ v, int s, int qblocks, float scale,
-                                                                    int causal) {
+                                                                    const float *__restrict__ v, int s, int qblocks, int pair,
+                                                                    float scale, int causal) {
     constexpr int D = 32 * DB, DQ = D / 4, KEYS = 32 * NB;
     constexpr int KPITCH = KEYS + 1;  // float4 per d-quad slice (+1: the tile stores of consecutive quads spread over the banks)
     constexpr int VPITCH = D + 8;     // floats per key row (+8: the two lane halves, 4 keys apart, use different banks)
@@ -193,9 +208,10 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
     __shared__ __align__(16) float vt[2 * VSTAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int64_t bh = blockIdx.x / qblocks;
-    // blocks of late queries have the most keys to visit under the causal mask: they go first
-    const int qb = qblocks - 1 - (int)(blockIdx.x % qblocks);
+    int rank;
+    int64_t bh;
+    attn_item(qblocks, pair, rank, bh);
+    const int qb = qblocks - 1 - rank;  // late queries have the most keys to visit under the causal mask
     const int qi = qb * AF_QUERIES + wave * 32 + r;  // this lane's query
     const int ql = min(qi, s - 1);                   // (queries beyond the end compute on the last one and store nothing)
     const float *qrow = q + (bh * s + ql) * (int64_t)D;
@@ -348,6 +364,20 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
         if (h == 0) lse[bh * s + qi] = m * 0.6931471805599453f + logf(l);  // back from log2 units
     }
 }
+// The distance in launch order between the two workgroups that share a CU (see attn_item): the number of
+// CUs when at least two workgroups of `kernel` fit one, otherwise a value no grid reaches.
+template <auto Kernel>
+static int attn_pair() {
+    static int fit = 0;  // per kernel instantiation; the answer does not change while the process lives
+    if (fit == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, Kernel, ATT_TPB, 0) != hipSuccess) (void)hipGetLastError();
+        fit = n >= 1 ? n : 1;
+    }
+    const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
+    return fit >= 2 ? cus : 0x7fffffff;
+}
+
 bool attn_fused_supported(int64_t d) { return d == 32 || d == 64 || d == 96 || d == 128; }
 int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k, const float *v, int64_t bh, int64_t s, int64_t d,
                          float scale, int causal) {
@@ -358,7 +388,7 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
     if (s > 0x7fffff00LL || bh * qblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
-#define MNI_AF(DBV, NBV) hipLaunchKernelGGL((attn_fused_fwd_kernel<DBV, NBV>), grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, scale, causal)
+#define MNI_AF(DBV, NBV) hipLaunchKernelGGL((attn_fused_fwd_kernel<DBV, NBV>), grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, attn_pair<attn_fused_fwd_kernel<DBV, NBV>>(), scale, causal)
     switch (d / 32) {
         // 64 keys per step while two workgroups still fit a CU's LDS, 32 beyond
         case 1: MNI_AF(1, 2); break;
@@ -383,7 +413,7 @@ template <int DB>
 __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_kernel(float *__restrict__ dq, const float *__restrict__ q,
                                                                        const float *__restrict__ k, const float *__restrict__ v,
                                                                        const float *__restrict__ dout, const float *__restrict__ lse,
-                                                                       const float *__restrict__ di, int s, int qblocks, float scale,
+                                                                       const float *__restrict__ di, int s, int qblocks, int pair, float scale,
                                                                        int causal) {
     constexpr int D = 32 * DB, DQ = D / 4, KEYS = 32;
     constexpr int TPITCH = KEYS + 1;  // float4 per d-quad slice of a [d/4][key] tile
@@ -395,8 +425,10 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
     __shared__ __align__(16) float kr[2 * RSTAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int64_t bh = blockIdx.x / qblocks;
-    const int qb = qblocks - 1 - (int)(blockIdx.x % qblocks);  // late query blocks (most keys under the mask) first
+    int rank;
+    int64_t bh;
+    attn_item(qblocks, pair, rank, bh);
+    const int qb = qblocks - 1 - rank;  // late query blocks have the most keys under the mask
     const int qi = qb * AF_QUERIES + wave * 32 + r;
     const int ql = min(qi, s - 1);
     const int64_t row = bh * s + ql;
@@ -511,7 +543,7 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
     if (s > 0x7fffff00LL || bh * qblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
-#define MNI_AB(DBV) hipLaunchKernelGGL(attn_fused_bwd_dq_kernel<DBV>, grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, scale, causal)
+#define MNI_AB(DBV) hipLaunchKernelGGL(attn_fused_bwd_dq_kernel<DBV>, grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, attn_pair<attn_fused_bwd_dq_kernel<DBV>>(), scale, causal)
     switch (d / 32) {
         case 1: MNI_AB(1); break;
         case 2: MNI_AB(2); break;
@@ -535,7 +567,7 @@ template <int DB>
 __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv_kernel(
     float *__restrict__ dk, float *__restrict__ dv, const float *__restrict__ q, const float *__restrict__ k,
     const float *__restrict__ v, const float *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ di, int s,
-    int kblocks, float scale, int causal) {
+    int kblocks, int pair, float scale, int causal) {
     constexpr int D = 32 * DB, DQ = D / 4, QT = 32;
     constexpr int TPITCH = QT + 1, RPITCH = D + 8;
     constexpr int TSTAGE = DQ * TPITCH, RSTAGE = QT * RPITCH;
@@ -548,8 +580,9 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
     __shared__ __align__(16) float dt[2 * QT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int64_t bh = blockIdx.x / kblocks;
-    const int kb = (int)(blockIdx.x % kblocks);  // early key blocks see the most queries under the mask: they come first anyway
+    int kb;  // early key blocks see the most queries under the mask
+    int64_t bh;
+    attn_item(kblocks, pair, kb, bh);
     const int kj = kb * AF_QUERIES + wave * 32 + r;  // this lane's key
     const int kl = min(kj, s - 1);
     const int64_t base = bh * s;
@@ -680,7 +713,7 @@ int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float 
     if (s > 0x7fffff00LL || bh * kblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
     const dim3 grid((unsigned)(bh * kblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
-#define MNI_AK(DBV) hipLaunchKernelGGL(attn_fused_bwd_dkv_kernel<DBV>, grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, scale, causal)
+#define MNI_AK(DBV) hipLaunchKernelGGL(attn_fused_bwd_dkv_kernel<DBV>, grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, attn_pair<attn_fused_bwd_dkv_kernel<DBV>>(), scale, causal)
     switch (d / 32) {
         case 1: MNI_AK(1); break;
         case 2: MNI_AK(2); break;
