@@ -182,14 +182,20 @@ typedef float att_f16 __attribute__((ext_vector_type(16)));
 // Which block of which head a workgroup takes.  Under the causal mask the blocks of a head differ in
 // work by a factor of up to their number, and the kernels below keep two workgroups on a CU, so what
 // counts is the sum of the two that share one.  The hardware hands workgroup x and workgroup x + CUs to
-// the same CU while the first two per CU are being placed.  So the first `pair` workgroups take the
-// heaviest blocks in falling order and the next `pair` the blocks that follow in rising order -- heavy
-// meets light on every CU -- and whatever is left goes on in falling order to the slots that free up.
-// rank 0 is the heaviest block; pair = CUs when two workgroups fit a CU, a huge value otherwise.
+// the same CU while the first two per CU are being placed.  With the blocks numbered from the heaviest
+// (t = 0) and `pair` = CUs, the w = min(total - pair, pair) CUs that receive a second workgroup get
+// blocks pair - w + x and pair + w - 1 - x: the lightest 2w of the first 2 pair blocks, folded so that
+// heavy meets light, while the heaviest blocks run alone.  What is left after 2 pair workgroups goes on
+// in falling order to the slots that free up.  pair is a huge value when only one workgroup fits a CU.
 __device__ __forceinline__ void attn_item(int nblocks, int pair, int &rank, int64_t &bh) {
     const int total = (int)gridDim.x, heads = total / nblocks;
     int t = (int)blockIdx.x;
-    if (t >= pair && t - pair < pair) t = pair + min(total - pair, pair) - 1 - (t - pair);
+    if (total > pair && t - pair < pair) {
+        const int w = min(total - pair, pair);
+        if (t < w) t += pair - w;
+        else if (t < pair) t -= w;
+        else t = pair + w - 1 - (t - pair);
+    }
     rank = t / heads;
     bh = t % heads;
 }
