@@ -132,6 +132,37 @@ def test_long_attention_backward_against_float64(rocm_native, bh, s, d, causal):
         assert max_err(got[1][b], ds.T @ q64) <= tol * float(np.abs(q).max()) * scale * 2
 
 
+@pytest.mark.parametrize("bh,s,d", [(75, 512, 32), (40, 1000, 64), (64, 1024, 32), (50, 1750, 32), (65, 512, 32), (9, 3800, 32)])
+def test_attention_grids_beyond_one_workgroup_per_cu_against_float64(rocm_native, bh, s, d):
+    """More workgroups than the 256 CUs: the kernels then hand out the causal blocks in folded order (the
+    lightest blocks as second workgroups of the CUs that hold the matching heavy ones), for grids of 300, 320,
+    512, 700, 260 and 270 workgroups -- a partly filled second row, a full one, and a tail past it.  Every block
+    must still be computed exactly once: forward and all three gradients against the closed form in float64."""
+    rocm_native.resetEngine()
+    gpu = bind(rocm_native)
+    q, k, v, w = (synth.normal(11, (bh, s, d), stream=i) for i in range(4))
+    scale = 1.0 / math.sqrt(d)
+    Q, K, V = (_t(gpu, a, True) for a in (q, k, v))
+    out = gpu.flashAttention(Q, K, V, scale, True)
+    got_out = out.numpy()
+    out.mul(_t(gpu, w)).sum().backward()
+    got = [T.grad.numpy() for T in (Q, K, V)]
+    tol = 1e-4 * math.sqrt(s) * float(np.abs(w).max()) * float(np.abs(v).max())
+    mask = np.tri(s, dtype=bool)
+    for b in range(bh):
+        q64, k64, v64, w64 = (a[b].astype(np.float64) for a in (q, k, v, w))
+        sc = np.where(mask, (q64 @ k64.T) * scale, -np.inf)
+        p = np.exp(sc - sc.max(1, keepdims=True))
+        p /= p.sum(1, keepdims=True)
+        o = p @ v64
+        assert max_err(got_out[b], o) <= 1e-5 * float(np.abs(v).max()), b
+        dp = w64 @ v64.T
+        ds = p * (dp - (w64 * o).sum(1, keepdims=True)) * scale
+        assert max_err(got[2][b], p.T @ w64) <= tol, b
+        assert max_err(got[0][b], ds @ k64) <= tol * float(np.abs(k).max()) * scale * 2, b
+        assert max_err(got[1][b], ds.T @ q64) <= tol * float(np.abs(q).max()) * scale * 2, b
+
+
 def test_attention_known_answers_on_the_gpu(both):
     gpu, _ = both
     bh, s, d = 2, 70, 8
