@@ -371,6 +371,17 @@ def run_for_counters(r, which):
         for _ in range(5):
             api.flashAttention(q, k, v, 0.125, True)
             api.native.gcTensors([q._id, k._id, v._id])
+    elif which == "attention_bwd":
+        # forward + backward of the same attention: the query-owned and the key-owned backward kernels
+        from framework_amd.api import bind
+        api = bind(N.Native())
+        mk = lambda i, g: api.Tensor.fromFloat32(synth.normal(2, (8, 8192, 64), stream=i), [8, 8192, 64]).setRequiresGrad(g)
+        q, k, v, w = mk(0, True), mk(1, True), mk(2, True), mk(3, False)
+        for _ in range(3):
+            api.native.zeroGrad([t._id for t in (q, k, v)])
+            api.flashAttention(q, k, v, 0.125, True).mul(w).sum().backward()
+            grads = [g for g in (api.native.getGrad(t._id) for t in (q, k, v)) if g is not None]
+            api.native.gcTensors([t._id for t in (q, k, v, w)] + grads)
     else:
         x, w = r.to_device(synth.normal(4, (4, 4096), 0.02)), r.to_device(synth.normal(4, (4096, 4096), 0.02, stream=1))
         for _ in range(5):
@@ -415,7 +426,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
-    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "attention"], default=None,
+    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "attention", "attention_bwd"], default=None,
                     help="for rocprofv3 --pmc runs: launch a copy kernel of known size (64 MiB read + 64 MiB "
                          "written) 3 times, then the chosen product 5 times, and exit")
     args = ap.parse_args()
