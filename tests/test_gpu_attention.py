@@ -132,12 +132,15 @@ def test_long_attention_backward_against_float64(rocm_native, bh, s, d, causal):
         assert max_err(got[1][b], ds.T @ q64) <= tol * float(np.abs(q).max()) * scale * 2
 
 
-@pytest.mark.parametrize("bh,s,d", [(75, 512, 32), (40, 1000, 64), (64, 1024, 32), (50, 1750, 32), (65, 512, 32), (9, 3800, 32)])
+@pytest.mark.parametrize("bh,s,d", [(75, 512, 32), (40, 1000, 64), (64, 1024, 32), (50, 1750, 32), (65, 512, 32), (9, 3800, 32),
+                                    (70, 512, 96), (33, 1024, 128)])
 def test_attention_grids_beyond_one_workgroup_per_cu_against_float64(rocm_native, bh, s, d):
     """More workgroups than the 256 CUs: the kernels then hand out the causal blocks in folded order (the
     lightest blocks as second workgroups of the CUs that hold the matching heavy ones), for grids of 300, 320,
-    512, 700, 260 and 270 workgroups -- a partly filled second row, a full one, and a tail past it.  Every block
-    must still be computed exactly once: forward and all three gradients against the closed form in float64."""
+    512, 700, 260 and 270 workgroups -- a partly filled second row, a full one, and a tail past it -- and for
+    head dims 96 and 128, whose backward kernels fit one workgroup per CU and take the blocks in falling order.
+    Every block must still be computed exactly once: forward and all three gradients against the closed form in
+    float64."""
     rocm_native.resetEngine()
     gpu = bind(rocm_native)
     q, k, v, w = (synth.normal(11, (bh, s, d), stream=i) for i in range(4))
