@@ -200,12 +200,19 @@ __device__ __forceinline__ void attn_item(int nblocks, int pair, int &rank, int6
     bh = t % heads;
 }
 static constexpr int AF_QUERIES = 128;
-template <int DB, int NB>  // head dim = 32 * DB, keys per step = 32 * NB
+// SPLIT (with 64 keys per step): the workgroup owns 64 queries instead of 128 and its wavefronts pair up on
+// them, one taking keys 0 .. 31 and the other keys 32 .. 63 of every tile; the two partial results (running
+// maximum, sum and output) meet in LDS at the end.  Half the MFMAs per wavefront and step: for grids too
+// small to fill the chip, where the time is that of the longest chain of steps.
+template <int DB, int NB, bool SPLIT>  // head dim = 32 * DB, keys per step = 32 * NB
 __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__restrict__ out, float *__restrict__ lse,
                                                                     const float *__restrict__ q, const float *__restrict__ k,
                                                                     const float *__restrict__ v, int s, int qblocks, int pair,
                                                                     float scale, int causal) {
+    static_assert(!SPLIT || NB == 2, "the split form takes 64-key tiles");
     constexpr int D = 32 * DB, DQ = D / 4, KEYS = 32 * NB;
+    constexpr int QB = SPLIT ? 64 : AF_QUERIES;  // queries per workgroup
+    constexpr int NBW = SPLIT ? 1 : NB;          // blocks of 32 keys a wavefront takes out of a tile
     constexpr int KPITCH = KEYS + 1;  // float4 per d-quad slice (+1: the tile stores of consecutive quads spread over the banks)
     constexpr int VPITCH = D + 8;     // floats per key row (+8: the two lane halves, 4 keys apart, use different banks)
     constexpr int KSTAGE = DQ * KPITCH, VSTAGE = KEYS * VPITCH;
@@ -214,11 +221,13 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
     __shared__ __align__(16) float vt[2 * VSTAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
+    const int grp = SPLIT ? (wave & 1) : wave;      // which 32 queries of the workgroup
+    const int koff = SPLIT ? 32 * (wave >> 1) : 0;  // first key of a tile this wavefront takes
     int rank;
     int64_t bh;
     attn_item(qblocks, pair, rank, bh);
     const int qb = qblocks - 1 - rank;  // late queries have the most keys to visit under the causal mask
-    const int qi = qb * AF_QUERIES + wave * 32 + r;  // this lane's query
+    const int qi = qb * QB + grp * 32 + r;  // this lane's query
     const int ql = min(qi, s - 1);                   // (queries beyond the end compute on the last one and store nothing)
     const float *qrow = q + (bh * s + ql) * (int64_t)D;
     const float *kbase = k + bh * s * (int64_t)D, *vbase = v + bh * s * (int64_t)D;
@@ -232,9 +241,9 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
         for (int e = 0; e < 16; ++e) oacc[b][e] = 0.f;
     float m = -INFINITY, l = 0.f;
     // keys this workgroup needs: all of them, or those up to its last query
-    const int nkeys = causal ? min(s, (qb + 1) * AF_QUERIES) : s;
+    const int nkeys = causal ? min(s, (qb + 1) * QB) : s;
     const int nsteps = (nkeys + KEYS - 1) / KEYS;
-    const int wave_first = qb * AF_QUERIES + wave * 32;  // first query of this wavefront
+    const int wave_first = qb * QB + grp * 32;  // first query of this wavefront
     const int wave_last = min(wave_first + 31, s - 1);   // and its last
     const float scale2 = scale * 1.4426950408889634f;    // scores in units of log2
 
@@ -274,23 +283,23 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
         const int cur = step & 1;
         MNI_AF_REQUEST(min(step + 1, nsteps - 1))
         // a wavefront whose queries all come before this key tile has nothing to add (causal)
-        if (!causal || k0 <= wave_last) {
+        if ((!causal || k0 + koff <= wave_last) && k0 + koff < s) {
             const float4 *ks = kt + cur * KSTAGE;
             const float *vs = vt + cur * VSTAGE;
-            att_f16 sacc[NB];
-            bool live[NB];  // under the causal mask the later 32 keys of a step may all lie past this wavefront
+            att_f16 sacc[NBW];
+            bool live[NBW];  // under the causal mask the later 32 keys of a step may all lie past this wavefront
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                live[nb] = !causal || k0 + 32 * nb <= wave_last;
+            for (int nb = 0; nb < NBW; ++nb) {
+                live[nb] = !causal || k0 + koff + 32 * nb <= wave_last;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) sacc[nb][e] = 0.f;
                 if (live[nb]) {
                     // key fragments are fetched from LDS one d chunk ahead of the MFMAs that use them
-                    float4 ka = ks[h * KPITCH + 32 * nb + r];
+                    float4 ka = ks[h * KPITCH + koff + 32 * nb + r];
 #pragma unroll
                     for (int c = 0; c < D / 8; ++c) {
                         float4 na = ka;
-                        if (c + 1 < D / 8) na = ks[(2 * (c + 1) + h) * KPITCH + 32 * nb + r];
+                        if (c + 1 < D / 8) na = ks[(2 * (c + 1) + h) * KPITCH + koff + 32 * nb + r];
                         sacc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qf[c].x, sacc[nb], 0, 0, 0);
                         sacc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qf[c].y, sacc[nb], 0, 0, 0);
                         sacc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qf[c].z, sacc[nb], 0, 0, 0);
@@ -302,21 +311,21 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
             // From here on in units of log2: p = 2^(x - max) is one v_exp_f32.  Only a tile that
             // reaches past the last key or across the diagonal of this wavefront needs the mask.
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
+            for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) sacc[nb][e] *= scale2;
             if (k0 + KEYS > s || (causal && k0 + KEYS - 1 > wave_first)) {
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
+                for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        const int key = k0 + 32 * nb + 8 * (e >> 2) + 4 * h + (e & 3);
+                        const int key = k0 + koff + 32 * nb + 8 * (e >> 2) + 4 * h + (e & 3);
                         if (!(key < s && (!causal || key <= ql))) sacc[nb][e] = -INFINITY;
                     }
             }
             float mx = m;
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
+            for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[nb][e]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -324,7 +333,7 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
             const float alpha = __builtin_amdgcn_exp2f(m - mx);
             float psum = 0.f;
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
+            for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     sacc[nb][e] = __builtin_amdgcn_exp2f(sacc[nb][e] - mx);
@@ -342,13 +351,13 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
                     for (int e = 0; e < 16; ++e) oacc[b][e] *= alpha;
                 }
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
+                for (int nb = 0; nb < NBW; ++nb) {
                     if (!live[nb]) continue;
 #pragma unroll
                     for (int c = 0; c < 4; ++c)
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
-                            oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[(32 * nb + 8 * c + 4 * h + j) * VPITCH + 32 * b + r],
+                            oacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[(koff + 32 * nb + 8 * c + 4 * h + j) * VPITCH + 32 * b + r],
                                                                            sacc[nb][4 * c + j], oacc[b], 0, 0, 0);
                 }
             }
@@ -358,6 +367,32 @@ __global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__res
     }
 #undef MNI_AF_REQUEST
 #undef MNI_AF_PARK
+    if constexpr (SPLIT) {
+        // The wavefronts of the second key half hand (output, maximum, sum) to their partners through the
+        // tile memory, which the loop's last barrier has released: element x of lane l at [grp][x][l].
+        constexpr int NX = 16 * DB + 2;
+        static_assert(2 * NX * 64 * sizeof(float) <= sizeof(kt), "merge buffer must fit the key tiles");
+        float *mb = reinterpret_cast<float *>(kt) + grp * NX * 64 + lane;
+        if (koff != 0) {
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mb[(16 * b + e) * 64] = oacc[b][e];
+            mb[16 * DB * 64] = m;
+            mb[(16 * DB + 1) * 64] = l;
+        }
+        __syncthreads();
+        if (koff != 0) return;
+        const float m1 = mb[16 * DB * 64], l1 = mb[(16 * DB + 1) * 64];
+        const float mx = fmaxf(m, m1);  // m is finite: key 0 belongs to this half
+        const float a0 = __builtin_amdgcn_exp2f(m - mx), a1 = __builtin_amdgcn_exp2f(m1 - mx);
+        l = l * a0 + l1 * a1;
+        m = mx;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[b][e] = oacc[b][e] * a0 + mb[(16 * b + e) * 64] * a1;
+    }
     if (qi < s) {
         const float inv = 1.0f / l;
         float *orow = out + (bh * s + qi) * (int64_t)D;
@@ -390,17 +425,24 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
     if (bh <= 0 || s <= 0) return MNI_OK;
     if (!attn_fused_supported(d)) return set_error(MNI_ERR_INVALID, "fused attention: head dim %lld is not 32, 64, 96 or 128", (long long)d);
     MNI_TRY(ensure_init());
-    const int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
-    if (s > 0x7fffff00LL || bh * qblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
+    if (s > 0x7fffff00LL || bh * qblocks > 0x3fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    // Fewer than two blocks of 128 queries per CU: blocks of 64 with the keys of a tile split over two wavefronts,
+    // so that the chain of steps each wavefront has to run is half as long (head dims with 64-key tiles).
+    // Larger grids keep the CUs busy either way and pay for reading every tile twice as often.
+    const bool split = d <= 64 && bh * qblocks < 2 * (ctx().compute_units > 0 ? ctx().compute_units : 256);
+    if (split) qblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
-#define MNI_AF(DBV, NBV) hipLaunchKernelGGL((attn_fused_fwd_kernel<DBV, NBV>), grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, attn_pair<attn_fused_fwd_kernel<DBV, NBV>>(), scale, causal)
+#define MNI_AF(DBV, NBV, SPV)                                                                                               \
+    hipLaunchKernelGGL((attn_fused_fwd_kernel<DBV, NBV, SPV>), grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, \
+                       attn_pair<attn_fused_fwd_kernel<DBV, NBV, SPV>>(), scale, causal)
     switch (d / 32) {
         // 64 keys per step while two workgroups still fit a CU's LDS, 32 beyond
-        case 1: MNI_AF(1, 2); break;
-        case 2: MNI_AF(2, 2); break;
-        case 3: MNI_AF(3, 1); break;
-        default: MNI_AF(4, 1); break;
+        case 1: if (split) MNI_AF(1, 2, true); else MNI_AF(1, 2, false); break;
+        case 2: if (split) MNI_AF(2, 2, true); else MNI_AF(2, 2, false); break;
+        case 3: MNI_AF(3, 1, false); break;
+        default: MNI_AF(4, 1, false); break;
     }
 #undef MNI_AF
     return check_launch("attn_fused_forward");

@@ -64,7 +64,9 @@ def test_softmax_negative_dim_gradient_is_the_reference_one(both):
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("bh,s,d", [(2, 4, 8), (3, 37, 20), (1, 1, 4), (4, 130, 64), (2, 1100, 16),
                                     # head dims of the one-kernel forward: key / query tails, one block, several blocks
-                                    (2, 300, 32), (1, 257, 96), (2, 129, 128), (1, 31, 64), (3, 1, 32), (1, 640, 64)])
+                                    (2, 300, 32), (1, 257, 96), (2, 129, 128), (1, 31, 64), (3, 1, 32), (1, 640, 64),
+                                    # around the edges of the two key halves of a 64-key tile (split forward)
+                                    (2, 33, 32), (1, 64, 64), (2, 97, 64), (3, 32, 32)])
 def test_attention_forward_and_backward_match_the_oracle(both, bh, s, d, causal):
     gpu, cpu = both
     q, k, v = (synth.normal(5, (bh, s, d), stream=i) for i in range(3))
@@ -133,12 +135,14 @@ def test_long_attention_backward_against_float64(rocm_native, bh, s, d, causal):
 
 
 @pytest.mark.parametrize("bh,s,d", [(75, 512, 32), (40, 1000, 64), (64, 1024, 32), (50, 1750, 32), (65, 512, 32), (9, 3800, 32),
-                                    (70, 512, 96), (33, 1024, 128)])
+                                    (70, 512, 96), (33, 1024, 128), (70, 1024, 64)])
 def test_attention_grids_beyond_one_workgroup_per_cu_against_float64(rocm_native, bh, s, d):
     """More workgroups than the 256 CUs: the kernels then hand out the causal blocks in folded order (the
     lightest blocks as second workgroups of the CUs that hold the matching heavy ones), for grids of 300, 320,
     512, 700, 260 and 270 workgroups -- a partly filled second row, a full one, and a tail past it -- and for
     head dims 96 and 128, whose backward kernels fit one workgroup per CU and take the blocks in falling order.
+    Below 512 blocks of 128 queries the forward for head dims 32 and 64 runs in its split form (64 queries per
+    workgroup, the keys of a tile shared between two wavefronts); 512, 560 and 700 blocks take the unsplit one.
     Every block must still be computed exactly once: forward and all three gradients against the closed form in
     float64."""
     rocm_native.resetEngine()
