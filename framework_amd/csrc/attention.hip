@@ -419,6 +419,15 @@ static int attn_pair() {
     return fit >= 2 ? cus : 0x7fffffff;
 }
 
+// Whether a grid of `blocks` 128-query (or 128-key) blocks runs in the split form (head dims whose forward
+// tiles hold 64 keys): fewer than two blocks per CU -- at most one for the key-owned backward at head dim 64,
+// whose split form fills the LDS of a CU with one workgroup and loses to the unsplit one beyond that.
+static bool attn_split(int64_t d, int64_t blocks, bool key_owned = false) {
+    const int64_t cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
+    if (d > 64) return false;
+    return key_owned && d > 32 ? blocks <= cus : blocks < 2 * cus;
+}
+
 bool attn_fused_supported(int64_t d) { return d == 32 || d == 64 || d == 96 || d == 128; }
 int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k, const float *v, int64_t bh, int64_t s, int64_t d,
                          float scale, int causal) {
@@ -430,7 +439,7 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
     // Fewer than two blocks of 128 queries per CU: blocks of 64 with the keys of a tile split over two wavefronts,
     // so that the chain of steps each wavefront has to run is half as long (head dims with 64-key tiles).
     // Larger grids keep the CUs busy either way and pay for reading every tile twice as often.
-    const bool split = d <= 64 && bh * qblocks < 2 * (ctx().compute_units > 0 ? ctx().compute_units : 256);
+    const bool split = attn_split(d, bh * qblocks);
     if (split) qblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
@@ -457,13 +466,16 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
 // registers; lse and di are one scalar per lane; dS^T stays in the accumulator
 // registers and is operand B of dQ^T += K^T dS^T, whose operand A is the key
 // tile once more, kept in LDS a second time as plain [key][d] rows.
-template <int DB>
-__global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_kernel(float *__restrict__ dq, const float *__restrict__ q,
+// SPLIT: as in the forward, 64 queries per workgroup and 64 keys per step, of which a wavefront takes 32;
+// the two partial dq of a query are plain sums and are added through the tile memory at the end.
+template <int DB, bool SPLIT>
+__global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void attn_fused_bwd_dq_kernel(float *__restrict__ dq, const float *__restrict__ q,
                                                                        const float *__restrict__ k, const float *__restrict__ v,
                                                                        const float *__restrict__ dout, const float *__restrict__ lse,
                                                                        const float *__restrict__ di, int s, int qblocks, int pair, float scale,
                                                                        int causal) {
-    constexpr int D = 32 * DB, DQ = D / 4, KEYS = 32;
+    constexpr int D = 32 * DB, DQ = D / 4, KEYS = SPLIT ? 64 : 32;
+    constexpr int QB = SPLIT ? 64 : AF_QUERIES;
     constexpr int TPITCH = KEYS + 1;  // float4 per d-quad slice of a [d/4][key] tile
     constexpr int RPITCH = D + 8;     // floats per row of the [key][d] copy of the key tile
     constexpr int TSTAGE = DQ * TPITCH, RSTAGE = KEYS * RPITCH;
@@ -473,11 +485,13 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
     __shared__ __align__(16) float kr[2 * RSTAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
+    const int grp = SPLIT ? (wave & 1) : wave;      // which 32 queries of the workgroup
+    const int koff = SPLIT ? 32 * (wave >> 1) : 0;  // first key of a tile this wavefront takes
     int rank;
     int64_t bh;
     attn_item(qblocks, pair, rank, bh);
     const int qb = qblocks - 1 - rank;  // late query blocks have the most keys under the mask
-    const int qi = qb * AF_QUERIES + wave * 32 + r;
+    const int qi = qb * QB + grp * 32 + r;
     const int ql = min(qi, s - 1);
     const int64_t row = bh * s + ql;
     const float *kbase = k + bh * s * (int64_t)D, *vbase = v + bh * s * (int64_t)D;
@@ -494,9 +508,9 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
     for (int b = 0; b < DB; ++b)
 #pragma unroll
         for (int e = 0; e < 16; ++e) qacc[b][e] = 0.f;
-    const int nkeys = causal ? min(s, (qb + 1) * AF_QUERIES) : s;
+    const int nkeys = causal ? min(s, (qb + 1) * QB) : s;
     const int nsteps = (nkeys + KEYS - 1) / KEYS;
-    const int wave_first = qb * AF_QUERIES + wave * 32;
+    const int wave_first = qb * QB + grp * 32;
     const int wave_last = min(wave_first + 31, s - 1);
 
     float4 kreg[NLD], vreg[NLD];
@@ -528,7 +542,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
         const int k0 = step * KEYS;
         const int cur = step & 1;
         MNI_AB_REQUEST(min(step + 1, nsteps - 1))
-        if (!causal || k0 <= wave_last) {
+        if ((!causal || k0 + koff <= wave_last) && k0 + koff < s) {
             const float4 *ks = kt + cur * TSTAGE, *vs = vt + cur * TSTAGE;
             const float *krow = kr + cur * RSTAGE;
             att_f16 sacc, pacc;
@@ -536,7 +550,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
             for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; pacc[e] = 0.f; }
 #pragma unroll
             for (int c = 0; c < D / 8; ++c) {
-                const float4 ka = ks[(2 * c + h) * TPITCH + r], va = vs[(2 * c + h) * TPITCH + r];
+                const float4 ka = ks[(2 * c + h) * TPITCH + koff + r], va = vs[(2 * c + h) * TPITCH + koff + r];
                 sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qf[c].x, sacc, 0, 0, 0);
                 pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(va.x, gf[c].x, pacc, 0, 0, 0);
                 sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qf[c].y, sacc, 0, 0, 0);
@@ -553,7 +567,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
                 const float p = __builtin_amdgcn_exp2f(sacc[e] * scale2 - lse2);
                 float ds = p * (pacc[e] - dil) * scale;
                 if (edge) {
-                    const int key = k0 + 8 * (e >> 2) + 4 * h + (e & 3);
+                    const int key = k0 + koff + 8 * (e >> 2) + 4 * h + (e & 3);
                     if (!(key < s && (!causal || key <= ql))) ds = 0.f;
                 }
                 sacc[e] = ds;
@@ -564,7 +578,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        qacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[(8 * c + 4 * h + j) * RPITCH + 32 * b + r], sacc[4 * c + j],
+                        qacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[(koff + 8 * c + 4 * h + j) * RPITCH + 32 * b + r], sacc[4 * c + j],
                                                                        qacc[b], 0, 0, 0);
         }
         MNI_AB_PARK(cur ^ 1)
@@ -572,6 +586,23 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
     }
 #undef MNI_AB_REQUEST
 #undef MNI_AB_PARK
+    if constexpr (SPLIT) {
+        // element x of lane l at [grp][x][l] of the tile memory, which the loop's last barrier has released
+        static_assert(2 * 16 * DB * 64 * sizeof(float) <= sizeof(kt), "merge buffer must fit the key tiles");
+        float *mb = reinterpret_cast<float *>(kt) + grp * 16 * DB * 64 + lane;
+        if (koff != 0) {
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) mb[(16 * b + e) * 64] = qacc[b][e];
+        }
+        __syncthreads();
+        if (koff != 0) return;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) qacc[b][e] += mb[(16 * b + e) * 64];
+    }
     if (qi < s) {
         float *orow = dq + (bh * s + qi) * (int64_t)D;
 #pragma unroll
@@ -587,16 +618,20 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
     if (bh <= 0 || s <= 0) return MNI_OK;
     if (!attn_fused_supported(d)) return set_error(MNI_ERR_INVALID, "fused attention: head dim %lld is not 32, 64, 96 or 128", (long long)d);
     MNI_TRY(ensure_init());
-    const int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
-    if (s > 0x7fffff00LL || bh * qblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
+    if (s > 0x7fffff00LL || bh * qblocks > 0x3fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    const bool split = attn_split(d, bh * qblocks);
+    if (split) qblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
-#define MNI_AB(DBV) hipLaunchKernelGGL(attn_fused_bwd_dq_kernel<DBV>, grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, attn_pair<attn_fused_bwd_dq_kernel<DBV>>(), scale, causal)
+#define MNI_AB(DBV, SPV)                                                                                                       \
+    hipLaunchKernelGGL((attn_fused_bwd_dq_kernel<DBV, SPV>), grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, \
+                       attn_pair<attn_fused_bwd_dq_kernel<DBV, SPV>>(), scale, causal)
     switch (d / 32) {
-        case 1: MNI_AB(1); break;
-        case 2: MNI_AB(2); break;
-        case 3: MNI_AB(3); break;
-        default: MNI_AB(4); break;
+        case 1: if (split) MNI_AB(1, true); else MNI_AB(1, false); break;
+        case 2: if (split) MNI_AB(2, true); else MNI_AB(2, false); break;
+        case 3: MNI_AB(3, false); break;
+        default: MNI_AB(4, false); break;
     }
 #undef MNI_AB
     return check_launch("attn_fused_backward_dq");
@@ -611,12 +646,15 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
 // accumulator registers as operand B of dV^T += dO^T P and dK^T += Q^T dS, whose
 // operands A are the dO / query tiles once more, kept as plain [query][d] rows.
 // Under the causal mask a key block starts at its own first query.
-template <int DB>
-__global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv_kernel(
+// SPLIT: 64 keys per workgroup and 64 queries per step, of which a wavefront takes 32; the two partial dk and
+// dv of a key are plain sums and are added through the tile memory at the end.
+template <int DB, bool SPLIT>
+__global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void attn_fused_bwd_dkv_kernel(
     float *__restrict__ dk, float *__restrict__ dv, const float *__restrict__ q, const float *__restrict__ k,
     const float *__restrict__ v, const float *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ di, int s,
     int kblocks, int pair, float scale, int causal) {
-    constexpr int D = 32 * DB, DQ = D / 4, QT = 32;
+    constexpr int D = 32 * DB, DQ = D / 4, QT = SPLIT ? 64 : 32;
+    constexpr int KB = SPLIT ? 64 : AF_QUERIES;  // keys per workgroup
     constexpr int TPITCH = QT + 1, RPITCH = D + 8;
     constexpr int TSTAGE = DQ * TPITCH, RSTAGE = QT * RPITCH;
     constexpr int NLD = QT * DQ / ATT_TPB;
@@ -628,10 +666,12 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
     __shared__ __align__(16) float dt[2 * QT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
+    const int grp = SPLIT ? (wave & 1) : wave;      // which 32 keys of the workgroup
+    const int qoff = SPLIT ? 32 * (wave >> 1) : 0;  // first query of a tile this wavefront takes
     int kb;  // early key blocks see the most queries under the mask
     int64_t bh;
     attn_item(kblocks, pair, kb, bh);
-    const int kj = kb * AF_QUERIES + wave * 32 + r;  // this lane's key
+    const int kj = kb * KB + grp * 32 + r;  // this lane's key
     const int kl = min(kj, s - 1);
     const int64_t base = bh * s;
     const float *qbase = q + base * (int64_t)D, *gbase = dout + base * (int64_t)D;
@@ -647,9 +687,9 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
     for (int b = 0; b < DB; ++b)
 #pragma unroll
         for (int e = 0; e < 16; ++e) { kacc[b][e] = 0.f; vacc[b][e] = 0.f; }
-    const int q_begin = causal ? kb * AF_QUERIES : 0;  // queries before the block's first key see none of its keys
+    const int q_begin = causal ? kb * KB : 0;  // queries before the block's first key see none of its keys
     const int nsteps = (s - q_begin + QT - 1) / QT;    // >= 1: the block holds at least one key < s
-    const int wave_first = kb * AF_QUERIES + wave * 32;  // first key of this wavefront
+    const int wave_first = kb * KB + grp * 32;  // first key of this wavefront
 
     float4 qreg[NLD], greg[NLD];
     float lreg, dreg;
@@ -668,8 +708,8 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
         qreg[i] = *reinterpret_cast<const float4 *>(qbase + src);                                     \
         greg[i] = *reinterpret_cast<const float4 *>(gbase + src);                                     \
     }                                                                                                 \
-    lreg = lse[base + min(q_begin + (STEP) * QT + (tid & 31), s - 1)] * 1.4426950408889634f;           \
-    dreg = di[base + min(q_begin + (STEP) * QT + (tid & 31), s - 1)];
+    lreg = lse[base + min(q_begin + (STEP) * QT + (tid & (QT - 1)), s - 1)] * 1.4426950408889634f;           \
+    dreg = di[base + min(q_begin + (STEP) * QT + (tid & (QT - 1)), s - 1)];
 #define MNI_AK_PARK(STAGE)                                                                            \
     _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
         qt[(STAGE) * TSTAGE + t_slot[i]] = qreg[i];                                                   \
@@ -686,7 +726,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
         const int cur = step & 1;
         MNI_AK_REQUEST(min(step + 1, nsteps - 1))
         // a wavefront whose keys all come after this query tile receives nothing from it (causal)
-        if (!causal || q0 + QT - 1 >= wave_first) {
+        if ((!causal || q0 + qoff + 31 >= wave_first) && q0 + qoff < s) {
             const float4 *qs = qt + cur * TSTAGE, *gs = gt + cur * TSTAGE;
             const float *qrow = qr + cur * RSTAGE, *grow = gr + cur * RSTAGE;
             att_f16 sacc, pacc;
@@ -694,7 +734,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
             for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; pacc[e] = 0.f; }
 #pragma unroll
             for (int c = 0; c < D / 8; ++c) {
-                const float4 qa = qs[(2 * c + h) * TPITCH + r], ga = gs[(2 * c + h) * TPITCH + r];
+                const float4 qa = qs[(2 * c + h) * TPITCH + qoff + r], ga = gs[(2 * c + h) * TPITCH + qoff + r];
                 sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.x, kf[c].x, sacc, 0, 0, 0);
                 pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ga.x, vf[c].x, pacc, 0, 0, 0);
                 sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa.y, kf[c].y, sacc, 0, 0, 0);
@@ -708,15 +748,15 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
             const bool edge = q0 + QT > s || kj >= s || (causal && q0 < wave_first + 32);
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
-                const float4 l4 = *reinterpret_cast<const float4 *>(lt + cur * QT + 8 * g4 + 4 * h);
-                const float4 d4 = *reinterpret_cast<const float4 *>(dt + cur * QT + 8 * g4 + 4 * h);
+                const float4 l4 = *reinterpret_cast<const float4 *>(lt + cur * QT + qoff + 8 * g4 + 4 * h);
+                const float4 d4 = *reinterpret_cast<const float4 *>(dt + cur * QT + qoff + 8 * g4 + 4 * h);
                 const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int e = 4 * g4 + j;
                     float p = __builtin_amdgcn_exp2f(sacc[e] * scale2 - ls[j]);
                     if (edge) {
-                        const int query = q0 + 8 * g4 + 4 * h + j;
+                        const int query = q0 + qoff + 8 * g4 + 4 * h + j;
                         if (!(query < s && kj < s && (!causal || kj <= query))) p = 0.f;
                     }
                     sacc[e] = p;
@@ -729,7 +769,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const int at = (8 * c + 4 * h + j) * RPITCH + 32 * b + r;
+                        const int at = (qoff + 8 * c + 4 * h + j) * RPITCH + 32 * b + r;
                         vacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(grow[at], sacc[4 * c + j], vacc[b], 0, 0, 0);
                         kacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(qrow[at], pacc[4 * c + j], kacc[b], 0, 0, 0);
                     }
@@ -739,6 +779,29 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
     }
 #undef MNI_AK_REQUEST
 #undef MNI_AK_PARK
+    if constexpr (SPLIT) {
+        // element x of lane l at [grp][x][l] of the tile memory, which the loop's last barrier has released
+        static_assert(2 * 32 * DB * 64 * sizeof(float) <= sizeof(qt), "merge buffer must fit the query tiles");
+        float *mb = reinterpret_cast<float *>(qt) + grp * 32 * DB * 64 + lane;
+        if (qoff != 0) {
+#pragma unroll
+            for (int b = 0; b < DB; ++b)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    mb[(32 * b + e) * 64] = kacc[b][e];
+                    mb[(32 * b + 16 + e) * 64] = vacc[b][e];
+                }
+        }
+        __syncthreads();
+        if (qoff != 0) return;
+#pragma unroll
+        for (int b = 0; b < DB; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                kacc[b][e] += mb[(32 * b + e) * 64];
+                vacc[b][e] += mb[(32 * b + 16 + e) * 64];
+            }
+    }
     if (kj < s) {
         float *krow = dk + (base + kj) * (int64_t)D, *vrow = dv + (base + kj) * (int64_t)D;
 #pragma unroll
@@ -757,16 +820,20 @@ int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float 
     if (bh <= 0 || s <= 0) return MNI_OK;
     if (!attn_fused_supported(d)) return set_error(MNI_ERR_INVALID, "fused attention: head dim %lld is not 32, 64, 96 or 128", (long long)d);
     MNI_TRY(ensure_init());
-    const int64_t kblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
-    if (s > 0x7fffff00LL || bh * kblocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    int64_t kblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
+    if (s > 0x7fffff00LL || bh * kblocks > 0x3fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
+    const bool split = attn_split(d, bh * kblocks, true);
+    if (split) kblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * kblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
-#define MNI_AK(DBV) hipLaunchKernelGGL(attn_fused_bwd_dkv_kernel<DBV>, grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, attn_pair<attn_fused_bwd_dkv_kernel<DBV>>(), scale, causal)
+#define MNI_AK(DBV, SPV)                                                                                                            \
+    hipLaunchKernelGGL((attn_fused_bwd_dkv_kernel<DBV, SPV>), grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, \
+                       attn_pair<attn_fused_bwd_dkv_kernel<DBV, SPV>>(), scale, causal)
     switch (d / 32) {
-        case 1: MNI_AK(1); break;
-        case 2: MNI_AK(2); break;
-        case 3: MNI_AK(3); break;
-        default: MNI_AK(4); break;
+        case 1: if (split) MNI_AK(1, true); else MNI_AK(1, false); break;
+        case 2: if (split) MNI_AK(2, true); else MNI_AK(2, false); break;
+        case 3: MNI_AK(3, false); break;
+        default: MNI_AK(4, false); break;
     }
 #undef MNI_AK
     return check_launch("attn_fused_backward_dkv");
