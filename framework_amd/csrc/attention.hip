@@ -203,9 +203,10 @@ static constexpr int AF_QUERIES = 128;
 // SPLIT (with 64 keys per step): the workgroup owns 64 queries instead of 128 and its wavefronts pair up on
 // them, one taking keys 0 .. 31 and the other keys 32 .. 63 of every tile; the two partial results (running
 // maximum, sum and output) meet in LDS at the end.  Half the MFMAs per wavefront and step: for grids too
-// small to fill the chip, where the time is that of the longest chain of steps.
+// small to fill the chip, where the time is that of the longest chain of steps (every head dim; 96 and 128
+// then take 64-key tiles too, one workgroup per CU).
 template <int DB, int NB, bool SPLIT>  // head dim = 32 * DB, keys per step = 32 * NB
-__global__ __launch_bounds__(ATT_TPB, 2) void attn_fused_fwd_kernel(float *__restrict__ out, float *__restrict__ lse,
+__global__ __launch_bounds__(ATT_TPB, (SPLIT && DB > 2 ? 1 : 2)) void attn_fused_fwd_kernel(float *__restrict__ out, float *__restrict__ lse,
                                                                     const float *__restrict__ q, const float *__restrict__ k,
                                                                     const float *__restrict__ v, int s, int qblocks, int pair,
                                                                     float scale, int causal) {
@@ -419,13 +420,16 @@ static int attn_pair() {
     return fit >= 2 ? cus : 0x7fffffff;
 }
 
-// Whether a grid of `blocks` 128-query (or 128-key) blocks runs in the split form (head dims whose forward
-// tiles hold 64 keys): fewer than two blocks per CU -- at most one for the key-owned backward at head dim 64,
-// whose split form fills the LDS of a CU with one workgroup and loses to the unsplit one beyond that.
-static bool attn_split(int64_t d, int64_t blocks, bool key_owned = false) {
+// Whether a grid of `blocks` 128-query (or 128-key) blocks runs in the split form.  Up to one block per CU
+// always where the form exists (the forward at every head dim, the backward kernels at 32 and 64); up to two
+// where two split workgroups still fit a CU, which leaves out the forward at 96 / 128 and the key-owned
+// backward at 64 (their split forms fill the LDS with one workgroup and lose to the unsplit ones beyond that).
+enum { ATT_FWD, ATT_DQ, ATT_DKV };
+static bool attn_split(int kernel, int64_t d, int64_t blocks) {
     const int64_t cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
-    if (d > 64) return false;
-    return key_owned && d > 32 ? blocks <= cus : blocks < 2 * cus;
+    if (d > 64 && kernel != ATT_FWD) return false;
+    const bool one_per_cu = d > 64 || (kernel == ATT_DKV && d > 32);
+    return one_per_cu ? blocks <= cus : blocks < 2 * cus;
 }
 
 bool attn_fused_supported(int64_t d) { return d == 32 || d == 64 || d == 96 || d == 128; }
@@ -436,10 +440,10 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
     MNI_TRY(ensure_init());
     int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
     if (s > 0x7fffff00LL || bh * qblocks > 0x3fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
-    // Fewer than two blocks of 128 queries per CU: blocks of 64 with the keys of a tile split over two wavefronts,
-    // so that the chain of steps each wavefront has to run is half as long (head dims with 64-key tiles).
-    // Larger grids keep the CUs busy either way and pay for reading every tile twice as often.
-    const bool split = attn_split(d, bh * qblocks);
+    // Few blocks of 128 queries per CU: blocks of 64 with the keys of a 64-key tile split over two wavefronts,
+    // so that the chain of steps each wavefront has to run is half as long.  Larger grids keep the CUs busy
+    // either way and pay for reading every tile twice as often.
+    const bool split = attn_split(ATT_FWD, d, bh * qblocks);
     if (split) qblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
@@ -450,8 +454,8 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
         // 64 keys per step while two workgroups still fit a CU's LDS, 32 beyond
         case 1: if (split) MNI_AF(1, 2, true); else MNI_AF(1, 2, false); break;
         case 2: if (split) MNI_AF(2, 2, true); else MNI_AF(2, 2, false); break;
-        case 3: MNI_AF(3, 1, false); break;
-        default: MNI_AF(4, 1, false); break;
+        case 3: if (split) MNI_AF(3, 2, true); else MNI_AF(3, 1, false); break;
+        default: if (split) MNI_AF(4, 2, true); else MNI_AF(4, 1, false); break;
     }
 #undef MNI_AF
     return check_launch("attn_fused_forward");
@@ -620,7 +624,7 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
     MNI_TRY(ensure_init());
     int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
     if (s > 0x7fffff00LL || bh * qblocks > 0x3fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
-    const bool split = attn_split(d, bh * qblocks);
+    const bool split = attn_split(ATT_DQ, d, bh * qblocks);
     if (split) qblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
@@ -822,7 +826,7 @@ int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float 
     MNI_TRY(ensure_init());
     int64_t kblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
     if (s > 0x7fffff00LL || bh * kblocks > 0x3fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
-    const bool split = attn_split(d, bh * kblocks, true);
+    const bool split = attn_split(ATT_DKV, d, bh * kblocks);
     if (split) kblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * kblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
