@@ -481,12 +481,10 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
     constexpr int D = 32 * DB, DQ = D / 4, KEYS = SPLIT ? 64 : 32;
     constexpr int QB = SPLIT ? 64 : AF_QUERIES;
     constexpr int TPITCH = KEYS + 1;  // float4 per d-quad slice of a [d/4][key] tile
-    constexpr int RPITCH = D + 8;     // floats per row of the [key][d] copy of the key tile
-    constexpr int TSTAGE = DQ * TPITCH, RSTAGE = KEYS * RPITCH;
+    constexpr int TSTAGE = DQ * TPITCH;
     constexpr int NLD = KEYS * DQ / ATT_TPB;  // float4 of each tile per thread (1 .. 4)
     __shared__ float4 kt[2 * TSTAGE];
     __shared__ float4 vt[2 * TSTAGE];
-    __shared__ __align__(16) float kr[2 * RSTAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int grp = SPLIT ? (wave & 1) : wave;      // which 32 queries of the workgroup
@@ -518,14 +516,13 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
     const int wave_last = min(wave_first + 31, s - 1);
 
     float4 kreg[NLD], vreg[NLD];
-    int src_off[NLD], t_slot[NLD], r_slot[NLD], key_of[NLD];
+    int src_off[NLD], t_slot[NLD], key_of[NLD];
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
         const int f = tid + ATT_TPB * i;
         key_of[i] = f / DQ;
         src_off[i] = 4 * (f % DQ);
         t_slot[i] = (f % DQ) * TPITCH + f / DQ;
-        r_slot[i] = (f / DQ) * RPITCH + 4 * (f % DQ);
     }
 #define MNI_AB_REQUEST(STEP)                                                                          \
     _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
@@ -537,7 +534,6 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
     _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
         kt[(STAGE) * TSTAGE + t_slot[i]] = kreg[i];                                                   \
         vt[(STAGE) * TSTAGE + t_slot[i]] = vreg[i];                                                   \
-        *reinterpret_cast<float4 *>(kr + (STAGE) * RSTAGE + r_slot[i]) = kreg[i];                     \
     }
     MNI_AB_REQUEST(0)
     MNI_AB_PARK(0)
@@ -548,7 +544,9 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
         MNI_AB_REQUEST(min(step + 1, nsteps - 1))
         if ((!causal || k0 + koff <= wave_last) && k0 + koff < s) {
             const float4 *ks = kt + cur * TSTAGE, *vs = vt + cur * TSTAGE;
-            const float *krow = kr + cur * RSTAGE;
+            // the key tile read along d for dQ^T += K^T dS^T: element (key, d) is component d % 4 of quad [d / 4][key];
+            // 4 lanes share a quad and the next 4 are a whole slice further, which keeps them on different banks
+            const float *krow = reinterpret_cast<const float *>(ks) + ((r >> 2) * TPITCH + koff + 4 * h) * 4 + (r & 3);
             att_f16 sacc, pacc;
 #pragma unroll
             for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; pacc[e] = 0.f; }
@@ -582,7 +580,7 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        qacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[(koff + 8 * c + 4 * h + j) * RPITCH + 32 * b + r], sacc[4 * c + j],
+                        qacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[(8 * b * TPITCH + 8 * c + j) * 4], sacc[4 * c + j],
                                                                        qacc[b], 0, 0, 0);
         }
         MNI_AB_PARK(cur ^ 1)
@@ -659,13 +657,11 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
     int kblocks, int pair, float scale, int causal) {
     constexpr int D = 32 * DB, DQ = D / 4, QT = SPLIT ? 64 : 32;
     constexpr int KB = SPLIT ? 64 : AF_QUERIES;  // keys per workgroup
-    constexpr int TPITCH = QT + 1, RPITCH = D + 8;
-    constexpr int TSTAGE = DQ * TPITCH, RSTAGE = QT * RPITCH;
+    constexpr int TPITCH = QT + 1;
+    constexpr int TSTAGE = DQ * TPITCH;
     constexpr int NLD = QT * DQ / ATT_TPB;
     __shared__ float4 qt[2 * TSTAGE];
     __shared__ float4 gt[2 * TSTAGE];
-    __shared__ __align__(16) float qr[2 * RSTAGE];
-    __shared__ __align__(16) float gr[2 * RSTAGE];
     __shared__ __align__(16) float lt[2 * QT];
     __shared__ __align__(16) float dt[2 * QT];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -697,14 +693,13 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
 
     float4 qreg[NLD], greg[NLD];
     float lreg, dreg;
-    int src_off[NLD], t_slot[NLD], r_slot[NLD], row_of[NLD];
+    int src_off[NLD], t_slot[NLD], row_of[NLD];
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
         const int f = tid + ATT_TPB * i;
         row_of[i] = f / DQ;
         src_off[i] = 4 * (f % DQ);
         t_slot[i] = (f % DQ) * TPITCH + f / DQ;
-        r_slot[i] = (f / DQ) * RPITCH + 4 * (f % DQ);
     }
 #define MNI_AK_REQUEST(STEP)                                                                          \
     _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
@@ -718,8 +713,6 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
     _Pragma("unroll") for (int i = 0; i < NLD; ++i) {                                                 \
         qt[(STAGE) * TSTAGE + t_slot[i]] = qreg[i];                                                   \
         gt[(STAGE) * TSTAGE + t_slot[i]] = greg[i];                                                   \
-        *reinterpret_cast<float4 *>(qr + (STAGE) * RSTAGE + r_slot[i]) = qreg[i];                     \
-        *reinterpret_cast<float4 *>(gr + (STAGE) * RSTAGE + r_slot[i]) = greg[i];                     \
     }                                                                                                 \
     if (tid < QT) { lt[(STAGE) * QT + tid] = lreg; dt[(STAGE) * QT + tid] = dreg; }
     MNI_AK_REQUEST(0)
@@ -732,7 +725,11 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
         // a wavefront whose keys all come after this query tile receives nothing from it (causal)
         if ((!causal || q0 + qoff + 31 >= wave_first) && q0 + qoff < s) {
             const float4 *qs = qt + cur * TSTAGE, *gs = gt + cur * TSTAGE;
-            const float *qrow = qr + cur * RSTAGE, *grow = gr + cur * RSTAGE;
+            // the same tiles read along d for dV^T += dO^T P and dK^T += Q^T dS: element (query, d) is component d % 4 of
+            // quad [d / 4][query]; 4 lanes share a quad and the next 4 are a whole slice further, which keeps them on
+            // different banks
+            const float *qrow = reinterpret_cast<const float *>(qs) + ((r >> 2) * TPITCH + qoff + 4 * h) * 4 + (r & 3);
+            const float *grow = reinterpret_cast<const float *>(gs) + ((r >> 2) * TPITCH + qoff + 4 * h) * 4 + (r & 3);
             att_f16 sacc, pacc;
 #pragma unroll
             for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; pacc[e] = 0.f; }
@@ -773,7 +770,7 @@ __global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const int at = (qoff + 8 * c + 4 * h + j) * RPITCH + 32 * b + r;
+                        const int at = (8 * b * TPITCH + 8 * c + j) * 4;
                         vacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(grow[at], sacc[4 * c + j], vacc[b], 0, 0, 0);
                         kacc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(qrow[at], pacc[4 * c + j], kacc[b], 0, 0, 0);
                     }
