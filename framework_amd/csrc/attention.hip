@@ -420,16 +420,11 @@ static int attn_pair() {
     return fit >= 2 ? cus : 0x7fffffff;
 }
 
-// Whether a grid of `blocks` 128-query (or 128-key) blocks runs in the split form.  Up to one block per CU
-// always where the form exists (the forward at every head dim, the backward kernels at 32 and 64); up to two
-// where two split workgroups still fit a CU, which leaves out the forward at 96 / 128 and the key-owned
-// backward at 64 (their split forms fill the LDS with one workgroup and lose to the unsplit ones beyond that).
-enum { ATT_FWD, ATT_DQ, ATT_DKV };
-static bool attn_split(int kernel, int64_t d, int64_t blocks) {
+// Whether a grid of `blocks` 128-query (or 128-key) blocks runs in the split form: fewer than two blocks per CU
+// at head dims 32 and 64, where two split workgroups fit a CU; at most one at 96 and 128, where one does.
+static bool attn_split(int64_t d, int64_t blocks) {
     const int64_t cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
-    if (d > 64 && kernel != ATT_FWD) return false;
-    const bool one_per_cu = d > 64 || (kernel == ATT_DKV && d > 32);
-    return one_per_cu ? blocks <= cus : blocks < 2 * cus;
+    return d > 64 ? blocks <= cus : blocks < 2 * cus;
 }
 
 bool attn_fused_supported(int64_t d) { return d == 32 || d == 64 || d == 96 || d == 128; }
@@ -443,7 +438,7 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
     // Few blocks of 128 queries per CU: blocks of 64 with the keys of a 64-key tile split over two wavefronts,
     // so that the chain of steps each wavefront has to run is half as long.  Larger grids keep the CUs busy
     // either way and pay for reading every tile twice as often.
-    const bool split = attn_split(ATT_FWD, d, bh * qblocks);
+    const bool split = attn_split(d, bh * qblocks);
     if (split) qblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
@@ -469,11 +464,11 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
 // tiles from LDS ([d/4][key] float4) and the lane's own q / dO rows from
 // registers; lse and di are one scalar per lane; dS^T stays in the accumulator
 // registers and is operand B of dQ^T += K^T dS^T, whose operand A is the key
-// tile once more, kept in LDS a second time as plain [key][d] rows.
+// tile once more, read along d out of the same [d/4][key] quads.
 // SPLIT: as in the forward, 64 queries per workgroup and 64 keys per step, of which a wavefront takes 32;
 // the two partial dq of a query are plain sums and are added through the tile memory at the end.
 template <int DB, bool SPLIT>
-__global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void attn_fused_bwd_dq_kernel(float *__restrict__ dq, const float *__restrict__ q,
+__global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_kernel(float *__restrict__ dq, const float *__restrict__ q,
                                                                        const float *__restrict__ k, const float *__restrict__ v,
                                                                        const float *__restrict__ dout, const float *__restrict__ lse,
                                                                        const float *__restrict__ di, int s, int qblocks, int pair, float scale,
@@ -622,7 +617,7 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
     MNI_TRY(ensure_init());
     int64_t qblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
     if (s > 0x7fffff00LL || bh * qblocks > 0x3fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
-    const bool split = attn_split(ATT_DQ, d, bh * qblocks);
+    const bool split = attn_split(d, bh * qblocks);
     if (split) qblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
@@ -632,8 +627,8 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
     switch (d / 32) {
         case 1: if (split) MNI_AB(1, true); else MNI_AB(1, false); break;
         case 2: if (split) MNI_AB(2, true); else MNI_AB(2, false); break;
-        case 3: MNI_AB(3, false); break;
-        default: MNI_AB(4, false); break;
+        case 3: if (split) MNI_AB(3, true); else MNI_AB(3, false); break;
+        default: if (split) MNI_AB(4, true); else MNI_AB(4, false); break;
     }
 #undef MNI_AB
     return check_launch("attn_fused_backward_dq");
@@ -646,12 +641,12 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
 // ([d/4][query] float4); lane (key r, half h) receives queries 8(e/4) + 4h + e%4,
 // whose lse and di come from LDS four at a time.  P and dS stay in the
 // accumulator registers as operand B of dV^T += dO^T P and dK^T += Q^T dS, whose
-// operands A are the dO / query tiles once more, kept as plain [query][d] rows.
+// operands A are the dO / query tiles once more, read along d out of the same quads.
 // Under the causal mask a key block starts at its own first query.
 // SPLIT: 64 keys per workgroup and 64 queries per step, of which a wavefront takes 32; the two partial dk and
 // dv of a key are plain sums and are added through the tile memory at the end.
 template <int DB, bool SPLIT>
-__global__ __launch_bounds__(ATT_TPB, ((SPLIT ? 2 * DB : DB) <= 2 ? 2 : 1)) void attn_fused_bwd_dkv_kernel(
+__global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv_kernel(
     float *__restrict__ dk, float *__restrict__ dv, const float *__restrict__ q, const float *__restrict__ k,
     const float *__restrict__ v, const float *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ di, int s,
     int kblocks, int pair, float scale, int causal) {
@@ -823,7 +818,7 @@ int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float 
     MNI_TRY(ensure_init());
     int64_t kblocks = (s + AF_QUERIES - 1) / AF_QUERIES;
     if (s > 0x7fffff00LL || bh * kblocks > 0x3fffffffLL) return set_error(MNI_ERR_INVALID, "fused attention: extent out of range");
-    const bool split = attn_split(ATT_DKV, d, bh * kblocks);
+    const bool split = attn_split(d, bh * kblocks);
     if (split) kblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * kblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
@@ -833,8 +828,8 @@ int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float 
     switch (d / 32) {
         case 1: if (split) MNI_AK(1, true); else MNI_AK(1, false); break;
         case 2: if (split) MNI_AK(2, true); else MNI_AK(2, false); break;
-        case 3: MNI_AK(3, false); break;
-        default: MNI_AK(4, false); break;
+        case 3: if (split) MNI_AK(3, true); else MNI_AK(3, false); break;
+        default: if (split) MNI_AK(4, true); else MNI_AK(4, false); break;
     }
 #undef MNI_AK
     return check_launch("attn_fused_backward_dkv");
