@@ -135,14 +135,17 @@ def test_long_attention_backward_against_float64(rocm_native, bh, s, d, causal):
 
 
 @pytest.mark.parametrize("bh,s,d", [(75, 512, 32), (40, 1000, 64), (64, 1024, 32), (50, 1750, 32), (65, 512, 32), (9, 3800, 32),
-                                    (70, 512, 96), (33, 1024, 128), (70, 1024, 64)])
+                                    (70, 512, 96), (33, 1024, 128), (70, 1024, 64),
+                                    # the last grids that still take the split forms: 511 blocks at 64, 256 at 128
+                                    (73, 896, 64), (32, 1024, 128)])
 def test_attention_grids_beyond_one_workgroup_per_cu_against_float64(rocm_native, bh, s, d):
     """More workgroups than the 256 CUs: the kernels then hand out the causal blocks in folded order (the
     lightest blocks as second workgroups of the CUs that hold the matching heavy ones), for grids of 300, 320,
     512, 700, 260 and 270 workgroups -- a partly filled second row, a full one, and a tail past it -- and for
     head dims 96 and 128, whose backward kernels fit one workgroup per CU and take the blocks in falling order.
-    Below 512 blocks of 128 queries the forward for head dims 32 and 64 runs in its split form (64 queries per
-    workgroup, the keys of a tile shared between two wavefronts); 512, 560 and 700 blocks take the unsplit one.
+    Below 512 blocks of 128 queries at head dims 32 and 64, and up to 256 at 96 and 128, all three kernels run
+    in their split forms (64 queries or keys per workgroup, a tile shared between two wavefronts); the grids
+    beyond take the unsplit ones.
     Every block must still be computed exactly once: forward and all three gradients against the closed form in
     float64."""
     rocm_native.resetEngine()
