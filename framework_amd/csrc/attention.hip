@@ -467,13 +467,15 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
 // tile once more, read along d out of the same [d/4][key] quads.
 // SPLIT: as in the forward, 64 queries per workgroup and 64 keys per step, of which a wavefront takes 32;
 // the two partial dq of a query are plain sums and are added through the tile memory at the end.
-template <int DB, bool SPLIT>
+// WIDE: 128 queries per workgroup as in the plain form, but 64 keys per step, both halves taken by every
+// wavefront in turn: half as many tile hand-overs and barriers per key.
+template <int DB, bool SPLIT, bool WIDE>
 __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_kernel(float *__restrict__ dq, const float *__restrict__ q,
                                                                        const float *__restrict__ k, const float *__restrict__ v,
                                                                        const float *__restrict__ dout, const float *__restrict__ lse,
                                                                        const float *__restrict__ di, int s, int qblocks, int pair, float scale,
                                                                        int causal) {
-    constexpr int D = 32 * DB, DQ = D / 4, KEYS = SPLIT ? 64 : 32;
+    constexpr int D = 32 * DB, DQ = D / 4, KEYS = SPLIT || WIDE ? 64 : 32;
     constexpr int QB = SPLIT ? 64 : AF_QUERIES;
     constexpr int TPITCH = KEYS + 1;  // float4 per d-quad slice of a [d/4][key] tile
     constexpr int TSTAGE = DQ * TPITCH;
@@ -483,7 +485,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int grp = SPLIT ? (wave & 1) : wave;      // which 32 queries of the workgroup
-    const int koff = SPLIT ? 32 * (wave >> 1) : 0;  // first key of a tile this wavefront takes
+    const int koff0 = SPLIT ? 32 * (wave >> 1) : 0;  // first key of a tile this wavefront takes
     int rank;
     int64_t bh;
     attn_item(qblocks, pair, rank, bh);
@@ -537,6 +539,8 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
         const int k0 = step * KEYS;
         const int cur = step & 1;
         MNI_AB_REQUEST(min(step + 1, nsteps - 1))
+#pragma unroll 1
+        for (int koff = koff0; koff < (WIDE ? 64 : koff0 + 32); koff += 32)
         if ((!causal || k0 + koff <= wave_last) && k0 + koff < s) {
             const float4 *ks = kt + cur * TSTAGE, *vs = vt + cur * TSTAGE;
             // the key tile read along d for dQ^T += K^T dS^T: element (key, d) is component d % 4 of quad [d / 4][key];
@@ -558,7 +562,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
                 pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(va.w, gf[c].w, pacc, 0, 0, 0);
             }
             // dS^T = P^T (dP^T - di) scale, 0 where the mask (or the end of the keys) forbids
-            const bool edge = k0 + KEYS > s || (causal && k0 + KEYS - 1 > wave_first);
+            const bool edge = k0 + koff + 32 > s || (causal && k0 + koff + 31 > wave_first);
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const float p = __builtin_amdgcn_exp2f(sacc[e] * scale2 - lse2);
@@ -587,14 +591,14 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dq_
         // element x of lane l at [grp][x][l] of the tile memory, which the loop's last barrier has released
         static_assert(2 * 16 * DB * 64 * sizeof(float) <= sizeof(kt), "merge buffer must fit the key tiles");
         float *mb = reinterpret_cast<float *>(kt) + grp * 16 * DB * 64 + lane;
-        if (koff != 0) {
+        if (koff0 != 0) {
 #pragma unroll
             for (int b = 0; b < DB; ++b)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) mb[(16 * b + e) * 64] = qacc[b][e];
         }
         __syncthreads();
-        if (koff != 0) return;
+        if (koff0 != 0) return;
 #pragma unroll
         for (int b = 0; b < DB; ++b)
 #pragma unroll
@@ -621,9 +625,9 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
     if (split) qblocks = (s + 63) / 64;
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
-#define MNI_AB(DBV, SPV)                                                                                                       \
-    hipLaunchKernelGGL((attn_fused_bwd_dq_kernel<DBV, SPV>), grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, \
-                       attn_pair<attn_fused_bwd_dq_kernel<DBV, SPV>>(), scale, causal)
+#define MNI_AB(DBV, SPV)                                                                                                               \
+    hipLaunchKernelGGL((attn_fused_bwd_dq_kernel<DBV, SPV, !SPV>), grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, \
+                       attn_pair<attn_fused_bwd_dq_kernel<DBV, SPV, !SPV>>(), scale, causal)
     switch (d / 32) {
         case 1: if (split) MNI_AB(1, true); else MNI_AB(1, false); break;
         case 2: if (split) MNI_AB(2, true); else MNI_AB(2, false); break;
@@ -645,12 +649,14 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
 // Under the causal mask a key block starts at its own first query.
 // SPLIT: 64 keys per workgroup and 64 queries per step, of which a wavefront takes 32; the two partial dk and
 // dv of a key are plain sums and are added through the tile memory at the end.
-template <int DB, bool SPLIT>
+// WIDE: 128 keys per workgroup as in the plain form, but 64 queries per step, both halves taken by every
+// wavefront in turn.
+template <int DB, bool SPLIT, bool WIDE>
 __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv_kernel(
     float *__restrict__ dk, float *__restrict__ dv, const float *__restrict__ q, const float *__restrict__ k,
     const float *__restrict__ v, const float *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ di, int s,
     int kblocks, int pair, float scale, int causal) {
-    constexpr int D = 32 * DB, DQ = D / 4, QT = SPLIT ? 64 : 32;
+    constexpr int D = 32 * DB, DQ = D / 4, QT = SPLIT || WIDE ? 64 : 32;
     constexpr int KB = SPLIT ? 64 : AF_QUERIES;  // keys per workgroup
     constexpr int TPITCH = QT + 1;
     constexpr int TSTAGE = DQ * TPITCH;
@@ -662,7 +668,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int grp = SPLIT ? (wave & 1) : wave;      // which 32 keys of the workgroup
-    const int qoff = SPLIT ? 32 * (wave >> 1) : 0;  // first query of a tile this wavefront takes
+    const int qoff0 = SPLIT ? 32 * (wave >> 1) : 0;  // first query of a tile this wavefront takes
     int kb;  // early key blocks see the most queries under the mask
     int64_t bh;
     attn_item(kblocks, pair, kb, bh);
@@ -718,6 +724,8 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
         const int cur = step & 1;
         MNI_AK_REQUEST(min(step + 1, nsteps - 1))
         // a wavefront whose keys all come after this query tile receives nothing from it (causal)
+#pragma unroll 1
+        for (int qoff = qoff0; qoff < (WIDE ? 64 : qoff0 + 32); qoff += 32)
         if ((!causal || q0 + qoff + 31 >= wave_first) && q0 + qoff < s) {
             const float4 *qs = qt + cur * TSTAGE, *gs = gt + cur * TSTAGE;
             // the same tiles read along d for dV^T += dO^T P and dK^T += Q^T dS: element (query, d) is component d % 4 of
@@ -741,7 +749,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
                 pacc = __builtin_amdgcn_mfma_f32_32x32x2f32(ga.w, vf[c].w, pacc, 0, 0, 0);
             }
             // P and dS for the queries 8 g + 4 h + 0..3 of accumulator elements 4 g .. 4 g + 3
-            const bool edge = q0 + QT > s || kj >= s || (causal && q0 < wave_first + 32);
+            const bool edge = q0 + qoff + 32 > s || kj >= s || (causal && q0 + qoff < wave_first + 32);
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const float4 l4 = *reinterpret_cast<const float4 *>(lt + cur * QT + qoff + 8 * g4 + 4 * h);
@@ -779,7 +787,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
         // element x of lane l at [grp][x][l] of the tile memory, which the loop's last barrier has released
         static_assert(2 * 32 * DB * 64 * sizeof(float) <= sizeof(qt), "merge buffer must fit the query tiles");
         float *mb = reinterpret_cast<float *>(qt) + grp * 32 * DB * 64 + lane;
-        if (qoff != 0) {
+        if (qoff0 != 0) {
 #pragma unroll
             for (int b = 0; b < DB; ++b)
 #pragma unroll
@@ -789,7 +797,7 @@ __global__ __launch_bounds__(ATT_TPB, (DB <= 2 ? 2 : 1)) void attn_fused_bwd_dkv
                 }
         }
         __syncthreads();
-        if (qoff != 0) return;
+        if (qoff0 != 0) return;
 #pragma unroll
         for (int b = 0; b < DB; ++b)
 #pragma unroll
@@ -823,8 +831,8 @@ int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float 
     const dim3 grid((unsigned)(bh * kblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
 #define MNI_AK(DBV, SPV)                                                                                                            \
-    hipLaunchKernelGGL((attn_fused_bwd_dkv_kernel<DBV, SPV>), grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, \
-                       attn_pair<attn_fused_bwd_dkv_kernel<DBV, SPV>>(), scale, causal)
+    hipLaunchKernelGGL((attn_fused_bwd_dkv_kernel<DBV, SPV, !SPV>), grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, \
+                       attn_pair<attn_fused_bwd_dkv_kernel<DBV, SPV, !SPV>>(), scale, causal)
     switch (d / 32) {
         case 1: if (split) MNI_AK(1, true); else MNI_AK(1, false); break;
         case 2: if (split) MNI_AK(2, true); else MNI_AK(2, false); break;
