@@ -440,7 +440,7 @@ int k_mul_backward_same(float *ga, float *gb, const float *g, const float *a, co
 // src/native/src/utils.rs:39-66) and the batch reduction of a broadcast matmul
 // operand.  Two deterministic passes: row blocks into partials, then partials
 // in block order.
-static constexpr int CS_ROWS = 128;  // rows per block in pass 1
+static constexpr int CS_ROWS = 32;  // rows per block in pass 1 (a [4096, 768] gradient then gives 384 workgroups, not 96)
 __global__ void colsum_partial_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t rows,
                                       int64_t cols) {
     const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -449,6 +449,13 @@ __global__ void colsum_partial_kernel(float *__restrict__ part, const float *__r
     const int64_t r1 = min(rows, r0 + CS_ROWS);
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     int64_t r = r0;
+    for (; r + 7 < r1; r += 8) {  // 8 loads in flight, four running sums
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = a[(r + e) * cols + c];
+        s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
+        s0 += v[4]; s1 += v[5]; s2 += v[6]; s3 += v[7];
+    }
     for (; r + 3 < r1; r += 4) {
         s0 += a[r * cols + c];
         s1 += a[(r + 1) * cols + c];
