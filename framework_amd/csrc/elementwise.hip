@@ -1004,10 +1004,34 @@ __global__ void ce_bwd_kernel(float *__restrict__ dl, const float *__restrict__ 
         dl[idx] = p * scale;
     }
 }
+// The same on 16-byte pieces, rows on the second grid axis: no division per element.
+__global__ void ce_bwd4_kernel(float4 *__restrict__ dl, const float4 *__restrict__ sm, const int32_t *__restrict__ targets,
+                               const float *__restrict__ grad, int64_t n, int64_t v4) {
+    const float scale = grad[0] / (float)n;
+    for (int64_t row = blockIdx.y; row < n; row += gridDim.y) {
+        const int64_t t = targets[row];
+        for (int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; j < v4; j += (int64_t)gridDim.x * blockDim.x) {
+            float4 p = sm[row * v4 + j];
+            const int64_t at = t - 4 * j;  // 0 .. 3 when the target's column is in this piece
+            if (at == 0) p.x -= 1.0f;
+            if (at == 1) p.y -= 1.0f;
+            if (at == 2) p.z -= 1.0f;
+            if (at == 3) p.w -= 1.0f;
+            dl[row * v4 + j] = make_float4(p.x * scale, p.y * scale, p.z * scale, p.w * scale);
+        }
+    }
+}
 int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t *targets, const float *grad_scalar,
                              int64_t n, int64_t v) {
     MNI_TRY(ensure_init());
     if (n * v <= 0) return MNI_OK;
+    if (v % 4 == 0 && al16(dlogits) && al16(softmax)) {
+        const int64_t v4 = v / 4;
+        const unsigned gx = (unsigned)min((int64_t)64, (v4 + TPB - 1) / TPB), gy = (unsigned)min(n, (int64_t)65535);
+        hipLaunchKernelGGL(ce_bwd4_kernel, dim3(gx, gy), dim3(TPB), 0, ctx().stream, (float4 *)dlogits, (const float4 *)softmax, targets,
+                           grad_scalar, n, v4);
+        return check_launch("ce_backward");
+    }
     hipLaunchKernelGGL(ce_bwd_kernel, dim3(grid_for(n * v, TPB * 2)), dim3(TPB), 0, ctx().stream, dlogits, softmax, targets, grad_scalar, n, v);
     return check_launch("ce_backward");
 }
