@@ -959,6 +959,57 @@ __global__ void ce_rows_cached_kernel(float *__restrict__ row_loss, float *__res
         row_loss[row] = -logf(e / sum);
     }
 }
+// Long rows: one workgroup per row, NV 16-byte pieces per thread, maximum and sum through LDS (the four
+// wavefront sums are added in wavefront order).  A wavefront per row would hold 128 registers of logits at
+// 8192 classes, and a few thousand such wavefronts do not fit the chip in one round.
+template <int NV>
+__global__ __launch_bounds__(256) void ce_rows_wg_kernel(float *__restrict__ row_loss, float *__restrict__ sm,
+                                                         const float *__restrict__ logits, const int32_t *__restrict__ targets,
+                                                         int64_t n, int64_t v) {
+    __shared__ float red[2][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t row = blockIdx.x;
+    const int64_t v4 = v >> 2;
+    const float4 *x = reinterpret_cast<const float4 *>(logits + row * v);
+    float4 *p = reinterpret_cast<float4 *>(sm + row * v);
+    float4 r[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t j = tid + 256 * i;
+        r[i] = j < v4 ? x[j] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) mx = fmaxf(fmaxf(mx, fmaxf(r[i].x, r[i].y)), fmaxf(r[i].z, r[i].w));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    if (lane == 0) red[0][wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        if (tid + 256 * i < v4) {
+            r[i].x = expf(r[i].x - mx); r[i].y = expf(r[i].y - mx); r[i].z = expf(r[i].z - mx); r[i].w = expf(r[i].w - mx);
+            sum += r[i].x; sum += r[i].y; sum += r[i].z; sum += r[i].w;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane == 0) red[1][wave] = sum;
+    __syncthreads();
+    sum = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t j = tid + 256 * i;
+        if (j < v4) p[j] = make_float4(r[i].x / sum, r[i].y / sum, r[i].z / sum, r[i].w / sum);
+    }
+    if (tid == 0) {
+        const int32_t t = targets[row];
+        const float e = expf(logits[row * v + t] - mx);
+        row_loss[row] = -logf(e / sum);
+    }
+}
 __global__ void ce_mean_kernel(float *__restrict__ loss, const float *__restrict__ row_loss, int64_t n) {
     const int lane = threadIdx.x;
     float s = 0.f;
@@ -979,8 +1030,8 @@ int k_cross_entropy(float *loss, float *softmax, const float *logits, const int3
         hipLaunchKernelGGL(ce_rows_cached_kernel<2>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
     else if (vec && v <= 64 * 4 * 8)
         hipLaunchKernelGGL(ce_rows_cached_kernel<8>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
-    else if (vec && v <= 64 * 4 * 32)
-        hipLaunchKernelGGL(ce_rows_cached_kernel<32>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
+    else if (vec && v <= 256 * 4 * 8 && n <= 0x7fffffffLL)
+        hipLaunchKernelGGL(ce_rows_wg_kernel<8>, dim3((unsigned)n), dim3(256), 0, st, (float *)rl, softmax, logits, targets, n, v);
     else
         hipLaunchKernelGGL(ce_rows_kernel, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
     int rc = check_launch("ce_rows");
