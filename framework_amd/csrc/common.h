@@ -45,7 +45,28 @@ struct DeviceCtx {
     unsigned *skinny_flags = nullptr;
     size_t skinny_flag_cap = 0;  // entries
     unsigned skinny_epoch = 0;
+    // Device status word in pinned host memory that kernels can write: a kernel
+    // whose bounded wait for another workgroup expires stores a DEVICE_STATUS_*
+    // code there (and NaN into its outputs).  Every call that waits for the
+    // stream reads the word afterwards and fails loudly when it is set.
+    unsigned *status_host = nullptr;  // host address
+    unsigned *status_dev = nullptr;   // the same word as kernels address it
+    // Workspace source of the current sgemm call: null = the caching allocator;
+    // otherwise the product's partial sums are placed in this preallocated
+    // block of `scratch_bytes` (the entry point that must not allocate).
+    float *scratch = nullptr;
+    size_t scratch_bytes = 0;
 };
+enum { DEVICE_STATUS_OK = 0, DEVICE_STATUS_STREAMK_WAIT = 1, DEVICE_STATUS_SKINNY_WAIT = 2 };
+// hipStreamSynchronize on the library's stream, then the device status word:
+// MNI_ERR_HIP naming the kernel when a bounded wait expired since the last check.
+int sync_stream_checked(const char *what);
+// The status word alone, for callers that have already waited (on an event).
+int check_device_status(const char *what);
+// Workspace of one product: from ctx().scratch when set (error when `bytes`
+// exceeds it), else from the caching allocator.  Release with gemm_ws_free.
+int gemm_ws_alloc(void **p, size_t bytes);
+void gemm_ws_free(void *p);
 DeviceCtx &ctx();
 
 // Every extern "C" entry point holds this for its whole duration: the engine

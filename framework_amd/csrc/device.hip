@@ -93,6 +93,12 @@ static int init_device(int device) {
     MNI_HIP_CHECK(hipMalloc((void **)&c.skinny_flags, c.skinny_flag_cap * sizeof(unsigned)));
     MNI_HIP_CHECK(hipMemset(c.skinny_flags, 0, c.skinny_flag_cap * sizeof(unsigned)));
     c.skinny_epoch = 0;
+    // Pinned, device-visible host memory: a kernel writes the word over the
+    // bus in the rare case it has something to report, the host reads it for
+    // free after every wait.
+    MNI_HIP_CHECK(hipHostMalloc((void **)&c.status_host, 64, hipHostMallocMapped));
+    memset(c.status_host, 0, 64);
+    MNI_HIP_CHECK(hipHostGetDevicePointer((void **)&c.status_dev, c.status_host, 0));
     c.ready = true;
     return MNI_OK;
 }
@@ -100,6 +106,37 @@ static int init_device(int device) {
 int ensure_init() {
     if (ctx().ready) return MNI_OK;
     return init_device(0);
+}
+
+int sync_stream_checked(const char *what) {
+    MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+    return check_device_status(what);
+}
+
+int check_device_status(const char *what) {
+    DeviceCtx &c = ctx();
+    if (!c.status_host) return MNI_OK;
+    const unsigned st = *(volatile unsigned *)c.status_host;
+    if (st == DEVICE_STATUS_OK) return MNI_OK;
+    *(volatile unsigned *)c.status_host = DEVICE_STATUS_OK;
+    const char *who = st == DEVICE_STATUS_STREAMK_WAIT  ? "gemm_mfma_kernel (stream-K): a finishing workgroup gave up waiting for a partial tile"
+                      : st == DEVICE_STATUS_SKINNY_WAIT ? "skinny_cols_kernel: a reducing workgroup gave up waiting for a K-slice partial"
+                                                        : "a kernel reported an unknown status";
+    return set_error(MNI_ERR_HIP, "%s: device status %u -- %s; results written since the last synchronisation hold NaN where "
+                                  "the wait expired", what, st, who);
+}
+
+int gemm_ws_alloc(void **p, size_t bytes) {
+    DeviceCtx &c = ctx();
+    if (!c.scratch) return dev_alloc(p, bytes);
+    if (bytes > c.scratch_bytes)
+        return set_error(MNI_ERR_INVALID, "sgemm_noalloc: this product needs %zu bytes of workspace, the fixed scratch holds %zu",
+                         bytes, c.scratch_bytes);
+    *p = c.scratch;
+    return MNI_OK;
+}
+void gemm_ws_free(void *p) {
+    if (p && p != (void *)ctx().scratch) dev_free(p);
 }
 
 int check_launch(const char *what) {
@@ -228,16 +265,14 @@ int mni_rocm_h2d(void *dst, const void *src, size_t bytes) {
     MNI_TRY(ensure_init());
     if (bytes == 0) return MNI_OK;
     MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
-    MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
-    return MNI_OK;
+    return sync_stream_checked("h2d");
 }
 int mni_rocm_d2h(void *dst, const void *src, size_t bytes) {
     MNI_API_GUARD;
     MNI_TRY(ensure_init());
     if (bytes == 0) return MNI_OK;
     MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
-    MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
-    return MNI_OK;
+    return sync_stream_checked("d2h");
 }
 int mni_rocm_d2d(void *dst, const void *src, size_t bytes) {
     MNI_API_GUARD;
@@ -249,7 +284,13 @@ int mni_rocm_d2d(void *dst, const void *src, size_t bytes) {
 int mni_rocm_sync(void) {
     MNI_API_GUARD;
     MNI_TRY(ensure_init());
-    MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+    return sync_stream_checked("sync");
+}
+
+int mni_rocm_test_raise_device_status(unsigned code) {
+    MNI_API_GUARD;
+    MNI_TRY(ensure_init());
+    *(volatile unsigned *)ctx().status_host = code;
     return MNI_OK;
 }
 
@@ -272,7 +313,7 @@ int mni_rocm_event_elapsed_ms(void *start, void *stop, float *ms) {
     MNI_API_GUARD;
     MNI_HIP_CHECK(hipEventSynchronize((hipEvent_t)stop));
     MNI_HIP_CHECK(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
-    return MNI_OK;
+    return check_device_status("event_elapsed_ms");
 }
 int mni_rocm_event_destroy(void *event) {
     MNI_API_GUARD;

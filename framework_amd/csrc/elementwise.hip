@@ -442,11 +442,11 @@ int k_mul_backward_same(float *ga, float *gb, const float *g, const float *a, co
 // in block order.
 static constexpr int CS_ROWS = 32;  // rows per block in pass 1 (a [4096, 768] gradient then gives 384 workgroups, not 96)
 __global__ void colsum_partial_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t rows,
-                                      int64_t cols) {
+                                      int64_t cols, int64_t rows_per_block) {
     const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= cols) return;
-    const int64_t r0 = (int64_t)blockIdx.y * CS_ROWS;
-    const int64_t r1 = min(rows, r0 + CS_ROWS);
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = min(rows, r0 + rows_per_block);
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     int64_t r = r0;
     for (; r + 7 < r1; r += 8) {  // 8 loads in flight, four running sums
@@ -464,6 +464,41 @@ __global__ void colsum_partial_kernel(float *__restrict__ part, const float *__r
     }
     for (; r < r1; ++r) s0 += a[r * cols + c];
     part[(int64_t)blockIdx.y * cols + c] = (s0 + s1) + (s2 + s3);
+}
+// Few columns (a reduction to a scalar or to a short vector): a thread per
+// column would leave most of a wavefront idle, so the 256 threads of a block
+// form `lanes` = 256 / cols row lanes of cols threads each; row lane l takes
+// rows l, l + lanes, ... of the block's CN_ROWS * lanes rows (consecutive
+// threads read consecutive floats), and the lanes are added in lane order.
+static constexpr int CN_COLS = 64;   // widest matrix that takes this form
+static constexpr int CN_ROWS = 32;   // rows per thread
+__global__ __launch_bounds__(256) void colsum_narrow_kernel(float *__restrict__ part, const float *__restrict__ a,
+                                                            int64_t rows, int cols, int lanes) {
+    __shared__ float sh[256];
+    const int t = threadIdx.x;
+    const int l = t / cols, c = t - l * cols;
+    const int64_t r0 = (int64_t)blockIdx.x * CN_ROWS * lanes;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (l < lanes) {
+#pragma unroll
+        for (int i0 = 0; i0 < CN_ROWS; i0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int64_t r = r0 + l + (int64_t)(i0 + e) * lanes;
+                v[e] = r < rows ? a[r * cols + c] : 0.0f;
+            }
+            s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
+            s0 += v[4]; s1 += v[5]; s2 += v[6]; s3 += v[7];
+        }
+    }
+    sh[t] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (t < cols) {
+        float v = sh[t];
+        for (int k = 1; k < lanes; ++k) v += sh[k * cols + t];
+        part[(int64_t)blockIdx.x * cols + t] = v;
+    }
 }
 // Pass 2: 64 columns per block, the partials dealt to four thread groups as
 // contiguous quarters (a quarter of the loads per thread, all in flight at
@@ -498,23 +533,37 @@ int k_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
     if (cols <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (rows <= 0) return k_fill(out, 0.0f, cols);
-    const int64_t nparts = (rows + CS_ROWS - 1) / CS_ROWS;
-    if (nparts > 65535) return set_error(MNI_ERR_INVALID, "colsum: too many rows (%lld)", (long long)rows);
     const dim3 block(TPB);
+    // Row blocks: 32 rows each; more when the second grid axis (65535 blocks)
+    // would not hold them.  Few columns and many rows: the row-lane form.
+    const bool narrow = cols <= CN_COLS && rows >= 4 * CN_ROWS;
+    const int lanes = narrow ? 256 / (int)cols : 0;
+    int64_t rows_per_block = narrow ? (int64_t)CN_ROWS * lanes : CS_ROWS;
+    int64_t nparts = (rows + rows_per_block - 1) / rows_per_block;
+    if (!narrow && nparts > 65535) {
+        rows_per_block = ((rows + 65534) / 65535 + 7) / 8 * 8;
+        nparts = (rows + rows_per_block - 1) / rows_per_block;
+    }
+    if (nparts > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "colsum: too many rows (%lld)", (long long)rows);
     const unsigned gx = (unsigned)((cols + TPB - 1) / TPB);
-    if (nparts == 1) {
-        hipLaunchKernelGGL(colsum_partial_kernel, dim3(gx, 1), block, 0, ctx().stream, out, a, rows, cols);
-        return check_launch("colsum");
-    }
     void *part = nullptr;
-    MNI_TRY(dev_alloc(&part, (size_t)nparts * cols * sizeof(float)));
-    hipLaunchKernelGGL(colsum_partial_kernel, dim3(gx, (unsigned)nparts), block, 0, ctx().stream, (float *)part, a, rows, cols);
+    if (nparts > 1) MNI_TRY(dev_alloc(&part, (size_t)nparts * cols * sizeof(float)));
+    float *dst = nparts > 1 ? (float *)part : out;
+    if (narrow)
+        hipLaunchKernelGGL(colsum_narrow_kernel, dim3((unsigned)nparts), dim3(256), 0, ctx().stream, dst, a, rows, (int)cols, lanes);
+    else
+        hipLaunchKernelGGL(colsum_partial_kernel, dim3(gx, (unsigned)nparts), block, 0, ctx().stream, dst, a, rows, cols, rows_per_block);
     int rc = check_launch("colsum_partial");
-    if (rc == MNI_OK) {
-        hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, out, (const float *)part, nparts, cols);
-        rc = check_launch("colsum_final");
+    if (rc == MNI_OK && nparts > 1) {
+        if (nparts > 1024) {
+            // many partials: they are a tall matrix themselves
+            rc = k_colsum(out, (const float *)part, nparts, cols);
+        } else {
+            hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, out, (const float *)part, nparts, cols);
+            rc = check_launch("colsum_final");
+        }
     }
-    dev_free(part);
+    if (part) dev_free(part);
     return rc;
 }
 
@@ -551,12 +600,13 @@ int k_bias_gelu(float *out, const float *x, const float *bias, int64_t rows, int
 static constexpr int BG_ROWS = 16;  // rows per block in the backward pass
 template <typename V, int W>
 __global__ void bias_gelu_bwd_kernel(V *__restrict__ dx, V *__restrict__ part, const V *__restrict__ g,
-                                     const V *__restrict__ x, const V *__restrict__ bias, int64_t rows, int64_t colsv) {
-    // colsv = columns in units of V (float or float4); thread = one V column, BG_ROWS rows
+                                     const V *__restrict__ x, const V *__restrict__ bias, int64_t rows, int64_t colsv,
+                                     int64_t rows_per_block) {
+    // colsv = columns in units of V (float or float4); thread = one V column, rows_per_block rows
     const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= colsv) return;
-    const int64_t r0 = (int64_t)blockIdx.y * BG_ROWS;
-    const int64_t r1 = min(rows, r0 + BG_ROWS);
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = min(rows, r0 + rows_per_block);
     float b[W], s[W];
     {
         const V bv = bias[c];
@@ -587,8 +637,12 @@ int k_bias_gelu_backward(float *dx, float *dbias, const float *g, const float *x
     if (cols <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (rows <= 0) return k_fill(dbias, 0.0f, cols);
-    const int64_t nparts = (rows + BG_ROWS - 1) / BG_ROWS;
-    if (nparts > 65535) return set_error(MNI_ERR_INVALID, "bias_gelu backward: too many rows (%lld)", (long long)rows);
+    int64_t rows_per_block = BG_ROWS;
+    int64_t nparts = (rows + rows_per_block - 1) / rows_per_block;
+    if (nparts > 65535) {  // the second grid axis holds no more
+        rows_per_block = (rows + 65534) / 65535;
+        nparts = (rows + rows_per_block - 1) / rows_per_block;
+    }
     const bool vec = cols % 4 == 0 && al16(dx) && al16(g) && al16(x) && al16(bias) && al16(dbias);
     const int64_t colsv = vec ? cols / 4 : cols;
     const dim3 block(TPB);
@@ -598,10 +652,10 @@ int k_bias_gelu_backward(float *dx, float *dbias, const float *g, const float *x
     float *dst = nparts > 1 ? (float *)part : dbias;
     if (vec)
         hipLaunchKernelGGL((bias_gelu_bwd_kernel<float4, 4>), dim3(gx, (unsigned)nparts), block, 0, ctx().stream, (float4 *)dx,
-                           (float4 *)dst, (const float4 *)g, (const float4 *)x, (const float4 *)bias, rows, colsv);
+                           (float4 *)dst, (const float4 *)g, (const float4 *)x, (const float4 *)bias, rows, colsv, rows_per_block);
     else
         hipLaunchKernelGGL((bias_gelu_bwd_kernel<float, 1>), dim3(gx, (unsigned)nparts), block, 0, ctx().stream, dx, dst, g, x,
-                           bias, rows, colsv);
+                           bias, rows, colsv, rows_per_block);
     int rc = check_launch("bias_gelu_backward");
     if (rc == MNI_OK && nparts > 1) {
         hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dbias,

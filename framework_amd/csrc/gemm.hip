@@ -34,7 +34,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_MFMA_STREAMK)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_DIRECT)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -95,7 +95,7 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         s.out = d.C; s.o_bs = d.c_batch_stride; s.bias = d.bias;
         s.epilogue = d.epilogue; s.accumulate = d.accumulate;
         s.ws = nullptr; s.split_k = 1; s.k_per_slice = s.K;
-        s.groups = 0; s.fused = 0; s.xcds = 0; s.flags = nullptr; s.epoch = 0;
+        s.groups = 0; s.fused = 0; s.xcds = 0; s.flags = nullptr; s.epoch = 0; s.status = ctx().status_dev;
 
         const bool w_batch_ok = s.w_bcount <= 1 || (s.w_bs % 4) == 0;
         const bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
@@ -126,7 +126,7 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
             void *ws = nullptr;
             if (split > 1) {
                 const size_t bytes = (size_t)split * s.batch * s.rows * s.cols * sizeof(float);
-                *rc = dev_alloc(&ws, bytes);
+                *rc = gemm_ws_alloc(&ws, bytes);
                 if (*rc != MNI_OK) return true;
                 s.ws = (float *)ws;
             }
@@ -148,7 +148,7 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
                 r.epilogue = s.epilogue; r.accumulate = s.accumulate; r.bias_on_rows = s.bias_on_rows;
                 *rc = launch_skinny_reduce(r);
             }
-            if (ws) dev_free(ws);
+            gemm_ws_free(ws);
             return true;
         }
         if (w_dots && d.split_k <= 1) {
@@ -163,6 +163,14 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
 }
 
 // ---- MFMA path ----------------------------------------------------------------
+// Which products go to the register-direct kernel by themselves: 0 = none,
+// else the number of wavefronts that share K.
+static int direct_plan(const GemmLaunch &g, int cus) {
+    (void)g;
+    (void)cus;
+    return 0;
+}
+
 static int run_mfma(const mni_gemm_desc &d) {
     GemmLaunch g;
     g.A = d.A.ptr; g.B = d.B.ptr; g.C = d.C; g.bias = d.bias; g.ws = nullptr;
@@ -182,6 +190,29 @@ static int run_mfma(const mni_gemm_desc &d) {
     const int amode = g.K == 0 ? 2 : classify(g.a_cs, g.a_rs);
     // op(B)(k, n): K stride = row_stride, N stride = col_stride.
     const int bmode = g.K == 0 ? 2 : classify(g.b_rs, g.b_cs);
+
+    // Register-direct form: forced, or chosen for batched products of many small tiles.
+    {
+        int ksplit = 0;
+        if (d.algo == MNI_ALGO_DIRECT) {
+            if (!gemm_direct_eligible(g, amode, bmode))
+                return set_error(MNI_ERR_INVALID, "sgemm: operand layouts not eligible for the direct kernel (each operand "
+                                                  "contiguous along K with K %% 4 == 0, or along M / N with an even extent)");
+            if (d.split_k != 0 && d.split_k != 1 && d.split_k != 4)
+                return set_error(MNI_ERR_INVALID, "sgemm: the direct kernel takes split_k 0, 1 or 4");
+            ksplit = d.split_k == 4 ? 4 : 1;
+        } else if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_direct_eligible(g, amode, bmode)) {
+            ksplit = direct_plan(g, cus);
+        }
+        if (ksplit) {
+            g.tiles_m = (g.M + 63) / 64;
+            g.tiles_n = (g.N + 63) / 64;
+            g.split_k = 1;
+            g.k_per_slice = g.K;
+            g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
+            return launch_gemm_direct(g, amode, bmode, ksplit);
+        }
+    }
 
     // Can the K steps of tiles of this shape be dealt over the stream-K grid?
     // In every XCD's stream-K region each workgroup must own at least
@@ -266,7 +297,7 @@ static int run_mfma(const mni_gemm_desc &d) {
     g.tiles_m = (g.M + bm - 1) / bm;
     g.tiles_n = (g.N + bn - 1) / bn;
 
-    g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0;
+    g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
     void *ws = nullptr;
     if (streamk) {
         g.split_k = 1;
@@ -276,10 +307,10 @@ static int run_mfma(const mni_gemm_desc &d) {
         g.sk_wpx = cus / c.xcd_count * gemm_mfma_resident_per_cu(bm, bn);
         g.sk_flags = c.skinny_flags;
         MNI_TRY(next_epoch(&g.sk_epoch));
-        MNI_TRY(dev_alloc(&ws, (size_t)g.sk_xcds * g.sk_wpx * bm * bn * sizeof(float)));
+        MNI_TRY(gemm_ws_alloc(&ws, (size_t)g.sk_xcds * g.sk_wpx * bm * bn * sizeof(float)));
         g.ws = (float *)ws;
         const int rc = launch_gemm_mfma(g, amode, bmode, bm, bn);
-        dev_free(ws);
+        gemm_ws_free(ws);
         return rc;
     }
 
@@ -305,13 +336,13 @@ static int run_mfma(const mni_gemm_desc &d) {
 
     if (split > 1) {
         const size_t bytes = (size_t)split * g.batch * g.M * g.N * sizeof(float);
-        MNI_TRY(dev_alloc(&ws, bytes));
+        MNI_TRY(gemm_ws_alloc(&ws, bytes));
         g.ws = (float *)ws;
     }
     int rc = launch_gemm_mfma(g, amode, bmode, bm, bn);
     if (rc == MNI_OK && split > 1)
         rc = finish_split(g.ws, g.C, g.bias, split, g.batch, g.M, g.N, g.ldc, 1, g.c_bs, g.epilogue, g.accumulate, 0);
-    if (ws) dev_free(ws);
+    gemm_ws_free(ws);
     return rc;
 }
 
@@ -360,6 +391,7 @@ extern "C" int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int w
     (void)hipEventDestroy(e1);
     if (rc != MNI_OK) return rc;
     if (he != hipSuccess) return set_error(MNI_ERR_HIP, "sgemm_timed: %s", hipGetErrorString(he));
+    MNI_TRY(check_device_status("sgemm_timed"));
     *avg_ms = ms / (float)iters;
     return MNI_OK;
 }

@@ -27,6 +27,7 @@ struct GemmLaunch {
     int streamk, sk_wpx, sk_xcds;
     unsigned *sk_flags;
     unsigned sk_epoch;
+    unsigned *status;  // device status word: set when a finisher's bounded wait expires
 };
 
 // tile_m, tile_n in {128, 64}; g.tiles_m / g.tiles_n count tiles of that size
@@ -34,6 +35,12 @@ int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int 
 // workgroups that stay resident per CU for a tile shape (what the stream-K grid is sized by)
 int gemm_mfma_resident_per_cu(int tile_m, int tile_n);
 int gemm_mfma_tile_k();
+// Register-direct form for batched products of many small tiles (gemm_direct.hip):
+// 64 x 64 tiles (g.tiles_m / g.tiles_n count those), one wavefront per tile
+// (ksplit 1) or four wavefronts sharing K (ksplit 4).  amode / bmode as for
+// the tile kernel; both must be 0 or 1 and pass gemm_direct_eligible.
+bool gemm_direct_eligible(const GemmLaunch &g, int amode, int bmode);
+int launch_gemm_direct(const GemmLaunch &g, int amode, int bmode, int ksplit);
 
 // Skinny (GEMV-shaped) products: X (MR x K, MR <= 16) against a large W.
 //   out[b](i, j) = sum_k X[b](i, k) * W[b](k, j),  i < rows, j < cols
@@ -58,6 +65,7 @@ struct SkinnyLaunch {
     int fused, xcds;
     unsigned *flags;
     unsigned epoch;
+    unsigned *status;  // device status word: set when a reducer's bounded wait expires
 };
 // W with unit stride along j (cols): lanes own columns, K split over wavefronts and slices.
 int launch_skinny_cols(const SkinnyLaunch &s);

@@ -79,7 +79,7 @@ static constexpr int BK = 32;
 static constexpr int KQ = BK / 4;           // K quads per tile
 static constexpr int PAD = 2;               // float4 of padding per K-quad slice
 static constexpr int NTHREADS = 256;
-static constexpr int SK_WAIT_LIMIT = 1 << 20;  // polls before a finisher gives up and writes NaN
+static constexpr int SK_WAIT_LIMIT = 1 << 20;  // polls before a finisher gives up, writes NaN and sets the status word
 
 __device__ __forceinline__ unsigned load_mark(const unsigned *p) {
     // sc1: answered by the XCD's L2, never by this CU's L1
@@ -631,6 +631,8 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
             }
         }
         lost = __syncthreads_or(!ok) != 0;
+        // Tell the host: the next call that waits for the stream fails with this code.
+        if (lost && tid == 0) *g.status = DEVICE_STATUS_STREAMK_WAIT;
     }
     float *const slot = g.ws + (int64_t)bid * (BM * BN);  // ROLE_PART: where this workgroup parks its tile
     // all wavefronts are past their last LDS read (barrier at the end of the K loop)
@@ -729,7 +731,7 @@ int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int 
     if ((int64_t)g.tiles_m * g.tiles_n * g.batch <= 0) return MNI_OK;
     if (g.streamk) {
         // what the kernel's arithmetic assumes about its grid and buffers
-        if (g.split_k != 1 || g.sk_xcds < 1 || g.sk_wpx < 1 || g.sk_wpx > NTHREADS || !g.ws || !g.sk_flags)
+        if (g.split_k != 1 || g.sk_xcds < 1 || g.sk_wpx < 1 || g.sk_wpx > NTHREADS || !g.ws || !g.sk_flags || !g.status)
             return set_error(MNI_ERR_INVALID, "sgemm: inconsistent stream-K launch");
     }
     const int64_t blocks = g.streamk ? (int64_t)g.sk_xcds * g.sk_wpx : (int64_t)g.tiles_m * g.tiles_n * g.batch * g.split_k;

@@ -226,6 +226,13 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
             arrived = __all(all);
             if (!arrived) __builtin_amdgcn_s_sleep(2);
         }
+        // Tell the host: the next call that waits for the stream fails with this code.
+        if (!arrived && tid == 0) *s.status = DEVICE_STATUS_SKINNY_WAIT;
+        // The partials are read with ordinary loads.  A 128-byte line of the
+        // workspace can be shared by two units when cols is not a multiple of
+        // 32, so this CU's L1 may hold such a line from before the other
+        // unit's partial landed: drop the L1 contents once, after the flags.
+        asm volatile("buffer_inv sc1" ::: "memory");
 
         constexpr int TB = 16;  // partials in flight per lane
         const int64_t slice_stride = (int64_t)batch * rows * s.cols;
@@ -445,7 +452,7 @@ int launch_skinny_cols(const SkinnyLaunch &s) {
     const bool fused = s.fused && s.split_k > 1;
     dim3 grid(groups, s.split_k, s.batch);
     if (fused) {
-        if (s.xcds <= 0 || !s.flags || !s.ws) return set_error(MNI_ERR_INVALID, "single-launch skinny product without flags/partials");
+        if (s.xcds <= 0 || !s.flags || !s.ws || !s.status) return set_error(MNI_ERR_INVALID, "single-launch skinny product without flags/partials");
         const int64_t units = (int64_t)groups * s.batch;
         grid = dim3((unsigned)((units + s.xcds - 1) / s.xcds * s.xcds), s.split_k);
     }

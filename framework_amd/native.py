@@ -23,7 +23,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmni_rocm.so")
 BAD_ID = 0xFFFFFFFF
 MAX_DIMS = 8
 EPI_NONE, EPI_BIAS, EPI_BIAS_RELU, EPI_BIAS_GELU = 0, 1, 2, 3
-ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL, ALGO_SKINNY_TWO_PASS, ALGO_MFMA_STREAMK = 0, 1, 2, 3, 4, 5
+ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL, ALGO_SKINNY_TWO_PASS, ALGO_MFMA_STREAMK, ALGO_DIRECT = 0, 1, 2, 3, 4, 5, 6
 
 _f32p = C.POINTER(C.c_float)
 _i64p = C.POINTER(C.c_int64)
@@ -60,6 +60,7 @@ SIGNATURES = {
     "mni_rocm_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "mni_rocm_d2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "mni_rocm_sync": (C.c_int, []),
+    "mni_rocm_test_raise_device_status": (C.c_int, [C.c_uint]),
     "mni_rocm_event_create": (C.c_int, [C.POINTER(C.c_void_p)]),
     "mni_rocm_event_record": (C.c_int, [C.c_void_p]),
     "mni_rocm_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
@@ -217,6 +218,9 @@ class Rocm:
 
     def sync(self):
         self._check(self.lib.mni_rocm_sync())
+
+    def test_raise_device_status(self, code):
+        self._check(self.lib.mni_rocm_test_raise_device_status(code))
 
     def event(self):
         e = C.c_void_p()

@@ -71,6 +71,17 @@ int mni_rocm_h2d(void *dst, const void *src, size_t bytes);
 int mni_rocm_d2h(void *dst, const void *src, size_t bytes);
 int mni_rocm_d2d(void *dst, const void *src, size_t bytes);
 int mni_rocm_sync(void);
+/* Device status.  A kernel that has to wait for other workgroups of its own
+ * launch (the single-launch K-slice reduction of the skinny kernel, the
+ * stream-K tile fix-up) waits a bounded number of polls; if the wait expires
+ * it writes NaN into the outputs concerned and a code into a status word, and
+ * the next call that waits for the stream (mni_rocm_sync, h2d, d2h,
+ * event_elapsed_ms, sgemm_timed and every engine call built on them, such as
+ * mni_to_float32 / mni_get_scalar) returns MNI_ERR_HIP with a message naming
+ * the kernel, and clears the word.  mni_rocm_test_raise_device_status sets
+ * the word from the host, so that this error path can be exercised without
+ * making a kernel hang.  No counterpart in the reference. */
+int mni_rocm_test_raise_device_status(unsigned code);
 
 /* Stream-ordered timing marks on the library's stream (HIP events). */
 int mni_rocm_event_create(void **event);
@@ -98,9 +109,14 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * device's workgroup-to-XCD mapping was not confirmed); SKINNY = the bandwidth
  * kernels (error if the shape or layout is not eligible); SKINNY_TWO_PASS = the
  * same with the K-slice partials summed by a second launch instead of inside
- * the first.  AUTO picks among them. */
+ * the first; DIRECT = the register-direct MFMA kernel for batched products of
+ * many small tiles (64 x 64 tiles, operands read from memory straight into the
+ * matrix instruction's registers; split_k 0 or 1 = one wavefront per tile,
+ * split_k 4 = four wavefronts sharing K; error if the operand layouts are not
+ * eligible: each operand contiguous along K with K % 4 == 0, or along M / N
+ * with that extent even).  AUTO picks among them. */
 enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
-       MNI_ALGO_MFMA_STREAMK = 5 };
+       MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),
@@ -179,7 +195,8 @@ uint32_t mni_sum_all(uint32_t a);                                         /* lib
 uint32_t mni_mean_all(uint32_t a);                                        /* lib.rs:267-277 */
 uint32_t mni_view(uint32_t a, const int64_t *shape, int ndim);            /* lib.rs:279-285 */
 uint32_t mni_permute(uint32_t a, const int64_t *dims, int ndim);          /* lib.rs:287-293 */
-uint32_t mni_contiguous(uint32_t a);                                      /* KV cache for incremental decoding (src/native/src/lib.rs:586-676 -> ops/kv_cache.rs): per cache
+uint32_t mni_contiguous(uint32_t a);                                      /* lib.rs:295-300 */
+/* KV cache for incremental decoding (src/native/src/lib.rs:586-676 -> ops/kv_cache.rs): per cache
  * [batch * heads, max_seq_len, head_dim] keys and values in device memory, fp32 or int8 with one f32 scale per
  * row (quantize_row_i8, kv_cache.rs:357-370).  The reference keeps the cache in host memory and decodes on the
  * CPU; here append and decode are kernels.  Ids start at 1 and restart after mni_reset_engine.
@@ -265,7 +282,6 @@ uint32_t mni_softmax_op(uint32_t a, int64_t dim);
  * five backward products) with row kernels for scale / causal mask /
  * normalisation.  Either replaces the per-key loop of kernels/flash_attention.cu. */
 uint32_t mni_flash_attention(uint32_t q, uint32_t k, uint32_t v, double scale, int causal);
-/* lib.rs:295-300 */
 uint32_t mni_cross_entropy_loss(uint32_t logits, const int64_t *targets, size_t n); /* lib.rs:328-336 */
 int mni_adamw_step(const uint32_t *ids, size_t n, double lr, double beta1, double beta2,
                    double eps, double weight_decay, int64_t step);        /* lib.rs:400-412 */

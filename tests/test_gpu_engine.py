@@ -429,6 +429,24 @@ def test_unbroadcast_patterns_vs_oracle(gpu, orc):
         assert_close(x, y, 1e-5, str(shape))
 
 
+def test_scalar_and_bias_gradients_of_large_tensors_vs_oracle(gpu, orc):
+    # a broadcast operand's gradient is a sum over every element of a [3000, 1024] tensor (3.07M rows of one
+    # column: more row blocks than one grid axis holds), and over its 3000 rows for a [1024] operand
+    x = synth.normal(21, (3000, 1024))
+    g = synth.normal(22, (3000, 1024), stream=1)
+
+    def script(api):
+        a = T(api, x, True)
+        c, d, e = T(api, np.array([1.0]), True), T(api, np.zeros(1024), True), T(api, np.full((1, 1), 0.5), True)
+        a.add(c).sub(d).mul(e).mul(T(api, g)).sum().backward()
+        return [c.grad.numpy(), d.grad.numpy(), e.grad.numpy(), a.grad.numpy()]
+    for (got, want), k in zip(zip(*both(gpu, orc, script)), (3072000, 3000, 3072000, 1)):
+        assert got.shape == want.shape
+        # the oracle adds in flat order in float32; bound both against the float64 sum
+        tol = 1e-4 * np.sqrt(k) * 4.0 * 5.0
+        assert max_err(got, want) <= tol
+
+
 def test_reductions_views_and_activations_vs_oracle(gpu, orc):
     x = synth.normal(1, (3, 5, 300))
 

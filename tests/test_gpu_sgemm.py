@@ -446,6 +446,23 @@ def test_skinny_batched_and_vs_oracle(dev, oracle_native):
         assert max_err(got[i], oracle_native.sgemm_ikj(a[i], w[0])) <= gemm_tol(4096, a, w)
 
 
+@pytest.mark.parametrize("algo", SKINNY_ALGOS)
+def test_skinny_cols_units_sharing_a_cache_line(dev, algo):
+    # N = 2100: 9 column groups, and rows of the partials that are not whole
+    # 128-byte lines, so the end of one unit's row shares a line with the
+    # start of another unit's row (both units on the same XCD: groups 0 and 8)
+    a = synth.normal(1, (4, 4096), 0.02)
+    w = synth.normal(2, (4096, 2100), 0.02, stream=1)
+    want = a.astype(np.float64) @ w.astype(np.float64)
+    first = run_gemm(dev, a, w, algo=algo)[0]
+    assert max_err(first, want) <= gemm_tol(4096, a, w)
+    for _ in range(20):
+        assert np.array_equal(run_gemm(dev, a, w, algo=algo)[0], first)
+    ai = synth.small_ints(3, (4, 4096), 3)
+    wi = synth.small_ints(4, (4096, 2100), 3, stream=1)
+    assert np.array_equal(run_gemm(dev, ai, wi, algo=algo)[0], (ai.astype(np.int64) @ wi.astype(np.int64)).astype(np.float32))
+
+
 def test_skinny_ineligible_is_an_error_only_when_forced(dev, rocm):
     a = synth.small_ints(1, (40, 30), 3)
     b = synth.small_ints(2, (30, 50), 3, stream=1)
@@ -496,6 +513,13 @@ def test_strided_copy_add_bias_colsum_axpy_fill(dev, rocm):
     dbig, cs2 = dev.put(big), dev.empty(33)
     rocm.colsum(cs2, dbig, 5000, 33)
     assert max_err(rocm.to_host(cs2, (33,)), big.astype(np.float64).sum(0)) <= gemm_tol(5000, big, np.ones(1))
+    # more row blocks than the second grid axis holds (2.2M rows of 4 columns, in both forms), and few
+    # columns against many rows (the row-lane form): integer inputs, so any summation order is exact
+    tall = synth.small_ints(5, (2200000, 4), 3)
+    dtall, cs3 = dev.put(tall), dev.empty(128)
+    for rows, cols in ((2200000, 4), (100000, 88), (2200000 * 4, 1), (275000, 32), (200, 44)):
+        rocm.colsum(cs3, dtall, rows, cols)
+        assert np.array_equal(rocm.to_host(cs3, (cols,)), tall.ravel()[:rows * cols].reshape(rows, cols).astype(np.int64).sum(0).astype(np.float32))
     rocm.axpy(out, da, 2.0, a.size)
     assert np.array_equal(rocm.to_host(out, (300, 96)), a + bias + 2 * a)
     rocm.fill(out, 3.5, 7)
@@ -584,6 +608,40 @@ def test_config5b_tall_k_weight_gradient(dev, rocm):
     rows, cols = slice(100, 116), slice(900, 932)
     want = X[:, rows].astype(np.float64).T @ dY[:, cols].astype(np.float64)
     assert max_err(got[rows, cols], want) <= gemm_tol(65536, X, dY)
+
+
+def test_device_status_word_makes_the_next_wait_fail(dev, rocm):
+    # What a kernel does when its bounded wait for another workgroup expires (NaN into the output, a code
+    # into the status word) cannot be provoked without hanging a kernel; the host side can: set the word
+    # the way such a kernel would and see that every waiting call reports it once and then recovers.
+    x = dev.put(np.ones(8, np.float32))
+    for code, text in ((1, "stream-K"), (2, "skinny_cols_kernel")):
+        rocm.test_raise_device_status(code)
+        with pytest.raises(N.MniError, match=text):
+            rocm.sync()
+        rocm.sync()  # cleared by the report
+        rocm.test_raise_device_status(code)
+        with pytest.raises(N.MniError, match="device status %d" % code):
+            rocm.to_host(x, (8,))
+        assert np.array_equal(rocm.to_host(x, (8,)), np.ones(8, np.float32))
+    rocm.test_raise_device_status(2)
+    e0, e1 = rocm.event(), rocm.event()
+    rocm.record(e0)
+    rocm.record(e1)
+    with pytest.raises(N.MniError, match="device status 2"):
+        rocm.elapsed_ms(e0, e1)
+    assert rocm.elapsed_ms(e0, e1) >= 0.0
+    rocm.event_destroy(e0)
+    rocm.event_destroy(e1)
+    # the engine's read-backs go through the same check
+    from framework_amd.native import Native
+    nat = Native()
+    t = nat.fromFloat32(np.arange(4, dtype=np.float32), [4])
+    rocm.test_raise_device_status(1)
+    with pytest.raises(N.MniError, match="device status 1"):
+        nat.toFloat32(t)
+    assert np.array_equal(nat.toFloat32(t), np.arange(4, dtype=np.float32))
+    nat.freeTensor(t)
 
 
 def test_sgemm_timed_runs_the_products_and_reports_a_duration(dev, rocm):
