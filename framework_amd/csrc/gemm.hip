@@ -34,7 +34,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_DIRECT)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_PANEL)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -166,9 +166,29 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
 // Which products go to the register-direct kernel by themselves: 0 = none,
 // else the number of wavefronts that share K.
 static int direct_plan(const GemmLaunch &g, int cus) {
-    (void)g;
-    (void)cus;
+    // Four wavefronts per 64 x 64 tile, a quarter of K each: when about one such
+    // workgroup exists per CU (between half and five quarters of the CUs; with
+    // more, the tile kernel's larger tiles and resident rounds win, with fewer,
+    // K slices across workgroups) and K is long enough to be worth splitting but
+    // not so long that two 32-deep phases in flight per wavefront starve it.
+    // Measured on MI355X against the tile kernel's plans, microseconds:
+    // [32 x 512 x 512] x [512 x 64] 16.7 vs 22.7, its transposed twin 15.9 vs 22.8,
+    // K = 256: 11.6 vs 17.0, 32 x (128 x 128 x 512) 15.6 vs 27.0,
+    // 16 x (1024 x 64 x 1024) 27.2 vs 30.5; 64 batches of the first 31.2 vs 31.0,
+    // 128 batches 59 vs 44, 4 x (2048 x 64 x 2048) 43.9 vs 33.3.
+    const int64_t tiles = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) * g.batch;
+    if (tiles * 2 >= cus && tiles * 4 <= 5LL * cus && g.K >= 128 && (g.K <= 1024 || (tiles >= cus && g.K <= 4096))) return 4;
     return 0;
+}
+
+// Whether a short-K product of two K-contiguous operands goes to the panel kernel by itself.
+static bool panel_plan(const GemmLaunch &g, int cus) {
+    // When its 128 x 128 tiles give more than half the CUs a workgroup.  Measured on MI355X against the
+    // tile kernel's plans, microseconds: 32 x (512 x 512 x 64) 13.8 vs 19.5, 8 x (1024 x 1024 x 64) 13.0 vs
+    // 18.5, 4096 x 4096 x 64 22.3 vs 34.9, K = 32: 9.9 vs 13.7, 16 x (384 x 384 x 64) 8.1 vs 8.7; at
+    // 8 x (512 x 512 x 64), 128 tiles, the tile kernel's 64 x 64 tiles are ahead, 7.4 vs 8.0.
+    const int64_t tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
+    return tiles * 2 > cus;
 }
 
 static int run_mfma(const mni_gemm_desc &d) {
@@ -191,6 +211,18 @@ static int run_mfma(const mni_gemm_desc &d) {
     // op(B)(k, n): K stride = row_stride, N stride = col_stride.
     const int bmode = g.K == 0 ? 2 : classify(g.b_rs, g.b_cs);
 
+    // Short-K panel form: forced, or chosen when its 128 x 128 tiles fill the machine.
+    if (d.algo == MNI_ALGO_PANEL || (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_panel_eligible(g, amode, bmode) && panel_plan(g, cus))) {
+        if (!gemm_panel_eligible(g, amode, bmode))
+            return set_error(MNI_ERR_INVALID, "sgemm: the short-K panel kernel takes two K-contiguous operands with K <= 64, K %% 4 == 0");
+        if (d.split_k > 1) return set_error(MNI_ERR_INVALID, "sgemm: the short-K panel kernel takes no split_k");
+        g.tiles_m = (g.M + 127) / 128;
+        g.tiles_n = (g.N + 127) / 128;
+        g.split_k = 1;
+        g.k_per_slice = g.K;
+        g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
+        return launch_gemm_panel(g, amode, bmode);
+    }
     // Register-direct form: forced, or chosen for batched products of many small tiles.
     {
         int ksplit = 0;

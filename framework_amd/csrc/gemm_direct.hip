@@ -206,8 +206,15 @@ __global__ __launch_bounds__(64 * KSPLIT, (KSPLIT == 1 || NPH == 0) ? 2 : 1) voi
             load_phase(ra[s], pa, s * DPHASE);
             load_phase(rb[s], pb, s * DPHASE);
         }
+        // Left alone, the instruction scheduler moves every load down to its
+        // first use to save registers, and the kernel then waits for memory
+        // once per load.  Requests first, arithmetic after.
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int s = 0; s < NPH; ++s) mfma_phase<AMODE, BMODE>(acc, ra[s], rb[s]);
+        for (int s = 0; s < NPH; ++s) {
+            mfma_phase<AMODE, BMODE>(acc, ra[s], rb[s]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     } else {
         const int nfull = klen / DPHASE;
         if (nfull > 0) {
@@ -220,13 +227,20 @@ __global__ __launch_bounds__(64 * KSPLIT, (KSPLIT == 1 || NPH == 0) ? 2 : 1) voi
             load_phase(b0, pb, 0);
             load_phase(a1, pa, min(1, nfull - 1) * DPHASE);
             load_phase(b1, pb, min(1, nfull - 1) * DPHASE);
+            // (the fences keep requests and arithmetic in this order: left alone, the
+            // scheduler moves every load down to its first use to save registers)
+            __builtin_amdgcn_sched_barrier(0);
             for (int p = 0; p < nfull; p += 2) {
                 mfma_phase<AMODE, BMODE>(acc, a0, b0);
+                __builtin_amdgcn_sched_barrier(0);
                 load_phase(a0, pa, min(p + 2, nfull - 1) * DPHASE);
                 load_phase(b0, pb, min(p + 2, nfull - 1) * DPHASE);
+                __builtin_amdgcn_sched_barrier(0);
                 if (p + 1 < nfull) mfma_phase<AMODE, BMODE>(acc, a1, b1);
+                __builtin_amdgcn_sched_barrier(0);
                 load_phase(a1, pa, min(p + 3, nfull - 1) * DPHASE);
                 load_phase(b1, pb, min(p + 3, nfull - 1) * DPHASE);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         if (nfull * DPHASE < klen) {

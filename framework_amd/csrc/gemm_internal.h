@@ -41,6 +41,10 @@ int gemm_mfma_tile_k();
 // the tile kernel; both must be 0 or 1 and pass gemm_direct_eligible.
 bool gemm_direct_eligible(const GemmLaunch &g, int amode, int bmode);
 int launch_gemm_direct(const GemmLaunch &g, int amode, int bmode, int ksplit);
+// Short-K form for two K-contiguous operands (gemm_panel.hip): 128 x 128 tiles
+// (g.tiles_m / g.tiles_n count those), all of K <= 64 at once.
+bool gemm_panel_eligible(const GemmLaunch &g, int amode, int bmode);
+int launch_gemm_panel(const GemmLaunch &g, int amode, int bmode);
 
 // Skinny (GEMV-shaped) products: X (MR x K, MR <= 16) against a large W.
 //   out[b](i, j) = sum_k X[b](i, k) * W[b](k, j),  i < rows, j < cols

@@ -23,7 +23,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmni_rocm.so")
 BAD_ID = 0xFFFFFFFF
 MAX_DIMS = 8
 EPI_NONE, EPI_BIAS, EPI_BIAS_RELU, EPI_BIAS_GELU = 0, 1, 2, 3
-ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL, ALGO_SKINNY_TWO_PASS, ALGO_MFMA_STREAMK, ALGO_DIRECT = 0, 1, 2, 3, 4, 5, 6
+ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL, ALGO_SKINNY_TWO_PASS, ALGO_MFMA_STREAMK, ALGO_DIRECT, ALGO_PANEL = 0, 1, 2, 3, 4, 5, 6, 7
 
 _f32p = C.POINTER(C.c_float)
 _i64p = C.POINTER(C.c_int64)
@@ -67,6 +67,8 @@ SIGNATURES = {
     "mni_rocm_event_destroy": (C.c_int, [C.c_void_p]),
     "mni_rocm_sgemm": (C.c_int, [C.POINTER(GemmDesc)]),
     "mni_rocm_sgemm_timed": (C.c_int, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
+    "mni_rocm_yardstick_timed": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_size_t, C.c_int, C.c_int,
+                                           C.c_int, C.POINTER(C.c_float)]),
     "mni_rocm_strided_copy": (C.c_int, [C.c_void_p, C.c_void_p, _i64p, _i64p, C.c_int]),
     "mni_rocm_add_bias": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
     "mni_rocm_colsum": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
@@ -270,6 +272,15 @@ class Rocm:
         d.split_k = split_k
         d.algo = algo
         return d
+
+    def yardstick_timed(self, kind, nbytes, dst=None, srcs=(), nontemporal=True, blocks_per_cu=8, warmup=5, iters=50):
+        """Average ms per launch of a streaming kernel: kind "empty", "read", "write" or "copy"."""
+        code = {"empty": 0, "read": 1, "write": 2, "copy": 3}[kind]
+        arr = (C.c_void_p * max(len(srcs), 1))(*srcs)
+        ms = C.c_float(0)
+        self._check(self.lib.mni_rocm_yardstick_timed(code, 1 if nontemporal else 0, dst, arr, len(srcs), nbytes, blocks_per_cu,
+                                                      warmup, iters, C.byref(ms)))
+        return ms.value
 
     def strided_copy(self, dst, src, shape, strides):
         self._check(self.lib.mni_rocm_strided_copy(dst, src, _i64_array(shape), _i64_array(strides), len(shape)))

@@ -114,9 +114,12 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * matrix instruction's registers; split_k 0 or 1 = one wavefront per tile,
  * split_k 4 = four wavefronts sharing K; error if the operand layouts are not
  * eligible: each operand contiguous along K with K % 4 == 0, or along M / N
- * with that extent even).  AUTO picks among them. */
+ * with that extent even); PANEL = the short-K kernel for two K-contiguous
+ * operands (A row-major, B given as its transpose; K <= 64, K % 4 == 0; error
+ * otherwise): 128 x 128 tiles, all of K at once, stores of one part of a tile
+ * under the MFMAs of the next.  AUTO picks among them. */
 enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
-       MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6 };
+       MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),
@@ -143,6 +146,20 @@ int mni_rocm_sgemm(const mni_gemm_desc *desc);
  * and returns the average milliseconds per launch.  Issuing from C keeps the
  * host ahead of kernels that take only a few microseconds. */
 int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms);
+
+/* Measurement aid (no counterpart in the reference): what the device gives a
+ * kernel that only streams.  `iters` launches between two HIP events on the
+ * library's stream after `warmup` untimed ones; the average milliseconds per
+ * launch is returned.  EMPTY: a one-wavefront kernel that does nothing (the
+ * cost of a launch in a back-to-back sequence).  READ: `bytes` bytes of
+ * srcs[launch % nsrc] are read with 16-byte loads, 8 in flight per lane, and
+ * nothing is written (several sources in rotation make the pass cold in the
+ * last-level cache).  WRITE: `bytes` bytes of dst are written.  COPY: both.
+ * `nontemporal` selects streaming loads / stores; the grid is blocks_per_cu
+ * workgroups of 256 threads per compute unit.  Sizes are multiples of 16. */
+enum { MNI_YARDSTICK_EMPTY = 0, MNI_YARDSTICK_READ = 1, MNI_YARDSTICK_WRITE = 2, MNI_YARDSTICK_COPY = 3 };
+int mni_rocm_yardstick_timed(int kind, int nontemporal, void *dst, const void *const *srcs, int nsrc, size_t bytes,
+                             int blocks_per_cu, int warmup, int iters, float *avg_ms);
 
 /* dst (contiguous, `shape`) = gather of src by `src_strides` (elements).
  * Replaces permute_f32 (src/native/kernels/elementwise.cu:67-81) and the host

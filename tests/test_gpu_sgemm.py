@@ -347,6 +347,122 @@ def test_streamk_is_refused_where_it_cannot_work(dev, rocm):
 
 # ---- skinny kernels ----------------------------------------------------------------
 
+# ---- register-direct kernel (batched products of many small tiles) ------------------------------
+
+DIRECT_SHAPES = [(64, 64, 64), (512, 512, 64), (130, 70, 64), (100, 64, 512), (64, 200, 520), (34, 36, 36), (2, 2, 4),
+                 (192, 128, 128), (66, 130, 1000)]
+
+
+@pytest.mark.parametrize("m,n,k", DIRECT_SHAPES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("parts", [1, 4])
+def test_direct_integer_exact_all_layouts(dev, m, n, k, ta, tb, parts):
+    # every extent is even and K a multiple of 4, so all four layouts are eligible; edges inside tiles,
+    # K tails inside phases, wavefronts without any K of their own (K = 4 split four ways)
+    a = synth.small_ints(m + k, (3, k, m) if ta else (3, m, k), 4)
+    b = synth.small_ints(n + k, (3, n, k) if tb else (3, k, n), 4, stream=1)
+    got = run_gemm(dev, a, b, ta, tb, algo=N.ALGO_DIRECT, split_k=parts)
+    A = a.transpose(0, 2, 1) if ta else a
+    B = b.transpose(0, 2, 1) if tb else b
+    assert np.array_equal(got, np.einsum("bmk,bkn->bmn", A.astype(np.int64), B.astype(np.int64)).astype(np.float32))
+
+
+@pytest.mark.parametrize("parts", [1, 4])
+def test_direct_odd_extents_where_the_layout_allows(dev, parts):
+    # an operand that is contiguous along K may have any number of rows
+    a = synth.small_ints(1, (77, 40), 4)
+    bt = synth.small_ints(2, (51, 40), 4, stream=1)
+    got = run_gemm(dev, a, bt, False, True, algo=N.ALGO_DIRECT, split_k=parts)[0]
+    assert np.array_equal(got, (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float32))
+
+
+@pytest.mark.parametrize("parts", [1, 4])
+def test_direct_normal_inputs_batch_rule_epilogue_accumulate(dev, rocm, oracle_native, parts):
+    a = synth.normal(1, (6, 96, 200))
+    w = synth.normal(2, (2, 200, 72), stream=1)   # batch b reads w[b % 2]
+    bias = synth.normal(3, (72,), stream=2)
+    c0 = synth.normal(4, (6, 96, 72), stream=3)
+    dA, dW, dbias, dC = dev.put(a), dev.put(w), dev.put(bias), dev.put(c0)
+    rocm.sgemm(96, 72, 200, dA, dW, dC, batch=6, a_batch=(96 * 200, 6), b_batch=(200 * 72, 2), bias=dbias,
+               epilogue=N.EPI_BIAS_RELU, accumulate=True, algo=N.ALGO_DIRECT, split_k=parts)
+    got = rocm.to_host(dC, (6, 96, 72))
+    for b in range(6):
+        want = np.maximum(oracle_native.sgemm_ikj(a[b], w[b % 2]) + bias, 0) + c0[b]
+        assert max_err(got[b], want) <= gemm_tol(200, a, w)
+
+
+def test_direct_is_refused_for_layouts_it_cannot_read(dev, rocm):
+    a, b = synth.small_ints(1, (64, 30), 3), synth.small_ints(2, (30, 64), 3, stream=1)
+    dA, dB, dC = dev.put(a), dev.put(b), dev.empty(64 * 64)
+    with pytest.raises(N.MniError, match="not eligible for the direct kernel"):
+        rocm.sgemm(64, 64, 30, dA, dB, dC, algo=N.ALGO_DIRECT)  # A contiguous along K, K % 4 != 0
+    with pytest.raises(N.MniError, match="split_k 0, 1 or 4"):
+        rocm.sgemm(64, 64, 28, dA, dB, dC, a_strides=(30, 1), algo=N.ALGO_DIRECT, split_k=3)
+    with pytest.raises(N.MniError, match="not eligible for the direct kernel"):
+        rocm.sgemm(64, 64, 15, dA, dB, dC, a_strides=(2, 128), algo=N.ALGO_DIRECT)  # neither axis contiguous
+
+
+# ---- short-K panel kernel (two K-contiguous operands, all of K at once) ---------------------------
+
+@pytest.mark.parametrize("m,n,k,batch", [(128, 128, 64, 1), (512, 512, 64, 3), (200, 150, 64, 2), (130, 257, 48, 1), (64, 40, 32, 2),
+                                         (300, 129, 20, 1), (1, 1, 4, 1), (129, 3, 36, 1)])
+def test_panel_integer_exact(dev, m, n, k, batch):
+    # edges inside tiles (rows beyond them re-read the last row), K below the kernel's 32 / 64 (zero quads)
+    a = synth.small_ints(m + k, (batch, m, k), 4)
+    bt = synth.small_ints(n + k, (batch, n, k), 4, stream=1)
+    got = run_gemm(dev, a, bt, False, True, algo=N.ALGO_PANEL)
+    assert np.array_equal(got, np.einsum("bmk,bnk->bmn", a.astype(np.int64), bt.astype(np.int64)).astype(np.float32))
+
+
+def test_panel_normal_inputs_batch_rule_epilogue_accumulate(dev, rocm, oracle_native):
+    a = synth.normal(1, (5, 140, 64))
+    wt = synth.normal(2, (2, 136, 64), stream=1)   # batch b reads wt[b % 2]
+    bias = synth.normal(3, (136,), stream=2)
+    c0 = synth.normal(4, (5, 140, 136), stream=3)
+    for epi, f in ((N.EPI_NONE, lambda z: z), (N.EPI_BIAS_RELU, lambda z: np.maximum(z + bias, 0))):
+        dA, dW, dbias, dC = dev.put(a), dev.put(wt), dev.put(bias), dev.put(c0)
+        rocm.sgemm(140, 136, 64, dA, dW, dC, batch=5, a_batch=(140 * 64, 5), b_strides=(1, 64), b_batch=(136 * 64, 2),
+                   bias=dbias if epi else None, epilogue=epi, accumulate=True, algo=N.ALGO_PANEL)
+        got = rocm.to_host(dC, (5, 140, 136))
+        for b in range(5):
+            want = f(oracle_native.sgemm_ikj(a[b], wt[b % 2].T.copy())) + c0[b]
+            assert max_err(got[b], want) <= gemm_tol(64, a, wt)
+
+
+def test_panel_is_refused_for_shapes_it_cannot_take(dev, rocm):
+    a, b = synth.small_ints(1, (64, 68), 3), synth.small_ints(2, (68, 64), 3, stream=1)
+    dA, dB, dC = dev.put(a), dev.put(b), dev.empty(64 * 64)
+    with pytest.raises(N.MniError, match="short-K panel kernel takes two K-contiguous operands"):
+        rocm.sgemm(64, 64, 68, dA, dB, dC, b_strides=(1, 68), algo=N.ALGO_PANEL)   # K > 64
+    with pytest.raises(N.MniError, match="short-K panel kernel takes two K-contiguous operands"):
+        rocm.sgemm(64, 64, 64, dA, dB, dC, a_strides=(68, 1), algo=N.ALGO_PANEL)   # B contiguous along N
+    with pytest.raises(N.MniError, match="no split_k"):
+        rocm.sgemm(64, 64, 64, dA, dB, dC, a_strides=(68, 1), b_strides=(1, 68), algo=N.ALGO_PANEL, split_k=2)
+
+
+def test_planner_sends_attention_shaped_products_to_the_new_kernels(dev, rocm):
+    # scores (short K, both operands K-contiguous) and the two backward products (one workgroup per CU,
+    # long thin operand) at a size where the planner picks the panel / direct kernels by itself; the
+    # results must be the forced kernels' bits
+    q = synth.normal(1, (16, 512, 64), 0.125)
+    ds = synth.normal(2, (16, 512, 512), stream=1)
+    dQ, dS = dev.put(q), dev.put(ds)
+    outs = []
+    for algo, split in ((N.ALGO_AUTO, 0), (N.ALGO_PANEL, 0)):
+        dC = dev.empty(16 * 512 * 512)
+        rocm.sgemm(512, 512, 64, dQ, dQ, dC, batch=16, a_batch=(512 * 64, 16), b_strides=(1, 64), b_batch=(512 * 64, 16), algo=algo, split_k=split)
+        outs.append(rocm.to_host(dC, (16, 512, 512)))
+    assert np.array_equal(outs[0], outs[1])
+    assert max_err(outs[0][3], q[3].astype(np.float64) @ q[3].T.astype(np.float64)) <= gemm_tol(64, q, q)
+    outs = []
+    for algo, split in ((N.ALGO_AUTO, 0), (N.ALGO_DIRECT, 4)):
+        dC = dev.empty(16 * 512 * 64)
+        rocm.sgemm(512, 64, 512, dS, dQ, dC, batch=16, a_batch=(512 * 512, 16), b_batch=(512 * 64, 16), algo=algo, split_k=split)
+        outs.append(rocm.to_host(dC, (16, 512, 64)))
+    assert np.array_equal(outs[0], outs[1])
+    assert max_err(outs[0][5], ds[5].astype(np.float64) @ q[5].astype(np.float64)) <= gemm_tol(512, ds, q)
+
+
 def test_single_launch_skinny_path_is_available(rocm):
     # MI355X deals workgroups over its 8 XCDs round-robin; were the probe to fail,
     # ALGO_SKINNY would quietly run as ALGO_SKINNY_TWO_PASS and the tests below
