@@ -56,6 +56,9 @@ struct DeviceCtx {
     // block of `scratch_bytes` (the entry point that must not allocate).
     float *scratch = nullptr;
     size_t scratch_bytes = 0;
+    // Device address and size of the library's static workspace (see device.hip).
+    float *noalloc_scratch = nullptr;
+    size_t noalloc_scratch_bytes = 0;
 };
 enum { DEVICE_STATUS_OK = 0, DEVICE_STATUS_STREAMK_WAIT = 1, DEVICE_STATUS_SKINNY_WAIT = 2 };
 // hipStreamSynchronize on the library's stream, then the device status word:

@@ -34,6 +34,15 @@ DeviceCtx &ctx() {
     return c;
 }
 
+// Workspace of mni_rocm_sgemm_noalloc, the entry point for callers that cannot
+// allocate: the K-slice / stream-K partial sums of one product.  Part of the
+// code object, so the device holds it from the moment the library is loaded
+// until the process ends.  On the host this name is only a handle for
+// hipGetSymbolAddress; the device address is looked up once in init_device and
+// kept in the device context, and that address is what kernels are given.
+static constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)32 << 20;
+static __device__ __align__(256) float scratch[NOALLOC_SCRATCH_BYTES / sizeof(float)];
+
 // Which XCD a workgroup runs on: the hardware id, read by one lane.
 __global__ void xcc_probe_kernel(unsigned *out) {
     if (threadIdx.x == 0) {
@@ -99,6 +108,11 @@ static int init_device(int device) {
     MNI_HIP_CHECK(hipHostMalloc((void **)&c.status_host, 64, hipHostMallocMapped));
     memset(c.status_host, 0, 64);
     MNI_HIP_CHECK(hipHostGetDevicePointer((void **)&c.status_dev, c.status_host, 0));
+    // Device address of the static workspace on this device (the library drives one device).
+    float *scratch_ptr = nullptr;
+    MNI_HIP_CHECK(hipGetSymbolAddress((void **)&scratch_ptr, HIP_SYMBOL(scratch)));
+    c.noalloc_scratch = scratch_ptr;
+    c.noalloc_scratch_bytes = NOALLOC_SCRATCH_BYTES;
     c.ready = true;
     return MNI_OK;
 }
@@ -286,6 +300,24 @@ int mni_rocm_sync(void) {
     MNI_TRY(ensure_init());
     return sync_stream_checked("sync");
 }
+
+int mni_rocm_sgemm_noalloc(const mni_gemm_desc *desc) {
+    MNI_API_GUARD;
+    if (!desc) return set_error(MNI_ERR_INVALID, "sgemm_noalloc: null descriptor");
+    DeviceCtx &c = ctx();
+    // Initialisation allocates (stream, flag array); this call must not, so it does not initialise.
+    if (!c.ready || !c.noalloc_scratch)
+        return set_error(MNI_ERR_INVALID, "sgemm_noalloc: call mni_rocm_init first (this entry point allocates nothing, "
+                                          "initialisation does)");
+    c.scratch = c.noalloc_scratch;
+    c.scratch_bytes = c.noalloc_scratch_bytes;
+    const int rc = sgemm(*desc);
+    c.scratch = nullptr;
+    c.scratch_bytes = 0;
+    return rc;
+}
+
+size_t mni_rocm_sgemm_noalloc_workspace_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
 
 int mni_rocm_test_raise_device_status(unsigned code) {
     MNI_API_GUARD;

@@ -66,6 +66,8 @@ SIGNATURES = {
     "mni_rocm_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "mni_rocm_event_destroy": (C.c_int, [C.c_void_p]),
     "mni_rocm_sgemm": (C.c_int, [C.POINTER(GemmDesc)]),
+    "mni_rocm_sgemm_noalloc": (C.c_int, [C.POINTER(GemmDesc)]),
+    "mni_rocm_sgemm_noalloc_workspace_bytes": (C.c_size_t, []),
     "mni_rocm_sgemm_timed": (C.c_int, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
     "mni_rocm_yardstick_timed": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_size_t, C.c_int, C.c_int,
                                            C.c_int, C.POINTER(C.c_float)]),
@@ -245,6 +247,14 @@ class Rocm:
         element strides of op(A) (M x K) and op(B) (K x N); default row-major."""
         d = self.gemm_desc(M, N, K, A, B, Cptr, **kw)
         self._check(self.lib.mni_rocm_sgemm(C.byref(d)))
+
+    def sgemm_noalloc(self, M, N, K, A, B, Cptr, **kw):
+        """sgemm with the plan's workspace taken from the library's fixed block: no allocation during the call."""
+        d = self.gemm_desc(M, N, K, A, B, Cptr, **kw)
+        self._check(self.lib.mni_rocm_sgemm_noalloc(C.byref(d)))
+
+    def sgemm_noalloc_workspace_bytes(self):
+        return int(self.lib.mni_rocm_sgemm_noalloc_workspace_bytes())
 
     def sgemm_timed(self, descs, warmup, iters):
         """Average ms per launch of the products in `descs` (made by gemm_desc),

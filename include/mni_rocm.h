@@ -140,6 +140,23 @@ typedef struct {
     int32_t algo;        /* MNI_ALGO_*                                      */
 } mni_gemm_desc;
 int mni_rocm_sgemm(const mni_gemm_desc *desc);
+/* The same product for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  Identical kernels, plans and results as
+ * mni_rocm_sgemm, but the partial sums of a split-K, stream-K or skinny plan
+ * go to a fixed 32 MiB workspace that is part of the library's code object
+ * instead of a block from the caching allocator, and nothing is allocated or
+ * freed during the call.  Requires a prior mni_rocm_init (initialisation
+ * allocates; this call refuses to initialise).  A product whose plan needs
+ * more than mni_rocm_sgemm_noalloc_workspace_bytes() fails with
+ * MNI_ERR_INVALID and a message giving both sizes (every plan the library
+ * chooses by itself fits; an explicit split_k over a large C may not).  All
+ * calls share the one workspace: they are ordered on the library's stream,
+ * so they do not race with each other, but the workspace keeps the last
+ * call's partials and two processes' or two libraries' calls on the same
+ * device memory would.  Nothing in it needs to start at zero. */
+int mni_rocm_sgemm_noalloc(const mni_gemm_desc *desc);
+size_t mni_rocm_sgemm_noalloc_workspace_bytes(void);
 /* Measurement aid (no counterpart in the reference): runs descs[0], descs[1],
  * ... descs[count-1], descs[0], ... back to back on the library's stream,
  * `warmup` untimed launches and then `iters` launches between two HIP events,
