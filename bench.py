@@ -17,10 +17,14 @@ One JSON line is printed:
 * cpu_baseline  the CPU oracle (a C restatement of the reference's
               single-threaded CPU backend) timed on this host on a bounded
               sample of the same product (the first 2048 rows of A);
-* extra       the other configurations of the path, for information: the
-              decode-shaped GEMV against HBM bandwidth, the tall-K weight
-              gradient, attention-shaped batched products, and the README-MLP
-              and FFN training steps in ms.
+* extra       the other configurations of the path, each with its own
+              `roofline` (algorithmic flops / bytes against the roof that
+              bounds it) and `cpu_baseline` (the oracle on a bounded sample):
+              the decode-shaped GEMV against HBM bandwidth (cold first), the
+              tall-K weight gradient, the three attention-shaped batched
+              products, the README-MLP step (launches per step) and the FFN
+              training step; plus what this device gives a kernel that only
+              streams (read / write / copy yardsticks, an empty launch).
 
 Only one GPU is used; --gpus above 1 is refused.
 """
@@ -42,10 +46,20 @@ from framework_amd import native as N  # noqa: E402
 PEAK_FP32_MATRIX_TFLOPS = 157.3  # MI355X dense fp32 MFMA: 256 CU x 256 FLOP/clk x 2.4 GHz
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per gemm_mfma_kernel launch at 4096^3, from the rocprofv3 --pmc
-# runs summarised in profiles/gemm_mfma_4096_pmc.txt (FETCH_SIZE + WRITE_SIZE,
-# scaled by a copy kernel of known size).  None until measured.
-MEASURED_HBM_BYTES_4096 = 797.2e6
+SETTLE_LAUNCHES = 25  # untimed launches ahead of the --warmup steps (see bench_headline)
+
+
+def profile_traffic(name):
+    """HBM-side bytes per launch of a kernel as its committed rocprofv3 --pmc summary under profiles/ states them
+    (FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a copy kernel of known size): the
+    line `traffic = <x> MB`.  None when the summary is absent."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic = ([0-9.]+) MB", text)
+    return float(m.group(1)) * 1e6 if m else None
 
 
 def time_launches(r, fn, warmup, iters):
@@ -72,7 +86,7 @@ def bench_headline(r, steps, warmup):
     step = lambda: r.sgemm(M, Nn, K, dA, dB, dC)
     # The uploads above leave the GPU idle, and its clocks need ~20 ms of work to settle
     # (the first launches after an idle spell run 10 % slow): settle first, then the W warm-up steps.
-    for _ in range(25):
+    for _ in range(SETTLE_LAUNCHES):
         step()
     for _ in range(warmup):
         step()
@@ -95,61 +109,166 @@ def bench_headline(r, steps, warmup):
     return wall_ms, kernel_ms, 2.0 * M * Nn * K, (a, b), err
 
 
-def bench_extras(r):
-    out = {}
-    # config 5a: decode-shaped GEMV x[4,4096] W[4096,4096], HBM-bound
+def roofline(bound, kernel, seconds, flops, nbytes, traffic=None):
+    """Roofline object of one kernel launch (or one step): algorithmic flops and bytes against the datasheet
+    peaks; `frac` is taken against the roof that bounds the work."""
+    tf, gb = flops / seconds / 1e12, nbytes / seconds / 1e9
+    out = {"bound": bound, "kernel": kernel, "us": seconds * 1e6, "algorithmic_flops": flops, "algorithmic_bytes": nbytes,
+           "TFLOP/s": tf, "GB/s": gb, "frac_mfma": tf / PEAK_FP32_MATRIX_TFLOPS, "frac_hbm": gb / PEAK_HBM_GBPS, "traffic": traffic}
+    if bound == "mfma":
+        out.update(achieved=tf, peak=PEAK_FP32_MATRIX_TFLOPS, unit="TFLOP/s", frac=tf / PEAK_FP32_MATRIX_TFLOPS)
+    else:
+        out.update(achieved=gb, peak=PEAK_HBM_GBPS, unit="GB/s", frac=gb / PEAK_HBM_GBPS)
+    return out
+
+
+def oracle_api():
+    from framework_amd.api import bind
+    from oracle.native import OracleNative
+    orc = bind(OracleNative())
+    orc.native.resetEngine()
+    return orc
+
+
+def cpu_time(fn, reps=1):
+    """Wall clock of fn() on this host (the oracle is single-threaded), best of `reps`."""
+    best = None
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return best
+
+
+def cpu_note(sample):
+    return {"cores": 1, "kind": "port", "sample": sample + "; oracle/mni_oracle.c (-O3 -ffp-contract=off, no -march=native), "
+            "1 of %d logical cores" % (os.cpu_count() or 0)}
+
+
+def bench_yardsticks(r):
+    """What the device gives a kernel that only streams, measured in this run: the figures the bandwidth-bound
+    rows below are to be read against, next to the datasheet's 8 TB/s."""
+    MB = 1 << 20
+    bufs = [r.malloc(64 * MB) for _ in range(9)]
+    for b in bufs:
+        r.fill(b, 1.0, 16 * MB)
+    out = {"empty_launch_us": r.yardstick_timed("empty", 0, iters=500) * 1e3}
+
+    def line(ms, nbytes):
+        return {"us": ms * 1e3, "GB/s": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBPS}
+    n = 64 * MB
+    out["hbm_read_yardstick_warm"] = dict(line(r.yardstick_timed("read", n, srcs=bufs[:1], iters=200), n),
+                                          note="the same 64 MiB every launch: served by the 256 MiB Infinity Cache")
+    out["hbm_read_yardstick_cold"] = dict(line(r.yardstick_timed("read", n, srcs=bufs[:8], iters=200), n),
+                                          note="eight 64 MiB buffers in rotation (512 MiB working set): served by HBM")
+    out["hbm_write_yardstick_32MiB"] = line(r.yardstick_timed("write", 32 * MB, dst=bufs[8], iters=200), 32 * MB)
+    out["hbm_copy_yardstick_64MiB"] = line(r.yardstick_timed("copy", n, dst=bufs[8], srcs=bufs[:1], iters=100), 2 * n)
+    for b in bufs:
+        r.free(b)
+    return out
+
+
+def bench_extras(r, with_cpu):
+    out = bench_yardsticks(r)
+    # ---- config 5a: decode-shaped GEMV x[4,4096] W[4096,4096], HBM-bound --------------------------------------
     x = synth.normal(4, (4, 4096), 0.02)
     w = synth.normal(4, (4096, 4096), 0.02, stream=1)
     dx, dw, dy = r.to_device(x), r.to_device(w), r.malloc(4 * 4096 * 4)
-    # launches of a few microseconds are issued from C (mni_rocm_sgemm_timed) so that the host stays ahead
-    ms = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 10, 200)
     by = 4.0 * (4096 * 4096 + 2 * 4 * 4096)
-    out["config5a_gemv"] = {"us": ms * 1e3, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / PEAK_HBM_GBPS,
-                            "note": "W (64 MiB) is re-read every launch and fits the 256 MiB Infinity Cache"}
-    # the same after 3000 launches (~40 ms) of it: memory-bound work runs ~5 % slower once the part has been
-    # streaming for a while than in a short burst
-    ms = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 3000, 1000)
-    out["config5a_gemv_sustained"] = {"us": ms * 1e3, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / PEAK_HBM_GBPS}
-    # the same product over 8 different W in turn (512 MiB working set): HBM-resident
+    fl = 2.0 * 4 * 4096 * 4096
+    kern = "skinny_cols_kernel<4, true, true, false, true>"
+    # launches of a few microseconds are issued from C (mni_rocm_sgemm_timed) so that the host stays ahead
     ws = [r.to_device(w) for _ in range(8)]
-    ms = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, p, dy) for p in ws], 16, 200)
-    out["config5a_gemv_cold"] = {"us": ms * 1e3, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / PEAK_HBM_GBPS}
+    ms_cold = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, p, dy) for p in ws], 16, 200)
+    ms_warm = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 10, 200)
+    ms_sus = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 3000, 1000)
+    got = r.to_host(dy, (4, 4096))
+    c5a = {"roofline": dict(roofline("hbm", kern, ms_cold * 1e-3, fl, by, traffic=profile_traffic("skinny_gemv_4x4096x4096.txt")),
+                            note="cold: eight different W in rotation (512 MiB working set), every byte comes from HBM"),
+           "warm": dict(roofline("hbm", kern, ms_warm * 1e-3, fl, by),
+                        note="the same W (64 MiB) every launch: it stays in the 256 MiB Infinity Cache, so this is not an HBM figure"),
+           "warm_sustained": dict(roofline("hbm", kern, ms_sus * 1e-3, fl, by), note="the same after 3000 launches (~40 ms) of it"),
+           "vs_read_yardstick": {"cold": out["hbm_read_yardstick_cold"]["us"] / (ms_cold * 1e3),
+                                 "warm": out["hbm_read_yardstick_warm"]["us"] / (ms_warm * 1e3),
+                                 "note": "time of a pure read of the same 64 MiB / time of the product"}}
+    if with_cpu:
+        orc = oracle_api()
+        X, W = orc.Tensor.fromFloat32(x, [4, 4096]), orc.Tensor.fromFloat32(w, [4096, 4096])
+        res = []
+        dt = cpu_time(lambda: res.append(X.matmul(W)), reps=3)
+        ref = res[-1].numpy()
+        c5a["max_err_vs_oracle"] = float(np.max(np.abs(got.astype(np.float64) - ref)))
+        c5a["cpu_baseline"] = dict(cpu_note("the whole product, best of 3"), value=dt * 1e3, unit="ms", **{"GB/s": by / dt / 1e9})
+        orc.native.resetEngine()
+    out["config5a_gemv"] = c5a
     for p in ws + [dx, dw, dy]:
         r.free(p)
-    # config 5b: X^T[1024,65536] dY[65536,1024], X^T as a view, split-K
+    # ---- config 5b: X^T[1024,65536] dY[65536,1024], X^T as a view, split-K -------------------------------------
     X = synth.normal(5, (65536, 1024))
     dX, dG, dO = r.to_device(X), r.to_device(X), r.malloc(1024 * 1024 * 4)
     # (30 launches of warm-up: the upload above leaves the GPU idle and its clocks take ~20 ms to settle)
     ms = time_launches(r, lambda: r.sgemm(1024, 1024, 65536, dX, dG, dO, a_strides=(1, 1024)), 30, 20)
     fl = 2.0 * 1024 * 1024 * 65536
-    out["config5b_tall_k"] = {"us": ms * 1e3, "TFLOP/s": fl / ms / 1e9, "frac_mfma": fl / ms / 1e9 / PEAK_FP32_MATRIX_TFLOPS}
+    by = 4.0 * (2 * 65536 * 1024 + 1024 * 1024)
+    c5b = {"roofline": roofline("mfma", "gemm_mfma_kernel<1, 1, 2, 2, false> + splitk_reduce_kernel", ms * 1e-3, fl, by)}
+    if with_cpu:
+        rows = 8192  # an eighth of K: the oracle gathers X^T into a contiguous copy, then runs its i-k-j loop
+        orc = oracle_api()
+        Xs = orc.Tensor.fromFloat32(X[:rows], [rows, 1024])
+        dt = cpu_time(lambda: Xs.permute(1, 0).matmul(Xs))
+        c5b["cpu_baseline"] = dict(cpu_note("the first %d of 65536 K rows (%.1f GFLOP), gather of the transposed view included" % (rows, 2.0 * 1024 * 1024 * rows / 1e9)),
+                                   value=2.0 * 1024 * 1024 * rows / dt / 1e12, unit="TFLOP/s", seconds=dt)
+        orc.native.resetEngine()
+    out["config5b_tall_k"] = c5b
     for p in (dX, dG, dO):
         r.free(p)
     del X
-    # config 3: Q K^T (K^T a permuted view), dQ, dK^T -- batched, near the ridge
+    # ---- config 3: Q K^T (K^T a permuted view), dQ, dK^T -- batched, near the ridge -------------------------------
     q = synth.normal(2, (32, 512, 64)) / np.float32(8)
+    kk = synth.normal(2, (32, 512, 64), stream=1) / np.float32(8)
     ds = synth.normal(2, (32, 512, 512), stream=2)
-    dq, dk, dds = r.to_device(q), r.to_device(q), r.to_device(ds)
+    dq, dk, dds = r.to_device(q), r.to_device(kk), r.to_device(ds)
     s_out, g_out = r.malloc(32 * 512 * 512 * 4), r.malloc(32 * 512 * 64 * 4)
     fl = 2.0 * 32 * 512 * 512 * 64
-    ms_f = r.sgemm_timed([r.gemm_desc(512, 512, 64, dq, dk, s_out, batch=32, a_batch=(512 * 64, 32),
-                                      b_strides=(1, 64), b_batch=(512 * 64, 32))], 5, 100)
-    ms_q = r.sgemm_timed([r.gemm_desc(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32),
-                                      b_batch=(512 * 64, 32))], 5, 100)
-    ms_k = r.sgemm_timed([r.gemm_desc(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64),
-                                      a_batch=(512 * 64, 32), b_batch=(512 * 512, 32))], 5, 100)
     by = 4.0 * 32 * (512 * 64 * 2 + 512 * 512)
-    out["config3_attention_scores"] = {
-        "fwd_us": ms_f * 1e3, "dq_us": ms_q * 1e3, "dkT_us": ms_k * 1e3,
-        "TFLOP/s": 3 * fl / (ms_f + ms_q + ms_k) / 1e9, "GB/s": 3 * by / (ms_f + ms_q + ms_k) / 1e6}
+    prods = [("scores", "gemm_panel_kernel<8>", r.gemm_desc(512, 512, 64, dq, dk, s_out, batch=32, a_batch=(512 * 64, 32),
+                                                             b_strides=(1, 64), b_batch=(512 * 64, 32))),
+             ("dQ", "gemm_direct_kernel<0, 1, 4, 4>", r.gemm_desc(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32),
+                                                                  b_batch=(512 * 64, 32))),
+             ("dKT", "gemm_direct_kernel<1, 1, 4, 4>", r.gemm_desc(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64),
+                                                                   a_batch=(512 * 64, 32), b_batch=(512 * 512, 32)))]
+    c3 = {}
+    total = 0.0
+    for name, kern, desc in prods:
+        ms = r.sgemm_timed([desc], 10, 200)
+        total += ms
+        # each product moves 41.9 MB and 1.07 GFLOP: the matrix pipe needs 6.8 us for it, HBM 5.2 us
+        c3[name] = roofline("mfma", kern, ms * 1e-3, fl, by)
+    c3["roofline"] = dict(roofline("mfma", "the three products", total * 1e-3, 3 * fl, 3 * by),
+                          note="arithmetic intensity 25.6 flop/B against a ridge of 19.7: the matrix pipe bounds it (20.5 us for all "
+                               "three), HBM is close behind (15.7 us); an empty launch in the same sequence takes "
+                               "%.2f us" % out["empty_launch_us"])
+    if with_cpu:
+        nb = 2  # batches of the 32
+        orc = oracle_api()
+        Q = orc.Tensor.fromFloat32(q[:nb], [nb, 512, 64]).setRequiresGrad(True)
+        K = orc.Tensor.fromFloat32(kk[:nb], [nb, 512, 64]).setRequiresGrad(True)
+        G = orc.Tensor.fromFloat32(ds[:nb], [nb, 512, 512])
+        dt = cpu_time(lambda: Q.matmul(K.permute(0, 2, 1)).mul(G).sum().backward())
+        c3["cpu_baseline"] = dict(cpu_note("%d of 32 batches: forward through the permuted view, backward to dQ and dK (incl. the oracle's "
+                                           "transposes, clones and the mul/sum that seed the gradient)" % nb),
+                                  value=dt * 1e3 * 32 / nb, unit="ms (scaled to 32 batches)", seconds=dt)
+        orc.native.resetEngine()
+    out["config3_attention_scores"] = c3
     for p in (dq, dk, dds, s_out, g_out):
         r.free(p)
-    # configs 1 and 4: training steps through the engine (wall clock, trailing sync)
+    # ---- configs 1 and 4: training steps through the engine (wall clock, trailing sync) -------------------------
     from framework_amd.api import bind
     api = bind(N.Native())
 
-    def T(a, grad=False):
-        t = api.Tensor.fromFloat32(a, list(a.shape))
+    def T(a, grad=False, on=None):
+        t = (on or api).Tensor.fromFloat32(a, list(a.shape))
         return t.setRequiresGrad(True) if grad else t
 
     def time_step(step, keep, n, warm):
@@ -157,23 +276,30 @@ def bench_extras(r):
             step()
             api.native.gcTensors(keep())
         r.sync()
-        total = 0.0
+        total, launches = 0.0, 0
         for _ in range(n):
+            l0 = r.launch_count()
             t0 = time.perf_counter()
             step()
             r.sync()
             total += time.perf_counter() - t0
+            launches = r.launch_count() - l0
             api.native.gcTensors(keep())
-        return total * 1e3 / n
+        return total * 1e3 / n, launches
 
     # config 4: FFN step X[4096,1024] -> 4096 (GELU) -> 1024, reference mseLoss, fwd + bwd
+    d, h, rows = 1024, 4096, 4096
+    x4, t4 = synth.normal(3, (rows, d)), synth.normal(3, (rows, d), stream=3)
+    w1, w2 = synth.uniform(3, (d, h), -1 / 32, 1 / 32, stream=1), synth.uniform(3, (h, d), -1 / 64, 1 / 64, stream=2)
+    gemm_flops = 6 * 2.0 * rows * d * h
+    gemm_bytes = 4.0 * (2 * (rows * d + d * h + rows * h) + (rows * h + h * d + rows * d) + (rows * h + rows * d + h * d)
+                        + (rows * d + d * h + rows * h) + (rows * d + rows * h + d * h))  # operands + result of the six products
     for fused in (False, True):
         api.native.resetEngine()
-        d, h, rows = 1024, 4096, 4096
-        x = T(synth.normal(3, (rows, d)), True)
-        tg = T(synth.normal(3, (rows, d), stream=3))
-        l1 = api.Linear(d, h, weight=synth.uniform(3, (d, h), -1 / 32, 1 / 32, stream=1), bias=np.zeros(h, np.float32), fused=fused, activation="gelu")
-        l2 = api.Linear(h, d, weight=synth.uniform(3, (h, d), -1 / 64, 1 / 64, stream=2), bias=np.zeros(d, np.float32), fused=fused)
+        x = T(x4, True)
+        tg = T(t4)
+        l1 = api.Linear(d, h, weight=w1, bias=np.zeros(h, np.float32), fused=fused, activation="gelu")
+        l2 = api.Linear(h, d, weight=w2, bias=np.zeros(d, np.float32), fused=fused)
         params = l1.parameters() + l2.parameters()
 
         def step4():
@@ -187,29 +313,67 @@ def bench_extras(r):
                 if g is not None:
                     ids.append(g)
             return ids
-        ms = time_step(step4, keep4, 20, 15)  # 30 ms of warm-up: the clocks take tens of milliseconds to settle after an idle spell
+        ms, launches = time_step(step4, keep4, 20, 15)  # 30 ms of warm-up: the clocks take tens of milliseconds to settle after an idle spell
         out["config4_ffn_step" + ("_fused_linear" if fused else "")] = {
-            "ms": ms, "gemm_TFLOP/s_if_all_gemm": 6 * 2.0 * rows * d * h / ms / 1e9}
+            "ms": ms, "launches_per_step": launches,
+            "roofline": dict(roofline("mfma", "whole step (six gemm_mfma_kernel launches + elementwise)", ms * 1e-3, gemm_flops, gemm_bytes),
+                             note="flops and bytes of the six products only; the step's elementwise kernels add ~0.7 GB of traffic and no counted flops")}
+    if with_cpu:
+        rs = 256  # rows of the 4096
+        orc = oracle_api()
+        xo = T(x4[:rs], True, orc)
+        to = T(t4[:rs], False, orc)
+        o1 = orc.Linear(d, h, weight=w1, bias=np.zeros(h, np.float32))
+        o2 = orc.Linear(h, d, weight=w2, bias=np.zeros(d, np.float32))
+        dt = cpu_time(lambda: orc.mseLoss(o2.forward(o1.forward(xo).gelu()), to).backward())
+        out["config4_ffn_step"]["cpu_baseline"] = dict(cpu_note("the first %d of 4096 rows of X (%.1f GFLOP of the 206.2), forward + backward" % (rs, gemm_flops * rs / rows / 1e9)),
+                                                       value=gemm_flops * rs / rows / dt / 1e12, unit="TFLOP/s", seconds=dt,
+                                                       ms_scaled_to_4096_rows=dt * 1e3 * rows / rs)
+        orc.native.resetEngine()
     # config 1: README MLP step (32x10 -> 64 -> 3, cross-entropy, Adam): launch-latency bound
     api.native.resetEngine()
-    x1 = T(synth.uniform(0, (32, 10)))
-    m1 = api.Linear(10, 64, weight=synth.uniform(0, (10, 64), -0.316, 0.316, stream=1), bias=synth.uniform(0, (64,), -0.316, 0.316, stream=2))
-    m2 = api.Linear(64, 3, weight=synth.uniform(0, (64, 3), -0.125, 0.125, stream=3), bias=synth.uniform(0, (3,), -0.125, 0.125, stream=4))
-    params1 = m1.parameters() + m2.parameters()
+    c1 = dict(x=synth.uniform(0, (32, 10)), w1=synth.uniform(0, (10, 64), -0.316, 0.316, stream=1), b1=synth.uniform(0, (64,), -0.316, 0.316, stream=2),
+              w2=synth.uniform(0, (64, 3), -0.125, 0.125, stream=3), b2=synth.uniform(0, (3,), -0.125, 0.125, stream=4))
     targets = [[int(t)] for t in synth.integers(0, (32,), 0, 3, stream=5)]
-    opt = api.Adam(params1, lr=1e-3)
 
-    def step1():
-        opt.zeroGrad()
-        api.crossEntropyLoss(m2.forward(m1.forward(x1).relu()), targets).backward()
-        opt.step()
+    def build1(a):
+        x1 = T(c1["x"], False, a)
+        m1 = a.Linear(10, 64, weight=c1["w1"], bias=c1["b1"])
+        m2 = a.Linear(64, 3, weight=c1["w2"], bias=c1["b2"])
+        ps = m1.parameters() + m2.parameters()
+        opt = a.Adam(ps, lr=1e-3)
 
-    def keep1():
-        ids = [x1._id] + [p.value._id for p in params1]
-        ids += [g for g in (api.native.getGrad(p.value._id) for p in params1) if g is not None]
-        return ids
-    out["config1_readme_mlp_step"] = {"ms": time_step(step1, keep1, 20, 5)}
-    # attention on the batched GEMM at the config-3 shapes: flashAttention(q, k, v) [32, 512, 64], causal
+        def step():
+            opt.zeroGrad()
+            a.crossEntropyLoss(m2.forward(m1.forward(x1).relu()), targets).backward()
+            opt.step()
+
+        def keep():
+            ids = [x1._id] + [p.value._id for p in ps]
+            return ids + [g for g in (a.native.getGrad(p.value._id) for p in ps) if g is not None]
+        return step, keep
+    step1, keep1 = build1(api)
+    ms, launches = time_step(step1, keep1, 20, 5)
+    out["config1_readme_mlp_step"] = {"ms": ms, "launches_per_step": launches,
+                                      "roofline": {"bound": "launch latency", "kernel": "%d kernel launches + 2 small copies per step" % launches,
+                                                   "us_per_launch": ms * 1e3 / max(launches, 1), "empty_launch_us": out["empty_launch_us"],
+                                                   "algorithmic_flops": 0.16e6, "frac": None,
+                                                   "note": "0.16 MFLOP and < 0.1 MB per step: neither roof applies; the step is the sum of its launch "
+                                                           "latencies and of the host's own work per op"}}
+    if with_cpu:
+        orc = oracle_api()
+        so, ko = build1(orc)
+        for _ in range(3):
+            so()
+            orc.native.gcTensors(ko())
+        t0 = time.perf_counter()
+        for _ in range(50):
+            so()
+            orc.native.gcTensors(ko())
+        out["config1_readme_mlp_step"]["cpu_baseline"] = dict(cpu_note("the whole step, mean of 50 (through the same Python binding)"),
+                                                              value=(time.perf_counter() - t0) / 50 * 1e3, unit="ms")
+        orc.native.resetEngine()
+    # ---- "next" rows: attention on the batched GEMM shapes, KV-cache decode ---------------------------------------
     api.native.resetEngine()
     bh, s, d = 32, 512, 64
     qa, ka, va = (T(synth.normal(2, (bh, s, d), stream=i) / np.float32(8 if i < 2 else 1), True) for i in range(3))
@@ -218,17 +382,17 @@ def bench_extras(r):
     def keep_att():
         ids = [t._id for t in (qa, ka, va, wa)]
         return ids + [g for g in (api.native.getGrad(t._id) for t in (qa, ka, va)) if g is not None]
-    ms_fwd = time_step(lambda: api.flashAttention(qa, ka, va, 0.125, True), keep_att, 20, 5)
+    ms_fwd, _ = time_step(lambda: api.flashAttention(qa, ka, va, 0.125, True), keep_att, 20, 5)
 
     def att_step():
         api.native.zeroGrad([qa._id, ka._id, va._id])
         api.flashAttention(qa, ka, va, 0.125, True).mul(wa).sum().backward()
-    ms_all = time_step(att_step, keep_att, 20, 5)
+    ms_all, _ = time_step(att_step, keep_att, 20, 5)
     # the one-kernel forward on long sequences ([8, 8192, 64] and [16, 4096, 128], causal): useful flops = half of dense
     for lb, ls, ld in ((8, 8192, 64), (16, 4096, 128)):
         ql, kl, vl = (T(synth.normal(2, (lb, ls, ld), stream=i)) for i in range(3))
         keep_long = lambda: [ql._id, kl._id, vl._id] + keep_att()
-        ms_long = time_step(lambda: api.flashAttention(ql, kl, vl, 1.0 / math.sqrt(ld), True), keep_long, 10, 3)
+        ms_long, _ = time_step(lambda: api.flashAttention(ql, kl, vl, 1.0 / math.sqrt(ld), True), keep_long, 10, 3)
         out["attention_fwd_%dx%dx%d_causal" % (lb, ls, ld)] = {"ms": ms_long, "useful_TFLOP/s": 2.0 * lb * ls * ls * ld / ms_long / 1e9}
         api.native.gcTensors(keep_att())
     dense = 2.0 * bh * s * s * d  # one s x s x d product, mask not exploited
@@ -254,93 +418,9 @@ def bench_extras(r):
         r.sync()
         us = (time.perf_counter() - t0) / 20 * 1e6
         by = 2.0 * bsz * nh * (hist + 12) * hd * (1 if quantized else 4)
-        out["kv_decode_8x32x128_hist4096_" + ("int8" if quantized else "fp32")] = {"us": us, "GB/s": by / us / 1e3}
+        out["kv_decode_8x32x128_hist4096_" + ("int8" if quantized else "fp32")] = {"us": us, "GB/s": by / us / 1e3, "frac_hbm": by / us / 1e3 / PEAK_HBM_GBPS}
         cache.free()
         api.native.gcTensors([])
-    # language-model training step: 2 blocks of width 768 (12 heads), 8 x 512 tokens, vocabulary 8192;
-    # dataset windows, embeddings, dropout, attention, residual + layernorm, GELU MLP, cross-entropy on
-    # buffered targets, clipped AdamW -- everything device-resident
-    api.native.resetEngine()
-    nat = api.native
-    V, D, H, Tn, Bn, L = 8192, 768, 12, 512, 8, 2
-    hd_ = D // H
-    nat.seed(1)
-    u = lambda seed, shape, b: synth.uniform(seed, shape, -b, b)
-    lin = lambda sd, i, o, act=None: api.Linear(i, o, weight=u(sd, (i, o), 1 / math.sqrt(i)), bias=np.zeros(o, np.float32), fused=True, activation=act)
-    tok, pos = api.Embedding(V, D, weight=u(1, (V, D), 0.05)), api.Embedding(Tn, D, weight=u(2, (Tn, D), 0.05))
-    layers = [dict(q=lin(10 + l, D, D), k=lin(20 + l, D, D), v=lin(30 + l, D, D), proj=lin(40 + l, D, D), fc=lin(50 + l, D, 4 * D, "gelu"),
-                   out=lin(60 + l, 4 * D, D), g1=api.Parameter(T(np.ones(D, np.float32), True)), b1=api.Parameter(T(np.zeros(D, np.float32), True)),
-                   g2=api.Parameter(T(np.ones(D, np.float32), True)), b2=api.Parameter(T(np.zeros(D, np.float32), True))) for l in range(L)]
-    head = lin(3, D, V)
-    lm_params = [tok.weight, pos.weight] + head.parameters()
-    for ly in layers:
-        for kname in ("q", "k", "v", "proj", "fc", "out"):
-            lm_params += ly[kname].parameters()
-        lm_params += [ly["g1"], ly["b1"], ly["g2"], ly["b2"]]
-    lm_opt = api.Adam(lm_params, lr=1e-3)
-    ds = nat.createDataset((np.arange(1 << 20, dtype=np.int64) * 2654435761 % V).astype(np.int32))
-    posidx = [list(range(Tn))] * Bn
-    heads = lambda t: t.view(Bn, Tn, H, hd_).permute(0, 2, 1, 3).contiguous().view(Bn * H, Tn, hd_)
-
-    def lm_step():
-        inp, tgt = nat.sampleBatch(ds, Tn, Bn)
-        h = api.dropout(tok.forwardGpu(inp, Bn, Tn).add(pos.forward(posidx)), 0.1)
-        for ly in layers:
-            att = api.flashAttention(heads(ly["q"].forward(h)), heads(ly["k"].forward(h)), heads(ly["v"].forward(h)), 1 / math.sqrt(hd_), True)
-            att = att.view(Bn, H, Tn, hd_).permute(0, 2, 1, 3).contiguous().view(Bn, Tn, D)
-            h1 = api.residualLayerNorm(api.dropout(ly["proj"].forward(att), 0.1), h, ly["g1"].value, ly["b1"].value)
-            h = api.residualLayerNorm(api.dropout(ly["out"].forward(ly["fc"].forward(h1)), 0.1), h1, ly["g2"].value, ly["b2"].value)
-        loss = api.crossEntropyLossGpu(head.forward(h), tgt)
-        lm_opt.zeroGrad()
-        loss.backward()
-        lm_opt.step(1.0)
-        nat.freeIntBuffer(inp)
-        nat.freeIntBuffer(tgt)
-
-    def keep_lm():
-        ids = [p.value._id for p in lm_params]
-        return ids + [g for g in (nat.getGrad(p.value._id) for p in lm_params) if g is not None]
-    ms = time_step(lm_step, keep_lm, 15, 6)
-    per_tok = 6.0 * (L * 12 * D * D + D * V) + L * 3.5 * 4 * Tn * D  # matmul FLOPs per token, fwd + bwd (attention counted dense)
-    out["lm_step_2x768_8x512_vocab8192"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3, "matmul_TFLOP/s": per_tok * Bn * Tn / ms / 1e9}
-    # token-side kernels on their own (wall clock per call incl. host issue; bytes = algorithmic)
-    api.native.resetEngine()
-    xt, rt = T(synth.normal(7, (8192, 768))), T(synth.normal(7, (8192, 768), stream=1))
-    gm, bt = T(np.ones(768, np.float32)), T(np.zeros(768, np.float32))
-    wemb = T(u(8, (32768, 768), 0.05), True)
-    idx = np.asarray(synth.integers(9, (8192,), 0, 32768), dtype=np.int64)
-
-    def keep_tok():
-        g = nat.getGrad(wemb._id)
-        return [t._id for t in (xt, rt, gm, bt, wemb)] + ([g] if g is not None else [])
-
-    def timed(fn, n=20):
-        # every call is followed by a collection (untimed), as in a training loop, so buffers come from the allocator's cache
-        total = 0.0
-        for it in range(n + 3):
-            r.sync()
-            t0 = time.perf_counter()
-            fn()
-            r.sync()
-            if it >= 3:
-                total += time.perf_counter() - t0
-            nat.gcTensors(keep_tok())
-        return total / n * 1e6
-    nb = 8192 * 768 * 4.0
-    us_d = timed(lambda: nat.dropoutOp(xt._id, 0.1, True))
-    us_l = timed(lambda: nat.residualLayernorm(xt._id, rt._id, gm._id, bt._id, 1e-5))
-    us_e = timed(lambda: nat.embeddingForward(wemb._id, idx, 8, 1024))
-
-    def emb_fb():
-        nat.zeroGrad([wemb._id])
-        api.Tensor(nat.embeddingForward(wemb._id, idx, 8, 1024)).mul(xt.view(8, 1024, 768)).sum().backward()
-    us_eb = timed(emb_fb, 10)
-    out["token_ops_8192x768"] = {
-        "dropout_us": us_d, "dropout_GB/s": 2 * nb / us_d / 1e3,
-        "residual_layernorm_us": us_l, "residual_layernorm_GB/s": 4 * nb / us_l / 1e3,
-        "embedding_forward_us": us_e, "embedding_forward_GB/s": 2 * nb / us_e / 1e3,
-        "embedding_forward_backward_vocab32768_us": us_eb,
-        "note": "one call, then a sync; embedding_forward includes the host-to-device copy of 8192 indices"}
     api.native.resetEngine()
     return out
 
@@ -445,17 +525,17 @@ def main():
     line = {
         "metric": "fp32 matmul TFLOP/s", "value": value, "unit": "TFLOP/s",
         "pct_of_fp32_matrix_peak": 100.0 * value / PEAK_FP32_MATRIX_TFLOPS,
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall_ms,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_launches": SETTLE_LAUNCHES, "ms_per_step": wall_ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "single fp32 matmul A[4096,4096] x B[4096,4096], A,B ~ N(0,1) seed 1, row-major, forward only",
                    "M": 4096, "N": 4096, "K": 4096, "device": info["name"].strip(), "compute_units": info["compute_units"],
                    "max_err_vs_f64_sample": err},
         "roofline": {"bound": "mfma", "kernel": "gemm_mfma_kernel<0, 1, 2, 2, false>", "achieved": achieved,
                      "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MATRIX_TFLOPS,
-                     "kernel_ms": kernel_ms, "algorithmic_flops": flops, "traffic": MEASURED_HBM_BYTES_4096},
+                     "kernel_ms": kernel_ms, "algorithmic_flops": flops, "traffic": profile_traffic("gemm_mfma_4096_pmc.txt")},
     }
     if not args.no_extras:
-        line["extra"] = bench_extras(r)
+        line["extra"] = bench_extras(r, not args.no_cpu)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a, b, args.cpu_sample_seconds)
     print(json.dumps(line))

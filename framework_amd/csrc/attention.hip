@@ -63,9 +63,9 @@ int k_softmax(float *out, const float *x, int64_t outer, int64_t n, int64_t inne
     if (outer * n * inner <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (inner == 1)
-        hipLaunchKernelGGL(softmax_rows_kernel, dim3(rows_grid(outer)), dim3(ATT_TPB), 0, ctx().stream, out, x, outer, n);
+        MNI_KERNEL_LAUNCH(softmax_rows_kernel, dim3(rows_grid(outer)), dim3(ATT_TPB), 0, ctx().stream, out, x, outer, n);
     else
-        hipLaunchKernelGGL(softmax_strided_kernel, dim3((unsigned)((outer * inner + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB), 0,
+        MNI_KERNEL_LAUNCH(softmax_strided_kernel, dim3((unsigned)((outer * inner + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB), 0,
                            ctx().stream, out, x, outer, n, inner);
     return check_launch("softmax");
 }
@@ -95,9 +95,9 @@ int k_softmax_backward(float *out, const float *sm, const float *g, int64_t oute
     if (outer * n * inner <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (inner == 1)
-        hipLaunchKernelGGL(softmax_bwd_rows_kernel, dim3(rows_grid(outer)), dim3(ATT_TPB), 0, ctx().stream, out, sm, g, outer, n);
+        MNI_KERNEL_LAUNCH(softmax_bwd_rows_kernel, dim3(rows_grid(outer)), dim3(ATT_TPB), 0, ctx().stream, out, sm, g, outer, n);
     else
-        hipLaunchKernelGGL(softmax_bwd_strided_kernel, dim3((unsigned)((outer * inner + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB),
+        MNI_KERNEL_LAUNCH(softmax_bwd_strided_kernel, dim3((unsigned)((outer * inner + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB),
                            0, ctx().stream, out, sm, g, outer, n, inner);
     return check_launch("softmax_backward");
 }
@@ -154,7 +154,7 @@ __global__ void attn_softmax_kernel(float *__restrict__ scores, float *__restric
 int k_attn_softmax(float *scores, float *lse, int64_t rows, int64_t s, float scale, int causal) {
     if (rows <= 0 || s <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(attn_softmax_kernel, dim3(rows_grid(rows)), dim3(ATT_TPB), 0, ctx().stream, scores, lse, rows, (int)s,
+    MNI_KERNEL_LAUNCH(attn_softmax_kernel, dim3(rows_grid(rows)), dim3(ATT_TPB), 0, ctx().stream, scores, lse, rows, (int)s,
                        scale, causal);
     return check_launch("attn_softmax");
 }
@@ -443,7 +443,7 @@ int k_attn_fused_forward(float *out, float *lse, const float *q, const float *k,
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
 #define MNI_AF(DBV, NBV, SPV)                                                                                               \
-    hipLaunchKernelGGL((attn_fused_fwd_kernel<DBV, NBV, SPV>), grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, \
+    MNI_KERNEL_LAUNCH((attn_fused_fwd_kernel<DBV, NBV, SPV>), grid, block, 0, st, out, lse, q, k, v, (int)s, (int)qblocks, \
                        attn_pair<attn_fused_fwd_kernel<DBV, NBV, SPV>>(), scale, causal)
     switch (d / 32) {
         // 64 keys per step while two workgroups still fit a CU's LDS, 32 beyond
@@ -626,7 +626,7 @@ int k_attn_fused_backward_dq(float *dq, const float *q, const float *k, const fl
     const dim3 grid((unsigned)(bh * qblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
 #define MNI_AB(DBV, SPV)                                                                                                               \
-    hipLaunchKernelGGL((attn_fused_bwd_dq_kernel<DBV, SPV, !SPV>), grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, \
+    MNI_KERNEL_LAUNCH((attn_fused_bwd_dq_kernel<DBV, SPV, !SPV>), grid, block, 0, st, dq, q, k, v, dout, lse, di, (int)s, (int)qblocks, \
                        attn_pair<attn_fused_bwd_dq_kernel<DBV, SPV, !SPV>>(), scale, causal)
     switch (d / 32) {
         case 1: if (split) MNI_AB(1, true); else MNI_AB(1, false); break;
@@ -831,7 +831,7 @@ int k_attn_fused_backward_dkv(float *dk, float *dv, const float *q, const float 
     const dim3 grid((unsigned)(bh * kblocks)), block(ATT_TPB);
     hipStream_t st = ctx().stream;
 #define MNI_AK(DBV, SPV)                                                                                                            \
-    hipLaunchKernelGGL((attn_fused_bwd_dkv_kernel<DBV, SPV, !SPV>), grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, \
+    MNI_KERNEL_LAUNCH((attn_fused_bwd_dkv_kernel<DBV, SPV, !SPV>), grid, block, 0, st, dk, dv, q, k, v, dout, lse, di, (int)s, (int)kblocks, \
                        attn_pair<attn_fused_bwd_dkv_kernel<DBV, SPV, !SPV>>(), scale, causal)
     switch (d / 32) {
         case 1: if (split) MNI_AK(1, true); else MNI_AK(1, false); break;
@@ -857,7 +857,7 @@ __global__ void rowdot_kernel(float *__restrict__ out, const float *__restrict__
 int k_rowdot(float *out, const float *a, const float *b, int64_t rows, int64_t d) {
     if (rows <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(rowdot_kernel, dim3(rows_grid(rows)), dim3(ATT_TPB), 0, ctx().stream, out, a, b, rows, d);
+    MNI_KERNEL_LAUNCH(rowdot_kernel, dim3(rows_grid(rows)), dim3(ATT_TPB), 0, ctx().stream, out, a, b, rows, d);
     return check_launch("rowdot");
 }
 
@@ -885,7 +885,7 @@ int k_attn_backward(float *scores, float *dp, const float *lse, const float *di,
     MNI_TRY(ensure_init());
     int64_t blocks = (n + ATT_TPB * 4 - 1) / (ATT_TPB * 4);
     if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL(attn_bwd_kernel, dim3((unsigned)blocks), dim3(ATT_TPB), 0, ctx().stream, scores, dp, lse, di, rows,
+    MNI_KERNEL_LAUNCH(attn_bwd_kernel, dim3((unsigned)blocks), dim3(ATT_TPB), 0, ctx().stream, scores, dp, lse, di, rows,
                        (int)s, scale, causal);
     return check_launch("attn_backward");
 }
@@ -938,10 +938,10 @@ int k_kv_append(void *kc, void *vc, float *ks, float *vs, const float *k, const 
     if (bh * d <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (quantized)
-        hipLaunchKernelGGL(kv_append_i8_kernel, dim3(rows_grid(2 * bh)), dim3(ATT_TPB), 0, ctx().stream, (signed char *)kc,
+        MNI_KERNEL_LAUNCH(kv_append_i8_kernel, dim3(rows_grid(2 * bh)), dim3(ATT_TPB), 0, ctx().stream, (signed char *)kc,
                            (signed char *)vc, ks, vs, k, v, bh, d, max_seq, pos);
     else
-        hipLaunchKernelGGL(kv_append_f32_kernel, dim3((unsigned)((bh * d + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB), 0,
+        MNI_KERNEL_LAUNCH(kv_append_f32_kernel, dim3((unsigned)((bh * d + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB), 0,
                            ctx().stream, (float *)kc, (float *)vc, k, v, bh * d, d, max_seq, pos);
     return check_launch("kv_append");
 }
@@ -1179,7 +1179,7 @@ template <bool Q8>
 static bool launch_kv_decode_vec(const KvDecode &a, dim3 grid, size_t lds) {
     const int pieces = (int)(a.d / (Q8 ? 16 : 4));
     hipStream_t st = ctx().stream;
-#define MNI_KVV(L) hipLaunchKernelGGL((kv_decode_vec_kernel<Q8, L>), grid, dim3(ATT_TPB), lds, st, a)
+#define MNI_KVV(L) MNI_KERNEL_LAUNCH((kv_decode_vec_kernel<Q8, L>), grid, dim3(ATT_TPB), lds, st, a)
     if (pieces <= 1) MNI_KVV(1);
     else if (pieces <= 2) MNI_KVV(2);
     else if (pieces <= 4) MNI_KVV(4);
@@ -1245,12 +1245,12 @@ int k_kv_decode(float *out, const void *kc, const void *vc, const float *ks, con
     }
     if (!launched) {
         const size_t lds = (size_t)(d + chunk + ATT_TPB) * sizeof(float);
-        if (quantized) hipLaunchKernelGGL((kv_decode_kernel<true>), grid, dim3(ATT_TPB), lds, ctx().stream, a);
-        else hipLaunchKernelGGL((kv_decode_kernel<false>), grid, dim3(ATT_TPB), lds, ctx().stream, a);
+        if (quantized) MNI_KERNEL_LAUNCH((kv_decode_kernel<true>), grid, dim3(ATT_TPB), lds, ctx().stream, a);
+        else MNI_KERNEL_LAUNCH((kv_decode_kernel<false>), grid, dim3(ATT_TPB), lds, ctx().stream, a);
     }
     int rc = check_launch("kv_decode");
     if (rc == MNI_OK && splits > 1) {
-        hipLaunchKernelGGL(kv_combine_kernel, dim3((unsigned)bh), dim3(ATT_TPB), 0, ctx().stream, out, (const float *)part, d,
+        MNI_KERNEL_LAUNCH(kv_combine_kernel, dim3((unsigned)bh), dim3(ATT_TPB), 0, ctx().stream, out, (const float *)part, d,
                            (int)splits);
         rc = check_launch("kv_combine");
     }

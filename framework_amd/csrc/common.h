@@ -56,6 +56,8 @@ struct DeviceCtx {
     // block of `scratch_bytes` (the entry point that must not allocate).
     float *scratch = nullptr;
     size_t scratch_bytes = 0;
+    // Kernels launched since the library was loaded (bookkeeping for latency-bound steps).
+    uint64_t launches = 0;
     // Device address and size of the library's static workspace (see device.hip).
     float *noalloc_scratch = nullptr;
     size_t noalloc_scratch_bytes = 0;
@@ -87,6 +89,12 @@ int dev_clear_cache();
 size_t dev_cached_bytes();  // bytes held in free lists
 
 // ---- launch helpers --------------------------------------------------------
+// Every kernel launch of the library goes through this, so that launches can be counted.
+#define MNI_KERNEL_LAUNCH(...)          \
+    do {                                \
+        ++::mni::ctx().launches;        \
+        hipLaunchKernelGGL(__VA_ARGS__); \
+    } while (0)
 int check_launch(const char *what);  // hipGetLastError after a kernel launch
 
 // gemm.hip

@@ -61,7 +61,7 @@ static int probe_xcd_mapping(DeviceCtx &c) {
     constexpr int BLOCKS = 24 * 29 * 3;
     unsigned *dev = nullptr;
     MNI_HIP_CHECK(hipMalloc((void **)&dev, BLOCKS * sizeof(unsigned)));
-    hipLaunchKernelGGL(xcc_probe_kernel, grid, dim3(64), 0, c.stream, dev);
+    MNI_KERNEL_LAUNCH(xcc_probe_kernel, grid, dim3(64), 0, c.stream, dev);
     std::vector<unsigned> host(BLOCKS);
     hipError_t e = hipMemcpyAsync(host.data(), dev, BLOCKS * sizeof(unsigned), hipMemcpyDeviceToHost, c.stream);
     if (e == hipSuccess) e = hipStreamSynchronize(c.stream);
@@ -318,6 +318,11 @@ int mni_rocm_sgemm_noalloc(const mni_gemm_desc *desc) {
 }
 
 size_t mni_rocm_sgemm_noalloc_workspace_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
+
+uint64_t mni_rocm_launch_count(void) {
+    MNI_API_GUARD;
+    return ctx().launches;
+}
 
 int mni_rocm_test_raise_device_status(unsigned code) {
     MNI_API_GUARD;

@@ -56,10 +56,10 @@ int k_fill(float *dst, float v, int64_t n) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (al16(dst) && (n % 4) == 0) {
-        hipLaunchKernelGGL(fill4_kernel, dim3(grid_for(n / 4, TPB * 4)), dim3(TPB), 0, ctx().stream,
+        MNI_KERNEL_LAUNCH(fill4_kernel, dim3(grid_for(n / 4, TPB * 4)), dim3(TPB), 0, ctx().stream,
                            reinterpret_cast<float4 *>(dst), v, n / 4);
     } else {
-        hipLaunchKernelGGL(fill_kernel, dim3(grid_for(n, TPB * 4)), dim3(TPB), 0, ctx().stream, dst, v, n);
+        MNI_KERNEL_LAUNCH(fill_kernel, dim3(grid_for(n, TPB * 4)), dim3(TPB), 0, ctx().stream, dst, v, n);
     }
     return check_launch("fill");
 }
@@ -84,10 +84,10 @@ int k_axpy(float *dst, const float *src, float alpha, int64_t n) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (al16(dst) && al16(src) && (n % 4) == 0) {
-        hipLaunchKernelGGL(axpy4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+        MNI_KERNEL_LAUNCH(axpy4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
                            reinterpret_cast<float4 *>(dst), reinterpret_cast<const float4 *>(src), alpha, n / 4);
     } else {
-        hipLaunchKernelGGL(axpy_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, dst, src, alpha, n);
+        MNI_KERNEL_LAUNCH(axpy_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, dst, src, alpha, n);
     }
     return check_launch("axpy");
 }
@@ -100,7 +100,7 @@ __global__ void scale_kernel(float *__restrict__ dst, float s, int64_t n) {
 int k_scale_inplace(float *dst, float s, int64_t n) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(scale_kernel, dim3(grid_for(n, TPB * 4)), dim3(TPB), 0, ctx().stream, dst, s, n);
+    MNI_KERNEL_LAUNCH(scale_kernel, dim3(grid_for(n, TPB * 4)), dim3(TPB), 0, ctx().stream, dst, s, n);
     return check_launch("scale");
 }
 
@@ -194,7 +194,7 @@ int k_strided_copy(float *dst, const float *src, const int64_t *shape, const int
         if (uniform && batch <= 65535) {
             dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32), (unsigned)batch);
             if (grid.y <= 65535) {
-                hipLaunchKernelGGL(transpose_tile_kernel, grid, dim3(256), 0, ctx().stream, dst, src, rows, cols,
+                MNI_KERNEL_LAUNCH(transpose_tile_kernel, grid, dim3(256), 0, ctx().stream, dst, src, rows, cols,
                                    strides[ndim - 1], bs);
                 return check_launch("transpose_tile");
             }
@@ -207,14 +207,14 @@ int k_strided_copy(float *dst, const float *src, const int64_t *shape, const int
         if (aligned) {
             d.ndim = ndim - 1;
             for (int i = 0; i < ndim - 1; ++i) { d.shape[i] = shape[i]; d.strides[i] = strides[i]; }
-            hipLaunchKernelGGL(gather4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+            MNI_KERNEL_LAUNCH(gather4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
                                reinterpret_cast<float4 *>(dst), src, d, shape[ndim - 1] / 4, n / 4);
             return check_launch("gather4");
         }
     }
     d.ndim = ndim;
     for (int i = 0; i < ndim; ++i) { d.shape[i] = shape[i]; d.strides[i] = strides[i]; }
-    hipLaunchKernelGGL(gather_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, dst, src, d, n);
+    MNI_KERNEL_LAUNCH(gather_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, dst, src, d, n);
     return check_launch("gather");
 }
 
@@ -253,7 +253,7 @@ int k_binary_broadcast(float *out, const float *a, const float *b, const Strided
     int64_t n = 1;
     for (int i = 0; i < d.ndim; ++i) n *= d.shape[i];
     if (n <= 0) return MNI_OK;
-    hipLaunchKernelGGL(binary_bcast_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, d, n, op, p);
+    MNI_KERNEL_LAUNCH(binary_bcast_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, d, n, op, p);
     return check_launch("binary_broadcast");
 }
 
@@ -277,11 +277,11 @@ int k_binary_same(float *out, const float *a, const float *b, int64_t n, int op,
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (al16(out) && al16(a) && al16(b) && (n % 4) == 0) {
-        hipLaunchKernelGGL(binary_same4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+        MNI_KERNEL_LAUNCH(binary_same4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
                            reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(a),
                            reinterpret_cast<const float4 *>(b), n / 4, op, p);
     } else {
-        hipLaunchKernelGGL(binary_same_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, n, op, p);
+        MNI_KERNEL_LAUNCH(binary_same_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, b, n, op, p);
     }
     return check_launch("binary_same");
 }
@@ -309,7 +309,7 @@ int k_div_backward(float *ga, float *gb, const float *g, const float *a, const f
     int64_t n = 1;
     for (int i = 0; i < d.ndim; ++i) n *= d.shape[i];
     if (n <= 0) return MNI_OK;
-    hipLaunchKernelGGL(div_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, ga, gb, g, a, b, d, n);
+    MNI_KERNEL_LAUNCH(div_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, ga, gb, g, a, b, d, n);
     return check_launch("div_backward");
 }
 
@@ -334,11 +334,11 @@ int k_add_bias(float *out, const float *a, const float *bias, int64_t rows, int6
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (al16(out) && al16(a) && al16(bias) && (cols % 4) == 0) {
-        hipLaunchKernelGGL(add_bias4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+        MNI_KERNEL_LAUNCH(add_bias4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
                            reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(a),
                            reinterpret_cast<const float4 *>(bias), n / 4, cols / 4);
     } else {
-        hipLaunchKernelGGL(add_bias_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, bias, n, cols);
+        MNI_KERNEL_LAUNCH(add_bias_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, a, bias, n, cols);
     }
     return check_launch("add_bias");
 }
@@ -374,10 +374,10 @@ int k_unary(float *out, const float *x, int64_t n, int op, float s) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (al16(out) && al16(x) && (n % 4) == 0) {
-        hipLaunchKernelGGL(unary4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+        MNI_KERNEL_LAUNCH(unary4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
                            reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(x), n / 4, op, s);
     } else {
-        hipLaunchKernelGGL(unary_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, n, op, s);
+        MNI_KERNEL_LAUNCH(unary_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, n, op, s);
     }
     return check_launch("unary");
 }
@@ -395,7 +395,7 @@ __global__ void unary_bwd_kernel(float *__restrict__ out, const float *__restric
 int k_unary_backward(float *out, const float *g, const float *x, int64_t n, int op) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(unary_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, x, n, op);
+    MNI_KERNEL_LAUNCH(unary_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, x, n, op);
     return check_launch("unary_backward");
 }
 
@@ -413,7 +413,7 @@ __global__ void unary2_bwd_kernel(float *__restrict__ out, const float *__restri
 int k_unary2_backward(float *out, const float *g, const float *saved, int64_t n, int op, float s) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(unary2_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, saved, n, op, s);
+    MNI_KERNEL_LAUNCH(unary2_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, saved, n, op, s);
     return check_launch("unary2_backward");
 }
 
@@ -431,7 +431,7 @@ __global__ void mul_bwd_kernel(float *__restrict__ ga, float *__restrict__ gb, c
 int k_mul_backward_same(float *ga, float *gb, const float *g, const float *a, const float *b, int64_t n) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(mul_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, ga, gb, g, a, b, n);
+    MNI_KERNEL_LAUNCH(mul_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, ga, gb, g, a, b, n);
     return check_launch("mul_backward");
 }
 
@@ -550,16 +550,16 @@ int k_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
     if (nparts > 1) MNI_TRY(dev_alloc(&part, (size_t)nparts * cols * sizeof(float)));
     float *dst = nparts > 1 ? (float *)part : out;
     if (narrow)
-        hipLaunchKernelGGL(colsum_narrow_kernel, dim3((unsigned)nparts), dim3(256), 0, ctx().stream, dst, a, rows, (int)cols, lanes);
+        MNI_KERNEL_LAUNCH(colsum_narrow_kernel, dim3((unsigned)nparts), dim3(256), 0, ctx().stream, dst, a, rows, (int)cols, lanes);
     else
-        hipLaunchKernelGGL(colsum_partial_kernel, dim3(gx, (unsigned)nparts), block, 0, ctx().stream, dst, a, rows, cols, rows_per_block);
+        MNI_KERNEL_LAUNCH(colsum_partial_kernel, dim3(gx, (unsigned)nparts), block, 0, ctx().stream, dst, a, rows, cols, rows_per_block);
     int rc = check_launch("colsum_partial");
     if (rc == MNI_OK && nparts > 1) {
         if (nparts > 1024) {
             // many partials: they are a tall matrix themselves
             rc = k_colsum(out, (const float *)part, nparts, cols);
         } else {
-            hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, out, (const float *)part, nparts, cols);
+            MNI_KERNEL_LAUNCH(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, out, (const float *)part, nparts, cols);
             rc = check_launch("colsum_final");
         }
     }
@@ -591,10 +591,10 @@ int k_bias_gelu(float *out, const float *x, const float *bias, int64_t rows, int
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (cols % 4 == 0 && al16(out) && al16(x) && al16(bias))
-        hipLaunchKernelGGL(bias_gelu4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream, (float4 *)out,
+        MNI_KERNEL_LAUNCH(bias_gelu4_kernel, dim3(grid_for(n / 4, TPB * 2)), dim3(TPB), 0, ctx().stream, (float4 *)out,
                            (const float4 *)x, (const float4 *)bias, n / 4, cols / 4);
     else
-        hipLaunchKernelGGL(bias_gelu_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, bias, n, cols);
+        MNI_KERNEL_LAUNCH(bias_gelu_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, bias, n, cols);
     return check_launch("bias_gelu");
 }
 static constexpr int BG_ROWS = 16;  // rows per block in the backward pass
@@ -651,14 +651,14 @@ int k_bias_gelu_backward(float *dx, float *dbias, const float *g, const float *x
     if (nparts > 1) MNI_TRY(dev_alloc(&part, (size_t)nparts * cols * sizeof(float)));
     float *dst = nparts > 1 ? (float *)part : dbias;
     if (vec)
-        hipLaunchKernelGGL((bias_gelu_bwd_kernel<float4, 4>), dim3(gx, (unsigned)nparts), block, 0, ctx().stream, (float4 *)dx,
+        MNI_KERNEL_LAUNCH((bias_gelu_bwd_kernel<float4, 4>), dim3(gx, (unsigned)nparts), block, 0, ctx().stream, (float4 *)dx,
                            (float4 *)dst, (const float4 *)g, (const float4 *)x, (const float4 *)bias, rows, colsv, rows_per_block);
     else
-        hipLaunchKernelGGL((bias_gelu_bwd_kernel<float, 1>), dim3(gx, (unsigned)nparts), block, 0, ctx().stream, dx, dst, g, x,
+        MNI_KERNEL_LAUNCH((bias_gelu_bwd_kernel<float, 1>), dim3(gx, (unsigned)nparts), block, 0, ctx().stream, dx, dst, g, x,
                            bias, rows, colsv, rows_per_block);
     int rc = check_launch("bias_gelu_backward");
     if (rc == MNI_OK && nparts > 1) {
-        hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dbias,
+        MNI_KERNEL_LAUNCH(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dbias,
                            (const float *)part, nparts, cols);
         rc = check_launch("colsum_final");
     }
@@ -702,9 +702,9 @@ int k_max_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t in
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (inner == 1 && dim >= 256)
-        hipLaunchKernelGGL(max_rows_kernel, dim3(grid_for(outer, 4)), dim3(TPB), 0, ctx().stream, out, a, outer, dim);
+        MNI_KERNEL_LAUNCH(max_rows_kernel, dim3(grid_for(outer, 4)), dim3(TPB), 0, ctx().stream, out, a, outer, dim);
     else
-        hipLaunchKernelGGL(max_dim_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, inner);
+        MNI_KERNEL_LAUNCH(max_dim_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, inner);
     return check_launch("max_dim");
 }
 __global__ void max_bwd_kernel(float *__restrict__ out, const float *__restrict__ x, const float *__restrict__ mx,
@@ -721,7 +721,7 @@ int k_max_backward(float *out, const float *x, const float *mx, const float *g, 
     const int64_t n = outer * dim * inner;
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(max_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, mx, g, dim, inner, n);
+    MNI_KERNEL_LAUNCH(max_bwd_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, mx, g, dim, inner, n);
     return check_launch("max_backward");
 }
 
@@ -753,7 +753,7 @@ int k_layernorm(float *out, float *mean, float *rstd, const float *x, const floa
                 int64_t c, float eps) {
     if (rows <= 0 || c <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(layernorm_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, mean, rstd, x, gamma, beta,
+    MNI_KERNEL_LAUNCH(layernorm_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, mean, rstd, x, gamma, beta,
                        rows, c, eps);
     return check_launch("layernorm");
 }
@@ -801,7 +801,7 @@ int k_layernorm_backward(float *dx, float *dgamma, float *dbeta, const float *g,
     if (c <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (rows <= 0) { MNI_TRY(k_fill(dgamma, 0.0f, c)); return k_fill(dbeta, 0.0f, c); }
-    hipLaunchKernelGGL(layernorm_bwd_rows_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, dx, g, x, gamma, mean,
+    MNI_KERNEL_LAUNCH(layernorm_bwd_rows_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, dx, g, x, gamma, mean,
                        rstd, rows, c);
     MNI_TRY(check_launch("layernorm_backward_rows"));
     const int64_t nparts = (rows + BG_ROWS - 1) / BG_ROWS;
@@ -810,12 +810,12 @@ int k_layernorm_backward(float *dx, float *dgamma, float *dbeta, const float *g,
     MNI_TRY(dev_alloc(&part, (size_t)2 * nparts * c * sizeof(float)));
     float *pg = (float *)part, *pb = pg + nparts * c;
     const unsigned gx = (unsigned)((c + TPB - 1) / TPB);
-    hipLaunchKernelGGL(layernorm_bwd_cols_kernel, dim3(gx, (unsigned)nparts), dim3(TPB), 0, ctx().stream, pg, pb, g, x, mean,
+    MNI_KERNEL_LAUNCH(layernorm_bwd_cols_kernel, dim3(gx, (unsigned)nparts), dim3(TPB), 0, ctx().stream, pg, pb, g, x, mean,
                        rstd, rows, c);
     int rc = check_launch("layernorm_backward_cols");
     if (rc == MNI_OK) {
-        hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(c), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dgamma, (const float *)pg, nparts, c);
-        hipLaunchKernelGGL(colsum_final_kernel, colsum_final_grid(c), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dbeta, (const float *)pb, nparts, c);
+        MNI_KERNEL_LAUNCH(colsum_final_kernel, colsum_final_grid(c), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dgamma, (const float *)pg, nparts, c);
+        MNI_KERNEL_LAUNCH(colsum_final_kernel, colsum_final_grid(c), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dbeta, (const float *)pb, nparts, c);
         rc = check_launch("colsum_final");
     }
     dev_free(part);
@@ -855,10 +855,10 @@ int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if (inner == 1 && dim >= 256) {
-        hipLaunchKernelGGL(reduce_rows_kernel, dim3(grid_for(outer, 4)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, div);
+        MNI_KERNEL_LAUNCH(reduce_rows_kernel, dim3(grid_for(outer, 4)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, div);
         return check_launch("reduce_rows");
     }
-    hipLaunchKernelGGL(reduce_inner_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, inner, div);
+    MNI_KERNEL_LAUNCH(reduce_inner_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, inner, div);
     return check_launch("reduce_inner");
 }
 
@@ -877,7 +877,7 @@ int k_expand_dim(float *out, const float *g, int64_t outer, int64_t dim, int64_t
     const int64_t n = outer * dim * inner;
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(expand_dim_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, outer, dim, inner, div, n);
+    MNI_KERNEL_LAUNCH(expand_dim_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, g, outer, dim, inner, div, n);
     return check_launch("expand_dim");
 }
 
@@ -936,7 +936,7 @@ int k_unbroadcast(float *out, const float *g, const int64_t *gshape, int gnd, co
         else if (ext != gshape[k]) return set_error(MNI_ERR_INVALID, "unbroadcast: shapes do not broadcast");
     }
     if (on <= 0) return MNI_OK;
-    hipLaunchKernelGGL(unbroadcast_kernel, dim3(grid_for(on, TPB)), dim3(TPB), 0, ctx().stream, out, g, d, on, red_total);
+    MNI_KERNEL_LAUNCH(unbroadcast_kernel, dim3(grid_for(on, TPB)), dim3(TPB), 0, ctx().stream, out, g, d, on, red_total);
     return check_launch("unbroadcast");
 }
 
@@ -1081,16 +1081,16 @@ int k_cross_entropy(float *loss, float *softmax, const float *logits, const int3
     const dim3 grid(grid_for(n, 4)), block(TPB);
     hipStream_t st = ctx().stream;
     if (vec && v <= 64 * 4 * 2)
-        hipLaunchKernelGGL(ce_rows_cached_kernel<2>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
+        MNI_KERNEL_LAUNCH(ce_rows_cached_kernel<2>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
     else if (vec && v <= 64 * 4 * 8)
-        hipLaunchKernelGGL(ce_rows_cached_kernel<8>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
+        MNI_KERNEL_LAUNCH(ce_rows_cached_kernel<8>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
     else if (vec && v <= 256 * 4 * 8 && n <= 0x7fffffffLL)
-        hipLaunchKernelGGL(ce_rows_wg_kernel<8>, dim3((unsigned)n), dim3(256), 0, st, (float *)rl, softmax, logits, targets, n, v);
+        MNI_KERNEL_LAUNCH(ce_rows_wg_kernel<8>, dim3((unsigned)n), dim3(256), 0, st, (float *)rl, softmax, logits, targets, n, v);
     else
-        hipLaunchKernelGGL(ce_rows_kernel, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
+        MNI_KERNEL_LAUNCH(ce_rows_kernel, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
     int rc = check_launch("ce_rows");
     if (rc == MNI_OK) {
-        hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(64), 0, ctx().stream, loss, (const float *)rl, n);
+        MNI_KERNEL_LAUNCH(ce_mean_kernel, dim3(1), dim3(64), 0, ctx().stream, loss, (const float *)rl, n);
         rc = check_launch("ce_mean");
     }
     dev_free(rl);
@@ -1133,11 +1133,11 @@ int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t
     if (v % 4 == 0 && al16(dlogits) && al16(softmax)) {
         const int64_t v4 = v / 4;
         const unsigned gx = (unsigned)min((int64_t)64, (v4 + TPB - 1) / TPB), gy = (unsigned)min(n, (int64_t)65535);
-        hipLaunchKernelGGL(ce_bwd4_kernel, dim3(gx, gy), dim3(TPB), 0, ctx().stream, (float4 *)dlogits, (const float4 *)softmax, targets,
+        MNI_KERNEL_LAUNCH(ce_bwd4_kernel, dim3(gx, gy), dim3(TPB), 0, ctx().stream, (float4 *)dlogits, (const float4 *)softmax, targets,
                            grad_scalar, n, v4);
         return check_launch("ce_backward");
     }
-    hipLaunchKernelGGL(ce_bwd_kernel, dim3(grid_for(n * v, TPB * 2)), dim3(TPB), 0, ctx().stream, dlogits, softmax, targets, grad_scalar, n, v);
+    MNI_KERNEL_LAUNCH(ce_bwd_kernel, dim3(grid_for(n * v, TPB * 2)), dim3(TPB), 0, ctx().stream, dlogits, softmax, targets, grad_scalar, n, v);
     return check_launch("ce_backward");
 }
 
@@ -1174,13 +1174,13 @@ int sumsq_blocks(int64_t n) {
 int k_sumsq_partials(double *part, const float *g, int64_t n) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(sumsq_kernel, dim3(sumsq_blocks(n)), dim3(TPB), 0, ctx().stream, part, g, n);
+    MNI_KERNEL_LAUNCH(sumsq_kernel, dim3(sumsq_blocks(n)), dim3(TPB), 0, ctx().stream, part, g, n);
     return check_launch("sumsq");
 }
 int k_sumsq_finish(double *out, const double *part, int nparts) {
     if (nparts <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), dim3(TPB), 0, ctx().stream, out, part, nparts);
+    MNI_KERNEL_LAUNCH(sumsq_final_kernel, dim3(1), dim3(TPB), 0, ctx().stream, out, part, nparts);
     return check_launch("sumsq_final");
 }
 int k_sumsq_f64(double *out, const float *g, int64_t n) {
@@ -1218,7 +1218,7 @@ int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, f
             float bc1, float bc2) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(adamw_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, p, m, v, g, n, lr, b1, b2, eps, wd, bc1, bc2);
+    MNI_KERNEL_LAUNCH(adamw_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, p, m, v, g, n, lr, b1, b2, eps, wd, bc1, bc2);
     return check_launch("adamw");
 }
 
@@ -1283,14 +1283,14 @@ static int multi_check(const MultiTensor &t) {
 int k_adamw_multi(const MultiTensor &t, float lr, float b1, float b2, float eps, float wd, float bc1, float bc2) {
     MNI_TRY(ensure_init());
     MNI_TRY(multi_check(t));
-    hipLaunchKernelGGL(multi_tensor_kernel<true>, dim3(t.block_start[t.count]), dim3(TPB), 0, ctx().stream, t, (double *)nullptr, lr, b1,
+    MNI_KERNEL_LAUNCH(multi_tensor_kernel<true>, dim3(t.block_start[t.count]), dim3(TPB), 0, ctx().stream, t, (double *)nullptr, lr, b1,
                        b2, eps, wd, bc1, bc2);
     return check_launch("adamw_multi");
 }
 int k_sumsq_multi(const MultiTensor &t, double *part) {
     MNI_TRY(ensure_init());
     MNI_TRY(multi_check(t));
-    hipLaunchKernelGGL(multi_tensor_kernel<false>, dim3(t.block_start[t.count]), dim3(TPB), 0, ctx().stream, t, part, 0.f, 0.f, 0.f,
+    MNI_KERNEL_LAUNCH(multi_tensor_kernel<false>, dim3(t.block_start[t.count]), dim3(TPB), 0, ctx().stream, t, part, 0.f, 0.f, 0.f,
                        0.f, 0.f, 0.f, 0.f);
     return check_launch("sumsq_multi");
 }

@@ -95,7 +95,7 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         s.out = d.C; s.o_bs = d.c_batch_stride; s.bias = d.bias;
         s.epilogue = d.epilogue; s.accumulate = d.accumulate;
         s.ws = nullptr; s.split_k = 1; s.k_per_slice = s.K;
-        s.groups = 0; s.fused = 0; s.xcds = 0; s.flags = nullptr; s.epoch = 0; s.status = ctx().status_dev;
+        s.groups = 0; s.flags = nullptr; s.epoch = 0; s.status = ctx().status_dev;
 
         const bool w_batch_ok = s.w_bcount <= 1 || (s.w_bs % 4) == 0;
         const bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
@@ -123,24 +123,26 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
             kps = (kps + pass - 1) / pass * pass;
             split = (s.K + kps - 1) / kps;
             s.split_k = split; s.k_per_slice = kps;
+            // One launch when the partials of a unit can stay inside one XCD's
+            // L2 and its arrival flags fit the library's flag array.  Its partial
+            // rows are whole 128-byte lines, so that no line is shared by two units.
+            DeviceCtx &c = ctx();
+            const int64_t flag_count = (int64_t)groups * s.batch * split;
+            const bool fused = split > 1 && d.algo != MNI_ALGO_SKINNY_TWO_PASS && c.xcd_count > 0 && c.skinny_flags &&
+                               flag_count <= (int64_t)c.skinny_flag_cap;
             void *ws = nullptr;
             if (split > 1) {
-                const size_t bytes = (size_t)split * s.batch * s.rows * s.cols * sizeof(float);
+                const size_t bytes = (size_t)split * s.batch * s.rows * skinny_ws_pitch(s.cols, fused) * sizeof(float);
                 *rc = gemm_ws_alloc(&ws, bytes);
                 if (*rc != MNI_OK) return true;
                 s.ws = (float *)ws;
             }
-            // One launch when the partials of a unit can stay inside one XCD's
-            // L2 and its arrival flags fit the library's flag array.
-            DeviceCtx &c = ctx();
-            const int64_t flag_count = (int64_t)groups * s.batch * split;
-            if (split > 1 && d.algo != MNI_ALGO_SKINNY_TWO_PASS && c.xcd_count > 0 && c.skinny_flags &&
-                flag_count <= (int64_t)c.skinny_flag_cap) {
+            if (fused) {
                 *rc = next_epoch(&s.epoch);
-                s.fused = 1; s.xcds = c.xcd_count; s.flags = c.skinny_flags;
+                s.flags = c.skinny_flags;
             }
-            if (*rc == MNI_OK) *rc = launch_skinny_cols(s);
-            if (*rc == MNI_OK && split > 1 && !s.fused) {
+            if (*rc == MNI_OK) *rc = launch_skinny_cols(s, fused ? c.xcd_count : 0);
+            if (*rc == MNI_OK && split > 1 && !fused) {
                 ReduceLaunch r;
                 r.ws = s.ws; r.out = s.out; r.bias = s.bias;
                 r.slices = split; r.batch = s.batch; r.rows = s.rows; r.cols = s.cols;

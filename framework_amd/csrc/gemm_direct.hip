@@ -351,11 +351,11 @@ template <int AMODE, int BMODE>
 static void launch_direct_modes(const GemmLaunch &g, int ksplit, dim3 grid) {
     hipStream_t s = ctx().stream;
     if (ksplit == 1) {
-        if (g.K == 2 * DPHASE) hipLaunchKernelGGL((gemm_direct_kernel<AMODE, BMODE, 1, 2>), grid, dim3(64), 0, s, g);
-        else hipLaunchKernelGGL((gemm_direct_kernel<AMODE, BMODE, 1, 0>), grid, dim3(64), 0, s, g);
+        if (g.K == 2 * DPHASE) MNI_KERNEL_LAUNCH((gemm_direct_kernel<AMODE, BMODE, 1, 2>), grid, dim3(64), 0, s, g);
+        else MNI_KERNEL_LAUNCH((gemm_direct_kernel<AMODE, BMODE, 1, 0>), grid, dim3(64), 0, s, g);
     } else {
-        if (g.K == 4 * 4 * DPHASE) hipLaunchKernelGGL((gemm_direct_kernel<AMODE, BMODE, 4, 4>), grid, dim3(256), 0, s, g);
-        else hipLaunchKernelGGL((gemm_direct_kernel<AMODE, BMODE, 4, 0>), grid, dim3(256), 0, s, g);
+        if (g.K == 4 * 4 * DPHASE) MNI_KERNEL_LAUNCH((gemm_direct_kernel<AMODE, BMODE, 4, 4>), grid, dim3(256), 0, s, g);
+        else MNI_KERNEL_LAUNCH((gemm_direct_kernel<AMODE, BMODE, 4, 0>), grid, dim3(256), 0, s, g);
     }
 }
 

@@ -54,7 +54,8 @@ struct SkinnyLaunch {
     const float *W;
     float *out;
     const float *bias;  // indexed by bias_on_rows ? i : j
-    float *ws;          // partials [slice][batch][rows][cols]
+    float *ws;          // partials [slice][batch][rows][pitch]: pitch = cols, or, in the single-launch form, cols
+                        // rounded up to whole 128-byte lines (skinny_ws_pitch), so that no line is shared by two units
     int rows, cols, K, batch;
     int groups;  // column groups of skinny_cols_block_cols() (skinny_cols only)
     int64_t x_rs, x_cs, x_bs;  // X(i, k)
@@ -63,16 +64,19 @@ struct SkinnyLaunch {
     int64_t o_rs, o_cs, o_bs;
     int split_k, k_per_slice;
     int epilogue, accumulate, bias_on_rows;
-    // Single-launch form (fused != 0, split_k > 1): arrival flags
-    // [unit][split_k] with unit = b * groups + column group, the value that
-    // marks this launch, and the number of XCDs the units are dealt over.
-    int fused, xcds;
+    // Single-launch form (split_k > 1): arrival flags [unit][split_k] with
+    // unit = b * groups + column group, and the value that marks this launch.
+    // (The struct is the kernel argument: it is kept to three 64-byte lines,
+    // a fourth costs the kernel's start a further scalar fetch.)
     unsigned *flags;
     unsigned epoch;
     unsigned *status;  // device status word: set when a reducer's bounded wait expires
 };
 // W with unit stride along j (cols): lanes own columns, K split over wavefronts and slices.
-int launch_skinny_cols(const SkinnyLaunch &s);
+// xcds > 0: the single-launch form, units dealt over that many XCDs; 0: partials left for a reduction launch.
+int launch_skinny_cols(const SkinnyLaunch &s, int xcds);
+// floats per row of the K-slice partials
+int skinny_ws_pitch(int cols, bool single_launch);
 // W with unit stride along k: one wavefront per output column, shuffle reduce.
 int launch_skinny_dots(const SkinnyLaunch &s);
 int skinny_cols_block_cols();

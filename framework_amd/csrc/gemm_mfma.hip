@@ -715,8 +715,8 @@ static void launch_modes(const GemmLaunch &g, int amode, int bmode, dim3 grid) {
     hipStream_t s = ctx().stream;
 #define MNI_LAUNCH(AM, BMO)                                                                        \
     do {                                                                                           \
-        if (g.streamk) hipLaunchKernelGGL((gemm_mfma_kernel<AM, BMO, TM, TN, true>), grid, block, 0, s, g);   \
-        else hipLaunchKernelGGL((gemm_mfma_kernel<AM, BMO, TM, TN, false>), grid, block, 0, s, g);            \
+        if (g.streamk) MNI_KERNEL_LAUNCH((gemm_mfma_kernel<AM, BMO, TM, TN, true>), grid, block, 0, s, g);   \
+        else MNI_KERNEL_LAUNCH((gemm_mfma_kernel<AM, BMO, TM, TN, false>), grid, block, 0, s, g);            \
     } while (0)
     if (amode == 2 || bmode == 2) MNI_LAUNCH(2, 2);
     else if (amode == 0 && bmode == 0) MNI_LAUNCH(0, 0);

@@ -222,8 +222,8 @@ int launch_gemm_panel(const GemmLaunch &g, int amode, int bmode) {
     if (blocks <= 0) return MNI_OK;
     if (blocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "sgemm: too many tiles (%lld)", (long long)blocks);
     const dim3 grid((unsigned)blocks), block(256);
-    if (g.K <= 32) hipLaunchKernelGGL((gemm_panel_kernel<4>), grid, block, 0, ctx().stream, g);
-    else hipLaunchKernelGGL((gemm_panel_kernel<8>), grid, block, 0, ctx().stream, g);
+    if (g.K <= 32) MNI_KERNEL_LAUNCH((gemm_panel_kernel<4>), grid, block, 0, ctx().stream, g);
+    else MNI_KERNEL_LAUNCH((gemm_panel_kernel<8>), grid, block, 0, ctx().stream, g);
     return check_launch("gemm_panel_kernel");
 }
 

@@ -83,6 +83,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
     const int64_t o_cs = LEAN ? 1 : s.o_cs;
     const int x_bcount = LEAN ? 1 : s.x_bcount, w_bcount = LEAN ? 1 : s.w_bcount;
     __shared__ float4 red[SK_WAVES - 1][MR][64];
+    const int ws_pitch = FUSED ? (s.cols + 31) & ~31 : s.cols;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -197,10 +198,10 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
             }
         }
         if (s.split_k > 1 && col_ok) {
-            float *ws = s.ws + (((int64_t)slice * batch + b) * rows) * (int64_t)s.cols + col0;
+            float *ws = s.ws + (((int64_t)slice * batch + b) * rows) * (int64_t)ws_pitch + col0;
 #pragma unroll
             for (int i = 0; i < MR; ++i)
-                if (i < rows) *reinterpret_cast<float4 *>(ws + (int64_t)i * s.cols) = acc[i];
+                if (i < rows) *reinterpret_cast<float4 *>(ws + (int64_t)i * ws_pitch) = acc[i];
         }
     }
 
@@ -226,23 +227,23 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
             arrived = __all(all);
             if (!arrived) __builtin_amdgcn_s_sleep(2);
         }
-        // Tell the host: the next call that waits for the stream fails with this code.
-        if (!arrived && tid == 0) *s.status = DEVICE_STATUS_SKINNY_WAIT;
-        // The partials are read with ordinary loads.  A 128-byte line of the
-        // workspace can be shared by two units when cols is not a multiple of
-        // 32, so this CU's L1 may hold such a line from before the other
-        // unit's partial landed: drop the L1 contents once, after the flags.
-        asm volatile("buffer_inv sc1" ::: "memory");
+        // The partials are read with ordinary loads.  That is safe because no
+        // 128-byte line of the workspace is shared by two units: its row pitch
+        // is a whole number of lines (ws_pitch), so this CU's L1 cannot hold a
+        // line of this unit from before its partials landed.
 
         constexpr int TB = 16;  // partials in flight per lane
-        const int64_t slice_stride = (int64_t)batch * rows * s.cols;
+        const int64_t slice_stride = (int64_t)batch * rows * ws_pitch;
         for (int row = q; row < rows; row += reducers) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
             if (!arrived) {
+                // NaN into the output and a code into the status word: the next call that
+                // waits for the stream fails with it
                 const float nan = __builtin_nanf("");
                 t = f32x4{nan, nan, nan, nan};
+                if (tid == 0) *s.status = DEVICE_STATUS_SKINNY_WAIT;
             } else if (col_ok) {
-                const float *p = s.ws + ((int64_t)b * rows + row) * (int64_t)s.cols + col0;
+                const float *p = s.ws + ((int64_t)b * rows + row) * (int64_t)ws_pitch + col0;
                 for (int s0 = wave; s0 < s.split_k; s0 += SK_WAVES * TB) {
                     f32x4 v[TB];
 #pragma unroll
@@ -429,12 +430,12 @@ static void launch_skinny_cols_mr(const SkinnyLaunch &s, dim3 grid, bool fused) 
                       s.o_rs % 4 == 0 && (reinterpret_cast<uintptr_t>(s.out) & 15) == 0 &&
                       s.epilogue == MNI_EPI_NONE && !s.accumulate;
     if (lean) {
-        hipLaunchKernelGGL((skinny_cols_kernel<MR, true, true, false, true>), grid, block, 0, st, s);
+        MNI_KERNEL_LAUNCH((skinny_cols_kernel<MR, true, true, false, true>), grid, block, 0, st, s);
         return;
     }
     switch (variant) {
 #define MNI_SK(V, XC, FUSED, TAIL) \
-    case V: hipLaunchKernelGGL((skinny_cols_kernel<MR, XC, FUSED, TAIL, false>), grid, block, 0, st, s); break;
+    case V: MNI_KERNEL_LAUNCH((skinny_cols_kernel<MR, XC, FUSED, TAIL, false>), grid, block, 0, st, s); break;
         MNI_SK(0, false, false, false) MNI_SK(1, false, false, true)
         MNI_SK(2, false, true, false)  MNI_SK(3, false, true, true)
         MNI_SK(4, true, false, false)  MNI_SK(5, true, false, true)
@@ -443,18 +444,20 @@ static void launch_skinny_cols_mr(const SkinnyLaunch &s, dim3 grid, bool fused) 
     }
 }
 
-int launch_skinny_cols(const SkinnyLaunch &s) {
+int skinny_ws_pitch(int cols, bool single_launch) { return single_launch ? (cols + 31) & ~31 : cols; }
+
+int launch_skinny_cols(const SkinnyLaunch &s, int xcds) {
     if (s.rows <= 0 || s.cols <= 0 || s.batch <= 0) return MNI_OK;
     const int groups = (s.cols + SK_COLS - 1) / SK_COLS;
     if (s.groups != groups) return set_error(MNI_ERR_INVALID, "skinny launch: column group count not set");
     if (s.k_per_slice % SK_UNROLL != 0 && s.split_k > 1)
         return set_error(MNI_ERR_INVALID, "skinny launch: a K slice must be whole groups of %d rows", SK_UNROLL);
-    const bool fused = s.fused && s.split_k > 1;
+    const bool fused = xcds > 0 && s.split_k > 1;
     dim3 grid(groups, s.split_k, s.batch);
     if (fused) {
-        if (s.xcds <= 0 || !s.flags || !s.ws || !s.status) return set_error(MNI_ERR_INVALID, "single-launch skinny product without flags/partials");
+        if (!s.flags || !s.ws || !s.status) return set_error(MNI_ERR_INVALID, "single-launch skinny product without flags/partials");
         const int64_t units = (int64_t)groups * s.batch;
-        grid = dim3((unsigned)((units + s.xcds - 1) / s.xcds * s.xcds), s.split_k);
+        grid = dim3((unsigned)((units + xcds - 1) / xcds * xcds), s.split_k);
     }
     if (s.rows <= 4) launch_skinny_cols_mr<4>(s, grid, fused);
     else if (s.rows <= 8) launch_skinny_cols_mr<8>(s, grid, fused);
@@ -466,7 +469,7 @@ int launch_skinny_cols(const SkinnyLaunch &s) {
 int launch_skinny_reduce(const ReduceLaunch &r) {
     const int64_t total = (int64_t)r.rows * r.cols * r.batch;
     if (total <= 0) return MNI_OK;
-    hipLaunchKernelGGL(skinny_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(64 * RED_GROUPS), 0, ctx().stream, r);
+    MNI_KERNEL_LAUNCH(skinny_reduce_kernel, dim3((unsigned)((total + 63) / 64)), dim3(64 * RED_GROUPS), 0, ctx().stream, r);
     return check_launch("skinny_reduce_kernel");
 }
 
@@ -474,9 +477,9 @@ int launch_skinny_dots(const SkinnyLaunch &s) {
     if (s.rows <= 0 || s.cols <= 0 || s.batch <= 0) return MNI_OK;
     dim3 grid((s.cols + 15) / 16, s.batch), block(256);
     hipStream_t st = ctx().stream;
-    if (s.rows <= 4) hipLaunchKernelGGL((skinny_dots_kernel<4>), grid, block, 0, st, s);
-    else if (s.rows <= 8) hipLaunchKernelGGL((skinny_dots_kernel<8>), grid, block, 0, st, s);
-    else if (s.rows <= 16) hipLaunchKernelGGL((skinny_dots_kernel<16>), grid, block, 0, st, s);
+    if (s.rows <= 4) MNI_KERNEL_LAUNCH((skinny_dots_kernel<4>), grid, block, 0, st, s);
+    else if (s.rows <= 8) MNI_KERNEL_LAUNCH((skinny_dots_kernel<8>), grid, block, 0, st, s);
+    else if (s.rows <= 16) MNI_KERNEL_LAUNCH((skinny_dots_kernel<16>), grid, block, 0, st, s);
     else return set_error(MNI_ERR_INVALID, "skinny kernel takes at most 16 rows, got %d", s.rows);
     return check_launch("skinny_dots_kernel");
 }
@@ -485,7 +488,7 @@ int launch_splitk_reduce(const ReduceLaunch &r) {
     const int64_t total = (int64_t)r.rows * r.cols * r.batch;
     if (total <= 0) return MNI_OK;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
-    hipLaunchKernelGGL(splitk_reduce_kernel, grid, block, 0, ctx().stream, r);
+    MNI_KERNEL_LAUNCH(splitk_reduce_kernel, grid, block, 0, ctx().stream, r);
     return check_launch("splitk_reduce_kernel");
 }
 

@@ -85,7 +85,7 @@ __global__ void random_fill_kernel(float *__restrict__ out, int64_t n, uint64_t 
 int k_random_fill(float *out, int64_t n, uint64_t seed, uint64_t offset, int mode) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(random_fill_kernel, dim3(grid_for((n + 3) / 4, TPB * 2)), dim3(TPB), 0, ctx().stream, out, n, seed, offset,
+    MNI_KERNEL_LAUNCH(random_fill_kernel, dim3(grid_for((n + 3) / 4, TPB * 2)), dim3(TPB), 0, ctx().stream, out, n, seed, offset,
                        mode);
     return check_launch("random_fill");
 }
@@ -119,7 +119,7 @@ __global__ void dropout_kernel(float *__restrict__ out, const float *__restrict_
 int k_dropout(float *out, const float *x, int64_t n, float rate, float scale, uint64_t seed, uint64_t offset) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(dropout_kernel, dim3(grid_for((n + 3) / 4, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, n, rate, scale,
+    MNI_KERNEL_LAUNCH(dropout_kernel, dim3(grid_for((n + 3) / 4, TPB * 2)), dim3(TPB), 0, ctx().stream, out, x, n, rate, scale,
                        seed, offset);
     return check_launch("dropout");
 }
@@ -142,7 +142,7 @@ int k_sample_windows(int32_t *inputs, int32_t *targets, const int32_t *data, con
     const int64_t total = block * batch;
     if (total <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(sample_windows_kernel, dim3(grid_for(total, TPB)), dim3(TPB), 0, ctx().stream, inputs, targets, data,
+    MNI_KERNEL_LAUNCH(sample_windows_kernel, dim3(grid_for(total, TPB)), dim3(TPB), 0, ctx().stream, inputs, targets, data,
                        starts, block, total);
     return check_launch("sample_windows");
 }
@@ -170,10 +170,10 @@ int k_embedding_forward(float *out, const float *w, const int32_t *idx, int64_t 
     if (tokens <= 0 || dim <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
     if ((dim % 4) == 0 && al16(out) && al16(w))
-        hipLaunchKernelGGL(embedding_gather4_kernel, dim3(grid_for(tokens * dim / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
+        MNI_KERNEL_LAUNCH(embedding_gather4_kernel, dim3(grid_for(tokens * dim / 4, TPB * 2)), dim3(TPB), 0, ctx().stream,
                            reinterpret_cast<float4 *>(out), reinterpret_cast<const float4 *>(w), idx, dim / 4, tokens * dim / 4);
     else
-        hipLaunchKernelGGL(embedding_gather_kernel, dim3(grid_for(tokens * dim, TPB * 2)), dim3(TPB), 0, ctx().stream, out, w,
+        MNI_KERNEL_LAUNCH(embedding_gather_kernel, dim3(grid_for(tokens * dim, TPB * 2)), dim3(TPB), 0, ctx().stream, out, w,
                            idx, dim, tokens * dim);
     return check_launch("embedding_forward");
 }
@@ -278,28 +278,28 @@ int k_embedding_backward(float *dw, const float *g, const int32_t *idx, int64_t 
     MNI_TRY(k_fill(reinterpret_cast<float *>(count), 0.0f, 2 * vocab));
     hipStream_t st = ctx().stream;
     if (tokens > 0) {
-        hipLaunchKernelGGL(emb_count_kernel, dim3(grid_for(tokens, TPB)), dim3(TPB), 0, st, count, idx, tokens);
+        MNI_KERNEL_LAUNCH(emb_count_kernel, dim3(grid_for(tokens, TPB)), dim3(TPB), 0, st, count, idx, tokens);
         MNI_TRY(check_launch("embedding_count"));
     }
-    hipLaunchKernelGGL(emb_scan_kernel, dim3(1), dim3(1024), 0, st, start, (const int32_t *)count, vocab);
+    MNI_KERNEL_LAUNCH(emb_scan_kernel, dim3(1), dim3(1024), 0, st, start, (const int32_t *)count, vocab);
     MNI_TRY(check_launch("embedding_scan"));
     if (tokens > 0) {
-        hipLaunchKernelGGL(emb_fill_kernel, dim3(grid_for(tokens, TPB)), dim3(TPB), 0, st, list, cursor, (const int32_t *)start,
+        MNI_KERNEL_LAUNCH(emb_fill_kernel, dim3(grid_for(tokens, TPB)), dim3(TPB), 0, st, list, cursor, (const int32_t *)start,
                            idx, tokens);
         MNI_TRY(check_launch("embedding_fill"));
-        hipLaunchKernelGGL(emb_order_kernel, dim3(grid_for(tokens, TPB)), dim3(TPB), 0, st, sorted, (const int32_t *)list,
+        MNI_KERNEL_LAUNCH(emb_order_kernel, dim3(grid_for(tokens, TPB)), dim3(TPB), 0, st, sorted, (const int32_t *)list,
                            (const int32_t *)start, idx, tokens);
         MNI_TRY(check_launch("embedding_order"));
     }
     if ((dim % 4) == 0 && al16(dw) && al16(g)) {
         const int64_t dimv = dim / 4;
         const int threads = dimv >= 256 ? 256 : dimv >= 128 ? 128 : 64;
-        hipLaunchKernelGGL(emb_accumulate_kernel<float4>, dim3((unsigned)vocab, 1), dim3(threads), 0, st,
+        MNI_KERNEL_LAUNCH(emb_accumulate_kernel<float4>, dim3((unsigned)vocab, 1), dim3(threads), 0, st,
                            reinterpret_cast<float4 *>(dw), reinterpret_cast<const float4 *>(g), (const int32_t *)sorted,
                            (const int32_t *)start, dimv);
     } else {
         const int threads = dim >= 256 ? 256 : dim >= 128 ? 128 : 64;
-        hipLaunchKernelGGL(emb_accumulate_kernel<float>, dim3((unsigned)vocab, 1), dim3(threads), 0, st, dw, g,
+        MNI_KERNEL_LAUNCH(emb_accumulate_kernel<float>, dim3((unsigned)vocab, 1), dim3(threads), 0, st, dw, g,
                            (const int32_t *)sorted, (const int32_t *)start, dim);
     }
     return check_launch("embedding_accumulate");
@@ -341,7 +341,7 @@ int k_tile(float *out, const float *in, const int64_t *in_shape, const int64_t *
     }
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(tile_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, in, d, n);
+    MNI_KERNEL_LAUNCH(tile_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, out, in, d, n);
     return check_launch("tile");
 }
 
@@ -379,7 +379,7 @@ int k_residual_layernorm(float *out, float *res, float *mean, float *rstd, const
                          const float *gamma, const float *beta, int64_t rows, int64_t c, float eps) {
     if (rows <= 0 || c <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(residual_layernorm_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, res, mean, rstd, x,
+    MNI_KERNEL_LAUNCH(residual_layernorm_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, res, mean, rstd, x,
                        residual, gamma, beta, rows, c, eps);
     return check_launch("residual_layernorm");
 }
@@ -401,7 +401,7 @@ __global__ void scale_check_kernel(float *__restrict__ g, float s, int64_t n, fl
 int k_scale_check(float *g, float s, int64_t n, float *flag) {
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    hipLaunchKernelGGL(scale_check_kernel, dim3(grid_for(n, TPB * 4)), dim3(TPB), 0, ctx().stream, g, s, n, flag);
+    MNI_KERNEL_LAUNCH(scale_check_kernel, dim3(grid_for(n, TPB * 4)), dim3(TPB), 0, ctx().stream, g, s, n, flag);
     return check_launch("scale_check");
 }
 

@@ -94,18 +94,18 @@ extern "C" int mni_rocm_yardstick_timed(int kind, int nontemporal, void *dst, co
     auto launch = [&](int it) {
         const f32x4 *src = reads ? (const f32x4 *)srcs[it % nsrc] : nullptr;
         switch (kind) {
-        case MNI_YARDSTICK_EMPTY: hipLaunchKernelGGL(ys_empty_kernel, dim3(1), dim3(64), 0, c.stream); break;
+        case MNI_YARDSTICK_EMPTY: MNI_KERNEL_LAUNCH(ys_empty_kernel, dim3(1), dim3(64), 0, c.stream); break;
         case MNI_YARDSTICK_READ:
-            if (nontemporal) hipLaunchKernelGGL((ys_read_kernel<true>), grid, block, 0, c.stream, src, n4, sink);
-            else hipLaunchKernelGGL((ys_read_kernel<false>), grid, block, 0, c.stream, src, n4, sink);
+            if (nontemporal) MNI_KERNEL_LAUNCH((ys_read_kernel<true>), grid, block, 0, c.stream, src, n4, sink);
+            else MNI_KERNEL_LAUNCH((ys_read_kernel<false>), grid, block, 0, c.stream, src, n4, sink);
             break;
         case MNI_YARDSTICK_WRITE:
-            if (nontemporal) hipLaunchKernelGGL((ys_write_kernel<true>), grid, block, 0, c.stream, (f32x4 *)dst, n4, 1.0f);
-            else hipLaunchKernelGGL((ys_write_kernel<false>), grid, block, 0, c.stream, (f32x4 *)dst, n4, 1.0f);
+            if (nontemporal) MNI_KERNEL_LAUNCH((ys_write_kernel<true>), grid, block, 0, c.stream, (f32x4 *)dst, n4, 1.0f);
+            else MNI_KERNEL_LAUNCH((ys_write_kernel<false>), grid, block, 0, c.stream, (f32x4 *)dst, n4, 1.0f);
             break;
         default:
-            if (nontemporal) hipLaunchKernelGGL((ys_copy_kernel<true>), grid, block, 0, c.stream, (f32x4 *)dst, src, n4);
-            else hipLaunchKernelGGL((ys_copy_kernel<false>), grid, block, 0, c.stream, (f32x4 *)dst, src, n4);
+            if (nontemporal) MNI_KERNEL_LAUNCH((ys_copy_kernel<true>), grid, block, 0, c.stream, (f32x4 *)dst, src, n4);
+            else MNI_KERNEL_LAUNCH((ys_copy_kernel<false>), grid, block, 0, c.stream, (f32x4 *)dst, src, n4);
         }
     };
     int it = 0;

@@ -61,6 +61,7 @@ SIGNATURES = {
     "mni_rocm_d2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "mni_rocm_sync": (C.c_int, []),
     "mni_rocm_test_raise_device_status": (C.c_int, [C.c_uint]),
+    "mni_rocm_launch_count": (C.c_uint64, []),
     "mni_rocm_event_create": (C.c_int, [C.POINTER(C.c_void_p)]),
     "mni_rocm_event_record": (C.c_int, [C.c_void_p]),
     "mni_rocm_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
@@ -225,6 +226,9 @@ class Rocm:
 
     def test_raise_device_status(self, code):
         self._check(self.lib.mni_rocm_test_raise_device_status(code))
+
+    def launch_count(self):
+        return int(self.lib.mni_rocm_launch_count())
 
     def event(self):
         e = C.c_void_p()

@@ -83,6 +83,10 @@ int mni_rocm_sync(void);
  * making a kernel hang.  No counterpart in the reference. */
 int mni_rocm_test_raise_device_status(unsigned code);
 
+/* Kernels launched by the library since it was loaded (copies not counted):
+ * what a latency-bound training step is made of.  No counterpart in the reference. */
+uint64_t mni_rocm_launch_count(void);
+
 /* Stream-ordered timing marks on the library's stream (HIP events). */
 int mni_rocm_event_create(void **event);
 int mni_rocm_event_record(void *event);
