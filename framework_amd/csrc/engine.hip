@@ -121,6 +121,15 @@ struct Engine {
     bool rng_ready = false;
     uint64_t rng_seed = 0, rng_offset = 0;
     std::mt19937_64 host_rng;
+    // While Tape::backward runs: what a fused Linear needs to see of the walk in order to hand the
+    // gradient of its input straight through the GELU of the Linear that produced it.
+    const Tape *bw_tape = nullptr;
+    const std::vector<int64_t> *bw_out2entry = nullptr;  // tensor id -> tape entry that produced it
+    const std::vector<int> *bw_consumers = nullptr;      // tensor id -> tape entries that read it
+    const std::vector<int64_t> *bw_grads = nullptr;      // tensor id -> gradient gathered so far
+    // output id of a GELU Linear -> its bias gradient, when the gradient that reaches it has already been
+    // taken through gelu' by the entry that consumed it
+    std::map<uint32_t, uint32_t> preact_db;
 };
 static Engine &eng() {
     // Never destroyed: releasing device buffers from a static destructor would
@@ -339,7 +348,9 @@ static int make_operand(const Tensor &t, bool transpose, mni_operand *op, BufP *
 // C = op(A) * op(B) on tensors, batch rule of ops/matmul.rs:54-60.
 // ta / tb: use the operand with its last two dims swapped (transpose_last2,
 // ops/matmul.rs:258-284, without the copy).
-static uint32_t matmul_tensors(uint32_t a, bool ta, uint32_t b, bool tb, const float *bias, int epilogue) {
+// aux / colsum_part: the second buffer and the strip sums of the MNI_EPI_BIAS_GELU_DUAL / MNI_EPI_DGELU epilogues.
+static uint32_t matmul_tensors(uint32_t a, bool ta, uint32_t b, bool tb, const float *bias, int epilogue, float *aux = nullptr,
+                               float *colsum_part = nullptr) {
     Tensor *A = get(a), *B = get(b);
     if (!A || !B) return MNI_BAD_ID;
     const int and_ = (int)A->shape.size(), bnd = (int)B->shape.size();
@@ -378,6 +389,7 @@ static uint32_t matmul_tensors(uint32_t a, bool ta, uint32_t b, bool tb, const f
     d.M = m; d.N = n; d.K = k; d.batch = batch;
     d.C = out->p; d.ldc = n; d.c_batch_stride = m * n;
     d.bias = bias; d.epilogue = epilogue;
+    d.aux = aux; d.colsum_part = colsum_part;
     if (sgemm(d) != MNI_OK) return MNI_BAD_ID;
     return insert_contig(std::move(out), out_shape);
 }
@@ -413,7 +425,14 @@ static uint32_t unbroadcast_tensor(uint32_t full, const Shape &orig_shape) {
 
 // ops/matmul.rs:199-222 matmul_backward: dA = unbroadcast(dC * B^T),
 // dB = unbroadcast(A^T * dC); both always.
-static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out) {
+// through_gelu (fused Linear only): A is the output of a GELU Linear with pre-activation z and bias; dA then
+// leaves the product already multiplied by gelu'(z + bias), with its strip sums in colsum_part.
+struct ThroughGelu {
+    const float *bias;
+    float *z;
+    float *colsum_part;
+};
+static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out, const ThroughGelu *through_gelu = nullptr) {
     const uint32_t a = e.inputs[0], b = e.inputs[1];
     Tensor *A = get(a), *B = get(b), *G = get(grad);
     if (!A || !B || !G) return MNI_ERR_FREED;
@@ -421,7 +440,9 @@ static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out) {
 
     // dA
     {
-        const uint32_t full = matmul_tensors(grad, false, b, true, nullptr, MNI_EPI_NONE);
+        const uint32_t full = through_gelu ? matmul_tensors(grad, false, b, true, through_gelu->bias, MNI_EPI_DGELU, through_gelu->z,
+                                                            through_gelu->colsum_part)
+                                           : matmul_tensors(grad, false, b, true, nullptr, MNI_EPI_NONE);
         if (full == MNI_BAD_ID) return MNI_ERR_INVALID;
         const uint32_t ga = unbroadcast_tensor(full, a_shape);
         free_tensor(full);
@@ -1250,19 +1271,20 @@ static uint32_t linear_op(uint32_t x, uint32_t w, uint32_t bias, int act) {
         set_error(MNI_ERR_INVALID, "linear: bias must be a contiguous [out] vector");
         return MNI_BAD_ID;
     }
-    // GELU needs its pre-activation in backward: the product is kept without
-    // the bias and one pass applies bias + GELU (ops/fused.rs:247-273); plain
-    // bias and ReLU ride in the GEMM epilogue.
+    // GELU needs its pre-activation in backward: the product's epilogue writes it (without the bias) and
+    // gelu(product + bias) side by side (the reference fuses bias + GELU into one pass after the product,
+    // ops/fused.rs:247-273); plain bias and ReLU ride in the epilogue as one output.
     const BufP bias_buf = Bv->buf;
     uint32_t out, aux = MNI_BAD_ID;
     if (act == MNI_EPI_BIAS_GELU) {
-        aux = matmul_tensors(x, false, w, false, nullptr, MNI_EPI_NONE);
+        int64_t n_out = W->shape[1];
+        for (size_t i = 0; i + 1 < X->shape.size(); ++i) n_out *= X->shape[i];
+        BufP o = new_buf((size_t)(n_out > 0 ? n_out : 1));
+        if (!o) return MNI_BAD_ID;
+        aux = matmul_tensors(x, false, w, false, bias_buf->p, MNI_EPI_BIAS_GELU_DUAL, o->p);
         if (aux == MNI_BAD_ID) return MNI_BAD_ID;
-        Tensor *Z = get(aux);
-        const int64_t c = Z->shape.back();
-        BufP o = new_buf((size_t)Z->size);
-        if (!o || k_bias_gelu(o->p, Z->buf->p, bias_buf->p, c ? Z->size / c : 0, c) != MNI_OK) return MNI_BAD_ID;
-        out = insert_contig(std::move(o), Z->shape);
+        const Shape zshape = get(aux)->shape;
+        out = insert_contig(std::move(o), zshape);
     } else {
         out = matmul_tensors(x, false, w, false, bias_buf->p, act);
         if (out == MNI_BAD_ID) return MNI_BAD_ID;
@@ -1278,7 +1300,14 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
     uint32_t g = grad;
     bool own_g = false;
     int64_t db_id = -1;
-    if (e.act == MNI_EPI_BIAS_GELU) {
+    Engine &en = eng();
+    const auto pre = en.preact_db.find(e.output_id);
+    if (e.act == MNI_EPI_BIAS_GELU && pre != en.preact_db.end()) {
+        // the entry that consumed this layer's output has already taken the gradient through gelu'
+        // (in the epilogue of its own product) and summed the bias gradient
+        db_id = pre->second;
+        en.preact_db.erase(pre);
+    } else if (e.act == MNI_EPI_BIAS_GELU) {
         // dZ = dOut * gelu'(z + bias) and db = column sums of dZ in one pass (ops/fused.rs:316-351)
         Tensor *G = get(grad), *Z = get(e.aux), *Bv = get(e.inputs[2]);
         if (!G || !Z || !Bv) return MNI_ERR_FREED;
@@ -1306,7 +1335,48 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
     }
     Entry mm;
     mm.op = OP_MATMUL; mm.n_inputs = 2; mm.inputs[0] = e.inputs[0]; mm.inputs[1] = e.inputs[1];
-    int rc = matmul_backward(g, mm, out);
+    // Is the input the output of a GELU Linear that nobody else reads?  Then dX leaves this layer's product
+    // as dZ of that one: gelu'(z + bias) applied and the bias gradient's strip sums taken in the epilogue
+    // (instead of a pass over dX and z of its own), and that layer's backward starts from dZ.
+    ThroughGelu tg = {nullptr, nullptr, nullptr};
+    BufP strips;
+    uint32_t producer_out = MNI_BAD_ID;
+    int64_t strip_rows = 0, strip_cols = 0;
+    if (en.bw_tape) {
+        const uint32_t x = e.inputs[0];
+        Tensor *X = get(x);
+        const int64_t pi = x < en.bw_out2entry->size() ? (*en.bw_out2entry)[x] : -1;
+        if (X && pi >= 0 && !X->requires_grad && is_contiguous(*X) && X->shape.size() >= 2 && (*en.bw_consumers)[x] == 1 &&
+            (*en.bw_grads)[x] < 0) {
+            const Entry &P = en.bw_tape->entries[(size_t)pi];
+            Tensor *Z = P.op == OP_LINEAR && P.act == MNI_EPI_BIAS_GELU && P.output_id == x ? get(P.aux) : nullptr;
+            Tensor *PB = Z ? get(P.inputs[2]) : nullptr;
+            if (Z && PB && is_contiguous(*Z) && Z->shape == X->shape && en.preact_db.find(x) == en.preact_db.end()) {
+                strip_cols = X->shape.back();
+                const int64_t m = X->shape[X->shape.size() - 2];
+                strip_rows = mni_rocm_sgemm_colsum_rows(m, strip_cols && m ? X->size / (strip_cols * m) : 0);
+                if (strip_rows > 0 && strip_cols > 0) strips = new_buf((size_t)(strip_rows * strip_cols));
+                if (strips) {
+                    tg.bias = PB->buf->p;
+                    tg.z = Z->buf->p;
+                    tg.colsum_part = strips->p;
+                    producer_out = x;
+                }
+            }
+        }
+    }
+    int rc = matmul_backward(g, mm, out, tg.z ? &tg : nullptr);
+    if (rc == MNI_OK && tg.z) {
+        // bias gradient of the producing layer: the strips added up, in strip order
+        Tensor *PB = get(en.bw_tape->entries[(size_t)(*en.bw_out2entry)[producer_out]].inputs[2]);
+        BufP db = PB ? new_buf((size_t)strip_cols) : nullptr;
+        if (!db) rc = MNI_ERR_NOMEM;
+        else rc = k_colsum(db->p, strips->p, strip_rows, strip_cols);
+        if (rc == MNI_OK) {
+            const Shape bshape = PB->shape;
+            en.preact_db[producer_out] = insert_contig(std::move(db), bshape);
+        }
+    }
     if (rc == MNI_OK) {
         if (db_id >= 0) out[2] = db_id;
         else {
@@ -1731,7 +1801,24 @@ static int tape_backward(Tape &tp, uint32_t loss) {
             }
         }
     }
+    // how many entries read each tensor (what the fused Linear's backward needs to know, see linear_backward)
+    std::vector<int> consumers(nslots, 0);
+    for (const Entry &en : tp.entries)
+        if (en.output_id < nslots && relevant[en.output_id])
+            for (int i = 0; i < en.n_inputs; ++i)
+                if (en.inputs[i] < nslots) ++consumers[en.inputs[i]];
     std::vector<int64_t> grads(nslots, -1);
+    struct WalkScope {  // publishes the walk to the ops for the duration of this call
+        Engine &e;
+        WalkScope(Engine &e_, const Tape *t, const std::vector<int64_t> *o, const std::vector<int> *c, const std::vector<int64_t> *g) : e(e_) {
+            e.bw_tape = t; e.bw_out2entry = o; e.bw_consumers = c; e.bw_grads = g;
+        }
+        ~WalkScope() {
+            e.bw_tape = nullptr; e.bw_out2entry = nullptr; e.bw_consumers = nullptr; e.bw_grads = nullptr;
+            for (auto &kv : e.preact_db) free_tensor(kv.second);  // (none are left when the walk completed)
+            e.preact_db.clear();
+        }
+    } walk_scope(eng(), &tp, &out2entry, &consumers, &grads);
     {
         const Shape shape = get(loss)->shape;
         const uint32_t g = filled(shape, 1.0f);  // ones_like for any loss shape, autograd.rs:143

@@ -29,8 +29,17 @@ static int validate(const mni_gemm_desc &d) {
     if (d.A.batch_count < 1 || d.B.batch_count < 1)
         return set_error(MNI_ERR_INVALID, "sgemm: operand batch_count must be >= 1");
     if (d.ldc < d.N) return set_error(MNI_ERR_INVALID, "sgemm: ldc (%lld) < N (%lld)", (long long)d.ldc, (long long)d.N);
-    if (d.epilogue < MNI_EPI_NONE || d.epilogue > MNI_EPI_BIAS_GELU)
+    if (d.epilogue < MNI_EPI_NONE || d.epilogue > MNI_EPI_DGELU)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown epilogue %d", d.epilogue);
+    if (d.epilogue >= MNI_EPI_BIAS_GELU_DUAL) {
+        if (!d.aux) return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs the aux pointer", d.epilogue);
+        if (d.accumulate || d.split_k > 1)
+            return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d takes neither accumulate nor split_k", d.epilogue);
+        if (d.algo != MNI_ALGO_AUTO && d.algo != MNI_ALGO_MFMA && d.algo != MNI_ALGO_MFMA_SMALL)
+            return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d runs on the MFMA tile kernel only", d.epilogue);
+    }
+    if (d.colsum_part && d.epilogue != MNI_EPI_DGELU)
+        return set_error(MNI_ERR_INVALID, "sgemm: colsum_part goes with the DGELU epilogue only");
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
@@ -214,7 +223,8 @@ static int run_mfma(const mni_gemm_desc &d) {
     const int bmode = g.K == 0 ? 2 : classify(g.b_rs, g.b_cs);
 
     // Short-K panel form: forced, or chosen when its 128 x 128 tiles fill the machine.
-    if (d.algo == MNI_ALGO_PANEL || (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_panel_eligible(g, amode, bmode) && panel_plan(g, cus))) {
+    if (d.algo == MNI_ALGO_PANEL || (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.epilogue < MNI_EPI_BIAS_GELU_DUAL &&
+                                     gemm_panel_eligible(g, amode, bmode) && panel_plan(g, cus))) {
         if (!gemm_panel_eligible(g, amode, bmode))
             return set_error(MNI_ERR_INVALID, "sgemm: the short-K panel kernel takes two K-contiguous operands with K <= 64, K %% 4 == 0");
         if (d.split_k > 1) return set_error(MNI_ERR_INVALID, "sgemm: the short-K panel kernel takes no split_k");
@@ -235,7 +245,7 @@ static int run_mfma(const mni_gemm_desc &d) {
             if (d.split_k != 0 && d.split_k != 1 && d.split_k != 4)
                 return set_error(MNI_ERR_INVALID, "sgemm: the direct kernel takes split_k 0, 1 or 4");
             ksplit = d.split_k == 4 ? 4 : 1;
-        } else if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_direct_eligible(g, amode, bmode)) {
+        } else if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.epilogue < MNI_EPI_BIAS_GELU_DUAL && gemm_direct_eligible(g, amode, bmode)) {
             ksplit = direct_plan(g, cus);
         }
         if (ksplit) {
@@ -275,7 +285,14 @@ static int run_mfma(const mni_gemm_desc &d) {
     int bm = g.M <= 64 ? 64 : 128, bn = g.N <= 64 ? 64 : 128;
     bool streamk = false;
     bool whole_tiles = false;  // one workgroup per tile, no K slices
-    if (d.algo == MNI_ALGO_MFMA_SMALL) {
+    // The two-output and the gelu'-scaling epilogues exist in the one-workgroup-per-tile form only;
+    // strip sums for the bias gradient are laid out for 128-row tiles.
+    const bool fused_gelu = d.epilogue >= MNI_EPI_BIAS_GELU_DUAL;
+    if (fused_gelu) {
+        whole_tiles = true;
+        if (d.algo == MNI_ALGO_MFMA_SMALL) bm = bn = 64;
+        if (d.colsum_part) bm = 128;
+    } else if (d.algo == MNI_ALGO_MFMA_SMALL) {
         bm = bn = 64;
     } else if (d.algo == MNI_ALGO_AUTO || d.algo == MNI_ALGO_MFMA_STREAMK) {
         const int64_t big_tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
@@ -332,6 +349,13 @@ static int run_mfma(const mni_gemm_desc &d) {
     g.tiles_n = (g.N + bn - 1) / bn;
 
     g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
+    if (fused_gelu) {
+        g.split_k = 1;
+        g.k_per_slice = g.K > 0 ? g.K : 1;
+        g.aux_out = d.aux;                // shares its slot with the K-slice partials, which this form never has
+        g.colsum_part = d.colsum_part;    // shares its slot with the stream-K marks
+        return launch_gemm_mfma(g, amode, bmode, bm, bn);
+    }
     void *ws = nullptr;
     if (streamk) {
         g.split_k = 1;
@@ -384,7 +408,7 @@ int sgemm(const mni_gemm_desc &d) {
     MNI_TRY(ensure_init());
     MNI_TRY(validate(d));
     if (d.M == 0 || d.N == 0 || d.batch == 0) return MNI_OK;
-    if (d.algo == MNI_ALGO_AUTO || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS) {
+    if ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS) {
         int rc;
         if (try_skinny(d, &rc)) return rc;
         if (d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS)
@@ -401,6 +425,12 @@ extern "C" int mni_rocm_sgemm(const mni_gemm_desc *desc) {
     MNI_API_GUARD;
     if (!desc) return mni::set_error(MNI_ERR_INVALID, "sgemm: null descriptor");
     return mni::sgemm(*desc);
+}
+
+extern "C" int64_t mni_rocm_sgemm_colsum_rows(int64_t M, int64_t batch) {
+    // two strips per 128-row tile (the planner keeps 128-row tiles when strip sums are asked for)
+    if (M <= 0 || batch <= 0) return 0;
+    return batch * ((M + 127) / 128) * 2;
 }
 
 extern "C" int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms) {

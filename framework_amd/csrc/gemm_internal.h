@@ -12,7 +12,16 @@ struct GemmLaunch {
     const float *B;
     float *C;
     const float *bias;
-    float *ws;  // split-K partials [slice][batch][M][N]
+    // One pointer, three mutually exclusive uses (a fourth 64-byte line of kernel
+    // arguments would cost every launch a further scalar fetch): the split-K /
+    // stream-K partials; with MNI_EPI_BIAS_GELU_DUAL the second output
+    // gelu(C + bias), laid out like C; with MNI_EPI_DGELU the saved
+    // pre-activation z (C then becomes acc * gelu'(z + bias)), laid out like C.
+    union {
+        float *ws;  // split-K partials [slice][batch][M][N]
+        float *aux_out;
+        const float *aux_in;
+    };
     int M, N, K, batch;
     int64_t a_rs, a_cs, a_bs;
     int64_t b_rs, b_cs, b_bs;
@@ -25,7 +34,12 @@ struct GemmLaunch {
     // persistent workgroups; `ws` then holds one tile-sized partial per
     // workgroup and sk_flags one arrival mark per workgroup, set to sk_epoch.
     int streamk, sk_wpx, sk_xcds;
-    unsigned *sk_flags;
+    // stream-K arrival marks; with MNI_EPI_DGELU (never stream-K) the column sums
+    // of C per 64-row (32-row for 64-row tiles) strip, [batch][2 tiles_m][N], or null
+    union {
+        unsigned *sk_flags;
+        float *colsum_part;
+    };
     unsigned sk_epoch;
     unsigned *status;  // device status word: set when a finisher's bounded wait expires
 };

@@ -243,10 +243,29 @@ __device__ __forceinline__ void tile_piece(int x, float4 *__restrict__ tile, con
     }
 }
 
+// tanh through the hardware's exp2 and reciprocal: 1 - 2 / (1 + e^{2x}) (exact limits at both ends, absolute
+// error ~1e-6).  The library's tanhf costs some forty instructions, and an epilogue that calls it once per
+// element while the matrix pipe waits made the fused GELU products 25 us slower than the plain ones plus a
+// separate pass; this form costs five.
+__device__ __forceinline__ float fast_tanh(float x) {
+    const float t = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);  // e^{2x} = 2^{2x log2(e)}
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + t);
+}
+
 __device__ __forceinline__ float gelu_tanh(float x) {
     // tanh-approximation GELU of the reference (src/native/src/ops/activation.rs:15-18)
     const float s = 0.7978845608028654f;  // sqrt(2/pi)
-    return 0.5f * x * (1.0f + tanhf(s * (x + 0.044715f * x * x * x)));
+    return 0.5f * x * (1.0f + fast_tanh(s * (x + 0.044715f * x * x * x)));
+}
+
+__device__ __forceinline__ float gelu_tanh_grad(float x) {
+    // src/native/src/ops/activation.rs:20-28
+    const float s = 0.7978845608028654f;
+    const float inner = s * (x + 0.044715f * x * x * x);
+    const float th = fast_tanh(inner);
+    const float sech2 = 1.0f - th * th;
+    const float d_inner = s * (1.0f + 3.0f * 0.044715f * x * x);
+    return 0.5f * (1.0f + th) + 0.5f * x * sech2 * d_inner;
 }
 
 __device__ __forceinline__ float pick(const float4 &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
@@ -635,6 +654,11 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         if (lost && tid == 0) *g.status = DEVICE_STATUS_STREAMK_WAIT;
     }
     float *const slot = g.ws + (int64_t)bid * (BM * BN);  // ROLE_PART: where this workgroup parks its tile
+    // Fused backward of a GELU layer (MNI_EPI_DGELU, whole tiles only): the lane's four columns, summed
+    // over the rows of this wavefront's strip, on the way to the bias gradient.
+    const bool dual = !SK && !partial && g.epilogue == MNI_EPI_BIAS_GELU_DUAL;
+    const bool dgelu = !SK && !partial && g.epilogue == MNI_EPI_DGELU;
+    float csum[4] = {0.f, 0.f, 0.f, 0.f};
     // all wavefronts are past their last LDS read (barrier at the end of the K loop)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -671,7 +695,39 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
             }
             if (row < g.M && col < g.N) {
                 float *dst = Cb + (int64_t)row * ldc + col;
-                if (!partial) {
+                if (dual) {
+                    // C keeps the product; the activated value goes to the second output, laid out like C
+                    float *dst2 = g.aux_out + (int64_t)batch * g.c_bs + (int64_t)row * ldc + col;
+                    float w[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) w[e] = gelu_tanh(v[e] + bias4[e]);
+                    if (col + 3 < g.N) {
+                        typedef float f32x4_t __attribute__((ext_vector_type(4)));
+                        const f32x4_t o4 = {w[0], w[1], w[2], w[3]};
+                        __builtin_nontemporal_store(o4, reinterpret_cast<f32x4_t *>(dst2));
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < g.N) dst2[e] = w[e];
+                    }
+                } else if (dgelu) {
+                    // C = product * gelu'(z + bias), z the saved pre-activation laid out like C
+                    const float *zp = g.aux_in + (int64_t)batch * g.c_bs + (int64_t)row * ldc + col;
+                    float z[4] = {0.f, 0.f, 0.f, 0.f};
+                    if (col + 3 < g.N) {
+                        const float4 z4 = *reinterpret_cast<const float4 *>(zp);
+                        z[0] = z4.x; z[1] = z4.y; z[2] = z4.z; z[3] = z4.w;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < g.N) z[e] = zp[e];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = col + e < g.N ? v[e] * gelu_tanh_grad(z[e] + bias4[e]) : 0.0f;
+                        csum[e] += v[e];
+                    }
+                } else if (!partial) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         v[e] += bias4[e];
@@ -698,6 +754,20 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
             }
         }
         __syncthreads();
+    }
+    if (dgelu && g.colsum_part) {
+        // lanes that share columns (same lane % LANES_PER_ROW) are added by butterfly steps; strip
+        // (batch, tile row, wm) owns one row of the partial matrix
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int off = LANES_PER_ROW; off < 64; off <<= 1) csum[e] += __shfl_xor(csum[e], off, 64);
+        if (lane < LANES_PER_ROW) {
+            float *cp = g.colsum_part + (((int64_t)batch * g.tiles_m + tm) * 2 + wm) * (int64_t)g.N;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < g.N) cp[col + e] = csum[e];
+        }
     }
     if (SK && role == ROLE_PART) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of the tile has reached L2

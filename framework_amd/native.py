@@ -22,7 +22,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmni_rocm.so")
 
 BAD_ID = 0xFFFFFFFF
 MAX_DIMS = 8
-EPI_NONE, EPI_BIAS, EPI_BIAS_RELU, EPI_BIAS_GELU = 0, 1, 2, 3
+EPI_NONE, EPI_BIAS, EPI_BIAS_RELU, EPI_BIAS_GELU, EPI_BIAS_GELU_DUAL, EPI_DGELU = 0, 1, 2, 3, 4, 5
 ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL, ALGO_SKINNY_TWO_PASS, ALGO_MFMA_STREAMK, ALGO_DIRECT, ALGO_PANEL = 0, 1, 2, 3, 4, 5, 6, 7
 
 _f32p = C.POINTER(C.c_float)
@@ -44,7 +44,7 @@ class GemmDesc(C.Structure):
                 ("A", Operand), ("B", Operand),
                 ("C", C.c_void_p), ("ldc", C.c_int64), ("c_batch_stride", C.c_int64),
                 ("bias", C.c_void_p), ("epilogue", C.c_int32), ("accumulate", C.c_int32),
-                ("split_k", C.c_int32), ("algo", C.c_int32)]
+                ("split_k", C.c_int32), ("algo", C.c_int32), ("aux", C.c_void_p), ("colsum_part", C.c_void_p)]
 
 
 # name -> (restype, argtypes): every symbol include/mni_rocm.h declares.
@@ -67,6 +67,7 @@ SIGNATURES = {
     "mni_rocm_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "mni_rocm_event_destroy": (C.c_int, [C.c_void_p]),
     "mni_rocm_sgemm": (C.c_int, [C.POINTER(GemmDesc)]),
+    "mni_rocm_sgemm_colsum_rows": (C.c_int64, [C.c_int64, C.c_int64]),
     "mni_rocm_sgemm_noalloc": (C.c_int, [C.POINTER(GemmDesc)]),
     "mni_rocm_sgemm_noalloc_workspace_bytes": (C.c_size_t, []),
     "mni_rocm_sgemm_timed": (C.c_int, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
@@ -260,6 +261,9 @@ class Rocm:
     def sgemm_noalloc_workspace_bytes(self):
         return int(self.lib.mni_rocm_sgemm_noalloc_workspace_bytes())
 
+    def sgemm_colsum_rows(self, M, batch=1):
+        return int(self.lib.mni_rocm_sgemm_colsum_rows(M, batch))
+
     def sgemm_timed(self, descs, warmup, iters):
         """Average ms per launch of the products in `descs` (made by gemm_desc),
         cycled back to back and issued from C."""
@@ -270,7 +274,8 @@ class Rocm:
 
     @staticmethod
     def gemm_desc(M, N, K, A, B, Cptr, *, batch=1, a_strides=None, b_strides=None, a_batch=(0, 1), b_batch=(0, 1),
-                  ldc=None, c_batch_stride=None, bias=None, epilogue=EPI_NONE, accumulate=False, split_k=0, algo=ALGO_AUTO):
+                  ldc=None, c_batch_stride=None, bias=None, epilogue=EPI_NONE, accumulate=False, split_k=0, algo=ALGO_AUTO,
+                  aux=None, colsum_part=None):
         d = GemmDesc()
         d.M, d.N, d.K, d.batch = M, N, K, batch
         ars, acs = a_strides if a_strides is not None else (K, 1)
@@ -285,6 +290,8 @@ class Rocm:
         d.accumulate = 1 if accumulate else 0
         d.split_k = split_k
         d.algo = algo
+        d.aux = aux
+        d.colsum_part = colsum_part
         return d
 
     def yardstick_timed(self, kind, nbytes, dst=None, srcs=(), nontemporal=True, blocks_per_cu=8, warmup=5, iters=50):

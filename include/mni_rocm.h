@@ -106,7 +106,14 @@ typedef struct {
     int64_t batch_count; /* >= 1 */
 } mni_operand;
 
-enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_GELU = 3 };
+/* NONE .. BIAS_GELU: C = f(product + bias).  The last two carry the fused Linear of a GELU layer through its
+ * backward (the reference fuses bias + GELU and their backward outside the product, src/native/src/ops/fused.rs:247-351):
+ *   BIAS_GELU_DUAL  C = product (the pre-activation without its bias, which the backward needs) and
+ *                   aux = gelu(product + bias), written by the same epilogue;
+ *   DGELU           C = product * gelu'(aux + bias) with aux the saved pre-activation, and, when colsum_part is
+ *                   given, the column sums of C per strip of rows (summed afterwards: the bias gradient).
+ * Both need `aux` laid out like C (same ldc and batch stride) and take no accumulate and no split_k. */
+enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_GELU = 3, MNI_EPI_BIAS_GELU_DUAL = 4, MNI_EPI_DGELU = 5 };
 /* MFMA = the MFMA tile kernel, one workgroup per tile and K slice, 128-wide tiles;
  * MFMA_SMALL = the same forced to 64 x 64 tiles; MFMA_STREAMK = the tile kernel
  * with the K steps of all tiles dealt evenly over a resident grid (error if the
@@ -142,8 +149,12 @@ typedef struct {
     int32_t accumulate;  /* non-zero: C += result                            */
     int32_t split_k;     /* 0 = choose, 1 = never, n > 1 = exactly n slices */
     int32_t algo;        /* MNI_ALGO_*                                      */
+    float *aux;          /* BIAS_GELU_DUAL: second output; DGELU: saved pre-activation (read); else NULL */
+    float *colsum_part;  /* DGELU: mni_rocm_sgemm_colsum_rows(M, batch) x N floats of strip sums, or NULL */
 } mni_gemm_desc;
 int mni_rocm_sgemm(const mni_gemm_desc *desc);
+/* Rows of the colsum_part matrix a DGELU product of this height and batch count writes. */
+int64_t mni_rocm_sgemm_colsum_rows(int64_t M, int64_t batch);
 /* The same product for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
  * No counterpart in the reference.  Identical kernels, plans and results as

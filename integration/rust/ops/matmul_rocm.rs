@@ -29,6 +29,8 @@ fn product(store: &mut TensorStore, a: MniOperand, b: MniOperand, m: usize, n: u
         accumulate: 0,
         split_k: 0,
         algo: MNI_ALGO_AUTO,
+        aux: std::ptr::null_mut(),
+        colsum_part: std::ptr::null_mut(),
     };
     check(unsafe { mni_rocm_sgemm(&desc) });
     out

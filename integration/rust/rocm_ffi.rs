@@ -23,6 +23,8 @@ pub const MNI_EPI_NONE: i32 = 0;
 pub const MNI_EPI_BIAS: i32 = 1;
 pub const MNI_EPI_BIAS_RELU: i32 = 2;
 pub const MNI_EPI_BIAS_GELU: i32 = 3;
+pub const MNI_EPI_BIAS_GELU_DUAL: i32 = 4;
+pub const MNI_EPI_DGELU: i32 = 5;
 
 pub const MNI_ALGO_AUTO: i32 = 0;
 
@@ -55,6 +57,8 @@ pub struct MniGemmDesc {
     pub accumulate: i32,
     pub split_k: i32,
     pub algo: i32,
+    pub aux: *mut f32,
+    pub colsum_part: *mut f32,
 }
 
 #[link(name = "mni_rocm")]
@@ -73,6 +77,7 @@ extern "C" {
     pub fn mni_rocm_test_raise_device_status(code: c_uint) -> c_int;
     pub fn mni_rocm_launch_count() -> u64;
     pub fn mni_rocm_sgemm(desc: *const MniGemmDesc) -> c_int;
+    pub fn mni_rocm_sgemm_colsum_rows(m: i64, batch: i64) -> i64;
     pub fn mni_rocm_sgemm_noalloc(desc: *const MniGemmDesc) -> c_int;
     pub fn mni_rocm_sgemm_noalloc_workspace_bytes() -> usize;
     pub fn mni_rocm_strided_copy(dst: *mut f32, src: *const f32, shape: *const i64, src_strides: *const i64, ndim: c_int) -> c_int;

@@ -42,7 +42,8 @@ def test_binding_covers_every_declared_symbol():
 def test_struct_layout_matches_header():
     # mni_operand: pointer + 4 x int64; mni_gemm_desc as laid out in the header
     assert ctypes.sizeof(native.Operand) == 40
-    assert ctypes.sizeof(native.GemmDesc) == 4 * 8 + 2 * 40 + 8 + 8 + 8 + 8 + 4 * 4
+    assert ctypes.sizeof(native.GemmDesc) == 4 * 8 + 2 * 40 + 8 + 8 + 8 + 8 + 4 * 4 + 2 * 8
+    assert native.GemmDesc.aux.offset == 160 and native.GemmDesc.colsum_part.offset == 168
     assert native.GemmDesc.A.offset == 32 and native.GemmDesc.B.offset == 72
     assert native.GemmDesc.C.offset == 112 and native.GemmDesc.bias.offset == 136
 

@@ -272,13 +272,17 @@ def ffn_inputs(rows, d, h):
     return x, w1, w2, t
 
 
-def ffn_script(api, x, w1, w2, t, fused=False):
+def ffn_script(api, x, w1, w2, t, fused=False, fused_gelu=False, b1=None):
+    """fused: each Linear is one product with a bias epilogue.  fused_gelu: the first Linear also carries
+    its GELU (two outputs from one epilogue), and in the backward the second Linear's product hands dX
+    straight through gelu' to the first (no pre-activation tensor is visible then: hpre is None)."""
     d, h = w1.shape
-    l1 = api.Linear(d, h, weight=w1, bias=np.zeros(h, np.float32), fused=fused)
-    l2 = api.Linear(h, d, weight=w2, bias=np.zeros(d, np.float32), fused=fused)
+    b1 = np.zeros(h, np.float32) if b1 is None else b1
+    l1 = api.Linear(d, h, weight=w1, bias=b1, fused=fused or fused_gelu, activation="gelu" if fused_gelu else None)
+    l2 = api.Linear(h, d, weight=w2, bias=np.zeros(d, np.float32), fused=fused or fused_gelu)
     X = T(api, x, True)
-    hpre = l1.forward(X)
-    hact = hpre.gelu()
+    hpre = None if fused_gelu else l1.forward(X)
+    hact = l1.forward(X) if fused_gelu else hpre.gelu()
     y = l2.forward(hact)
     loss = api.mseLoss(y, T(api, t))
     loss.backward()
@@ -287,11 +291,12 @@ def ffn_script(api, x, w1, w2, t, fused=False):
 
 def test_config4_ffn_step_reduced_vs_oracle(gpu, orc):
     x, w1, w2, t = ffn_inputs(256, 128, 512)
-    for fused in (False, True):
+    b1 = synth.uniform(3, (512,), -0.3, 0.3, stream=4)   # the benchmark's bias is zero; a non-zero one exercises z + b
+    for fused, fused_gelu, bias1 in ((False, False, None), (True, False, None), (True, True, None), (True, True, b1)):
         gpu.native.resetEngine()
         orc.native.resetEngine()
-        g = ffn_script(gpu, x, w1, w2, t, fused)
-        o = ffn_script(orc, x, w1, w2, t)
+        g = ffn_script(gpu, x, w1, w2, t, fused, fused_gelu, bias1)
+        o = ffn_script(orc, x, w1, w2, t, b1=bias1)
         assert g["loss"].shape == [256, 1]
         assert_close(g["y"].numpy(), o["y"].numpy(), gemm_tol(512, o["hact"].numpy(), w2), "y")
         assert_close(g["loss"].numpy(), o["loss"].numpy(), 1e-4, "loss")
@@ -304,18 +309,30 @@ def test_config4_ffn_step_reduced_vs_oracle(gpu, orc):
         assert_close(g["X"].grad.numpy(), o["X"].grad.numpy(), gemm_tol(512, dh, w1) * 2, "dX")
 
 
-def test_config4_ffn_step_full_size_relations(gpu):
+@pytest.mark.parametrize("fused_gelu", [False, True])
+def test_config4_ffn_step_full_size_relations(gpu, fused_gelu):
     # X[4096,1024] -> 4096 -> 1024: too slow for the scalar oracle, so every
     # product of the step is checked on sampled rows/columns in float64 from
-    # the tensors the GPU itself produced.
+    # the tensors the GPU itself produced.  fused_gelu: the step the benchmark
+    # times as "fused" (GELU and its backward inside the products' epilogues).
     x, w1, w2, t = ffn_inputs(4096, 1024, 4096)
-    g = ffn_script(gpu, x, w1, w2, t)
-    hpre, hact, y = g["hpre"].numpy(), g["hact"].numpy(), g["y"].numpy()
+    g = ffn_script(gpu, x, w1, w2, t, fused_gelu, fused_gelu)
+    hact, y = g["hact"].numpy(), g["y"].numpy()
     rows = np.array([0, 1, 2047, 4095])
     x64, w164, w264 = x.astype(np.float64), w1.astype(np.float64), w2.astype(np.float64)
-    assert_close(hpre[rows], x64[rows] @ w164, gemm_tol(1024, x, w1), "X W1")
     gelu = lambda v: 0.5 * v * (1 + np.tanh(math.sqrt(2 / math.pi) * (v + 0.044715 * v ** 3)))
-    assert_close(hact[rows], gelu(hpre[rows].astype(np.float64)), 1e-5, "gelu")
+    if fused_gelu:
+        # the pre-activation never leaves the engine: take it in float64 where it is needed
+        class Pre:
+            def __getitem__(self, idx):
+                r, c = idx if isinstance(idx, tuple) else (idx, slice(None))
+                return (x64[r] @ w164[:, c]).astype(np.float64)
+        hpre = Pre()
+        assert_close(hact[rows], gelu(hpre[rows]), gemm_tol(1024, x, w1), "gelu(X W1)")
+    else:
+        hpre = g["hpre"].numpy()
+        assert_close(hpre[rows], x64[rows] @ w164, gemm_tol(1024, x, w1), "X W1")
+        assert_close(hact[rows], gelu(hpre[rows].astype(np.float64)), 1e-5, "gelu")
     assert_close(y[rows], hact[rows].astype(np.float64) @ w264, gemm_tol(4096, hact, w2), "H W2")
     loss = g["loss"].numpy()
     assert loss.shape == (4096, 1)

@@ -248,6 +248,76 @@ def test_bias_epilogues(dev, rocm, algo, epi):
         assert max_err(got2, got) <= 1e-6 * max(1.0, np.abs(z).max())
 
 
+def _gelu64(v):
+    return 0.5 * v * (1 + np.tanh(np.sqrt(2 / np.pi) * (v + 0.044715 * v ** 3)))
+
+
+def _gelu_grad64(v):
+    s = np.sqrt(2 / np.pi)
+    th = np.tanh(s * (v + 0.044715 * v ** 3))
+    return 0.5 * (1 + th) + 0.5 * v * (1 - th * th) * s * (1 + 3 * 0.044715 * v * v)
+
+
+@pytest.mark.parametrize("m,n,k,batch,algo", [(256, 384, 160, 1, N.ALGO_AUTO), (130, 70, 96, 3, N.ALGO_AUTO), (70, 200, 64, 2, N.ALGO_MFMA_SMALL),
+                                              (1, 5, 8, 1, N.ALGO_AUTO)])
+def test_two_output_gelu_epilogue(dev, rocm, m, n, k, batch, algo):
+    # C = product, aux = gelu(product + bias): the forward of a fused GELU Linear
+    a = synth.normal(1, (batch, m, k))
+    b = synth.normal(2, (k, n), 0.3, stream=1)
+    bias = synth.normal(3, (n,), stream=2)
+    dA, dB, dbias = dev.put(a), dev.put(b), dev.put(bias)
+    dC, dH = dev.empty(batch * m * n, fill=-7.0), dev.empty(batch * m * n, fill=-7.0)
+    rocm.sgemm(m, n, k, dA, dB, dC, batch=batch, a_batch=(m * k, batch), bias=dbias, epilogue=N.EPI_BIAS_GELU_DUAL, aux=dH, algo=algo)
+    z = a.astype(np.float64) @ b.astype(np.float64)
+    assert max_err(rocm.to_host(dC, (batch, m, n)), z) <= gemm_tol(k, a, b)
+    assert max_err(rocm.to_host(dH, (batch, m, n)), _gelu64(z + bias)) <= gemm_tol(k, a, b)
+
+
+@pytest.mark.parametrize("m,n,k,batch,algo,strips", [(256, 384, 160, 1, N.ALGO_AUTO, True), (130, 70, 96, 3, N.ALGO_AUTO, True),
+                                                     (70, 200, 64, 2, N.ALGO_MFMA_SMALL, False), (40, 36, 200, 1, N.ALGO_AUTO, True)])
+def test_gelu_backward_epilogue_with_strip_sums(dev, rocm, m, n, k, batch, algo, strips):
+    # C = product * gelu'(z + bias) and the column sums of C per strip of rows: the gradient of a Linear's
+    # input taken through the GELU of the layer that produced it, with that layer's bias gradient
+    g = synth.normal(1, (batch, m, k))
+    wt = synth.normal(2, (n, k), 0.3, stream=1)          # the weight [n, k] used transposed
+    z = synth.normal(3, (batch, m, n), stream=2)
+    bias = synth.normal(4, (n,), stream=3)
+    dG, dW, dZ, dbias = dev.put(g), dev.put(wt), dev.put(z), dev.put(bias)
+    dC = dev.empty(batch * m * n, fill=-7.0)
+    rows = rocm.sgemm_colsum_rows(m, batch)
+    assert rows == batch * ((m + 127) // 128) * 2
+    dP = dev.empty(rows * n, fill=-7.0) if strips else None
+    rocm.sgemm(m, n, k, dG, dW, dC, batch=batch, a_batch=(m * k, batch), b_strides=(1, k), bias=dbias, epilogue=N.EPI_DGELU, aux=dZ,
+               colsum_part=dP, algo=algo)
+    want = (g.astype(np.float64) @ wt.T.astype(np.float64)) * _gelu_grad64(z.astype(np.float64) + bias)
+    got = rocm.to_host(dC, (batch, m, n))
+    tol = gemm_tol(k, g, wt) * 1.2
+    assert max_err(got, want) <= tol
+    if strips:
+        part = rocm.to_host(dP, (rows, n))
+        assert max_err(part.astype(np.float64).sum(0), want.sum((0, 1))) <= tol * np.sqrt(batch * m)
+        # strip r holds rows 64 r' .. of its batch: each strip is the sum of exactly its own rows
+        per_batch = rows // batch
+        for bi in range(batch):
+            for st in range(per_batch):
+                lo, hi = 64 * st, min(m, 64 * (st + 1))
+                exp = got[bi, lo:hi].astype(np.float64).sum(0) if lo < m else np.zeros(n)
+                assert max_err(part[bi * per_batch + st], exp) <= 1e-4 * max(1.0, np.abs(got).max()) * 8
+
+
+def test_fused_gelu_epilogues_reject_what_they_cannot_do(dev, rocm):
+    a, b = dev.put(np.ones((64, 64), np.float32)), dev.put(np.ones((64, 64), np.float32))
+    c, bias = dev.empty(64 * 64), dev.put(np.zeros(64, np.float32))
+    with pytest.raises(N.MniError, match="needs the aux pointer"):
+        rocm.sgemm(64, 64, 64, a, b, c, bias=bias, epilogue=N.EPI_BIAS_GELU_DUAL)
+    with pytest.raises(N.MniError, match="neither accumulate nor split_k"):
+        rocm.sgemm(64, 64, 64, a, b, c, bias=bias, epilogue=N.EPI_DGELU, aux=c, split_k=2)
+    with pytest.raises(N.MniError, match="MFMA tile kernel only"):
+        rocm.sgemm(4, 64, 64, a, b, c, bias=bias, epilogue=N.EPI_DGELU, aux=c, algo=N.ALGO_SKINNY)
+    with pytest.raises(N.MniError, match="colsum_part goes with the DGELU epilogue"):
+        rocm.sgemm(64, 64, 64, a, b, c, bias=bias, epilogue=N.EPI_BIAS, colsum_part=c)
+
+
 def test_accumulate(dev, rocm):
     a = synth.small_ints(1, (100, 50), 3)
     b = synth.small_ints(2, (50, 60), 3, stream=1)

@@ -14,7 +14,7 @@ C_TO_RUST = {
     "float": "f32", "double": "f64",
     "void *": "*mut c_void", "const void *": "*const c_void", "void **": "*mut *mut c_void",
     "char *": "*mut c_char", "const char *": "*const c_char", "int *": "*mut c_int",
-    "float *": "*mut f32", "const float *": "*const f32", "const int64_t *": "*const i64",
+    "float *": "*mut f32", "int64_t": "i64", "const float *": "*const f32", "const int64_t *": "*const i64",
     "const mni_gemm_desc *": "*const MniGemmDesc", "mni_operand": "MniOperand",
 }
 
