@@ -443,6 +443,18 @@ def run_for_counters(r, which):
         a, b = r.to_device(synth.normal(1, (4096, 3072))), r.to_device(synth.normal(1, (3072, 768), stream=1))
         for _ in range(5):
             r.sgemm(4096, 768, 3072, a, b, dst)
+    elif which == "config3":
+        # the three attention-shaped batched products of configuration 3 (scores through the panel kernel, dQ and
+        # dK^T through the register-direct kernel), 5 launches each
+        q, ds = synth.normal(2, (32, 512, 64)) / np.float32(8), synth.normal(2, (32, 512, 512), stream=2)
+        dq, dk, dds = r.to_device(q), r.to_device(q), r.to_device(ds)
+        g_out = r.malloc(32 * 512 * 64 * 4)
+        for _ in range(5):
+            r.sgemm(512, 512, 64, dq, dk, dst, batch=32, a_batch=(512 * 64, 32), b_strides=(1, 64), b_batch=(512 * 64, 32))
+        for _ in range(5):
+            r.sgemm(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32), b_batch=(512 * 64, 32))
+        for _ in range(5):
+            r.sgemm(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64), a_batch=(512 * 64, 32), b_batch=(512 * 512, 32))
     elif which == "attention":
         # the one-kernel attention forward on [8, 8192, 64], causal, through the engine entry point
         from framework_amd.api import bind
@@ -506,7 +518,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
-    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "attention", "attention_bwd"], default=None,
+    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "attention", "attention_bwd"], default=None,
                     help="for rocprofv3 --pmc runs: launch a copy kernel of known size (64 MiB read + 64 MiB "
                          "written) 3 times, then the chosen product 5 times, and exit")
     args = ap.parse_args()
