@@ -179,10 +179,11 @@ def bench_extras(r, with_cpu):
     fl = 2.0 * 4 * 4096 * 4096
     kern = "skinny_cols_kernel<4, true, true, false, true>"
     # launches of a few microseconds are issued from C (mni_rocm_sgemm_timed) so that the host stays ahead
-    ws = [r.to_device(w) for _ in range(8)]
-    ms_cold = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, p, dy) for p in ws], 16, 200)
     ms_warm = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 10, 200)
     ms_sus = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 3000, 1000)
+    ws = [r.to_device(w) for _ in range(8)]
+    ms_cold = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, p, dy) for p in ws], 16, 200)
+    r.sgemm(4, 4096, 4096, dx, dw, dy)
     got = r.to_host(dy, (4, 4096))
     c5a = {"roofline": dict(roofline("hbm", kern, ms_cold * 1e-3, fl, by, traffic=profile_traffic("skinny_gemv_4x4096x4096.txt")),
                             note="cold: eight different W in rotation (512 MiB working set), every byte comes from HBM"),
