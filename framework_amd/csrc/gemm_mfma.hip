@@ -27,15 +27,15 @@
 //
 // Operand layouts (transposes folded into the load path).  An operand whose K
 // axis has unit stride (A row-major, or B given as its transpose) is loaded
-// with 16-byte loads along K and stored to LDS as is.  An operand whose M/N
-// axis has unit stride (B row-major, or A given as its transpose) is loaded as
-// a 4(k) x 4(mn) micro-tile with 16-byte loads along M/N and transposed in
-// registers on the way to LDS.  The 16-byte loads need no more than the 4-byte
-// alignment every float has (the memory system splits a load that straddles a
-// cache line), so odd leading dimensions and offset bases take these paths
-// too.  Anything else (neither axis contiguous, K tails, edges of an M/N-
-// contiguous operand off a multiple of 4) takes guarded scalar loads into the
-// same register layout.
+// with 16-byte loads along K.  An operand whose M/N axis has unit stride (B
+// row-major, or A given as its transpose) is loaded with 4-byte loads, each
+// wavefront instruction covering 64 consecutive rows of one K value, four of
+// them filling the register quad that holds a row's K quad.  Either way the
+// registers are stored to LDS as they are.  The loads need no more than the
+// 4-byte alignment every float has (the memory system splits a 16-byte load
+// that straddles a cache line), so odd leading dimensions and offset bases take
+// these paths too.  Anything else (neither axis contiguous, K tails) takes
+// guarded scalar loads into the same register layout.
 //
 // K loop.  Tile kt+1 sits in staging registers while tile kt is multiplied out
 // of LDS; in the last quarter of a step the staged tile goes to the other LDS
@@ -44,12 +44,18 @@
 // MFMA of that quarter; LDS is read in the first three quarters and written
 // in the last).
 // The loop exists twice.  The general form chooses between fast and guarded
-// loads per step.  The steady form (interior tile, whole K steps; a partial
-// last step and the two before it are left to the general form) has no such
-// choice and loads unconditionally: when the staging registers
-// have two possible producers the compiler merges them with register copies
-// that wait for the data right behind the request, which stalls every step
-// for a memory round trip.
+// loads per step.  The steady form (whole K steps; a partial last step and the
+// two before it are left to the general form) has no such choice and loads
+// unconditionally: when the staging registers have two possible producers the
+// compiler merges them with register copies that wait for the data right
+// behind the request, which stalls every step for a memory round trip.  The
+// steady form is also free of vector-ALU instructions: on this chip every one
+// of them is paid for in fp32 MFMA issue time (measured: one v_mov per MFMA
+// takes 8 % off a loop of MFMAs, an address add 15 %; LDS accesses, buffer
+// loads and scalar instructions take nothing).  So it is unrolled over the two
+// LDS stages (every LDS address a fixed register plus an immediate), loads go
+// through buffer instructions whose moving parts (tile base, K advance, row
+// pitch) are scalar, and nothing is shuffled between load and LDS store.
 //
 // Work distribution.  Classic form: one workgroup per (tile, batch, K slice);
 // with more than one slice the partials go to a workspace and a second kernel
@@ -96,19 +102,26 @@ __device__ __forceinline__ unsigned load_mark(const unsigned *p) {
 __device__ __forceinline__ int lds_row(int r) { return r ^ ((r >> 4) & 3); }
 
 // ---- global -> register loads ---------------------------------------------
-// A tile side has ROWS = 128 or 64 rows (m for A, n for B) and BK = 32 K values.
+// A tile side has ROWS = 256, 128 or 64 rows (m for A, n for B) and BK = 32 K
+// values: ROWS / 32 float4 per thread.
 // Register layout LAYOUT 0 (K contiguous): thread owns float4 #(tid + 256 i),
-//   i < ROWS/32, where float4 #f is row f/8, K quad f%8.
-// Register layout LAYOUT 1 (M/N contiguous): thread owns the 4 x 4 micro-tile
-//   rows 4*(tid % (ROWS/4))..+3, K quad tid / (ROWS/4) (threads whose quad is
-//   >= 8 own nothing: half of them when ROWS = 64); v[j] holds k = 4*quad + j
-//   across the four rows.
+//   i < ROWS/32, where float4 #f is row f/8, K quad f%8: one 16-byte load each.
+// Register layout LAYOUT 1 (M/N contiguous): thread owns row tid % ROWS and the
+//   K quads tid / ROWS + (256 / ROWS) p, p < ROWS/32; v[p] holds the quad's four
+//   K values, fetched by four 4-byte loads (64 lanes = 256 consecutive bytes
+//   each).  Either way a register quad is what one LDS slot holds, so nothing
+//   is shuffled between the load and the LDS store: every vector-ALU instruction
+//   in the K loop takes its cycles from the fp32 MFMAs (a v_mov per MFMA costs
+//   8 % of the matrix rate on this chip; loads, LDS traffic and scalar work cost
+//   nothing), so the loop is built to contain none.
+template <int ROWS> __device__ constexpr int stage_regs() { return ROWS / 32 > 4 ? ROWS / 32 : 4; }
+template <int ROWS> __device__ constexpr int quad_stride() { return NTHREADS / ROWS; }  // K quads covered per pass (layout 1)
 
-// Rows at or beyond `rows` (an edge tile; a multiple of 4 for layout 1) are
-// read from the last valid row or row quad instead: what they contribute lands
-// in accumulator rows / columns that the epilogue never stores.
+// Rows at or beyond `rows` (an edge tile) are read from the last valid row
+// instead: what they contribute lands in accumulator rows / columns that the
+// epilogue never stores.
 template <int LAYOUT, int ROWS>
-__device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t ld, int rows, int tid, float4 (&v)[4]) {
+__device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t ld, int rows, int tid, float4 (&v)[stage_regs<ROWS>()]) {
     if (LAYOUT == 0) {
 #pragma unroll
         for (int i = 0; i < ROWS / 32; ++i) {
@@ -117,16 +130,15 @@ __device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t l
             v[i] = *reinterpret_cast<const float4 *>(p + (int64_t)row * ld + 4 * q);
         }
     } else {
-        constexpr int R4 = ROWS / 4;
-        int r4 = min(tid % R4, rows / 4 - 1), q = tid / R4;
-        // Threads beyond the tile (half of them when ROWS = 64) own nothing;
-        // they load what their partner 8 quads below loads and never store
-        // it.  Loading under a predicate instead would make every load a merge
-        // with the old register contents, which waits for the data on the spot.
-        q %= KQ;
+        constexpr int QS = quad_stride<ROWS>();
+        const int n = min(tid % ROWS, rows - 1), q0 = tid / ROWS;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            v[j] = *reinterpret_cast<const float4 *>(p + 4 * r4 + (int64_t)(4 * q + j) * ld);
+        for (int ps = 0; ps < ROWS / 32; ++ps) {
+            float t[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) t[j] = p[n + (int64_t)(4 * (q0 + QS * ps) + j) * ld];
+            v[ps] = make_float4(t[0], t[1], t[2], t[3]);
+        }
     }
 }
 
@@ -134,112 +146,110 @@ __device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t l
 // rows >= rmax or k >= kmax read as zero.
 template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void load_guarded(const float *__restrict__ p, int64_t rs, int64_t cs, int rmax,
-                                             int kmax, int tid, float4 (&v)[4]) {
+                                             int kmax, int tid, float4 (&v)[stage_regs<ROWS>()]) {
     // Edge tiles and K tails only.  The empty asm makes the element addresses
     // get computed here, on use: computed once ahead of the K loop they would
     // occupy sixteen register pairs for the whole loop.
     asm volatile("" : "+v"(tid));
-    if (LAYOUT == 0) {
 #pragma unroll
-        for (int i = 0; i < ROWS / 32; ++i) {
-            int f = tid + NTHREADS * i;
-            int row = f >> 3, q = f & 7;
-            float t[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                int k = 4 * q + e;
-                t[e] = (row < rmax && k < kmax) ? p[(int64_t)row * rs + (int64_t)k * cs] : 0.0f;
-            }
-            v[i] = make_float4(t[0], t[1], t[2], t[3]);
+    for (int i = 0; i < ROWS / 32; ++i) {
+        int row, q;
+        if (LAYOUT == 0) {
+            const int f = tid + NTHREADS * i;
+            row = f >> 3, q = f & 7;
+        } else {
+            row = tid % ROWS, q = tid / ROWS + quad_stride<ROWS>() * i;
         }
-    } else {
-        constexpr int R4 = ROWS / 4;
-        int r4 = tid % R4, q = tid / R4;
-        if (q < KQ) {
+        float t[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                int k = 4 * q + j;
-                float t[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    int row = 4 * r4 + e;
-                    t[e] = (row < rmax && k < kmax) ? p[(int64_t)row * rs + (int64_t)k * cs] : 0.0f;
-                }
-                v[j] = make_float4(t[0], t[1], t[2], t[3]);
-            }
+        for (int e = 0; e < 4; ++e) {
+            int k = 4 * q + e;
+            t[e] = (row < rmax && k < kmax) ? p[(int64_t)row * rs + (int64_t)k * cs] : 0.0f;
         }
+        v[i] = make_float4(t[0], t[1], t[2], t[3]);
     }
 }
 
 // ---- register -> LDS --------------------------------------------------------
+// float4 slot of piece i of this thread within a tile stage
 template <int LAYOUT, int ROWS>
-__device__ __forceinline__ void store_lds(float4 *__restrict__ tile, int tid, const float4 (&v)[4]) {
+__device__ __forceinline__ int lds_slot(int tid, int i) {
     constexpr int SLICE = ROWS + PAD;
+    if (LAYOUT == 0) {
+        const int f = tid + NTHREADS * i;
+        return (f & 7) * SLICE + lds_row(f >> 3);
+    }
+    return (tid / ROWS + quad_stride<ROWS>() * i) * SLICE + lds_row(tid % ROWS);
+}
+
+template <int LAYOUT, int ROWS>
+__device__ __forceinline__ void store_lds(float4 *__restrict__ tile, int tid, const float4 (&v)[stage_regs<ROWS>()]) {
+#pragma unroll
+    for (int i = 0; i < ROWS / 32; ++i) tile[lds_slot<LAYOUT, ROWS>(tid, i)] = v[i];
+}
+
+// ---- the steady K loop's transfers -------------------------------------------
+// In the steady loop a tile side moves in pieces dealt out behind the MFMAs:
+// first the ROWS/32 LDS stores of the staged tile, then the loads that refill
+// the staging registers.  The loads are buffer loads: the tile's base address
+// and the K advance sit in the scalar resource descriptor, row offsets that
+// depend on the leading dimension in a scalar offset, and the only vector
+// register involved is a per-thread byte offset computed once ahead of the loop.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+struct StageAddr {
+    int voff[8];  // layout 0: byte offset of piece i; layout 1: voff[0] = byte offset of the thread's row
+    int quad0;    // layout 1: byte offset of the thread's first K row, 4 * (tid / ROWS) * ld * 4 (uniform per wavefront)
+    int ldb;      // leading dimension in bytes
+};
+
+template <int LAYOUT, int ROWS>
+__device__ __forceinline__ StageAddr stage_addr(int64_t ld, int rows, int tid) {
+    StageAddr s;
+    s.ldb = (int)ld * 4;
+    s.quad0 = 0;
     if (LAYOUT == 0) {
 #pragma unroll
         for (int i = 0; i < ROWS / 32; ++i) {
-            int f = tid + NTHREADS * i;
-            int row = f >> 3, q = f & 7;
-            tile[q * SLICE + lds_row(row)] = v[i];
+            const int f = tid + NTHREADS * i;
+            s.voff[i] = (min(f >> 3, rows - 1) * (int)ld + 4 * (f & 7)) * 4;
         }
     } else {
-        constexpr int R4 = ROWS / 4;
-        int r4 = tid % R4, q = tid / R4;
-        // The 4 x 4 transpose is sixteen register moves, written out so that
-        // they stay here, a whole K step after the loads were issued.  Left to
-        // the compiler they end up merged into the loop-carried copy of the
-        // staging registers, right behind the loads, and wait for data that
-        // was only just requested.
-        float4 o[4];
-#define MNI_TRANSPOSE_ROW(dst, c)                                                                     \
-    asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7"        \
-                 : "=&v"(dst.x), "=&v"(dst.y), "=&v"(dst.z), "=&v"(dst.w)                              \
-                 : "v"(v[0].c), "v"(v[1].c), "v"(v[2].c), "v"(v[3].c))
-        MNI_TRANSPOSE_ROW(o[0], x);
-        MNI_TRANSPOSE_ROW(o[1], y);
-        MNI_TRANSPOSE_ROW(o[2], z);
-        MNI_TRANSPOSE_ROW(o[3], w);
-#undef MNI_TRANSPOSE_ROW
-        if (NTHREADS / R4 <= KQ || q < KQ) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) tile[q * SLICE + lds_row(4 * r4 + e)] = o[e];
-        }
+        s.voff[0] = min(tid % ROWS, rows - 1) * 4;
+        s.quad0 = __builtin_amdgcn_readfirstlane(tid / ROWS) * 4 * s.ldb;
     }
+    return s;
 }
 
-// One piece of a tile transfer, so that the last chunk of a K step can deal
-// them out one per MFMA.  A tile side is `pieces<LAYOUT, ROWS>()` pieces: for
-// layout 0 float4 #i is stored (first half) and then loaded anew (second
-// half); for layout 1 pieces 0..3 transpose and store row e of the micro-tile
-// and pieces 4..7 load v[j].
-template <int LAYOUT, int ROWS>
-__device__ constexpr int tile_pieces() { return LAYOUT == 0 ? 2 * (ROWS / 32) : 8; }
+// Whether the offsets above fit the 32-bit offset fields of a buffer load.
+template <int ROWS>
+__device__ __forceinline__ bool stage_addr_fits(int64_t ld) { return ld > 0 && ld * 4 * (ROWS > BK ? ROWS : BK) < (int64_t)0x7fffffff; }
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t stage_rsrc(const float *p) {
+    // raw buffer: stride 0, no range limit (rows are clamped by the caller), 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p), 0, -1, 0x00020000);
+}
 
 template <int LAYOUT, int ROWS>
-__device__ __forceinline__ void tile_piece(int x, float4 *__restrict__ tile, const float *__restrict__ p, int64_t ld,
-                                           int rows, int tid, float4 (&v)[4]) {
-    constexpr int SLICE = ROWS + PAD;
-    if (LAYOUT == 0) {
-        constexpr int NV = ROWS / 32;
-        const int i = x < NV ? x : x - NV;
-        const int f = tid + NTHREADS * i;
-        const int row = f >> 3, q = f & 7;
-        if (x < NV) tile[q * SLICE + lds_row(row)] = v[i];
-        else v[i] = *reinterpret_cast<const float4 *>(p + (int64_t)min(row, rows - 1) * ld + 4 * q);
+__device__ constexpr int tile_pieces() { return LAYOUT == 0 ? 2 * (ROWS / 32) : 5 * (ROWS / 32); }
+
+template <int LAYOUT, int ROWS>
+__device__ __forceinline__ void tile_piece(int x, float4 *__restrict__ tile, __amdgpu_buffer_rsrc_t rsrc, const StageAddr &sa,
+                                           int tid, float4 (&v)[stage_regs<ROWS>()]) {
+    constexpr int NV = ROWS / 32;
+    if (x < NV) {
+        tile[lds_slot<LAYOUT, ROWS>(tid, x)] = v[x];
+    } else if (LAYOUT == 0) {
+        const floatx4 t = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, sa.voff[x - NV], 0, 0));
+        v[x - NV] = make_float4(t.x, t.y, t.z, t.w);
     } else {
-        constexpr int R4 = ROWS / 4;
-        const int r4 = tid % R4, q = tid / R4;
-        if (x < 4) {
-            float4 o;
-            if (x == 0) asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7" : "=&v"(o.x), "=&v"(o.y), "=&v"(o.z), "=&v"(o.w) : "v"(v[0].x), "v"(v[1].x), "v"(v[2].x), "v"(v[3].x));
-            if (x == 1) asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7" : "=&v"(o.x), "=&v"(o.y), "=&v"(o.z), "=&v"(o.w) : "v"(v[0].y), "v"(v[1].y), "v"(v[2].y), "v"(v[3].y));
-            if (x == 2) asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7" : "=&v"(o.x), "=&v"(o.y), "=&v"(o.z), "=&v"(o.w) : "v"(v[0].z), "v"(v[1].z), "v"(v[2].z), "v"(v[3].z));
-            if (x == 3) asm volatile("v_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7" : "=&v"(o.x), "=&v"(o.y), "=&v"(o.z), "=&v"(o.w) : "v"(v[0].w), "v"(v[1].w), "v"(v[2].w), "v"(v[3].w));
-            if (NTHREADS / R4 <= KQ || q < KQ) tile[q * SLICE + lds_row(4 * r4 + x)] = o;
-        } else {
-            const int j = x - 4;
-            v[j] = *reinterpret_cast<const float4 *>(p + 4 * min(r4, rows / 4 - 1) + (int64_t)(4 * (q % KQ) + j) * ld);
-        }
+        const int y = x - NV, ps = y >> 2, j = y & 3;
+        const float t = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+            rsrc, sa.voff[0], sa.quad0 + (4 * quad_stride<ROWS>() * ps + j) * sa.ldb, 0));
+        if (j == 0) v[ps].x = t;
+        if (j == 1) v[ps].y = t;
+        if (j == 2) v[ps].z = t;
+        if (j == 3) v[ps].w = t;
     }
 }
 
@@ -431,11 +441,10 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         g.B + (int64_t)(batch % g.b_bcount) * g.b_bs + (int64_t)n0 * g.b_cs + (int64_t)k_begin * g.b_rs;
     const int mrem = g.M - m0, nrem = g.N - n0;
     // Fast loads also serve an edge tile (rows beyond the edge re-read the last
-    // valid ones), except that 16-byte loads along M/N need the edge on a
-    // multiple of 4.
+    // valid ones).
     const int a_rows = min(mrem, BM), b_rows = min(nrem, BN);
-    const bool a_fast = AMODE == 0 || (AMODE == 1 && a_rows % 4 == 0);
-    const bool b_fast = BMODE == 0 || (BMODE == 1 && b_rows % 4 == 0);
+    const bool a_fast = AMODE != 2;
+    const bool b_fast = BMODE != 2;
     // leading dimension seen by the fast loaders
     const int64_t a_ld = AMODE == 0 ? g.a_rs : g.a_cs;
     const int64_t b_ld = BMODE == 0 ? g.b_cs : g.b_rs;
@@ -448,41 +457,36 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    float4 ra[4], rb[4];
+    float4 ra[stage_regs<BM>()], rb[stage_regs<BN>()];
 
-    // STEADY: the tile is interior and K is a whole number of steps, so every
-    // load of the K loop is a fast one; the loop then has no branch that
-    // produces staging registers on two paths.
-    auto load_a = [&](int kt, auto steady) {  // A tile: rows = m, element (m, k) at Ap[m * a_rs + k * a_cs]
+    auto load_a = [&](int kt) {  // A tile: rows = m, element (m, k) at Ap[m * a_rs + k * a_cs]
         const int k0 = kt * BK;
         const int krem = klen - k0;
-        if (decltype(steady)::value || (a_fast && krem >= BK)) {
+        if (a_fast && krem >= BK) {
             if (AMODE == 0) load_fast<0, BM>(Ap + (int64_t)k0, a_ld, a_rows, tid, ra);
             else load_fast<1, BM>(Ap + (int64_t)k0 * a_ld, a_ld, a_rows, tid, ra);
         } else {
             load_guarded<AL, BM>(Ap + (int64_t)k0 * g.a_cs, g.a_rs, g.a_cs, mrem, krem, tid, ra);
         }
     };
-    auto load_b = [&](int kt, auto steady) {  // B tile: rows = n, element (n, k) at Bp[n * b_cs + k * b_rs]
+    auto load_b = [&](int kt) {  // B tile: rows = n, element (n, k) at Bp[n * b_cs + k * b_rs]
         const int k0 = kt * BK;
         const int krem = klen - k0;
-        if (decltype(steady)::value || (b_fast && krem >= BK)) {
+        if (b_fast && krem >= BK) {
             if (BMODE == 0) load_fast<0, BN>(Bp + (int64_t)k0, b_ld, b_rows, tid, rb);
             else load_fast<1, BN>(Bp + (int64_t)k0 * b_ld, b_ld, b_rows, tid, rb);
         } else {
             load_guarded<BL, BN>(Bp + (int64_t)k0 * g.b_rs, g.b_cs, g.b_rs, nrem, krem, tid, rb);
         }
     };
-    typedef std::integral_constant<bool, false> General;
-    typedef std::integral_constant<bool, true> Steady;
 
     // Prologue: tile 0 goes to LDS stage 0, tile 1 into the staging registers.
     if (nkt > 0) {
-        load_a(0, General());
-        load_b(0, General());
+        load_a(0);
+        load_b(0);
         store_lds<AL, BM>(stage_a(0), tid, ra);
         store_lds<BL, BN>(stage_b(0), tid, rb);
-        if (nkt > 1) { load_a(1, General()); load_b(1, General()); }
+        if (nkt > 1) { load_a(1); load_b(1); }
     }
     __syncthreads();
 
@@ -506,99 +510,123 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
             for (int jj = 0; jj < TN; ++jj)
                 acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(pick(fa[i], j), pick(fb[jj], j), acc[i][jj], 0, 0, 0);
     };
+    // The first three quarters of a K step: MFMAs of chunk c with the fragment
+    // reads of chunk c + 1 between the groups.
+    auto chunk = [&](const float4 *As, const float4 *Bs, int c) {
+        const int qa = (2 * (c + 1) + h) * SLICE_A, qb = (2 * (c + 1) + h) * SLICE_B;
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) na[i] = As[qa + a_row[i]];
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < (TN + 1) / 2; ++j) nb[j] = Bs[qb + b_row[j]];
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(2);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = (TN + 1) / 2; j < TN; ++j) nb[j] = Bs[qb + b_row[j]];
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(3);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = na[i];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = nb[j];
+    };
 
-    auto k_loop = [&](auto steady, int kt_begin, int kt_end) {
-    constexpr bool ST = decltype(steady)::value;
-    for (int kt = kt_begin; kt < kt_end; ++kt) {
-        const int cur = kt & 1;
-        // Steady form: the stores and loads run unconditionally (the last two
-        // steps park and fetch the final tile again, which nobody reads), so
-        // the staging registers have one producer.
-        const bool more = ST || kt + 1 < nkt;
-        const bool more2 = ST || kt + 2 < nkt;
-        const int kt2 = ST ? min(kt + 2, nkt - 1) : kt + 2;
-
+    // Steady form of a K step (every load a fast one; the stage is a
+    // compile-time constant, the loop below is unrolled over both, so that
+    // every LDS address is a register fixed ahead of the loop plus an immediate).
+    // The staged tile goes to LDS and tile kt + 2 is requested piece by piece,
+    // one or two pieces behind each MFMA of the last chunk, so that none of it
+    // has to be issued with the matrix pipe idle.  The last two steps park and
+    // fetch the final tile again, which nobody reads: the staging registers have
+    // one producer, and no branch on which the compiler could merge two with
+    // register copies that wait for the data right behind the request.
+    const StageAddr sa_a = stage_addr<AL, BM>(a_ld, a_rows, tid), sa_b = stage_addr<BL, BN>(b_ld, b_rows, tid);
+    auto steady_step = [&](auto stage, int kt) {
+        constexpr int cur = decltype(stage)::value;
+        const int kt2 = min(kt + 2, nkt - 1);
         const float4 *As = stage_a(cur), *Bs = stage_b(cur);
 #pragma unroll
         for (int i = 0; i < TM; ++i) fa[i] = As[h * SLICE_A + a_row[i]];
 #pragma unroll
         for (int j = 0; j < TN; ++j) fb[j] = Bs[h * SLICE_B + b_row[j]];
 #pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) {
-            const bool last = c == NCHUNK - 1;
-            const int qa = (2 * (c + 1) + h) * SLICE_A, qb = (2 * (c + 1) + h) * SLICE_B;
-            if (ST && last) {
-                // Steady form: the staged tile goes to LDS and tile kt+2 is
-                // requested piece by piece, one or two pieces behind each MFMA, so
-                // that none of it has to be issued with the matrix pipe idle.
-                constexpr int PA = tile_pieces<AL, BM>(), PB = tile_pieces<BL, BN>();
-                constexpr int SLOTS = 4 * TM * TN, PER = (PA + PB + SLOTS - 1) / SLOTS;
-                const float *pa = AMODE == 0 ? Ap + (int64_t)kt2 * BK : Ap + (int64_t)kt2 * BK * a_ld;
-                const float *pb = BMODE == 0 ? Bp + (int64_t)kt2 * BK : Bp + (int64_t)kt2 * BK * b_ld;
-                int slot = 0;
+        for (int c = 0; c < NCHUNK - 1; ++c) chunk(As, Bs, c);
+        constexpr int PA = tile_pieces<AL, BM>(), PB = tile_pieces<BL, BN>();
+        constexpr int SLOTS = 4 * TM * TN, PER = (PA + PB + SLOTS - 1) / SLOTS;
+        const __amdgpu_buffer_rsrc_t ra_src = stage_rsrc(AMODE == 0 ? Ap + (int64_t)kt2 * BK : Ap + (int64_t)kt2 * BK * a_ld);
+        const __amdgpu_buffer_rsrc_t rb_src = stage_rsrc(BMODE == 0 ? Bp + (int64_t)kt2 * BK : Bp + (int64_t)kt2 * BK * b_ld);
+        int slot = 0;
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                        for (int jj = 0; jj < TN; ++jj) {
-                            __builtin_amdgcn_sched_barrier(0);
-                            acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(pick(fa[i], j), pick(fb[jj], j), acc[i][jj], 0, 0, 0);
-                            __builtin_amdgcn_sched_barrier(0);
+                for (int jj = 0; jj < TN; ++jj) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x2f32(pick(fa[i], j), pick(fb[jj], j), acc[i][jj], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                            for (int x = slot * PER; x < (slot + 1) * PER; ++x) {
-                                if (x < PA) tile_piece<AL, BM>(x, stage_a(cur ^ 1), pa, a_ld, a_rows, tid, ra);
-                                else if (x < PA + PB) tile_piece<BL, BN>(x - PA, stage_b(cur ^ 1), pb, b_ld, b_rows, tid, rb);
-                            }
-                            ++slot;
-                        }
-                __builtin_amdgcn_sched_barrier(0);
-                continue;
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_group(0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (!last) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i) na[i] = As[qa + a_row[i]];
-            } else if (more) {
-                // The staging registers hold tile kt+1 (requested a whole K step
-                // ago); once they are in LDS they are refilled with tile kt+2.
-                store_lds<AL, BM>(stage_a(cur ^ 1), tid, ra);
-                if (more2) load_a(kt2, steady);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_group(1);
-            __builtin_amdgcn_sched_barrier(0);
-            if (!last) nb[0] = Bs[qb + b_row[0]];
-            else if (more) {
-                store_lds<BL, BN>(stage_b(cur ^ 1), tid, rb);
-                if (more2) load_b(kt2, steady);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_group(2);
-            __builtin_amdgcn_sched_barrier(0);
-            if (!last && TN > 1) nb[TN - 1] = Bs[qb + b_row[TN - 1]];
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_group(3);
-            __builtin_amdgcn_sched_barrier(0);
-            if (!last) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i) fa[i] = na[i];
-#pragma unroll
-                for (int j = 0; j < TN; ++j) fb[j] = nb[j];
-            }
-        }
+                    for (int x = slot * PER; x < (slot + 1) * PER; ++x) {
+                        if (x < PA) tile_piece<AL, BM>(x, stage_a(cur ^ 1), ra_src, sa_a, tid, ra);
+                        else if (x < PA + PB) tile_piece<BL, BN>(x - PA, stage_b(cur ^ 1), rb_src, sa_b, tid, rb);
+                    }
+                    ++slot;
+                }
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
-    }
     };
-    // An interior tile runs the steady form; when K ends in a partial step, up
-    // to the step that requests that last tile (two steps ahead), and the
-    // general form takes the remaining three.
+
+    // General form: chooses between fast and guarded loads per step.
+    auto general_step = [&](int kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < nkt, more2 = kt + 2 < nkt;
+        const float4 *As = stage_a(cur), *Bs = stage_b(cur);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = As[h * SLICE_A + a_row[i]];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = Bs[h * SLICE_B + b_row[j]];
+#pragma unroll
+        for (int c = 0; c < NCHUNK - 1; ++c) chunk(As, Bs, c);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) {
+            // The staging registers hold tile kt+1 (requested a whole K step
+            // ago); once they are in LDS they are refilled with tile kt+2.
+            store_lds<AL, BM>(stage_a(cur ^ 1), tid, ra);
+            if (more2) load_a(kt + 2);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) {
+            store_lds<BL, BN>(stage_b(cur ^ 1), tid, rb);
+            if (more2) load_b(kt + 2);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(2);
+        mfma_group(3);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+    };
+    // A tile whose fast loads fit the buffer-load offsets runs pairs of steady
+    // steps; when K ends in a partial step, up to the step that requests that
+    // last tile (two steps ahead), and the general form takes what remains.
     int nsteady = 0;
-    if (AMODE != 2 && BMODE != 2 && a_fast && b_fast) nsteady = klen % BK == 0 ? nkt : max(nkt - 3, 0);
-    k_loop(Steady(), 0, nsteady);
-    k_loop(General(), nsteady, nkt);
+    if (a_fast && b_fast && stage_addr_fits<BM>(a_ld) && stage_addr_fits<BN>(b_ld))
+        nsteady = (klen % BK == 0 ? nkt : max(nkt - 3, 0)) & ~1;
+    for (int kt = 0; kt < nsteady; kt += 2) {
+        steady_step(std::integral_constant<int, 0>(), kt);
+        steady_step(std::integral_constant<int, 1>(), kt + 1);
+    }
+    for (int kt = nsteady; kt < nkt; ++kt) general_step(kt);
 
     // ---- epilogue -----------------------------------------------------------
     // A 32 x 32 MFMA block leaves lane l with column l%32 and rows
@@ -660,8 +688,12 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     const bool dgelu = !SK && !partial && g.epilogue == MNI_EPI_DGELU;
     float csum[4] = {0.f, 0.f, 0.f, 0.f};
     // all wavefronts are past their last LDS read (barrier at the end of the K loop)
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    // One 32-row strip of the wavefront's blocks at a time.  The strip index is a compile-time constant (a
+    // lambda called once per value, not a loop): were the loop left rolled -- the body is long, and with
+    // four strips the unroller declines -- the accumulators would be indexed at run time, live in scratch
+    // memory, and every MFMA of the K loop would be followed by a store of its result.
+    auto epilogue_strip = [&](auto strip) {
+        constexpr int i = decltype(strip)::value;
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -754,7 +786,11 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
             }
         }
         __syncthreads();
-    }
+    };
+    epilogue_strip(std::integral_constant<int, 0>());
+    if constexpr (TM > 1) epilogue_strip(std::integral_constant<int, 1>());
+    if constexpr (TM > 2) epilogue_strip(std::integral_constant<int, 2>());
+    if constexpr (TM > 3) epilogue_strip(std::integral_constant<int, 3>());
     if (dgelu && g.colsum_part) {
         // lanes that share columns (same lane % LANES_PER_ROW) are added by butterfly steps; strip
         // (batch, tile row, wm) owns one row of the partial matrix
