@@ -276,12 +276,11 @@ static int run_mfma(const mni_gemm_desc &d) {
     };
 
     // Tile shape and work distribution.  A side is 64 wide when that extent is
-    // at most 64 (no half-empty tiles).  Otherwise: 128 x 128 tiles when every
-    // resident workgroup gets a good stretch of K steps out of them, 64 x 64
-    // when not.  With the tile chosen: one workgroup per tile when the tiles
-    // fill their rounds on the machine well; else stream-K, which has no
-    // rounds to fill; else (device mapping unknown, tiny product) K slices and
-    // a reduction pass.
+    // at most 64 (no half-empty tiles).  Otherwise: one workgroup per tile of
+    // the biggest shape that deals the CUs equal loads; failing that, stream-K
+    // (which has no rounds to fill) over 128 x 128 tiles when there are more of
+    // them than workgroup slots and over 64 x 64 tiles when not; else (device
+    // mapping unknown, tiny product) K slices and a reduction pass.
     int bm = g.M <= 64 ? 64 : 128, bn = g.N <= 64 ? 64 : 128;
     bool streamk = false;
     bool whole_tiles = false;  // one workgroup per tile, no K slices
@@ -297,39 +296,40 @@ static int run_mfma(const mni_gemm_desc &d) {
     } else if (d.algo == MNI_ALGO_AUTO || d.algo == MNI_ALGO_MFMA_STREAMK) {
         const int64_t big_tiles = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
         const int64_t big_slots = (int64_t)cus * gemm_mfma_resident_per_cu(bm, bn);
-        if (ktiles >= 8 && d.split_k == 0 && sk_device) {
-            if (big_tiles * ktiles >= 20 * big_slots) {
-                // plenty of K steps per workgroup slot: big tiles
-                const int64_t rounds = (big_tiles + big_slots - 1) / big_slots;
-                whole_tiles = big_tiles * 100 >= rounds * big_slots * 93;
-                if (!whole_tiles && bm == 128 && bn == 128 && (amode == 0 || bmode == 0) && ktiles <= 64) {
-                    // Tiles halved along one side may fill their rounds where
-                    // 128 x 128 does not.  Over a few rounds of moderate K they
-                    // beat stream-K (they run within 5 % of the big tile; over
-                    // many rounds or a long K stream-K's fix-up of one last
-                    // round costs less than that).
-                    // The short side goes to an operand that is K-contiguous: one
-                    // that is transposed on the way to LDS keeps all threads busy
-                    // with its loads only at 128.
-                    const int hm = amode == 0 ? 64 : 128, hn = amode == 0 ? 128 : 64;
-                    const int64_t half_tiles = (int64_t)((g.M + hm - 1) / hm) * ((g.N + hn - 1) / hn) * g.batch;
-                    const int64_t half_slots = (int64_t)cus * gemm_mfma_resident_per_cu(hm, hn);
-                    const int64_t half_rounds = (half_tiles + half_slots - 1) / half_slots;
-                    if (half_rounds <= 3 && half_tiles * 100 >= half_rounds * half_slots * 93) {
-                        whole_tiles = true;
-                        bm = hm;
-                        bn = hn;
-                    }
+        // One workgroup per tile when some tile shape deals the CUs equal loads: a CU's matrix pipe is
+        // shared by the workgroups resident on it, so what counts is tiles per CU, not per workgroup slot
+        // (768 tiles of 128 x 128 on 256 CUs run as fast per tile as 1024 do), and at least two per CU,
+        // because one workgroup alone leaves a SIMD a single wavefront and its stalls uncovered.  The K
+        // loop issues no vector-ALU work whatever the tile shape, so a smaller tile costs only its extra
+        // L2 traffic: the biggest shape whose last round is at least 95 % full wins.  (Measured: whole
+        // tiles take ideal / fill, stream-K ideal x 1.03-1.05; 2560^3 with 64 x 64 tiles at 89 % loses 10 %
+        // to stream-K, 4096 x 768 x 3072 with 64 x 64 tiles at 100 % beats it by 10 %.)
+        if (ktiles >= 8 && d.split_k == 0 && d.algo == MNI_ALGO_AUTO) {
+            // Up to 32 K steps the smaller shapes run 1-3 % ahead (more workgroups to overlap prologues and
+            // epilogues with), except with A given as its transpose.
+            const int cand[4][2] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
+            const bool small_first = ktiles <= 32 && amode != 1;
+            for (int i = 0; i < 4 && !whole_tiles; ++i) {
+                const int cm = cand[small_first ? 3 - i : i][0], cn = cand[small_first ? 3 - i : i][1];
+                if (cm > bm || cn > bn) continue;
+                const int64_t tiles = (int64_t)((g.M + cm - 1) / cm) * ((g.N + cn - 1) / cn) * g.batch;
+                const int64_t per_cu = (tiles + cus - 1) / cus;
+                if (per_cu >= 2 && tiles * 100 >= per_cu * cus * 95) {
+                    whole_tiles = true;
+                    bm = cm;
+                    bn = cn;
                 }
-                // (under 3/16 of the slots: long K over few tiles, left to the K slices below)
-                if (!whole_tiles && big_tiles * 16 >= 3 * big_slots) streamk = streamk_fits(bm, bn, 8);
+            }
+        }
+        if (whole_tiles) {
+            // settled above
+        } else if (ktiles >= 8 && d.split_k == 0 && sk_device) {
+            if (big_tiles >= big_slots && big_tiles * ktiles >= 20 * big_slots) {
+                // more big tiles than workgroup slots and plenty of K steps per slot: stream-K over big tiles
+                streamk = streamk_fits(bm, bn, 8);
             } else {
-                const int64_t tiles = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) * g.batch;
-                const int64_t slots = (int64_t)cus * gemm_mfma_resident_per_cu(64, 64);
-                const int64_t rounds = (tiles + slots - 1) / slots;
-                whole_tiles = tiles * 100 >= rounds * slots * 70;
-                if (!whole_tiles) streamk = streamk_fits(64, 64, 8);
-                if (whole_tiles || streamk) bm = bn = 64;
+                streamk = streamk_fits(64, 64, 8);
+                if (streamk) bm = bn = 64;
             }
         } else {
             // short K, a requested split, or no stream-K on this device: 64 x 64 when
