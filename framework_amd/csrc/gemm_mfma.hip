@@ -16,26 +16,28 @@
 // the last MFMAs of step t are refilled with tile t+2 right away, so a load has
 // a whole step of MFMAs to land before it is needed.
 //
-// LDS layout.  Both operand tiles are stored "K-quad major":
-//     tile[k/4][row][k%4]        (row = m for A, n for B; one float4 per row)
-// so that one ds_read_b128 gives a lane the four K values it feeds to four
-// consecutive MFMAs, and the 32 lanes of a half-wave read 32 consecutive
-// float4 (conflict-free).  The MFMA takes k = lane/32 from each lane; because
-// A and B use the same (k/4, k%4) split, lane half h contracts k = 8c+4h+j at
-// MFMA j of chunk c, and the order of the K sum is the only thing that differs
-// from a textbook loop.
-//
-// Operand layouts (transposes folded into the load path).  An operand whose K
-// axis has unit stride (A row-major, or B given as its transpose) is loaded
-// with 16-byte loads along K.  An operand whose M/N axis has unit stride (B
-// row-major, or A given as its transpose) is loaded with 4-byte loads, each
-// wavefront instruction covering 64 consecutive rows of one K value, four of
-// them filling the register quad that holds a row's K quad.  Either way the
-// registers are stored to LDS as they are.  The loads need no more than the
-// 4-byte alignment every float has (the memory system splits a 16-byte load
-// that straddles a cache line), so odd leading dimensions and offset bases take
-// these paths too.  Anything else (neither axis contiguous, K tails) takes
-// guarded scalar loads into the same register layout.
+// LDS layout and operand layouts (transposes folded into the load path).  The
+// MFMA takes k = lane/32 from each lane, so a lane feeds four consecutive MFMAs
+// from four K values of one row (m for A, n for B); lane half h contracts
+// k = 8c+4h+j at MFMA j of chunk c for both operands, and the order of the K
+// sum is the only thing that differs from a textbook loop.
+// An operand whose K axis has unit stride (A row-major, or B given as its
+// transpose) is loaded with 16-byte loads along K and stored "K-quad major",
+//     tile[k/4][row][k%4]        (one float4 per row),
+// so that one ds_read_b128 gives a lane its four K values and the 32 lanes of a
+// half-wave read 32 consecutive float4 (conflict-free).
+// An operand whose M/N axis has unit stride (B row-major, or A given as its
+// transpose) is loaded with 16-byte loads along M/N and stored as it comes,
+//     tile[k][row],
+// and a lane gathers its four K values with four 4-byte reads (32 consecutive
+// floats per half-wave, the halves 32 banks apart).  Nothing is transposed in
+// registers: LDS instructions are free where vector-ALU instructions are not
+// (see the K loop below).
+// The 16-byte loads need no more than the 4-byte alignment every float has (the
+// memory system splits a load that straddles a cache line), so odd leading
+// dimensions and offset bases take these paths too.  Anything else (neither
+// axis contiguous, K tails, edges of an M/N-contiguous operand off a multiple
+// of 4) takes guarded scalar loads into the same register layout.
 //
 // K loop.  Tile kt+1 sits in staging registers while tile kt is multiplied out
 // of LDS; in the last quarter of a step the staged tile goes to the other LDS
@@ -103,41 +105,36 @@ __device__ __forceinline__ int lds_row(int r) { return r ^ ((r >> 4) & 3); }
 
 // ---- global -> register loads ---------------------------------------------
 // A tile side has ROWS = 256, 128 or 64 rows (m for A, n for B) and BK = 32 K
-// values: ROWS / 32 float4 per thread.
+// values: ROWS / 32 16-byte pieces per thread.
 // Register layout LAYOUT 0 (K contiguous): thread owns float4 #(tid + 256 i),
-//   i < ROWS/32, where float4 #f is row f/8, K quad f%8: one 16-byte load each.
-// Register layout LAYOUT 1 (M/N contiguous): thread owns row tid % ROWS and the
-//   K quads tid / ROWS + (256 / ROWS) p, p < ROWS/32; v[p] holds the quad's four
-//   K values, fetched by four 4-byte loads (64 lanes = 256 consecutive bytes
-//   each).  Either way a register quad is what one LDS slot holds, so nothing
-//   is shuffled between the load and the LDS store: every vector-ALU instruction
-//   in the K loop takes its cycles from the fp32 MFMAs (a v_mov per MFMA costs
-//   8 % of the matrix rate on this chip; loads, LDS traffic and scalar work cost
-//   nothing), so the loop is built to contain none.
+//   i < ROWS/32, where float4 #f is row f/8, K quad f%8: four K values of one
+//   row, which is what one LDS slot holds.
+// Register layout LAYOUT 1 (M/N contiguous): thread owns rows 4 r4 .. 4 r4 + 3,
+//   r4 = tid % (ROWS/4), at the K values tid / (ROWS/4) + (1024 / ROWS) i,
+//   i < ROWS/32: one 16-byte load along M/N each.  Its four components belong
+//   to four different LDS slots and are stored there one by one (4-byte LDS
+//   stores).  Nothing is shuffled in registers in either layout: every
+//   vector-ALU instruction in the K loop takes its cycles from the fp32 MFMAs (a
+//   v_mov per MFMA costs 8 % of the matrix rate on this chip; loads, LDS
+//   traffic and scalar work cost nothing), so the loop is built to contain none.
 template <int ROWS> __device__ constexpr int stage_regs() { return ROWS / 32 > 4 ? ROWS / 32 : 4; }
-template <int ROWS> __device__ constexpr int quad_stride() { return NTHREADS / ROWS; }  // K quads covered per pass (layout 1)
+template <int ROWS> __device__ constexpr int k_stride() { return 4 * NTHREADS / ROWS; }  // K rows covered per pass (layout 1)
 
-// Rows at or beyond `rows` (an edge tile) are read from the last valid row
-// instead: what they contribute lands in accumulator rows / columns that the
-// epilogue never stores.
+// Rows at or beyond `rows` (an edge tile; a multiple of 4 for layout 1) are
+// read from the last valid row or row quad instead: what they contribute lands
+// in accumulator rows / columns that the epilogue never stores.
 template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void load_fast(const float *__restrict__ p, int64_t ld, int rows, int tid, float4 (&v)[stage_regs<ROWS>()]) {
-    if (LAYOUT == 0) {
 #pragma unroll
-        for (int i = 0; i < ROWS / 32; ++i) {
+    for (int i = 0; i < ROWS / 32; ++i) {
+        if (LAYOUT == 0) {
             int f = tid + NTHREADS * i;
             int row = min(f >> 3, rows - 1), q = f & 7;
             v[i] = *reinterpret_cast<const float4 *>(p + (int64_t)row * ld + 4 * q);
-        }
-    } else {
-        constexpr int QS = quad_stride<ROWS>();
-        const int n = min(tid % ROWS, rows - 1), q0 = tid / ROWS;
-#pragma unroll
-        for (int ps = 0; ps < ROWS / 32; ++ps) {
-            float t[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) t[j] = p[n + (int64_t)(4 * (q0 + QS * ps) + j) * ld];
-            v[ps] = make_float4(t[0], t[1], t[2], t[3]);
+        } else {
+            constexpr int R4 = ROWS / 4;
+            const int r4 = min(tid % R4, rows / 4 - 1), k = tid / R4 + k_stride<ROWS>() * i;
+            v[i] = *reinterpret_cast<const float4 *>(p + 4 * r4 + (int64_t)k * ld);
         }
     }
 }
@@ -153,53 +150,75 @@ __device__ __forceinline__ void load_guarded(const float *__restrict__ p, int64_
     asm volatile("" : "+v"(tid));
 #pragma unroll
     for (int i = 0; i < ROWS / 32; ++i) {
-        int row, q;
-        if (LAYOUT == 0) {
-            const int f = tid + NTHREADS * i;
-            row = f >> 3, q = f & 7;
-        } else {
-            row = tid % ROWS, q = tid / ROWS + quad_stride<ROWS>() * i;
-        }
         float t[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            int k = 4 * q + e;
+            int row, k;
+            if (LAYOUT == 0) {
+                const int f = tid + NTHREADS * i;
+                row = f >> 3, k = 4 * (f & 7) + e;
+            } else {
+                row = 4 * (tid % (ROWS / 4)) + e, k = tid / (ROWS / 4) + k_stride<ROWS>() * i;
+            }
             t[e] = (row < rmax && k < kmax) ? p[(int64_t)row * rs + (int64_t)k * cs] : 0.0f;
         }
         v[i] = make_float4(t[0], t[1], t[2], t[3]);
     }
 }
 
-// ---- register -> LDS --------------------------------------------------------
-// float4 slot of piece i of this thread within a tile stage
+// ---- register -> LDS, LDS -> MFMA operands -----------------------------------
+// A tile stage in LDS, by layout:
+//   0: float4 tile[K quad][row] (pitch ROWS + PAD slots): a register quad is one
+//      slot, and one ds_read_b128 gives a lane the K values of four MFMAs;
+//   1: float  tile[k][row] (pitch ROWS + 8 floats): a register quad (four rows
+//      at one K value) is 16 contiguous bytes, and a lane gathers its four K
+//      values with four 4-byte reads.  The pitch puts the rows of K value k + 4
+//      -- what the other half of the wavefront reads -- 32 banks further on.
+// LDS instructions cost the matrix pipe nothing; a transpose in registers
+// would.
 template <int LAYOUT, int ROWS>
-__device__ __forceinline__ int lds_slot(int tid, int i) {
-    constexpr int SLICE = ROWS + PAD;
+__device__ constexpr int stage_slots() { return LAYOUT == 0 ? KQ * (ROWS + PAD) : BK * (ROWS + 8) / 4; }  // float4 per stage
+
+template <int LAYOUT, int ROWS>
+__device__ __forceinline__ void store_piece(float4 *__restrict__ tile, int tid, int i, const float4 &v) {
     if (LAYOUT == 0) {
         const int f = tid + NTHREADS * i;
-        return (f & 7) * SLICE + lds_row(f >> 3);
+        tile[(f & 7) * (ROWS + PAD) + lds_row(f >> 3)] = v;
+    } else {
+        const int k = tid / (ROWS / 4) + k_stride<ROWS>() * i;
+        tile[k * ((ROWS + 8) / 4) + tid % (ROWS / 4)] = v;
     }
-    return (tid / ROWS + quad_stride<ROWS>() * i) * SLICE + lds_row(tid % ROWS);
 }
 
 template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void store_lds(float4 *__restrict__ tile, int tid, const float4 (&v)[stage_regs<ROWS>()]) {
 #pragma unroll
-    for (int i = 0; i < ROWS / 32; ++i) tile[lds_slot<LAYOUT, ROWS>(tid, i)] = v[i];
+    for (int i = 0; i < ROWS / 32; ++i) store_piece<LAYOUT, ROWS>(tile, tid, i, v[i]);
+}
+
+// What a lane keeps per MFMA block row: where row `row` of the tile sits in a stage.
+template <int LAYOUT>
+__device__ __forceinline__ int frag_row(int row) { return LAYOUT == 0 ? lds_row(row) : row; }
+
+// K values 8 c + 4 h + 0..3 of the row: the operands of the four MFMA groups of chunk c for lane half h.
+template <int LAYOUT, int ROWS>
+__device__ __forceinline__ float4 frag_load(const float4 *__restrict__ tile, int c, int h, int frow) {
+    if (LAYOUT == 0) return tile[(2 * c + h) * (ROWS + PAD) + frow];
+    const float *t = reinterpret_cast<const float *>(tile) + (8 * c + 4 * h) * (ROWS + 8) + frow;
+    return make_float4(t[0], t[ROWS + 8], t[2 * (ROWS + 8)], t[3 * (ROWS + 8)]);
 }
 
 // ---- the steady K loop's transfers -------------------------------------------
 // In the steady loop a tile side moves in pieces dealt out behind the MFMAs:
 // first the ROWS/32 LDS stores of the staged tile, then the loads that refill
 // the staging registers.  The loads are buffer loads: the tile's base address
-// and the K advance sit in the scalar resource descriptor, row offsets that
-// depend on the leading dimension in a scalar offset, and the only vector
-// register involved is a per-thread byte offset computed once ahead of the loop.
+// and the K advance sit in the scalar resource descriptor, offsets that depend
+// on the leading dimension in a scalar offset, and the only vector register
+// involved is a per-thread byte offset computed once ahead of the loop.
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 struct StageAddr {
-    int voff[8];  // layout 0: byte offset of piece i; layout 1: voff[0] = byte offset of the thread's row
-    int quad0;    // layout 1: byte offset of the thread's first K row, 4 * (tid / ROWS) * ld * 4 (uniform per wavefront)
+    int voff[8];  // layout 0: byte offset of piece i; layout 1: voff[0] = byte offset of the thread's row quad at its first K row
     int ldb;      // leading dimension in bytes
 };
 
@@ -207,7 +226,6 @@ template <int LAYOUT, int ROWS>
 __device__ __forceinline__ StageAddr stage_addr(int64_t ld, int rows, int tid) {
     StageAddr s;
     s.ldb = (int)ld * 4;
-    s.quad0 = 0;
     if (LAYOUT == 0) {
 #pragma unroll
         for (int i = 0; i < ROWS / 32; ++i) {
@@ -215,8 +233,7 @@ __device__ __forceinline__ StageAddr stage_addr(int64_t ld, int rows, int tid) {
             s.voff[i] = (min(f >> 3, rows - 1) * (int)ld + 4 * (f & 7)) * 4;
         }
     } else {
-        s.voff[0] = min(tid % ROWS, rows - 1) * 4;
-        s.quad0 = __builtin_amdgcn_readfirstlane(tid / ROWS) * 4 * s.ldb;
+        s.voff[0] = 16 * min(tid % (ROWS / 4), rows / 4 - 1) + (tid / (ROWS / 4)) * s.ldb;
     }
     return s;
 }
@@ -230,26 +247,20 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t stage_rsrc(const float *p) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p), 0, -1, 0x00020000);
 }
 
-template <int LAYOUT, int ROWS>
-__device__ constexpr int tile_pieces() { return LAYOUT == 0 ? 2 * (ROWS / 32) : 5 * (ROWS / 32); }
+template <int ROWS>
+__device__ constexpr int tile_pieces() { return 2 * (ROWS / 32); }
 
 template <int LAYOUT, int ROWS>
 __device__ __forceinline__ void tile_piece(int x, float4 *__restrict__ tile, __amdgpu_buffer_rsrc_t rsrc, const StageAddr &sa,
                                            int tid, float4 (&v)[stage_regs<ROWS>()]) {
     constexpr int NV = ROWS / 32;
     if (x < NV) {
-        tile[lds_slot<LAYOUT, ROWS>(tid, x)] = v[x];
-    } else if (LAYOUT == 0) {
-        const floatx4 t = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, sa.voff[x - NV], 0, 0));
-        v[x - NV] = make_float4(t.x, t.y, t.z, t.w);
+        store_piece<LAYOUT, ROWS>(tile, tid, x, v[x]);
     } else {
-        const int y = x - NV, ps = y >> 2, j = y & 3;
-        const float t = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-            rsrc, sa.voff[0], sa.quad0 + (4 * quad_stride<ROWS>() * ps + j) * sa.ldb, 0));
-        if (j == 0) v[ps].x = t;
-        if (j == 1) v[ps].y = t;
-        if (j == 2) v[ps].z = t;
-        if (j == 3) v[ps].w = t;
+        const int i = x - NV;
+        const floatx4 t = __builtin_bit_cast(floatx4, LAYOUT == 0 ? __builtin_amdgcn_raw_buffer_load_b128(rsrc, sa.voff[i], 0, 0)
+                                                                  : __builtin_amdgcn_raw_buffer_load_b128(rsrc, sa.voff[0], k_stride<ROWS>() * i * sa.ldb, 0));
+        v[i] = make_float4(t.x, t.y, t.z, t.w);
     }
 }
 
@@ -299,11 +310,10 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     constexpr int AL = AMODE == 1 ? 1 : 0;
     constexpr int BL = BMODE == 1 ? 1 : 0;
     constexpr int BM = 64 * TM, BN = 64 * TN;
-    constexpr int SLICE_A = BM + PAD, SLICE_B = BN + PAD;
     // One LDS block: two stages of the A tile, two of the B tile; the epilogue
     // reuses it to turn the MFMA accumulator layout into row-contiguous 16-byte
     // stores.
-    constexpr int STAGE_A = KQ * SLICE_A, STAGE_B = KQ * SLICE_B;
+    constexpr int STAGE_A = stage_slots<AL, BM>(), STAGE_B = stage_slots<BL, BN>();
     __shared__ float4 lds[2 * STAGE_A + 2 * STAGE_B];
     auto stage_a = [&](int st) -> float4 * { return lds + st * STAGE_A; };
     auto stage_b = [&](int st) -> float4 * { return lds + 2 * STAGE_A + st * STAGE_B; };
@@ -364,9 +374,9 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     // float4 slots of this lane's A row blocks and B column blocks
     int a_row[TM], b_row[TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) a_row[i] = lds_row(wm * (32 * TM) + 32 * i + r);
+    for (int i = 0; i < TM; ++i) a_row[i] = frag_row<AL>(wm * (32 * TM) + 32 * i + r);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) b_row[j] = lds_row(wn * (32 * TN) + 32 * j + r);
+    for (int j = 0; j < TN; ++j) b_row[j] = frag_row<BL>(wn * (32 * TN) + 32 * j + r);
 
     int64_t pid;
     int role, k_begin, k_end, slice = 0;
@@ -441,10 +451,11 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         g.B + (int64_t)(batch % g.b_bcount) * g.b_bs + (int64_t)n0 * g.b_cs + (int64_t)k_begin * g.b_rs;
     const int mrem = g.M - m0, nrem = g.N - n0;
     // Fast loads also serve an edge tile (rows beyond the edge re-read the last
-    // valid ones).
+    // valid ones), except that 16-byte loads along M/N need the edge on a
+    // multiple of 4.
     const int a_rows = min(mrem, BM), b_rows = min(nrem, BN);
-    const bool a_fast = AMODE != 2;
-    const bool b_fast = BMODE != 2;
+    const bool a_fast = AMODE == 0 || (AMODE == 1 && a_rows % 4 == 0);
+    const bool b_fast = BMODE == 0 || (BMODE == 1 && b_rows % 4 == 0);
     // leading dimension seen by the fast loaders
     const int64_t a_ld = AMODE == 0 ? g.a_rs : g.a_cs;
     const int64_t b_ld = BMODE == 0 ? g.b_cs : g.b_rs;
@@ -513,22 +524,21 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     // The first three quarters of a K step: MFMAs of chunk c with the fragment
     // reads of chunk c + 1 between the groups.
     auto chunk = [&](const float4 *As, const float4 *Bs, int c) {
-        const int qa = (2 * (c + 1) + h) * SLICE_A, qb = (2 * (c + 1) + h) * SLICE_B;
         __builtin_amdgcn_sched_barrier(0);
         mfma_group(0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) na[i] = As[qa + a_row[i]];
+        for (int i = 0; i < TM; ++i) na[i] = frag_load<AL, BM>(As, c + 1, h, a_row[i]);
         __builtin_amdgcn_sched_barrier(0);
         mfma_group(1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < (TN + 1) / 2; ++j) nb[j] = Bs[qb + b_row[j]];
+        for (int j = 0; j < (TN + 1) / 2; ++j) nb[j] = frag_load<BL, BN>(Bs, c + 1, h, b_row[j]);
         __builtin_amdgcn_sched_barrier(0);
         mfma_group(2);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = (TN + 1) / 2; j < TN; ++j) nb[j] = Bs[qb + b_row[j]];
+        for (int j = (TN + 1) / 2; j < TN; ++j) nb[j] = frag_load<BL, BN>(Bs, c + 1, h, b_row[j]);
         __builtin_amdgcn_sched_barrier(0);
         mfma_group(3);
         __builtin_amdgcn_sched_barrier(0);
@@ -553,12 +563,12 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         const int kt2 = min(kt + 2, nkt - 1);
         const float4 *As = stage_a(cur), *Bs = stage_b(cur);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = As[h * SLICE_A + a_row[i]];
+        for (int i = 0; i < TM; ++i) fa[i] = frag_load<AL, BM>(As, 0, h, a_row[i]);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = Bs[h * SLICE_B + b_row[j]];
+        for (int j = 0; j < TN; ++j) fb[j] = frag_load<BL, BN>(Bs, 0, h, b_row[j]);
 #pragma unroll
         for (int c = 0; c < NCHUNK - 1; ++c) chunk(As, Bs, c);
-        constexpr int PA = tile_pieces<AL, BM>(), PB = tile_pieces<BL, BN>();
+        constexpr int PA = tile_pieces<BM>(), PB = tile_pieces<BN>();
         constexpr int SLOTS = 4 * TM * TN, PER = (PA + PB + SLOTS - 1) / SLOTS;
         const __amdgpu_buffer_rsrc_t ra_src = stage_rsrc(AMODE == 0 ? Ap + (int64_t)kt2 * BK : Ap + (int64_t)kt2 * BK * a_ld);
         const __amdgpu_buffer_rsrc_t rb_src = stage_rsrc(BMODE == 0 ? Bp + (int64_t)kt2 * BK : Bp + (int64_t)kt2 * BK * b_ld);
@@ -589,9 +599,9 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         const bool more = kt + 1 < nkt, more2 = kt + 2 < nkt;
         const float4 *As = stage_a(cur), *Bs = stage_b(cur);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = As[h * SLICE_A + a_row[i]];
+        for (int i = 0; i < TM; ++i) fa[i] = frag_load<AL, BM>(As, 0, h, a_row[i]);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = Bs[h * SLICE_B + b_row[j]];
+        for (int j = 0; j < TN; ++j) fb[j] = frag_load<BL, BN>(Bs, 0, h, b_row[j]);
 #pragma unroll
         for (int c = 0; c < NCHUNK - 1; ++c) chunk(As, Bs, c);
         __builtin_amdgcn_sched_barrier(0);
