@@ -324,9 +324,14 @@ static int run_mfma(const mni_gemm_desc &d) {
         if (whole_tiles) {
             // settled above
         } else if (ktiles >= 8 && d.split_k == 0 && sk_device) {
-            if (big_tiles >= big_slots && big_tiles * ktiles >= 20 * big_slots) {
+            const bool long_k = big_tiles * ktiles >= 20 * big_slots;
+            if (long_k && big_tiles >= big_slots) {
                 // more big tiles than workgroup slots and plenty of K steps per slot: stream-K over big tiles
                 streamk = streamk_fits(bm, bn, 8);
+            } else if (long_k && big_tiles * 16 < 3 * big_slots && ((int64_t)g.M + g.N) * g.K * 4 > (128LL << 20)) {
+                // A handful of big tiles over a K so long that the operands outgrow the Infinity Cache:
+                // 64 x 64 tiles would stream them twice as often (1024 x 1024 x 65536: 1127 us against
+                // 1015 us for 128 x 128 tiles in K slices, the plan below)
             } else {
                 streamk = streamk_fits(64, 64, 8);
                 if (streamk) bm = bn = 64;
