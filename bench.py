@@ -166,6 +166,12 @@ def bench_yardsticks(r):
     out["hbm_copy_yardstick_64MiB"] = line(r.yardstick_timed("copy", n, dst=bufs[8], srcs=bufs[:1], iters=100), 2 * n)
     for b in bufs:
         r.free(b)
+    # What the matrix pipe gives a loop of nothing but fp32 MFMAs (two wavefronts per SIMD, as the tile kernel has),
+    # and with one or two register moves behind every MFMA: the vector ALU's issue time comes out of the MFMAs'.
+    tf = [r.mfma_yardstick(v) for v in (0, 1, 2)]
+    out["mfma_yardstick"] = {"TFLOP/s": tf[0], "frac_mfma": tf[0] / PEAK_FP32_MATRIX_TFLOPS,
+                             "with_1_v_mov_per_mfma": tf[1], "with_2_v_mov_per_mfma": tf[2],
+                             "note": "v_mfma_f32_32x32x2_f32 on four independent accumulators per wavefront, nothing else in the loop"}
     return out
 
 

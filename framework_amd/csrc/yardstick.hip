@@ -1,6 +1,6 @@
-// Memory-system yardsticks, timed the way mni_rocm_sgemm_timed times products:
-// an empty launch, a pure read, a pure write and a copy of a caller-supplied
-// buffer.  They say what this device gives a kernel that does nothing but
+// Yardsticks, timed the way mni_rocm_sgemm_timed times products: an empty
+// launch, a pure read, a pure write and a copy of a caller-supplied buffer, and
+// a loop of nothing but MFMAs.  They say what this device gives a kernel that does nothing but
 // stream -- the figure a bandwidth-bound product (the skinny kernels, the
 // batched attention-shaped products) is to be held against, next to the
 // datasheet's.  No counterpart in the reference.
@@ -67,9 +67,80 @@ __global__ __launch_bounds__(YS_THREADS) void ys_copy_kernel(f32x4 *__restrict__
     for (; p < hi; p += YS_THREADS) dst[p] = src[p];
 }
 
+// What the matrix pipe gives a loop of nothing but fp32 MFMAs, and what it
+// still gives when every MFMA is followed by VALU vector-ALU instructions that
+// depend on nothing: on this chip the fp32 MFMA and the vector ALU share issue
+// time, so the second figure is what any kernel pays per address computation or
+// register move inside its MFMA loop.  Four independent accumulators per
+// wavefront (an MFMA never waits for the one before it).
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <int VALU>
+__global__ __launch_bounds__(YS_THREADS) void ys_mfma_kernel(float *sink, int rounds) {
+    floatx16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+    const float a = threadIdx.x * 1e-6f, b = blockIdx.x * 1e-6f;
+    float x = a, y = b;
+    for (int it = 0; it < rounds; ++it) {
+#pragma unroll
+        for (int rep = 0; rep < 4; ++rep)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int v = 0; v < VALU; ++v) asm volatile("v_mov_b32 %0, %1" : "=v"(x) : "v"(y));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    }
+    float s = x;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s += acc[i][e];
+    if (s == -1.2345678e38f) *sink = s;
+}
+
 }  // namespace mni
 
 using namespace mni;
+
+extern "C" int mni_rocm_mfma_yardstick_timed(int valu_per_mfma, int waves_per_simd, int mfmas_per_wave, int warmup, int iters, float *avg_ms) {
+    MNI_API_GUARD;
+    MNI_TRY(ensure_init());
+    if (valu_per_mfma < 0 || valu_per_mfma > 2 || waves_per_simd < 1 || waves_per_simd > 2 || mfmas_per_wave < 16 || mfmas_per_wave % 16 != 0 ||
+        iters <= 0 || warmup < 0 || !avg_ms)
+        return set_error(MNI_ERR_INVALID, "mfma yardstick: bad arguments");
+    DeviceCtx &c = ctx();
+    const dim3 grid((unsigned)((c.compute_units > 0 ? c.compute_units : 256) * waves_per_simd)), block(YS_THREADS);
+    float *sink = (float *)c.skinny_flags;  // never written
+    const int rounds = mfmas_per_wave / 16;
+    auto launch = [&]() {
+        if (valu_per_mfma == 0) MNI_KERNEL_LAUNCH((ys_mfma_kernel<0>), grid, block, 0, c.stream, sink, rounds);
+        else if (valu_per_mfma == 1) MNI_KERNEL_LAUNCH((ys_mfma_kernel<1>), grid, block, 0, c.stream, sink, rounds);
+        else MNI_KERNEL_LAUNCH((ys_mfma_kernel<2>), grid, block, 0, c.stream, sink, rounds);
+    };
+    for (int i = 0; i < warmup; ++i) launch();
+    MNI_TRY(check_launch("mfma yardstick"));
+    hipEvent_t e0, e1;
+    MNI_HIP_CHECK(hipEventCreate(&e0));
+    MNI_HIP_CHECK(hipEventCreate(&e1));
+    hipError_t he = hipEventRecord(e0, c.stream);
+    for (int i = 0; i < iters; ++i) launch();
+    if (he == hipSuccess) he = hipEventRecord(e1, c.stream);
+    if (he == hipSuccess) he = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (he != hipSuccess) return set_error(MNI_ERR_HIP, "mfma yardstick: %s", hipGetErrorString(he));
+    MNI_TRY(check_launch("mfma yardstick"));
+    *avg_ms = ms / (float)iters;
+    return MNI_OK;
+}
 
 extern "C" int mni_rocm_yardstick_timed(int kind, int nontemporal, void *dst, const void *const *srcs, int nsrc, size_t bytes,
                                         int blocks_per_cu, int warmup, int iters, float *avg_ms) {

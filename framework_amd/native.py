@@ -73,6 +73,7 @@ SIGNATURES = {
     "mni_rocm_sgemm_timed": (C.c_int, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
     "mni_rocm_yardstick_timed": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_size_t, C.c_int, C.c_int,
                                            C.c_int, C.POINTER(C.c_float)]),
+    "mni_rocm_mfma_yardstick_timed": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
     "mni_rocm_strided_copy": (C.c_int, [C.c_void_p, C.c_void_p, _i64p, _i64p, C.c_int]),
     "mni_rocm_add_bias": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
     "mni_rocm_colsum": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
@@ -302,6 +303,13 @@ class Rocm:
         self._check(self.lib.mni_rocm_yardstick_timed(code, 1 if nontemporal else 0, dst, arr, len(srcs), nbytes, blocks_per_cu,
                                                       warmup, iters, C.byref(ms)))
         return ms.value
+
+    def mfma_yardstick(self, valu_per_mfma=0, waves_per_simd=2, mfmas_per_wave=32768, warmup=2, iters=5):
+        """TFLOP/s of a loop of nothing but fp32 MFMAs with `valu_per_mfma` independent v_mov_b32 behind each."""
+        ms = C.c_float(0)
+        self._check(self.lib.mni_rocm_mfma_yardstick_timed(valu_per_mfma, waves_per_simd, mfmas_per_wave, warmup, iters, C.byref(ms)))
+        cus = self.device_info()["compute_units"]
+        return cus * 4 * waves_per_simd * mfmas_per_wave * 4096.0 / (ms.value * 1e-3) / 1e12
 
     def strided_copy(self, dst, src, shape, strides):
         self._check(self.lib.mni_rocm_strided_copy(dst, src, _i64_array(shape), _i64_array(strides), len(shape)))

@@ -192,6 +192,17 @@ int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int 
 enum { MNI_YARDSTICK_EMPTY = 0, MNI_YARDSTICK_READ = 1, MNI_YARDSTICK_WRITE = 2, MNI_YARDSTICK_COPY = 3 };
 int mni_rocm_yardstick_timed(int kind, int nontemporal, void *dst, const void *const *srcs, int nsrc, size_t bytes,
                              int blocks_per_cu, int warmup, int iters, float *avg_ms);
+/* Measurement aid (no counterpart in the reference): what the matrix pipe
+ * gives a loop of nothing but fp32 MFMAs.  Every wavefront issues
+ * `mfmas_per_wave` (a multiple of 16) v_mfma_f32_32x32x2_f32 on four
+ * independent accumulators, each followed by `valu_per_mfma` (0..2) v_mov_b32
+ * that depend on nothing; the grid is `waves_per_simd` (1 or 2) workgroups of
+ * four wavefronts per compute unit.  Returns the average milliseconds per
+ * launch; the rate is CUs * 4 * waves_per_simd * mfmas_per_wave * 4096 flop
+ * over that.  The figure with valu_per_mfma = 0 is the ceiling an MFMA-bound
+ * product is held against next to the datasheet's; the others show what every
+ * vector-ALU instruction inside an MFMA loop costs on this device. */
+int mni_rocm_mfma_yardstick_timed(int valu_per_mfma, int waves_per_simd, int mfmas_per_wave, int warmup, int iters, float *avg_ms);
 
 /* dst (contiguous, `shape`) = gather of src by `src_strides` (elements).
  * Replaces permute_f32 (src/native/kernels/elementwise.cu:67-81) and the host

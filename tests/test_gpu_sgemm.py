@@ -842,3 +842,12 @@ def test_sgemm_timed_runs_the_products_and_reports_a_duration(dev, rocm):
         assert np.array_equal(rocm.to_host(dC, (64, 80)), (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
     with pytest.raises(N.MniError):
         rocm.sgemm_timed(descs, 0, 0)
+
+
+def test_mfma_yardstick_runs_and_shows_what_a_register_move_costs(rocm):
+    pure = rocm.mfma_yardstick(0, mfmas_per_wave=8192)
+    moved = rocm.mfma_yardstick(2, mfmas_per_wave=8192)
+    assert 100.0 < pure < 160.0          # TFLOP/s: below the 157.3 datasheet peak, well above any product
+    assert moved < pure                  # vector-ALU instructions take their issue time from the MFMAs
+    with pytest.raises(N.MniError, match="bad arguments"):
+        rocm.mfma_yardstick(3)
