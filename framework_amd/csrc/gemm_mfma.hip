@@ -264,29 +264,28 @@ __device__ __forceinline__ void tile_piece(int x, float4 *__restrict__ tile, __a
     }
 }
 
-// tanh through the hardware's exp2 and reciprocal: 1 - 2 / (1 + e^{2x}) (exact limits at both ends, absolute
-// error ~1e-6).  The library's tanhf costs some forty instructions, and an epilogue that calls it once per
-// element while the matrix pipe waits made the fused GELU products 25 us slower than the plain ones plus a
-// separate pass; this form costs five.
-__device__ __forceinline__ float fast_tanh(float x) {
-    const float t = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);  // e^{2x} = 2^{2x log2(e)}
-    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + t);
+// GELU (tanh approximation, src/native/src/ops/activation.rs:15-28) in the epilogues.  With u = s (x + c x^3),
+// s = sqrt(2/pi), c = 0.044715:  0.5 (1 + tanh u) = 1 / (1 + e^{-2u}) =: sig, so
+//     gelu(x)  = x sig
+//     gelu'(x) = sig + 0.5 x sech^2(u) u' = sig (1 + x (1 - sig) 2u'),   2u' = 2s + 6sc x^2,
+// through the hardware's exp2 and reciprocal (exact limits at both ends, absolute error ~1e-6): seven instructions for
+// the value, eleven for the derivative.  The count matters: an epilogue's vector-ALU instructions are paid for in MFMA
+// time of the workgroup that shares the SIMDs (the library's tanhf, some forty instructions, made the fused GELU
+// products 25 us slower than the plain ones plus a separate pass).
+__device__ __forceinline__ float gelu_sig(float x, float x2) {
+    const float c0 = -2.0f * 0.7978845608028654f * 1.4426950408889634f;             // -2 s log2(e)
+    const float c1 = -2.0f * 0.7978845608028654f * 0.044715f * 1.4426950408889634f;  // -2 s c log2(e)
+    const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(x2, c1, c0));           // e^{-2u}
+    return __builtin_amdgcn_rcpf(1.0f + e);
 }
 
-__device__ __forceinline__ float gelu_tanh(float x) {
-    // tanh-approximation GELU of the reference (src/native/src/ops/activation.rs:15-18)
-    const float s = 0.7978845608028654f;  // sqrt(2/pi)
-    return 0.5f * x * (1.0f + fast_tanh(s * (x + 0.044715f * x * x * x)));
-}
+__device__ __forceinline__ float gelu_tanh(float x) { return x * gelu_sig(x, x * x); }
 
 __device__ __forceinline__ float gelu_tanh_grad(float x) {
-    // src/native/src/ops/activation.rs:20-28
-    const float s = 0.7978845608028654f;
-    const float inner = s * (x + 0.044715f * x * x * x);
-    const float th = fast_tanh(inner);
-    const float sech2 = 1.0f - th * th;
-    const float d_inner = s * (1.0f + 3.0f * 0.044715f * x * x);
-    return 0.5f * (1.0f + th) + 0.5f * x * sech2 * d_inner;
+    const float x2 = x * x;
+    const float sig = gelu_sig(x, x2);
+    const float du2 = __builtin_fmaf(x2, 6.0f * 0.7978845608028654f * 0.044715f, 2.0f * 0.7978845608028654f);  // 2u'
+    return sig * __builtin_fmaf(x * du2, 1.0f - sig, 1.0f);
 }
 
 __device__ __forceinline__ float pick(const float4 &v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; }
@@ -697,7 +696,30 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     const bool dual = !SK && !partial && g.epilogue == MNI_EPI_BIAS_GELU_DUAL;
     const bool dgelu = !SK && !partial && g.epilogue == MNI_EPI_DGELU;
     float csum[4] = {0.f, 0.f, 0.f, 0.f};
-    // all wavefronts are past their last LDS read (barrier at the end of the K loop)
+    // The saved pre-activations of this wavefront's part of the tile are requested here, all at once, so that the
+    // strips below find them in registers instead of waiting for a memory round trip per strip (columns in whole
+    // quads only: N % 4 == 0; rows and quads beyond the edge re-read the last valid ones and are not used).
+    constexpr int PASSES = 32 / ROWS_PER_PASS;
+    float4 zpre[TM][PASSES];
+    const bool zvec = dgelu && g.N % 4 == 0 && g.N >= 4;
+    if (zvec) {
+        const float *zb = g.aux_in + (int64_t)batch * g.c_bs + min(col, g.N - 4);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int pass = 0; pass < PASSES; ++pass) {
+                const int row = min(m0 + wm * (32 * TM) + 32 * i + prow + ROWS_PER_PASS * pass, g.M - 1);
+                zpre[i][pass] = *reinterpret_cast<const float4 *>(zb + (int64_t)row * ldc);
+            }
+    }
+    // All wavefronts are past their last LDS read (barrier at the end of the K loop), and a patch belongs to one
+    // wavefront: its lanes exchange values through it, which needs the LDS accesses kept in program order (they are
+    // executed in order per wavefront) but no workgroup barrier.
+    auto wave_sync = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
     // One 32-row strip of the wavefront's blocks at a time.  The strip index is a compile-time constant (a
     // lambda called once per value, not a loop): were the loop left rolled -- the body is long, and with
     // four strips the unroller declines -- the accumulators would be indexed at run time, live in scratch
@@ -708,7 +730,7 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) patch[(8 * (e >> 2) + 4 * h + (e & 3)) * PW + 32 * j + r] = acc[i][j][e];
-        __syncthreads();
+        wave_sync();
 #pragma unroll
         for (int pass = 0; pass < 32 / ROWS_PER_PASS; ++pass) {
             const int lr = prow + ROWS_PER_PASS * pass;
@@ -756,7 +778,9 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
                     // C = product * gelu'(z + bias), z the saved pre-activation laid out like C
                     const float *zp = g.aux_in + (int64_t)batch * g.c_bs + (int64_t)row * ldc + col;
                     float z[4] = {0.f, 0.f, 0.f, 0.f};
-                    if (col + 3 < g.N) {
+                    if (zvec) {
+                        z[0] = zpre[i][pass].x; z[1] = zpre[i][pass].y; z[2] = zpre[i][pass].z; z[3] = zpre[i][pass].w;
+                    } else if (col + 3 < g.N) {
                         const float4 z4 = *reinterpret_cast<const float4 *>(zp);
                         z[0] = z4.x; z[1] = z4.y; z[2] = z4.z; z[3] = z4.w;
                     } else {
@@ -795,12 +819,14 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
                 }
             }
         }
-        __syncthreads();
+        wave_sync();
     };
     epilogue_strip(std::integral_constant<int, 0>());
     if constexpr (TM > 1) epilogue_strip(std::integral_constant<int, 1>());
     if constexpr (TM > 2) epilogue_strip(std::integral_constant<int, 2>());
     if constexpr (TM > 3) epilogue_strip(std::integral_constant<int, 3>());
+    // (stream-K: the next segment's prologue writes LDS that other wavefronts' patches still occupy)
+    if (SK) __syncthreads();
     if (dgelu && g.colsum_part) {
         // lanes that share columns (same lane % LANES_PER_ROW) are added by butterfly steps; strip
         // (batch, tile row, wm) owns one row of the partial matrix
