@@ -130,6 +130,31 @@ def test_edge_tiles_in_padded_buffers(dev, m, n, k, lda, ldb, ta, tb):
         assert np.array_equal(r.to_host(dC, (m, n)), want), algo
 
 
+@pytest.mark.parametrize("ld", [4194300, 4194308])
+@pytest.mark.parametrize("ta", [False, True])
+def test_row_pitches_at_the_limit_of_32_bit_byte_offsets(dev, rocm, ld, ta):
+    """The steady K loop addresses a tile through 32-bit byte offsets from the tile's base (buffer loads); a
+    128-row tile side at a pitch of 2^22 floats is where they stop fitting.  Just below the limit the offsets
+    reach 2.13e9; just above it the tile takes the loop with 64-bit addresses (64-row tiles still fit).  A sits
+    in rows of `ld` floats (16 MiB apart), everything between the rows is never touched."""
+    m, n, k = 130, 70, 96
+    rows = k if ta else m            # stored rows of A
+    a = synth.small_ints(ld % 97, (rows, m if ta else k), 4)
+    b = synth.small_ints(5, (k, n), 4, stream=1)
+    dA = rocm.malloc(rows * ld * 4)
+    try:
+        for i in range(rows):
+            rocm._check(rocm.lib.mni_rocm_h2d(dA + i * ld * 4, a[i].ctypes.data, a[i].nbytes))
+        dB, dC = dev.put(b), dev.empty(m * n)
+        want = ((a.T if ta else a).astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+        for algo in (N.ALGO_MFMA, N.ALGO_MFMA_SMALL, N.ALGO_AUTO):
+            rocm.fill(dC, -7.0, m * n)
+            rocm.sgemm(m, n, k, dA, dB, dC, a_strides=(1, ld) if ta else (ld, 1), algo=algo)
+            assert np.array_equal(rocm.to_host(dC, (m, n)), want), algo
+    finally:
+        rocm.free(dA)
+
+
 @pytest.mark.parametrize("m,n,k", [(257, 259, 261), (1000, 1001, 515)])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 def test_odd_leading_dimensions_and_offset_bases(dev, m, n, k, ta, tb):
