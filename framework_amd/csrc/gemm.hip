@@ -177,18 +177,18 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
 // Which products go to the register-direct kernel by themselves: 0 = none,
 // else the number of wavefronts that share K.
 static int direct_plan(const GemmLaunch &g, int cus) {
-    // Four wavefronts per 64 x 64 tile, a quarter of K each: when about one such
-    // workgroup exists per CU (between half and five quarters of the CUs; with
-    // more, the tile kernel's larger tiles and resident rounds win, with fewer,
-    // K slices across workgroups) and K is long enough to be worth splitting but
-    // not so long that two 32-deep phases in flight per wavefront starve it.
-    // Measured on MI355X against the tile kernel's plans, microseconds:
-    // [32 x 512 x 512] x [512 x 64] 16.7 vs 22.7, its transposed twin 15.9 vs 22.8,
-    // K = 256: 11.6 vs 17.0, 32 x (128 x 128 x 512) 15.6 vs 27.0,
-    // 16 x (1024 x 64 x 1024) 27.2 vs 30.5; 64 batches of the first 31.2 vs 31.0,
-    // 128 batches 59 vs 44, 4 x (2048 x 64 x 2048) 43.9 vs 33.3.
-    const int64_t tiles = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) * g.batch;
-    if (tiles * 2 >= cus && tiles * 4 <= 5LL * cus && g.K >= 128 && (g.K <= 1024 || (tiles >= cus && g.K <= 4096))) return 4;
+    // None any more.  The kernel was built for batched products of about one
+    // 64 x 64 tile per CU (the backward products of an attention layer), where
+    // the tile kernel then spent its time waiting on loads.  Since the tile
+    // kernel's K loop carries no vector-ALU work, its 64 x 64 tiles in one K
+    // slice are ahead on every such shape (MI355X, microseconds, direct with
+    // four wavefronts sharing K against tile): [32 x 512 x 512] x [512 x 64] 16.4
+    // vs 13.7, its transposed twin 15.7 vs 13.7, K = 256: 11.5 vs 9.1, K = 1024:
+    // 27.4 vs 21.3, 32 x (128 x 128 x 512) 15.4 vs 13.0, 16 x (1024 x 64 x 1024)
+    // 27.2 vs 21.5, 40 batches of the first 29.6 vs 20.5.  MNI_ALGO_DIRECT
+    // still selects it.
+    (void)g;
+    (void)cus;
     return 0;
 }
 
@@ -333,15 +333,26 @@ static int run_mfma(const mni_gemm_desc &d) {
                 // 64 x 64 tiles would stream them twice as often (1024 x 1024 x 65536: 1127 us against
                 // 1015 us for 128 x 128 tiles in K slices, the plan below)
             } else {
-                streamk = streamk_fits(64, 64, 8);
-                if (streamk) bm = bn = 64;
+                const int64_t tiles64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) * g.batch;
+                if (tiles64 <= cus || (tiles64 <= 2LL * cus && ktiles <= 32)) {
+                    // At most one 64 x 64 tile per CU (or two, of a short K): one workgroup per tile and all of K
+                    // when at least half the CUs get one -- splitting K to fill the other workgroup slots costs a
+                    // reduction pass and gains nothing (32 x (512 x 64 x 512): 13.7 us whole, 19.0 in two K slices,
+                    // 19.8 stream-K; 40 batches, 1.25 tiles per CU: 20.6 whole, 27.5 stream-K) -- and K slices
+                    // below when fewer do (8 batches: 11.8 in two slices, 12.9 whole).
+                    bm = bn = 64;
+                    whole_tiles = tiles64 * 2 >= cus;
+                } else {
+                    streamk = streamk_fits(64, 64, 8);
+                    if (streamk) bm = bn = 64;
+                }
             }
         } else {
             // short K, a requested split, or no stream-K on this device: 64 x 64 when
             // 128 x 128 tiles would leave the machine with few, short-lived workgroups
-            const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
+            const int64_t t128 = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
             const int64_t big_split = d.split_k > 0 ? d.split_k : (ktiles / 8 > 0 ? ktiles / 8 : 1);
-            if (bm == 128 && bn == 128 && ((g.K <= 256 && t128 < 4LL * cus) || t128 * big_split < 2LL * cus)) bm = bn = 64;
+            if ((bm == 128 || bn == 128) && ((g.K <= 256 && t128 < 4LL * cus) || t128 * big_split < 2LL * cus)) bm = bn = 64;
         }
         if (d.algo == MNI_ALGO_MFMA_STREAMK && !streamk) {
             if (!sk_device) return set_error(MNI_ERR_INVALID, "sgemm: stream-K needs a confirmed workgroup-to-XCD mapping");

@@ -535,10 +535,10 @@ def test_panel_is_refused_for_shapes_it_cannot_take(dev, rocm):
         rocm.sgemm(64, 64, 64, dA, dB, dC, a_strides=(68, 1), b_strides=(1, 68), algo=N.ALGO_PANEL, split_k=2)
 
 
-def test_planner_sends_attention_shaped_products_to_the_new_kernels(dev, rocm):
-    # scores (short K, both operands K-contiguous) and the two backward products (one workgroup per CU,
-    # long thin operand) at a size where the planner picks the panel / direct kernels by itself; the
-    # results must be the forced kernels' bits
+def test_planner_choices_for_attention_shaped_products(dev, rocm):
+    # scores (short K, both operands K-contiguous) go to the panel kernel by themselves; the two backward
+    # products (about one 64 x 64 tile per CU, a long thin operand) to the tile kernel's 64 x 64 tiles in one K
+    # slice, one launch each; the results must be the forced plans' bits
     q = synth.normal(1, (16, 512, 64), 0.125)
     ds = synth.normal(2, (16, 512, 512), stream=1)
     dQ, dS = dev.put(q), dev.put(ds)
@@ -549,13 +549,24 @@ def test_planner_sends_attention_shaped_products_to_the_new_kernels(dev, rocm):
         outs.append(rocm.to_host(dC, (16, 512, 512)))
     assert np.array_equal(outs[0], outs[1])
     assert max_err(outs[0][3], q[3].astype(np.float64) @ q[3].T.astype(np.float64)) <= gemm_tol(64, q, q)
-    outs = []
-    for algo, split in ((N.ALGO_AUTO, 0), (N.ALGO_DIRECT, 4)):
+    outs, launches = [], []
+    for algo, split in ((N.ALGO_AUTO, 0), (N.ALGO_MFMA_SMALL, 1), (N.ALGO_DIRECT, 4)):
         dC = dev.empty(16 * 512 * 64)
+        before = rocm.launch_count()
         rocm.sgemm(512, 64, 512, dS, dQ, dC, batch=16, a_batch=(512 * 512, 16), b_batch=(512 * 64, 16), algo=algo, split_k=split)
+        launches.append(rocm.launch_count() - before)
         outs.append(rocm.to_host(dC, (16, 512, 64)))
+    assert np.array_equal(outs[0], outs[1]) and launches[0] == 1
+    for got in outs:
+        assert max_err(got[5], ds[5].astype(np.float64) @ q[5].astype(np.float64)) <= gemm_tol(512, ds, q)
+    # its transposed twin, dK^T = Q^T dS
+    outs = []
+    for algo, split in ((N.ALGO_AUTO, 0), (N.ALGO_MFMA_SMALL, 1)):
+        dC = dev.empty(16 * 64 * 512)
+        rocm.sgemm(64, 512, 512, dQ, dS, dC, batch=16, a_strides=(1, 64), a_batch=(512 * 64, 16), b_batch=(512 * 512, 16), algo=algo, split_k=split)
+        outs.append(rocm.to_host(dC, (16, 64, 512)))
     assert np.array_equal(outs[0], outs[1])
-    assert max_err(outs[0][5], ds[5].astype(np.float64) @ q[5].astype(np.float64)) <= gemm_tol(512, ds, q)
+    assert max_err(outs[0][7], q[7].T.astype(np.float64) @ ds[7].astype(np.float64)) <= gemm_tol(512, q, ds)
 
 
 def test_single_launch_skinny_path_is_available(rocm):
