@@ -168,7 +168,8 @@ def bench_yardsticks(r):
         r.free(b)
     # What the matrix pipe gives a loop of nothing but fp32 MFMAs (two wavefronts per SIMD, as the tile kernel has),
     # and with one or two register moves behind every MFMA: the vector ALU's issue time comes out of the MFMAs'.
-    tf = [r.mfma_yardstick(v) for v in (0, 1, 2)]
+    r.mfma_yardstick(0, warmup=20, iters=1)  # ~40 ms of nothing but MFMAs first: the clocks take that long to settle
+    tf = [r.mfma_yardstick(v, warmup=3, iters=10) for v in (0, 1, 2)]
     out["mfma_yardstick"] = {"TFLOP/s": tf[0], "frac_mfma": tf[0] / PEAK_FP32_MATRIX_TFLOPS,
                              "with_1_v_mov_per_mfma": tf[1], "with_2_v_mov_per_mfma": tf[2],
                              "note": "v_mfma_f32_32x32x2_f32 on four independent accumulators per wavefront, nothing else in the loop"}
@@ -241,9 +242,9 @@ def bench_extras(r, with_cpu):
     by = 4.0 * 32 * (512 * 64 * 2 + 512 * 512)
     prods = [("scores", "gemm_panel_kernel<8>", r.gemm_desc(512, 512, 64, dq, dk, s_out, batch=32, a_batch=(512 * 64, 32),
                                                              b_strides=(1, 64), b_batch=(512 * 64, 32))),
-             ("dQ", "gemm_direct_kernel<0, 1, 4, 4>", r.gemm_desc(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32),
+             ("dQ", "gemm_mfma_kernel<0, 1, 1, 1, false>", r.gemm_desc(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32),
                                                                   b_batch=(512 * 64, 32))),
-             ("dKT", "gemm_direct_kernel<1, 1, 4, 4>", r.gemm_desc(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64),
+             ("dKT", "gemm_mfma_kernel<1, 1, 1, 1, false>", r.gemm_desc(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64),
                                                                    a_batch=(512 * 64, 32), b_batch=(512 * 512, 32)))]
     c3 = {}
     total = 0.0
