@@ -99,6 +99,8 @@ int check_launch(const char *what);  // hipGetLastError after a kernel launch
 
 // gemm.hip
 int sgemm(const mni_gemm_desc &d);
+// Two independent products, in one launch where the paired tile kernel takes them (gemm.hip).
+int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1);
 
 // elementwise.hip: internal launchers (device pointers, element strides)
 struct StridedDesc {

@@ -349,14 +349,21 @@ static int make_operand(const Tensor &t, bool transpose, mni_operand *op, BufP *
 // ta / tb: use the operand with its last two dims swapped (transpose_last2,
 // ops/matmul.rs:258-284, without the copy).
 // aux / colsum_part: the second buffer and the strip sums of the MNI_EPI_BIAS_GELU_DUAL / MNI_EPI_DGELU epilogues.
-static uint32_t matmul_tensors(uint32_t a, bool ta, uint32_t b, bool tb, const float *bias, int epilogue, float *aux = nullptr,
-                               float *colsum_part = nullptr) {
+struct PreparedMatmul {
+    mni_gemm_desc d;
+    BufP out, keep_a, keep_b;  // the result buffer; contiguous copies the operands needed, alive until the launch is issued
+    Shape out_shape;
+};
+
+// Everything of a product but the launch: checks, broadcast of the batch dims, operand descriptors, result buffer.
+static bool prepare_matmul(uint32_t a, bool ta, uint32_t b, bool tb, const float *bias, int epilogue, float *aux, float *colsum_part,
+                           PreparedMatmul *pm) {
     Tensor *A = get(a), *B = get(b);
-    if (!A || !B) return MNI_BAD_ID;
+    if (!A || !B) return false;
     const int and_ = (int)A->shape.size(), bnd = (int)B->shape.size();
     if (and_ < 2 || bnd < 2) {
         set_error(MNI_ERR_INVALID, "matmul requires at least 2D tensors");
-        return MNI_BAD_ID;
+        return false;
     }
     int64_t m = A->shape[and_ - 2], k = A->shape[and_ - 1];
     if (ta) std::swap(m, k);
@@ -364,34 +371,40 @@ static uint32_t matmul_tensors(uint32_t a, bool ta, uint32_t b, bool tb, const f
     if (tb) std::swap(k2, n);
     if (k != k2) {
         set_error(MNI_ERR_INVALID, "matmul inner dimensions must match: %lld vs %lld", (long long)k, (long long)k2);
-        return MNI_BAD_ID;
+        return false;
     }
     const Shape a_batch(A->shape.begin(), A->shape.end() - 2), b_batch(B->shape.begin(), B->shape.end() - 2);
-    Shape out_shape;
+    Shape &out_shape = pm->out_shape;
     if (!broadcast_shape(a_batch, b_batch, &out_shape)) {
         set_error(MNI_ERR_INVALID, "matmul batch shapes are not broadcastable");
-        return MNI_BAD_ID;
+        return false;
     }
     if (out_shape.size() + 2 > MNI_MAX_DIMS) {
         set_error(MNI_ERR_INVALID, "matmul result rank exceeds %d", MNI_MAX_DIMS);
-        return MNI_BAD_ID;
+        return false;
     }
     const int64_t batch = shape_size(out_shape);
     out_shape.push_back(m);
     out_shape.push_back(n);
 
-    mni_gemm_desc d;
+    mni_gemm_desc &d = pm->d;
     memset(&d, 0, sizeof d);
-    BufP keep_a, keep_b;
-    if (make_operand(*A, ta, &d.A, &keep_a) != MNI_OK || make_operand(*B, tb, &d.B, &keep_b) != MNI_OK) return MNI_BAD_ID;
-    BufP out = new_buf((size_t)shape_size(out_shape));
-    if (!out) return MNI_BAD_ID;
+    if (make_operand(*A, ta, &d.A, &pm->keep_a) != MNI_OK || make_operand(*B, tb, &d.B, &pm->keep_b) != MNI_OK) return false;
+    pm->out = new_buf((size_t)shape_size(out_shape));
+    if (!pm->out) return false;
     d.M = m; d.N = n; d.K = k; d.batch = batch;
-    d.C = out->p; d.ldc = n; d.c_batch_stride = m * n;
+    d.C = pm->out->p; d.ldc = n; d.c_batch_stride = m * n;
     d.bias = bias; d.epilogue = epilogue;
     d.aux = aux; d.colsum_part = colsum_part;
-    if (sgemm(d) != MNI_OK) return MNI_BAD_ID;
-    return insert_contig(std::move(out), out_shape);
+    return true;
+}
+
+static uint32_t matmul_tensors(uint32_t a, bool ta, uint32_t b, bool tb, const float *bias, int epilogue, float *aux = nullptr,
+                               float *colsum_part = nullptr) {
+    PreparedMatmul pm;
+    if (!prepare_matmul(a, ta, b, tb, bias, epilogue, aux, colsum_part, &pm)) return MNI_BAD_ID;
+    if (sgemm(pm.d) != MNI_OK) return MNI_BAD_ID;
+    return insert_contig(std::move(pm.out), pm.out_shape);
 }
 
 // Sum `full` (contiguous, full_shape) down to `orig_shape`
@@ -438,55 +451,62 @@ static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out, const Th
     if (!A || !B || !G) return MNI_ERR_FREED;
     const Shape a_shape = A->shape, b_shape = B->shape;
 
-    // dA
+    // The two products are independent of each other, so both are set up first and issued together
+    // (mni_rocm_sgemm_pair's rule decides whether that is one launch or two).
+    // dA = dC * B^T
+    PreparedMatmul pa;
+    if (!(through_gelu ? prepare_matmul(grad, false, b, true, through_gelu->bias, MNI_EPI_DGELU, through_gelu->z, through_gelu->colsum_part, &pa)
+                       : prepare_matmul(grad, false, b, true, nullptr, MNI_EPI_NONE, nullptr, nullptr, &pa)))
+        return MNI_ERR_INVALID;
+    // dB = A^T * dC.  When B has no batch of its own and A / dC stack their batch
+    // matrices at a uniform row pitch, sum over the batch inside one product
+    // by extending K to batch * M (the split-K path then fills the machine).
+    PreparedMatmul pb;
+    A = get(a); B = get(b); G = get(grad);
+    const int and_ = (int)A->shape.size(), gnd = (int)G->shape.size();
+    int64_t b_bcount = 1;
+    for (size_t i = 0; i + 2 < b_shape.size(); ++i) b_bcount *= b_shape[i];
+    int64_t g_batch = 1;
+    for (int i = 0; i < gnd - 2; ++i) g_batch *= G->shape[i];
+    bool folded = false;
+    if (b_bcount == 1 && g_batch > 1 && is_contiguous(*A) && is_contiguous(*G)) {
+        int64_t a_batch = 1;
+        for (int i = 0; i < and_ - 2; ++i) a_batch *= A->shape[i];
+        if (a_batch == g_batch) {
+            const int64_t m = A->shape[and_ - 2], k = A->shape[and_ - 1], n = G->shape[gnd - 1];
+            mni_gemm_desc &d = pb.d;
+            memset(&d, 0, sizeof d);
+            pb.out = new_buf((size_t)(k * n));
+            if (!pb.out) return MNI_ERR_NOMEM;
+            d.M = k; d.N = n; d.K = g_batch * m; d.batch = 1;
+            d.A.ptr = A->buf->p; d.A.row_stride = 1; d.A.col_stride = k; d.A.batch_count = 1;
+            d.B.ptr = G->buf->p; d.B.row_stride = n; d.B.col_stride = 1; d.B.batch_count = 1;
+            d.C = pb.out->p; d.ldc = n; d.c_batch_stride = k * n;
+            pb.out_shape = {k, n};
+            folded = true;
+        }
+    }
+    if (!folded && !prepare_matmul(a, true, grad, false, nullptr, MNI_EPI_NONE, nullptr, nullptr, &pb)) return MNI_ERR_INVALID;
+    MNI_TRY(sgemm_pair(pa.d, pb.d));
+
     {
-        const uint32_t full = through_gelu ? matmul_tensors(grad, false, b, true, through_gelu->bias, MNI_EPI_DGELU, through_gelu->z,
-                                                            through_gelu->colsum_part)
-                                           : matmul_tensors(grad, false, b, true, nullptr, MNI_EPI_NONE);
+        const uint32_t full = insert_contig(std::move(pa.out), pa.out_shape);
         if (full == MNI_BAD_ID) return MNI_ERR_INVALID;
         const uint32_t ga = unbroadcast_tensor(full, a_shape);
         free_tensor(full);
         if (ga == MNI_BAD_ID) return MNI_ERR_INVALID;
         out[0] = ga;
     }
-    // dB.  When B has no batch of its own and A / dC stack their batch
-    // matrices at a uniform row pitch, sum over the batch inside one product
-    // by extending K to batch * M (the split-K path then fills the machine).
     {
-        A = get(a); B = get(b); G = get(grad);
-        const int and_ = (int)A->shape.size(), gnd = (int)G->shape.size();
-        int64_t b_bcount = 1;
-        for (size_t i = 0; i + 2 < b_shape.size(); ++i) b_bcount *= b_shape[i];
-        int64_t g_batch = 1;
-        for (int i = 0; i < gnd - 2; ++i) g_batch *= G->shape[i];
-        bool folded = false;
-        if (b_bcount == 1 && g_batch > 1 && is_contiguous(*A) && is_contiguous(*G)) {
-            int64_t a_batch = 1;
-            for (int i = 0; i < and_ - 2; ++i) a_batch *= A->shape[i];
-            if (a_batch == g_batch) {
-                const int64_t m = A->shape[and_ - 2], k = A->shape[and_ - 1], n = G->shape[gnd - 1];
-                mni_gemm_desc d;
-                memset(&d, 0, sizeof d);
-                BufP outb = new_buf((size_t)(k * n));
-                if (!outb) return MNI_ERR_NOMEM;
-                d.M = k; d.N = n; d.K = g_batch * m; d.batch = 1;
-                d.A.ptr = A->buf->p; d.A.row_stride = 1; d.A.col_stride = k; d.A.batch_count = 1;
-                d.B.ptr = G->buf->p; d.B.row_stride = n; d.B.col_stride = 1; d.B.batch_count = 1;
-                d.C = outb->p; d.ldc = n; d.c_batch_stride = k * n;
-                MNI_TRY(sgemm(d));
-                Shape kn = {k, n};
-                const uint32_t full = insert_contig(std::move(outb), kn);
-                // b_shape may carry leading ones ([1, K, N]); same element count.
-                Tensor *F = get(full);
-                F->shape = b_shape;
-                F->strides = compute_strides(b_shape);
-                out[1] = full;
-                folded = true;
-            }
-        }
-        if (!folded) {
-            const uint32_t full = matmul_tensors(a, true, grad, false, nullptr, MNI_EPI_NONE);
-            if (full == MNI_BAD_ID) return MNI_ERR_INVALID;
+        const uint32_t full = insert_contig(std::move(pb.out), pb.out_shape);
+        if (full == MNI_BAD_ID) return MNI_ERR_INVALID;
+        if (folded) {
+            // b_shape may carry leading ones ([1, K, N]); same element count.
+            Tensor *F = get(full);
+            F->shape = b_shape;
+            F->strides = compute_strides(b_shape);
+            out[1] = full;
+        } else {
             const uint32_t gb = unbroadcast_tensor(full, b_shape);
             free_tensor(full);
             if (gb == MNI_BAD_ID) return MNI_ERR_INVALID;

@@ -46,6 +46,9 @@ struct GemmLaunch {
 
 // tile_m, tile_n in {128, 64}; g.tiles_m / g.tiles_n count tiles of that size
 int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int tile_n);
+// Two independent products of 64 x 64 tiles (one workgroup per tile, all of K) in one launch; amode0 must be 0 and bmode1 1.
+bool gemm_mfma_pair_eligible(int amode0, int bmode0, int amode1, int bmode1);
+int launch_gemm_mfma_pair(const GemmLaunch &g0, int amode0, int bmode0, const GemmLaunch &g1, int amode1, int bmode1);
 // workgroups that stay resident per CU for a tile shape (what the stream-K grid is sized by)
 int gemm_mfma_resident_per_cu(int tile_m, int tile_n);
 int gemm_mfma_tile_k();

@@ -297,23 +297,26 @@ __device__ __forceinline__ float pick(const float4 &v, int j) { return j == 0 ? 
 // short-K products where smaller tiles waste less and fill the machine better.
 // SK: the stream-K form (a loop over this workgroup's segments); otherwise the
 // body runs once for the (tile, batch, slice) named by the workgroup id.
+typedef const GemmLaunch __attribute__((address_space(4))) *LaunchPtr;
+
+// float4 slots of LDS a workgroup needs: two stages of the A tile, two of the B tile; the epilogue reuses the
+// block to turn the MFMA accumulator layout into row-contiguous 16-byte stores.
+template <int AMODE, int BMODE, int TM, int TN>
+__device__ constexpr int gemm_lds_slots() {
+    return 2 * stage_slots<AMODE == 1 ? 1 : 0, 64 * TM>() + 2 * stage_slots<BMODE == 1 ? 1 : 0, 64 * TN>();
+}
+
+// The work of one workgroup.  gp: the launch descriptor in the kernel-argument segment (read through scalar
+// loads, afresh for every stream-K segment, instead of being held in scalar registers across the K loop);
+// wg / nwg: this workgroup's number and the number of workgroups of this product, numbered the way the
+// hardware deals workgroups to XCDs (wg % 8 is the XCD); lds: gemm_lds_slots() float4.
 template <int AMODE, int BMODE, int TM, int TN, bool SK>
-__global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_kernel(const GemmLaunch launch_args) {
-    // The launch descriptor is read through the kernel-argument segment, so
-    // that the stream-K form can read it afresh for every segment (scalar
-    // loads) instead of holding all of it in scalar registers across the loop.
-    (void)launch_args;
-    typedef const GemmLaunch __attribute__((address_space(4))) *LaunchPtr;
-    LaunchPtr gp = (LaunchPtr)__builtin_amdgcn_kernarg_segment_ptr();
+__device__ __forceinline__ void gemm_mfma_body(LaunchPtr gp, const unsigned wg, const unsigned nwg, float4 *__restrict__ lds) {
 #define g (*gp)
     constexpr int AL = AMODE == 1 ? 1 : 0;
     constexpr int BL = BMODE == 1 ? 1 : 0;
     constexpr int BM = 64 * TM, BN = 64 * TN;
-    // One LDS block: two stages of the A tile, two of the B tile; the epilogue
-    // reuses it to turn the MFMA accumulator layout into row-contiguous 16-byte
-    // stores.
     constexpr int STAGE_A = stage_slots<AL, BM>(), STAGE_B = stage_slots<BL, BN>();
-    __shared__ float4 lds[2 * STAGE_A + 2 * STAGE_B];
     auto stage_a = [&](int st) -> float4 * { return lds + st * STAGE_A; };
     auto stage_b = [&](int st) -> float4 * { return lds + 2 * STAGE_A + st * STAGE_B; };
 
@@ -349,7 +352,7 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
         return sh;
     };
     if (SK) {
-        const Share sh = share_of(blockIdx.x);
+        const Share sh = share_of(wg);
         seg_hi = sh.hi;
         dp_tile = sh.dp0;
         if (seg_hi <= sh.lo && dp_tile >= sh.tiles) return;
@@ -360,7 +363,7 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     // segment (the empty asm hides that it never changes): hoisted out of the
     // segment loop, those addresses would stay live across it and spill.
     int tid = threadIdx.x;
-    unsigned bid = blockIdx.x;
+    unsigned bid = wg;
     if (SK) {
         asm volatile("" : "+v"(tid));
         asm volatile("" : "+s"(gp));
@@ -385,8 +388,8 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     if (!SK) {
         // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
         // Renumber so that every XCD works on one contiguous run of tiles.
-        pid = blockIdx.x;
-        const int64_t total = gridDim.x;
+        pid = wg;
+        const int64_t total = nwg;
         const int64_t q = total >> 3, rr = total & 7;
         const int64_t x = pid & 7, i = pid >> 3;
         pid = (x < rr ? x * (q + 1) : rr * (q + 1) + (x - rr) * q) + i;
@@ -851,6 +854,38 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
 #undef g
 }
 
+template <int AMODE, int BMODE, int TM, int TN, bool SK>
+__global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_kernel(const GemmLaunch launch_args) {
+    (void)launch_args;
+    __shared__ float4 lds[gemm_lds_slots<AMODE, BMODE, TM, TN>()];
+    gemm_mfma_body<AMODE, BMODE, TM, TN, SK>((LaunchPtr)__builtin_amdgcn_kernarg_segment_ptr(), blockIdx.x, gridDim.x, lds);
+}
+
+// Two independent products of 64 x 64 tiles in one launch: workgroups [0, wgs0) work on the first (wgs0 = its tile
+// count rounded up to a multiple of 8, so that the second product's numbering starts on XCD 0 as well; the
+// padding workgroups leave at once), the rest on the second.  For the two backward products of a batched matmul
+// (src/native/src/ops/matmul.rs:199-222) when each of them alone is about one tile per CU: together they give
+// every SIMD two wavefronts, and they share one launch, one ramp-up and one tail.
+struct GemmPairLaunch {
+    GemmLaunch g[2];
+    unsigned wgs0, tiles0, tiles1;
+};
+
+template <int AM0, int BM0, int AM1, int BM1>
+__global__ __launch_bounds__(NTHREADS, 4) void gemm_mfma_pair_kernel(const GemmPairLaunch pair_args) {
+    (void)pair_args;
+    typedef const GemmPairLaunch __attribute__((address_space(4))) *PairPtr;
+    PairPtr pp = (PairPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    constexpr int S0 = gemm_lds_slots<AM0, BM0, 1, 1>(), S1 = gemm_lds_slots<AM1, BM1, 1, 1>();
+    __shared__ float4 lds[S0 > S1 ? S0 : S1];
+    const unsigned wg = blockIdx.x;
+    if (wg < pp->wgs0) {
+        if (wg < pp->tiles0) gemm_mfma_body<AM0, BM0, 1, 1, false>(&pp->g[0], wg, pp->tiles0, lds);
+    } else {
+        gemm_mfma_body<AM1, BM1, 1, 1, false>(&pp->g[1], wg - pp->wgs0, pp->tiles1, lds);
+    }
+}
+
 template <int TM, int TN>
 static void launch_modes(const GemmLaunch &g, int amode, int bmode, dim3 grid) {
     dim3 block(NTHREADS);
@@ -885,6 +920,35 @@ int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int 
     else if (tile_m == 64 && tile_n == 64) launch_modes<1, 1>(g, amode, bmode, grid);
     else return set_error(MNI_ERR_INVALID, "sgemm: unsupported tile %d x %d", tile_m, tile_n);
     return check_launch("gemm_mfma_kernel");
+}
+
+// The product pairs a matmul backward gives rise to: product 0 has dC (row-major) as its A, product 1 has dC as
+// its B; 64 x 64 tiles (g.tiles_m / g.tiles_n count those), one workgroup per tile, all of K.
+bool gemm_mfma_pair_eligible(int amode0, int bmode0, int amode1, int bmode1) {
+    return amode0 == 0 && bmode0 <= 1 && amode1 <= 1 && bmode1 == 1;
+}
+
+int launch_gemm_mfma_pair(const GemmLaunch &g0, int amode0, int bmode0, const GemmLaunch &g1, int amode1, int bmode1) {
+    if (!gemm_mfma_pair_eligible(amode0, bmode0, amode1, bmode1))
+        return set_error(MNI_ERR_INVALID, "sgemm: product pair not eligible for the paired tile kernel");
+    const int64_t t0 = (int64_t)g0.tiles_m * g0.tiles_n * g0.batch, t1 = (int64_t)g1.tiles_m * g1.tiles_n * g1.batch;
+    if (g0.tiles_m != (g0.M + 63) / 64 || g0.tiles_n != (g0.N + 63) / 64 || g1.tiles_m != (g1.M + 63) / 64 ||
+        g1.tiles_n != (g1.N + 63) / 64 || t0 <= 0 || t1 <= 0 || t0 + t1 + 8 > 0x7fffffffLL || g0.split_k != 1 || g1.split_k != 1 ||
+        g0.streamk || g1.streamk)
+        return set_error(MNI_ERR_INVALID, "sgemm: paired tile kernel launched with a wrong plan");
+    GemmPairLaunch p;
+    p.g[0] = g0;
+    p.g[1] = g1;
+    p.tiles0 = (unsigned)t0;
+    p.tiles1 = (unsigned)t1;
+    p.wgs0 = (unsigned)((t0 + 7) / 8 * 8);
+    const dim3 grid(p.wgs0 + p.tiles1), block(NTHREADS);
+    hipStream_t s = ctx().stream;
+    if (bmode0 == 0 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 0, 1>), grid, block, 0, s, p);
+    else if (bmode0 == 0 && amode1 == 1) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 1, 1>), grid, block, 0, s, p);
+    else if (bmode0 == 1 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 0, 1>), grid, block, 0, s, p);
+    else MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 1, 1>), grid, block, 0, s, p);
+    return check_launch("gemm_mfma_pair_kernel");
 }
 
 int gemm_mfma_tile_k() { return BK; }

@@ -71,6 +71,8 @@ SIGNATURES = {
     "mni_rocm_sgemm_noalloc": (C.c_int, [C.POINTER(GemmDesc)]),
     "mni_rocm_sgemm_noalloc_workspace_bytes": (C.c_size_t, []),
     "mni_rocm_sgemm_timed": (C.c_int, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
+    "mni_rocm_sgemm_pair_timed": (C.c_int, [C.POINTER(GemmDesc), C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
+    "mni_rocm_sgemm_pair": (C.c_int, [C.POINTER(GemmDesc), C.POINTER(GemmDesc)]),
     "mni_rocm_yardstick_timed": (C.c_int, [C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_void_p), C.c_int, C.c_size_t, C.c_int, C.c_int,
                                            C.c_int, C.POINTER(C.c_float)]),
     "mni_rocm_mfma_yardstick_timed": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]),
@@ -271,6 +273,17 @@ class Rocm:
         arr = (GemmDesc * len(descs))(*descs)
         ms = C.c_float(0)
         self._check(self.lib.mni_rocm_sgemm_timed(arr, len(descs), warmup, iters, C.byref(ms)))
+        return ms.value
+
+    def sgemm_pair(self, first, second):
+        """Two independent products (descriptors made by gemm_desc), in one launch where the library pairs them."""
+        self._check(self.lib.mni_rocm_sgemm_pair(C.byref(first), C.byref(second)))
+
+    def sgemm_pair_timed(self, descs, warmup, iters):
+        """Average ms per pair: descs holds pairs (0 with 1, 2 with 3, ...), cycled back to back and issued from C."""
+        arr = (GemmDesc * len(descs))(*descs)
+        ms = C.c_float(0)
+        self._check(self.lib.mni_rocm_sgemm_pair_timed(arr, len(descs), warmup, iters, C.byref(ms)))
         return ms.value
 
     @staticmethod

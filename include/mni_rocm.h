@@ -172,12 +172,25 @@ int64_t mni_rocm_sgemm_colsum_rows(int64_t M, int64_t batch);
  * device memory would.  Nothing in it needs to start at zero. */
 int mni_rocm_sgemm_noalloc(const mni_gemm_desc *desc);
 size_t mni_rocm_sgemm_noalloc_workspace_bytes(void);
+/* Two products that do not depend on each other: neither reads what the other
+ * writes and their outputs do not overlap.  Replaces the two gemm calls of
+ * matmul_backward (src/native/src/ops/matmul.rs:199-222: dA = dC * B^T and
+ * dB = A^T * dC), which the reference issues one after the other.  When each
+ * product alone is a batch of about one 64 x 64 tile per compute unit, both
+ * run in one launch (every SIMD gets a second wavefront; one ramp-up, one
+ * tail); otherwise this is mni_rocm_sgemm(first) followed by
+ * mni_rocm_sgemm(second).  The results are those of the separate calls bit
+ * for bit. */
+int mni_rocm_sgemm_pair(const mni_gemm_desc *first, const mni_gemm_desc *second);
 /* Measurement aid (no counterpart in the reference): runs descs[0], descs[1],
  * ... descs[count-1], descs[0], ... back to back on the library's stream,
  * `warmup` untimed launches and then `iters` launches between two HIP events,
  * and returns the average milliseconds per launch.  Issuing from C keeps the
  * host ahead of kernels that take only a few microseconds. */
 int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms);
+/* The same for mni_rocm_sgemm_pair: descs holds count / 2 pairs (descs[0] with
+ * descs[1], descs[2] with descs[3], ...); the average is per pair. */
+int mni_rocm_sgemm_pair_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms);
 
 /* Measurement aid (no counterpart in the reference): what the device gives a
  * kernel that only streams.  `iters` launches between two HIP events on the

@@ -569,6 +569,76 @@ def test_planner_choices_for_attention_shaped_products(dev, rocm):
     assert max_err(outs[0][7], q[7].T.astype(np.float64) @ ds[7].astype(np.float64)) <= gemm_tol(512, q, ds)
 
 
+# ---- two independent products in one launch (the backward pair of a batched matmul) ----------------
+
+def _pair_descs(rocm, dev, batch, t, d, kview, ds, q, k):
+    """dQ = dS K and dK^T = Q^T dS for S = Q K^T; kview: K^T given as a permuted view (the forward's B
+    operand), so dQ's B is K row-major; else the forward's B is K^T stored [d, t] and dQ's B is its transpose."""
+    dDS, dQm, dKm = dev.put(ds), dev.put(q), dev.put(k)
+    o0, o1 = dev.empty(batch * t * d), dev.empty(batch * t * d)
+    if kview:
+        d0 = rocm.gemm_desc(t, d, t, dDS, dKm, o0, batch=batch, a_batch=(t * t, batch), b_batch=(t * d, batch))
+        d1 = rocm.gemm_desc(d, t, t, dQm, dDS, o1, batch=batch, a_strides=(1, d), a_batch=(t * d, batch), b_batch=(t * t, batch))
+    else:
+        d0 = rocm.gemm_desc(t, d, t, dDS, dKm, o0, batch=batch, a_batch=(t * t, batch), b_strides=(1, t), b_batch=(t * d, batch))
+        d1 = rocm.gemm_desc(d, t, t, dQm, dDS, o1, batch=batch, a_batch=(t * d, batch), b_batch=(t * t, batch))
+    return d0, d1, o0, o1
+
+
+@pytest.mark.parametrize("batch,t,d,kview", [(16, 512, 64, True), (16, 512, 64, False), (32, 256, 128, True), (20, 500, 62, True),
+                                             (64, 512, 64, True)])
+def test_pair_launch_gives_the_bits_of_separate_launches(dev, rocm, batch, t, d, kview):
+    # sizes at which each product alone is planned as 64 x 64 tiles, one workgroup per tile, so the pair goes out as
+    # one launch (the fourth with edges inside tiles and a K tail; the last with two tiles per CU each); integer
+    # inputs pin the values, normal inputs the order of the K sum
+    for make in (lambda s, shape, st: synth.small_ints(s, shape, 3, stream=st), lambda s, shape, st: synth.normal(s, shape, stream=st)):
+        ds = make(1, (batch, t, t), 0)
+        q = make(2, (batch, t, d) if kview else (batch, d, t), 1)
+        k = make(3, (batch, t, d) if kview else (batch, d, t), 2)
+        d0, d1, o0, o1 = _pair_descs(rocm, dev, batch, t, d, kview, ds, q, k)
+        before = rocm.launch_count()
+        rocm.sgemm_pair(d0, d1)
+        launches = rocm.launch_count() - before
+        got0, got1 = rocm.to_host(o0, (batch, t, d)), rocm.to_host(o1, (batch, d, t))
+        rocm.fill(o0, -1.0, batch * t * d)
+        rocm.fill(o1, -1.0, batch * t * d)
+        rocm._check(rocm.lib.mni_rocm_sgemm(d0))
+        rocm._check(rocm.lib.mni_rocm_sgemm(d1))
+        assert np.array_equal(got0, rocm.to_host(o0, (batch, t, d)))
+        assert np.array_equal(got1, rocm.to_host(o1, (batch, d, t)))
+        assert launches == 1
+        if np.all(ds == np.round(ds)):
+            K = k if kview else k.transpose(0, 2, 1)
+            Q = q if kview else q.transpose(0, 2, 1)
+            assert np.array_equal(got0, np.einsum("bij,bjd->bid", ds.astype(np.int64), K.astype(np.int64)).astype(np.float32))
+            assert np.array_equal(got1, np.einsum("bid,bij->bdj", Q.astype(np.int64), ds.astype(np.int64)).astype(np.float32))
+
+
+def test_pair_launch_of_small_and_of_big_products(dev, rocm, oracle_native):
+    # a pair of small products (a few tiles each) may share a launch too; either way the values are right
+    a = synth.normal(1, (96, 200))
+    b = synth.normal(2, (200, 72), stream=1)
+    g = synth.normal(3, (96, 72), stream=2)
+    dA, dB, dG = dev.put(a), dev.put(b), dev.put(g)
+    oa, ob = dev.empty(96 * 200), dev.empty(200 * 72)
+    d0 = rocm.gemm_desc(96, 200, 72, dG, dB, oa, b_strides=(1, 72))
+    d1 = rocm.gemm_desc(200, 72, 96, dA, dG, ob, a_strides=(1, 200))
+    rocm.sgemm_pair(d0, d1)
+    assert max_err(rocm.to_host(oa, (96, 200)), oracle_native.sgemm_ikj(g, b.T.copy())) <= gemm_tol(72, g, b)
+    assert max_err(rocm.to_host(ob, (200, 72)), oracle_native.sgemm_ikj(a.T.copy(), g)) <= gemm_tol(96, a, g)
+    with pytest.raises(N.MniError, match="null descriptor"):
+        rocm._check(rocm.lib.mni_rocm_sgemm_pair(None, None))
+    # a big pair: each product fills the machine by itself and is launched by itself
+    n = 2048
+    big = synth.normal(4, (n, n))
+    dBig, o2, o3 = dev.put(big), dev.empty(n * n), dev.empty(n * n)
+    before = rocm.launch_count()
+    rocm.sgemm_pair(rocm.gemm_desc(n, n, n, dBig, dBig, o2, b_strides=(1, n)), rocm.gemm_desc(n, n, n, dBig, dBig, o3, a_strides=(1, n)))
+    assert rocm.launch_count() - before >= 2
+    assert max_err(rocm.to_host(o2, (n, n)), big.astype(np.float64) @ big.T.astype(np.float64)) <= gemm_tol(n, big, big)
+    assert max_err(rocm.to_host(o3, (n, n)), big.T.astype(np.float64) @ big.astype(np.float64)) <= gemm_tol(n, big, big)
+
+
 def test_single_launch_skinny_path_is_available(rocm):
     # MI355X deals workgroups over its 8 XCDs round-robin; were the probe to fail,
     # ALGO_SKINNY would quietly run as ALGO_SKINNY_TWO_PASS and the tests below
