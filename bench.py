@@ -247,16 +247,23 @@ def bench_extras(r, with_cpu):
              ("dKT", "gemm_mfma_kernel<1, 1, 1, 1, false>", r.gemm_desc(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64),
                                                                    a_batch=(512 * 64, 32), b_batch=(512 * 512, 32)))]
     c3 = {}
-    total = 0.0
+    each = {}
     for name, kern, desc in prods:
-        ms = r.sgemm_timed([desc], 10, 200)
-        total += ms
+        each[name] = r.sgemm_timed([desc], 10, 200)
         # each product moves 41.9 MB and 1.07 GFLOP: the matrix pipe needs 6.8 us for it, HBM 5.2 us
-        c3[name] = roofline("mfma", kern, ms * 1e-3, fl, by)
-    c3["roofline"] = dict(roofline("mfma", "the three products", total * 1e-3, 3 * fl, 3 * by),
+        c3[name] = roofline("mfma", kern, each[name] * 1e-3, fl, by)
+    # the two gradients as the engine's matmul backward issues them: one paired launch (mni_rocm_sgemm_pair)
+    g_out2 = r.malloc(32 * 512 * 64 * 4)
+    pair = [prods[1][2], r.gemm_desc(64, 512, 512, dq, dds, g_out2, batch=32, a_strides=(1, 64), a_batch=(512 * 64, 32), b_batch=(512 * 512, 32))]
+    ms_pair = r.sgemm_pair_timed(pair, 10, 200)
+    c3["dQ_and_dKT_paired"] = dict(roofline("mfma", "gemm_mfma_pair_kernel<0, 1, 1, 1>", ms_pair * 1e-3, 2 * fl, 2 * by),
+                                   note="both gradients in one launch; one after the other they take %.1f us" % ((each["dQ"] + each["dKT"]) * 1e3))
+    total = each["scores"] + ms_pair
+    c3["roofline"] = dict(roofline("mfma", "the three products (scores, then both gradients in one launch)", total * 1e-3, 3 * fl, 3 * by),
                           note="arithmetic intensity 25.6 flop/B against a ridge of 19.7: the matrix pipe bounds it (20.5 us for all "
                                "three), HBM is close behind (15.7 us); an empty launch in the same sequence takes "
-                               "%.2f us" % out["empty_launch_us"])
+                               "%.2f us; three separate launches take %.1f us" % (out["empty_launch_us"], sum(each.values()) * 1e3))
+    r.free(g_out2)
     if with_cpu:
         nb = 2  # batches of the 32
         orc = oracle_api()
@@ -453,7 +460,7 @@ def run_for_counters(r, which):
             r.sgemm(4096, 768, 3072, a, b, dst)
     elif which == "config3":
         # the three attention-shaped batched products of configuration 3 (scores through the panel kernel, dQ and
-        # dK^T through the register-direct kernel), 5 launches each
+        # dK^T through the tile kernel's 64 x 64 tiles), 5 launches each, then the two gradients as one paired launch
         q, ds = synth.normal(2, (32, 512, 64)) / np.float32(8), synth.normal(2, (32, 512, 512), stream=2)
         dq, dk, dds = r.to_device(q), r.to_device(q), r.to_device(ds)
         g_out = r.malloc(32 * 512 * 64 * 4)
@@ -463,6 +470,10 @@ def run_for_counters(r, which):
             r.sgemm(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32), b_batch=(512 * 64, 32))
         for _ in range(5):
             r.sgemm(64, 512, 512, dq, dds, g_out, batch=32, a_strides=(1, 64), a_batch=(512 * 64, 32), b_batch=(512 * 512, 32))
+        g_out2 = r.malloc(32 * 512 * 64 * 4)
+        for _ in range(5):
+            r.sgemm_pair(r.gemm_desc(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32), b_batch=(512 * 64, 32)),
+                         r.gemm_desc(64, 512, 512, dq, dds, g_out2, batch=32, a_strides=(1, 64), a_batch=(512 * 64, 32), b_batch=(512 * 512, 32)))
     elif which == "attention":
         # the one-kernel attention forward on [8, 8192, 64], causal, through the engine entry point
         from framework_amd.api import bind

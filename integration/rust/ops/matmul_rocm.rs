@@ -13,6 +13,13 @@ use smallvec::smallvec;
 /// out[..., M, N] = op_a[..., M, K] * op_b[..., K, N]; batch b of an operand
 /// with fewer batches reads batch `b % count` (the CPU arm's rule, :55-56).
 fn product(store: &mut TensorStore, a: MniOperand, b: MniOperand, m: usize, n: usize, k: usize, batch: usize, out_shape: &[usize]) -> TensorId {
+    let (out, desc) = describe(store, a, b, m, n, k, batch, out_shape);
+    check(unsafe { mni_rocm_sgemm(&desc) });
+    out
+}
+
+/// A result tensor and the descriptor of the product that fills it; nothing is launched.
+fn describe(store: &mut TensorStore, a: MniOperand, b: MniOperand, m: usize, n: usize, k: usize, batch: usize, out_shape: &[usize]) -> (TensorId, MniGemmDesc) {
     let out = store.uninit(out_shape);
     let desc = MniGemmDesc {
         m: m as i64,
@@ -32,8 +39,7 @@ fn product(store: &mut TensorStore, a: MniOperand, b: MniOperand, m: usize, n: u
         aux: std::ptr::null_mut(),
         colsum_part: std::ptr::null_mut(),
     };
-    check(unsafe { mni_rocm_sgemm(&desc) });
-    out
+    (out, desc)
 }
 
 struct Dims {
@@ -118,11 +124,13 @@ pub fn matmul_backward(grad: TensorId, saved: &SavedContext, store: &mut TensorS
         let mut ga_shape = d.out_shape.clone();
         let nd = ga_shape.len();
         ga_shape[nd - 1] = d.k;
-        let ga = product(store, og, transposed(ob), d.m, d.k, d.n, d.batch, &ga_shape);
+        let (ga, desc_a) = describe(store, og, transposed(ob), d.m, d.k, d.n, d.batch, &ga_shape);
         // dB[.., K, N] = A^T[.., K, M] * dC[.., M, N]
         let mut gb_shape = d.out_shape.clone();
         gb_shape[nd - 2] = d.k;
-        let gb = product(store, transposed(oa), og, d.k, d.n, d.m, d.batch, &gb_shape);
+        let (gb, desc_b) = describe(store, transposed(oa), og, d.k, d.n, d.m, d.batch, &gb_shape);
+        // the two products do not depend on each other: issued together, in one launch where the library pairs them
+        check(unsafe { mni_rocm_sgemm_pair(&desc_a, &desc_b) });
         for t in [ta, tb, tg].into_iter().flatten() {
             store.free(t);
         }

@@ -77,6 +77,7 @@ extern "C" {
     pub fn mni_rocm_test_raise_device_status(code: c_uint) -> c_int;
     pub fn mni_rocm_launch_count() -> u64;
     pub fn mni_rocm_sgemm(desc: *const MniGemmDesc) -> c_int;
+    pub fn mni_rocm_sgemm_pair(first: *const MniGemmDesc, second: *const MniGemmDesc) -> c_int;
     pub fn mni_rocm_sgemm_colsum_rows(m: i64, batch: i64) -> i64;
     pub fn mni_rocm_sgemm_noalloc(desc: *const MniGemmDesc) -> c_int;
     pub fn mni_rocm_sgemm_noalloc_workspace_bytes() -> usize;
