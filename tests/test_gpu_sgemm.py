@@ -585,11 +585,12 @@ def _pair_descs(rocm, dev, batch, t, d, kview, ds, q, k):
     return d0, d1, o0, o1
 
 
-@pytest.mark.parametrize("batch,t,d,kview", [(16, 512, 64, True), (16, 512, 64, False), (32, 256, 128, True), (20, 500, 62, True),
+@pytest.mark.parametrize("batch,t,d,kview", [(16, 512, 64, True), (16, 512, 64, False), (32, 256, 128, True), (20, 500, 62, True), (20, 448, 64, True),
                                              (64, 512, 64, True)])
 def test_pair_launch_gives_the_bits_of_separate_launches(dev, rocm, batch, t, d, kview):
     # sizes at which each product alone is planned as 64 x 64 tiles, one workgroup per tile, so the pair goes out as
-    # one launch (the fourth with edges inside tiles and a K tail; the last with two tiles per CU each); integer
+    # one launch (the fourth with edges inside tiles and a K tail; the fifth with a tile count that is no multiple
+    # of 8, so that padding workgroups exist; the last with two tiles per CU each); integer
     # inputs pin the values, normal inputs the order of the K sum
     for make in (lambda s, shape, st: synth.small_ints(s, shape, 3, stream=st), lambda s, shape, st: synth.normal(s, shape, stream=st)):
         ds = make(1, (batch, t, t), 0)
