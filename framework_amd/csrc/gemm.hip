@@ -43,7 +43,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_PANEL)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_TINY)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -445,6 +445,20 @@ int sgemm(const mni_gemm_desc &d) {
     MNI_TRY(ensure_init());
     MNI_TRY(validate(d));
     if (d.M == 0 || d.N == 0 || d.batch == 0) return MNI_OK;
+    if (d.algo == MNI_ALGO_TINY || (d.algo == MNI_ALGO_AUTO && d.split_k == 0)) {
+        // A product that a launch's worth of threads computes outright (the README example's sizes: measured
+        // 2-3 us each against 4-13 us through the skinny and tile kernels).
+        GemmLaunch g;
+        fill_launch(g, d);
+        g.tiles_m = g.tiles_n = 1; g.split_k = 1; g.k_per_slice = g.K > 0 ? g.K : 1;
+        g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = ctx().status_dev;
+        if (d.algo == MNI_ALGO_TINY) {
+            if (d.epilogue > MNI_EPI_BIAS_GELU || d.split_k > 1)
+                return set_error(MNI_ERR_INVALID, "sgemm: the tiny-product kernel takes no split_k and no fused GELU epilogue");
+            return launch_gemm_tiny(g);
+        }
+        if (gemm_tiny_eligible(g)) return launch_gemm_tiny(g);
+    }
     if ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS) {
         int rc;
         if (try_skinny(d, &rc)) return rc;
@@ -478,6 +492,11 @@ int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1) {
         // (min(M, N) <= 16 may go to the skinny kernels, which sgemm tries before run_mfma)
         pair = d.M > 16 && d.N > 16 && d.K > 0 && d.batch > 0 && d.algo == MNI_ALGO_AUTO && d.split_k == 0;
         if (!pair) break;
+        {
+            GemmLaunch t;
+            fill_launch(t, d);
+            if (gemm_tiny_eligible(t)) { pair = false; break; }  // sgemm computes those outright
+        }
         MNI_TRY(run_mfma(d, &plan[i]));
         pair = plan[i].kind == PlanProbe::TILE && plan[i].bm == 64 && plan[i].bn == 64 && plan[i].split == 1;
         if (pair) tiles += (int64_t)plan[i].g.tiles_m * plan[i].g.tiles_n * plan[i].g.batch;

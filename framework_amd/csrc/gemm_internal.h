@@ -58,6 +58,9 @@ int gemm_mfma_tile_k();
 // the tile kernel; both must be 0 or 1 and pass gemm_direct_eligible.
 bool gemm_direct_eligible(const GemmLaunch &g, int amode, int bmode);
 int launch_gemm_direct(const GemmLaunch &g, int amode, int bmode, int ksplit);
+// One thread per output, sequential K (gemm_tiny.hip): a few thousand outputs of a short K, any strides.
+bool gemm_tiny_eligible(const GemmLaunch &g);
+int launch_gemm_tiny(const GemmLaunch &g);
 // Short-K form for two K-contiguous operands (gemm_panel.hip): 128 x 128 tiles
 // (g.tiles_m / g.tiles_n count those), all of K <= 64 at once.
 bool gemm_panel_eligible(const GemmLaunch &g, int amode, int bmode);

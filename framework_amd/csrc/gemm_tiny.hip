@@ -1,0 +1,103 @@
+// Products so small that a launch is most of their cost: one thread per output
+// element, a sequential loop over K.
+//
+//   C[b] = epilogue( op(A)[b] (M x K)  *  op(B)[b] (K x N) )
+//
+// The reference's README example (src/native/src/ops/matmul.rs:18-78 with
+// [32, 10] x [10, 64] and [32, 64] x [64, 3], and the four backward products of
+// ops/matmul.rs:199-222 on the same sizes) is made of such products: a few
+// thousand outputs, K of 3 to 64.  The tile and skinny kernels are built to
+// stream large operands; on these sizes they spend 4 to 13 us on set-up,
+// barriers, K slices and reductions that have nothing to work on.
+//
+// Every output is the reference CPU arm's own sum: products rounded to fp32,
+// added in k order, no fused multiply-add (ops/matmul.rs:62-69 is an i-k-j
+// loop of `c += a * b`), so this kernel reproduces that arm bit for bit, for
+// any strides.
+#include "common.h"
+#include "gemm_internal.h"
+
+namespace mni {
+
+static constexpr int TINY_THREADS = 256;
+
+__device__ __forceinline__ float tiny_gelu(float x) {
+    // tanh-approximation GELU of the reference (src/native/src/ops/activation.rs:15-18)
+    const float s = 0.7978845608028654f;
+    return 0.5f * x * (1.0f + tanhf(s * (x + 0.044715f * x * x * x)));
+}
+
+// A4 / W4: op(A) / op(B) has unit stride along K and is read four K values at a time.
+template <bool A4, bool W4>
+__global__ __launch_bounds__(TINY_THREADS) void gemm_tiny_kernel(const GemmLaunch g) {
+#pragma clang fp contract(off)  // products are rounded before they are added: no fused multiply-add in this function
+    const int64_t per = (int64_t)g.M * g.N;
+    const int64_t idx = (int64_t)blockIdx.x * TINY_THREADS + threadIdx.x;
+    if (idx >= per * g.batch) return;
+    const int b = (int)(idx / per);
+    const int r = (int)(idx - (int64_t)b * per);
+    const int m = r / g.N, n = r - m * g.N;
+    const float *__restrict__ a = g.A + (int64_t)(b % g.a_bcount) * g.a_bs + (int64_t)m * g.a_rs;
+    const float *__restrict__ w = g.B + (int64_t)(b % g.b_bcount) * g.b_bs + (int64_t)n * g.b_cs;
+    float acc = 0.0f;
+    // An operand whose K axis has unit stride is read four K values at a time (16-byte loads need no more than the
+    // 4-byte alignment every float has): with one row per lane, every 4-byte load of it would touch as many
+    // cache lines as there are lanes.
+    constexpr bool a4 = A4, w4 = W4;
+    const int k4 = (a4 || w4) ? g.K & ~3 : 0;
+#pragma unroll 4
+    for (int k = 0; k < k4; k += 4) {
+        float av[4], wv[4];
+        if (a4) {
+            const float4 t = *reinterpret_cast<const float4 *>(a + k);
+            av[0] = t.x; av[1] = t.y; av[2] = t.z; av[3] = t.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) av[j] = a[(int64_t)(k + j) * g.a_cs];
+        }
+        if (w4) {
+            const float4 t = *reinterpret_cast<const float4 *>(w + k);
+            wv[0] = t.x; wv[1] = t.y; wv[2] = t.z; wv[3] = t.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wv[j] = w[(int64_t)(k + j) * g.b_rs];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = acc + av[j] * wv[j];
+    }
+#pragma unroll 16
+    for (int k = k4; k < g.K; ++k) acc = acc + a[(int64_t)k * g.a_cs] * w[(int64_t)k * g.b_rs];
+    if (g.epilogue != MNI_EPI_NONE) {
+        acc += g.bias[n];
+        if (g.epilogue == MNI_EPI_BIAS_RELU) acc = fmaxf(acc, 0.0f);
+        else if (g.epilogue == MNI_EPI_BIAS_GELU) acc = tiny_gelu(acc);
+    }
+    float *dst = g.C + (int64_t)b * g.c_bs + (int64_t)m * g.ldc + n;
+    *dst = g.accumulate ? acc + *dst : acc;
+}
+
+// Few outputs and a short K: what a launch of 256-thread workgroups computes in about the time the launch takes.
+// Measured on MI355X against the tile kernel's 64 x 64 tiles (us): 32 x 64 x 10 2.6 / 5.3, 32 x 3 x 64 4.7 / 6.7,
+// 64 x 64 x 64 3.3 / 5.4, 256 x 256 x 64 3.5 / 5.8, 128 x 64 x 128 4.6 / 6.6, 128 x 128 x 256 7.1 / 8.6.
+bool gemm_tiny_eligible(const GemmLaunch &g) {
+    const int64_t outputs = (int64_t)g.M * g.N * g.batch;
+    return g.epilogue <= MNI_EPI_BIAS_GELU && outputs > 0 && outputs <= 65536 && g.K <= 256 && outputs * (g.K > 0 ? g.K : 1) <= (1 << 22);
+}
+
+int launch_gemm_tiny(const GemmLaunch &g) {
+    if (g.epilogue > MNI_EPI_BIAS_GELU) return set_error(MNI_ERR_INVALID, "sgemm: the tiny-product kernel has no fused GELU epilogues");
+    const int64_t outputs = (int64_t)g.M * g.N * g.batch;
+    if (outputs <= 0) return MNI_OK;
+    const int64_t blocks = (outputs + TINY_THREADS - 1) / TINY_THREADS;
+    if (blocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "sgemm: too many outputs for the tiny-product kernel");
+    const dim3 grid((unsigned)blocks), block(TINY_THREADS);
+    hipStream_t st = ctx().stream;
+    const bool a4 = g.a_cs == 1 && g.K >= 4, w4 = g.b_rs == 1 && g.K >= 4;
+    if (a4 && w4) MNI_KERNEL_LAUNCH((gemm_tiny_kernel<true, true>), grid, block, 0, st, g);
+    else if (a4) MNI_KERNEL_LAUNCH((gemm_tiny_kernel<true, false>), grid, block, 0, st, g);
+    else if (w4) MNI_KERNEL_LAUNCH((gemm_tiny_kernel<false, true>), grid, block, 0, st, g);
+    else MNI_KERNEL_LAUNCH((gemm_tiny_kernel<false, false>), grid, block, 0, st, g);
+    return check_launch("gemm_tiny_kernel");
+}
+
+}  // namespace mni

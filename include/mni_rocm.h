@@ -128,9 +128,12 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * with that extent even); PANEL = the short-K kernel for two K-contiguous
  * operands (A row-major, B given as its transpose; K <= 64, K % 4 == 0; error
  * otherwise): 128 x 128 tiles, all of K at once, stores of one part of a tile
- * under the MFMAs of the next.  AUTO picks among them. */
+ * under the MFMAs of the next; TINY = one thread per output element and a
+ * sequential sum over K, products rounded and added one by one as the
+ * reference's CPU arm does (bit-identical to it), for products of a few
+ * thousand outputs.  AUTO picks among them. */
 enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
-       MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7 };
+       MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7, MNI_ALGO_TINY = 8 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),

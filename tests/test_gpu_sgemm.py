@@ -569,6 +569,55 @@ def test_planner_choices_for_attention_shaped_products(dev, rocm):
     assert max_err(outs[0][7], q[7].T.astype(np.float64) @ ds[7].astype(np.float64)) <= gemm_tol(512, q, ds)
 
 
+# ---- tiny products: one thread per output, the reference CPU arm's own sum ---------------------------
+
+@pytest.mark.parametrize("m,n,k", [(32, 64, 10), (32, 3, 64), (32, 64, 3), (32, 10, 64), (64, 3, 32), (10, 64, 32), (1, 1, 1), (7, 5, 3),
+                                   (64, 64, 64), (33, 17, 130), (100, 60, 7)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_tiny_products_are_the_reference_sum_bit_for_bit(dev, oracle_native, m, n, k, ta, tb):
+    # the README example's six products among them; normal inputs: every output must be the oracle's i-k-j sum
+    # (products rounded, added in k order) to the last bit, whatever the layout, forced and chosen by the planner
+    a = synth.normal(m + k, (k, m) if ta else (m, k))
+    b = synth.normal(n + k, (n, k) if tb else (k, n), stream=1)
+    want = oracle_native.sgemm_ikj(np.ascontiguousarray(a.T) if ta else a, np.ascontiguousarray(b.T) if tb else b)
+    for algo in (N.ALGO_TINY, N.ALGO_AUTO):
+        got = run_gemm(dev, a, b, ta, tb, algo=algo)[0]
+        assert np.array_equal(got, want), algo
+
+
+def test_tiny_products_batch_rule_strides_epilogues_accumulate(dev, rocm, oracle_native):
+    a = synth.normal(1, (6, 20, 12))
+    w = synth.normal(2, (2, 12, 9), stream=1)     # batch b reads w[b % 2]
+    bias = synth.normal(3, (9,), stream=2)
+    c0 = synth.normal(4, (6, 20, 11), stream=3)   # C sits in rows of 11 floats
+    for epi, f in ((N.EPI_NONE, lambda z: z), (N.EPI_BIAS, lambda z: z + bias), (N.EPI_BIAS_RELU, lambda z: np.maximum(z + bias, 0)),
+                   (N.EPI_BIAS_GELU, lambda z: None)):   # tanh-approximation GELU, in float64 below
+        dA, dW, dbias, dC = dev.put(a), dev.put(w), dev.put(bias), dev.put(c0)
+        before = rocm.launch_count()
+        rocm.sgemm(20, 9, 12, dA, dW, dC, batch=6, a_batch=(20 * 12, 6), b_batch=(12 * 9, 2), ldc=11, c_batch_stride=20 * 11,
+                   bias=dbias if epi else None, epilogue=epi, accumulate=True)
+        assert rocm.launch_count() - before == 1
+        got = rocm.to_host(dC, (6, 20, 11))
+        assert np.array_equal(got[:, :, 9:], c0[:, :, 9:])   # the padding of C is untouched
+        for bb in range(6):
+            z = oracle_native.sgemm_ikj(a[bb], w[bb % 2])
+            want = f(z)
+            if want is None:
+                s_ = np.float32(0.7978845608028654)
+                zb = (z + bias).astype(np.float64)
+                want = (0.5 * zb * (1.0 + np.tanh(s_ * (zb + 0.044715 * zb ** 3)))).astype(np.float32)
+            assert max_err(got[bb, :, :9], want + c0[bb, :, :9]) <= 2e-6 * max(1.0, float(np.abs(want).max()))
+    # neither axis of A contiguous, B a column slice of a wider matrix
+    wide_a = synth.small_ints(5, (16, 2 * 24), 4)
+    wide_b = synth.small_ints(6, (24, 40), 4, stream=1)
+    dA, dB, dC = dev.put(wide_a), dev.put(wide_b), dev.empty(16 * 8)
+    rocm.sgemm(16, 8, 24, dA, dB + 4 * 5, dC, a_strides=(48, 2), b_strides=(40, 1), algo=N.ALGO_TINY)
+    want = wide_a[:, ::2].astype(np.int64) @ wide_b[:, 5:13].astype(np.int64)
+    assert np.array_equal(rocm.to_host(dC, (16, 8)), want.astype(np.float32))
+    with pytest.raises(N.MniError, match="no split_k and no fused GELU"):
+        rocm.sgemm(16, 8, 24, dA, dB, dC, algo=N.ALGO_TINY, split_k=2)
+
+
 # ---- two independent products in one launch (the backward pair of a batched matmul) ----------------
 
 def _pair_descs(rocm, dev, batch, t, d, kview, ds, q, k):
