@@ -17,7 +17,15 @@ def bind(native):
     class Tensor:  # src/tensor.ts:9-252
         def __init__(self, id, shape=None):
             self._id = id
-            self._shape = list(shape) if shape is not None else [int(s) for s in native.tensorShape(id)]
+            # the reference asks native.tensorShape(id) here when no shape is given; this mirror asks on first use
+            # (most results of a training step are passed on by id and never asked for their shape)
+            self._known_shape = list(shape) if shape is not None else None
+
+        @property
+        def _shape(self):
+            if self._known_shape is None:
+                self._known_shape = [int(s) for s in native.tensorShape(self._id)]
+            return self._known_shape
 
         @property
         def shape(self):

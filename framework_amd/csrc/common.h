@@ -51,6 +51,14 @@ struct DeviceCtx {
     // stream reads the word afterwards and fails loudly when it is set.
     unsigned *status_host = nullptr;  // host address
     unsigned *status_dev = nullptr;   // the same word as kernels address it
+    // A second word in the same pinned block: a kernel leaves a 32-bit result there, tagged with the number
+    // the host gave it, and the host reads it without a copy or a wait for the stream (wait_result_word).
+    unsigned long long *result_host = nullptr;
+    unsigned long long *result_dev = nullptr;
+    unsigned result_seq = 0;
+    // Pinned, device-visible buffer that small device-to-host reads arrive in (mni_rocm_d2h).
+    unsigned *fetch_host = nullptr;
+    unsigned *fetch_dev = nullptr;
     // Workspace source of the current sgemm call: null = the caching allocator;
     // otherwise the product's partial sums are placed in this preallocated
     // block of `scratch_bytes` (the entry point that must not allocate).
@@ -61,7 +69,32 @@ struct DeviceCtx {
     // Device address and size of the library's static workspace (see device.hip).
     float *noalloc_scratch = nullptr;
     size_t noalloc_scratch_bytes = 0;
+    // Pinned staging slots for small host-to-device uploads that must not stall the host (upload_small).
+    static constexpr int STAGE_SLOTS = 16;
+    static constexpr size_t STAGE_BYTES = 16384;
+    char *stage_host = nullptr;            // STAGE_SLOTS x STAGE_BYTES, pinned
+    hipEvent_t stage_done[STAGE_SLOTS] = {};
+    bool stage_used[STAGE_SLOTS] = {};
+    unsigned stage_next = 0;
 };
+// Host-to-device upload of `bytes` bytes on the library's stream.  Up to STAGE_BYTES the data is copied into a
+// pinned staging slot and the transfer is only enqueued: the host does not wait for the stream (an ordinary
+// mni_rocm_h2d drains everything queued so far), and `src` may be reused at once.  Larger uploads wait.
+int upload_small(void *dst, const void *src, size_t bytes);
+// A kernel hands one 32-bit value to the host: next_result_tag() clears the result word and returns the tag for
+// the launch; the kernel's last act is one 8-byte store of (tag << 32 | value) to ctx().result_dev;
+// wait_result_word() returns the value once that store has arrived.  It watches the word for a short while
+// (a kernel that is next in line delivers within microseconds), then waits for the stream; false in *delivered
+// if even then the word has not come (the caller has another way to the value).
+#ifdef __HIPCC__
+// One 8-byte store to pinned host memory: the host sees the tag and the value together or not at all, and
+// after everything this thread wrote before.
+__device__ __forceinline__ void post_result_word(unsigned long long *word, unsigned tag, unsigned value) {
+    __hip_atomic_store(word, ((unsigned long long)tag << 32) | (unsigned long long)value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+#endif
+unsigned next_result_tag();
+int wait_result_word(unsigned tag, unsigned *value, bool *delivered);
 enum { DEVICE_STATUS_OK = 0, DEVICE_STATUS_STREAMK_WAIT = 1, DEVICE_STATUS_SKINNY_WAIT = 2 };
 // hipStreamSynchronize on the library's stream, then the device status word:
 // MNI_ERR_HIP naming the kernel when a bounded wait expired since the last check.
@@ -135,7 +168,9 @@ int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t
 int k_expand_dim(float *out, const float *g, int64_t outer, int64_t dim, int64_t inner, float div);
 // generic unbroadcast: out (orig shape, contiguous) = sum of g over broadcast dims
 int k_unbroadcast(float *out, const float *g, const int64_t *gshape, int gnd, const int64_t *oshape, int ond);
-int k_cross_entropy(float *loss, float *softmax, const float *logits, const int32_t *targets,
+// targets: device buffer of n values.  targets_host: null when `targets` already holds them; otherwise the values
+// (each in [0, v)), which the call brings to `targets` itself.
+int k_cross_entropy(float *loss, float *softmax, const float *logits, int32_t *targets, const int32_t *targets_host,
                     int64_t n, int64_t v);
 int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t *targets,
                              const float *grad_scalar, int64_t n, int64_t v);
@@ -191,7 +226,9 @@ int k_sumsq_f64(double *out, const float *g, int64_t n);  // out += sum g^2 (dev
 // one tensor (sumsq_blocks(n) doubles), then out += sum of all partials.
 int sumsq_blocks(int64_t n);
 int k_sumsq_partials(double *part, const float *g, int64_t n);
-int k_sumsq_finish(double *out, const double *part, int nparts);
+// result_word / tag: when given, (float)out[0] also goes to that word (see wait_result_word).
+int k_sumsq_finish(double *out, const double *part, int nparts, bool overwrite = false, unsigned long long *result_word = nullptr,
+                   unsigned tag = 0);
 int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, float b1, float b2,
             float eps, float wd, float bc1, float bc2);
 // Many tensors in one launch.  Tensor i owns workgroups [block_start[i], block_start[i + 1]), one per
@@ -208,5 +245,9 @@ struct MultiTensor {
 int multi_tensor_blocks(int64_t n);
 int k_adamw_multi(const MultiTensor &t, float lr, float b1, float b2, float eps, float wd, float bc1, float bc2);
 int k_sumsq_multi(const MultiTensor &t, double *part);
+// Up to SUMSQ_SOLO_BLOCKS workgroups' worth of gradients: one workgroup computes the partial sums one after the
+// other and adds them up, in the order of k_sumsq_multi + k_sumsq_finish (same value); out[0] = the sum.
+constexpr int SUMSQ_SOLO_BLOCKS = 16;
+int k_sumsq_solo(const MultiTensor &t, double *out, unsigned long long *result_word, unsigned tag);
 
 }  // namespace mni

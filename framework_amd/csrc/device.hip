@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <chrono>
+
 #include <unordered_map>
 #include <vector>
 
@@ -102,12 +104,19 @@ static int init_device(int device) {
     MNI_HIP_CHECK(hipMalloc((void **)&c.skinny_flags, c.skinny_flag_cap * sizeof(unsigned)));
     MNI_HIP_CHECK(hipMemset(c.skinny_flags, 0, c.skinny_flag_cap * sizeof(unsigned)));
     c.skinny_epoch = 0;
+    // Pinned staging slots of upload_small, and one event per slot that says when its transfer has left it.
+    MNI_HIP_CHECK(hipHostMalloc((void **)&c.stage_host, DeviceCtx::STAGE_SLOTS * DeviceCtx::STAGE_BYTES, hipHostMallocDefault));
+    for (int i = 0; i < DeviceCtx::STAGE_SLOTS; ++i) MNI_HIP_CHECK(hipEventCreateWithFlags(&c.stage_done[i], hipEventDisableTiming));
     // Pinned, device-visible host memory: a kernel writes the word over the
     // bus in the rare case it has something to report, the host reads it for
     // free after every wait.
     MNI_HIP_CHECK(hipHostMalloc((void **)&c.status_host, 64, hipHostMallocMapped));
     memset(c.status_host, 0, 64);
     MNI_HIP_CHECK(hipHostGetDevicePointer((void **)&c.status_dev, c.status_host, 0));
+    MNI_HIP_CHECK(hipHostMalloc((void **)&c.fetch_host, DeviceCtx::STAGE_BYTES, hipHostMallocMapped));
+    MNI_HIP_CHECK(hipHostGetDevicePointer((void **)&c.fetch_dev, c.fetch_host, 0));
+    c.result_host = (unsigned long long *)(c.status_host + 2);  // bytes 8..15 of the block
+    c.result_dev = (unsigned long long *)(c.status_dev + 2);
     // Device address of the static workspace on this device (the library drives one device).
     float *scratch_ptr = nullptr;
     MNI_HIP_CHECK(hipGetSymbolAddress((void **)&scratch_ptr, HIP_SYMBOL(scratch)));
@@ -122,9 +131,60 @@ int ensure_init() {
     return init_device(0);
 }
 
-int sync_stream_checked(const char *what) {
+// Watches the result word for `tag` for at most `micros` microseconds.
+static bool poll_result_word(unsigned tag, unsigned *value, int micros) {
+    volatile unsigned long long *w = ctx().result_host;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (;;) {
+        for (int i = 0; i < 64; ++i) {
+            const unsigned long long v = *w;
+            if ((unsigned)(v >> 32) == tag) {
+                if (value) *value = (unsigned)v;
+                return true;
+            }
+            __builtin_ia32_pause();
+        }
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(micros)) return false;
+    }
+}
+static int blocking_sync(const char *what) {
     MNI_HIP_CHECK(hipStreamSynchronize(ctx().stream));
     return check_device_status(what);
+}
+unsigned next_result_tag() {
+    DeviceCtx &c = ctx();
+    if (++c.result_seq == 0) ++c.result_seq;
+    *(volatile unsigned long long *)c.result_host = 0;  // (every earlier result has been waited for)
+    return c.result_seq;
+}
+int wait_result_word(unsigned tag, unsigned *value, bool *delivered) {
+    *delivered = true;
+    if (poll_result_word(tag, value, 200)) return MNI_OK;
+    MNI_TRY(blocking_sync("waiting for a kernel's result"));
+    *delivered = poll_result_word(tag, value, 0);
+    return MNI_OK;
+}
+
+__global__ void marker_kernel(unsigned long long *word, unsigned tag) { post_result_word(word, tag, 0u); }
+// Up to DeviceCtx::STAGE_BYTES of device memory into pinned host memory, then the tag.
+__global__ __launch_bounds__(256) void fetch_small_kernel(unsigned *__restrict__ host, const unsigned *__restrict__ src, int words,
+                                                          unsigned long long *word, unsigned tag) {
+    for (int i = threadIdx.x; i < words; i += 256) host[i] = src[i];
+    __threadfence_system();
+    __syncthreads();
+    if (threadIdx.x == 0) post_result_word(word, tag, 0u);
+}
+
+// The stream runs in order, so a one-thread kernel queued now runs when everything before it is done; it
+// writes a tag to pinned host memory and the host watches for it.  That takes a few microseconds after the
+// last kernel ends; the runtime's own wait queues a barrier and sleeps on an interrupt, some twenty more.  Work
+// that lasts longer than the watch falls back on the runtime's wait.
+int sync_stream_checked(const char *what) {
+    DeviceCtx &c = ctx();
+    const unsigned tag = next_result_tag();
+    hipLaunchKernelGGL(marker_kernel, dim3(1), dim3(1), 0, c.stream, c.result_dev, tag);  // (not counted as a launch of the caller's work)
+    if (hipGetLastError() == hipSuccess && poll_result_word(tag, nullptr, 150)) return check_device_status(what);
+    return blocking_sync(what);
 }
 
 int check_device_status(const char *what) {
@@ -245,6 +305,23 @@ size_t dev_cached_bytes() { return allocator().cached; }
 
 using namespace mni;
 
+namespace mni {
+int upload_small(void *dst, const void *src, size_t bytes) {
+    MNI_TRY(ensure_init());
+    if (bytes == 0) return MNI_OK;
+    DeviceCtx &c = ctx();
+    if (bytes > DeviceCtx::STAGE_BYTES || !c.stage_host) return mni_rocm_h2d(dst, src, bytes);
+    const unsigned slot = c.stage_next++ % DeviceCtx::STAGE_SLOTS;
+    if (c.stage_used[slot]) MNI_HIP_CHECK(hipEventSynchronize(c.stage_done[slot]));  // sixteen uploads ago: long done
+    char *host = c.stage_host + (size_t)slot * DeviceCtx::STAGE_BYTES;
+    memcpy(host, src, bytes);
+    MNI_HIP_CHECK(hipMemcpyAsync(dst, host, bytes, hipMemcpyHostToDevice, c.stream));
+    MNI_HIP_CHECK(hipEventRecord(c.stage_done[slot], c.stream));
+    c.stage_used[slot] = true;
+    return MNI_OK;
+}
+}  // namespace mni
+
 extern "C" {
 
 int mni_rocm_init(int device) { MNI_API_GUARD; return init_device(device); }
@@ -285,7 +362,21 @@ int mni_rocm_d2h(void *dst, const void *src, size_t bytes) {
     MNI_API_GUARD;
     MNI_TRY(ensure_init());
     if (bytes == 0) return MNI_OK;
-    MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
+    DeviceCtx &c = ctx();
+    if (bytes <= DeviceCtx::STAGE_BYTES && bytes % 4 == 0 && ((uintptr_t)src & 3) == 0 && c.fetch_host) {
+        // a small read (a loss, a norm, a few hundred values): a kernel brings it to pinned host memory and
+        // says so; no copy to set up, no barrier to wait behind
+        const unsigned tag = next_result_tag();
+        hipLaunchKernelGGL(fetch_small_kernel, dim3(1), dim3(256), 0, c.stream, c.fetch_dev, (const unsigned *)src, (int)(bytes / 4),
+                           c.result_dev, tag);
+        MNI_TRY(check_launch("fetch_small_kernel"));
+        int rc = MNI_OK;
+        if (poll_result_word(tag, nullptr, 150)) rc = check_device_status("d2h");
+        else rc = blocking_sync("d2h");
+        if (rc == MNI_OK) memcpy(dst, c.fetch_host, bytes);
+        return rc;
+    }
+    MNI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, c.stream));
     return sync_stream_checked("d2h");
 }
 int mni_rocm_d2d(void *dst, const void *src, size_t bytes) {

@@ -6,6 +6,8 @@
 // and the 256-thread one-element-per-thread kernels of its cuda arm
 // (src/native/kernels/elementwise.cu) with 16-byte accesses where the layout
 // allows.
+#include <string.h>
+
 #include "common.h"
 
 // The reference's cpu arm rounds every multiply and every add separately (Rust
@@ -944,11 +946,8 @@ int k_unbroadcast(float *out, const float *g, const int64_t *gshape, int gnd, co
 // src/native/src/ops/loss.rs:24-67: per row max, exp, normalise, -ln p[target];
 // loss = mean over rows.  One wavefront per row; the row losses are summed by
 // a single wavefront in a fixed order.
-__global__ void ce_rows_kernel(float *__restrict__ row_loss, float *__restrict__ sm, const float *__restrict__ logits,
-                               const int32_t *__restrict__ targets, int64_t n, int64_t v) {
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (row >= n) return;
+__device__ __forceinline__ float ce_row(float *__restrict__ sm, const float *__restrict__ logits, const int32_t t,
+                                        const int64_t row, const int lane, const int64_t v) {
     const float *x = logits + row * v;
     float *p = sm + row * v;
     float mx = -INFINITY;
@@ -964,20 +963,22 @@ __global__ void ce_rows_kernel(float *__restrict__ row_loss, float *__restrict__
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
     for (int64_t j = lane; j < v; j += 64) p[j] = p[j] / sum;
-    if (lane == 0) {
-        const int32_t t = targets[row];
-        const float e = expf(x[t] - mx);
-        row_loss[row] = -logf(e / sum);
-    }
+    const float e = expf(x[t] - mx);
+    return -logf(e / sum);  // the row's loss (every lane holds it)
+}
+__global__ void ce_rows_kernel(float *__restrict__ row_loss, float *__restrict__ sm, const float *__restrict__ logits,
+                               const int32_t *__restrict__ targets, int64_t n, int64_t v) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n) return;
+    const float l = ce_row(sm, logits, targets[row], row, lane, v);
+    if (lane == 0) row_loss[row] = l;
 }
 // The same with the row held in registers (NV 16-byte pieces per lane): the
 // logits are read once and the probabilities written once.
 template <int NV>
-__global__ void ce_rows_cached_kernel(float *__restrict__ row_loss, float *__restrict__ sm, const float *__restrict__ logits,
-                                      const int32_t *__restrict__ targets, int64_t n, int64_t v) {
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (row >= n) return;
+__device__ __forceinline__ float ce_row_cached(float *__restrict__ sm, const float *__restrict__ logits, const int32_t t,
+                                               const int64_t row, const int lane, const int64_t v) {
     const int64_t v4 = v >> 2;
     const float4 *x = reinterpret_cast<const float4 *>(logits + row * v);
     float4 *p = reinterpret_cast<float4 *>(sm + row * v);
@@ -1007,11 +1008,17 @@ __global__ void ce_rows_cached_kernel(float *__restrict__ row_loss, float *__res
         const int64_t j = lane + 64 * i;
         if (j < v4) p[j] = make_float4(r[i].x / sum, r[i].y / sum, r[i].z / sum, r[i].w / sum);
     }
-    if (lane == 0) {
-        const int32_t t = targets[row];
-        const float e = expf(logits[row * v + t] - mx);
-        row_loss[row] = -logf(e / sum);
-    }
+    const float e = expf(logits[row * v + t] - mx);
+    return -logf(e / sum);
+}
+template <int NV>
+__global__ void ce_rows_cached_kernel(float *__restrict__ row_loss, float *__restrict__ sm, const float *__restrict__ logits,
+                                      const int32_t *__restrict__ targets, int64_t n, int64_t v) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n) return;
+    const float l = ce_row_cached<NV>(sm, logits, targets[row], row, lane, v);
+    if (lane == 0) row_loss[row] = l;
 }
 // Long rows: one workgroup per row, NV 16-byte pieces per thread, maximum and sum through LDS (the four
 // wavefront sums are added in wavefront order).  A wavefront per row would hold 128 registers of logits at
@@ -1072,12 +1079,59 @@ __global__ void ce_mean_kernel(float *__restrict__ loss, const float *__restrict
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
     if (lane == 0) loss[0] = s / (float)n;
 }
-int k_cross_entropy(float *loss, float *softmax, const float *logits, const int32_t *targets, int64_t n, int64_t v) {
+// A small batch in one launch: one workgroup of sixteen wavefronts, which take the rows in turn (four each at
+// most) and leave the row losses in LDS; the first wavefront then adds them in ce_mean_kernel's order.  Same
+// sums as the two launches.  EMBED: the targets arrive in the kernel arguments (no upload has to be queued for
+// sixty-four numbers) and are written to `targets` for the backward pass.
+constexpr int CE_SMALL_ROWS = 64;
+constexpr int64_t CE_SMALL_VALUES = 16384;
+struct CeTargets {
+    int32_t t[CE_SMALL_ROWS];
+};
+template <int NV, bool EMBED>  // NV 0: ce_row, else ce_row_cached<NV>
+__global__ __launch_bounds__(1024) void ce_small_kernel(float *__restrict__ loss, float *__restrict__ sm, const float *__restrict__ logits,
+                                                        int32_t *__restrict__ targets, int n, int64_t v, const CeTargets given) {
+    __shared__ float row_loss[CE_SMALL_ROWS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int row = wave; row < n; row += 16) {
+        const int32_t t = EMBED ? given.t[row] : targets[row];
+        float l;
+        if constexpr (NV == 0) l = ce_row(sm, logits, t, row, lane, v);
+        else l = ce_row_cached<NV>(sm, logits, t, row, lane, v);
+        if (lane == 0) {
+            row_loss[row] = l;
+            if (EMBED) targets[row] = t;
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float s = 0.f;
+    for (int i = lane; i < n; i += 64) s += row_loss[i];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (lane == 0) loss[0] = s / (float)n;
+}
+// targets: device buffer of n values.  targets_host: null when `targets` already holds them; otherwise the
+// values, which this call brings to `targets` (checked by the caller to lie in [0, v)).
+int k_cross_entropy(float *loss, float *softmax, const float *logits, int32_t *targets, const int32_t *targets_host, int64_t n, int64_t v) {
     MNI_TRY(ensure_init());
     if (n <= 0 || v <= 0) return set_error(MNI_ERR_INVALID, "cross_entropy: empty logits");
+    const bool vec = (v % 4) == 0 && al16(logits) && al16(softmax);
+    if (n <= CE_SMALL_ROWS && n * v <= CE_SMALL_VALUES && (!vec || v <= 64 * 4 * 2)) {
+        CeTargets given;
+        memset(&given, 0, sizeof given);
+        if (targets_host) memcpy(given.t, targets_host, (size_t)n * sizeof(int32_t));
+        const dim3 grid(1), block(1024);
+        hipStream_t st = ctx().stream;
+        if (vec && targets_host) MNI_KERNEL_LAUNCH((ce_small_kernel<2, true>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, given);
+        else if (vec) MNI_KERNEL_LAUNCH((ce_small_kernel<2, false>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, given);
+        else if (targets_host) MNI_KERNEL_LAUNCH((ce_small_kernel<0, true>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, given);
+        else MNI_KERNEL_LAUNCH((ce_small_kernel<0, false>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, given);
+        return check_launch("ce_small");
+    }
+    if (targets_host) MNI_TRY(upload_small(targets, targets_host, (size_t)n * sizeof(int32_t)));
     void *rl = nullptr;
     MNI_TRY(dev_alloc(&rl, (size_t)n * sizeof(float)));
-    const bool vec = (v % 4) == 0 && al16(logits) && al16(softmax);
     const dim3 grid(grid_for(n, 4)), block(TPB);
     hipStream_t st = ctx().stream;
     if (vec && v <= 64 * 4 * 2)
@@ -1155,16 +1209,26 @@ __global__ void sumsq_kernel(double *__restrict__ part, const float *__restrict_
     __syncthreads();
     if (threadIdx.x == 0) part[blockIdx.x] = (sh[0] + sh[1]) + (sh[2] + sh[3]);
 }
-// out[0] += sum of part[0..nparts): one workgroup, fixed order
-__global__ void sumsq_final_kernel(double *__restrict__ out, const double *__restrict__ part, int nparts) {
-    __shared__ double sh[4];
+// Sum of part[0..nparts) by one workgroup of TPB threads in a fixed order; the value in thread 0 (sh: four doubles of LDS).
+__device__ __forceinline__ double sum_partials(const double *part, int nparts, double *sh) {
     double s = 0.0;
-    for (int p = threadIdx.x; p < nparts; p += blockDim.x) s += part[p];
+    for (int p = threadIdx.x; p < nparts; p += TPB) s += part[p];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
     if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
     __syncthreads();
-    if (threadIdx.x == 0) out[0] += (sh[0] + sh[1]) + (sh[2] + sh[3]);
+    return (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+// out[0] (+)= sum of part[0..nparts): one workgroup, fixed order
+__global__ __launch_bounds__(TPB) void sumsq_final_kernel(double *__restrict__ out, const double *__restrict__ part, int nparts, int overwrite,
+                                                          unsigned long long *result_word, unsigned tag) {
+    __shared__ double sh[4];
+    const double s = sum_partials(part, nparts, sh);
+    if (threadIdx.x == 0) {
+        const double total = (overwrite ? 0.0 : out[0]) + s;
+        out[0] = total;
+        if (result_word) post_result_word(result_word, tag, __float_as_uint((float)total));
+    }
 }
 int sumsq_blocks(int64_t n) {
     if (n <= 0) return 0;
@@ -1177,10 +1241,11 @@ int k_sumsq_partials(double *part, const float *g, int64_t n) {
     MNI_KERNEL_LAUNCH(sumsq_kernel, dim3(sumsq_blocks(n)), dim3(TPB), 0, ctx().stream, part, g, n);
     return check_launch("sumsq");
 }
-int k_sumsq_finish(double *out, const double *part, int nparts) {
-    if (nparts <= 0) return MNI_OK;
+int k_sumsq_finish(double *out, const double *part, int nparts, bool overwrite, unsigned long long *result_word, unsigned tag) {
+    if (nparts <= 0 && !overwrite && !result_word) return MNI_OK;
     MNI_TRY(ensure_init());
-    MNI_KERNEL_LAUNCH(sumsq_final_kernel, dim3(1), dim3(TPB), 0, ctx().stream, out, part, nparts);
+    MNI_KERNEL_LAUNCH(sumsq_final_kernel, dim3(1), dim3(TPB), 0, ctx().stream, out, part, nparts < 0 ? 0 : nparts, overwrite ? 1 : 0,
+                       result_word, tag);
     return check_launch("sumsq_final");
 }
 int k_sumsq_f64(double *out, const float *g, int64_t n) {
@@ -1226,6 +1291,16 @@ int k_adamw(float *p, float *m, float *v, const float *g, int64_t n, float lr, f
 // dozens of parameters, most of them a few hundred values long): the table
 // rides in the kernel arguments, a workgroup takes MULTI_CHUNK elements of the
 // tensor its index falls into.
+// Sum of squares of g[lo..hi) in f64 by one workgroup of TPB threads; the value in thread 0 (sh: four doubles of LDS).
+__device__ __forceinline__ double chunk_sumsq(const float *__restrict__ g, int64_t lo, int64_t hi, double *sh) {
+    double sq = 0.0;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += TPB) { const double x = (double)g[i]; sq += x * x; }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = sq;
+    __syncthreads();
+    return (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
 template <bool ADAM>
 __global__ void multi_tensor_kernel(const MultiTensor t, double *__restrict__ part, float lr, float b1, float b2, float eps,
                                     float wd, float bc1, float bc2) {
@@ -1260,13 +1335,29 @@ __global__ void multi_tensor_kernel(const MultiTensor t, double *__restrict__ pa
         }
     } else {
         __shared__ double sh[4];
-        double sq = 0.0;
-        for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) { const double x = (double)g[i]; sq += x * x; }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
-        if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = sq;
-        __syncthreads();
-        if (threadIdx.x == 0) part[blockIdx.x] = (sh[0] + sh[1]) + (sh[2] + sh[3]);
+        const double sq = chunk_sumsq(g, lo, hi, sh);
+        if (threadIdx.x == 0) part[blockIdx.x] = sq;
+    }
+}
+__global__ __launch_bounds__(TPB) void sumsq_solo_kernel(const MultiTensor t, double *__restrict__ out, unsigned long long *result_word,
+                                                         unsigned tag) {
+    __shared__ double sh[4];
+    __shared__ double part[SUMSQ_SOLO_BLOCKS];
+    const int blocks = t.block_start[t.count];
+    int ti = 0;
+    for (int b = 0; b < blocks; ++b) {
+        while (ti + 1 < t.count && b >= t.block_start[ti + 1]) ++ti;
+        const int64_t n = t.n[ti];
+        const int64_t lo = (int64_t)(b - t.block_start[ti]) * MULTI_CHUNK;
+        const int64_t hi = lo + MULTI_CHUNK < n ? lo + MULTI_CHUNK : n;
+        const double sq = chunk_sumsq(t.g[ti], lo, hi, sh);
+        if (threadIdx.x == 0) part[b] = sq;
+        __syncthreads();  // sh is reused; part[b] is visible
+    }
+    const double total = sum_partials(part, blocks, sh);
+    if (threadIdx.x == 0) {
+        out[0] = total;
+        if (result_word) post_result_word(result_word, tag, __float_as_uint((float)total));
     }
 }
 int multi_tensor_blocks(int64_t n) { return (int)((n + MULTI_CHUNK - 1) / MULTI_CHUNK); }
@@ -1286,6 +1377,13 @@ int k_adamw_multi(const MultiTensor &t, float lr, float b1, float b2, float eps,
     MNI_KERNEL_LAUNCH(multi_tensor_kernel<true>, dim3(t.block_start[t.count]), dim3(TPB), 0, ctx().stream, t, (double *)nullptr, lr, b1,
                        b2, eps, wd, bc1, bc2);
     return check_launch("adamw_multi");
+}
+int k_sumsq_solo(const MultiTensor &t, double *out, unsigned long long *result_word, unsigned tag) {
+    MNI_TRY(ensure_init());
+    MNI_TRY(multi_check(t));
+    if (t.block_start[t.count] > SUMSQ_SOLO_BLOCKS) return set_error(MNI_ERR_INVALID, "sumsq_solo: more than %d chunks", SUMSQ_SOLO_BLOCKS);
+    MNI_KERNEL_LAUNCH(sumsq_solo_kernel, dim3(1), dim3(TPB), 0, ctx().stream, t, out, result_word, tag);
+    return check_launch("sumsq_solo");
 }
 int k_sumsq_multi(const MultiTensor &t, double *part) {
     MNI_TRY(ensure_init());

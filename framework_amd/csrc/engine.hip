@@ -18,6 +18,7 @@
 #include <vector>
 
 #include "common.h"
+#include <functional>
 
 namespace mni {
 namespace {
@@ -130,6 +131,9 @@ struct Engine {
     // output id of a GELU Linear -> its bias gradient, when the gradient that reaches it has already been
     // taken through gelu' by the entry that consumed it
     std::map<uint32_t, uint32_t> preact_db;
+    // One float holding 1.0, shared by every scalar loss as the gradient backward() starts from (writers copy
+    // a shared buffer before they touch it, so nobody changes it).
+    BufP one;
 };
 static Engine &eng() {
     // Never destroyed: releasing device buffers from a static destructor would
@@ -856,12 +860,11 @@ static uint32_t cross_entropy_op(uint32_t logits, const int64_t *targets, size_t
     void *tp = nullptr;
     if (dev_alloc(&tp, (size_t)n * sizeof(int32_t)) != MNI_OK) return MNI_BAD_ID;
     std::shared_ptr<void> tdev(tp, [](void *p) { dev_free(p); });
-    if (mni_rocm_h2d(tp, t32.data(), (size_t)n * sizeof(int32_t)) != MNI_OK) return MNI_BAD_ID;
     BufP x = contiguous_buf(*L);
     BufP sm = x ? new_buf((size_t)(n * v)) : nullptr;
     BufP loss = sm ? new_buf(1) : nullptr;
     if (!loss) return MNI_BAD_ID;
-    if (k_cross_entropy(loss->p, sm->p, x->p, (const int32_t *)tp, n, v) != MNI_OK) return MNI_BAD_ID;
+    if (k_cross_entropy(loss->p, sm->p, x->p, (int32_t *)tp, t32.data(), n, v) != MNI_OK) return MNI_BAD_ID;
     const uint32_t loss_id = insert_contig(std::move(loss), Shape{1});
     const uint32_t sm_id = insert_contig(std::move(sm), shape);
     Entry e;
@@ -1539,7 +1542,7 @@ static int sample_batch(uint32_t dataset, int64_t block, int64_t batch, uint32_t
     inp.data = dev_ints((size_t)(batch * block));
     tgt.data = dev_ints((size_t)(batch * block));
     if (!dstarts || !inp.data || !tgt.data) return MNI_ERR_NOMEM;
-    MNI_TRY(mni_rocm_h2d(dstarts.get(), starts.data(), (size_t)batch * sizeof(int32_t)));
+    MNI_TRY(upload_small(dstarts.get(), starts.data(), (size_t)batch * sizeof(int32_t)));
     const std::shared_ptr<void> src = ds->data;
     inp.len = tgt.len = batch * block;
     inp.lo = tgt.lo = ds->lo;
@@ -1599,7 +1602,7 @@ static uint32_t embedding_forward(uint32_t weight, const int64_t *indices, size_
     for (int64_t i = 0; i < tokens; ++i) i32[(size_t)i] = (int32_t)indices[i];
     std::shared_ptr<void> dev = dev_ints((size_t)tokens);
     if (!dev) return MNI_BAD_ID;
-    if (tokens && mni_rocm_h2d(dev.get(), i32.data(), (size_t)tokens * sizeof(int32_t)) != MNI_OK) return MNI_BAD_ID;
+    if (tokens && upload_small(dev.get(), i32.data(), (size_t)tokens * sizeof(int32_t)) != MNI_OK) return MNI_BAD_ID;
     return embedding_common(weight, std::move(dev), batch, seq_len);
 }
 static uint32_t embedding_forward_gpu(uint32_t weight, uint32_t int_buf, int64_t batch, int64_t seq_len) {
@@ -1647,7 +1650,7 @@ static uint32_t cross_entropy_gpu_op(uint32_t logits, uint32_t int_buf) {
     BufP sm = x ? new_buf((size_t)(n * v)) : nullptr;
     BufP loss = sm ? new_buf(1) : nullptr;
     if (!loss) return MNI_BAD_ID;
-    if (k_cross_entropy(loss->p, sm->p, x->p, (const int32_t *)tdev.get(), n, v) != MNI_OK) return MNI_BAD_ID;
+    if (k_cross_entropy(loss->p, sm->p, x->p, (int32_t *)tdev.get(), nullptr, n, v) != MNI_OK) return MNI_BAD_ID;
     const uint32_t loss_id = insert_contig(std::move(loss), Shape{1});
     const uint32_t sm_id = insert_contig(std::move(sm), Shape{n, v});
     Entry e;
@@ -1841,7 +1844,18 @@ static int tape_backward(Tape &tp, uint32_t loss) {
     } walk_scope(eng(), &tp, &out2entry, &consumers, &grads);
     {
         const Shape shape = get(loss)->shape;
-        const uint32_t g = filled(shape, 1.0f);  // ones_like for any loss shape, autograd.rs:143
+        uint32_t g;  // ones_like for any loss shape, autograd.rs:143
+        if (shape_size(shape) == 1) {
+            Engine &e = eng();
+            if (!e.one) {
+                e.one = new_buf(1);
+                if (!e.one) return MNI_ERR_NOMEM;
+                if (k_fill(e.one->p, 1.0f, 1) != MNI_OK) { e.one = nullptr; return MNI_ERR_HIP; }
+            }
+            g = insert_contig(BufP(e.one), shape);
+        } else {
+            g = filled(shape, 1.0f);
+        }
         if (g == MNI_BAD_ID) return MNI_ERR_NOMEM;
         grads[loss] = g;
     }
@@ -1884,7 +1898,9 @@ static float powi_f32(float a, int b) {  // f32::powi (compiler-rt __powisf2)
 }
 
 // ops/optimizer.rs:126-138 grad_norm
-static int grad_norm(const uint32_t *ids, size_t n, float *out) {
+// before_read: issued after the norm's kernels and before the host waits for the value (work that does not
+// depend on it then runs while the copy is in flight).
+static int grad_norm(const uint32_t *ids, size_t n, float *out, const std::function<int()> &before_read = nullptr) {
     // Workgroups of multi-tensor launches leave one partial sum each in one
     // buffer; a single kernel adds them up.
     std::vector<Tensor *> gs;
@@ -1899,11 +1915,20 @@ static int grad_norm(const uint32_t *ids, size_t n, float *out) {
         gs.push_back(G);
         nparts += multi_tensor_blocks(G->size);
     }
+    if (nparts == 0) {  // no gradients
+        if (before_read) MNI_TRY(before_read());
+        *out = 0.0f;
+        return MNI_OK;
+    }
     void *acc = nullptr;
     MNI_TRY(dev_alloc(&acc, (size_t)(nparts + 1) * sizeof(double)));
     std::shared_ptr<void> guard(acc, [](void *p) { dev_free(p); });
     double *total = (double *)acc, *part = total + 1;
-    MNI_TRY(k_fill((float *)total, 0.0f, 2));  // one double
+    // The sum also goes, as a float, to a word of pinned host memory: the host then has it a few microseconds
+    // after the kernel that wrote it, with no copy to order and no wait for what was queued behind it.
+    const unsigned tag = next_result_tag();
+    unsigned long long *word = ctx().result_dev;
+    const bool solo = gs.size() <= (size_t)MULTI_MAX && nparts <= SUMSQ_SOLO_BLOCKS;
     int64_t at = 0;
     for (size_t first = 0; first < gs.size(); first += MULTI_MAX) {
         MultiTensor t;
@@ -1918,13 +1943,24 @@ static int grad_norm(const uint32_t *ids, size_t n, float *out) {
             blocks += multi_tensor_blocks(G->size);
         }
         t.block_start[t.count] = blocks;
-        MNI_TRY(k_sumsq_multi(t, part + at));
+        if (solo) MNI_TRY(k_sumsq_solo(t, total, word, tag));  // a small model: partial sums and their sum in one launch
+        else MNI_TRY(k_sumsq_multi(t, part + at));
         at += blocks;
     }
-    MNI_TRY(k_sumsq_finish(total, part, (int)nparts));
-    double sq = 0.0;
-    MNI_TRY(mni_rocm_d2h(&sq, total, sizeof(double)));
-    *out = sqrtf((float)sq);
+    if (!solo) MNI_TRY(k_sumsq_finish(total, part, (int)nparts, true, word, tag));
+    if (before_read) MNI_TRY(before_read());
+    unsigned bits = 0;
+    bool delivered = false;
+    MNI_TRY(wait_result_word(tag, &bits, &delivered));
+    float sq;
+    if (delivered) {
+        memcpy(&sq, &bits, sizeof sq);
+    } else {
+        double sq64 = 0.0;
+        MNI_TRY(mni_rocm_d2h(&sq64, total, sizeof(double)));
+        sq = (float)sq64;
+    }
+    *out = sqrtf(sq);
     return MNI_OK;
 }
 
@@ -2022,7 +2058,7 @@ uint32_t mni_from_float32(const float *data, size_t len, const int64_t *shape, i
         return MNI_BAD_ID;
     }
     BufP b = new_buf((size_t)n);
-    if (!b || mni_rocm_h2d(b->p, data, (size_t)n * sizeof(float)) != MNI_OK) return MNI_BAD_ID;
+    if (!b || upload_small(b->p, data, (size_t)n * sizeof(float)) != MNI_OK) return MNI_BAD_ID;
     return insert_contig(std::move(b), s);
 }
 int mni_tensor_shape(uint32_t id, int64_t *out, int cap) {
@@ -2236,12 +2272,17 @@ double mni_clip_and_step(const uint32_t *ids, size_t n, double lr, double beta1,
                          double weight_decay, int64_t step, double max_grad_norm) {  // optimizer.rs:224-245
     MNI_API_GUARD;
     float norm = 0.f;
-    if (grad_norm(ids, n, &norm) != MNI_OK) return -1.0;
     const float mg = (float)max_grad_norm;
-    if (mg > 0.0f && norm > mg)
+    auto update = [&] { return adamw_step(ids, n, (float)lr, (float)beta1, (float)beta2, (float)eps, (float)weight_decay, (uint32_t)step); };
+    if (!(mg > 0.0f)) {
+        // no clipping asked for: the update does not depend on the norm and is issued before the host waits for it
+        if (grad_norm(ids, n, &norm, update) != MNI_OK) return -1.0;
+        return (double)norm;
+    }
+    if (grad_norm(ids, n, &norm) != MNI_OK) return -1.0;
+    if (norm > mg)
         if (scale_grads(ids, n, mg / norm) != MNI_OK) return -1.0;
-    if (adamw_step(ids, n, (float)lr, (float)beta1, (float)beta2, (float)eps, (float)weight_decay, (uint32_t)step) != MNI_OK)
-        return -1.0;
+    if (update() != MNI_OK) return -1.0;
     return (double)norm;
 }
 void mni_reset_engine(void) {

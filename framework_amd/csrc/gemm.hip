@@ -484,6 +484,20 @@ int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1) {
     DeviceCtx &c = ctx();
     const int cus = c.compute_units > 0 ? c.compute_units : 256;
     const mni_gemm_desc *ds[2] = {&d0, &d1};
+    {
+        // two products of a few thousand outputs each (sgemm would give each a launch of the tiny-product kernel)
+        GemmLaunch t[2] = {};
+        bool tiny = true;
+        for (int i = 0; i < 2 && tiny; ++i) {
+            const mni_gemm_desc &d = *ds[i];
+            tiny = d.M > 0 && d.N > 0 && d.K > 0 && d.batch > 0 && d.algo == MNI_ALGO_AUTO && d.split_k == 0;
+            if (tiny) {
+                fill_launch(t[i], d);
+                tiny = gemm_tiny_eligible(t[i]);
+            }
+        }
+        if (tiny) return launch_gemm_tiny_pair(t[0], t[1]);
+    }
     PlanProbe plan[2];
     int64_t tiles = 0;
     bool pair = true;

@@ -61,6 +61,7 @@ int launch_gemm_direct(const GemmLaunch &g, int amode, int bmode, int ksplit);
 // One thread per output, sequential K (gemm_tiny.hip): a few thousand outputs of a short K, any strides.
 bool gemm_tiny_eligible(const GemmLaunch &g);
 int launch_gemm_tiny(const GemmLaunch &g);
+int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1);  // two eligible, independent products in one launch
 // Short-K form for two K-contiguous operands (gemm_panel.hip): 128 x 128 tiles
 // (g.tiles_m / g.tiles_n count those), all of K <= 64 at once.
 bool gemm_panel_eligible(const GemmLaunch &g, int amode, int bmode);

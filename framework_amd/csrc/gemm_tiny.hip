@@ -28,11 +28,11 @@ __device__ __forceinline__ float tiny_gelu(float x) {
 }
 
 // A4 / W4: op(A) / op(B) has unit stride along K and is read four K values at a time.
+// idx: the output this thread computes, counted over batch, rows and columns.
 template <bool A4, bool W4>
-__global__ __launch_bounds__(TINY_THREADS) void gemm_tiny_kernel(const GemmLaunch g) {
+__device__ __forceinline__ void gemm_tiny_output(const GemmLaunch &g, const int64_t idx) {
 #pragma clang fp contract(off)  // products are rounded before they are added: no fused multiply-add in this function
     const int64_t per = (int64_t)g.M * g.N;
-    const int64_t idx = (int64_t)blockIdx.x * TINY_THREADS + threadIdx.x;
     if (idx >= per * g.batch) return;
     const int b = (int)(idx / per);
     const int r = (int)(idx - (int64_t)b * per);
@@ -75,6 +75,28 @@ __global__ __launch_bounds__(TINY_THREADS) void gemm_tiny_kernel(const GemmLaunc
     float *dst = g.C + (int64_t)b * g.c_bs + (int64_t)m * g.ldc + n;
     *dst = g.accumulate ? acc + *dst : acc;
 }
+template <bool A4, bool W4>
+__global__ __launch_bounds__(TINY_THREADS) void gemm_tiny_kernel(const GemmLaunch g) {
+    gemm_tiny_output<A4, W4>(g, (int64_t)blockIdx.x * TINY_THREADS + threadIdx.x);
+}
+// Two independent products in one launch: workgroups [0, blocks0) compute the first, the rest the second.
+// form: bit 0 = A4, bit 1 = W4 of each product.
+struct TinyPairLaunch {
+    GemmLaunch g[2];
+    unsigned blocks0;
+    int form[2];
+};
+__global__ __launch_bounds__(TINY_THREADS) void gemm_tiny_pair_kernel(const TinyPairLaunch p) {
+    const bool second = blockIdx.x >= p.blocks0;
+    const GemmLaunch &g = second ? p.g[1] : p.g[0];
+    const int64_t idx = (int64_t)(blockIdx.x - (second ? p.blocks0 : 0u)) * TINY_THREADS + threadIdx.x;
+    switch (second ? p.form[1] : p.form[0]) {
+        case 0: gemm_tiny_output<false, false>(g, idx); break;
+        case 1: gemm_tiny_output<true, false>(g, idx); break;
+        case 2: gemm_tiny_output<false, true>(g, idx); break;
+        default: gemm_tiny_output<true, true>(g, idx); break;
+    }
+}
 
 // Few outputs and a short K: what a launch of 256-thread workgroups computes in about the time the launch takes.
 // Measured on MI355X against the tile kernel's 64 x 64 tiles (us): 32 x 64 x 10 2.6 / 5.3, 32 x 3 x 64 4.7 / 6.7,
@@ -84,20 +106,39 @@ bool gemm_tiny_eligible(const GemmLaunch &g) {
     return g.epilogue <= MNI_EPI_BIAS_GELU && outputs > 0 && outputs <= 65536 && g.K <= 256 && outputs * (g.K > 0 ? g.K : 1) <= (1 << 22);
 }
 
+static int tiny_form(const GemmLaunch &g) { return (g.a_cs == 1 && g.K >= 4 ? 1 : 0) | (g.b_rs == 1 && g.K >= 4 ? 2 : 0); }
+static int64_t tiny_blocks(const GemmLaunch &g) { return ((int64_t)g.M * g.N * g.batch + TINY_THREADS - 1) / TINY_THREADS; }
+
 int launch_gemm_tiny(const GemmLaunch &g) {
     if (g.epilogue > MNI_EPI_BIAS_GELU) return set_error(MNI_ERR_INVALID, "sgemm: the tiny-product kernel has no fused GELU epilogues");
     const int64_t outputs = (int64_t)g.M * g.N * g.batch;
     if (outputs <= 0) return MNI_OK;
-    const int64_t blocks = (outputs + TINY_THREADS - 1) / TINY_THREADS;
+    const int64_t blocks = tiny_blocks(g);
     if (blocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "sgemm: too many outputs for the tiny-product kernel");
     const dim3 grid((unsigned)blocks), block(TINY_THREADS);
     hipStream_t st = ctx().stream;
-    const bool a4 = g.a_cs == 1 && g.K >= 4, w4 = g.b_rs == 1 && g.K >= 4;
-    if (a4 && w4) MNI_KERNEL_LAUNCH((gemm_tiny_kernel<true, true>), grid, block, 0, st, g);
-    else if (a4) MNI_KERNEL_LAUNCH((gemm_tiny_kernel<true, false>), grid, block, 0, st, g);
-    else if (w4) MNI_KERNEL_LAUNCH((gemm_tiny_kernel<false, true>), grid, block, 0, st, g);
-    else MNI_KERNEL_LAUNCH((gemm_tiny_kernel<false, false>), grid, block, 0, st, g);
+    switch (tiny_form(g)) {
+        case 3: MNI_KERNEL_LAUNCH((gemm_tiny_kernel<true, true>), grid, block, 0, st, g); break;
+        case 1: MNI_KERNEL_LAUNCH((gemm_tiny_kernel<true, false>), grid, block, 0, st, g); break;
+        case 2: MNI_KERNEL_LAUNCH((gemm_tiny_kernel<false, true>), grid, block, 0, st, g); break;
+        default: MNI_KERNEL_LAUNCH((gemm_tiny_kernel<false, false>), grid, block, 0, st, g); break;
+    }
     return check_launch("gemm_tiny_kernel");
+}
+
+// Both products must pass gemm_tiny_eligible; neither may read what the other writes.
+int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1) {
+    if (!gemm_tiny_eligible(g0) || !gemm_tiny_eligible(g1))
+        return set_error(MNI_ERR_INVALID, "sgemm_pair: the tiny-product pair takes two products that each fit the tiny-product kernel");
+    TinyPairLaunch p;
+    p.g[0] = g0;
+    p.g[1] = g1;
+    p.blocks0 = (unsigned)tiny_blocks(g0);
+    p.form[0] = tiny_form(g0);
+    p.form[1] = tiny_form(g1);
+    const dim3 grid(p.blocks0 + (unsigned)tiny_blocks(g1)), block(TINY_THREADS);
+    MNI_KERNEL_LAUNCH(gemm_tiny_pair_kernel, grid, block, 0, ctx().stream, p);
+    return check_launch("gemm_tiny_pair_kernel");
 }
 
 }  // namespace mni

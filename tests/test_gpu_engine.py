@@ -530,6 +530,33 @@ def test_entry_points_serialise_concurrent_callers(rocm_native):
     assert errors == []
 
 
+@pytest.mark.parametrize("sizes", [[5], [640, 64, 192, 3], [4096 * 16], [4096 * 16 + 1], [100000, 7], [33] * 49, [4096] * 16 + [1]])
+def test_grad_norm_small_models_in_one_launch_and_large_ones_in_two(gpu, sizes):
+    # up to sixteen 4096-value chunks of gradients are summed by one workgroup in one launch; beyond that (or with more
+    # tensors than one launch's table holds) by a launch of partial sums and one that adds them.  Either way the
+    # norm reaches the host through pinned memory; the value is checked against float64.
+    Tn = gpu.Tensor
+    ws, want = [], 0.0
+    for i, n in enumerate(sizes):
+        x = synth.normal(n + i, (n,), stream=i)
+        w = Tn.fromFloat32(np.zeros(n, np.float32), [n]).setRequiresGrad(True)
+        w.mul(Tn.fromFloat32(x, [n])).sum().backward()
+        ws.append(w)
+        want += float(np.sum(x.astype(np.float64) ** 2))
+    ids = [w._id for w in ws]
+    got = gpu.native.gradNorm(ids)
+    assert abs(got - np.sqrt(want)) <= 2e-7 * np.sqrt(want)
+    assert gpu.native.gradNorm(ids) == got          # the same sums in the same order
+    # a step without clipping returns the same norm (its update is queued before the host looks at the norm) and
+    # moves every parameter by lr (Adam's first step is lr * g / (|g| + eps))
+    opt = gpu.Adam([gpu.Parameter(w) for w in ws], lr=0.01)
+    assert opt.step() == got
+    assert all(np.mean(np.abs(w.numpy()) > 0.009) > 0.999 for w in ws)
+    # with clipping: the norm is read first, the gradients are scaled to the limit, then the update
+    assert opt.step(maxGradNorm=got / 4) == got
+    assert abs(gpu.native.gradNorm(ids) - got / 4) <= 1e-6 * got
+
+
 def test_cleared_gradients_read_as_zeros_and_accumulate_from_zero(gpu):
     # zeroGrad only marks a gradient; the zeros appear when it is read, and the first accumulation replaces them
     Tn = gpu.Tensor

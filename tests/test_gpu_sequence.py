@@ -195,9 +195,12 @@ def test_int_buffer_forms_equal_the_host_forms(both):
         gpu.crossEntropyLossGpu(_t(gpu, np.zeros((4, 50))), bad)
 
 
-@pytest.mark.parametrize("n,v", [(5, 3), (33, 512), (17, 516), (64, 2048), (9, 2050), (12, 4100), (40, 8192), (6, 8196), (3, 20000)])
+@pytest.mark.parametrize("n,v", [(5, 3), (33, 512), (17, 516), (64, 2048), (9, 2050), (12, 4100), (40, 8192), (6, 8196), (3, 20000),
+                                 (1, 2), (32, 3), (64, 3), (65, 3), (33, 496), (64, 256), (16, 1001), (2, 8190)])
 def test_cross_entropy_row_kernels_match_the_oracle(both, n, v):
-    # every row-kernel variant: scalar rows, rows cached in registers at two depths, a workgroup per row, long rows
+    # every row-kernel variant: scalar rows, rows cached in registers at two depths, a workgroup per row, long rows;
+    # from (1, 2) on, batches small enough for the single launch (rows and their mean by one workgroup) and
+    # their neighbours just outside it
     logits = synth.normal(n + v, (n, v)) * 3.0
     targets = [[int(t)] for t in np.random.default_rng(v).integers(0, v, size=n)]
     res = []

@@ -689,6 +689,33 @@ def test_pair_launch_of_small_and_of_big_products(dev, rocm, oracle_native):
     assert max_err(rocm.to_host(o3, (n, n)), big.T.astype(np.float64) @ big.astype(np.float64)) <= gemm_tol(n, big, big)
 
 
+@pytest.mark.parametrize("m,h,c", [(32, 64, 3), (32, 10, 64), (7, 5, 3), (128, 64, 64), (33, 257, 9)])
+def test_pair_of_tiny_products_is_one_launch_with_the_reference_sums(dev, rocm, oracle_native, m, h, c):
+    # the backward pair of a small Linear (x [m, h] . w [h, c]; dx = g . w^T, dw = x^T . g): products the tiny-product
+    # kernel takes go out as one launch, each output still the reference CPU arm's sum bit for bit
+    x = synth.normal(m, (m, h))
+    w = synth.normal(h, (h, c), stream=1)
+    g = synth.normal(c, (m, c), stream=2)
+    dX, dW, dG = dev.put(x), dev.put(w), dev.put(g)
+    ox, ow = dev.empty(m * h), dev.empty(h * c)
+    d0 = rocm.gemm_desc(m, h, c, dG, dW, ox, b_strides=(1, c))   # g . w^T
+    d1 = rocm.gemm_desc(h, c, m, dX, dG, ow, a_strides=(1, h))   # x^T . g
+    before = rocm.launch_count()
+    rocm.sgemm_pair(d0, d1)
+    assert rocm.launch_count() - before == 1
+    got0, got1 = rocm.to_host(ox, (m, h)), rocm.to_host(ow, (h, c))
+    assert np.array_equal(got0, oracle_native.sgemm_ikj(g, w.T.copy()))
+    assert np.array_equal(got1, oracle_native.sgemm_ikj(x.T.copy(), g))
+    # accumulate on one side, a bias on the other: the two products keep their own epilogues
+    bias = synth.normal(3, (c,), stream=3)
+    dBias = dev.put(bias)
+    d2 = rocm.gemm_desc(m, h, c, dG, dW, ox, b_strides=(1, c), accumulate=1)
+    d3 = rocm.gemm_desc(h, c, m, dX, dG, ow, a_strides=(1, h), bias=dBias, epilogue=N.EPI_BIAS)
+    rocm.sgemm_pair(d2, d3)
+    assert np.array_equal(rocm.to_host(ox, (m, h)), got0 + got0)
+    assert np.array_equal(rocm.to_host(ow, (h, c)), got1 + bias[None, :])
+
+
 def test_single_launch_skinny_path_is_available(rocm):
     # MI355X deals workgroups over its 8 XCDs round-robin; were the probe to fail,
     # ALGO_SKINNY would quietly run as ALGO_SKINNY_TWO_PASS and the tests below
