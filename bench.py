@@ -351,30 +351,42 @@ def bench_extras(r, with_cpu):
               w2=synth.uniform(0, (64, 3), -0.125, 0.125, stream=3), b2=synth.uniform(0, (3,), -0.125, 0.125, stream=4))
     targets = [[int(t)] for t in synth.integers(0, (32,), 0, 3, stream=5)]
 
-    def build1(a):
+    def build1(a, fused=False):
         x1 = T(c1["x"], False, a)
-        m1 = a.Linear(10, 64, weight=c1["w1"], bias=c1["b1"])
-        m2 = a.Linear(64, 3, weight=c1["w2"], bias=c1["b2"])
+        m1 = a.Linear(10, 64, weight=c1["w1"], bias=c1["b1"], fused=fused, activation="relu")
+        m2 = a.Linear(64, 3, weight=c1["w2"], bias=c1["b2"], fused=fused)
         ps = m1.parameters() + m2.parameters()
         opt = a.Adam(ps, lr=1e-3)
 
         def step():
             opt.zeroGrad()
-            a.crossEntropyLoss(m2.forward(m1.forward(x1).relu()), targets).backward()
+            a.crossEntropyLoss(m2.forward(m1.forward(x1)), targets).backward()
             opt.step()
 
         def keep():
             ids = [x1._id] + [p.value._id for p in ps]
             return ids + [g for g in (a.native.getGrad(p.value._id) for p in ps) if g is not None]
         return step, keep
-    step1, keep1 = build1(api)
-    ms, launches = time_step(step1, keep1, 20, 5)
-    out["config1_readme_mlp_step"] = {"ms": ms, "launches_per_step": launches,
-                                      "roofline": {"bound": "launch latency", "kernel": "%d kernel launches + 2 small copies per step" % launches,
-                                                   "us_per_launch": ms * 1e3 / max(launches, 1), "empty_launch_us": out["empty_launch_us"],
-                                                   "algorithmic_flops": 0.16e6, "frac": None,
-                                                   "note": "0.16 MFLOP and < 0.1 MB per step: neither roof applies; the step is the sum of its launch "
-                                                           "latencies and of the host's own work per op"}}
+    for fused in (False, True):
+        api.native.resetEngine()
+        step1, keep1 = build1(api, fused)
+        ms, launches = time_step(step1, keep1, 200, 20)
+        # the same steps without a wait after each: what a training loop that does not read the loss sees
+        r.sync()
+        t0 = time.perf_counter()
+        for _ in range(200):
+            step1()
+            api.native.gcTensors(keep1())
+        r.sync()
+        ms_loop = (time.perf_counter() - t0) / 200 * 1e3
+        out["config1_readme_mlp_step" + ("_fused_linear" if fused else "")] = {
+            "ms": ms, "ms_per_step_in_a_loop_of_200": ms_loop, "launches_per_step": launches,
+            "roofline": {"bound": "launch latency", "kernel": "%d kernel launches per step" % launches,
+                         "us_per_launch": ms * 1e3 / max(launches, 1), "empty_launch_us": out["empty_launch_us"],
+                         "algorithmic_flops": 0.16e6, "frac": None,
+                         "note": "0.16 MFLOP and < 0.1 MB per step: neither roof applies; the step is the sum of its launch "
+                                 "latencies and of the host's own work per op.  ms: each step followed by a wait for the device"}}
+    api.native.resetEngine()
     if with_cpu:
         orc = oracle_api()
         so, ko = build1(orc)

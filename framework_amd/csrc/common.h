@@ -170,8 +170,10 @@ int k_expand_dim(float *out, const float *g, int64_t outer, int64_t dim, int64_t
 int k_unbroadcast(float *out, const float *g, const int64_t *gshape, int gnd, const int64_t *oshape, int ond);
 // targets: device buffer of n values.  targets_host: null when `targets` already holds them; otherwise the values
 // (each in [0, v)), which the call brings to `targets` itself.
+// grad_for_one (may be null): n * v floats; a small batch's launch also leaves there the gradient of the logits for
+// an upstream gradient of exactly one, and *wrote_grad says whether it did.
 int k_cross_entropy(float *loss, float *softmax, const float *logits, int32_t *targets, const int32_t *targets_host,
-                    int64_t n, int64_t v);
+                    int64_t n, int64_t v, float *grad_for_one = nullptr, bool *wrote_grad = nullptr);
 int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t *targets,
                              const float *grad_scalar, int64_t n, int64_t v);
 int k_bias_gelu(float *out, const float *x, const float *bias, int64_t rows, int64_t cols);

@@ -946,8 +946,11 @@ int k_unbroadcast(float *out, const float *g, const int64_t *gshape, int gnd, co
 // src/native/src/ops/loss.rs:24-67: per row max, exp, normalise, -ln p[target];
 // loss = mean over rows.  One wavefront per row; the row losses are summed by
 // a single wavefront in a fixed order.
+// dl (may be null): the row's gradient for an upstream gradient of one, (p - onehot) * dl_scale, as ce_bwd_kernel
+// would compute it with scale = 1 / rows.
 __device__ __forceinline__ float ce_row(float *__restrict__ sm, const float *__restrict__ logits, const int32_t t,
-                                        const int64_t row, const int lane, const int64_t v) {
+                                        const int64_t row, const int lane, const int64_t v, float *__restrict__ dl = nullptr,
+                                        const float dl_scale = 0.f) {
     const float *x = logits + row * v;
     float *p = sm + row * v;
     float mx = -INFINITY;
@@ -962,7 +965,11 @@ __device__ __forceinline__ float ce_row(float *__restrict__ sm, const float *__r
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-    for (int64_t j = lane; j < v; j += 64) p[j] = p[j] / sum;
+    for (int64_t j = lane; j < v; j += 64) {
+        const float q = p[j] / sum;
+        p[j] = q;
+        if (dl) dl[row * v + j] = (j == t ? q - 1.0f : q) * dl_scale;
+    }
     const float e = expf(x[t] - mx);
     return -logf(e / sum);  // the row's loss (every lane holds it)
 }
@@ -978,7 +985,8 @@ __global__ void ce_rows_kernel(float *__restrict__ row_loss, float *__restrict__
 // logits are read once and the probabilities written once.
 template <int NV>
 __device__ __forceinline__ float ce_row_cached(float *__restrict__ sm, const float *__restrict__ logits, const int32_t t,
-                                               const int64_t row, const int lane, const int64_t v) {
+                                               const int64_t row, const int lane, const int64_t v, float *__restrict__ dl = nullptr,
+                                               const float dl_scale = 0.f) {
     const int64_t v4 = v >> 2;
     const float4 *x = reinterpret_cast<const float4 *>(logits + row * v);
     float4 *p = reinterpret_cast<float4 *>(sm + row * v);
@@ -1006,7 +1014,16 @@ __device__ __forceinline__ float ce_row_cached(float *__restrict__ sm, const flo
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int64_t j = lane + 64 * i;
-        if (j < v4) p[j] = make_float4(r[i].x / sum, r[i].y / sum, r[i].z / sum, r[i].w / sum);
+        if (j < v4) {
+            const float4 q = make_float4(r[i].x / sum, r[i].y / sum, r[i].z / sum, r[i].w / sum);
+            p[j] = q;
+            if (dl) {
+                const int64_t c = 4 * j;
+                reinterpret_cast<float4 *>(dl + row * v)[j] =
+                    make_float4((c == t ? q.x - 1.0f : q.x) * dl_scale, (c + 1 == t ? q.y - 1.0f : q.y) * dl_scale,
+                                (c + 2 == t ? q.z - 1.0f : q.z) * dl_scale, (c + 3 == t ? q.w - 1.0f : q.w) * dl_scale);
+            }
+        }
     }
     const float e = expf(logits[row * v + t] - mx);
     return -logf(e / sum);
@@ -1090,14 +1107,15 @@ struct CeTargets {
 };
 template <int NV, bool EMBED>  // NV 0: ce_row, else ce_row_cached<NV>
 __global__ __launch_bounds__(1024) void ce_small_kernel(float *__restrict__ loss, float *__restrict__ sm, const float *__restrict__ logits,
-                                                        int32_t *__restrict__ targets, int n, int64_t v, const CeTargets given) {
+                                                        int32_t *__restrict__ targets, int n, int64_t v, float *__restrict__ dl,
+                                                        const CeTargets given) {
     __shared__ float row_loss[CE_SMALL_ROWS];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int row = wave; row < n; row += 16) {
         const int32_t t = EMBED ? given.t[row] : targets[row];
         float l;
-        if constexpr (NV == 0) l = ce_row(sm, logits, t, row, lane, v);
-        else l = ce_row_cached<NV>(sm, logits, t, row, lane, v);
+        if constexpr (NV == 0) l = ce_row(sm, logits, t, row, lane, v, dl, 1.0f / (float)n);
+        else l = ce_row_cached<NV>(sm, logits, t, row, lane, v, dl, 1.0f / (float)n);
         if (lane == 0) {
             row_loss[row] = l;
             if (EMBED) targets[row] = t;
@@ -1113,7 +1131,11 @@ __global__ __launch_bounds__(1024) void ce_small_kernel(float *__restrict__ loss
 }
 // targets: device buffer of n values.  targets_host: null when `targets` already holds them; otherwise the
 // values, which this call brings to `targets` (checked by the caller to lie in [0, v)).
-int k_cross_entropy(float *loss, float *softmax, const float *logits, int32_t *targets, const int32_t *targets_host, int64_t n, int64_t v) {
+// grad_for_one (may be null): n * v floats; a small batch's launch also leaves there the gradient of the logits
+// for an upstream gradient of exactly one (what backward() of the loss itself asks for), and *wrote_grad says so.
+int k_cross_entropy(float *loss, float *softmax, const float *logits, int32_t *targets, const int32_t *targets_host, int64_t n, int64_t v,
+                    float *grad_for_one, bool *wrote_grad) {
+    if (wrote_grad) *wrote_grad = false;
     MNI_TRY(ensure_init());
     if (n <= 0 || v <= 0) return set_error(MNI_ERR_INVALID, "cross_entropy: empty logits");
     const bool vec = (v % 4) == 0 && al16(logits) && al16(softmax);
@@ -1123,10 +1145,12 @@ int k_cross_entropy(float *loss, float *softmax, const float *logits, int32_t *t
         if (targets_host) memcpy(given.t, targets_host, (size_t)n * sizeof(int32_t));
         const dim3 grid(1), block(1024);
         hipStream_t st = ctx().stream;
-        if (vec && targets_host) MNI_KERNEL_LAUNCH((ce_small_kernel<2, true>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, given);
-        else if (vec) MNI_KERNEL_LAUNCH((ce_small_kernel<2, false>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, given);
-        else if (targets_host) MNI_KERNEL_LAUNCH((ce_small_kernel<0, true>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, given);
-        else MNI_KERNEL_LAUNCH((ce_small_kernel<0, false>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, given);
+        float *dl = wrote_grad && (!vec || al16(grad_for_one)) ? grad_for_one : nullptr;
+        if (dl) *wrote_grad = true;
+        if (vec && targets_host) MNI_KERNEL_LAUNCH((ce_small_kernel<2, true>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, dl, given);
+        else if (vec) MNI_KERNEL_LAUNCH((ce_small_kernel<2, false>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, dl, given);
+        else if (targets_host) MNI_KERNEL_LAUNCH((ce_small_kernel<0, true>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, dl, given);
+        else MNI_KERNEL_LAUNCH((ce_small_kernel<0, false>), grid, block, 0, st, loss, softmax, logits, targets, (int)n, v, dl, given);
         return check_launch("ce_small");
     }
     if (targets_host) MNI_TRY(upload_small(targets, targets_host, (size_t)n * sizeof(int32_t)));

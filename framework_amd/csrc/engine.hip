@@ -80,6 +80,7 @@ struct Entry {
     uint32_t aux2 = MNI_BAD_ID; // attention log-sum-exp
     uint32_t aux3 = MNI_BAD_ID; // residual + layernorm: the saved sum x + residual
     std::shared_ptr<void> targets;  // device int32 targets / embedding indices
+    BufP ce_grad_for_one;           // cross-entropy of a small batch: d loss / d logits, computed with the loss
     int64_t ce_n = 0, ce_v = 0;
     uint64_t rng_seed = 0, rng_offset = 0;  // dropout: where its mask starts in the random stream
 };
@@ -864,12 +865,17 @@ static uint32_t cross_entropy_op(uint32_t logits, const int64_t *targets, size_t
     BufP sm = x ? new_buf((size_t)(n * v)) : nullptr;
     BufP loss = sm ? new_buf(1) : nullptr;
     if (!loss) return MNI_BAD_ID;
-    if (k_cross_entropy(loss->p, sm->p, x->p, (int32_t *)tp, t32.data(), n, v) != MNI_OK) return MNI_BAD_ID;
+    // (a loss that is differentiated is nearly always the root of backward(): its small-batch kernel writes the
+    // gradient for that case while it holds the probabilities)
+    BufP dl = eng().tape.enabled && n * v <= 16384 ? new_buf((size_t)(n * v)) : nullptr;
+    bool wrote = false;
+    if (k_cross_entropy(loss->p, sm->p, x->p, (int32_t *)tp, t32.data(), n, v, dl ? dl->p : nullptr, &wrote) != MNI_OK) return MNI_BAD_ID;
     const uint32_t loss_id = insert_contig(std::move(loss), Shape{1});
     const uint32_t sm_id = insert_contig(std::move(sm), shape);
     Entry e;
     e.op = OP_CROSSENTROPY; e.output_id = loss_id; e.n_inputs = 1; e.inputs[0] = logits;
     e.aux = sm_id; e.targets = tdev; e.ce_n = n; e.ce_v = v;
+    if (wrote) e.ce_grad_for_one = std::move(dl);
     eng().tape.record(std::move(e));
     return loss_id;
 }
@@ -878,6 +884,10 @@ static int cross_entropy_backward(uint32_t grad, const Entry &e, int64_t *out) {
     Tensor *G = get(grad), *S = get(e.aux);
     if (!G || !S) return MNI_ERR_FREED;
     const Shape shape = S->shape;
+    if (e.ce_grad_for_one && eng().one && G->buf == eng().one) {  // the upstream gradient is the constant 1.0
+        out[0] = insert_contig(BufP(e.ce_grad_for_one), shape);
+        return MNI_OK;
+    }
     BufP o = new_buf((size_t)(e.ce_n * e.ce_v));
     if (!o) return MNI_ERR_NOMEM;
     MNI_TRY(k_cross_entropy_backward(o->p, S->buf->p, (const int32_t *)e.targets.get(), G->buf->p, e.ce_n, e.ce_v));

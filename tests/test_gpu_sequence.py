@@ -211,6 +211,14 @@ def test_cross_entropy_row_kernels_match_the_oracle(both, n, v):
         res.append((loss.item(), lg.grad.numpy()))
     assert abs(res[0][0] - res[1][0]) < 4e-6 * abs(res[1][0])
     assert max_err(res[0][1], res[1][1]) < 4e-6 * float(np.abs(res[1][1]).max())   # the row sum runs in another order
+    # backward() from the loss itself (a small batch's gradient for that case is written by the forward launch)
+    direct = []
+    for api in both:
+        lg = _t(api, logits, True)
+        api.crossEntropyLoss(lg, targets).backward()
+        direct.append(lg.grad.numpy())
+    assert max_err(direct[0], direct[1]) < 4e-6 * float(np.abs(direct[1]).max())
+    assert max_err(direct[0] * np.float32(3.0), res[0][1]) < 1e-6 * float(np.abs(res[0][1]).max())
     lp = logits.astype(np.float64)
     want = np.mean(np.log(np.exp(lp - lp.max(1, keepdims=True)).sum(1)) + lp.max(1) - lp[np.arange(n), [t[0] for t in targets]])
     assert abs(res[0][0] - want) < 1e-5 * abs(want)
