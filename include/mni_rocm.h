@@ -66,7 +66,12 @@ int mni_rocm_malloc(void **ptr, size_t bytes);
 int mni_rocm_free(void *ptr);
 int mni_rocm_clear_cache(void);
 /* Copies.  h2d/d2h synchronise the stream before returning (the reference's
- * memcpy_stod / memcpy_dtov, src/native/src/tensor.rs:364-387,460-469). */
+ * memcpy_stod / memcpy_dtov, src/native/src/tensor.rs:364-387,460-469).
+ * mni_rocm_sync, and mni_rocm_d2h of up to 16 KB, wait by queueing a small
+ * kernel that writes a tag (and the data) to pinned host memory and watching
+ * for it for up to 150 us, then fall back on hipStreamSynchronize: a wait
+ * ends a few microseconds after the last kernel, and spins for that long at
+ * most. */
 int mni_rocm_h2d(void *dst, const void *src, size_t bytes);
 int mni_rocm_d2h(void *dst, const void *src, size_t bytes);
 int mni_rocm_d2d(void *dst, const void *src, size_t bytes);
@@ -181,7 +186,9 @@ size_t mni_rocm_sgemm_noalloc_workspace_bytes(void);
  * dB = A^T * dC), which the reference issues one after the other.  When each
  * product alone is a batch of about one 64 x 64 tile per compute unit, both
  * run in one launch (every SIMD gets a second wavefront; one ramp-up, one
- * tail); otherwise this is mni_rocm_sgemm(first) followed by
+ * tail); so do two products of a few thousand outputs each (what
+ * MNI_ALGO_AUTO gives to the tiny-product kernel: the gradients of a small
+ * Linear); otherwise this is mni_rocm_sgemm(first) followed by
  * mni_rocm_sgemm(second).  The results are those of the separate calls bit
  * for bit. */
 int mni_rocm_sgemm_pair(const mni_gemm_desc *first, const mni_gemm_desc *second);
