@@ -19,7 +19,9 @@
 //      so that one 16-byte LDS read hands a lane the four K values it feeds to
 //      four consecutive MFMAs (lane = row % 32 + 32 (k / 4 % 2));
 //   3. each wavefront pulls its 64 + 64 rows of operand fragments into
-//      registers (the panels are dead after that and LDS is reused);
+//      registers (the panels are dead after that and LDS is reused); steps
+//      2 and 3 run in two halves, the rows of every wavefront's first block
+//      first, so that its MFMAs start when half the pieces have arrived;
 //   4. its four 32 x 32 blocks are computed one after the other, all of K per
 //      block, and while the matrix pipe runs block b + 1 the accumulators of
 //      block b go through a wavefront-private LDS patch (the MFMA layout holds
@@ -79,35 +81,55 @@ __global__ __launch_bounds__(256, 2) void gemm_panel_kernel(const GemmLaunch g) 
     const float *Ab = g.A + (int64_t)(batch % g.a_bcount) * g.a_bs;
     const float *Bb = g.B + (int64_t)(batch % g.b_bcount) * g.b_bs;
     const int kq = g.K >> 2;
+    // The pieces are requested in two halves, rows {0..31, 64..95} of both panels first: those are the rows of
+    // every wavefront's first block (rows 64 wm + 0..31 of A against rows 64 wn + 0..31 of B), whose MFMAs then
+    // run while the other half is still on its way.  Piece x of a thread is row tid / KQ + (256 / KQ) order[x].
+    constexpr int HALF = PER_THREAD / 2;
+    constexpr int ROWS_PER_PASS = 256 / KQ;  // 16 (K <= 64) or 32 (K <= 32)
+    auto piece_row = [&](int x) {
+        // PER_THREAD 8: passes of 16 rows in the order 0 1 4 5 | 2 3 6 7; PER_THREAD 4: passes of 32 rows, 0 2 | 1 3
+        const int pass = PER_THREAD == 8 ? ((x & 4) ? (x & 1) + 2 + ((x & 2) << 1) : (x & 1) + ((x & 2) << 1)) : ((x & 1) << 1) + (x >> 1);
+        return tid / KQ + ROWS_PER_PASS * pass;
+    };
     f32x4 va[PER_THREAD], vb[PER_THREAD];
 #pragma unroll
     for (int x = 0; x < PER_THREAD; ++x) {
-        const int f = tid + 256 * x;
-        const int row = f / KQ, q = f % KQ;
+        const int row = piece_row(x), q = tid % KQ;
         const bool ok = KQ * 4 == 64 && g.K == 64 ? true : q < kq;
         const float *pa = Ab + (int64_t)min(m0 + row, g.M - 1) * g.a_rs + 4 * q;   // op(A)(m, k): a_cs == 1
         const float *pb = Bb + (int64_t)min(n0 + row, g.N - 1) * g.b_cs + 4 * q;   // op(B)(k, n): b_rs == 1
         va[x] = ok ? *reinterpret_cast<const f32x4 *>(pa) : f32x4{0.f, 0.f, 0.f, 0.f};
         vb[x] = ok ? *reinterpret_cast<const f32x4 *>(pb) : f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    // ---- 2. panels to LDS ------------------------------------------------------------
-#pragma unroll
-    for (int x = 0; x < PER_THREAD; ++x) {
-        const int f = tid + 256 * x;
-        const int row = f / KQ, q = f % KQ;
-        As[q * PSLICE + row] = va[x];
-        Bs[q * PSLICE + row] = vb[x];
-    }
-    __syncthreads();
-    // ---- 3. this wavefront's fragments: rows 64 wm + 32 a + i of A, 64 wn + 32 q + i of B ------
+    // ---- 2. the first half to LDS, and this wavefront's fragments of it ---------------------------
+    // fragments: rows 64 wm + 32 a + i of A, 64 wn + 32 q + i of B
     f32x4 fa[2][NCH], fb[2][NCH];
+    auto stage = [&](int half) {
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+        for (int x = half * HALF; x < (half + 1) * HALF; ++x) {
+            const int row = piece_row(x), q = tid % KQ;
+            As[q * PSLICE + row] = va[x];
+            Bs[q * PSLICE + row] = vb[x];
+        }
+        __syncthreads();
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            fa[a][c] = As[(2 * c + h) * PSLICE + 64 * wm + 32 * a + i];
-            fb[a][c] = Bs[(2 * c + h) * PSLICE + 64 * wn + 32 * a + i];
+            fa[half][c] = As[(2 * c + h) * PSLICE + 64 * wm + 32 * half + i];
+            fb[half][c] = Bs[(2 * c + h) * PSLICE + 64 * wn + 32 * half + i];
         }
+    };
+    stage(0);
+    __builtin_amdgcn_sched_barrier(0);
+    floatx16 acc[2];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[0][e] = 0.0f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(pk_pick(fa[0][c], j), pk_pick(fb[0][c], j), acc[0], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- 3. the second half, behind the first block's MFMAs ------------------------------------------
+    stage(1);
     __syncthreads();  // the panels are dead: LDS now holds the wavefronts' patches
 
     // ---- 4. block by block, stores of one block under the MFMAs of the next -------------
@@ -121,7 +143,6 @@ __global__ __launch_bounds__(256, 2) void gemm_panel_kernel(const GemmLaunch g) 
     // else the wavefront has to do is placed in the gaps between the MFMAs of the NEXT block: the 16
     // patch writes of the block just finished, then the 4 patch reads, then the 4 global stores.
     // Two accumulators alternate.  sched_barrier pins the order.
-    floatx16 acc[2];
     f32x4 pv[4];  // patch rows on their way to memory
     // lane (i, h) holds column i, rows 8 (e / 4) + 4 h + e % 4 of the block
     auto patch_write = [&](const floatx16 &d, int e) { patch[(8 * (e >> 2) + 4 * h + (e & 3)) * PPITCH + i] = d[e]; };
@@ -160,12 +181,6 @@ __global__ __launch_bounds__(256, 2) void gemm_panel_kernel(const GemmLaunch g) 
     constexpr int NM = 4 * NCH;  // MFMAs per block (16 or 32)
     // what goes behind MFMA t of the next block (NM = 32: writes at t = 0..15, reads 18..21, stores 24..27;
     // NM = 16: a write behind every MFMA, reads and stores after the block)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) acc[0][e] = 0.0f;
-#pragma unroll
-    for (int c = 0; c < NCH; ++c)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(pk_pick(fa[0][c], j), pk_pick(fb[0][c], j), acc[0], 0, 0, 0);
     auto blocks = [&](auto fast) {
 #pragma unroll
     for (int blk = 0; blk < 4; ++blk) {
