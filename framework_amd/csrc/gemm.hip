@@ -219,6 +219,34 @@ struct PlanProbe {
     GemmLaunch g;  // kind TILE: the launch descriptor, complete
 };
 
+// K slices for a product of `tiles` 64 x 64 tiles (at most one per CU) of `ktiles` K steps each.
+// Estimated microseconds of a plan with s slices:
+//   (per_cu (steps + 3) + 3) c  +  [s > 1]  (2.5 + 2 s out_bytes / 5 TB/s)
+// per_cu = workgroups on the fullest CU, steps = K steps per slice, c = 0.55 us per K step of a workgroup that
+// has its CU to itself and 0.48 when several share one (they cover each other's barriers and LDS round trips);
+// three steps' worth of prologue and epilogue per workgroup and per launch; the reduction pass costs a launch
+// and reads what the slices wrote.  Fitted to, and within 10 % of, 60 measured plans: M = 24..384 against
+// (N, K) = (4096, 4096), (4096, 1024), (1024, 4096), (11008, 4096), (4096, 11008), s = 1..16; e.g.
+// 64 x 4096 x 4096: s = 1, 2, 4, 8, 16 measured 68.0 / 40.2 / 25.4 / 26.7 / 30.5 us, estimated 73.7 / 41.8 / 25.1 /
+// 25.6 / 31.8.  The smallest s within 3 % of the best estimate wins; slices keep at least 8 K steps.
+static int split_for_few_tiles(int64_t tiles, int ktiles, int cus, int64_t out_bytes) {
+    static const int cand[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
+    double best = 0.0;
+    int best_s = 1;
+    for (int s : cand) {
+        if (s > 1 && ktiles / s < 8) break;
+        const int64_t per_cu = (tiles * s + cus - 1) / cus;
+        const int steps = (ktiles + s - 1) / s;
+        double t = ((double)per_cu * (steps + 3) + 3) * (per_cu > 1 ? 0.48 : 0.55);
+        if (s > 1) t += 2.5 + 2.0 * s * (double)out_bytes / 5.0e6;
+        if (s == 1 || t < best * 0.97) {
+            best = t;
+            best_s = s;
+        }
+    }
+    return best_s;
+}
+
 static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
     GemmLaunch g;
     fill_launch(g, d);
@@ -297,6 +325,7 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
     int bm = g.M <= 64 ? 64 : 128, bn = g.N <= 64 ? 64 : 128;
     bool streamk = false;
     bool whole_tiles = false;  // one workgroup per tile, no K slices
+    int planned_split = 0;     // K slices chosen by the planner (0: by the slot rule further down)
     // The two-output and the gelu'-scaling epilogues exist in the one-workgroup-per-tile form only;
     // strip sums for the bias gradient are laid out for 128-row tiles.
     const bool fused_gelu = d.epilogue >= MNI_EPI_BIAS_GELU_DUAL;
@@ -341,20 +370,24 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
             if (long_k && big_tiles >= big_slots) {
                 // more big tiles than workgroup slots and plenty of K steps per slot: stream-K over big tiles
                 streamk = streamk_fits(bm, bn, 8);
-            } else if (long_k && big_tiles * 16 < 3 * big_slots && ((int64_t)g.M + g.N) * g.K * 4 > (128LL << 20)) {
+            } else if (long_k && ktiles >= 512 && big_tiles * 16 < 3 * big_slots && ((int64_t)g.M + g.N) * g.K * 4 > (128LL << 20)) {
                 // A handful of big tiles over a K so long that the operands outgrow the Infinity Cache:
                 // 64 x 64 tiles would stream them twice as often (1024 x 1024 x 65536: 1127 us against
                 // 1015 us for 128 x 128 tiles in K slices, the plan below)
             } else {
                 const int64_t tiles64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) * g.batch;
-                if (tiles64 <= cus || (tiles64 <= 2LL * cus && ktiles <= 32)) {
-                    // At most one 64 x 64 tile per CU (or two, of a short K): one workgroup per tile and all of K
-                    // when at least half the CUs get one -- splitting K to fill the other workgroup slots costs a
-                    // reduction pass and gains nothing (32 x (512 x 64 x 512): 13.7 us whole, 19.0 in two K slices,
-                    // 19.8 stream-K; 40 batches, 1.25 tiles per CU: 20.6 whole, 27.5 stream-K) -- and K slices
-                    // below when fewer do (8 batches: 11.8 in two slices, 12.9 whole).
+                if (tiles64 <= cus) {
+                    // At most one 64 x 64 tile per CU: K slices by the cost model of split_for_few_tiles (one
+                    // slice, i.e. no reduction pass, wins for short K: 32 x (512 x 64 x 512) 13.7 us whole, 19.0 in
+                    // two K slices, 19.8 stream-K; several for long K: 128 x 4096 x 4096 69.6 us whole, 40.1 in four).
                     bm = bn = 64;
-                    whole_tiles = tiles64 * 2 >= cus;
+                    planned_split = split_for_few_tiles(tiles64, ktiles, cus, (int64_t)g.M * g.N * g.batch * 4);
+                    whole_tiles = planned_split == 1;
+                } else if (tiles64 <= 2LL * cus && ktiles <= 32) {
+                    // up to two per CU, of a short K: one workgroup per tile (40 batches of the product above,
+                    // 1.25 tiles per CU: 20.6 us whole, 27.5 stream-K)
+                    bm = bn = 64;
+                    whole_tiles = true;
                 } else {
                     streamk = streamk_fits(64, 64, 8);
                     if (streamk) bm = bn = 64;
@@ -405,7 +438,7 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
 
     // Split K when the output tiles alone cannot fill the machine (two
     // workgroups fit on each CU).  Slices are whole K steps.
-    int split = whole_tiles ? 1 : d.split_k;
+    int split = whole_tiles ? 1 : (planned_split > 0 && d.split_k == 0 ? planned_split : d.split_k);
     if (split == 0) {
         const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n * g.batch;
         const int64_t slots = (bm * bn >= 128 * 128 ? 2LL : 4LL) * cus;

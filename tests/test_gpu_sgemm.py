@@ -689,6 +689,22 @@ def test_pair_launch_of_small_and_of_big_products(dev, rocm, oracle_native):
     assert max_err(rocm.to_host(o3, (n, n)), big.T.astype(np.float64) @ big.astype(np.float64)) <= gemm_tol(n, big, big)
 
 
+@pytest.mark.parametrize("m,n,k", [(24, 4096, 4096), (96, 4096, 4096), (128, 1024, 4096), (192, 4096, 1024), (48, 11008, 1024), (64, 512, 16384),
+                                   (200, 1000, 3000)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+def test_products_of_few_tiles_in_planned_k_slices_integer_exact(dev, rocm, m, n, k, ta, tb):
+    # 17 to a few hundred rows against a large operand: fewer 64 x 64 tiles than CUs, so the planner's cost model
+    # picks the number of K slices (1 to 16 over these shapes); whatever it picks, the sums are exact and the
+    # launches are the product and at most one reduction
+    a = synth.small_ints(m + k, (k, m) if ta else (m, k), 3)
+    b = synth.small_ints(n + k, (n, k) if tb else (k, n), 3, stream=1)
+    want = ((a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(np.float32)
+    before = rocm.launch_count()
+    got = run_gemm(dev, a, b, ta, tb)[0]
+    assert np.array_equal(got, want)
+    assert rocm.launch_count() - before <= 3   # (the output buffer's fill, the product, the reduction)
+
+
 @pytest.mark.parametrize("m,h,c", [(32, 64, 3), (32, 10, 64), (7, 5, 3), (128, 64, 64), (33, 257, 9)])
 def test_pair_of_tiny_products_is_one_launch_with_the_reference_sums(dev, rocm, oracle_native, m, h, c):
     # the backward pair of a small Linear (x [m, h] . w [h, c]; dx = g . w^T, dw = x^T . g): products the tiny-product
