@@ -44,6 +44,9 @@ struct DeviceCtx {
     // launch marks them with a fresh epoch so they never need clearing.
     unsigned *skinny_flags = nullptr;
     size_t skinny_flag_cap = 0;  // entries
+    // Arrival counters of the few-rows kernel's K slices, one per (batch, column group); zero between launches.
+    unsigned *fewrows_counters = nullptr;
+    size_t fewrows_counter_cap = 0;
     unsigned skinny_epoch = 0;
     // Device status word in pinned host memory that kernels can write: a kernel
     // whose bounded wait for another workgroup expires stores a DEVICE_STATUS_*

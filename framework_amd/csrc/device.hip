@@ -104,6 +104,9 @@ static int init_device(int device) {
     MNI_HIP_CHECK(hipMalloc((void **)&c.skinny_flags, c.skinny_flag_cap * sizeof(unsigned)));
     MNI_HIP_CHECK(hipMemset(c.skinny_flags, 0, c.skinny_flag_cap * sizeof(unsigned)));
     c.skinny_epoch = 0;
+    c.fewrows_counter_cap = 4096;
+    MNI_HIP_CHECK(hipMalloc((void **)&c.fewrows_counters, c.fewrows_counter_cap * sizeof(unsigned)));
+    MNI_HIP_CHECK(hipMemset(c.fewrows_counters, 0, c.fewrows_counter_cap * sizeof(unsigned)));
     // Pinned staging slots of upload_small, and one event per slot that says when its transfer has left it.
     MNI_HIP_CHECK(hipHostMalloc((void **)&c.stage_host, DeviceCtx::STAGE_SLOTS * DeviceCtx::STAGE_BYTES, hipHostMallocDefault));
     for (int i = 0; i < DeviceCtx::STAGE_SLOTS; ++i) MNI_HIP_CHECK(hipEventCreateWithFlags(&c.stage_done[i], hipEventDisableTiming));

@@ -43,7 +43,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_TINY)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_FEWROWS)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -137,8 +137,18 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
             // rows are whole 128-byte lines, so that no line is shared by two units.
             DeviceCtx &c = ctx();
             const int64_t flag_count = (int64_t)groups * s.batch * split;
-            const bool fused = split > 1 && d.algo != MNI_ALGO_SKINNY_TWO_PASS && c.xcd_count > 0 && c.skinny_flags &&
-                               flag_count <= (int64_t)c.skinny_flag_cap;
+            bool fused = split > 1 && d.algo != MNI_ALGO_SKINNY_TWO_PASS && c.xcd_count > 0 && c.skinny_flags &&
+                         flag_count <= (int64_t)c.skinny_flag_cap;
+            if (fused) {
+                // The reducers of a unit (the workgroups of its last min(rows, slices) slices) wait for all of its
+                // slices while they hold their places on the CUs: every reducer of an XCD must fit on it at once,
+                // or the first ones could fill it and wait for slices that are never dispatched.
+                const int cus = c.compute_units > 0 ? c.compute_units : 256;
+                const int64_t units_per_xcd = ((int64_t)groups * s.batch + c.xcd_count - 1) / c.xcd_count;
+                const int64_t reducers_per_xcd = units_per_xcd * (s.rows < split ? s.rows : split);
+                const int64_t room_per_xcd = (int64_t)skinny_cols_fused_occupancy(s) * (cus / c.xcd_count);
+                fused = reducers_per_xcd <= room_per_xcd;
+            }
             void *ws = nullptr;
             if (split > 1) {
                 const size_t bytes = (size_t)split * s.batch * s.rows * skinny_ws_pitch(s.cols, fused) * sizeof(float);
@@ -214,10 +224,29 @@ static void fill_launch(GemmLaunch &g, const mni_gemm_desc &d) {
 
 // What run_mfma would launch for a product, for a caller that wants to know before anything is launched.
 struct PlanProbe {
-    enum { TILE = 0, PANEL = 1, DIRECT = 2, TILE_FUSED_GELU = 3, TILE_STREAMK = 4 };
+    enum { TILE = 0, PANEL = 1, DIRECT = 2, TILE_FUSED_GELU = 3, TILE_STREAMK = 4, FEWROWS = 5 };
     int kind, bm, bn, split, amode, bmode;
     GemmLaunch g;  // kind TILE: the launch descriptor, complete
 };
+
+// K slices of the few-rows kernel: one workgroup per CU (more gain nothing: with one, the loop already runs close
+// to both the memory system's and the matrix pipe's rate), slices of at least 128 K values (four blocks per
+// wavefront), at most 32 of them (the last workgroup of a column group adds them up).  Measured against every
+// other count on 19 (N, K) pairs from 512 x 512 to 50304 x 768: within 10 % of the best everywhere.
+static int fewrows_split(const GemmLaunch &g, int cus) {
+    const int64_t groups = (int64_t)((g.N + 127) / 128) * g.batch;
+    int64_t split = cus / groups;
+    if (split > g.K / 128) split = g.K / 128;
+    if (split > 32) split = 32;
+    return split < 1 ? 1 : (int)split;
+}
+// Whether the few-rows kernel is the plan for an eligible product: from about 512 x 512 of W on it is ahead of the
+// tile kernel's 64 x 64 tiles in K slices (us, 32 rows: 512 x 512 7.8 / 15.1, 1024 x 1024 8.8 / 11.7, 4096 x 4096
+// 19.1 / 24.4, 8192 x 8192 46.6 / 70.4, 50304 x 768 35.0 / 50.4, 1024 x 16384 24.3 / 29.7); below, and for short K, not.
+static bool fewrows_plan(const GemmLaunch &g, int cus) {
+    (void)cus;
+    return g.K >= 256 && (int64_t)g.N * g.K >= (1 << 18);
+}
 
 // K slices for a product of `tiles` 64 x 64 tiles (at most one per CU) of `ktiles` K steps each.
 // Estimated microseconds of a plan with s slices:
@@ -274,6 +303,38 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
         g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
         if (probe) { probe->kind = PlanProbe::PANEL; return MNI_OK; }
         return launch_gemm_panel(g, amode, bmode);
+    }
+    // Few-rows form (17 to 32 rows against a wide N-contiguous operand): forced, or chosen by fewrows_plan.
+    {
+        // (its K slices meet in one XCD's L2: the workgroup-to-XCD mapping must be the confirmed round-robin over 8)
+        const bool fr_ok = gemm_fewrows_eligible(g, amode, bmode) && (size_t)((g.N + 127) / 128) * g.batch <= c.fewrows_counter_cap && c.xcd_count == 8;
+        int fr_split = 0;
+        if (d.algo == MNI_ALGO_FEWROWS) {
+            if (!fr_ok)
+                return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel takes 17 to 32 rows of a K-contiguous A against an N-contiguous B, "
+                                                  "K %% 8 == 0, N %% 4 == 0, 16-byte aligned");
+            fr_split = d.split_k > 0 ? d.split_k : fewrows_split(g, cus);
+        } else if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && fr_ok && fewrows_plan(g, cus)) {
+            fr_split = fewrows_split(g, cus);
+        }
+        if (fr_split > 0) {
+            g.tiles_m = 1;
+            g.tiles_n = (g.N + 127) / 128;
+            const int per = ((g.K + fr_split - 1) / fr_split + 31) / 32 * 32;
+            g.k_per_slice = per;
+            g.split_k = (g.K + per - 1) / per;
+            g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_epoch = 0; g.status = c.status_dev;
+            g.sk_flags = c.fewrows_counters;
+            if (probe) { probe->kind = PlanProbe::FEWROWS; return MNI_OK; }
+            void *fws = nullptr;
+            if (g.split_k > 1) {
+                MNI_TRY(gemm_ws_alloc(&fws, (size_t)g.split_k * g.batch * g.M * g.N * sizeof(float)));
+                g.ws = (float *)fws;
+            }
+            const int rc = launch_gemm_fewrows(g, amode, bmode);
+            gemm_ws_free(fws);
+            return rc;
+        }
     }
     // Register-direct form: forced, or chosen for batched products of many small tiles.
     {

@@ -62,6 +62,12 @@ int launch_gemm_direct(const GemmLaunch &g, int amode, int bmode, int ksplit);
 bool gemm_tiny_eligible(const GemmLaunch &g);
 int launch_gemm_tiny(const GemmLaunch &g);
 int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1);  // two eligible, independent products in one launch
+// 17 to 32 rows of a K-contiguous A against a wide N-contiguous B, both straight into MFMA registers (gemm_fewrows.hip):
+// g.tiles_n counts column groups of 128, g.split_k K slices of g.k_per_slice (a multiple of 32).  With split_k > 1:
+// partials [slice][batch][M][N] in g.ws and one counter per (batch, column group) in g.sk_flags, zero between launches
+// (the workgroup that completes a count adds the slices up and returns the counter to zero).
+bool gemm_fewrows_eligible(const GemmLaunch &g, int amode, int bmode);
+int launch_gemm_fewrows(const GemmLaunch &g, int amode, int bmode);
 // Short-K form for two K-contiguous operands (gemm_panel.hip): 128 x 128 tiles
 // (g.tiles_m / g.tiles_n count those), all of K <= 64 at once.
 bool gemm_panel_eligible(const GemmLaunch &g, int amode, int bmode);
@@ -96,6 +102,8 @@ struct SkinnyLaunch {
 // W with unit stride along j (cols): lanes own columns, K split over wavefronts and slices.
 // xcds > 0: the single-launch form, units dealt over that many XCDs; 0: partials left for a reduction launch.
 int launch_skinny_cols(const SkinnyLaunch &s, int xcds);
+// workgroups of the single-launch form of `s` that fit one CU together (0: unknown)
+int skinny_cols_fused_occupancy(const SkinnyLaunch &s);
 // floats per row of the K-slice partials
 int skinny_ws_pitch(int cols, bool single_launch);
 // W with unit stride along k: one wavefront per output column, shuffle reduce.

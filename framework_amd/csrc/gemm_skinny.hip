@@ -48,9 +48,15 @@ __device__ __forceinline__ float sk_epilogue(float v, float bias, int epilogue) 
 //    holding the last R = min(rows, slices) slices of a unit then act as
 //    reducers, one output row each: they poll the unit's flags with loads that
 //    skip the CU's L1, read the row's partials from L2 and apply the epilogue.
-//    Reducers have the highest workgroup ids of the grid, so everything they
-//    wait for has been dispatched before them and never waits itself; the poll
-//    is bounded all the same and a reducer that gives up writes NaN.
+//    Reducers wait for every slice of their unit, the later reducers' own
+//    included, and a workgroup that waits keeps its place on its CU: were there
+//    more reducers on an XCD than workgroups fit on it together, the first
+//    ones could fill it and wait for slices that are never dispatched.  The
+//    host therefore takes this form only when all reducers of an XCD fit on it
+//    at once (skinny_cols_fused_occupancy); the non-reducers ahead of them in
+//    the grid never wait and make room as they finish.  The poll is bounded
+//    all the same, and a reducer that gives up writes NaN and raises the
+//    device status word.
 //    Measured on MI355X for x[4,4096] W[4096,4096]: 12.2 us against 15.8 us for
 //    two launches.  What does not work here: one arrival counter per unit
 //    (returning atomics on one address serialise at ~145 ns each in L2: +9 us
@@ -445,6 +451,37 @@ static void launch_skinny_cols_mr(const SkinnyLaunch &s, dim3 grid, bool fused) 
 }
 
 int skinny_ws_pitch(int cols, bool single_launch) { return single_launch ? (cols + 31) & ~31 : cols; }
+
+// How many workgroups of the single-launch form that `s` would run as fit one CU together (what the runtime's
+// occupancy calculation says for that instantiation: between 1 for the 16-row general form, whose 253 VGPRs
+// leave room for one wavefront per SIMD, and 6).  0 if the query fails.
+template <int MR>
+static int skinny_cols_fused_occupancy_mr(const SkinnyLaunch &s) {
+    const int variant = (s.x_cs == 1 ? 4 : 0) | 2 | (s.K % SK_UNROLL != 0 ? 1 : 0);
+    const bool lean = variant == 6 && s.batch == 1 && s.rows == MR && s.cols % SK_COLS == 0 && s.o_cs == 1 &&
+                      s.o_rs % 4 == 0 && (reinterpret_cast<uintptr_t>(s.out) & 15) == 0 &&
+                      s.epilogue == MNI_EPI_NONE && !s.accumulate;  // (the rule of launch_skinny_cols_mr)
+    static int cache[5] = {-1, -1, -1, -1, -1};  // per (lean, x contiguous, tail)
+    const int slot = lean ? 4 : (variant & 4 ? 2 : 0) | (variant & 1);
+    if (cache[slot] < 0) {
+        int n = 0;
+        hipError_t e;
+        if (lean) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, true, true, false, true>, SK_THREADS, 0);
+        else if (slot == 0) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, false, true, false, false>, SK_THREADS, 0);
+        else if (slot == 1) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, false, true, true, false>, SK_THREADS, 0);
+        else if (slot == 2) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, true, true, false, false>, SK_THREADS, 0);
+        else e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, true, true, true, false>, SK_THREADS, 0);
+        if (e != hipSuccess) { (void)hipGetLastError(); n = 0; }
+        cache[slot] = n;
+    }
+    return cache[slot];
+}
+int skinny_cols_fused_occupancy(const SkinnyLaunch &s) {
+    if (s.rows <= 4) return skinny_cols_fused_occupancy_mr<4>(s);
+    if (s.rows <= 8) return skinny_cols_fused_occupancy_mr<8>(s);
+    if (s.rows <= 16) return skinny_cols_fused_occupancy_mr<16>(s);
+    return 0;
+}
 
 int launch_skinny_cols(const SkinnyLaunch &s, int xcds) {
     if (s.rows <= 0 || s.cols <= 0 || s.batch <= 0) return MNI_OK;

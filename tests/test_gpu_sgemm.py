@@ -705,6 +705,48 @@ def test_products_of_few_tiles_in_planned_k_slices_integer_exact(dev, rocm, m, n
     assert rocm.launch_count() - before <= 3   # (the output buffer's fill, the product, the reduction)
 
 
+@pytest.mark.parametrize("m,n,k,split", [(32, 256, 256, 0), (17, 128, 64, 0), (32, 4096, 4096, 0), (24, 1000, 520, 0), (32, 512, 1024, 1), (20, 640, 2056, 3),
+                                         (32, 4096, 1024, 16), (31, 132, 72, 0), (29, 11008, 512, 0), (32, 2048, 8192, 5), (18, 50304, 256, 0)])
+def test_fewrows_integer_exact(dev, rocm, m, n, k, split):
+    # 17 to 32 rows against a wide N-contiguous operand: W straight into MFMA registers, K slices summed by the last
+    # workgroup of a column group to arrive.  Edges in M and N, slices that do not divide K, one slice, more slices
+    # than CUs per column group; forced and (where the planner picks it) by itself, twice in a row (the arrival
+    # counters must be back at zero).
+    a = synth.small_ints(m + k, (m, k), 3)
+    b = synth.small_ints(n + k, (k, n), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    for _ in range(2):
+        assert np.array_equal(run_gemm(dev, a, b, algo=N.ALGO_FEWROWS, split_k=split)[0], want)
+    assert np.array_equal(run_gemm(dev, a, b)[0], want)
+
+
+def test_fewrows_normal_inputs_batch_epilogues_accumulate(dev, rocm, oracle_native):
+    m, n, k, batch = 27, 640, 1024, 3
+    a = synth.normal(1, (batch, m, k))
+    w = synth.normal(2, (1, k, n), stream=1)          # one W for all batches (the reference's broadcast rule)
+    bias = synth.normal(3, (n,), stream=2)
+    tol = gemm_tol(k, a, w)
+    want = np.stack([oracle_native.sgemm_ikj(a[b], w[0]) for b in range(batch)])
+    for algo in (N.ALGO_FEWROWS, N.ALGO_AUTO):
+        assert max_err(run_gemm(dev, a, w, algo=algo), want) <= tol
+    dBias = dev.put(bias)
+    for epi, f in ((N.EPI_BIAS, lambda z: z), (N.EPI_BIAS_RELU, lambda z: np.maximum(z, 0)),
+                   (N.EPI_BIAS_GELU, lambda z: 0.5 * z * (1 + np.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3))))):
+        for split in (1, 0):
+            got = run_gemm(dev, a, w, algo=N.ALGO_FEWROWS, split_k=split, bias=dBias, epilogue=epi)
+            assert max_err(got, f(want.astype(np.float64) + bias[None, None, :])) <= tol + 1e-5
+    # accumulate: C += A W on a C that holds something
+    dA, dW = dev.put(a), dev.put(w)
+    dC = dev.put(want.copy())
+    rocm.sgemm(m, n, k, dA, dW, dC, batch=batch, a_batch=(m * k, batch), b_batch=(k * n, 1), accumulate=True, algo=N.ALGO_FEWROWS)
+    assert max_err(rocm.to_host(dC, (batch, m, n)), 2.0 * want.astype(np.float64)) <= 2 * tol
+    # what it does not take is refused when forced
+    with pytest.raises(N.MniError, match="few-rows kernel takes 17 to 32 rows"):
+        run_gemm(dev, synth.normal(1, (40, 256)), synth.normal(2, (256, 256)), algo=N.ALGO_FEWROWS)
+    with pytest.raises(N.MniError, match="few-rows kernel takes 17 to 32 rows"):
+        run_gemm(dev, synth.normal(1, (256, 32)), synth.normal(2, (256, 256)), ta=True, algo=N.ALGO_FEWROWS)
+
+
 @pytest.mark.parametrize("m,h,c", [(32, 64, 3), (32, 10, 64), (7, 5, 3), (128, 64, 64), (33, 257, 9)])
 def test_pair_of_tiny_products_is_one_launch_with_the_reference_sums(dev, rocm, oracle_native, m, h, c):
     # the backward pair of a small Linear (x [m, h] . w [h, c]; dx = g . w^T, dw = x^T . g): products the tiny-product
@@ -751,6 +793,21 @@ def test_skinny_cols_integer_exact(dev, m, algo):
     assert np.array_equal(run_gemm(dev, a, b, algo=algo)[0], want)
     for split in (1, 3, 11):  # 3 slices < 13 rows: reducers take several rows each
         assert np.array_equal(run_gemm(dev, a, b, algo=algo, split_k=split)[0], want)
+
+
+@pytest.mark.parametrize("m,n,k", [(12, 8192, 2048), (12, 11008, 1024), (8, 50304, 768), (13, 4096, 4096), (16, 50304, 256), (5, 32000, 512), (9, 2048, 8192)])
+def test_skinny_cols_wide_outputs_integer_exact(dev, rocm, m, n, k):
+    # Many column groups: the reducers of the single-launch form (the workgroups of a unit's last min(rows, slices)
+    # K slices, which wait for all of its slices) must all fit on their XCD together, or the first ones fill it and
+    # wait for slices that are never dispatched.  The 16-row general form fits one workgroup per CU (253 VGPRs): at
+    # 12 x 8192 x 8192 its 48 reducers per XCD met 32 places, gave up and wrote NaN.  The host now takes the
+    # two-launch form whenever the reducers would not fit.
+    a = synth.small_ints(m + n, (m, k), 3)
+    b = synth.small_ints(n + k, (k, n), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    for algo in (N.ALGO_AUTO, N.ALGO_SKINNY):
+        assert np.array_equal(run_gemm(dev, a, b, algo=algo)[0], want)
+    rocm.sync()   # (a wait that expired would be reported here)
 
 
 @pytest.mark.parametrize("m", [4, 8, 16])
