@@ -248,6 +248,17 @@ static bool fewrows_plan(const GemmLaunch &g, int cus) {
     return g.K >= 256 && (int64_t)g.N * g.K >= (1 << 18);
 }
 
+// Whether run_mfma would give the product to the few-rows kernel by itself.
+static bool fewrows_takes(const mni_gemm_desc &d) {
+    if (d.K == 0 || d.epilogue >= MNI_EPI_BIAS_GELU_DUAL) return false;
+    GemmLaunch g;
+    fill_launch(g, d);
+    DeviceCtx &c = ctx();
+    const int amode = classify(g.a_cs, g.a_rs), bmode = classify(g.b_rs, g.b_cs);
+    return gemm_fewrows_eligible(g, amode, bmode) && (size_t)((g.N + 127) / 128) * g.batch <= c.fewrows_counter_cap && c.xcd_count == 8 &&
+           fewrows_plan(g, c.compute_units > 0 ? c.compute_units : 256);
+}
+
 // K slices for a product of `tiles` 64 x 64 tiles (at most one per CU) of `ktiles` K steps each.
 // Estimated microseconds of a plan with s slices:
 //   (per_cu (steps + 3) + 3) c  +  [s > 1]  (2.5 + 2 s out_bytes / 5 TB/s)
@@ -304,14 +315,14 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
         if (probe) { probe->kind = PlanProbe::PANEL; return MNI_OK; }
         return launch_gemm_panel(g, amode, bmode);
     }
-    // Few-rows form (17 to 32 rows against a wide N-contiguous operand): forced, or chosen by fewrows_plan.
+    // Few-rows form (9 to 32 rows against a wide N-contiguous operand): forced, or chosen by fewrows_plan.
     {
         // (its K slices meet in one XCD's L2: the workgroup-to-XCD mapping must be the confirmed round-robin over 8)
         const bool fr_ok = gemm_fewrows_eligible(g, amode, bmode) && (size_t)((g.N + 127) / 128) * g.batch <= c.fewrows_counter_cap && c.xcd_count == 8;
         int fr_split = 0;
         if (d.algo == MNI_ALGO_FEWROWS) {
             if (!fr_ok)
-                return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel takes 17 to 32 rows of a K-contiguous A against an N-contiguous B, "
+                return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel takes 9 to 32 rows of a K-contiguous A against an N-contiguous B, "
                                                   "K %% 8 == 0, N %% 4 == 0, 16-byte aligned");
             fr_split = d.split_k > 0 ? d.split_k : fewrows_split(g, cus);
         } else if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && fr_ok && fewrows_plan(g, cus)) {
@@ -553,7 +564,12 @@ int sgemm(const mni_gemm_desc &d) {
         }
         if (gemm_tiny_eligible(g)) return launch_gemm_tiny(g);
     }
-    if ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS) {
+    // 9 to 16 rows against a wide N-contiguous operand: the few-rows MFMA kernel is level with or ahead of the skinny
+    // kernel's 16-row forms (us, few-rows against skinny: 16 x 4096 x 4096 18.6 / 21.5, 12 rows 18.6 / 30.5,
+    // 16 x 8192 x 8192 46 / 58, 16 x 1024 x 1024 8.5 / 8.4; at 8 rows the skinny kernel leads, 15.2 / 18.6)
+    const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M > 8 && d.M <= 16 && fewrows_takes(d);
+    if (!to_fewrows &&
+        ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS)) {
         int rc;
         if (try_skinny(d, &rc)) return rc;
         if (d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS)

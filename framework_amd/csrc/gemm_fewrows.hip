@@ -1,8 +1,8 @@
 // A few dozen rows against a wide, N-contiguous operand on the MFMA matrix cores:
 //
-//   C[b] (M x N) = epilogue( A[b] (M x K)  *  W[b] (K x N) ),   16 < M <= 32
+//   C[b] (M x N) = epilogue( A[b] (M x K)  *  W[b] (K x N) ),   8 < M <= 32
 //
-// A K-contiguous, W N-contiguous -- `x.matmul(weight)` with a [in, out] weight and a batch of 17 to 32 rows
+// A K-contiguous, W N-contiguous -- `x.matmul(weight)` with a [in, out] weight and a batch of 9 to 32 rows
 // (reference call site: src/native/src/ops/matmul.rs:18-78 through src/nn.ts:20-25), the shape of batched
 // decoding.  W is read once and is what the product costs (32 rows against 4096 x 4096: 64 MiB of W, ~10 us of
 // HBM time, 7 us of MFMAs).  The tile kernel spends its time elsewhere on this shape: its smallest tile pads
@@ -248,9 +248,9 @@ __global__ __launch_bounds__(256, 2) void gemm_fewrows_kernel(const GemmLaunch g
 
 static bool fr_aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-// 17 to 32 rows of a K-contiguous A against an N-contiguous W, everything in whole 16-byte pieces.
+// 9 to 32 rows of a K-contiguous A against an N-contiguous W, everything in whole 16-byte pieces.
 bool gemm_fewrows_eligible(const GemmLaunch &g, int amode, int bmode) {
-    if (amode != 0 || bmode != 1 || g.M <= 16 || g.M > FR_ROWS || g.epilogue > MNI_EPI_BIAS_GELU) return false;
+    if (amode != 0 || bmode != 1 || g.M <= 8 || g.M > FR_ROWS || g.epilogue > MNI_EPI_BIAS_GELU) return false;
     if (g.K < 64 || g.K % 8 != 0 || g.N < FR_COLS || g.N % 4 != 0) return false;
     if (g.a_rs % 4 != 0 || g.b_rs % 4 != 0 || g.a_bs % 4 != 0 || g.b_bs % 4 != 0) return false;
     if (!fr_aligned16(g.A) || !fr_aligned16(g.B)) return false;
@@ -262,7 +262,7 @@ bool gemm_fewrows_eligible(const GemmLaunch &g, int amode, int bmode) {
 // g.tiles_n = column groups of 128; g.split_k slices of g.k_per_slice (a multiple of 32).
 int launch_gemm_fewrows(const GemmLaunch &g, int amode, int bmode) {
     if (!gemm_fewrows_eligible(g, amode, bmode))
-        return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel takes 17 to 32 rows of a K-contiguous A against an N-contiguous B, "
+        return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel takes 9 to 32 rows of a K-contiguous A against an N-contiguous B, "
                                           "K %% 8 == 0, N %% 4 == 0, 16-byte aligned");
     if (g.tiles_n != (g.N + FR_COLS - 1) / FR_COLS || g.split_k < 1 || g.k_per_slice % 32 != 0 || g.k_per_slice <= 0 ||
         (int64_t)g.split_k * g.k_per_slice < g.K || (g.split_k > 1 && (!g.ws || !g.sk_flags)) ||

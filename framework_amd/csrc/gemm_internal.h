@@ -62,7 +62,7 @@ int launch_gemm_direct(const GemmLaunch &g, int amode, int bmode, int ksplit);
 bool gemm_tiny_eligible(const GemmLaunch &g);
 int launch_gemm_tiny(const GemmLaunch &g);
 int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1);  // two eligible, independent products in one launch
-// 17 to 32 rows of a K-contiguous A against a wide N-contiguous B, both straight into MFMA registers (gemm_fewrows.hip):
+// 9 to 32 rows of a K-contiguous A against a wide N-contiguous B, both straight into MFMA registers (gemm_fewrows.hip):
 // g.tiles_n counts column groups of 128, g.split_k K slices of g.k_per_slice (a multiple of 32).  With split_k > 1:
 // partials [slice][batch][M][N] in g.ws and one counter per (batch, column group) in g.sk_flags, zero between launches
 // (the workgroup that completes a count adds the slices up and returns the counter to zero).

@@ -706,9 +706,10 @@ def test_products_of_few_tiles_in_planned_k_slices_integer_exact(dev, rocm, m, n
 
 
 @pytest.mark.parametrize("m,n,k,split", [(32, 256, 256, 0), (17, 128, 64, 0), (32, 4096, 4096, 0), (24, 1000, 520, 0), (32, 512, 1024, 1), (20, 640, 2056, 3),
-                                         (32, 4096, 1024, 16), (31, 132, 72, 0), (29, 11008, 512, 0), (32, 2048, 8192, 5), (18, 50304, 256, 0)])
+                                         (32, 4096, 1024, 16), (31, 132, 72, 0), (29, 11008, 512, 0), (32, 2048, 8192, 5), (18, 50304, 256, 0),
+                                         (9, 512, 512, 0), (12, 8192, 2048, 0), (16, 4096, 4096, 0)])
 def test_fewrows_integer_exact(dev, rocm, m, n, k, split):
-    # 17 to 32 rows against a wide N-contiguous operand: W straight into MFMA registers, K slices summed by the last
+    # 9 to 32 rows against a wide N-contiguous operand: W straight into MFMA registers, K slices summed by the last
     # workgroup of a column group to arrive.  Edges in M and N, slices that do not divide K, one slice, more slices
     # than CUs per column group; forced and (where the planner picks it) by itself, twice in a row (the arrival
     # counters must be back at zero).
@@ -741,9 +742,9 @@ def test_fewrows_normal_inputs_batch_epilogues_accumulate(dev, rocm, oracle_nati
     rocm.sgemm(m, n, k, dA, dW, dC, batch=batch, a_batch=(m * k, batch), b_batch=(k * n, 1), accumulate=True, algo=N.ALGO_FEWROWS)
     assert max_err(rocm.to_host(dC, (batch, m, n)), 2.0 * want.astype(np.float64)) <= 2 * tol
     # what it does not take is refused when forced
-    with pytest.raises(N.MniError, match="few-rows kernel takes 17 to 32 rows"):
+    with pytest.raises(N.MniError, match="few-rows kernel takes 9 to 32 rows"):
         run_gemm(dev, synth.normal(1, (40, 256)), synth.normal(2, (256, 256)), algo=N.ALGO_FEWROWS)
-    with pytest.raises(N.MniError, match="few-rows kernel takes 17 to 32 rows"):
+    with pytest.raises(N.MniError, match="few-rows kernel takes 9 to 32 rows"):
         run_gemm(dev, synth.normal(1, (256, 32)), synth.normal(2, (256, 256)), ta=True, algo=N.ALGO_FEWROWS)
 
 
