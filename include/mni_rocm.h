@@ -125,7 +125,9 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * device's workgroup-to-XCD mapping was not confirmed); SKINNY = the bandwidth
  * kernels (error if the shape or layout is not eligible); SKINNY_TWO_PASS = the
  * same with the K-slice partials summed by a second launch instead of inside
- * the first; DIRECT = the register-direct MFMA kernel for batched products of
+ * the first (SKINNY itself takes the second launch when the reducing
+ * workgroups of the single launch would not all fit the device at once);
+ * DIRECT = the register-direct MFMA kernel for batched products of
  * many small tiles (64 x 64 tiles, operands read from memory straight into the
  * matrix instruction's registers; split_k 0 or 1 = one wavefront per tile,
  * split_k 4 = four wavefronts sharing K; error if the operand layouts are not
@@ -136,7 +138,12 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * under the MFMAs of the next; TINY = one thread per output element and a
  * sequential sum over K, products rounded and added one by one as the
  * reference's CPU arm does (bit-identical to it), for products of a few
- * thousand outputs.  AUTO picks among them. */
+ * thousand outputs; FEWROWS = 9 to 32 rows of a K-contiguous A against a
+ * wide N-contiguous B (a batch of token rows against a [in, out] weight): B
+ * read once, straight into the matrix instruction's registers, K slices
+ * (split_k, 0 = chosen) summed inside the launch (error unless K % 8 == 0,
+ * N % 4 == 0, N >= 128, K >= 64, operands and C 16-byte aligned with row
+ * strides in whole 16 bytes).  AUTO picks among them. */
 enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
        MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7, MNI_ALGO_TINY = 8, MNI_ALGO_FEWROWS = 9 };
 
