@@ -886,14 +886,37 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_mfma_pair_kernel(const GemmP
     }
 }
 
+// Workgroups of a stream-K instantiation that fit one CU together, by the runtime's occupancy calculation (asked once).
+template <int AM, int BMO, int TM, int TN>
+static int streamk_occupancy() {
+    static int n = -1;
+    if (n < 0) {
+        int v = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, gemm_mfma_kernel<AM, BMO, TM, TN, true>, NTHREADS, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            v = 0;
+        }
+        n = v;
+    }
+    return n;
+}
+
 template <int TM, int TN>
-static void launch_modes(const GemmLaunch &g, int amode, int bmode, dim3 grid) {
+static int launch_modes(const GemmLaunch &g, int amode, int bmode, dim3 grid) {
     dim3 block(NTHREADS);
     hipStream_t s = ctx().stream;
+    // A stream-K finisher waits for partial tiles of other workgroups of its XCD: the whole grid must be resident
+    // at once.  The planner sizes it by gemm_mfma_resident_per_cu; here that figure is held against what the
+    // runtime says about the instantiation that is about to run.
+    const int cus_per_xcd = g.streamk && g.sk_xcds > 0 ? (ctx().compute_units > 0 ? ctx().compute_units : 256) / g.sk_xcds : 0;
 #define MNI_LAUNCH(AM, BMO)                                                                        \
     do {                                                                                           \
-        if (g.streamk) MNI_KERNEL_LAUNCH((gemm_mfma_kernel<AM, BMO, TM, TN, true>), grid, block, 0, s, g);   \
-        else MNI_KERNEL_LAUNCH((gemm_mfma_kernel<AM, BMO, TM, TN, false>), grid, block, 0, s, g);            \
+        if (g.streamk) {                                                                           \
+            if ((int64_t)streamk_occupancy<AM, BMO, TM, TN>() * cus_per_xcd < g.sk_wpx)           \
+                return set_error(MNI_ERR_INVALID, "sgemm: stream-K grid of %d workgroups per XCD, but %d fit a CU", g.sk_wpx, \
+                                 streamk_occupancy<AM, BMO, TM, TN>());                           \
+            MNI_KERNEL_LAUNCH((gemm_mfma_kernel<AM, BMO, TM, TN, true>), grid, block, 0, s, g);   \
+        } else MNI_KERNEL_LAUNCH((gemm_mfma_kernel<AM, BMO, TM, TN, false>), grid, block, 0, s, g);            \
     } while (0)
     if (amode == 2 || bmode == 2) MNI_LAUNCH(2, 2);
     else if (amode == 0 && bmode == 0) MNI_LAUNCH(0, 0);
@@ -901,6 +924,7 @@ static void launch_modes(const GemmLaunch &g, int amode, int bmode, dim3 grid) {
     else if (amode == 1 && bmode == 0) MNI_LAUNCH(1, 0);
     else MNI_LAUNCH(1, 1);
 #undef MNI_LAUNCH
+    return MNI_OK;
 }
 
 // tile_m / tile_n: 128 or 64 (g.tiles_m / g.tiles_n must be counted in those units)
@@ -914,11 +938,13 @@ int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int 
     const int64_t blocks = g.streamk ? (int64_t)g.sk_xcds * g.sk_wpx : (int64_t)g.tiles_m * g.tiles_n * g.batch * g.split_k;
     if (blocks > 0x7fffffffLL) return set_error(MNI_ERR_INVALID, "sgemm: too many tiles (%lld)", (long long)blocks);
     dim3 grid((unsigned)blocks);
-    if (tile_m == 128 && tile_n == 128) launch_modes<2, 2>(g, amode, bmode, grid);
-    else if (tile_m == 128 && tile_n == 64) launch_modes<2, 1>(g, amode, bmode, grid);
-    else if (tile_m == 64 && tile_n == 128) launch_modes<1, 2>(g, amode, bmode, grid);
-    else if (tile_m == 64 && tile_n == 64) launch_modes<1, 1>(g, amode, bmode, grid);
+    int rc;
+    if (tile_m == 128 && tile_n == 128) rc = launch_modes<2, 2>(g, amode, bmode, grid);
+    else if (tile_m == 128 && tile_n == 64) rc = launch_modes<2, 1>(g, amode, bmode, grid);
+    else if (tile_m == 64 && tile_n == 128) rc = launch_modes<1, 2>(g, amode, bmode, grid);
+    else if (tile_m == 64 && tile_n == 64) rc = launch_modes<1, 1>(g, amode, bmode, grid);
     else return set_error(MNI_ERR_INVALID, "sgemm: unsupported tile %d x %d", tile_m, tile_n);
+    MNI_TRY(rc);
     return check_launch("gemm_mfma_kernel");
 }
 
