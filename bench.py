@@ -210,6 +210,20 @@ def bench_extras(r, with_cpu):
         c5a["cpu_baseline"] = dict(cpu_note("the whole product, best of 3"), value=dt * 1e3, unit="ms", **{"GB/s": by / dt / 1e9})
         orc.native.resetEngine()
     out["config5a_gemv"] = c5a
+    # the same W against batches of token rows (batched decoding): 8 rows through the skinny kernel, 16 and 32 through
+    # the few-rows MFMA kernel, 64 through the tile kernel; W cold (eight in rotation) -- not a BASELINE config
+    rows_out = {}
+    for mrows in (8, 16, 32, 64):
+        xb = r.to_device(synth.normal(5, (mrows, 4096)))
+        yb = r.malloc(mrows * 4096 * 4)
+        descs = [r.gemm_desc(mrows, 4096, 4096, xb, wp, yb) for wp in ws]
+        us = r.sgemm_timed(descs, 300, 200) * 1e3
+        byb = 4.0 * (4096 * 4096 + 2 * mrows * 4096)
+        rows_out["%d_rows" % mrows] = {"us": us, "GB/s": byb / us / 1e3, "frac_hbm": byb / us / 1e3 / PEAK_HBM_GBPS,
+                                       "TFLOP/s": 2.0 * mrows * 4096 * 4096 / us / 1e6}
+        r.free(xb)
+        r.free(yb)
+    out["decode_batch_rows_x_4096x4096_cold"] = rows_out
     for p in ws + [dx, dw, dy]:
         r.free(p)
     # ---- config 5b: X^T[1024,65536] dY[65536,1024], X^T as a view, split-K -------------------------------------
@@ -248,14 +262,17 @@ def bench_extras(r, with_cpu):
                                                                    a_batch=(512 * 64, 32), b_batch=(512 * 512, 32)))]
     c3 = {}
     each = {}
+    # 1500 untimed launches (~25 ms) first: after the host-side work above the clocks are down, and the first ~20 ms of
+    # any timing run 10 % slow (the headline's settle launches and config 4's warm-up steps are there for the same reason)
+    C3_WARM = 1500
     for name, kern, desc in prods:
-        each[name] = r.sgemm_timed([desc], 10, 200)
+        each[name] = r.sgemm_timed([desc], C3_WARM, 200)
         # each product moves 41.9 MB and 1.07 GFLOP: the matrix pipe needs 6.8 us for it, HBM 5.2 us
         c3[name] = roofline("mfma", kern, each[name] * 1e-3, fl, by)
     # the two gradients as the engine's matmul backward issues them: one paired launch (mni_rocm_sgemm_pair)
     g_out2 = r.malloc(32 * 512 * 64 * 4)
     pair = [prods[1][2], r.gemm_desc(64, 512, 512, dq, dds, g_out2, batch=32, a_strides=(1, 64), a_batch=(512 * 64, 32), b_batch=(512 * 512, 32))]
-    ms_pair = r.sgemm_pair_timed(pair, 10, 200)
+    ms_pair = r.sgemm_pair_timed(pair, C3_WARM, 200)
     c3["dQ_and_dKT_paired"] = dict(roofline("mfma", "gemm_mfma_pair_kernel<0, 1, 1, 1>", ms_pair * 1e-3, 2 * fl, 2 * by),
                                    note="both gradients in one launch; one after the other they take %.1f us" % ((each["dQ"] + each["dKT"]) * 1e3))
     total = each["scores"] + ms_pair
@@ -486,6 +503,14 @@ def run_for_counters(r, which):
         for _ in range(5):
             r.sgemm_pair(r.gemm_desc(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32), b_batch=(512 * 64, 32)),
                          r.gemm_desc(64, 512, 512, dq, dds, g_out2, batch=32, a_strides=(1, 64), a_batch=(512 * 64, 32), b_batch=(512 * 512, 32)))
+    elif which == "fewrows":
+        # 32 token rows against a [4096, 4096] weight (the few-rows kernel) and against an [8192, 8192] one, 5 launches each
+        x = r.to_device(synth.normal(4, (32, 8192), 0.02))
+        w = r.to_device(synth.normal(4, (8192, 8192), 0.02, stream=1))
+        for _ in range(5):
+            r.sgemm(32, 4096, 4096, x, w, dst)
+        for _ in range(5):
+            r.sgemm(32, 8192, 8192, x, w, dst)
     elif which == "attention":
         # the one-kernel attention forward on [8, 8192, 64], causal, through the engine entry point
         from framework_amd.api import bind
@@ -549,7 +574,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
-    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "attention", "attention_bwd"], default=None,
+    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "fewrows", "attention", "attention_bwd"], default=None,
                     help="for rocprofv3 --pmc runs: launch a copy kernel of known size (64 MiB read + 64 MiB "
                          "written) 3 times, then the chosen product 5 times, and exit")
     args = ap.parse_args()
