@@ -784,11 +784,11 @@ __global__ void layernorm_bwd_rows_kernel(float *__restrict__ dx, const float *_
 // dgamma / dbeta: column sums of g * xhat and g over row blocks, partials summed in block order
 __global__ void layernorm_bwd_cols_kernel(float *__restrict__ pgamma, float *__restrict__ pbeta, const float *__restrict__ g,
                                           const float *__restrict__ x, const float *__restrict__ mean,
-                                          const float *__restrict__ rstd, int64_t rows, int64_t c) {
+                                          const float *__restrict__ rstd, int64_t rows, int64_t c, int64_t rows_per_block) {
     const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (j >= c) return;
-    const int64_t r0 = (int64_t)blockIdx.y * BG_ROWS;
-    const int64_t r1 = min(rows, r0 + BG_ROWS);
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = min(rows, r0 + rows_per_block);
     float sg = 0.f, sb = 0.f;
     for (int64_t r = r0; r < r1; ++r) {
         const float gv = g[r * c + j];
@@ -806,14 +806,16 @@ int k_layernorm_backward(float *dx, float *dgamma, float *dbeta, const float *g,
     MNI_KERNEL_LAUNCH(layernorm_bwd_rows_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, dx, g, x, gamma, mean,
                        rstd, rows, c);
     MNI_TRY(check_launch("layernorm_backward_rows"));
-    const int64_t nparts = (rows + BG_ROWS - 1) / BG_ROWS;
-    if (nparts > 65535) return set_error(MNI_ERR_INVALID, "layernorm backward: too many rows (%lld)", (long long)rows);
+    // row blocks of BG_ROWS; more rows per block when the second grid axis (65535 blocks) would not hold them all
+    int64_t rows_per_block = BG_ROWS;
+    if ((rows + rows_per_block - 1) / rows_per_block > 65535) rows_per_block = (rows + 65534) / 65535;
+    const int64_t nparts = (rows + rows_per_block - 1) / rows_per_block;
     void *part = nullptr;
     MNI_TRY(dev_alloc(&part, (size_t)2 * nparts * c * sizeof(float)));
     float *pg = (float *)part, *pb = pg + nparts * c;
     const unsigned gx = (unsigned)((c + TPB - 1) / TPB);
     MNI_KERNEL_LAUNCH(layernorm_bwd_cols_kernel, dim3(gx, (unsigned)nparts), dim3(TPB), 0, ctx().stream, pg, pb, g, x, mean,
-                       rstd, rows, c);
+                       rstd, rows, c, rows_per_block);
     int rc = check_launch("layernorm_backward_cols");
     if (rc == MNI_OK) {
         MNI_KERNEL_LAUNCH(colsum_final_kernel, colsum_final_grid(c), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, dgamma, (const float *)pg, nparts, c);

@@ -110,6 +110,22 @@ def test_max_matches_the_oracle_exactly(both, shape, dim):
     assert np.array_equal(res[0][0], x.max(axis=dim, keepdims=True))
 
 
+def test_layernorm_backward_of_more_rows_than_one_grid_axis_of_row_blocks(gpu):
+    # 1.2 M rows of 8: the column sums for gamma and beta run over more 16-row blocks than the second grid axis holds,
+    # so a block takes more rows; checked against float64 (the oracle would need minutes)
+    rows, c = 1_200_000, 8
+    x = synth.normal(20, (rows, c), 2.0)
+    g = synth.uniform(21, (c,), 0.5, 1.5, stream=1)
+    b = synth.normal(22, (c,), stream=2)
+    w = synth.normal(23, (rows, c), stream=3)
+    X, G, B = _t(gpu, x, True), _t(gpu, g, True), _t(gpu, b, True)
+    gpu.layerNorm(X, G, B, 1e-5).mul(_t(gpu, w)).sum().backward()
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    xhat = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5)
+    assert max_err(G.grad.numpy(), (w64 * xhat).sum(0)) <= 1e-4 * math.sqrt(rows) * float(np.abs(w).max()) * 3
+    assert max_err(B.grad.numpy(), w64.sum(0)) <= 1e-4 * math.sqrt(rows) * float(np.abs(w).max())
+
+
 @pytest.mark.parametrize("shape", [(2, 3), (64, 768), (4, 33, 100), (5000, 16)])
 def test_layernorm_matches_the_oracle(both, shape):
     gpu, cpu = both
