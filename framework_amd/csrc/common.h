@@ -90,10 +90,11 @@ int upload_small(void *dst, const void *src, size_t bytes);
 // (a kernel that is next in line delivers within microseconds), then waits for the stream; false in *delivered
 // if even then the word has not come (the caller has another way to the value).
 #ifdef __HIPCC__
-// One 8-byte store to pinned host memory: the host sees the tag and the value together or not at all, and
-// after everything this thread wrote before.
+// One 8-byte store to pinned host memory: the host sees the tag and the value together or not at all.  Relaxed: a
+// release at system scope would write the whole L2 back first (microseconds, with the host waiting); a kernel that
+// hands over more than the word fences what it wrote itself (fetch_small_kernel).
 __device__ __forceinline__ void post_result_word(unsigned long long *word, unsigned tag, unsigned value) {
-    __hip_atomic_store(word, ((unsigned long long)tag << 32) | (unsigned long long)value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    __hip_atomic_store(word, ((unsigned long long)tag << 32) | (unsigned long long)value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 #endif
 unsigned next_result_tag();

@@ -1367,20 +1367,34 @@ __global__ void multi_tensor_kernel(const MultiTensor t, double *__restrict__ pa
 }
 __global__ __launch_bounds__(TPB) void sumsq_solo_kernel(const MultiTensor t, double *__restrict__ out, unsigned long long *result_word,
                                                          unsigned tag) {
-    __shared__ double sh[4];
+    // The host waits for this kernel, so the chunks are not taken one after the other by the whole workgroup (a
+    // round trip to memory each) but four at a time, one per wavefront.  A wavefront plays the four wavefronts of
+    // chunk_sumsq in turn -- lane l of "wavefront" w adds up elements lo + 64 w + l, + 256, ... -- so every sum
+    // is formed in the order of the multi-launch form: same value.
     __shared__ double part[SUMSQ_SOLO_BLOCKS];
+    __shared__ double fin[4];
     const int blocks = t.block_start[t.count];
-    int ti = 0;
-    for (int b = 0; b < blocks; ++b) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int b = wave; b < blocks; b += TPB / 64) {
+        int ti = 0;
         while (ti + 1 < t.count && b >= t.block_start[ti + 1]) ++ti;
         const int64_t n = t.n[ti];
         const int64_t lo = (int64_t)(b - t.block_start[ti]) * MULTI_CHUNK;
         const int64_t hi = lo + MULTI_CHUNK < n ? lo + MULTI_CHUNK : n;
-        const double sq = chunk_sumsq(t.g[ti], lo, hi, sh);
-        if (threadIdx.x == 0) part[b] = sq;
-        __syncthreads();  // sh is reused; part[b] is visible
+        const float *__restrict__ g = t.g[ti];
+        double s[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            double v = 0.0;
+            for (int64_t i = lo + 64 * w + lane; i < hi; i += TPB) { const double x = (double)g[i]; v += x * x; }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+            s[w] = v;
+        }
+        if (lane == 0) part[b] = (s[0] + s[1]) + (s[2] + s[3]);
     }
-    const double total = sum_partials(part, blocks, sh);
+    __syncthreads();
+    const double total = sum_partials(part, blocks, fin);
     if (threadIdx.x == 0) {
         out[0] = total;
         if (result_word) post_result_word(result_word, tag, __float_as_uint((float)total));
