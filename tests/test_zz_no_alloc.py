@@ -17,6 +17,7 @@ SPLITK = (1024, 1024, 8192, (1, 1024), N.ALGO_AUTO, 0)  # A^T view, 8 K slices o
 GEMV = (4, 4096, 4096, None, N.ALGO_AUTO, 0)            # skinny kernel, 64 K slices reduced inside the launch
 SMALL_SPLIT = (200, 136, 1000, None, N.ALGO_MFMA, 5)    # ragged edges, explicit split
 NO_WORKSPACE = (512, 512, 64, None, N.ALGO_AUTO, 0)     # one workgroup per tile: no partials at all
+FEWROWS = (24, 4096, 2048, None, N.ALGO_AUTO, 0)        # few-rows kernel: 8 K slices summed by the last workgroup to arrive
 
 
 def _operands(rocm, case, seed):
@@ -33,7 +34,8 @@ def _run(rocm, fn, case, dA, dB, dC):
     return rocm.to_host(dC, (M, Nn))
 
 
-@pytest.mark.parametrize("first,second", [(STREAMK, GEMV), (SPLITK, SMALL_SPLIT), (GEMV, NO_WORKSPACE), (STREAMK, SPLITK)])
+@pytest.mark.parametrize("first,second", [(STREAMK, GEMV), (SPLITK, SMALL_SPLIT), (GEMV, NO_WORKSPACE), (STREAMK, SPLITK), (SPLITK, FEWROWS),
+                                          (FEWROWS, GEMV)])
 def test_two_calls_in_a_row_match_the_allocating_entry_point(rocm, first, second):
     bufs = []
     try:
