@@ -82,7 +82,11 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
     // LEAN (the decode shape): one batch, exactly MR rows, whole 256-column
     // groups, row-major output, no epilogue -- known at compile time, so the
     // general case's address arithmetic and guards drop out of a kernel whose
-    // whole life is a few microseconds.
+    // whole life is a few microseconds.  Instantiated for every row count from
+    // 1 to 8 (and 16): with the count a run-time value below MR the guards come
+    // back and cost 0.4 (4 rows) to 0.9 us (8 rows); with the count rounded up
+    // to 4 or 8, x[1,4096] W[4096,4096] took 12.8 us against 11.7, 5 rows 15.7
+    // against 13.4 (MI355X, W in the Infinity Cache).
     static_assert(!LEAN || (XC && FUSED && !TAIL), "LEAN implies XC, FUSED, !TAIL");
     const int rows = LEAN ? MR : s.rows, batch = LEAN ? 1 : s.batch;
     const int epilogue = LEAN ? (int)MNI_EPI_NONE : s.epilogue, accumulate = LEAN ? 0 : s.accumulate;
@@ -140,6 +144,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
                 float xv[4][U];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    if (i0 + i >= MR) continue;  // (MR need not be a multiple of 4)
                     const int ii = min(i0 + i, rows - 1);
                     if (XC) {  // X rows contiguous along k: one scalar load of U floats
                         const float *__restrict__ xr = X + (int64_t)ii * s.x_rs + k0;
@@ -153,6 +158,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
                 }
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    if (i0 + i >= MR) continue;
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
                         acc[i0 + i].x += xv[i][u] * w[u].x;
@@ -460,17 +466,28 @@ __global__ __launch_bounds__(256) void splitk_reduce4_kernel(const ReduceLaunch 
 int skinny_cols_block_cols() { return SK_COLS; }
 int skinny_cols_rows_per_pass() { return SK_WAVES * SK_UNROLL; }
 
+// The decode shape, for which the single-launch form has an instantiation per row count (1 to 8, and 16): X rows
+// contiguous, K in whole groups of SK_UNROLL rows, one batch, whole 256-column groups, row-major 16-byte aligned
+// output, no epilogue.
+static bool skinny_decode_shape(const SkinnyLaunch &s) {
+    return s.x_cs == 1 && s.K % SK_UNROLL == 0 && s.batch == 1 && (s.rows <= 8 || s.rows == 16) && s.cols % SK_COLS == 0 &&
+           s.o_cs == 1 && s.o_rs % 4 == 0 && (reinterpret_cast<uintptr_t>(s.out) & 15) == 0 && s.epilogue == MNI_EPI_NONE &&
+           !s.accumulate;
+}
+#define MNI_SK_DECODE_ROWS(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(16)
+
 template <int MR>
 static void launch_skinny_cols_mr(const SkinnyLaunch &s, dim3 grid, bool fused) {
     const dim3 block(SK_THREADS);
     hipStream_t st = ctx().stream;
     const int variant = (s.x_cs == 1 ? 4 : 0) | (fused ? 2 : 0) | (s.K % SK_UNROLL != 0 ? 1 : 0);
-    const bool lean = variant == 6 && s.batch == 1 && s.rows == MR && s.cols % SK_COLS == 0 && s.o_cs == 1 &&
-                      s.o_rs % 4 == 0 && (reinterpret_cast<uintptr_t>(s.out) & 15) == 0 &&
-                      s.epilogue == MNI_EPI_NONE && !s.accumulate;
-    if (lean) {
-        MNI_KERNEL_LAUNCH((skinny_cols_kernel<MR, true, true, false, true>), grid, block, 0, st, s);
-        return;
+    if (fused && skinny_decode_shape(s)) {
+        switch (s.rows) {
+#define MNI_SK_LEAN(R) \
+    case R: MNI_KERNEL_LAUNCH((skinny_cols_kernel<R, true, true, false, true>), grid, block, 0, st, s); return;
+            MNI_SK_DECODE_ROWS(MNI_SK_LEAN)
+#undef MNI_SK_LEAN
+        }
     }
     switch (variant) {
 #define MNI_SK(V, XC, FUSED, TAIL) \
@@ -491,16 +508,28 @@ int skinny_ws_pitch(int cols, bool single_launch) { return single_launch ? (cols
 template <int MR>
 static int skinny_cols_fused_occupancy_mr(const SkinnyLaunch &s) {
     const int variant = (s.x_cs == 1 ? 4 : 0) | 2 | (s.K % SK_UNROLL != 0 ? 1 : 0);
-    const bool lean = variant == 6 && s.batch == 1 && s.rows == MR && s.cols % SK_COLS == 0 && s.o_cs == 1 &&
-                      s.o_rs % 4 == 0 && (reinterpret_cast<uintptr_t>(s.out) & 15) == 0 &&
-                      s.epilogue == MNI_EPI_NONE && !s.accumulate;  // (the rule of launch_skinny_cols_mr)
-    static int cache[5] = {-1, -1, -1, -1, -1};  // per (lean, x contiguous, tail)
-    const int slot = lean ? 4 : (variant & 4 ? 2 : 0) | (variant & 1);
+    if (skinny_decode_shape(s)) {  // (the rule of launch_skinny_cols_mr)
+        static int by_rows[17] = {-1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1, -1};
+        if (by_rows[s.rows] < 0) {
+            int n = 0;
+            hipError_t e = hipErrorInvalidValue;
+            switch (s.rows) {
+#define MNI_SK_LEAN(R) \
+    case R: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<R, true, true, false, true>, SK_THREADS, 0); break;
+                MNI_SK_DECODE_ROWS(MNI_SK_LEAN)
+#undef MNI_SK_LEAN
+            }
+            if (e != hipSuccess) { (void)hipGetLastError(); n = 0; }
+            by_rows[s.rows] = n;
+        }
+        return by_rows[s.rows];
+    }
+    static int cache[4] = {-1, -1, -1, -1};  // per (x contiguous, tail)
+    const int slot = (variant & 4 ? 2 : 0) | (variant & 1);
     if (cache[slot] < 0) {
         int n = 0;
         hipError_t e;
-        if (lean) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, true, true, false, true>, SK_THREADS, 0);
-        else if (slot == 0) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, false, true, false, false>, SK_THREADS, 0);
+        if (slot == 0) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, false, true, false, false>, SK_THREADS, 0);
         else if (slot == 1) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, false, true, true, false>, SK_THREADS, 0);
         else if (slot == 2) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, true, true, false, false>, SK_THREADS, 0);
         else e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<MR, true, true, true, false>, SK_THREADS, 0);

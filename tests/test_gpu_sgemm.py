@@ -811,14 +811,28 @@ def test_skinny_cols_wide_outputs_integer_exact(dev, rocm, m, n, k):
     rocm.sync()   # (a wait that expired would be reported here)
 
 
-@pytest.mark.parametrize("m", [4, 8, 16])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8, 16])
 def test_skinny_cols_decode_shape_integer_exact(dev, m):
-    # whole column groups, full row blocks, plain output: the specialised single-launch kernel
+    # whole column groups, plain output: the single-launch kernel specialised for the row count
     a = synth.small_ints(m, (m, 2048), 4)
     b = synth.small_ints(m + 1, (2048, 768), 4, stream=1)
     want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
     assert np.array_equal(run_gemm(dev, a, b, algo=N.ALGO_SKINNY)[0], want)
     assert np.array_equal(run_gemm(dev, a, b, algo=N.ALGO_SKINNY, split_k=5)[0], want)
+    assert np.array_equal(run_gemm(dev, a, b)[0], want)  # (what the planner picks for the shape)
+
+
+@pytest.mark.parametrize("m", [1, 3, 5, 7])
+def test_skinny_cols_decode_shape_normal_inputs(dev, m):
+    # the kernels specialised for a row count: within tolerance of a float64 product and of the two-launch form,
+    # and the same bits launch after launch
+    k, n = 4096, 1024
+    a = synth.normal(m, (m, k)); b = synth.normal(m + 1, (k, n), stream=1)
+    one = run_gemm(dev, a, b, algo=N.ALGO_SKINNY)[0]
+    assert np.array_equal(one, run_gemm(dev, a, b, algo=N.ALGO_SKINNY)[0])
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.abs(one - ref).max() <= gemm_tol(k, a, b)
+    assert max_err(one, run_gemm(dev, a, b, algo=N.ALGO_SKINNY_TWO_PASS)[0]) <= gemm_tol(k, a, b)
 
 
 @pytest.mark.parametrize("algo", SKINNY_ALGOS)
