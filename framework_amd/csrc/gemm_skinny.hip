@@ -80,16 +80,17 @@ template <int MR, bool XC, bool FUSED, bool TAIL, bool LEAN>
 __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLaunch s) {
     constexpr int U = SK_UNROLL;
     // LEAN (the decode shape): one batch, exactly MR rows, whole 256-column
-    // groups, row-major output, no epilogue -- known at compile time, so the
-    // general case's address arithmetic and guards drop out of a kernel whose
-    // whole life is a few microseconds.  Instantiated for every row count from
+    // groups, row-major output, a bias (if any) along the columns -- known at
+    // compile time, so the general case's address arithmetic and guards drop
+    // out of a kernel whose whole life is a few microseconds.  (The epilogue
+    // stays a run-time choice: it is applied once per output at the very end.)  Instantiated for every row count from
     // 1 to 8 (and 16): with the count a run-time value below MR the guards come
     // back and cost 0.4 (4 rows) to 0.9 us (8 rows); with the count rounded up
     // to 4 or 8, x[1,4096] W[4096,4096] took 12.8 us against 11.7, 5 rows 15.7
     // against 13.4 (MI355X, W in the Infinity Cache).
     static_assert(!LEAN || (XC && FUSED && !TAIL), "LEAN implies XC, FUSED, !TAIL");
     const int rows = LEAN ? MR : s.rows, batch = LEAN ? 1 : s.batch;
-    const int epilogue = LEAN ? (int)MNI_EPI_NONE : s.epilogue, accumulate = LEAN ? 0 : s.accumulate;
+    const int epilogue = s.epilogue, accumulate = s.accumulate;
     const int64_t o_cs = LEAN ? 1 : s.o_cs;
     const int x_bcount = LEAN ? 1 : s.x_bcount, w_bcount = LEAN ? 1 : s.w_bcount;
     __shared__ float4 red[SK_WAVES - 1][MR][64];
@@ -126,6 +127,28 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
     float4 acc[MR];
 #pragma unroll
     for (int i = 0; i < MR; ++i) acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+    // Decode shape: the bias (and, when nothing but a sum follows, the old output of an accumulating call) joins
+    // the sum as part of the first K slice's partial.  That workgroup is dispatched first and is done long before
+    // the reducers need its partial, so the loads cost nothing; asked for by the reducers -- whose own slices are
+    // the last to finish -- they put a dependent round trip (0.85 us for one row) at the end of the kernel.
+    const bool lean_activation = LEAN && epilogue >= MNI_EPI_BIAS_RELU;
+    if (LEAN && slice == 0 && wave == 0 && alive) {
+        if (epilogue != MNI_EPI_NONE) {
+            float bv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[e] = s.bias[col0 + e];
+#pragma unroll
+            for (int i = 0; i < MR; ++i) acc[i] = make_float4(bv[0], bv[1], bv[2], bv[3]);
+        }
+        if (accumulate && !lean_activation) {
+#pragma unroll
+            for (int i = 0; i < MR; ++i) {
+                const float4 old = *reinterpret_cast<const float4 *>(s.out + (int64_t)i * s.o_rs + col0);
+                acc[i].x += old.x; acc[i].y += old.y; acc[i].z += old.z; acc[i].w += old.w;
+            }
+        }
+    }
 
     for (int k0 = k_begin + wave * U; k0 < k_end; k0 += SK_WAVES * U) {
         f32x4 w[U];
@@ -280,7 +303,16 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
                 }
                 float *out = s.out + (int64_t)b * s.o_bs;
                 if (LEAN) {
-                    *reinterpret_cast<float4 *>(out + (int64_t)row * s.o_rs + col0) = make_float4(r[0], r[1], r[2], r[3]);
+                    float4 *dst = reinterpret_cast<float4 *>(out + (int64_t)row * s.o_rs + col0);
+                    if (lean_activation) {  // (the bias came in with the first slice's partial)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) r[e] = sk_epilogue(r[e], 0.0f, epilogue);
+                        if (accumulate) {
+                            const float4 old = *dst;
+                            r[0] += old.x; r[1] += old.y; r[2] += old.z; r[3] += old.w;
+                        }
+                    }
+                    *dst = make_float4(r[0], r[1], r[2], r[3]);
                     continue;
                 }
 #pragma unroll
@@ -468,11 +500,11 @@ int skinny_cols_rows_per_pass() { return SK_WAVES * SK_UNROLL; }
 
 // The decode shape, for which the single-launch form has an instantiation per row count (1 to 8, and 16): X rows
 // contiguous, K in whole groups of SK_UNROLL rows, one batch, whole 256-column groups, row-major 16-byte aligned
-// output, no epilogue.
+// output, the bias (if any) one value per column.
 static bool skinny_decode_shape(const SkinnyLaunch &s) {
     return s.x_cs == 1 && s.K % SK_UNROLL == 0 && s.batch == 1 && (s.rows <= 8 || s.rows == 16) && s.cols % SK_COLS == 0 &&
-           s.o_cs == 1 && s.o_rs % 4 == 0 && (reinterpret_cast<uintptr_t>(s.out) & 15) == 0 && s.epilogue == MNI_EPI_NONE &&
-           !s.accumulate;
+           s.o_cs == 1 && s.o_rs % 4 == 0 && (reinterpret_cast<uintptr_t>(s.out) & 15) == 0 && !s.bias_on_rows &&
+           s.epilogue <= MNI_EPI_BIAS_GELU;
 }
 #define MNI_SK_DECODE_ROWS(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(16)
 

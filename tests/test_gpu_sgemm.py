@@ -822,6 +822,31 @@ def test_skinny_cols_decode_shape_integer_exact(dev, m):
     assert np.array_equal(run_gemm(dev, a, b)[0], want)  # (what the planner picks for the shape)
 
 
+@pytest.mark.parametrize("m", [1, 4, 6, 16])
+def test_skinny_cols_decode_shape_epilogues_and_accumulate(dev, rocm, m):
+    # bias, activation and accumulation in the kernels specialised for a row count (the bias and, without an
+    # activation, the old output enter the sum with the first K slice)
+    k, n = 1024, 512
+    a = synth.small_ints(m, (m, k), 3); b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+    bias = synth.small_ints(m + 2, (n,), 5, stream=2); old = synth.small_ints(m + 3, (m, n), 9, stream=3)
+    prod = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float64)
+    dA, dB, dBias = dev.put(a), dev.put(b), dev.put(bias)
+    for epi, accumulate in [(N.EPI_NONE, True), (N.EPI_BIAS, False), (N.EPI_BIAS, True), (N.EPI_BIAS_RELU, False),
+                            (N.EPI_BIAS_RELU, True), (N.EPI_BIAS_GELU, False), (N.EPI_BIAS_GELU, True)]:
+        z = prod + (bias if epi != N.EPI_NONE else 0.0)
+        if epi == N.EPI_BIAS_RELU: z = np.maximum(z, 0.0)
+        if epi == N.EPI_BIAS_GELU: z = 0.5 * z * (1.0 + np.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        want = z + (old if accumulate else 0.0)
+        for algo in (N.ALGO_AUTO, N.ALGO_SKINNY, N.ALGO_SKINNY_TWO_PASS):
+            dC = dev.put(old)
+            rocm.sgemm(m, n, k, dA, dB, dC, bias=dBias if epi != N.EPI_NONE else None, epilogue=epi, accumulate=accumulate, algo=algo)
+            got = rocm.to_host(dC, (m, n))
+            if epi == N.EPI_BIAS_GELU:
+                assert np.abs(got - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), (epi, accumulate, algo)
+            else:
+                assert np.array_equal(got, want.astype(np.float32)), (epi, accumulate, algo)
+
+
 @pytest.mark.parametrize("m", [1, 3, 5, 7])
 def test_skinny_cols_decode_shape_normal_inputs(dev, m):
     # the kernels specialised for a row count: within tolerance of a float64 product and of the two-launch form,
