@@ -104,7 +104,7 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         s.out = d.C; s.o_bs = d.c_batch_stride; s.bias = d.bias;
         s.epilogue = d.epilogue; s.accumulate = d.accumulate;
         s.ws = nullptr; s.split_k = 1; s.k_per_slice = s.K;
-        s.groups = 0; s.flags = nullptr; s.epoch = 0; s.status = ctx().status_dev;
+        s.groups = 0; s.flags = nullptr; s.epoch = 0; s.max_reducers = 16; s.status = ctx().status_dev;
 
         const bool w_batch_ok = s.w_bcount <= 1 || (s.w_bs % 4) == 0;
         const bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
@@ -143,11 +143,16 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
                 // The reducers of a unit (the workgroups of its last min(rows, slices) slices) wait for all of its
                 // slices while they hold their places on the CUs: every reducer of an XCD must fit on it at once,
                 // or the first ones could fill it and wait for slices that are never dispatched.
+                // With more rows than that leaves room for, a unit gets fewer reducers, each taking several rows.
                 const int cus = c.compute_units > 0 ? c.compute_units : 256;
                 const int64_t units_per_xcd = ((int64_t)groups * s.batch + c.xcd_count - 1) / c.xcd_count;
-                const int64_t reducers_per_xcd = units_per_xcd * (s.rows < split ? s.rows : split);
                 const int64_t room_per_xcd = (int64_t)skinny_cols_fused_occupancy(s) * (cus / c.xcd_count);
-                fused = reducers_per_xcd <= room_per_xcd;
+                // (Up to 8 rows: 8 x 50304 x 768 33.6 us with 5 reducers per unit against 43.2 in two launches.  Not the
+                // 16-row form, one workgroup per CU: 12 x 8192 x 8192 72.5 us with 8 reducers per unit, 58.2 in two launches.)
+                const int64_t per_unit = room_per_xcd / units_per_xcd;
+                const int64_t wanted = s.rows < split ? s.rows : split;
+                fused = s.rows <= 8 ? per_unit >= 1 : per_unit >= wanted;
+                s.max_reducers = (int)(per_unit < 16 ? per_unit : 16);
             }
             void *ws = nullptr;
             if (split > 1) {

@@ -97,6 +97,9 @@ struct SkinnyLaunch {
     // a fourth costs the kernel's start a further scalar fetch.)
     unsigned *flags;
     unsigned epoch;
+    // Single-launch form: at most this many workgroups per unit add up its slices (each then takes every
+    // max_reducers-th row).  Reducers hold their places while they wait, so all of an XCD's must fit on it at once.
+    int max_reducers;
     unsigned *status;  // device status word: set when a reducer's bounded wait expires
 };
 // W with unit stride along j (cols): lanes own columns, K split over wavefronts and slices.

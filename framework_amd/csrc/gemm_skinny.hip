@@ -52,9 +52,11 @@ __device__ __forceinline__ float sk_epilogue(float v, float bias, int epilogue) 
 //    included, and a workgroup that waits keeps its place on its CU: were there
 //    more reducers on an XCD than workgroups fit on it together, the first
 //    ones could fill it and wait for slices that are never dispatched.  The
-//    host therefore takes this form only when all reducers of an XCD fit on it
-//    at once (skinny_cols_fused_occupancy); the non-reducers ahead of them in
-//    the grid never wait and make room as they finish.  The poll is bounded
+//    host therefore limits the reducers of a unit (max_reducers; each then
+//    takes every max_reducers-th row) so that all reducers of an XCD fit on it
+//    at once (skinny_cols_fused_occupancy), and takes the two-launch form when
+//    not even one per unit does; the non-reducers ahead of them in the grid
+//    never wait and make room as they finish.  The poll is bounded
 //    all the same, and a reducer that gives up writes NaN and raises the
 //    device status word.
 //    Measured on MI355X for x[4,4096] W[4096,4096]: 12.2 us against 15.8 us for
@@ -246,7 +248,7 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the partial has reached L2
             if (lane == 0) flags[slice] = s.epoch;
         }
-        const int reducers = min(rows, s.split_k);
+        const int reducers = min(min(rows, s.split_k), s.max_reducers);
         const int q = s.split_k - 1 - slice;
         if (q >= reducers) return;
 
