@@ -177,7 +177,11 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
             gemm_ws_free(ws);
             return true;
         }
-        if (w_dots && d.split_k <= 1) {
+        // W contiguous along K: one wavefront per output column.  By itself only up to 8 rows -- its 16-row
+        // instantiation is behind the tile kernel's 64 x 64 tiles in K slices on every shape measured (MI355X, us,
+        // dots at 9 / 16 rows against tiles: [50304, 768] 80 / 95 against 48, [4096, 4096] 26 / 28 against 24,
+        // [1024, 4096] 22 / 25 against 12, [11008, 4096] 56 / 61 against 58).
+        if (w_dots && d.split_k <= 1 && (s.rows <= 8 || d.algo != MNI_ALGO_AUTO)) {
             *rc = launch_skinny_dots(s);
             return true;
         }
