@@ -109,8 +109,29 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         const bool w_batch_ok = s.w_bcount <= 1 || (s.w_bs % 4) == 0;
         const bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
         const bool x_batch_ok = s.x_bcount <= 1 || (s.x_bs % 4) == 0;
-        const bool w_dots = s.w_rs == 1 && (s.w_cs % 4) == 0 && (s.K % 4) == 0 && aligned16(s.W) && w_batch_ok &&
-                            s.x_cs == 1 && (s.x_rs % 4) == 0 && aligned16(s.X) && x_batch_ok;
+        // (the pitch of X only matters from the second row on)
+        const bool x_dots = s.x_cs == 1 && (s.rows == 1 || (s.x_rs % 4) == 0) && aligned16(s.X) && x_batch_ok;
+        const bool w_dots_w = s.w_rs == 1 && (s.w_cs % 4) == 0 && (s.K % 4) == 0 && aligned16(s.W) && w_batch_ok;
+        bool w_dots = w_dots_w && x_dots;
+        // By itself the dots kernel takes up to 8 rows of a K of at least 512 (see below).  Then it also pays to
+        // bring a small operand that is not laid out along K -- the [K, n] weight of a head with a few outputs
+        // under a tall activation matrix -- into that layout first, with one small copy launch, when the big
+        // operand is worth it (65536 x 768 against [768, 2]: 72 us through the tile kernel, 31 + 3 this way).
+        void *packed = nullptr;
+        // (At 8 rows the copy eats what the kernel gains over the tile kernel -- unless that kernel is on its slow
+        // loads because the row count is not a multiple of 4.)
+        if (w_dots_w && !x_dots && !w_cols && d.algo == MNI_ALGO_AUTO && d.split_k <= 1 && (s.rows <= 4 || (s.rows <= 8 && s.rows % 4 != 0)) &&
+            s.K >= 512 &&
+            (int64_t)s.cols * s.K * s.batch >= (2LL << 20)) {
+            const int64_t xb = s.x_bcount > 1 ? s.x_bcount : 1;
+            *rc = gemm_ws_alloc(&packed, (size_t)(xb * s.rows * s.K) * sizeof(float));
+            if (*rc != MNI_OK) return true;
+            const int64_t shape[3] = {xb, s.rows, s.K}, strides[3] = {s.x_bs, s.x_rs, s.x_cs};
+            *rc = k_strided_copy((float *)packed, s.X, shape, strides, 3);
+            if (*rc != MNI_OK) { gemm_ws_free(packed); return true; }
+            s.X = (const float *)packed; s.x_cs = 1; s.x_rs = s.K; s.x_bs = (int64_t)s.rows * s.K;
+            w_dots = true;
+        }
 
         if (w_cols) {
             // Slice K until about 4 workgroups per CU exist (every CU streams,
@@ -181,10 +202,13 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         // instantiation is behind the tile kernel's 64 x 64 tiles in K slices on every shape measured (MI355X, us,
         // dots at 9 / 16 rows against tiles: [50304, 768] 80 / 95 against 48, [4096, 4096] 26 / 28 against 24,
         // [1024, 4096] 22 / 25 against 12, [11008, 4096] 56 / 61 against 58).
-        if (w_dots && d.split_k <= 1 && (s.rows <= 8 || d.algo != MNI_ALGO_AUTO)) {
+        // Nor for a short K, where half its lanes have nothing to load (100000 x 128 against 8 columns: 55 us, tiles 22).
+        if (w_dots && d.split_k <= 1 && ((s.rows <= 8 && s.K >= 512) || d.algo != MNI_ALGO_AUTO)) {
             *rc = launch_skinny_dots(s);
+            gemm_ws_free(packed);
             return true;
         }
+        gemm_ws_free(packed);
         // Both extents small: the other orientation may be eligible.
         if (attempt == 0 && !swapped && d.N <= 16) swapped = true;
         else break;
@@ -585,6 +609,28 @@ int sgemm(const mni_gemm_desc &d) {
             return set_error(MNI_ERR_INVALID,
                              "sgemm: shape/layout not eligible for the skinny kernels "
                              "(needs min(M,N) <= 16 and 16-byte aligned unit-stride W)");
+    }
+    // A small N-contiguous B whose rows are not whole 16-byte pieces (N = 10 under a tall A) leaves the tile
+    // kernel its element-wise loads of B; copied once into a K-contiguous layout it is read in 16-byte pieces
+    // (65536 x 768 against [768, 10]: 77 us as given, 50 with the copy).  Not in the entry point that may not
+    // allocate: the plan's own workspace has the one fixed block.
+    if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && !ctx().scratch && d.B.col_stride == 1 && d.N > 1 &&
+        (d.B.row_stride % 4 != 0 || !aligned16(d.B.ptr) || (d.B.batch_count > 1 && d.B.batch_stride % 4 != 0)) && d.K % 4 == 0 &&
+        d.K * d.N * d.B.batch_count <= (1 << 18) && d.M * d.K * d.batch >= 16 * d.K * d.N * d.B.batch_count && d.M * d.K * d.batch >= (1LL << 20)) {
+        void *packed = nullptr;
+        MNI_TRY(gemm_ws_alloc(&packed, (size_t)(d.K * d.N * d.B.batch_count) * sizeof(float)));
+        const int64_t shape[3] = {d.B.batch_count, d.N, d.K}, strides[3] = {d.B.batch_stride, d.B.col_stride, d.B.row_stride};
+        int rc = k_strided_copy((float *)packed, d.B.ptr, shape, strides, 3);
+        if (rc == MNI_OK) {
+            mni_gemm_desc d2 = d;
+            d2.B.ptr = (const float *)packed;
+            d2.B.row_stride = 1;
+            d2.B.col_stride = d.K;
+            d2.B.batch_stride = d.K * d.N;
+            rc = run_mfma(d2);
+        }
+        gemm_ws_free(packed);
+        return rc;
     }
     return run_mfma(d);
 }

@@ -899,6 +899,29 @@ def test_skinny_single_launch_repeats_and_matches_two_pass(dev, rocm):
     assert max_err(first, two) <= gemm_tol(4096, a, w)
 
 
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 9, 10, 13, 17])
+def test_few_output_columns_under_a_tall_operand_integer_exact(dev, rocm, n):
+    # A head with a few outputs: the [K, n] weight is small and, for most n, not laid out for 16-byte loads.  The
+    # planner copies it into a K-contiguous layout first (for the dots kernel up to 8 columns, for the tile
+    # kernel beyond) when the tall operand is big enough to pay for the extra launch; same sums either way.
+    m, k = 2048, 640
+    a = synth.small_ints(n, (m, k), 3); b = synth.small_ints(n + 1, (k, n), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b)[0], want)
+    # batched, with one weight per batch and with a shared one
+    a3 = synth.small_ints(n + 2, (3, 1024, 512), 3); b3 = synth.small_ints(n + 3, (3, 512, n), 3, stream=1)
+    want3 = np.einsum("bmk,bkn->bmn", a3.astype(np.int64), b3.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a3, b3), want3)
+    want1 = np.einsum("bmk,kn->bmn", a3.astype(np.int64), b3[0].astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a3, b3[:1]), want1)
+    # with a bias along the few columns, accumulating
+    bias = synth.small_ints(n + 4, (n,), 5, stream=2); old = synth.small_ints(n + 5, (m, n), 9, stream=3)
+    dA, dB, dBias, dC = dev.put(a), dev.put(b), dev.put(bias), dev.put(old)
+    rocm.sgemm(m, n, k, dA, dB, dC, bias=dBias, epilogue=N.EPI_BIAS_RELU, accumulate=True)
+    z = np.maximum(want.astype(np.float64) + bias, 0.0) + old
+    assert np.array_equal(rocm.to_host(dC, (m, n)), z.astype(np.float32))
+
+
 @pytest.mark.parametrize("m", [1, 4, 16])
 def test_skinny_dots_integer_exact(dev, m):
     a = synth.small_ints(m, (m, 1024), 4)
