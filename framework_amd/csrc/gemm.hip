@@ -43,7 +43,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_FEWROWS)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_OUTER)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -257,7 +257,7 @@ static void fill_launch(GemmLaunch &g, const mni_gemm_desc &d) {
 
 // What run_mfma would launch for a product, for a caller that wants to know before anything is launched.
 struct PlanProbe {
-    enum { TILE = 0, PANEL = 1, DIRECT = 2, TILE_FUSED_GELU = 3, TILE_STREAMK = 4, FEWROWS = 5 };
+    enum { TILE = 0, PANEL = 1, DIRECT = 2, TILE_FUSED_GELU = 3, TILE_STREAMK = 4, FEWROWS = 5, OUTER = 6 };
     int kind, bm, bn, split, amode, bmode;
     GemmLaunch g;  // kind TILE: the launch descriptor, complete
 };
@@ -272,6 +272,19 @@ static int fewrows_split(const GemmLaunch &g, int cus) {
     if (split > g.K / 128) split = g.K / 128;
     if (split > 32) split = 32;
     return split < 1 ? 1 : (int)split;
+}
+// Whether the short-K outer-product kernel is the plan for an eligible product.  It costs what writing C costs
+// plus ~0.2 us per pair of K values of a wavefront; the tile kernel's 64 x 64 tiles pay a fixed prologue and
+// epilogue per tile and little per K step.  Measured on MI355X, us, outer against tiles, K = 8 / 32 / 64:
+// 4096 x 4096 17.2 / 20.2 / 29.0 against 28.7 / 26.0 / 33.1 (K = 128: 49.4 / 46.3); 4096 x 11008 34.3 / 40.1 / 67.6
+// against 68.4 / 62.2 / 82.7; 2048 x 2048 6.7 / 9.0 / 12.2 against 10.1 / 9.3 / 11.0; 768 x 3072 6.4 / 8.6 / 11.7
+// against 8.7 / 8.0 / 9.3; 768 x 768 5.5 / 7.7 / 10.8 against 6.0 / 5.7 / 6.1.
+static bool outer_plan(const GemmLaunch &g, int cus) {
+    (void)cus;
+    const int64_t outputs = (int64_t)g.M * g.N * g.batch;
+    if (outputs >= (1LL << 24)) return g.K <= 64;
+    if (outputs >= (1LL << 21)) return g.K <= 24;
+    return outputs >= (1LL << 16) && g.K <= 8;
 }
 // Whether the few-rows kernel is the plan for an eligible product: from about 512 x 512 of W on it is ahead of the
 // tile kernel's 64 x 64 tiles in K slices (us, 32 rows: 512 x 512 7.8 / 15.1, 1024 x 1024 8.8 / 11.7, 4096 x 4096
@@ -347,6 +360,20 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
         g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
         if (probe) { probe->kind = PlanProbe::PANEL; return MNI_OK; }
         return launch_gemm_panel(g, amode, bmode);
+    }
+    // Short-K outer-product form (both operands contiguous along the output axes): forced, or chosen by outer_plan.
+    if (d.algo == MNI_ALGO_OUTER || (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_outer_eligible(g) && outer_plan(g, cus))) {
+        if (!gemm_outer_eligible(g))
+            return set_error(MNI_ERR_INVALID, "sgemm: the short-K outer-product kernel takes an A contiguous along M and a B contiguous along N, "
+                                              "K <= 128, N %% 4 == 0, B and C 16-byte aligned, no epilogue");
+        if (d.split_k > 1) return set_error(MNI_ERR_INVALID, "sgemm: the short-K outer-product kernel takes no split_k");
+        g.tiles_m = (g.M + 127) / 128;
+        g.tiles_n = (g.N + 127) / 128;
+        g.split_k = 1;
+        g.k_per_slice = g.K;
+        g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
+        if (probe) { probe->kind = PlanProbe::OUTER; return MNI_OK; }
+        return launch_gemm_outer(g);
     }
     // Few-rows form (9 to 32 rows against a wide N-contiguous operand): forced, or chosen by fewrows_plan.
     {

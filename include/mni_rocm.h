@@ -143,9 +143,15 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * read once, straight into the matrix instruction's registers, K slices
  * (split_k, 0 = chosen) summed inside the launch (error unless K % 8 == 0,
  * N % 4 == 0, N >= 128, K >= 64, operands and C 16-byte aligned with row
- * strides in whole 16 bytes).  AUTO picks among them. */
+ * strides in whole 16 bytes); OUTER = a short K (<= 128) under a large
+ * output with A contiguous along M and B along N -- the weight gradient
+ * X^T dY of a small batch: both operands straight into the matrix
+ * instruction's registers, the cost of writing C (error unless N % 4 == 0,
+ * B and C 16-byte aligned with row strides in whole 16 bytes, no epilogue;
+ * accumulate is honoured).  AUTO picks among them. */
 enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
-       MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7, MNI_ALGO_TINY = 8, MNI_ALGO_FEWROWS = 9 };
+       MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7, MNI_ALGO_TINY = 8, MNI_ALGO_FEWROWS = 9,
+       MNI_ALGO_OUTER = 10 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),

@@ -899,6 +899,51 @@ def test_skinny_single_launch_repeats_and_matches_two_pass(dev, rocm):
     assert max_err(first, two) <= gemm_tol(4096, a, w)
 
 
+@pytest.mark.parametrize("nin,nout,rows,batch", [(128, 128, 8, 1), (100, 132, 7, 1), (33, 4, 1, 1), (300, 260, 33, 2), (257, 516, 128, 3),
+                                                 (64, 64, 2, 1), (1000, 640, 5, 1), (31, 1028, 19, 4)])
+def test_outer_product_kernel_integer_exact(dev, rocm, nin, nout, rows, batch):
+    # dW[b] = X[b]^T dY[b] of a small batch: K = its rows, A the transposed view of X, both operands contiguous along
+    # the output axes.  Forced and as planned; overwriting and accumulating; edges in both extents, odd K.
+    x = synth.small_ints(rows + nin, (batch, rows, nin), 3); dy = synth.small_ints(rows + nout, (batch, rows, nout), 3, stream=1)
+    old = synth.small_ints(5, (batch, nin, nout), 7, stream=2)
+    want = np.einsum("bki,bkn->bin", x.astype(np.int64), dy.astype(np.int64)).astype(np.float32)
+    dX, dY = dev.put(x), dev.put(dy)
+    for algo in (N.ALGO_OUTER, N.ALGO_AUTO, N.ALGO_MFMA_SMALL):
+        for accumulate in (False, True):
+            dC = dev.put(old)
+            rocm.sgemm(nin, nout, rows, dX, dY, dC, batch=batch, a_strides=(1, nin), a_batch=(rows * nin, batch),
+                       b_batch=(rows * nout, batch), accumulate=accumulate, algo=algo)
+            assert np.array_equal(rocm.to_host(dC, (batch, nin, nout)), want + (old if accumulate else 0)), (algo, accumulate)
+    # one X against a dY per batch (X's batch count 1), into a padded C
+    dC = dev.empty(batch * nin * (nout + 4), fill=-7.0)
+    rocm.sgemm(nin, nout, rows, dX, dY, dC, batch=batch, a_strides=(1, nin), a_batch=(0, 1), b_batch=(rows * nout, batch),
+               ldc=nout + 4, c_batch_stride=nin * (nout + 4), algo=N.ALGO_OUTER)
+    got = rocm.to_host(dC, (batch, nin, nout + 4))
+    want1 = np.einsum("ki,bkn->bin", x[0].astype(np.int64), dy.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(got[:, :, :nout], want1) and np.all(got[:, :, nout:] == -7.0)
+
+
+def test_outer_product_kernel_is_the_plan_for_a_small_batch_weight_gradient_and_refuses_other_layouts(dev, rocm):
+    rows, nin, nout = 16, 2048, 4096
+    x = synth.normal(1, (rows, nin)); dy = synth.normal(2, (rows, nout), stream=1)
+    dX, dY, dC = dev.put(x), dev.put(dy), dev.empty(nin * nout)
+    before = rocm.launch_count()
+    rocm.sgemm(nin, nout, rows, dX, dY, dC, a_strides=(1, nin))
+    assert rocm.launch_count() - before == 1
+    got = rocm.to_host(dC, (nin, nout))
+    ref = x.astype(np.float64).T @ dy.astype(np.float64)
+    assert np.abs(got - ref).max() <= gemm_tol(rows, x, dy)
+    forced = dev.empty(nin * nout)
+    rocm.sgemm(nin, nout, rows, dX, dY, forced, a_strides=(1, nin), algo=N.ALGO_OUTER)
+    assert np.array_equal(rocm.to_host(forced, (nin, nout)), got)  # the planner's choice was this kernel
+    bias = dev.put(np.zeros(nout, np.float32))
+    for kw in (dict(), dict(a_strides=(1, nin), bias=bias, epilogue=N.EPI_BIAS), dict(a_strides=(1, nin), split_k=2)):
+        with pytest.raises(N.MniError):   # K-contiguous A; an epilogue; K slices
+            rocm.sgemm(nin, nout, rows, dX, dY, dC, algo=N.ALGO_OUTER, **kw)
+    with pytest.raises(N.MniError):       # K beyond the kernel's limit
+        rocm.sgemm(64, 64, 200, dX, dY, dC, a_strides=(1, 64), algo=N.ALGO_OUTER)
+
+
 @pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 9, 10, 13, 17])
 def test_few_output_columns_under_a_tall_operand_integer_exact(dev, rocm, n):
     # A head with a few outputs: the [K, n] weight is small and, for most n, not laid out for 16-byte loads.  The
