@@ -225,6 +225,23 @@ def bench_extras(r, with_cpu):
         r.free(xb)
         r.free(yb)
     out["decode_batch_rows_x_4096x4096_cold"] = rows_out
+    # the weight gradient of the same layer under a small batch: dW[4096,4096] = X^T[4096,rows] dY[rows,4096], X^T as a
+    # view (matmul_backward's second product with K = the batch's rows): bound by writing dW -- not a BASELINE config
+    grad_out = {}
+    dwg = r.malloc(4096 * 4096 * 4)
+    for mrows in (8, 32):
+        xb = r.to_device(synth.normal(6, (mrows, 4096)))
+        gb = r.to_device(synth.normal(7, (mrows, 4096)))
+        for accumulate in (False, True):
+            d = r.gemm_desc(4096, 4096, mrows, xb, gb, dwg, a_strides=(1, 4096), accumulate=accumulate)
+            us = r.sgemm_timed([d], 300, 200) * 1e3
+            byb = 4.0 * (4096 * 4096 * (2 if accumulate else 1) + 2 * mrows * 4096)
+            grad_out["%d_rows%s" % (mrows, "_accumulating" if accumulate else "")] = {
+                "us": us, "GB/s": byb / us / 1e3, "frac_hbm": byb / us / 1e3 / PEAK_HBM_GBPS, "TFLOP/s": 2.0 * mrows * 4096 * 4096 / us / 1e6}
+        r.free(xb)
+        r.free(gb)
+    r.free(dwg)
+    out["weight_gradient_4096x4096_of_a_small_batch"] = grad_out
     for p in ws + [dx, dw, dy]:
         r.free(p)
     # ---- config 5b: X^T[1024,65536] dY[65536,1024], X^T as a view, split-K -------------------------------------
