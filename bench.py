@@ -529,6 +529,13 @@ def run_for_counters(r, which):
             r.sgemm(32, 4096, 4096, x, w, dst)
         for _ in range(5):
             r.sgemm(32, 8192, 8192, x, w, dst)
+    elif which == "outer":
+        # the weight gradient of a [4096, 4096] layer under 8 rows (the outer-product kernel), overwriting and
+        # accumulating, 5 launches each
+        x, gy = r.to_device(synth.normal(6, (8, 4096))), r.to_device(synth.normal(7, (8, 4096)))
+        for accumulate in (False, True):
+            for _ in range(5):
+                r.sgemm(4096, 4096, 8, x, gy, dst, a_strides=(1, 4096), accumulate=accumulate)
     elif which == "attention":
         # the one-kernel attention forward on [8, 8192, 64], causal, through the engine entry point
         from framework_amd.api import bind
@@ -592,7 +599,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
-    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "fewrows", "attention", "attention_bwd"], default=None,
+    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "fewrows", "outer", "attention", "attention_bwd"], default=None,
                     help="for rocprofv3 --pmc runs: launch a copy kernel of known size (64 MiB read + 64 MiB "
                          "written) 3 times, then the chosen product 5 times, and exit")
     args = ap.parse_args()
