@@ -479,10 +479,11 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
         // tiles take ideal / fill, stream-K ideal x 1.03-1.05; 2560^3 with 64 x 64 tiles at 89 % loses 10 %
         // to stream-K, 4096 x 768 x 3072 with 64 x 64 tiles at 100 % beats it by 10 %.)
         if (ktiles >= 8 && d.split_k == 0 && d.algo == MNI_ALGO_AUTO) {
-            // Up to 32 K steps the smaller shapes run 1-3 % ahead (more workgroups to overlap prologues and
-            // epilogues with), except with A given as its transpose.
+            // Up to 32 K steps the smaller shapes run ahead (more workgroups to overlap prologues and epilogues
+            // with): 1-3 % with A along K, and with A given as its transpose 4096 x 11008 x 128 137.5 -> 119.4 us,
+            // 768 x 3072 x 256 24.3 -> 17.3, 8192 x 8192 x 128 187.5 -> 173.6, 4096 x 4096 x 1024 246.5 -> 244.6.
             const int cand[4][2] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
-            const bool small_first = ktiles <= 32 && amode != 1;
+            const bool small_first = ktiles <= 32;
             for (int i = 0; i < 4 && !whole_tiles; ++i) {
                 const int cm = cand[small_first ? 3 - i : i][0], cn = cand[small_first ? 3 - i : i][1];
                 if (cm > bm || cn > bn) continue;
@@ -522,7 +523,14 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
                     whole_tiles = true;
                 } else {
                     streamk = streamk_fits(64, 64, 8);
-                    if (streamk) bm = bn = 64;
+                    if (streamk) {
+                        bm = bn = 64;
+                    } else if (ktiles <= 32) {
+                        // too few K steps to deal: whole 64 x 64 tiles all the same, the last round part empty
+                        // (768 x 3072 x 256, 576 tiles: 17.5 us against 24.4 for 128 x 128 tiles in K slices)
+                        bm = bn = 64;
+                        whole_tiles = true;
+                    }
                 }
             }
         } else {
@@ -530,7 +538,11 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
             // 128 x 128 tiles would leave the machine with few, short-lived workgroups
             const int64_t t128 = (int64_t)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
             const int64_t big_split = d.split_k > 0 ? d.split_k : (ktiles / 8 > 0 ? ktiles / 8 : 1);
-            if ((bm == 128 || bn == 128) && ((g.K <= 256 && t128 < 4LL * cus) || t128 * big_split < 2LL * cus)) bm = bn = 64;
+            // (fewer than 8 K steps: 64 x 64 whatever the tile count -- a tile is mostly prologue and epilogue, and the
+            // small ones overlap them better; in every layout 4096 x 11008 x 64 98 -> 82 us, 8192 x 8192 x 128 187 -> 173,
+            // 2048 x 8192 x 32 30.6 -> 26.8, 4096 x 4096 x 192 62 -> 60)
+            if ((bm == 128 || bn == 128) && ((ktiles < 8 && d.split_k == 0) || (g.K <= 256 && t128 < 4LL * cus) || t128 * big_split < 2LL * cus))
+                bm = bn = 64;
         }
         if (d.algo == MNI_ALGO_MFMA_STREAMK && !streamk) {
             if (!sk_device) return set_error(MNI_ERR_INVALID, "sgemm: stream-K needs a confirmed workgroup-to-XCD mapping");
