@@ -274,17 +274,17 @@ static int fewrows_split(const GemmLaunch &g, int cus) {
     return split < 1 ? 1 : (int)split;
 }
 // Whether the short-K outer-product kernel is the plan for an eligible product.  It costs what writing C costs
-// plus ~0.2 us per pair of K values of a wavefront; the tile kernel's 64 x 64 tiles pay a fixed prologue and
-// epilogue per tile and little per K step.  Measured on MI355X, us, outer against tiles, K = 8 / 32 / 64:
-// 4096 x 4096 17.2 / 20.2 / 29.0 against 28.7 / 26.0 / 33.1 (K = 128: 49.4 / 46.3); 4096 x 11008 34.3 / 40.1 / 67.6
-// against 68.4 / 62.2 / 82.7; 2048 x 2048 6.7 / 9.0 / 12.2 against 10.1 / 9.3 / 11.0; 768 x 3072 6.4 / 8.6 / 11.7
-// against 8.7 / 8.0 / 9.3; 768 x 768 5.5 / 7.7 / 10.8 against 6.0 / 5.7 / 6.1.
+// plus the MFMAs of a wavefront's K pairs, which nothing hides when all wavefronts start together; the tile
+// kernel's 64 x 64 tiles pay a fixed prologue and epilogue per tile and little per K step.  Measured on MI355X,
+// us, outer against tiles, K = 8 / 32 / 64 / 128: 4096 x 4096 15.3 / 18.1 / 23.8 / 38.0 against 29.0 / 25.9 / 33.0 /
+// 46.4; 4096 x 11008 32.6 / 41.0 / 62.2 / 102 against 68.4 / 61.9 / 82.4 / 119; 2048 x 2048 5.7 / 6.9 / 8.9 / 12.3
+// against 10.2 / 9.2 / 11.0 / 14.2; 768 x 3072 3.9 / 5.9 / 7.8 / 11.7 against 8.1 / 7.9 / 9.3 / 11.8; 768 x 768
+// 3.6 / 5.1 / 7.0 / 10.8 against 5.9 / 5.7 / 6.1 / 7.2.
 static bool outer_plan(const GemmLaunch &g, int cus) {
     (void)cus;
     const int64_t outputs = (int64_t)g.M * g.N * g.batch;
-    if (outputs >= (1LL << 24)) return g.K <= 64;
-    if (outputs >= (1LL << 21)) return g.K <= 24;
-    return outputs >= (1LL << 16) && g.K <= 8;
+    if (outputs >= (1LL << 21)) return true;  // (eligible: K <= 128)
+    return outputs >= (1LL << 16) && g.K <= 48;  // (512 x 512: K = 48 5.9 against 6.8, K = 64 6.9 against 6.0)
 }
 // Whether the few-rows kernel is the plan for an eligible product: from about 512 x 512 of W on it is ahead of the
 // tile kernel's 64 x 64 tiles in K slices (us, 32 rows: 512 x 512 7.8 / 15.1, 1024 x 1024 8.8 / 11.7, 4096 x 4096

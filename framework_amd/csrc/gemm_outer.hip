@@ -47,45 +47,70 @@ __global__ __launch_bounds__(256) void gemm_outer_kernel(const GemmLaunch g) {
     const int batch = blockIdx.z;
     if (m0 >= g.M) return;  // (a whole wavefront; nothing in this kernel waits for another wavefront)
 
-    // rows beyond M repeat the last one, columns beyond N (N % 4 == 0) the last four: neither is stored
-    const float *ap = g.A + (int64_t)(batch % g.a_bcount) * g.a_bs + min(m0 + i, g.M - 1);
-    const float *bp = g.B + (int64_t)(batch % g.b_bcount) * g.b_bs + min(n0 + 4 * i, g.N - 4);
+    // rows beyond M repeat the last one, columns beyond N (N % 4 == 0) the last four: neither is stored.
+    // Loads are buffer loads whose per-lane part (row or column, and which of the pair's two K values) is fixed
+    // and whose moving part (the K pair) is a scalar offset: the loop has no vector-ALU work between its MFMAs
+    // (computing addresses and zeroing the unused half of an odd K per load made a K pair cost 470 cycles for
+    // 256 of MFMAs).
+    const __amdgpu_buffer_rsrc_t ar = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(g.A + (int64_t)(batch % g.a_bcount) * g.a_bs), 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(g.B + (int64_t)(batch % g.b_bcount) * g.b_bs), 0, -1, 0x00020000);
+    const int arow = min(m0 + i, g.M - 1), bcol = min(n0 + 4 * i, g.N - 4);
+    const int a_cs = (int)g.a_cs, b_rs = (int)g.b_rs;  // (offsets fit 32 bits: checked at launch)
+    const int va = (arow + h * a_cs) * 4, vb = (bcol + h * b_rs) * 4;
+    const int sa = 8 * a_cs, sb = 8 * b_rs;  // bytes from one K pair to the next
     floatx16 acc[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[j][e] = 0.0f;
-
-    // K values 2 s + h; one past an odd K repeats the last (a valid address) and is multiplied as zeros.  The
-    // next group of OU_PAIRS pairs is requested before the current one is multiplied (a group is one round trip
-    // to memory, and a small output has no other wavefront to hide it behind).  No branch around a load: the
-    // compiler would then wait for every load in flight at each use; requests past the end repeat the last row.
-    const int pairs = (g.K + 1) >> 1;
-    float a[OU_PAIRS], an[OU_PAIRS];
-    f32x4 b[OU_PAIRS], bn[OU_PAIRS];
-    auto request = [&](int s0, float (&ra)[OU_PAIRS], f32x4 (&rb)[OU_PAIRS]) {
-#pragma unroll
-        for (int u = 0; u < OU_PAIRS; ++u) {
-            const int k = min(2 * (s0 + u) + h, g.K - 1);
-            ra[u] = ap[(int64_t)k * g.a_cs];
-            rb[u] = *reinterpret_cast<const f32x4 *>(bp + (int64_t)k * g.b_rs);
-        }
+    auto multiply = [&](float av, const f32x4 &bv) {
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv.x, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv.y, acc[1], 0, 0, 0);
+        acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv.z, acc[2], 0, 0, 0);
+        acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv.w, acc[3], 0, 0, 0);
     };
-    request(0, a, b);
-    for (int s0 = 0; s0 < pairs; s0 += OU_PAIRS) {
-        request(s0 + OU_PAIRS, an, bn);
+
+    // K values 2 s + h.  Whole groups of OU_PAIRS pairs first, the next group requested before the current one
+    // is multiplied (a group is one round trip to memory, and a small output has no other wavefront to hide it
+    // behind); then the remaining pairs, requested ahead of everything: their K indices are clamped to the last
+    // row (a valid address) and what lies past an odd K is multiplied as zeros.
+    const int pairs = (g.K + 1) >> 1;
+    const int whole = (g.K >> 1) / OU_PAIRS;           // groups in which every K value exists
+    const int rest0 = whole * OU_PAIRS;                 // first pair of the remainder
+    float at[OU_PAIRS];
+    f32x4 bt[OU_PAIRS];
 #pragma unroll
-        for (int u = 0; u < OU_PAIRS; ++u) {
-            const bool live = 2 * (s0 + u) + h < g.K;
-            const float av = live ? a[u] : 0.0f;
-            const f32x4 bv = live ? b[u] : f32x4{0.f, 0.f, 0.f, 0.f};
-            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv.x, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv.y, acc[1], 0, 0, 0);
-            acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv.z, acc[2], 0, 0, 0);
-            acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv.w, acc[3], 0, 0, 0);
+    for (int u = 0; u < OU_PAIRS; ++u) {
+        const int k = min(2 * (rest0 + u) + h, g.K - 1);
+        at[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, (arow + k * a_cs) * 4, 0, 0));
+        bt[u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(br, (bcol + k * b_rs) * 4, 0, 0));
+    }
+    if (whole > 0) {
+        float a[OU_PAIRS], an[OU_PAIRS];
+        f32x4 b[OU_PAIRS], bn[OU_PAIRS];
+        auto request = [&](int group, float (&ra)[OU_PAIRS], f32x4 (&rb)[OU_PAIRS]) {
+#pragma unroll
+            for (int u = 0; u < OU_PAIRS; ++u) {
+                ra[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ar, va, (group * OU_PAIRS + u) * sa, 0));
+                rb[u] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(br, vb, (group * OU_PAIRS + u) * sb, 0));
+            }
+        };
+        request(0, a, b);
+        for (int group = 0; group < whole; ++group) {
+            request(min(group + 1, whole - 1), an, bn);  // (past the last group: the last again, unused)
+#pragma unroll
+            for (int u = 0; u < OU_PAIRS; ++u) multiply(a[u], b[u]);
+#pragma unroll
+            for (int u = 0; u < OU_PAIRS; ++u) { a[u] = an[u]; b[u] = bn[u]; }
         }
+    }
 #pragma unroll
-        for (int u = 0; u < OU_PAIRS; ++u) { a[u] = an[u]; b[u] = bn[u]; }
+    for (int u = 0; u < OU_PAIRS; ++u) {
+        if (rest0 + u >= pairs) break;  // (uniform)
+        const bool live = 2 * (rest0 + u) + h < g.K;
+        multiply(live ? at[u] : 0.0f, live ? bt[u] : f32x4{0.f, 0.f, 0.f, 0.f});
     }
 
     // element e of lane (i, h): row 8 (e / 4) + 4 h + e % 4, columns n0 + 4 i + (accumulator index)
@@ -124,6 +149,8 @@ bool gemm_outer_eligible(const GemmLaunch &g) {
     if (g.a_rs != 1 || g.b_cs != 1) return false;
     if (g.b_rs % 4 != 0 || (g.b_bcount > 1 && g.b_bs % 4 != 0) || !ou_aligned16(g.B)) return false;
     if (g.ldc % 4 != 0 || (g.batch > 1 && g.c_bs % 4 != 0) || !ou_aligned16(g.C)) return false;
+    // byte offsets inside one batch of A and of B are 32-bit in the kernel
+    if (g.a_cs < 0 || g.b_rs < 0 || ((int64_t)g.K * g.a_cs + g.M) * 4 >= 0x7fffffffLL || ((int64_t)g.K * g.b_rs + g.N) * 4 >= 0x7fffffffLL) return false;
     return true;
 }
 
