@@ -283,7 +283,9 @@ static int fewrows_split(const GemmLaunch &g, int cus) {
 static bool outer_plan(const GemmLaunch &g, int cus) {
     (void)cus;
     const int64_t outputs = (int64_t)g.M * g.N * g.batch;
-    if (outputs >= (1LL << 21)) return true;  // (eligible: K <= 128)
+    // (K = 192 / 256 / 512: 4096 x 4096 53.9 / 70.4 / 129 against 60.3 / 74.5 / 131, 8192 x 8192 202 / 260 / 497 against 230 /
+    // 286 / 510, 2048 x 2048 16.3 / 20.2 / 47.8 against 17.7 / 21.2 / 35.7, 4096 x 11008 156 / 200 / 376 against 156 / 193 / 344)
+    if (outputs >= (1LL << 21)) return g.K <= 256;
     return outputs >= (1LL << 16) && g.K <= 48;  // (512 x 512: K = 48 5.9 against 6.8, K = 64 6.9 against 6.0)
 }
 // Whether the few-rows kernel is the plan for an eligible product: from about 512 x 512 of W on it is ahead of the
@@ -365,7 +367,7 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
     if (d.algo == MNI_ALGO_OUTER || (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_outer_eligible(g) && outer_plan(g, cus))) {
         if (!gemm_outer_eligible(g))
             return set_error(MNI_ERR_INVALID, "sgemm: the short-K outer-product kernel takes an A contiguous along M and a B contiguous along N, "
-                                              "K <= 128, N %% 4 == 0, B and C 16-byte aligned, no epilogue");
+                                              "K <= 512, N %% 4 == 0, B and C 16-byte aligned, no epilogue");
         if (d.split_k > 1) return set_error(MNI_ERR_INVALID, "sgemm: the short-K outer-product kernel takes no split_k");
         g.tiles_m = (g.M + 127) / 128;
         g.tiles_n = (g.N + 127) / 128;

@@ -68,7 +68,7 @@ int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1);  // two e
 // (the workgroup that completes a count adds the slices up and returns the counter to zero).
 bool gemm_fewrows_eligible(const GemmLaunch &g, int amode, int bmode);
 int launch_gemm_fewrows(const GemmLaunch &g, int amode, int bmode);
-// Short-K form for an A contiguous along M and a B contiguous along N (gemm_outer.hip): K <= 128 outer products,
+// Short-K form for an A contiguous along M and a B contiguous along N (gemm_outer.hip): K <= 512 outer products,
 // both operands straight into MFMA registers, no epilogue; g.accumulate honoured.
 bool gemm_outer_eligible(const GemmLaunch &g);
 int launch_gemm_outer(const GemmLaunch &g);

@@ -1,6 +1,6 @@
 // A short K under a large output, both operands contiguous along the OUTPUT axes:
 //
-//   C[b] (M x N) (+)= op(A)[b] (M x K) * B[b] (K x N),   K <= 128,
+//   C[b] (M x N) (+)= op(A)[b] (M x K) * B[b] (K x N),   K <= 512,
 //   op(A)(m, k) = A[k * a_cs + m]  (A stored [K, M]: the transposed view of an [rows, in] activation),
 //   B(k, n) = B[k * b_rs + n]
 //
@@ -35,7 +35,7 @@ static constexpr int OU_ROWS = 32;    // rows per wavefront
 static constexpr int OU_COLS = 128;   // columns per wavefront (and workgroup)
 static constexpr int OU_WAVES = 4;    // row blocks per workgroup
 static constexpr int OU_PAIRS = 4;    // pairs of K values requested together
-static constexpr int OU_MAX_K = 128;
+static constexpr int OU_MAX_K = 512;
 
 // g.tiles_n = column groups of 128, g.tiles_m = groups of 128 rows.
 __global__ __launch_bounds__(256) void gemm_outer_kernel(const GemmLaunch g) {
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void gemm_outer_kernel(const GemmLaunch g) {
 
 static bool ou_aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-// A contiguous along M, B along N (16-byte pieces of B and C), K at most 128, no epilogue.
+// A contiguous along M, B along N (16-byte pieces of B and C), K at most 512, no epilogue.
 bool gemm_outer_eligible(const GemmLaunch &g) {
     if (g.K < 1 || g.K > OU_MAX_K || g.M < 1 || g.N < 4 || g.N % 4 != 0 || g.epilogue != MNI_EPI_NONE) return false;
     if (g.a_rs != 1 || g.b_cs != 1) return false;

@@ -143,7 +143,7 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * read once, straight into the matrix instruction's registers, K slices
  * (split_k, 0 = chosen) summed inside the launch (error unless K % 8 == 0,
  * N % 4 == 0, N >= 128, K >= 64, operands and C 16-byte aligned with row
- * strides in whole 16 bytes); OUTER = a short K (<= 128) under a large
+ * strides in whole 16 bytes); OUTER = a short K (<= 512) under a large
  * output with A contiguous along M and B along N -- the weight gradient
  * X^T dY of a small batch: both operands straight into the matrix
  * instruction's registers, the cost of writing C (error unless N % 4 == 0,

@@ -900,7 +900,7 @@ def test_skinny_single_launch_repeats_and_matches_two_pass(dev, rocm):
 
 
 @pytest.mark.parametrize("nin,nout,rows,batch", [(128, 128, 8, 1), (100, 132, 7, 1), (33, 4, 1, 1), (300, 260, 33, 2), (257, 516, 128, 3),
-                                                 (64, 64, 2, 1), (1000, 640, 5, 1), (31, 1028, 19, 4)])
+                                                 (64, 64, 2, 1), (1000, 640, 5, 1), (31, 1028, 19, 4), (260, 132, 301, 1), (128, 256, 512, 2)])
 def test_outer_product_kernel_integer_exact(dev, rocm, nin, nout, rows, batch):
     # dW[b] = X[b]^T dY[b] of a small batch: K = its rows, A the transposed view of X, both operands contiguous along
     # the output axes.  Forced and as planned; overwriting and accumulating; edges in both extents, odd K.
@@ -941,7 +941,7 @@ def test_outer_product_kernel_is_the_plan_for_a_small_batch_weight_gradient_and_
         with pytest.raises(N.MniError):   # K-contiguous A; an epilogue; K slices
             rocm.sgemm(nin, nout, rows, dX, dY, dC, algo=N.ALGO_OUTER, **kw)
     with pytest.raises(N.MniError):       # K beyond the kernel's limit
-        rocm.sgemm(64, 64, 200, dX, dY, dC, a_strides=(1, 64), algo=N.ALGO_OUTER)
+        rocm.sgemm(32, 32, 600, dX, dY, dC, a_strides=(1, 32), algo=N.ALGO_OUTER)
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 9, 10, 13, 17])
