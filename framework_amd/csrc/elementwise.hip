@@ -854,10 +854,62 @@ __global__ void reduce_rows_kernel(float *__restrict__ out, const float *__restr
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
     if (lane == 0) out[row] = s / div;
 }
+// A few long rows (the sum of a whole tensor: one row of millions): a wavefront per chunk of a row first, the
+// chunk sums are a short matrix for the forms above.  Lanes stride the chunk, 8 loads in flight, four running
+// sums folded in a fixed order.
+static constexpr int64_t RC_CHUNK = 8192;
+__global__ void reduce_chunks_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t nchunks_total, int64_t dim,
+                                     int64_t chunks) {
+    const int lane = threadIdx.x & 63;
+    const int64_t idx = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (idx >= nchunks_total) return;
+    const int64_t o = idx / chunks, c = idx - o * chunks;
+    const int64_t len = min(RC_CHUNK, dim - c * RC_CHUNK);
+    const float *p = a + o * dim + c * RC_CHUNK;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int64_t d = lane;
+    for (; d + 7 * 64 < len; d += 8 * 64) {
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = p[d + e * 64];
+        s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
+        s0 += v[4]; s1 += v[5]; s2 += v[6]; s3 += v[7];
+    }
+    for (; d < len; d += 64) s0 += p[d];
+    float s = (s0 + s1) + (s2 + s3);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (lane == 0) part[idx] = s;
+}
+__global__ void div_inplace_kernel(float *__restrict__ x, float div, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = x[i] / div;
+}
 int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t inner, float div) {
     const int64_t n = outer * inner;
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
+    if (inner == 1 && dim >= 4 * RC_CHUNK && outer < 4096) {
+        // (a wavefront per row would leave the few rows to a few wavefronts: 16 M elements in one row took 58 ms)
+        const int64_t chunks = (dim + RC_CHUNK - 1) / RC_CHUNK, total = outer * chunks;
+        void *part = nullptr;
+        MNI_TRY(dev_alloc(&part, (size_t)total * sizeof(float)));
+        MNI_KERNEL_LAUNCH(reduce_chunks_kernel, dim3(grid_for(total, 4)), dim3(TPB), 0, ctx().stream, (float *)part, a, total, dim, chunks);
+        int rc = check_launch("reduce_chunks");
+        if (rc == MNI_OK) rc = k_reduce_dim(out, (const float *)part, outer, chunks, 1, div);
+        dev_free(part);
+        return rc;
+    }
+    if (inner > 1 && dim >= 256 && n < 32768 && outer <= 64) {
+        // Few outputs under a long reduced axis (the column sums of a tall matrix): a thread per output would
+        // walk the axis alone (4096 x 4096 summed over its rows: 977 us); the two-pass column sum per outer slice.
+        for (int64_t o = 0; o < outer; ++o) MNI_TRY(k_colsum(out + o * inner, a + o * dim * inner, dim, inner));
+        if (div != 1.0f) {
+            MNI_KERNEL_LAUNCH(div_inplace_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx().stream, out, div, n);
+            return check_launch("div_inplace");
+        }
+        return MNI_OK;
+    }
     if (inner == 1 && dim >= 256) {
         MNI_KERNEL_LAUNCH(reduce_rows_kernel, dim3(grid_for(outer, 4)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, div);
         return check_launch("reduce_rows");

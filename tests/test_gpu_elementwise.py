@@ -110,6 +110,35 @@ def test_max_matches_the_oracle_exactly(both, shape, dim):
     assert np.array_equal(res[0][0], x.max(axis=dim, keepdims=True))
 
 
+@pytest.mark.parametrize("shape", [(1 << 22,), (8, 1 << 18), (3, 32768 + 5), (2048, 2048), (2, 50000, 7), (100000, 3), (1, 33000), (300, 40)])
+def test_sums_and_means_over_long_axes_and_of_whole_tensors(both, shape):
+    # sum / mean (src/native/src/ops/reduce.rs:13-46,169-184) where the reduced axis is long and the outputs few: a
+    # row of millions is summed chunk by chunk over the whole device, the column sums of a tall matrix in two passes
+    # (a wavefront per row, or a thread per output, took 58 ms for one row of 16 M elements).  Against float64; the
+    # oracle too where it is quick.
+    gpu, cpu = both
+    a = synth.normal(sum(shape), shape)
+    a64 = a.astype(np.float64)
+    t = _t(gpu, a)
+    for dim in (None, -1, 0):
+        for mean in (False, True):
+            got = (t.mean() if mean else t.sum()) if dim is None else (t.mean(dim) if mean else t.sum(dim))
+            want = (a64.mean(keepdims=True) if mean else a64.sum(keepdims=True)) if dim is None else \
+                   (a64.mean(dim, keepdims=True) if mean else a64.sum(dim, keepdims=True))
+            nred = a.size / want.size
+            tol = 1e-5 * math.sqrt(nred) * float(np.abs(a).max()) / (nred if mean else 1.0) + 1e-7
+            assert list(got.shape) == list(want.shape), (dim, mean)
+            assert max_err(got.numpy(), want) <= tol, (dim, mean)
+    if a.size <= 1 << 19:
+        tc = _t(cpu, a)
+        for dim in (-1, 0):
+            assert max_err(t.sum(dim).numpy(), tc.sum(dim).numpy()) <= 1e-5 * math.sqrt(a.size) * float(np.abs(a).max())
+    # backward of a whole-tensor mean: every element gets 1 / n
+    X = _t(gpu, a, True)
+    X.mean().backward()
+    assert np.allclose(X.grad.numpy(), 1.0 / a.size, rtol=1e-6, atol=0)
+
+
 def test_layernorm_backward_of_more_rows_than_one_grid_axis_of_row_blocks(gpu):
     # 1.2 M rows of 8: the column sums for gamma and beta run over more 16-row blocks than the second grid axis holds,
     # so a block takes more rows; checked against float64 (the oracle would need minutes)
