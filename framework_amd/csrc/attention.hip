@@ -43,6 +43,75 @@ __global__ void softmax_rows_kernel(float *__restrict__ out, const float *__rest
     sum = wave_sum(sum);
     for (int64_t j = lane; j < n; j += 64) o[j] = o[j] / sum;
 }
+// lines of a few values: a thread per line (a wavefront per line leaves 60 lanes idle: 1 M lines of 4 took 250 us)
+__global__ void softmax_short_kernel(float *__restrict__ out, const float *__restrict__ x, int64_t rows, int n) {
+    const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= rows) return;
+    const float *p = x + row * n;
+    float *o = out + row * n;
+    float v[16];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        v[j] = j < n ? p[j] : -INFINITY;
+        mx = fmaxf(mx, v[j]);
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        v[j] = j < n ? expf(v[j] - mx) : 0.0f;
+        sum += v[j];
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+        if (j < n) o[j] = v[j] / sum;
+}
+// long contiguous lines: a workgroup per line (a wavefront alone walks a vocabulary-sized line 786 steps at a
+// time, three times over: 8 x 50304 took 624 us)
+__global__ __launch_bounds__(1024) void softmax_lines_kernel(float *__restrict__ out, const float *__restrict__ x, int64_t n, int vec) {
+    __shared__ float red[32];
+    float mx, sum;
+    softmax_line_workgroup(out + (int64_t)blockIdx.x * n, x + (int64_t)blockIdx.x * n, n, vec != 0, red, mx, sum);
+}
+// lines of up to 1024 NV values in whole 16-byte pieces: a workgroup per line holds it in registers -- one read, one write
+template <int NV>
+__global__ __launch_bounds__(256) void softmax_lines_cached_kernel(float *__restrict__ out, const float *__restrict__ x, int64_t n) {
+    __shared__ float red[2][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t n4 = n >> 2;
+    const float4 *p = reinterpret_cast<const float4 *>(x + (int64_t)blockIdx.x * n);
+    float4 *o = reinterpret_cast<float4 *>(out + (int64_t)blockIdx.x * n);
+    float4 r[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t j = tid + 256 * i;
+        r[i] = j < n4 ? p[j] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) mx = fmaxf(fmaxf(mx, fmaxf(r[i].x, r[i].y)), fmaxf(r[i].z, r[i].w));
+    mx = wave_max(mx);
+    if (lane == 0) red[0][wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        if (tid + 256 * i < n4) {
+            r[i].x = expf(r[i].x - mx); r[i].y = expf(r[i].y - mx); r[i].z = expf(r[i].z - mx); r[i].w = expf(r[i].w - mx);
+            sum += r[i].x; sum += r[i].y; sum += r[i].z; sum += r[i].w;
+        }
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) red[1][wave] = sum;
+    __syncthreads();
+    sum = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t j = tid + 256 * i;
+        if (j < n4) o[j] = make_float4(r[i].x / sum, r[i].y / sum, r[i].z / sum, r[i].w / sum);
+    }
+}
 // lines with a stride (inner > 1): one thread per line, neighbours coalesce
 __global__ void softmax_strided_kernel(float *__restrict__ out, const float *__restrict__ x, int64_t outer, int64_t n,
                                        int64_t inner) {
@@ -62,7 +131,14 @@ __global__ void softmax_strided_kernel(float *__restrict__ out, const float *__r
 int k_softmax(float *out, const float *x, int64_t outer, int64_t n, int64_t inner) {
     if (outer * n * inner <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    if (inner == 1)
+    if (inner == 1 && n <= 16 && outer >= 4096) {
+        MNI_KERNEL_LAUNCH(softmax_short_kernel, dim3((unsigned)((outer + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB), 0, ctx().stream, out, x, outer, (int)n);
+    } else if (inner == 1 && n >= 1024 && outer <= 0x7fffffffLL) {
+        const int vec = n % 4 == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)x & 15) == 0;
+        if (vec && n <= 2048) MNI_KERNEL_LAUNCH(softmax_lines_cached_kernel<2>, dim3((unsigned)outer), dim3(256), 0, ctx().stream, out, x, n);
+        else if (vec && n <= 8192) MNI_KERNEL_LAUNCH(softmax_lines_cached_kernel<8>, dim3((unsigned)outer), dim3(256), 0, ctx().stream, out, x, n);
+        else MNI_KERNEL_LAUNCH(softmax_lines_kernel, dim3((unsigned)outer), dim3(n <= 16384 ? 256 : 1024), 0, ctx().stream, out, x, n, vec);
+    } else if (inner == 1)
         MNI_KERNEL_LAUNCH(softmax_rows_kernel, dim3(rows_grid(outer)), dim3(ATT_TPB), 0, ctx().stream, out, x, outer, n);
     else
         MNI_KERNEL_LAUNCH(softmax_strided_kernel, dim3((unsigned)((outer * inner + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB), 0,

@@ -96,6 +96,63 @@ int upload_small(void *dst, const void *src, size_t bytes);
 __device__ __forceinline__ void post_result_word(unsigned long long *word, unsigned tag, unsigned value) {
     __hip_atomic_store(word, ((unsigned long long)tag << 32) | (unsigned long long)value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
+// One workgroup (blockDim.x threads, whole wavefronts, at most 1024) turns one contiguous line of n values into its
+// softmax, o[j] = exp(p[j] - max) / sum, in three passes over the line (the second and third re-read what the
+// workgroup itself touched: L2), and hands max and sum to every thread.  `vec`: n % 4 == 0 and both lines 16-byte
+// aligned.  `red`: 32 floats of LDS.  Sums are taken per thread, then per wavefront, then in wavefront order.
+__device__ __forceinline__ void softmax_line_workgroup(float *__restrict__ o, const float *__restrict__ p, int64_t n, bool vec,
+                                                       float *red, float &mx_out, float &sum_out) {
+    const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+    const int64_t n4 = n >> 2;
+    const float4 *p4 = reinterpret_cast<const float4 *>(p);
+    float4 *o4 = reinterpret_cast<float4 *>(o);
+    float mx = -INFINITY;
+    if (vec) {
+        for (int64_t j = tid; j < n4; j += nt) {
+            const float4 v = p4[j];
+            mx = fmaxf(fmaxf(mx, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+        }
+    } else {
+        for (int64_t j = tid; j < n; j += nt) mx = fmaxf(mx, p[j]);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = red[0];
+    for (int w = 1; w < nw; ++w) mx = fmaxf(mx, red[w]);
+    float sum = 0.f;
+    if (vec) {
+        for (int64_t j = tid; j < n4; j += nt) {
+            float4 v = p4[j];
+            v.x = expf(v.x - mx); v.y = expf(v.y - mx); v.z = expf(v.z - mx); v.w = expf(v.w - mx);
+            o4[j] = v;
+            sum += v.x; sum += v.y; sum += v.z; sum += v.w;
+        }
+    } else {
+        for (int64_t j = tid; j < n; j += nt) {
+            const float e = expf(p[j] - mx);
+            o[j] = e;
+            sum += e;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane == 0) red[16 + wave] = sum;
+    __syncthreads();
+    sum = red[16];
+    for (int w = 1; w < nw; ++w) sum += red[16 + w];
+    if (vec) {
+        for (int64_t j = tid; j < n4; j += nt) {
+            float4 v = o4[j];  // (written by this thread)
+            o4[j] = make_float4(v.x / sum, v.y / sum, v.z / sum, v.w / sum);
+        }
+    } else {
+        for (int64_t j = tid; j < n; j += nt) o[j] = o[j] / sum;
+    }
+    mx_out = mx;
+    sum_out = sum;
+}
 #endif
 unsigned next_result_tag();
 int wait_result_word(unsigned tag, unsigned *value, bool *delivered);

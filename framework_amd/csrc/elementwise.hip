@@ -699,10 +699,72 @@ __global__ void max_rows_kernel(float *__restrict__ out, const float *__restrict
     }
     if (lane == 0) out[row] = m;
 }
+// A long reduced axis under few outputs, in two levels (a maximum does not depend on the order it is taken in): the
+// axis is cut into `parts` blocks of `blk`, a thread takes the maximum of one block for one output, and the block
+// maxima are a shorter axis for the forms above.  (One thread per output walked a million rows alone: 90 ms.)
+__global__ void max_dim_blocks_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t outer, int64_t dim, int64_t inner,
+                                      int64_t blk, int64_t parts) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= outer * parts * inner) return;
+    const int64_t i = idx % inner, op = idx / inner, p = op % parts, o = op / parts;
+    const int64_t d0 = p * blk, d1 = min(dim, d0 + blk);
+    const float *q = a + o * dim * inner + i;
+    float m = -INFINITY;
+    for (int64_t d = d0; d < d1; ++d) {
+        const float v = q[d * inner];
+        if (v > m) m = v;
+    }
+    part[idx] = m;
+}
+// The same for a few long contiguous rows: a wavefront per chunk of a row, lanes striding it.
+static constexpr int64_t MC_CHUNK = 8192;
+__global__ void max_chunks_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t total, int64_t dim, int64_t chunks) {
+    const int lane = threadIdx.x & 63;
+    const int64_t idx = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (idx >= total) return;
+    const int64_t o = idx / chunks, c = idx - o * chunks;
+    const int64_t len = min(MC_CHUNK, dim - c * MC_CHUNK);
+    const float *p = a + o * dim + c * MC_CHUNK;
+    float m = -INFINITY;
+    for (int64_t d = lane; d < len; d += 64) {
+        const float v = p[d];
+        if (v > m) m = v;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float o2 = __shfl_xor(m, off, 64);
+        if (o2 > m) m = o2;
+    }
+    if (lane == 0) part[idx] = m;
+}
 int k_max_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t inner) {
     const int64_t n = outer * inner;
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
+    if (inner == 1 && dim >= 4 * MC_CHUNK && outer < 4096) {
+        const int64_t chunks = (dim + MC_CHUNK - 1) / MC_CHUNK, total = outer * chunks;
+        void *part = nullptr;
+        MNI_TRY(dev_alloc(&part, (size_t)total * sizeof(float)));
+        MNI_KERNEL_LAUNCH(max_chunks_kernel, dim3(grid_for(total, 4)), dim3(TPB), 0, ctx().stream, (float *)part, a, total, dim, chunks);
+        int rc = check_launch("max_chunks");
+        if (rc == MNI_OK) rc = k_max_dim(out, (const float *)part, outer, chunks, 1);
+        dev_free(part);
+        return rc;
+    }
+    if (inner > 1 && n < 32768 && dim >= 2048) {
+        const int64_t want = (1 << 17) / n;                      // blocks per output for ~128 K threads
+        const int64_t blk = max((int64_t)32, (dim + want - 1) / want), parts = (dim + blk - 1) / blk;
+        if (parts > 1) {
+            void *part = nullptr;
+            MNI_TRY(dev_alloc(&part, (size_t)(outer * parts * inner) * sizeof(float)));
+            MNI_KERNEL_LAUNCH(max_dim_blocks_kernel, dim3(grid_for(outer * parts * inner, TPB)), dim3(TPB), 0, ctx().stream, (float *)part, a,
+                               outer, dim, inner, blk, parts);
+            int rc = check_launch("max_dim_blocks");
+            if (rc == MNI_OK) rc = k_max_dim(out, (const float *)part, outer, parts, inner);
+            dev_free(part);
+            return rc;
+        }
+    }
     if (inner == 1 && dim >= 256)
         MNI_KERNEL_LAUNCH(max_rows_kernel, dim3(grid_for(outer, 4)), dim3(TPB), 0, ctx().stream, out, a, outer, dim);
     else
@@ -1142,6 +1204,21 @@ __global__ __launch_bounds__(256) void ce_rows_wg_kernel(float *__restrict__ row
         row_loss[row] = -logf(e / sum);
     }
 }
+// Rows beyond what the forms above hold in registers (a vocabulary of tens of thousands, or a row not in whole
+// 16-byte pieces): a workgroup per row, three passes over the row.
+__global__ __launch_bounds__(1024) void ce_rows_wide_kernel(float *__restrict__ row_loss, float *__restrict__ sm,
+                                                            const float *__restrict__ logits, const int32_t *__restrict__ targets,
+                                                            int64_t v, int vec) {
+    __shared__ float red[32];
+    const int64_t row = blockIdx.x;
+    float mx, sum;
+    softmax_line_workgroup(sm + row * v, logits + row * v, v, vec != 0, red, mx, sum);
+    if (threadIdx.x == 0) {
+        const int32_t t = targets[row];
+        const float e = expf(logits[row * v + t] - mx);
+        row_loss[row] = -logf(e / sum);
+    }
+}
 __global__ void ce_mean_kernel(float *__restrict__ loss, const float *__restrict__ row_loss, int64_t n) {
     const int lane = threadIdx.x;
     float s = 0.f;
@@ -1218,6 +1295,8 @@ int k_cross_entropy(float *loss, float *softmax, const float *logits, int32_t *t
         MNI_KERNEL_LAUNCH(ce_rows_cached_kernel<8>, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
     else if (vec && v <= 256 * 4 * 8 && n <= 0x7fffffffLL)
         MNI_KERNEL_LAUNCH(ce_rows_wg_kernel<8>, dim3((unsigned)n), dim3(256), 0, st, (float *)rl, softmax, logits, targets, n, v);
+    else if (v >= 1024 && n <= 0x7fffffffLL)
+        MNI_KERNEL_LAUNCH(ce_rows_wide_kernel, dim3((unsigned)n), dim3(v <= 16384 ? 256 : 1024), 0, st, (float *)rl, softmax, logits, targets, v, vec ? 1 : 0);
     else
         MNI_KERNEL_LAUNCH(ce_rows_kernel, grid, block, 0, st, (float *)rl, softmax, logits, targets, n, v);
     int rc = check_launch("ce_rows");

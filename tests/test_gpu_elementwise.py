@@ -139,6 +139,42 @@ def test_sums_and_means_over_long_axes_and_of_whole_tensors(both, shape):
     assert np.allclose(X.grad.numpy(), 1.0 / a.size, rtol=1e-6, atol=0)
 
 
+@pytest.mark.parametrize("shape,dim", [((4, 1 << 18), -1), ((1, 1 << 20), -1), ((2048, 2048), 0), ((1 << 18, 4), 0), ((2, 3, 1 << 16), -1),
+                                       ((2, 40000, 5), 1), ((3, 32768 + 5), 1)])
+def test_max_over_a_long_axis_under_few_outputs_is_exact(gpu, shape, dim):
+    # taken in two levels (chunks of a long row, blocks of a tall matrix): a maximum is exact whatever the order
+    a = synth.normal(sum(shape), shape)
+    assert np.array_equal(_t(gpu, a).max(dim).numpy(), a.max(axis=dim, keepdims=True))
+
+
+@pytest.mark.parametrize("shape", [(8, 50304), (5, 50257), (3, 70000), (100000, 4), (5000, 13), (300, 4096), (64, 8192), (7, 1030)])
+def test_softmax_and_cross_entropy_over_long_and_short_lines(both, shape):
+    # softmax over the last axis (src/native/src/ops/reduce.rs softmax) and the cross-entropy on top of it
+    # (src/native/src/ops/loss.rs:24-67) for lines of vocabulary length under a handful of rows (a workgroup per
+    # line; a wavefront per line took 624 us for 8 x 50304), lines held in registers, and lines of a few values
+    # (a thread per line).  Against float64, and against the oracle where it is quick.
+    gpu, cpu = both
+    a = synth.normal(shape[0] + shape[1], shape, 3.0)
+    a64 = a.astype(np.float64)
+    e = np.exp(a64 - a64.max(-1, keepdims=True))
+    want = e / e.sum(-1, keepdims=True)
+    got = gpu.softmax(_t(gpu, a), -1).numpy()
+    assert max_err(got, want) <= 2e-6
+    assert np.abs(got.astype(np.float64).sum(-1) - 1.0).max() <= 1e-4
+    if shape[0] <= 5000:
+        targets = [int(t) for t in (np.arange(shape[0]) * 7919) % shape[1]]
+        want_loss = float(np.mean(-np.log(want[np.arange(shape[0]), targets])))
+        L = _t(gpu, a, True)
+        loss = gpu.crossEntropyLoss(L, targets)
+        assert abs(float(loss.numpy().ravel()[0]) - want_loss) <= 1e-5 * max(1.0, abs(want_loss))
+        loss.backward()
+        onehot = np.zeros(shape); onehot[np.arange(shape[0]), targets] = 1.0
+        assert max_err(L.grad.numpy(), (want - onehot) / shape[0]) <= 2e-6
+        if a.size <= 1 << 19:
+            Lc = _t(cpu, a, True)
+            assert abs(float(cpu.crossEntropyLoss(Lc, targets).numpy().ravel()[0]) - float(loss.numpy().ravel()[0])) <= 1e-5 * max(1.0, abs(want_loss))
+
+
 def test_layernorm_backward_of_more_rows_than_one_grid_axis_of_row_blocks(gpu):
     # 1.2 M rows of 8: the column sums for gamma and beta run over more 16-row blocks than the second grid axis holds,
     # so a block takes more rows; checked against float64 (the oracle would need minutes)
