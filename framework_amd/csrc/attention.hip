@@ -158,6 +158,22 @@ __global__ void softmax_bwd_rows_kernel(float *__restrict__ out, const float *__
     dot = wave_sum(dot);
     for (int64_t j = lane; j < n; j += 64) out[row * n + j] = s[j] * (gr[j] - dot);
 }
+// long lines: a workgroup per line (sums per thread, per wavefront, then in wavefront order)
+__global__ __launch_bounds__(1024) void softmax_bwd_lines_kernel(float *__restrict__ out, const float *__restrict__ sm,
+                                                                 const float *__restrict__ g, int64_t n) {
+    __shared__ float red[16];
+    const int tid = threadIdx.x, nt = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+    const float *s = sm + (int64_t)blockIdx.x * n, *gr = g + (int64_t)blockIdx.x * n;
+    float *o = out + (int64_t)blockIdx.x * n;
+    float dot = 0.f;
+    for (int64_t j = tid; j < n; j += nt) dot += gr[j] * s[j];
+    dot = wave_sum(dot);
+    if (lane == 0) red[wave] = dot;
+    __syncthreads();
+    dot = red[0];
+    for (int w = 1; w < nw; ++w) dot += red[w];
+    for (int64_t j = tid; j < n; j += nt) o[j] = s[j] * (gr[j] - dot);
+}
 __global__ void softmax_bwd_strided_kernel(float *__restrict__ out, const float *__restrict__ sm,
                                            const float *__restrict__ g, int64_t outer, int64_t n, int64_t inner) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -170,7 +186,9 @@ __global__ void softmax_bwd_strided_kernel(float *__restrict__ out, const float 
 int k_softmax_backward(float *out, const float *sm, const float *g, int64_t outer, int64_t n, int64_t inner) {
     if (outer * n * inner <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    if (inner == 1)
+    if (inner == 1 && n >= 2048 && outer <= 0x7fffffffLL)
+        MNI_KERNEL_LAUNCH(softmax_bwd_lines_kernel, dim3((unsigned)outer), dim3(n <= 16384 ? 256 : 1024), 0, ctx().stream, out, sm, g, n);
+    else if (inner == 1)
         MNI_KERNEL_LAUNCH(softmax_bwd_rows_kernel, dim3(rows_grid(outer)), dim3(ATT_TPB), 0, ctx().stream, out, sm, g, outer, n);
     else
         MNI_KERNEL_LAUNCH(softmax_bwd_strided_kernel, dim3((unsigned)((outer * inner + ATT_TPB - 1) / ATT_TPB)), dim3(ATT_TPB),

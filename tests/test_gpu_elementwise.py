@@ -161,6 +161,12 @@ def test_softmax_and_cross_entropy_over_long_and_short_lines(both, shape):
     got = gpu.softmax(_t(gpu, a), -1).numpy()
     assert max_err(got, want) <= 2e-6
     assert np.abs(got.astype(np.float64).sum(-1) - 1.0).max() <= 1e-4
+    if shape[0] <= 5000:   # its gradient: p * (w - sum(p * w)) per line (the axis given as 1: the reference reads -1 back as 0)
+        w = synth.normal(3, shape, stream=2)
+        X = _t(gpu, a, True)
+        gpu.softmax(X, 1).mul(_t(gpu, w)).sum().backward()
+        w64 = w.astype(np.float64)
+        assert max_err(X.grad.numpy(), want * (w64 - (want * w64).sum(-1, keepdims=True))) <= 1e-5 * float(np.abs(w).max())
     if shape[0] <= 5000:
         targets = [int(t) for t in (np.arange(shape[0]) * 7919) % shape[1]]
         want_loss = float(np.mean(-np.log(want[np.arange(shape[0]), targets])))
