@@ -225,6 +225,10 @@ int k_mul_backward_same(float *ga, float *gb, const float *g, const float *a, co
 int k_colsum(float *out, const float *a, int64_t rows, int64_t cols);
 // out[o, i] = (sum_d a[o, d, i]) / div
 int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t inner, float div);
+// layernorm (residual == nullptr) or residual + layernorm of rows of 1024 to 16384 values, a workgroup per row;
+// false (nothing launched) when the rows do not fit that form
+bool launch_layernorm_workgroups(float *out, float *res, float *mean, float *rstd, const float *x, const float *residual,
+                                 const float *gamma, const float *beta, int64_t rows, int64_t c, float eps);
 // out[o, d, i] = g[o, i] / div
 int k_expand_dim(float *out, const float *g, int64_t outer, int64_t dim, int64_t inner, float div);
 // generic unbroadcast: out (orig shape, contiguous) = sum of g over broadcast dims

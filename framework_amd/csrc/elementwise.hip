@@ -813,10 +813,89 @@ __global__ void layernorm_kernel(float *__restrict__ out, float *__restrict__ me
     for (int64_t j = lane; j < c; j += 64) out[row * c + j] = (p[j] - m) * r * gamma[j] + beta[j];
     if (lane == 0) { mean[row] = m; rstd[row] = r; }
 }
+// Rows of 1024 to 16384 values in whole 16-byte pieces: a workgroup per row holds the row in registers -- one
+// read, one write, two LDS reductions (a wavefront walked a 4096-wide row 64 steps at a time, three times over:
+// 21 us for a single row).  RESIDUAL: the row is x + residual, which is also written out (res).
+template <int NV, bool RESIDUAL>
+__global__ __launch_bounds__(256) void layernorm_wg_kernel(float *__restrict__ out, float *__restrict__ res, float *__restrict__ mean,
+                                                           float *__restrict__ rstd, const float *__restrict__ x,
+                                                           const float *__restrict__ residual, const float *__restrict__ gamma,
+                                                           const float *__restrict__ beta, int64_t c, float eps) {
+    __shared__ float red[2][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t row = blockIdx.x, c4 = c >> 2;
+    const float4 *p = reinterpret_cast<const float4 *>(x + row * c);
+    float4 v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t j = tid + 256 * i;
+        v[i] = j < c4 ? p[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (RESIDUAL) {
+        const float4 *q = reinterpret_cast<const float4 *>(residual + row * c);
+        float4 *ps = reinterpret_cast<float4 *>(res + row * c);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int64_t j = tid + 256 * i;
+            if (j < c4) {
+                const float4 r4 = q[j];
+                v[i].x += r4.x; v[i].y += r4.y; v[i].z += r4.z; v[i].w += r4.w;
+                ps[j] = v[i];
+            }
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) { s += v[i].x; s += v[i].y; s += v[i].z; s += v[i].w; }  // (pieces past the row are zeros)
+    s = ew_wave_sum(s);
+    if (lane == 0) red[0][wave] = s;
+    __syncthreads();
+    const float m = ((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / (float)c;
+    float var = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        if (tid + 256 * i < c4) {
+            const float dx = v[i].x - m, dy = v[i].y - m, dz = v[i].z - m, dw = v[i].w - m;
+            var += dx * dx; var += dy * dy; var += dz * dz; var += dw * dw;
+        }
+    }
+    var = ew_wave_sum(var);
+    if (lane == 0) red[1][wave] = var;
+    __syncthreads();
+    const float r = 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / (float)c + eps);
+    const float4 *g4 = reinterpret_cast<const float4 *>(gamma), *b4 = reinterpret_cast<const float4 *>(beta);
+    float4 *o = reinterpret_cast<float4 *>(out + row * c);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t j = tid + 256 * i;
+        if (j < c4) {
+            const float4 gg = g4[j], bb = b4[j];
+            o[j] = make_float4((v[i].x - m) * r * gg.x + bb.x, (v[i].y - m) * r * gg.y + bb.y, (v[i].z - m) * r * gg.z + bb.z,
+                               (v[i].w - m) * r * gg.w + bb.w);
+        }
+    }
+    if (tid == 0) { mean[row] = m; rstd[row] = r; }
+}
+// Launches the form above when the row fits it; false when it does not.
+bool launch_layernorm_workgroups(float *out, float *res, float *mean, float *rstd, const float *x, const float *residual,
+                                 const float *gamma, const float *beta, int64_t rows, int64_t c, float eps) {
+    if (c < 1024 || c > 16384 || c % 4 != 0 || rows > 0x7fffffffLL) return false;
+    if (!al16(out) || !al16(x) || !al16(gamma) || !al16(beta) || (residual && (!al16(residual) || !al16(res)))) return false;
+    const dim3 grid((unsigned)rows), block(256);
+    hipStream_t st = ctx().stream;
+    if (residual && c <= 2048) MNI_KERNEL_LAUNCH((layernorm_wg_kernel<2, true>), grid, block, 0, st, out, res, mean, rstd, x, residual, gamma, beta, c, eps);
+    else if (residual && c <= 8192) MNI_KERNEL_LAUNCH((layernorm_wg_kernel<8, true>), grid, block, 0, st, out, res, mean, rstd, x, residual, gamma, beta, c, eps);
+    else if (residual) MNI_KERNEL_LAUNCH((layernorm_wg_kernel<16, true>), grid, block, 0, st, out, res, mean, rstd, x, residual, gamma, beta, c, eps);
+    else if (c <= 2048) MNI_KERNEL_LAUNCH((layernorm_wg_kernel<2, false>), grid, block, 0, st, out, res, mean, rstd, x, residual, gamma, beta, c, eps);
+    else if (c <= 8192) MNI_KERNEL_LAUNCH((layernorm_wg_kernel<8, false>), grid, block, 0, st, out, res, mean, rstd, x, residual, gamma, beta, c, eps);
+    else MNI_KERNEL_LAUNCH((layernorm_wg_kernel<16, false>), grid, block, 0, st, out, res, mean, rstd, x, residual, gamma, beta, c, eps);
+    return true;
+}
 int k_layernorm(float *out, float *mean, float *rstd, const float *x, const float *gamma, const float *beta, int64_t rows,
                 int64_t c, float eps) {
     if (rows <= 0 || c <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
+    if (launch_layernorm_workgroups(out, nullptr, mean, rstd, x, nullptr, gamma, beta, rows, c, eps)) return check_launch("layernorm");
     MNI_KERNEL_LAUNCH(layernorm_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, mean, rstd, x, gamma, beta,
                        rows, c, eps);
     return check_launch("layernorm");

@@ -379,6 +379,7 @@ int k_residual_layernorm(float *out, float *res, float *mean, float *rstd, const
                          const float *gamma, const float *beta, int64_t rows, int64_t c, float eps) {
     if (rows <= 0 || c <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
+    if (launch_layernorm_workgroups(out, res, mean, rstd, x, residual, gamma, beta, rows, c, eps)) return check_launch("residual_layernorm");
     MNI_KERNEL_LAUNCH(residual_layernorm_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, res, mean, rstd, x,
                        residual, gamma, beta, rows, c, eps);
     return check_launch("residual_layernorm");

@@ -197,7 +197,7 @@ def test_layernorm_backward_of_more_rows_than_one_grid_axis_of_row_blocks(gpu):
     assert max_err(B.grad.numpy(), w64.sum(0)) <= 1e-4 * math.sqrt(rows) * float(np.abs(w).max())
 
 
-@pytest.mark.parametrize("shape", [(2, 3), (64, 768), (4, 33, 100), (5000, 16)])
+@pytest.mark.parametrize("shape", [(2, 3), (64, 768), (4, 33, 100), (5000, 16), (8, 4096), (3, 1024), (2, 8192), (5, 2052), (2, 8196), (3, 16384), (2, 16388)])
 def test_layernorm_matches_the_oracle(both, shape):
     gpu, cpu = both
     c = shape[-1]

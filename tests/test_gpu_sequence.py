@@ -240,7 +240,7 @@ def test_tile_matches_numpy_and_the_oracle(both):
         gpu.tile(_t(gpu, a), [2])
 
 
-@pytest.mark.parametrize("rows,c", [(33, 70), (4, 4), (512, 768), (7, 1), (1, 1000)])
+@pytest.mark.parametrize("rows,c", [(33, 70), (4, 4), (512, 768), (7, 1), (1, 1000), (8, 4096), (3, 1024), (2, 8192), (5, 2052)])
 def test_residual_layernorm_matches_the_oracle(both, rows, c):
     xv, rv = synth.normal(1, (rows, c)), synth.normal(2, (rows, c), stream=1)
     gv, bv = synth.uniform(3, (c,), 0.5, 1.5), synth.normal(4, (c,), stream=2)
