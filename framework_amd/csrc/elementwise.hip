@@ -718,13 +718,14 @@ __global__ void max_dim_blocks_kernel(float *__restrict__ part, const float *__r
 }
 // The same for a few long contiguous rows: a wavefront per chunk of a row, lanes striding it.
 static constexpr int64_t MC_CHUNK = 8192;
-__global__ void max_chunks_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t total, int64_t dim, int64_t chunks) {
+__global__ void max_chunks_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t total, int64_t dim, int64_t chunks,
+                                  int64_t chunk) {
     const int lane = threadIdx.x & 63;
     const int64_t idx = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (idx >= total) return;
     const int64_t o = idx / chunks, c = idx - o * chunks;
-    const int64_t len = min(MC_CHUNK, dim - c * MC_CHUNK);
-    const float *p = a + o * dim + c * MC_CHUNK;
+    const int64_t len = min(chunk, dim - c * chunk);
+    const float *p = a + o * dim + c * chunk;
     float m = -INFINITY;
     for (int64_t d = lane; d < len; d += 64) {
         const float v = p[d];
@@ -741,11 +742,12 @@ int k_max_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t in
     const int64_t n = outer * inner;
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    if (inner == 1 && dim >= 4 * MC_CHUNK && outer < 4096) {
-        const int64_t chunks = (dim + MC_CHUNK - 1) / MC_CHUNK, total = outer * chunks;
+    if (inner == 1 && outer < 4096 && (dim >= 4 * MC_CHUNK || (dim >= MC_CHUNK && outer <= 512))) {
+        const int64_t chunk = dim >= 4 * MC_CHUNK ? MC_CHUNK : MC_CHUNK / 8;
+        const int64_t chunks = (dim + chunk - 1) / chunk, total = outer * chunks;
         void *part = nullptr;
         MNI_TRY(dev_alloc(&part, (size_t)total * sizeof(float)));
-        MNI_KERNEL_LAUNCH(max_chunks_kernel, dim3(grid_for(total, 4)), dim3(TPB), 0, ctx().stream, (float *)part, a, total, dim, chunks);
+        MNI_KERNEL_LAUNCH(max_chunks_kernel, dim3(grid_for(total, 4)), dim3(TPB), 0, ctx().stream, (float *)part, a, total, dim, chunks, chunk);
         int rc = check_launch("max_chunks");
         if (rc == MNI_OK) rc = k_max_dim(out, (const float *)part, outer, chunks, 1);
         dev_free(part);
@@ -1000,13 +1002,13 @@ __global__ void reduce_rows_kernel(float *__restrict__ out, const float *__restr
 // sums folded in a fixed order.
 static constexpr int64_t RC_CHUNK = 8192;
 __global__ void reduce_chunks_kernel(float *__restrict__ part, const float *__restrict__ a, int64_t nchunks_total, int64_t dim,
-                                     int64_t chunks) {
+                                     int64_t chunks, int64_t chunk) {
     const int lane = threadIdx.x & 63;
     const int64_t idx = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (idx >= nchunks_total) return;
     const int64_t o = idx / chunks, c = idx - o * chunks;
-    const int64_t len = min(RC_CHUNK, dim - c * RC_CHUNK);
-    const float *p = a + o * dim + c * RC_CHUNK;
+    const int64_t len = min(chunk, dim - c * chunk);
+    const float *p = a + o * dim + c * chunk;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     int64_t d = lane;
     for (; d + 7 * 64 < len; d += 8 * 64) {
@@ -1030,12 +1032,14 @@ int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t
     const int64_t n = outer * inner;
     if (n <= 0) return MNI_OK;
     MNI_TRY(ensure_init());
-    if (inner == 1 && dim >= 4 * RC_CHUNK && outer < 4096) {
-        // (a wavefront per row would leave the few rows to a few wavefronts: 16 M elements in one row took 58 ms)
-        const int64_t chunks = (dim + RC_CHUNK - 1) / RC_CHUNK, total = outer * chunks;
+    if (inner == 1 && outer < 4096 && (dim >= 4 * RC_CHUNK || (dim >= RC_CHUNK && outer <= 512))) {
+        // (a wavefront per row would leave the few rows to a few wavefronts: 16 M elements in one row took 58 ms,
+        // 8 rows of 16384 27 us; shorter chunks for the shorter rows)
+        const int64_t chunk = dim >= 4 * RC_CHUNK ? RC_CHUNK : RC_CHUNK / 8;
+        const int64_t chunks = (dim + chunk - 1) / chunk, total = outer * chunks;
         void *part = nullptr;
         MNI_TRY(dev_alloc(&part, (size_t)total * sizeof(float)));
-        MNI_KERNEL_LAUNCH(reduce_chunks_kernel, dim3(grid_for(total, 4)), dim3(TPB), 0, ctx().stream, (float *)part, a, total, dim, chunks);
+        MNI_KERNEL_LAUNCH(reduce_chunks_kernel, dim3(grid_for(total, 4)), dim3(TPB), 0, ctx().stream, (float *)part, a, total, dim, chunks, chunk);
         int rc = check_launch("reduce_chunks");
         if (rc == MNI_OK) rc = k_reduce_dim(out, (const float *)part, outer, chunks, 1, div);
         dev_free(part);

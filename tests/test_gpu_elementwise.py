@@ -110,7 +110,7 @@ def test_max_matches_the_oracle_exactly(both, shape, dim):
     assert np.array_equal(res[0][0], x.max(axis=dim, keepdims=True))
 
 
-@pytest.mark.parametrize("shape", [(1 << 22,), (8, 1 << 18), (3, 32768 + 5), (2048, 2048), (2, 50000, 7), (100000, 3), (1, 33000), (300, 40)])
+@pytest.mark.parametrize("shape", [(1 << 22,), (8, 1 << 18), (3, 32768 + 5), (2048, 2048), (2, 50000, 7), (100000, 3), (1, 33000), (300, 40), (8, 16384), (5, 9000)])
 def test_sums_and_means_over_long_axes_and_of_whole_tensors(both, shape):
     # sum / mean (src/native/src/ops/reduce.rs:13-46,169-184) where the reduced axis is long and the outputs few: a
     # row of millions is summed chunk by chunk over the whole device, the column sums of a tall matrix in two passes
@@ -140,7 +140,7 @@ def test_sums_and_means_over_long_axes_and_of_whole_tensors(both, shape):
 
 
 @pytest.mark.parametrize("shape,dim", [((4, 1 << 18), -1), ((1, 1 << 20), -1), ((2048, 2048), 0), ((1 << 18, 4), 0), ((2, 3, 1 << 16), -1),
-                                       ((2, 40000, 5), 1), ((3, 32768 + 5), 1)])
+                                       ((2, 40000, 5), 1), ((3, 32768 + 5), 1), ((8, 16384), 1), ((5, 9000), -1)])
 def test_max_over_a_long_axis_under_few_outputs_is_exact(gpu, shape, dim):
     # taken in two levels (chunks of a long row, blocks of a tall matrix): a maximum is exact whatever the order
     a = synth.normal(sum(shape), shape)
