@@ -446,6 +446,30 @@ def test_unbroadcast_patterns_vs_oracle(gpu, orc):
         assert_close(x, y, 1e-5, str(shape))
 
 
+@pytest.mark.parametrize("full,small", [((512, 2048), (512, 1)), ((16, 256, 96), (1, 256, 1)), ((4, 1 << 18), (4, 1)),
+                                        ((8, 6, 128, 128), (8, 1, 1, 128)), ((8, 6, 128, 128), (1, 6, 1, 1)), ((3, 70, 5000), (70, 1)),
+                                        ((2, 300, 40), (2, 1, 40))])
+def test_unbroadcast_of_few_outputs_under_many_values(gpu, orc, full, small):
+    # utils::unbroadcast (src/native/src/utils.rs:39-66) where the operand's gradient has few elements, each the sum
+    # of many: one reduced axis after the other (row sums of a matrix, a mask broadcast over heads and queries, ...),
+    # not one thread per output.  Against float64; against the oracle too where it is quick.
+    x, y, w = synth.normal(1, full), synth.normal(2, small, stream=1), synth.normal(3, full, stream=2)
+    X, Y = T(gpu, x, True), T(gpu, y, True)
+    X.mul(Y).mul(T(gpu, w)).sum().backward()
+    nd = len(full)
+    al = (1,) * (nd - len(small)) + tuple(small)
+    axes = tuple(i for i in range(nd) if al[i] == 1 and full[i] != 1)
+    want = (x.astype(np.float64) * w.astype(np.float64)).sum(axis=axes, keepdims=True).reshape(small)
+    nred = int(np.prod([full[i] for i in axes]))
+    assert max_err(Y.grad.numpy(), want) <= 1e-5 * math.sqrt(nred) * float(np.abs(x).max()) * float(np.abs(w).max())
+    if int(np.prod(full)) <= 1 << 20:
+        def script(api):
+            a, b = T(api, x, True), T(api, y, True)
+            a.mul(b).mul(T(api, w)).sum().backward()
+            return b.grad.numpy()
+        assert_close(script(gpu), script(orc), 1e-5 * math.sqrt(nred) * 16, str(small))
+
+
 def test_scalar_and_bias_gradients_of_large_tensors_vs_oracle(gpu, orc):
     # a broadcast operand's gradient is a sum over every element of a [3000, 1024] tensor (3.07M rows of one
     # column: more row blocks than one grid axis holds), and over its 3000 rows for a [1024] operand
