@@ -184,7 +184,7 @@ def bench_extras(r, with_cpu):
     dx, dw, dy = r.to_device(x), r.to_device(w), r.malloc(4 * 4096 * 4)
     by = 4.0 * (4096 * 4096 + 2 * 4 * 4096)
     fl = 2.0 * 4 * 4096 * 4096
-    kern = "skinny_cols_kernel<4, true, true, false, true>"
+    kern = "skinny_cols_kernel<4, true, true, false, true, true>"
     # launches of a few microseconds are issued from C (mni_rocm_sgemm_timed) so that the host stays ahead
     ms_warm = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 10, 200)
     ms_sus = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 3000, 1000)

@@ -78,7 +78,7 @@ __device__ __forceinline__ unsigned sk_load_flag(const unsigned *p) {
 // groups (K % SK_UNROLL == 0), which removes the guarded path and its address
 // arithmetic from the kernel; this kernel lives for a few microseconds, so the
 // length of its prologue shows.
-template <int MR, bool XC, bool FUSED, bool TAIL, bool LEAN>
+template <int MR, bool XC, bool FUSED, bool TAIL, bool LEAN, bool PLAIN = false>
 __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLaunch s) {
     constexpr int U = SK_UNROLL;
     // LEAN (the decode shape): one batch, exactly MR rows, whole 256-column
@@ -92,7 +92,10 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_cols_kernel(const SkinnyLau
     // against 13.4 (MI355X, W in the Infinity Cache).
     static_assert(!LEAN || (XC && FUSED && !TAIL), "LEAN implies XC, FUSED, !TAIL");
     const int rows = LEAN ? MR : s.rows, batch = LEAN ? 1 : s.batch;
-    const int epilogue = s.epilogue, accumulate = s.accumulate;
+    // PLAIN (with LEAN): no epilogue and no accumulation either -- the benchmark's product; carrying the two as
+    // run-time values cost it 0.15 of its 12.4 us.
+    static_assert(!PLAIN || LEAN, "PLAIN implies LEAN");
+    const int epilogue = PLAIN ? (int)MNI_EPI_NONE : s.epilogue, accumulate = PLAIN ? 0 : s.accumulate;
     const int64_t o_cs = LEAN ? 1 : s.o_cs;
     const int x_bcount = LEAN ? 1 : s.x_bcount, w_bcount = LEAN ? 1 : s.w_bcount;
     __shared__ float4 red[SK_WAVES - 1][MR][64];
@@ -516,9 +519,13 @@ static void launch_skinny_cols_mr(const SkinnyLaunch &s, dim3 grid, bool fused) 
     hipStream_t st = ctx().stream;
     const int variant = (s.x_cs == 1 ? 4 : 0) | (fused ? 2 : 0) | (s.K % SK_UNROLL != 0 ? 1 : 0);
     if (fused && skinny_decode_shape(s)) {
+        const bool plain = s.epilogue == MNI_EPI_NONE && !s.accumulate;
         switch (s.rows) {
 #define MNI_SK_LEAN(R) \
-    case R: MNI_KERNEL_LAUNCH((skinny_cols_kernel<R, true, true, false, true>), grid, block, 0, st, s); return;
+    case R: \
+        if (plain) MNI_KERNEL_LAUNCH((skinny_cols_kernel<R, true, true, false, true, true>), grid, block, 0, st, s); \
+        else MNI_KERNEL_LAUNCH((skinny_cols_kernel<R, true, true, false, true>), grid, block, 0, st, s); \
+        return;
             MNI_SK_DECODE_ROWS(MNI_SK_LEAN)
 #undef MNI_SK_LEAN
         }
@@ -549,7 +556,7 @@ static int skinny_cols_fused_occupancy_mr(const SkinnyLaunch &s) {
             hipError_t e = hipErrorInvalidValue;
             switch (s.rows) {
 #define MNI_SK_LEAN(R) \
-    case R: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<R, true, true, false, true>, SK_THREADS, 0); break;
+    case R: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, skinny_cols_kernel<R, true, true, false, true>, SK_THREADS, 0); break;  /* (the plain form needs no more) */
                 MNI_SK_DECODE_ROWS(MNI_SK_LEAN)
 #undef MNI_SK_LEAN
             }
