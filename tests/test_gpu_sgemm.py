@@ -944,6 +944,26 @@ def test_outer_product_kernel_is_the_plan_for_a_small_batch_weight_gradient_and_
         rocm.sgemm(32, 32, 600, dX, dY, dC, a_strides=(1, 32), algo=N.ALGO_OUTER)
 
 
+@pytest.mark.parametrize("m,n,k", [(1001, 1003, 999), (1538, 1537, 1400), (2048, 1027, 1500), (1281, 2050, 1300)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_big_products_with_edges_off_a_multiple_of_four_integer_exact(dev, rocm, m, n, k, ta, tb):
+    # An operand contiguous along M or N with that extent off a multiple of 4: the product is cut into the part that
+    # ends on a multiple of 4 and a strip of 1 to 3 rows / columns (both, and their corner, when both operands are
+    # such).  Same sums; with a bias and accumulation across the cut as well.
+    a = synth.small_ints(m + k, (k, m) if ta else (m, k), 3)
+    b = synth.small_ints(n + k, (n, k) if tb else (k, n), 3, stream=1)
+    opa = a.T if ta else a
+    opb = b.T if tb else b
+    want = (opa.astype(np.int64) @ opb.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b, ta=ta, tb=tb)[0], want)
+    bias = synth.small_ints(7, (n,), 5, stream=2); old = synth.small_ints(8, (m, n), 9, stream=3)
+    dA, dB, dBias, dC = dev.put(a), dev.put(b), dev.put(bias), dev.put(old)
+    rocm.sgemm(m, n, k, dA, dB, dC, a_strides=(1, m) if ta else None, b_strides=(1, k) if tb else None, bias=dBias,
+               epilogue=N.EPI_BIAS_RELU, accumulate=True)
+    z = np.maximum(want.astype(np.float64) + bias, 0.0) + old
+    assert np.array_equal(rocm.to_host(dC, (m, n)), z.astype(np.float32))
+
+
 @pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 7, 8, 9, 10, 13, 17])
 def test_few_output_columns_under_a_tall_operand_integer_exact(dev, rocm, n):
     # A head with a few outputs: the [K, n] weight is small and, for most n, not laid out for 16-byte loads.  The
