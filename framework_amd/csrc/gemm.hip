@@ -684,9 +684,16 @@ int sgemm(const mni_gemm_desc &d) {
     // kernel its element-wise loads of B; copied once into a K-contiguous layout it is read in 16-byte pieces
     // (65536 x 768 against [768, 10]: 77 us as given, 50 with the copy).  Not in the entry point that may not
     // allocate: the plan's own workspace has the one fixed block.
-    if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && !ctx().scratch && d.B.col_stride == 1 && d.N > 1 &&
-        (d.B.row_stride % 4 != 0 || !aligned16(d.B.ptr) || (d.B.batch_count > 1 && d.B.batch_stride % 4 != 0)) && d.K % 4 == 0 &&
-        d.K * d.N * d.B.batch_count <= (1 << 18) && d.M * d.K * d.batch >= 16 * d.K * d.N * d.B.batch_count && d.M * d.K * d.batch >= (1LL << 20)) {
+    // The same copy pays for a B of up to 16 MB whose N is off a multiple of 4 under a product of 1 to 6 GFLOP (too
+    // small to be cut into a main part and a strip): its edge tiles would take the element-wise loop and the
+    // launch would wait for them (1001 x 1003 x 999: 41 us as given, 24 with B given K-contiguous).
+    const double flops = 2.0 * (double)d.M * (double)d.N * (double)d.K * (double)d.batch;
+    const bool small_b = (d.B.row_stride % 4 != 0 || !aligned16(d.B.ptr) || (d.B.batch_count > 1 && d.B.batch_stride % 4 != 0)) && d.K % 4 == 0 &&
+                         d.K * d.N * d.B.batch_count <= (1 << 18) && d.M * d.K * d.batch >= 16 * d.K * d.N * d.B.batch_count &&
+                         d.M * d.K * d.batch >= (1LL << 20);
+    const bool ragged_b = d.N % 4 != 0 && d.N >= 64 && d.M >= 64 && d.B.row_stride != 1 && flops >= 1e9 && flops < 6e9 &&
+                          d.K * d.N * d.B.batch_count <= (1 << 22) && d.epilogue <= MNI_EPI_BIAS_GELU;
+    if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && !ctx().scratch && d.B.col_stride == 1 && d.N > 1 && (small_b || ragged_b)) {
         void *packed = nullptr;
         MNI_TRY(gemm_ws_alloc(&packed, (size_t)(d.K * d.N * d.B.batch_count) * sizeof(float)));
         const int64_t shape[3] = {d.B.batch_count, d.N, d.K}, strides[3] = {d.B.batch_stride, d.B.col_stride, d.B.row_stride};
