@@ -693,20 +693,35 @@ int sgemm(const mni_gemm_desc &d) {
                          d.M * d.K * d.batch >= (1LL << 20);
     const bool ragged_b = d.N % 4 != 0 && d.N >= 64 && d.M >= 64 && d.B.row_stride != 1 && flops >= 1e9 && flops < 6e9 &&
                           d.K * d.N * d.B.batch_count <= (1 << 22) && d.epilogue <= MNI_EPI_BIAS_GELU;
-    if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && !ctx().scratch && d.B.col_stride == 1 && d.N > 1 && (small_b || ragged_b)) {
-        void *packed = nullptr;
-        MNI_TRY(gemm_ws_alloc(&packed, (size_t)(d.K * d.N * d.B.batch_count) * sizeof(float)));
-        const int64_t shape[3] = {d.B.batch_count, d.N, d.K}, strides[3] = {d.B.batch_stride, d.B.col_stride, d.B.row_stride};
-        int rc = k_strided_copy((float *)packed, d.B.ptr, shape, strides, 3);
-        if (rc == MNI_OK) {
-            mni_gemm_desc d2 = d;
-            d2.B.ptr = (const float *)packed;
+    // (and for an A given as its transpose whose M is off a multiple of 4: 1001 x 1003 x 999 transposed-A 56 us)
+    const bool ragged_a = d.M % 4 != 0 && d.M >= 64 && d.N >= 64 && d.A.row_stride == 1 && d.A.col_stride != 1 && flops >= 1e9 && flops < 6e9 &&
+                          d.M * d.K * d.A.batch_count <= (1 << 22) && d.epilogue <= MNI_EPI_BIAS_GELU;
+    const bool pack_b = d.B.col_stride == 1 && d.N > 1 && (small_b || ragged_b);
+    if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && !ctx().scratch && (pack_b || ragged_a)) {
+        void *packed_a = nullptr, *packed_b = nullptr;
+        mni_gemm_desc d2 = d;
+        int rc = MNI_OK;
+        if (pack_b) {
+            rc = gemm_ws_alloc(&packed_b, (size_t)(d.K * d.N * d.B.batch_count) * sizeof(float));
+            const int64_t shape[3] = {d.B.batch_count, d.N, d.K}, strides[3] = {d.B.batch_stride, d.B.col_stride, d.B.row_stride};
+            if (rc == MNI_OK) rc = k_strided_copy((float *)packed_b, d.B.ptr, shape, strides, 3);
+            d2.B.ptr = (const float *)packed_b;
             d2.B.row_stride = 1;
             d2.B.col_stride = d.K;
             d2.B.batch_stride = d.K * d.N;
-            rc = run_mfma(d2);
         }
-        gemm_ws_free(packed);
+        if (rc == MNI_OK && ragged_a) {
+            rc = gemm_ws_alloc(&packed_a, (size_t)(d.M * d.K * d.A.batch_count) * sizeof(float));
+            const int64_t shape[3] = {d.A.batch_count, d.M, d.K}, strides[3] = {d.A.batch_stride, d.A.row_stride, d.A.col_stride};
+            if (rc == MNI_OK) rc = k_strided_copy((float *)packed_a, d.A.ptr, shape, strides, 3);
+            d2.A.ptr = (const float *)packed_a;
+            d2.A.row_stride = d.K;
+            d2.A.col_stride = 1;
+            d2.A.batch_stride = d.M * d.K;
+        }
+        if (rc == MNI_OK) rc = run_mfma(d2);
+        gemm_ws_free(packed_a);
+        gemm_ws_free(packed_b);
         return rc;
     }
     return run_mfma(d);
