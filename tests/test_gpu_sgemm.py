@@ -944,6 +944,28 @@ def test_outer_product_kernel_is_the_plan_for_a_small_batch_weight_gradient_and_
         rocm.sgemm(32, 32, 600, dX, dY, dC, a_strides=(1, 32), algo=N.ALGO_OUTER)
 
 
+@pytest.mark.parametrize("batch,m,n,k", [(64, 16, 132, 256), (100, 1, 64, 512), (7, 33, 260, 100), (3, 128, 128, 64), (40, 5, 1024, 768)])
+def test_batches_of_a_against_one_shared_b_integer_exact(dev, rocm, batch, m, n, k):
+    # x[B, T, d] . W[d, n]: the batches of A are stacked at a uniform pitch, as are those of C, so the library runs one
+    # product of B x T rows (1024 products of one row each took 6.5 ms against 0.3).  Same values as batch by batch; not
+    # collapsed when C's batches are padded apart or A is itself broadcast.
+    a = synth.small_ints(batch + m, (batch, m, k), 3); b = synth.small_ints(n + k, (1, k, n), 3, stream=1)
+    want = np.einsum("bmk,kn->bmn", a.astype(np.int64), b[0].astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b), want)
+    bias = synth.small_ints(9, (n,), 5, stream=2)
+    dA, dB, dBias = dev.put(a), dev.put(b), dev.put(bias)
+    pad = m * n + 8                                        # C's batches apart: stays a batch of products
+    dC = dev.empty(batch * pad, fill=-7.0)
+    rocm.sgemm(m, n, k, dA, dB, dC, batch=batch, a_batch=(m * k, batch), b_batch=(0, 1), c_batch_stride=pad, bias=dBias, epilogue=N.EPI_BIAS)
+    got = rocm.to_host(dC, (batch, pad))
+    assert np.array_equal(got[:, :m * n].reshape(batch, m, n), want + bias) and np.all(got[:, m * n:] == -7.0)
+    dC2 = dev.empty(batch * m * n, fill=-7.0)             # the same, C contiguous: one product
+    before = rocm.launch_count()
+    rocm.sgemm(m, n, k, dA, dB, dC2, batch=batch, a_batch=(m * k, batch), b_batch=(0, 1), bias=dBias, epilogue=N.EPI_BIAS)
+    assert rocm.launch_count() - before <= 3
+    assert np.array_equal(rocm.to_host(dC2, (batch, m, n)), want + bias)
+
+
 @pytest.mark.parametrize("m,n,k", [(1001, 1003, 999), (1538, 1537, 1400), (2048, 1027, 1500), (1281, 2050, 1300)])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 def test_big_products_with_edges_off_a_multiple_of_four_integer_exact(dev, rocm, m, n, k, ta, tb):
