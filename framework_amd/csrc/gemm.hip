@@ -627,7 +627,8 @@ int sgemm(const mni_gemm_desc &d) {
     // Batches of A against one shared B, stacked at a uniform row pitch in A and in C (x[B, T, d] . W[d, n], and the
     // dX of it): one product of B x T rows.  As a batch of small products every batch pads its few rows to a tile
     // and reads B again ([1024, 1, 4096] . [4096, 4096]: 6.5 ms as 1024 products of one row, 0.3 as one of 1024 rows).
-    if (d.batch > 1 && d.B.batch_count == 1 && d.A.batch_count == d.batch && d.A.batch_stride == d.M * d.A.row_stride &&
+    if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.batch > 1 && d.B.batch_count == 1 && d.A.batch_count == d.batch &&
+        d.A.batch_stride == d.M * d.A.row_stride &&
         d.c_batch_stride == d.M * d.ldc && d.epilogue <= MNI_EPI_BIAS_GELU && d.M * d.batch <= 0x7fffffffLL) {
         mni_gemm_desc one = d;
         one.M = d.M * d.batch;

@@ -101,9 +101,15 @@ __global__ __launch_bounds__(TINY_THREADS) void gemm_tiny_pair_kernel(const Tiny
 // Few outputs and a short K: what a launch of 256-thread workgroups computes in about the time the launch takes.
 // Measured on MI355X against the tile kernel's 64 x 64 tiles (us): 32 x 64 x 10 2.6 / 5.3, 32 x 3 x 64 4.7 / 6.7,
 // 64 x 64 x 64 3.3 / 5.4, 256 x 256 x 64 3.5 / 5.8, 128 x 64 x 128 4.6 / 6.6, 128 x 128 x 256 7.1 / 8.6.
+// Also a large batch of products of at most 256 outputs each, which would each pad a 64 x 64 tile (us, this kernel
+// against the tile kernel: 65536 x (4 x 4 x 4) 6.1 / 223, 4096 x (8 x 8 x 64) 6.2 / 27.0, 4096 x (16 x 16 x 16) 6.8 / 25.2,
+// 8192 x (64 x 1 x 64) 27.7 / 62.4, 8192 x (1 x 64 x 64) 20.9 / 26.5; 1024 x (32 x 32 x 32) 10.1 / 8.6 stays with tiles).
 bool gemm_tiny_eligible(const GemmLaunch &g) {
     const int64_t outputs = (int64_t)g.M * g.N * g.batch;
-    return g.epilogue <= MNI_EPI_BIAS_GELU && outputs > 0 && outputs <= 65536 && g.K <= 256 && outputs * (g.K > 0 ? g.K : 1) <= (1 << 22);
+    if (g.epilogue > MNI_EPI_BIAS_GELU || outputs <= 0) return false;
+    const int64_t k = g.K > 0 ? g.K : 1;
+    if (outputs <= 65536 && g.K <= 256 && outputs * k <= (1 << 22)) return true;
+    return g.batch >= 64 && (int64_t)g.M * g.N <= 256 && g.K <= 128 && outputs * k <= (1 << 27);
 }
 
 static int tiny_form(const GemmLaunch &g) { return (g.a_cs == 1 && g.K >= 4 ? 1 : 0) | (g.b_rs == 1 && g.K >= 4 ? 2 : 0); }

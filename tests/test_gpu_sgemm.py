@@ -944,6 +944,19 @@ def test_outer_product_kernel_is_the_plan_for_a_small_batch_weight_gradient_and_
         rocm.sgemm(32, 32, 600, dX, dY, dC, a_strides=(1, 32), algo=N.ALGO_OUTER)
 
 
+@pytest.mark.parametrize("batch,m,n,k", [(4096, 8, 8, 64), (20000, 3, 3, 3), (300, 16, 16, 128), (2048, 1, 64, 64), (2048, 64, 1, 64), (70, 2, 100, 7)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+def test_large_batches_of_tiny_products_integer_exact(dev, batch, m, n, k, ta, tb):
+    # thousands of products of at most 256 outputs each: one thread per output over the whole batch, not a padded
+    # 64 x 64 tile per product (65536 x (4 x 4 x 4): 223 us -> 6)
+    a = synth.small_ints(batch + m, (batch, k, m) if ta else (batch, m, k), 3)
+    b = synth.small_ints(batch + n, (batch, n, k) if tb else (batch, k, n), 3, stream=1)
+    opa = a.transpose(0, 2, 1) if ta else a
+    opb = b.transpose(0, 2, 1) if tb else b
+    want = np.einsum("bmk,bkn->bmn", opa.astype(np.int64), opb.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b, ta=ta, tb=tb), want)
+
+
 @pytest.mark.parametrize("batch,m,n,k", [(64, 16, 132, 256), (100, 1, 64, 512), (7, 33, 260, 100), (3, 128, 128, 64), (40, 5, 1024, 768)])
 def test_batches_of_a_against_one_shared_b_integer_exact(dev, rocm, batch, m, n, k):
     # x[B, T, d] . W[d, n]: the batches of A are stacked at a uniform pitch, as are those of C, so the library runs one
