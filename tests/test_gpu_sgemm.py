@@ -957,6 +957,16 @@ def test_large_batches_of_tiny_products_integer_exact(dev, batch, m, n, k, ta, t
     assert np.array_equal(run_gemm(dev, a, b, ta=ta, tb=tb), want)
 
 
+@pytest.mark.parametrize("batch,n,k", [(256, 4096, 128), (32, 8192, 64), (1024, 512, 64), (16, 1000, 100), (40, 333, 7), (64, 2048, 4)])
+def test_one_row_per_batch_against_k_contiguous_b_integer_exact(dev, batch, n, k):
+    # q[B, 1, d] . K[B, n, d]^T, the scores of one new token per head: a thread per score reads its own row of K
+    # (256 x (1 x 4096 x 128): 166 us through tiles -> 122)
+    a = synth.small_ints(batch + k, (batch, 1, k), 3)
+    b = synth.small_ints(batch + n, (batch, n, k), 3, stream=1)
+    want = np.einsum("bmk,bnk->bmn", a.astype(np.int64), b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b, tb=True), want)
+
+
 @pytest.mark.parametrize("batch,m,n,k", [(64, 16, 132, 256), (100, 1, 64, 512), (7, 33, 260, 100), (3, 128, 128, 64), (40, 5, 1024, 768)])
 def test_batches_of_a_against_one_shared_b_integer_exact(dev, rocm, batch, m, n, k):
     # x[B, T, d] . W[d, n]: the batches of A are stacked at a uniform pitch, as are those of C, so the library runs one
