@@ -203,7 +203,9 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         // dots at 9 / 16 rows against tiles: [50304, 768] 80 / 95 against 48, [4096, 4096] 26 / 28 against 24,
         // [1024, 4096] 22 / 25 against 12, [11008, 4096] 56 / 61 against 58).
         // Nor for a short K, where half its lanes have nothing to load (100000 x 128 against 8 columns: 55 us, tiles 22).
-        if (w_dots && d.split_k <= 1 && ((s.rows <= 8 && s.K >= 512) || d.algo != MNI_ALGO_AUTO)) {
+        // (One row: from K = 384, 64 x (1 x 4096 x 384) 72 us against 105 through tiles; at K = 256 130 against 144, and the
+        // thread-per-output kernel's 121 is ahead of both.)
+        if (w_dots && d.split_k <= 1 && ((s.rows <= 8 && (s.K >= 512 || (s.rows == 1 && s.K >= 384))) || d.algo != MNI_ALGO_AUTO)) {
             *rc = launch_skinny_dots(s);
             gemm_ws_free(packed);
             return true;
@@ -241,6 +243,10 @@ static bool panel_plan(const GemmLaunch &g, int cus) {
     // tile kernel's plans, microseconds: 32 x (512 x 512 x 64) 13.8 vs 19.5, 8 x (1024 x 1024 x 64) 13.0 vs
     // 18.5, 4096 x 4096 x 64 22.3 vs 34.9, K = 32: 9.9 vs 13.7, 16 x (384 x 384 x 64) 8.1 vs 8.7; at
     // 8 x (512 x 512 x 64), 128 tiles, the tile kernel's 64 x 64 tiles are ahead, 7.4 vs 8.0.
+    // Not up to 64 rows or columns, where half or more of every tile would be padding (us, panel against 64 x 64 tiles):
+    // 64 x (64 x 4096 x 64) 53 / 34, 64 x (4096 x 32 x 64) 49 / 33, 1024 x (64 x 256 x 64) 55 / 37, 256 x (2 x 4096 x 64) 163 / 104;
+    // from 96 on it is ahead: 64 x (96 x 4096 x 64) 53 / 62, 1024 x (96 x 96 x 32) 14 / 26, 1024 x (128 x 128 x 64) 29 / 36.
+    if (g.M <= 64 || g.N <= 64) return false;
     const int64_t tiles = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
     return tiles * 2 > cus;
 }

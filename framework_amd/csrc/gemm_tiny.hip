@@ -112,8 +112,11 @@ bool gemm_tiny_eligible(const GemmLaunch &g) {
     if (g.batch >= 64 && (int64_t)g.M * g.N <= 256 && g.K <= 128 && outputs * k <= (1 << 27)) return true;
     // One row per batch against a B stored K-contiguous with a short K (q . K^T of one new token per head): a thread per
     // output reads its own row of B in 16-byte pieces; 256 x (1 x 4096 x 128) 122 us against 166 through tiles,
-    // 1024 x (1 x 512 x 64) 27 against 85, 32 x (1 x 8192 x 64) 15 against 45.
-    return g.M == 1 && g.batch >= 16 && g.b_rs == 1 && g.K >= 4 && g.K <= 128 && outputs * k <= (1LL << 28);
+    // 1024 x (1 x 512 x 64) 27 against 85, 32 x (1 x 8192 x 64) 15 against 45, 4 x (1 x 65536 x 64) 15 against 45,
+    // 128 x (1 x 4096 x 256) 121 against 144.  Two rows up to K = 64 (256 x (2 x 4096 x 64) 82 against 104; at K = 128
+    // 187 against 166, and four rows 329 against 166).
+    if (g.batch < 4 || g.b_rs != 1 || g.K < 4 || outputs * k > (1LL << 28)) return false;
+    return (g.M == 1 && g.K <= 256) || (g.M == 2 && g.K <= 64);
 }
 
 static int tiny_form(const GemmLaunch &g) { return (g.a_cs == 1 && g.K >= 4 ? 1 : 0) | (g.b_rs == 1 && g.K >= 4 ? 2 : 0); }

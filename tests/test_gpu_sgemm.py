@@ -957,11 +957,14 @@ def test_large_batches_of_tiny_products_integer_exact(dev, batch, m, n, k, ta, t
     assert np.array_equal(run_gemm(dev, a, b, ta=ta, tb=tb), want)
 
 
-@pytest.mark.parametrize("batch,n,k", [(256, 4096, 128), (32, 8192, 64), (1024, 512, 64), (16, 1000, 100), (40, 333, 7), (64, 2048, 4)])
-def test_one_row_per_batch_against_k_contiguous_b_integer_exact(dev, batch, n, k):
+@pytest.mark.parametrize("batch,m,n,k", [(256, 1, 4096, 128), (32, 1, 8192, 64), (1024, 1, 512, 64), (16, 1, 1000, 100), (40, 1, 333, 7), (64, 1, 2048, 4),
+                                         (4, 1, 65536, 64), (32, 1, 4096, 256), (16, 1, 4096, 384), (128, 2, 4096, 64), (64, 2, 1024, 128),
+                                         (16, 64, 4096, 64), (16, 4096, 32, 64), (16, 96, 1024, 64)])
+def test_few_rows_per_batch_against_k_contiguous_b_integer_exact(dev, batch, m, n, k):
     # q[B, 1, d] . K[B, n, d]^T, the scores of one new token per head: a thread per score reads its own row of K
-    # (256 x (1 x 4096 x 128): 166 us through tiles -> 122)
-    a = synth.small_ints(batch + k, (batch, 1, k), 3)
+    # (256 x (1 x 4096 x 128): 166 us through tiles -> 122); K = 384 goes to the dots kernel, two rows of K <= 64 to the
+    # thread-per-output kernel, up to 64 rows or columns of K <= 64 to 64 x 64 tiles rather than 128 x 128 panels
+    a = synth.small_ints(batch + k, (batch, m, k), 3)
     b = synth.small_ints(batch + n, (batch, n, k), 3, stream=1)
     want = np.einsum("bmk,bnk->bmn", a.astype(np.int64), b.astype(np.int64)).astype(np.float32)
     assert np.array_equal(run_gemm(dev, a, b, tb=True), want)
