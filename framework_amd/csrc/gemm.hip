@@ -107,7 +107,11 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         s.groups = 0; s.flags = nullptr; s.epoch = 0; s.max_reducers = 16; s.status = ctx().status_dev;
 
         const bool w_batch_ok = s.w_bcount <= 1 || (s.w_bs % 4) == 0;
-        const bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
+        bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
+        // (Many small products of 9 to 16 rows: the 16-row form gives a workgroup 256 columns, and under that many most
+        // of it idles -- 8192 x (16 x 64 x 16) 109 us against 47 through tiles.  Nor with a short K: 2048 x (16 x 256 x 32)
+        // 40 against 43, but 48 against 24 through the outer-product kernel when A is given as its transpose.)
+        if (d.algo == MNI_ALGO_AUTO && s.rows > 8 && s.batch > 1 && (s.cols < 256 || s.K < 64)) w_cols = false;
         const bool x_batch_ok = s.x_bcount <= 1 || (s.x_bs % 4) == 0;
         // (the pitch of X only matters from the second row on)
         const bool x_dots = s.x_cs == 1 && (s.rows == 1 || (s.x_rs % 4) == 0) && aligned16(s.X) && x_batch_ok;
@@ -291,6 +295,14 @@ static bool outer_plan(const GemmLaunch &g, int cus) {
     const int64_t outputs = (int64_t)g.M * g.N * g.batch;
     // (K = 192 / 256 / 512: 4096 x 4096 53.9 / 70.4 / 129 against 60.3 / 74.5 / 131, 8192 x 8192 202 / 260 / 497 against 230 /
     // 286 / 510, 2048 x 2048 16.3 / 20.2 / 47.8 against 17.7 / 21.2 / 35.7, 4096 x 11008 156 / 200 / 376 against 156 / 193 / 344)
+    // A wavefront's block is 32 x 128, the tile kernel's smallest tile 64 x 64: not where this kernel would pad small
+    // or narrow products more than tiles do (us, this kernel against tiles: 2048 x (64 x 64 x 64) 38 / 23,
+    // 2048 x (64 x 32 x 64) 39 / 21, 512 x (128 x 64 x 128) 19 / 15; level padding or less: 4096 x (32 x 64 x 32) 24 / 27,
+    // 1024 x (80 x 80 x 80) 24 / 45, 2048 x (16 x 256 x 32) 24 / 42, 8192 x (16 x 64 x 16) 28 / 47).
+    const int64_t mn = (int64_t)g.M * g.N;
+    const int64_t own_pad = (int64_t)((g.M + 31) / 32 * 32) * ((g.N + 127) / 128 * 128);
+    const int64_t tile_pad = (int64_t)((g.M + 63) / 64 * 64) * ((g.N + 63) / 64 * 64);
+    if (own_pad > tile_pad && own_pad * 9 > mn * 10) return false;
     if (outputs >= (1LL << 21)) return g.K <= 256;
     return outputs >= (1LL << 16) && g.K <= 48;  // (512 x 512: K = 48 5.9 against 6.8, K = 64 6.9 against 6.0)
 }

@@ -109,7 +109,10 @@ bool gemm_tiny_eligible(const GemmLaunch &g) {
     if (g.epilogue > MNI_EPI_BIAS_GELU || outputs <= 0) return false;
     const int64_t k = g.K > 0 ? g.K : 1;
     if (outputs <= 65536 && g.K <= 256 && outputs * k <= (1 << 22)) return true;
-    if (g.batch >= 64 && (int64_t)g.M * g.N <= 256 && g.K <= 128 && outputs * k <= (1 << 27)) return true;
+    // (With B along K and several columns, neighbouring lanes read rows of B 4 K bytes apart and the limit is 2^25:
+    // 4096 x (16 x 16 x 64) with B transposed 38 / 30, 2048 x (16 x 16 x 128) 37 / 23, 4096 x (8 x 8 x 64) 11 / 28.)
+    const int64_t many_limit = g.b_rs == 1 && g.N > 1 && g.M > 1 ? (1 << 25) : (1 << 27);
+    if (g.batch >= 64 && (int64_t)g.M * g.N <= 256 && g.K <= 128 && outputs * k <= many_limit) return true;
     // One row per batch against a B stored K-contiguous with a short K (q . K^T of one new token per head): a thread per
     // output reads its own row of B in 16-byte pieces; 256 x (1 x 4096 x 128) 122 us against 166 through tiles,
     // 1024 x (1 x 512 x 64) 27 against 85, 32 x (1 x 8192 x 64) 15 against 45, 4 x (1 x 65536 x 64) 15 against 45,

@@ -970,6 +970,21 @@ def test_few_rows_per_batch_against_k_contiguous_b_integer_exact(dev, batch, m, 
     assert np.array_equal(run_gemm(dev, a, b, tb=True), want)
 
 
+@pytest.mark.parametrize("batch,m,n,k,ta,tb", [(512, 64, 64, 64, True, False), (512, 64, 32, 64, True, False), (256, 80, 80, 80, True, False),
+                                               (512, 32, 64, 32, True, False), (1024, 16, 64, 16, False, False), (1024, 16, 64, 16, True, False),
+                                               (256, 16, 256, 32, True, False), (256, 16, 256, 32, False, False), (2048, 16, 16, 64, False, True),
+                                               (1024, 16, 16, 32, False, True), (300, 12, 100, 20, False, False), (3, 4096, 4160, 16, True, False)])
+def test_many_small_products_under_the_planner_integer_exact(dev, batch, m, n, k, ta, tb):
+    # attention-sized products of short sequences, forward and backward: which of the outer-product kernel (32 x 128 blocks),
+    # 64 x 64 tiles, the 16-row column kernel and the thread-per-output kernel takes them depends on how much each would pad
+    a = synth.small_ints(batch + m, (batch, k, m) if ta else (batch, m, k), 3)
+    b = synth.small_ints(batch + n, (batch, n, k) if tb else (batch, k, n), 3, stream=1)
+    opa = a.transpose(0, 2, 1) if ta else a
+    opb = b.transpose(0, 2, 1) if tb else b
+    want = np.einsum("bmk,bkn->bmn", opa.astype(np.int64), opb.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b, ta=ta, tb=tb), want)
+
+
 @pytest.mark.parametrize("batch,m,n,k", [(64, 16, 132, 256), (100, 1, 64, 512), (7, 33, 260, 100), (3, 128, 128, 64), (40, 5, 1024, 768)])
 def test_batches_of_a_against_one_shared_b_integer_exact(dev, rocm, batch, m, n, k):
     # x[B, T, d] . W[d, n]: the batches of A are stacked at a uniform pitch, as are those of C, so the library runs one
