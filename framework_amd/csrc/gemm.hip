@@ -111,7 +111,8 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         // (Many small products of 9 to 16 rows: the 16-row form gives a workgroup 256 columns, and under that many most
         // of it idles -- 8192 x (16 x 64 x 16) 109 us against 47 through tiles.  Nor with a short K: 2048 x (16 x 256 x 32)
         // 40 against 43, but 48 against 24 through the outer-product kernel when A is given as its transpose.)
-        if (d.algo == MNI_ALGO_AUTO && s.rows > 8 && s.batch > 1 && (s.cols < 256 || s.K < 64)) w_cols = false;
+        // (A single narrow product likewise: 16 x 16 x 16384 61 us against 17 through tiles in K slices, 10 x 128 x 16384 59 / 29.)
+        if (d.algo == MNI_ALGO_AUTO && s.rows > 8 && (s.cols < 256 || (s.batch > 1 && s.K < 64))) w_cols = false;
         const bool x_batch_ok = s.x_bcount <= 1 || (s.x_bs % 4) == 0;
         // (the pitch of X only matters from the second row on)
         const bool x_dots = s.x_cs == 1 && (s.rows == 1 || (s.x_rs % 4) == 0) && aligned16(s.X) && x_batch_ok;
@@ -334,13 +335,15 @@ static bool fewrows_takes(const mni_gemm_desc &d) {
 // and reads what the slices wrote.  Fitted to, and within 10 % of, 60 measured plans: M = 24..384 against
 // (N, K) = (4096, 4096), (4096, 1024), (1024, 4096), (11008, 4096), (4096, 11008), s = 1..16; e.g.
 // 64 x 4096 x 4096: s = 1, 2, 4, 8, 16 measured 68.0 / 40.2 / 25.4 / 26.7 / 30.5 us, estimated 73.7 / 41.8 / 25.1 /
-// 25.6 / 31.8.  The smallest s within 3 % of the best estimate wins; slices keep at least 8 K steps.
+// 25.6 / 31.8.  The smallest s within 3 % of the best estimate wins; slices keep at least 8 K steps (2 when K has at most 32).
 static int split_for_few_tiles(int64_t tiles, int ktiles, int cus, int64_t out_bytes) {
     static const int cand[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64};
     double best = 0.0;
     int best_s = 1;
     for (int s : cand) {
-        if (s > 1 && ktiles / s < 8) break;
+        // (Up to 32 K steps a slice may be as short as two: 64 x 512 x 512 in 1 / 2 / 4 / 8 slices measured 12.9 / 11.1 / 8.7 /
+        // 8.4 us, estimated 12.1 / 10.2 / 8.0 / 6.9; 256 x 512 x 512 13.0 / 11.4 / 9.3 / 9.6; 64 x 1024 x 256 8.9 / 9.2 / 7.9 / 8.4.)
+        if (s > 1 && ktiles / s < (ktiles <= 32 ? 2 : 8)) break;
         const int64_t per_cu = (tiles * s + cus - 1) / cus;
         const int steps = (ktiles + s - 1) / s;
         double t = ((double)per_cu * (steps + 3) + 3) * (per_cu > 1 ? 0.48 : 0.55);

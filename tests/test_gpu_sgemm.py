@@ -985,6 +985,19 @@ def test_many_small_products_under_the_planner_integer_exact(dev, batch, m, n, k
     assert np.array_equal(run_gemm(dev, a, b, ta=ta, tb=tb), want)
 
 
+@pytest.mark.parametrize("m,n,k,ta,tb", [(16384, 16, 16, False, False), (16384, 16, 16, False, True), (784, 128, 64, True, False), (1024, 256, 32, False, False),
+                                         (4096, 10, 128, False, False), (4096, 64, 10, False, True), (64, 256, 256, False, True), (64, 512, 512, False, True),
+                                         (256, 512, 512, False, False), (64, 1024, 256, False, True), (16, 16, 16384, True, False), (64, 10, 16384, True, False),
+                                         (128, 10, 1024, True, False), (300, 300, 64, True, False)])
+def test_small_layers_under_the_planner_integer_exact(dev, m, n, k, ta, tb):
+    # the products of Linear layers of 10 to 512 features under batches of 64 to 16384 rows (forward, dX, dW): thread-per-output
+    # kernel up to 2^18 outputs, short K slices for a handful of 64 x 64 tiles, no 16-row column kernel under 256 columns
+    a = synth.small_ints(m + k, (k, m) if ta else (m, k), 2)
+    b = synth.small_ints(n + k, (n, k) if tb else (k, n), 2, stream=1)
+    want = ((a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, b, ta, tb)[0], want)
+
+
 @pytest.mark.parametrize("batch,m,n,k", [(64, 16, 132, 256), (100, 1, 64, 512), (7, 33, 260, 100), (3, 128, 128, 64), (40, 5, 1024, 768)])
 def test_batches_of_a_against_one_shared_b_integer_exact(dev, rocm, batch, m, n, k):
     # x[B, T, d] . W[d, n]: the batches of A are stacked at a uniform pitch, as are those of C, so the library runs one
