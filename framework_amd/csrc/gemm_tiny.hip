@@ -109,13 +109,14 @@ bool gemm_tiny_eligible(const GemmLaunch &g) {
     if (g.epilogue > MNI_EPI_BIAS_GELU || outputs <= 0) return false;
     const int64_t k = g.K > 0 ? g.K : 1;
     // With B along K and several columns, neighbouring lanes read rows of B 4 K bytes apart: 65536 outputs and 2^22
-    // multiply-adds at most (at K = 256 that is a little wide: 64 x 256 x 256 with B transposed 10.8 / 8.8).  With B along N
+    // multiply-adds at most, and beyond K = 128 only up to 1024 outputs (64 x 256 x 256 with B transposed 10.8 / 8.8,
+    // 64 x 32 x 256 10.7 / 8.5).  With B along N
     // up to 2^18 outputs and 2^23 multiply-adds: 16384 x 16 x 16
     // 3.4 / 6.0, 784 x 128 x 64 with A transposed 4.4 / 6.0, 1024 x 256 x 32 4.4 / 5.6, 4096 x 10 x 128 6.9 / 9.6; 256 x 256 x 256 7.7 / 8.9
     // stays with tiles.
     // (rows of B of up to 64 bytes are no such matter: 4096 x 64 x 10 with B transposed 3.6 / 6.1, 16384 x 16 x 16 3.8 / 5.9)
     const bool b_along_k = g.b_rs == 1 && g.N > 1 && g.K > 16;
-    if (b_along_k ? outputs <= 65536 && g.K <= 256 && outputs * k <= (1 << 22)
+    if (b_along_k ? outputs <= (g.K <= 128 ? 65536 : 1024) && g.K <= 256 && outputs * k <= (1 << 22)
                   : outputs <= (1 << 18) && g.K <= 256 && outputs * k <= (1 << 23)) return true;
     // (With B along K and several columns, neighbouring lanes read rows of B 4 K bytes apart and the limit is 2^25:
     // 4096 x (16 x 16 x 64) with B transposed 38 / 30, 2048 x (16 x 16 x 128) 37 / 23, 4096 x (8 x 8 x 64) 11 / 28.)
