@@ -116,6 +116,8 @@ bool gemm_tiny_eligible(const GemmLaunch &g) {
     // stays with tiles.
     // (rows of B of up to 64 bytes are no such matter: 4096 x 64 x 10 with B transposed 3.6 / 6.1, 16384 x 16 x 16 3.8 / 5.9)
     const bool b_along_k = g.b_rs == 1 && g.N > 1 && g.K > 16;
+    // (Up to 8 rows of a K beyond 128 are the column kernel's, which slices K: 1 x 256 x 256 4.2 against 6.9 here, 4 rows 4.8 / 7.1.)
+    if (g.batch == 1 && g.M <= 8 && g.K > 128 && g.N >= 64 && g.N % 4 == 0 && g.b_cs == 1) return false;
     if (b_along_k ? outputs <= (g.K <= 128 ? 65536 : 1024) && g.K <= 256 && outputs * k <= (1 << 22)
                   : outputs <= (1 << 18) && g.K <= 256 && outputs * k <= (1 << 23)) return true;
     // (With B along K and several columns, neighbouring lanes read rows of B 4 K bytes apart and the limit is 2^25:
