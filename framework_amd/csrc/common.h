@@ -48,6 +48,13 @@ struct DeviceCtx {
     unsigned *fewrows_counters = nullptr;
     size_t fewrows_counter_cap = 0;
     unsigned skinny_epoch = 0;
+    // K-slice partials and arrival counters of the decode product (gemv_units_kernel): the partials carry the
+    // launch's epoch as a tag, so the buffer is written by that kernel alone and by nothing else, ever.
+    void *gemv_pa = nullptr;  // gemv_slot_cap pieces of 16 bytes
+    void *gemv_pb = nullptr;  // gemv_slot_cap pieces of 8 bytes
+    size_t gemv_slot_cap = 0;
+    unsigned *gemv_counters = nullptr;
+    size_t gemv_counter_cap = 0;
     // Device status word in pinned host memory that kernels can write: a kernel
     // whose bounded wait for another workgroup expires stores a DEVICE_STATUS_*
     // code there (and NaN into its outputs).  Every call that waits for the
@@ -156,7 +163,7 @@ __device__ __forceinline__ void softmax_line_workgroup(float *__restrict__ o, co
 #endif
 unsigned next_result_tag();
 int wait_result_word(unsigned tag, unsigned *value, bool *delivered);
-enum { DEVICE_STATUS_OK = 0, DEVICE_STATUS_STREAMK_WAIT = 1, DEVICE_STATUS_SKINNY_WAIT = 2 };
+enum { DEVICE_STATUS_OK = 0, DEVICE_STATUS_STREAMK_WAIT = 1, DEVICE_STATUS_SKINNY_WAIT = 2, DEVICE_STATUS_GEMV_WAIT = 3 };
 // hipStreamSynchronize on the library's stream, then the device status word:
 // MNI_ERR_HIP naming the kernel when a bounded wait expired since the last check.
 int sync_stream_checked(const char *what);

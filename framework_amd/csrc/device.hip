@@ -107,6 +107,14 @@ static int init_device(int device) {
     c.fewrows_counter_cap = 4096;
     MNI_HIP_CHECK(hipMalloc((void **)&c.fewrows_counters, c.fewrows_counter_cap * sizeof(unsigned)));
     MNI_HIP_CHECK(hipMemset(c.fewrows_counters, 0, c.fewrows_counter_cap * sizeof(unsigned)));
+    c.gemv_slot_cap = 256 * 8 * 32;  // one workgroup per CU, 8 rows, 32 column lanes
+    MNI_HIP_CHECK(hipMalloc(&c.gemv_pa, c.gemv_slot_cap * 16));
+    MNI_HIP_CHECK(hipMalloc(&c.gemv_pb, c.gemv_slot_cap * 8));
+    MNI_HIP_CHECK(hipMemset(c.gemv_pa, 0, c.gemv_slot_cap * 16));
+    MNI_HIP_CHECK(hipMemset(c.gemv_pb, 0, c.gemv_slot_cap * 8));
+    c.gemv_counter_cap = 256 * 4;
+    MNI_HIP_CHECK(hipMalloc((void **)&c.gemv_counters, c.gemv_counter_cap * sizeof(unsigned)));
+    MNI_HIP_CHECK(hipMemset(c.gemv_counters, 0, c.gemv_counter_cap * sizeof(unsigned)));
     // Pinned staging slots of upload_small, and one event per slot that says when its transfer has left it.
     MNI_HIP_CHECK(hipHostMalloc((void **)&c.stage_host, DeviceCtx::STAGE_SLOTS * DeviceCtx::STAGE_BYTES, hipHostMallocDefault));
     for (int i = 0; i < DeviceCtx::STAGE_SLOTS; ++i) MNI_HIP_CHECK(hipEventCreateWithFlags(&c.stage_done[i], hipEventDisableTiming));
@@ -198,6 +206,7 @@ int check_device_status(const char *what) {
     *(volatile unsigned *)c.status_host = DEVICE_STATUS_OK;
     const char *who = st == DEVICE_STATUS_STREAMK_WAIT  ? "gemm_mfma_kernel (stream-K): a finishing workgroup gave up waiting for a partial tile"
                       : st == DEVICE_STATUS_SKINNY_WAIT ? "skinny_cols_kernel: a reducing workgroup gave up waiting for a K-slice partial"
+                      : st == DEVICE_STATUS_GEMV_WAIT   ? "gemv_units_kernel: the adding wavefront gave up waiting for a K-slice partial"
                                                         : "a kernel reported an unknown status";
     return set_error(MNI_ERR_HIP, "%s: device status %u -- %s; results written since the last synchronisation hold NaN where "
                                   "the wait expired", what, st, who);

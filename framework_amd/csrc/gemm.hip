@@ -43,7 +43,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_OUTER)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_GEMV)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -65,10 +65,47 @@ static int next_epoch(unsigned *epoch) {
     DeviceCtx &c = ctx();
     if (++c.skinny_epoch == 0) {
         MNI_TRY(k_fill((float *)c.skinny_flags, 0.0f, (int64_t)c.skinny_flag_cap));
+        MNI_TRY(k_fill((float *)c.gemv_pa, 0.0f, (int64_t)c.gemv_slot_cap * 4));  // (the decode product's tags are epochs too)
+        MNI_TRY(k_fill((float *)c.gemv_pb, 0.0f, (int64_t)c.gemv_slot_cap * 2));
         c.skinny_epoch = 1;
     }
     *epoch = c.skinny_epoch;
     return MNI_OK;
+}
+
+// ---- the decode product ---------------------------------------------------------
+// x[<= 8, K] against a row-major W[K, N] whose column and K extents deal the CUs one workgroup each (gemm_gemv.hip).
+// True when it took the product (errors through *rc).
+static bool try_gemv_units(const SkinnyLaunch &s, const mni_gemm_desc &d, int *rc) {
+    DeviceCtx &c = ctx();
+    if (d.algo != MNI_ALGO_AUTO && d.algo != MNI_ALGO_GEMV) return false;
+    if (d.split_k > 1 || s.batch != 1 || s.rows > 8 || s.x_cs != 1 || s.w_cs != 1 || s.o_cs != 1) return false;
+    if ((s.w_rs % 4) != 0 || !aligned16(s.W) || (s.o_rs % 4) != 0 || !aligned16(s.out)) return false;
+    if (s.w_rs > 0x7fffffffLL || s.x_rs > 0x7fffffffLL || s.o_rs > 0x7fffffffLL) return false;
+    if (s.epilogue > MNI_EPI_BIAS_GELU || s.bias_on_rows) return false;
+    if (s.epilogue != MNI_EPI_NONE && !aligned16(s.bias)) return false;
+    if (s.accumulate && s.epilogue >= MNI_EPI_BIAS_RELU) return false;  // (the old output would have to wait for the sum)
+    int slices = 0, trips = 0;
+    if (!gemv_units_plan(s.rows, s.cols, s.K, c.compute_units, c.xcd_count, &slices, &trips)) return false;
+    // Several trips per workgroup are taken one after the other (16 loads per lane, used up, the next 16): ahead of the
+    // column kernel's four small workgroups per CU up to 4096 columns (us, cold: 4 x 4096 x 8192 23.2 against 30.3,
+    // 4 x 4096 x 16384 46.3 / 54.6), level at 16384 and 32768 columns (44.9 / 43.8, 87.3 / 87.5), behind at 8192
+    // (4 x 8192 x 8192 52.0 against 45.0).  One trip: 4 x 4096 x 4096 12.8 / 14.4, 1 row 12.2 / 13.5, 8 rows 14.5 / 16.3,
+    // 4 x 8192 x 2048 13.0 / 14.6, 4 x 32768 x 512 12.9 / 15.6, 4 x 16384 x 1024 13.3 / 14.3.
+    if (d.algo == MNI_ALGO_AUTO && trips > 1 && s.cols > 4096) return false;
+    if (!c.gemv_pa || gemv_units_partial_slots(s.rows, s.cols, slices) > c.gemv_slot_cap ||
+        (size_t)(s.cols / 128) * GEMV_COUNTERS_PER_UNIT > c.gemv_counter_cap)
+        return false;
+    GemvLaunch g;
+    g.W = s.W; g.X = s.X; g.out = s.out; g.bias = s.bias;
+    g.pa = (decltype(g.pa))c.gemv_pa; g.pb = (decltype(g.pb))c.gemv_pb;
+    g.count = c.gemv_counters; g.status = c.status_dev;
+    g.units = s.cols / 128; g.slices = slices; g.trips = trips;
+    g.w_rs = (int)s.w_rs; g.x_rs = (int)s.x_rs; g.o_rs = (int)s.o_rs;
+    g.epilogue = s.epilogue; g.accumulate = s.accumulate;
+    *rc = next_epoch(&g.epoch);
+    if (*rc == MNI_OK) *rc = launch_gemv_units(g, s.rows);
+    return true;
 }
 
 // ---- skinny path --------------------------------------------------------------
@@ -106,6 +143,8 @@ static bool try_skinny(const mni_gemm_desc &d, int *rc) {
         s.ws = nullptr; s.split_k = 1; s.k_per_slice = s.K;
         s.groups = 0; s.flags = nullptr; s.epoch = 0; s.max_reducers = 16; s.status = ctx().status_dev;
 
+        if (!swapped && try_gemv_units(s, d, rc)) return true;
+        if (d.algo == MNI_ALGO_GEMV) return false;
         const bool w_batch_ok = s.w_bcount <= 1 || (s.w_bs % 4) == 0;
         bool w_cols = s.w_cs == 1 && (s.w_rs % 4) == 0 && (s.cols % 4) == 0 && aligned16(s.W) && w_batch_ok;
         // (Many small products of 9 to 16 rows: the 16-row form gives a workgroup 256 columns, and under that many most
@@ -707,9 +746,14 @@ int sgemm(const mni_gemm_desc &d) {
     // 16 x 8192 x 8192 46 / 58, 16 x 1024 x 1024 8.5 / 8.4; at 8 rows the skinny kernel leads, 15.2 / 18.6)
     const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M > 8 && d.M <= 16 && fewrows_takes(d);
     if (!to_fewrows &&
-        ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS)) {
+        ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS ||
+         d.algo == MNI_ALGO_GEMV)) {
         int rc;
         if (try_skinny(d, &rc)) return rc;
+        if (d.algo == MNI_ALGO_GEMV)
+            return set_error(MNI_ERR_INVALID,
+                             "sgemm: shape/layout not eligible for the decode product kernel (1 to 8 rows, one batch, row-major 16-byte "
+                             "aligned B and C, N / 128 a multiple of 8 that divides the compute units, K a multiple of 512 slices)");
         if (d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS)
             return set_error(MNI_ERR_INVALID,
                              "sgemm: shape/layout not eligible for the skinny kernels "

@@ -118,6 +118,31 @@ int launch_skinny_dots(const SkinnyLaunch &s);
 int skinny_cols_block_cols();
 int skinny_cols_rows_per_pass();  // K rows one workgroup covers per trip
 
+// The decode product (gemm_gemv.hip): up to 8 rows of a K-contiguous X against a row-major W, one workgroup of 16
+// wavefronts per CU; workgroup id -> (unit = id % units: 128 columns, slice = id / units: trips * 512 rows of K).
+// Partials carry the launch's tag (epoch) in every piece; pa / pb / count belong to the library (DeviceCtx) and are
+// written by nothing else.
+static constexpr int GEMV_MAX_SLICES = 8;
+static constexpr int GEMV_COUNTERS_PER_UNIT = 4;  // one per summing wavefront (rows * 32 threads)
+struct GemvLaunch {
+    const float *W;
+    const float *X;
+    float *out;
+    const float *bias;  // one value per column, 16-byte aligned, or null
+    float __attribute__((ext_vector_type(4))) *pa;  // [unit][slice][rows * 32] pieces {x, y, z, tag}
+    float __attribute__((ext_vector_type(2))) *pb;  // the same of {w, tag}
+    unsigned *count;   // [unit][GEMV_COUNTERS_PER_UNIT], zero between launches (each count wraps to zero with its last arrival)
+    unsigned *status;  // device status word: set when the adding wavefront's bounded wait for a partial expires
+    unsigned epoch;
+    int units, slices, trips;
+    int w_rs, x_rs, o_rs;
+    int epilogue, accumulate;
+};
+// Whether the kernel takes rows x K against K x cols on this device, and with how many K slices / trips per workgroup.
+bool gemv_units_plan(int rows, int cols, int K, int cus, int xcds, int *slices, int *trips);
+size_t gemv_units_partial_slots(int rows, int cols, int slices);  // pieces of pa (and of pb) the plan writes
+int launch_gemv_units(const GemvLaunch &p, int rows);
+
 // Sums split-K partials ws[slice][batch][rows][cols] in slice order and
 // applies the epilogue; out addressed with (o_bs, o_rs, o_cs).
 struct ReduceLaunch {

@@ -148,10 +148,17 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * X^T dY of a small batch: both operands straight into the matrix
  * instruction's registers, the cost of writing C (error unless N % 4 == 0,
  * B and C 16-byte aligned with row strides in whole 16 bytes, no epilogue;
- * accumulate is honoured).  AUTO picks among them. */
+ * accumulate is honoured); GEMV = the decode product, 1 to 8 rows of a
+ * K-contiguous A against a row-major B that is as large as the product is
+ * expensive: one workgroup per compute unit, 128 columns and a K slice each,
+ * the K slices summed inside the launch by whichever wavefront arrives last
+ * (error unless one batch, N % 128 == 0 with N / 128 a divisor of the 256
+ * compute units and a multiple of 8, K a multiple of 512 * 256 / (N / 128),
+ * B, C and the bias 16-byte aligned with row strides in whole 16 bytes, and
+ * no activation together with accumulate).  AUTO picks among them. */
 enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
        MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7, MNI_ALGO_TINY = 8, MNI_ALGO_FEWROWS = 9,
-       MNI_ALGO_OUTER = 10 };
+       MNI_ALGO_OUTER = 10, MNI_ALGO_GEMV = 11 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),

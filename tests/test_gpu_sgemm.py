@@ -847,6 +847,102 @@ def test_skinny_cols_decode_shape_epilogues_and_accumulate(dev, rocm, m):
                 assert np.array_equal(got, want.astype(np.float32)), (epi, accumulate, algo)
 
 
+# ---- the decode product kernel (one workgroup per CU, tagged K-slice partials, the last wavefront to arrive adds) ----
+def _gemv_gemm(dev, a, b, ldb=None, **kw):
+    """a [m, k] against b [k, n] stored with row pitch ldb."""
+    r = dev.r
+    m, k = a.shape
+    n = b.shape[1]
+    ldb = ldb or n
+    store = np.zeros((k, ldb), np.float32)
+    store[:, :n] = b
+    dA, dB = dev.put(a), dev.put(store)
+    dC = dev.empty(m * n, fill=-7.0)
+    r.sgemm(m, n, k, dA, dB, dC, b_strides=(ldb, 1), **kw)
+    return r.to_host(dC, (m, n))
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_decode_product_kernel_integer_exact(dev, rocm, m):
+    # 4096 x 4096: 32 units x 8 K slices of one trip (the form fixed at compile time); forced and as the planner's choice,
+    # and repeated: every launch must find the counters of the last one back at zero
+    a = synth.small_ints(m, (m, 4096), 3)
+    b = synth.small_ints(m + 1, (4096, 4096), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    for algo in (N.ALGO_GEMV, N.ALGO_AUTO, N.ALGO_GEMV):
+        assert np.array_equal(_gemv_gemm(dev, a, b, algo=algo), want), algo
+    rocm.sync()   # (an adding wavefront's expired wait would be reported here)
+
+
+@pytest.mark.parametrize("m,n,k", [(4, 4096, 8192), (3, 8192, 2048), (8, 8192, 4096), (5, 16384, 1024), (2, 32768, 512), (7, 32768, 1024),
+                                   (1, 4096, 16384), (6, 16384, 2048)])
+def test_decode_product_kernel_other_plans_integer_exact(dev, rocm, m, n, k):
+    # 8, 4, 2 slices and none at all (32768 columns: every workgroup owns its columns outright), one and several trips
+    a = synth.small_ints(m, (m, k), 3)
+    b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(_gemv_gemm(dev, a, b, algo=N.ALGO_GEMV), want)
+    assert np.array_equal(_gemv_gemm(dev, a, b), want)  # (the planner's choice, whichever kernel that is)
+    rocm.sync()
+
+
+@pytest.mark.parametrize("m,n,k", [(4, 4096, 4096), (1, 8192, 2048), (6, 32768, 512)])
+def test_decode_product_kernel_epilogues_accumulate_and_pitch(dev, rocm, m, n, k):
+    a = synth.small_ints(m, (m, k), 3); b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+    bias = synth.small_ints(m + 2, (n,), 5, stream=2); old = synth.small_ints(m + 3, (m, n), 9, stream=3)
+    prod = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float64)
+    ldb = n + 12  # rows of W 48 bytes apart from a power of two
+    store = np.zeros((k, ldb), np.float32); store[:, :n] = b
+    dA, dB, dBias = dev.put(a), dev.put(store), dev.put(bias)
+    for epi, accumulate in [(N.EPI_NONE, False), (N.EPI_NONE, True), (N.EPI_BIAS, False), (N.EPI_BIAS, True), (N.EPI_BIAS_RELU, False),
+                            (N.EPI_BIAS_GELU, False)]:
+        z = prod + (bias if epi != N.EPI_NONE else 0.0)
+        if epi == N.EPI_BIAS_RELU: z = np.maximum(z, 0.0)
+        if epi == N.EPI_BIAS_GELU: z = 0.5 * z * (1.0 + np.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        want = z + (old if accumulate else 0.0)
+        dC = dev.put(old)
+        rocm.sgemm(m, n, k, dA, dB, dC, b_strides=(ldb, 1), bias=dBias if epi != N.EPI_NONE else None, epilogue=epi, accumulate=accumulate,
+                   algo=N.ALGO_GEMV)
+        got = rocm.to_host(dC, (m, n))
+        if epi == N.EPI_BIAS_GELU:
+            assert np.abs(got - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), (epi, accumulate)
+        else:
+            assert np.array_equal(got, want.astype(np.float32)), (epi, accumulate)
+    # an activation together with accumulate is not this kernel's: refused when forced, taken by another under the planner
+    dC = dev.put(old)
+    with pytest.raises(N.MniError):
+        rocm.sgemm(m, n, k, dA, dB, dC, b_strides=(ldb, 1), bias=dBias, epilogue=N.EPI_BIAS_RELU, accumulate=True, algo=N.ALGO_GEMV)
+    rocm.sgemm(m, n, k, dA, dB, dC, b_strides=(ldb, 1), bias=dBias, epilogue=N.EPI_BIAS_RELU, accumulate=True)
+    assert np.array_equal(rocm.to_host(dC, (m, n)), (np.maximum(prod + bias, 0.0) + old).astype(np.float32))
+
+
+def test_decode_product_kernel_normal_inputs_and_repeats(dev, rocm):
+    # within the tolerance of a float64 product and of the column kernel; the same bits launch after launch (the sums
+    # are formed in a fixed order whichever wavefront adds the slices up)
+    m, k, n = 4, 4096, 4096
+    a = synth.normal(31, (m, k), 0.02); b = synth.normal(32, (k, n), 0.02, stream=1)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    first = _gemv_gemm(dev, a, b, algo=N.ALGO_GEMV)
+    assert max_err(first, want) <= gemm_tol(k, a, b)
+    assert max_err(_gemv_gemm(dev, a, b, algo=N.ALGO_SKINNY), want) <= gemm_tol(k, a, b)
+    dA, dB = dev.put(a), dev.put(b)
+    dC = dev.empty(m * n, fill=-7.0)
+    for _ in range(50):
+        rocm.sgemm(m, n, k, dA, dB, dC, algo=N.ALGO_GEMV)
+    assert np.array_equal(rocm.to_host(dC, (m, n)), first)
+
+
+def test_decode_product_kernel_ineligible_is_an_error_only_when_forced(dev, rocm):
+    a = synth.small_ints(1, (4, 1024), 3); b = synth.small_ints(2, (1024, 768), 3, stream=1)  # 6 units: not a multiple of 8
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    with pytest.raises(N.MniError):
+        _gemv_gemm(dev, a, b, algo=N.ALGO_GEMV)
+    assert np.array_equal(_gemv_gemm(dev, a, b), want)
+    a9 = synth.small_ints(3, (9, 4096), 3); b9 = synth.small_ints(4, (4096, 4096), 3, stream=1)  # 9 rows
+    with pytest.raises(N.MniError):
+        _gemv_gemm(dev, a9, b9, algo=N.ALGO_GEMV)
+
+
 @pytest.mark.parametrize("m", [1, 3, 5, 7])
 def test_skinny_cols_decode_shape_normal_inputs(dev, m):
     # the kernels specialised for a row count: within tolerance of a float64 product and of the two-launch form,
