@@ -1702,6 +1702,38 @@ int mni_rocm_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
     if (cols > 0 && (!out || (rows > 0 && !a))) return set_error(MNI_ERR_INVALID, "colsum: null argument");
     return k_colsum(out, a, rows, cols);
 }
+int mni_rocm_unbroadcast(float *out, const float *g, const int64_t *g_shape, int g_ndim, const int64_t *to_shape, int to_ndim) {
+    MNI_API_GUARD;
+    MNI_TRY(ensure_init());
+    if (g_ndim < 0 || to_ndim < 0 || g_ndim > MNI_MAX_DIMS || to_ndim > g_ndim) return set_error(MNI_ERR_INVALID, "unbroadcast: bad ranks %d -> %d", g_ndim, to_ndim);
+    if ((g_ndim > 0 && !g_shape) || (to_ndim > 0 && !to_shape)) return set_error(MNI_ERR_INVALID, "unbroadcast: null shape");
+    int64_t gn = 1, on = 1;
+    for (int k = 0; k < g_ndim; ++k) { if (g_shape[k] < 0) return set_error(MNI_ERR_INVALID, "unbroadcast: negative extent"); gn *= g_shape[k]; }
+    for (int k = 0; k < to_ndim; ++k) { if (to_shape[k] < 0) return set_error(MNI_ERR_INVALID, "unbroadcast: negative extent"); on *= to_shape[k]; }
+    // right-aligned: every extent of `to` is the gradient's or 1 (src/native/src/utils.rs:3-20 run backwards)
+    const int off = g_ndim - to_ndim;
+    bool same = true;
+    for (int k = 0; k < g_ndim; ++k) {
+        const int64_t ext = k < off ? 1 : to_shape[k - off];
+        if (ext != g_shape[k] && ext != 1) return set_error(MNI_ERR_INVALID, "unbroadcast: shapes do not broadcast");
+        same = same && ext == g_shape[k];
+    }
+    if (on == 0) return MNI_OK;
+    if (!out || (gn > 0 && !g)) return set_error(MNI_ERR_INVALID, "unbroadcast: null argument");
+    if (gn == 0) return k_fill(out, 0.0f, on);
+    if (same) {
+        const int64_t shape1[1] = {on}, stride1[1] = {1};
+        return k_strided_copy(out, g, shape1, stride1, 1);
+    }
+    // Only leading dims summed away ([R.., C..] -> [C..] or [1.., C..]): the two-pass column sum.
+    int lead = 0;
+    while (lead < to_ndim && to_shape[lead] == 1) ++lead;
+    const int core = to_ndim - lead;
+    bool suffix = true;
+    for (int i = 0; suffix && i < core; ++i) suffix = g_shape[g_ndim - core + i] == to_shape[lead + i];
+    if (suffix) return k_colsum(out, g, gn / on, on);
+    return k_unbroadcast(out, g, g_shape, g_ndim, to_shape, to_ndim);
+}
 int mni_rocm_axpy(float *dst, const float *src, float alpha, int64_t n) {
     MNI_API_GUARD;
     if (n < 0) return set_error(MNI_ERR_INVALID, "axpy: negative length");

@@ -151,6 +151,9 @@ bool gemm_outer_eligible(const GemmLaunch &g) {
     if (g.ldc % 4 != 0 || (g.batch > 1 && g.c_bs % 4 != 0) || !ou_aligned16(g.C)) return false;
     // byte offsets inside one batch of A and of B are 32-bit in the kernel
     if (g.a_cs < 0 || g.b_rs < 0 || ((int64_t)g.K * g.a_cs + g.M) * 4 >= 0x7fffffffLL || ((int64_t)g.K * g.b_rs + g.N) * 4 >= 0x7fffffffLL) return false;
+    // the batch and the row blocks are grid dimensions y and z of the launch (65535 each; four row blocks per workgroup
+    // once the grid is large): a product beyond that is the tile kernel's, whose grid is one-dimensional
+    if (g.batch > 65535 || (g.M + OU_ROWS - 1) / OU_ROWS > 4LL * 65535) return false;
     return true;
 }
 

@@ -79,6 +79,7 @@ SIGNATURES = {
     "mni_rocm_strided_copy": (C.c_int, [C.c_void_p, C.c_void_p, _i64p, _i64p, C.c_int]),
     "mni_rocm_add_bias": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
     "mni_rocm_colsum": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
+    "mni_rocm_unbroadcast": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int, C.POINTER(C.c_int64), C.c_int]),
     "mni_rocm_axpy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_float, C.c_int64]),
     "mni_rocm_fill": (C.c_int, [C.c_void_p, C.c_float, C.c_int64]),
     "mni_zeros": (C.c_uint32, [_i64p, C.c_int]),
@@ -332,6 +333,11 @@ class Rocm:
 
     def colsum(self, out, a, rows, cols):
         self._check(self.lib.mni_rocm_colsum(out, a, rows, cols))
+
+    def unbroadcast(self, out, g, g_shape, to_shape):
+        gs = (C.c_int64 * max(len(g_shape), 1))(*g_shape)
+        ts = (C.c_int64 * max(len(to_shape), 1))(*to_shape)
+        self._check(self.lib.mni_rocm_unbroadcast(out, g, gs, len(g_shape), ts, len(to_shape)))
 
     def axpy(self, dst, src, alpha, n):
         self._check(self.lib.mni_rocm_axpy(dst, src, alpha, n))

@@ -257,6 +257,13 @@ int mni_rocm_add_bias(float *out, const float *a, const float *bias, int64_t row
 /* out[c] = sum_r a[r, c]          (bias gradient; replaces the host unbroadcast of
  * add_backward, src/native/src/ops/elementwise.rs:213-231) */
 int mni_rocm_colsum(float *out, const float *a, int64_t rows, int64_t cols);
+/* out (contiguous, `to_shape`) = g (contiguous, `g_shape`) summed over every dim that broadcasting `to_shape` up to
+ * `g_shape` had stretched: the missing leading dims and every dim where to_shape is 1 and g_shape is not, interior
+ * ones included ([2,3,M,K] -> [2,1,M,K]).  Each output is an f32 sum in the gradient's flat order.  Replaces
+ * utils::unbroadcast (src/native/src/utils.rs:39-66) as matmul_backward (src/native/src/ops/matmul.rs:206-218) and
+ * add_backward (src/native/src/ops/elementwise.rs:199-231) call it, which the reference's cuda arm runs on the host.
+ * Equal shapes copy; up to 8 dims; error if the shapes do not broadcast. */
+int mni_rocm_unbroadcast(float *out, const float *g, const int64_t *g_shape, int g_ndim, const int64_t *to_shape, int to_ndim);
 /* dst[i] += alpha * src[i]        (add_f32 in accumulate_grad / add_inplace,
  * src/native/src/tensor.rs:475-508) */
 int mni_rocm_axpy(float *dst, const float *src, float alpha, int64_t n);

@@ -8,7 +8,7 @@
 use crate::autograd::{BackwardOp, SavedContext, Tape, TapeEntry};
 use crate::rocm_ffi::*;
 use crate::tensor::{shape_size, TensorId, TensorStore};
-use crate::utils::{broadcast_shape, unbroadcast};
+use crate::utils::broadcast_shape;
 use smallvec::smallvec;
 
 pub fn add(a: TensorId, b: TensorId, store: &mut TensorStore, tape: &mut Tape) -> TensorId {
@@ -54,21 +54,19 @@ pub fn add_backward(grad: TensorId, saved: &SavedContext, store: &mut TensorStor
             if shape == grad_shape.as_slice() {
                 return store.clone_device(grad, shape);
             }
-            // leading dims broadcast (the bias case: [rows, C] -> [C]): a column sum on the device
-            let cols = shape_size(shape);
-            let suffix = grad_shape.len() >= shape.len() && grad_shape[grad_shape.len() - shape.len()..] == *shape;
-            if suffix {
-                let g = store.ensure_contiguous(grad);
-                let out = store.uninit(shape);
-                let rows = shape_size(&grad_shape) / cols;
-                check(unsafe { mni_rocm_colsum(store.dev_ptr_mut(out), store.dev_ptr(g), rows as i64, cols as i64) });
-                if g != grad {
-                    store.free(g);
-                }
-                return out;
+            // every broadcast dim summed on the device (the bias case [rows, C] -> [C] is the library's column sum;
+            // interior dims of extent 1 go through its general form): utils::unbroadcast (utils.rs:39-66)
+            let g = store.ensure_contiguous(grad);
+            let out = store.uninit(shape);
+            let from64: Vec<i64> = grad_shape.iter().map(|&d| d as i64).collect();
+            let to64: Vec<i64> = shape.iter().map(|&d| d as i64).collect();
+            check(unsafe {
+                mni_rocm_unbroadcast(store.dev_ptr_mut(out), store.dev_ptr(g), from64.as_ptr(), from64.len() as i32, to64.as_ptr(), to64.len() as i32)
+            });
+            if g != grad {
+                store.free(g);
             }
-            let host = store.to_host(grad);
-            store.from_vec(unbroadcast(&host, &grad_shape, shape), shape)
+            out
         };
         let ga = one(store, &a_shape);
         let gb = one(store, &b_shape);

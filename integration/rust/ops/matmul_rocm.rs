@@ -93,17 +93,24 @@ pub fn matmul_no_grad(a: TensorId, b: TensorId, store: &mut TensorStore) -> Tens
     forward(a, b, store)
 }
 
-/// Sum a gradient of shape `from` down to `to` (leading dims only: that is
-/// what a broadcast batch leaves): rows = what was broadcast, cols = the rest.
-fn unbroadcast_leading(store: &mut TensorStore, g: TensorId, to: &[usize]) -> TensorId {
+/// Sum a gradient down to the shape of the operand it belongs to: every dim that the batch broadcast had stretched,
+/// the missing leading ones and interior ones of extent 1 alike (`a[2,1,M,K] * b[2,3,K,N]` sums dim 1 of the
+/// `[2,3,M,K]` gradient).  `utils::unbroadcast` (utils.rs:39-66) on the device.
+pub(crate) fn unbroadcast_device(store: &mut TensorStore, g: TensorId, to: &[usize]) -> TensorId {
     let from = store.shape(g).to_vec();
     if from == to {
         return g;
     }
-    let cols = shape_size(to);
-    let rows = shape_size(&from) / cols;
+    let gc = store.ensure_contiguous(g);
     let out = store.uninit(to);
-    check(unsafe { mni_rocm_colsum(store.dev_ptr_mut(out), store.dev_ptr(g), rows as i64, cols as i64) });
+    let from64: Vec<i64> = from.iter().map(|&d| d as i64).collect();
+    let to64: Vec<i64> = to.iter().map(|&d| d as i64).collect();
+    check(unsafe {
+        mni_rocm_unbroadcast(store.dev_ptr_mut(out), store.dev_ptr(gc), from64.as_ptr(), from64.len() as i32, to64.as_ptr(), to64.len() as i32)
+    });
+    if gc != g {
+        store.free(gc);
+    }
     store.free(g);
     out
 }
@@ -135,9 +142,8 @@ pub fn matmul_backward(grad: TensorId, saved: &SavedContext, store: &mut TensorS
             store.free(t);
         }
         // a broadcast operand receives the sum over the batches it served
-        // (right-aligned shapes: the missing dims are the leading ones)
-        let ga = unbroadcast_leading(store, ga, &a_shape);
-        let gb = unbroadcast_leading(store, gb, &b_shape);
+        let ga = unbroadcast_device(store, ga, &a_shape);
+        let gb = unbroadcast_device(store, gb, &b_shape);
         vec![Some(ga), Some(gb)]
     } else {
         vec![None, None]

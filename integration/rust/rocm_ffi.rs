@@ -84,6 +84,7 @@ extern "C" {
     pub fn mni_rocm_strided_copy(dst: *mut f32, src: *const f32, shape: *const i64, src_strides: *const i64, ndim: c_int) -> c_int;
     pub fn mni_rocm_add_bias(out: *mut f32, a: *const f32, bias: *const f32, rows: i64, cols: i64) -> c_int;
     pub fn mni_rocm_colsum(out: *mut f32, a: *const f32, rows: i64, cols: i64) -> c_int;
+    pub fn mni_rocm_unbroadcast(out: *mut f32, g: *const f32, g_shape: *const i64, g_ndim: c_int, to_shape: *const i64, to_ndim: c_int) -> c_int;
     pub fn mni_rocm_axpy(dst: *mut f32, src: *const f32, alpha: f32, n: i64) -> c_int;
     pub fn mni_rocm_fill(dst: *mut f32, value: f32, n: i64) -> c_int;
 }

@@ -1019,6 +1019,23 @@ def test_outer_product_kernel_integer_exact(dev, rocm, nin, nout, rows, batch):
     assert np.array_equal(got[:, :, :nout], want1) and np.all(got[:, :, nout:] == -7.0)
 
 
+def test_more_batches_than_a_grid_dimension_holds_go_to_the_tile_kernel(dev, rocm):
+    # 70000 x (32 x 64 x 32) with A given as its transpose: what the outer-product kernel would take but for its batch in
+    # grid dimension z (65535); the planner must fall through to the tile kernel instead of failing, and a forced
+    # outer-product launch must say why it cannot
+    batch, m, n, k = 70000, 32, 64, 32
+    x = synth.small_ints(1, (1, k, m), 3); dy = synth.small_ints(2, (1, k, n), 3, stream=1)
+    want = (x[0].astype(np.int64).T @ dy[0].astype(np.int64)).astype(np.float32)
+    dX, dY = dev.put(x), dev.put(dy)
+    dC = dev.empty(batch * m * n, fill=-7.0)
+    rocm.sgemm(m, n, k, dX, dY, dC, batch=batch, a_strides=(1, m), a_batch=(0, 1), b_batch=(0, 1))
+    got = rocm.to_host(dC, (batch, m, n))
+    assert np.array_equal(got[0], want) and np.array_equal(got[65535], want) and np.array_equal(got[-1], want)
+    assert np.all(got == want[None])
+    with pytest.raises(N.MniError):
+        rocm.sgemm(m, n, k, dX, dY, dC, batch=batch, a_strides=(1, m), a_batch=(0, 1), b_batch=(0, 1), algo=N.ALGO_OUTER)
+
+
 def test_outer_product_kernel_is_the_plan_for_a_small_batch_weight_gradient_and_refuses_other_layouts(dev, rocm):
     rows, nin, nout = 16, 2048, 4096
     x = synth.normal(1, (rows, nin)); dy = synth.normal(2, (rows, nout), stream=1)
@@ -1407,3 +1424,61 @@ def test_mfma_yardstick_runs_and_shows_what_a_register_move_costs(rocm):
     assert moved < pure                  # vector-ALU instructions take their issue time from the MFMAs
     with pytest.raises(N.MniError, match="bad arguments"):
         rocm.mfma_yardstick(3)
+
+
+# ---- the kernel-level ABI driven the way the Rust `rocm` arm of matmul_backward drives it ----------------------------
+def _rust_arm_matmul_backward(dev, a, b, g):
+    """dA, dB of C = A B for an upstream gradient g, through mni_rocm_sgemm_pair and mni_rocm_unbroadcast exactly as
+    integration/rust/ops/matmul_rocm.rs issues them: the two products with the transposed operand as a stride swap
+    and the batch rule `b % count`, then each gradient summed down to its operand's shape."""
+    r = dev.r
+    m, k = a.shape[-2:]
+    n = b.shape[-1]
+    out_batch = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+    batch = int(np.prod(out_batch, dtype=np.int64))
+    a_count, b_count = int(np.prod(a.shape[:-2], dtype=np.int64)), int(np.prod(b.shape[:-2], dtype=np.int64))
+    dA, dB, dG = dev.put(a), dev.put(b), dev.put(g)
+    ga_full, gb_full = dev.empty(batch * m * k), dev.empty(batch * k * n)
+    first = r.gemm_desc(m, k, n, dG, dB, ga_full, batch=batch, a_strides=(n, 1), a_batch=(m * n, batch),
+                        b_strides=(1, n), b_batch=(k * n, b_count))          # dA = dC * B^T
+    second = r.gemm_desc(k, n, m, dA, dG, gb_full, batch=batch, a_strides=(1, k), a_batch=(m * k, a_count),
+                         b_strides=(n, 1), b_batch=(m * n, batch))           # dB = A^T * dC
+    r.sgemm_pair(first, second)
+    ga, gb = dev.empty(a.size), dev.empty(b.size)
+    r.unbroadcast(ga, ga_full, list(out_batch) + [m, k], list(a.shape))
+    r.unbroadcast(gb, gb_full, list(out_batch) + [k, n], list(b.shape))
+    return r.to_host(ga, a.shape), r.to_host(gb, b.shape)
+
+
+@pytest.mark.parametrize("a_shape,b_shape", [((2, 1, 5, 7), (2, 3, 7, 4)), ((1, 6, 9), (4, 9, 5)), ((3, 8, 6), (6, 10)),
+                                             ((2, 3, 4, 6), (1, 3, 6, 5)), ((4, 1, 1, 3, 8), (4, 2, 5, 8, 2))])
+def test_rust_arm_call_sequence_gradients_vs_oracle(dev, orc, a_shape, b_shape):
+    # an interior batch dim of extent 1 (a[2,1,M,K] against b[2,3,K,N]) is summed along that dim, not along the
+    # leading one; the oracle's matmul_backward (ops/matmul.rs:199-222 with utils.rs:39-66) is the reference
+    a = synth.small_ints(1, a_shape, 3); b = synth.small_ints(2, b_shape, 3, stream=1)
+    out_batch = np.broadcast_shapes(a_shape[:-2], b_shape[:-2])
+    # (an operand with fewer batches is read at batch % count, the reference's rule (ops/matmul.rs:55-56), by the
+    # oracle and by the kernel alike; test_oracle_matmul pins the rule itself)
+    g = synth.small_ints(3, tuple(out_batch) + (a_shape[-2], b_shape[-1]), 2, stream=2)
+    A = orc.Tensor.fromFloat32(a, list(a_shape)).setRequiresGrad(True)
+    B = orc.Tensor.fromFloat32(b, list(b_shape)).setRequiresGrad(True)
+    A.matmul(B).mul(orc.Tensor.fromFloat32(g, list(g.shape))).sum().backward()
+    want_a, want_b = A.grad.numpy(), B.grad.numpy()
+    ga, gb = _rust_arm_matmul_backward(dev, a, b, g)
+    assert np.array_equal(ga, want_a) and np.array_equal(gb, want_b)
+
+
+def test_kernel_level_unbroadcast_patterns_and_errors(dev, rocm):
+    g = synth.small_ints(4, (2, 3, 4, 5), 4)
+    dG = dev.put(g)
+    for to, axes in (([2, 1, 4, 5], (1,)), ([3, 1, 5], (0, 2)), ([5], (0, 1, 2)), ([1], (0, 1, 2, 3)), ([2, 3, 4, 5], ()), ([1, 1, 4, 1], (0, 1, 3)),
+                     ([4, 5], (0, 1))):
+        out = dev.empty(int(np.prod(to)))
+        rocm.unbroadcast(out, dG, list(g.shape), to)
+        want = g.astype(np.int64).sum(axis=axes, keepdims=True).reshape(to).astype(np.float32) if axes else g
+        assert np.array_equal(rocm.to_host(out, tuple(to)), want), to
+    out = dev.empty(40)
+    with pytest.raises(N.MniError):
+        rocm.unbroadcast(out, dG, list(g.shape), [2, 4, 5])      # 2 does not broadcast against 3
+    with pytest.raises(N.MniError):
+        rocm.unbroadcast(out, dG, [4, 5], [2, 4, 5])             # more dims than the gradient has

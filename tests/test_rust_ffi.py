@@ -88,6 +88,16 @@ def test_the_calls_the_arms_make_are_all_declared():
     assert used and used <= set(rust_functions()), sorted(used - set(rust_functions()))
 
 
+def test_broadcast_gradients_are_reduced_by_the_general_device_sum():
+    # matmul_backward and add_backward sum a gradient over every broadcast dim, interior ones of extent 1 included
+    # (utils.rs:39-66): the arms hand both shapes to mni_rocm_unbroadcast and never guess a (rows, cols) column sum
+    for rel in ("ops/matmul_rocm.rs", "ops/elementwise_rocm.rs"):
+        text = open(os.path.join(ROOT, "integration", "rust", rel)).read()
+        back = text[text.index("_backward("):]
+        assert "mni_rocm_unbroadcast(" in text and "mni_rocm_colsum(" not in back, rel
+        assert "to_host(" not in back, rel  # (no host round trip for a broadcast gradient)
+
+
 def test_structs_have_the_headers_fields_in_order():
     for c_name, r_name in (("mni_operand", "MniOperand"), ("mni_gemm_desc", "MniGemmDesc")):
         c_fields, r_fields = header_struct(c_name), rust_struct(r_name)
