@@ -71,7 +71,24 @@ def build(force=False, verbose=True):
     if verbose:
         print("built %s (%d translation units recompiled)" % (LIB, len(jobs)))
     build_node_addon(force or bool(jobs), verbose)
+    build_step_bench(force or bool(jobs), verbose)
     return LIB
+
+
+STEP_BENCH = os.path.join(HERE, "lib", "mlp_step_bench")
+
+
+def build_step_bench(force=False, verbose=True):
+    """The README training step driven through the engine-level C ABI from plain C (csrc/mlp_step_bench.c): what a
+    step costs without a language binding in the loop.  bench.py runs it beside its own (ctypes) figure."""
+    src = os.path.join(CSRC, "mlp_step_bench.c")
+    inc = os.path.normpath(os.path.join(CSRC, "..", "..", "include"))
+    if force or _stale(STEP_BENCH, [src, LIB, os.path.join(inc, "mni_rocm.h")]):
+        _run(["gcc", "-O2", "-std=c11", "-D_POSIX_C_SOURCE=199309L", "-Wall", "-I" + inc, src, "-o", STEP_BENCH, "-L" + os.path.dirname(LIB), "-lmni_rocm",
+              "-Wl,-rpath,$ORIGIN"])
+        if verbose:
+            print("built %s" % STEP_BENCH)
+    return STEP_BENCH
 
 
 NODE_ADDON = os.path.join(HERE, "lib", "mni_rocm.node")

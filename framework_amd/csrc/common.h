@@ -201,7 +201,10 @@ int check_launch(const char *what);  // hipGetLastError after a kernel launch
 // gemm.hip
 int sgemm(const mni_gemm_desc &d);
 // Two independent products, in one launch where the paired tile kernel takes them (gemm.hip).
-int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1);
+// `colsum` (may be null): column sums the caller needs as well (a Linear's bias gradient); computed in the same launch
+// when the pair goes out as one launch of the tiny-product kernel and the matrix is small, and colsum->done says so.
+struct PairColsum;
+int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1, PairColsum *colsum = nullptr);
 
 // elementwise.hip: internal launchers (device pointers, element strides)
 struct StridedDesc {
@@ -323,5 +326,8 @@ int k_sumsq_multi(const MultiTensor &t, double *part);
 // other and adds them up, in the order of k_sumsq_multi + k_sumsq_finish (same value); out[0] = the sum.
 constexpr int SUMSQ_SOLO_BLOCKS = 16;
 int k_sumsq_solo(const MultiTensor &t, double *out, unsigned long long *result_word, unsigned tag);
+// The same launch then clips the gradients in place (norm > max_norm > 0) and applies AdamW to every tensor of the table.
+int k_clip_and_step_solo(const MultiTensor &t, double *out, unsigned long long *result_word, unsigned tag, float max_norm, float lr, float b1,
+                         float b2, float eps, float wd, float bc1, float bc2);
 
 }  // namespace mni

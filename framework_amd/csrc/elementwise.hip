@@ -1612,8 +1612,15 @@ __global__ void multi_tensor_kernel(const MultiTensor t, double *__restrict__ pa
         if (threadIdx.x == 0) part[blockIdx.x] = sq;
     }
 }
+// STEP: the same workgroup then clips (gradients scaled in place when their norm exceeds max_norm > 0, as
+// clip_and_step does before its update, src/native/src/ops/optimizer.rs:224-245) and applies the AdamW update to
+// every tensor of the table: a model of a few thousand parameters takes its whole optimiser step in one launch.
+struct SoloStep {
+    float max_norm, lr, b1, b2, eps, wd, bc1, bc2;
+};
+template <bool STEP>
 __global__ __launch_bounds__(TPB) void sumsq_solo_kernel(const MultiTensor t, double *__restrict__ out, unsigned long long *result_word,
-                                                         unsigned tag) {
+                                                         unsigned tag, const SoloStep a) {
     // The host waits for this kernel, so the chunks are not taken one after the other by the whole workgroup (a
     // round trip to memory each) but four at a time, one per wavefront.  A wavefront plays the four wavefronts of
     // chunk_sumsq in turn -- lane l of "wavefront" w adds up elements lo + 64 w + l, + 256, ... -- so every sum
@@ -1646,6 +1653,28 @@ __global__ __launch_bounds__(TPB) void sumsq_solo_kernel(const MultiTensor t, do
         out[0] = total;
         if (result_word) post_result_word(result_word, tag, __float_as_uint((float)total));
     }
+    if (!STEP) return;
+    const float norm = sqrtf((float)total);  // (every thread holds the total)
+    const bool clip = a.max_norm > 0.0f && norm > a.max_norm;
+    const float scale = clip ? a.max_norm / norm : 1.0f;
+    for (int ti = 0; ti < t.count; ++ti) {
+        float *__restrict__ p = t.p[ti], *__restrict__ m = t.m[ti], *__restrict__ v = t.v[ti];
+        float *g = const_cast<float *>(t.g[ti]);
+        const int64_t n = t.n[ti];
+        for (int64_t i = threadIdx.x; i < n; i += TPB) {
+            float gv = g[i];
+            if (clip) { gv *= scale; g[i] = gv; }
+            float pv = p[i];
+            if (a.wd > 0.0f) pv *= 1.0f - a.lr * a.wd;
+            const float mv = a.b1 * m[i] + (1.0f - a.b1) * gv;
+            const float vv = a.b2 * v[i] + (1.0f - a.b2) * gv * gv;
+            m[i] = mv;
+            v[i] = vv;
+            const float m_hat = mv / a.bc1;
+            const float v_hat = vv / a.bc2;
+            p[i] = pv - a.lr * m_hat / (sqrtf(v_hat) + a.eps);
+        }
+    }
 }
 int multi_tensor_blocks(int64_t n) { return (int)((n + MULTI_CHUNK - 1) / MULTI_CHUNK); }
 static int multi_check(const MultiTensor &t) {
@@ -1669,8 +1698,17 @@ int k_sumsq_solo(const MultiTensor &t, double *out, unsigned long long *result_w
     MNI_TRY(ensure_init());
     MNI_TRY(multi_check(t));
     if (t.block_start[t.count] > SUMSQ_SOLO_BLOCKS) return set_error(MNI_ERR_INVALID, "sumsq_solo: more than %d chunks", SUMSQ_SOLO_BLOCKS);
-    MNI_KERNEL_LAUNCH(sumsq_solo_kernel, dim3(1), dim3(TPB), 0, ctx().stream, t, out, result_word, tag);
+    MNI_KERNEL_LAUNCH(sumsq_solo_kernel<false>, dim3(1), dim3(TPB), 0, ctx().stream, t, out, result_word, tag, SoloStep{});
     return check_launch("sumsq_solo");
+}
+int k_clip_and_step_solo(const MultiTensor &t, double *out, unsigned long long *result_word, unsigned tag, float max_norm, float lr, float b1,
+                         float b2, float eps, float wd, float bc1, float bc2) {
+    MNI_TRY(ensure_init());
+    MNI_TRY(multi_check(t));
+    if (t.block_start[t.count] > SUMSQ_SOLO_BLOCKS) return set_error(MNI_ERR_INVALID, "clip_and_step_solo: more than %d chunks", SUMSQ_SOLO_BLOCKS);
+    MNI_KERNEL_LAUNCH(sumsq_solo_kernel<true>, dim3(1), dim3(TPB), 0, ctx().stream, t, out, result_word, tag,
+                       SoloStep{max_norm, lr, b1, b2, eps, wd, bc1, bc2});
+    return check_launch("clip_and_step_solo");
 }
 int k_sumsq_multi(const MultiTensor &t, double *part) {
     MNI_TRY(ensure_init());

@@ -18,6 +18,7 @@
 #include <vector>
 
 #include "common.h"
+#include "gemm_internal.h"
 #include <functional>
 
 namespace mni {
@@ -450,7 +451,8 @@ struct ThroughGelu {
     float *z;
     float *colsum_part;
 };
-static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out, const ThroughGelu *through_gelu = nullptr) {
+// bias_sums (fused Linear only, may be null): column sums of the upstream gradient wanted along with the two products.
+static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out, const ThroughGelu *through_gelu = nullptr, PairColsum *bias_sums = nullptr) {
     const uint32_t a = e.inputs[0], b = e.inputs[1];
     Tensor *A = get(a), *B = get(b), *G = get(grad);
     if (!A || !B || !G) return MNI_ERR_FREED;
@@ -492,7 +494,7 @@ static int matmul_backward(uint32_t grad, const Entry &e, int64_t *out, const Th
         }
     }
     if (!folded && !prepare_matmul(a, true, grad, false, nullptr, MNI_EPI_NONE, nullptr, nullptr, &pb)) return MNI_ERR_INVALID;
-    MNI_TRY(sgemm_pair(pa.d, pb.d));
+    MNI_TRY(sgemm_pair(pa.d, pb.d, bias_sums));
 
     {
         const uint32_t full = insert_contig(std::move(pa.out), pa.out_shape);
@@ -1398,7 +1400,19 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
             }
         }
     }
-    int rc = matmul_backward(g, mm, out, tg.z ? &tg : nullptr);
+    // The bias gradient (column sums of g over its rows) rides in the launch of the two products when they are small
+    // enough to go out as one launch of the tiny-product kernel: a training step of a few thousand parameters is the
+    // sum of its launches.
+    PairColsum sums = {nullptr, nullptr, 0, 0, false};
+    BufP db_early;
+    if (db_id < 0) {
+        Tensor *G = get(g), *Bv = get(e.inputs[2]);
+        if (G && Bv && is_contiguous(*G) && !G->shape.empty() && G->shape.back() == Bv->size && Bv->size > 0 && G->size / Bv->size <= 256) {
+            db_early = new_buf((size_t)Bv->size);
+            if (db_early) sums = PairColsum{G->buf->p, db_early->p, G->size / Bv->size, Bv->size, false};
+        }
+    }
+    int rc = matmul_backward(g, mm, out, tg.z ? &tg : nullptr, sums.out ? &sums : nullptr);
     if (rc == MNI_OK && tg.z) {
         // bias gradient of the producing layer: the strips added up, in strip order
         Tensor *PB = get(en.bw_tape->entries[(size_t)(*en.bw_out2entry)[producer_out]].inputs[2]);
@@ -1417,7 +1431,7 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
             if (!Bv) rc = MNI_ERR_FREED;
             else {
                 const Shape bshape = Bv->shape;
-                const uint32_t gb = unbroadcast_tensor(g, bshape);
+                const uint32_t gb = sums.done ? insert_contig(std::move(db_early), bshape) : unbroadcast_tensor(g, bshape);
                 if (gb == MNI_BAD_ID) rc = MNI_ERR_INVALID;
                 else out[2] = gb;
             }
@@ -2023,6 +2037,76 @@ static int adamw_step(const uint32_t *ids, size_t n, float lr, float b1, float b
     return flush();
 }
 
+// A model of a few thousand parameters: gradient norm, clipping and the AdamW update of clip_and_step
+// (ops/optimizer.rs:224-245) as one launch of one workgroup.  *handled = false when the parameter list is not of that
+// kind (nothing has been launched then).  Same sums and the same update arithmetic as the separate launches.
+static int clip_and_step_solo(const uint32_t *ids, size_t n, float lr, float b1, float b2, float eps, float wd, uint32_t step, float max_norm,
+                              float *norm_out, bool *handled) {
+    *handled = false;
+    if (n == 0 || n > (size_t)MULTI_MAX) return MNI_OK;
+    MultiTensor t;
+    memset(&t, 0, sizeof t);
+    int blocks = 0;
+    int64_t total = 0;
+    for (size_t p = 0; p < n; ++p) {
+        Tensor *T = get(ids[p]);
+        if (!T) return MNI_ERR_FREED;
+        if (T->grad < 0) continue;
+        Tensor *G = get((uint32_t)T->grad);
+        if (!G) return MNI_ERR_FREED;
+        if (T->size <= 0 || G->size != T->size || !is_contiguous(*G) || !G->buf || (int64_t)G->buf->n != G->size) return MNI_OK;
+        for (int i = 0; i < t.count; ++i)
+            if (t.p[i] == T->buf->p) return MNI_OK;  // (the same parameter twice must see its first update)
+        total += T->size;
+        blocks += multi_tensor_blocks(T->size);
+        if (total > 8192 || blocks > SUMSQ_SOLO_BLOCKS) return MNI_OK;
+        ++t.count;
+    }
+    if (t.count == 0) return MNI_OK;
+    // second pass: buffers made private and moments created (launches of their own only on the first step)
+    t.count = 0;
+    blocks = 0;
+    for (size_t p = 0; p < n; ++p) {
+        Tensor *T = get(ids[p]);
+        if (T->grad < 0) continue;
+        Tensor *G = get((uint32_t)T->grad);
+        if (!T->adam_m) {
+            T->adam_m = new_buf((size_t)T->size);
+            T->adam_v = new_buf((size_t)T->size);
+            if (!T->adam_m || !T->adam_v) return MNI_ERR_NOMEM;
+            MNI_TRY(k_fill(T->adam_m->p, 0.f, T->size));
+            MNI_TRY(k_fill(T->adam_v->p, 0.f, T->size));
+        }
+        MNI_TRY(make_unique(*T));
+        if (max_norm > 0.0f) MNI_TRY(make_unique(*G));  // (clipping scales the gradient in place)
+        const int i = t.count++;
+        t.block_start[i] = blocks;
+        t.p[i] = T->buf->p; t.m[i] = T->adam_m->p; t.v[i] = T->adam_v->p; t.g[i] = G->buf->p; t.n[i] = T->size;
+        blocks += multi_tensor_blocks(T->size);
+    }
+    t.block_start[t.count] = blocks;
+    void *acc = nullptr;
+    MNI_TRY(dev_alloc(&acc, sizeof(double)));
+    std::shared_ptr<void> guard(acc, [](void *q) { dev_free(q); });
+    const unsigned tag = next_result_tag();
+    const float bc1 = 1.0f - powi_f32(b1, (int)step), bc2 = 1.0f - powi_f32(b2, (int)step);
+    MNI_TRY(k_clip_and_step_solo(t, (double *)acc, ctx().result_dev, tag, max_norm, lr, b1, b2, eps, wd, bc1, bc2));
+    *handled = true;
+    unsigned bits = 0;
+    bool delivered = false;
+    MNI_TRY(wait_result_word(tag, &bits, &delivered));
+    float sq;
+    if (delivered) {
+        memcpy(&sq, &bits, sizeof sq);
+    } else {
+        double sq64 = 0.0;
+        MNI_TRY(mni_rocm_d2h(&sq64, acc, sizeof(double)));
+        sq = (float)sq64;
+    }
+    *norm_out = sqrtf(sq);
+    return MNI_OK;
+}
+
 static int scale_grads(const uint32_t *ids, size_t n, float scale) {
     for (size_t p = 0; p < n; ++p) {
         Tensor *T = get(ids[p]);
@@ -2283,6 +2367,13 @@ double mni_clip_and_step(const uint32_t *ids, size_t n, double lr, double beta1,
     MNI_API_GUARD;
     float norm = 0.f;
     const float mg = (float)max_grad_norm;
+    {
+        bool handled = false;
+        if (clip_and_step_solo(ids, n, (float)lr, (float)beta1, (float)beta2, (float)eps, (float)weight_decay, (uint32_t)step, mg > 0.0f ? mg : 0.0f,
+                               &norm, &handled) != MNI_OK)
+            return -1.0;
+        if (handled) return (double)norm;
+    }
     auto update = [&] { return adamw_step(ids, n, (float)lr, (float)beta1, (float)beta2, (float)eps, (float)weight_decay, (uint32_t)step); };
     if (!(mg > 0.0f)) {
         // no clipping asked for: the update does not depend on the norm and is issued before the host waits for it

@@ -813,7 +813,8 @@ int sgemm(const mni_gemm_desc &d) {
 // and its transposed twin: 13.4 + 13.6 us one after the other, 20.9 us together (64 batches of the first in one
 // launch take the same 20.8).  Otherwise one after the other.  Same kernel body and same order of every sum either
 // way, so the results are those of the separate calls bit for bit.
-int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1) {
+int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1, PairColsum *colsum) {
+    if (colsum) colsum->done = false;
     MNI_TRY(ensure_init());
     MNI_TRY(validate(d0));
     MNI_TRY(validate(d1));
@@ -832,7 +833,14 @@ int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1) {
                 tiny = gemm_tiny_eligible(t[i]);
             }
         }
-        if (tiny) return launch_gemm_tiny_pair(t[0], t[1]);
+        if (tiny) {
+            // (a thread per column walks the rows alone: only for a matrix a launch's worth of threads reads in a moment)
+            const bool with_sums = colsum && colsum->src && colsum->out && colsum->rows > 0 && colsum->rows <= 256 && colsum->cols > 0 &&
+                                   colsum->cols <= 4096 && colsum->rows * colsum->cols <= (1 << 16);
+            MNI_TRY(launch_gemm_tiny_pair(t[0], t[1], with_sums ? colsum : nullptr));
+            if (with_sums) colsum->done = true;
+            return MNI_OK;
+        }
     }
     PlanProbe plan[2];
     int64_t tiles = 0;

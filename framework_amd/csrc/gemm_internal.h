@@ -61,7 +61,15 @@ int launch_gemm_direct(const GemmLaunch &g, int amode, int bmode, int ksplit);
 // One thread per output, sequential K (gemm_tiny.hip): a few thousand outputs of a short K, any strides.
 bool gemm_tiny_eligible(const GemmLaunch &g);
 int launch_gemm_tiny(const GemmLaunch &g);
-int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1);  // two eligible, independent products in one launch
+// Column sums of a contiguous [rows, cols] matrix (rows added in order) that a paired launch of two tiny products
+// computes along with them; `done` says whether it did.
+struct PairColsum {
+    const float *src;
+    float *out;
+    int64_t rows, cols;
+    bool done;
+};
+int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1, const PairColsum *colsum = nullptr);  // two eligible, independent products in one launch
 // 9 to 32 rows of a K-contiguous A against a wide N-contiguous B, both straight into MFMA registers (gemm_fewrows.hip):
 // g.tiles_n counts column groups of 128, g.split_k K slices of g.k_per_slice (a multiple of 32).  With split_k > 1:
 // partials [slice][batch][M][N] in g.ws and one counter per (batch, column group) in g.sk_flags, zero between launches

@@ -81,12 +81,26 @@ __global__ __launch_bounds__(TINY_THREADS) void gemm_tiny_kernel(const GemmLaunc
 }
 // Two independent products in one launch: workgroups [0, blocks0) compute the first, the rest the second.
 // form: bit 0 = A4, bit 1 = W4 of each product.
+// A third job rides along when asked for: the column sums of a contiguous [rows, cols] matrix, one thread per column,
+// rows added in order -- the bias gradient of a Linear, utils::unbroadcast's own sum (src/native/src/utils.rs:55-64).
 struct TinyPairLaunch {
     GemmLaunch g[2];
-    unsigned blocks0;
+    unsigned blocks0, blocks01;  // workgroups of the first product; of both products
     int form[2];
+    const float *cs_src;
+    float *cs_out;
+    int cs_rows, cs_cols;
 };
 __global__ __launch_bounds__(TINY_THREADS) void gemm_tiny_pair_kernel(const TinyPairLaunch p) {
+    if (blockIdx.x >= p.blocks01) {
+        const int col = (int)(blockIdx.x - p.blocks01) * TINY_THREADS + threadIdx.x;
+        if (col >= p.cs_cols) return;
+        const float *__restrict__ src = p.cs_src + col;
+        float s = 0.0f;
+        for (int r = 0; r < p.cs_rows; ++r) s += src[(int64_t)r * p.cs_cols];
+        p.cs_out[col] = s;
+        return;
+    }
     const bool second = blockIdx.x >= p.blocks0;
     const GemmLaunch &g = second ? p.g[1] : p.g[0];
     const int64_t idx = (int64_t)(blockIdx.x - (second ? p.blocks0 : 0u)) * TINY_THREADS + threadIdx.x;
@@ -154,16 +168,23 @@ int launch_gemm_tiny(const GemmLaunch &g) {
 }
 
 // Both products must pass gemm_tiny_eligible; neither may read what the other writes.
-int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1) {
+int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1, const PairColsum *colsum) {
     if (!gemm_tiny_eligible(g0) || !gemm_tiny_eligible(g1))
         return set_error(MNI_ERR_INVALID, "sgemm_pair: the tiny-product pair takes two products that each fit the tiny-product kernel");
     TinyPairLaunch p;
     p.g[0] = g0;
     p.g[1] = g1;
     p.blocks0 = (unsigned)tiny_blocks(g0);
+    p.blocks01 = p.blocks0 + (unsigned)tiny_blocks(g1);
     p.form[0] = tiny_form(g0);
     p.form[1] = tiny_form(g1);
-    const dim3 grid(p.blocks0 + (unsigned)tiny_blocks(g1)), block(TINY_THREADS);
+    p.cs_src = nullptr; p.cs_out = nullptr; p.cs_rows = 0; p.cs_cols = 0;
+    unsigned extra = 0;
+    if (colsum && colsum->rows > 0 && colsum->cols > 0) {
+        p.cs_src = colsum->src; p.cs_out = colsum->out; p.cs_rows = (int)colsum->rows; p.cs_cols = (int)colsum->cols;
+        extra = (unsigned)((colsum->cols + TINY_THREADS - 1) / TINY_THREADS);
+    }
+    const dim3 grid(p.blocks01 + extra), block(TINY_THREADS);
     MNI_KERNEL_LAUNCH(gemm_tiny_pair_kernel, grid, block, 0, ctx().stream, p);
     return check_launch("gemm_tiny_pair_kernel");
 }
