@@ -2,6 +2,7 @@
 """Benchmark of the fp32 matmul hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+    python bench.py --planner-check        (MNI_ALGO_AUTO against the recorded best forced plan per shape)
 
 A step is one pass of the hot path over one batch of synthetic input: the
 single fp32 product A[4096,4096] x B[4096,4096] (A, B ~ N(0,1), seed 1,
@@ -17,14 +18,19 @@ One JSON line is printed:
 * cpu_baseline  the CPU oracle (a C restatement of the reference's
               single-threaded CPU backend) timed on this host on a bounded
               sample of the same product (the first 2048 rows of A);
-* extra       the other configurations of the path, each with its own
-              `roofline` (algorithmic flops / bytes against the roof that
-              bounds it) and `cpu_baseline` (the oracle on a bounded sample):
-              the decode-shaped GEMV against HBM bandwidth (cold first), the
-              tall-K weight gradient, the three attention-shaped batched
-              products, the README-MLP step (launches per step) and the FFN
-              training step; plus what this device gives a kernel that only
-              streams (read / write / copy yardsticks, an empty launch).
+* other       rows that are not among the configurations the metric is quoted
+              on (what the device gives a kernel that only streams or only
+              multiplies, batched decoding, small-batch weight gradients,
+              attention, the KV cache) -- printed first;
+* extra       the other four configurations, printed LAST and kept short so
+              that they survive in a record that keeps the end of the line:
+              config1 (README MLP step: ms through a plain-C loop over the
+              engine ABI, the ctypes figure beside it, launches per step),
+              config3 (the three attention-shaped batched products), config4
+              (FFN training step), config5a (decode GEMV against HBM
+              bandwidth, weights cold) and config5b (tall-K weight gradient),
+              each with `frac` against the roof that bounds it, `traffic`
+              from the committed counter summaries, and a `cpu_baseline`.
 
 Only one GPU is used; --gpus above 1 is refused.
 """
@@ -122,6 +128,52 @@ def roofline(bound, kernel, seconds, flops, nbytes, traffic=None):
     return out
 
 
+def sig(x, digits=4):
+    """x rounded to a few significant digits (the record keeps the end of the line: every byte counts)."""
+    if isinstance(x, float):
+        return float("%.*g" % (digits, x))
+    if isinstance(x, dict):
+        return {k: sig(v, digits) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [sig(v, digits) for v in x]
+    return x
+
+
+def brief(roof, **more):
+    """The fields of a roofline object that a reader of the record needs."""
+    out = {k: roof[k] for k in ("us", "frac", "bound", "kernel", "achieved", "peak", "unit", "traffic") if k in roof}
+    out.update(more)
+    return sig(out)
+
+
+def brief_cpu(cpu):
+    return sig({k: cpu[k] for k in ("value", "unit", "cores", "kind", "sample") if k in cpu})
+
+
+def profile_value(name, label):
+    """A figure from a committed profile summary: the number on the line `<label> = <x>`."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+    except OSError:
+        return None
+    m = re.search(re.escape(label) + r" = ([0-9.]+)", text)
+    return float(m.group(1)) if m else None
+
+
+def c_loop_step(fused):
+    """The README step driven from plain C over the engine ABI (framework_amd/lib/mlp_step_bench, built with the library):
+    its JSON line, or None when the program is not there."""
+    import subprocess
+    exe = os.path.join(ROOT, "framework_amd", "lib", "mlp_step_bench")
+    if not os.path.exists(exe):
+        return None
+    p = subprocess.run([exe, "1" if fused else "0", "1000", "100"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
+    if p.returncode != 0:
+        return {"error": (p.stderr or p.stdout).strip()[-200:]}
+    return json.loads(p.stdout.strip().splitlines()[-1])
+
+
 def oracle_api():
     from framework_amd.api import bind
     from oracle.native import OracleNative
@@ -184,7 +236,7 @@ def bench_extras(r, with_cpu):
     dx, dw, dy = r.to_device(x), r.to_device(w), r.malloc(4 * 4096 * 4)
     by = 4.0 * (4096 * 4096 + 2 * 4 * 4096)
     fl = 2.0 * 4 * 4096 * 4096
-    kern = "skinny_cols_kernel<4, true, true, false, true, true>"
+    kern = "gemv_units_kernel<4, false, true>"
     # launches of a few microseconds are issued from C (mni_rocm_sgemm_timed) so that the host stays ahead
     ms_warm = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 10, 200)
     ms_sus = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, dw, dy)], 3000, 1000)
@@ -192,7 +244,7 @@ def bench_extras(r, with_cpu):
     ms_cold = r.sgemm_timed([r.gemm_desc(4, 4096, 4096, dx, p, dy) for p in ws], 16, 200)
     r.sgemm(4, 4096, 4096, dx, dw, dy)
     got = r.to_host(dy, (4, 4096))
-    c5a = {"roofline": dict(roofline("hbm", kern, ms_cold * 1e-3, fl, by, traffic=profile_traffic("skinny_gemv_4x4096x4096.txt")),
+    c5a = {"roofline": dict(roofline("hbm", kern, ms_cold * 1e-3, fl, by, traffic=profile_traffic("gemv_units_4x4096x4096.txt")),
                             note="cold: eight different W in rotation (512 MiB working set), every byte comes from HBM"),
            "warm": dict(roofline("hbm", kern, ms_warm * 1e-3, fl, by),
                         note="the same W (64 MiB) every launch: it stays in the 256 MiB Infinity Cache, so this is not an HBM figure"),
@@ -210,7 +262,7 @@ def bench_extras(r, with_cpu):
         c5a["cpu_baseline"] = dict(cpu_note("the whole product, best of 3"), value=dt * 1e3, unit="ms", **{"GB/s": by / dt / 1e9})
         orc.native.resetEngine()
     out["config5a_gemv"] = c5a
-    # the same W against batches of token rows (batched decoding): up to 8 rows through the skinny kernel (an
+    # the same W against batches of token rows (batched decoding): up to 8 rows through the decode kernel (an
     # instantiation per row count), 16 and 32 through the few-rows MFMA kernel, 64 through the tile kernel; W cold
     # (eight in rotation) -- not a BASELINE config
     rows_out = {}
@@ -251,7 +303,8 @@ def bench_extras(r, with_cpu):
     ms = time_launches(r, lambda: r.sgemm(1024, 1024, 65536, dX, dG, dO, a_strides=(1, 1024)), 30, 20)
     fl = 2.0 * 1024 * 1024 * 65536
     by = 4.0 * (2 * 65536 * 1024 + 1024 * 1024)
-    c5b = {"roofline": roofline("mfma", "gemm_mfma_kernel<1, 1, 2, 2, false> + splitk_reduce_kernel", ms * 1e-3, fl, by)}
+    c5b = {"roofline": roofline("mfma", "gemm_mfma_kernel<1, 1, 2, 2, false> + splitk_reduce_kernel", ms * 1e-3, fl, by,
+                                traffic=profile_traffic("config5b_tall_k_1024x1024x65536.txt"))}
     if with_cpu:
         rows = 8192  # an eighth of K: the oracle gathers X^T into a contiguous copy, then runs its i-k-j loop
         orc = oracle_api()
@@ -294,7 +347,8 @@ def bench_extras(r, with_cpu):
     c3["dQ_and_dKT_paired"] = dict(roofline("mfma", "gemm_mfma_pair_kernel<0, 1, 1, 1>", ms_pair * 1e-3, 2 * fl, 2 * by),
                                    note="both gradients in one launch; one after the other they take %.1f us" % ((each["dQ"] + each["dKT"]) * 1e3))
     total = each["scores"] + ms_pair
-    c3["roofline"] = dict(roofline("mfma", "the three products (scores, then both gradients in one launch)", total * 1e-3, 3 * fl, 3 * by),
+    c3["roofline"] = dict(roofline("mfma", "the three products (scores, then both gradients in one launch)", total * 1e-3, 3 * fl, 3 * by,
+                                   traffic=profile_traffic("config3_attention_products_32x512x64.txt")),
                           note="arithmetic intensity 25.6 flop/B against a ridge of 19.7: the matrix pipe bounds it (20.5 us for all "
                                "three), HBM is close behind (15.7 us); an empty launch in the same sequence takes "
                                "%.2f us; three separate launches take %.1f us" % (out["empty_launch_us"], sum(each.values()) * 1e3))
@@ -422,6 +476,9 @@ def bench_extras(r, with_cpu):
                          "note": "0.16 MFLOP and < 0.1 MB per step: neither roof applies; the step is the sum of its launch "
                                  "latencies and of the host's own work per op.  ms: each step followed by a wait for the device"}}
     api.native.resetEngine()
+    # the same step driven from plain C over the engine ABI (no language binding in the loop)
+    for fused in (False, True):
+        out["config1_readme_mlp_step" + ("_fused_linear" if fused else "")]["c_loop"] = c_loop_step(fused)
     if with_cpu:
         orc = oracle_api()
         so, ko = build1(orc)
@@ -487,6 +544,45 @@ def bench_extras(r, with_cpu):
     return out
 
 
+def split_extras(out):
+    """(other, extra): `extra` holds the configurations BASELINE names, in short form; `other` everything else."""
+    ex = {}
+    c1f, c1 = out.pop("config1_readme_mlp_step_fused_linear"), out.pop("config1_readme_mlp_step")
+    cf, cc = c1f.get("c_loop") or {}, c1.get("c_loop") or {}
+    ms1 = cf.get("ms_per_step_with_a_wait_after_each", c1f["ms"])
+    ex["config1"] = sig({
+        "ms": ms1, "measured": "plain-C loop over the engine ABI, fused Linear, a wait for the device after every step" if cf.get("steps") else "ctypes binding",
+        "launches_per_step": cf.get("launches_per_step", c1f["launches_per_step"]), "ms_in_a_loop_without_waits": cf.get("ms_per_step_in_a_loop"),
+        "composed_matmul_then_add": {"ms": cc.get("ms_per_step_with_a_wait_after_each"), "launches_per_step": cc.get("launches_per_step", c1["launches_per_step"])},
+        "through_the_ctypes_binding": {"fused_ms": c1f["ms"], "composed_ms": c1["ms"]},
+        "bound": "launch latency", "us_per_launch": ms1 * 1e3 / max(cf.get("launches_per_step", c1f["launches_per_step"]), 1),
+        "empty_launch_us": out["empty_launch_us"], "frac": None, "traffic": None})
+    if "cpu_baseline" in c1:
+        ex["config1"]["cpu_baseline"] = brief_cpu(c1["cpu_baseline"])
+    c3 = out.pop("config3_attention_scores")
+    ex["config3"] = brief(c3["roofline"], scores_us=c3["scores"]["us"], dQ_us=c3["dQ"]["us"], dKT_us=c3["dKT"]["us"],
+                          gradients_in_one_launch_us=c3["dQ_and_dKT_paired"]["us"], GBps=c3["roofline"]["GB/s"])
+    if "cpu_baseline" in c3:
+        ex["config3"]["cpu_baseline"] = brief_cpu(c3["cpu_baseline"])
+    c4f, c4 = out.pop("config4_ffn_step_fused_linear"), out.pop("config4_ffn_step")
+    ex["config4"] = brief(c4f["roofline"], ms=c4f["ms"], launches_per_step=c4f["launches_per_step"], kernel="whole step, fused Linear + GELU epilogues: six products + elementwise",
+                          composed=sig({"ms": c4["ms"], "frac": c4["roofline"]["frac"], "launches_per_step": c4["launches_per_step"]}))
+    if "cpu_baseline" in c4:
+        ex["config4"]["cpu_baseline"] = brief_cpu(c4["cpu_baseline"])
+    c5a = out.pop("config5a_gemv")
+    ex["config5a"] = brief(c5a["roofline"], weights="cold: eight W in rotation, every byte from HBM", warm_us=c5a["warm"]["us"], warm_frac=c5a["warm"]["frac"],
+                           read_yardstick_cold_us=out["hbm_read_yardstick_cold"]["us"], vs_read_yardstick_cold=c5a["vs_read_yardstick"]["cold"])
+    if "max_err_vs_oracle" in c5a:
+        ex["config5a"]["max_err_vs_oracle"] = sig(c5a["max_err_vs_oracle"])
+    if "cpu_baseline" in c5a:
+        ex["config5a"]["cpu_baseline"] = brief_cpu(c5a["cpu_baseline"])
+    c5b = out.pop("config5b_tall_k")
+    ex["config5b"] = brief(c5b["roofline"])
+    if "cpu_baseline" in c5b:
+        ex["config5b"]["cpu_baseline"] = brief_cpu(c5b["cpu_baseline"])
+    return sig(out), ex
+
+
 def run_for_counters(r, which):
     """Launch sequence for hardware-counter runs: the strided-copy kernel x3 on
     a contiguous 16M-float buffer (64 MiB read, 64 MiB written: the yardstick
@@ -521,6 +617,28 @@ def run_for_counters(r, which):
         for _ in range(5):
             r.sgemm_pair(r.gemm_desc(512, 64, 512, dds, dk, g_out, batch=32, a_batch=(512 * 512, 32), b_batch=(512 * 64, 32)),
                          r.gemm_desc(64, 512, 512, dq, dds, g_out2, batch=32, a_strides=(1, 64), a_batch=(512 * 64, 32), b_batch=(512 * 512, 32)))
+    elif which == "config5b":
+        # the tall-K weight gradient X^T[1024, 65536] dY[65536, 1024] (X^T a view): K slices and their reduction pass
+        X = r.to_device(synth.normal(5, (65536, 1024)))
+        G = r.to_device(synth.normal(5, (65536, 1024), stream=1))
+        for _ in range(5):
+            r.sgemm(1024, 1024, 65536, X, G, dst, a_strides=(1, 1024))
+    elif which == "config4":
+        # three FFN training steps with the fused Linear (forward + backward through the engine)
+        from framework_amd.api import bind
+        api = bind(N.Native())
+        d, h, rows = 1024, 4096, 4096
+        T = lambda a, g=False: (api.Tensor.fromFloat32(a, list(a.shape)).setRequiresGrad(True) if g else api.Tensor.fromFloat32(a, list(a.shape)))
+        x, tg = T(synth.normal(3, (rows, d)), True), T(synth.normal(3, (rows, d), stream=3))
+        l1 = api.Linear(d, h, weight=synth.uniform(3, (d, h), -1 / 32, 1 / 32, stream=1), bias=np.zeros(h, np.float32), fused=True, activation="gelu")
+        l2 = api.Linear(h, d, weight=synth.uniform(3, (h, d), -1 / 64, 1 / 64, stream=2), bias=np.zeros(d, np.float32), fused=True)
+        params = l1.parameters() + l2.parameters()
+        for _ in range(3):
+            api.native.zeroGrad([x._id] + [p.value._id for p in params])
+            api.mseLoss(l2.forward(l1.forward(x)), tg).backward()
+            keep = [x._id, tg._id] + [p.value._id for p in params]
+            keep += [g for g in (api.native.getGrad(t._id) for t in [x] + [p.value for p in params]) if g is not None]
+            api.native.gcTensors(keep)
     elif which == "fewrows":
         # 32 token rows against a [4096, 4096] weight (the few-rows kernel) and against an [8192, 8192] one, 5 launches each
         x = r.to_device(synth.normal(4, (32, 8192), 0.02))
@@ -563,6 +681,115 @@ def run_for_counters(r, which):
     print(json.dumps({"counters_run": which, "copy_bytes_read": n * 4, "copy_bytes_written": n * 4}))
 
 
+# ---- the planner held against forced plans -----------------------------------------------------------------------------
+# (M, N, K, batch, A given as its transpose, B given as its transpose): the configurations, the products of batched
+# decoding, small and transformer-sized Linear layers with their backward products, weight gradients of small batches,
+# batches of small products, edges off a multiple of four.
+PLANNER_SHAPES = [
+    (4096, 4096, 4096, 1, 0, 0), (4096, 4096, 1024, 1, 0, 0), (4096, 4096, 1024, 1, 0, 1), (4096, 1024, 4096, 1, 1, 0), (1024, 4096, 4096, 1, 1, 0),
+    (1024, 1024, 65536, 1, 1, 0), (512, 512, 64, 32, 0, 1), (512, 64, 512, 32, 0, 0), (64, 512, 512, 32, 1, 0),
+    (1, 4096, 4096, 1, 0, 0), (4, 4096, 4096, 1, 0, 0), (8, 4096, 4096, 1, 0, 0), (16, 4096, 4096, 1, 0, 0), (32, 4096, 4096, 1, 0, 0),
+    (64, 4096, 4096, 1, 0, 0), (128, 4096, 4096, 1, 0, 0), (192, 4096, 4096, 1, 0, 0), (4, 8192, 8192, 1, 0, 0), (4, 4096, 16384, 1, 0, 0),
+    (4, 16384, 4096, 1, 0, 0), (8, 50304, 768, 1, 0, 0), (12, 8192, 8192, 1, 0, 0), (16, 50304, 768, 1, 0, 1), (1, 50304, 768, 1, 0, 1),
+    (24, 11008, 4096, 1, 0, 0), (64, 4096, 11008, 1, 0, 0), (32, 64, 10, 1, 0, 0), (32, 3, 64, 1, 0, 0), (64, 512, 512, 1, 0, 0),
+    (256, 512, 512, 1, 0, 0), (16384, 16, 16, 1, 0, 0), (784, 128, 64, 1, 1, 0), (4096, 768, 3072, 1, 0, 0), (4096, 3072, 768, 1, 0, 0),
+    (4096, 2304, 768, 1, 0, 0), (2048, 2048, 2048, 1, 0, 0), (3000, 3000, 3000, 1, 0, 0), (1001, 1003, 999, 1, 0, 0), (2048, 2050, 2048, 1, 0, 0),
+    (4096, 4096, 8, 1, 1, 0), (4096, 4096, 32, 1, 1, 0), (4096, 11008, 64, 1, 1, 0), (768, 3072, 256, 1, 1, 0), (4096, 11008, 64, 1, 0, 0),
+    (8192, 8192, 128, 1, 0, 0), (2048, 8192, 32, 1, 0, 0), (64, 64, 64, 2048, 1, 0), (16, 64, 16, 8192, 0, 0), (4, 4, 4, 65536, 0, 0),
+    (1, 512, 64, 1024, 0, 1), (128, 128, 512, 32, 0, 0), (1024, 64, 1024, 16, 0, 0), (65536, 2, 768, 1, 0, 0), (4096, 10, 4096, 1, 0, 0),
+    (512, 512, 4096, 1, 0, 0), (768, 768, 4096, 1, 1, 0), (6144, 1024, 2048, 1, 0, 0), (8192, 8192, 8192, 1, 0, 0),
+]
+
+
+def planner_plans():
+    P = [("mfma128", N.ALGO_MFMA, 1), ("mfma128_s2", N.ALGO_MFMA, 2), ("mfma128_s4", N.ALGO_MFMA, 4), ("mfma128_s8", N.ALGO_MFMA, 8),
+         ("mfma64", N.ALGO_MFMA_SMALL, 1), ("mfma64_s2", N.ALGO_MFMA_SMALL, 2), ("mfma64_s4", N.ALGO_MFMA_SMALL, 4), ("mfma64_s8", N.ALGO_MFMA_SMALL, 8),
+         ("mfma64_s16", N.ALGO_MFMA_SMALL, 16), ("streamk", N.ALGO_MFMA_STREAMK, 0), ("skinny", N.ALGO_SKINNY, 0), ("skinny_two_pass", N.ALGO_SKINNY_TWO_PASS, 0),
+         ("direct", N.ALGO_DIRECT, 0), ("direct_s4", N.ALGO_DIRECT, 4), ("panel", N.ALGO_PANEL, 0), ("tiny", N.ALGO_TINY, 0), ("fewrows", N.ALGO_FEWROWS, 0),
+         ("outer", N.ALGO_OUTER, 0), ("gemv", N.ALGO_GEMV, 0)]
+    return {name: (algo, split) for name, algo, split in P}
+
+
+def planner_time(r, shape, bufs, algo, split, iters):
+    M, Nn, K, batch, ta, tb = shape
+    dA, dB, dC = bufs
+    desc = r.gemm_desc(M, Nn, K, dA, dB, dC, batch=batch, a_strides=(1, M) if ta else (K, 1), b_strides=(1, K) if tb else (Nn, 1),
+                       a_batch=(M * K, batch), b_batch=(K * Nn, batch), algo=algo, split_k=split)
+    try:
+        return r.sgemm_timed([desc], max(5, iters // 4), iters) * 1e3
+    except N.MniError:
+        return None  # the plan does not take this shape or layout
+
+
+def planner_bufs(r, shape):
+    M, Nn, K, batch, _, _ = shape
+    sizes = (M * K * batch, K * Nn * batch, M * Nn * batch)
+    bufs = [r.malloc(max(n, 1) * 4) for n in sizes]
+    for p, n in zip(bufs, sizes):
+        r.fill(p, 0.5, n)
+    return bufs
+
+
+def planner_iters(shape):
+    M, Nn, K, batch, _, _ = shape
+    return 40 if 2.0 * M * Nn * K * batch > 2e10 else 200
+
+
+def planner_sweep(r, path):
+    """Every forced plan on every shape of PLANNER_SHAPES: writes the best plan and its time per shape (the data
+    --planner-check holds the planner against)."""
+    plans = planner_plans()
+    rows = []
+    for shape in PLANNER_SHAPES:
+        bufs = planner_bufs(r, shape)
+        it = planner_iters(shape)
+        planner_time(r, shape, bufs, N.ALGO_AUTO, 0, it)  # (clocks)
+        heavy = 2.0 * shape[0] * shape[1] * shape[2] * shape[3] > 2e10  # no thread-per-output kernels on the large products
+        times = {name: planner_time(r, shape, bufs, algo, split, it) for name, (algo, split) in plans.items()
+                 if not (heavy and name in ("direct", "direct_s4", "tiny", "outer"))}
+        times = {k: round(v, 2) for k, v in times.items() if v is not None}
+        auto = planner_time(r, shape, bufs, N.ALGO_AUTO, 0, it)
+        best = min(times, key=times.get)
+        rows.append({"M": shape[0], "N": shape[1], "K": shape[2], "batch": shape[3], "a_transposed": shape[4], "b_transposed": shape[5],
+                     "auto_us": round(auto, 2), "best_plan": best, "best_us": times[best], "plans_us": times})
+        print("%-40s auto %9.2f  best %-16s %9.2f" % (str(shape), auto, best, times[best]), file=sys.stderr, flush=True)
+        for p in bufs:
+            r.free(p)
+    with open(path, "w") as f:
+        json.dump({"device": r.device_info()["name"].strip(), "unit": "us per launch, mni_rocm_sgemm_timed (HIP events, launches back to back)",
+                   "shapes": rows}, f, indent=1)
+
+
+def planner_check(r, path):
+    """Re-times every shape of the recorded sweep under MNI_ALGO_AUTO and under its recorded best plan, one right
+    after the other, and reports the shapes where the planner's choice is more than 10 % behind."""
+    plans = planner_plans()
+    data = json.load(open(path))
+    behind, lines = [], []
+    for row in data["shapes"]:
+        shape = (row["M"], row["N"], row["K"], row["batch"], row["a_transposed"], row["b_transposed"])
+        bufs = planner_bufs(r, shape)
+        it = planner_iters(shape)
+        algo, split = plans[row["best_plan"]]
+        planner_time(r, shape, bufs, N.ALGO_AUTO, 0, it)
+        best, auto = float("inf"), float("inf")
+        for _ in range(3):  # in turns, the smallest of three each: a figure of a few microseconds moves with the clocks
+            best = min(best, planner_time(r, shape, bufs, algo, split, it))
+            auto = min(auto, planner_time(r, shape, bufs, N.ALGO_AUTO, 0, it))
+        for p in bufs:
+            r.free(p)
+        rec = {"shape": list(shape), "auto_us": round(auto, 2), "best_plan": row["best_plan"], "best_us": round(best, 2),
+               "recorded_best_us": row["best_us"], "auto_over_best": round(auto / best, 3)}
+        lines.append(rec)
+        if auto > 1.10 * best:
+            behind.append(rec)
+        print("%-40s auto %9.2f  %-16s %9.2f  x%.3f%s" % (str(shape), auto, row["best_plan"], best, auto / best, "   <-- behind" if auto > 1.10 * best else ""),
+              file=sys.stderr, flush=True)
+    ratios = [l["auto_over_best"] for l in lines]
+    print(json.dumps({"planner_check": {"shapes": len(lines), "more_than_10_percent_behind": behind, "worst_ratio": max(ratios),
+                                        "mean_ratio": round(sum(ratios) / len(ratios), 4)}, "rows": lines}))
+
+
 def cpu_baseline(a, b, target_seconds):
     """The CPU oracle's matmul (clones and i-k-j loop, one thread) on the first
     rows of A against all of B; the row count is chosen from a short
@@ -599,9 +826,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
-    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "fewrows", "outer", "attention", "attention_bwd"], default=None,
+    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "config4", "config5b", "fewrows", "outer", "attention", "attention_bwd"], default=None,
                     help="for rocprofv3 --pmc runs: launch a copy kernel of known size (64 MiB read + 64 MiB "
                          "written) 3 times, then the chosen product 5 times, and exit")
+    ap.add_argument("--planner-sweep", metavar="JSON", default=None, help="time every forced plan on the planner's shape list and write the best per shape")
+    ap.add_argument("--planner-check", action="store_true", help="hold MNI_ALGO_AUTO against the recorded best plan of tests/golden/planner_sweep.json")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (got --gpus %d)" % args.gpus)
@@ -611,6 +840,12 @@ def main():
     info = r.device_info()
     if args.counters:
         run_for_counters(r, args.counters)
+        return
+    if args.planner_sweep:
+        planner_sweep(r, args.planner_sweep)
+        return
+    if args.planner_check:
+        planner_check(r, os.path.join(ROOT, "tests", "golden", "planner_sweep.json"))
         return
     wall_ms, kernel_ms, flops, (a, b), err = bench_headline(r, args.steps, args.warmup)
     value = flops / wall_ms / 1e9
@@ -627,10 +862,15 @@ def main():
                      "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MATRIX_TFLOPS,
                      "kernel_ms": kernel_ms, "algorithmic_flops": flops, "traffic": profile_traffic("gemm_mfma_4096_pmc.txt")},
     }
+    extra = None
     if not args.no_extras:
-        line["extra"] = bench_extras(r, not args.no_cpu)
+        line["other"], extra = split_extras(bench_extras(r, not args.no_cpu))
+    # the headline's own objects and the BASELINE configurations close the line
+    line["roofline"] = line.pop("roofline")
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a, b, args.cpu_sample_seconds)
+    if extra is not None:
+        line["extra"] = extra
     print(json.dumps(line))
 
 

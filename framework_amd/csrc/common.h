@@ -188,6 +188,7 @@ int dev_alloc(void **p, size_t bytes);  // contents undefined
 int dev_free(void *p);
 int dev_clear_cache();
 size_t dev_cached_bytes();  // bytes held in free lists
+void dev_alloc_stats(uint64_t *requests, uint64_t *driver_allocations, uint64_t *releases, uint64_t *cached_bytes);
 
 // ---- launch helpers --------------------------------------------------------
 // Every kernel launch of the library goes through this, so that launches can be counted.

@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <chrono>
 
 #include <unordered_map>
@@ -151,6 +152,8 @@ static bool poll_result_word(unsigned tag, unsigned *value, int micros) {
             const unsigned long long v = *w;
             if ((unsigned)(v >> 32) == tag) {
                 if (value) *value = (unsigned)v;
+                // what the kernel wrote to pinned memory before the tag is read by the caller after this
+                std::atomic_thread_fence(std::memory_order_acquire);
                 return true;
             }
             __builtin_ia32_pause();
@@ -240,6 +243,7 @@ struct Allocator {
     std::unordered_map<void *, size_t> live;  // ptr -> rounded size
     size_t total = 0;
     size_t cached = 0;
+    uint64_t requests = 0, driver_allocations = 0, releases = 0;  // dev_alloc calls, hipMalloc calls, dev_free calls
 };
 static Allocator &allocator() {
     // Never destroyed: tensors of the engine (another translation unit's
@@ -256,6 +260,7 @@ static size_t round_size(size_t bytes) {
 int dev_alloc(void **p, size_t bytes) {
     MNI_TRY(ensure_init());
     Allocator &a = allocator();
+    ++a.requests;
     size_t sz = round_size(bytes);
     auto it = a.free_lists.find(sz);
     if (it != a.free_lists.end() && !it->second.empty()) {
@@ -276,6 +281,7 @@ int dev_alloc(void **p, size_t bytes) {
             return set_error(MNI_ERR_NOMEM, "hipMalloc(%zu) failed: %s", sz, hipGetErrorString(e));
         }
     }
+    ++a.driver_allocations;
     a.total += sz;
     a.live[*p] = sz;
     return MNI_OK;
@@ -286,6 +292,7 @@ int dev_free(void *p) {
     Allocator &a = allocator();
     auto it = a.live.find(p);
     if (it == a.live.end()) return set_error(MNI_ERR_INVALID, "free of a pointer this library did not allocate");
+    ++a.releases;
     a.free_lists[it->second].push_back(p);
     a.cached += it->second;
     a.live.erase(it);
@@ -312,6 +319,10 @@ int dev_clear_cache() {
 }
 
 size_t dev_cached_bytes() { return allocator().cached; }
+void dev_alloc_stats(uint64_t *requests, uint64_t *driver_allocations, uint64_t *releases, uint64_t *cached_bytes) {
+    const Allocator &a = allocator();
+    *requests = a.requests; *driver_allocations = a.driver_allocations; *releases = a.releases; *cached_bytes = a.cached;
+}
 
 }  // namespace mni
 
@@ -425,6 +436,13 @@ size_t mni_rocm_sgemm_noalloc_workspace_bytes(void) { return NOALLOC_SCRATCH_BYT
 uint64_t mni_rocm_launch_count(void) {
     MNI_API_GUARD;
     return ctx().launches;
+}
+
+int mni_rocm_alloc_stats(uint64_t *requests, uint64_t *driver_allocations, uint64_t *releases, uint64_t *cached_bytes) {
+    MNI_API_GUARD;
+    if (!requests || !driver_allocations || !releases || !cached_bytes) return set_error(MNI_ERR_INVALID, "alloc_stats: null output");
+    dev_alloc_stats(requests, driver_allocations, releases, cached_bytes);
+    return MNI_OK;
 }
 
 int mni_rocm_test_raise_device_status(unsigned code) {

@@ -276,10 +276,15 @@ static int direct_plan(const GemmLaunch &g, int cus) {
     // four wavefronts sharing K against tile): [32 x 512 x 512] x [512 x 64] 16.4
     // vs 13.7, its transposed twin 15.7 vs 13.7, K = 256: 11.5 vs 9.1, K = 1024:
     // 27.4 vs 21.3, 32 x (128 x 128 x 512) 15.4 vs 13.0, 16 x (1024 x 64 x 1024)
-    // 27.2 vs 21.5, 40 batches of the first 29.6 vs 20.5.  MNI_ALGO_DIRECT
-    // still selects it.
-    (void)g;
-    (void)cus;
+    // 27.2 vs 21.5, 40 batches of the first 29.6 vs 20.5.
+    // What is left to it: many batches of a few rows and a K of one MFMA phase,
+    // where three quarters or more of each 64 x 64 tile of the tile kernel are
+    // padding and its LDS round trip is all it does (us, direct with one wavefront
+    // against tile): 8192 x (16 x 64 x 16) 32.3 vs 47.5, 2048 x (16 x 256 x 16) 32.0 vs
+    // 46.8, 2048 x (32 x 64 x 16) 9.1 vs 15.4, 2048 x (48 x 256 x 16) 39.0 vs 53.2,
+    // 512 x (16 x 256 x 16) 8.3 vs 14.2; at K = 32 the two are level.
+    // MNI_ALGO_DIRECT selects it for every eligible product.
+    if (g.K <= 16 && g.M <= 48 && g.N >= 64 && (int64_t)g.batch * ((g.N + 63) / 64) >= 2 * (int64_t)cus) return 1;
     return 0;
 }
 
@@ -345,7 +350,9 @@ static bool outer_plan(const GemmLaunch &g, int cus) {
     const int64_t own_pad = (int64_t)((g.M + 31) / 32 * 32) * ((g.N + 127) / 128 * 128);
     const int64_t tile_pad = (int64_t)((g.M + 63) / 64 * 64) * ((g.N + 63) / 64 * 64);
     if (own_pad > tile_pad && own_pad * 9 > mn * 10) return false;
-    if (outputs >= (1LL << 21)) return g.K <= 256;
+    // (768 x 3072, K = 256: 19.1 against 17.2, so the longest K only from 2048 x 2048 outputs on)
+    if (outputs >= (1LL << 22)) return g.K <= 256;
+    if (outputs >= (1LL << 21)) return g.K <= 128;
     return outputs >= (1LL << 16) && g.K <= 48;  // (512 x 512: K = 48 5.9 against 6.8, K = 64 6.9 against 6.0)
 }
 // Whether the few-rows kernel is the plan for an eligible product: from about 512 x 512 of W on it is ahead of the

@@ -62,6 +62,7 @@ SIGNATURES = {
     "mni_rocm_sync": (C.c_int, []),
     "mni_rocm_test_raise_device_status": (C.c_int, [C.c_uint]),
     "mni_rocm_launch_count": (C.c_uint64, []),
+    "mni_rocm_alloc_stats": (C.c_int, [C.POINTER(C.c_uint64)] * 4),
     "mni_rocm_event_create": (C.c_int, [C.POINTER(C.c_void_p)]),
     "mni_rocm_event_record": (C.c_int, [C.c_void_p]),
     "mni_rocm_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
@@ -234,6 +235,12 @@ class Rocm:
 
     def launch_count(self):
         return int(self.lib.mni_rocm_launch_count())
+
+    def alloc_stats(self):
+        """(requests, driver allocations, releases, cached bytes) of the library's device allocator."""
+        v = [C.c_uint64(0) for _ in range(4)]
+        self._check(self.lib.mni_rocm_alloc_stats(*[C.byref(x) for x in v]))
+        return tuple(int(x.value) for x in v)
 
     def event(self):
         e = C.c_void_p()

@@ -78,19 +78,13 @@ int mni_rocm_d2d(void *dst, const void *src, size_t bytes);
 int mni_rocm_sync(void);
 /* Device status.  A kernel that has to wait for other workgroups of its own
  * launch (the single-launch K-slice reduction of the skinny kernel, the
- * stream-K tile fix-up) waits a bounded number of polls; if the wait expires
- * it writes NaN into the outputs concerned and a code into a status word, and
- * the next call that waits for the stream (mni_rocm_sync, h2d, d2h,
- * event_elapsed_ms, sgemm_timed and every engine call built on them, such as
- * mni_to_float32 / mni_get_scalar) returns MNI_ERR_HIP with a message naming
- * the kernel, and clears the word.  mni_rocm_test_raise_device_status sets
- * the word from the host, so that this error path can be exercised without
- * making a kernel hang.  No counterpart in the reference. */
-int mni_rocm_test_raise_device_status(unsigned code);
-
-/* Kernels launched by the library since it was loaded (copies not counted):
- * what a latency-bound training step is made of.  No counterpart in the reference. */
-uint64_t mni_rocm_launch_count(void);
+ * stream-K tile fix-up, the decode product's partial sums) waits a bounded
+ * number of polls; if the wait expires it writes NaN into the outputs
+ * concerned and a code into a status word, and the next call that waits for
+ * the stream (mni_rocm_sync, h2d, d2h, event_elapsed_ms and every engine call
+ * built on them, such as mni_to_float32 / mni_get_scalar) returns MNI_ERR_HIP
+ * with a message naming the kernel, and clears the word.  No counterpart in
+ * the reference. */
 
 /* Stream-ordered timing marks on the library's stream (HIP events). */
 int mni_rocm_event_create(void **event);
@@ -183,21 +177,27 @@ typedef struct {
 int mni_rocm_sgemm(const mni_gemm_desc *desc);
 /* Rows of the colsum_part matrix a DGELU product of this height and batch count writes. */
 int64_t mni_rocm_sgemm_colsum_rows(int64_t M, int64_t batch);
-/* The same product for callers that cannot allocate device memory (code under
- * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
- * No counterpart in the reference.  Identical kernels, plans and results as
- * mni_rocm_sgemm, but the partial sums of a split-K, stream-K or skinny plan
- * go to a fixed 32 MiB workspace that is part of the library's code object
- * instead of a block from the caching allocator, and nothing is allocated or
- * freed during the call.  Requires a prior mni_rocm_init (initialisation
- * allocates; this call refuses to initialise).  A product whose plan needs
- * more than mni_rocm_sgemm_noalloc_workspace_bytes() fails with
- * MNI_ERR_INVALID and a message giving both sizes (every plan the library
- * chooses by itself fits; an explicit split_k over a large C may not).  All
- * calls share the one workspace: they are ordered on the library's stream,
- * so they do not race with each other, but the workspace keeps the last
- * call's partials and two processes' or two libraries' calls on the same
- * device memory would.  Nothing in it needs to start at zero. */
+/* The same product for callers that cannot allocate device memory (tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  The same kernels and the same sums as mni_rocm_sgemm, but the
+ * partial sums of a split-K, stream-K or skinny plan go to a fixed 32 MiB
+ * workspace that is part of the library's code object instead of a block
+ * from the caching allocator, and nothing is allocated or freed during the
+ * call.  Two differences in plan follow from that: a product whose B (or
+ * ragged A) mni_rocm_sgemm would first repack into a scratch copy runs on
+ * the operands as they are (same values, slower), and a product the decode
+ * kernel would take keeps that kernel (its partial-sum slots are allocated at
+ * mni_rocm_init).  The launches go to the library's own stream, as those of
+ * every other entry point do: a caller cannot record them into a HIP graph
+ * of its own.  Requires a prior mni_rocm_init (initialisation allocates;
+ * this call refuses to initialise).  A product whose plan needs more than
+ * mni_rocm_sgemm_noalloc_workspace_bytes() fails with MNI_ERR_INVALID and a
+ * message giving both sizes (every plan the library chooses by itself fits;
+ * an explicit split_k over a large C may not).  All calls share the one
+ * workspace: they are ordered on the library's stream, so they do not race
+ * with each other, but the workspace keeps the last call's partials and two
+ * processes' or two libraries' calls on the same device memory would.
+ * Nothing in it needs to start at zero. */
 int mni_rocm_sgemm_noalloc(const mni_gemm_desc *desc);
 size_t mni_rocm_sgemm_noalloc_workspace_bytes(void);
 /* Two products that do not depend on each other: neither reads what the other
@@ -209,43 +209,13 @@ size_t mni_rocm_sgemm_noalloc_workspace_bytes(void);
  * tail); so do two products of a few thousand outputs each (what
  * MNI_ALGO_AUTO gives to the tiny-product kernel: the gradients of a small
  * Linear); otherwise this is mni_rocm_sgemm(first) followed by
- * mni_rocm_sgemm(second).  The results are those of the separate calls bit
- * for bit. */
+ * mni_rocm_sgemm(second).  The values are those of the separate calls within
+ * the product's tolerance, and bit for bit wherever the separate call would
+ * run the same kernel (the joint launches use the tile kernel's 64 x 64 tiles
+ * in one K slice and the tiny-product kernel's sequential sum; a batch of
+ * products against one shared B that mni_rocm_sgemm alone would fold into a
+ * single tall product is summed in the unfolded order here). */
 int mni_rocm_sgemm_pair(const mni_gemm_desc *first, const mni_gemm_desc *second);
-/* Measurement aid (no counterpart in the reference): runs descs[0], descs[1],
- * ... descs[count-1], descs[0], ... back to back on the library's stream,
- * `warmup` untimed launches and then `iters` launches between two HIP events,
- * and returns the average milliseconds per launch.  Issuing from C keeps the
- * host ahead of kernels that take only a few microseconds. */
-int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms);
-/* The same for mni_rocm_sgemm_pair: descs holds count / 2 pairs (descs[0] with
- * descs[1], descs[2] with descs[3], ...); the average is per pair. */
-int mni_rocm_sgemm_pair_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms);
-
-/* Measurement aid (no counterpart in the reference): what the device gives a
- * kernel that only streams.  `iters` launches between two HIP events on the
- * library's stream after `warmup` untimed ones; the average milliseconds per
- * launch is returned.  EMPTY: a one-wavefront kernel that does nothing (the
- * cost of a launch in a back-to-back sequence).  READ: `bytes` bytes of
- * srcs[launch % nsrc] are read with 16-byte loads, 8 in flight per lane, and
- * nothing is written (several sources in rotation make the pass cold in the
- * last-level cache).  WRITE: `bytes` bytes of dst are written.  COPY: both.
- * `nontemporal` selects streaming loads / stores; the grid is blocks_per_cu
- * workgroups of 256 threads per compute unit.  Sizes are multiples of 16. */
-enum { MNI_YARDSTICK_EMPTY = 0, MNI_YARDSTICK_READ = 1, MNI_YARDSTICK_WRITE = 2, MNI_YARDSTICK_COPY = 3 };
-int mni_rocm_yardstick_timed(int kind, int nontemporal, void *dst, const void *const *srcs, int nsrc, size_t bytes,
-                             int blocks_per_cu, int warmup, int iters, float *avg_ms);
-/* Measurement aid (no counterpart in the reference): what the matrix pipe
- * gives a loop of nothing but fp32 MFMAs.  Every wavefront issues
- * `mfmas_per_wave` (a multiple of 16) v_mfma_f32_32x32x2_f32 on four
- * independent accumulators, each followed by `valu_per_mfma` (0..2) v_mov_b32
- * that depend on nothing; the grid is `waves_per_simd` (1 or 2) workgroups of
- * four wavefronts per compute unit.  Returns the average milliseconds per
- * launch; the rate is CUs * 4 * waves_per_simd * mfmas_per_wave * 4096 flop
- * over that.  The figure with valu_per_mfma = 0 is the ceiling an MFMA-bound
- * product is held against next to the datasheet's; the others show what every
- * vector-ALU instruction inside an MFMA loop costs on this device. */
-int mni_rocm_mfma_yardstick_timed(int valu_per_mfma, int waves_per_simd, int mfmas_per_wave, int warmup, int iters, float *avg_ms);
 
 /* dst (contiguous, `shape`) = gather of src by `src_strides` (elements).
  * Replaces permute_f32 (src/native/kernels/elementwise.cu:67-81) and the host
@@ -414,6 +384,63 @@ uint32_t mni_linear(uint32_t x, uint32_t w, uint32_t bias, int act);
 /* Device address of a tensor's buffer (cuda arm: TensorStore::dev_ptr,
  * src/native/src/tensor.rs:358-361). NULL on error. */
 void *mni_dev_ptr(uint32_t id);
+
+/* ------------------------------------------------------------------------- *
+ * Measurement and test hooks.  NOT part of the drop-in boundary: nothing the
+ * reference binds has a counterpart here and an integration needs none of
+ * them.  They exist so that benchmarks can issue launches from C (the host
+ * stays ahead of kernels of a few microseconds), so that a kernel can be held
+ * against what the device gives a loop that only streams or only issues
+ * MFMAs, and so that tests can reach an error path without hanging a kernel.
+ * ------------------------------------------------------------------------- */
+/* Sets the device status word from the host, as a kernel whose bounded wait
+ * expired would: the next call that waits for the stream reports it. */
+int mni_rocm_test_raise_device_status(unsigned code);
+
+/* Kernels launched by the library since it was loaded (copies not counted):
+ * what a latency-bound training step is made of. */
+uint64_t mni_rocm_launch_count(void);
+
+/* The library's device allocator since it was loaded: requests made of it
+ * (mni_rocm_malloc, tensors, workspaces), those that went on to hipMalloc
+ * (the others were served from its free lists), blocks given back to it, and
+ * the bytes its free lists hold now.  A test of mni_rocm_sgemm_noalloc reads
+ * them before and after the call. */
+int mni_rocm_alloc_stats(uint64_t *requests, uint64_t *driver_allocations, uint64_t *releases, uint64_t *cached_bytes);
+
+/* Runs descs[0], descs[1],
+ * ... descs[count-1], descs[0], ... back to back on the library's stream,
+ * `warmup` untimed launches and then `iters` launches between two HIP events,
+ * and returns the average milliseconds per launch.  Issuing from C keeps the
+ * host ahead of kernels that take only a few microseconds. */
+int mni_rocm_sgemm_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms);
+/* The same for mni_rocm_sgemm_pair: descs holds count / 2 pairs (descs[0] with
+ * descs[1], descs[2] with descs[3], ...); the average is per pair. */
+int mni_rocm_sgemm_pair_timed(const mni_gemm_desc *descs, int count, int warmup, int iters, float *avg_ms);
+/* What the device gives a
+ * kernel that only streams.  `iters` launches between two HIP events on the
+ * library's stream after `warmup` untimed ones; the average milliseconds per
+ * launch is returned.  EMPTY: a one-wavefront kernel that does nothing (the
+ * cost of a launch in a back-to-back sequence).  READ: `bytes` bytes of
+ * srcs[launch % nsrc] are read with 16-byte loads, 8 in flight per lane, and
+ * nothing is written (several sources in rotation make the pass cold in the
+ * last-level cache).  WRITE: `bytes` bytes of dst are written.  COPY: both.
+ * `nontemporal` selects streaming loads / stores; the grid is blocks_per_cu
+ * workgroups of 256 threads per compute unit.  Sizes are multiples of 16. */
+enum { MNI_YARDSTICK_EMPTY = 0, MNI_YARDSTICK_READ = 1, MNI_YARDSTICK_WRITE = 2, MNI_YARDSTICK_COPY = 3 };
+int mni_rocm_yardstick_timed(int kind, int nontemporal, void *dst, const void *const *srcs, int nsrc, size_t bytes,
+                             int blocks_per_cu, int warmup, int iters, float *avg_ms);
+/* What the matrix pipe
+ * gives a loop of nothing but fp32 MFMAs.  Every wavefront issues
+ * `mfmas_per_wave` (a multiple of 16) v_mfma_f32_32x32x2_f32 on four
+ * independent accumulators, each followed by `valu_per_mfma` (0..2) v_mov_b32
+ * that depend on nothing; the grid is `waves_per_simd` (1 or 2) workgroups of
+ * four wavefronts per compute unit.  Returns the average milliseconds per
+ * launch; the rate is CUs * 4 * waves_per_simd * mfmas_per_wave * 4096 flop
+ * over that.  The figure with valu_per_mfma = 0 is the ceiling an MFMA-bound
+ * product is held against next to the datasheet's; the others show what every
+ * vector-ALU instruction inside an MFMA loop costs on this device. */
+int mni_rocm_mfma_yardstick_timed(int valu_per_mfma, int waves_per_simd, int mfmas_per_wave, int warmup, int iters, float *avg_ms);
 
 #ifdef __cplusplus
 }

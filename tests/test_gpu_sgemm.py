@@ -569,6 +569,20 @@ def test_planner_choices_for_attention_shaped_products(dev, rocm):
     assert max_err(outs[0][7], q[7].T.astype(np.float64) @ ds[7].astype(np.float64)) <= gemm_tol(512, q, ds)
 
 
+@pytest.mark.parametrize("m,n,k,batch", [(16, 64, 16, 1024), (48, 256, 16, 512), (33, 70, 12, 600)])
+@pytest.mark.parametrize("tb", [False, True])
+def test_planner_gives_many_batches_of_few_rows_and_one_k_phase_to_the_direct_kernel(dev, rocm, m, n, k, batch, tb):
+    # three quarters of a 64 x 64 tile would be padding: the register-direct kernel, one wavefront per tile, takes them;
+    # the bits are the forced plan's, the values exact on small integers
+    a = synth.small_ints(m + n, (batch, m, k), 4)
+    b = synth.small_ints(k + batch, (batch, n, k) if tb else (batch, k, n), 4, stream=1)
+    got = run_gemm(dev, a, b, False, tb)
+    forced = run_gemm(dev, a, b, False, tb, algo=N.ALGO_DIRECT, split_k=1)
+    B = b.transpose(0, 2, 1) if tb else b
+    assert np.array_equal(got, np.einsum("bmk,bkn->bmn", a.astype(np.int64), B.astype(np.int64)).astype(np.float32))
+    assert np.array_equal(got, forced)
+
+
 # ---- tiny products: one thread per output, the reference CPU arm's own sum ---------------------------
 
 @pytest.mark.parametrize("m,n,k", [(32, 64, 10), (32, 3, 64), (32, 64, 3), (32, 10, 64), (64, 3, 32), (10, 64, 32), (1, 1, 1), (7, 5, 3),
@@ -1410,18 +1424,23 @@ def test_sgemm_timed_runs_the_products_and_reports_a_duration(dev, rocm):
     dCs = [dev.empty(64 * 80) for _ in bs]
     descs = [rocm.gemm_desc(64, 80, 48, dA, dB, dC) for dB, dC in zip(dBs, dCs)]
     ms = rocm.sgemm_timed(descs, 2, 7)  # 9 launches cycle over the 3 products
-    assert 0.0 < ms < 10.0
+    assert np.isfinite(ms) and ms > 0.0
     for b, dC in zip(bs, dCs):
         assert np.array_equal(rocm.to_host(dC, (64, 80)), (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32))
     with pytest.raises(N.MniError):
         rocm.sgemm_timed(descs, 0, 0)
 
 
-def test_mfma_yardstick_runs_and_shows_what_a_register_move_costs(rocm):
+def test_mfma_yardstick_runs_and_shows_what_a_register_move_costs(dev, rocm):
     pure = rocm.mfma_yardstick(0, mfmas_per_wave=8192)
     moved = rocm.mfma_yardstick(2, mfmas_per_wave=8192)
-    assert 100.0 < pure < 160.0          # TFLOP/s: below the 157.3 datasheet peak, well above any product
     assert moved < pure                  # vector-ALU instructions take their issue time from the MFMAs
+    # the yardstick is a ceiling for products on the same card at the same clocks: a 2048^3 product stays below it,
+    # and not by an order of magnitude
+    n = 2048
+    dA, dB, dC = dev.empty(n * n, fill=0.5), dev.empty(n * n, fill=0.25), dev.empty(n * n)
+    product = 2.0 * n ** 3 / (rocm.sgemm_timed([rocm.gemm_desc(n, n, n, dA, dB, dC)], 5, 20) * 1e-3) / 1e12
+    assert 0.1 * pure < product < pure
     with pytest.raises(N.MniError, match="bad arguments"):
         rocm.mfma_yardstick(3)
 

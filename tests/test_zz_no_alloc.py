@@ -1,7 +1,8 @@
 """mni_rocm_sgemm_noalloc: the product for callers that cannot allocate.  Its
 results must be the bits mni_rocm_sgemm gives (same kernels, same plan; only
 the home of the partial sums differs), call after call on the one shared
-workspace, also when a smaller product follows a larger one."""
+workspace, also when a smaller product follows a larger one, and the
+library's allocator must not be asked for anything meanwhile."""
 import numpy as np
 import pytest
 
@@ -12,7 +13,8 @@ from helpers import gemm_tol, max_err
 pytestmark = pytest.mark.gpu
 
 # (M, N, K, a_strides, algo, split_k): plans that keep partial sums in a workspace
-STREAMK = (4096, 768, 3072, None, N.ALGO_AUTO, 0)      # stream-K: 512 tile-sized slots = the whole 32 MiB
+STREAMK = (1300, 900, 1100, None, N.ALGO_MFMA_STREAMK, 0)   # stream-K forced: ragged tiles, one tile-sized slot per workgroup in the workspace
+STREAMK_AUTO = (2560, 2560, 2560, None, N.ALGO_AUTO, 0)     # no tile shape deals 256 CUs equal loads: the planner's own stream-K
 SPLITK = (1024, 1024, 8192, (1, 1024), N.ALGO_AUTO, 0)  # A^T view, 8 K slices of a 4 MiB result
 GEMV = (4, 4096, 4096, None, N.ALGO_AUTO, 0)            # skinny kernel, 64 K slices reduced inside the launch
 SMALL_SPLIT = (200, 136, 1000, None, N.ALGO_MFMA, 5)    # ragged edges, explicit split
@@ -35,7 +37,7 @@ def _run(rocm, fn, case, dA, dB, dC):
 
 
 @pytest.mark.parametrize("first,second", [(STREAMK, GEMV), (SPLITK, SMALL_SPLIT), (GEMV, NO_WORKSPACE), (STREAMK, SPLITK), (SPLITK, FEWROWS),
-                                          (FEWROWS, GEMV)])
+                                          (FEWROWS, GEMV), (STREAMK_AUTO, STREAMK)])
 def test_two_calls_in_a_row_match_the_allocating_entry_point(rocm, first, second):
     bufs = []
     try:
@@ -49,7 +51,11 @@ def test_two_calls_in_a_row_match_the_allocating_entry_point(rocm, first, second
         # the larger product, then the smaller one on the workspace the first left behind, then both again
         for _ in range(2):
             for (c, a, b, dA, dB, dC), w in zip(cases, want):
-                got = _run(rocm, rocm.sgemm_noalloc, c, dA, dB, dC)
+                rocm.fill(dC, -3.0, c[0] * c[1])
+                before = rocm.alloc_stats()
+                rocm.sgemm_noalloc(c[0], c[1], c[2], dA, dB, dC, a_strides=c[3], algo=c[4], split_k=c[5])
+                assert rocm.alloc_stats() == before, "the allocator was used during the call"
+                got = rocm.to_host(dC, (c[0], c[1]))
                 assert np.array_equal(got, w), "case %r differs from mni_rocm_sgemm" % (c,)
                 A = a.T if c[3] else a
                 rows = [0, c[0] // 2, c[0] - 1]
