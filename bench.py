@@ -408,7 +408,7 @@ def bench_extras(r, with_cpu):
 
         def step4():
             api.native.zeroGrad([x._id] + [p.value._id for p in params])
-            api.mseLoss(l2.forward(l1.forward(x)), tg).backward()
+            api.mseLoss(l2.forward(l1.forward(x)), tg, fused=fused).backward()
 
         def keep4():
             ids = [x._id, tg._id] + [p.value._id for p in params]
@@ -624,7 +624,7 @@ def run_for_counters(r, which):
         for _ in range(5):
             r.sgemm(1024, 1024, 65536, X, G, dst, a_strides=(1, 1024))
     elif which == "config4":
-        # three FFN training steps with the fused Linear (forward + backward through the engine)
+        # 24 FFN training steps with the fused Linear and the fused loss (forward + backward through the engine)
         from framework_amd.api import bind
         api = bind(N.Native())
         d, h, rows = 1024, 4096, 4096
@@ -633,9 +633,9 @@ def run_for_counters(r, which):
         l1 = api.Linear(d, h, weight=synth.uniform(3, (d, h), -1 / 32, 1 / 32, stream=1), bias=np.zeros(h, np.float32), fused=True, activation="gelu")
         l2 = api.Linear(h, d, weight=synth.uniform(3, (h, d), -1 / 64, 1 / 64, stream=2), bias=np.zeros(d, np.float32), fused=True)
         params = l1.parameters() + l2.parameters()
-        for _ in range(3):
+        for _ in range(24):  # (the clocks settle over the first twenty: the last steps of the trace are the ones to read)
             api.native.zeroGrad([x._id] + [p.value._id for p in params])
-            api.mseLoss(l2.forward(l1.forward(x)), tg).backward()
+            api.mseLoss(l2.forward(l1.forward(x)), tg, fused=True).backward()
             keep = [x._id, tg._id] + [p.value._id for p in params]
             keep += [g for g in (api.native.getGrad(t._id) for t in [x] + [p.value for p in params]) if g is not None]
             api.native.gcTensors(keep)

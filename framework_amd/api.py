@@ -233,7 +233,9 @@ def bind(native):
         def forward(self, x):
             return x.gelu()
 
-    def mseLoss(pred, target):  # src/nn.ts:161-165: mean(-1) twice
+    def mseLoss(pred, target, fused=False):  # src/nn.ts:161-165: mean(-1) twice
+        if fused and hasattr(native, "mseLoss") and list(pred.shape) == list(target.shape):
+            return Tensor(native.mseLoss(pred._id, target._id))  # opt-in: the same values from one pass
         diff = pred.sub(target)
         sq = diff.mul(diff)
         return Tensor(native.meanOp(Tensor(native.meanOp(sq._id, -1))._id, -1))

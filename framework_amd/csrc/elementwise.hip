@@ -539,6 +539,12 @@ int k_colsum(float *out, const float *a, int64_t rows, int64_t cols) {
     // Row blocks: 32 rows each; more when the second grid axis (65535 blocks)
     // would not hold them.  Few columns and many rows: the row-lane form.
     const bool narrow = cols <= CN_COLS && rows >= 4 * CN_ROWS;
+    // A few dozen rows (the strip sums a product's epilogue leaves for a bias gradient) are what the second pass
+    // is made for: one launch, not a pass of 32-row blocks and then their sum.
+    if (!narrow && rows > CS_ROWS && rows <= 256) {
+        MNI_KERNEL_LAUNCH(colsum_final_kernel, colsum_final_grid(cols), dim3(CF_COLS * CF_GROUPS), 0, ctx().stream, out, a, rows, cols);
+        return check_launch("colsum_final");
+    }
     const int lanes = narrow ? 256 / (int)cols : 0;
     int64_t rows_per_block = narrow ? (int64_t)CN_ROWS * lanes : CS_ROWS;
     int64_t nparts = (rows + rows_per_block - 1) / rows_per_block;
@@ -1061,6 +1067,85 @@ int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t
     }
     MNI_KERNEL_LAUNCH(reduce_inner_kernel, dim3(grid_for(n, TPB)), dim3(TPB), 0, ctx().stream, out, a, outer, dim, inner, div);
     return check_launch("reduce_inner");
+}
+
+// ---- mean of squared differences along the last dim, one pass each way ------------------------------------
+// What mseLoss composes from sub, mul and two means (src/nn.ts:161-165; the second mean runs over the size-1 dim
+// the first one leaves, so the loss is one value per row): out[r] = sum_c (p[r, c] - t[r, c])^2 / dim.
+// One wavefront per row, lanes stride the row (16-byte pieces when the row allows), sums folded in a fixed order.
+__global__ void mse_rows_kernel(float *__restrict__ out, const float *__restrict__ p, const float *__restrict__ t, int64_t rows,
+                                int64_t dim, float div, int vec) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *pr = p + row * dim, *tr = t + row * dim;
+    float s = 0.f;
+    if (vec) {
+        const int64_t n4 = dim >> 2;
+        for (int64_t d = lane; d < n4; d += 64) {
+            const float4 a = reinterpret_cast<const float4 *>(pr)[d], b = reinterpret_cast<const float4 *>(tr)[d];
+            const float x = a.x - b.x, y = a.y - b.y, z = a.z - b.z, w = a.w - b.w;
+            s += x * x; s += y * y; s += z * z; s += w * w;
+        }
+    } else {
+        for (int64_t d = lane; d < dim; d += 64) {
+            const float x = pr[d] - tr[d];
+            s += x * x;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (lane == 0) out[row] = s / div;
+}
+int k_mse_rows(float *out, const float *p, const float *t, int64_t rows, int64_t dim) {
+    if (rows <= 0) return MNI_OK;
+    if (dim <= 0) return set_error(MNI_ERR_INVALID, "mse: empty rows");
+    MNI_TRY(ensure_init());
+    const int vec = dim % 4 == 0 && ((uintptr_t)p & 15) == 0 && ((uintptr_t)t & 15) == 0;
+    MNI_KERNEL_LAUNCH(mse_rows_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, p, t, rows, dim, (float)dim, vec);
+    return check_launch("mse_rows");
+}
+// Its backward in one pass: what mean_backward (g / dim), mul_backward (g d for each of the two operands, added up) and
+// sub_backward (the negative for the target) leave behind: dp[r, c] = (g[r] / dim) d + (g[r] / dim) d with
+// d = p - t, and dt = -dp when it is wanted.
+__global__ void mse_rows_backward_kernel(float *__restrict__ dp, float *__restrict__ dt, const float *__restrict__ p,
+                                         const float *__restrict__ t, const float *__restrict__ g, int64_t dim, float div, int64_t n) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; idx < n; idx += step) {
+        const float gr = g[idx / dim] / div;
+        const float v = gr * (p[idx] - t[idx]);
+        const float o = 2.0f * v;  // (v + v, out of reach of a contraction into one fused multiply-add)
+        dp[idx] = o;
+        if (dt) dt[idx] = -o;
+    }
+}
+__global__ void mse_rows_backward4_kernel(float4 *__restrict__ dp, float4 *__restrict__ dt, const float4 *__restrict__ p,
+                                          const float4 *__restrict__ t, const float *__restrict__ g, int64_t dim4, float div, int64_t n4) {
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t step = (int64_t)gridDim.x * blockDim.x;
+    for (; idx < n4; idx += step) {
+        const float gr = g[idx / dim4] / div;
+        const float4 a = p[idx], b = t[idx];
+        float4 o;
+        o.x = gr * (a.x - b.x); o.y = gr * (a.y - b.y); o.z = gr * (a.z - b.z); o.w = gr * (a.w - b.w);
+        o.x *= 2.0f; o.y *= 2.0f; o.z *= 2.0f; o.w *= 2.0f;  // (v + v, out of reach of a contraction into one fused multiply-add)
+        dp[idx] = o;
+        if (dt) dt[idx] = make_float4(-o.x, -o.y, -o.z, -o.w);
+    }
+}
+int k_mse_rows_backward(float *dp, float *dt, const float *p, const float *t, const float *g, int64_t rows, int64_t dim) {
+    const int64_t n = rows * dim;
+    if (n <= 0) return MNI_OK;
+    MNI_TRY(ensure_init());
+    const bool al = (((uintptr_t)dp | (uintptr_t)dt | (uintptr_t)p | (uintptr_t)t) & 15) == 0;
+    if (dim % 4 == 0 && al) {
+        MNI_KERNEL_LAUNCH(mse_rows_backward4_kernel, dim3(grid_for(n / 4, TPB)), dim3(TPB), 0, ctx().stream, (float4 *)dp, (float4 *)dt,
+                          (const float4 *)p, (const float4 *)t, g, dim / 4, (float)dim, n / 4);
+        return check_launch("mse_rows_backward4");
+    }
+    MNI_KERNEL_LAUNCH(mse_rows_backward_kernel, dim3(grid_for(n, TPB * 2)), dim3(TPB), 0, ctx().stream, dp, dt, p, t, g, dim, (float)dim, n);
+    return check_launch("mse_rows_backward");
 }
 
 // sum_backward / mean_backward (src/native/src/ops/reduce.rs:94-118,232-263)

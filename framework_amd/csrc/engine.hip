@@ -64,7 +64,7 @@ enum Op {  // subset of src/native/src/autograd.rs:28-62 plus the fused Linear
     OP_SUM, OP_MEAN, OP_VIEW, OP_PERMUTE, OP_CONTIGUOUS, OP_CROSSENTROPY, OP_LINEAR,
     OP_SOFTMAX, OP_FLASHATTENTION, OP_BIASGELU,
     OP_EXP, OP_LOG, OP_DIV, OP_SIGMOID, OP_POW, OP_MAX, OP_LAYERNORM,
-    OP_EMBEDDING, OP_DROPOUT, OP_RESIDUALLAYERNORM
+    OP_EMBEDDING, OP_DROPOUT, OP_RESIDUALLAYERNORM, OP_MSEROWS
 };
 
 // src/native/src/autograd.rs:65-70 TapeEntry
@@ -894,6 +894,52 @@ static int cross_entropy_backward(uint32_t grad, const Entry &e, int64_t *out) {
     if (!o) return MNI_ERR_NOMEM;
     MNI_TRY(k_cross_entropy_backward(o->p, S->buf->p, (const int32_t *)e.targets.get(), G->buf->p, e.ce_n, e.ce_v));
     out[0] = insert_contig(std::move(o), shape);
+    return MNI_OK;
+}
+
+// Opt-in fused form of mseLoss (src/nn.ts:161-165: sub, mul, mean(-1), mean(-1)): one pass over both operands, one
+// tape entry.  The result is what the composition gives, one mean per row of the last dim (the second mean of the
+// composition runs over the size-1 dim the first one leaves).
+static uint32_t mse_rows_op(uint32_t pred, uint32_t target) {
+    Tensor *P = get(pred), *T = get(target);
+    if (!P || !T) return MNI_BAD_ID;
+    if (P->shape != T->shape || P->shape.empty() || P->size <= 0) {
+        set_error(MNI_ERR_INVALID, "mse_loss: prediction and target must have the same non-empty shape (no broadcasting)");
+        return MNI_BAD_ID;
+    }
+    Shape out_shape = P->shape;
+    const int64_t dim = out_shape.back();
+    out_shape.back() = 1;
+    const int64_t rows = P->size / dim;
+    BufP p = contiguous_buf(*P);
+    BufP t = p ? contiguous_buf(*get(target)) : nullptr;
+    BufP o = t ? new_buf((size_t)rows) : nullptr;
+    if (!o || k_mse_rows(o->p, p->p, t->p, rows, dim) != MNI_OK) return MNI_BAD_ID;
+    const uint32_t id = insert_contig(std::move(o), out_shape);
+    Entry e;
+    e.op = OP_MSEROWS; e.output_id = id; e.n_inputs = 2; e.inputs[0] = pred; e.inputs[1] = target;
+    eng().tape.record(std::move(e));
+    return id;
+}
+static int mse_rows_backward(uint32_t grad, const Entry &e, int64_t *out) {
+    Tensor *G = get(grad), *P = get(e.inputs[0]), *T = get(e.inputs[1]);
+    if (!G || !P || !T) return MNI_ERR_FREED;
+    const Shape shape = P->shape;
+    const int64_t dim = shape.back(), rows = P->size / dim;
+    if (G->size != rows) return set_error(MNI_ERR_INVALID, "mse_loss backward: gradient of %lld values for %lld rows", (long long)G->size, (long long)rows);
+    // the target's gradient only where something will take it: a tensor that asks for one, or one the tape produced
+    Engine &en = eng();
+    const uint32_t tid = e.inputs[1];
+    const bool want_t = T->requires_grad || (en.bw_out2entry && tid < en.bw_out2entry->size() && (*en.bw_out2entry)[tid] >= 0);
+    BufP g = contiguous_buf(*G);
+    BufP p = g ? contiguous_buf(*get(e.inputs[0])) : nullptr;
+    BufP t = p ? contiguous_buf(*get(e.inputs[1])) : nullptr;
+    BufP dp = t ? new_buf((size_t)(rows * dim)) : nullptr;
+    BufP dt = dp && want_t ? new_buf((size_t)(rows * dim)) : nullptr;
+    if (!dp || (want_t && !dt)) return MNI_ERR_NOMEM;
+    MNI_TRY(k_mse_rows_backward(dp->p, dt ? dt->p : nullptr, p->p, t->p, g->p, rows, dim));
+    out[0] = insert_contig(std::move(dp), shape);
+    if (dt) out[1] = insert_contig(std::move(dt), shape);
     return MNI_OK;
 }
 
@@ -1794,6 +1840,7 @@ static int dispatch_backward(const Entry &e, uint32_t grad, int64_t *out) {  // 
     case OP_EMBEDDING: return embedding_backward(grad, e, out);
     case OP_DROPOUT: return dropout_backward(grad, e, out);
     case OP_RESIDUALLAYERNORM: return residual_layernorm_backward(grad, e, out);
+    case OP_MSEROWS: return mse_rows_backward(grad, e, out);
     }
     return set_error(MNI_ERR_INVALID, "unknown tape op %d", e.op);
 }
@@ -2247,6 +2294,7 @@ uint32_t mni_matmul(uint32_t a, uint32_t b) {
     return out;
 }
 uint32_t mni_linear(uint32_t x, uint32_t w, uint32_t bias, int act) { MNI_API_GUARD; return linear_op(x, w, bias, act); }
+uint32_t mni_mse_loss(uint32_t pred, uint32_t target) { MNI_API_GUARD; return mse_rows_op(pred, target); }
 
 uint32_t mni_sum_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return reduce_op(a, dim, false); }
 uint32_t mni_mean_op(uint32_t a, int64_t dim) { MNI_API_GUARD; return reduce_op(a, dim, true); }

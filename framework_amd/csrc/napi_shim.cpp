@@ -321,6 +321,10 @@ napi_value Linear(napi_env env, napi_callback_info info) {
     const int act = a.n > 3 ? (int)get_i64(env, a.v[3]) : MNI_EPI_BIAS;
     return ret_id(env, mni_linear(get_u32(env, a.v[0]), get_u32(env, a.v[1]), get_u32(env, a.v[2]), act));
 }
+napi_value MseLoss(napi_env env, napi_callback_info info) {  // fused form of src/nn.ts:161-165
+    Args a(env, info);
+    return ret_id(env, mni_mse_loss(get_u32(env, a.v[0]), get_u32(env, a.v[1])));
+}
 
 FROM_SHAPE(RandTensor, mni_rand_tensor)    // lib.rs:60-64
 FROM_SHAPE(RandnTensor, mni_randn_tensor)  // lib.rs:67-71
@@ -422,7 +426,7 @@ NAPI_MODULE_INIT() {
         EXPORT("sumAll", SumAll), EXPORT("meanAll", MeanAll), EXPORT("view", View), EXPORT("permute", Permute),
         EXPORT("contiguous", Contiguous), EXPORT("crossEntropyLoss", CrossEntropyLoss), EXPORT("adamwStep", AdamwStep),
         EXPORT("gradNorm", GradNorm), EXPORT("clipGradNorm", ClipGradNorm), EXPORT("clipAndStep", ClipAndStep),
-        EXPORT("resetEngine", ResetEngine), EXPORT("gcTensors", GcTensors), EXPORT("linear", Linear),
+        EXPORT("resetEngine", ResetEngine), EXPORT("gcTensors", GcTensors), EXPORT("linear", Linear), EXPORT("mseLoss", MseLoss),
         EXPORT("softmaxOp", SoftmaxOp), EXPORT("biasGelu", BiasGelu),
         EXPORT("expOp", ExpOp), EXPORT("logOp", LogOp), EXPORT("sigmoid", Sigmoid), EXPORT("powOp", PowOp),
         EXPORT("div", Div), EXPORT("lt", Lt), EXPORT("eqOp", EqOp), EXPORT("gt", Gt), EXPORT("isClose", IsClose),

@@ -149,6 +149,7 @@ SIGNATURES = {
     "mni_reset_engine": (None, []),
     "mni_gc_tensors": (C.c_int, [_u32p, C.c_size_t]),
     "mni_linear": (C.c_uint32, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_int]),
+    "mni_mse_loss": (C.c_uint32, [C.c_uint32, C.c_uint32]),
     "mni_dev_ptr": (C.c_void_p, [C.c_uint32]),
 }
 
@@ -454,6 +455,9 @@ class Native:
 
     def linear(self, x, w, bias, act=EPI_BIAS):
         return self._id(self.lib.mni_linear(x, w, bias, act))
+
+    def mseLoss(self, pred, target):
+        return self._id(self.lib.mni_mse_loss(pred, target))
 
     def gelu(self, a):
         return self._id(self.lib.mni_gelu(a))

@@ -381,6 +381,15 @@ int mni_gc_tensors(const uint32_t *keep, size_t n);                       /* lib
  * act: MNI_EPI_BIAS (none), MNI_EPI_BIAS_RELU or MNI_EPI_BIAS_GELU. */
 uint32_t mni_linear(uint32_t x, uint32_t w, uint32_t bias, int act);
 
+/* Opt-in fused mseLoss: what src/nn.ts:161-165 composes from sub, mul and two
+ * mean(-1) calls, in one pass and one tape entry whose backward is one pass
+ * too.  Same result as the composition: one mean of squared differences per
+ * row of the last dim, shape [..., 1] (the composition's second mean runs
+ * over the size-1 dim the first one leaves).  Shapes must be equal; a caller
+ * that needs broadcasting keeps the composition.  Feature-detected like
+ * mni_linear. */
+uint32_t mni_mse_loss(uint32_t pred, uint32_t target);
+
 /* Device address of a tensor's buffer (cuda arm: TensorStore::dev_ptr,
  * src/native/src/tensor.rs:358-361). NULL on error. */
 void *mni_dev_ptr(uint32_t id);

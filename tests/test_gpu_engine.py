@@ -272,7 +272,7 @@ def ffn_inputs(rows, d, h):
     return x, w1, w2, t
 
 
-def ffn_script(api, x, w1, w2, t, fused=False, fused_gelu=False, b1=None):
+def ffn_script(api, x, w1, w2, t, fused=False, fused_gelu=False, b1=None, fused_mse=False):
     """fused: each Linear is one product with a bias epilogue.  fused_gelu: the first Linear also carries
     its GELU (two outputs from one epilogue), and in the backward the second Linear's product hands dX
     straight through gelu' to the first (no pre-activation tensor is visible then: hpre is None)."""
@@ -284,7 +284,7 @@ def ffn_script(api, x, w1, w2, t, fused=False, fused_gelu=False, b1=None):
     hpre = None if fused_gelu else l1.forward(X)
     hact = l1.forward(X) if fused_gelu else hpre.gelu()
     y = l2.forward(hact)
-    loss = api.mseLoss(y, T(api, t))
+    loss = api.mseLoss(y, T(api, t), fused=True) if fused_mse else api.mseLoss(y, T(api, t))
     loss.backward()
     return {"hpre": hpre, "hact": hact, "y": y, "loss": loss, "X": X, "l1": l1, "l2": l2}
 
@@ -292,10 +292,11 @@ def ffn_script(api, x, w1, w2, t, fused=False, fused_gelu=False, b1=None):
 def test_config4_ffn_step_reduced_vs_oracle(gpu, orc):
     x, w1, w2, t = ffn_inputs(256, 128, 512)
     b1 = synth.uniform(3, (512,), -0.3, 0.3, stream=4)   # the benchmark's bias is zero; a non-zero one exercises z + b
-    for fused, fused_gelu, bias1 in ((False, False, None), (True, False, None), (True, True, None), (True, True, b1)):
+    for fused, fused_gelu, bias1, fused_mse in ((False, False, None, False), (True, False, None, False), (True, True, None, False), (True, True, b1, False),
+                                                (True, True, b1, True)):
         gpu.native.resetEngine()
         orc.native.resetEngine()
-        g = ffn_script(gpu, x, w1, w2, t, fused, fused_gelu, bias1)
+        g = ffn_script(gpu, x, w1, w2, t, fused, fused_gelu, bias1, fused_mse)
         o = ffn_script(orc, x, w1, w2, t, b1=bias1)
         assert g["loss"].shape == [256, 1]
         assert_close(g["y"].numpy(), o["y"].numpy(), gemm_tol(512, o["hact"].numpy(), w2), "y")
@@ -316,7 +317,7 @@ def test_config4_ffn_step_full_size_relations(gpu, fused_gelu):
     # the tensors the GPU itself produced.  fused_gelu: the step the benchmark
     # times as "fused" (GELU and its backward inside the products' epilogues).
     x, w1, w2, t = ffn_inputs(4096, 1024, 4096)
-    g = ffn_script(gpu, x, w1, w2, t, fused_gelu, fused_gelu)
+    g = ffn_script(gpu, x, w1, w2, t, fused_gelu, fused_gelu, fused_mse=fused_gelu)
     hact, y = g["hact"].numpy(), g["y"].numpy()
     rows = np.array([0, 1, 2047, 4095])
     x64, w164, w264 = x.astype(np.float64), w1.astype(np.float64), w2.astype(np.float64)
@@ -360,6 +361,44 @@ def test_config4_ffn_step_full_size_relations(gpu, fused_gelu):
     dz_cols = dh_cols * (0.5 * (1 + thc) + 0.5 * vc * (1 - thc * thc) * s * (1 + 3 * 0.044715 * vc * vc))
     assert_close(gw1[:, hc], x64.T @ dz_cols, gemm_tol(4096, x, dz_cols) * 2, "dW1 = X^T dZ")
     assert_close(g["l1"].bias.value.grad.numpy()[hc], dz_cols.sum(0), gemm_tol(4096, dz_cols, np.ones(1)) * 2, "db1")
+
+
+@pytest.mark.parametrize("shape", [(256, 128), (7, 33), (3, 5, 40), (1, 1), (64, 4096)])
+def test_fused_mse_loss_is_the_composition_in_one_pass(gpu, orc, shape):
+    # forward: one mean of squared differences per row of the last dim, shape [..., 1] like the composition's two
+    # mean(-1) calls; backward: the composition's own arithmetic ((g / dim) d + (g / dim) d), so the same bits
+    p, t = synth.normal(11, shape), synth.normal(12, shape, stream=1)
+    up = synth.normal(13, shape[:-1] + (1,), stream=2)
+    res = {}
+    for name, api, fused in (("fused", gpu, True), ("composed", gpu, False), ("oracle", orc, False)):
+        api.native.resetEngine()
+        P, Tt = T(api, p, True), T(api, t, True)
+        loss = api.mseLoss(P, Tt, fused=True) if fused else api.mseLoss(P, Tt)
+        loss.mul(T(api, up)).backward()  # (a different upstream gradient for every row)
+        res[name] = (loss.shape, loss.numpy(), P.grad.numpy(), Tt.grad.numpy())
+    assert res["fused"][0] == res["composed"][0] == list(shape[:-1]) + [1]
+    assert_close(res["fused"][1], res["oracle"][1], 1e-5 * max(1.0, float(np.abs(res["oracle"][1]).max())), "loss")
+    assert_close(res["fused"][1], res["composed"][1], 1e-5 * max(1.0, float(np.abs(res["oracle"][1]).max())), "loss vs composed")
+    assert np.array_equal(res["fused"][2], res["composed"][2]) and np.array_equal(res["fused"][3], res["composed"][3])
+    assert_close(res["fused"][2], res["oracle"][2], 1e-6 * max(1.0, float(np.abs(res["oracle"][2]).max())), "dpred")
+    assert np.array_equal(res["fused"][3], -res["fused"][2])
+
+
+def test_fused_mse_loss_views_plain_targets_and_errors(gpu):
+    # a permuted prediction is gathered first; a target that asks for no gradient gets none; shapes must be equal
+    p, t = synth.normal(21, (40, 24)), synth.normal(22, (24, 40), stream=1)
+    P, Tt = T(gpu, p, True), T(gpu, t)
+    loss = gpu.mseLoss(P.permute(1, 0), Tt, fused=True)
+    loss.backward()
+    want = ((p.T.astype(np.float64) - t) ** 2).mean(1, keepdims=True)
+    assert_close(loss.numpy(), want, 1e-5, "loss of a permuted view")
+    assert_close(P.grad.numpy(), (2 * (p.T.astype(np.float64) - t) / 40).T, 1e-6, "gradient through the view")
+    assert Tt.grad is None
+    with pytest.raises(Exception, match="same non-empty shape"):
+        gpu.native.mseLoss(P._id, T(gpu, synth.normal(23, (24,)))._id)
+    # broadcasting keeps the composition
+    l2 = gpu.mseLoss(T(gpu, t), T(gpu, t[0]), fused=True)
+    assert l2.shape == [24, 1]
 
 
 # ---- configuration 5 through the engine ------------------------------------------------------------------
