@@ -136,6 +136,10 @@ struct Engine {
     // One float holding 1.0, shared by every scalar loss as the gradient backward() starts from (writers copy
     // a shared buffer before they touch it, so nobody changes it).
     BufP one;
+    // The same for the last loss that was not a scalar (the reference's mseLoss leaves one value per row): a buffer of
+    // that many ones, refilled only when the size changes.
+    BufP ones;
+    int64_t ones_n = 0;
 };
 static Engine &eng() {
     // Never destroyed: releasing device buffers from a static destructor would
@@ -1924,6 +1928,16 @@ static int tape_backward(Tape &tp, uint32_t loss) {
                 if (k_fill(e.one->p, 1.0f, 1) != MNI_OK) { e.one = nullptr; return MNI_ERR_HIP; }
             }
             g = insert_contig(BufP(e.one), shape);
+        } else if (shape_size(shape) <= (1 << 20)) {
+            Engine &e = eng();
+            const int64_t n = shape_size(shape);
+            if (!e.ones || e.ones_n != n) {
+                e.ones = new_buf((size_t)n);
+                e.ones_n = n;
+                if (!e.ones) { e.ones_n = 0; return MNI_ERR_NOMEM; }
+                if (k_fill(e.ones->p, 1.0f, n) != MNI_OK) { e.ones = nullptr; e.ones_n = 0; return MNI_ERR_HIP; }
+            }
+            g = insert_contig(BufP(e.ones), shape);
         } else {
             g = filled(shape, 1.0f);
         }
