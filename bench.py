@@ -277,6 +277,25 @@ def bench_extras(r, with_cpu):
         r.free(xb)
         r.free(yb)
     out["decode_batch_rows_x_4096x4096_cold"] = rows_out
+    # token rows against a weight stored [out, in] (a tied language-model head: logits = x E^T with E [50304, 768]), E cold
+    # (four in rotation, 618 MB) -- not a BASELINE config
+    head_out = {}
+    vocab, dm = 50304, 768
+    es = [r.malloc(vocab * dm * 4) for _ in range(4)]
+    for e in es:
+        r.fill(e, 0.01, vocab * dm)
+    for mrows in (1, 8, 16):
+        xb = r.to_device(synth.normal(7, (mrows, dm)))
+        yb = r.malloc(mrows * vocab * 4)
+        descs = [r.gemm_desc(mrows, vocab, dm, xb, e, yb, b_strides=(1, dm)) for e in es]
+        us = r.sgemm_timed(descs, 100, 200) * 1e3
+        byb = 4.0 * (vocab * dm + mrows * dm + mrows * vocab)
+        head_out["%d_rows" % mrows] = {"us": us, "GB/s": byb / us / 1e3, "frac_hbm": byb / us / 1e3 / PEAK_HBM_GBPS}
+        r.free(xb)
+        r.free(yb)
+    for e in es:
+        r.free(e)
+    out["rows_x_transposed_50304x768_weight_cold"] = head_out
     # the weight gradient of the same layer under a small batch: dW[4096,4096] = X^T[4096,rows] dY[rows,4096], X^T as a
     # view (matmul_backward's second product with K = the batch's rows): bound by writing dW -- not a BASELINE config
     grad_out = {}
@@ -691,7 +710,7 @@ PLANNER_SHAPES = [
     (1, 4096, 4096, 1, 0, 0), (4, 4096, 4096, 1, 0, 0), (8, 4096, 4096, 1, 0, 0), (16, 4096, 4096, 1, 0, 0), (32, 4096, 4096, 1, 0, 0),
     (64, 4096, 4096, 1, 0, 0), (128, 4096, 4096, 1, 0, 0), (192, 4096, 4096, 1, 0, 0), (4, 8192, 8192, 1, 0, 0), (4, 4096, 16384, 1, 0, 0),
     (4, 16384, 4096, 1, 0, 0), (8, 50304, 768, 1, 0, 0), (12, 8192, 8192, 1, 0, 0), (16, 50304, 768, 1, 0, 1), (1, 50304, 768, 1, 0, 1),
-    (24, 11008, 4096, 1, 0, 0), (64, 4096, 11008, 1, 0, 0), (32, 64, 10, 1, 0, 0), (32, 3, 64, 1, 0, 0), (64, 512, 512, 1, 0, 0),
+    (24, 11008, 4096, 1, 0, 0), (64, 4096, 11008, 1, 0, 0), (8, 50304, 768, 1, 0, 1), (16, 32000, 1024, 1, 0, 1), (32, 64, 10, 1, 0, 0), (32, 3, 64, 1, 0, 0), (64, 512, 512, 1, 0, 0),
     (256, 512, 512, 1, 0, 0), (16384, 16, 16, 1, 0, 0), (784, 128, 64, 1, 1, 0), (4096, 768, 3072, 1, 0, 0), (4096, 3072, 768, 1, 0, 0),
     (4096, 2304, 768, 1, 0, 0), (2048, 2048, 2048, 1, 0, 0), (3000, 3000, 3000, 1, 0, 0), (1001, 1003, 999, 1, 0, 0), (2048, 2050, 2048, 1, 0, 0),
     (4096, 4096, 8, 1, 1, 0), (4096, 4096, 32, 1, 1, 0), (4096, 11008, 64, 1, 1, 0), (768, 3072, 256, 1, 1, 0), (4096, 11008, 64, 1, 0, 0),
@@ -706,7 +725,7 @@ def planner_plans():
          ("mfma64", N.ALGO_MFMA_SMALL, 1), ("mfma64_s2", N.ALGO_MFMA_SMALL, 2), ("mfma64_s4", N.ALGO_MFMA_SMALL, 4), ("mfma64_s8", N.ALGO_MFMA_SMALL, 8),
          ("mfma64_s16", N.ALGO_MFMA_SMALL, 16), ("streamk", N.ALGO_MFMA_STREAMK, 0), ("skinny", N.ALGO_SKINNY, 0), ("skinny_two_pass", N.ALGO_SKINNY_TWO_PASS, 0),
          ("direct", N.ALGO_DIRECT, 0), ("direct_s4", N.ALGO_DIRECT, 4), ("panel", N.ALGO_PANEL, 0), ("tiny", N.ALGO_TINY, 0), ("fewrows", N.ALGO_FEWROWS, 0),
-         ("outer", N.ALGO_OUTER, 0), ("gemv", N.ALGO_GEMV, 0)]
+         ("outer", N.ALGO_OUTER, 0), ("gemv", N.ALGO_GEMV, 0), ("fewrows_nt", N.ALGO_FEWROWS_NT, 0)]
     return {name: (algo, split) for name, algo, split in P}
 
 

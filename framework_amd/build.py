@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "lib", "obj")
 LIB = os.path.join(HERE, "lib", "libmni_rocm.so")
-SOURCES = ["device.hip", "gemm_mfma.hip", "gemm_direct.hip", "gemm_panel.hip", "gemm_tiny.hip", "gemm_fewrows.hip", "gemm_outer.hip", "gemm_skinny.hip", "gemm_gemv.hip", "gemm.hip", "elementwise.hip", "yardstick.hip", "attention.hip", "sequence.hip", "engine.hip"]
+SOURCES = ["device.hip", "gemm_mfma.hip", "gemm_direct.hip", "gemm_panel.hip", "gemm_tiny.hip", "gemm_fewrows.hip", "gemm_outer.hip", "gemm_skinny.hip", "gemm_gemv.hip", "gemm_fewrows_nt.hip", "gemm.hip", "elementwise.hip", "yardstick.hip", "attention.hip", "sequence.hip", "engine.hip"]
 HEADERS = ["common.h", "gemm_internal.h", os.path.join("..", "..", "include", "mni_rocm.h")]
 
 # -packed-fp32-ops is switched off for device code: hipcc must not form

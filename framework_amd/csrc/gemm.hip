@@ -43,7 +43,7 @@ static int validate(const mni_gemm_desc &d) {
     if (d.epilogue != MNI_EPI_NONE && !d.bias)
         return set_error(MNI_ERR_INVALID, "sgemm: epilogue %d needs a bias pointer", d.epilogue);
     if (d.split_k < 0) return set_error(MNI_ERR_INVALID, "sgemm: split_k < 0");
-    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_GEMV)
+    if (d.algo < MNI_ALGO_AUTO || d.algo > MNI_ALGO_FEWROWS_NT)
         return set_error(MNI_ERR_INVALID, "sgemm: unknown algo %d", d.algo);
     return MNI_OK;
 }
@@ -363,6 +363,19 @@ static bool fewrows_plan(const GemmLaunch &g, int cus) {
     return g.K >= 256 && (int64_t)g.N * g.K >= (1 << 18);
 }
 
+// Whether the few-rows kernel for a K-contiguous B is the plan for an eligible product.  Measured on MI355X (us, cold W,
+// this kernel against the planner's choice without it -- the dots kernel up to 8 rows, 64 x 64 tiles in K slices beyond):
+// 16 x 50304 x 768 33.3 / 49.9, 9 rows 32.3 / 49.4, 8 rows 31.9 / 44.8, 4 rows 31.0 / 31.5, 2 rows 29.9 / 29.1, 1 row 31.2 / 28.7;
+// 16 x 16384 x 768 13.8 / 16.6, 16 x 8192 x 768 9.5 / 13.1, 16 x 4096 x 768 7.5 / 9.7, 16 x 4096 x 1984 15.5 / 22.7,
+// 8 x 32768 x 1984 53.0 / 66.1, 16 x 128256 x 512 70.2 / 74.4, 16 x 32000 x 1024 37.4 / 38.4; behind with a short K, where
+// the sum over a wavefront's sixteen blocks at the end of every group of four columns weighs (16 x 65536 x 256 37.3 / 20.2,
+// 12 x 262144 x 64 129 / 30), under 4096 columns (12 x 2048 x 1024 10.0 / 9.1), with four rows or fewer
+// (4 x 32000 x 1024 36.2 / 29.1) and beyond 16 rows, where eight LDS reads and 32 MFMAs per load add up
+// (32 x 50304 x 768 56.4 / 51.3).
+static bool fewrows_nt_plan(const GemmLaunch &g, int cus) {
+    (void)cus;
+    return g.M > 4 && g.M <= 16 && g.K >= 512 && g.N >= 4096;
+}
 // Whether run_mfma would give the product to the few-rows kernel by itself.
 static bool fewrows_takes(const mni_gemm_desc &d) {
     if (d.K == 0 || d.epilogue >= MNI_EPI_BIAS_GELU_DUAL) return false;
@@ -370,8 +383,10 @@ static bool fewrows_takes(const mni_gemm_desc &d) {
     fill_launch(g, d);
     DeviceCtx &c = ctx();
     const int amode = classify(g.a_cs, g.a_rs), bmode = classify(g.b_rs, g.b_cs);
+    const int cus = c.compute_units > 0 ? c.compute_units : 256;
+    if (gemm_fewrows_nt_eligible(g, amode, bmode) && fewrows_nt_plan(g, cus)) return true;  // (its twin for a K-contiguous B)
     return gemm_fewrows_eligible(g, amode, bmode) && (size_t)((g.N + 127) / 128) * g.batch <= c.fewrows_counter_cap && c.xcd_count == 8 &&
-           fewrows_plan(g, c.compute_units > 0 ? c.compute_units : 256);
+           fewrows_plan(g, cus);
 }
 
 // K slices for a product of `tiles` 64 x 64 tiles (at most one per CU) of `ktiles` K steps each.
@@ -445,6 +460,14 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
         g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
         if (probe) { probe->kind = PlanProbe::OUTER; return MNI_OK; }
         return launch_gemm_outer(g);
+    }
+    // Few rows against a wide K-contiguous operand (a weight stored [out, in]): forced, or chosen by fewrows_nt_plan.
+    if (d.algo == MNI_ALGO_FEWROWS_NT || (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_fewrows_nt_eligible(g, amode, bmode) && fewrows_nt_plan(g, cus))) {
+        if (!gemm_fewrows_nt_eligible(g, amode, bmode) || d.split_k > 1)
+            return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel for a K-contiguous B takes one product of up to 32 rows of a K-contiguous A, K %% 64 == 0 and "
+                                              "short enough for A to sit in LDS (1984, 960 beyond 16 rows), operands 16-byte aligned, no split_k");
+        if (probe) { probe->kind = PlanProbe::FEWROWS; return MNI_OK; }
+        return launch_gemm_fewrows_nt(g, amode, bmode);
     }
     // Few-rows form (9 to 32 rows against a wide N-contiguous operand): forced, or chosen by fewrows_plan.
     {
@@ -751,7 +774,7 @@ int sgemm(const mni_gemm_desc &d) {
     // 9 to 16 rows against a wide N-contiguous operand: the few-rows MFMA kernel is level with or ahead of the skinny
     // kernel's 16-row forms (us, few-rows against skinny: 16 x 4096 x 4096 18.6 / 21.5, 12 rows 18.6 / 30.5,
     // 16 x 8192 x 8192 46 / 58, 16 x 1024 x 1024 8.5 / 8.4; at 8 rows the skinny kernel leads, 15.2 / 18.6)
-    const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M > 8 && d.M <= 16 && fewrows_takes(d);
+    const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M > 4 && d.M <= 16 && fewrows_takes(d);
     if (!to_fewrows &&
         ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS ||
          d.algo == MNI_ALGO_GEMV)) {

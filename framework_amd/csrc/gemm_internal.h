@@ -151,6 +151,20 @@ bool gemv_units_plan(int rows, int cols, int K, int cus, int xcds, int *slices, 
 size_t gemv_units_partial_slots(int rows, int cols, int slices);  // pieces of pa (and of pb) the plan writes
 int launch_gemv_units(const GemvLaunch &p, int rows);
 
+// Up to 32 rows against a wide K-contiguous operand (gemm_fewrows_nt.hip): a wavefront per 16 columns and all of K, A in LDS.
+static constexpr int FEWROWS_NT_LDS_FLOATS = 32768;  // 16 (or 32) rows of K + 4 floats
+struct FewNtLaunch {
+    const float *X;     // [M, K], rows x_rs apart
+    const float *W;     // [N, K], rows w_cs apart
+    float *out;         // [M, N], rows o_rs apart
+    const float *bias;  // one value per column, or null
+    int M, N, K;
+    int64_t x_rs, w_cs, o_rs;
+    int epilogue, accumulate;
+};
+bool gemm_fewrows_nt_eligible(const GemmLaunch &g, int amode, int bmode);
+int launch_gemm_fewrows_nt(const GemmLaunch &g, int amode, int bmode);
+
 // Sums split-K partials ws[slice][batch][rows][cols] in slice order and
 // applies the epilogue; out addressed with (o_bs, o_rs, o_cs).
 struct ReduceLaunch {

@@ -23,7 +23,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmni_rocm.so")
 BAD_ID = 0xFFFFFFFF
 MAX_DIMS = 8
 EPI_NONE, EPI_BIAS, EPI_BIAS_RELU, EPI_BIAS_GELU, EPI_BIAS_GELU_DUAL, EPI_DGELU = 0, 1, 2, 3, 4, 5
-ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL, ALGO_SKINNY_TWO_PASS, ALGO_MFMA_STREAMK, ALGO_DIRECT, ALGO_PANEL, ALGO_TINY, ALGO_FEWROWS, ALGO_OUTER, ALGO_GEMV = 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11
+ALGO_AUTO, ALGO_MFMA, ALGO_SKINNY, ALGO_MFMA_SMALL, ALGO_SKINNY_TWO_PASS, ALGO_MFMA_STREAMK, ALGO_DIRECT, ALGO_PANEL, ALGO_TINY, ALGO_FEWROWS, ALGO_OUTER, ALGO_GEMV, ALGO_FEWROWS_NT = 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12
 
 _f32p = C.POINTER(C.c_float)
 _i64p = C.POINTER(C.c_int64)

@@ -149,10 +149,16 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * (error unless one batch, N % 128 == 0 with N / 128 a divisor of the 256
  * compute units and a multiple of 8, K a multiple of 512 * 256 / (N / 128),
  * B, C and the bias 16-byte aligned with row strides in whole 16 bytes, and
- * no activation together with accumulate).  AUTO picks among them. */
+ * no activation together with accumulate); FEWROWS_NT = up to 32 rows of a
+ * K-contiguous A against a wide B that is K-contiguous too (a weight stored
+ * [out, in], given as its transposed view): a wavefront per 16 columns and
+ * all of K on the 16 x 16 x 4 MFMA, A resident in LDS, no sums across
+ * wavefronts (error unless one batch, K % 64 == 0 and at most 1984, 960
+ * beyond 16 rows, both operands 16-byte aligned with pitches in whole 16
+ * bytes, no split_k).  AUTO picks among them. */
 enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
        MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7, MNI_ALGO_TINY = 8, MNI_ALGO_FEWROWS = 9,
-       MNI_ALGO_OUTER = 10, MNI_ALGO_GEMV = 11 };
+       MNI_ALGO_OUTER = 10, MNI_ALGO_GEMV = 11, MNI_ALGO_FEWROWS_NT = 12 };
 
 /* C[b] (M x N, row stride ldc, unit column stride) = epilogue(op(A)[b] (M x K) * op(B)[b] (K x N)).
  * Replaces dev.blas.gemm / gemm_strided_batched (src/native/src/ops/matmul.rs:150-189),

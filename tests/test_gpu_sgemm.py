@@ -957,6 +957,61 @@ def test_decode_product_kernel_ineligible_is_an_error_only_when_forced(dev, rocm
         _gemv_gemm(dev, a9, b9, algo=N.ALGO_GEMV)
 
 
+# ---- few rows against a wide K-contiguous operand (a weight stored [out, in]): a wavefront per 16 columns, all of K ----
+@pytest.mark.parametrize("m,n,k", [(16, 50304, 768), (9, 20000, 256), (32, 16400, 512), (17, 16384, 960), (12, 33000, 1984), (1, 4096, 64),
+                                   (8, 1000, 128), (32, 70, 320), (16, 16, 1984), (5, 4099, 768), (3, 9001, 512), (8, 16384, 768)])
+def test_fewrows_nt_kernel_integer_exact(dev, rocm, m, n, k):
+    # one and two 16-row sets, column counts off a multiple of 16, K at both ends of what fits LDS, K off a multiple of
+    # the ring of loads, fewer column groups than CUs; forced and as the planner's choice
+    a = synth.small_ints(m + n, (m, k), 3)
+    bt = synth.small_ints(n + k, (n, k), 3, stream=1)
+    want = (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(run_gemm(dev, a, bt, False, True, algo=N.ALGO_FEWROWS_NT)[0], want)
+    assert np.array_equal(run_gemm(dev, a, bt, False, True)[0], want)  # (the planner's choice, whichever kernel that is)
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 20000, 768), (24, 16390, 256)])
+def test_fewrows_nt_kernel_epilogues_accumulate_and_pitches(dev, rocm, m, n, k):
+    a = synth.small_ints(m, (m, k), 3); bt = synth.small_ints(m + 1, (n, k), 3, stream=1)
+    bias = synth.small_ints(m + 2, (n,), 5, stream=2); old = synth.small_ints(m + 3, (m, n), 9, stream=3)
+    prod = (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float64)
+    lda, ldb, ldc = k + 8, k + 12, n + 3  # pitches off their extents (operands in whole 16-byte pieces, C any)
+    sa = np.zeros((m, lda), np.float32); sa[:, :k] = a
+    sb = np.zeros((n, ldb), np.float32); sb[:, :k] = bt
+    dA, dB, dBias = dev.put(sa), dev.put(sb), dev.put(bias)
+    for epi, accumulate in [(N.EPI_NONE, False), (N.EPI_NONE, True), (N.EPI_BIAS, False), (N.EPI_BIAS, True), (N.EPI_BIAS_RELU, True),
+                            (N.EPI_BIAS_GELU, False)]:
+        z = prod + (bias if epi != N.EPI_NONE else 0.0)
+        if epi == N.EPI_BIAS_RELU: z = np.maximum(z, 0.0)
+        if epi == N.EPI_BIAS_GELU: z = 0.5 * z * (1.0 + np.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        want = z + (old if accumulate else 0.0)
+        sc = np.full((m, ldc), -5.0, np.float32); sc[:, :n] = old
+        dC = dev.put(sc)
+        rocm.sgemm(m, n, k, dA, dB, dC, a_strides=(lda, 1), b_strides=(1, ldb), ldc=ldc, bias=dBias if epi != N.EPI_NONE else None, epilogue=epi,
+                   accumulate=accumulate, algo=N.ALGO_FEWROWS_NT)
+        got = rocm.to_host(dC, (m, ldc))
+        assert np.all(got[:, n:] == -5.0), "the padding of C was written"
+        if epi == N.EPI_BIAS_GELU:
+            assert np.abs(got[:, :n] - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), (epi, accumulate)
+        else:
+            assert np.array_equal(got[:, :n], want.astype(np.float32)), (epi, accumulate)
+
+
+def test_fewrows_nt_kernel_normal_inputs_and_what_it_refuses(dev, rocm):
+    m, n, k = 16, 50304, 768
+    a = synth.normal(51, (m, k), 0.05); bt = synth.normal(52, (n, k), 0.05, stream=1)
+    want = a.astype(np.float64) @ bt.T.astype(np.float64)
+    got = run_gemm(dev, a, bt, False, True, algo=N.ALGO_FEWROWS_NT)[0]
+    assert max_err(got, want) <= gemm_tol(k, a, bt)
+    assert np.array_equal(got, run_gemm(dev, a, bt, False, True, algo=N.ALGO_FEWROWS_NT)[0])
+    # 40 rows; K off a multiple of 64; K beyond what LDS holds for 32 rows; a row-major B
+    for mm, kk, tb in ((40, 256, True), (16, 208, True), (32, 1024, True), (16, 256, False)):
+        aa = synth.small_ints(1, (mm, kk), 3)
+        bb = synth.small_ints(2, (20000, kk) if tb else (kk, 20000), 3, stream=1)
+        with pytest.raises(N.MniError, match="few-rows kernel for a K-contiguous B"):
+            run_gemm(dev, aa, bb, False, tb, algo=N.ALGO_FEWROWS_NT)
+
+
 @pytest.mark.parametrize("m", [1, 3, 5, 7])
 def test_skinny_cols_decode_shape_normal_inputs(dev, m):
     # the kernels specialised for a row count: within tolerance of a float64 product and of the two-launch form,
