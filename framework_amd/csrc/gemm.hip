@@ -79,32 +79,46 @@ static int next_epoch(unsigned *epoch) {
 static bool try_gemv_units(const SkinnyLaunch &s, const mni_gemm_desc &d, int *rc) {
     DeviceCtx &c = ctx();
     if (d.algo != MNI_ALGO_AUTO && d.algo != MNI_ALGO_GEMV) return false;
-    if (d.split_k > 1 || s.batch != 1 || s.rows > 8 || s.x_cs != 1 || s.w_cs != 1 || s.o_cs != 1) return false;
+    if (d.split_k > 1 || s.batch != 1 || s.rows > 16 || s.x_cs != 1 || s.w_cs != 1 || s.o_cs != 1) return false;
     if ((s.w_rs % 4) != 0 || !aligned16(s.W) || (s.o_rs % 4) != 0 || !aligned16(s.out)) return false;
     if (s.w_rs > 0x7fffffffLL || s.x_rs > 0x7fffffffLL || s.o_rs > 0x7fffffffLL) return false;
     if (s.epilogue > MNI_EPI_BIAS_GELU || s.bias_on_rows) return false;
     if (s.epilogue != MNI_EPI_NONE && !aligned16(s.bias)) return false;
     if (s.accumulate && s.epilogue >= MNI_EPI_BIAS_RELU) return false;  // (the old output would have to wait for the sum)
-    int slices = 0, trips = 0;
-    if (!gemv_units_plan(s.rows, s.cols, s.K, c.compute_units, c.xcd_count, &slices, &trips)) return false;
-    // Several trips per workgroup are taken one after the other (16 loads per lane, used up, the next 16): ahead of the
-    // column kernel's four small workgroups per CU up to 4096 columns (us, cold: 4 x 4096 x 8192 23.2 against 30.3,
-    // 4 x 4096 x 16384 46.3 / 54.6), level at 16384 and 32768 columns (44.9 / 43.8, 87.3 / 87.5), behind at 8192
-    // (4 x 8192 x 8192 52.0 against 45.0).  One trip: 4 x 4096 x 4096 12.8 / 14.4, 1 row 12.2 / 13.5, 8 rows 14.5 / 16.3,
-    // 4 x 8192 x 2048 13.0 / 14.6, 4 x 32768 x 512 12.9 / 15.6, 4 x 16384 x 1024 13.3 / 14.3.
-    if (d.algo == MNI_ALGO_AUTO && trips > 1 && s.cols > 4096) return false;
-    if (!c.gemv_pa || gemv_units_partial_slots(s.rows, s.cols, slices) > c.gemv_slot_cap ||
-        (size_t)(s.cols / 128) * GEMV_COUNTERS_PER_UNIT > c.gemv_counter_cap)
+    // Two forms.  Up to 8 rows on 4 x 4 x 1 blocks (128-column units, a kernel per row count); up to 16 rows on the
+    // 16 x 16 x 4 MFMA (64-column units, X in 16-byte pieces), whose time does not depend on the row count.  Measured on
+    // MI355X, us, cold W, the first against the second: 4096 x 4096 1 row 12.2 / 13.7, 4 rows 12.8 / 13.8, 6 rows 13.5 / 13.8,
+    // 7 rows 14.3 / 13.8, 8 rows 14.5 / 13.8 (16 rows 14.1: 20.9 through the few-rows kernel); 8192 x 8192 4 rows 51.2 / 42.4
+    // (the column kernel 45.0), 8 rows 52.4 / 43.0; 16384 x 1024 4 rows 13.3 / 12.4, 8 rows 15.0 / 12.6; 4096 x 8192 4 rows
+    // 23.1 / 23.8, 8 rows 24.9 / 24.0.
+    int slices = 0, trips = 0, slices16 = 0, trips16 = 0;
+    const bool narrow_ok = s.rows <= 8 && c.gemv_pa && gemv_units_plan(s.rows, s.cols, s.K, c.compute_units, c.xcd_count, &slices, &trips) &&
+                           gemv_units_partial_slots(s.rows, s.cols, slices) <= c.gemv_slot_cap &&
+                           (size_t)(s.cols / 128) * GEMV_COUNTERS_PER_UNIT <= c.gemv_counter_cap;
+    const bool wide_ok = c.gemv_pa && (s.x_rs % 4) == 0 && aligned16(s.X) &&
+                         gemv_units16_plan(s.rows, s.cols, s.K, c.compute_units, c.xcd_count, &slices16, &trips16) &&
+                         gemv_units16_partial_slots(s.cols, slices16) <= c.gemv_slot_cap &&
+                         (size_t)(s.cols / 64) * GEMV_COUNTERS_PER_UNIT <= c.gemv_counter_cap;
+    const bool prefer_wide = s.rows > 6 || s.cols > 4096;
+    const bool wide = wide_ok && (prefer_wide || !narrow_ok);
+    if (!wide && !narrow_ok) return false;
+    if (wide) {
+        slices = slices16;
+        trips = trips16;
+    } else if (d.algo == MNI_ALGO_AUTO && trips > 1 && s.cols > 4096) {
+        // (several trips of the narrow form beyond 4096 columns: the column kernel's four small workgroups per CU are
+        // ahead, 4 x 8192 x 8192 52.0 against 45.0; reached only where the wide form cannot take the product)
         return false;
+    }
     GemvLaunch g;
     g.W = s.W; g.X = s.X; g.out = s.out; g.bias = s.bias;
     g.pa = (decltype(g.pa))c.gemv_pa; g.pb = (decltype(g.pb))c.gemv_pb;
     g.count = c.gemv_counters; g.status = c.status_dev;
-    g.units = s.cols / 128; g.slices = slices; g.trips = trips;
+    g.units = s.cols / (wide ? 64 : 128); g.slices = slices; g.trips = trips;
     g.w_rs = (int)s.w_rs; g.x_rs = (int)s.x_rs; g.o_rs = (int)s.o_rs;
-    g.epilogue = s.epilogue; g.accumulate = s.accumulate;
+    g.epilogue = s.epilogue; g.accumulate = s.accumulate; g.rows = s.rows;
     *rc = next_epoch(&g.epoch);
-    if (*rc == MNI_OK) *rc = launch_gemv_units(g, s.rows);
+    if (*rc == MNI_OK) *rc = wide ? launch_gemv_units16(g) : launch_gemv_units(g, s.rows);
     return true;
 }
 
@@ -774,6 +788,18 @@ int sgemm(const mni_gemm_desc &d) {
     // 9 to 16 rows against a wide N-contiguous operand: the few-rows MFMA kernel is level with or ahead of the skinny
     // kernel's 16-row forms (us, few-rows against skinny: 16 x 4096 x 4096 18.6 / 21.5, 12 rows 18.6 / 30.5,
     // 16 x 8192 x 8192 46 / 58, 16 x 1024 x 1024 8.5 / 8.4; at 8 rows the skinny kernel leads, 15.2 / 18.6)
+    // 9 to 16 rows of the decode shape: the 16-row form of the decode product ahead of the few-rows kernel
+    if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M > 8 && d.M <= 16 && d.batch == 1 && d.K > 0 && d.epilogue <= MNI_EPI_BIAS_GELU) {
+        SkinnyLaunch s;
+        s.rows = (int)d.M; s.cols = (int)d.N; s.K = (int)d.K; s.batch = 1;
+        s.X = d.A.ptr; s.x_rs = d.A.row_stride; s.x_cs = d.A.col_stride; s.x_bs = 0; s.x_bcount = 1;
+        s.W = d.B.ptr; s.w_rs = d.B.row_stride; s.w_cs = d.B.col_stride; s.w_bs = 0; s.w_bcount = 1;
+        s.out = d.C; s.o_rs = d.ldc; s.o_cs = 1; s.o_bs = 0; s.bias = d.bias; s.bias_on_rows = 0;
+        s.epilogue = d.epilogue; s.accumulate = d.accumulate;
+        s.ws = nullptr; s.split_k = 1; s.k_per_slice = s.K; s.groups = 0; s.flags = nullptr; s.epoch = 0; s.max_reducers = 16; s.status = ctx().status_dev;
+        int rc16 = MNI_OK;
+        if (try_gemv_units(s, d, &rc16)) return rc16;
+    }
     const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M > 4 && d.M <= 16 && fewrows_takes(d);
     if (!to_fewrows &&
         ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS ||
@@ -782,8 +808,9 @@ int sgemm(const mni_gemm_desc &d) {
         if (try_skinny(d, &rc)) return rc;
         if (d.algo == MNI_ALGO_GEMV)
             return set_error(MNI_ERR_INVALID,
-                             "sgemm: shape/layout not eligible for the decode product kernel (1 to 8 rows, one batch, row-major 16-byte "
-                             "aligned B and C, N / 128 a multiple of 8 that divides the compute units, K a multiple of 512 slices)");
+                             "sgemm: shape/layout not eligible for the decode product kernel (1 to 16 rows, one batch, row-major 16-byte "
+                             "aligned B and C, N / 128 (N / 64 beyond 8 rows) a multiple of 8 that divides the compute units, K a multiple of "
+                             "512 (1024) slices)");
         if (d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS)
             return set_error(MNI_ERR_INVALID,
                              "sgemm: shape/layout not eligible for the skinny kernels "

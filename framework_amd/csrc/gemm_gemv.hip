@@ -301,4 +301,207 @@ int launch_gemv_units(const GemvLaunch &p, int rows) {
     return check_launch("gemv_units_kernel");
 }
 
+
+// ---- the same product for 9 to 16 rows --------------------------------------------------------------------------
+// What changes against gemv_units_kernel: the accumulators.  With the 4 x 4 x 1 blocks a lane keeps rows x 4 columns
+// of sums (64 registers at 16 rows, next to the 64 its loads are in flight in); v_mfma_f32_16x16x4_f32 keeps a
+// 16 x 16 tile in four registers.  Lane (n = lane & 15, q = lane >> 4) loads 16 bytes of W: row q of the instruction's
+// four, columns 4 n .. 4 n + 3 of the unit's 64 -- 256 contiguous bytes of each of four consecutive rows -- and MFMA j
+// takes component j (lane n stands for column 4 n + j; the result's columns are permuted the same way: register v of
+// accumulators 0..3 is four adjacent columns of row 4 q + v).  A unit is 64 columns, so there are twice the units and
+// half the K slices of the 8-row form; a wavefront owns 64 consecutive rows of K per trip (16 loads of four rows),
+// a workgroup 1024.  X for those rows (16 rows x 64 values, 256 contiguous bytes per row) goes through a
+// wavefront-private piece of LDS, one value per lane and load as the A operand (row n, K row q).  From the LDS sum
+// across the 16 wavefronts on -- 256 summing threads, tagged partial sums, counting in, the last arrival adds -- the
+// code is the 8-row form's.
+static constexpr int GW_UNIT_COLS = 64, GW_WAVE_ROWS = 4 * GV_U, GW_TRIP_ROWS = GV_WAVES * GW_WAVE_ROWS;  // 64 rows per wavefront, 1024 per trip
+static constexpr int GW_XPITCH = GW_WAVE_ROWS + 4;  // floats per row of X in LDS (lanes (n, q) then read 64 different banks)
+static constexpr int GW_PIECES = 16 * 16;           // 16-byte pieces of a workgroup's 16 x 64 tile
+
+template <bool EPI>
+__global__ __launch_bounds__(GV_THREADS) void gemv_units16_kernel(const GemvLaunch p) {
+    constexpr int U = GV_U, SMAX = GEMV_MAX_SLICES;
+    __shared__ __attribute__((aligned(16))) float xs[GV_WAVES][16][GW_XPITCH];
+    __shared__ f32x4 red[GV_WAVES][GW_PIECES];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int id = blockIdx.x;
+    const int unit = id % p.units, slice = id / p.units;
+    const int S = p.slices, trips = p.trips, rows = p.rows;
+    const int n = lane & 15, q = lane >> 4;
+
+    // Everything the end of the kernel needs is fetched from the argument block and worked out now, not after the
+    // last byte of W has arrived.
+    const unsigned epoch = p.epoch;
+    const int tl = tid < GW_PIECES ? tid : 0;  // summing threads: (row tl >> 4, column quad tl & 15)
+    const int64_t slot = GW_PIECES;
+    f32x4 *const unit_a = p.pa + (int64_t)unit * S * slot;
+    f32x2 *const unit_b = p.pb + (int64_t)unit * S * slot;
+    f32x4 *const my_a = unit_a + (int64_t)slice * slot + tl;
+    f32x2 *const my_b = unit_b + (int64_t)slice * slot + tl;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(unit_a, 0, -1, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(unit_b, 0, -1, 0x00020000);
+    unsigned *const my_count = p.count + unit * GEMV_COUNTERS_PER_UNIT + wave;
+    const bool my_row = (tl >> 4) < rows;
+    f32x4 *const my_out = reinterpret_cast<f32x4 *>(p.out + (int64_t)(my_row ? tl >> 4 : 0) * p.o_rs + unit * GW_UNIT_COLS + (tl & 15) * 4);
+    unsigned *const status = p.status;
+    const int epilogue = EPI ? p.epilogue : (int)MNI_EPI_NONE;
+    asm volatile("" ::"v"(my_a), "v"(my_b), "s"(my_count), "v"(my_out), "s"(epoch), "s"(status));
+    // The first slice's partial carries the bias and, when only a sum follows, the old output of an accumulating call.
+    f32x4 extra = {0.f, 0.f, 0.f, 0.f};
+    if (EPI && slice == 0 && tid < GW_PIECES) {
+        if (epilogue != MNI_EPI_NONE) extra = *reinterpret_cast<const f32x4 *>(p.bias + unit * GW_UNIT_COLS + (tl & 15) * 4);
+        if (p.accumulate && my_row) extra += *my_out;
+    }
+
+    f32x4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int64_t w_rs = p.w_rs;
+    const int k0 = slice * trips * GW_TRIP_ROWS + wave * GW_WAVE_ROWS;  // this wavefront's first row of K
+    const float *__restrict__ Wc = p.W + (int64_t)(k0 + q) * w_rs + unit * GW_UNIT_COLS + n * 4;
+    // X: lane (row = lane >> 2, quarter = lane & 3) takes 64 bytes of its row (rows past `rows` repeat the last one: their
+    // sums are never stored), four 16-byte loads
+    const int xr = lane >> 2, xq = lane & 3;
+    const float *__restrict__ xp = p.X + (int64_t)min(xr, rows - 1) * p.x_rs + k0 + 16 * xq;
+    for (int trip = 0; trip < trips; ++trip) {
+        f32x4 xg[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) xg[e] = *reinterpret_cast<const f32x4 *>(xp + 4 * e);
+        __builtin_amdgcn_sched_barrier(0);
+        f32x4 w[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) w[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(Wc + (int64_t)u * 4 * w_rs));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) *reinterpret_cast<f32x4 *>(&xs[wave][xr][16 * xq + 4 * e]) = xg[e];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // same wavefront: its LDS writes are done, no barrier needed
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float a = xs[wave][n][4 * u + q];  // row n of X, the K row of this lane's piece of load u
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, w[u][j], acc[j], 0, 0, 0);
+        }
+        Wc += (int64_t)GW_TRIP_ROWS * w_rs;
+        xp += GW_TRIP_ROWS;
+        // (the next trip overwrites this wavefront's piece of xs: LDS operations of one wavefront complete in order)
+    }
+    // register v of accumulators 0..3 is row 4 q + v, columns 4 n .. 4 n + 3: one 16-byte piece
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][(4 * q + v) * 16 + n] = f32x4{acc[0][v], acc[1][v], acc[2][v], acc[3][v]};
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    if (tid >= GW_PIECES) return;
+
+    // all 16 wavefronts' sums at once, then added in wavefront order
+    f32x4 e[GV_WAVES];
+#pragma unroll
+    for (int w2 = 0; w2 < GV_WAVES; ++w2) e[w2] = red[w2][tid];
+    __builtin_amdgcn_sched_barrier(0);
+    f32x4 t = e[0];
+#pragma unroll
+    for (int w2 = 1; w2 < GV_WAVES; ++w2) t += e[w2];
+    if (EPI) t += extra;
+    auto finish = [&](f32x4 v) {
+        if (EPI) {
+            if (epilogue == MNI_EPI_BIAS_RELU) v = f32x4{fmaxf(v.x, 0.f), fmaxf(v.y, 0.f), fmaxf(v.z, 0.f), fmaxf(v.w, 0.f)};
+            else if (epilogue == MNI_EPI_BIAS_GELU) v = f32x4{gv_gelu(v.x), gv_gelu(v.y), gv_gelu(v.z), gv_gelu(v.w)};
+        }
+        if (my_row) *my_out = v;
+    };
+    if (S == 1) { finish(t); return; }  // (uniform over the grid)
+
+    const float tag = __uint_as_float(epoch);
+    *my_a = f32x4{t.x, t.y, t.z, tag};
+    *my_b = f32x2{t.w, tag};
+    // lane 0 counts the wavefront in; no branch, so nothing waits for the answer here
+    unsigned rank;
+    {
+        unsigned long long saved;
+        asm volatile("s_mov_b64 %1, exec\n\ts_mov_b64 exec, 1\n\tglobal_atomic_inc %0, %2, %3, off sc0\n\ts_mov_b64 exec, %1"
+                     : "=&v"(rank), "=&s"(saved)
+                     : "v"(my_count), "v"(S - 1)
+                     : "memory");
+    }
+    f32x4 a[SMAX];
+    f32x2 b[SMAX];
+    const int other = slice + 1 < S ? slice + 1 : 0;
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) {
+        const unsigned so = (s == slice || s >= S) ? other : s;  // (never the own slot, never past the last)
+        a[s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, tl * 16, so * (GW_PIECES * 16), 0));
+        b[s] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(rb, tl * 8, so * (GW_PIECES * 8), 0));
+    }
+    // Everything asked for above has to be back before the count is looked at (and the requests must not sink below
+    // the branch that follows).
+    static_assert(SMAX == 8, "operand list below");
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(rank), "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]), "+v"(b[0]),
+                   "+v"(b[1]), "+v"(b[2]), "+v"(b[3]), "+v"(b[4]), "+v"(b[5]), "+v"(b[6]), "+v"(b[7])
+                 :
+                 : "memory");
+    rank = __builtin_amdgcn_readfirstlane(rank);
+    if (rank != (unsigned)(S - 1)) return;
+
+    bool ok = false;
+    for (int spin = 0; spin < GV_SPIN_LIMIT; ++spin) {
+        unsigned bad = 0;
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) {
+            const unsigned d = (__float_as_uint(a[s].w) ^ epoch) | (__float_as_uint(b[s].y) ^ epoch);
+            bad |= (s == slice || s >= S) ? 0u : d;
+        }
+        ok = __all(bad == 0);
+        if (ok) break;
+        __builtin_amdgcn_s_sleep(2);
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) {
+            const unsigned so = (s == slice || s >= S) ? other : s;
+            a[s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, tl * 16, so * (GW_PIECES * 16), 16));  // sc1: past this CU's L1
+            b[s] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(rb, tl * 8, so * (GW_PIECES * 8), 16));
+        }
+    }
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) {
+        const f32x4 v = s == slice ? t : f32x4{a[s].x, a[s].y, a[s].z, b[s].x};
+        if (s < S) sum += v;
+    }
+    if (!ok) {
+        // NaN into the output and a code into the status word: the next call that waits for the stream fails with it
+        const float nan = __builtin_nanf("");
+        sum = f32x4{nan, nan, nan, nan};
+        if (lane == 0) *status = DEVICE_STATUS_GEMV_WAIT;
+    }
+    finish(sum);
+}
+
+bool gemv_units16_plan(int rows, int cols, int K, int cus, int xcds, int *slices, int *trips) {
+    if (rows < 1 || rows > 16 || xcds != 8 || cus != 256) return false;
+    if (cols <= 0 || cols % GW_UNIT_COLS != 0) return false;
+    const int units = cols / GW_UNIT_COLS;
+    if (units % xcds != 0 || units > cus || cus % units != 0) return false;
+    const int s = cus / units;  // one workgroup per CU
+    if (s > GEMV_MAX_SLICES) return false;
+    if (K < s * GW_TRIP_ROWS || K % (s * GW_TRIP_ROWS) != 0) return false;
+    *slices = s;
+    *trips = K / (s * GW_TRIP_ROWS);
+    return true;
+}
+
+size_t gemv_units16_partial_slots(int cols, int slices) { return (size_t)(cols / GW_UNIT_COLS) * slices * GW_PIECES; }
+
+int launch_gemv_units16(const GemvLaunch &p) {
+    if (p.units <= 0 || p.units % 8 != 0 || p.slices < 1 || p.slices > GEMV_MAX_SLICES || p.trips < 1 || p.rows < 1 || p.rows > 16 ||
+        (int64_t)p.units * p.slices > 256 || p.w_rs < p.units * GW_UNIT_COLS || p.o_rs < p.units * GW_UNIT_COLS ||
+        (p.rows > 1 && p.x_rs < p.slices * p.trips * GW_TRIP_ROWS))
+        return set_error(MNI_ERR_INVALID, "decode product, 16-row form: bad plan (units %d, slices %d, trips %d, rows %d)", p.units, p.slices, p.trips, p.rows);
+    const dim3 grid((unsigned)(p.units * p.slices)), block(GV_THREADS);
+    hipStream_t st = ctx().stream;
+    if (p.epilogue != MNI_EPI_NONE || p.accumulate) MNI_KERNEL_LAUNCH((gemv_units16_kernel<true>), grid, block, 0, st, p);
+    else MNI_KERNEL_LAUNCH((gemv_units16_kernel<false>), grid, block, 0, st, p);
+    return check_launch("gemv_units16_kernel");
+}
+
 }  // namespace mni

@@ -145,11 +145,16 @@ struct GemvLaunch {
     int units, slices, trips;
     int w_rs, x_rs, o_rs;
     int epilogue, accumulate;
+    int rows;  // (the 16-row form: rows of X that exist; the forms up to 8 rows are compiled per row count)
 };
 // Whether the kernel takes rows x K against K x cols on this device, and with how many K slices / trips per workgroup.
 bool gemv_units_plan(int rows, int cols, int K, int cus, int xcds, int *slices, int *trips);
 size_t gemv_units_partial_slots(int rows, int cols, int slices);  // pieces of pa (and of pb) the plan writes
 int launch_gemv_units(const GemvLaunch &p, int rows);
+// The same for up to 16 rows: units of 64 columns, 1024 rows of K per workgroup and trip.
+bool gemv_units16_plan(int rows, int cols, int K, int cus, int xcds, int *slices, int *trips);
+size_t gemv_units16_partial_slots(int cols, int slices);
+int launch_gemv_units16(const GemvLaunch &p);
 
 // Up to 32 rows against a wide K-contiguous operand (gemm_fewrows_nt.hip): a wavefront per 16 columns and all of K, A in LDS.
 static constexpr int FEWROWS_NT_LDS_FLOATS = 32768;  // 16 (or 32) rows of K + 4 floats

@@ -952,9 +952,86 @@ def test_decode_product_kernel_ineligible_is_an_error_only_when_forced(dev, rocm
     with pytest.raises(N.MniError):
         _gemv_gemm(dev, a, b, algo=N.ALGO_GEMV)
     assert np.array_equal(_gemv_gemm(dev, a, b), want)
-    a9 = synth.small_ints(3, (9, 4096), 3); b9 = synth.small_ints(4, (4096, 4096), 3, stream=1)  # 9 rows
+    a17 = synth.small_ints(3, (17, 4096), 3); b17 = synth.small_ints(4, (4096, 4096), 3, stream=1)  # 17 rows
     with pytest.raises(N.MniError):
-        _gemv_gemm(dev, a9, b9, algo=N.ALGO_GEMV)
+        _gemv_gemm(dev, a17, b17, algo=N.ALGO_GEMV)
+
+
+@pytest.mark.parametrize("m,n,k", [(7, 4096, 4096), (8, 4096, 4096), (4, 8192, 8192), (8, 16384, 1024), (5, 32768, 512)])
+def test_decode_product_both_forms_give_exact_sums(dev, rocm, m, n, k):
+    # from 7 rows, or beyond 4096 columns, the 16-row form is preferred; an X whose pitch is not a whole number of 16-byte
+    # pieces is outside that form and keeps the per-row-count kernels in use for these shapes
+    a = synth.small_ints(m, (m, k), 3)
+    b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(_gemv_gemm(dev, a, b, algo=N.ALGO_GEMV), want)
+    lda = k + 1
+    sa = np.zeros((m, lda), np.float32); sa[:, :k] = a
+    dA, dB, dC = dev.put(sa), dev.put(b), dev.empty(m * n, fill=-7.0)
+    before = rocm.launch_count()
+    rocm.sgemm(m, n, k, dA, dB, dC, a_strides=(lda, 1), algo=N.ALGO_GEMV)
+    assert rocm.launch_count() - before == 1
+    assert np.array_equal(rocm.to_host(dC, (m, n)), want)
+    rocm.sync()
+
+
+@pytest.mark.parametrize("m", [9, 10, 13, 16])
+def test_decode_product_16_row_form_integer_exact(dev, rocm, m):
+    # 4096 x 4096: 64 units of 64 columns x 4 K slices of one trip; forced and as the planner's choice, and repeated
+    a = synth.small_ints(m, (m, 4096), 3)
+    b = synth.small_ints(m + 1, (4096, 4096), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    for algo in (N.ALGO_GEMV, N.ALGO_AUTO, N.ALGO_GEMV):
+        assert np.array_equal(_gemv_gemm(dev, a, b, algo=algo), want), algo
+    rocm.sync()   # (an adding wavefront's expired wait would be reported here)
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 8192, 8192), (12, 16384, 4096), (9, 16384, 1024), (16, 4096, 8192), (11, 2048, 8192), (16, 8192, 2048)])
+def test_decode_product_16_row_form_other_plans_integer_exact(dev, rocm, m, n, k):
+    # 8, 4, 2 slices and none at all (16384 columns: every workgroup owns its columns outright), one and several trips
+    a = synth.small_ints(m, (m, k), 3)
+    b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(_gemv_gemm(dev, a, b, algo=N.ALGO_GEMV), want)
+    assert np.array_equal(_gemv_gemm(dev, a, b), want)  # (the planner's choice, whichever kernel that is)
+    rocm.sync()
+
+
+def test_decode_product_16_row_form_epilogues_accumulate_pitches_and_repeats(dev, rocm):
+    m, n, k = 13, 4096, 4096
+    a = synth.small_ints(m, (m, k), 3); b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+    bias = synth.small_ints(m + 2, (n,), 5, stream=2); old = synth.small_ints(m + 3, (m, n), 9, stream=3)
+    prod = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float64)
+    lda, ldb, ldc = k + 8, n + 12, n + 4
+    sa = np.zeros((m, lda), np.float32); sa[:, :k] = a
+    sb = np.zeros((k, ldb), np.float32); sb[:, :n] = b
+    dA, dB, dBias = dev.put(sa), dev.put(sb), dev.put(bias)
+    for epi, accumulate in [(N.EPI_NONE, False), (N.EPI_NONE, True), (N.EPI_BIAS, False), (N.EPI_BIAS, True), (N.EPI_BIAS_RELU, False),
+                            (N.EPI_BIAS_GELU, False)]:
+        z = prod + (bias if epi != N.EPI_NONE else 0.0)
+        if epi == N.EPI_BIAS_RELU: z = np.maximum(z, 0.0)
+        if epi == N.EPI_BIAS_GELU: z = 0.5 * z * (1.0 + np.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        want = z + (old if accumulate else 0.0)
+        sc = np.full((m, ldc), -5.0, np.float32); sc[:, :n] = old
+        dC = dev.put(sc)
+        rocm.sgemm(m, n, k, dA, dB, dC, a_strides=(lda, 1), b_strides=(ldb, 1), ldc=ldc, bias=dBias if epi != N.EPI_NONE else None, epilogue=epi,
+                   accumulate=accumulate, algo=N.ALGO_GEMV)
+        got = rocm.to_host(dC, (m, ldc))
+        assert np.all(got[:, n:] == -5.0), "the padding of C was written"
+        if epi == N.EPI_BIAS_GELU:
+            assert np.abs(got[:, :n] - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), (epi, accumulate)
+        else:
+            assert np.array_equal(got[:, :n], want.astype(np.float32)), (epi, accumulate)
+    # normal inputs: within tolerance, and the same bits launch after launch
+    an = synth.normal(61, (16, k), 0.02); bn = synth.normal(62, (k, n), 0.02, stream=1)
+    first = _gemv_gemm(dev, an, bn, algo=N.ALGO_GEMV)
+    assert max_err(first, an.astype(np.float64) @ bn.astype(np.float64)) <= gemm_tol(k, an, bn)
+    dA2, dB2 = dev.put(an), dev.put(bn)
+    dC2 = dev.empty(16 * n, fill=-7.0)
+    for _ in range(50):
+        rocm.sgemm(16, n, k, dA2, dB2, dC2, algo=N.ALGO_GEMV)
+    assert np.array_equal(rocm.to_host(dC2, (16, n)), first)
+    rocm.sync()
 
 
 # ---- few rows against a wide K-contiguous operand (a weight stored [out, in]): a wavefront per 16 columns, all of K ----
