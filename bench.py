@@ -262,9 +262,9 @@ def bench_extras(r, with_cpu):
         c5a["cpu_baseline"] = dict(cpu_note("the whole product, best of 3"), value=dt * 1e3, unit="ms", **{"GB/s": by / dt / 1e9})
         orc.native.resetEngine()
     out["config5a_gemv"] = c5a
-    # the same W against batches of token rows (batched decoding): up to 8 rows through the decode kernel (an
-    # instantiation per row count), 16 and 32 through the few-rows MFMA kernel, 64 through the tile kernel; W cold
-    # (eight in rotation) -- not a BASELINE config
+    # the same W against batches of token rows (batched decoding): up to 32 rows through the decode kernel (a form per
+    # row count up to 6 rows, one or two sets of 16 rows on the 16 x 16 x 4 MFMA beyond), 64 through the tile kernel;
+    # W cold (eight in rotation) -- not a BASELINE config
     rows_out = {}
     for mrows in (1, 2, 8, 16, 32, 64):
         xb = r.to_device(synth.normal(5, (mrows, 4096)))

@@ -108,12 +108,12 @@ static int init_device(int device) {
     c.fewrows_counter_cap = 4096;
     MNI_HIP_CHECK(hipMalloc((void **)&c.fewrows_counters, c.fewrows_counter_cap * sizeof(unsigned)));
     MNI_HIP_CHECK(hipMemset(c.fewrows_counters, 0, c.fewrows_counter_cap * sizeof(unsigned)));
-    c.gemv_slot_cap = 256 * 8 * 32;  // one workgroup per CU, 8 rows, 32 column lanes
+    c.gemv_slot_cap = 256 * 512;  // one workgroup per CU, a tile of up to 32 rows x 64 columns (or 8 x 128) in 16-byte pieces
     MNI_HIP_CHECK(hipMalloc(&c.gemv_pa, c.gemv_slot_cap * 16));
     MNI_HIP_CHECK(hipMalloc(&c.gemv_pb, c.gemv_slot_cap * 8));
     MNI_HIP_CHECK(hipMemset(c.gemv_pa, 0, c.gemv_slot_cap * 16));
     MNI_HIP_CHECK(hipMemset(c.gemv_pb, 0, c.gemv_slot_cap * 8));
-    c.gemv_counter_cap = 256 * 4;
+    c.gemv_counter_cap = 256 * 8;
     MNI_HIP_CHECK(hipMalloc((void **)&c.gemv_counters, c.gemv_counter_cap * sizeof(unsigned)));
     MNI_HIP_CHECK(hipMemset(c.gemv_counters, 0, c.gemv_counter_cap * sizeof(unsigned)));
     // Pinned staging slots of upload_small, and one event per slot that says when its transfer has left it.

@@ -74,31 +74,34 @@ static int next_epoch(unsigned *epoch) {
 }
 
 // ---- the decode product ---------------------------------------------------------
-// x[<= 8, K] against a row-major W[K, N] whose column and K extents deal the CUs one workgroup each (gemm_gemv.hip).
+// x[<= 32, K] against a row-major W[K, N] whose column and K extents deal the CUs one workgroup each (gemm_gemv.hip).
 // True when it took the product (errors through *rc).
 static bool try_gemv_units(const SkinnyLaunch &s, const mni_gemm_desc &d, int *rc) {
     DeviceCtx &c = ctx();
     if (d.algo != MNI_ALGO_AUTO && d.algo != MNI_ALGO_GEMV) return false;
-    if (d.split_k > 1 || s.batch != 1 || s.rows > 16 || s.x_cs != 1 || s.w_cs != 1 || s.o_cs != 1) return false;
+    if (d.split_k > 1 || s.batch != 1 || s.rows > 32 || s.x_cs != 1 || s.w_cs != 1 || s.o_cs != 1) return false;
     if ((s.w_rs % 4) != 0 || !aligned16(s.W) || (s.o_rs % 4) != 0 || !aligned16(s.out)) return false;
     if (s.w_rs > 0x7fffffffLL || s.x_rs > 0x7fffffffLL || s.o_rs > 0x7fffffffLL) return false;
     if (s.epilogue > MNI_EPI_BIAS_GELU || s.bias_on_rows) return false;
     if (s.epilogue != MNI_EPI_NONE && !aligned16(s.bias)) return false;
     if (s.accumulate && s.epilogue >= MNI_EPI_BIAS_RELU) return false;  // (the old output would have to wait for the sum)
-    // Two forms.  Up to 8 rows on 4 x 4 x 1 blocks (128-column units, a kernel per row count); up to 16 rows on the
-    // 16 x 16 x 4 MFMA (64-column units, X in 16-byte pieces), whose time does not depend on the row count.  Measured on
-    // MI355X, us, cold W, the first against the second: 4096 x 4096 1 row 12.2 / 13.7, 4 rows 12.8 / 13.8, 6 rows 13.5 / 13.8,
-    // 7 rows 14.3 / 13.8, 8 rows 14.5 / 13.8 (16 rows 14.1: 20.9 through the few-rows kernel); 8192 x 8192 4 rows 51.2 / 42.4
-    // (the column kernel 45.0), 8 rows 52.4 / 43.0; 16384 x 1024 4 rows 13.3 / 12.4, 8 rows 15.0 / 12.6; 4096 x 8192 4 rows
-    // 23.1 / 23.8, 8 rows 24.9 / 24.0.
+    // Two forms.  Up to 8 rows on 4 x 4 x 1 blocks (128-column units, a kernel per row count); up to 32 rows on the
+    // 16 x 16 x 4 MFMA (64-column units, X in 16-byte pieces, one or two sets of 16 rows), whose time depends on the number
+    // of sets only.  Measured on MI355X, us, cold W, the first against the second: 4096 x 4096 1 row 12.2 / 13.7,
+    // 4 rows 12.8 / 13.8, 6 rows 13.5 / 13.8, 7 rows 14.3 / 13.8, 8 rows 14.5 / 13.8 (16 rows 14.1: 20.9 through the
+    // few-rows kernel); 8192 x 8192 4 rows 51.2 / 42.4 (the column kernel 45.0), 8 rows 52.4 / 43.0; 16384 x 1024 4 rows
+    // 13.3 / 12.4, 8 rows 15.0 / 12.6; 4096 x 8192 4 rows 23.1 / 23.8, 8 rows 24.9 / 24.0.
     int slices = 0, trips = 0, slices16 = 0, trips16 = 0;
     const bool narrow_ok = s.rows <= 8 && c.gemv_pa && gemv_units_plan(s.rows, s.cols, s.K, c.compute_units, c.xcd_count, &slices, &trips) &&
                            gemv_units_partial_slots(s.rows, s.cols, slices) <= c.gemv_slot_cap &&
                            (size_t)(s.cols / 128) * GEMV_COUNTERS_PER_UNIT <= c.gemv_counter_cap;
-    const bool wide_ok = c.gemv_pa && (s.x_rs % 4) == 0 && aligned16(s.X) &&
+    const bool wide_ok = c.gemv_pa && (s.x_rs % 4) == 0 && aligned16(s.X) && gemv_units16_pitches_ok(s.w_rs, s.x_rs) &&
                          gemv_units16_plan(s.rows, s.cols, s.K, c.compute_units, c.xcd_count, &slices16, &trips16) &&
-                         gemv_units16_partial_slots(s.cols, slices16) <= c.gemv_slot_cap &&
-                         (size_t)(s.cols / 64) * GEMV_COUNTERS_PER_UNIT <= c.gemv_counter_cap;
+                         gemv_units16_partial_slots(s.rows, s.cols, slices16) <= c.gemv_slot_cap &&
+                         gemv_units16_counters(s.rows, s.cols) <= c.gemv_counter_cap;
+    // Two sets of rows, us against the few-rows MFMA kernel: 32 x 4096 x 4096 16.5 / 21.4, 17 rows 16.0 / 20.9,
+    // 32 x 16384 x 1024 14.7 / 20.6, 32 x 4096 x 8192 28.2 / 33.8, 32 x 8192 x 2048 16.6 / 20.2; 32 x 8192 x 8192 50.4 / 50.0
+    if (s.rows > 16 && d.algo == MNI_ALGO_AUTO && (int64_t)s.cols * s.K >= (1LL << 26)) return false;
     const bool prefer_wide = s.rows > 6 || s.cols > 4096;
     const bool wide = wide_ok && (prefer_wide || !narrow_ok);
     if (!wide && !narrow_ok) return false;
@@ -788,8 +791,10 @@ int sgemm(const mni_gemm_desc &d) {
     // 9 to 16 rows against a wide N-contiguous operand: the few-rows MFMA kernel is level with or ahead of the skinny
     // kernel's 16-row forms (us, few-rows against skinny: 16 x 4096 x 4096 18.6 / 21.5, 12 rows 18.6 / 30.5,
     // 16 x 8192 x 8192 46 / 58, 16 x 1024 x 1024 8.5 / 8.4; at 8 rows the skinny kernel leads, 15.2 / 18.6)
-    // 9 to 16 rows of the decode shape: the 16-row form of the decode product ahead of the few-rows kernel
-    if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M > 8 && d.M <= 16 && d.batch == 1 && d.K > 0 && d.epilogue <= MNI_EPI_BIAS_GELU) {
+    // 9 to 32 rows of the decode shape come first: there the 16 x 16 x 4 form of the decode product is ahead of both
+    // (16 x 4096 x 4096 14.1 us, 32 rows 16.5)
+    if ((d.algo == MNI_ALGO_AUTO || d.algo == MNI_ALGO_GEMV) && d.split_k == 0 && d.M > 8 && d.M <= 32 && d.batch == 1 && d.K > 0 &&
+        d.epilogue <= MNI_EPI_BIAS_GELU) {
         SkinnyLaunch s;
         s.rows = (int)d.M; s.cols = (int)d.N; s.K = (int)d.K; s.batch = 1;
         s.X = d.A.ptr; s.x_rs = d.A.row_stride; s.x_cs = d.A.col_stride; s.x_bs = 0; s.x_bcount = 1;
@@ -808,9 +813,9 @@ int sgemm(const mni_gemm_desc &d) {
         if (try_skinny(d, &rc)) return rc;
         if (d.algo == MNI_ALGO_GEMV)
             return set_error(MNI_ERR_INVALID,
-                             "sgemm: shape/layout not eligible for the decode product kernel (1 to 16 rows, one batch, row-major 16-byte "
-                             "aligned B and C, N / 128 (N / 64 beyond 8 rows) a multiple of 8 that divides the compute units, K a multiple of "
-                             "512 (1024) slices)");
+                             "sgemm: shape/layout not eligible for the decode product kernel (1 to 32 rows, one batch, row-major 16-byte "
+                             "aligned B and C, N / 128 (N / 64 beyond 8 rows, with a 16-byte aligned A) a multiple of 8 that divides the "
+                             "compute units, K a multiple of 512 (1024) times the compute units left per unit of columns)");
         if (d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS)
             return set_error(MNI_ERR_INVALID,
                              "sgemm: shape/layout not eligible for the skinny kernels "

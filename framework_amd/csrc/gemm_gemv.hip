@@ -302,7 +302,7 @@ int launch_gemv_units(const GemvLaunch &p, int rows) {
 }
 
 
-// ---- the same product for 9 to 16 rows --------------------------------------------------------------------------
+// ---- the same product for up to 32 rows -------------------------------------------------------------------------
 // What changes against gemv_units_kernel: the accumulators.  With the 4 x 4 x 1 blocks a lane keeps rows x 4 columns
 // of sums (64 registers at 16 rows, next to the 64 its loads are in flight in); v_mfma_f32_16x16x4_f32 keeps a
 // 16 x 16 tile in four registers.  Lane (n = lane & 15, q = lane >> 4) loads 16 bytes of W: row q of the instruction's
@@ -310,21 +310,31 @@ int launch_gemv_units(const GemvLaunch &p, int rows) {
 // takes component j (lane n stands for column 4 n + j; the result's columns are permuted the same way: register v of
 // accumulators 0..3 is four adjacent columns of row 4 q + v).  A unit is 64 columns, so there are twice the units and
 // half the K slices of the 8-row form; a wavefront owns 64 consecutive rows of K per trip (16 loads of four rows),
-// a workgroup 1024.  X for those rows (16 rows x 64 values, 256 contiguous bytes per row) goes through a
-// wavefront-private piece of LDS, one value per lane and load as the A operand (row n, K row q).  From the LDS sum
-// across the 16 wavefronts on -- 256 summing threads, tagged partial sums, counting in, the last arrival adds -- the
-// code is the 8-row form's.
+// a workgroup 1024.  X for those rows (16 or 32 rows x 64 values, 256 contiguous bytes per row) is loaded straight into
+// a wavefront-private piece of LDS, and read from there one value per lane and load as the A operand (row n, K row q);
+// with 17 to 32 rows every load of W is multiplied with two sets of 16 rows (eight MFMAs instead of four).  From the
+// LDS sum across the 16 wavefronts on -- 256 summing threads per set, tagged partial sums, counting in, the last
+// arrival adds -- the code is the 8-row form's.
 static constexpr int GW_UNIT_COLS = 64, GW_WAVE_ROWS = 4 * GV_U, GW_TRIP_ROWS = GV_WAVES * GW_WAVE_ROWS;  // 64 rows per wavefront, 1024 per trip
-static constexpr int GW_XPITCH = GW_WAVE_ROWS + 4;  // floats per row of X in LDS (lanes (n, q) then read 64 different banks)
-static constexpr int GW_PIECES = 16 * 16;           // 16-byte pieces of a workgroup's 16 x 64 tile
+static constexpr int GW_PIECES = 16 * 16;  // 16-byte pieces of a 16 x 64 tile
+// pitch of X (floats) up to which the byte offsets of its buffer loads, 124 x_rs + 240 at most, stay below 2^31
+static constexpr int GW_MAX_X_PITCH = 1 << 24;
 
-template <bool EPI>
+// SETS: sets of 16 rows (1: up to 16 rows, 2: up to 32 -- the same loads of W multiplied with two sets of rows of X)
+template <int SETS, bool EPI>
 __global__ __launch_bounds__(GV_THREADS) void gemv_units16_kernel(const GemvLaunch p) {
     constexpr int U = GV_U, SMAX = GEMV_MAX_SLICES;
-    __shared__ __attribute__((aligned(16))) float xs[GV_WAVES][16][GW_XPITCH];
-    __shared__ f32x4 red[GV_WAVES][GW_PIECES];
+    constexpr int XROWS = 16 * SETS, PIECES = GW_PIECES * SETS, NCOUNT = GEMV_COUNTERS_PER_UNIT * SETS;
+    constexpr int XS_BYTES = GV_WAVES * XROWS * GW_WAVE_ROWS * 4, RED_BYTES = GV_WAVES * PIECES * 16;
+    static_assert(U == 16, "the wait for X below counts the loads of W behind it");
+    // X during the loop, the wavefronts' tiles after it: the same piece of LDS.  A wavefront's tile is as large as its X
+    // and takes its place, so no wavefront writes where another still reads.
+    static_assert(XS_BYTES == RED_BYTES, "a wavefront's tile goes where its X was");
+    __shared__ __attribute__((aligned(1024))) char lds[XS_BYTES];
+    f32x4(*red)[PIECES] = reinterpret_cast<f32x4(*)[PIECES]>(lds);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    float *const xs = reinterpret_cast<float *>(lds) + wave * (XROWS * GW_WAVE_ROWS);  // this wavefront's XROWS x 64 values of X
     const int id = blockIdx.x;
     const int unit = id % p.units, slice = id / p.units;
     const int S = p.slices, trips = p.trips, rows = p.rows;
@@ -333,67 +343,98 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_units16_kernel(const GemvLaun
     // Everything the end of the kernel needs is fetched from the argument block and worked out now, not after the
     // last byte of W has arrived.
     const unsigned epoch = p.epoch;
-    const int tl = tid < GW_PIECES ? tid : 0;  // summing threads: (row tl >> 4, column quad tl & 15)
-    const int64_t slot = GW_PIECES;
+    const int tl = tid < PIECES ? tid : 0;  // summing threads: (row tl >> 4, column quad tl & 15)
+    const int64_t slot = PIECES;
     f32x4 *const unit_a = p.pa + (int64_t)unit * S * slot;
     f32x2 *const unit_b = p.pb + (int64_t)unit * S * slot;
     f32x4 *const my_a = unit_a + (int64_t)slice * slot + tl;
     f32x2 *const my_b = unit_b + (int64_t)slice * slot + tl;
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(unit_a, 0, -1, 0x00020000);
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(unit_b, 0, -1, 0x00020000);
-    unsigned *const my_count = p.count + unit * GEMV_COUNTERS_PER_UNIT + wave;
+    unsigned *const my_count = p.count + unit * NCOUNT + wave;
     const bool my_row = (tl >> 4) < rows;
     f32x4 *const my_out = reinterpret_cast<f32x4 *>(p.out + (int64_t)(my_row ? tl >> 4 : 0) * p.o_rs + unit * GW_UNIT_COLS + (tl & 15) * 4);
     unsigned *const status = p.status;
     const int epilogue = EPI ? p.epilogue : (int)MNI_EPI_NONE;
-    asm volatile("" ::"v"(my_a), "v"(my_b), "s"(my_count), "v"(my_out), "s"(epoch), "s"(status));
+    // (with two sets of rows the loop takes every register: there the per-lane addresses are worked out after it)
+    if (SETS == 1) asm volatile("" ::"v"(my_a), "v"(my_b), "s"(my_count), "v"(my_out), "s"(epoch), "s"(status));
+    else asm volatile("" ::"s"(my_count), "s"(epoch), "s"(status));
     // The first slice's partial carries the bias and, when only a sum follows, the old output of an accumulating call.
     f32x4 extra = {0.f, 0.f, 0.f, 0.f};
-    if (EPI && slice == 0 && tid < GW_PIECES) {
-        if (epilogue != MNI_EPI_NONE) extra = *reinterpret_cast<const f32x4 *>(p.bias + unit * GW_UNIT_COLS + (tl & 15) * 4);
-        if (p.accumulate && my_row) extra += *my_out;
-    }
+    auto fetch_extra = [&]() {
+        if (EPI && slice == 0 && tid < PIECES) {
+            if (epilogue != MNI_EPI_NONE) extra = *reinterpret_cast<const f32x4 *>(p.bias + unit * GW_UNIT_COLS + (tl & 15) * 4);
+            if (p.accumulate && my_row) extra += *my_out;
+        }
+    };
+    if (SETS == 1) fetch_extra();
 
-    f32x4 acc[4];
+    f32x4 acc[SETS][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < SETS; ++s)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[s][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int64_t w_rs = p.w_rs;
     const int k0 = slice * trips * GW_TRIP_ROWS + wave * GW_WAVE_ROWS;  // this wavefront's first row of K
-    const float *__restrict__ Wc = p.W + (int64_t)(k0 + q) * w_rs + unit * GW_UNIT_COLS + n * 4;
-    // X: lane (row = lane >> 2, quarter = lane & 3) takes 64 bytes of its row (rows past `rows` repeat the last one: their
-    // sums are never stored), four 16-byte loads
-    const int xr = lane >> 2, xq = lane & 3;
-    const float *__restrict__ xp = p.X + (int64_t)min(xr, rows - 1) * p.x_rs + k0 + 16 * xq;
-    for (int trip = 0; trip < trips; ++trip) {
-        f32x4 xg[4];
+    // W: an address per lane for the first load and a byte step that is the same for all lanes (plain loads: the same
+    // loads as buffer loads with scalar offsets cost half a microsecond more on a one-trip product, 14.5 against 14.0 us
+    // at 16 x 4096 x 4096, and gain as much on 16 x 8192 x 8192, 43.3 against 43.9)
+    const char *Wk = reinterpret_cast<const char *>(p.W + (int64_t)(k0 + q) * w_rs + unit * GW_UNIT_COLS + n * 4);
+    // X goes from memory straight into LDS, a load instruction per four rows: lane (q, n) brings a 16-byte piece of row
+    // 4 e + q and the hardware puts the wavefront's 64 pieces side by side in lane order, 256 bytes per row.  Which piece
+    // of its row a lane brings is its n xor-ed with the row's number within the set: piece u of row r then sits at place
+    // u ^ r, and the sixteen lanes that read the same u of sixteen rows (the A operand below) hit sixteen different groups
+    // of four banks.  Rows past `rows` repeat the last one: their sums are never stored.
+    const char *Xk = reinterpret_cast<const char *>(p.X + k0);
+    int xoff[4 * SETS];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) xg[e] = *reinterpret_cast<const f32x4 *>(xp + 4 * e);
+    for (int e = 0; e < 4 * SETS; ++e) {
+        const int row = 4 * e + q;
+        xoff[e] = (min(row, rows - 1) * p.x_rs + 4 * (n ^ (row & 15))) * 4;
+    }
+    const int a_idx = n * GW_WAVE_ROWS + q, n4 = 4 * n;  // (row n of a set, K row q of a load's four)
+    for (int trip = 0; trip < trips; ++trip) {
+        const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(Xk), 0, -1, 0x00020000);
+        // X goes out ahead of W: it is wanted first, and loads complete in the order of issue.  (The cast: with an element
+        // of an array of template-dependent size as the argument, the host pass drops the kernel's launch stub.)
+#pragma unroll
+        for (int e = 0; e < 4 * SETS; ++e)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void *)(xs + 256 * e), 16, static_cast<int>(xoff[e]), 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         f32x4 w[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) w[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(Wc + (int64_t)u * 4 * w_rs));
+        for (int u = 0; u < U; ++u) w[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(Wk + (int64_t)u * 16 * w_rs));
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) *reinterpret_cast<f32x4 *>(&xs[wave][xr][16 * xq + 4 * e]) = xg[e];
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // same wavefront: its LDS writes are done, no barrier needed
+        // X is in LDS when no more than the 16 loads of W are outstanding (the compiler does not know that the loads
+        // into LDS and the reads below touch the same bytes)
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const float a = xs[wave][n][4 * u + q];  // row n of X, the K row of this lane's piece of load u
+            // K row 4 u + q of this trip is value q of piece u: place u ^ n of row n
+            float a[SETS];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, w[u][j], acc[j], 0, 0, 0);
+            for (int s = 0; s < SETS; ++s) a[s] = xs[s * 16 * GW_WAVE_ROWS + a_idx + ((4 * u) ^ n4)];
+#pragma unroll
+            for (int s = 0; s < SETS; ++s)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[s][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s], w[u][j], acc[s][j], 0, 0, 0);
         }
-        Wc += (int64_t)GW_TRIP_ROWS * w_rs;
-        xp += GW_TRIP_ROWS;
-        // (the next trip overwrites this wavefront's piece of xs: LDS operations of one wavefront complete in order)
+        Wk += (int64_t)GW_TRIP_ROWS * 4 * w_rs;
+        Xk += GW_TRIP_ROWS * 4;
+        // the next trip's X overwrites this one's: every read of it has to be back first
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
     }
-    // register v of accumulators 0..3 is row 4 q + v, columns 4 n .. 4 n + 3: one 16-byte piece
+    if (SETS > 1) fetch_extra();  // (back by the time the LDS sum is done)
+    // register v of accumulators 0..3 is row 16 s + 4 q + v, columns 4 n .. 4 n + 3: one 16-byte piece
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][(4 * q + v) * 16 + n] = f32x4{acc[0][v], acc[1][v], acc[2][v], acc[3][v]};
+    for (int s = 0; s < SETS; ++s)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][(16 * s + 4 * q + v) * 16 + n] = f32x4{acc[s][0][v], acc[s][1][v], acc[s][2][v], acc[s][3][v]};
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-    if (tid >= GW_PIECES) return;
-
+    if (tid >= PIECES) return;
     // all 16 wavefronts' sums at once, then added in wavefront order
     f32x4 e[GV_WAVES];
 #pragma unroll
@@ -430,8 +471,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_units16_kernel(const GemvLaun
 #pragma unroll
     for (int s = 0; s < SMAX; ++s) {
         const unsigned so = (s == slice || s >= S) ? other : s;  // (never the own slot, never past the last)
-        a[s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, tl * 16, so * (GW_PIECES * 16), 0));
-        b[s] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(rb, tl * 8, so * (GW_PIECES * 8), 0));
+        a[s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, tl * 16, so * (PIECES * 16), 0));
+        b[s] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(rb, tl * 8, so * (PIECES * 8), 0));
     }
     // Everything asked for above has to be back before the count is looked at (and the requests must not sink below
     // the branch that follows).
@@ -458,8 +499,8 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_units16_kernel(const GemvLaun
 #pragma unroll
         for (int s = 0; s < SMAX; ++s) {
             const unsigned so = (s == slice || s >= S) ? other : s;
-            a[s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, tl * 16, so * (GW_PIECES * 16), 16));  // sc1: past this CU's L1
-            b[s] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(rb, tl * 8, so * (GW_PIECES * 8), 16));
+            a[s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, tl * 16, so * (PIECES * 16), 16));  // sc1: past this CU's L1
+            b[s] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(rb, tl * 8, so * (PIECES * 8), 16));
         }
     }
     f32x4 sum = {0.f, 0.f, 0.f, 0.f};
@@ -477,8 +518,10 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_units16_kernel(const GemvLaun
     finish(sum);
 }
 
+bool gemv_units16_pitches_ok(int64_t w_rs, int64_t x_rs) { return w_rs > 0 && w_rs <= 0x7fffffffLL && x_rs >= 0 && x_rs <= GW_MAX_X_PITCH; }
+
 bool gemv_units16_plan(int rows, int cols, int K, int cus, int xcds, int *slices, int *trips) {
-    if (rows < 1 || rows > 16 || xcds != 8 || cus != 256) return false;
+    if (rows < 1 || rows > 32 || xcds != 8 || cus != 256) return false;
     if (cols <= 0 || cols % GW_UNIT_COLS != 0) return false;
     const int units = cols / GW_UNIT_COLS;
     if (units % xcds != 0 || units > cus || cus % units != 0) return false;
@@ -490,17 +533,25 @@ bool gemv_units16_plan(int rows, int cols, int K, int cus, int xcds, int *slices
     return true;
 }
 
-size_t gemv_units16_partial_slots(int cols, int slices) { return (size_t)(cols / GW_UNIT_COLS) * slices * GW_PIECES; }
+size_t gemv_units16_partial_slots(int rows, int cols, int slices) { return (size_t)(cols / GW_UNIT_COLS) * slices * GW_PIECES * (rows > 16 ? 2 : 1); }
+size_t gemv_units16_counters(int rows, int cols) { return (size_t)(cols / GW_UNIT_COLS) * GEMV_COUNTERS_PER_UNIT * (rows > 16 ? 2 : 1); }
 
 int launch_gemv_units16(const GemvLaunch &p) {
-    if (p.units <= 0 || p.units % 8 != 0 || p.slices < 1 || p.slices > GEMV_MAX_SLICES || p.trips < 1 || p.rows < 1 || p.rows > 16 ||
+    if (p.units <= 0 || p.units % 8 != 0 || p.slices < 1 || p.slices > GEMV_MAX_SLICES || p.trips < 1 || p.rows < 1 || p.rows > 32 ||
         (int64_t)p.units * p.slices > 256 || p.w_rs < p.units * GW_UNIT_COLS || p.o_rs < p.units * GW_UNIT_COLS ||
-        (p.rows > 1 && p.x_rs < p.slices * p.trips * GW_TRIP_ROWS))
+        (p.rows > 1 && p.x_rs < p.slices * p.trips * GW_TRIP_ROWS) || p.x_rs > GW_MAX_X_PITCH || p.x_rs < 0 ||
+        (p.x_rs % 4) != 0 || ((uintptr_t)p.X & 15) != 0 || ((uintptr_t)p.W & 15) != 0 || (p.w_rs % 4) != 0)
         return set_error(MNI_ERR_INVALID, "decode product, 16-row form: bad plan (units %d, slices %d, trips %d, rows %d)", p.units, p.slices, p.trips, p.rows);
     const dim3 grid((unsigned)(p.units * p.slices)), block(GV_THREADS);
     hipStream_t st = ctx().stream;
-    if (p.epilogue != MNI_EPI_NONE || p.accumulate) MNI_KERNEL_LAUNCH((gemv_units16_kernel<true>), grid, block, 0, st, p);
-    else MNI_KERNEL_LAUNCH((gemv_units16_kernel<false>), grid, block, 0, st, p);
+    const bool epi = p.epilogue != MNI_EPI_NONE || p.accumulate;
+    if (p.rows > 16) {
+        if (epi) MNI_KERNEL_LAUNCH((gemv_units16_kernel<2, true>), grid, block, 0, st, p);
+        else MNI_KERNEL_LAUNCH((gemv_units16_kernel<2, false>), grid, block, 0, st, p);
+    } else {
+        if (epi) MNI_KERNEL_LAUNCH((gemv_units16_kernel<1, true>), grid, block, 0, st, p);
+        else MNI_KERNEL_LAUNCH((gemv_units16_kernel<1, false>), grid, block, 0, st, p);
+    }
     return check_launch("gemv_units16_kernel");
 }
 

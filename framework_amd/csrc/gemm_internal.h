@@ -151,9 +151,11 @@ struct GemvLaunch {
 bool gemv_units_plan(int rows, int cols, int K, int cus, int xcds, int *slices, int *trips);
 size_t gemv_units_partial_slots(int rows, int cols, int slices);  // pieces of pa (and of pb) the plan writes
 int launch_gemv_units(const GemvLaunch &p, int rows);
-// The same for up to 16 rows: units of 64 columns, 1024 rows of K per workgroup and trip.
+// The same for up to 32 rows (two sets of 16): units of 64 columns, 1024 rows of K per workgroup and trip.
 bool gemv_units16_plan(int rows, int cols, int K, int cus, int xcds, int *slices, int *trips);
-size_t gemv_units16_partial_slots(int cols, int slices);
+size_t gemv_units16_partial_slots(int rows, int cols, int slices);
+bool gemv_units16_pitches_ok(int64_t w_rs, int64_t x_rs);  // the kernel's 32-bit byte offsets hold for these pitches
+size_t gemv_units16_counters(int rows, int cols);  // counters the plan uses (one per summing wavefront and unit)
 int launch_gemv_units16(const GemvLaunch &p);
 
 // Up to 32 rows against a wide K-contiguous operand (gemm_fewrows_nt.hip): a wavefront per 16 columns and all of K, A in LDS.

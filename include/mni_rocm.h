@@ -142,14 +142,18 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * X^T dY of a small batch: both operands straight into the matrix
  * instruction's registers, the cost of writing C (error unless N % 4 == 0,
  * B and C 16-byte aligned with row strides in whole 16 bytes, no epilogue;
- * accumulate is honoured); GEMV = the decode product, 1 to 8 rows of a
+ * accumulate is honoured); GEMV = the decode product, 1 to 32 rows of a
  * K-contiguous A against a row-major B that is as large as the product is
- * expensive: one workgroup per compute unit, 128 columns and a K slice each,
- * the K slices summed inside the launch by whichever wavefront arrives last
- * (error unless one batch, N % 128 == 0 with N / 128 a divisor of the 256
- * compute units and a multiple of 8, K a multiple of 512 * 256 / (N / 128),
- * B, C and the bias 16-byte aligned with row strides in whole 16 bytes, and
- * no activation together with accumulate); FEWROWS_NT = up to 32 rows of a
+ * expensive: one workgroup per compute unit, a unit of columns and a K slice
+ * each, the K slices summed inside the launch by whichever wavefront arrives
+ * last.  Two forms: units of 128 columns for 1 to 8 rows, units of 64 for
+ * up to 32 rows (A 16-byte aligned with a row stride in whole 16 bytes);
+ * where both fit, the faster one is taken.  (Error unless one batch, N a
+ * multiple of the unit with N / unit a divisor of the 256 compute units and
+ * a multiple of 8, K a multiple of 512 (units of 128) or 1024 (units of 64)
+ * times 256 / (N / unit), B, C and the bias 16-byte aligned with row strides
+ * in whole 16 bytes, and no activation together with accumulate);
+ * FEWROWS_NT = up to 32 rows of a
  * K-contiguous A against a wide B that is K-contiguous too (a weight stored
  * [out, in], given as its transposed view): a wavefront per 16 columns and
  * all of K on the 16 x 16 x 4 MFMA, A resident in LDS, no sums across

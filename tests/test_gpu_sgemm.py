@@ -952,9 +952,9 @@ def test_decode_product_kernel_ineligible_is_an_error_only_when_forced(dev, rocm
     with pytest.raises(N.MniError):
         _gemv_gemm(dev, a, b, algo=N.ALGO_GEMV)
     assert np.array_equal(_gemv_gemm(dev, a, b), want)
-    a17 = synth.small_ints(3, (17, 4096), 3); b17 = synth.small_ints(4, (4096, 4096), 3, stream=1)  # 17 rows
+    a33 = synth.small_ints(3, (33, 4096), 3); b33 = synth.small_ints(4, (4096, 4096), 3, stream=1)  # 33 rows
     with pytest.raises(N.MniError):
-        _gemv_gemm(dev, a17, b17, algo=N.ALGO_GEMV)
+        _gemv_gemm(dev, a33, b33, algo=N.ALGO_GEMV)
 
 
 @pytest.mark.parametrize("m,n,k", [(7, 4096, 4096), (8, 4096, 4096), (4, 8192, 8192), (8, 16384, 1024), (5, 32768, 512)])
@@ -1031,6 +1031,59 @@ def test_decode_product_16_row_form_epilogues_accumulate_pitches_and_repeats(dev
     for _ in range(50):
         rocm.sgemm(16, n, k, dA2, dB2, dC2, algo=N.ALGO_GEMV)
     assert np.array_equal(rocm.to_host(dC2, (16, n)), first)
+    rocm.sync()
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 4096, 4096), (32, 4096, 4096), (24, 4096, 4096), (32, 8192, 8192), (20, 16384, 1024), (31, 16384, 4096),
+                                   (32, 2048, 8192), (19, 8192, 2048), (32, 4096, 16384)])
+def test_decode_product_two_sets_of_rows_integer_exact(dev, rocm, m, n, k):
+    # 17 to 32 rows: the same loads of W multiplied with two sets of 16 rows; 8, 4, 2 slices and none, one and several trips
+    a = synth.small_ints(m, (m, k), 3)
+    b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    for algo in (N.ALGO_GEMV, N.ALGO_AUTO, N.ALGO_GEMV):
+        assert np.array_equal(_gemv_gemm(dev, a, b, algo=algo), want), algo
+    rocm.sync()
+
+
+def test_decode_product_two_sets_of_rows_epilogues_accumulate_pitches_and_repeats(dev, rocm):
+    m, n, k = 27, 4096, 4096
+    a = synth.small_ints(m, (m, k), 3); b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+    bias = synth.small_ints(m + 2, (n,), 5, stream=2); old = synth.small_ints(m + 3, (m, n), 9, stream=3)
+    prod = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float64)
+    lda, ldb, ldc = k + 8, n + 12, n + 4
+    sa = np.zeros((m, lda), np.float32); sa[:, :k] = a
+    sb = np.zeros((k, ldb), np.float32); sb[:, :n] = b
+    dA, dB, dBias = dev.put(sa), dev.put(sb), dev.put(bias)
+    for epi, accumulate in [(N.EPI_NONE, False), (N.EPI_NONE, True), (N.EPI_BIAS, False), (N.EPI_BIAS, True), (N.EPI_BIAS_RELU, False),
+                            (N.EPI_BIAS_GELU, False)]:
+        z = prod + (bias if epi != N.EPI_NONE else 0.0)
+        if epi == N.EPI_BIAS_RELU: z = np.maximum(z, 0.0)
+        if epi == N.EPI_BIAS_GELU: z = 0.5 * z * (1.0 + np.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        want = z + (old if accumulate else 0.0)
+        sc = np.full((m, ldc), -5.0, np.float32); sc[:, :n] = old
+        dC = dev.put(sc)
+        rocm.sgemm(m, n, k, dA, dB, dC, a_strides=(lda, 1), b_strides=(ldb, 1), ldc=ldc, bias=dBias if epi != N.EPI_NONE else None, epilogue=epi,
+                   accumulate=accumulate, algo=N.ALGO_GEMV)
+        got = rocm.to_host(dC, (m, ldc))
+        assert np.all(got[:, n:] == -5.0), "the padding of C was written"
+        if epi == N.EPI_BIAS_GELU:
+            assert np.abs(got[:, :n] - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), (epi, accumulate)
+        else:
+            assert np.array_equal(got[:, :n], want.astype(np.float32)), (epi, accumulate)
+    # normal inputs: within tolerance, the same bits launch after launch, also with other decode launches in between
+    an = synth.normal(71, (32, k), 0.02); bn = synth.normal(72, (k, n), 0.02, stream=1)
+    first = _gemv_gemm(dev, an, bn, algo=N.ALGO_GEMV)
+    assert max_err(first, an.astype(np.float64) @ bn.astype(np.float64)) <= gemm_tol(k, an, bn)
+    dA2, dB2 = dev.put(an), dev.put(bn)
+    dC2 = dev.empty(32 * n, fill=-7.0)
+    dC4 = dev.empty(4 * n, fill=-7.0)
+    for i in range(50):
+        rocm.sgemm(32, n, k, dA2, dB2, dC2, algo=N.ALGO_GEMV)
+        if i % 3 == 0: rocm.sgemm(4, n, k, dA2, dB2, dC4, algo=N.ALGO_GEMV)   # (the other forms share the partial sums' buffer)
+        if i % 5 == 0: rocm.sgemm(16, n, k, dA2, dB2, dC2, algo=N.ALGO_GEMV)
+    rocm.sgemm(32, n, k, dA2, dB2, dC2, algo=N.ALGO_GEMV)
+    assert np.array_equal(rocm.to_host(dC2, (32, n)), first)
     rocm.sync()
 
 
