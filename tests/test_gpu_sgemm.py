@@ -1087,6 +1087,26 @@ def test_decode_product_two_sets_of_rows_epilogues_accumulate_pitches_and_repeat
     rocm.sync()
 
 
+@pytest.mark.parametrize("m", [12, 29])
+def test_decode_product_16_row_forms_take_operands_off_a_128_byte_boundary(dev, rocm, m):
+    # X, W and C 16 bytes (X: 48) past a 128-byte boundary, as rows of a larger tensor are: the loads of X into LDS then start in
+    # the middle of a cache line; several trips and K slices (8192 x 8192: 2 slices of 4 trips)
+    for n, k in ((4096, 4096), (8192, 8192)):
+        a = synth.small_ints(m, (m, k), 3); b = synth.small_ints(m + 1, (k, n), 3, stream=1)
+        want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+        fa = np.zeros(m * k + 12, np.float32); fa[12:] = a.ravel()
+        fb = np.zeros(k * n + 4, np.float32); fb[4:] = b.ravel()
+        dA, dB = dev.put(fa), dev.put(fb)
+        dC = dev.empty(m * n + 4, fill=-7.0)
+        before = rocm.launch_count()
+        rocm.sgemm(m, n, k, dA + 4 * 12, dB + 4 * 4, dC + 4 * 4, algo=N.ALGO_GEMV)
+        assert rocm.launch_count() - before == 1
+        got = rocm.to_host(dC, (m * n + 4,))
+        assert np.all(got[:4] == -7.0)
+        assert np.array_equal(got[4:].reshape(m, n), want)
+    rocm.sync()
+
+
 # ---- few rows against a wide K-contiguous operand (a weight stored [out, in]): a wavefront per 16 columns, all of K ----
 @pytest.mark.parametrize("m,n,k", [(16, 50304, 768), (9, 20000, 256), (32, 16400, 512), (17, 16384, 960), (12, 33000, 1984), (1, 4096, 64),
                                    (8, 1000, 128), (32, 70, 320), (16, 16, 1984), (5, 4099, 768), (3, 9001, 512), (8, 16384, 768)])
