@@ -410,6 +410,16 @@ def bench_extras(r, with_cpu):
             api.native.gcTensors(keep())
         return total * 1e3 / n, launches
 
+    def time_steps_back_to_back(step, keep, n):
+        """n steps issued one after the other (the bookkeeping between them included), one wait at the end."""
+        r.sync()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            step()
+            api.native.gcTensors(keep())
+        r.sync()
+        return (time.perf_counter() - t0) * 1e3 / n
+
     # config 4: FFN step X[4096,1024] -> 4096 (GELU) -> 1024, reference mseLoss, fwd + bwd
     d, h, rows = 1024, 4096, 4096
     x4, t4 = synth.normal(3, (rows, d)), synth.normal(3, (rows, d), stream=3)
@@ -437,8 +447,9 @@ def bench_extras(r, with_cpu):
                     ids.append(g)
             return ids
         ms, launches = time_step(step4, keep4, 20, 15)  # 30 ms of warm-up: the clocks take tens of milliseconds to settle after an idle spell
+        ms_loop = time_steps_back_to_back(step4, keep4, 15)
         out["config4_ffn_step" + ("_fused_linear" if fused else "")] = {
-            "ms": ms, "launches_per_step": launches,
+            "ms": ms, "launches_per_step": launches, "ms_in_a_loop_without_waits": ms_loop,
             "roofline": dict(roofline("mfma", "whole step (six gemm_mfma_kernel launches + elementwise)", ms * 1e-3, gemm_flops, gemm_bytes),
                              note="flops and bytes of the six products only; the step's elementwise kernels add ~0.7 GB of traffic and no counted flops")}
     if with_cpu:
@@ -585,6 +596,7 @@ def split_extras(out):
         ex["config3"]["cpu_baseline"] = brief_cpu(c3["cpu_baseline"])
     c4f, c4 = out.pop("config4_ffn_step_fused_linear"), out.pop("config4_ffn_step")
     ex["config4"] = brief(c4f["roofline"], ms=c4f["ms"], launches_per_step=c4f["launches_per_step"], kernel="whole step, fused Linear + GELU epilogues: six products + elementwise",
+                          ms_in_a_loop_without_waits=c4f["ms_in_a_loop_without_waits"],
                           composed=sig({"ms": c4["ms"], "frac": c4["roofline"]["frac"], "launches_per_step": c4["launches_per_step"]}))
     if "cpu_baseline" in c4:
         ex["config4"]["cpu_baseline"] = brief_cpu(c4["cpu_baseline"])
