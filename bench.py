@@ -450,7 +450,8 @@ def bench_extras(r, with_cpu):
         ms_loop = time_steps_back_to_back(step4, keep4, 15)
         out["config4_ffn_step" + ("_fused_linear" if fused else "")] = {
             "ms": ms, "launches_per_step": launches, "ms_in_a_loop_without_waits": ms_loop,
-            "roofline": dict(roofline("mfma", "whole step (six gemm_mfma_kernel launches + elementwise)", ms * 1e-3, gemm_flops, gemm_bytes),
+            "roofline": dict(roofline("mfma", "whole step (six gemm_mfma_kernel launches + elementwise)", ms * 1e-3, gemm_flops, gemm_bytes,
+                                      traffic=profile_traffic("config4_ffn_step.txt") if fused else None),
                              note="flops and bytes of the six products only; the step's elementwise kernels add ~0.7 GB of traffic and no counted flops")}
     if with_cpu:
         rs = 256  # rows of the 4096
