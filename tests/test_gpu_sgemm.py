@@ -997,8 +997,8 @@ def test_decode_product_16_row_form_other_plans_integer_exact(dev, rocm, m, n, k
     rocm.sync()
 
 
-def test_decode_product_16_row_form_epilogues_accumulate_pitches_and_repeats(dev, rocm):
-    m, n, k = 13, 4096, 4096
+@pytest.mark.parametrize("m,n,k", [(13, 4096, 4096), (11, 16384, 2048)])   # (K slices summed by the last arrival; no slices: every workgroup finishes its own)
+def test_decode_product_16_row_form_epilogues_accumulate_pitches_and_repeats(dev, rocm, m, n, k):
     a = synth.small_ints(m, (m, k), 3); b = synth.small_ints(m + 1, (k, n), 3, stream=1)
     bias = synth.small_ints(m + 2, (n,), 5, stream=2); old = synth.small_ints(m + 3, (m, n), 9, stream=3)
     prod = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float64)
@@ -1046,8 +1046,8 @@ def test_decode_product_two_sets_of_rows_integer_exact(dev, rocm, m, n, k):
     rocm.sync()
 
 
-def test_decode_product_two_sets_of_rows_epilogues_accumulate_pitches_and_repeats(dev, rocm):
-    m, n, k = 27, 4096, 4096
+@pytest.mark.parametrize("m,n,k", [(27, 4096, 4096), (21, 16384, 1024)])
+def test_decode_product_two_sets_of_rows_epilogues_accumulate_pitches_and_repeats(dev, rocm, m, n, k):
     a = synth.small_ints(m, (m, k), 3); b = synth.small_ints(m + 1, (k, n), 3, stream=1)
     bias = synth.small_ints(m + 2, (n,), 5, stream=2); old = synth.small_ints(m + 3, (m, n), 9, stream=3)
     prod = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float64)
