@@ -181,6 +181,18 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_units_kernel(const GemvLaunch
     __builtin_amdgcn_s_barrier();
     if (tid >= MR * CL) return;
 
+    // Lane 0 counts the wavefront in -- now, before the workgroup's sums are added up and stored: the answer takes 0.6 us,
+    // the LDS sum and the stores 0.3-0.8, and whoever turns out to be the last arrival checks the tags of what it fetched
+    // anyway (a partial of a workgroup that counted in earlier and has not stored yet is fetched again).  Under an exec
+    // mask from inline asm: no divergent branch, so nothing waits for the answer here.
+    unsigned rank = 0;
+    if (S > 1) {  // (uniform over the grid)
+        unsigned long long saved;
+        asm volatile("s_mov_b64 %1, exec\n\ts_mov_b64 exec, 1\n\tglobal_atomic_inc %0, %2, %3, off sc0\n\ts_mov_b64 exec, %1"
+                     : "=&v"(rank), "=&s"(saved)
+                     : "v"(my_count), "v"(S - 1)
+                     : "memory");
+    }
     // all 16 wavefronts' sums at once, then added in wavefront order
     f32x4 e[GV_WAVES];
 #pragma unroll
@@ -202,15 +214,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_units_kernel(const GemvLaunch
     const float tag = __uint_as_float(epoch);
     *my_a = f32x4{t.x, t.y, t.z, tag};
     *my_b = f32x2{t.w, tag};
-    // lane 0 counts the wavefront in; no branch, so nothing waits for the answer here
-    unsigned rank;
-    {
-        unsigned long long saved;
-        asm volatile("s_mov_b64 %1, exec\n\ts_mov_b64 exec, 1\n\tglobal_atomic_inc %0, %2, %3, off sc0\n\ts_mov_b64 exec, %1"
-                     : "=&v"(rank), "=&s"(saved)
-                     : "v"(my_count), "v"(S - 1)
-                     : "memory");
-    }
     f32x4 a[SMAX];
     f32x2 b[SMAX];
     const int other = slice + 1 < S ? slice + 1 : 0;
@@ -435,6 +438,18 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_units16_kernel(const GemvLaun
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     if (tid >= PIECES) return;
+    // Lane 0 counts the wavefront in -- now, before the workgroup's sums are added up and stored: the answer takes 0.6 us,
+    // the LDS sum and the stores 0.3-0.8, and whoever turns out to be the last arrival checks the tags of what it fetched
+    // anyway (a partial of a workgroup that counted in earlier and has not stored yet is fetched again).  Under an exec
+    // mask from inline asm: no divergent branch, so nothing waits for the answer here.
+    unsigned rank = 0;
+    if (S > 1) {  // (uniform over the grid)
+        unsigned long long saved;
+        asm volatile("s_mov_b64 %1, exec\n\ts_mov_b64 exec, 1\n\tglobal_atomic_inc %0, %2, %3, off sc0\n\ts_mov_b64 exec, %1"
+                     : "=&v"(rank), "=&s"(saved)
+                     : "v"(my_count), "v"(S - 1)
+                     : "memory");
+    }
     // all 16 wavefronts' sums at once, then added in wavefront order
     f32x4 e[GV_WAVES];
 #pragma unroll
@@ -456,15 +471,6 @@ __global__ __launch_bounds__(GV_THREADS) void gemv_units16_kernel(const GemvLaun
     const float tag = __uint_as_float(epoch);
     *my_a = f32x4{t.x, t.y, t.z, tag};
     *my_b = f32x2{t.w, tag};
-    // lane 0 counts the wavefront in; no branch, so nothing waits for the answer here
-    unsigned rank;
-    {
-        unsigned long long saved;
-        asm volatile("s_mov_b64 %1, exec\n\ts_mov_b64 exec, 1\n\tglobal_atomic_inc %0, %2, %3, off sc0\n\ts_mov_b64 exec, %1"
-                     : "=&v"(rank), "=&s"(saved)
-                     : "v"(my_count), "v"(S - 1)
-                     : "memory");
-    }
     f32x4 a[SMAX];
     f32x2 b[SMAX];
     const int other = slice + 1 < S ? slice + 1 : 0;
