@@ -620,7 +620,21 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
                 // 1015 us for 128 x 128 tiles in K slices, the plan below)
             } else {
                 const int64_t tiles64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) * g.batch;
-                if (tiles64 <= cus) {
+                const int64_t wide = g.N % 128 == 0 ? (int64_t)(g.N / 128) : 0;  // 64 x 128 tiles of a product of up to 64 rows
+                if (g.M > 32 && g.M <= 64 && g.batch == 1 && tiles64 <= cus && wide > 0 && cus % wide == 0 && cus / wide <= 16 &&
+                    ktiles >= 8 * (cus / wide) && (int64_t)g.N * g.K >= (1LL << 24)) {
+                    // 33 to 64 rows against a weight that outgrows the L2s (batched decoding; the weight comes from HBM):
+                    // 64 x 128 tiles in as many K slices as give every CU one workgroup read B in 512-byte pieces of a row,
+                    // which is what streams best.  Cold B, us, against 64 x 64 tiles in the slices of the model below:
+                    // 64 x 4096 x 4096 25.6 / 27.4, 33 rows 25.2 / 27.0, 64 x 8192 x 8192 69.8 / 73.1, 64 x 4096 x 8192 40.1 / 45.3,
+                    // 64 x 8192 x 2048 25.1 / 27.1, 64 x 2048 x 8192 26.2 / 29.6, 64 x 4096 x 11008 50.5 / 52.1 (with B in the
+                    // Infinity Cache the small tiles are 3 % ahead: 23.3 / 24.1 at 4096 x 4096).  Below 2^24 elements of B the
+                    // small tiles lead: 64 x 2048 x 4096 17.8 / 17.1, 4096 x 2048 17.2 / 16.4, 8192 x 1024 17.2 / 16.6, 2048 x 2048 15.8 / 12.7.
+                    bm = 64;
+                    bn = 128;
+                    planned_split = (int)(cus / wide);
+                    whole_tiles = planned_split == 1;
+                } else if (tiles64 <= cus) {
                     // At most one 64 x 64 tile per CU: K slices by the cost model of split_for_few_tiles (one
                     // slice, i.e. no reduction pass, wins for short K: 32 x (512 x 64 x 512) 13.7 us whole, 19.0 in
                     // two K slices, 19.8 stream-K; several for long K: 128 x 4096 x 4096 69.6 us whole, 40.1 in four).

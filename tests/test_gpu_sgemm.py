@@ -583,6 +583,22 @@ def test_planner_gives_many_batches_of_few_rows_and_one_k_phase_to_the_direct_ke
     assert np.array_equal(got, forced)
 
 
+@pytest.mark.parametrize("m,n,k", [(33, 4096, 4096), (64, 2048, 8192), (50, 8192, 2048), (64, 16384, 1024)])
+def test_planner_gives_33_to_64_rows_against_a_large_weight_wide_tiles_in_k_slices(dev, rocm, m, n, k):
+    # 64 x 128 tiles in 256 / (N / 128) K slices, one workgroup per CU, and their reduction pass: exact on small integers, with and
+    # without the bias epilogue, and the bits of the forced plan
+    a = synth.small_ints(m + n, (m, k), 3)
+    b = synth.small_ints(k + m, (k, n), 3, stream=1)
+    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    got = run_gemm(dev, a, b)[0]
+    assert np.array_equal(got, want)
+    assert np.array_equal(got, run_gemm(dev, a, b, algo=N.ALGO_MFMA, split_k=256 // (n // 128))[0])
+    bias = synth.small_ints(n, (n,), 5, stream=2)
+    dA, dB, dBias, dC = dev.put(a), dev.put(b), dev.put(bias), dev.empty(m * n, fill=-3.0)
+    rocm.sgemm(m, n, k, dA, dB, dC, bias=dBias, epilogue=N.EPI_BIAS_RELU)
+    assert np.array_equal(rocm.to_host(dC, (m, n)), np.maximum(want + bias, 0.0).astype(np.float32))
+
+
 # ---- tiny products: one thread per output, the reference CPU arm's own sum ---------------------------
 
 @pytest.mark.parametrize("m,n,k", [(32, 64, 10), (32, 3, 64), (32, 64, 3), (32, 10, 64), (64, 3, 32), (10, 64, 32), (1, 1, 1), (7, 5, 3),
