@@ -634,6 +634,15 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
                     bn = 128;
                     planned_split = (int)(cus / wide);
                     whole_tiles = planned_split == 1;
+                } else if (g.M > 64 && g.M <= 128 && g.batch == 1 && tiles64 <= cus && wide > 0 && cus % wide == 0 && cus / wide <= 16 &&
+                           ktiles >= 8 * (cus / wide) && g.K >= 8192 && (int64_t)g.N * g.K >= (1LL << 25)) {
+                    // 65 to 128 rows against a long K of a large weight: the same with 128 x 128 tiles.  Cold B, us, against
+                    // 64 x 64 tiles: 128 x 8192 x 8192 126.8 / 133.8, 80 rows 125.1 / 132.5, 128 x 4096 x 8192 69.4 / 71.4,
+                    // 128 x 4096 x 11008 89.2 / 92.8; level at 4096 x 4096 and 2048 x 8192, behind at 8192 x 2048 and shorter K.
+                    bm = 128;
+                    bn = 128;
+                    planned_split = (int)(cus / wide);
+                    whole_tiles = planned_split == 1;
                 } else if (tiles64 <= cus) {
                     // At most one 64 x 64 tile per CU: K slices by the cost model of split_for_few_tiles (one
                     // slice, i.e. no reduction pass, wins for short K: 32 x (512 x 64 x 512) 13.7 us whole, 19.0 in

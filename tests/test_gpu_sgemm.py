@@ -583,13 +583,14 @@ def test_planner_gives_many_batches_of_few_rows_and_one_k_phase_to_the_direct_ke
     assert np.array_equal(got, forced)
 
 
-@pytest.mark.parametrize("m,n,k", [(33, 4096, 4096), (64, 2048, 8192), (50, 8192, 2048), (64, 16384, 1024)])
+@pytest.mark.parametrize("m,n,k", [(33, 4096, 4096), (64, 2048, 8192), (50, 8192, 2048), (64, 16384, 1024), (96, 4096, 8192), (128, 8192, 8192),
+                                   (70, 4096, 11008)])
 def test_planner_gives_33_to_64_rows_against_a_large_weight_wide_tiles_in_k_slices(dev, rocm, m, n, k):
-    # 64 x 128 tiles in 256 / (N / 128) K slices, one workgroup per CU, and their reduction pass: exact on small integers, with and
-    # without the bias epilogue, and the bits of the forced plan
+    # 64 x 128 tiles (128 x 128 from 65 rows, for a long K) in 256 / (N / 128) K slices, one workgroup per CU, and their reduction pass:
+    # exact on small integers, with and without the bias epilogue, and the bits of the forced plan
     a = synth.small_ints(m + n, (m, k), 3)
     b = synth.small_ints(k + m, (k, n), 3, stream=1)
-    want = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)  # (exact: the sums stay far below 2^53)
     got = run_gemm(dev, a, b)[0]
     assert np.array_equal(got, want)
     assert np.array_equal(got, run_gemm(dev, a, b, algo=N.ALGO_MFMA, split_k=256 // (n // 128))[0])
