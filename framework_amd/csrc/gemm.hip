@@ -583,24 +583,25 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
         const int64_t big_slots = (int64_t)cus * gemm_mfma_resident_per_cu(bm, bn);
         // One workgroup per tile when some tile shape deals the CUs equal loads: a CU's matrix pipe is
         // shared by the workgroups resident on it, so what counts is tiles per CU, not per workgroup slot
-        // (768 tiles of 128 x 128 on 256 CUs run as fast per tile as 1024 do), and at least two per CU,
-        // because one workgroup alone leaves a SIMD a single wavefront and its stalls uncovered.  The K
-        // loop issues no vector-ALU work whatever the tile shape, so a smaller tile costs only its extra
-        // L2 traffic: the biggest shape whose last round is at least 95 % full wins.  (Measured: whole
-        // tiles take ideal / fill, stream-K ideal x 1.03-1.05; 2560^3 with 64 x 64 tiles at 89 % loses 10 %
-        // to stream-K, 4096 x 768 x 3072 with 64 x 64 tiles at 100 % beats it by 10 %.)
+        // (768 tiles of 128 x 128 on 256 CUs run as fast per tile as 1024 do).  The biggest shape whose last
+        // round is at least 95 % full wins; at least two tiles per CU, except that 128 x 128 tiles may come one
+        // per CU when K is 1024 and more.  (Measured: whole tiles take ideal / fill, stream-K ideal x 1.03-1.05;
+        // 2560^3 with 64 x 64 tiles at 89 % loses 10 % to stream-K, 4096 x 768 x 3072 with 64 x 64 tiles at 100 % beats
+        // it by 10 %.)  Big before small whatever the K: on operands of normally distributed values, us, 128 x 128
+        // against what smaller tiles the same rule picked before: 4096 x 4096 x 1024 247.9 / 262.2 (64 x 64), x 512
+        // 133.4 / 140.9, 4096 x 3072 x 768 146.0 / 151.2, 4096 x 1024 x 4096 239.7 / 248.7 (128 x 64, two per CU), its
+        // transposed forms 238-243 / 248-251.  An earlier version of this rule preferred the small shapes up to 32 K
+        // steps on the strength of products of constants (4096 x 4096 x 1024: 244.6 / 246.5 there): constants toggle few
+        // bits, the matrix pipe draws less and clocks higher, and the ranking of the tile shapes turns round.
         if (ktiles >= 8 && d.split_k == 0 && d.algo == MNI_ALGO_AUTO) {
-            // Up to 32 K steps the smaller shapes run ahead (more workgroups to overlap prologues and epilogues
-            // with): 1-3 % with A along K, and with A given as its transpose 4096 x 11008 x 128 137.5 -> 119.4 us,
-            // 768 x 3072 x 256 24.3 -> 17.3, 8192 x 8192 x 128 187.5 -> 173.6, 4096 x 4096 x 1024 246.5 -> 244.6.
             const int cand[4][2] = {{128, 128}, {128, 64}, {64, 128}, {64, 64}};
-            const bool small_first = ktiles <= 32;
             for (int i = 0; i < 4 && !whole_tiles; ++i) {
-                const int cm = cand[small_first ? 3 - i : i][0], cn = cand[small_first ? 3 - i : i][1];
+                const int cm = cand[i][0], cn = cand[i][1];
                 if (cm > bm || cn > bn) continue;
                 const int64_t tiles = (int64_t)((g.M + cm - 1) / cm) * ((g.N + cn - 1) / cn) * g.batch;
                 const int64_t per_cu = (tiles + cus - 1) / cus;
-                if (per_cu >= 2 && tiles * 100 >= per_cu * cus * 95) {
+                const bool alone_ok = cm == 128 && cn == 128 && g.K >= 1024;  // (one 128 x 128 workgroup per CU, a K long enough to hide its start and end)
+                if ((per_cu >= 2 || alone_ok) && tiles * 100 >= per_cu * cus * 95) {
                     whole_tiles = true;
                     bm = cm;
                     bn = cn;
