@@ -99,9 +99,9 @@ static bool try_gemv_units(const SkinnyLaunch &s, const mni_gemm_desc &d, int *r
                          gemv_units16_plan(s.rows, s.cols, s.K, c.compute_units, c.xcd_count, &slices16, &trips16) &&
                          gemv_units16_partial_slots(s.rows, s.cols, slices16) <= c.gemv_slot_cap &&
                          gemv_units16_counters(s.rows, s.cols) <= c.gemv_counter_cap;
-    // Two sets of rows, us against the few-rows MFMA kernel: 32 x 4096 x 4096 16.5 / 21.4, 17 rows 16.0 / 20.9,
-    // 32 x 16384 x 1024 14.7 / 20.6, 32 x 4096 x 8192 28.2 / 33.8, 32 x 8192 x 2048 16.6 / 20.2; 32 x 8192 x 8192 50.4 / 50.0
-    if (s.rows > 16 && d.algo == MNI_ALGO_AUTO && (int64_t)s.cols * s.K >= (1LL << 26)) return false;
+    // Two sets of rows, us against the few-rows MFMA kernel (cold W of normally distributed values): 32 x 4096 x 4096 16.4 / 21.5,
+    // 24 rows 16.1 / 21.4, 32 x 8192 x 4096 28.2 / 30.8, 32 x 4096 x 8192 28.3 / 33.9, 32 x 8192 x 8192 52.4 / 52.6, 24 rows 50.0 / 52.6,
+    // 32 x 4096 x 16384 52.3 / 55.5, 32 x 16384 x 4096 50.2 / 52.2: taken wherever it is eligible.
     const bool prefer_wide = s.rows > 6 || s.cols > 4096;
     const bool wide = wide_ok && (prefer_wide || !narrow_ok);
     if (!wide && !narrow_ok) return false;
