@@ -130,9 +130,14 @@ struct Engine {
     const std::vector<int64_t> *bw_out2entry = nullptr;  // tensor id -> tape entry that produced it
     const std::vector<int> *bw_consumers = nullptr;      // tensor id -> tape entries that read it
     const std::vector<int64_t> *bw_grads = nullptr;      // tensor id -> gradient gathered so far
-    // output id of a GELU Linear -> its bias gradient, when the gradient that reaches it has already been
-    // taken through gelu' by the entry that consumed it
-    std::map<uint32_t, uint32_t> preact_db;
+    // output id of a GELU Linear -> the strip sums of its bias gradient ([rows, cols]: the gradient is their column
+    // sums), when the gradient that reaches it has already been taken through gelu' by the entry that consumed it.
+    // That layer's own backward adds the strips up, in the launch of its two products where that launch takes them.
+    struct PendingStrips {
+        BufP strips;
+        int64_t rows, cols;
+    };
+    std::map<uint32_t, PendingStrips> preact_strips;
     // One float holding 1.0, shared by every scalar loss as the gradient backward() starts from (writers copy
     // a shared buffer before they touch it, so nobody changes it).
     BufP one;
@@ -1386,12 +1391,13 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
     bool own_g = false;
     int64_t db_id = -1;
     Engine &en = eng();
-    const auto pre = en.preact_db.find(e.output_id);
-    if (e.act == MNI_EPI_BIAS_GELU && pre != en.preact_db.end()) {
+    Engine::PendingStrips pend = {nullptr, 0, 0};
+    const auto pre = en.preact_strips.find(e.output_id);
+    if (e.act == MNI_EPI_BIAS_GELU && pre != en.preact_strips.end()) {
         // the entry that consumed this layer's output has already taken the gradient through gelu'
-        // (in the epilogue of its own product) and summed the bias gradient
-        db_id = pre->second;
-        en.preact_db.erase(pre);
+        // (in the epilogue of its own product) and left the bias gradient as strip sums
+        pend = std::move(pre->second);
+        en.preact_strips.erase(pre);
     } else if (e.act == MNI_EPI_BIAS_GELU) {
         // dZ = dOut * gelu'(z + bias) and db = column sums of dZ in one pass (ops/fused.rs:316-351)
         Tensor *G = get(grad), *Z = get(e.aux), *Bv = get(e.inputs[2]);
@@ -1436,7 +1442,7 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
             const Entry &P = en.bw_tape->entries[(size_t)pi];
             Tensor *Z = P.op == OP_LINEAR && P.act == MNI_EPI_BIAS_GELU && P.output_id == x ? get(P.aux) : nullptr;
             Tensor *PB = Z ? get(P.inputs[2]) : nullptr;
-            if (Z && PB && is_contiguous(*Z) && Z->shape == X->shape && en.preact_db.find(x) == en.preact_db.end()) {
+            if (Z && PB && is_contiguous(*Z) && Z->shape == X->shape && en.preact_strips.find(x) == en.preact_strips.end()) {
                 strip_cols = X->shape.back();
                 const int64_t m = X->shape[X->shape.size() - 2];
                 strip_rows = mni_rocm_sgemm_colsum_rows(m, strip_cols && m ? X->size / (strip_cols * m) : 0);
@@ -1450,30 +1456,26 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
             }
         }
     }
-    // The bias gradient (column sums of g over its rows) rides in the launch of the two products when they are small
-    // enough to go out as one launch of the tiny-product kernel: a training step of a few thousand parameters is the
-    // sum of its launches.
+    // The bias gradient (column sums of g over its rows, or of the strip sums left by the consumer) rides in the launch
+    // of the two products when they go out as one launch that takes it: a training step of a few thousand parameters
+    // is the sum of its launches, and under two big products the sums cost nothing.
     PairColsum sums = {nullptr, nullptr, 0, 0, false};
     BufP db_early;
-    if (db_id < 0) {
+    if (pend.strips) {
+        db_early = new_buf((size_t)pend.cols);
+        if (!db_early) return MNI_ERR_NOMEM;
+        sums = PairColsum{pend.strips->p, db_early->p, pend.rows, pend.cols, false};
+    } else if (db_id < 0) {
         Tensor *G = get(g), *Bv = get(e.inputs[2]);
-        if (G && Bv && is_contiguous(*G) && !G->shape.empty() && G->shape.back() == Bv->size && Bv->size > 0 && G->size / Bv->size <= 256) {
+        if (G && Bv && is_contiguous(*G) && !G->shape.empty() && G->shape.back() == Bv->size && Bv->size > 0) {
             db_early = new_buf((size_t)Bv->size);
             if (db_early) sums = PairColsum{G->buf->p, db_early->p, G->size / Bv->size, Bv->size, false};
         }
     }
     int rc = matmul_backward(g, mm, out, tg.z ? &tg : nullptr, sums.out ? &sums : nullptr);
-    if (rc == MNI_OK && tg.z) {
-        // bias gradient of the producing layer: the strips added up, in strip order
-        Tensor *PB = get(en.bw_tape->entries[(size_t)(*en.bw_out2entry)[producer_out]].inputs[2]);
-        BufP db = PB ? new_buf((size_t)strip_cols) : nullptr;
-        if (!db) rc = MNI_ERR_NOMEM;
-        else rc = k_colsum(db->p, strips->p, strip_rows, strip_cols);
-        if (rc == MNI_OK) {
-            const Shape bshape = PB->shape;
-            en.preact_db[producer_out] = insert_contig(std::move(db), bshape);
-        }
-    }
+    if (rc == MNI_OK && tg.z) en.preact_strips[producer_out] = Engine::PendingStrips{strips, strip_rows, strip_cols};
+    // (the strips added up in strip order, when the launch above did not take them)
+    if (rc == MNI_OK && pend.strips && !sums.done) rc = k_colsum(db_early->p, pend.strips->p, pend.rows, pend.cols);
     if (rc == MNI_OK) {
         if (db_id >= 0) out[2] = db_id;
         else {
@@ -1481,7 +1483,7 @@ static int linear_backward(uint32_t grad, const Entry &e, int64_t *out) {
             if (!Bv) rc = MNI_ERR_FREED;
             else {
                 const Shape bshape = Bv->shape;
-                const uint32_t gb = sums.done ? insert_contig(std::move(db_early), bshape) : unbroadcast_tensor(g, bshape);
+                const uint32_t gb = (sums.done || pend.strips) ? insert_contig(std::move(db_early), bshape) : unbroadcast_tensor(g, bshape);
                 if (gb == MNI_BAD_ID) rc = MNI_ERR_INVALID;
                 else out[2] = gb;
             }
@@ -1913,8 +1915,7 @@ static int tape_backward(Tape &tp, uint32_t loss) {
         }
         ~WalkScope() {
             e.bw_tape = nullptr; e.bw_out2entry = nullptr; e.bw_consumers = nullptr; e.bw_grads = nullptr;
-            for (auto &kv : e.preact_db) free_tensor(kv.second);  // (none are left when the walk completed)
-            e.preact_db.clear();
+            e.preact_strips.clear();  // (none are left when the walk completed)
         }
     } walk_scope(eng(), &tp, &out2entry, &consumers, &grads);
     {

@@ -333,7 +333,7 @@ static void fill_launch(GemmLaunch &g, const mni_gemm_desc &d) {
 struct PlanProbe {
     enum { TILE = 0, PANEL = 1, DIRECT = 2, TILE_FUSED_GELU = 3, TILE_STREAMK = 4, FEWROWS = 5, OUTER = 6 };
     int kind, bm, bn, split, amode, bmode;
-    GemmLaunch g;  // kind TILE: the launch descriptor, complete
+    GemmLaunch g;  // kinds TILE and TILE_FUSED_GELU: the launch descriptor, complete
 };
 
 // K slices of the few-rows kernel: one workgroup per CU (more gain nothing: with one, the loop already runs close
@@ -695,7 +695,12 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
         g.k_per_slice = g.K > 0 ? g.K : 1;
         g.aux_out = d.aux;                // shares its slot with the K-slice partials, which this form never has
         g.colsum_part = d.colsum_part;    // shares its slot with the stream-K marks
-        if (probe) { probe->kind = PlanProbe::TILE_FUSED_GELU; return MNI_OK; }
+        if (probe) {
+            probe->kind = PlanProbe::TILE_FUSED_GELU;
+            probe->bm = bm; probe->bn = bn; probe->split = 1; probe->amode = amode; probe->bmode = bmode;
+            probe->g = g;
+            return MNI_OK;
+        }
         return launch_gemm_mfma(g, amode, bmode, bm, bn);
     }
     void *ws = nullptr;
@@ -893,12 +898,18 @@ int sgemm(const mni_gemm_desc &d) {
 }
 
 // Two products that do not depend on each other (neither reads what the other writes; the outputs do not
-// overlap).  One launch when run_mfma's plan for each of them alone is the tile kernel's 64 x 64 tiles, one
-// workgroup per tile and all of K (batched products of about a tile per CU): together they give every SIMD a
-// second wavefront and share one launch, one ramp-up and one tail.  Measured on 32 x (512 x 64 x 512)
-// and its transposed twin: 13.4 + 13.6 us one after the other, 20.9 us together (64 batches of the first in one
-// launch take the same 20.8).  Otherwise one after the other.  Same kernel body and same order of every sum either
-// way, so the results are those of the separate calls bit for bit.
+// overlap).  One launch when run_mfma's plan for each of them alone is one workgroup per tile of the tile kernel and
+// all of K, on 64 x 64 tiles both or on 128 x 128 tiles both.  Small tiles (batched products of about a tile per
+// CU): together they give every SIMD a second wavefront and share one launch, one ramp-up and one tail.  Measured on
+// 32 x (512 x 64 x 512) and its transposed twin: 13.4 + 13.6 us one after the other, 20.9 us together (64 batches of
+// the first in one launch take the same 20.8).  Big tiles (the two gradients of a Linear layer): the second product's
+// workgroups start where the first one's run out, so one drain and one fill of the machine go, and two products of
+// one tile per CU each give every CU its second workgroup.  Measured on normally distributed operands, the pair
+// issued back to back separately / as one launch, us: the gradients of [4096, 1024] . [1024, 4096] 489.6 / 473.0, of
+// [4096, 4096] . [4096, 1024] (1024 tiles of K = 1024 behind 256 of K = 4096) 494.8 / 483.7, of 2048^3 259.8 / 245.4,
+// [4096, 2048] . [2048, 2048] 484.2 / 474.1, [2048, 4096] . [4096, 1024] 257.1 / 250.6, [8192, 1024] . [1024, 4096]
+// 943.2 / 922.3, 4096^3 1853.3 / 1849.4.  Otherwise one after the other.  Same kernel body and same order of every sum
+// either way, so the results are those of the separate calls bit for bit.
 int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1, PairColsum *colsum) {
     if (colsum) colsum->done = false;
     MNI_TRY(ensure_init());
@@ -930,7 +941,7 @@ int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1, PairColsum *col
     }
     PlanProbe plan[2];
     int64_t tiles = 0;
-    bool pair = true;
+    bool pair = true, big = true;
     for (int i = 0; i < 2 && pair; ++i) {
         const mni_gemm_desc &d = *ds[i];
         // (min(M, N) <= 16 may go to the skinny kernels, which sgemm tries before run_mfma)
@@ -942,12 +953,28 @@ int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1, PairColsum *col
             if (gemm_tiny_eligible(t)) { pair = false; break; }  // sgemm computes those outright
         }
         MNI_TRY(run_mfma(d, &plan[i]));
-        pair = plan[i].kind == PlanProbe::TILE && plan[i].bm == 64 && plan[i].bn == 64 && plan[i].split == 1;
+        const bool whole = (plan[i].kind == PlanProbe::TILE || plan[i].kind == PlanProbe::TILE_FUSED_GELU) && plan[i].split == 1 &&
+                           plan[i].bm == plan[i].bn;
+        // 128 x 128 tiles: only products that sgemm would hand to run_mfma as they are (no batch to fold into the rows, no
+        // ragged edge to cut off or operand to repack: every extent a multiple of 4)
+        big = big && whole && plan[i].bm == 128 && d.batch == 1 && d.M % 4 == 0 && d.N % 4 == 0 && d.K % 4 == 0;
+        pair = whole && (plan[i].bm == 64 ? plan[i].kind == PlanProbe::TILE : big);
         if (pair) tiles += (int64_t)plan[i].g.tiles_m * plan[i].g.tiles_n * plan[i].g.batch;
     }
-    // up to four 64 x 64 workgroups fit a CU; beyond that a joint launch has nothing left to fill
-    if (pair && tiles <= 4LL * cus && gemm_mfma_pair_eligible(plan[0].amode, plan[0].bmode, plan[1].amode, plan[1].bmode))
-        return launch_gemm_mfma_pair(plan[0].g, plan[0].amode, plan[0].bmode, plan[1].g, plan[1].amode, plan[1].bmode);
+    if (pair && plan[0].bm == plan[1].bm && gemm_mfma_pair_eligible(plan[0].amode, plan[0].bmode, plan[1].amode, plan[1].bmode)) {
+        // 64 x 64: up to four workgroups fit a CU; beyond that a joint launch has nothing left to fill.  128 x 128: whatever
+        // the tile counts (see above).
+        if ((plan[0].bm == 64 && tiles <= 4LL * cus) || (plan[0].bm == 128 && big)) {
+            // the caller's column sums ride along: workgroups behind the tiles that read the matrix once in the launch's tail
+            // (4096 x 1024: two launches of 4.6 us each otherwise; config 4's step 1.512 -> 1.500 ms with both bias
+            // gradients taken this way)
+            const bool with_sums = colsum && gemm_mfma_pair_takes_colsum(*colsum);
+            MNI_TRY(launch_gemm_mfma_pair(plan[0].g, plan[0].amode, plan[0].bmode, plan[1].g, plan[1].amode, plan[1].bmode, plan[0].bm,
+                                          with_sums ? colsum : nullptr));
+            if (with_sums) colsum->done = true;
+            return MNI_OK;
+        }
+    }
     MNI_TRY(sgemm(d0));
     return sgemm(d1);
 }

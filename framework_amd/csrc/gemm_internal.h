@@ -46,9 +46,22 @@ struct GemmLaunch {
 
 // tile_m, tile_n in {128, 64}; g.tiles_m / g.tiles_n count tiles of that size
 int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int tile_n);
-// Two independent products of 64 x 64 tiles (one workgroup per tile, all of K) in one launch; amode0 must be 0 and bmode1 1.
+// Column sums of a contiguous [rows, cols] matrix that a paired launch computes along with its two products (in the
+// tiny-product pair: rows added in order; in the tile kernel's pair: in 64 interleaved groups of rows, the groups then
+// added in order); `done` says whether the launch did.
+struct PairColsum {
+    const float *src;
+    float *out;
+    int64_t rows, cols;
+    bool done;
+};
+// Two independent products, both of 64 x 64 or both of 128 x 128 tiles (`tile`; one workgroup per tile, all of K) in one
+// launch; amode0 must be 0 and bmode1 1.
 bool gemm_mfma_pair_eligible(int amode0, int bmode0, int amode1, int bmode1);
-int launch_gemm_mfma_pair(const GemmLaunch &g0, int amode0, int bmode0, const GemmLaunch &g1, int amode1, int bmode1);
+// `colsum` (may be null): column sums computed by extra workgroups of the same launch; must satisfy gemm_mfma_pair_takes_colsum.
+bool gemm_mfma_pair_takes_colsum(const PairColsum &cs);
+int launch_gemm_mfma_pair(const GemmLaunch &g0, int amode0, int bmode0, const GemmLaunch &g1, int amode1, int bmode1, int tile,
+                          const PairColsum *colsum = nullptr);
 // workgroups that stay resident per CU for a tile shape (what the stream-K grid is sized by)
 int gemm_mfma_resident_per_cu(int tile_m, int tile_n);
 int gemm_mfma_tile_k();
@@ -61,14 +74,6 @@ int launch_gemm_direct(const GemmLaunch &g, int amode, int bmode, int ksplit);
 // One thread per output, sequential K (gemm_tiny.hip): a few thousand outputs of a short K, any strides.
 bool gemm_tiny_eligible(const GemmLaunch &g);
 int launch_gemm_tiny(const GemmLaunch &g);
-// Column sums of a contiguous [rows, cols] matrix (rows added in order) that a paired launch of two tiny products
-// computes along with them; `done` says whether it did.
-struct PairColsum {
-    const float *src;
-    float *out;
-    int64_t rows, cols;
-    bool done;
-};
 int launch_gemm_tiny_pair(const GemmLaunch &g0, const GemmLaunch &g1, const PairColsum *colsum = nullptr);  // two eligible, independent products in one launch
 // 9 to 32 rows of a K-contiguous A against a wide N-contiguous B, both straight into MFMA registers (gemm_fewrows.hip):
 // g.tiles_n counts column groups of 128, g.split_k K slices of g.k_per_slice (a multiple of 32).  With split_k > 1:

@@ -861,28 +861,92 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
     gemm_mfma_body<AMODE, BMODE, TM, TN, SK>((LaunchPtr)__builtin_amdgcn_kernarg_segment_ptr(), blockIdx.x, gridDim.x, lds);
 }
 
-// Two independent products of 64 x 64 tiles in one launch: workgroups [0, wgs0) work on the first (wgs0 = its tile
-// count rounded up to a multiple of 8, so that the second product's numbering starts on XCD 0 as well; the
-// padding workgroups leave at once), the rest on the second.  For the two backward products of a batched matmul
-// (src/native/src/ops/matmul.rs:199-222) when each of them alone is about one tile per CU: together they give
-// every SIMD two wavefronts, and they share one launch, one ramp-up and one tail.
+// Two independent products in one launch, both on 64 x 64 tiles or both on 128 x 128 (T = 1, 2), one workgroup per
+// tile and all of K: workgroups [0, wgs_lead) work on the product named by `lead` (wgs_lead = its tile count rounded
+// up to a multiple of 8, so that the other product's numbering starts on XCD 0 as well; the padding workgroups
+// leave at once), the rest on the other.  For the two backward products of a matmul
+// (src/native/src/ops/matmul.rs:199-222): when each of them alone is about one tile per CU, together they give
+// every SIMD a second wavefront; and whatever their size they share one launch, one ramp-up and one tail.  The
+// product with the longer K leads, so that its long-lived workgroups are dealt first and the short ones fill in
+// behind them.
 struct GemmPairLaunch {
     GemmLaunch g[2];
-    unsigned wgs0, tiles0, tiles1;
+    unsigned lead, wgs_lead, tiles0, tiles1;
+    // Column sums that ride along (a Linear layer's bias gradient: the sums of the matrix both products read): cs_out[c] =
+    // sum over r of cs_src[r, c] for a contiguous [cs_rows, cs_cols] matrix, by cs_wgs workgroups behind the products'
+    // (0: none), PAIR_CS_COLS columns each.  Behind, because a workgroup ahead of the tiles would take a tile's place in
+    // the first round on a machine the tiles fill exactly, and that tile would run alone at the end; at the end they
+    // start as the first tiles finish and run in the raggedness of the launch's tail.
+    const float *cs_src;
+    float *cs_out;
+    int cs_rows, cs_cols;
+    unsigned cs_wgs;
 };
+typedef const GemmPairLaunch __attribute__((address_space(4))) *PairPtr;
 
-template <int AM0, int BM0, int AM1, int BM1>
-__global__ __launch_bounds__(NTHREADS, 4) void gemm_mfma_pair_kernel(const GemmPairLaunch pair_args) {
+constexpr int PAIR_CS_COLS = 8, PAIR_CS_GROUPS = 128, PAIR_CS_DEPTH = 8;
+static_assert(NTHREADS == 2 * PAIR_CS_GROUPS && PAIR_CS_COLS == 8, "the column sums of a paired launch split 256 threads into 2 column quads x 128 row groups");
+
+// Workgroup b of the column sums: thread (quad, group) adds rows group, group + 128, ... of its four columns (eight
+// loads in flight), the groups are added in order through LDS.  cs_cols is a multiple of 4 and both pointers are
+// 16-byte aligned (checked by the launcher).
+__device__ __forceinline__ void pair_colsum_role(PairPtr pp, const unsigned b, float4 *__restrict__ lds) {
+    const int tid = threadIdx.x, cq = tid & 1, rg = tid >> 1;
+    const int rows = pp->cs_rows, cols = pp->cs_cols;
+    const int col = (int)b * PAIR_CS_COLS + 4 * cq;
+    float4 acc[PAIR_CS_DEPTH];
+#pragma unroll
+    for (int u = 0; u < PAIR_CS_DEPTH; ++u) acc[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (col < cols) {
+        const float *__restrict__ p = pp->cs_src + col;
+        int r = rg;
+        for (; r + PAIR_CS_GROUPS * (PAIR_CS_DEPTH - 1) < rows; r += PAIR_CS_GROUPS * PAIR_CS_DEPTH) {
+            float4 v[PAIR_CS_DEPTH];
+#pragma unroll
+            for (int u = 0; u < PAIR_CS_DEPTH; ++u) v[u] = *reinterpret_cast<const float4 *>(p + (int64_t)(r + PAIR_CS_GROUPS * u) * cols);
+#pragma unroll
+            for (int u = 0; u < PAIR_CS_DEPTH; ++u) { acc[u].x += v[u].x; acc[u].y += v[u].y; acc[u].z += v[u].z; acc[u].w += v[u].w; }
+        }
+        for (; r < rows; r += PAIR_CS_GROUPS) {
+            const float4 v = *reinterpret_cast<const float4 *>(p + (int64_t)r * cols);
+            acc[0].x += v.x; acc[0].y += v.y; acc[0].z += v.z; acc[0].w += v.w;
+        }
+    }
+#pragma unroll
+    for (int w = PAIR_CS_DEPTH / 2; w >= 1; w >>= 1)
+#pragma unroll
+        for (int u = 0; u < w; ++u) { acc[u].x += acc[u + w].x; acc[u].y += acc[u + w].y; acc[u].z += acc[u + w].z; acc[u].w += acc[u + w].w; }
+    lds[tid] = acc[0];
+    __syncthreads();
+    if (tid < 2 && col < cols) {
+        float4 t = lds[tid];
+        for (int g = 1; g < PAIR_CS_GROUPS; ++g) {
+            const float4 v = lds[2 * g + tid];
+            t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+        }
+        *reinterpret_cast<float4 *>(pp->cs_out + col) = t;
+    }
+}
+
+template <int AM0, int BM0, int AM1, int BM1, int T>
+__global__ __launch_bounds__(NTHREADS, (T >= 2 ? 2 : 4)) void gemm_mfma_pair_kernel(const GemmPairLaunch pair_args) {
     (void)pair_args;
-    typedef const GemmPairLaunch __attribute__((address_space(4))) *PairPtr;
     PairPtr pp = (PairPtr)__builtin_amdgcn_kernarg_segment_ptr();
-    constexpr int S0 = gemm_lds_slots<AM0, BM0, 1, 1>(), S1 = gemm_lds_slots<AM1, BM1, 1, 1>();
+    constexpr int S0 = gemm_lds_slots<AM0, BM0, T, T>(), S1 = gemm_lds_slots<AM1, BM1, T, T>();
+    static_assert(S0 >= NTHREADS && S1 >= NTHREADS, "the column sums park one float4 per thread");
     __shared__ float4 lds[S0 > S1 ? S0 : S1];
-    const unsigned wg = blockIdx.x;
-    if (wg < pp->wgs0) {
-        if (wg < pp->tiles0) gemm_mfma_body<AM0, BM0, 1, 1, false>(&pp->g[0], wg, pp->tiles0, lds);
+    const unsigned b = blockIdx.x, tile_wgs = pp->wgs_lead + (pp->lead ? pp->tiles0 : pp->tiles1);
+    if (b >= tile_wgs) {
+        pair_colsum_role(pp, b - tile_wgs, lds);
+        return;
+    }
+    const bool in_lead = b < pp->wgs_lead;
+    const unsigned wg = in_lead ? b : b - pp->wgs_lead;
+    const unsigned which = in_lead ? pp->lead : 1u - pp->lead;
+    if (which == 0) {
+        if (wg < pp->tiles0) gemm_mfma_body<AM0, BM0, T, T, false>(&pp->g[0], wg, pp->tiles0, lds);
     } else {
-        gemm_mfma_body<AM1, BM1, 1, 1, false>(&pp->g[1], wg - pp->wgs0, pp->tiles1, lds);
+        if (wg < pp->tiles1) gemm_mfma_body<AM1, BM1, T, T, false>(&pp->g[1], wg, pp->tiles1, lds);
     }
 }
 
@@ -949,31 +1013,53 @@ int launch_gemm_mfma(const GemmLaunch &g, int amode, int bmode, int tile_m, int 
 }
 
 // The product pairs a matmul backward gives rise to: product 0 has dC (row-major) as its A, product 1 has dC as
-// its B; 64 x 64 tiles (g.tiles_m / g.tiles_n count those), one workgroup per tile, all of K.
+// its B; tiles of `tile` x `tile` (64 or 128; g.tiles_m / g.tiles_n count those), one workgroup per tile, all of K.
 bool gemm_mfma_pair_eligible(int amode0, int bmode0, int amode1, int bmode1) {
     return amode0 == 0 && bmode0 <= 1 && amode1 <= 1 && bmode1 == 1;
 }
 
-int launch_gemm_mfma_pair(const GemmLaunch &g0, int amode0, int bmode0, const GemmLaunch &g1, int amode1, int bmode1) {
+template <int T>
+static void launch_pair_modes(const GemmPairLaunch &p, int bmode0, int amode1, dim3 grid) {
+    const dim3 block(NTHREADS);
+    hipStream_t s = ctx().stream;
+    if (bmode0 == 0 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 0, 1, T>), grid, block, 0, s, p);
+    else if (bmode0 == 0 && amode1 == 1) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 1, 1, T>), grid, block, 0, s, p);
+    else if (bmode0 == 1 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 0, 1, T>), grid, block, 0, s, p);
+    else MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 1, 1, T>), grid, block, 0, s, p);
+}
+
+bool gemm_mfma_pair_takes_colsum(const PairColsum &cs) {
+    return cs.src && cs.out && cs.rows > 0 && cs.cols > 0 && cs.cols % 4 == 0 && cs.rows <= 0x7fffffffLL && cs.cols <= (1LL << 24) &&
+           ((uintptr_t)cs.src & 15) == 0 && ((uintptr_t)cs.out & 15) == 0;
+}
+
+int launch_gemm_mfma_pair(const GemmLaunch &g0, int amode0, int bmode0, const GemmLaunch &g1, int amode1, int bmode1, int tile,
+                          const PairColsum *colsum) {
     if (!gemm_mfma_pair_eligible(amode0, bmode0, amode1, bmode1))
         return set_error(MNI_ERR_INVALID, "sgemm: product pair not eligible for the paired tile kernel");
+    if (tile != 64 && tile != 128) return set_error(MNI_ERR_INVALID, "sgemm: paired tile kernel takes tiles of 64 or 128");
+    if (colsum && !gemm_mfma_pair_takes_colsum(*colsum))
+        return set_error(MNI_ERR_INVALID, "sgemm: the paired tile kernel's column sums take a 16-byte aligned matrix of a multiple of 4 columns");
     const int64_t t0 = (int64_t)g0.tiles_m * g0.tiles_n * g0.batch, t1 = (int64_t)g1.tiles_m * g1.tiles_n * g1.batch;
-    if (g0.tiles_m != (g0.M + 63) / 64 || g0.tiles_n != (g0.N + 63) / 64 || g1.tiles_m != (g1.M + 63) / 64 ||
-        g1.tiles_n != (g1.N + 63) / 64 || t0 <= 0 || t1 <= 0 || t0 + t1 + 8 > 0x7fffffffLL || g0.split_k != 1 || g1.split_k != 1 ||
-        g0.streamk || g1.streamk)
+    if (g0.tiles_m != (g0.M + tile - 1) / tile || g0.tiles_n != (g0.N + tile - 1) / tile || g1.tiles_m != (g1.M + tile - 1) / tile ||
+        g1.tiles_n != (g1.N + tile - 1) / tile || t0 <= 0 || t1 <= 0 || t0 + t1 + (1LL << 22) > 0x7fffffffLL || g0.split_k != 1 || g1.split_k != 1 ||
+        g0.streamk || g1.streamk || g0.K <= 0 || g1.K <= 0 || g0.k_per_slice < g0.K || g1.k_per_slice < g1.K)
         return set_error(MNI_ERR_INVALID, "sgemm: paired tile kernel launched with a wrong plan");
     GemmPairLaunch p;
     p.g[0] = g0;
     p.g[1] = g1;
     p.tiles0 = (unsigned)t0;
     p.tiles1 = (unsigned)t1;
-    p.wgs0 = (unsigned)((t0 + 7) / 8 * 8);
-    const dim3 grid(p.wgs0 + p.tiles1), block(NTHREADS);
-    hipStream_t s = ctx().stream;
-    if (bmode0 == 0 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 0, 1>), grid, block, 0, s, p);
-    else if (bmode0 == 0 && amode1 == 1) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 1, 1>), grid, block, 0, s, p);
-    else if (bmode0 == 1 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 0, 1>), grid, block, 0, s, p);
-    else MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 1, 1>), grid, block, 0, s, p);
+    p.lead = g1.K > g0.K ? 1u : 0u;
+    p.wgs_lead = (unsigned)(((p.lead ? t1 : t0) + 7) / 8 * 8);
+    p.cs_src = colsum ? colsum->src : nullptr;
+    p.cs_out = colsum ? colsum->out : nullptr;
+    p.cs_rows = colsum ? (int)colsum->rows : 0;
+    p.cs_cols = colsum ? (int)colsum->cols : 0;
+    p.cs_wgs = colsum ? (unsigned)((colsum->cols + PAIR_CS_COLS - 1) / PAIR_CS_COLS) : 0u;   // (at most 2^21)
+    const dim3 grid(p.wgs_lead + (p.lead ? p.tiles0 : p.tiles1) + p.cs_wgs);
+    if (tile == 128) launch_pair_modes<2>(p, bmode0, amode1, grid);
+    else launch_pair_modes<1>(p, bmode0, amode1, grid);
     return check_launch("gemm_mfma_pair_kernel");
 }
 

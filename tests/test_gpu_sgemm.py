@@ -709,15 +709,78 @@ def test_pair_launch_of_small_and_of_big_products(dev, rocm, oracle_native):
     assert max_err(rocm.to_host(ob, (200, 72)), oracle_native.sgemm_ikj(a.T.copy(), g)) <= gemm_tol(96, a, g)
     with pytest.raises(N.MniError, match="null descriptor"):
         rocm._check(rocm.lib.mni_rocm_sgemm_pair(None, None))
-    # a big pair: each product fills the machine by itself and is launched by itself
+    # a pair with an extent off a multiple of 4 (its edge tiles could not be read in 16-byte pieces along that axis: sgemm cuts
+    # such a product up first): each product is launched by itself
     n = 2048
     big = synth.normal(4, (n, n))
-    dBig, o2, o3 = dev.put(big), dev.empty(n * n), dev.empty(n * n)
+    odd = synth.normal(5, (n - 2, n), stream=1)
+    dBig, dOdd, o2, o3 = dev.put(big), dev.put(odd), dev.empty((n - 2) * n), dev.empty(n * n)
     before = rocm.launch_count()
-    rocm.sgemm_pair(rocm.gemm_desc(n, n, n, dBig, dBig, o2, b_strides=(1, n)), rocm.gemm_desc(n, n, n, dBig, dBig, o3, a_strides=(1, n)))
+    rocm.sgemm_pair(rocm.gemm_desc(n - 2, n, n, dOdd, dBig, o2, b_strides=(1, n)), rocm.gemm_desc(n, n, n - 2, dOdd, dOdd, o3, a_strides=(1, n)))
     assert rocm.launch_count() - before >= 2
-    assert max_err(rocm.to_host(o2, (n, n)), big.astype(np.float64) @ big.T.astype(np.float64)) <= gemm_tol(n, big, big)
-    assert max_err(rocm.to_host(o3, (n, n)), big.T.astype(np.float64) @ big.astype(np.float64)) <= gemm_tol(n, big, big)
+    assert max_err(rocm.to_host(o2, (n - 2, n)), odd.astype(np.float64) @ big.T.astype(np.float64)) <= gemm_tol(n, odd, big)
+    assert max_err(rocm.to_host(o3, (n, n)), odd.T.astype(np.float64) @ odd.astype(np.float64)) <= gemm_tol(n, odd, odd)
+
+
+def _linear_backward_descs(rocm, dev, M, K, Nn, g, x, w, **first):
+    """dx = g . w^T and dw = x^T . g of y[M, Nn] = x[M, K] . w[K, Nn]."""
+    dG, dX, dW = dev.put(g), dev.put(x), dev.put(w)
+    o0, o1 = dev.empty(M * K, fill=-3.0), dev.empty(K * Nn, fill=-3.0)
+    d0 = rocm.gemm_desc(M, K, Nn, dG, dW, o0, b_strides=(1, Nn), **first)
+    d1 = rocm.gemm_desc(K, Nn, M, dX, dG, o1, a_strides=(1, K))
+    return d0, d1, o0, o1
+
+
+@pytest.mark.parametrize("M,K,Nn", [(2048, 2048, 2048), (2044, 2048, 2040), (1920, 2176, 1920), (4096, 4096, 1024)])
+def test_pair_launch_of_big_tiles_gives_the_bits_of_separate_launches(dev, rocm, M, K, Nn):
+    # the two gradients of a Linear layer, each planned alone as whole 128 x 128 tiles: one launch (the second with edges
+    # inside tiles; the third with 255 tiles each, so that a padding workgroup exists; the last with 1024 tiles of
+    # K = 1024 behind 256 of K = 4096, which lead); integer inputs pin the values, normal inputs the order of the K sum
+    for make in (lambda s, shape, st: synth.small_ints(s, shape, 3, stream=st), lambda s, shape, st: synth.normal(s, shape, stream=st)):
+        g, x, w = make(1, (M, Nn), 0), make(2, (M, K), 1), make(3, (K, Nn), 2)
+        d0, d1, o0, o1 = _linear_backward_descs(rocm, dev, M, K, Nn, g, x, w)
+        before = rocm.launch_count()
+        rocm.sgemm_pair(d0, d1)
+        launches = rocm.launch_count() - before
+        got0, got1 = rocm.to_host(o0, (M, K)), rocm.to_host(o1, (K, Nn))
+        rocm.fill(o0, -1.0, M * K)
+        rocm.fill(o1, -1.0, K * Nn)
+        rocm._check(rocm.lib.mni_rocm_sgemm(d0))
+        rocm._check(rocm.lib.mni_rocm_sgemm(d1))
+        assert np.array_equal(got0, rocm.to_host(o0, (M, K)))
+        assert np.array_equal(got1, rocm.to_host(o1, (K, Nn)))
+        assert launches == 1
+        if np.all(g == np.round(g)):
+            assert np.array_equal(got0, (g.astype(np.float64) @ w.T.astype(np.float64)).astype(np.float32))
+            assert np.array_equal(got1, (x.T.astype(np.float64) @ g.astype(np.float64)).astype(np.float32))
+
+
+def test_pair_launch_of_big_tiles_with_the_gelu_backward_epilogue(dev, rocm):
+    # the same pair behind a GELU Linear: the first product scales by gelu'(z + bias) and leaves strip sums for that layer's
+    # bias gradient; still one launch, and the bits of the two products launched apart
+    M, K, Nn = 2048, 2048, 2048
+    g, x, w = synth.normal(1, (M, Nn)), synth.normal(2, (M, K), stream=1), synth.normal(3, (K, Nn), 0.3, stream=2)
+    z, bias = synth.normal(4, (M, K), stream=3), synth.normal(5, (K,), stream=4)
+    dZ, dbias = dev.put(z), dev.put(bias)
+    rows = rocm.sgemm_colsum_rows(M, 1)
+    dP = dev.empty(rows * K, fill=-7.0)
+    d0, d1, o0, o1 = _linear_backward_descs(rocm, dev, M, K, Nn, g, x, w, bias=dbias, epilogue=N.EPI_DGELU, aux=dZ, colsum_part=dP)
+    before = rocm.launch_count()
+    rocm.sgemm_pair(d0, d1)
+    assert rocm.launch_count() - before == 1
+    got0, got1, part = rocm.to_host(o0, (M, K)), rocm.to_host(o1, (K, Nn)), rocm.to_host(dP, (rows, K))
+    rocm.fill(o0, -1.0, M * K)
+    rocm.fill(o1, -1.0, K * Nn)
+    rocm.fill(dP, -1.0, rows * K)
+    rocm._check(rocm.lib.mni_rocm_sgemm(d0))
+    rocm._check(rocm.lib.mni_rocm_sgemm(d1))
+    assert np.array_equal(got0, rocm.to_host(o0, (M, K)))
+    assert np.array_equal(got1, rocm.to_host(o1, (K, Nn)))
+    assert np.array_equal(part, rocm.to_host(dP, (rows, K)))
+    want = (g.astype(np.float64) @ w.T.astype(np.float64)) * _gelu_grad64(z.astype(np.float64) + bias)
+    assert max_err(got0, want) <= gemm_tol(Nn, g, w) * 1.2
+    assert max_err(part.astype(np.float64).sum(0), want.sum(0)) <= gemm_tol(Nn, g, w) * 1.2 * np.sqrt(M)
+    assert max_err(got1, x.T.astype(np.float64) @ g.astype(np.float64)) <= gemm_tol(M, x, g)
 
 
 @pytest.mark.parametrize("m,n,k", [(24, 4096, 4096), (96, 4096, 4096), (128, 1024, 4096), (192, 4096, 1024), (48, 11008, 1024), (64, 512, 16384),
