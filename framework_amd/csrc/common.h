@@ -251,7 +251,7 @@ int k_unbroadcast(float *out, const float *g, const int64_t *gshape, int gnd, co
 int k_cross_entropy(float *loss, float *softmax, const float *logits, int32_t *targets, const int32_t *targets_host,
                     int64_t n, int64_t v, float *grad_for_one = nullptr, bool *wrote_grad = nullptr);
 // out[r] = mean_c (p - t)^2 and its backward (dt may be null)
-int k_mse_rows(float *out, const float *p, const float *t, int64_t rows, int64_t dim);
+int k_mse_rows(float *out, const float *p, const float *t, int64_t rows, int64_t dim, float *seeded = nullptr);  // seeded: also the gradient for an upstream gradient of ones
 int k_mse_rows_backward(float *dp, float *dt, const float *p, const float *t, const float *g, int64_t rows, int64_t dim);
 int k_cross_entropy_backward(float *dlogits, const float *softmax, const int32_t *targets,
                              const float *grad_scalar, int64_t n, int64_t v);

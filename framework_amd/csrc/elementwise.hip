@@ -1073,12 +1073,16 @@ int k_reduce_dim(float *out, const float *a, int64_t outer, int64_t dim, int64_t
 // What mseLoss composes from sub, mul and two means (src/nn.ts:161-165; the second mean runs over the size-1 dim
 // the first one leaves, so the loss is one value per row): out[r] = sum_c (p[r, c] - t[r, c])^2 / dim.
 // One wavefront per row, lanes stride the row (16-byte pieces when the row allows), sums folded in a fixed order.
+// `seeded` (may be null): the gradient for an upstream gradient of all ones, written in the same pass with the
+// arithmetic of the backward kernels below, so that a backward() rooted at this loss has nothing left to launch.
 __global__ void mse_rows_kernel(float *__restrict__ out, const float *__restrict__ p, const float *__restrict__ t, int64_t rows,
-                                int64_t dim, float div, int vec) {
+                                int64_t dim, float div, int vec, float *__restrict__ seeded) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= rows) return;
     const float *pr = p + row * dim, *tr = t + row * dim;
+    float *sr = seeded ? seeded + row * dim : nullptr;
+    const float gr = 1.0f / div;
     float s = 0.f;
     if (vec) {
         const int64_t n4 = dim >> 2;
@@ -1086,23 +1090,30 @@ __global__ void mse_rows_kernel(float *__restrict__ out, const float *__restrict
             const float4 a = reinterpret_cast<const float4 *>(pr)[d], b = reinterpret_cast<const float4 *>(tr)[d];
             const float x = a.x - b.x, y = a.y - b.y, z = a.z - b.z, w = a.w - b.w;
             s += x * x; s += y * y; s += z * z; s += w * w;
+            if (sr) {
+                float4 o;
+                o.x = gr * x; o.y = gr * y; o.z = gr * z; o.w = gr * w;
+                o.x *= 2.0f; o.y *= 2.0f; o.z *= 2.0f; o.w *= 2.0f;
+                reinterpret_cast<float4 *>(sr)[d] = o;
+            }
         }
     } else {
         for (int64_t d = lane; d < dim; d += 64) {
             const float x = pr[d] - tr[d];
             s += x * x;
+            if (sr) sr[d] = 2.0f * (gr * x);
         }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
     if (lane == 0) out[row] = s / div;
 }
-int k_mse_rows(float *out, const float *p, const float *t, int64_t rows, int64_t dim) {
+int k_mse_rows(float *out, const float *p, const float *t, int64_t rows, int64_t dim, float *seeded) {
     if (rows <= 0) return MNI_OK;
     if (dim <= 0) return set_error(MNI_ERR_INVALID, "mse: empty rows");
     MNI_TRY(ensure_init());
-    const int vec = dim % 4 == 0 && ((uintptr_t)p & 15) == 0 && ((uintptr_t)t & 15) == 0;
-    MNI_KERNEL_LAUNCH(mse_rows_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, p, t, rows, dim, (float)dim, vec);
+    const int vec = dim % 4 == 0 && (((uintptr_t)p | (uintptr_t)t | (uintptr_t)seeded) & 15) == 0;
+    MNI_KERNEL_LAUNCH(mse_rows_kernel, dim3(grid_for(rows, 4)), dim3(TPB), 0, ctx().stream, out, p, t, rows, dim, (float)dim, vec, seeded);
     return check_launch("mse_rows");
 }
 // Its backward in one pass: what mean_backward (g / dim), mul_backward (g d for each of the two operands, added up) and

@@ -82,6 +82,7 @@ struct Entry {
     uint32_t aux3 = MNI_BAD_ID; // residual + layernorm: the saved sum x + residual
     std::shared_ptr<void> targets;  // device int32 targets / embedding indices
     BufP ce_grad_for_one;           // cross-entropy of a small batch: d loss / d logits, computed with the loss
+    BufP mse_grad_for_ones;         // fused mseLoss: d loss / d prediction for an upstream gradient of ones, computed with the loss
     int64_t ce_n = 0, ce_v = 0;
     uint64_t rng_seed = 0, rng_offset = 0;  // dropout: where its mask starts in the random stream
 };
@@ -923,10 +924,15 @@ static uint32_t mse_rows_op(uint32_t pred, uint32_t target) {
     BufP p = contiguous_buf(*P);
     BufP t = p ? contiguous_buf(*get(target)) : nullptr;
     BufP o = t ? new_buf((size_t)rows) : nullptr;
-    if (!o || k_mse_rows(o->p, p->p, t->p, rows, dim) != MNI_OK) return MNI_BAD_ID;
+    // (a loss that is differentiated is nearly always the root of backward(), whose gradient is ones_like(loss),
+    // autograd.rs:143: the forward pass, which holds p - t anyway, writes the gradient for that case: one pass over
+    // the operands instead of two)
+    BufP seeded = o && eng().tape.enabled ? new_buf((size_t)(rows * dim)) : nullptr;
+    if (!o || k_mse_rows(o->p, p->p, t->p, rows, dim, seeded ? seeded->p : nullptr) != MNI_OK) return MNI_BAD_ID;
     const uint32_t id = insert_contig(std::move(o), out_shape);
     Entry e;
     e.op = OP_MSEROWS; e.output_id = id; e.n_inputs = 2; e.inputs[0] = pred; e.inputs[1] = target;
+    e.mse_grad_for_ones = std::move(seeded);
     eng().tape.record(std::move(e));
     return id;
 }
@@ -940,6 +946,11 @@ static int mse_rows_backward(uint32_t grad, const Entry &e, int64_t *out) {
     Engine &en = eng();
     const uint32_t tid = e.inputs[1];
     const bool want_t = T->requires_grad || (en.bw_out2entry && tid < en.bw_out2entry->size() && (*en.bw_out2entry)[tid] >= 0);
+    if (e.mse_grad_for_ones && !want_t && ((en.ones && G->buf == en.ones) || (en.one && G->buf == en.one))) {
+        // the upstream gradient is backward()'s own seed of ones: the forward pass has left the result
+        out[0] = insert_contig(BufP(e.mse_grad_for_ones), shape);
+        return MNI_OK;
+    }
     BufP g = contiguous_buf(*G);
     BufP p = g ? contiguous_buf(*get(e.inputs[0])) : nullptr;
     BufP t = p ? contiguous_buf(*get(e.inputs[1])) : nullptr;

@@ -966,8 +966,8 @@ int sgemm_pair(const mni_gemm_desc &d0, const mni_gemm_desc &d1, PairColsum *col
         // the tile counts (see above).
         if ((plan[0].bm == 64 && tiles <= 4LL * cus) || (plan[0].bm == 128 && big)) {
             // the caller's column sums ride along: workgroups behind the tiles that read the matrix once in the launch's tail
-            // (4096 x 1024: two launches of 4.6 us each otherwise; config 4's step 1.512 -> 1.500 ms with both bias
-            // gradients taken this way)
+            // (4096 x 1024: two launches of 4.6 us each otherwise; the training step of a 4096 x 1024 -> 4096 -> 1024
+            // network 1.512 -> 1.500 ms with both bias gradients taken this way)
             const bool with_sums = colsum && gemm_mfma_pair_takes_colsum(*colsum);
             MNI_TRY(launch_gemm_mfma_pair(plan[0].g, plan[0].amode, plan[0].bmode, plan[1].g, plan[1].amode, plan[1].bmode, plan[0].bm,
                                           with_sums ? colsum : nullptr));

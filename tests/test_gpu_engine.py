@@ -384,6 +384,36 @@ def test_fused_mse_loss_is_the_composition_in_one_pass(gpu, orc, shape):
     assert np.array_equal(res["fused"][3], -res["fused"][2])
 
 
+@pytest.mark.parametrize("shape", [(256, 128), (7, 33), (1, 5), (4096, 1024)])
+def test_fused_mse_loss_rooted_backward_takes_the_gradient_the_forward_pass_left(gpu, shape):
+    # backward() rooted at the loss starts from ones: the forward pass has already written the gradient for that case,
+    # with the arithmetic of the backward kernel, so the bits are those of the composition and nothing is launched for
+    # it; a target that wants a gradient, or a second use of the loss, takes the backward kernel
+    p, t = synth.normal(31, shape), synth.normal(32, shape, stream=1)
+    res = {}
+    for fused in (True, False):
+        gpu.native.resetEngine()
+        P = T(gpu, p, True)
+        loss = gpu.mseLoss(P, T(gpu, t), fused=True) if fused else gpu.mseLoss(P, T(gpu, t))
+        before = int(gpu.native.lib.mni_rocm_launch_count())
+        loss.backward()
+        res[fused] = (P.grad.numpy(), int(gpu.native.lib.mni_rocm_launch_count()) - before)
+    assert np.array_equal(res[True][0], res[False][0])
+    assert_close(res[True][0], 2 * (p.astype(np.float64) - t) / shape[-1], 1e-6 * max(1.0, float(np.abs(p - t).max())), "dpred")
+    assert res[True][1] <= 1   # (at most the fill of a seed of a new size)
+    gpu.native.resetEngine()
+    P, Tt = T(gpu, p, True), T(gpu, t, True)
+    gpu.mseLoss(P, Tt, fused=True).backward()
+    assert np.array_equal(P.grad.numpy(), res[False][0]) and np.array_equal(Tt.grad.numpy(), -res[False][0])
+    gpu.native.resetEngine()
+    gpu.native.noGradStart()
+    try:
+        loss = gpu.mseLoss(T(gpu, p), T(gpu, t), fused=True)
+    finally:
+        gpu.native.noGradEnd()
+    assert_close(loss.numpy(), ((p.astype(np.float64) - t) ** 2).mean(-1, keepdims=True), 1e-5, "loss without a tape")
+
+
 def test_fused_mse_loss_views_plain_targets_and_errors(gpu):
     # a permuted prediction is gathered first; a target that asks for no gradient gets none; shapes must be equal
     p, t = synth.normal(21, (40, 24)), synth.normal(22, (24, 40), stream=1)
