@@ -310,7 +310,9 @@ __device__ constexpr int gemm_lds_slots() {
 // loads, afresh for every stream-K segment, instead of being held in scalar registers across the K loop);
 // wg / nwg: this workgroup's number and the number of workgroups of this product, numbered the way the
 // hardware deals workgroups to XCDs (wg % 8 is the XCD); lds: gemm_lds_slots() float4.
-template <int AMODE, int BMODE, int TM, int TN, bool SK>
+// FRESH: the body runs inside a loop of its caller (as it does inside its own loop over stream-K segments): what a thread
+// derives from its id is then derived afresh on every call instead of staying live across the K loop.
+template <int AMODE, int BMODE, int TM, int TN, bool SK, bool FRESH = SK>
 __device__ __forceinline__ void gemm_mfma_body(LaunchPtr gp, const unsigned wg, const unsigned nwg, float4 *__restrict__ lds) {
 #define g (*gp)
     constexpr int AL = AMODE == 1 ? 1 : 0;
@@ -364,7 +366,7 @@ __device__ __forceinline__ void gemm_mfma_body(LaunchPtr gp, const unsigned wg, 
     // segment loop, those addresses would stay live across it and spill.
     int tid = threadIdx.x;
     unsigned bid = wg;
-    if (SK) {
+    if (SK || FRESH) {
         asm volatile("" : "+v"(tid));
         asm volatile("" : "+s"(gp));
         asm volatile("" : "+s"(bid));
@@ -872,6 +874,13 @@ __global__ __launch_bounds__(NTHREADS, (TM * TN >= 2 ? 2 : 4)) void gemm_mfma_ke
 struct GemmPairLaunch {
     GemmLaunch g[2];
     unsigned lead, wgs_lead, tiles0, tiles1;
+    // The other product's workgroups: wgs_other of them, each working through `chunk` tiles one after the other (tiles w,
+    // w + wgs_other, ...).  chunk > 1 when the lead's K is that many times the other's and the whole launch is resident
+    // at once: every workgroup then has the same number of K steps before it, and which CU gets how many of the short
+    // tiles is no longer left to the order in which workgroup slots happen to fall free (1024 tiles of K = 1024 behind
+    // 256 of K = 4096 took 492 us on most launches and 546 on one in four; four short tiles per workgroup: every launch
+    // the same).
+    unsigned wgs_other, chunk;
     // Column sums that ride along (a Linear layer's bias gradient: the sums of the matrix both products read): cs_out[c] =
     // sum over r of cs_src[r, c] for a contiguous [cs_rows, cs_cols] matrix, by cs_wgs workgroups behind the products'
     // (0: none), PAIR_CS_COLS columns each.  Behind, because a workgroup ahead of the tiles would take a tile's place in
@@ -928,14 +937,15 @@ __device__ __forceinline__ void pair_colsum_role(PairPtr pp, const unsigned b, f
     }
 }
 
-template <int AM0, int BM0, int AM1, int BM1, int T>
+// CHUNKED: the instantiation for chunk > 1 (a loop around the body; the plain one keeps the body's straight-line code)
+template <int AM0, int BM0, int AM1, int BM1, int T, bool CHUNKED>
 __global__ __launch_bounds__(NTHREADS, (T >= 2 ? 2 : 4)) void gemm_mfma_pair_kernel(const GemmPairLaunch pair_args) {
     (void)pair_args;
     PairPtr pp = (PairPtr)__builtin_amdgcn_kernarg_segment_ptr();
     constexpr int S0 = gemm_lds_slots<AM0, BM0, T, T>(), S1 = gemm_lds_slots<AM1, BM1, T, T>();
     static_assert(S0 >= NTHREADS && S1 >= NTHREADS, "the column sums park one float4 per thread");
     __shared__ float4 lds[S0 > S1 ? S0 : S1];
-    const unsigned b = blockIdx.x, tile_wgs = pp->wgs_lead + (pp->lead ? pp->tiles0 : pp->tiles1);
+    const unsigned b = blockIdx.x, tile_wgs = pp->wgs_lead + pp->wgs_other;
     if (b >= tile_wgs) {
         pair_colsum_role(pp, b - tile_wgs, lds);
         return;
@@ -943,10 +953,27 @@ __global__ __launch_bounds__(NTHREADS, (T >= 2 ? 2 : 4)) void gemm_mfma_pair_ker
     const bool in_lead = b < pp->wgs_lead;
     const unsigned wg = in_lead ? b : b - pp->wgs_lead;
     const unsigned which = in_lead ? pp->lead : 1u - pp->lead;
-    if (which == 0) {
-        if (wg < pp->tiles0) gemm_mfma_body<AM0, BM0, T, T, false>(&pp->g[0], wg, pp->tiles0, lds);
+    if constexpr (!CHUNKED) {
+        if (which == 0) {
+            if (wg < pp->tiles0) gemm_mfma_body<AM0, BM0, T, T, false>(&pp->g[0], wg, pp->tiles0, lds);
+        } else {
+            if (wg < pp->tiles1) gemm_mfma_body<AM1, BM1, T, T, false>(&pp->g[1], wg, pp->tiles1, lds);
+        }
     } else {
-        if (wg < pp->tiles1) gemm_mfma_body<AM1, BM1, T, T, false>(&pp->g[1], wg, pp->tiles1, lds);
+        const unsigned reps = in_lead ? 1u : pp->chunk, stride = pp->wgs_other;
+        if (which == 0) {
+            for (unsigned rep = 0; rep < reps; ++rep) {
+                const unsigned w = wg + rep * stride;
+                if (w < pp->tiles0) gemm_mfma_body<AM0, BM0, T, T, false, true>(&pp->g[0], w, pp->tiles0, lds);
+                if (rep + 1 < reps) __syncthreads();  // (the next tile's prologue writes LDS that this one's epilogue still reads)
+            }
+        } else {
+            for (unsigned rep = 0; rep < reps; ++rep) {
+                const unsigned w = wg + rep * stride;
+                if (w < pp->tiles1) gemm_mfma_body<AM1, BM1, T, T, false, true>(&pp->g[1], w, pp->tiles1, lds);
+                if (rep + 1 < reps) __syncthreads();
+            }
+        }
     }
 }
 
@@ -1018,14 +1045,14 @@ bool gemm_mfma_pair_eligible(int amode0, int bmode0, int amode1, int bmode1) {
     return amode0 == 0 && bmode0 <= 1 && amode1 <= 1 && bmode1 == 1;
 }
 
-template <int T>
+template <int T, bool CHUNKED>
 static void launch_pair_modes(const GemmPairLaunch &p, int bmode0, int amode1, dim3 grid) {
     const dim3 block(NTHREADS);
     hipStream_t s = ctx().stream;
-    if (bmode0 == 0 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 0, 1, T>), grid, block, 0, s, p);
-    else if (bmode0 == 0 && amode1 == 1) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 1, 1, T>), grid, block, 0, s, p);
-    else if (bmode0 == 1 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 0, 1, T>), grid, block, 0, s, p);
-    else MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 1, 1, T>), grid, block, 0, s, p);
+    if (bmode0 == 0 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 0, 1, T, CHUNKED>), grid, block, 0, s, p);
+    else if (bmode0 == 0 && amode1 == 1) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 0, 1, 1, T, CHUNKED>), grid, block, 0, s, p);
+    else if (bmode0 == 1 && amode1 == 0) MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 0, 1, T, CHUNKED>), grid, block, 0, s, p);
+    else MNI_KERNEL_LAUNCH((gemm_mfma_pair_kernel<0, 1, 1, 1, T, CHUNKED>), grid, block, 0, s, p);
 }
 
 bool gemm_mfma_pair_takes_colsum(const PairColsum &cs) {
@@ -1052,14 +1079,24 @@ int launch_gemm_mfma_pair(const GemmLaunch &g0, int amode0, int bmode0, const Ge
     p.tiles1 = (unsigned)t1;
     p.lead = g1.K > g0.K ? 1u : 0u;
     p.wgs_lead = (unsigned)(((p.lead ? t1 : t0) + 7) / 8 * 8);
+    {
+        const int64_t k_lead = p.lead ? g1.K : g0.K, k_other = p.lead ? g0.K : g1.K, t_other = p.lead ? t0 : t1;
+        const int64_t c = k_lead / k_other;
+        const int64_t slots = (int64_t)(ctx().compute_units > 0 ? ctx().compute_units : 256) * gemm_mfma_resident_per_cu(tile, tile);
+        const bool even = c >= 2 && c <= 8 && t_other % c == 0 && (t_other / c) % 8 == 0 && (int64_t)p.wgs_lead + t_other / c <= slots;
+        p.chunk = even ? (unsigned)c : 1u;
+        p.wgs_other = (unsigned)(t_other / p.chunk);
+    }
     p.cs_src = colsum ? colsum->src : nullptr;
     p.cs_out = colsum ? colsum->out : nullptr;
     p.cs_rows = colsum ? (int)colsum->rows : 0;
     p.cs_cols = colsum ? (int)colsum->cols : 0;
     p.cs_wgs = colsum ? (unsigned)((colsum->cols + PAIR_CS_COLS - 1) / PAIR_CS_COLS) : 0u;   // (at most 2^21)
-    const dim3 grid(p.wgs_lead + (p.lead ? p.tiles0 : p.tiles1) + p.cs_wgs);
-    if (tile == 128) launch_pair_modes<2>(p, bmode0, amode1, grid);
-    else launch_pair_modes<1>(p, bmode0, amode1, grid);
+    const dim3 grid(p.wgs_lead + p.wgs_other + p.cs_wgs);
+    if (tile == 128 && p.chunk > 1) launch_pair_modes<2, true>(p, bmode0, amode1, grid);
+    else if (tile == 128) launch_pair_modes<2, false>(p, bmode0, amode1, grid);
+    else if (p.chunk > 1) launch_pair_modes<1, true>(p, bmode0, amode1, grid);
+    else launch_pair_modes<1, false>(p, bmode0, amode1, grid);
     return check_launch("gemm_mfma_pair_kernel");
 }
 

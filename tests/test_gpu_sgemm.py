@@ -731,11 +731,12 @@ def _linear_backward_descs(rocm, dev, M, K, Nn, g, x, w, **first):
     return d0, d1, o0, o1
 
 
-@pytest.mark.parametrize("M,K,Nn", [(2048, 2048, 2048), (2044, 2048, 2040), (1920, 2176, 1920), (4096, 4096, 1024)])
+@pytest.mark.parametrize("M,K,Nn", [(2048, 2048, 2048), (2044, 2048, 2040), (1920, 2176, 1920), (4096, 4096, 1024), (1024, 4096, 2048)])
 def test_pair_launch_of_big_tiles_gives_the_bits_of_separate_launches(dev, rocm, M, K, Nn):
     # the two gradients of a Linear layer, each planned alone as whole 128 x 128 tiles: one launch (the second with edges
-    # inside tiles; the third with 255 tiles each, so that a padding workgroup exists; the last with 1024 tiles of
-    # K = 1024 behind 256 of K = 4096, which lead); integer inputs pin the values, normal inputs the order of the K sum
+    # inside tiles; the third with 255 tiles each, so that a padding workgroup exists; the fourth with 1024 tiles of
+    # K = 1024 behind 256 of K = 4096, which lead, four short tiles to a workgroup; the last with the first product
+    # leading and two tiles to a workgroup of the second); integer inputs pin the values, normal inputs the order of the K sum
     for make in (lambda s, shape, st: synth.small_ints(s, shape, 3, stream=st), lambda s, shape, st: synth.normal(s, shape, stream=st)):
         g, x, w = make(1, (M, Nn), 0), make(2, (M, K), 1), make(3, (K, Nn), 2)
         d0, d1, o0, o1 = _linear_backward_descs(rocm, dev, M, K, Nn, g, x, w)
