@@ -278,6 +278,20 @@ def bench_extras(r, with_cpu):
         r.free(xb)
         r.free(yb)
     out["decode_batch_rows_x_4096x4096_cold"] = rows_out
+    # the same buffers read as W stored [out, in]: rows . W^T, the layout of dX = dY W^T under a small batch (matmul_backward's
+    # first product against a weight kept [in, out]) and of a Linear whose weight is kept transposed -- not a BASELINE config
+    rows_t = {}
+    for mrows in (1, 4, 8, 16):
+        xb = r.to_device(synth.normal(5, (mrows, 4096)))
+        yb = r.malloc(mrows * 4096 * 4)
+        descs = [r.gemm_desc(mrows, 4096, 4096, xb, wp, yb, b_strides=(1, 4096)) for wp in ws]
+        r.sgemm_timed(descs, 100, 200)
+        us = min(r.sgemm_timed(descs, 20, 200) for _ in range(3)) * 1e3
+        byb = 4.0 * (4096 * 4096 + 2 * mrows * 4096)
+        rows_t["%d_rows" % mrows] = {"us": us, "GB/s": byb / us / 1e3, "frac_hbm": byb / us / 1e3 / PEAK_HBM_GBPS}
+        r.free(xb)
+        r.free(yb)
+    out["rows_x_transposed_4096x4096_weight_cold"] = rows_t
     # token rows against a weight stored [out, in] (a tied language-model head: logits = x E^T with E [50304, 768]), E cold
     # (four in rotation, 618 MB) -- not a BASELINE config
     head_out = {}

@@ -393,6 +393,50 @@ static bool fewrows_nt_plan(const GemmLaunch &g, int cus) {
     (void)cus;
     return g.M > 4 && g.M <= 16 && g.K >= 512 && g.N >= 4096;
 }
+// K slices for the sliced form of that kernel (0: not this form).  A slice is a run of steps of 64 values of K, at most
+// as many as the kernel keeps in flight; a workgroup is 64 columns x one slice and has a CU to itself, so a plan costs
+// rounds of workgroups x steps of the longest slice, plus something per slice for the sum at the end.
+static int fewrows_nt_slices(const GemmLaunch &g, int cus, int want) {
+    const int ksteps = g.K / 64, maxs = fewrows_nt_max_steps(g.M);
+    const int smin = std::max(2, (ksteps + maxs - 1) / maxs), smax = std::min(ksteps, FEWROWS_NT_MAX_SLICES);
+    if (smin > smax) return 0;
+    if (want > 0) return want >= smin && want <= smax ? want : 0;
+    const int64_t units8 = 8 * (int64_t)(((g.N + 63) / 64 + 7) / 8);
+    int best = 0;
+    double best_cost = 0.0;
+    for (int s = smin; s <= smax; ++s) {
+        // a round of workgroups costs its steps (0.7 us each: 256 CUs x 64 columns x 64 values) and about 5 us besides
+        // (A into LDS ahead of the first request for W; partial sums acknowledged, counted and added behind the last)
+        const int64_t rounds = (units8 * s + cus - 1) / cus;
+        const double cost = (double)rounds * ((ksteps + s - 1) / s + 7);
+        if (best == 0 || cost < best_cost - 1e-9) { best = s; best_cost = cost; }
+    }
+    return best;
+}
+// Measured cold on MI355X (us; this form / the dots kernel / 64 x 64 tiles in K slices), W [N, K]:
+//    rows    4096 x 4096        8192 x 8192         32000 x 4096          4096 x 11008        1024 x 8192         4096 x 2048         2048 x 2048
+//      1   14.2 / 17.7 / 24.7   49.5 / 54.0 / 87.2   94.9 /  96.5 / 127   36.3 / 43.5 / 64.7   14.3 / 21.4 / 18.2   12.1 / 10.2 / 15.2   12.7 /  8.0 / 14.3
+//      4   14.5 / 18.7 / 25.1   51.1 / 55.3 / 88.3   96.7 /  97.6 / 129   38.1 / 44.5 / 65.0   15.1 / 22.9 / 18.4   12.4 / 11.3 / 15.1   13.2 /  9.2 / 14.6
+//      8   15.1 / 22.8 / 25.3   53.8 / 61.6 / 88.5  100.3 / 113.7 / 129   41.9 / 51.8 / 65.5   17.1 / 30.6 / 18.9   13.1 / 14.9 / 15.6   14.3 / 12.7 / 14.8
+//     16   17.1 / 31.7 / 25.7   62.7 / 88.6 / 89.6  112.5 / 167.5 / 131   52.4 / 67.4 / 66.4   21.9 / 45.2 / 19.1   15.4 / 22.0 / 15.9   17.2 / 20.1 / 15.1
+// (the same weights stored [K, N] take 12.2-14.1 us at 4096 x 4096 through the decode product).  With 17 to 32 rows the 32
+// MFMAs per load weigh: 41-45 us against the tiles' 28 at 4096 x 4096.
+static bool fewrows_nt_sliced_plan(const GemmLaunch &g, int cus) {
+    (void)cus;
+    const int kmax = FEWROWS_NT_LDS_FLOATS / 16 - 16;  // (up to there the unsliced form holds A in LDS)
+    if (g.M > 16 || g.K <= kmax || (int64_t)g.N * g.K < (1 << 23)) return false;
+    return g.M > 8 ? g.N >= 2048 : (g.K >= 4096 || g.M >= 8);
+}
+// Whether run_mfma gives the product to the sliced form by itself.
+static bool fewrows_nt_sliced_takes(const GemmLaunch &g, int amode, int bmode) {
+    DeviceCtx &c = ctx();
+    const int cus = c.compute_units > 0 ? c.compute_units : 256;
+    if (!gemm_fewrows_nt_sliced_eligible(g, amode, bmode) || c.xcd_count != 8 || (size_t)((g.N + 63) / 64 + 7) > c.fewrows_counter_cap) return false;
+    if (!fewrows_nt_sliced_plan(g, cus)) return false;
+    const int fs = fewrows_nt_slices(g, cus, 0);
+    // (a caller that cannot allocate gets the plan only when the fixed scratch holds its partial sums)
+    return fs > 0 && !(c.scratch && fewrows_nt_sliced_ws_floats(g.N, fs) * sizeof(float) > c.scratch_bytes);
+}
 // Whether run_mfma would give the product to the few-rows kernel by itself.
 static bool fewrows_takes(const mni_gemm_desc &d) {
     if (d.K == 0 || d.epilogue >= MNI_EPI_BIAS_GELU_DUAL) return false;
@@ -402,6 +446,7 @@ static bool fewrows_takes(const mni_gemm_desc &d) {
     const int amode = classify(g.a_cs, g.a_rs), bmode = classify(g.b_rs, g.b_cs);
     const int cus = c.compute_units > 0 ? c.compute_units : 256;
     if (gemm_fewrows_nt_eligible(g, amode, bmode) && fewrows_nt_plan(g, cus)) return true;  // (its twin for a K-contiguous B)
+    if (fewrows_nt_sliced_takes(g, amode, bmode)) return true;
     return gemm_fewrows_eligible(g, amode, bmode) && (size_t)((g.N + 127) / 128) * g.batch <= c.fewrows_counter_cap && c.xcd_count == 8 &&
            fewrows_plan(g, cus);
 }
@@ -477,6 +522,28 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
         g.streamk = 0; g.sk_wpx = 0; g.sk_xcds = 0; g.sk_flags = nullptr; g.sk_epoch = 0; g.status = c.status_dev;
         if (probe) { probe->kind = PlanProbe::OUTER; return MNI_OK; }
         return launch_gemm_outer(g);
+    }
+    // The same in K slices: forced with a split_k or a K beyond the unsliced form's LDS, or chosen by fewrows_nt_sliced_plan.
+    {
+        const bool fs_ok = gemm_fewrows_nt_sliced_eligible(g, amode, bmode) && c.xcd_count == 8 && (size_t)((g.N + 63) / 64 + 7) <= c.fewrows_counter_cap;
+        int fs = 0;
+        if (d.algo == MNI_ALGO_FEWROWS_NT && (d.split_k > 1 || !gemm_fewrows_nt_eligible(g, amode, bmode))) {
+            fs = fs_ok ? fewrows_nt_slices(g, cus, d.split_k > 1 ? d.split_k : 0) : 0;
+            if (fs == 0)
+                return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel for a K-contiguous B takes one product of up to 32 rows of a K-contiguous A, operands "
+                                                  "16-byte aligned, K %% 64 == 0; at most 1984 (960 beyond 16 rows) in one piece, or in 2 to 16 slices (split_k) of at "
+                                                  "most 1024 (768) each");
+        } else if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && fewrows_nt_sliced_takes(g, amode, bmode)) {
+            fs = fewrows_nt_slices(g, cus, 0);
+        }
+        if (fs > 0) {
+            if (probe) { probe->kind = PlanProbe::FEWROWS; return MNI_OK; }
+            void *fws = nullptr;
+            MNI_TRY(gemm_ws_alloc(&fws, fewrows_nt_sliced_ws_floats(g.N, fs) * sizeof(float)));
+            const int rc = launch_gemm_fewrows_nt_sliced(g, amode, bmode, fs, (float *)fws, c.fewrows_counters);
+            gemm_ws_free(fws);
+            return rc;
+        }
     }
     // Few rows against a wide K-contiguous operand (a weight stored [out, in]): forced, or chosen by fewrows_nt_plan.
     if (d.algo == MNI_ALGO_FEWROWS_NT || (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_fewrows_nt_eligible(g, amode, bmode) && fewrows_nt_plan(g, cus))) {
@@ -834,7 +901,8 @@ int sgemm(const mni_gemm_desc &d) {
         int rc16 = MNI_OK;
         if (try_gemv_units(s, d, &rc16)) return rc16;
     }
-    const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M > 4 && d.M <= 16 && fewrows_takes(d);
+    // (the sliced form of the kernel for a K-contiguous B also takes 1 to 4 rows: 4 x 4096 x 4096 14.6 us against the dots kernel's 18.7)
+    const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M <= 16 && fewrows_takes(d);
     if (!to_fewrows &&
         ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS ||
          d.algo == MNI_ALGO_GEMV)) {

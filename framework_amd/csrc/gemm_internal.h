@@ -173,9 +173,21 @@ struct FewNtLaunch {
     int M, N, K;
     int64_t x_rs, w_cs, o_rs;
     int epilogue, accumulate;
+    // the form with K in slices only (null / zero otherwise):
+    float *ws;        // partial sums [column block of 64][slice][column 64][row 16]
+    unsigned *count;  // one counter per column block, zero between launches (each wraps to zero with its last arrival)
+    int slices;       // K slices: runs of K's steps of 64 values, the first ksteps % slices of them one step longer
+    int ksteps;       // K / 64
 };
 bool gemm_fewrows_nt_eligible(const GemmLaunch &g, int amode, int bmode);
 int launch_gemm_fewrows_nt(const GemmLaunch &g, int amode, int bmode);
+// The same product with K beyond what LDS holds of A, or too few columns to give every CU a workgroup: K in slices
+// (workgroup = 64 columns x one slice), the slices of a column block added up by the last of them to arrive.
+static constexpr int FEWROWS_NT_MAX_SLICES = 16;
+bool gemm_fewrows_nt_sliced_eligible(const GemmLaunch &g, int amode, int bmode);
+int fewrows_nt_max_steps(int rows);  // steps of 64 values of K a slice may have with that many rows of A
+size_t fewrows_nt_sliced_ws_floats(int N, int slices);
+int launch_gemm_fewrows_nt_sliced(const GemmLaunch &g, int amode, int bmode, int slices, float *ws, unsigned *count);
 
 // Sums split-K partials ws[slice][batch][rows][cols] in slice order and
 // applies the epilogue; out addressed with (o_bs, o_rs, o_cs).

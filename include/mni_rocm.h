@@ -155,11 +155,14 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * in whole 16 bytes, and no activation together with accumulate);
  * FEWROWS_NT = up to 32 rows of a
  * K-contiguous A against a wide B that is K-contiguous too (a weight stored
- * [out, in], given as its transposed view): a wavefront per 16 columns and
- * all of K on the 16 x 16 x 4 MFMA, A resident in LDS, no sums across
- * wavefronts (error unless one batch, K % 64 == 0 and at most 1984, 960
- * beyond 16 rows, both operands 16-byte aligned with pitches in whole 16
- * bytes, no split_k).  AUTO picks among them. */
+ * [out, in], given as its transposed view): a wavefront per 4 columns on
+ * the 4 x 4 x 1 MFMA, A resident in LDS; with K up to 1984 (960 beyond 16
+ * rows) all of K per wavefront and no sums across wavefronts, with a larger
+ * K, or with a split_k of 2 to 16, K in that many slices of at most 1024
+ * values (768 beyond 16 rows) that the last workgroup of a column block to
+ * arrive adds up (error unless one batch, K % 64 == 0 and within those
+ * limits, both operands 16-byte aligned with pitches in whole 16 bytes).
+ * AUTO picks among them. */
 enum { MNI_ALGO_AUTO = 0, MNI_ALGO_MFMA = 1, MNI_ALGO_SKINNY = 2, MNI_ALGO_MFMA_SMALL = 3, MNI_ALGO_SKINNY_TWO_PASS = 4,
        MNI_ALGO_MFMA_STREAMK = 5, MNI_ALGO_DIRECT = 6, MNI_ALGO_PANEL = 7, MNI_ALGO_TINY = 8, MNI_ALGO_FEWROWS = 9,
        MNI_ALGO_OUTER = 10, MNI_ALGO_GEMV = 11, MNI_ALGO_FEWROWS_NT = 12 };

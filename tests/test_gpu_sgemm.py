@@ -1235,12 +1235,73 @@ def test_fewrows_nt_kernel_normal_inputs_and_what_it_refuses(dev, rocm):
     got = run_gemm(dev, a, bt, False, True, algo=N.ALGO_FEWROWS_NT)[0]
     assert max_err(got, want) <= gemm_tol(k, a, bt)
     assert np.array_equal(got, run_gemm(dev, a, bt, False, True, algo=N.ALGO_FEWROWS_NT)[0])
-    # 40 rows; K off a multiple of 64; K beyond what LDS holds for 32 rows; a row-major B
-    for mm, kk, tb in ((40, 256, True), (16, 208, True), (32, 1024, True), (16, 256, False)):
+    # 40 rows; K off a multiple of 64; a row-major B  (a K beyond what LDS holds of A goes to the form with K in slices)
+    for mm, kk, tb in ((40, 256, True), (16, 208, True), (16, 256, False)):
         aa = synth.small_ints(1, (mm, kk), 3)
         bb = synth.small_ints(2, (20000, kk) if tb else (kk, 20000), 3, stream=1)
         with pytest.raises(N.MniError, match="few-rows kernel for a K-contiguous B"):
             run_gemm(dev, aa, bb, False, tb, algo=N.ALGO_FEWROWS_NT)
+
+
+@pytest.mark.parametrize("m,n,k,split", [(16, 4096, 4096, 0), (16, 4096, 4096, 8), (16, 4096, 4096, 16), (9, 1000, 2048, 0), (1, 4096, 4096, 0),
+                                          (4, 2050, 5120, 5), (8, 11008, 4096, 0), (12, 192, 2816, 3), (16, 64, 512, 2), (32, 4096, 4096, 0),
+                                          (17, 1111, 1536, 2), (24, 8192, 3072, 0), (3, 70, 1024, 4), (13, 3000, 2112, 0), (32, 500, 1088, 0),
+                                          (7, 4096, 2240, 3)])
+def test_fewrows_nt_kernel_in_k_slices_integer_exact(dev, rocm, m, n, k, split):
+    # K beyond what LDS holds of A: workgroups of 64 columns x one K slice, the last slice of a column block to arrive adds
+    # them.  Even and uneven slices, column counts off a multiple of 64 and under one block, 1 to 32 rows; forced (with
+    # and without a slice count) and as the planner's choice; twice in a row (the counters wrap back to zero)
+    a = synth.small_ints(m + n, (m, k), 3)
+    bt = synth.small_ints(n + k, (n, k), 3, stream=1)
+    want = (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float32)
+    for _ in range(2):
+        assert np.array_equal(run_gemm(dev, a, bt, False, True, algo=N.ALGO_FEWROWS_NT, split_k=split)[0], want)
+    assert np.array_equal(run_gemm(dev, a, bt, False, True)[0], want)  # (the planner's choice, whichever kernel that is)
+
+
+@pytest.mark.parametrize("m,n,k,split", [(16, 4100, 2048, 2), (30, 2000, 1536, 3)])
+def test_fewrows_nt_kernel_in_k_slices_epilogues_accumulate_and_pitches(dev, rocm, m, n, k, split):
+    a = synth.small_ints(m, (m, k), 3); bt = synth.small_ints(m + 1, (n, k), 3, stream=1)
+    bias = synth.small_ints(m + 2, (n,), 5, stream=2); old = synth.small_ints(m + 3, (m, n), 9, stream=3)
+    prod = (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float64)
+    lda, ldb, ldc = k + 8, k + 12, n + 3  # pitches off their extents (operands in whole 16-byte pieces, C any)
+    sa = np.zeros((m, lda), np.float32); sa[:, :k] = a
+    sb = np.zeros((n, ldb), np.float32); sb[:, :k] = bt
+    dA, dB, dBias = dev.put(sa), dev.put(sb), dev.put(bias)
+    for epi, accumulate in [(N.EPI_NONE, False), (N.EPI_NONE, True), (N.EPI_BIAS, False), (N.EPI_BIAS, True), (N.EPI_BIAS_RELU, True),
+                            (N.EPI_BIAS_GELU, False)]:
+        z = prod + (bias if epi != N.EPI_NONE else 0.0)
+        if epi == N.EPI_BIAS_RELU: z = np.maximum(z, 0.0)
+        if epi == N.EPI_BIAS_GELU: z = 0.5 * z * (1.0 + np.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        want = z + (old if accumulate else 0.0)
+        sc = np.full((m, ldc), -5.0, np.float32); sc[:, :n] = old
+        dC = dev.put(sc)
+        rocm.sgemm(m, n, k, dA, dB, dC, a_strides=(lda, 1), b_strides=(1, ldb), ldc=ldc, bias=dBias if epi != N.EPI_NONE else None, epilogue=epi,
+                   accumulate=accumulate, algo=N.ALGO_FEWROWS_NT, split_k=split)
+        got = rocm.to_host(dC, (m, ldc))
+        assert np.all(got[:, n:] == -5.0), "the padding of C was written"
+        if epi == N.EPI_BIAS_GELU:
+            assert np.abs(got[:, :n] - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), (epi, accumulate)
+        else:
+            assert np.array_equal(got[:, :n], want.astype(np.float32)), (epi, accumulate)
+
+
+def test_fewrows_nt_kernel_in_k_slices_normal_inputs_and_what_it_refuses(dev, rocm):
+    m, n, k = 16, 4096, 4096
+    a = synth.normal(61, (m, k), 0.05); bt = synth.normal(62, (n, k), 0.05, stream=1)
+    want = a.astype(np.float64) @ bt.T.astype(np.float64)
+    got = run_gemm(dev, a, bt, False, True)[0]
+    assert max_err(got, want) <= gemm_tol(k, a, bt)
+    for _ in range(3):  # the same bits whoever of a column block's slices arrives last
+        assert np.array_equal(got, run_gemm(dev, a, bt, False, True)[0])
+    assert np.array_equal(got, run_gemm(dev, a, bt, False, True, algo=N.ALGO_FEWROWS_NT, split_k=4)[0])
+    # slices longer than 16 steps of 64; more slices than steps; more than 16 slices; K off a multiple of 64; 32 rows of a K
+    # that 16 slices of 12 steps do not cover
+    for mm, kk, split in ((16, 4096, 2), (16, 256, 5), (16, 8192, 17), (16, 2400, 3), (32, 12352, 0)):
+        aa = synth.small_ints(1, (mm, kk), 3)
+        bb = synth.small_ints(2, (512, kk), 3, stream=1)
+        with pytest.raises(N.MniError, match="few-rows kernel for a K-contiguous B"):
+            run_gemm(dev, aa, bb, False, True, algo=N.ALGO_FEWROWS_NT, split_k=split)
 
 
 @pytest.mark.parametrize("m", [1, 3, 5, 7])
