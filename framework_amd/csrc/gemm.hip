@@ -389,9 +389,18 @@ static bool fewrows_plan(const GemmLaunch &g, int cus) {
 // 12 x 262144 x 64 129 / 30), under 4096 columns (12 x 2048 x 1024 10.0 / 9.1), with four rows or fewer
 // (4 x 32000 x 1024 36.2 / 29.1) and beyond 16 rows, where eight LDS reads and 32 MFMAs per load add up
 // (32 x 50304 x 768 56.4 / 51.3).
+// Since A's values for a step are asked of LDS a step ahead (this kernel / the dots kernel up to 8 rows / tiles, us, cold):
+// 1 x 50304 x 768 24.9 / 28.8 / 47.8, 4 rows 27.0 / 31.3, 16 rows 33.5, 32 rows 47.2 / - / 53.5; 1 x 16384 x 768 9.9 / 12.1, 4 x 4096 x 768
+// 5.3 / 6.9, 4 x 32768 x 1984 42.0 / 50.4, 4 x 2048 x 1024 5.6 / 7.2, 3 x 1024 x 1024 4.7 / 6.3, 2 x 8192 x 640 6.4 / 7.7, 8 x 2048 x 1024 6.4 / 10.2,
+// 16 x 2048 x 1024 9.1 / 16.5 / 14.3, 16 x 3072 x 1536 10.6 / 18.4 / 15.6, 20 x 12288 x 768 15.6 / - / 24.1, 32 x 8192 x 768 12.8 / - / 16.8; level at
+// 1 x 32000 x 1024 (27.8 / 27.3) and 2 x 4096 x 1984 (9.2 / 9.1); behind at K = 512 and below (4 x 128256 x 512 57.0 / 51.3, 1 x 65536 x 256
+// 25.7 / 20.2) and, beyond 16 rows, wherever K is not 768: the steps past the last in the ring of 12 loads multiply zeros, 32 MFMAs each
+// (24 x 8192 x 960 17.4 against 15.5, 32 x 32000 x 960 50.4 against 36.5).
 static bool fewrows_nt_plan(const GemmLaunch &g, int cus) {
     (void)cus;
-    return g.M > 4 && g.M <= 16 && g.K >= 512 && g.N >= 4096;
+    if (g.M > 16) return g.K == 768 && g.N >= 8192;
+    if (g.M > 4) return g.K >= 512 && g.N >= 2048;
+    return g.K >= 640 && g.N >= 1024;
 }
 // K slices for the sliced form of that kernel (0: not this form).  A slice is a run of steps of 64 values of K, at most
 // as many as the kernel keeps in flight; a workgroup is 64 columns x one slice and has a CU to itself, so a plan costs
@@ -902,7 +911,7 @@ int sgemm(const mni_gemm_desc &d) {
         if (try_gemv_units(s, d, &rc16)) return rc16;
     }
     // (the sliced form of the kernel for a K-contiguous B also takes 1 to 4 rows: 4 x 4096 x 4096 14.6 us against the dots kernel's 18.7)
-    const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M <= 16 && fewrows_takes(d);
+    const bool to_fewrows = d.algo == MNI_ALGO_AUTO && d.split_k == 0 && d.M <= 32 && fewrows_takes(d);
     if (!to_fewrows &&
         ((d.algo == MNI_ALGO_AUTO && d.epilogue < MNI_EPI_BIAS_GELU_DUAL) || d.algo == MNI_ALGO_SKINNY || d.algo == MNI_ALGO_SKINNY_TWO_PASS ||
          d.algo == MNI_ALGO_GEMV)) {

@@ -43,6 +43,7 @@ __device__ __forceinline__ float fn_pick(const f32x4 &v, int j) { return j == 0 
 template <int SETS>
 __global__ __launch_bounds__(FN_THREADS) void gemm_fewrows_nt_kernel(const FewNtLaunch p) {
     __shared__ __attribute__((aligned(16))) float xs[FEWROWS_NT_LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float zeros[256];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 3, b = lane >> 2;
@@ -57,10 +58,12 @@ __global__ __launch_bounds__(FN_THREADS) void gemm_fewrows_nt_kernel(const FewNt
         const f32x4 v = *reinterpret_cast<const f32x4 *>(p.X + (int64_t)min(row, M - 1) * p.x_rs + 4 * c4);
         *reinterpret_cast<f32x4 *>(&xs[row * pitch + 4 * c4]) = v;
     }
+    if (tid < 256) zeros[tid] = 0.0f;
     __syncthreads();
 
     const int ngroups = (N + 3) >> 2;
     const float *xrow = &xs[j * pitch + 4 * b];  // (as the A operand this lane is row 4 s + j of the set)
+    const float *zrow = &zeros[4 * lane];
     for (int g = blockIdx.x + (int)gridDim.x * wave; g < ngroups; g += (int)gridDim.x * FN_WAVES) {
         const int col = 4 * g + j;
         const float *wp = p.W + (int64_t)min(col, N - 1) * p.w_cs + 4 * b;  // columns past N repeat the last one: never stored
@@ -68,26 +71,36 @@ __global__ __launch_bounds__(FN_THREADS) void gemm_fewrows_nt_kernel(const FewNt
 #pragma unroll
         for (int s = 0; s < SETS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
         // No branch around a request: the compiler counts the loads in flight per path and waits for the fewest.
-        // Requests beyond the last step repeat it (the lines are in the L1 by then); steps beyond it multiply zeros.
+        // Requests beyond the last step repeat it (the lines are in the L1 by then); steps beyond it read zeros for A (a
+        // select on the values would have to wait for them where they are asked for).
         f32x4 wr[FN_RING];
 #pragma unroll
         for (int r = 0; r < FN_RING; ++r) wr[r] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(wp + 64 * min(r, steps - 1)));
+        // A's values for a step are asked of LDS a step ahead (up to 16 rows; with 32 the registers do not reach): the round
+        // trip to LDS in front of every group of MFMAs is what a wavefront otherwise waits out alone.
+        constexpr int XB = SETS <= 4 ? 2 : 1;
+        f32x4 xa[XB][SETS];
+        auto fetch = [&](int t, f32x4 *dst) {
+            const float *src = t < steps ? xrow + 64 * t : zrow;  // (uniform choice)
+            const int set_pitch = t < steps ? 4 * pitch : 0;
+#pragma unroll
+            for (int s = 0; s < SETS; ++s) dst[s] = *reinterpret_cast<const f32x4 *>(src + s * set_pitch);
+        };
+        static_assert(FN_RING % 2 == 0, "the two buffers of A alternate with the step's parity");
+        if (XB == 2) fetch(0, xa[0]);
         for (int t0 = 0; t0 < steps; t0 += FN_RING) {
 #pragma unroll
             for (int r = 0; r < FN_RING; ++r) {
                 const int t = t0 + r;
-                const bool live = t < steps;
-                const int tl = min(t, steps - 1);
-                f32x4 xa[SETS];
-#pragma unroll
-                for (int s = 0; s < SETS; ++s) {
-                    xa[s] = *reinterpret_cast<const f32x4 *>(xrow + s * 4 * pitch + 64 * tl);
-                    if (!live) xa[s] = f32x4{0.f, 0.f, 0.f, 0.f};
-                }
+                if (XB == 2) fetch(t + 1, xa[(r + 1) & 1]);
+                else fetch(t, xa[0]);
+                const f32x4 *x = xa[XB == 2 ? (r & 1) : 0];
+                // (a uniform branch around the MFMAs of the steps past the last -- their operands are zeros -- made the compiler
+                // spill and the 16-row product take 48 us instead of 33)
 #pragma unroll
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
-                    for (int s = 0; s < SETS; ++s) acc[s] = __builtin_amdgcn_mfma_f32_4x4x1f32(fn_pick(xa[s], c), fn_pick(wr[r], c), acc[s], 0, 0, 0);
+                    for (int s = 0; s < SETS; ++s) acc[s] = __builtin_amdgcn_mfma_f32_4x4x1f32(fn_pick(x[s], c), fn_pick(wr[r], c), acc[s], 0, 0, 0);
                 wr[r] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(wp + 64 * min(t + FN_RING, steps - 1)));
             }
         }
