@@ -702,6 +702,14 @@ def run_for_counters(r, which):
         for mrows in (16, 32):
             for i in range(16):
                 r.sgemm(mrows, 4096, 4096, x, ws[i % 8], dst)
+    elif which == "nt_rows":
+        # 4 and 16 token rows against a [4096, 4096] weight stored [out, in] (rows . W^T: dX = dY W^T of a small batch), eight weights
+        # in rotation (every byte of W from HBM): the few-rows kernel for a K-contiguous weight with K in slices, 16 launches each
+        x = r.to_device(synth.normal(4, (16, 4096), 0.02))
+        ws = [r.to_device(synth.normal(4, (4096, 4096), 0.02, stream=1 + i)) for i in range(8)]
+        for mrows in (4, 16):
+            for i in range(16):
+                r.sgemm(mrows, 4096, 4096, x, ws[i % 8], dst, b_strides=(1, 4096))
     elif which == "outer":
         # the weight gradient of a [4096, 4096] layer under 8 rows (the outer-product kernel), overwriting and
         # accumulating, 5 launches each
@@ -889,7 +897,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations")
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
-    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "config4", "config5b", "fewrows", "decode_rows", "outer", "attention", "attention_bwd"], default=None,
+    ap.add_argument("--counters", choices=["gemm", "gemv", "streamk", "config3", "config4", "config5b", "fewrows", "decode_rows", "nt_rows", "outer", "attention", "attention_bwd"], default=None,
                     help="for rocprofv3 --pmc runs: launch a copy kernel of known size (64 MiB read + 64 MiB "
                          "written) 3 times, then the chosen product 5 times, and exit")
     ap.add_argument("--planner-sweep", metavar="JSON", default=None, help="time every forced plan on the planner's shape list and write the best per shape")
