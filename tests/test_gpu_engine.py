@@ -94,6 +94,8 @@ CASES = [
     ((2, 1, 6, 4), (1, 3, 4, 5)),     # the modulo batch rule
     ((2, 300), (300, 512)),           # skinny
     ((600, 32), (32, 3)),             # few output columns
+    ((6, 2048), (2048, 4096)),        # a small batch under a wide layer: dA = dC B^T reads B K-contiguous, K = 4096 in slices
+    ((3, 1024), (1024, 1280)),        # the same with a K of 1280: all of it per wavefront
 ]
 
 
