@@ -1304,6 +1304,25 @@ def test_fewrows_nt_kernel_in_k_slices_normal_inputs_and_what_it_refuses(dev, ro
             run_gemm(dev, aa, bb, False, True, algo=N.ALGO_FEWROWS_NT, split_k=split)
 
 
+def test_fewrows_kernels_share_their_counters_launch_after_launch(dev, rocm):
+    # the sliced kernel for a K-contiguous B and the few-rows kernel for a row-major B count their K slices in at the same
+    # array of counters (every count wraps back to zero with its last arrival): products of different unit and slice counts
+    # one after the other, ten rounds, every result integer-exact
+    cases = []
+    for m, n, k, tb, split, algo in ((16, 4096, 4096, True, 4, N.ALGO_FEWROWS_NT), (8, 1000, 2048, True, 2, N.ALGO_FEWROWS_NT),
+                                     (24, 1280, 4096, False, 0, N.ALGO_FEWROWS), (5, 2112, 3072, True, 3, N.ALGO_FEWROWS_NT),
+                                     (12, 640, 8192, False, 0, N.ALGO_FEWROWS), (3, 520, 4096, True, 16, N.ALGO_FEWROWS_NT)):
+        a = synth.small_ints(m + n, (m, k), 3)
+        b = synth.small_ints(n + k, (n, k) if tb else (k, n), 3, stream=1)
+        want = (a.astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(np.float32)
+        cases.append((m, n, k, dev.put(a), dev.put(b), dev.empty(m * n, fill=-7.0), tb, split, algo, want))
+    for _ in range(10):
+        for m, n, k, dA, dB, dC, tb, split, algo, want in cases:
+            rocm.sgemm(m, n, k, dA, dB, dC, b_strides=(1, k) if tb else (n, 1), algo=algo, split_k=split)
+    for m, n, k, dA, dB, dC, tb, split, algo, want in cases:
+        assert np.array_equal(rocm.to_host(dC, (m, n)), want), (m, n, k)
+
+
 @pytest.mark.parametrize("m", [1, 3, 5, 7])
 def test_skinny_cols_decode_shape_normal_inputs(dev, m):
     # the kernels specialised for a row count: within tolerance of a float64 product and of the two-launch form,
