@@ -176,9 +176,10 @@ int launch_gemm_fewrows_nt(const GemmLaunch &g, int amode, int bmode) {
 // of the chip one group each however K is cut.  So a workgroup takes 64 columns (a group per wavefront) and one slice
 // of K -- a run of steps of 64 values, at most 16 of them (12 beyond 16 rows) -- and:
 //   * A's slice goes from memory straight into LDS (wavefront w brings row w, and row w + 16 of 32: a load instruction
-//     per block, 1 KB, which the hardware lays down in lane order, i.e. as the row lies in memory); the loads of W are
-//     issued right behind and stay in flight across the workgroup's one barrier: loads complete in the order of issue, so
-//     `s_waitcnt vmcnt(RING)` says A has landed when only W's are outstanding.
+//     per four steps, 1 KB, which the hardware lays down in lane order, i.e. as the row lies in memory) and is waited
+//     for before anybody asks for W: a CU takes requests only as fast as earlier ones are answered, and behind the first
+//     wavefronts' loads of W the barrier that says "A is in LDS" would fall when most of W is in, with every MFMA of the
+//     workgroup still to come.
 //   * the steps are gemm_fewrows_nt_kernel's; a slice is at most RING steps long, so all of its W is requested before the
 //     first MFMA and there is no loop.
 //   * the slices of a column block run on one XCD (workgroup id = 8 q + XCD; q = block of eight column blocks x slice),
