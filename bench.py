@@ -292,6 +292,27 @@ def bench_extras(r, with_cpu):
         r.free(xb)
         r.free(yb)
     out["rows_x_transposed_4096x4096_weight_cold"] = rows_t
+    # the decode product against larger row-major weights (the shapes of a 7B-class model's layers), 4 rows, cold (two or three
+    # weights in rotation, more than the Infinity Cache holds): what the launch, the first access and the sum of the K slices cost
+    # weighs less the longer the stream is -- not a BASELINE config
+    big_out = {}
+    for (n_, k_) in ((11008, 4096), (8192, 8192), (32000, 4096)):
+        nbuf = 3 if n_ * k_ * 4 < (200 << 20) else 2
+        wb = [r.malloc(n_ * k_ * 4) for _ in range(nbuf)]
+        for w_ in wb:
+            r.fill(w_, 0.01, n_ * k_)
+        xb = r.to_device(synth.normal(5, (4, k_)))
+        yb = r.malloc(4 * n_ * 4)
+        descs = [r.gemm_desc(4, n_, k_, xb, w_, yb) for w_ in wb]
+        r.sgemm_timed(descs, 20, 60)
+        us = min(r.sgemm_timed(descs, 10, 60) for _ in range(3)) * 1e3
+        byb = 4.0 * (n_ * k_ + 4 * k_ + 4 * n_)
+        big_out["4x%dx%d" % (n_, k_)] = {"us": us, "GB/s": byb / us / 1e3, "frac_hbm": byb / us / 1e3 / PEAK_HBM_GBPS}
+        r.free(xb)
+        r.free(yb)
+        for w_ in wb:
+            r.free(w_)
+    out["decode_gemv_larger_weights_cold"] = big_out
     # token rows against a weight stored [out, in] (a tied language-model head: logits = x E^T with E [50304, 768]), E cold
     # (four in rotation, 618 MB) -- not a BASELINE config
     head_out = {}
