@@ -75,3 +75,57 @@ def test_random_products_are_integer_exact(rocm, seed):
         assert np.array_equal(got.astype(np.float64), want), what
         ran += 1
     assert ran >= 100
+
+
+FEW_M = [1, 2, 3, 4, 5, 7, 8, 9, 12, 16, 17, 24, 32]
+FEW_N = [64, 65, 132, 1003, 1024, 2048, 2050, 4096, 4100, 8192]
+FEW_K = [64, 256, 512, 640, 768, 960, 1024, 1088, 1984, 2048, 2112, 3072, 4096]
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_random_few_rows_against_wide_operands_are_integer_exact(rocm, seed):
+    # the decode family under the planner: 1 to 32 rows against a wide B, three times in four stored K-contiguous (a weight kept
+    # [out, in]); pitches off their extents (whole 16 bytes or not), operands that start 1 or 4 floats into their allocation,
+    # epilogues, accumulation.  The padding of A and B holds a huge value that must never reach C.
+    r = rocm
+    rng = random.Random(seed)
+    gen = np.random.default_rng(seed)
+    for case in range(60):
+        m, n, k = rng.choice(FEW_M), rng.choice(FEW_N), rng.choice(FEW_K)
+        while n * k > (1 << 24):
+            n = rng.choice(FEW_N)
+        tb = rng.random() < 0.75
+        pad_a, pad_b = rng.choice([0, 0, 4, 8, 3]), rng.choice([0, 0, 4, 12, 1])
+        off_a, off_b = rng.choice([0, 0, 4, 1]), rng.choice([0, 0, 4, 2])
+        sb = (n, k) if tb else (k, n)
+        lda, ldb = k + pad_a, sb[1] + pad_b
+        a = np.full((m, lda), HUGE, np.float32)
+        b = np.full((sb[0], ldb), HUGE, np.float32)
+        a[:, :k] = gen.integers(-3, 4, (m, k))
+        b[:, :sb[1]] = gen.integers(-3, 4, sb)
+        ldc = n + rng.choice([0, 0, 1, 5])
+        c0 = gen.integers(-3, 4, (m, ldc)).astype(np.float32)
+        bias = gen.integers(-3, 4, n).astype(np.float32)
+        epi = rng.choice([N.EPI_NONE, N.EPI_NONE, N.EPI_BIAS, N.EPI_BIAS_RELU])
+        acc = rng.random() < 0.25
+        what = dict(case=case, m=m, n=n, k=k, tb=tb, lda=lda, ldb=ldb, off_a=off_a, off_b=off_b, ldc=ldc, epi=epi, acc=acc)
+        d_a = r.to_device(np.concatenate([np.full(off_a, HUGE, np.float32), a.ravel()]))
+        d_b = r.to_device(np.concatenate([np.full(off_b, HUGE, np.float32), b.ravel()]))
+        d_c, d_bias = r.to_device(c0), r.to_device(bias)
+        try:
+            r.sgemm(m, n, k, d_a + 4 * off_a, d_b + 4 * off_b, d_c, a_strides=(lda, 1), b_strides=(1, ldb) if tb else (ldb, 1), ldc=ldc,
+                    epilogue=epi, bias=d_bias if epi != N.EPI_NONE else None, accumulate=acc)
+            got = r.to_host(d_c, (m, ldc))
+        finally:
+            for ptr in (d_a, d_b, d_c, d_bias):
+                r.free(ptr)
+        opb = b[:, :sb[1]].T if tb else b[:, :sb[1]]
+        want = a[:, :k].astype(np.float64) @ opb.astype(np.float64)
+        if epi != N.EPI_NONE:
+            want = want + bias
+        if epi == N.EPI_BIAS_RELU:
+            want = np.maximum(want, 0.0)
+        if acc:
+            want = want + c0[:, :n]
+        assert np.array_equal(got[:, :n], want.astype(np.float32)), what
+        assert np.array_equal(got[:, n:], c0[:, n:]), ("the padding of C was written", what)
