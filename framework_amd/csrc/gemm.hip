@@ -396,10 +396,13 @@ static bool fewrows_plan(const GemmLaunch &g, int cus) {
 // 1 x 32000 x 1024 (27.8 / 27.3) and 2 x 4096 x 1984 (9.2 / 9.1); behind at K = 512 and below (4 x 128256 x 512 57.0 / 51.3, 1 x 65536 x 256
 // 25.7 / 20.2) and, beyond 16 rows, wherever K is not 768: the steps past the last in the ring of 12 loads multiply zeros, 32 MFMAs each
 // (24 x 8192 x 960 17.4 against 15.5, 32 x 32000 x 960 50.4 against 36.5).
+// (K beyond 1984: where A still fits LDS -- 2048 values of up to 16 rows, 4096 of up to 8, 8192 of up to 4 -- fewrows_nt_sliced_plan
+// decides between this form and the sliced one, and comes first.)
 static bool fewrows_nt_plan(const GemmLaunch &g, int cus) {
     (void)cus;
     if (g.M > 16) return g.K == 768 && g.N >= 8192;
-    if (g.M > 4) return g.K >= 512 && g.N >= 2048;
+    if (g.M > 8) return g.K >= 512 && g.N >= 2048;
+    if (g.M > 4) return g.K >= 512 && g.N >= 1024;  // (8 x 1024 x 4096 11.7 against 16.8; 16 rows 21.6 against 12.3)
     return g.K >= 640 && g.N >= 1024;
 }
 // K slices for the sliced form of that kernel (0: not this form).  A slice is a run of steps of 64 values of K, at most
@@ -422,18 +425,26 @@ static int fewrows_nt_slices(const GemmLaunch &g, int cus, int want) {
     }
     return best;
 }
-// Measured cold on MI355X (us; this form / the dots kernel / 64 x 64 tiles in K slices), W [N, K]:
+// Measured cold on MI355X (us; the sliced form / the dots kernel / 64 x 64 tiles in K slices), W [N, K]:
 //    rows    4096 x 4096        8192 x 8192         32000 x 4096          4096 x 11008        1024 x 8192         4096 x 2048         2048 x 2048
 //      1   14.2 / 17.7 / 24.7   49.5 / 54.0 / 87.2   94.9 /  96.5 / 127   36.3 / 43.5 / 64.7   14.3 / 21.4 / 18.2   12.1 / 10.2 / 15.2   12.7 /  8.0 / 14.3
 //      4   14.5 / 18.7 / 25.1   51.1 / 55.3 / 88.3   96.7 /  97.6 / 129   38.1 / 44.5 / 65.0   15.1 / 22.9 / 18.4   12.4 / 11.3 / 15.1   13.2 /  9.2 / 14.6
 //      8   15.1 / 22.8 / 25.3   53.8 / 61.6 / 88.5  100.3 / 113.7 / 129   41.9 / 51.8 / 65.5   17.1 / 30.6 / 18.9   13.1 / 14.9 / 15.6   14.3 / 12.7 / 14.8
 //     16   17.1 / 31.7 / 25.7   62.7 / 88.6 / 89.6  112.5 / 167.5 / 131   52.4 / 67.4 / 66.4   21.9 / 45.2 / 19.1   15.4 / 22.0 / 15.9   17.2 / 20.1 / 15.1
 // (the same weights stored [K, N] take 12.2-14.1 us at 4096 x 4096 through the decode product).  With 17 to 32 rows the 32
-// MFMAs per load weigh: 41-45 us against the tiles' 28 at 4096 x 4096.
+// MFMAs per load weigh: 41-45 us against the tiles' 28 at 4096 x 4096.  Where LDS holds all of A's K the unsliced form is the third
+// choice, and from about 5000 columns on the first: 1 x 32000 x 4096 81.9, 1 x 8192 x 8192 45.5, 8 x 32000 x 4096 84.8, 8 x 14336 x 4096 41.6,
+// 1 x 2048 x 2048 6.5, 4 x 4096 x 2048 9.5, 8 x 4096 x 2048 10.4, 16 x 4096 x 2048 14.0.
 static bool fewrows_nt_sliced_plan(const GemmLaunch &g, int cus) {
     (void)cus;
-    const int kmax = FEWROWS_NT_LDS_FLOATS / 16 - 16;  // (up to there the unsliced form holds A in LDS)
-    if (g.M > 16 || g.K <= kmax || (int64_t)g.N * g.K < (1 << 23)) return false;
+    // (up to there the unsliced form holds A in LDS: 2048 values of up to 16 rows, 4096 of up to 8, 8192 of up to 4)
+    const int kmax = FEWROWS_NT_LDS_FLOATS / (g.M > 8 ? 16 : g.M > 4 ? 8 : 4) - 16;
+    if (g.M > 16 || (int64_t)g.N * g.K < (1 << 23)) return false;
+    // Where the unsliced form holds A it is ahead from about 5000 columns on -- nothing to add up, no rounds of workgroups (us,
+    // unsliced / sliced: 8 x 5120 x 4096 19.7 / 25.1, 4 x 6144 x 4096 20.8 / 24.3, 4 x 8192 x 8192 47.2 / 51.1, 8 x 14336 x 4096 41.7 / 51.0,
+    // 1 x 32000 x 4096 81.9 / 94.7, 16 x 16384 x 2048 29.9 / 32.0) -- and behind at 4096, where three wavefronts in four have no group
+    // of columns (4 x 4096 x 4096 16.0 / 14.5, 8 rows 17.4 / 15.1).
+    if (g.K <= kmax && (g.N >= 5120 || g.K <= 2048)) return false;
     return g.M > 8 ? g.N >= 2048 : (g.K >= 4096 || g.M >= 8);
 }
 // Whether run_mfma gives the product to the sliced form by itself.
@@ -540,7 +551,7 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
             fs = fs_ok ? fewrows_nt_slices(g, cus, d.split_k > 1 ? d.split_k : 0) : 0;
             if (fs == 0)
                 return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel for a K-contiguous B takes one product of up to 32 rows of a K-contiguous A, operands "
-                                                  "16-byte aligned, K %% 64 == 0; at most 1984 (960 beyond 16 rows) in one piece, or in 2 to 16 slices (split_k) of at "
+                                                  "16-byte aligned, K %% 64 == 0; at most 8192 / 4096 / 2048 / 960 for up to 4 / 8 / 16 / 32 rows in one piece, or in 2 to 16 slices (split_k) of at "
                                                   "most 1024 (768) each");
         } else if (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && fewrows_nt_sliced_takes(g, amode, bmode)) {
             fs = fewrows_nt_slices(g, cus, 0);
@@ -558,7 +569,7 @@ static int run_mfma(const mni_gemm_desc &d, PlanProbe *probe = nullptr) {
     if (d.algo == MNI_ALGO_FEWROWS_NT || (d.algo == MNI_ALGO_AUTO && d.split_k == 0 && gemm_fewrows_nt_eligible(g, amode, bmode) && fewrows_nt_plan(g, cus))) {
         if (!gemm_fewrows_nt_eligible(g, amode, bmode) || d.split_k > 1)
             return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel for a K-contiguous B takes one product of up to 32 rows of a K-contiguous A, K %% 64 == 0 and "
-                                              "short enough for A to sit in LDS (1984, 960 beyond 16 rows), operands 16-byte aligned, no split_k");
+                                              "short enough for A to sit in LDS (8192 / 4096 / 2048 / 960 for up to 4 / 8 / 16 / 32 rows), operands 16-byte aligned, no split_k");
         if (probe) { probe->kind = PlanProbe::FEWROWS; return MNI_OK; }
         return launch_gemm_fewrows_nt(g, amode, bmode);
     }

@@ -16,7 +16,7 @@
 //     of the load is the B operand of the MFMAs for K value 64 t + 4 b + c, one MFMA per set of four rows of A, whose
 //     A operand lane (b, i) reads from LDS: row 4 s + i, the same K value.  Every block accumulates its own sixteenth
 //     of K; the blocks are added up at the end of the group with four butterfly steps over the lanes' block bits.
-//   * A (up to 32 rows x K) sits in LDS for the whole kernel, rows K + 16 floats apart (the 16-byte reads of the first
+//   * A (the 4, 8, 16 or 32 rows of the instantiation x K: K up to 8192, 4096, 2048, 960) sits in LDS for the whole kernel, rows K + 16 floats apart (the 16-byte reads of the first
 //     sixteen lanes -- four rows, four blocks -- then hit sixteen different bank groups).
 //   * One workgroup of 16 wavefronts per CU; column group g belongs to workgroup g % workgroups, wavefront
 //     g / workgroups % 16 (then round again): every CU gets the same number of groups to within one.  Twelve loads
@@ -140,7 +140,7 @@ static bool fn_aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 bool gemm_fewrows_nt_eligible(const GemmLaunch &g, int amode, int bmode) {
     if (amode != 0 || bmode != 0 || g.batch != 1 || g.M < 1 || g.M > 32 || g.N < 1 || g.epilogue > MNI_EPI_BIAS_GELU) return false;
     if (g.K < 64 || g.K % 64 != 0) return false;
-    const int rows = g.M > 16 ? 32 : 16;
+    const int rows = g.M > 16 ? 32 : g.M > 8 ? 16 : g.M > 4 ? 8 : 4;  // (rows of A the kernel's instantiation keeps in LDS)
     if ((int64_t)rows * (g.K + FN_XPAD) > FEWROWS_NT_LDS_FLOATS) return false;
     if (g.a_rs % 4 != 0 || g.b_cs % 4 != 0 || !fn_aligned16(g.A) || !fn_aligned16(g.B)) return false;
     if (g.a_rs < g.K || g.b_cs < g.K || g.ldc < g.N) return false;
@@ -151,8 +151,8 @@ bool gemm_fewrows_nt_eligible(const GemmLaunch &g, int amode, int bmode) {
 int launch_gemm_fewrows_nt(const GemmLaunch &g, int amode, int bmode) {
     if (!gemm_fewrows_nt_eligible(g, amode, bmode))
         return set_error(MNI_ERR_INVALID, "sgemm: the few-rows kernel for a K-contiguous B takes one product of up to 32 rows of a K-contiguous A, "
-                                          "K %% 64 == 0 and at most %d (%d beyond 16 rows), both operands 16-byte aligned with pitches in whole 16 bytes",
-                         FEWROWS_NT_LDS_FLOATS / 16 - FN_XPAD, FEWROWS_NT_LDS_FLOATS / 32 - FN_XPAD);
+                                          "K %% 64 == 0 and at most 8192 / 4096 / 2048 / 960 for up to 4 / 8 / 16 / 32 rows, both operands 16-byte aligned with "
+                                          "pitches in whole 16 bytes");
     FewNtLaunch p;
     p.X = g.A; p.W = g.B; p.out = g.C; p.bias = g.bias;
     p.M = g.M; p.N = g.N; p.K = g.K;

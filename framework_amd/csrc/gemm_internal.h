@@ -164,7 +164,7 @@ size_t gemv_units16_counters(int rows, int cols);  // counters the plan uses (on
 int launch_gemv_units16(const GemvLaunch &p);
 
 // Up to 32 rows against a wide K-contiguous operand (gemm_fewrows_nt.hip): a wavefront per 16 columns and all of K, A in LDS.
-static constexpr int FEWROWS_NT_LDS_FLOATS = 32768;  // 16 (or 32) rows of K + 4 floats
+static constexpr int FEWROWS_NT_LDS_FLOATS = 33024;  // 4, 8, 16 or 32 rows of K + 16 floats: 8 rows of 4096, 16 of 2048
 struct FewNtLaunch {
     const float *X;     // [M, K], rows x_rs apart
     const float *W;     // [N, K], rows w_cs apart

@@ -156,8 +156,9 @@ enum { MNI_EPI_NONE = 0, MNI_EPI_BIAS = 1, MNI_EPI_BIAS_RELU = 2, MNI_EPI_BIAS_G
  * FEWROWS_NT = up to 32 rows of a
  * K-contiguous A against a wide B that is K-contiguous too (a weight stored
  * [out, in], given as its transposed view): a wavefront per 4 columns on
- * the 4 x 4 x 1 MFMA, A resident in LDS; with K up to 1984 (960 beyond 16
- * rows) all of K per wavefront and no sums across wavefronts, with a larger
+ * the 4 x 4 x 1 MFMA, A resident in LDS; with K up to 8192 / 4096 / 2048 /
+ * 960 for up to 4 / 8 / 16 / 32 rows all of K per wavefront and no sums
+ * across wavefronts, with a larger
  * K, or with a split_k of 2 to 16, K in that many slices of at most 1024
  * values (768 beyond 16 rows) that the last workgroup of a column block to
  * arrive adds up (error unless one batch, K % 64 == 0 and within those

@@ -1190,10 +1190,11 @@ def test_decode_product_16_row_forms_take_operands_off_a_128_byte_boundary(dev, 
 
 # ---- few rows against a wide K-contiguous operand (a weight stored [out, in]): a wavefront per 16 columns, all of K ----
 @pytest.mark.parametrize("m,n,k", [(16, 50304, 768), (9, 20000, 256), (32, 16400, 512), (17, 16384, 960), (12, 33000, 1984), (1, 4096, 64),
-                                   (8, 1000, 128), (32, 70, 320), (16, 16, 1984), (5, 4099, 768), (3, 9001, 512), (8, 16384, 768)])
+                                   (8, 1000, 128), (32, 70, 320), (16, 16, 1984), (5, 4099, 768), (3, 9001, 512), (8, 16384, 768),
+                                   (4, 5000, 8192), (8, 6144, 4096), (2, 300, 4096), (16, 5120, 2048), (7, 2052, 4032)])
 def test_fewrows_nt_kernel_integer_exact(dev, rocm, m, n, k):
-    # one and two 16-row sets, column counts off a multiple of 16, K at both ends of what fits LDS, K off a multiple of
-    # the ring of loads, fewer column groups than CUs; forced and as the planner's choice
+    # one to eight sets of four rows, column counts off a multiple of 16, K at both ends of what fits LDS (8192 values of 4 rows,
+    # 4096 of 8, 2048 of 16), K off a multiple of the ring of loads, fewer column groups than CUs; forced and as the planner's choice
     a = synth.small_ints(m + n, (m, k), 3)
     bt = synth.small_ints(n + k, (n, k), 3, stream=1)
     want = (a.astype(np.int64) @ bt.T.astype(np.int64)).astype(np.float32)
