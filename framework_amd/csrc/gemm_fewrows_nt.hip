@@ -76,31 +76,42 @@ __global__ __launch_bounds__(FN_THREADS) void gemm_fewrows_nt_kernel(const FewNt
         f32x4 wr[FN_RING];
 #pragma unroll
         for (int r = 0; r < FN_RING; ++r) wr[r] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(wp + 64 * min(r, steps - 1)));
-        // A's values for a step are asked of LDS a step ahead (up to 16 rows; with 32 the registers do not reach): the round
-        // trip to LDS in front of every group of MFMAs is what a wavefront otherwise waits out alone.
-        constexpr int XB = SETS <= 4 ? 2 : 1;
-        f32x4 xa[XB][SETS];
-        auto fetch = [&](int t, f32x4 *dst) {
-            const float *src = t < steps ? xrow + 64 * t : zrow;  // (uniform choice)
+        // A's values are asked of LDS ahead of the MFMAs that use them -- the round trip to LDS in front of every group of MFMAs is
+        // what a wavefront otherwise waits out alone.  Up to 16 rows: a step ahead, two sets of registers that alternate with
+        // the step's parity.  With 32 rows (eight sets of four) the registers do not reach for that.
+        constexpr int HS = SETS <= 4 ? SETS : SETS / 2;  // sets per buffer
+        f32x4 xa[2][HS];
+        auto fetch = [&](int t, int s0, f32x4 *dst) {
+            const float *src = t < steps ? xrow + 64 * t + s0 * 4 * pitch : zrow;  // (uniform choice)
             const int set_pitch = t < steps ? 4 * pitch : 0;
 #pragma unroll
-            for (int s = 0; s < SETS; ++s) dst[s] = *reinterpret_cast<const f32x4 *>(src + s * set_pitch);
+            for (int s = 0; s < HS; ++s) dst[s] = *reinterpret_cast<const f32x4 *>(src + s * set_pitch);
+        };
+        auto mfmas = [&](int r, int s0, const f32x4 *x) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int s = 0; s < HS; ++s) acc[s0 + s] = __builtin_amdgcn_mfma_f32_4x4x1f32(fn_pick(x[s], c), fn_pick(wr[r], c), acc[s0 + s], 0, 0, 0);
         };
         static_assert(FN_RING % 2 == 0, "the two buffers of A alternate with the step's parity");
-        if (XB == 2) fetch(0, xa[0]);
+        if (SETS <= 4) fetch(0, 0, xa[0]);
         for (int t0 = 0; t0 < steps; t0 += FN_RING) {
 #pragma unroll
             for (int r = 0; r < FN_RING; ++r) {
                 const int t = t0 + r;
-                if (XB == 2) fetch(t + 1, xa[(r + 1) & 1]);
-                else fetch(t, xa[0]);
-                const f32x4 *x = xa[XB == 2 ? (r & 1) : 0];
                 // (a uniform branch around the MFMAs of the steps past the last -- their operands are zeros -- made the compiler
                 // spill and the 16-row product take 48 us instead of 33)
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-#pragma unroll
-                    for (int s = 0; s < SETS; ++s) acc[s] = __builtin_amdgcn_mfma_f32_4x4x1f32(fn_pick(x[s], c), fn_pick(wr[r], c), acc[s], 0, 0, 0);
+                if (SETS <= 4) {
+                    fetch(t + 1, 0, xa[(r + 1) & 1]);
+                    mfmas(r, 0, xa[r & 1]);
+                } else {
+                    // (the halves of a step alternating, as in the sliced form below, make the compiler spill here: the ring's
+                    // twelve addresses are live as well)
+                    fetch(t, 0, xa[0]);
+                    fetch(t, HS, xa[1]);
+                    mfmas(r, 0, xa[0]);
+                    mfmas(r, HS, xa[1]);
+                }
                 wr[r] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(wp + 64 * min(t + FN_RING, steps - 1)));
             }
         }
@@ -261,32 +272,39 @@ __global__ __launch_bounds__(FN_THREADS) void gemm_fewrows_nt_sliced_kernel(cons
     for (int s = 0; s < SETS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
     const float *xrow = &xs[j * pitch + 4 * b];  // (as the A operand this lane is row 4 s + j of the set)
     const float *zrow = &zeros[4 * lane];
-    // A's values for a step are asked of LDS a step ahead (up to 16 rows; with 32 the registers do not reach): alone on its SIMD
-    // for most of its steps -- the wavefronts get their W one after the other -- a wavefront would otherwise wait out an LDS
-    // round trip in front of every group of MFMAs.
-    constexpr int XB = SETS <= 4 ? 2 : 1;
-    f32x4 xa[XB][SETS];
+    // A's values are asked of LDS ahead of the MFMAs that use them: alone on its SIMD for most of its steps -- the wavefronts get
+    // their W one after the other -- a wavefront would otherwise wait out an LDS round trip in front of every group of MFMAs.
+    // Up to 16 rows a step ahead (two sets of registers that alternate with the step's parity); with 32 rows the halves of a
+    // step alternate (sets 4-7 under the MFMAs of sets 0-3, sets 0-3 of the next step under those of sets 4-7).
+    constexpr int HS = SETS <= 4 ? SETS : SETS / 2;  // sets per buffer
+    f32x4 xa[2][HS];
     // (steps past the slice's last read zeros for A: a select on the values would have to wait for them where they are asked for)
-    auto fetch = [&](int t, f32x4 *dst) {
-        const float *src = t < steps ? xrow + 64 * t : zrow;  // (uniform choice)
+    auto fetch = [&](int t, int s0, f32x4 *dst) {
+        const float *src = t < steps ? xrow + 64 * t + s0 * 4 * pitch : zrow;  // (uniform choice)
         const int set_pitch = t < steps ? 4 * pitch : 0;
 #pragma unroll
-        for (int s = 0; s < SETS; ++s) dst[s] = *reinterpret_cast<const f32x4 *>(src + s * set_pitch);
+        for (int s = 0; s < HS; ++s) dst[s] = *reinterpret_cast<const f32x4 *>(src + s * set_pitch);
     };
-    if (XB == 2) fetch(0, xa[0]);
-    // a slice is at most RING steps long (fewrows_nt_max_steps)
-#pragma unroll
-    for (int r = 0; r < RING; ++r) {
-        if (XB == 2) {
-            if (r + 1 < RING) fetch(r + 1, xa[(r + 1) & 1]);
-        } else {
-            fetch(r, xa[0]);
-        }
-        const f32x4 *x = xa[XB == 2 ? (r & 1) : 0];
+    auto mfmas = [&](int r, int s0, const f32x4 *x) {
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
-            for (int s = 0; s < SETS; ++s) acc[s] = __builtin_amdgcn_mfma_f32_4x4x1f32(fn_pick(x[s], c), fn_pick(wr[r], c), acc[s], 0, 0, 0);
+            for (int s = 0; s < HS; ++s) acc[s0 + s] = __builtin_amdgcn_mfma_f32_4x4x1f32(fn_pick(x[s], c), fn_pick(wr[r], c), acc[s0 + s], 0, 0, 0);
+    };
+    fetch(0, 0, xa[0]);
+    // a slice is at most RING steps long (fewrows_nt_max_steps)
+#pragma unroll
+    for (int r = 0; r < RING; ++r) {
+        if (SETS <= 4) {
+            if (r + 1 < RING) fetch(r + 1, 0, xa[(r + 1) & 1]);
+            mfmas(r, 0, xa[r & 1]);
+        } else {
+            fetch(r, HS, xa[1]);
+            mfmas(r, 0, xa[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (r + 1 < RING) fetch(r + 1, 0, xa[0]);
+            mfmas(r, HS, xa[1]);
+        }
         __builtin_amdgcn_sched_barrier(0);  // (or every step's reads of A are hoisted to the top)
     }
     // the sixteen blocks' shares of K, added up over the lanes' block bits (every lane ends with the whole sum)
