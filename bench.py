@@ -731,6 +731,16 @@ def run_for_counters(r, which):
         for mrows in (4, 16):
             for i in range(16):
                 r.sgemm(mrows, 4096, 4096, x, ws[i % 8], dst, b_strides=(1, 4096))
+        # ... and 1 and 8 rows against a [14336, 4096] weight of the same layout, two in rotation (470 MB): the unsliced form (all of K
+        # per wavefront, no partial sums), 8 launches each
+        for w in ws:
+            r.free(w)
+        wl = [r.malloc(14336 * 4096 * 4) for _ in range(2)]
+        for w in wl:
+            r.fill(w, 0.01, 14336 * 4096)
+        for mrows in (1, 8):
+            for i in range(8):
+                r.sgemm(mrows, 14336, 4096, x, wl[i % 2], dst, b_strides=(1, 4096))
     elif which == "outer":
         # the weight gradient of a [4096, 4096] layer under 8 rows (the outer-product kernel), overwriting and
         # accumulating, 5 launches each
