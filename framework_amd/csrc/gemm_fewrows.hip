@@ -152,8 +152,9 @@ __global__ __launch_bounds__(256, 2) void gemm_fewrows_kernel(const GemmLaunch g
             for (int bb = 0; bb < FR_CHUNK; ++bb) {
                 const int b = c * FR_CHUNK + bb;
                 const int d = bb % FR_DEPTH;
-                f32x4 a = Ac[(2 * bb + h) * FR_PITCH + i];
-                if (b > last) a = f32x4{0.f, 0.f, 0.f, 0.f};
+                // (blocks beyond the range: their quads of A were stored as zeros by a_request, so nothing is selected here -- a
+                // select on the values would have to wait for them right behind the read)
+                const f32x4 a = Ac[(2 * bb + h) * FR_PITCH + i];
 #pragma unroll
                 for (int u = 0; u < 4; ++u)
 #pragma unroll
